@@ -1,0 +1,195 @@
+/*
+ * tq_hip.h -- C ABI of libtq_hip.so, the MI355X (gfx950) TurboQuant KV-cache kernels.
+ *
+ * The reference project is pure Python and has no FFI of its own; each entry
+ * point below names the reference function (file:line, relative to the
+ * reference checkout) whose arithmetic it replaces.  The host side that mirrors
+ * the reference's Python API binds these symbols with ctypes.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless the comment says "host";
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream);
+ *   - `dtype` tags the element type of floating inputs: TQ_F32 / TQ_F16 / TQ_BF16;
+ *   - the caller allocates every output and the decode workspace; no entry
+ *     point allocates, frees or synchronises;
+ *   - the library keeps no mutable global state: calls on different streams
+ *     may overlap;
+ *   - return value: 0 on success, a negative TQ_E* code for a rejected argument
+ *     (nothing was launched), or a positive hipError_t from the launch.
+ */
+#ifndef TQ_HIP_H
+#define TQ_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TQ_ABI_VERSION 1
+
+enum { TQ_F32 = 0, TQ_F16 = 1, TQ_BF16 = 2 };
+
+enum {
+  TQ_OK = 0,
+  TQ_EINVAL = -1,       /* a size, stride or enum is out of range                */
+  TQ_EUNSUPPORTED = -2, /* a legal request this build has no kernel for          */
+  TQ_ENULL = -3         /* a required pointer is NULL                            */
+};
+
+#define TQ_PAGE_TOKENS 16
+#define TQ_MAX_TERMS 15
+
+/* Per-layer constants of the key quantiser (reference quantizer.py:101-127,186-212).
+ * All arrays live in device memory and are owned by the caller. */
+typedef struct tq_layer {
+  int32_t d;               /* head_dim; multiple of 64, 64..768                             */
+  int32_t mse_bits;        /* bits of the Lloyd-Max stage = key_bits - 1, 1..4              */
+  const float *Pi;         /* d*d row-major rotation (rotation.py:17-40)                    */
+  const float *PiT;        /* its transpose, row-major                                      */
+  const float *S;          /* d*d row-major Gaussian sketch (rotation.py:43-56)             */
+  const float *ST;         /* its transpose, row-major                                      */
+  const float *centroids;  /* 2^mse_bits                                                    */
+  const float *thresholds; /* 2^mse_bits - 1 interior boundaries (quantizer.py:127)         */
+  float qjl_scale;         /* sqrt(pi/2)/d (quantizer.py:212)                               */
+  /* Walsh expansion of the codebook over the index bits, used by the decode
+   * kernel: centroids[idx] = term_const + sum_t term_coef[t] * parity(idx & term_mask[t]).
+   * Filled by tq_layer_fill_terms from the host copy of the centroids.          */
+  int32_t n_terms;
+  int32_t term_mask[TQ_MAX_TERMS];
+  float term_coef[TQ_MAX_TERMS];
+  float term_const;
+} tq_layer;
+
+/* Geometry of one page = TQ_PAGE_TOKENS tokens of one KV head (new design; the
+ * reference keeps python lists of chunk tensors, store.py:59-63).  Offsets are
+ * in bytes from the start of the page.
+ *   planes : key_bits bit-planes (MSE index bits high..low, then the QJL sign),
+ *            each stored as [d/32 words][16 tokens] uint32; bit i of word j of
+ *            token n is coordinate 32*j+i.
+ *   norm   : 16 key norms in the input dtype (2 or 4 bytes) ; rnorm : 16 fp32 ||r||.
+ *   vdata  : per channel a little-endian field of 16*value_bits bits, token n's
+ *            code at bit value_bits*n ; channels consecutive.
+ *   vscale / vzero : [d/group][16 tokens] in the input dtype.                 */
+typedef struct tq_page_layout {
+  int32_t d, mse_bits, value_bits, group_size, dtype;
+  int32_t off_planes, off_norm, off_rnorm, off_vdata, off_vscale, off_vzero;
+  int32_t page_bytes;      /* stride between (page, head) records, multiple of 128 */
+} tq_page_layout;
+
+int tq_version(void);
+
+/* Host helper: fills the term_* fields of `layer` from a HOST array of its
+ * 2^mse_bits centroids; coefficients below 1e-9 of the largest are dropped. */
+int tq_layer_fill_terms(tq_layer *layer /*host*/, const float *centroids_host);
+
+/* Host helper: computes the page geometry for inputs of `dtype`;
+ * value_bits 2 or 4, d a multiple of 64 and of group_size (>= 16).                     */
+int tq_page_layout_init(tq_page_layout *out /*host*/, int d, int mse_bits, int value_bits,
+                        int group_size, int dtype);
+
+/* ---- parity entry points on the reference's own tensor layouts ------------------ */
+
+/* idx = #{t : !(y <= thresholds[t])}, packed little-end-first into bytes, 1/2/4/4
+ * bits per index for mse_bits 1/2/3/4 (quantizer.py:144 + _pack_indices :38-69).
+ * y is (n_vec, d) fp32 contiguous; idx_out is (n_vec, ceil(d/per_byte)).          */
+int tq_bucketize_pack(const float *y, int64_t n_vec, int d, const float *thresholds, int mse_bits,
+                      uint8_t *idx_out, void *stream);
+
+/* bit j of byte k = (p[8k+j] > 0) (quantizer.py:214-222). p is (n_vec, d) fp32.    */
+int tq_sign_pack(const float *p, int64_t n_vec, int d, uint8_t *sign_out, void *stream);
+
+/* TurboQuantProd.quantize (quantizer.py:231-257 with :129-165 inlined).
+ * x is (n_vec, d) with `row_stride` elements between vectors.  norm_out has the
+ * input dtype, rnorm_out is fp32.  y_dbg / p_dbg (nullable, (n_vec,d) fp32)
+ * receive the rotated unit vector and the projected residual.  With
+ * mse_only != 0 only the first stage runs (TurboQuantMSE.quantize :129-149) and
+ * sign_out / rnorm_out may be NULL.                                               */
+int tq_quantize_keys(const void *x, int dtype, int64_t n_vec, int64_t row_stride, const tq_layer *layer,
+                     uint8_t *idx_out, uint8_t *sign_out, void *norm_out, float *rnorm_out,
+                     float *y_dbg, float *p_dbg, int mse_only, void *stream);
+
+/* quantize_values (kv_cache.py:45-98): per-group min/max affine codes, computed
+ * with the per-operation rounding of the input dtype.  bits 2, 4 or 8.
+ * data_out (n_vec, d*bits/8), scale_out / zero_out (n_vec, d/group) input dtype.  */
+int tq_quantize_values(const void *v, int dtype, int64_t n_vec, int64_t row_stride, int d, int group_size,
+                       int bits, uint8_t *data_out, void *scale_out, void *zero_out, void *stream);
+
+/* TurboQuantMSE.dequantize / TurboQuantProd.dequantize (quantizer.py:151-165,
+ * 259-272) -> out (n_vec, d) fp32.  norm_dtype tags `norms`.  signs / rnorms may
+ * be NULL for the MSE-only form.                                                  */
+int tq_dequant_keys(const uint8_t *idx, const uint8_t *signs, const void *norms, int norm_dtype,
+                    const float *rnorms, int64_t n_vec, const tq_layer *layer, float *out, void *stream);
+
+/* dequantize_values (kv_cache.py:101-116) -> out (n_vec, d) fp32.                  */
+int tq_dequant_values(const uint8_t *data, const void *scales, const void *zeros, int dtype, int64_t n_vec,
+                      int d, int group_size, int bits, float *out, void *stream);
+
+/* TurboQuantProd.attention_score (quantizer.py:274-302) in the rotated-query
+ * form of triton_kernels.py:49-53,138: for each of `batch` independent
+ * problems, scores[b, i, k] = norm_k * <q_i Pi^T, c[idx_k]> + qjl_scale * rnorm_k *
+ * <q_i S^T, sigma_k>.  q (batch, n_q, d) `dtype`; key arrays (batch, n_k, ...);
+ * scores (batch, n_q, n_k) fp32; no 1/sqrt(d).  work is a caller buffer of
+ * 2*batch*n_q*d floats for the rotated and sketched queries.                      */
+int tq_score(const void *q, int dtype, int64_t batch, int64_t n_q, const uint8_t *idx, const uint8_t *signs,
+             const void *norms, int norm_dtype, const float *rnorms, int64_t n_k, const tq_layer *layer,
+             float *scores, float *work, void *stream);
+
+/* q_rot = q Pi^T and q_sk = q S^T in fp32 for `rows` vectors of `dtype`
+ * (triton_kernels.py:527-528); the prologue of tq_score and of the decode kernel. */
+int tq_rotate_query(const void *q, int dtype, int64_t rows, const tq_layer *layer, float *q_rot, float *q_sk,
+                    void *stream);
+
+/* ---- paged store ---------------------------------------------------------------- */
+
+/* Quantise T new tokens of each of B sequences and write them into pages
+ * (fused a8 + a11 of the reference, store.py:73-90, for a batch of sequences).
+ * k, v: element (b, t, h, :) at  base + b*stride_b + t*stride_t + h*stride_h  (in
+ * elements), innermost dimension contiguous.  Token t of sequence b goes to
+ * logical position start_pos[b] + t, i.e. page block_table[b*max_pages + pos/16],
+ * slot pos%16.  start_pos may be NULL (all zero).  pool is (num_pages, H, page_bytes). */
+int tq_append_kv_paged(const void *k, const void *v, int dtype, int B, int T, int H, int64_t stride_b,
+                       int64_t stride_t, int64_t stride_h, const int32_t *start_pos, const int32_t *block_table,
+                       int max_pages, const tq_layer *layer, const tq_page_layout *layout, uint8_t *pool,
+                       int64_t num_pages, void *stream);
+
+/* Gather a sequence's pages back into the reference's flat tensors
+ * (store.py:92-114 get_flat_cache): idx (H, n_tok, d*eff/8), signs (H, n_tok, d/8),
+ * norms (H, n_tok) input dtype, rnorms fp32, v_data (H, n_tok, d*vb/8),
+ * v_scales / v_zeros (H, n_tok, d/group).  block_table is this sequence's row.    */
+int tq_pool_export(const uint8_t *pool, int64_t num_pages, int H, const int32_t *block_table, int n_tok,
+                   const tq_page_layout *layout, uint8_t *idx, uint8_t *signs, void *norms, float *rnorms,
+                   uint8_t *v_data, void *v_scales, void *v_zeros, void *stream);
+
+/* Bytes of workspace tq_decode_attn_paged needs for these sizes.                   */
+size_t tq_decode_workspace_bytes(int B, int Hq, int d, int n_split);
+
+/* Fused decode attention over the paged compressed history plus an optional
+ * exact tail (compute_hybrid_attention, score.py:29-173; kernel semantics of
+ * triton_kernels.py:209-356 with GQA sharing, paging and split-K added).
+ * q (B, Hq, d) `dtype` contiguous (it need not be the pages' dtype); query head h
+ * reads KV head h / (Hq/Hkv).
+ * seq_lens[b] compressed tokens of sequence b sit in block_table[b*bt_stride + i]
+ * (bt_stride = 0 shares one table among all b).  recent_k / recent_v (nullable)
+ * hold exact tokens (b, r, h, :) `dtype`, element strides rs_b, rs_r, rs_h, with
+ * recent_len[b] valid rows (NULL = recent_rows for all).  out (B, Hq, d) `dtype`:
+ * softmax(sm_scale * [scores_hist ; q k_recent^T]) [v_hist ; v_recent]; all-empty
+ * rows give zeros.                                                                */
+int tq_decode_attn_paged(const void *q, int dtype, int B, int Hq, int Hkv, const uint8_t *pool,
+                         int64_t num_pages, const int32_t *block_table, int bt_stride, const int32_t *seq_lens,
+                         float sm_scale, const tq_layer *layer, const tq_page_layout *layout,
+                         const void *recent_k, const void *recent_v, int recent_rows, int64_t rs_b,
+                         int64_t rs_r, int64_t rs_h, const int32_t *recent_len, void *out, void *workspace,
+                         int n_split, void *stream);
+
+/* Log-sum-exp merge of n_parts partial results per (b, query head):
+ * parts (B*Hq, n_parts, d+2) fp32 = [running max, sum of exp, un-normalised acc];
+ * out (B*Hq, d) `dtype`.  The same operator a context-parallel shard exchange
+ * would use.                                                                      */
+int tq_decode_merge(const float *parts, int64_t rows, int n_parts, int d, int dtype, void *out, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TQ_HIP_H */

@@ -1,0 +1,161 @@
+"""ctypes binding of libtq_hip.so (declarations: include/tq_hip.h).
+
+The library is loaded on first use.  There is no fallback: if the shared object
+is missing or a tensor is not on a GPU the call raises.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+import math
+import os
+from typing import Optional
+
+import torch
+
+TQ_F32, TQ_F16, TQ_BF16 = 0, 1, 2
+TQ_PAGE_TOKENS = 16
+TQ_MAX_TERMS = 15
+ABI_VERSION = 1
+
+_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libtq_hip.so")
+_lib: Optional[C.CDLL] = None
+
+_ERR = {-1: "TQ_EINVAL (a size, stride or enum is out of range)",
+        -2: "TQ_EUNSUPPORTED (no kernel for this shape / bit-width)",
+        -3: "TQ_ENULL (a required pointer is NULL)"}
+
+
+class TqLayer(C.Structure):
+    _fields_ = [
+        ("d", C.c_int32), ("mse_bits", C.c_int32),
+        ("Pi", C.c_void_p), ("PiT", C.c_void_p), ("S", C.c_void_p), ("ST", C.c_void_p),
+        ("centroids", C.c_void_p), ("thresholds", C.c_void_p),
+        ("qjl_scale", C.c_float),
+        ("n_terms", C.c_int32),
+        ("term_mask", C.c_int32 * TQ_MAX_TERMS),
+        ("term_coef", C.c_float * TQ_MAX_TERMS),
+        ("term_const", C.c_float),
+    ]
+
+
+class TqPageLayout(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in (
+        "d", "mse_bits", "value_bits", "group_size", "dtype",
+        "off_planes", "off_norm", "off_rnorm", "off_vdata", "off_vscale", "off_vzero", "page_bytes")]
+
+
+_vp, _i, _i64, _f = C.c_void_p, C.c_int, C.c_int64, C.c_float
+_SIGNATURES = {
+    "tq_version": (C.c_int, []),
+    "tq_layer_fill_terms": (C.c_int, [C.POINTER(TqLayer), C.POINTER(C.c_float)]),
+    "tq_page_layout_init": (C.c_int, [C.POINTER(TqPageLayout), _i, _i, _i, _i, _i]),
+    "tq_bucketize_pack": (C.c_int, [_vp, _i64, _i, _vp, _i, _vp, _vp]),
+    "tq_sign_pack": (C.c_int, [_vp, _i64, _i, _vp, _vp]),
+    "tq_quantize_keys": (C.c_int, [_vp, _i, _i64, _i64, C.POINTER(TqLayer), _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp]),
+    "tq_quantize_values": (C.c_int, [_vp, _i, _i64, _i64, _i, _i, _i, _vp, _vp, _vp, _vp]),
+    "tq_dequant_keys": (C.c_int, [_vp, _vp, _vp, _i, _vp, _i64, C.POINTER(TqLayer), _vp, _vp]),
+    "tq_dequant_values": (C.c_int, [_vp, _vp, _vp, _i, _i64, _i, _i, _i, _vp, _vp]),
+    "tq_score": (C.c_int, [_vp, _i, _i64, _i64, _vp, _vp, _vp, _i, _vp, _i64, C.POINTER(TqLayer), _vp, _vp, _vp]),
+    "tq_rotate_query": (C.c_int, [_vp, _i, _i64, C.POINTER(TqLayer), _vp, _vp, _vp]),
+    "tq_append_kv_paged": (C.c_int, [_vp, _vp, _i, _i, _i, _i, _i64, _i64, _i64, _vp, _vp, _i,
+                                     C.POINTER(TqLayer), C.POINTER(TqPageLayout), _vp, _i64, _vp]),
+    "tq_pool_export": (C.c_int, [_vp, _i64, _i, _vp, _i, C.POINTER(TqPageLayout), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "tq_decode_workspace_bytes": (C.c_size_t, [_i, _i, _i, _i]),
+    "tq_decode_attn_paged": (C.c_int, [_vp, _i, _i, _i, _i, _vp, _i64, _vp, _i, _vp, _f, C.POINTER(TqLayer),
+                                       C.POINTER(TqPageLayout), _vp, _vp, _i, _i64, _i64, _i64, _vp, _vp, _vp, _i, _vp]),
+    "tq_decode_merge": (C.c_int, [_vp, _i64, _i, _i, _i, _vp, _vp]),
+}
+
+EXPORTED_SYMBOLS = tuple(_SIGNATURES)
+
+
+def library_path() -> str:
+    return _LIB_PATH
+
+
+def lib() -> C.CDLL:
+    """Load libtq_hip.so (once) and attach the prototypes."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            raise RuntimeError(
+                f"{_LIB_PATH} is missing: build it with `python -m turboquant_amd.build` "
+                "(there is no CPU or PyTorch fallback for the TurboQuant kernels)")
+        handle = C.CDLL(_LIB_PATH)
+        for name, (res, args) in _SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype, fn.argtypes = res, args
+        got = handle.tq_version()
+        if got != ABI_VERSION:
+            raise RuntimeError(f"libtq_hip.so has ABI version {got}, the bindings expect {ABI_VERSION}")
+        _lib = handle
+    return _lib
+
+
+def check(rc: int, what: str):
+    if rc == 0:
+        return
+    if rc < 0:
+        raise ValueError(f"{what}: {_ERR.get(rc, rc)}")
+    raise RuntimeError(f"{what}: HIP error {rc}")
+
+
+def dtype_tag(dt: torch.dtype) -> int:
+    if dt == torch.float32:
+        return TQ_F32
+    if dt == torch.float16:
+        return TQ_F16
+    if dt == torch.bfloat16:
+        return TQ_BF16
+    raise TypeError(f"TurboQuant kernels take float32, float16 or bfloat16 tensors, not {dt}")
+
+
+def require_gpu(t: torch.Tensor, name: str) -> torch.Tensor:
+    if not t.is_cuda:
+        raise RuntimeError(
+            f"{name} lives on {t.device}: the TurboQuant kernels run on the GPU only and have no CPU path")
+    return t
+
+
+def ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def stream_ptr(device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def walsh_terms(centroids_host: torch.Tensor, mse_bits: int, layer: TqLayer):
+    arr = (C.c_float * (1 << mse_bits))(*[float(v) for v in centroids_host.tolist()])
+    layer.mse_bits = mse_bits
+    check(lib().tq_layer_fill_terms(C.byref(layer), arr), "tq_layer_fill_terms")
+
+
+def make_layer(d: int, mse_bits: int, Pi: torch.Tensor, PiT: torch.Tensor, centroids: torch.Tensor,
+               thresholds: torch.Tensor, S: Optional[torch.Tensor] = None, ST: Optional[torch.Tensor] = None,
+               centroids_host: Optional[torch.Tensor] = None) -> TqLayer:
+    """Describe a layer's constants to the library.  The tensors must stay alive
+    while the struct is in use; they must be fp32, contiguous and on one GPU."""
+    for name, t in (("Pi", Pi), ("PiT", PiT), ("centroids", centroids), ("thresholds", thresholds), ("S", S), ("ST", ST)):
+        if t is None:
+            continue
+        require_gpu(t, name)
+        if t.dtype != torch.float32 or not t.is_contiguous():
+            raise TypeError(f"{name} must be a contiguous float32 tensor")
+    ly = TqLayer()
+    ly.d, ly.mse_bits = d, mse_bits
+    ly.Pi, ly.PiT = Pi.data_ptr(), PiT.data_ptr()
+    ly.S = None if S is None else S.data_ptr()
+    ly.ST = None if ST is None else ST.data_ptr()
+    ly.centroids, ly.thresholds = centroids.data_ptr(), thresholds.data_ptr()
+    ly.qjl_scale = math.sqrt(math.pi / 2.0) / d
+    walsh_terms(centroids_host if centroids_host is not None else centroids.detach().cpu(), mse_bits, ly)
+    return ly
+
+
+def make_page_layout(d: int, mse_bits: int, value_bits: int, group_size: int, dtype: torch.dtype) -> TqPageLayout:
+    L = TqPageLayout()
+    check(lib().tq_page_layout_init(C.byref(L), d, mse_bits, value_bits, group_size, dtype_tag(dtype)),
+          "tq_page_layout_init")
+    return L

@@ -1,0 +1,113 @@
+// Shared device helpers for the TurboQuant gfx950 kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/tq_hip.h"
+
+#define TQ_WAVE 64
+
+#define TQ_CHECK_LAUNCH()                         \
+  do {                                            \
+    hipError_t e__ = hipGetLastError();           \
+    if (e__ != hipSuccess) return (int)e__;       \
+  } while (0)
+
+namespace tq {
+
+// ---- 16-bit float <-> fp32, bit-level so that the rounding is explicit --------------
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
+
+// round-to-nearest-even, NaN kept quiet: the rounding torch applies when an op
+// on bf16 tensors is computed in fp32 and stored back.
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+__device__ __forceinline__ float f16_bits_to_f32(uint16_t b) {
+  _Float16 h;
+  __builtin_memcpy(&h, &b, 2);
+  return (float)h;
+}
+
+__device__ __forceinline__ uint16_t f32_to_f16_bits(float f) {
+  _Float16 h = (_Float16)f;  // v_cvt_f16_f32: round-to-nearest-even
+  uint16_t b;
+  __builtin_memcpy(&b, &h, 2);
+  return b;
+}
+
+// DT is one of the TQ_F32 / TQ_F16 / TQ_BF16 tags.
+template <int DT>
+struct Elem;
+template <>
+struct Elem<TQ_F32> {
+  using storage = float;
+  static __device__ __forceinline__ float load(const void* p, int64_t i) { return ((const float*)p)[i]; }
+  static __device__ __forceinline__ void store(void* p, int64_t i, float v) { ((float*)p)[i] = v; }
+  static __device__ __forceinline__ float round(float v) { return v; }
+};
+template <>
+struct Elem<TQ_F16> {
+  using storage = uint16_t;
+  static __device__ __forceinline__ float load(const void* p, int64_t i) { return f16_bits_to_f32(((const uint16_t*)p)[i]); }
+  static __device__ __forceinline__ void store(void* p, int64_t i, float v) { ((uint16_t*)p)[i] = f32_to_f16_bits(v); }
+  static __device__ __forceinline__ float round(float v) { return f16_bits_to_f32(f32_to_f16_bits(v)); }
+};
+template <>
+struct Elem<TQ_BF16> {
+  using storage = uint16_t;
+  static __device__ __forceinline__ float load(const void* p, int64_t i) { return bf16_bits_to_f32(((const uint16_t*)p)[i]); }
+  static __device__ __forceinline__ void store(void* p, int64_t i, float v) { ((uint16_t*)p)[i] = f32_to_bf16_bits(v); }
+  static __device__ __forceinline__ float round(float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); }
+};
+
+__device__ __forceinline__ float load_as_f32(const void* p, int64_t i, int dt) {
+  if (dt == TQ_F32) return ((const float*)p)[i];
+  uint16_t b = ((const uint16_t*)p)[i];
+  return dt == TQ_F16 ? f16_bits_to_f32(b) : bf16_bits_to_f32(b);
+}
+
+__device__ __forceinline__ void store_from_f32(void* p, int64_t i, float v, int dt) {
+  if (dt == TQ_F32) ((float*)p)[i] = v;
+  else ((uint16_t*)p)[i] = dt == TQ_F16 ? f32_to_f16_bits(v) : f32_to_bf16_bits(v);
+}
+
+// ---- wave reductions ---------------------------------------------------------------
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+// ---- index packing of the reference's flat layout (quantizer.py:38-69) --------------
+
+__host__ __device__ __forceinline__ int eff_bits(int mse_bits) { return mse_bits == 1 ? 1 : (mse_bits == 2 ? 2 : (mse_bits <= 4 ? 4 : 8)); }
+__host__ __device__ __forceinline__ int idx_row_bytes(int d, int mse_bits) {
+  int per = 8 / eff_bits(mse_bits);
+  return (d + per - 1) / per;
+}
+
+// ---- page geometry -----------------------------------------------------------------
+
+// word j (32 coordinates) of plane p for token n
+__device__ __forceinline__ int plane_word_off(const tq_page_layout& L, int p, int j, int n) {
+  return L.off_planes + (((p * (L.d >> 5)) + j) * TQ_PAGE_TOKENS + n) * 4;
+}
+
+__device__ __forceinline__ const uint8_t* page_ptr(const uint8_t* pool, int64_t page, int H, int h, int page_bytes) {
+  return pool + (page * H + h) * (int64_t)page_bytes;
+}
+
+}  // namespace tq

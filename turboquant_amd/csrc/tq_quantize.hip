@@ -1,0 +1,664 @@
+// Quantise path: key quantiser (rotation, Lloyd-Max bucketise, residual, QJL sign
+// sketch), value group quantiser, and the writers for the flat (reference)
+// layout and for the paged store.
+//
+// One workgroup handles a tile of TQ_PAGE_TOKENS (16) vectors of one head with
+// d threads, thread j owning coordinate j of every vector of the tile.  The
+// three d x d contractions run in fp32 on the vector ALUs with the tile staged
+// in LDS; matrices are read column-coalesced from their row-major transposes.
+
+#include <type_traits>
+
+#include "tq_common.h"
+
+namespace tq {
+
+constexpr int TILE = TQ_PAGE_TOKENS;
+
+// ------------------------------------------------------------------------------------
+// parity entry points: bucketise+pack and sign-pack from given fp32 tensors
+// ------------------------------------------------------------------------------------
+
+__global__ void bucketize_pack_kernel(const float* __restrict__ y, int64_t n_vec, int d, const float* __restrict__ thr,
+                                      int mse_bits, uint8_t* __restrict__ out) {
+  const int eff = eff_bits(mse_bits), per = 8 / eff, row = idx_row_bytes(d, mse_bits);
+  const int n_thr = (1 << mse_bits) - 1;
+  int64_t gid = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+  if (gid >= n_vec * row) return;
+  int64_t v = gid / row;
+  int k = (int)(gid - v * row);
+  unsigned byte = 0;
+  for (int s = 0; s < per; ++s) {
+    int c = k * per + s;
+    if (c >= d) break;
+    float val = y[v * d + c];
+    unsigned idx = 0;
+    for (int t = 0; t < n_thr; ++t) idx += !(val <= thr[t]);
+    byte |= idx << (eff * s);
+  }
+  out[gid] = (uint8_t)byte;
+}
+
+__global__ void sign_pack_kernel(const float* __restrict__ p, int64_t n_vec, int d, uint8_t* __restrict__ out) {
+  const int row = (d + 7) / 8;
+  int64_t gid = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+  if (gid >= n_vec * row) return;
+  int64_t v = gid / row;
+  int k = (int)(gid - v * row);
+  unsigned byte = 0;
+  for (int s = 0; s < 8; ++s) {
+    int c = k * 8 + s;
+    if (c < d && p[v * d + c] > 0.0f) byte |= 1u << s;
+  }
+  out[gid] = (uint8_t)byte;
+}
+
+// ------------------------------------------------------------------------------------
+// tile sources: where the 16 vectors of a tile come from and which are valid
+// ------------------------------------------------------------------------------------
+
+struct FlatSource {          // (n_vec, d) with a row stride
+  int64_t n_vec, row_stride;
+  __device__ bool locate(int tile, int slot, int64_t& elem_off) const {
+    int64_t v = (int64_t)tile * TILE + slot;
+    elem_off = v * row_stride;
+    return v < n_vec;
+  }
+};
+
+struct PagedSource {         // (b, t, h, :) strided, tokens mapped onto 16-token pages
+  int B, T, H, tiles_per_seq;
+  int64_t stride_b, stride_t, stride_h;
+  const int32_t* start_pos;
+  // tile index -> (b, page slot window, head)
+  __device__ void decode(int tile, int& b, int& lpage, int& h) const {
+    h = tile % H;
+    int r = tile / H;
+    int pg = r % tiles_per_seq;
+    b = r / tiles_per_seq;
+    int s0 = start_pos ? start_pos[b] : 0;
+    lpage = s0 / TILE + pg;
+  }
+  __device__ bool locate(int tile, int slot, int64_t& elem_off) const {
+    int b, lpage, h;
+    decode(tile, b, lpage, h);
+    int s0 = start_pos ? start_pos[b] : 0;
+    int t = lpage * TILE + slot - s0;
+    elem_off = b * stride_b + (int64_t)t * stride_t + h * stride_h;
+    return t >= 0 && t < T;
+  }
+};
+
+// ------------------------------------------------------------------------------------
+// key tile
+// ------------------------------------------------------------------------------------
+
+struct KeyFlatSink {
+  uint8_t* idx;
+  uint8_t* sign;
+  void* norm;
+  float* rnorm;
+  float* y_dbg;
+  float* p_dbg;
+};
+
+struct KeyPagedSink {
+  uint8_t* pool;
+  const int32_t* block_table;
+  int max_pages;
+  tq_page_layout L;
+};
+
+template <int DT, class Source, class Sink>
+__global__ void __launch_bounds__(1024)
+key_tile_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, int mse_only) {
+  using E = Elem<DT>;
+  const int d = ly.d, j = threadIdx.x, tile = blockIdx.x;
+  const int lane = j & 63, wave = j >> 6, n_wave = d >> 6;
+  const int mb = ly.mse_bits, n_thr = (1 << mb) - 1;
+
+  extern __shared__ __align__(16) unsigned char smem[];
+  float* sx = (float*)smem;                 // [TILE][d] input as fp32
+  float* su = sx + TILE * d;                // [TILE][d] unit vector -> centroid values -> residual
+  uint8_t* sidx = (uint8_t*)(su + TILE * d);  // [TILE][d]
+  uint8_t* ssgn = sidx + TILE * d;          // [TILE][d]
+  float* snorm = (float*)(ssgn + TILE * d); // [TILE] norm as fp32 (value of the input dtype)
+  float* srn = snorm + TILE;                // [TILE]
+  float* scent = srn + TILE;                // [16] centroids
+  int* svalid = (int*)(scent + 16);         // [TILE]
+
+  if (j < (1 << mb)) scent[j] = ly.centroids[j];
+  // (1) stage the tile
+  for (int t = 0; t < TILE; ++t) {
+    int64_t off;
+    bool ok = src.locate(tile, t, off);
+    sx[t * d + j] = ok ? E::load(x, off + j) : 0.0f;
+    if (j == 0) svalid[t] = ok;
+  }
+  __syncthreads();
+  {  // nothing to do for a tile without tokens (tail tiles of the paged grid)
+    int any = 0;
+    for (int t = 0; t < TILE; ++t) any |= svalid[t];
+    if (!any) return;
+  }
+  // (2) norm in the input dtype (quantizer.py:136)
+  for (int t = wave; t < TILE; t += n_wave) {
+    float ss = 0.0f;
+    for (int i = lane; i < d; i += 64) { float a = sx[t * d + i]; ss += a * a; }
+    ss = wave_sum(ss);
+    if (lane == 0) snorm[t] = E::round(sqrtf(ss));
+  }
+  __syncthreads();
+  // (3) unit vector, still in the input dtype (quantizer.py:138)
+  for (int t = 0; t < TILE; ++t) {
+    float den = E::round(snorm[t] + 1e-10f);
+    su[t * d + j] = E::round(sx[t * d + j] / den);
+  }
+  __syncthreads();
+  // (4) y = u Pi^T (fp32), bucketise
+  float acc[TILE];
+#pragma unroll
+  for (int t = 0; t < TILE; ++t) acc[t] = 0.0f;
+  for (int i = 0; i < d; i += 4) {
+    float m0 = ly.PiT[(int64_t)(i + 0) * d + j], m1 = ly.PiT[(int64_t)(i + 1) * d + j];
+    float m2 = ly.PiT[(int64_t)(i + 2) * d + j], m3 = ly.PiT[(int64_t)(i + 3) * d + j];
+#pragma unroll
+    for (int t = 0; t < TILE; ++t) {
+      float4 u = *(const float4*)(su + t * d + i);
+      acc[t] = fmaf(u.x, m0, acc[t]); acc[t] = fmaf(u.y, m1, acc[t]);
+      acc[t] = fmaf(u.z, m2, acc[t]); acc[t] = fmaf(u.w, m3, acc[t]);
+    }
+  }
+  __syncthreads();   // everyone is done reading su
+#pragma unroll
+  for (int t = 0; t < TILE; ++t) {
+    float yv = acc[t];
+    unsigned idx = 0;
+    for (int k = 0; k < n_thr; ++k) idx += !(yv <= ly.thresholds[k]);
+    sidx[t * d + j] = (uint8_t)idx;
+    su[t * d + j] = scent[idx];
+    if constexpr (std::is_same<Sink, KeyFlatSink>::value) {
+      if (sink.y_dbg && svalid[t]) sink.y_dbg[((int64_t)tile * TILE + t) * d + j] = yv;
+    }
+  }
+  __syncthreads();
+  if (!mse_only) {
+    // (5) x_hat = (c Pi) * norm ; r = x - x_hat ; rho = ||r|| (quantizer.py:241-245)
+#pragma unroll
+    for (int t = 0; t < TILE; ++t) acc[t] = 0.0f;
+    for (int i = 0; i < d; i += 4) {
+      float m0 = ly.Pi[(int64_t)(i + 0) * d + j], m1 = ly.Pi[(int64_t)(i + 1) * d + j];
+      float m2 = ly.Pi[(int64_t)(i + 2) * d + j], m3 = ly.Pi[(int64_t)(i + 3) * d + j];
+#pragma unroll
+      for (int t = 0; t < TILE; ++t) {
+        float4 u = *(const float4*)(su + t * d + i);
+        acc[t] = fmaf(u.x, m0, acc[t]); acc[t] = fmaf(u.y, m1, acc[t]);
+        acc[t] = fmaf(u.z, m2, acc[t]); acc[t] = fmaf(u.w, m3, acc[t]);
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int t = 0; t < TILE; ++t) su[t * d + j] = sx[t * d + j] - acc[t] * snorm[t];
+    __syncthreads();
+    for (int t = wave; t < TILE; t += n_wave) {
+      float ss = 0.0f;
+      for (int i = lane; i < d; i += 64) { float a = su[t * d + i]; ss += a * a; }
+      ss = wave_sum(ss);
+      if (lane == 0) srn[t] = sqrtf(ss);
+    }
+    // (6) p = r S^T ; sign bits (quantizer.py:248-249)
+#pragma unroll
+    for (int t = 0; t < TILE; ++t) acc[t] = 0.0f;
+    for (int i = 0; i < d; i += 4) {
+      float m0 = ly.ST[(int64_t)(i + 0) * d + j], m1 = ly.ST[(int64_t)(i + 1) * d + j];
+      float m2 = ly.ST[(int64_t)(i + 2) * d + j], m3 = ly.ST[(int64_t)(i + 3) * d + j];
+#pragma unroll
+      for (int t = 0; t < TILE; ++t) {
+        float4 u = *(const float4*)(su + t * d + i);
+        acc[t] = fmaf(u.x, m0, acc[t]); acc[t] = fmaf(u.y, m1, acc[t]);
+        acc[t] = fmaf(u.z, m2, acc[t]); acc[t] = fmaf(u.w, m3, acc[t]);
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < TILE; ++t) {
+      ssgn[t * d + j] = acc[t] > 0.0f;
+      if constexpr (std::is_same<Sink, KeyFlatSink>::value) {
+        if (sink.p_dbg && svalid[t]) sink.p_dbg[((int64_t)tile * TILE + t) * d + j] = acc[t];
+      }
+    }
+  }
+  __syncthreads();
+
+  // (7) write
+  if constexpr (std::is_same<Sink, KeyFlatSink>::value) {
+    const int eff = eff_bits(mb), per = 8 / eff, row = idx_row_bytes(d, mb), srow = d >> 3;
+    for (int o = j; o < TILE * row; o += d) {
+      int t = o / row, k = o - t * row;
+      if (!svalid[t]) continue;
+      unsigned byte = 0;
+      for (int s = 0; s < per; ++s) {
+        int c = k * per + s;
+        if (c < d) byte |= (unsigned)sidx[t * d + c] << (eff * s);
+      }
+      sink.idx[((int64_t)tile * TILE + t) * row + k] = (uint8_t)byte;
+    }
+    if (!mse_only) {
+      for (int o = j; o < TILE * srow; o += d) {
+        int t = o / srow, k = o - t * srow;
+        if (!svalid[t]) continue;
+        unsigned byte = 0;
+        for (int s = 0; s < 8; ++s) byte |= (unsigned)ssgn[t * d + k * 8 + s] << s;
+        sink.sign[((int64_t)tile * TILE + t) * srow + k] = (uint8_t)byte;
+      }
+    }
+    if (j < TILE && svalid[j]) {
+      int64_t v = (int64_t)tile * TILE + j;
+      E::store(sink.norm, v, snorm[j]);
+      if (!mse_only) sink.rnorm[v] = srn[j];
+    }
+  } else {
+    int b, lpage, h;
+    src.decode(tile, b, lpage, h);
+    const tq_page_layout& L = sink.L;
+    int64_t page = sink.block_table[(int64_t)b * sink.max_pages + lpage];
+    uint8_t* pg = sink.pool + (page * src.H + h) * (int64_t)L.page_bytes;
+    const int words = d >> 5, planes = mb + 1;
+    for (int o = j; o < planes * words * TILE; o += d) {
+      int n = o % TILE, r = o / TILE;
+      int w = r % words, p = r / words;
+      if (!svalid[n]) continue;
+      uint32_t bits = 0;
+      if (p < mb) {
+        int sh = mb - 1 - p;
+        for (int i = 0; i < 32; ++i) bits |= (uint32_t)((sidx[n * d + w * 32 + i] >> sh) & 1) << i;
+      } else {
+        for (int i = 0; i < 32; ++i) bits |= (uint32_t)ssgn[n * d + w * 32 + i] << i;
+      }
+      *(uint32_t*)(pg + plane_word_off(L, p, w, n)) = bits;
+    }
+    if (j < TILE && svalid[j]) {
+      E::store(pg + L.off_norm, j, snorm[j]);
+      ((float*)(pg + L.off_rnorm))[j] = srn[j];
+    }
+  }
+}
+
+static size_t key_tile_smem(int d) { return (size_t)TILE * d * (4 + 4 + 1 + 1) + (TILE * 2 + 16) * 4 + TILE * 4; }
+
+// ------------------------------------------------------------------------------------
+// value tile (kv_cache.py:45-98)
+// ------------------------------------------------------------------------------------
+
+struct ValFlatSink {
+  uint8_t* data;
+  void* scale;
+  void* zero;
+};
+struct ValPagedSink {
+  uint8_t* pool;
+  const int32_t* block_table;
+  int max_pages;
+  tq_page_layout L;
+};
+
+template <int DT, class Source, class Sink>
+__global__ void __launch_bounds__(1024)
+value_tile_kernel(const void* __restrict__ v, Source src, int d, int gs, int bits, Sink sink) {
+  using E = Elem<DT>;
+  const int j = threadIdx.x, tile = blockIdx.x, ng = d / gs;
+  extern __shared__ __align__(16) unsigned char smem[];
+  float* sv = (float*)smem;                   // [TILE][d]
+  float* sscale = sv + TILE * d;              // [TILE][ng]
+  float* szero = sscale + TILE * ng;          // [TILE][ng]
+  uint8_t* scode = (uint8_t*)(szero + TILE * ng);  // [TILE][d]
+  int* svalid = (int*)(scode + TILE * d);     // [TILE]
+
+  for (int t = 0; t < TILE; ++t) {
+    int64_t off;
+    bool ok = src.locate(tile, t, off);
+    sv[t * d + j] = ok ? E::load(v, off + j) : 0.0f;
+    if (j == 0) svalid[t] = ok;
+  }
+  __syncthreads();
+  {
+    int any = 0;
+    for (int t = 0; t < TILE; ++t) any |= svalid[t];
+    if (!any) return;
+  }
+  const float levels = (float)((1 << bits) - 1);
+  for (int o = j; o < TILE * ng; o += d) {
+    int t = o / ng, g = o - t * ng;
+    const float* row = sv + t * d + g * gs;
+    float lo = row[0], hi = row[0];
+    bool has_nan = false;
+    for (int i = 0; i < gs; ++i) {
+      float a = row[(i + j) % gs];           // rotate the start to spread LDS banks
+      has_nan |= (a != a);
+      lo = fminf(lo, a);
+      hi = fmaxf(hi, a);
+    }
+    if (has_nan) lo = hi = __uint_as_float(0x7fc00000u);   // torch min/max propagate NaN
+    float sc = E::round(E::round(hi - lo) / levels);
+    float floor_v = E::round(1e-10f);
+    sc = (sc != sc) ? sc : fmaxf(sc, floor_v);
+    sscale[o] = sc;
+    szero[o] = lo;
+  }
+  __syncthreads();
+  for (int t = 0; t < TILE; ++t) {
+    int g = j / gs;
+    float sc = sscale[t * ng + g], z = szero[t * ng + g];
+    float q = E::round(E::round(sv[t * d + j] - z) / sc);
+    q = rintf(q);
+    q = fminf(fmaxf(q, 0.0f), levels);
+    scode[t * d + j] = (q != q) ? (uint8_t)0 : (uint8_t)q;
+  }
+  __syncthreads();
+
+  if constexpr (std::is_same<Sink, ValFlatSink>::value) {
+    const int per = 8 / bits, row = d / per;
+    for (int o = j; o < TILE * row; o += d) {
+      int t = o / row, k = o - t * row;
+      if (!svalid[t]) continue;
+      unsigned byte = 0;
+      for (int s = 0; s < per; ++s) byte |= (unsigned)scode[t * d + k * per + s] << (bits * s);
+      sink.data[((int64_t)tile * TILE + t) * row + k] = (uint8_t)byte;
+    }
+    for (int o = j; o < TILE * ng; o += d) {
+      int t = o / ng, g = o - t * ng;
+      if (!svalid[t]) continue;
+      int64_t at = ((int64_t)tile * TILE + t) * ng + g;
+      E::store(sink.scale, at, sscale[o]);
+      E::store(sink.zero, at, szero[o]);
+    }
+  } else {
+    int b, lpage, h;
+    src.decode(tile, b, lpage, h);
+    const tq_page_layout& L = sink.L;
+    int64_t page = sink.block_table[(int64_t)b * sink.max_pages + lpage];
+    uint8_t* pg = sink.pool + (page * src.H + h) * (int64_t)L.page_bytes;
+    // channel j: a field of 16*bits bits, token n at bit bits*n; read-modify-write keeps
+    // the codes of slots this call does not touch
+    const int wpc = bits / 2;                         // 32-bit words per channel
+    uint32_t* field = (uint32_t*)(pg + L.off_vdata) + j * wpc;
+    const int per_word = 32 / bits;
+    for (int w = 0; w < wpc; ++w) {
+      uint32_t neu = 0, mask = 0;
+      for (int s = 0; s < per_word; ++s) {
+        int n = w * per_word + s;
+        if (svalid[n]) {
+          neu |= (uint32_t)scode[n * d + j] << (bits * s);
+          mask |= ((1u << bits) - 1u) << (bits * s);
+        }
+      }
+      uint32_t old = (mask == 0xffffffffu) ? 0u : field[w];
+      field[w] = (old & ~mask) | neu;
+    }
+    for (int o = j; o < TILE * ng; o += d) {
+      int n = o % TILE, g = o / TILE;
+      if (!svalid[n]) continue;
+      E::store(pg + L.off_vscale, g * TILE + n, sscale[n * ng + g]);
+      E::store(pg + L.off_vzero, g * TILE + n, szero[n * ng + g]);
+    }
+  }
+}
+
+static size_t value_tile_smem(int d, int gs) { return (size_t)TILE * d * 5 + (size_t)TILE * (d / gs) * 8 + TILE * 4; }
+
+// ------------------------------------------------------------------------------------
+// page -> flat export (store.py:92-114)
+// ------------------------------------------------------------------------------------
+
+__device__ __forceinline__ void copy_elem(void* dst, int64_t di, const void* src, int64_t si, int dt) {
+  if (dt == TQ_F32) ((uint32_t*)dst)[di] = ((const uint32_t*)src)[si];
+  else ((uint16_t*)dst)[di] = ((const uint16_t*)src)[si];
+}
+
+__global__ void pool_export_kernel(const uint8_t* __restrict__ pool, int H, const int32_t* __restrict__ block_table,
+                                   int n_tok, tq_page_layout L, uint8_t* idx, uint8_t* signs, void* norms,
+                                   float* rnorms, uint8_t* v_data, void* v_scales, void* v_zeros) {
+  const int d = L.d, mb = L.mse_bits, vb = L.value_bits, ng = d / L.group_size;
+  const int lpage = blockIdx.x, h = blockIdx.y, j = threadIdx.x;
+  const uint8_t* pg = pool + ((int64_t)block_table[lpage] * H + h) * (int64_t)L.page_bytes;
+  const int eff = eff_bits(mb), per = 8 / eff, row = idx_row_bytes(d, mb), srow = d >> 3;
+  const int vrow = d * vb / 8, vper = 8 / vb;
+  for (int n = 0; n < TILE; ++n) {
+    int tok = lpage * TILE + n;
+    if (tok >= n_tok) break;
+    int64_t flat = (int64_t)h * n_tok + tok;
+    for (int k = j; k < row; k += blockDim.x) {
+      unsigned byte = 0;
+      for (int s = 0; s < per; ++s) {
+        int c = k * per + s;
+        if (c >= d) break;
+        unsigned id = 0;
+        for (int p = 0; p < mb; ++p) {
+          uint32_t w = *(const uint32_t*)(pg + plane_word_off(L, p, c >> 5, n));
+          id = (id << 1) | ((w >> (c & 31)) & 1u);
+        }
+        byte |= id << (eff * s);
+      }
+      idx[flat * row + k] = (uint8_t)byte;
+    }
+    for (int k = j; k < srow; k += blockDim.x) {
+      uint32_t w = *(const uint32_t*)(pg + plane_word_off(L, mb, k >> 2, n));
+      signs[flat * srow + k] = (uint8_t)(w >> ((k & 3) * 8));
+    }
+    for (int k = j; k < vrow; k += blockDim.x) {
+      unsigned byte = 0;
+      for (int s = 0; s < vper; ++s) {
+        int c = k * vper + s;
+        const uint32_t* field = (const uint32_t*)(pg + L.off_vdata) + c * (vb / 2);
+        int bit = vb * n;
+        byte |= ((field[bit >> 5] >> (bit & 31)) & ((1u << vb) - 1u)) << (vb * s);
+      }
+      v_data[flat * vrow + k] = (uint8_t)byte;
+    }
+    for (int g = j; g < ng; g += blockDim.x) {
+      copy_elem(v_scales, flat * ng + g, pg + L.off_vscale, g * TILE + n, L.dtype);
+      copy_elem(v_zeros, flat * ng + g, pg + L.off_vzero, g * TILE + n, L.dtype);
+    }
+    if (j == 0) {
+      copy_elem(norms, flat, pg + L.off_norm, n, L.dtype);
+      rnorms[flat] = ((const float*)(pg + L.off_rnorm))[n];
+    }
+  }
+}
+
+}  // namespace tq
+
+// ======================================================================================
+// C ABI
+// ======================================================================================
+
+using namespace tq;
+
+static int check_layer(const tq_layer* ly, bool need_sketch) {
+  if (!ly) return TQ_ENULL;
+  if (ly->d < 64 || ly->d > 768 || (ly->d & 63)) return TQ_EUNSUPPORTED;
+  if (ly->mse_bits < 1 || ly->mse_bits > 4) return TQ_EUNSUPPORTED;
+  if (!ly->Pi || !ly->PiT || !ly->centroids || !ly->thresholds) return TQ_ENULL;
+  if (need_sketch && (!ly->S || !ly->ST)) return TQ_ENULL;
+  return TQ_OK;
+}
+
+extern "C" int tq_version(void) { return TQ_ABI_VERSION; }
+
+extern "C" int tq_layer_fill_terms(tq_layer* layer, const float* c) {
+  if (!layer || !c) return TQ_ENULL;
+  const int mb = layer->mse_bits;
+  if (mb < 1 || mb > 4) return TQ_EUNSUPPORTED;
+  const int n = 1 << mb;
+  double w[16], wmax = 0.0;
+  for (int s = 0; s < n; ++s) {           // Walsh coefficient of bit-subset s
+    double a = 0.0;
+    for (int b = 0; b < n; ++b) a += (__builtin_popcount(b & s) & 1) ? -(double)c[b] : (double)c[b];
+    w[s] = a / n;
+    if (s && (w[s] < 0 ? -w[s] : w[s]) > wmax) wmax = w[s] < 0 ? -w[s] : w[s];
+  }
+  // c[idx] = sum_s w_s (-1)^{parity(idx&s)} = c[0] - 2 sum_{s>0} w_s parity(idx&s)
+  layer->n_terms = 0;
+  layer->term_const = c[0];
+  for (int s = 1; s < n; ++s) {
+    double a = w[s] < 0 ? -w[s] : w[s];
+    if (a <= 1e-9 * wmax) continue;
+    layer->term_mask[layer->n_terms] = s;
+    layer->term_coef[layer->n_terms] = (float)(-2.0 * w[s]);
+    layer->n_terms++;
+  }
+  return TQ_OK;
+}
+
+extern "C" int tq_page_layout_init(tq_page_layout* L, int d, int mse_bits, int value_bits, int group_size, int dtype) {
+  if (!L) return TQ_ENULL;
+  if (d < 64 || d > 768 || (d & 63)) return TQ_EUNSUPPORTED;
+  if (mse_bits < 1 || mse_bits > 4) return TQ_EUNSUPPORTED;
+  if (value_bits != 2 && value_bits != 4) return TQ_EUNSUPPORTED;
+  if (group_size < 16 || d % group_size) return TQ_EINVAL;
+  if (dtype < TQ_F32 || dtype > TQ_BF16) return TQ_EINVAL;
+  const int es = dtype == TQ_F32 ? 4 : 2;
+  L->d = d; L->mse_bits = mse_bits; L->value_bits = value_bits; L->group_size = group_size; L->dtype = dtype;
+  int off = 0;
+  L->off_planes = off; off += (mse_bits + 1) * (d / 8) * TQ_PAGE_TOKENS;
+  L->off_norm = off;   off += es * TQ_PAGE_TOKENS;
+  L->off_rnorm = off;  off += 4 * TQ_PAGE_TOKENS;
+  L->off_vdata = off;  off += d * value_bits * 2;
+  L->off_vscale = off; off += (d / group_size) * TQ_PAGE_TOKENS * es;
+  L->off_vzero = off;  off += (d / group_size) * TQ_PAGE_TOKENS * es;
+  L->page_bytes = (off + 127) & ~127;
+  return TQ_OK;
+}
+
+extern "C" int tq_bucketize_pack(const float* y, int64_t n_vec, int d, const float* thresholds, int mse_bits,
+                                 uint8_t* idx_out, void* stream) {
+  if (!y || !thresholds || !idx_out) return TQ_ENULL;
+  if (n_vec < 0 || d <= 0 || mse_bits < 1 || mse_bits > 8) return TQ_EINVAL;
+  if (n_vec == 0) return TQ_OK;
+  int64_t total = n_vec * idx_row_bytes(d, mse_bits);
+  bucketize_pack_kernel<<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream>>>(
+      y, n_vec, d, thresholds, mse_bits, idx_out);
+  TQ_CHECK_LAUNCH();
+  return TQ_OK;
+}
+
+extern "C" int tq_sign_pack(const float* p, int64_t n_vec, int d, uint8_t* sign_out, void* stream) {
+  if (!p || !sign_out) return TQ_ENULL;
+  if (n_vec < 0 || d <= 0) return TQ_EINVAL;
+  if (n_vec == 0) return TQ_OK;
+  int64_t total = n_vec * ((d + 7) / 8);
+  sign_pack_kernel<<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream>>>(p, n_vec, d, sign_out);
+  TQ_CHECK_LAUNCH();
+  return TQ_OK;
+}
+
+template <class Source, class Sink>
+static int launch_key(const void* x, int dtype, const Source& src, const tq_layer& ly, const Sink& sink, int mse_only,
+                      int64_t tiles, hipStream_t st) {
+  size_t smem = key_tile_smem(ly.d);
+  dim3 grid((unsigned)tiles), block(ly.d);
+#define TQ_LAUNCH_KEY(DT)                                                                              \
+  {                                                                                                    \
+    auto kern = key_tile_kernel<DT, Source, Sink>;                                                     \
+    if (smem > 48 * 1024) {                                                                            \
+      hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem); \
+      if (e != hipSuccess) return (int)e;                                                              \
+    }                                                                                                  \
+    kern<<<grid, block, smem, st>>>(x, src, ly, sink, mse_only);                                       \
+  }
+  switch (dtype) {
+    case TQ_F32: TQ_LAUNCH_KEY(TQ_F32) break;
+    case TQ_F16: TQ_LAUNCH_KEY(TQ_F16) break;
+    case TQ_BF16: TQ_LAUNCH_KEY(TQ_BF16) break;
+    default: return TQ_EINVAL;
+  }
+#undef TQ_LAUNCH_KEY
+  TQ_CHECK_LAUNCH();
+  return TQ_OK;
+}
+
+template <class Source, class Sink>
+static int launch_value(const void* v, int dtype, const Source& src, int d, int gs, int bits, const Sink& sink,
+                        int64_t tiles, hipStream_t st) {
+  size_t smem = value_tile_smem(d, gs);
+  dim3 grid((unsigned)tiles), block(d);
+#define TQ_LAUNCH_VAL(DT)                                                                              \
+  {                                                                                                    \
+    auto kern = value_tile_kernel<DT, Source, Sink>;                                                   \
+    if (smem > 48 * 1024) {                                                                            \
+      hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem); \
+      if (e != hipSuccess) return (int)e;                                                              \
+    }                                                                                                  \
+    kern<<<grid, block, smem, st>>>(v, src, d, gs, bits, sink);                                        \
+  }
+  switch (dtype) {
+    case TQ_F32: TQ_LAUNCH_VAL(TQ_F32) break;
+    case TQ_F16: TQ_LAUNCH_VAL(TQ_F16) break;
+    case TQ_BF16: TQ_LAUNCH_VAL(TQ_BF16) break;
+    default: return TQ_EINVAL;
+  }
+#undef TQ_LAUNCH_VAL
+  TQ_CHECK_LAUNCH();
+  return TQ_OK;
+}
+
+extern "C" int tq_quantize_keys(const void* x, int dtype, int64_t n_vec, int64_t row_stride, const tq_layer* layer,
+                                uint8_t* idx_out, uint8_t* sign_out, void* norm_out, float* rnorm_out, float* y_dbg,
+                                float* p_dbg, int mse_only, void* stream) {
+  int rc = check_layer(layer, !mse_only);
+  if (rc) return rc;
+  if (!x || !idx_out || !norm_out) return TQ_ENULL;
+  if (!mse_only && (!sign_out || !rnorm_out)) return TQ_ENULL;
+  if (n_vec < 0 || row_stride < layer->d) return TQ_EINVAL;
+  if (n_vec == 0) return TQ_OK;
+  FlatSource src{n_vec, row_stride};
+  KeyFlatSink sink{idx_out, sign_out, norm_out, rnorm_out, y_dbg, p_dbg};
+  return launch_key(x, dtype, src, *layer, sink, mse_only, (n_vec + TILE - 1) / TILE, (hipStream_t)stream);
+}
+
+extern "C" int tq_quantize_values(const void* v, int dtype, int64_t n_vec, int64_t row_stride, int d, int group_size,
+                                  int bits, uint8_t* data_out, void* scale_out, void* zero_out, void* stream) {
+  if (!v || !data_out || !scale_out || !zero_out) return TQ_ENULL;
+  if (d < 64 || d > 768 || (d & 63)) return TQ_EUNSUPPORTED;
+  if (bits != 2 && bits != 4 && bits != 8) return TQ_EUNSUPPORTED;
+  if (group_size < 16 || d % group_size || n_vec < 0 || row_stride < d) return TQ_EINVAL;
+  if (n_vec == 0) return TQ_OK;
+  FlatSource src{n_vec, row_stride};
+  ValFlatSink sink{data_out, scale_out, zero_out};
+  return launch_value(v, dtype, src, d, group_size, bits, sink, (n_vec + TILE - 1) / TILE, (hipStream_t)stream);
+}
+
+extern "C" int tq_append_kv_paged(const void* k, const void* v, int dtype, int B, int T, int H, int64_t stride_b,
+                                  int64_t stride_t, int64_t stride_h, const int32_t* start_pos,
+                                  const int32_t* block_table, int max_pages, const tq_layer* layer,
+                                  const tq_page_layout* layout, uint8_t* pool, int64_t num_pages, void* stream) {
+  int rc = check_layer(layer, true);
+  if (rc) return rc;
+  if (!k || !v || !block_table || !layout || !pool) return TQ_ENULL;
+  if (dtype != layout->dtype || layout->d != layer->d || layout->mse_bits != layer->mse_bits) return TQ_EINVAL;
+  if (B < 0 || T < 0 || H <= 0 || max_pages <= 0 || num_pages <= 0) return TQ_EINVAL;
+  if (B == 0 || T == 0) return TQ_OK;
+  // a run of T tokens starting anywhere inside a page touches at most this many pages
+  // (the run may begin at any of the 16 slots of its first page when start_pos is given)
+  const int tiles_per_seq = start_pos ? (T + TILE - 2) / TILE + 1 : (T + TILE - 1) / TILE;
+  PagedSource src{B, T, H, tiles_per_seq, stride_b, stride_t, stride_h, start_pos};
+  int64_t tiles = (int64_t)B * tiles_per_seq * H;
+  KeyPagedSink ks{pool, block_table, max_pages, *layout};
+  rc = launch_key(k, dtype, src, *layer, ks, 0, tiles, (hipStream_t)stream);
+  if (rc) return rc;
+  ValPagedSink vs{pool, block_table, max_pages, *layout};
+  return launch_value(v, dtype, src, layer->d, layout->group_size, layout->value_bits, vs, tiles, (hipStream_t)stream);
+}
+
+extern "C" int tq_pool_export(const uint8_t* pool, int64_t num_pages, int H, const int32_t* block_table, int n_tok,
+                              const tq_page_layout* layout, uint8_t* idx, uint8_t* signs, void* norms, float* rnorms,
+                              uint8_t* v_data, void* v_scales, void* v_zeros, void* stream) {
+  if (!pool || !block_table || !layout || !idx || !signs || !norms || !rnorms || !v_data || !v_scales || !v_zeros)
+    return TQ_ENULL;
+  if (H <= 0 || n_tok < 0 || num_pages <= 0) return TQ_EINVAL;
+  if (n_tok == 0) return TQ_OK;
+  dim3 grid((n_tok + TILE - 1) / TILE, H), block(64);
+  pool_export_kernel<<<grid, block, 0, (hipStream_t)stream>>>(pool, H, block_table, n_tok, *layout, idx, signs, norms,
+                                                             rnorms, v_data, v_scales, v_zeros);
+  TQ_CHECK_LAUNCH();
+  return TQ_OK;
+}

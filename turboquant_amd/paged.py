@@ -1,0 +1,165 @@
+"""Paged compressed KV pool for batches of sequences (new design).
+
+The reference keeps one python list of chunk tensors per layer and therefore
+one sequence (store.py:59-63; integration/vllm.py:139-145).  This module is the
+batch-aware store underneath: a pool of 16-token pages per layer, block tables
+and sequence lengths, written by the fused quantise kernel and read by the fused
+decode-attention kernel.  `CompressedKVStore` (store.py mirror) is a
+single-sequence view over it.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+import math
+from typing import Optional
+
+import torch
+
+from . import _ffi
+from .quantizer import TurboQuantProd
+
+PAGE_TOKENS = _ffi.TQ_PAGE_TOKENS
+
+
+class PagedKVPool:
+    """(num_pages, num_kv_heads, page_bytes) uint8 pool + its geometry."""
+
+    def __init__(self, quantizer: TurboQuantProd, num_kv_heads: int, num_pages: int, value_bits: int = 2,
+                 value_group_size: int = 32, dtype: torch.dtype = torch.bfloat16, device=None):
+        self.quantizer = quantizer
+        self.head_dim = quantizer.dim
+        self.num_kv_heads = num_kv_heads
+        self.value_bits = value_bits
+        self.value_group_size = min(value_group_size, self.head_dim)
+        self.dtype = dtype
+        self.device = torch.device(device) if device is not None else quantizer.S.device
+        if self.device.type != "cuda":
+            raise RuntimeError("PagedKVPool needs a GPU device: the TurboQuant kernels have no CPU path")
+        self.layout = _ffi.make_page_layout(self.head_dim, quantizer.bits - 1, value_bits, self.value_group_size, dtype)
+        self.num_pages = int(num_pages)
+        self.data = torch.zeros(self.num_pages, num_kv_heads, self.layout.page_bytes, dtype=torch.uint8,
+                                device=self.device)
+
+    @property
+    def page_bytes(self) -> int:
+        return self.layout.page_bytes
+
+    def grow(self, num_pages: int):
+        """Enlarge the pool, keeping existing pages."""
+        if num_pages <= self.num_pages:
+            return
+        bigger = torch.zeros(num_pages, self.num_kv_heads, self.layout.page_bytes, dtype=torch.uint8, device=self.device)
+        bigger[: self.num_pages] = self.data
+        self.data, self.num_pages = bigger, int(num_pages)
+
+    # ---- write ------------------------------------------------------------------
+    def append(self, key: torch.Tensor, value: torch.Tensor, block_table: torch.Tensor,
+               start_pos: Optional[torch.Tensor] = None):
+        """Quantise key/value (B, T, H, d) and store token t of sequence b at
+        logical position start_pos[b] + t through block_table (B, max_pages) int32."""
+        _ffi.require_gpu(key, "key")
+        if key.dim() != 4 or key.shape != value.shape:
+            raise ValueError("key and value must both be (B, T, H, d)")
+        B, T, H, d = key.shape
+        if H != self.num_kv_heads or d != self.head_dim:
+            raise ValueError(f"expected (B, T, {self.num_kv_heads}, {self.head_dim}), got {tuple(key.shape)}")
+        if key.dtype != self.dtype or value.dtype != self.dtype:
+            raise TypeError(f"pool was laid out for {self.dtype}")
+        if key.stride(-1) != 1 or value.stride(-1) != 1 or key.stride() != value.stride():
+            key, value = key.contiguous(), value.contiguous()
+        if block_table.dtype != torch.int32 or block_table.dim() != 2 or block_table.shape[0] != B:
+            raise ValueError("block_table must be int32 (B, max_pages)")
+        block_table = block_table.contiguous()
+        if start_pos is not None:
+            start_pos = start_pos.to(device=self.device, dtype=torch.int32).contiguous()
+        ly = self.quantizer._layer()
+        with torch.cuda.device(self.device):
+            _ffi.check(_ffi.lib().tq_append_kv_paged(
+                key.data_ptr(), value.data_ptr(), _ffi.dtype_tag(self.dtype), B, T, H, key.stride(0), key.stride(1),
+                key.stride(2), _ffi.ptr(start_pos), block_table.data_ptr(), block_table.shape[1], C.byref(ly),
+                C.byref(self.layout), self.data.data_ptr(), self.num_pages, _ffi.stream_ptr(self.device)),
+                "tq_append_kv_paged")
+
+    # ---- read -------------------------------------------------------------------
+    def export_flat(self, block_table_row: torch.Tensor, n_tok: int):
+        """Gather one sequence's pages into the reference's flat tensors
+        (H, n_tok, ...): idx, signs, norms, rnorms, v_data, v_scales, v_zeros."""
+        H, d, dev = self.num_kv_heads, self.head_dim, self.device
+        mb = self.quantizer.bits - 1
+        eff = 1 if mb == 1 else (2 if mb == 2 else 4)
+        ng = d // self.value_group_size
+        idx = torch.empty(H, n_tok, d * eff // 8, dtype=torch.uint8, device=dev)
+        signs = torch.empty(H, n_tok, d // 8, dtype=torch.uint8, device=dev)
+        norms = torch.empty(H, n_tok, dtype=self.dtype, device=dev)
+        rnorms = torch.empty(H, n_tok, dtype=torch.float32, device=dev)
+        v_data = torch.empty(H, n_tok, d * self.value_bits // 8, dtype=torch.uint8, device=dev)
+        v_scales = torch.empty(H, n_tok, ng, dtype=self.dtype, device=dev)
+        v_zeros = torch.empty(H, n_tok, ng, dtype=self.dtype, device=dev)
+        bt = block_table_row.to(device=dev, dtype=torch.int32).contiguous()
+        with torch.cuda.device(dev):
+            _ffi.check(_ffi.lib().tq_pool_export(
+                self.data.data_ptr(), self.num_pages, H, bt.data_ptr(), n_tok, C.byref(self.layout), idx.data_ptr(),
+                signs.data_ptr(), norms.data_ptr(), rnorms.data_ptr(), v_data.data_ptr(), v_scales.data_ptr(),
+                v_zeros.data_ptr(), _ffi.stream_ptr(dev)), "tq_pool_export")
+        return idx, signs, norms, rnorms, v_data, v_scales, v_zeros
+
+    def default_splits(self, B: int, max_len: int) -> int:
+        """Enough (sequence, head, split) workgroups to fill 256 CUs a few times over."""
+        pages = max(1, (max_len + PAGE_TOKENS - 1) // PAGE_TOKENS)
+        want = max(1, math.ceil(2048 / max(1, B * self.num_kv_heads)))
+        return int(max(1, min(want, pages, 512)))
+
+    def workspace(self, B: int, Hq: int, n_split: int) -> torch.Tensor:
+        nbytes = _ffi.lib().tq_decode_workspace_bytes(B, Hq, self.head_dim, n_split)
+        return torch.empty(nbytes // 4, dtype=torch.float32, device=self.device)
+
+    def decode_attention(self, query: torch.Tensor, block_table: torch.Tensor, seq_lens: torch.Tensor,
+                         scale: Optional[float] = None, recent_k: Optional[torch.Tensor] = None,
+                         recent_v: Optional[torch.Tensor] = None, recent_len: Optional[torch.Tensor] = None,
+                         n_split: Optional[int] = None, workspace: Optional[torch.Tensor] = None,
+                         out: Optional[torch.Tensor] = None, max_len: Optional[int] = None) -> torch.Tensor:
+        """softmax(scale * [scores_hist ; q k_recent^T]) [v_hist ; v_recent] for one
+        query token per sequence.  query (B, Hq, d);
+        block_table (B, max_pages) or (max_pages,) shared; seq_lens (B,) int32;
+        recent_k / recent_v (B, R, H, d) exact tokens, recent_len (B,) valid rows."""
+        _ffi.require_gpu(query, "query")
+        B, Hq, d = query.shape
+        if d != self.head_dim or Hq % self.num_kv_heads:
+            raise ValueError(f"Incompatible GQA shapes: Q={Hq}, H_kv={self.num_kv_heads}, d={d}")
+        query = query.contiguous()
+        if scale is None:
+            scale = 1.0 / math.sqrt(d)
+        bt = block_table.contiguous()
+        bt_stride = 0 if bt.dim() == 1 else bt.shape[1]
+        seq_lens = seq_lens.to(device=self.device, dtype=torch.int32).contiguous()
+        if n_split is None:
+            if max_len is None:
+                max_len = (bt.shape[-1]) * PAGE_TOKENS
+            n_split = self.default_splits(B, max_len)
+        if workspace is None:
+            workspace = self.workspace(B, Hq, n_split)
+        if out is None:
+            out = torch.empty_like(query)
+        rk_ptr = rv_ptr = rl_ptr = None
+        rows = 0
+        rs = (0, 0, 0)
+        if recent_k is not None and recent_k.shape[1] > 0:
+            if recent_k.dtype != query.dtype or recent_v.dtype != query.dtype:
+                raise TypeError("recent_k / recent_v must have the query's dtype")
+            if recent_k.stride(-1) != 1 or recent_k.stride() != recent_v.stride():
+                recent_k, recent_v = recent_k.contiguous(), recent_v.contiguous()
+            rows = recent_k.shape[1]
+            rs = (recent_k.stride(0), recent_k.stride(1), recent_k.stride(2))
+            rk_ptr, rv_ptr = recent_k.data_ptr(), recent_v.data_ptr()
+            if recent_len is not None:
+                recent_len = recent_len.to(device=self.device, dtype=torch.int32).contiguous()
+                rl_ptr = recent_len.data_ptr()
+        ly = self.quantizer._layer()
+        with torch.cuda.device(self.device):
+            _ffi.check(_ffi.lib().tq_decode_attn_paged(
+                query.data_ptr(), _ffi.dtype_tag(query.dtype), B, Hq, self.num_kv_heads, self.data.data_ptr(),
+                self.num_pages, bt.data_ptr(), bt_stride, seq_lens.data_ptr(), float(scale), C.byref(ly),
+                C.byref(self.layout), rk_ptr, rv_ptr, rows, rs[0], rs[1], rs[2], rl_ptr, out.data_ptr(),
+                workspace.data_ptr(), n_split, _ffi.stream_ptr(self.device)), "tq_decode_attn_paged")
+        return out
