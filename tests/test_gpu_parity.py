@@ -1,0 +1,507 @@
+"""GPU: the HIP kernels, called through the C ABI, against the pinned oracle and
+the reference's golden vectors.
+
+Gates (from the north star): packed bytes bit-exact when the kernel is fed the
+reference's rotated / projected fp32 tensors; scores within 1e-3 relative to the
+score scale, |delta| <= 1e-3 * rms(scores), on identical packed bytes;
+attention outputs cosine >= 0.9999 on an identical packed store.  End-to-end
+quantisation (own rotation on the GPU) differs from a CPU BLAS only by fp32
+summation order; its index / sign flip rates are bounded here at 1e-4.
+"""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import tq_oracle as O
+from tests.helpers import (bit_mismatch, byte_mismatch, cosine, install_matrices, key_code, params_of, value_code)
+
+pytestmark = pytest.mark.gpu
+
+SCORE_TOL = 1e-3          # x rms(scores)
+COS_GATE = 0.9999
+FLIP_RATE = 1e-4
+
+
+def _import():
+    import ctypes as C
+    from turboquant_amd import _ffi
+    return C, _ffi
+
+
+def _progress(msg):
+    print(f"[gpu-parity] {msg}", flush=True)
+
+
+# ------------------------------------------------------------------ packing entry points
+def test_bucketize_and_sign_pack_bit_exact_on_reference_tensors(gpu, golden):
+    C, ffi = _import()
+    lib = ffi.lib()
+    z = golden.npz("config1_full")
+    jobs = [("config1", torch.from_numpy(z["y_head"]), torch.from_numpy(z["p_head"]), torch.from_numpy(z["thresholds"]),
+             2, z["mse_indices"][:256], z["qjl_signs"][:256])]
+    kc = golden.npz("key_cases")
+    for case in golden.cases("key_cases"):
+        d, bits, _ = [int(v) for v in kc[case + ".meta"]]
+        y = torch.from_numpy(kc[case + ".y"]).reshape(-1, d)
+        p = torch.from_numpy(kc[case + ".p"]).reshape(-1, d)
+        jobs.append((case, y, p, torch.from_numpy(kc[case + ".thresholds"]), bits - 1,
+                     kc[case + ".mse_indices"].reshape(y.shape[0], -1), kc[case + ".qjl_signs"].reshape(y.shape[0], -1)))
+    for name, y, p, thr, mb, want_idx, want_sgn in jobs:
+        _progress(f"pack {name} mb={mb} shape={tuple(y.shape)}")
+        n, d = y.shape
+        yd, pd, td = y.to(gpu).contiguous(), p.to(gpu).contiguous(), thr.to(gpu).contiguous()
+        idx = torch.zeros(n, want_idx.shape[1], dtype=torch.uint8, device=gpu)
+        sgn = torch.zeros(n, want_sgn.shape[1], dtype=torch.uint8, device=gpu)
+        ffi.check(lib.tq_bucketize_pack(yd.data_ptr(), n, d, td.data_ptr(), mb, idx.data_ptr(), None), "bucketize")
+        ffi.check(lib.tq_sign_pack(pd.data_ptr(), n, d, sgn.data_ptr(), None), "sign_pack")
+        torch.cuda.synchronize()
+        assert np.array_equal(idx.cpu().numpy(), want_idx), name
+        assert np.array_equal(sgn.cpu().numpy(), want_sgn), name
+
+
+def test_pack_ragged_dim_and_special_values(gpu):
+    C, ffi = _import()
+    lib = ffi.lib()
+    g = torch.Generator().manual_seed(9)
+    for mb, d in [(1, 13), (2, 13), (3, 77), (4, 5), (2, 128)]:
+        thr = torch.sort(torch.randn(2 ** mb - 1, generator=g) * 0.1).values
+        y = torch.randn(9, d, generator=g) * 0.1
+        y[0, 0], y[0, 1], y[0, 2] = float("nan"), float("inf"), -float("inf")
+        m = min(d, thr.numel())
+        y[1, :m] = thr[:m]                            # exact ties go to the lower bucket
+        want = O.pack_indices(O.bucketize(y, thr), mb)
+        idx = torch.zeros_like(want, device=gpu)
+        yd, td = y.to(gpu), thr.to(gpu)              # named, so the buffers outlive the launch
+        ffi.check(lib.tq_bucketize_pack(yd.data_ptr(), 9, d, td.data_ptr(), mb, idx.data_ptr(), None), "b")
+        p = torch.randn(9, d, generator=g)
+        p[0, :4] = torch.tensor([0.0, -0.0, float("nan"), 1e-40])
+        wsg = O.pack_signs(p)
+        sgn = torch.zeros_like(wsg, device=gpu)
+        pd = p.to(gpu)
+        ffi.check(lib.tq_sign_pack(pd.data_ptr(), 9, d, sgn.data_ptr(), None), "s")
+        torch.cuda.synchronize()
+        assert torch.equal(idx.cpu(), want), (mb, d)
+        assert torch.equal(sgn.cpu(), wsg), (mb, d)
+    # empty input is a no-op
+    ffi.check(lib.tq_sign_pack(pd.data_ptr(), 0, 8, sgn.data_ptr(), None), "empty")
+
+
+# ------------------------------------------------------------------ key quantiser, flat layout
+def _quantizer_for(prm, key_bits, gpu):
+    from turboquant_amd.quantizer import TurboQuantProd
+    tq = TurboQuantProd(prm.Pi.shape[0], bits=key_bits, device=gpu)
+    return install_matrices(tq, prm)
+
+
+def test_key_quantiser_end_to_end_vs_reference_vectors(gpu, golden):
+    kc = golden.npz("key_cases")
+    for case in golden.cases("key_cases"):
+        d, bits, _ = [int(v) for v in kc[case + ".meta"]]
+        if bits - 1 > 4:
+            continue
+        _progress(f"quantize_keys {case}")
+        prm = golden.key_params("key_cases", case)
+        tq = _quantizer_for(prm, bits, gpu)
+        x = golden.tensor("key_cases", case + ".x")
+        code, y, p = tq.quantize_traced(x.to(gpu))
+        torch.cuda.synchronize()
+        n_coord = x.numel()
+        want_idx = torch.from_numpy(kc[case + ".mse_indices"])
+        want_sgn = torch.from_numpy(kc[case + ".qjl_signs"])
+        assert code.mse_indices.shape == want_idx.shape and code.mse_indices.dtype == torch.uint8
+        assert code.qjl_signs.shape == want_sgn.shape
+        assert code.norms.dtype == x.dtype and code.residual_norms.dtype == torch.float32
+        idx_flips = byte_mismatch(code.mse_indices, want_idx)
+        sgn_flips = bit_mismatch(code.qjl_signs, want_sgn)
+        _progress(f"   index bytes differing {idx_flips}, sign bits differing {sgn_flips} of {n_coord}")
+        assert idx_flips <= max(1, FLIP_RATE * n_coord), case
+        assert sgn_flips <= max(2, FLIP_RATE * n_coord), case
+        ref_norm = golden.tensor("key_cases", case + ".norms").float()
+        got_norm = code.norms.float().cpu()
+        ulp = 2.0 ** -7 if x.dtype == torch.bfloat16 else (2.0 ** -10 if x.dtype == torch.float16 else 2.0 ** -22)
+        assert torch.all((got_norm - ref_norm).abs() <= ulp * ref_norm.abs() + 1e-30), case
+        if x.dtype != torch.float32:           # 16-bit norms: rounding hides the fp32 summation order
+            assert (got_norm != ref_norm).float().mean() < 0.02, case
+        ref_rn = torch.from_numpy(kc[case + ".residual_norms"])
+        assert torch.allclose(code.residual_norms.cpu(), ref_rn, rtol=2e-5, atol=1e-6), case
+        yr = torch.from_numpy(kc[case + ".y"])
+        ok = ~torch.isnan(yr)
+        assert (y.cpu()[ok] - yr[ok]).abs().max() < 2e-6, case
+        assert torch.equal(torch.isnan(y.cpu()), torch.isnan(yr)), case
+        pr = torch.from_numpy(kc[case + ".p"])
+        assert (p.cpu() - pr).abs().max() <= 1e-4 * pr.abs().max(), case
+        # feeding the kernel's own y / p back through the pack entry points reproduces its bytes
+        assert torch.equal(O.pack_indices(O.bucketize(y.cpu(), prm.thresholds), bits - 1), code.mse_indices.cpu())
+        assert torch.equal(O.pack_signs(p.cpu()), code.qjl_signs.cpu())
+
+
+def test_mse_only_quantiser_and_dequant(gpu, golden):
+    case = "fp32_d128_b4"
+    kc = golden.npz("key_cases")
+    prm = golden.key_params("key_cases", case)
+    tq = _quantizer_for(prm, 4, gpu)
+    x = golden.tensor("key_cases", case + ".x").to(gpu)
+    mq = tq.mse_quantizer.quantize(x)
+    full = tq.quantize(x)
+    assert torch.equal(mq.indices, full.mse_indices) and torch.equal(mq.norms, full.norms) and mq.bits == 3
+    ref_code = key_code(torch.from_numpy(kc[case + ".mse_indices"]), torch.from_numpy(kc[case + ".qjl_signs"]),
+                        torch.from_numpy(kc[case + ".residual_norms"]), golden.tensor("key_cases", case + ".norms"), 3)
+    from turboquant_amd.quantizer import MSEQuantized, ProdQuantized
+    deq = tq.mse_quantizer.dequantize(MSEQuantized(ref_code.mse_indices.to(gpu), ref_code.norms.to(gpu), 3)).cpu()
+    want = O.mse_dequantize(ref_code.mse_indices, ref_code.norms, prm)
+    assert (deq - want).abs().max() <= 2e-6 * want.abs().max()
+    rt = tq.mse_quantizer(x).cpu()
+    assert rt.shape == x.shape
+    assert ((rt - x.cpu()).norm(dim=-1) / x.cpu().norm(dim=-1).clamp_min(1e-6))[1:].pow(2).mean() < 0.06   # mse_total(3b)=0.034
+
+
+def test_prod_dequant_and_score_on_reference_bytes(gpu, golden):
+    from turboquant_amd.quantizer import ProdQuantized
+    kc = golden.npz("key_cases")
+    for case in golden.cases("key_cases"):
+        d, bits, _ = [int(v) for v in kc[case + ".meta"]]
+        if bits - 1 > 4:
+            continue
+        _progress(f"dequant+score {case}")
+        prm = golden.key_params("key_cases", case)
+        tq = _quantizer_for(prm, bits, gpu)
+        code = ProdQuantized(torch.from_numpy(kc[case + ".mse_indices"]).to(gpu),
+                             torch.from_numpy(kc[case + ".qjl_signs"]).to(gpu),
+                             torch.from_numpy(kc[case + ".residual_norms"]).to(gpu),
+                             golden.tensor("key_cases", case + ".norms").to(gpu), bits - 1)
+        deq = tq.dequantize(code).cpu()
+        want = torch.from_numpy(kc[case + ".dequant"])
+        assert (deq - want).abs().max() <= 4e-6 * want.abs().max(), case
+        q = golden.tensor("key_cases", case + ".q").to(gpu)
+        sc = tq.attention_score(q, code).cpu()
+        ref = torch.from_numpy(kc[case + ".scores"])
+        assert sc.shape == ref.shape and sc.dtype == torch.float32
+        rms = ref.pow(2).mean().sqrt()
+        assert (sc - ref).abs().max() <= SCORE_TOL * rms, case
+        assert (sc - ref).abs().max() <= 2e-5 * rms, case      # fp32 kernels sit far inside the gate
+
+
+def test_config1_scores_on_reference_bytes_and_round_trip(gpu, golden):
+    from turboquant_amd.quantizer import ProdQuantized
+    z = golden.npz("config1_full")
+    prm = O.KeyParams(torch.from_numpy(z["Pi"]), torch.from_numpy(z["S"]), torch.from_numpy(z["centroids"]),
+                      torch.from_numpy(z["thresholds"]), 2)
+    tq = _quantizer_for(prm, 3, gpu)
+    code = ProdQuantized(torch.from_numpy(z["mse_indices"]).to(gpu), torch.from_numpy(z["qjl_signs"]).to(gpu),
+                         torch.from_numpy(z["residual_norms"]).to(gpu), torch.from_numpy(z["norms"]).to(gpu), 2)
+    Q = torch.from_numpy(z["Q"]).to(gpu)
+    sc = tq.attention_score(Q, code).cpu()
+    ref = torch.from_numpy(z["scores"])
+    rms = float(ref.pow(2).mean().sqrt())
+    err = float((sc - ref).abs().max())
+    _progress(f"config1 scores: max|delta| {err:.3e} = {err / rms:.2e} x rms")
+    assert sc.shape == (32, 4096)
+    assert err <= SCORE_TOL * rms
+    # full round trip on the regenerated config-1 keys: bytes differ from the reference's only by
+    # fp32 summation order
+    g = torch.Generator(device="cpu").manual_seed(0)
+    K = torch.randn(4096, 128, generator=g, dtype=torch.float32)
+    K = K / K.norm(dim=-1, keepdim=True)
+    K = K * (0.5 + 1.5 * torch.rand(4096, generator=g)).unsqueeze(-1)
+    got = tq.quantize(K.to(gpu))
+    idx_flips = byte_mismatch(got.mse_indices, torch.from_numpy(z["mse_indices"]))
+    sgn_flips = bit_mismatch(got.qjl_signs, torch.from_numpy(z["qjl_signs"]))
+    _progress(f"config1 end-to-end: {idx_flips} index bytes, {sgn_flips} sign bits differ of 524288 coordinates")
+    assert idx_flips <= 52 and sgn_flips <= 52
+    assert torch.allclose(got.norms.cpu(), torch.from_numpy(z["norms"]), rtol=1e-6)
+    assert torch.allclose(got.residual_norms.cpu(), torch.from_numpy(z["residual_norms"]), rtol=2e-5)
+    sc2 = tq.attention_score(Q, got).cpu()
+    # a flipped sign moves one score by a few percent of rms; everything else agrees to 1e-5
+    assert ((sc2 - ref).abs() > 1e-4 * rms).float().mean() < 1e-3
+
+
+def test_attention_score_batched_and_broadcast(gpu):
+    from turboquant_amd.quantizer import TurboQuantProd
+    tq = TurboQuantProd(128, bits=3, device=gpu)
+    prm = params_of(tq)
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(2, 3, 70, 128, generator=g).bfloat16()
+    q = torch.randn(2, 3, 5, 128, generator=g).bfloat16()
+    code = tq.quantize(x.to(gpu))
+    sc = tq.attention_score(q.to(gpu), code).cpu()
+    host = key_code(code.mse_indices.cpu(), code.qjl_signs.cpu(), code.residual_norms.cpu(), code.norms.cpu(), 2)
+    want = O.attention_score(q, host, prm)
+    rms = want.pow(2).mean().sqrt()
+    assert sc.shape == (2, 3, 5, 70)
+    assert (sc - want).abs().max() <= 2e-5 * rms
+    one_q = q[:1, :1]
+    sc_b = tq.attention_score(one_q.to(gpu), code).cpu()           # query broadcast over the key batch dims
+    assert torch.allclose(sc_b, O.attention_score(one_q, host, prm), atol=float(2e-5 * rms))
+
+
+# ------------------------------------------------------------------ values
+def test_value_quantiser_bit_exact_vs_reference_vectors(gpu, golden):
+    from turboquant_amd.kv_cache import dequantize_values, quantize_values, ValueQuantized
+    z = golden.npz("values")
+    for case in golden.cases("values"):
+        tag, b, g_ = case.split("_")
+        bits, gs = int(b[1:]), int(g_[1:])
+        v = golden.tensor("values", case + ".v")
+        vq = quantize_values(v.to(gpu), bits=bits, group_size=gs)
+        assert vq.bits == bits and vq.scales.dtype == v.dtype and vq.zeros.dtype == v.dtype
+        assert np.array_equal(vq.data.cpu().numpy(), z[case + ".data"]), case
+        assert torch.equal(vq.scales.cpu(), golden.tensor("values", case + ".scales")), case
+        assert torch.equal(vq.zeros.cpu(), golden.tensor("values", case + ".zeros")), case
+        deq = dequantize_values(vq, gs).cpu()
+        assert np.array_equal(deq.numpy(), z[case + ".dequant"], equal_nan=True), case
+
+
+def test_value_quantiser_strided_rows_and_nan(gpu):
+    from turboquant_amd.kv_cache import quantize_values
+    g = torch.Generator().manual_seed(2)
+    big = torch.randn(37, 256, generator=g).bfloat16()
+    view = big[:, :128]                                     # row stride 256, 128 used
+    vq = quantize_values(view.to(gpu)[:, :], bits=4, group_size=32)
+    want = O.quantize_values(view.contiguous(), 4, 32)
+    assert torch.equal(vq.data.cpu(), want.data) and torch.equal(vq.scales.cpu(), want.scales)
+    v = torch.randn(3, 64, generator=g)
+    v[1, 5] = float("nan")
+    vq = quantize_values(v.to(gpu), bits=2, group_size=32)
+    want = O.quantize_values(v, 2, 32)
+    assert torch.equal(torch.isnan(vq.scales.cpu()), torch.isnan(want.scales))
+    assert torch.equal(vq.data.cpu()[[0, 2]], want.data[[0, 2]])
+
+
+# ------------------------------------------------------------------ paged store
+def _make_pool(gpu, d, key_bits, vb, H, n_pages, dtype=torch.bfloat16, seed=42, gs=32):
+    from turboquant_amd.paged import PagedKVPool
+    from turboquant_amd.quantizer import TurboQuantProd
+    tq = TurboQuantProd(d, bits=key_bits, device=gpu, seed=seed)
+    return PagedKVPool(tq, H, n_pages, value_bits=vb, value_group_size=gs, dtype=dtype, device=gpu), tq
+
+
+@pytest.mark.parametrize("d,key_bits,vb,dtype", [(128, 3, 4, torch.bfloat16), (256, 3, 2, torch.bfloat16),
+                                                   (64, 2, 2, torch.float16), (128, 4, 4, torch.bfloat16),
+                                                   (128, 5, 2, torch.float32)])
+def test_paged_append_equals_flat_quantise(gpu, d, key_bits, vb, dtype):
+    from turboquant_amd.kv_cache import quantize_values
+    H, T = 2, 75
+    pool, tq = _make_pool(gpu, d, key_bits, vb, H, 16, dtype)
+    g = torch.Generator().manual_seed(d + key_bits)
+    k = torch.randn(1, T, H, d, generator=g).to(dtype).to(gpu)
+    v = torch.randn(1, T, H, d, generator=g).to(dtype).to(gpu)
+    table = torch.randperm(16, generator=g).to(torch.int32).to(gpu)[None, :]     # scattered physical pages
+    # three appends with ragged boundaries: 0..20, 20..21, 21..75
+    for a, b in ((0, 20), (20, 21), (21, 75)):
+        pool.append(k[:, a:b], v[:, a:b], table, torch.tensor([a], dtype=torch.int32, device=gpu))
+    idx, sgn, norms, rnorms, vdata, vsc, vz = pool.export_flat(table[0], T)
+    ref = tq.quantize(k[0].transpose(0, 1))                 # (H, T, d)
+    refv = quantize_values(v[0].transpose(0, 1), bits=vb, group_size=32)
+    torch.cuda.synchronize()
+    assert torch.equal(idx, ref.mse_indices) and torch.equal(sgn, ref.qjl_signs)
+    assert torch.equal(norms, ref.norms) and torch.equal(rnorms, ref.residual_norms)
+    assert torch.equal(vdata, refv.data) and torch.equal(vsc, refv.scales) and torch.equal(vz, refv.zeros)
+    # and the same tokens appended in one go give the same pages
+    pool2, _ = _make_pool(gpu, d, key_bits, vb, H, 16, dtype)
+    pool2.append(k, v, table)
+    n_pg = (T + 15) // 16
+    used = table[0, :n_pg].long()
+    assert torch.equal(pool.data[used[:-1]], pool2.data[used[:-1]])
+
+
+def _store_from_oracle_view(pool, table_row, n_tok):
+    idx, sgn, norms, rnorms, vdata, vsc, vz = [t.cpu() for t in pool.export_flat(table_row, n_tok)]
+    return key_code(idx, sgn, rnorms, norms, pool.quantizer.bits - 1), value_code(vdata, vsc, vz, pool.value_bits)
+
+
+def _decode_case(gpu, d, key_bits, vb, B, Hq, Hkv, lens, recent, seed, n_split=None, dtype=torch.bfloat16):
+    g = torch.Generator().manual_seed(seed)
+    max_len = max(max(lens), 1)
+    pages_per_seq = (max_len + 15) // 16
+    n_pages = B * pages_per_seq + 3
+    pool, tq = _make_pool(gpu, d, key_bits, vb, Hkv, n_pages, dtype, seed=42 + 7 * (seed % 5))
+    perm = torch.randperm(n_pages, generator=g)[: B * pages_per_seq].to(torch.int32)
+    table = perm.reshape(B, pages_per_seq).to(gpu)
+    k = torch.randn(B, max_len, Hkv, d, generator=g).to(dtype)
+    v = torch.randn(B, max_len, Hkv, d, generator=g).to(dtype)
+    pool.append(k.to(gpu), v.to(gpu), table)
+    q = torch.randn(B, Hq, d, generator=g).to(dtype)
+    rk = rv = rl = None
+    if recent:
+        rk = torch.randn(B, max(recent), Hkv, d, generator=g).to(dtype)
+        rv = torch.randn(B, max(recent), Hkv, d, generator=g).to(dtype)
+        rl = torch.tensor(recent, dtype=torch.int32)
+    seq = torch.tensor(lens, dtype=torch.int32)
+    out = pool.decode_attention(q.to(gpu), table, seq.to(gpu), recent_k=None if rk is None else rk.to(gpu),
+                                recent_v=None if rv is None else rv.to(gpu),
+                                recent_len=None if rl is None else rl.to(gpu), n_split=n_split, max_len=max_len)
+    torch.cuda.synchronize()
+    prm = params_of(tq)
+    worst = 1.0
+    for b in range(B):
+        kc = vc = None
+        if lens[b]:
+            kc, vc = _store_from_oracle_view(pool, table[b], lens[b])
+        r = recent[b] if recent else 0
+        # MIN_HISTORY is host policy; the kernel itself attends to any non-empty history
+        want = O.hybrid_attention(q[b:b + 1], kc, vc, max(lens[b], O.MIN_HISTORY) if lens[b] else 0, prm, Hkv,
+                                  rk[b, :r] if r else None, rv[b, :r] if r else None)
+        got = out[b:b + 1].cpu()
+        assert got.dtype == q.dtype
+        if lens[b] == 0 and r == 0:
+            assert torch.count_nonzero(got) == 0
+            continue
+        c = cosine(got, want)
+        worst = min(worst, c)
+        assert c >= COS_GATE, (b, c)
+        assert (got.float() - want.float()).abs().max() <= 2 ** -7 * want.float().abs().max() + 1e-3, b
+    return worst
+
+
+@pytest.mark.parametrize("d,key_bits,vb,Hq,Hkv", [(128, 3, 4, 8, 2), (256, 3, 2, 16, 2), (128, 3, 2, 4, 4),
+                                                   (64, 3, 4, 4, 1), (128, 4, 4, 8, 2), (128, 2, 2, 6, 2)])
+def test_decode_attention_matches_oracle_on_the_same_store(gpu, d, key_bits, vb, Hq, Hkv):
+    _progress(f"decode d={d} kb={key_bits} vb={vb} Hq={Hq} Hkv={Hkv}")
+    worst = _decode_case(gpu, d, key_bits, vb, 3, Hq, Hkv, [200, 37, 512], None, seed=d + vb)
+    _progress(f"   worst cosine {worst:.7f}")
+
+
+def test_decode_attention_ragged_empty_and_hybrid_tail(gpu):
+    # empty sequence, history shorter than a page, page-aligned history, ragged exact tails
+    worst = _decode_case(gpu, 128, 3, 4, 5, 8, 2, [0, 5, 16, 33, 1000], [0, 3, 128, 0, 77], seed=77)
+    _progress(f"ragged+tail worst cosine {worst:.7f}")
+    worst = _decode_case(gpu, 128, 3, 2, 2, 8, 8, [0, 0], [40, 1], seed=78)          # exact tokens only
+    worst = _decode_case(gpu, 128, 3, 2, 2, 4, 2, [0, 64], None, seed=79)            # one row has nothing at all
+
+
+def test_decode_split_invariance_and_page_permutation(gpu):
+    from turboquant_amd.paged import PagedKVPool
+    g = torch.Generator().manual_seed(5)
+    d, Hkv, Hq, B, N = 128, 2, 8, 2, 1500
+    pool, tq = _make_pool(gpu, d, 3, 4, Hkv, 2 * 94 + 1)
+    k = torch.randn(B, N, Hkv, d, generator=g).bfloat16().to(gpu)
+    v = torch.randn(B, N, Hkv, d, generator=g).bfloat16().to(gpu)
+    q = torch.randn(B, Hq, d, generator=g).bfloat16().to(gpu)
+    t1 = torch.arange(2 * 94, dtype=torch.int32).reshape(2, 94).to(gpu)
+    pool.append(k, v, t1)
+    seq = torch.tensor([N, N - 7], dtype=torch.int32, device=gpu)
+    outs = [pool.decode_attention(q, t1, seq, n_split=s, max_len=N).float() for s in (1, 3, 32, 94)]
+    for o in outs[1:]:
+        assert (o - outs[0]).abs().max() <= 2 ** -7 * outs[0].abs().max()
+    # the same tokens behind a permuted page table give bit-identical results
+    pool2 = PagedKVPool(tq, Hkv, 2 * 94 + 1, value_bits=4, dtype=torch.bfloat16, device=gpu)
+    t2 = torch.randperm(2 * 94, generator=g).to(torch.int32).reshape(2, 94).to(gpu)
+    pool2.append(k, v, t2)
+    o2 = pool2.decode_attention(q, t2, seq, n_split=3, max_len=N).float()
+    assert torch.equal(o2, outs[1])
+
+
+def test_decode_constant_values_and_convexity(gpu):
+    # softmax weights are a convex combination: constant V comes back exactly (up to value
+    # quantisation of a constant group, which is exact) and outputs stay inside [min v, max v]
+    g = torch.Generator().manual_seed(6)
+    d, Hkv, Hq, N = 128, 1, 4, 300
+    pool, _ = _make_pool(gpu, d, 3, 2, Hkv, 20)
+    k = torch.randn(1, N, Hkv, d, generator=g).bfloat16().to(gpu)
+    v = torch.full((1, N, Hkv, d), 0.75).bfloat16().to(gpu)
+    t = torch.arange(19, dtype=torch.int32)[None].to(gpu)
+    pool.append(k, v, t)
+    q = torch.randn(1, Hq, d, generator=g).bfloat16().to(gpu)
+    out = pool.decode_attention(q, t, torch.tensor([N], dtype=torch.int32, device=gpu), max_len=N)
+    assert torch.all(out.float() == 0.75)
+
+
+# ------------------------------------------------------------------ store / capture / score API (reference call shapes)
+def test_store_flat_cache_matches_reference_golden(gpu, golden):
+    from turboquant_amd.score import compute_hybrid_attention
+    from turboquant_amd.store import CompressedKVStore
+    z = golden.npz("hybrid")
+    for case in golden.cases("hybrid"):
+        H, G, d, n_hist, n_recent, vb = [int(x) for x in z[case + ".meta"]]
+        _progress(f"hybrid {case}")
+        store = CompressedKVStore(d, H, key_bits=3, value_bits=vb, value_group_size=32, device=gpu, layer_idx=3)
+        cent, _, thr = O.codebook_tensors(golden.codebook(d, 2))
+        prm = O.KeyParams(torch.from_numpy(z[case + ".Pi"]), torch.from_numpy(z[case + ".S"]), cent, thr, 2)
+        install_matrices(store.quantizer, prm)
+        q = golden.tensor("hybrid", case + ".q").to(gpu)
+        if n_hist:
+            k = golden.tensor("hybrid", case + ".k").to(gpu)
+            v = golden.tensor("hybrid", case + ".v").to(gpu)
+            store.append_chunk(k[: n_hist // 2], v[: n_hist // 2])
+            store.append_chunk(k[n_hist // 2:], v[n_hist // 2:])
+            assert store.num_tokens == n_hist and store.num_chunks == 2
+            flat = store.get_flat_cache()
+            assert flat.num_tokens == n_hist and flat is store.get_flat_cache()
+            n_coord = n_hist * H * d
+            assert flat.prod_q.mse_indices.shape == z[case + ".mse_indices"].shape
+            assert byte_mismatch(flat.prod_q.mse_indices, torch.from_numpy(z[case + ".mse_indices"])) <= max(1, FLIP_RATE * n_coord)
+            assert bit_mismatch(flat.prod_q.qjl_signs, torch.from_numpy(z[case + ".qjl_signs"])) <= max(2, FLIP_RATE * n_coord)
+            assert torch.equal(flat.value_q.data.cpu(), torch.from_numpy(z[case + ".v_data"]))
+            assert torch.equal(flat.value_q.scales.cpu(), golden.tensor("hybrid", case + ".v_scales"))
+            assert torch.equal(flat.value_q.zeros.cpu(), golden.tensor("hybrid", case + ".v_zeros"))
+            assert store.memory_bytes() == int(z[case + ".memory_bytes"])
+        else:
+            assert store.get_flat_cache() is None
+        rk = golden.tensor("hybrid", case + ".recent_k").to(gpu) if n_recent else None
+        rv = golden.tensor("hybrid", case + ".recent_v").to(gpu) if n_recent else None
+        out = compute_hybrid_attention(q, store, rk, rv, num_query_heads=H * G).cpu()
+        ref = golden.tensor("hybrid", case + ".out")
+        assert out.shape == ref.shape and out.dtype == ref.dtype
+        c = cosine(out, ref)
+        _progress(f"   cosine vs reference output {c:.7f}")
+        assert c >= COS_GATE, case
+    # nothing stored, nothing recent: zeros (score.py:59-63); GQA mismatch raises
+    store = CompressedKVStore(128, 2, device=gpu)
+    q = torch.randn(1, 4, 128, device=gpu, dtype=torch.bfloat16)
+    assert torch.count_nonzero(compute_hybrid_attention(q, store, None, None, 4)) == 0
+    with pytest.raises(ValueError):
+        compute_hybrid_attention(torch.randn(1, 5, 128, device=gpu, dtype=torch.bfloat16), store,
+                                 torch.randn(3, 2, 128, device=gpu, dtype=torch.bfloat16),
+                                 torch.randn(3, 2, 128, device=gpu, dtype=torch.bfloat16), 5)
+
+
+def test_capture_engine_end_to_end_on_gpu(gpu):
+    from turboquant_amd.capture import KVCaptureEngine
+    from turboquant_amd.score import compute_hybrid_attention
+    from turboquant_amd.store import CompressedKVStore
+    g = torch.Generator().manual_seed(8)
+    H, G, d = 2, 4, 128
+    store = CompressedKVStore(d, H, key_bits=3, value_bits=4, device=gpu, layer_idx=1)
+    eng = KVCaptureEngine(store, ring_capacity=32, device=gpu)
+    k = torch.randn(500, H, d, generator=g).bfloat16()
+    v = torch.randn(500, H, d, generator=g).bfloat16()
+    eng.ingest_prefill(k[:300].to(gpu), v[:300].to(gpu), 300)
+    for t in range(300, 500):
+        eng.ingest_decode(k[t:t + 1].to(gpu), v[t:t + 1].to(gpu), 1)
+    assert eng.total_tokens == 500 and eng.total_buffered_tokens == 500 - store.num_tokens
+    assert store.num_tokens == 268 + 32 * 7 and store.num_chunks == 8
+    q = torch.randn(2, H * G, d, generator=g).bfloat16()
+    rk, rv = eng.ring.peek()
+    out = compute_hybrid_attention(q.to(gpu), store, rk, rv, num_query_heads=H * G).cpu()
+    flat = store.get_flat_cache()
+    kc = key_code(flat.prod_q.mse_indices.cpu(), flat.prod_q.qjl_signs.cpu(), flat.prod_q.residual_norms.cpu(),
+                  flat.prod_q.norms.cpu(), 2)
+    vc = value_code(flat.value_q.data.cpu(), flat.value_q.scales.cpu(), flat.value_q.zeros.cpu(), 4)
+    want = O.hybrid_attention(q, kc, vc, store.num_tokens, params_of(store.quantizer), H, rk.cpu(), rv.cpu())
+    assert cosine(out, want) >= COS_GATE
+    eng.reset()
+    assert eng.total_tokens == 0 and store.get_flat_cache() is None
+
+
+def test_kv_cache_object_against_reference_golden(gpu, golden):
+    from turboquant_amd.kv_cache import TurboQuantKVCache
+    z = golden.npz("kv_cache_object")
+    cache = TurboQuantKVCache(128, key_bits=3, value_bits=2, buffer_size=16, device=gpu, dtype=torch.float32, layer_idx=1)
+    cent, _, thr = O.codebook_tensors(golden.codebook(128, 2))
+    install_matrices(cache.key_quantizer, O.KeyParams(torch.from_numpy(z["Pi"]), torch.from_numpy(z["S"]), cent, thr, 2))
+    cache.prefill(torch.from_numpy(z["k"]).to(gpu), torch.from_numpy(z["v"]).to(gpu))
+    for i in range(5):
+        cache.append(torch.from_numpy(z[f"append_k{i}"]).to(gpu), torch.from_numpy(z[f"append_v{i}"]).to(gpu))
+    assert cache.get_seq_length() == int(z["seq_len"])
+    sc = cache.attention_scores(torch.from_numpy(z["q"]).to(gpu)).cpu()
+    ref = torch.from_numpy(z["scores"])
+    assert sc.shape == ref.shape
+    # a flipped sign bit moves single entries; everything else agrees tightly
+    assert ((sc - ref).abs() > 1e-4).float().mean() < 0.01
+    out = cache.attend(torch.softmax(sc.to(gpu), dim=-1)).cpu()
+    assert cosine(out, torch.from_numpy(z["out"])) >= COS_GATE
+    mem = cache.memory_bytes()
+    assert [mem[n] for n in ("quantized_keys", "quantized_values", "buffer", "total")] == z["memory"].tolist()

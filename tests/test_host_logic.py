@@ -1,0 +1,235 @@
+"""CPU: host-side logic of the package (no kernel launches): the C-ABI library
+loads and exports what include/tq_hip.h declares, argument checking, page
+geometry, codebook files, ring / capture policy against the reference's trace,
+and the loud failure on CPU tensors."""
+
+import ctypes as C
+import json
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+import turboquant_amd
+from turboquant_amd import _ffi
+from turboquant_amd.capture import KVCaptureEngine, RingBuffer
+from turboquant_amd.codebook import compute_lloyd_max_codebook, get_codebook, get_codebook_tensors
+from turboquant_amd.quantizer import TurboQuantMSE, TurboQuantProd, _pack_indices, _unpack_indices
+from turboquant_amd.kv_cache import ValueQuantized, quantize_values, unpack_values
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "tq_hip.h")).read()
+    declared = set(re.findall(r"\b(tq_[a-z_0-9]+)\s*\(", header))
+    assert declared, "no declarations found"
+    lib = _ffi.lib()
+    for name in sorted(declared):
+        assert hasattr(lib, name), f"{name} declared in tq_hip.h but not exported"
+    assert declared == set(_ffi.EXPORTED_SYMBOLS)
+    assert lib.tq_version() == _ffi.ABI_VERSION
+
+
+def test_argument_errors_are_reported_before_any_launch():
+    lib = _ffi.lib()
+    assert lib.tq_bucketize_pack(None, 4, 128, None, 2, None, None) == -3
+    assert lib.tq_sign_pack(None, 4, 128, None, None) == -3
+    ly = _ffi.TqLayer()
+    ly.d, ly.mse_bits = 100, 2                       # not a multiple of 64
+    assert lib.tq_quantize_keys(1, 0, 4, 128, C.byref(ly), 1, 1, 1, 1, None, None, 0, None) == -2
+    assert lib.tq_quantize_values(1, 0, 4, 128, 128, 48, 2, 1, 1, 1, None) == -1     # 128 % 48 != 0
+    assert lib.tq_quantize_values(1, 0, 4, 128, 128, 32, 3, 1, 1, 1, None) == -2     # 3-bit values
+    assert lib.tq_decode_workspace_bytes(0, 8, 128, 4) == 0
+    with pytest.raises(ValueError):
+        _ffi.check(-1, "x")
+    with pytest.raises(RuntimeError):
+        _ffi.check(700, "x")
+    with pytest.raises(TypeError):
+        _ffi.dtype_tag(torch.float64)
+
+
+@pytest.mark.parametrize("d,mb,vb,gs,dt,per_token", [
+    (128, 2, 4, 32, torch.bfloat16, 32 + 16 + 2 + 4 + 64 + 16),      # 134 B: fp32 residual norm
+    (256, 2, 2, 32, torch.bfloat16, 64 + 32 + 2 + 4 + 64 + 32),      # 198 B
+    (128, 2, 2, 32, torch.float16, 32 + 16 + 2 + 4 + 32 + 16),
+    (128, 3, 4, 64, torch.float32, 48 + 16 + 4 + 4 + 64 + 16),
+])
+def test_page_layout_geometry(d, mb, vb, gs, dt, per_token):
+    L = _ffi.make_page_layout(d, mb, vb, gs, dt)
+    assert L.off_planes == 0
+    offs = [L.off_planes, L.off_norm, L.off_rnorm, L.off_vdata, L.off_vscale, L.off_vzero]
+    assert offs == sorted(offs) and all(o % 16 == 0 for o in offs)
+    used = L.off_vzero + (d // gs) * 16 * (4 if dt == torch.float32 else 2)
+    assert used == 16 * per_token
+    assert L.page_bytes % 128 == 0 and used <= L.page_bytes < used + 128
+    with pytest.raises(ValueError):
+        _ffi.make_page_layout(100, 2, 2, 32, torch.bfloat16)
+    with pytest.raises(ValueError):
+        _ffi.make_page_layout(128, 2, 3, 32, torch.bfloat16)
+
+
+@pytest.mark.parametrize("d,mb", [(128, 1), (128, 2), (128, 3), (128, 4), (64, 2), (256, 2), (576, 3)])
+def test_walsh_terms_reconstruct_the_codebook(d, mb):
+    cb = get_codebook(d, mb)
+    cent = torch.tensor(cb["centroids"], dtype=torch.float32)
+    ly = _ffi.TqLayer()
+    _ffi.walsh_terms(cent, mb, ly)
+    assert 1 <= ly.n_terms <= 2 ** mb - 1
+    # a symmetric codebook is an odd function of the +-1 index bits: only odd-size subsets survive
+    assert ly.n_terms == 2 ** (mb - 1)
+    for idx in range(2 ** mb):
+        val = ly.term_const + sum(ly.term_coef[t] * (bin(idx & ly.term_mask[t]).count("1") & 1)
+                                  for t in range(ly.n_terms))
+        assert val == pytest.approx(float(cent[idx]), abs=2e-7)
+    # an asymmetric codebook keeps every subset
+    skew = torch.arange(2 ** mb, dtype=torch.float32) ** 2
+    _ffi.walsh_terms(skew, mb, ly)
+    for idx in range(2 ** mb):
+        val = ly.term_const + sum(ly.term_coef[t] * (bin(idx & ly.term_mask[t]).count("1") & 1)
+                                  for t in range(ly.n_terms))
+        assert val == pytest.approx(float(skew[idx]), abs=1e-4)
+
+
+def test_shipped_codebooks_equal_reference_files(golden):
+    for d, b in [(64, 1), (64, 2), (64, 3), (64, 4), (128, 1), (128, 2), (128, 3), (128, 4), (576, 3),
+                 (256, 1), (256, 2), (256, 3)]:
+        ref, got = golden.codebook(d, b), get_codebook(d, b)
+        assert got["d"] == d and got["bits"] == b
+        assert set(got) == {"centroids", "boundaries", "mse_per_coord", "mse_total", "d", "bits"}
+        assert np.allclose(got["centroids"], ref["centroids"], rtol=0, atol=1e-15)
+        # the fp32 tensors handed to the kernels are identical
+        c, e = get_codebook_tensors(d, b, "cpu")
+        assert torch.equal(c, torch.tensor(ref["centroids"], dtype=torch.float32))
+        # the middle boundary is 0 by symmetry; two of the reference's files hold -4e-17 / -3e-18 there
+        # (rounding noise of the machine that wrote them), everything else is identical in fp32
+        ref_e = torch.tensor(ref["boundaries"], dtype=torch.float32)
+        differs = (e != ref_e)
+        assert int(differs.sum()) <= 1 and torch.all(ref_e[differs].abs() < 1e-15) and torch.all(e[differs] == 0)
+
+
+def test_codebook_solver_known_answer(golden):
+    got = compute_lloyd_max_codebook(128, 2)
+    ref = golden.codebook(128, 2)
+    assert got["centroids"] == pytest.approx(ref["centroids"], abs=1e-15)
+    assert got["mse_total"] == pytest.approx(0.11600007032012699, abs=1e-13)
+    with pytest.raises(ValueError):
+        compute_lloyd_max_codebook(2, 1)
+
+
+def test_pack_helpers_match_reference_vectors(golden):
+    z = golden.npz("packing")
+    for bits in (1, 2, 3, 4, 5):
+        for d in (128, 13):
+            idx = torch.from_numpy(z[f"idx_b{bits}_d{d}"])
+            pk = _pack_indices(idx, bits)
+            assert pk.dtype == torch.uint8 and np.array_equal(pk.numpy(), z[f"packed_b{bits}_d{d}"])
+            assert np.array_equal(_unpack_indices(pk, bits, d).numpy(), z[f"unpacked_b{bits}_d{d}"])
+    vq = ValueQuantized(torch.tensor([[0b11100100, 0b00011011]], dtype=torch.uint8), None, None, 2)
+    assert unpack_values(vq).tolist() == [[0, 1, 2, 3, 3, 2, 1, 0]]
+    vq = ValueQuantized(torch.tensor([[0xA5]], dtype=torch.uint8), None, None, 4)
+    assert unpack_values(vq).tolist() == [[5, 10]]
+
+
+def test_public_surface():
+    assert turboquant_amd.__version__ == "0.2.0"
+    for name in ("compute_lloyd_max_codebook", "get_codebook", "TurboQuantMSE", "TurboQuantProd", "TurboQuantKVCache",
+                 "RingBuffer", "KVCaptureEngine", "CompressedKVStore", "compute_hybrid_attention"):
+        assert hasattr(turboquant_amd, name)
+    tq = TurboQuantProd(128, bits=3, device=torch.device("cpu"))
+    assert set(dict(tq.named_buffers())) >= {"S", "mse_quantizer.Pi", "mse_quantizer.centroids",
+                                             "mse_quantizer.boundaries", "mse_quantizer.decision_boundaries"}
+    assert set(tq.state_dict()) == {"S", "mse_quantizer.Pi", "mse_quantizer.centroids", "mse_quantizer.boundaries",
+                                    "mse_quantizer.decision_boundaries"}
+    assert tq.mse_quantizer.bits == 2 and tq.mse_quantizer.n_clusters == 4
+    with pytest.raises(AssertionError):
+        TurboQuantProd(128, bits=1, device=torch.device("cpu"))
+
+
+def test_no_cpu_fallback():
+    tq = TurboQuantProd(128, bits=3, device=torch.device("cpu"))
+    x = torch.randn(4, 128)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        tq.quantize(x)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        tq.mse_quantizer.quantize(x)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        quantize_values(x, 2, 32)
+
+
+class _TagStore:
+    def __init__(self, heads, dim):
+        self.num_kv_heads, self.head_dim, self.device = heads, dim, torch.device("cpu")
+        self.chunks = []
+
+    @property
+    def num_tokens(self):
+        return sum(len(c) for c in self.chunks)
+
+    def append_chunk(self, key, value):
+        assert torch.equal(key, value)
+        self.chunks.append([int(t) for t in key[:, 0, 0].float().tolist()])
+
+    def reset(self):
+        self.chunks = []
+
+
+def test_capture_engine_routes_tokens_like_the_reference(golden):
+    for tr in golden.json("capture_trace.json"):
+        if tr.get("double_prefill"):
+            st = _TagStore(1, 4)
+            eng = KVCaptureEngine(st, ring_capacity=4, device="cpu", dtype=torch.float32)
+            a = torch.arange(3.0).view(-1, 1, 1).expand(3, 1, 4)
+            eng.ingest_prefill(a, a, 3)
+            eng.ingest_prefill(a + 10, a + 10, 3)
+        else:
+            st = _TagStore(2, 8)
+            eng = KVCaptureEngine(st, ring_capacity=tr["capacity"], device="cpu", dtype=torch.float32)
+            tok = 0
+            if tr["prefill"]:
+                k = torch.arange(float(tr["prefill"])).view(-1, 1, 1).expand(tr["prefill"], 2, 8)
+                eng.ingest_prefill(k, k, tr["prefill"])
+                tok = tr["prefill"]
+            for _ in range(tr["decodes"]):
+                k = torch.full((1, 2, 8), float(tok))
+                eng.ingest_decode(k, k, 1)
+                tok += 1
+            if tr["flush"]:
+                eng.flush()
+            assert eng.total_compressed_tokens == tr["total_compressed"]
+            assert eng.total_buffered_tokens == tr["total_buffered"]
+            assert eng.total_tokens == tr["total_compressed"] + tr["total_buffered"]
+            assert eng.ring.total_written == tr["ring_total_written"]
+        peek = eng.ring.peek()
+        ring = [] if peek is None else [int(t) for t in peek[0][:, 0, 0].tolist()]
+        assert st.chunks == tr["chunks"]
+        assert ring == tr["ring"]
+
+
+def test_ring_buffer_contract():
+    rb = RingBuffer(4, 2, 8, "cpu", torch.float32)
+    assert rb.size == 0 and not rb.is_full and rb.peek() is None and rb.drain() is None
+    k = torch.arange(6.0).view(-1, 1, 1).expand(6, 2, 8)
+    spill = rb.write(k, k, 6)
+    assert spill is not None and spill[0][:, 0, 0].tolist() == [0, 1, 2, 3]
+    assert rb.size == 2 and rb.total_written == 6
+    assert rb.peek()[0][:, 0, 0].tolist() == [4, 5]
+    got = rb.drain()
+    assert got[0][:, 0, 0].tolist() == [4, 5] and rb.size == 0
+    rb.reset()
+    assert rb.total_written == 0
+
+
+def test_paged_cache_ingest_gathers_blocks_in_table_order():
+    st = _TagStore(1, 4)
+    eng = KVCaptureEngine(st, ring_capacity=4, device="cpu", dtype=torch.float32)
+    cache = torch.zeros(2, 5, 4, 1, 4)
+    table = torch.tensor([3, 0, 4])
+    for logical, phys in enumerate(table.tolist()):
+        for s in range(4):
+            cache[:, phys, s] = logical * 4 + s
+    eng.ingest_prefill_from_paged_cache(cache, 10, table, 4)
+    assert st.chunks == [[0, 1, 2, 3, 4, 5]]
+    assert eng.ring.peek()[0][:, 0, 0].tolist() == [6, 7, 8, 9]

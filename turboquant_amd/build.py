@@ -20,6 +20,9 @@ SOURCES = ["tq_quantize.hip", "tq_score.hip", "tq_decode.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # no implicit a*b+c fusion: the quantisers mirror separately rounded torch ops;
+    # the kernels call fmaf() explicitly wherever a fused multiply-add is wanted
+    "-ffp-contract=off",
     "-fno-gpu-rdc", "-Wall", "-Wno-unused-function",
 ]
 

@@ -23,7 +23,7 @@ def generate_rotation_matrix(d: int, device, dtype: torch.dtype = torch.float32,
     Its determinant can be -1; orthogonality is all the quantiser needs."""
     q_factor, r_factor = torch.linalg.qr(_seeded_gaussian(d, seed))
     col_sign = torch.sign(torch.diagonal(r_factor))
-    return (q_factor * col_sign[None, :]).to(device=device, dtype=dtype)
+    return (q_factor * col_sign[None, :]).contiguous().to(device=device, dtype=dtype)
 
 
 def generate_qjl_matrix(d: int, device, dtype: torch.dtype = torch.float32, seed: int = 12345) -> torch.Tensor:
