@@ -1,0 +1,290 @@
+"""Headline benchmark: compressed-KV decode attention GB/s (and % of HBM peak)
+plus quantize tokens/s, on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
+
+A step is one pass of the fused decode-attention path (query rotation, page
+streaming kernel, merge) over the long-context configuration: 4 sequences x
+131 072 context tokens, 16 query heads over 2 KV heads, head_dim 256, 3-bit keys
+(2-bit Lloyd-Max + 1-bit QJL), 2-bit values in groups of 32, 16-token pages.
+The compressed pools are resident in HBM before timing starts; steps rotate
+over several pools so that no step finds its pages in the 256 MB Infinity
+Cache.  `value` = algorithmic KV bytes per step / step time, with the
+reference's own byte accounting (norms, residual norms, scales and zeros at
+2 bytes): 196 B per (token, KV head).
+
+The same JSON line carries
+  roofline     : the page-streaming kernel alone (hipEvents around that stage),
+                 algorithmic bytes / its mean duration, against 8 TB/s;
+  quantize     : tokens/s of the fused paged quantise call on the prefill
+                 configuration (32 768 tokens x 8 KV heads, head_dim 128);
+  decode_gqa   : the 16 x 8192-token GQA decode configuration;
+  cpu_baseline : the CPU oracle's de-quantise-everything attention (the
+                 reference's production read path) timed on the host cores on
+                 one of the four sequences.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def student_t(shape, nu, gen, device):
+    import torch
+    z = torch.randn(*shape, generator=gen, device=device)
+    chi = torch.zeros(shape, device=device)
+    for _ in range(nu):
+        chi += torch.randn(*shape, generator=gen, device=device) ** 2
+    return z / torch.sqrt(chi / nu)
+
+
+def algorithmic_bytes_per_token_head(d, mse_bits, value_bits, group):
+    eff = 1 if mse_bits == 1 else (2 if mse_bits == 2 else 4)
+    return d * eff // 8 + d // 8 + 2 + 2 + d * value_bits // 8 + 2 * 2 * (d // group)
+
+
+class DecodeWorkload:
+    """B sequences of N compressed tokens in `n_pools` separate pools."""
+
+    def __init__(self, name, B, N, Hq, Hkv, d, key_bits, value_bits, n_pools, seed, dist, device):
+        import torch
+        from turboquant_amd.paged import PagedKVPool
+        from turboquant_amd.quantizer import TurboQuantProd
+        self.name, self.B, self.N, self.Hq, self.Hkv, self.d = name, B, N, Hq, Hkv, d
+        self.key_bits, self.value_bits = key_bits, value_bits
+        gen = torch.Generator(device=device).manual_seed(seed)
+        self.tq = TurboQuantProd(d, bits=key_bits, device=device)
+        pages_per_seq = (N + 15) // 16
+        n_pages = B * pages_per_seq
+        self.pools = []
+        perm = torch.randperm(n_pages, generator=gen, device=device).to(torch.int32)
+        self.table = perm.reshape(B, pages_per_seq).contiguous()
+        first = PagedKVPool(self.tq, Hkv, n_pages, value_bits=value_bits, value_group_size=32,
+                            dtype=torch.bfloat16, device=device)
+        chunk = 16384
+        for b in range(B):                      # sequence by sequence, in chunks, to bound the bf16 staging memory
+            for t0 in range(0, N, chunk):
+                t1 = min(N, t0 + chunk)
+                shape = (1, t1 - t0, Hkv, d)
+                if dist == "student_t5":
+                    k, v = student_t(shape, 5, gen, device), student_t(shape, 5, gen, device)
+                else:
+                    k = torch.randn(*shape, generator=gen, device=device)
+                    v = torch.randn(*shape, generator=gen, device=device)
+                first.append(k.bfloat16(), v.bfloat16(), self.table[b:b + 1],
+                             torch.tensor([t0], dtype=torch.int32, device=device))
+        self.pools.append(first)
+        for _ in range(n_pools - 1):
+            p = PagedKVPool(self.tq, Hkv, n_pages, value_bits=value_bits, value_group_size=32,
+                            dtype=torch.bfloat16, device=device)
+            p.data.copy_(first.data)
+            self.pools.append(p)
+        self.q = torch.randn(B, Hq, d, generator=gen, device=device).bfloat16()
+        self.seq = torch.full((B,), N, dtype=torch.int32, device=device)
+        self.n_split = first.default_splits(B, N)
+        self.ws = first.workspace(B, Hq, self.n_split)
+        self.out = torch.empty_like(self.q)
+        self.bytes = B * Hkv * N * algorithmic_bytes_per_token_head(d, key_bits - 1, value_bits, 32)
+        self.stored_bytes = B * Hkv * pages_per_seq * first.page_bytes
+
+    def step(self, i, stages=7):
+        pool = self.pools[i % len(self.pools)]
+        pool.decode_attention(self.q, self.table, self.seq, n_split=self.n_split, workspace=self.ws, out=self.out,
+                              max_len=self.N, stages=stages)
+
+
+def time_steps(fn, steps, warmup):
+    """(mean ms per step, wall ms per step) with HIP events on the launch stream."""
+    import torch
+    for i in range(warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for i in range(steps):
+        fn(warmup + i)
+    stop.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3 / steps
+    return start.elapsed_time(stop) / steps, wall
+
+
+def time_kernel_stage(work, steps, warmup):
+    """Mean duration of the page-streaming kernel alone: events bracket each
+    stage-2 launch separately, the other stages run untimed in between."""
+    import torch
+    for i in range(warmup):
+        work.step(i)
+    torch.cuda.synchronize()
+    total = 0.0
+    evs = []
+    for i in range(steps):
+        work.step(warmup + i, stages=1)
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        work.step(warmup + i, stages=2)
+        b.record()
+        work.step(warmup + i, stages=4)
+        evs.append((a, b))
+    torch.cuda.synchronize()
+    for a, b in evs:
+        total += a.elapsed_time(b)
+    return total / steps
+
+
+def cpu_decode_baseline(work):
+    """The oracle's de-quantise-all + dense attention on one sequence of the
+    workload, on the host cores."""
+    import torch
+    from oracle import tq_oracle as O
+    from tests.helpers import key_code, value_code, params_of
+    pool = work.pools[0]
+    idx, sgn, norms, rn, vd, vs, vz = [t.cpu() for t in pool.export_flat(work.table[0], work.N)]
+    kc = key_code(idx, sgn, rn, norms, work.key_bits - 1)
+    vc = value_code(vd, vs, vz, work.value_bits)
+    prm = params_of(work.tq)
+    q = work.q[:1].cpu()
+    times = []
+    out = None
+    for _ in range(3):
+        t0 = time.perf_counter()
+        out = O.hybrid_attention(q, kc, vc, work.N, prm, work.Hkv, None, None)
+        times.append(time.perf_counter() - t0)
+    sec = sorted(times)[1] if len(times) > 2 else min(times)
+    sample_bytes = work.bytes // work.B
+    return out, {"value": sample_bytes / sec / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(),
+                 "kind": "port", "seconds": sec,
+                 "sample": f"1 of {work.B} sequences ({work.N} tokens x {work.Hkv} KV heads), full-job time = x{work.B}"}
+
+
+def quantize_bench(device, steps, warmup):
+    import torch
+    from turboquant_amd.paged import PagedKVPool
+    from turboquant_amd.quantizer import TurboQuantProd
+    T, H, d = 32768, 8, 128
+    gen = torch.Generator(device=device).manual_seed(1)
+    k = torch.randn(1, T, H, d, generator=gen, device=device)
+    v = torch.randn(1, T, H, d, generator=gen, device=device)
+    for t in (k, v):
+        for h in range(H):
+            ch = torch.randperm(d, generator=gen, device=device)[:4]
+            t[0, :, h, ch] *= 20.0
+    k, v = k.bfloat16(), v.bfloat16()
+    tq = TurboQuantProd(d, bits=3, device=device)
+    pool = PagedKVPool(tq, H, T // 16, value_bits=2, value_group_size=32, dtype=torch.bfloat16, device=device)
+    table = torch.arange(T // 16, dtype=torch.int32, device=device)[None]
+    ms, _ = time_steps(lambda i: pool.append(k, v, table), steps, warmup)
+    flops = 3 * 2 * d * d * T * H
+    return {"tokens_per_s": T / (ms * 1e-3), "ms": ms, "tokens": T, "kv_heads": H, "head_dim": d,
+            "workload": "prefill quantize, 32768 tok x 8 KV heads, d=128, 3b keys + 2b values, pages of 16",
+            "contraction_tflops": flops / (ms * 1e-3) / 1e12,
+            "hbm_gbs": (T * (2 * H * d * 2 + H * 100)) / (ms * 1e-3) / 1e9}, (pool, k, v, table, tq)
+
+
+def cpu_quantize_baseline(k, v, tq, sample_tokens=4096):
+    import torch
+    from oracle import tq_oracle as O
+    from tests.helpers import params_of
+    prm = params_of(tq)
+    kk = k[0, :sample_tokens].transpose(0, 1).contiguous().cpu()      # (H, T, d)
+    vv = v[0, :sample_tokens].transpose(0, 1).contiguous().cpu()
+    times = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        O.prod_quantize(kk, prm)
+        O.quantize_values(vv, 2, 32)
+        times.append(time.perf_counter() - t0)
+    sec = sorted(times)[1]
+    return {"tokens_per_s": sample_tokens / sec, "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"{sample_tokens} of 32768 tokens x 8 KV heads"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    ap.add_argument("--context", type=int, default=131072, help="context tokens per sequence of the main workload")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the path has no cross-GPU step and this build runs on a single MI355X; "
+              "use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from turboquant_amd import _ffi
+    if not os.path.exists(_ffi.library_path()):
+        raise SystemExit("turboquant_amd/libtq_hip.so is missing; run `python -m turboquant_amd.build` first")
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+
+    main_w = DecodeWorkload("long-context decode", 4, args.context, 16, 2, 256, 3, 2, n_pools=4, seed=3,
+                            dist="student_t5", device=device)
+    ms, wall = time_steps(main_w.step, args.steps, args.warmup)
+    kern_ms = time_kernel_stage(main_w, args.steps, args.warmup)
+    value = main_w.bytes / (ms * 1e-3) / 1e9
+    achieved = main_w.bytes / (kern_ms * 1e-3) / 1e9
+
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "decode_pages_traffic.json")
+    if os.path.exists(tpath):
+        with open(tpath) as f:
+            t = json.load(f)
+        if t.get("context") == args.context:
+            traffic = t.get("hbm_bytes_per_launch")
+
+    gqa_w = DecodeWorkload("gqa decode", 16, 8192, 32, 8, 128, 3, 4, n_pools=4, seed=2, dist="normal", device=device)
+    gqa_ms, _ = time_steps(gqa_w.step, args.steps, args.warmup)
+    gqa_kern = time_kernel_stage(gqa_w, args.steps, args.warmup)
+
+    quant, (qpool, qk, qv, qtable, qtq) = quantize_bench(device, max(5, args.steps // 5), max(2, args.warmup // 5))
+
+    cpu = None
+    if not args.no_cpu:
+        ref_out, cpu = cpu_decode_baseline(main_w)
+        main_w.step(0)
+        torch.cuda.synchronize()
+        got = main_w.out[:1].float().cpu().flatten()
+        want = ref_out.float().flatten()
+        cpu["gpu_vs_oracle_cosine"] = float((got @ want) / (got.norm() * want.norm()))
+        quant["cpu_baseline"] = cpu_quantize_baseline(qk, qv, qtq)
+
+    line = {
+        "metric": "compressed-KV decode attn GB/s (% HBM peak) + quantize tokens/s, 1 GPU",
+        "value": value, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "u8 codes, fp32 accumulate", "data": "synthetic (seeded GPU generator; Student-t nu=5 K/V, bf16)",
+        "config": {"workload": f"long-context decode: 4 seq x {args.context} ctx, 16 q heads / 2 KV heads, head_dim 256, "
+                               "keys 3b (2b Lloyd-Max + 1b QJL, m=256), values 2b group 32, pages of 16, bf16 query",
+                   "algorithmic_bytes_per_step": main_w.bytes, "stored_bytes_per_step": main_w.stored_bytes,
+                   "n_split": main_w.n_split, "kv_pools_rotated": len(main_w.pools)},
+        "pct_hbm_peak": 100.0 * value / HBM_PEAK_GBS,
+        "wall_ms_per_step": wall,
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic, "kernel": "decode_pages_kernel",
+                     "kernel_ms": kern_ms},
+        "quantize": quant,
+        "decode_gqa": {"workload": "16 seq x 8192 ctx, 32 q heads / 8 KV heads, head_dim 128, keys 3b, values 4b",
+                       "GBps": gqa_w.bytes / (gqa_ms * 1e-3) / 1e9, "ms_per_step": gqa_ms,
+                       "kernel_GBps": gqa_w.bytes / (gqa_kern * 1e-3) / 1e9,
+                       "pct_hbm_peak": 100.0 * gqa_w.bytes / (gqa_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -183,6 +183,18 @@ int tq_decode_attn_paged(const void *q, int dtype, int B, int Hq, int Hkv, const
                          int64_t rs_r, int64_t rs_h, const int32_t *recent_len, void *out, void *workspace,
                          int n_split, void *stream);
 
+/* The same call restricted to some of its three stages, for timing them apart:
+ * bit 0 query rotation / sketch, bit 1 the page-streaming kernel (and the exact
+ * tail), bit 2 the merge.  stages = 7 is tq_decode_attn_paged.  A later stage
+ * expects the workspace an earlier call left behind.                            */
+int tq_decode_attn_paged_stages(const void *q, int dtype, int B, int Hq, int Hkv, const uint8_t *pool,
+                                int64_t num_pages, const int32_t *block_table, int bt_stride,
+                                const int32_t *seq_lens, float sm_scale, const tq_layer *layer,
+                                const tq_page_layout *layout, const void *recent_k, const void *recent_v,
+                                int recent_rows, int64_t rs_b, int64_t rs_r, int64_t rs_h,
+                                const int32_t *recent_len, void *out, void *workspace, int n_split, int stages,
+                                void *stream);
+
 /* Log-sum-exp merge of n_parts partial results per (b, query head):
  * parts (B*Hq, n_parts, d+2) fp32 = [running max, sum of exp, un-normalised acc];
  * out (B*Hq, d) `dtype`.  The same operator a context-parallel shard exchange

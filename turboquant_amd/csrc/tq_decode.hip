@@ -269,12 +269,13 @@ extern "C" int tq_decode_merge(const float* parts, int64_t rows, int n_parts, in
   return TQ_OK;
 }
 
-extern "C" int tq_decode_attn_paged(const void* q, int dtype, int B, int Hq, int Hkv, const uint8_t* pool,
-                                    int64_t num_pages, const int32_t* block_table, int bt_stride,
-                                    const int32_t* seq_lens, float sm_scale, const tq_layer* layer,
-                                    const tq_page_layout* layout, const void* recent_k, const void* recent_v,
-                                    int recent_rows, int64_t rs_b, int64_t rs_r, int64_t rs_h,
-                                    const int32_t* recent_len, void* out, void* workspace, int n_split, void* stream) {
+extern "C" int tq_decode_attn_paged_stages(const void* q, int dtype, int B, int Hq, int Hkv, const uint8_t* pool,
+                                           int64_t num_pages, const int32_t* block_table, int bt_stride,
+                                           const int32_t* seq_lens, float sm_scale, const tq_layer* layer,
+                                           const tq_page_layout* layout, const void* recent_k, const void* recent_v,
+                                           int recent_rows, int64_t rs_b, int64_t rs_r, int64_t rs_h,
+                                           const int32_t* recent_len, void* out, void* workspace, int n_split,
+                                           int stages, void* stream) {
   if (!q || !pool || !block_table || !seq_lens || !layer || !layout || !out || !workspace) return TQ_ENULL;
   if (B <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || n_split <= 0 || num_pages <= 0 || bt_stride < 0) return TQ_EINVAL;
   if (B > 65535 || Hkv > 65535) return TQ_EUNSUPPORTED;
@@ -291,12 +292,16 @@ extern "C" int tq_decode_attn_paged(const void* q, int dtype, int B, int Hq, int
   float* q_rot = parts + parts_floats(B, Hq, d, n_parts);
   float* q_sk = q_rot + (size_t)B * Hq * d;
 
-  int rc = tq_rotate_query(q, dtype, (int64_t)B * Hq, layer, q_rot, q_sk, stream);
-  if (rc) return rc;
+  if (stages & 1) {
+    int rc = tq_rotate_query(q, dtype, (int64_t)B * Hq, layer, q_rot, q_sk, stream);
+    if (rc) return rc;
+  }
+  if (!(stages & 6)) return TQ_OK;
 
   const int qsz = d * G + (d >> 5) * 4;
   size_t smem = (size_t)(2 * qsz + 16 + DEC_WAVES * G * 16 + DEC_WAVES * G * (d + 2)) * sizeof(float);
   dim3 grid(n_split, Hkv, B), block(DEC_WAVES * 64);
+  if (stages & 2) {
 #define TQ_LAUNCH_DEC(VB)                                                                                 \
   {                                                                                                       \
     auto kern = decode_pages_kernel<VB>;                                                                  \
@@ -312,8 +317,9 @@ extern "C" int tq_decode_attn_paged(const void* q, int dtype, int B, int Hq, int
   else TQ_LAUNCH_DEC(4)
 #undef TQ_LAUNCH_DEC
   TQ_CHECK_LAUNCH();
+  }
 
-  if (tail) {
+  if (tail && (stages & 2)) {
     size_t tsm = (size_t)(G * d + G * recent_rows + 2 * G) * sizeof(float);
     auto kern = exact_tail_kernel;
     if (tsm > 48 * 1024) {
@@ -324,9 +330,21 @@ extern "C" int tq_decode_attn_paged(const void* q, int dtype, int B, int Hq, int
                                                recent_len, sm_scale, parts, n_parts, n_split);
     TQ_CHECK_LAUNCH();
   }
+  if (!(stages & 4)) return TQ_OK;
   // without a tail the merge simply reads one part fewer
   merge_kernel<<<dim3((unsigned)(B * Hq)), dim3(d < 256 ? d : 256), 0, st>>>(parts, tail ? n_parts : n_split, n_parts, d,
                                                                             dtype, out);
   TQ_CHECK_LAUNCH();
   return TQ_OK;
+}
+
+extern "C" int tq_decode_attn_paged(const void* q, int dtype, int B, int Hq, int Hkv, const uint8_t* pool,
+                                    int64_t num_pages, const int32_t* block_table, int bt_stride,
+                                    const int32_t* seq_lens, float sm_scale, const tq_layer* layer,
+                                    const tq_page_layout* layout, const void* recent_k, const void* recent_v,
+                                    int recent_rows, int64_t rs_b, int64_t rs_r, int64_t rs_h,
+                                    const int32_t* recent_len, void* out, void* workspace, int n_split, void* stream) {
+  return tq_decode_attn_paged_stages(q, dtype, B, Hq, Hkv, pool, num_pages, block_table, bt_stride, seq_lens, sm_scale,
+                                     layer, layout, recent_k, recent_v, recent_rows, rs_b, rs_r, rs_h, recent_len, out,
+                                     workspace, n_split, 7, stream);
 }

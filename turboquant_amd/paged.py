@@ -118,11 +118,14 @@ class PagedKVPool:
                          scale: Optional[float] = None, recent_k: Optional[torch.Tensor] = None,
                          recent_v: Optional[torch.Tensor] = None, recent_len: Optional[torch.Tensor] = None,
                          n_split: Optional[int] = None, workspace: Optional[torch.Tensor] = None,
-                         out: Optional[torch.Tensor] = None, max_len: Optional[int] = None) -> torch.Tensor:
+                         out: Optional[torch.Tensor] = None, max_len: Optional[int] = None,
+                         stages: int = 7) -> torch.Tensor:
         """softmax(scale * [scores_hist ; q k_recent^T]) [v_hist ; v_recent] for one
         query token per sequence.  query (B, Hq, d);
         block_table (B, max_pages) or (max_pages,) shared; seq_lens (B,) int32;
-        recent_k / recent_v (B, R, H, d) exact tokens, recent_len (B,) valid rows."""
+        recent_k / recent_v (B, R, H, d) exact tokens, recent_len (B,) valid rows.
+        `stages` (bit 0 query rotation, bit 1 page kernel, bit 2 merge) exists for
+        timing the stages apart; 7 runs the whole thing."""
         _ffi.require_gpu(query, "query")
         B, Hq, d = query.shape
         if d != self.head_dim or Hq % self.num_kv_heads:
@@ -157,9 +160,9 @@ class PagedKVPool:
                 rl_ptr = recent_len.data_ptr()
         ly = self.quantizer._layer()
         with torch.cuda.device(self.device):
-            _ffi.check(_ffi.lib().tq_decode_attn_paged(
+            _ffi.check(_ffi.lib().tq_decode_attn_paged_stages(
                 query.data_ptr(), _ffi.dtype_tag(query.dtype), B, Hq, self.num_kv_heads, self.data.data_ptr(),
                 self.num_pages, bt.data_ptr(), bt_stride, seq_lens.data_ptr(), float(scale), C.byref(ly),
                 C.byref(self.layout), rk_ptr, rv_ptr, rows, rs[0], rs[1], rs[2], rl_ptr, out.data_ptr(),
-                workspace.data_ptr(), n_split, _ffi.stream_ptr(self.device)), "tq_decode_attn_paged")
+                workspace.data_ptr(), n_split, stages, _ffi.stream_ptr(self.device)), "tq_decode_attn_paged")
         return out
