@@ -64,17 +64,21 @@ typedef struct tq_layer {
 
 /* Geometry of one page = TQ_PAGE_TOKENS tokens of one KV head (new design; the
  * reference keeps python lists of chunk tensors, store.py:59-63).  Offsets are
- * in bytes from the start of the page.
- *   planes : key_bits bit-planes (MSE index bits high..low, then the QJL sign),
- *            each stored as [d/32 words][16 tokens] uint32; bit i of word j of
- *            token n is coordinate 32*j+i.
- *   norm   : 16 key norms in the input dtype (2 or 4 bytes) ; rnorm : 16 fp32 ||r||.
- *   vdata  : per channel a little-endian field of 16*value_bits bits, token n's
- *            code at bit value_bits*n ; channels consecutive.
- *   vscale / vzero : [d/group][16 tokens] in the input dtype.                 */
+ * in bytes from the start of the page; every section starts 16-byte aligned.
+ *   keys   : key_bits = mse_bits+1 bit-planes (index bits high..low, then the QJL
+ *            sign).  Word j of plane p of token n holds coordinates 32j..32j+31
+ *            (bit i = coordinate 32j+i).  With key_lane_major != 0 (d a multiple
+ *            of 128) the words are stored as [j%4][n][p][j/4], so that the
+ *            words one wavefront lane (token n, coordinate quarter j%4) consumes
+ *            are contiguous; otherwise as [p][j][n].
+ *   meta   : per token {float norm, float rnorm}: the key norm (a value of the
+ *            input dtype, widened losslessly) and ||r||.
+ *   vdata  : per channel c a little-endian field of 16*value_bits bits, token n's
+ *            code at bit value_bits*n; fields ordered [c%16][c/16].
+ *   vscale / vzero : [d/group][16 tokens] in the input dtype.                  */
 typedef struct tq_page_layout {
-  int32_t d, mse_bits, value_bits, group_size, dtype;
-  int32_t off_planes, off_norm, off_rnorm, off_vdata, off_vscale, off_vzero;
+  int32_t d, mse_bits, value_bits, group_size, dtype, key_lane_major;
+  int32_t off_keys, off_meta, off_vdata, off_vscale, off_vzero;
   int32_t page_bytes;      /* stride between (page, head) records, multiple of 128 */
 } tq_page_layout;
 

@@ -52,15 +52,16 @@ def test_argument_errors_are_reported_before_any_launch():
 
 
 @pytest.mark.parametrize("d,mb,vb,gs,dt,per_token", [
-    (128, 2, 4, 32, torch.bfloat16, 32 + 16 + 2 + 4 + 64 + 16),      # 134 B: fp32 residual norm
-    (256, 2, 2, 32, torch.bfloat16, 64 + 32 + 2 + 4 + 64 + 32),      # 198 B
-    (128, 2, 2, 32, torch.float16, 32 + 16 + 2 + 4 + 32 + 16),
+    (128, 2, 4, 32, torch.bfloat16, 32 + 16 + 4 + 4 + 64 + 16),      # 136 B: fp32 norm and residual norm
+    (256, 2, 2, 32, torch.bfloat16, 64 + 32 + 4 + 4 + 64 + 32),      # 200 B
+    (128, 2, 2, 32, torch.float16, 32 + 16 + 4 + 4 + 32 + 16),
     (128, 3, 4, 64, torch.float32, 48 + 16 + 4 + 4 + 64 + 16),
+    (64, 2, 2, 32, torch.bfloat16, 16 + 8 + 4 + 4 + 16 + 8),
 ])
 def test_page_layout_geometry(d, mb, vb, gs, dt, per_token):
     L = _ffi.make_page_layout(d, mb, vb, gs, dt)
-    assert L.off_planes == 0
-    offs = [L.off_planes, L.off_norm, L.off_rnorm, L.off_vdata, L.off_vscale, L.off_vzero]
+    assert L.off_keys == 0 and L.key_lane_major == (1 if d % 128 == 0 else 0)
+    offs = [L.off_keys, L.off_meta, L.off_vdata, L.off_vscale, L.off_vzero]
     assert offs == sorted(offs) and all(o % 16 == 0 for o in offs)
     used = L.off_vzero + (d // gs) * 16 * (4 if dt == torch.float32 else 2)
     assert used == 16 * per_token

@@ -41,8 +41,8 @@ class TqLayer(C.Structure):
 
 class TqPageLayout(C.Structure):
     _fields_ = [(n, C.c_int32) for n in (
-        "d", "mse_bits", "value_bits", "group_size", "dtype",
-        "off_planes", "off_norm", "off_rnorm", "off_vdata", "off_vscale", "off_vzero", "page_bytes")]
+        "d", "mse_bits", "value_bits", "group_size", "dtype", "key_lane_major",
+        "off_keys", "off_meta", "off_vdata", "off_vscale", "off_vzero", "page_bytes")]
 
 
 _vp, _i, _i64, _f = C.c_void_p, C.c_int, C.c_int64, C.c_float

@@ -101,13 +101,18 @@ __host__ __device__ __forceinline__ int idx_row_bytes(int d, int mse_bits) {
 
 // ---- page geometry -----------------------------------------------------------------
 
-// word j (32 coordinates) of plane p for token n
-__device__ __forceinline__ int plane_word_off(const tq_page_layout& L, int p, int j, int n) {
-  return L.off_planes + (((p * (L.d >> 5)) + j) * TQ_PAGE_TOKENS + n) * 4;
+// byte offset of word j (coordinates 32j..32j+31) of plane p of token n
+__host__ __device__ __forceinline__ int key_word_off(const tq_page_layout& L, int p, int j, int n) {
+  const int W = L.d >> 5, planes = L.mse_bits + 1;
+  if (L.key_lane_major) return L.off_keys + (((((j & 3) * TQ_PAGE_TOKENS + n) * planes + p) * (W >> 2)) + (j >> 2)) * 4;
+  return L.off_keys + ((p * W + j) * TQ_PAGE_TOKENS + n) * 4;
 }
 
-__device__ __forceinline__ const uint8_t* page_ptr(const uint8_t* pool, int64_t page, int H, int h, int page_bytes) {
-  return pool + (page * H + h) * (int64_t)page_bytes;
+// byte offset of the value field (16 * value_bits bits) of channel c
+__host__ __device__ __forceinline__ int vfield_off(const tq_page_layout& L, int c) {
+  return L.off_vdata + (((c & 15) * (L.d >> 4)) + (c >> 4)) * (L.value_bits * 2);
 }
+
+__host__ __device__ __forceinline__ int elem_bytes(int dtype) { return dtype == TQ_F32 ? 4 : 2; }
 
 }  // namespace tq

@@ -80,7 +80,7 @@ decode_pages_kernel(const float* __restrict__ q_rot, const float* __restrict__ q
     for (int g = 0; g < G_MAX; ++g) pm[g] = pq[g] = 0.0f;
     for (int w = kb; w < words; w += 4) {
       uint32_t pw[5];
-      for (int p = 0; p <= mb; ++p) pw[p] = *(const uint32_t*)(pg + plane_word_off(L, p, w, n));
+      for (int p = 0; p <= mb; ++p) pw[p] = *(const uint32_t*)(pg + key_word_off(L, p, w, n));
       for (int i = 0; i < 32; ++i) {
         unsigned id = 0;
         for (int p = 0; p < mb; ++p) id = (id << 1) | ((pw[p] >> i) & 1u);
@@ -97,8 +97,8 @@ decode_pages_kernel(const float* __restrict__ q_rot, const float* __restrict__ q
         }
       }
     }
-    const float nk = (n < n_valid) ? load_as_f32(pg + L.off_norm, n, L.dtype) : 0.0f;
-    const float rk = (n < n_valid) ? ly.qjl_scale * ((const float*)(pg + L.off_rnorm))[n] : 0.0f;
+    const float nk = (n < n_valid) ? ((const float*)(pg + L.off_meta))[2 * n] : 0.0f;
+    const float rk = (n < n_valid) ? ly.qjl_scale * ((const float*)(pg + L.off_meta))[2 * n + 1] : 0.0f;
 #pragma unroll
     for (int g = 0; g < G_MAX; ++g) {
       if (g < G) {
@@ -129,7 +129,7 @@ decode_pages_kernel(const float* __restrict__ q_rot, const float* __restrict__ q
     for (int c2 = 0; c2 < 12; ++c2) {
       if (c2 < cpl) {
         const int ch = lane + 64 * c2, grp = ch / L.group_size;
-        const uint32_t* field = (const uint32_t*)(pg + L.off_vdata) + ch * (VB / 2);
+        const uint32_t* field = (const uint32_t*)(pg + vfield_off(L, ch));
         uint32_t f0 = field[0], f1 = (VB == 4) ? field[1] : 0u;
         const int es = L.dtype == TQ_F32 ? 4 : 2;
         const uint8_t* sc_p = pg + L.off_vscale + grp * TQ_PAGE_TOKENS * es;
@@ -222,24 +222,44 @@ exact_tail_kernel(const void* __restrict__ q, int dtype, int Hq, int Hkv, int d,
   }
 }
 
-// n_parts partials are merged per row; consecutive rows are part_stride partials apart
-__global__ void merge_kernel(const float* __restrict__ parts, int n_parts, int part_stride, int d, int dtype,
-                             void* __restrict__ out) {
+// n_parts partials are merged per row; consecutive rows are part_stride partials apart.
+// One workgroup per row: the weights exp(m_s - M) are computed once into LDS, then
+// thread ch sums its channel over the parts (coalesced across threads).
+__global__ void __launch_bounds__(256)
+merge_kernel(const float* __restrict__ parts, int n_parts, int part_stride, int d, int dtype, void* __restrict__ out) {
+  extern __shared__ float s_w[];                 // [n_parts] weights, then [8] scratch
   const int64_t row = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const float* p = parts + row * part_stride * (int64_t)(d + 2);
+  float* scratch = s_w + n_parts;
   float mm = NEG_BIG;
-  for (int s = 0; s < n_parts; ++s) mm = fmaxf(mm, p[(int64_t)s * (d + 2)]);
-  for (int ch = threadIdx.x; ch < d; ch += blockDim.x) {
-    float ll = 0.0f, aa = 0.0f;
+  for (int s = tid; s < n_parts; s += blockDim.x) {
+    const float* r = p + (int64_t)s * (d + 2);
+    if (r[1] > 0.0f) mm = fmaxf(mm, r[0]);
+  }
+  mm = wave_max(mm);
+  if (lane == 0) scratch[wave] = mm;
+  __syncthreads();
+  mm = fmaxf(fmaxf(scratch[0], scratch[1]), fmaxf(scratch[2], scratch[3]));
+  float ll = 0.0f;
+  for (int s = tid; s < n_parts; s += blockDim.x) {
+    const float* r = p + (int64_t)s * (d + 2);
+    const float w = r[1] > 0.0f ? __expf(r[0] - mm) : 0.0f;
+    s_w[s] = w;
+    ll += w * r[1];
+  }
+  ll = wave_sum(ll);
+  if (lane == 0) scratch[4 + wave] = ll;
+  __syncthreads();
+  ll = scratch[4] + scratch[5] + scratch[6] + scratch[7];
+  const float inv = ll > 0.0f ? 1.0f / ll : 0.0f;
+  for (int ch = tid; ch < d; ch += blockDim.x) {
+    float aa = 0.0f;
     for (int s = 0; s < n_parts; ++s) {
-      const float* r = p + (int64_t)s * (d + 2);
-      if (r[1] > 0.0f) {
-        float w = __expf(r[0] - mm);
-        ll += w * r[1];
-        aa += w * r[2 + ch];
-      }
+      const float w = s_w[s];
+      if (w != 0.0f) aa = fmaf(w, p[(int64_t)s * (d + 2) + 2 + ch], aa);
     }
-    store_from_f32(out, row * d + ch, ll > 0.0f ? aa / ll : 0.0f, dtype);
+    store_from_f32(out, row * d + ch, aa * inv, dtype);
   }
 }
 
@@ -247,15 +267,21 @@ __global__ void merge_kernel(const float* __restrict__ parts, int n_parts, int p
 
 using namespace tq;
 
-extern "C" int tq_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* layer, float* q_rot,
-                               float* q_sk, void* stream);
+namespace tq {
+int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* layer, float* q_rot, float* q_sk,
+                        float* q_stat, hipStream_t st);
+int launch_decode_mfma(const float* q_rot, const float* q_sk, const float* q_stat, int B, int Hq, int Hkv,
+                       const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
+                       float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts,
+                       int n_split, hipStream_t st);
+}  // namespace tq
 
 static size_t parts_floats(int B, int Hq, int d, int n_parts) { return (size_t)B * Hq * n_parts * (d + 2); }
 
 extern "C" size_t tq_decode_workspace_bytes(int B, int Hq, int d, int n_split) {
   if (B <= 0 || Hq <= 0 || d <= 0 || n_split <= 0) return 0;
-  // partials for n_split history splits + 1 exact tail, then q_rot and q_sk
-  return (parts_floats(B, Hq, d, n_split + 1) + (size_t)2 * B * Hq * d) * sizeof(float);
+  // partials for n_split history splits + 1 exact tail, then q_rot, q_sk and 4 statistics per query row
+  return (parts_floats(B, Hq, d, n_split + 1) + (size_t)2 * B * Hq * d + (size_t)4 * B * Hq) * sizeof(float);
 }
 
 extern "C" int tq_decode_merge(const float* parts, int64_t rows, int n_parts, int d, int dtype, void* out,
@@ -263,8 +289,8 @@ extern "C" int tq_decode_merge(const float* parts, int64_t rows, int n_parts, in
   if (!parts || !out) return TQ_ENULL;
   if (rows < 0 || n_parts <= 0 || d <= 0 || dtype < TQ_F32 || dtype > TQ_BF16) return TQ_EINVAL;
   if (rows == 0) return TQ_OK;
-  merge_kernel<<<dim3((unsigned)rows), dim3(d < 256 ? d : 256), 0, (hipStream_t)stream>>>(parts, n_parts, n_parts, d, dtype,
-                                                                                          out);
+  merge_kernel<<<dim3((unsigned)rows), dim3(256), (n_parts + 8) * sizeof(float), (hipStream_t)stream>>>(
+      parts, n_parts, n_parts, d, dtype, out);
   TQ_CHECK_LAUNCH();
   return TQ_OK;
 }
@@ -291,9 +317,12 @@ extern "C" int tq_decode_attn_paged_stages(const void* q, int dtype, int B, int 
   float* parts = (float*)workspace;
   float* q_rot = parts + parts_floats(B, Hq, d, n_parts);
   float* q_sk = q_rot + (size_t)B * Hq * d;
+  float* q_stat = q_sk + (size_t)B * Hq * d;
 
   if (stages & 1) {
-    int rc = tq_rotate_query(q, dtype, (int64_t)B * Hq, layer, q_rot, q_sk, stream);
+    if (!layer->Pi || !layer->PiT || !layer->S || !layer->ST || !layer->centroids) return TQ_ENULL;
+    if (dtype < TQ_F32 || dtype > TQ_BF16) return TQ_EINVAL;
+    int rc = launch_rotate_query(q, dtype, (int64_t)B * Hq, layer, q_rot, q_sk, q_stat, st);
     if (rc) return rc;
   }
   if (!(stages & 6)) return TQ_OK;
@@ -301,7 +330,12 @@ extern "C" int tq_decode_attn_paged_stages(const void* q, int dtype, int B, int 
   const int qsz = d * G + (d >> 5) * 4;
   size_t smem = (size_t)(2 * qsz + 16 + DEC_WAVES * G * 16 + DEC_WAVES * G * (d + 2)) * sizeof(float);
   dim3 grid(n_split, Hkv, B), block(DEC_WAVES * 64);
-  if (stages & 2) {
+  int mf = TQ_EUNSUPPORTED;
+  if (stages & 2)
+    mf = launch_decode_mfma(q_rot, q_sk, q_stat, B, Hq, Hkv, pool, block_table, bt_stride, seq_lens, sm_scale, *layer,
+                            *layout, parts, n_parts, n_split, st);
+  if (mf > 0) return mf;
+  if ((stages & 2) && mf == TQ_EUNSUPPORTED) {      // no matrix-core kernel for this shape: general kernel
 #define TQ_LAUNCH_DEC(VB)                                                                                 \
   {                                                                                                       \
     auto kern = decode_pages_kernel<VB>;                                                                  \
@@ -332,8 +366,8 @@ extern "C" int tq_decode_attn_paged_stages(const void* q, int dtype, int B, int 
   }
   if (!(stages & 4)) return TQ_OK;
   // without a tail the merge simply reads one part fewer
-  merge_kernel<<<dim3((unsigned)(B * Hq)), dim3(d < 256 ? d : 256), 0, st>>>(parts, tail ? n_parts : n_split, n_parts, d,
-                                                                            dtype, out);
+  merge_kernel<<<dim3((unsigned)(B * Hq)), dim3(256), (n_parts + 8) * sizeof(float), st>>>(
+      parts, tail ? n_parts : n_split, n_parts, d, dtype, out);
   TQ_CHECK_LAUNCH();
   return TQ_OK;
 }

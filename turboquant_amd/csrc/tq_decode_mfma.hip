@@ -1,0 +1,559 @@
+// Page-streaming decode kernel on the matrix cores (gfx950, bf16 MFMA 16x16x32).
+//
+// The packed bits feed the matrix cores almost directly:
+//
+//  * keys.  A Lloyd-Max centroid is an affine function of the parities of subsets
+//    of its index bits (Walsh expansion; for the symmetric codebooks simply of
+//    the individual index bits), so  sum_j q_rot[j] c[idx_j]  is a sum of
+//    "query . bit-plane" contractions, exactly like the QJL term
+//    sum_j q_sk[j] (2 bit_j - 1).  A bf16 whose only set bit is bit p (7..14) is
+//    the power of two 2^(2^(p-7)-127); one AND per pair of coordinates turns a
+//    32-bit plane word into MFMA B operands, and the query operand carries the
+//    inverse power of two, so the products are exact.  The query is split into
+//    bf16 hi + lo parts that occupy two rows of the 16-row A operand, which
+//    gives fp32-class scores.
+//  * values.  A code is OR-ed into the top mantissa bits of bf16(2^vb), i.e.
+//    B = 2^vb + code exactly; the softmax weight times the group scale is the A
+//    operand, and a second MFMA with B = -2^vb removes the offset with the very
+//    same A.  The zero points go through one more MFMA (weights x zeros).
+//
+// One wavefront owns 64 tokens (4 pages) per iteration: lane (n, kb) = lane%16,
+// lane/16 is token n and coordinate quarter kb in the score stage, and (row,
+// page kb) in the value stage.  The key words of the next 64 tokens are
+// requested before the current ones are consumed; the value words of the current
+// 64 tokens are requested before its score stage.  Workgroups have 4 wavefronts;
+// WPS of them share a SIMD so that one wavefront's dependency stalls are filled
+// by another.
+
+#include <type_traits>
+
+#include "tq_common.h"
+
+namespace tq {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int MF_WAVES = 4;
+constexpr int BLK_TOK = 64;              // tokens per wavefront iteration
+constexpr float MF_NEG = -1.0e30f;
+constexpr int P_STRIDE = 20;             // floats per row of the LDS softmax-weight tile (16 + skew)
+constexpr int WAVE_LDS_FLOATS = 4 * 16 * P_STRIDE + 16 + 4 * 16 * 8;
+
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  f32x2 f = {lo, hi};
+  bf16x2 r = __builtin_convertvector(f, bf16x2);   // v_cvt_pk_bf16_f32, round to nearest even
+  uint32_t u;
+  __builtin_memcpy(&u, &r, 4);
+  return u;
+}
+__device__ __forceinline__ float bf16_round(float v) { return __uint_as_float(pack_bf16(v, 0.0f) << 16); }
+__device__ __forceinline__ f32x4 mfma(const u32x4& a, const u32x4& b, f32x4 c) {
+  bf16x8 av, bv;
+  __builtin_memcpy(&av, &a, 16);
+  __builtin_memcpy(&bv, &b, 16);
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, bv, c, 0, 0, 0);
+}
+// keeps a loop-invariant constant in a vector register, so that three-operand
+// bit instructions do not need two scalar operands
+__device__ __forceinline__ uint32_t in_vgpr(uint32_t v) {
+  asm volatile("" : "+v"(v));
+  return v;
+}
+
+template <int CTRL>
+__device__ __forceinline__ float dpp(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+// all-reduce over the 16 lanes of a DPP row (quad swaps, half-row mirror, row mirror)
+__device__ __forceinline__ float row_max16(float v) {
+  v = fmaxf(v, dpp<0xB1>(v));
+  v = fmaxf(v, dpp<0x4E>(v));
+  v = fmaxf(v, dpp<0x141>(v));
+  v = fmaxf(v, dpp<0x140>(v));
+  return v;
+}
+__device__ __forceinline__ float row_sum16(float v) {
+  v += dpp<0xB1>(v);
+  v += dpp<0x4E>(v);
+  v += dpp<0x141>(v);
+  v += dpp<0x140>(v);
+  return v;
+}
+
+// bit position p (inside each 16-bit half) that coordinate-pair `bit` of a plane
+// word occupies in the B operand of MFMA u = bit/4, register r = bit%4; the value
+// of that single-bit bf16 is 2^(2^(p-7) - 127)
+__host__ __device__ constexpr int bit_slot(int bit) { return bit <= 6 ? bit + 7 : (bit == 15 ? 14 : bit); }
+__host__ __device__ constexpr int slot_exponent(int p) { return (1 << (p - 7)) - 127; }
+
+// 32 coordinates of one plane word -> 16 dwords = B operands of 4 MFMAs
+__device__ __forceinline__ void expand_plane_word(uint32_t x, uint32_t (&b)[16]) {
+  const uint32_t xs = x << 7, xr = x >> 1;
+#pragma unroll
+  for (int bit = 0; bit < 16; ++bit) {
+    const uint32_t src = bit <= 6 ? xs : (bit == 15 ? xr : x);
+    b[bit] = src & (0x00010001u << bit_slot(bit));
+  }
+}
+
+// token held by element (r, h) of MFMA half u of the value stage
+template <int VB>
+__device__ __forceinline__ constexpr int v_token(int u, int r, int h) {
+  return VB == 2 ? 4 * u + r + 8 * h : 8 * u + r + 4 * h;
+}
+
+// D in {128, 256}; MB stored index bits; NX extra (multi-bit) Walsh terms; VB value bits;
+// GS value group size; WPS wavefronts per SIMD the register budget is sized for.
+template <int D, int MB, int NX, int VB, int GS, int WPS>
+__global__ void __launch_bounds__(MF_WAVES * 64, WPS)
+decode_mfma_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_sk, const float* __restrict__ q_stat,
+                   int Hq, int Hkv, const uint8_t* __restrict__ pool, const int32_t* __restrict__ block_table,
+                   int bt_stride, const int32_t* __restrict__ seq_lens, float sm_scale, tq_layer ly, tq_page_layout L,
+                   float* __restrict__ parts, int n_parts, int n_split) {
+  constexpr int WPL = D / 128;                // plane words per lane per plane per page
+  constexpr int NTP = MB + NX + 1;            // term planes fed to the MFMA (stored + XOR terms + sign)
+  constexpr int NKW = (MB + 1) * WPL;         // key dwords per lane per page
+  constexpr int CT = D / 16;                  // channel tiles
+  constexpr int VW = CT * VB / 2;             // value dwords per lane per block
+  constexpr int NG = D / GS, CTG = GS / 16;   // groups, channel tiles per group
+  constexpr int PIECES = 2 * NG;              // 16-byte pieces of scales per page
+  const int G = Hq / Hkv;                     // <= 8
+  const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 15, kb = lane >> 4;    // score stage: token / coordinate quarter; value stage: row / page
+  const float LOG2E = 1.4426950408889634f;
+
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  float* s_p = (float*)smem_raw + wave * WAVE_LDS_FLOATS;   // [4 pages][16 rows][P_STRIDE]
+  float* s_alpha = s_p + 4 * 16 * P_STRIDE;                 // [16]
+  uint32_t* s_scale = (uint32_t*)(s_alpha + 16);            // [4 pages][NG][8 dwords]
+  float* s_red = (float*)smem_raw;                          // after the loop: [MF_WAVES][G][D + 2]
+
+  float cmax = 0.0f;
+  for (int t = 0; t < ly.n_terms; ++t) cmax = fmaxf(cmax, fabsf(ly.term_coef[t]));
+
+  // ---------------------------------------------------------------- A operands of the score stage
+  // lane (row = n, kb): row -> (head g = row/2, part = row%2: bf16 hi / lo of the query)
+  u32x4 qa[NTP][WPL][4];
+  {
+    const int g = n >> 1, part = n & 1;
+    const bool live = g < G;
+    const int64_t qrow = (int64_t)b * Hq + h * G + (live ? g : 0);
+    const float* rot = q_rot + qrow * D;
+    const float* sk = q_sk + qrow * D;
+    const float m1 = fmaxf(q_stat[qrow * 4 + 0] * cmax, 1e-30f), m2 = fmaxf(q_stat[qrow * 4 + 1], 1e-30f);
+#pragma unroll
+    for (int tp = 0; tp < NTP; ++tp) {
+      // coefficient of this term plane: stored plane p <-> index bit MB-1-p; extra terms in table order
+      float coef = 0.0f;
+      if (tp < MB) {
+        for (int t = 0; t < ly.n_terms; ++t)
+          if (ly.term_mask[t] == (1 << (MB - 1 - tp))) coef = ly.term_coef[t];
+      } else if (tp < MB + NX) {
+        int seen = 0;
+        for (int t = 0; t < ly.n_terms; ++t) {
+          if (__builtin_popcount(ly.term_mask[t]) > 1) {
+            if (seen == tp - MB) coef = ly.term_coef[t];
+            ++seen;
+          }
+        }
+      }
+      const bool is_sign = tp == NTP - 1;
+      const float* src = is_sign ? sk : rot;
+      const float mul = live ? (is_sign ? 1.0f / m2 : coef / m1) : 0.0f;
+#pragma unroll
+      for (int i = 0; i < WPL; ++i) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          u32x4 reg;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int bit = 4 * u + r;
+            const float sc = __builtin_ldexpf(1.0f, -slot_exponent(bit_slot(bit)));
+            const int c0 = 32 * (4 * i + kb) + bit;
+            float v0 = src[c0] * mul * sc, v1 = src[c0 + 16] * mul * sc;
+            if (part) { v0 -= bf16_round(v0); v1 -= bf16_round(v1); }
+            reg[r] = pack_bf16(v0, v1);
+          }
+          qa[tp][i][u] = reg;
+        }
+      }
+    }
+  }
+  // score constants of the two heads this lane sees in the MFMA output (rows 4kb..4kb+3 = heads 2kb, 2kb+1)
+  float am[2], bm[2], aq[2], bq[2];
+  int xplanes[NX > 0 ? NX : 1];                 // which stored planes each extra term XORs
+  {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int g = 2 * kb + j;
+      const bool live = g < G;
+      const int64_t qrow = (int64_t)b * Hq + h * G + (live ? g : 0);
+      const float m1 = fmaxf(q_stat[qrow * 4 + 0] * cmax, 1e-30f), m2 = fmaxf(q_stat[qrow * 4 + 1], 1e-30f);
+      const float k = live ? sm_scale * LOG2E : 0.0f;
+      am[j] = k * m1;
+      bm[j] = k * ly.term_const * q_stat[qrow * 4 + 2];
+      aq[j] = 2.0f * k * ly.qjl_scale * m2;
+      bq[j] = -k * ly.qjl_scale * q_stat[qrow * 4 + 3];
+    }
+    int seen = 0;
+    for (int t = 0; t < ly.n_terms; ++t) {
+      if (__builtin_popcount(ly.term_mask[t]) > 1 && seen < NX) {
+        int pl = 0;
+        for (int k2 = 0; k2 < MB; ++k2)
+          if (ly.term_mask[t] & (1 << k2)) pl |= 1 << (MB - 1 - k2);
+        xplanes[seen++] = __builtin_amdgcn_readfirstlane(pl);
+      }
+    }
+  }
+
+  // ---------------------------------------------------------------- work range (all scalar)
+  const int seq_len = seq_lens[b];
+  const int n_pages = (seq_len + TQ_PAGE_TOKENS - 1) / TQ_PAGE_TOKENS;
+  const int n_blocks = (seq_len + BLK_TOK - 1) / BLK_TOK;
+  const int per_split = (n_blocks + n_split - 1) / n_split;
+  const int blk_begin = split * per_split;
+  const int blk_end = min(n_blocks, blk_begin + per_split);
+  const int32_t* bt = block_table + (int64_t)b * bt_stride;
+  const uint8_t* pool_h = pool + (int64_t)h * L.page_bytes;
+  const int64_t page_stride = (int64_t)Hkv * L.page_bytes;
+  const int off_keys = L.off_keys + lane * (NKW * 4), off_meta = L.off_meta + n * 8;
+  const int off_v = L.off_vdata + n * (VW * 4), off_zero = L.off_vzero + n * 32;
+  const int off_scale = L.off_vscale + (lane % PIECES) * 16;
+
+  f32x4 acc[CT];
+#pragma unroll
+  for (int c = 0; c < CT; ++c) acc[c] = f32x4{0, 0, 0, 0};
+  f32x4 zacc = {0, 0, 0, 0};
+  float m_run[2] = {MF_NEG, MF_NEG}, l_run[2] = {0.0f, 0.0f};
+
+  struct KeyRegs { uint32_t key[4][NKW]; f32x2 meta[4]; };
+  struct ValRegs { uint32_t v[VW]; u32x4 zero[2]; u32x4 scale; };
+
+  // page ids of block `blk` -> 4 scalars, clamped into the sequence's pages
+  auto page_ids = [&](int blk, int (&pid)[4]) {
+#pragma unroll
+    for (int pg = 0; pg < 4; ++pg) pid[pg] = bt[min(4 * blk + pg, n_pages - 1)];
+  };
+  auto load_keys = [&](const int (&pid)[4], KeyRegs& R) {
+#pragma unroll
+    for (int pg = 0; pg < 4; ++pg) {
+      const uint8_t* base = pool_h + pid[pg] * page_stride;
+      const uint32_t* kp = (const uint32_t*)(base + off_keys);
+#pragma unroll
+      for (int w = 0; w < NKW; ++w) R.key[pg][w] = kp[w];
+      R.meta[pg] = *(const f32x2*)(base + off_meta);
+    }
+  };
+  auto load_vals = [&](const int (&pid)[4], ValRegs& R) {
+    const int my_pid = kb == 0 ? pid[0] : (kb == 1 ? pid[1] : (kb == 2 ? pid[2] : pid[3]));
+    const uint8_t* vbase = pool_h + my_pid * page_stride;
+    const uint32_t* vp = (const uint32_t*)(vbase + off_v);
+#pragma unroll
+    for (int w = 0; w < VW; ++w) R.v[w] = vp[w];
+    if (n < NG) {
+      const u32x4* zp = (const u32x4*)(vbase + off_zero);
+      R.zero[0] = zp[0];
+      R.zero[1] = zp[1];
+    } else {
+      R.zero[0] = u32x4{0, 0, 0, 0};
+      R.zero[1] = u32x4{0, 0, 0, 0};
+    }
+    if (lane < 4 * PIECES) {
+      const int spg = lane / PIECES;
+      const int spid = spg == 0 ? pid[0] : (spg == 1 ? pid[1] : (spg == 2 ? pid[2] : pid[3]));
+      R.scale = *(const u32x4*)(pool_h + spid * page_stride + off_scale);
+    } else {
+      R.scale = u32x4{0, 0, 0, 0};
+    }
+  };
+
+  const uint32_t base_pat = in_vgpr(VB == 2 ? 0x40804080u : 0x41804180u);   // bf16 pairs of 2^VB
+  const uint32_t code_mask = in_vgpr(VB == 2 ? 0x00600060u : 0x00780078u);  // top mantissa bits
+  const uint32_t neg_pat = VB == 2 ? 0xC080C080u : 0xC180C180u;             // bf16 pairs of -2^VB
+  const u32x4 neg_base = {neg_pat, neg_pat, neg_pat, neg_pat};
+
+  // ---------------------------------------------------------------- one block of 64 tokens
+  auto compute = [&](int blk, const KeyRegs& K, const ValRegs& V, auto partial_tag) {
+    constexpr bool PARTIAL = decltype(partial_tag)::value;
+    // scales -> LDS ([page][group][16 tokens] bf16, as in the page)
+    if (lane < 4 * PIECES) *(u32x4*)(s_scale + lane * 4) = V.scale;
+    // ---- scores of the 4 pages
+    float s2[2][4];
+#pragma unroll
+    for (int pg = 0; pg < 4; ++pg) {
+      f32x4 dm = {0, 0, 0, 0}, dq = {0, 0, 0, 0};
+#pragma unroll
+      for (int i = 0; i < WPL; ++i) {
+#pragma unroll
+        for (int tp = 0; tp < NTP; ++tp) {
+          uint32_t x;
+          if (tp < MB) x = K.key[pg][tp * WPL + i];
+          else if (tp == NTP - 1) x = K.key[pg][MB * WPL + i];
+          else {
+            x = 0;
+#pragma unroll
+            for (int p = 0; p < MB; ++p) x ^= ((xplanes[tp - MB] >> p) & 1) ? K.key[pg][p * WPL + i] : 0u;
+          }
+          uint32_t bb[16];
+          expand_plane_word(x, bb);
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            u32x4 bv = {bb[4 * u], bb[4 * u + 1], bb[4 * u + 2], bb[4 * u + 3]};
+            if (tp == NTP - 1) dq = mfma(qa[tp][i][u], bv, dq);
+            else dm = mfma(qa[tp][i][u], bv, dm);
+          }
+        }
+      }
+      const float nk = K.meta[pg][0], rk = K.meta[pg][1];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const float vm = dm[2 * j] + dm[2 * j + 1], vq = dq[2 * j] + dq[2 * j + 1];
+        float s = fmaf(nk, fmaf(am[j], vm, bm[j]), rk * fmaf(aq[j], vq, bq[j]));
+        if (PARTIAL && (blk * BLK_TOK + pg * 16 + n >= seq_len)) s = MF_NEG;
+        s2[j][pg] = s;
+      }
+    }
+    // ---- online softmax (log2 domain); every lane of a 16-lane row ends with the same maximum
+    float alpha[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      float mx = fmaxf(fmaxf(s2[j][0], s2[j][1]), fmaxf(s2[j][2], s2[j][3]));
+      mx = row_max16(mx);
+      const float m_new = fmaxf(m_run[j], mx);
+      alpha[j] = __builtin_amdgcn_exp2f(m_run[j] - m_new);
+      m_run[j] = m_new;
+      float psum = 0.0f;
+#pragma unroll
+      for (int pg = 0; pg < 4; ++pg) {
+        const float p = __builtin_amdgcn_exp2f(s2[j][pg] - m_new);
+        psum += p;
+        s_p[(pg * 16 + 2 * kb + j) * P_STRIDE + n] = p;
+      }
+      l_run[j] = fmaf(l_run[j], alpha[j], psum);
+    }
+    const bool rescale = __builtin_amdgcn_ballot_w64(alpha[0] != 1.0f || alpha[1] != 1.0f) != 0;
+    if (rescale && n == 0) { s_alpha[2 * kb] = alpha[0]; s_alpha[2 * kb + 1] = alpha[1]; }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    if (rescale) {
+      const f32x4 a4 = *(const f32x4*)(s_alpha + 4 * kb);      // accumulator rows 4kb..4kb+3
+#pragma unroll
+      for (int c = 0; c < CT; ++c) acc[c] *= a4;
+      zacc *= a4;
+    }
+    // ---- value stage: lane = (row g = n, page kb)
+    float pr[16];
+    {
+      const f32x4* pp = (const f32x4*)(s_p + (kb * 16 + n) * P_STRIDE);
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        f32x4 t = pp[q4];
+        pr[4 * q4] = t[0]; pr[4 * q4 + 1] = t[1]; pr[4 * q4 + 2] = t[2]; pr[4 * q4 + 3] = t[3];
+      }
+    }
+    // validity of this lane's page tokens (last block only): bit t set = token t of page kb exists
+    uint32_t keep[8];
+    if (PARTIAL) {
+      const int nv = min(max(seq_len - (blk * BLK_TOK + kb * 16), 0), 16);
+      const uint32_t tokmask = (1u << nv) - 1u;
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        keep[i] = ((tokmask >> (2 * i)) & 1u ? 0x0000ffffu : 0u) | ((tokmask >> (2 * i + 1)) & 1u ? 0xffff0000u : 0u);
+    }
+    // zero points: weights (natural token order) x zeros
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      u32x4 ap, bz = V.zero[u];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        ap[r] = pack_bf16(pr[8 * u + 2 * r], pr[8 * u + 2 * r + 1]);
+        if (PARTIAL) bz[r] &= keep[4 * u + r];
+      }
+      zacc = mfma(ap, bz, zacc);
+    }
+#pragma unroll
+    for (int grp = 0; grp < NG; ++grp) {
+      // w = weight * scale for the 16 tokens of page kb, then the two A operands in the value token order
+      uint32_t sc[8];
+      {
+        const u32x4* sp = (const u32x4*)(s_scale + (kb * NG + grp) * 8);
+        const u32x4 s0 = sp[0], s1 = sp[1];
+        sc[0] = s0[0]; sc[1] = s0[1]; sc[2] = s0[2]; sc[3] = s0[3];
+        sc[4] = s1[0]; sc[5] = s1[1]; sc[6] = s1[2]; sc[7] = s1[3];
+      }
+      float w[16];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        uint32_t sd = sc[i];
+        if (PARTIAL) sd &= keep[i];
+        w[2 * i] = pr[2 * i] * __uint_as_float(sd << 16);
+        w[2 * i + 1] = pr[2 * i + 1] * __uint_as_float(sd & 0xffff0000u);
+      }
+      u32x4 aw[2];
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) aw[u][r] = pack_bf16(w[v_token<VB>(u, r, 0)], w[v_token<VB>(u, r, 1)]);
+#pragma unroll
+      for (int cc = 0; cc < CTG; ++cc) {
+        const int c = grp * CTG + cc;
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          u32x4 bc;
+          if (VB == 2) {
+            const uint32_t x = V.v[c];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const int f = 4 * u + r, sh = 5 - 2 * f;
+              const uint32_t y = sh >= 0 ? (x << sh) : (x >> (-sh));
+              bc[r] = (y & code_mask) | base_pat;
+            }
+          } else {
+            const uint32_t x = V.v[2 * c + u];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const int sh = 3 - 4 * r;
+              const uint32_t y = sh >= 0 ? (x << sh) : (x >> (-sh));
+              bc[r] = (y & code_mask) | base_pat;
+            }
+          }
+          acc[c] = mfma(aw[u], bc, acc[c]);
+          acc[c] = mfma(aw[u], neg_base, acc[c]);
+        }
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+  };
+
+  // ---------------------------------------------------------------- pipeline over this wave's blocks
+  {
+    KeyRegs KA, KB;
+    ValRegs VR;
+    int pid_cur[4], pid_nxt[4];
+    int blk = blk_begin + wave;
+    if (blk < blk_end) {
+      page_ids(blk, pid_cur);
+      load_keys(pid_cur, KA);
+    }
+    while (blk < blk_end) {
+      // even step: current keys in KA
+      {
+        const int nxt = blk + MF_WAVES;
+        load_vals(pid_cur, VR);
+        if (nxt < blk_end) { page_ids(nxt, pid_nxt); load_keys(pid_nxt, KB); }
+        if ((blk + 1) * BLK_TOK > seq_len) compute(blk, KA, VR, std::true_type{});
+        else compute(blk, KA, VR, std::false_type{});
+        blk = nxt;
+      }
+      if (blk >= blk_end) break;
+      // odd step: current keys in KB
+      {
+        const int nxt = blk + MF_WAVES;
+        load_vals(pid_nxt, VR);
+        if (nxt < blk_end) { page_ids(nxt, pid_cur); load_keys(pid_cur, KA); }
+        if ((blk + 1) * BLK_TOK > seq_len) compute(blk, KB, VR, std::true_type{});
+        else compute(blk, KB, VR, std::false_type{});
+        blk = nxt;
+      }
+    }
+  }
+
+  // ---------------------------------------------------------------- merge the 4 waves, write the partial
+  __syncthreads();      // every wave is done with its private LDS region
+  float* s_z = s_red + MF_WAVES * G * (D + 2);                 // [MF_WAVES][16 rows][16 groups]
+#pragma unroll
+  for (int i = 0; i < 4; ++i) s_z[(wave * 16 + 4 * kb + i) * 16 + n] = zacc[i];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const float lsum = row_sum16(l_run[j]);
+    const int g = 2 * kb + j;
+    if (n == 0 && g < G) {
+      float* r = s_red + (wave * G + g) * (D + 2);
+      r[0] = m_run[j] * 0.6931471805599453f;     // back to the natural-log domain of the partials
+      r[1] = lsum;
+    }
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+  for (int c = 0; c < CT; ++c) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int g = 4 * kb + i;
+      if (g < G) {
+        const float z = s_z[(wave * 16 + g) * 16 + c / CTG];
+        s_red[(wave * G + g) * (D + 2) + 2 + 16 * c + n] = acc[c][i] + z;
+      }
+    }
+  }
+  __syncthreads();
+  for (int o = tid; o < G * D; o += blockDim.x) {
+    const int g = o / D, ch = o - g * D;
+    float mm = MF_NEG;
+    for (int w = 0; w < MF_WAVES; ++w) mm = fmaxf(mm, s_red[(w * G + g) * (D + 2)]);
+    float ll = 0.0f, aa = 0.0f;
+    for (int w = 0; w < MF_WAVES; ++w) {
+      const float* r = s_red + (w * G + g) * (D + 2);
+      const float wgt = __expf(r[0] - mm);
+      ll += wgt * r[1];
+      aa += wgt * r[2 + ch];
+    }
+    float* out = parts + (((int64_t)b * Hq + h * G + g) * n_parts + split) * (D + 2);
+    if (ch == 0) { out[0] = mm; out[1] = ll; }
+    out[2 + ch] = aa;
+  }
+}
+
+template <int D, int MB, int NX, int VB, int GS, int WPS>
+static int launch_one(const float* q_rot, const float* q_sk, const float* q_stat, int B, int Hq, int Hkv,
+                      const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
+                      float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts, int n_split,
+                      hipStream_t st) {
+  const int G = Hq / Hkv;
+  size_t per_wave = (size_t)WAVE_LDS_FLOATS * sizeof(float);
+  size_t merge = (size_t)(MF_WAVES * G * (D + 2) + MF_WAVES * 16 * 16) * sizeof(float);
+  size_t smem = per_wave * MF_WAVES > merge ? per_wave * MF_WAVES : merge;
+  auto kern = decode_mfma_kernel<D, MB, NX, VB, GS, WPS>;
+  if (smem > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) return (int)e;
+  }
+  kern<<<dim3(n_split, Hkv, B), dim3(MF_WAVES * 64), smem, st>>>(q_rot, q_sk, q_stat, Hq, Hkv, pool, block_table,
+                                                                 bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts,
+                                                                 n_split);
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? TQ_OK : (int)e;
+}
+
+// Returns TQ_EUNSUPPORTED when the shape has no matrix-core kernel; the caller then
+// uses the general vector-ALU kernel.
+int launch_decode_mfma(const float* q_rot, const float* q_sk, const float* q_stat, int B, int Hq, int Hkv,
+                       const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
+                       float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts,
+                       int n_split, hipStream_t st) {
+  const int G = Hq / Hkv, d = ly.d, mb = ly.mse_bits, vb = L.value_bits, gs = L.group_size;
+  if (G > 8 || L.dtype != TQ_BF16 || !L.key_lane_major) return TQ_EUNSUPPORTED;
+  int nx = 0;
+  for (int t = 0; t < ly.n_terms; ++t)
+    if (__builtin_popcount(ly.term_mask[t]) > 1) ++nx;
+#define TQ_TRY(D_, MB_, NX_, VB_, GS_, WPS_)                                                                    \
+  if (d == D_ && mb == MB_ && nx == NX_ && vb == VB_ && gs == GS_)                                              \
+    return launch_one<D_, MB_, NX_, VB_, GS_, WPS_>(q_rot, q_sk, q_stat, B, Hq, Hkv, pool, block_table, bt_stride, \
+                                                    seq_lens, sm_scale, ly, L, parts, n_parts, n_split, st);
+  TQ_TRY(128, 2, 0, 2, 32, 2) TQ_TRY(128, 2, 0, 4, 32, 2) TQ_TRY(256, 2, 0, 2, 32, 1) TQ_TRY(256, 2, 0, 4, 32, 1)
+  TQ_TRY(128, 1, 0, 2, 32, 2) TQ_TRY(128, 1, 0, 4, 32, 2) TQ_TRY(256, 1, 0, 2, 32, 1) TQ_TRY(256, 1, 0, 4, 32, 1)
+  TQ_TRY(128, 3, 1, 2, 32, 1) TQ_TRY(128, 3, 1, 4, 32, 1)
+  TQ_TRY(128, 2, 0, 2, 64, 2) TQ_TRY(128, 2, 0, 4, 64, 2) TQ_TRY(256, 2, 0, 2, 64, 1) TQ_TRY(256, 2, 0, 4, 64, 1)
+#undef TQ_TRY
+  return TQ_EUNSUPPORTED;
+}
+
+}  // namespace tq

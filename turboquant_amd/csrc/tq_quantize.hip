@@ -274,11 +274,11 @@ key_tile_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
       } else {
         for (int i = 0; i < 32; ++i) bits |= (uint32_t)ssgn[n * d + w * 32 + i] << i;
       }
-      *(uint32_t*)(pg + plane_word_off(L, p, w, n)) = bits;
+      *(uint32_t*)(pg + key_word_off(L, p, w, n)) = bits;
     }
     if (j < TILE && svalid[j]) {
-      E::store(pg + L.off_norm, j, snorm[j]);
-      ((float*)(pg + L.off_rnorm))[j] = srn[j];
+      ((float*)(pg + L.off_meta))[2 * j] = snorm[j];
+      ((float*)(pg + L.off_meta))[2 * j + 1] = srn[j];
     }
   }
 }
@@ -380,7 +380,7 @@ value_tile_kernel(const void* __restrict__ v, Source src, int d, int gs, int bit
     // channel j: a field of 16*bits bits, token n at bit bits*n; read-modify-write keeps
     // the codes of slots this call does not touch
     const int wpc = bits / 2;                         // 32-bit words per channel
-    uint32_t* field = (uint32_t*)(pg + L.off_vdata) + j * wpc;
+    uint32_t* field = (uint32_t*)(pg + vfield_off(L, j));
     const int per_word = 32 / bits;
     for (int w = 0; w < wpc; ++w) {
       uint32_t neu = 0, mask = 0;
@@ -433,7 +433,7 @@ __global__ void pool_export_kernel(const uint8_t* __restrict__ pool, int H, cons
         if (c >= d) break;
         unsigned id = 0;
         for (int p = 0; p < mb; ++p) {
-          uint32_t w = *(const uint32_t*)(pg + plane_word_off(L, p, c >> 5, n));
+          uint32_t w = *(const uint32_t*)(pg + key_word_off(L, p, c >> 5, n));
           id = (id << 1) | ((w >> (c & 31)) & 1u);
         }
         byte |= id << (eff * s);
@@ -441,14 +441,14 @@ __global__ void pool_export_kernel(const uint8_t* __restrict__ pool, int H, cons
       idx[flat * row + k] = (uint8_t)byte;
     }
     for (int k = j; k < srow; k += blockDim.x) {
-      uint32_t w = *(const uint32_t*)(pg + plane_word_off(L, mb, k >> 2, n));
+      uint32_t w = *(const uint32_t*)(pg + key_word_off(L, mb, k >> 2, n));
       signs[flat * srow + k] = (uint8_t)(w >> ((k & 3) * 8));
     }
     for (int k = j; k < vrow; k += blockDim.x) {
       unsigned byte = 0;
       for (int s = 0; s < vper; ++s) {
         int c = k * vper + s;
-        const uint32_t* field = (const uint32_t*)(pg + L.off_vdata) + c * (vb / 2);
+        const uint32_t* field = (const uint32_t*)(pg + vfield_off(L, c));
         int bit = vb * n;
         byte |= ((field[bit >> 5] >> (bit & 31)) & ((1u << vb) - 1u)) << (vb * s);
       }
@@ -459,8 +459,8 @@ __global__ void pool_export_kernel(const uint8_t* __restrict__ pool, int H, cons
       copy_elem(v_zeros, flat * ng + g, pg + L.off_vzero, g * TILE + n, L.dtype);
     }
     if (j == 0) {
-      copy_elem(norms, flat, pg + L.off_norm, n, L.dtype);
-      rnorms[flat] = ((const float*)(pg + L.off_rnorm))[n];
+      store_from_f32(norms, flat, ((const float*)(pg + L.off_meta))[2 * n], L.dtype);
+      rnorms[flat] = ((const float*)(pg + L.off_meta))[2 * n + 1];
     }
   }
 }
@@ -518,10 +518,10 @@ extern "C" int tq_page_layout_init(tq_page_layout* L, int d, int mse_bits, int v
   if (dtype < TQ_F32 || dtype > TQ_BF16) return TQ_EINVAL;
   const int es = dtype == TQ_F32 ? 4 : 2;
   L->d = d; L->mse_bits = mse_bits; L->value_bits = value_bits; L->group_size = group_size; L->dtype = dtype;
+  L->key_lane_major = (d % 128 == 0) ? 1 : 0;
   int off = 0;
-  L->off_planes = off; off += (mse_bits + 1) * (d / 8) * TQ_PAGE_TOKENS;
-  L->off_norm = off;   off += es * TQ_PAGE_TOKENS;
-  L->off_rnorm = off;  off += 4 * TQ_PAGE_TOKENS;
+  L->off_keys = off;   off += (mse_bits + 1) * (d / 8) * TQ_PAGE_TOKENS;
+  L->off_meta = off;   off += 8 * TQ_PAGE_TOKENS;
   L->off_vdata = off;  off += d * value_bits * 2;
   L->off_vscale = off; off += (d / group_size) * TQ_PAGE_TOKENS * es;
   L->off_vzero = off;  off += (d / group_size) * TQ_PAGE_TOKENS * es;

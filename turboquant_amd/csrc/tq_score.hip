@@ -5,24 +5,51 @@
 
 namespace tq {
 
-// q_rot = q Pi^T, q_sk = q S^T for `rows` query vectors (triton_kernels.py:527-528).
-// One workgroup per row, d threads, fp32.
+// q_rot = q Pi^T, q_sk = q S^T for `rows` query vectors (triton_kernels.py:527-528), fp32.
+// One workgroup per row with d x 4 threads: thread (j, s) sums slice s of the
+// contraction for output column j, the four slices meet in LDS.  q_stat
+// (nullable) receives per row {max|q_rot|, max|q_sk|, sum q_rot, sum q_sk}, which
+// the matrix-core decode kernel uses to normalise and re-centre its operands.
 __global__ void __launch_bounds__(1024)
 rotate_query_kernel(const void* __restrict__ q, int dtype, tq_layer ly, float* __restrict__ q_rot,
-                    float* __restrict__ q_sk) {
-  extern __shared__ float sq[];
-  const int d = ly.d, j = threadIdx.x;
+                    float* __restrict__ q_sk, float* __restrict__ q_stat) {
+  extern __shared__ float sm[];
+  const int d = ly.d, tid = threadIdx.x, j = tid % d, sl = tid / d, n_sl = blockDim.x / d;
+  float* sq = sm;                 // [d]
+  float* pa = sm + d;             // [n_sl][d]
+  float* pb = pa + n_sl * d;      // [n_sl][d]
+  float* red = pb + n_sl * d;     // [4][16]
   const int64_t row = blockIdx.x;
-  sq[j] = load_as_f32(q, row * d + j, dtype);
+  if (tid < d) sq[tid] = load_as_f32(q, row * d + tid, dtype);
   __syncthreads();
+  const int per = d / n_sl, i0 = sl * per;
   float a = 0.0f, b = 0.0f;
-  for (int i = 0; i < d; ++i) {
-    float x = sq[i];
+  for (int i = i0; i < i0 + per; ++i) {
+    const float x = sq[i];
     a = fmaf(x, ly.PiT[(int64_t)i * d + j], a);
     b = fmaf(x, ly.ST[(int64_t)i * d + j], b);
   }
-  q_rot[row * d + j] = a;
-  q_sk[row * d + j] = b;
+  pa[sl * d + j] = a;
+  pb[sl * d + j] = b;
+  __syncthreads();
+  float ra = 0.0f, rb = 0.0f;
+  if (tid < d) {
+    for (int k = 0; k < n_sl; ++k) { ra += pa[k * d + tid]; rb += pb[k * d + tid]; }
+    q_rot[row * d + tid] = ra;
+    q_sk[row * d + tid] = rb;
+  }
+  if (q_stat) {
+    const int lane = tid & 63, wave = tid >> 6, n_wave = blockDim.x >> 6;
+    float ma = wave_max(tid < d ? fabsf(ra) : 0.0f), mb = wave_max(tid < d ? fabsf(rb) : 0.0f);
+    float sa = wave_sum(tid < d ? ra : 0.0f), sb = wave_sum(tid < d ? rb : 0.0f);
+    if (lane == 0) { red[wave] = ma; red[16 + wave] = mb; red[32 + wave] = sa; red[48 + wave] = sb; }
+    __syncthreads();
+    if (tid == 0) {
+      float m1 = 0.0f, m2 = 0.0f, s1 = 0.0f, s2 = 0.0f;
+      for (int w = 0; w < n_wave; ++w) { m1 = fmaxf(m1, red[w]); m2 = fmaxf(m2, red[16 + w]); s1 += red[32 + w]; s2 += red[48 + w]; }
+      q_stat[row * 4 + 0] = m1; q_stat[row * 4 + 1] = m2; q_stat[row * 4 + 2] = s1; q_stat[row * 4 + 3] = s2;
+    }
+  }
 }
 
 // scores[b, i, k] for a tile of QT queries and one key per thread.
@@ -152,6 +179,19 @@ static int check_layer_rd(const tq_layer* ly, bool need_sketch) {
   return TQ_OK;
 }
 
+namespace tq {
+int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* layer, float* q_rot, float* q_sk,
+                        float* q_stat, hipStream_t st) {
+  const int d = layer->d;
+  int n_sl = 4;
+  while (n_sl > 1 && (d * n_sl > 1024 || d % n_sl)) n_sl >>= 1;
+  size_t smem = (size_t)(d + 2 * n_sl * d + 64) * sizeof(float);
+  rotate_query_kernel<<<dim3((unsigned)rows), dim3(d * n_sl), smem, st>>>(q, dtype, *layer, q_rot, q_sk, q_stat);
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? TQ_OK : (int)e;
+}
+}  // namespace tq
+
 extern "C" int tq_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* layer, float* q_rot,
                                float* q_sk, void* stream) {
   int rc = check_layer_rd(layer, true);
@@ -159,10 +199,7 @@ extern "C" int tq_rotate_query(const void* q, int dtype, int64_t rows, const tq_
   if (!q || !q_rot || !q_sk) return TQ_ENULL;
   if (rows < 0 || dtype < TQ_F32 || dtype > TQ_BF16) return TQ_EINVAL;
   if (rows == 0) return TQ_OK;
-  rotate_query_kernel<<<dim3((unsigned)rows), dim3(layer->d), layer->d * sizeof(float), (hipStream_t)stream>>>(
-      q, dtype, *layer, q_rot, q_sk);
-  TQ_CHECK_LAUNCH();
-  return TQ_OK;
+  return launch_rotate_query(q, dtype, rows, layer, q_rot, q_sk, nullptr, (hipStream_t)stream);
 }
 
 extern "C" int tq_score(const void* q, int dtype, int64_t batch, int64_t n_q, const uint8_t* idx, const uint8_t* signs,

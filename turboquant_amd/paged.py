@@ -105,10 +105,15 @@ class PagedKVPool:
         return idx, signs, norms, rnorms, v_data, v_scales, v_zeros
 
     def default_splits(self, B: int, max_len: int) -> int:
-        """Enough (sequence, head, split) workgroups to fill 256 CUs a few times over."""
-        pages = max(1, (max_len + PAGE_TOKENS - 1) // PAGE_TOKENS)
-        want = max(1, math.ceil(2048 / max(1, B * self.num_kv_heads)))
-        return int(max(1, min(want, pages, 512)))
+        """Split count of the page-streaming kernel.  Its workgroups (4 wavefronts,
+        one per SIMD, each walking 64-token blocks) should number about two per CU
+        (256 CUs) while every wavefront still gets several blocks, because each
+        wavefront first builds its query operands."""
+        blocks = max(1, (max_len + 63) // 64)
+        pairs = max(1, B * self.num_kv_heads)
+        want = max(1, 512 // pairs)
+        longest = max(1, blocks // 16)          # keep >= 4 blocks per wavefront
+        return int(max(1, min(want, longest, 512)))
 
     def workspace(self, B: int, Hq: int, n_split: int) -> torch.Tensor:
         nbytes = _ffi.lib().tq_decode_workspace_bytes(B, Hq, self.head_dim, n_split)
