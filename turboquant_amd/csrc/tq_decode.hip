@@ -255,10 +255,10 @@ merge_kernel(const float* __restrict__ parts, int n_parts, int part_stride, int 
   const float inv = ll > 0.0f ? 1.0f / ll : 0.0f;
   for (int ch = tid; ch < d; ch += blockDim.x) {
     float aa = 0.0f;
-    for (int s = 0; s < n_parts; ++s) {
-      const float w = s_w[s];
-      if (w != 0.0f) aa = fmaf(w, p[(int64_t)s * (d + 2) + 2 + ch], aa);
-    }
+    // every part was written by its producer (empty ones as zeros), so the loads need no guard and
+    // stay independent of each other
+#pragma unroll 8
+    for (int s = 0; s < n_parts; ++s) aa = fmaf(s_w[s], p[(int64_t)s * (d + 2) + 2 + ch], aa);
     store_from_f32(out, row * d + ch, aa * inv, dtype);
   }
 }
@@ -269,8 +269,9 @@ using namespace tq;
 
 namespace tq {
 int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* layer, float* q_rot, float* q_sk,
-                        float* q_stat, hipStream_t st);
-int launch_decode_mfma(const float* q_rot, const float* q_sk, const float* q_stat, int B, int Hq, int Hkv,
+                        float* q_stat, uint32_t* qa_pack, int G, hipStream_t st);
+size_t decode_mfma_pack_words(int B, int Hkv, int d);
+int launch_decode_mfma(const uint32_t* qa_pack, const float* q_stat, int B, int Hq, int Hkv,
                        const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
                        float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts,
                        int n_split, hipStream_t st);
@@ -280,8 +281,10 @@ static size_t parts_floats(int B, int Hq, int d, int n_parts) { return (size_t)B
 
 extern "C" size_t tq_decode_workspace_bytes(int B, int Hq, int d, int n_split) {
   if (B <= 0 || Hq <= 0 || d <= 0 || n_split <= 0) return 0;
-  // partials for n_split history splits + 1 exact tail, then q_rot, q_sk and 4 statistics per query row
-  return (parts_floats(B, Hq, d, n_split + 1) + (size_t)2 * B * Hq * d + (size_t)4 * B * Hq) * sizeof(float);
+  // partials for n_split history splits + 1 exact tail, then q_rot, q_sk, 4 statistics per query row and
+  // the packed query operands of the matrix-core kernel (sized for the largest kernel: 9 term planes, 8 heads)
+  return (parts_floats(B, Hq, d, n_split + 1) + (size_t)2 * B * Hq * d + (size_t)4 * B * Hq) * sizeof(float) +
+         decode_mfma_pack_words(B, Hq, d) * sizeof(uint32_t);
 }
 
 extern "C" int tq_decode_merge(const float* parts, int64_t rows, int n_parts, int d, int dtype, void* out,
@@ -318,11 +321,14 @@ extern "C" int tq_decode_attn_paged_stages(const void* q, int dtype, int B, int 
   float* q_rot = parts + parts_floats(B, Hq, d, n_parts);
   float* q_sk = q_rot + (size_t)B * Hq * d;
   float* q_stat = q_sk + (size_t)B * Hq * d;
+  uint32_t* qa_pack = (uint32_t*)(q_stat + (size_t)4 * B * Hq);
+  const bool mfma_shape = G <= 8 && (d % 128) == 0 && layout->dtype == TQ_BF16;
 
   if (stages & 1) {
     if (!layer->Pi || !layer->PiT || !layer->S || !layer->ST || !layer->centroids) return TQ_ENULL;
     if (dtype < TQ_F32 || dtype > TQ_BF16) return TQ_EINVAL;
-    int rc = launch_rotate_query(q, dtype, (int64_t)B * Hq, layer, q_rot, q_sk, q_stat, st);
+    int rc = launch_rotate_query(q, dtype, (int64_t)B * Hq, layer, q_rot, q_sk, q_stat, mfma_shape ? qa_pack : nullptr,
+                                 G, st);
     if (rc) return rc;
   }
   if (!(stages & 6)) return TQ_OK;
@@ -332,7 +338,7 @@ extern "C" int tq_decode_attn_paged_stages(const void* q, int dtype, int B, int 
   dim3 grid(n_split, Hkv, B), block(DEC_WAVES * 64);
   int mf = TQ_EUNSUPPORTED;
   if (stages & 2)
-    mf = launch_decode_mfma(q_rot, q_sk, q_stat, B, Hq, Hkv, pool, block_table, bt_stride, seq_lens, sm_scale, *layer,
+    mf = launch_decode_mfma(qa_pack, q_stat, B, Hq, Hkv, pool, block_table, bt_stride, seq_lens, sm_scale, *layer,
                             *layout, parts, n_parts, n_split, st);
   if (mf > 0) return mf;
   if ((stages & 2) && mf == TQ_EUNSUPPORTED) {      // no matrix-core kernel for this shape: general kernel

@@ -110,8 +110,7 @@ __device__ __forceinline__ constexpr int v_token(int u, int r, int h) {
 // GS value group size; WPS wavefronts per SIMD the register budget is sized for.
 template <int D, int MB, int NX, int VB, int GS, int WPS>
 __global__ void __launch_bounds__(MF_WAVES * 64, WPS)
-decode_mfma_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_sk, const float* __restrict__ q_stat,
-                   int Hq, int Hkv, const uint8_t* __restrict__ pool, const int32_t* __restrict__ block_table,
+decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict__ q_stat, int Hq, int Hkv, const uint8_t* __restrict__ pool, const int32_t* __restrict__ block_table,
                    int bt_stride, const int32_t* __restrict__ seq_lens, float sm_scale, tq_layer ly, tq_page_layout L,
                    float* __restrict__ parts, int n_parts, int n_split) {
   constexpr int WPL = D / 128;                // plane words per lane per plane per page
@@ -138,52 +137,21 @@ decode_mfma_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
   for (int t = 0; t < ly.n_terms; ++t) cmax = fmaxf(cmax, fabsf(ly.term_coef[t]));
 
   // ---------------------------------------------------------------- A operands of the score stage
-  // lane (row = n, kb): row -> (head g = row/2, part = row%2: bf16 hi / lo of the query)
+  // lane (row = n, kb): row -> (head g = row/2, part = row%2: bf16 hi / lo of the query); the query
+  // kernel has stored them in register order, one coalesced 1 KB load per register quadruple
   u32x4 qa[NTP][WPL][4];
   {
-    const int g = n >> 1, part = n & 1;
-    const bool live = g < G;
-    const int64_t qrow = (int64_t)b * Hq + h * G + (live ? g : 0);
-    const float* rot = q_rot + qrow * D;
-    const float* sk = q_sk + qrow * D;
-    const float m1 = fmaxf(q_stat[qrow * 4 + 0] * cmax, 1e-30f), m2 = fmaxf(q_stat[qrow * 4 + 1], 1e-30f);
+    const u32x4* src = (const u32x4*)qa_pack + ((int64_t)b * Hkv + h) * (NTP * WPL * 4 * 64) + lane;
+    const bool live = (n >> 1) < G;
 #pragma unroll
-    for (int tp = 0; tp < NTP; ++tp) {
-      // coefficient of this term plane: stored plane p <-> index bit MB-1-p; extra terms in table order
-      float coef = 0.0f;
-      if (tp < MB) {
-        for (int t = 0; t < ly.n_terms; ++t)
-          if (ly.term_mask[t] == (1 << (MB - 1 - tp))) coef = ly.term_coef[t];
-      } else if (tp < MB + NX) {
-        int seen = 0;
-        for (int t = 0; t < ly.n_terms; ++t) {
-          if (__builtin_popcount(ly.term_mask[t]) > 1) {
-            if (seen == tp - MB) coef = ly.term_coef[t];
-            ++seen;
-          }
-        }
-      }
-      const bool is_sign = tp == NTP - 1;
-      const float* src = is_sign ? sk : rot;
-      const float mul = live ? (is_sign ? 1.0f / m2 : coef / m1) : 0.0f;
+    for (int tp = 0; tp < NTP; ++tp)
 #pragma unroll
-      for (int i = 0; i < WPL; ++i) {
+      for (int i = 0; i < WPL; ++i)
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-          u32x4 reg;
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const int bit = 4 * u + r;
-            const float sc = __builtin_ldexpf(1.0f, -slot_exponent(bit_slot(bit)));
-            const int c0 = 32 * (4 * i + kb) + bit;
-            float v0 = src[c0] * mul * sc, v1 = src[c0 + 16] * mul * sc;
-            if (part) { v0 -= bf16_round(v0); v1 -= bf16_round(v1); }
-            reg[r] = pack_bf16(v0, v1);
-          }
-          qa[tp][i][u] = reg;
+          u32x4 v = src[((tp * WPL + i) * 4 + u) * 64];
+          qa[tp][i][u] = live ? v : u32x4{0, 0, 0, 0};
         }
-      }
-    }
   }
   // score constants of the two heads this lane sees in the MFMA output (rows 4kb..4kb+3 = heads 2kb, 2kb+1)
   float am[2], bm[2], aq[2], bq[2];
@@ -279,11 +247,9 @@ decode_mfma_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
   const u32x4 neg_base = {neg_pat, neg_pat, neg_pat, neg_pat};
 
   // ---------------------------------------------------------------- one block of 64 tokens
-  auto compute = [&](int blk, const KeyRegs& K, const ValRegs& V, auto partial_tag) {
+  // scores of the 4 pages of block blk, online softmax, weights -> LDS
+  auto score_stage = [&](int blk, const KeyRegs& K, auto partial_tag) -> bool {
     constexpr bool PARTIAL = decltype(partial_tag)::value;
-    // scales -> LDS ([page][group][16 tokens] bf16, as in the page)
-    if (lane < 4 * PIECES) *(u32x4*)(s_scale + lane * 4) = V.scale;
-    // ---- scores of the 4 pages
     float s2[2][4];
 #pragma unroll
     for (int pg = 0; pg < 4; ++pg) {
@@ -339,6 +305,13 @@ decode_mfma_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
     }
     const bool rescale = __builtin_amdgcn_ballot_w64(alpha[0] != 1.0f || alpha[1] != 1.0f) != 0;
     if (rescale && n == 0) { s_alpha[2 * kb] = alpha[0]; s_alpha[2 * kb + 1] = alpha[1]; }
+    return rescale;
+  };
+  // weights x (codes, scales, zeros) of block blk into the accumulators
+  auto value_stage = [&](int blk, const ValRegs& V, bool rescale, auto partial_tag) {
+    constexpr bool PARTIAL = decltype(partial_tag)::value;
+    // scales -> LDS ([page][group][16 tokens] bf16, as in the page); first use of the value loads
+    if (lane < 4 * PIECES) *(u32x4*)(s_scale + lane * 4) = V.scale;
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -433,35 +406,29 @@ decode_mfma_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
   };
 
   // ---------------------------------------------------------------- pipeline over this wave's blocks
+  // Registers are reloaded as soon as their last reader is done: the key words of
+  // the next block are requested right after the score stage, its value words
+  // right after the value stage.
   {
-    KeyRegs KA, KB;
-    ValRegs VR;
-    int pid_cur[4], pid_nxt[4];
+    KeyRegs K;
+    ValRegs V;
+    int pid[4];
     int blk = blk_begin + wave;
     if (blk < blk_end) {
-      page_ids(blk, pid_cur);
-      load_keys(pid_cur, KA);
+      page_ids(blk, pid);
+      load_keys(pid, K);
+      load_vals(pid, V);
     }
     while (blk < blk_end) {
-      // even step: current keys in KA
-      {
-        const int nxt = blk + MF_WAVES;
-        load_vals(pid_cur, VR);
-        if (nxt < blk_end) { page_ids(nxt, pid_nxt); load_keys(pid_nxt, KB); }
-        if ((blk + 1) * BLK_TOK > seq_len) compute(blk, KA, VR, std::true_type{});
-        else compute(blk, KA, VR, std::false_type{});
-        blk = nxt;
-      }
-      if (blk >= blk_end) break;
-      // odd step: current keys in KB
-      {
-        const int nxt = blk + MF_WAVES;
-        load_vals(pid_nxt, VR);
-        if (nxt < blk_end) { page_ids(nxt, pid_cur); load_keys(pid_cur, KA); }
-        if ((blk + 1) * BLK_TOK > seq_len) compute(blk, KB, VR, std::true_type{});
-        else compute(blk, KB, VR, std::false_type{});
-        blk = nxt;
-      }
+      const int nxt = blk + MF_WAVES;
+      const bool last = (blk + 1) * BLK_TOK > seq_len;
+      const bool rescale = last ? score_stage(blk, K, std::true_type{}) : score_stage(blk, K, std::false_type{});
+      int pid_n[4];
+      if (nxt < blk_end) { page_ids(nxt, pid_n); load_keys(pid_n, K); }
+      if (last) value_stage(blk, V, rescale, std::true_type{});
+      else value_stage(blk, V, rescale, std::false_type{});
+      if (nxt < blk_end) load_vals(pid_n, V);
+      blk = nxt;
     }
   }
 
@@ -513,7 +480,7 @@ decode_mfma_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
 }
 
 template <int D, int MB, int NX, int VB, int GS, int WPS>
-static int launch_one(const float* q_rot, const float* q_sk, const float* q_stat, int B, int Hq, int Hkv,
+static int launch_one(const uint32_t* qa_pack, const float* q_stat, int B, int Hq, int Hkv,
                       const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
                       float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts, int n_split,
                       hipStream_t st) {
@@ -526,7 +493,7 @@ static int launch_one(const float* q_rot, const float* q_sk, const float* q_stat
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return (int)e;
   }
-  kern<<<dim3(n_split, Hkv, B), dim3(MF_WAVES * 64), smem, st>>>(q_rot, q_sk, q_stat, Hq, Hkv, pool, block_table,
+  kern<<<dim3(n_split, Hkv, B), dim3(MF_WAVES * 64), smem, st>>>(qa_pack, q_stat, Hq, Hkv, pool, block_table,
                                                                  bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts,
                                                                  n_split);
   hipError_t e = hipGetLastError();
@@ -535,7 +502,10 @@ static int launch_one(const float* q_rot, const float* q_sk, const float* q_stat
 
 // Returns TQ_EUNSUPPORTED when the shape has no matrix-core kernel; the caller then
 // uses the general vector-ALU kernel.
-int launch_decode_mfma(const float* q_rot, const float* q_sk, const float* q_stat, int B, int Hq, int Hkv,
+// words of packed query operands tq_decode_attn_paged reserves in its workspace
+size_t decode_mfma_pack_words(int B, int Hq, int d) { return (size_t)B * Hq * 9 * (d / 128 + 1) * 1024; }
+
+int launch_decode_mfma(const uint32_t* qa_pack, const float* q_stat, int B, int Hq, int Hkv,
                        const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
                        float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts,
                        int n_split, hipStream_t st) {
@@ -546,7 +516,7 @@ int launch_decode_mfma(const float* q_rot, const float* q_sk, const float* q_sta
     if (__builtin_popcount(ly.term_mask[t]) > 1) ++nx;
 #define TQ_TRY(D_, MB_, NX_, VB_, GS_, WPS_)                                                                    \
   if (d == D_ && mb == MB_ && nx == NX_ && vb == VB_ && gs == GS_)                                              \
-    return launch_one<D_, MB_, NX_, VB_, GS_, WPS_>(q_rot, q_sk, q_stat, B, Hq, Hkv, pool, block_table, bt_stride, \
+    return launch_one<D_, MB_, NX_, VB_, GS_, WPS_>(qa_pack, q_stat, B, Hq, Hkv, pool, block_table, bt_stride,    \
                                                     seq_lens, sm_scale, ly, L, parts, n_parts, n_split, st);
   TQ_TRY(128, 2, 0, 2, 32, 2) TQ_TRY(128, 2, 0, 4, 32, 2) TQ_TRY(256, 2, 0, 2, 32, 1) TQ_TRY(256, 2, 0, 4, 32, 1)
   TQ_TRY(128, 1, 0, 2, 32, 2) TQ_TRY(128, 1, 0, 4, 32, 2) TQ_TRY(256, 1, 0, 2, 32, 1) TQ_TRY(256, 1, 0, 4, 32, 1)

@@ -6,49 +6,163 @@
 namespace tq {
 
 // q_rot = q Pi^T, q_sk = q S^T for `rows` query vectors (triton_kernels.py:527-528), fp32.
-// One workgroup per row with d x 4 threads: thread (j, s) sums slice s of the
-// contraction for output column j, the four slices meet in LDS.  q_stat
-// (nullable) receives per row {max|q_rot|, max|q_sk|, sum q_rot, sum q_sk}, which
-// the matrix-core decode kernel uses to normalise and re-centre its operands.
-__global__ void __launch_bounds__(1024)
-rotate_query_kernel(const void* __restrict__ q, int dtype, tq_layer ly, float* __restrict__ q_rot,
-                    float* __restrict__ q_sk, float* __restrict__ q_stat) {
+// A workgroup handles R consecutive rows (the query heads of one KV head when
+// called from the decode path) and a slice of ROT_COLS output columns with
+// ROT_COLS x ROT_SLICES threads: thread (j, s) sums slice s of the contraction for
+// its column of every row, so each matrix element is read once per workgroup; the
+// slices meet in LDS.
+constexpr int ROT_MAX_ROWS = 8, ROT_COLS = 32, ROT_SLICES = 8;
+
+__global__ void __launch_bounds__(ROT_COLS * ROT_SLICES)
+rotate_query_kernel(const void* __restrict__ q, int dtype, int64_t rows, int R, tq_layer ly, float* __restrict__ q_rot,
+                    float* __restrict__ q_sk) {
   extern __shared__ float sm[];
-  const int d = ly.d, tid = threadIdx.x, j = tid % d, sl = tid / d, n_sl = blockDim.x / d;
-  float* sq = sm;                 // [d]
-  float* pa = sm + d;             // [n_sl][d]
-  float* pb = pa + n_sl * d;      // [n_sl][d]
-  float* red = pb + n_sl * d;     // [4][16]
-  const int64_t row = blockIdx.x;
-  if (tid < d) sq[tid] = load_as_f32(q, row * d + tid, dtype);
+  const int d = ly.d, tid = threadIdx.x, jl = tid % ROT_COLS, sl = tid / ROT_COLS;
+  const int j = blockIdx.y * ROT_COLS + jl;
+  float* sq = sm;                                  // [R][d] inputs
+  float* pa = sq + R * d;                          // [ROT_SLICES][R][ROT_COLS] partial sums
+  float* pb = pa + ROT_SLICES * R * ROT_COLS;
+  const int64_t row0 = (int64_t)blockIdx.x * R;
+  const int nr = (int)((rows - row0) < R ? (rows - row0) : R);
+  for (int o = tid; o < R * d; o += blockDim.x) sq[o] = o < nr * d ? load_as_f32(q, row0 * d + o, dtype) : 0.0f;
   __syncthreads();
-  const int per = d / n_sl, i0 = sl * per;
-  float a = 0.0f, b = 0.0f;
-  for (int i = i0; i < i0 + per; ++i) {
-    const float x = sq[i];
-    a = fmaf(x, ly.PiT[(int64_t)i * d + j], a);
-    b = fmaf(x, ly.ST[(int64_t)i * d + j], b);
-  }
-  pa[sl * d + j] = a;
-  pb[sl * d + j] = b;
-  __syncthreads();
-  float ra = 0.0f, rb = 0.0f;
-  if (tid < d) {
-    for (int k = 0; k < n_sl; ++k) { ra += pa[k * d + tid]; rb += pb[k * d + tid]; }
-    q_rot[row * d + tid] = ra;
-    q_sk[row * d + tid] = rb;
-  }
-  if (q_stat) {
-    const int lane = tid & 63, wave = tid >> 6, n_wave = blockDim.x >> 6;
-    float ma = wave_max(tid < d ? fabsf(ra) : 0.0f), mb = wave_max(tid < d ? fabsf(rb) : 0.0f);
-    float sa = wave_sum(tid < d ? ra : 0.0f), sb = wave_sum(tid < d ? rb : 0.0f);
-    if (lane == 0) { red[wave] = ma; red[16 + wave] = mb; red[32 + wave] = sa; red[48 + wave] = sb; }
-    __syncthreads();
-    if (tid == 0) {
-      float m1 = 0.0f, m2 = 0.0f, s1 = 0.0f, s2 = 0.0f;
-      for (int w = 0; w < n_wave; ++w) { m1 = fmaxf(m1, red[w]); m2 = fmaxf(m2, red[16 + w]); s1 += red[32 + w]; s2 += red[48 + w]; }
-      q_stat[row * 4 + 0] = m1; q_stat[row * 4 + 1] = m2; q_stat[row * 4 + 2] = s1; q_stat[row * 4 + 3] = s2;
+  const int per = d / ROT_SLICES, i0 = sl * per;
+  float a[ROT_MAX_ROWS], b[ROT_MAX_ROWS];
+#pragma unroll
+  for (int r = 0; r < ROT_MAX_ROWS; ++r) a[r] = b[r] = 0.0f;
+  // eight matrix rows at a time: all sixteen loads are in flight before the first use
+  for (int ib = i0; ib < i0 + per; ib += 8) {
+    float mp[8], ms[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      mp[k] = ly.PiT[(int64_t)(ib + k) * d + j];
+      ms[k] = ly.ST[(int64_t)(ib + k) * d + j];
     }
+#pragma unroll
+    for (int r = 0; r < ROT_MAX_ROWS; ++r) {
+      if (r < R) {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          const float x = sq[r * d + ib + k];
+          a[r] = fmaf(x, mp[k], a[r]);
+          b[r] = fmaf(x, ms[k], b[r]);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < ROT_MAX_ROWS; ++r) {
+    if (r < R) {
+      pa[(sl * R + r) * ROT_COLS + jl] = a[r];
+      pb[(sl * R + r) * ROT_COLS + jl] = b[r];
+    }
+  }
+  __syncthreads();
+  for (int o = tid; o < nr * ROT_COLS; o += blockDim.x) {
+    const int r = o / ROT_COLS, c = o - r * ROT_COLS;
+    float ra = 0.0f, rb = 0.0f;
+    for (int k = 0; k < ROT_SLICES; ++k) { ra += pa[(k * R + r) * ROT_COLS + c]; rb += pb[(k * R + r) * ROT_COLS + c]; }
+    q_rot[(row0 + r) * d + blockIdx.y * ROT_COLS + c] = ra;
+    q_sk[(row0 + r) * d + blockIdx.y * ROT_COLS + c] = rb;
+  }
+}
+
+// Operands of the matrix-core decode kernel for one GQA group (G query heads of one
+// KV head), from the finished q_rot / q_sk rows.
+// q_stat receives per row {max|q_rot|, max|q_sk|, sum q_rot, sum q_sk}.
+// qa_pack receives the score-stage A operands in register order:
+// [kv head][term plane][word i][mfma u][lane 0..63][4 dwords], where lane
+// (n, kb) = (2*g + part, coordinate quarter), g the head within the group, part 0/1
+// the bf16 hi / lo half of the value, and element (r, h) of a register quadruple is
+// coordinate 32*(4i+kb) + 4u + r + 16h scaled by the inverse of the power of two its
+// bit occupies in the B operand.
+__host__ __device__ constexpr int qa_bit_slot(int bit) { return bit <= 6 ? bit + 7 : (bit == 15 ? 14 : bit); }
+
+__global__ void __launch_bounds__(1024)
+pack_query_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_sk, int G, tq_layer ly,
+                  float* __restrict__ q_stat, uint32_t* __restrict__ qa_pack) {
+  extern __shared__ float sm[];
+  const int d = ly.d, tid = threadIdx.x;
+  float* sq = sm;                 // [G][d]
+  float* sk = sq + G * d;         // [G][d]
+  float* stat = sk + G * d;       // [G][4]
+  const int64_t group = blockIdx.x, row0 = group * G;
+  for (int o = tid; o < G * d; o += blockDim.x) { sq[o] = q_rot[row0 * d + o]; sk[o] = q_sk[row0 * d + o]; }
+  __syncthreads();
+  {
+    const int lane = tid & 63, wave = tid >> 6, n_wave = blockDim.x >> 6;
+    for (int r = wave; r < G; r += n_wave) {
+      float m1 = 0.0f, m2 = 0.0f, s1 = 0.0f, s2 = 0.0f;
+      for (int c = lane; c < d; c += 64) {
+        const float x = sq[r * d + c], y = sk[r * d + c];
+        m1 = fmaxf(m1, fabsf(x)); m2 = fmaxf(m2, fabsf(y)); s1 += x; s2 += y;
+      }
+      m1 = wave_max(m1); m2 = wave_max(m2); s1 = wave_sum(s1); s2 = wave_sum(s2);
+      if (lane == 0) {
+        stat[r * 4 + 0] = m1; stat[r * 4 + 1] = m2; stat[r * 4 + 2] = s1; stat[r * 4 + 3] = s2;
+        q_stat[(row0 + r) * 4 + 0] = m1; q_stat[(row0 + r) * 4 + 1] = m2;
+        q_stat[(row0 + r) * 4 + 2] = s1; q_stat[(row0 + r) * 4 + 3] = s2;
+      }
+    }
+  }
+  if (!qa_pack) return;
+  const int mb = ly.mse_bits;
+  int nx = 0;
+  float cmax = 0.0f;
+  for (int t = 0; t < ly.n_terms; ++t) {
+    cmax = fmaxf(cmax, fabsf(ly.term_coef[t]));
+    if (__builtin_popcount(ly.term_mask[t]) > 1) ++nx;
+  }
+  const int ntp = mb + nx + 1, wpl = d / 128;
+  float* coefs = stat + 4 * G;          // [ntp] coefficient of each term plane (1 for the sign plane)
+  float* scale = coefs + 16;            // [16] inverse power of two of each bit slot
+  if (tid < ntp) {
+    float coef = 1.0f;
+    if (tid < mb) {
+      coef = 0.0f;
+      for (int t = 0; t < ly.n_terms; ++t)
+        if (ly.term_mask[t] == (1 << (mb - 1 - tid))) coef = ly.term_coef[t];
+    } else if (tid < mb + nx) {
+      coef = 0.0f;
+      int seen = 0;
+      for (int t = 0; t < ly.n_terms; ++t) {
+        if (__builtin_popcount(ly.term_mask[t]) > 1) {
+          if (seen == tid - mb) coef = ly.term_coef[t];
+          ++seen;
+        }
+      }
+    }
+    coefs[tid] = coef;
+  }
+  if (tid >= 64 && tid < 80) scale[tid - 64] = ldexpf(1.0f, 127 - (1 << (qa_bit_slot(tid - 64) - 7)));
+  __syncthreads();
+  if (tid < G) {                        // per head: 1 / normaliser of the rotated and of the sketched query
+    stat[tid * 4 + 2] = 1.0f / fmaxf(stat[tid * 4 + 0] * cmax, 1e-30f);
+    stat[tid * 4 + 3] = 1.0f / fmaxf(stat[tid * 4 + 1], 1e-30f);
+  }
+  __syncthreads();
+  // one thread per output word, in storage order (coalesced stores); lanes of absent heads get zeros
+  const int total = ntp * wpl * 4 * 64 * 4;
+  uint32_t* dst = qa_pack + group * (int64_t)total;
+  for (int o = tid; o < total; o += blockDim.x) {
+    const int r = o & 3, lane = (o >> 2) & 63, u = (o >> 8) & 3;
+    const int i = (o >> 10) % wpl, tp = (o >> 10) / wpl;
+    const int kb = lane >> 4, g = (lane & 15) >> 1, part = lane & 1;
+    uint32_t packed = 0;
+    if (g < G) {
+      const bool is_sign = tp == ntp - 1;
+      const float* src = (is_sign ? sk : sq) + g * d;
+      const int bit = 4 * u + r;
+      const float mul = (is_sign ? stat[g * 4 + 3] : coefs[tp] * stat[g * 4 + 2]) * scale[bit];
+      const int c0 = 32 * (4 * i + kb) + bit;
+      float v0 = src[c0] * mul, v1 = src[c0 + 16] * mul;
+      if (part) {
+        v0 -= bf16_bits_to_f32(f32_to_bf16_bits(v0));
+        v1 -= bf16_bits_to_f32(f32_to_bf16_bits(v1));
+      }
+      packed = (uint32_t)f32_to_bf16_bits(v0) | ((uint32_t)f32_to_bf16_bits(v1) << 16);
+    }
+    dst[o] = packed;
   }
 }
 
@@ -181,14 +295,24 @@ static int check_layer_rd(const tq_layer* ly, bool need_sketch) {
 
 namespace tq {
 int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* layer, float* q_rot, float* q_sk,
-                        float* q_stat, hipStream_t st) {
+                        float* q_stat, uint32_t* qa_pack, int G, hipStream_t st) {
   const int d = layer->d;
-  int n_sl = 4;
-  while (n_sl > 1 && (d * n_sl > 1024 || d % n_sl)) n_sl >>= 1;
-  size_t smem = (size_t)(d + 2 * n_sl * d + 64) * sizeof(float);
-  rotate_query_kernel<<<dim3((unsigned)rows), dim3(d * n_sl), smem, st>>>(q, dtype, *layer, q_rot, q_sk, q_stat);
+  // rows per workgroup: the GQA group when the decode operands are wanted, else up to 8
+  const int R = (q_stat && G <= ROT_MAX_ROWS) ? G : (int)(rows < ROT_MAX_ROWS ? rows : ROT_MAX_ROWS);
+  if (R < 1 || d % ROT_COLS || d % (8 * ROT_SLICES)) return TQ_EUNSUPPORTED;
+  size_t smem = (size_t)(R * d + 2 * ROT_SLICES * R * ROT_COLS) * sizeof(float);
+  rotate_query_kernel<<<dim3((unsigned)((rows + R - 1) / R), d / ROT_COLS), dim3(ROT_COLS * ROT_SLICES), smem, st>>>(
+      q, dtype, rows, R, *layer, q_rot, q_sk);
   hipError_t e = hipGetLastError();
-  return e == hipSuccess ? TQ_OK : (int)e;
+  if (e != hipSuccess) return (int)e;
+  if (q_stat) {
+    if (G > ROT_MAX_ROWS * 2 || rows % G) return TQ_EUNSUPPORTED;
+    size_t psm = (size_t)(2 * G * d + 4 * G + 32) * sizeof(float);
+    pack_query_kernel<<<dim3((unsigned)(rows / G)), dim3(1024), psm, st>>>(q_rot, q_sk, G, *layer, q_stat, qa_pack);
+    e = hipGetLastError();
+    if (e != hipSuccess) return (int)e;
+  }
+  return TQ_OK;
 }
 }  // namespace tq
 
@@ -199,7 +323,7 @@ extern "C" int tq_rotate_query(const void* q, int dtype, int64_t rows, const tq_
   if (!q || !q_rot || !q_sk) return TQ_ENULL;
   if (rows < 0 || dtype < TQ_F32 || dtype > TQ_BF16) return TQ_EINVAL;
   if (rows == 0) return TQ_OK;
-  return launch_rotate_query(q, dtype, rows, layer, q_rot, q_sk, nullptr, (hipStream_t)stream);
+  return launch_rotate_query(q, dtype, rows, layer, q_rot, q_sk, nullptr, nullptr, 1, (hipStream_t)stream);
 }
 
 extern "C" int tq_score(const void* q, int dtype, int64_t batch, int64_t n_q, const uint8_t* idx, const uint8_t* signs,
