@@ -36,6 +36,7 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
 
 constexpr int MF_WAVES = 4;
 constexpr int BLK_TOK = 64;              // tokens per wavefront iteration
@@ -191,7 +192,7 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
   const uint8_t* pool_h = pool + (int64_t)h * L.page_bytes;
   const int64_t page_stride = (int64_t)Hkv * L.page_bytes;
   const int off_keys = L.off_keys + lane * (NKW * 4), off_meta = L.off_meta + n * 8;
-  const int off_v = L.off_vdata + n * (VW * 4), off_zero = L.off_vzero + n * 32;
+  const int off_v = L.off_vdata + n * (VW * 4);
   const int off_scale = L.off_vscale + (lane % PIECES) * 16;
 
   f32x4 acc[CT];
@@ -203,7 +204,8 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
   struct KeyRegs { uint32_t key[4][NKW]; f32x2 meta[4]; };
   struct ValRegs { uint32_t v[VW]; u32x4 zero[2]; u32x4 scale; };
 
-  // page ids of block `blk` -> 4 scalars, clamped into the sequence's pages
+  // page ids of block `blk` -> 4 scalars; a page past the end of the sequence (last block only) is
+  // replaced by the block's first page, which always exists
   auto page_ids = [&](int blk, int (&pid)[4]) {
 #pragma unroll
     for (int pg = 0; pg < 4; ++pg) pid[pg] = bt[min(4 * blk + pg, n_pages - 1)];
@@ -218,27 +220,22 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
       R.meta[pg] = *(const f32x2*)(base + off_meta);
     }
   };
+  // All loads below are unconditional (lanes without a group / piece of their own read a
+  // neighbour's): a load inside a branch would make the wait counters at the join conservative
+  // and serialise the prefetch.
+  const int off_zero_c = L.off_vzero + min(n, NG - 1) * 32;
+  const int spg = min(lane / PIECES, 3);
   auto load_vals = [&](const int (&pid)[4], ValRegs& R) {
     const int my_pid = kb == 0 ? pid[0] : (kb == 1 ? pid[1] : (kb == 2 ? pid[2] : pid[3]));
     const uint8_t* vbase = pool_h + my_pid * page_stride;
     const uint32_t* vp = (const uint32_t*)(vbase + off_v);
 #pragma unroll
     for (int w = 0; w < VW; ++w) R.v[w] = vp[w];
-    if (n < NG) {
-      const u32x4* zp = (const u32x4*)(vbase + off_zero);
-      R.zero[0] = zp[0];
-      R.zero[1] = zp[1];
-    } else {
-      R.zero[0] = u32x4{0, 0, 0, 0};
-      R.zero[1] = u32x4{0, 0, 0, 0};
-    }
-    if (lane < 4 * PIECES) {
-      const int spg = lane / PIECES;
-      const int spid = spg == 0 ? pid[0] : (spg == 1 ? pid[1] : (spg == 2 ? pid[2] : pid[3]));
-      R.scale = *(const u32x4*)(pool_h + spid * page_stride + off_scale);
-    } else {
-      R.scale = u32x4{0, 0, 0, 0};
-    }
+    const u32x4* zp = (const u32x4*)(vbase + off_zero_c);
+    R.zero[0] = zp[0];
+    R.zero[1] = zp[1];
+    const int spid = spg == 0 ? pid[0] : (spg == 1 ? pid[1] : (spg == 2 ? pid[2] : pid[3]));
+    R.scale = *(const u32x4*)(pool_h + spid * page_stride + off_scale);
   };
 
   const uint32_t base_pat = in_vgpr(VB == 2 ? 0x40804080u : 0x41804180u);   // bf16 pairs of 2^VB
@@ -422,12 +419,16 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
     while (blk < blk_end) {
       const int nxt = blk + MF_WAVES;
       const bool last = (blk + 1) * BLK_TOK > seq_len;
-      const bool rescale = last ? score_stage(blk, K, std::true_type{}) : score_stage(blk, K, std::false_type{});
+      // the block after this wave's last one does not exist: re-request the current one instead,
+      // so that the loads stay outside any branch
+      const int nxt_c = nxt < blk_end ? nxt : blk;
       int pid_n[4];
-      if (nxt < blk_end) { page_ids(nxt, pid_n); load_keys(pid_n, K); }
+      page_ids(nxt_c, pid_n);                            // scalar loads, consumed after the score stage
+      const bool rescale = last ? score_stage(blk, K, std::true_type{}) : score_stage(blk, K, std::false_type{});
+      load_keys(pid_n, K);
       if (last) value_stage(blk, V, rescale, std::true_type{});
       else value_stage(blk, V, rescale, std::false_type{});
-      if (nxt < blk_end) load_vals(pid_n, V);
+      load_vals(pid_n, V);
       blk = nxt;
     }
   }
