@@ -53,6 +53,10 @@ typedef struct tq_layer {
   const float *centroids;  /* 2^mse_bits                                                    */
   const float *thresholds; /* 2^mse_bits - 1 interior boundaries (quantizer.py:127)         */
   float qjl_scale;         /* sqrt(pi/2)/d (quantizer.py:212)                               */
+  /* Optional operands of the matrix-core quantise kernel: Pi, its transpose and S, each
+   * written as the exact sum of three bf16 matrices, stored [term][row][col] as raw
+   * bf16 bit patterns (3*d*d each).  NULL selects the vector-ALU kernel.            */
+  const uint16_t *Pi_split, *PiT_split, *S_split;
   /* Walsh expansion of the codebook over the index bits, used by the decode
    * kernel: centroids[idx] = term_const + sum_t term_coef[t] * parity(idx & term_mask[t]).
    * Filled by tq_layer_fill_terms from the host copy of the centroids.          */

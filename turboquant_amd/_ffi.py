@@ -32,6 +32,7 @@ class TqLayer(C.Structure):
         ("Pi", C.c_void_p), ("PiT", C.c_void_p), ("S", C.c_void_p), ("ST", C.c_void_p),
         ("centroids", C.c_void_p), ("thresholds", C.c_void_p),
         ("qjl_scale", C.c_float),
+        ("Pi_split", C.c_void_p), ("PiT_split", C.c_void_p), ("S_split", C.c_void_p),
         ("n_terms", C.c_int32),
         ("term_mask", C.c_int32 * TQ_MAX_TERMS),
         ("term_coef", C.c_float * TQ_MAX_TERMS),
@@ -137,7 +138,7 @@ def walsh_terms(centroids_host: torch.Tensor, mse_bits: int, layer: TqLayer):
 
 def make_layer(d: int, mse_bits: int, Pi: torch.Tensor, PiT: torch.Tensor, centroids: torch.Tensor,
                thresholds: torch.Tensor, S: Optional[torch.Tensor] = None, ST: Optional[torch.Tensor] = None,
-               centroids_host: Optional[torch.Tensor] = None) -> TqLayer:
+               centroids_host: Optional[torch.Tensor] = None, splits=None) -> TqLayer:
     """Describe a layer's constants to the library.  The tensors must stay alive
     while the struct is in use; they must be fp32, contiguous and on one GPU."""
     for name, t in (("Pi", Pi), ("PiT", PiT), ("centroids", centroids), ("thresholds", thresholds), ("S", S), ("ST", ST)):
@@ -153,8 +154,24 @@ def make_layer(d: int, mse_bits: int, Pi: torch.Tensor, PiT: torch.Tensor, centr
     ly.ST = None if ST is None else ST.data_ptr()
     ly.centroids, ly.thresholds = centroids.data_ptr(), thresholds.data_ptr()
     ly.qjl_scale = math.sqrt(math.pi / 2.0) / d
+    if splits is not None:
+        pi_s, pit_s, s_s = splits
+        ly.Pi_split, ly.PiT_split = pi_s.data_ptr(), pit_s.data_ptr()
+        ly.S_split = None if s_s is None else s_s.data_ptr()
     walsh_terms(centroids_host if centroids_host is not None else centroids.detach().cpu(), mse_bits, ly)
     return ly
+
+
+def split_bf16x3(m: torch.Tensor) -> torch.Tensor:
+    """fp32 matrix -> (3, rows, cols) int16 tensor of bf16 bit patterns whose three
+    terms sum to the matrix exactly (each term rounds the running remainder)."""
+    rest = m.float()
+    parts = []
+    for _ in range(3):
+        term = rest.to(torch.bfloat16)
+        parts.append(term)
+        rest = rest - term.float()
+    return torch.stack(parts).contiguous().view(torch.int16)
 
 
 def make_page_layout(d: int, mse_bits: int, value_bits: int, group_size: int, dtype: torch.dtype) -> TqPageLayout:

@@ -1,0 +1,137 @@
+// Pieces shared by the vector-ALU and the matrix-core key quantise kernels: where a
+// tile of 16 vectors comes from, where its codes go, and the two writers.
+#pragma once
+
+#include <type_traits>
+
+#include "tq_common.h"
+
+namespace tq {
+
+constexpr int TILE = TQ_PAGE_TOKENS;
+
+// ------------------------------------------------------------------------------------
+// tile sources: where the 16 vectors of a tile come from and which are valid
+// ------------------------------------------------------------------------------------
+
+struct FlatSource {          // (n_vec, d) with a row stride
+  int64_t n_vec, row_stride;
+  __device__ bool locate(int tile, int slot, int64_t& elem_off) const {
+    int64_t v = (int64_t)tile * TILE + slot;
+    elem_off = v * row_stride;
+    return v < n_vec;
+  }
+};
+
+struct PagedSource {         // (b, t, h, :) strided, tokens mapped onto 16-token pages
+  int B, T, H, tiles_per_seq;
+  int64_t stride_b, stride_t, stride_h;
+  const int32_t* start_pos;
+  // tile index -> (b, page slot window, head)
+  __device__ void decode(int tile, int& b, int& lpage, int& h) const {
+    h = tile % H;
+    int r = tile / H;
+    int pg = r % tiles_per_seq;
+    b = r / tiles_per_seq;
+    int s0 = start_pos ? start_pos[b] : 0;
+    lpage = s0 / TILE + pg;
+  }
+  __device__ bool locate(int tile, int slot, int64_t& elem_off) const {
+    int b, lpage, h;
+    decode(tile, b, lpage, h);
+    int s0 = start_pos ? start_pos[b] : 0;
+    int t = lpage * TILE + slot - s0;
+    elem_off = b * stride_b + (int64_t)t * stride_t + h * stride_h;
+    return t >= 0 && t < T;
+  }
+};
+
+// ------------------------------------------------------------------------------------
+// key tile
+// ------------------------------------------------------------------------------------
+
+struct KeyFlatSink {
+  uint8_t* idx;
+  uint8_t* sign;
+  void* norm;
+  float* rnorm;
+  float* y_dbg;
+  float* p_dbg;
+};
+
+struct KeyPagedSink {
+  uint8_t* pool;
+  const int32_t* block_table;
+  int max_pages;
+  tq_page_layout L;
+};
+
+
+// ------------------------------------------------------------------------------------
+// writers for one tile of 16 vectors, run by `nthreads` cooperating threads (tid = 0..nthreads-1).
+// sidx / ssgn hold one byte per (slot, coordinate): the Lloyd-Max index and the sign bit;
+// snorm / srn the key norm (as fp32) and the residual norm; svalid which slots exist.
+// ------------------------------------------------------------------------------------
+
+template <int DT>
+__device__ __forceinline__ void write_key_tile_flat(const KeyFlatSink& sink, int64_t tile, int d, int mb, int mse_only,
+                                                    const uint8_t* sidx, const uint8_t* ssgn, const float* snorm,
+                                                    const float* srn, const int* svalid, int tid, int nthreads) {
+  using E = Elem<DT>;
+  const int eff = eff_bits(mb), per = 8 / eff, row = idx_row_bytes(d, mb), srow = d >> 3;
+  for (int o = tid; o < TILE * row; o += nthreads) {
+    int t = o / row, k = o - t * row;
+    if (!svalid[t]) continue;
+    unsigned byte = 0;
+    for (int s = 0; s < per; ++s) {
+      int c = k * per + s;
+      if (c < d) byte |= (unsigned)sidx[t * d + c] << (eff * s);
+    }
+    sink.idx[(tile * TILE + t) * row + k] = (uint8_t)byte;
+  }
+  if (!mse_only) {
+    for (int o = tid; o < TILE * srow; o += nthreads) {
+      int t = o / srow, k = o - t * srow;
+      if (!svalid[t]) continue;
+      unsigned byte = 0;
+      for (int s = 0; s < 8; ++s) byte |= (unsigned)ssgn[t * d + k * 8 + s] << s;
+      sink.sign[(tile * TILE + t) * srow + k] = (uint8_t)byte;
+    }
+  }
+  if (tid < TILE && svalid[tid]) {
+    int64_t v = tile * TILE + tid;
+    E::store(sink.norm, v, snorm[tid]);
+    if (!mse_only) sink.rnorm[v] = srn[tid];
+  }
+}
+
+__device__ __forceinline__ void write_key_tile_paged(const KeyPagedSink& sink, const PagedSource& src, int tile, int d,
+                                                     int mb, const uint8_t* sidx, const uint8_t* ssgn,
+                                                     const float* snorm, const float* srn, const int* svalid, int tid,
+                                                     int nthreads) {
+  int b, lpage, h;
+  src.decode(tile, b, lpage, h);
+  const tq_page_layout& L = sink.L;
+  int64_t page = sink.block_table[(int64_t)b * sink.max_pages + lpage];
+  uint8_t* pg = sink.pool + (page * src.H + h) * (int64_t)L.page_bytes;
+  const int words = d >> 5, planes = mb + 1;
+  for (int o = tid; o < planes * words * TILE; o += nthreads) {
+    int n = o % TILE, r = o / TILE;
+    int w = r % words, p = r / words;
+    if (!svalid[n]) continue;
+    uint32_t bits = 0;
+    if (p < mb) {
+      int sh = mb - 1 - p;
+      for (int i = 0; i < 32; ++i) bits |= (uint32_t)((sidx[n * d + w * 32 + i] >> sh) & 1) << i;
+    } else {
+      for (int i = 0; i < 32; ++i) bits |= (uint32_t)ssgn[n * d + w * 32 + i] << i;
+    }
+    *(uint32_t*)(pg + key_word_off(L, p, w, n)) = bits;
+  }
+  if (tid < TILE && svalid[tid]) {
+    ((float*)(pg + L.off_meta))[2 * tid] = snorm[tid];
+    ((float*)(pg + L.off_meta))[2 * tid + 1] = srn[tid];
+  }
+}
+
+}  // namespace tq

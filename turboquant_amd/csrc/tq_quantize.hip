@@ -7,13 +7,9 @@
 // three d x d contractions run in fp32 on the vector ALUs with the tile staged
 // in LDS; matrices are read column-coalesced from their row-major transposes.
 
-#include <type_traits>
-
-#include "tq_common.h"
+#include "tq_quantize.h"
 
 namespace tq {
-
-constexpr int TILE = TQ_PAGE_TOKENS;
 
 // ------------------------------------------------------------------------------------
 // parity entry points: bucketise+pack and sign-pack from given fp32 tensors
@@ -52,62 +48,6 @@ __global__ void sign_pack_kernel(const float* __restrict__ p, int64_t n_vec, int
   }
   out[gid] = (uint8_t)byte;
 }
-
-// ------------------------------------------------------------------------------------
-// tile sources: where the 16 vectors of a tile come from and which are valid
-// ------------------------------------------------------------------------------------
-
-struct FlatSource {          // (n_vec, d) with a row stride
-  int64_t n_vec, row_stride;
-  __device__ bool locate(int tile, int slot, int64_t& elem_off) const {
-    int64_t v = (int64_t)tile * TILE + slot;
-    elem_off = v * row_stride;
-    return v < n_vec;
-  }
-};
-
-struct PagedSource {         // (b, t, h, :) strided, tokens mapped onto 16-token pages
-  int B, T, H, tiles_per_seq;
-  int64_t stride_b, stride_t, stride_h;
-  const int32_t* start_pos;
-  // tile index -> (b, page slot window, head)
-  __device__ void decode(int tile, int& b, int& lpage, int& h) const {
-    h = tile % H;
-    int r = tile / H;
-    int pg = r % tiles_per_seq;
-    b = r / tiles_per_seq;
-    int s0 = start_pos ? start_pos[b] : 0;
-    lpage = s0 / TILE + pg;
-  }
-  __device__ bool locate(int tile, int slot, int64_t& elem_off) const {
-    int b, lpage, h;
-    decode(tile, b, lpage, h);
-    int s0 = start_pos ? start_pos[b] : 0;
-    int t = lpage * TILE + slot - s0;
-    elem_off = b * stride_b + (int64_t)t * stride_t + h * stride_h;
-    return t >= 0 && t < T;
-  }
-};
-
-// ------------------------------------------------------------------------------------
-// key tile
-// ------------------------------------------------------------------------------------
-
-struct KeyFlatSink {
-  uint8_t* idx;
-  uint8_t* sign;
-  void* norm;
-  float* rnorm;
-  float* y_dbg;
-  float* p_dbg;
-};
-
-struct KeyPagedSink {
-  uint8_t* pool;
-  const int32_t* block_table;
-  int max_pages;
-  tq_page_layout L;
-};
 
 template <int DT, class Source, class Sink>
 __global__ void __launch_bounds__(1024)
@@ -230,57 +170,10 @@ key_tile_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
   __syncthreads();
 
   // (7) write
-  if constexpr (std::is_same<Sink, KeyFlatSink>::value) {
-    const int eff = eff_bits(mb), per = 8 / eff, row = idx_row_bytes(d, mb), srow = d >> 3;
-    for (int o = j; o < TILE * row; o += d) {
-      int t = o / row, k = o - t * row;
-      if (!svalid[t]) continue;
-      unsigned byte = 0;
-      for (int s = 0; s < per; ++s) {
-        int c = k * per + s;
-        if (c < d) byte |= (unsigned)sidx[t * d + c] << (eff * s);
-      }
-      sink.idx[((int64_t)tile * TILE + t) * row + k] = (uint8_t)byte;
-    }
-    if (!mse_only) {
-      for (int o = j; o < TILE * srow; o += d) {
-        int t = o / srow, k = o - t * srow;
-        if (!svalid[t]) continue;
-        unsigned byte = 0;
-        for (int s = 0; s < 8; ++s) byte |= (unsigned)ssgn[t * d + k * 8 + s] << s;
-        sink.sign[((int64_t)tile * TILE + t) * srow + k] = (uint8_t)byte;
-      }
-    }
-    if (j < TILE && svalid[j]) {
-      int64_t v = (int64_t)tile * TILE + j;
-      E::store(sink.norm, v, snorm[j]);
-      if (!mse_only) sink.rnorm[v] = srn[j];
-    }
-  } else {
-    int b, lpage, h;
-    src.decode(tile, b, lpage, h);
-    const tq_page_layout& L = sink.L;
-    int64_t page = sink.block_table[(int64_t)b * sink.max_pages + lpage];
-    uint8_t* pg = sink.pool + (page * src.H + h) * (int64_t)L.page_bytes;
-    const int words = d >> 5, planes = mb + 1;
-    for (int o = j; o < planes * words * TILE; o += d) {
-      int n = o % TILE, r = o / TILE;
-      int w = r % words, p = r / words;
-      if (!svalid[n]) continue;
-      uint32_t bits = 0;
-      if (p < mb) {
-        int sh = mb - 1 - p;
-        for (int i = 0; i < 32; ++i) bits |= (uint32_t)((sidx[n * d + w * 32 + i] >> sh) & 1) << i;
-      } else {
-        for (int i = 0; i < 32; ++i) bits |= (uint32_t)ssgn[n * d + w * 32 + i] << i;
-      }
-      *(uint32_t*)(pg + key_word_off(L, p, w, n)) = bits;
-    }
-    if (j < TILE && svalid[j]) {
-      ((float*)(pg + L.off_meta))[2 * j] = snorm[j];
-      ((float*)(pg + L.off_meta))[2 * j + 1] = srn[j];
-    }
-  }
+  if constexpr (std::is_same<Sink, KeyFlatSink>::value)
+    write_key_tile_flat<DT>(sink, tile, d, mb, mse_only, sidx, ssgn, snorm, srn, svalid, j, d);
+  else
+    write_key_tile_paged(sink, src, tile, d, mb, sidx, ssgn, snorm, srn, svalid, j, d);
 }
 
 static size_t key_tile_smem(int d) { return (size_t)TILE * d * (4 + 4 + 1 + 1) + (TILE * 2 + 16) * 4 + TILE * 4; }
@@ -551,9 +444,19 @@ extern "C" int tq_sign_pack(const float* p, int64_t n_vec, int d, uint8_t* sign_
   return TQ_OK;
 }
 
+namespace tq {
+template <class Source, class Sink>
+int launch_key_mfma(const void* x, int dtype, const Source& src, const tq_layer& ly, const Sink& sink, int mse_only,
+                    int64_t tiles, hipStream_t st);
+}
+
 template <class Source, class Sink>
 static int launch_key(const void* x, int dtype, const Source& src, const tq_layer& ly, const Sink& sink, int mse_only,
                       int64_t tiles, hipStream_t st) {
+  {  // matrix-core kernel when the layer carries split matrices and head_dim is 128 / 256
+    int rc = launch_key_mfma(x, dtype, src, ly, sink, mse_only, tiles, st);
+    if (rc != TQ_EUNSUPPORTED) return rc;
+  }
   size_t smem = key_tile_smem(ly.d);
   dim3 grid((unsigned)tiles), block(ly.d);
 #define TQ_LAUNCH_KEY(DT)                                                                              \

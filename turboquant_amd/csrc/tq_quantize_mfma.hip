@@ -1,0 +1,503 @@
+// Key quantiser on the matrix cores (gfx950, bf16 MFMA 16x16x32).
+//
+// The three d x d contractions of the reference (y = u Pi^T, x_hat = c[idx] Pi,
+// p = r S^T; quantizer.py:141,160,248) need fp32-class accuracy, because an index
+// or a sign flips whenever a result crosses a threshold.  Every fp32 number is the
+// exact sum of three bf16 numbers (8 + 8 + 8 significand bits), so each operand is
+// split into bf16 terms and the product is assembled from bf16 MFMAs whose partial
+// products are exact; terms (a, b) with a + b > 2 are below fp32 resolution and are
+// skipped.  The matrices are split once per layer on the host; inputs that already
+// are bf16 need a single term.
+//
+// One workgroup (4 wavefronts) owns TT = 8192/d vectors (TT/16 tiles of 16) and
+// keeps about 72 KB of LDS, so two workgroups share a compute unit and one's
+// epilogues overlap the other's MFMAs.  The vectors' operand terms sit in LDS (row
+// stride padded so that the 16 rows of an MFMA operand fall into different banks);
+// a wavefront owns d/64 column tiles of the output for all TT vectors, keeps the
+// matrix terms of the current 32-wide slice of the contraction in registers (next
+// slice prefetched), and re-reads the vector terms from LDS.  The matrix rows are
+// the MFMA's row operand, so a lane ends up with four consecutive output columns
+// of one vector: terms for the next contraction go back to LDS as 8-byte writes and
+// the index / sign bits of a vector are gathered into 32-bit plane words with two
+// cross-lane exchanges.  The three contractions are separated by workgroup barriers
+// because each needs complete rows of the previous result.
+
+#include <atomic>
+
+#include "tq_quantize.h"
+
+namespace tq {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ f32x4 mfma_bf16(const u32x4& rows, const u32x4& cols, f32x4 c) {
+  bf16x8 av, bv;
+  __builtin_memcpy(&av, &rows, 16);
+  __builtin_memcpy(&bv, &cols, 16);
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, bv, c, 0, 0, 0);
+}
+
+// two fp32 -> packed bf16 (first value in the low half), round to nearest even
+__device__ __forceinline__ uint32_t cvt_pk_bf16(float a, float b) {
+  f32x2 v = {a, b};
+  bf16x2 r = __builtin_convertvector(v, bf16x2);
+  uint32_t u;
+  __builtin_memcpy(&u, &r, 4);
+  return u;
+}
+
+// (v0, v1) = t[0] + t[1] + t[2] lane-wise, each term a packed pair of bf16: a term is
+// the rounding of what the previous terms left, and every remainder is exact in fp32
+__device__ __forceinline__ void split3_pk(float v0, float v1, uint32_t (&t)[3]) {
+  t[0] = cvt_pk_bf16(v0, v1);
+  float r0 = v0 - __uint_as_float(t[0] << 16), r1 = v1 - __uint_as_float(t[0] & 0xffff0000u);
+  t[1] = cvt_pk_bf16(r0, r1);
+  r0 -= __uint_as_float(t[1] << 16);
+  r1 -= __uint_as_float(t[1] & 0xffff0000u);
+  t[2] = cvt_pk_bf16(r0, r1);
+}
+
+// N consecutive elements of the input dtype from LDS (16-byte aligned) as fp32
+template <int DT, int N>
+__device__ __forceinline__ void load_run(const typename Elem<DT>::storage* p, float (&out)[N]) {
+  if constexpr (DT == TQ_F32) {
+#pragma unroll
+    for (int c = 0; c < N; c += 4) {
+      const f32x4 v = *(const f32x4*)(p + c);
+      out[c] = v.x; out[c + 1] = v.y; out[c + 2] = v.z; out[c + 3] = v.w;
+    }
+  } else if constexpr (N % 8 == 0) {
+#pragma unroll
+    for (int c = 0; c < N; c += 8) {
+      const u32x4 v = *(const u32x4*)(p + c);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        out[c + 2 * k] = Elem<DT>::load(&v, 2 * k);
+        out[c + 2 * k + 1] = Elem<DT>::load(&v, 2 * k + 1);
+      }
+    }
+  } else {
+    static_assert(N == 4, "runs of 4 or a multiple of 8");
+    const u32x2 v = *(const u32x2*)p;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) out[k] = Elem<DT>::load(&v, k);
+  }
+}
+
+template <int DT> struct InTerms;                       // bf16 terms that represent a value of the input dtype exactly
+template <> struct InTerms<TQ_BF16> { static constexpr int N = 1; };
+template <> struct InTerms<TQ_F16> { static constexpr int N = 2; };
+template <> struct InTerms<TQ_F32> { static constexpr int N = 3; };
+
+constexpr int KQ_WAVES = 4;
+constexpr int KQ_THREADS = KQ_WAVES * 64;
+constexpr int KQ_MAX_PLANES = 5;                        // 4 index bits + sign
+
+template <int D>
+struct KeyGeom {
+  static constexpr int TT = 8192 / D;                   // vectors per workgroup
+  static constexpr int MT = TT / 16;                    // 16-vector tiles per workgroup
+  static constexpr int NPW = D / 16 / KQ_WAVES;         // output column tiles per wavefront
+  static constexpr int KB = D / 32;                     // 32-wide slices of the contraction
+  static constexpr int RS = D + 8;                      // LDS row stride of a term tile, in bf16
+  static constexpr int W = D / 32;                      // 32-bit words per bit plane of a vector
+  static constexpr int TPR = KQ_THREADS / TT;           // threads that share a vector in the norm pass
+  static constexpr int SEG = D / TPR;                   // = 32 elements per thread
+};
+
+template <int DT, int D>
+struct KeySmem {
+  using G = KeyGeom<D>;
+  using S = typename Elem<DT>::storage;
+  static constexpr int XRS = D + 16 / (int)sizeof(S);                       // padded row of the input tile
+  static constexpr size_t off_x = 0;
+  static constexpr size_t off_terms = (size_t)G::TT * XRS * sizeof(S);      // 3 term tiles [TT][RS] bf16
+  static constexpr size_t off_planes = off_terms + 3 * (size_t)G::TT * G::RS * 2;   // [plane][TT][W] words
+  static constexpr size_t off_small = off_planes + (size_t)KQ_MAX_PLANES * G::TT * G::W * 4;
+  // snorm[TT] srn[TT] spart[4][TT] svalid[TT] sthr[16] slut[16] (8 bytes each)
+  static constexpr size_t bytes = off_small + (size_t)G::TT * (3 + KQ_WAVES) * 4 + 16 * 4 + 16 * 8;
+};
+
+// One contraction: out[t][n] = sum_k A[t][k] * M[n][k] for the wavefront's column tiles.
+// a_terms tiles in LDS ([term][TT][RS] bf16), matrix terms in global ([term][D][D] bf16, row n
+// holds the coefficients of output n).  NA vector terms, 3 matrix terms, pairs with a + b <= 2.
+// acc[m][c][i] = out[16 m + (lane & 15)][16 (wave NPW + c) + 4 (lane >> 4) + i].
+template <int D, int NA>
+__device__ __forceinline__ void contract(const uint16_t* a_terms, const uint16_t* __restrict__ m_terms, int wave,
+                                         int lane, f32x4 (&acc)[KeyGeom<D>::MT][KeyGeom<D>::NPW]) {
+  using Gm = KeyGeom<D>;
+  constexpr int MT = Gm::MT, NPW = Gm::NPW, KB = Gm::KB, RS = Gm::RS;
+  const int n = lane & 15, kb = lane >> 4;
+#pragma unroll
+  for (int m = 0; m < MT; ++m)
+#pragma unroll
+    for (int c = 0; c < NPW; ++c) acc[m][c] = f32x4{0, 0, 0, 0};
+  u32x4 bcur[NPW][3], bnxt[NPW][3];
+  auto load_b = [&](int kblk, u32x4 (&dst)[NPW][3]) {
+#pragma unroll
+    for (int c = 0; c < NPW; ++c) {
+      const int row = 16 * (wave * NPW + c) + n;
+#pragma unroll
+      for (int b = 0; b < 3; ++b)
+        dst[c][b] = *(const u32x4*)(m_terms + ((size_t)b * D + row) * D + 32 * kblk + 8 * kb);
+    }
+  };
+  load_b(0, bcur);
+#pragma unroll
+  for (int kblk = 0; kblk < KB; ++kblk) {
+    if (kblk + 1 < KB) load_b(kblk + 1, bnxt);
+    u32x4 av[MT][NA];
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int a = 0; a < NA; ++a)
+        av[m][a] = *(const u32x4*)(a_terms + ((size_t)a * Gm::TT + 16 * m + n) * RS + 32 * kblk + 8 * kb);
+    // consecutive MFMAs go to different accumulators
+#pragma unroll
+    for (int a = 0; a < NA; ++a)
+#pragma unroll
+      for (int b = 0; b < 3; ++b)
+        if (a + b <= 2) {
+#pragma unroll
+          for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int c = 0; c < NPW; ++c) acc[m][c] = mfma_bf16(bcur[c][b], av[m][a], acc[m][c]);
+        }
+    if (kblk + 1 < KB) {
+#pragma unroll
+      for (int c = 0; c < NPW; ++c)
+#pragma unroll
+        for (int b = 0; b < 3; ++b) bcur[c][b] = bnxt[c][b];
+    }
+  }
+}
+
+// OR a value over the four lanes that hold the same vector (lane & 15 equal)
+__device__ __forceinline__ uint32_t or_over_kb(uint32_t v) {
+  v |= (uint32_t)__shfl_xor((int)v, 16, 64);
+  v |= (uint32_t)__shfl_xor((int)v, 32, 64);
+  return v;
+}
+
+template <int DT, int D, class Source, class Sink>
+__global__ void __launch_bounds__(KQ_THREADS, 2)
+key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, int mse_only, int64_t n_tiles) {
+  using E = Elem<DT>;
+  using S = typename E::storage;
+  using Gm = KeyGeom<D>;
+  using Sm = KeySmem<DT, D>;
+  constexpr int TT = Gm::TT, MT = Gm::MT, NPW = Gm::NPW, RS = Gm::RS, W = Gm::W, NA1 = InTerms<DT>::N;
+  constexpr int XRS = Sm::XRS, TPR = Gm::TPR, SEG = Gm::SEG;
+  constexpr int CH = 16 / (int)sizeof(S);                       // elements per 16-byte chunk of the input
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n = lane & 15, kb = lane >> 4;
+  const int mb = ly.mse_bits, n_thr = (1 << mb) - 1;
+  const int64_t tile0 = (int64_t)blockIdx.x * MT;
+
+  extern __shared__ __align__(16) unsigned char smem[];
+  S* sx = (S*)(smem + Sm::off_x);                               // [TT][XRS] input
+  uint16_t* terms = (uint16_t*)(smem + Sm::off_terms);          // [3][TT][RS]: unit vector, then centroids, then residual
+  uint32_t* spl = (uint32_t*)(smem + Sm::off_planes);           // [plane][TT][W]
+  float* snorm = (float*)(smem + Sm::off_small);                // [TT]
+  float* srn = snorm + TT;                                      // [TT]
+  float* spart = srn + TT;                                      // [KQ_WAVES][TT] partial sums of r^2
+  int* svalid = (int*)(spart + KQ_WAVES * TT);                  // [TT]
+  float* sthr = (float*)(svalid + TT);                          // [16]
+  u32x2* slut = (u32x2*)(sthr + 16);                            // [16] bf16 terms of a centroid: {t0 | t1 << 16, t2}
+
+  if (tid < n_thr) sthr[tid] = ly.thresholds[tid];
+  if (tid < (1 << mb)) {
+    uint32_t t[3];
+    split3_pk(ly.centroids[tid], 0.0f, t);
+    slut[tid] = u32x2{(t[0] & 0xffffu) | (t[1] << 16), t[2] & 0xffffu};
+  }
+  // (1) stage TT vectors: every thread issues its 16-byte loads before it stores any
+  {
+    constexpr int CPR = D / CH;                                 // chunks per vector
+    constexpr int PER = TT * CPR / KQ_THREADS;                  // chunks per thread
+    u32x4 buf[PER];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int q = tid + KQ_THREADS * j, t = q / CPR, ck = q % CPR;
+      int64_t off;
+      const int64_t tile = tile0 + t / TILE;
+      const bool ok = tile < n_tiles && src.locate((int)tile, t % TILE, off);
+      buf[j] = ok ? *(const u32x4*)((const S*)x + off + ck * CH) : u32x4{0, 0, 0, 0};
+      if (ck == 0) svalid[t] = ok;
+    }
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int q = tid + KQ_THREADS * j, t = q / CPR, ck = q % CPR;
+      *(u32x4*)(sx + t * XRS + ck * CH) = buf[j];
+    }
+  }
+  __syncthreads();
+  // (2) norm, unit vector in the input dtype (quantizer.py:136-138), its bf16 terms.
+  //     TPR neighbouring threads share a vector, 32 coordinates each.
+  {
+    const int t = tid / TPR, seg = tid % TPR;
+    float xs[SEG];
+    load_run<DT, SEG>(sx + t * XRS + seg * SEG, xs);
+    float ss = 0.0f;
+#pragma unroll
+    for (int c = 0; c < SEG; ++c) ss += xs[c] * xs[c];
+#pragma unroll
+    for (int o = 1; o < TPR; o <<= 1) ss += __shfl_xor(ss, o, 64);
+    const float nrm = E::round(sqrtf(ss));
+    const float den = E::round(nrm + 1e-10f);
+    if (seg == 0) snorm[t] = nrm;
+#pragma unroll
+    for (int c8 = 0; c8 < SEG; c8 += 8) {
+      uint32_t pk[3][4];
+#pragma unroll
+      for (int c = 0; c < 8; c += 2) {
+        uint32_t tm[3];
+        split3_pk(E::round(xs[c8 + c] / den), E::round(xs[c8 + c + 1] / den), tm);
+#pragma unroll
+        for (int a = 0; a < 3; ++a) pk[a][c >> 1] = tm[a];
+      }
+#pragma unroll
+      for (int a = 0; a < NA1; ++a)
+        *(u32x4*)(terms + ((size_t)a * TT + t) * RS + seg * SEG + c8) = u32x4{pk[a][0], pk[a][1], pk[a][2], pk[a][3]};
+    }
+  }
+  __syncthreads();
+
+  f32x4 acc[MT][NPW];
+  // (3) y = u Pi^T, bucketise; index bit planes; centroid values as bf16 terms for the next contraction
+  contract<D, NA1>(terms, ly.Pi_split, wave, lane, acc);
+  __syncthreads();                                              // every wavefront has read the unit-vector terms
+  {
+    uint32_t idx[MT][NPW][4];
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int c = 0; c < NPW; ++c)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) idx[m][c][i] = 0;
+    for (int k = 0; k < n_thr; ++k) {                           // searchsorted: count thresholds below y (NaN counts all)
+      const float th = sthr[k];
+#pragma unroll
+      for (int m = 0; m < MT; ++m)
+#pragma unroll
+        for (int c = 0; c < NPW; ++c)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) idx[m][c][i] += !(acc[m][c][i] <= th);
+    }
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+      const int t = 16 * m + n;
+      for (int p = 0; p < mb; ++p) {
+        const int sh = mb - 1 - p;
+#pragma unroll
+        for (int wl = 0; wl < NPW / 2; ++wl) {
+          uint32_t v = 0;
+#pragma unroll
+          for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) v |= ((idx[m][2 * wl + h][i] >> sh) & 1u) << (16 * h + 4 * kb + i);
+          v = or_over_kb(v);
+          if (kb == 0) spl[(p * TT + t) * W + (wave * NPW) / 2 + wl] = v;
+        }
+      }
+#pragma unroll
+      for (int c = 0; c < NPW; ++c) {
+        const int col0 = 16 * (wave * NPW + c) + 4 * kb;
+        u32x2 e[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) e[i] = slut[idx[m][c][i]];
+        // term 0: low halves of .x, term 1: high halves of .x, term 2: low halves of .y
+        const u32x2 t0{(e[0].x & 0xffffu) | (e[1].x << 16), (e[2].x & 0xffffu) | (e[3].x << 16)};
+        const u32x2 t1{(e[0].x >> 16) | (e[1].x & 0xffff0000u), (e[2].x >> 16) | (e[3].x & 0xffff0000u)};
+        const u32x2 t2{e[0].y | (e[1].y << 16), e[2].y | (e[3].y << 16)};
+        *(u32x2*)(terms + ((size_t)0 * TT + t) * RS + col0) = t0;
+        *(u32x2*)(terms + ((size_t)1 * TT + t) * RS + col0) = t1;
+        *(u32x2*)(terms + ((size_t)2 * TT + t) * RS + col0) = t2;
+        if constexpr (std::is_same<Sink, KeyFlatSink>::value) {
+          if (sink.y_dbg && svalid[t]) *(f32x4*)(sink.y_dbg + (tile0 * TILE + t) * D + col0) = acc[m][c];
+        }
+      }
+    }
+  }
+  __syncthreads();
+  if (!mse_only) {
+    // (4) x_hat = (c Pi) * norm ; r = x - x_hat ; ||r||^2 partial sums ; r as bf16 terms (quantizer.py:241-245)
+    contract<D, 3>(terms, ly.PiT_split, wave, lane, acc);
+    __syncthreads();                                            // every wavefront has read the centroid terms
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+      const int t = 16 * m + n;
+      const float nrm = snorm[t];
+      float rs = 0.0f;
+#pragma unroll
+      for (int c = 0; c < NPW; ++c) {
+        const int col0 = 16 * (wave * NPW + c) + 4 * kb;
+        float r[4], xv[4];
+        load_run<DT, 4>(sx + t * XRS + col0, xv);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float xh = acc[m][c][i] * nrm;
+          r[i] = xv[i] - xh;
+          rs += r[i] * r[i];
+        }
+        uint32_t lo[3], hi[3];
+        split3_pk(r[0], r[1], lo);
+        split3_pk(r[2], r[3], hi);
+#pragma unroll
+        for (int a = 0; a < 3; ++a) *(u32x2*)(terms + ((size_t)a * TT + t) * RS + col0) = u32x2{lo[a], hi[a]};
+      }
+      rs += __shfl_xor(rs, 16, 64);
+      rs += __shfl_xor(rs, 32, 64);
+      if (kb == 0) spart[wave * TT + t] = rs;
+    }
+    __syncthreads();
+    if (tid < TT) {
+      float v = 0.0f;
+#pragma unroll
+      for (int w = 0; w < KQ_WAVES; ++w) v += spart[w * TT + tid];
+      srn[tid] = sqrtf(v);
+    }
+    // (5) p = r S^T ; sign bits (quantizer.py:248-249)
+    contract<D, 3>(terms, ly.S_split, wave, lane, acc);
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+      const int t = 16 * m + n;
+#pragma unroll
+      for (int wl = 0; wl < NPW / 2; ++wl) {
+        uint32_t v = 0;
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) v |= (uint32_t)(acc[m][2 * wl + h][i] > 0.0f) << (16 * h + 4 * kb + i);
+        v = or_over_kb(v);
+        if (kb == 0) spl[(mb * TT + t) * W + (wave * NPW) / 2 + wl] = v;
+      }
+      if constexpr (std::is_same<Sink, KeyFlatSink>::value) {
+        if (sink.p_dbg && svalid[t]) {
+#pragma unroll
+          for (int c = 0; c < NPW; ++c)
+            *(f32x4*)(sink.p_dbg + (tile0 * TILE + t) * D + 16 * (wave * NPW + c) + 4 * kb) = acc[m][c];
+        }
+      }
+    }
+  }
+  __syncthreads();
+  // (6) write
+  if constexpr (std::is_same<Sink, KeyFlatSink>::value) {
+    // flat format of the reference (quantizer.py:38-69): indices packed eff_bits apiece, signs 8 per byte
+    const int eff = eff_bits(mb), per = 8 / eff, row = idx_row_bytes(D, mb);
+    for (int o = tid; o < TT * row; o += KQ_THREADS) {
+      const int t = o / row, k = o - t * row;
+      if (!svalid[t]) continue;
+      unsigned byte = 0;
+      for (int s = 0; s < per; ++s) {
+        const int c = k * per + s;
+        unsigned v = 0;
+        for (int p = 0; p < mb; ++p) v |= ((spl[(p * TT + t) * W + (c >> 5)] >> (c & 31)) & 1u) << (mb - 1 - p);
+        byte |= v << (eff * s);
+      }
+      sink.idx[(tile0 * TILE + t) * row + k] = (uint8_t)byte;
+    }
+    if (!mse_only) {
+      for (int o = tid; o < TT * W; o += KQ_THREADS) {
+        const int t = o / W, w = o - t * W;
+        if (svalid[t]) ((uint32_t*)sink.sign)[(tile0 * TILE + t) * W + w] = spl[(mb * TT + t) * W + w];
+      }
+    }
+    if (tid < TT && svalid[tid]) {
+      const int64_t v = tile0 * TILE + tid;
+      E::store(sink.norm, v, snorm[tid]);
+      if (!mse_only) sink.rnorm[v] = srn[tid];
+    }
+  } else {
+    // pages: bit-plane words in page order (lane-major: [w & 3][token][plane][w >> 2]), so that
+    // neighbouring threads write neighbouring words
+    const tq_page_layout& L = sink.L;
+    const int planes = mb + 1, per_page = planes * W * TILE;
+    for (int o = tid; o < MT * per_page; o += KQ_THREADS) {
+      const int m = o / per_page;
+      int q = o - m * per_page;
+      const int jh = q % (W / 4); q /= (W / 4);
+      const int p = q % planes; q /= planes;
+      const int nn = q % TILE, jl = q / TILE;
+      const int64_t tile = tile0 + m;
+      if (tile >= n_tiles || !svalid[16 * m + nn]) continue;
+      int b, lpage, h;
+      src.decode((int)tile, b, lpage, h);
+      const int64_t page = sink.block_table[(int64_t)b * sink.max_pages + lpage];
+      uint8_t* pg = sink.pool + (page * src.H + h) * (int64_t)L.page_bytes;
+      const int w = jh * 4 + jl;
+      *(uint32_t*)(pg + key_word_off(L, p, w, nn)) = (p == mb && mse_only) ? 0u : spl[(p * TT + 16 * m + nn) * W + w];
+    }
+    if (tid < TT && svalid[tid]) {
+      const int64_t tile = tile0 + tid / TILE;
+      int b, lpage, h;
+      src.decode((int)tile, b, lpage, h);
+      const int64_t page = sink.block_table[(int64_t)b * sink.max_pages + lpage];
+      float* meta = (float*)(sink.pool + (page * src.H + h) * (int64_t)L.page_bytes + L.off_meta);
+      meta[2 * (tid % TILE)] = snorm[tid];
+      meta[2 * (tid % TILE) + 1] = mse_only ? 0.0f : srn[tid];
+    }
+  }
+}
+
+__host__ static bool aligned_for_chunks(const void* x, int dtype, const FlatSource& s) {
+  const int64_t ch = 16 / elem_bytes(dtype);
+  return (uintptr_t)x % 16 == 0 && s.row_stride % ch == 0;
+}
+__host__ static bool aligned_for_chunks(const void* x, int dtype, const PagedSource& s) {
+  const int64_t ch = 16 / elem_bytes(dtype);
+  return (uintptr_t)x % 16 == 0 && s.stride_b % ch == 0 && s.stride_t % ch == 0 && s.stride_h % ch == 0;
+}
+__host__ static bool sink_ok(const KeyFlatSink& s, int mse_only) {
+  return (uintptr_t)s.y_dbg % 16 == 0 && (uintptr_t)s.p_dbg % 16 == 0 && (mse_only || (uintptr_t)s.sign % 4 == 0);
+}
+__host__ static bool sink_ok(const KeyPagedSink& s, int) { return s.L.key_lane_major != 0; }
+
+template <int DT, int D, class Source, class Sink>
+static int launch_dt_d(const void* x, const Source& src, const tq_layer& ly, const Sink& sink, int mse_only, int64_t tiles,
+                       hipStream_t st) {
+  using Gm = KeyGeom<D>;
+  using Sm = KeySmem<DT, D>;
+  auto kern = key_mfma_kernel<DT, D, Source, Sink>;
+  static std::atomic<uint64_t> configured{0};           // per instantiation, one bit per device; the attribute is sticky
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return TQ_EINVAL;
+  if (dev >= 64 || !(configured.load() >> dev & 1)) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)Sm::bytes);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 64) configured.fetch_or(1ull << dev);
+  }
+  const int64_t groups = (tiles + Gm::MT - 1) / Gm::MT;
+  kern<<<dim3((unsigned)groups), dim3(KQ_THREADS), Sm::bytes, st>>>(x, src, ly, sink, mse_only, tiles);
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? TQ_OK : (int)e;
+}
+
+// TQ_EUNSUPPORTED when there is no matrix-core kernel for this call (head_dim other than
+// 128 / 256, no split matrices, or operands not aligned for 16-byte loads): the caller
+// falls back to the vector-ALU kernel.
+template <class Source, class Sink>
+int launch_key_mfma(const void* x, int dtype, const Source& src, const tq_layer& ly, const Sink& sink, int mse_only,
+                    int64_t tiles, hipStream_t st) {
+  if (!ly.Pi_split || !ly.PiT_split || (!mse_only && !ly.S_split)) return TQ_EUNSUPPORTED;
+  if (ly.mse_bits < 1 || ly.mse_bits > 4) return TQ_EUNSUPPORTED;
+  if (!aligned_for_chunks(x, dtype, src) || !sink_ok(sink, mse_only)) return TQ_EUNSUPPORTED;
+#define TQ_KQ(DT_, D_) \
+  if (dtype == DT_ && ly.d == D_) return launch_dt_d<DT_, D_, Source, Sink>(x, src, ly, sink, mse_only, tiles, st);
+  TQ_KQ(TQ_BF16, 128) TQ_KQ(TQ_BF16, 256) TQ_KQ(TQ_F16, 128) TQ_KQ(TQ_F16, 256) TQ_KQ(TQ_F32, 128) TQ_KQ(TQ_F32, 256)
+#undef TQ_KQ
+  return TQ_EUNSUPPORTED;
+}
+
+template int launch_key_mfma<FlatSource, KeyFlatSink>(const void*, int, const FlatSource&, const tq_layer&,
+                                                      const KeyFlatSink&, int, int64_t, hipStream_t);
+template int launch_key_mfma<PagedSource, KeyPagedSink>(const void*, int, const PagedSource&, const tq_layer&,
+                                                        const KeyPagedSink&, int, int64_t, hipStream_t);
+
+}  // namespace tq

@@ -105,6 +105,7 @@ class TurboQuantMSE(torch.nn.Module):
         # kernel-side companions (not part of the reference's state dict)
         self.register_buffer("_PiT", self.Pi.T.contiguous(), persistent=False)
         self._centroids_host = centroids.detach().float().cpu()
+        self._splits = None           # (Pi, Pi^T[, S]) as bf16 term triples, built on first GPU use
 
     # -- library plumbing ---------------------------------------------------------
     def _layer(self, S: Optional[torch.Tensor] = None, ST: Optional[torch.Tensor] = None) -> _ffi.TqLayer:
@@ -112,8 +113,14 @@ class TurboQuantMSE(torch.nn.Module):
             raise TypeError("the kernels need float32 rotation / codebook buffers")
         if self._PiT.device != self.Pi.device or self._PiT.data_ptr() == 0:
             self._PiT = self.Pi.T.contiguous()
+            self._splits = None
+        key = (self.Pi.data_ptr(), self.Pi._version, None if S is None else (S.data_ptr(), S._version))
+        if self._splits is None or self._splits[0] != key:
+            self._PiT = self.Pi.T.contiguous()
+            self._splits = (key, (_ffi.split_bf16x3(self.Pi), _ffi.split_bf16x3(self._PiT),
+                                  None if S is None else _ffi.split_bf16x3(S)))
         return _ffi.make_layer(self.dim, self.bits, self.Pi, self._PiT, self.centroids, self.decision_boundaries,
-                               S, ST, centroids_host=self._centroids_host)
+                               S, ST, centroids_host=self._centroids_host, splits=self._splits[1])
 
     def quantize(self, x: torch.Tensor) -> MSEQuantized:
         """x (..., d) -> packed indices (..., d*eff/8) and norms (...) in x's dtype."""
@@ -166,8 +173,9 @@ class TurboQuantProd(torch.nn.Module):
         self.qjl_scale = math.sqrt(math.pi / 2.0) / dim
 
     def _layer(self) -> _ffi.TqLayer:
-        if self._ST.device != self.S.device:
+        if self._ST.device != self.S.device or getattr(self, "_ST_version", None) != self.S._version:
             self._ST = self.S.T.contiguous()
+            self._ST_version = self.S._version
         return self.mse_quantizer._layer(self.S, self._ST)
 
     def quantize(self, x: torch.Tensor) -> ProdQuantized:
