@@ -16,12 +16,20 @@ constexpr int TILE = TQ_PAGE_TOKENS;
 
 struct FlatSource {          // (n_vec, d) with a row stride
   int64_t n_vec, row_stride;
+  struct TileRef { int64_t v0; };
+  __device__ TileRef tile_ref(int64_t tile) const { return TileRef{tile * TILE}; }
+  __device__ bool slot_off(const TileRef& r, int slot, int64_t& elem_off) const {
+    elem_off = (r.v0 + slot) * row_stride;
+    return r.v0 + slot < n_vec;
+  }
   __device__ bool locate(int tile, int slot, int64_t& elem_off) const {
     int64_t v = (int64_t)tile * TILE + slot;
     elem_off = v * row_stride;
     return v < n_vec;
   }
 };
+
+__device__ const int32_t k_zero_i32 = 0;
 
 struct PagedSource {         // (b, t, h, :) strided, tokens mapped onto 16-token pages
   int B, T, H, tiles_per_seq;
@@ -35,6 +43,23 @@ struct PagedSource {         // (b, t, h, :) strided, tokens mapped onto 16-toke
     b = r / tiles_per_seq;
     int s0 = start_pos ? start_pos[b] : 0;
     lpage = s0 / TILE + pg;
+  }
+  // the part of locate() that is the same for the 16 slots of a tile
+  struct TileRef { int64_t base; int t0; };
+  __device__ TileRef tile_ref(int64_t tile) const {
+    int h = (int)tile % H;
+    int r = (int)tile / H;
+    int pg = r % tiles_per_seq;
+    int b = r / tiles_per_seq;
+    // one unconditional load (no branch on the null pointer): a load under a branch makes the
+    // compiler wait for every outstanding load at the join
+    int s0 = *(start_pos ? start_pos + b : &k_zero_i32);
+    return TileRef{b * stride_b + h * stride_h, (s0 / TILE + pg) * TILE - s0};
+  }
+  __device__ bool slot_off(const TileRef& r, int slot, int64_t& elem_off) const {
+    int t = r.t0 + slot;
+    elem_off = r.base + (int64_t)t * stride_t;
+    return t >= 0 && t < T;
   }
   __device__ bool locate(int tile, int slot, int64_t& elem_off) const {
     int b, lpage, h;

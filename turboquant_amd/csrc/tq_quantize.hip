@@ -206,18 +206,27 @@ value_tile_kernel(const void* __restrict__ v, Source src, int d, int gs, int bit
   uint8_t* scode = (uint8_t*)(szero + TILE * ng);  // [TILE][d]
   int* svalid = (int*)(scode + TILE * d);     // [TILE]
 
-  for (int t = 0; t < TILE; ++t) {
-    int64_t off;
-    bool ok = src.locate(tile, t, off);
-    sv[t * d + j] = ok ? E::load(v, off + j) : 0.0f;
-    if (j == 0) svalid[t] = ok;
+  {
+    // all 16 loads are issued before any is used, and none sits under a branch (slots that
+    // do not exist read the first vector and are zeroed afterwards)
+    const typename Source::TileRef ref = src.tile_ref(tile);
+    float vals[TILE];
+    unsigned okm = 0;
+#pragma unroll
+    for (int t = 0; t < TILE; ++t) {
+      int64_t off;
+      const bool ok = src.slot_off(ref, t, off);
+      okm |= (unsigned)ok << t;
+      vals[t] = E::load(v, (ok ? off : 0) + j);
+    }
+    if (!okm) return;                          // uniform: validity depends on the slot only
+#pragma unroll
+    for (int t = 0; t < TILE; ++t) {
+      sv[t * d + j] = ((okm >> t) & 1) ? vals[t] : 0.0f;
+      if (j == 0) svalid[t] = (okm >> t) & 1;
+    }
   }
   __syncthreads();
-  {
-    int any = 0;
-    for (int t = 0; t < TILE; ++t) any |= svalid[t];
-    if (!any) return;
-  }
   const float levels = (float)((1 << bits) - 1);
   for (int o = j; o < TILE * ng; o += d) {
     int t = o / ng, g = o - t * ng;

@@ -9,9 +9,11 @@
 // skipped.  The matrices are split once per layer on the host; inputs that already
 // are bf16 need a single term.
 //
-// One workgroup (4 wavefronts) owns TT = 8192/d vectors (TT/16 tiles of 16) and
-// keeps about 72 KB of LDS, so two workgroups share a compute unit and one's
-// epilogues overlap the other's MFMAs.  The vectors' operand terms sit in LDS (row
+// Workgroups (4 wavefronts) are persistent: two per compute unit (about 75 KB of LDS
+// each), each looping over groups of TT = 8192/d vectors (TT/16 tiles of 16).  The next
+// group's vectors are fetched into registers while the current group is worked on, and
+// the matrix operand of a contraction is requested before the epilogue of the previous
+// one, so no global-memory latency sits on the critical path.  The vectors' operand terms sit in LDS (row
 // stride padded so that the 16 rows of an MFMA operand fall into different banks);
 // a wavefront owns d/64 column tiles of the output for all TT vectors, keeps the
 // matrix terms of the current 32-wide slice of the contraction in registers (next
@@ -123,57 +125,71 @@ struct KeySmem {
   static constexpr size_t bytes = off_small + (size_t)G::TT * (3 + KQ_WAVES) * 4 + 16 * 4 + 16 * 8;
 };
 
+// Register copy of the matrix operand: BUF slices of 32 contraction indices for the
+// wavefront's column tiles.  head_dim 128 holds a whole contraction (BUF = KB), so the
+// loads for the next contraction are issued before the current epilogue starts and their
+// latency hides behind it; head_dim 256 keeps a ring that runs BUF - 1 slices ahead.
+template <int D>
+struct MatRegs {
+  static constexpr int BUF = D == 128 ? 4 : 2;
+  u32x4 b[BUF][KeyGeom<D>::NPW][3];
+};
+
+// m_terms: [term][D][D] bf16 in global memory, row n holds the coefficients of output n
+template <int D>
+__device__ __forceinline__ void load_slice(const uint16_t* __restrict__ m_terms, int wave, int lane, int kblk,
+                                           u32x4 (&dst)[KeyGeom<D>::NPW][3]) {
+  // one 32-bit per-lane byte offset; everything else is a uniform constant added to the base pointer
+  const uint32_t lane_off = (uint32_t)(((16 * wave * KeyGeom<D>::NPW + (lane & 15)) * D + 8 * (lane >> 4)) * 2);
+#pragma unroll
+  for (int c = 0; c < KeyGeom<D>::NPW; ++c) {
+#pragma unroll
+    for (int b = 0; b < 3; ++b) {
+      const char* base = (const char*)m_terms + ((size_t)(b * D + 16 * c) * D + 32 * kblk) * 2;
+      dst[c][b] = *(const u32x4*)(base + lane_off);
+    }
+  }
+}
+
+template <int D>
+__device__ __forceinline__ void prefetch_matrix(const uint16_t* __restrict__ m_terms, int wave, int lane, MatRegs<D>& mr) {
+#pragma unroll
+  for (int k = 0; k < MatRegs<D>::BUF; ++k) load_slice<D>(m_terms, wave, lane, k, mr.b[k]);
+}
+
 // One contraction: out[t][n] = sum_k A[t][k] * M[n][k] for the wavefront's column tiles.
-// a_terms tiles in LDS ([term][TT][RS] bf16), matrix terms in global ([term][D][D] bf16, row n
-// holds the coefficients of output n).  NA vector terms, 3 matrix terms, pairs with a + b <= 2.
+// a_terms tiles in LDS ([term][TT][RS] bf16); the first BUF slices of M are in `mr` already.
+// NA vector terms, 3 matrix terms, pairs with a + b <= 2.
 // acc[m][c][i] = out[16 m + (lane & 15)][16 (wave NPW + c) + 4 (lane >> 4) + i].
 template <int D, int NA>
 __device__ __forceinline__ void contract(const uint16_t* a_terms, const uint16_t* __restrict__ m_terms, int wave,
-                                         int lane, f32x4 (&acc)[KeyGeom<D>::MT][KeyGeom<D>::NPW]) {
+                                         int lane, MatRegs<D>& mr, f32x4 (&acc)[KeyGeom<D>::MT][KeyGeom<D>::NPW]) {
   using Gm = KeyGeom<D>;
-  constexpr int MT = Gm::MT, NPW = Gm::NPW, KB = Gm::KB, RS = Gm::RS;
+  constexpr int MT = Gm::MT, NPW = Gm::NPW, KB = Gm::KB, RS = Gm::RS, BUF = MatRegs<D>::BUF;
   const int n = lane & 15, kb = lane >> 4;
 #pragma unroll
   for (int m = 0; m < MT; ++m)
 #pragma unroll
     for (int c = 0; c < NPW; ++c) acc[m][c] = f32x4{0, 0, 0, 0};
-  u32x4 bcur[NPW][3], bnxt[NPW][3];
-  auto load_b = [&](int kblk, u32x4 (&dst)[NPW][3]) {
-#pragma unroll
-    for (int c = 0; c < NPW; ++c) {
-      const int row = 16 * (wave * NPW + c) + n;
-#pragma unroll
-      for (int b = 0; b < 3; ++b)
-        dst[c][b] = *(const u32x4*)(m_terms + ((size_t)b * D + row) * D + 32 * kblk + 8 * kb);
-    }
-  };
-  load_b(0, bcur);
 #pragma unroll
   for (int kblk = 0; kblk < KB; ++kblk) {
-    if (kblk + 1 < KB) load_b(kblk + 1, bnxt);
-    u32x4 av[MT][NA];
-#pragma unroll
-    for (int m = 0; m < MT; ++m)
-#pragma unroll
-      for (int a = 0; a < NA; ++a)
-        av[m][a] = *(const u32x4*)(a_terms + ((size_t)a * Gm::TT + 16 * m + n) * RS + 32 * kblk + 8 * kb);
     // consecutive MFMAs go to different accumulators
 #pragma unroll
-    for (int a = 0; a < NA; ++a)
+    for (int a = 0; a < NA; ++a) {
+      u32x4 av[MT];
+#pragma unroll
+      for (int m = 0; m < MT; ++m)
+        av[m] = *(const u32x4*)(a_terms + ((size_t)a * Gm::TT + 16 * m + n) * RS + 32 * kblk + 8 * kb);
 #pragma unroll
       for (int b = 0; b < 3; ++b)
         if (a + b <= 2) {
 #pragma unroll
           for (int m = 0; m < MT; ++m)
 #pragma unroll
-            for (int c = 0; c < NPW; ++c) acc[m][c] = mfma_bf16(bcur[c][b], av[m][a], acc[m][c]);
+            for (int c = 0; c < NPW; ++c) acc[m][c] = mfma_bf16(mr.b[kblk % BUF][c][b], av[m], acc[m][c]);
         }
-    if (kblk + 1 < KB) {
-#pragma unroll
-      for (int c = 0; c < NPW; ++c)
-#pragma unroll
-        for (int b = 0; b < 3; ++b) bcur[c][b] = bnxt[c][b];
     }
+    if (kblk + BUF < KB) load_slice<D>(m_terms, wave, lane, kblk + BUF, mr.b[kblk % BUF]);
   }
 }
 
@@ -184,9 +200,12 @@ __device__ __forceinline__ uint32_t or_over_kb(uint32_t v) {
   return v;
 }
 
-template <int DT, int D, class Source, class Sink>
+// MSE_ONLY (the stage-1 quantiser alone: no residual, no signs) is a template parameter: as a
+// run-time flag it adds control flow that costs the register allocator its footing.
+template <int DT, int D, bool MSE_ONLY, class Source, class Sink>
 __global__ void __launch_bounds__(KQ_THREADS, 2)
-key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, int mse_only, int64_t n_tiles) {
+key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, int64_t n_tiles) {
+  constexpr int mse_only = MSE_ONLY;
   using E = Elem<DT>;
   using S = typename E::storage;
   using Gm = KeyGeom<D>;
@@ -194,10 +213,11 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
   constexpr int TT = Gm::TT, MT = Gm::MT, NPW = Gm::NPW, RS = Gm::RS, W = Gm::W, NA1 = InTerms<DT>::N;
   constexpr int XRS = Sm::XRS, TPR = Gm::TPR, SEG = Gm::SEG;
   constexpr int CH = 16 / (int)sizeof(S);                       // elements per 16-byte chunk of the input
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int n = lane & 15, kb = lane >> 4;
+  const int tid0 = threadIdx.x, wave0 = __builtin_amdgcn_readfirstlane(tid0 >> 6);
   const int mb = ly.mse_bits, n_thr = (1 << mb) - 1;
-  const int64_t tile0 = (int64_t)blockIdx.x * MT;
+  const int64_t n_groups = (n_tiles + MT - 1) / MT;             // a group = the TT vectors of one pass
+  MatRegs<D> mr;
+  prefetch_matrix<D>(ly.Pi_split, wave0, tid0 & 63, mr);        // in flight while the vectors are staged
 
   extern __shared__ __align__(16) unsigned char smem[];
   S* sx = (S*)(smem + Sm::off_x);                               // [TT][XRS] input
@@ -210,31 +230,59 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
   float* sthr = (float*)(svalid + TT);                          // [16]
   u32x2* slut = (u32x2*)(sthr + 16);                            // [16] bf16 terms of a centroid: {t0 | t1 << 16, t2}
 
-  if (tid < n_thr) sthr[tid] = ly.thresholds[tid];
-  if (tid < (1 << mb)) {
+  if (tid0 < n_thr) sthr[tid0] = ly.thresholds[tid0];
+  if (tid0 < (1 << mb)) {
     uint32_t t[3];
-    split3_pk(ly.centroids[tid], 0.0f, t);
-    slut[tid] = u32x2{(t[0] & 0xffffu) | (t[1] << 16), t[2] & 0xffffu};
+    split3_pk(ly.centroids[tid0], 0.0f, t);
+    slut[tid0] = u32x2{(t[0] & 0xffffu) | (t[1] << 16), t[2] & 0xffffu};
   }
-  // (1) stage TT vectors: every thread issues its 16-byte loads before it stores any
-  {
-    constexpr int CPR = D / CH;                                 // chunks per vector
-    constexpr int PER = TT * CPR / KQ_THREADS;                  // chunks per thread
-    u32x4 buf[PER];
+  // (1) staging: a thread holds its 16-byte chunks of the NEXT group in registers while the
+  //     current group is worked on, so the latency of the loads is never waited for.  The
+  //     KQ_THREADS chunks of one round lie in one tile, so the tile lookup is wavefront-uniform.
+  constexpr int CPR = D / CH;                                   // chunks per vector
+  constexpr int PER = TT * CPR / KQ_THREADS;                    // rounds
+  constexpr int RPR = KQ_THREADS / CPR;                         // vectors per round (<= 16)
+  static_assert(RPR <= TILE && TILE % RPR == 0, "a round of chunks stays inside one tile");
+  u32x4 xbuf[PER];
+  unsigned xok = 0;
+  typename Source::TileRef xref[PER];                           // tile lookups of the group to fetch next
+  auto lookup_x = [&](int64_t group) {
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
-      const int q = tid + KQ_THREADS * j, t = q / CPR, ck = q % CPR;
-      int64_t off;
-      const int64_t tile = tile0 + t / TILE;
-      const bool ok = tile < n_tiles && src.locate((int)tile, t % TILE, off);
-      buf[j] = ok ? *(const u32x4*)((const S*)x + off + ck * CH) : u32x4{0, 0, 0, 0};
-      if (ck == 0) svalid[t] = ok;
+      const int64_t tile = group * MT + (RPR * j) / TILE;
+      xref[j] = src.tile_ref(tile < n_tiles ? tile : 0);
     }
+  };
+  auto issue_x = [&](int64_t group, int tr, int ck) {
+    xok = 0;
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
-      const int q = tid + KQ_THREADS * j, t = q / CPR, ck = q % CPR;
-      *(u32x4*)(sx + t * XRS + ck * CH) = buf[j];
+      const int64_t tile = group * MT + (RPR * j) / TILE;
+      int64_t off = 0;
+      const bool ok = src.slot_off(xref[j], (RPR * j + tr) % TILE, off) && tile < n_tiles;
+      // unconditional load (a load under a branch makes every later wait a wait for all loads);
+      // slots that do not exist read the first vector and are zeroed when they are stored
+      xbuf[j] = *(const u32x4*)((const S*)x + (ok ? off : 0) + ck * CH);
+      xok |= (unsigned)ok << j;
     }
+  };
+  lookup_x(blockIdx.x);
+  issue_x(blockIdx.x, tid0 / CPR, tid0 % CPR);
+
+  for (int64_t g = blockIdx.x; g < n_groups; g += gridDim.x) {
+  // The thread index is re-read through an opaque copy in every pass: otherwise the compiler
+  // hoists all per-thread address arithmetic out of this loop and spills it.
+  int tid = tid0, wave = wave0;
+  asm volatile("" : "+v"(tid), "+s"(wave));
+  const int lane = tid & 63, n = lane & 15, kb = lane >> 4;
+  const int tr = tid / CPR, ck = tid % CPR;
+  const int64_t tile0 = g * MT;
+  lookup_x(g + gridDim.x);                                      // read long before issue_x needs it
+#pragma unroll
+  for (int j = 0; j < PER; ++j) {
+    const bool ok = (xok >> j) & 1;
+    *(u32x4*)(sx + (RPR * j + tr) * XRS + ck * CH) = ok ? xbuf[j] : u32x4{0, 0, 0, 0};
+    if (ck == 0) svalid[RPR * j + tr] = ok;
   }
   __syncthreads();
   // (2) norm, unit vector in the input dtype (quantizer.py:136-138), its bf16 terms.
@@ -256,10 +304,14 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
       uint32_t pk[3][4];
 #pragma unroll
       for (int c = 0; c < 8; c += 2) {
-        uint32_t tm[3];
-        split3_pk(E::round(xs[c8 + c] / den), E::round(xs[c8 + c + 1] / den), tm);
+        if constexpr (DT == TQ_BF16) {                          // the rounded quotient is its own single term
+          pk[0][c >> 1] = cvt_pk_bf16(xs[c8 + c] / den, xs[c8 + c + 1] / den);
+        } else {
+          uint32_t tm[3];
+          split3_pk(E::round(xs[c8 + c] / den), E::round(xs[c8 + c + 1] / den), tm);
 #pragma unroll
-        for (int a = 0; a < 3; ++a) pk[a][c >> 1] = tm[a];
+          for (int a = 0; a < 3; ++a) pk[a][c >> 1] = tm[a];
+        }
       }
 #pragma unroll
       for (int a = 0; a < NA1; ++a)
@@ -270,7 +322,8 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
 
   f32x4 acc[MT][NPW];
   // (3) y = u Pi^T, bucketise; index bit planes; centroid values as bf16 terms for the next contraction
-  contract<D, NA1>(terms, ly.Pi_split, wave, lane, acc);
+  contract<D, NA1>(terms, ly.Pi_split, wave, lane, mr, acc);
+  prefetch_matrix<D>(mse_only ? ly.Pi_split : ly.PiT_split, wave, lane, mr);   // lands during the epilogue
   __syncthreads();                                              // every wavefront has read the unit-vector terms
   {
     uint32_t idx[MT][NPW][4];
@@ -325,9 +378,11 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
     }
   }
   __syncthreads();
+  if (mse_only) issue_x(g + gridDim.x, tr, ck);
   if (!mse_only) {
     // (4) x_hat = (c Pi) * norm ; r = x - x_hat ; ||r||^2 partial sums ; r as bf16 terms (quantizer.py:241-245)
-    contract<D, 3>(terms, ly.PiT_split, wave, lane, acc);
+    contract<D, 3>(terms, ly.PiT_split, wave, lane, mr, acc);
+    prefetch_matrix<D>(ly.S_split, wave, lane, mr);
     __syncthreads();                                            // every wavefront has read the centroid terms
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
@@ -356,6 +411,7 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
       if (kb == 0) spart[wave * TT + t] = rs;
     }
     __syncthreads();
+    issue_x(g + gridDim.x, tr, ck);                                     // the input tile is free: fetch the next group
     if (tid < TT) {
       float v = 0.0f;
 #pragma unroll
@@ -363,7 +419,8 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
       srn[tid] = sqrtf(v);
     }
     // (5) p = r S^T ; sign bits (quantizer.py:248-249)
-    contract<D, 3>(terms, ly.S_split, wave, lane, acc);
+    contract<D, 3>(terms, ly.S_split, wave, lane, mr, acc);
+    prefetch_matrix<D>(ly.Pi_split, wave, lane, mr);            // for the next group
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
       const int t = 16 * m + n;
@@ -415,34 +472,35 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
       if (!mse_only) sink.rnorm[v] = srn[tid];
     }
   } else {
-    // pages: bit-plane words in page order (lane-major: [w & 3][token][plane][w >> 2]), so that
-    // neighbouring threads write neighbouring words
+    // pages: a wavefront writes the bit-plane words of one tile, so the page lookup is uniform;
+    // lanes run over (word, token) in page order (lane-major: [w & 3][token][plane][w >> 2])
     const tq_page_layout& L = sink.L;
-    const int planes = mb + 1, per_page = planes * W * TILE;
-    for (int o = tid; o < MT * per_page; o += KQ_THREADS) {
-      const int m = o / per_page;
-      int q = o - m * per_page;
-      const int jh = q % (W / 4); q /= (W / 4);
-      const int p = q % planes; q /= planes;
-      const int nn = q % TILE, jl = q / TILE;
+    constexpr int NSUB = KQ_WAVES / MT > 0 ? KQ_WAVES / MT : 1;   // wavefronts that share a tile
+    const int planes = mb + 1;
+    for (int m = wave % MT; m < MT; m += KQ_WAVES) {
       const int64_t tile = tile0 + m;
-      if (tile >= n_tiles || !svalid[16 * m + nn]) continue;
+      if (tile >= n_tiles) break;
       int b, lpage, h;
       src.decode((int)tile, b, lpage, h);
       const int64_t page = sink.block_table[(int64_t)b * sink.max_pages + lpage];
       uint8_t* pg = sink.pool + (page * src.H + h) * (int64_t)L.page_bytes;
-      const int w = jh * 4 + jl;
-      *(uint32_t*)(pg + key_word_off(L, p, w, nn)) = (p == mb && mse_only) ? 0u : spl[(p * TT + 16 * m + nn) * W + w];
+      for (int p = wave / MT; p < planes; p += NSUB) {
+#pragma unroll
+        for (int e = lane; e < W * TILE; e += 64) {
+          const int jh = e % (W / 4), nn = (e / (W / 4)) % TILE, jl = e / (W / 4) / TILE;
+          const int w = jh * 4 + jl;
+          if (svalid[16 * m + nn])
+            *(uint32_t*)(pg + key_word_off(L, p, w, nn)) = (p == mb && mse_only) ? 0u : spl[(p * TT + 16 * m + nn) * W + w];
+        }
+      }
+      if (wave / MT == 0 && lane < TILE && svalid[16 * m + lane]) {
+        float* meta = (float*)(pg + L.off_meta);
+        meta[2 * lane] = snorm[16 * m + lane];
+        meta[2 * lane + 1] = mse_only ? 0.0f : srn[16 * m + lane];
+      }
     }
-    if (tid < TT && svalid[tid]) {
-      const int64_t tile = tile0 + tid / TILE;
-      int b, lpage, h;
-      src.decode((int)tile, b, lpage, h);
-      const int64_t page = sink.block_table[(int64_t)b * sink.max_pages + lpage];
-      float* meta = (float*)(sink.pool + (page * src.H + h) * (int64_t)L.page_bytes + L.off_meta);
-      meta[2 * (tid % TILE)] = snorm[tid];
-      meta[2 * (tid % TILE) + 1] = mse_only ? 0.0f : srn[tid];
-    }
+  }
+  __syncthreads();                                              // the next group overwrites what the writers read
   }
 }
 
@@ -459,12 +517,12 @@ __host__ static bool sink_ok(const KeyFlatSink& s, int mse_only) {
 }
 __host__ static bool sink_ok(const KeyPagedSink& s, int) { return s.L.key_lane_major != 0; }
 
-template <int DT, int D, class Source, class Sink>
-static int launch_dt_d(const void* x, const Source& src, const tq_layer& ly, const Sink& sink, int mse_only, int64_t tiles,
+template <int DT, int D, bool MSE_ONLY, class Source, class Sink>
+static int launch_dt_d(const void* x, const Source& src, const tq_layer& ly, const Sink& sink, int64_t tiles,
                        hipStream_t st) {
   using Gm = KeyGeom<D>;
   using Sm = KeySmem<DT, D>;
-  auto kern = key_mfma_kernel<DT, D, Source, Sink>;
+  auto kern = key_mfma_kernel<DT, D, MSE_ONLY, Source, Sink>;
   static std::atomic<uint64_t> configured{0};           // per instantiation, one bit per device; the attribute is sticky
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return TQ_EINVAL;
@@ -473,8 +531,18 @@ static int launch_dt_d(const void* x, const Source& src, const tq_layer& ly, con
     if (e != hipSuccess) return (int)e;
     if (dev < 64) configured.fetch_or(1ull << dev);
   }
+  // persistent workgroups: as many as stay resident (LDS allows 160 KB / bytes per compute unit)
+  static std::atomic<int> n_cu{0};
+  if (!n_cu.load()) {
+    int v = 0;
+    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) v = 256;
+    n_cu.store(v);
+  }
+  const int per_cu = (int)(160 * 1024 / Sm::bytes) > 2 ? 2 : (int)(160 * 1024 / Sm::bytes);
   const int64_t groups = (tiles + Gm::MT - 1) / Gm::MT;
-  kern<<<dim3((unsigned)groups), dim3(KQ_THREADS), Sm::bytes, st>>>(x, src, ly, sink, mse_only, tiles);
+  const int64_t resident = (int64_t)n_cu.load() * (per_cu > 0 ? per_cu : 1);
+  const unsigned grid = (unsigned)(groups < resident ? groups : resident);
+  kern<<<dim3(grid), dim3(KQ_THREADS), Sm::bytes, st>>>(x, src, ly, sink, tiles);
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? TQ_OK : (int)e;
 }
@@ -488,8 +556,14 @@ int launch_key_mfma(const void* x, int dtype, const Source& src, const tq_layer&
   if (!ly.Pi_split || !ly.PiT_split || (!mse_only && !ly.S_split)) return TQ_EUNSUPPORTED;
   if (ly.mse_bits < 1 || ly.mse_bits > 4) return TQ_EUNSUPPORTED;
   if (!aligned_for_chunks(x, dtype, src) || !sink_ok(sink, mse_only)) return TQ_EUNSUPPORTED;
-#define TQ_KQ(DT_, D_) \
-  if (dtype == DT_ && ly.d == D_) return launch_dt_d<DT_, D_, Source, Sink>(x, src, ly, sink, mse_only, tiles, st);
+  constexpr bool paged = std::is_same<Sink, KeyPagedSink>::value;     // pages always hold the full code
+  if (paged && mse_only) return TQ_EUNSUPPORTED;
+#define TQ_KQ(DT_, D_)                                                                                     \
+  if (dtype == DT_ && ly.d == D_) {                                                                        \
+    if constexpr (!paged)                                                                                  \
+      if (mse_only) return launch_dt_d<DT_, D_, true, Source, Sink>(x, src, ly, sink, tiles, st);          \
+    return launch_dt_d<DT_, D_, false, Source, Sink>(x, src, ly, sink, tiles, st);                         \
+  }
   TQ_KQ(TQ_BF16, 128) TQ_KQ(TQ_BF16, 256) TQ_KQ(TQ_F16, 128) TQ_KQ(TQ_F16, 256) TQ_KQ(TQ_F32, 128) TQ_KQ(TQ_F32, 256)
 #undef TQ_KQ
   return TQ_EUNSUPPORTED;
