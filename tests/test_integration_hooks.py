@@ -1,0 +1,256 @@
+"""Attention-backend hooks against a fake model runner (the duck-typed contract
+of the reference's integration/vllm.py:361-441).  The CPU tests cover hook
+installation, mode routing and bookkeeping; the GPU test drives a prefill and
+decode steps through the compressed path and checks the hybrid output against
+the oracle on the same store."""
+
+import math
+import types
+
+import pytest
+import torch
+
+from turboquant_amd.integration import vllm as hooks
+from turboquant_amd import vllm_attn_backend as legacy
+
+
+class FakeMeta:
+    def __init__(self, n, max_q):
+        self.num_actual_tokens, self.max_query_len = n, max_q
+
+
+class FakeImpl:
+    """Exact-attention backend: keeps every K/V it is given, attends causally over them."""
+
+    def __init__(self, hq, hkv, d, separate_update=True):
+        self.num_heads, self.num_kv_heads, self.head_size = hq, hkv, d
+        self.scale = 1.0 / math.sqrt(d)
+        self.k, self.v = [], []
+        self.forward_calls = 0
+        if separate_update:
+            self.do_kv_cache_update = types.MethodType(FakeImpl._update, self)
+
+    def _update(self, layer, key, value, kv_cache, slot_mapping):
+        self.k.append(key.clone())
+        self.v.append(value.clone())
+
+    def forward(self, layer, query, key, value, kv_cache, attn_metadata, output=None, output_scale=None,
+                output_block_scale=None):
+        self.forward_calls += 1
+        n = query.shape[0] if attn_metadata is None else attn_metadata.num_actual_tokens
+        K = torch.cat(self.k).float() if self.k else key.float()
+        V = torch.cat(self.v).float() if self.v else value.float()
+        q = query[:n].reshape(n, self.num_heads, self.head_size).float()
+        rep = self.num_heads // self.num_kv_heads
+        Kx, Vx = K.repeat_interleave(rep, 1), V.repeat_interleave(rep, 1)
+        s = torch.einsum("thd,nhd->htn", q, Kx) * self.scale
+        N = Kx.shape[0]
+        mask = torch.arange(N)[None, :].to(s.device) > (N - n + torch.arange(n)[:, None].to(s.device))
+        s = s.masked_fill(mask[None], float("-inf"))
+        o = torch.einsum("htn,nhd->thd", s.softmax(-1), Vx).to(query.dtype)
+        res = o if query.dim() == 3 else o.reshape(n, -1)
+        if output is not None:
+            output[:n].copy_(res.reshape(output[:n].shape))
+            return output
+        return res
+
+
+class FakeMlaImpl:
+    def __init__(self):
+        self.num_kv_heads, self.kv_lora_rank = 1, 64
+        self.updates = 0
+
+    def do_kv_cache_update(self, kv_c_normed, k_pe, kv_cache, slot_mapping, kv_cache_dtype, k_scale):
+        self.updates += 1
+
+    def forward_mqa(self, q, kv_c_and_k_pe_cache, attn_metadata, layer):
+        return q
+
+
+class FakeModule:
+    def __init__(self, impl, device):
+        self.impl = impl
+        self.kv_cache = [torch.zeros(2, 4, 16, 2, 8, device=device)]
+
+
+def make_runner(device, n_layers=3, hq=4, hkv=2, d=64, separate_update=True, with_mla=False):
+    ctx = {}
+    for i in range(n_layers):
+        ctx[f"model.layers.{i}.attn"] = FakeModule(FakeImpl(hq, hkv, d, separate_update), device)
+    ctx["model.norm"] = types.SimpleNamespace()                       # no impl: skipped
+    if with_mla:
+        ctx["model.layers.9.mla"] = FakeModule(FakeMlaImpl(), device)
+    runner = types.SimpleNamespace(device=device,
+                                   compilation_config=types.SimpleNamespace(static_forward_context=ctx))
+    runner.kv_caches = [m.kv_cache[0] for m in ctx.values() if hasattr(m, "kv_cache")]
+    return runner
+
+
+def test_install_assigns_bits_kinds_and_seeds():
+    r = make_runner(torch.device("cpu"), n_layers=3, with_mla=True)
+    st = hooks.install_hooks(r, key_bits=3, value_bits=2, initial_layers_count=2, mode=hooks.MODE_CAPTURE_ONLY)
+    assert list(st) == ["model.layers.0.attn", "model.layers.1.attn", "model.layers.2.attn", "model.layers.9.mla"]
+    assert [s.config.key_bits for s in st.values()] == [4, 4, 3, 3]
+    assert [s.config.layer_idx for s in st.values()] == [0, 1, 2, 3]
+    assert [s.supports_hybrid for s in st.values()] == [True, True, True, False]
+    assert st["model.layers.9.mla"].config.head_dim == 64 and st["model.layers.9.mla"].config.backend_kind == "mla"
+    assert st["model.layers.0.attn"].config.num_query_heads == 4
+    assert st["model.layers.1.attn"].store.layer_idx == 1
+    assert r._tq_layer_states is st and r._tq_no_alloc is False
+    assert hooks.get_mode() == hooks.MODE_CAPTURE_ONLY
+    # per-layer rotation seeds differ (42 + 7 * layer, store.py:56 of the reference)
+    a, b = st["model.layers.0.attn"].store.quantizer, st["model.layers.2.attn"].store.quantizer
+    assert a.mse_quantizer.Pi.shape == (64, 64)
+    assert not torch.equal(st["model.layers.1.attn"].store.quantizer.mse_quantizer.Pi[:, :1],
+                           st["model.layers.2.attn"].store.quantizer.mse_quantizer.Pi[:, :1])
+    assert a is not b
+
+
+def test_modes_validate_and_legacy_names_map():
+    with pytest.raises(AssertionError):
+        hooks.set_mode("bogus")
+    legacy.set_mode(legacy.MODE_ACTIVE)
+    assert hooks.get_mode() == hooks.MODE_HYBRID and legacy.get_mode() == legacy.MODE_ACTIVE
+    legacy.set_mode(legacy.MODE_SHADOW)
+    assert hooks.get_mode() == hooks.MODE_CAPTURE_ONLY
+    with pytest.raises(AssertionError):
+        legacy.set_mode("hybrid")
+    r = make_runner(torch.device("cpu"), n_layers=1)
+    st = legacy.install_turboquant_hooks(r, buffer_size=32, mode=legacy.MODE_ACCUMULATE)
+    assert r._tq_states is st and st["model.layers.0.attn"].engine.ring.capacity == 32
+    assert hooks.get_mode() == hooks.MODE_CAPTURE_ONLY
+
+
+@pytest.mark.parametrize("separate_update", [True, False])
+def test_capture_routes_tokens_and_passthrough_output(separate_update):
+    dev = torch.device("cpu")
+    r = make_runner(dev, n_layers=1, separate_update=separate_update)
+    st = hooks.install_hooks(r, ring_capacity=128, initial_layers_count=0, mode=hooks.MODE_CAPTURE_ONLY)
+    state = st["model.layers.0.attn"]
+    impl = r.compilation_config.static_forward_context["model.layers.0.attn"].impl
+    g = torch.Generator().manual_seed(0)
+    k = torch.randn(40, 2, 64, generator=g).bfloat16()
+    v = torch.randn(40, 2, 64, generator=g).bfloat16()
+    q = torch.randn(40, 4 * 64, generator=g).bfloat16()
+    if separate_update:
+        impl.do_kv_cache_update(None, k, v, None, torch.arange(40))
+    out = torch.zeros(48, 4 * 64, dtype=torch.bfloat16)
+    res = impl.forward(None, q, k, v, None, FakeMeta(40, 40), output=out)
+    assert res is out and impl.forward_calls == 1 and out[:40].abs().sum() > 0 and out[40:].abs().sum() == 0
+    assert state.engine.ring.size == 40 and state.store.num_tokens == 0
+    # one decode token
+    k1, v1, q1 = k[:1] + 1, v[:1] - 1, q[:1]
+    if separate_update:
+        impl.do_kv_cache_update(None, k1, v1, None, torch.arange(1))
+    impl.forward(None, q1, k1, v1, None, FakeMeta(1, 1))
+    assert state.engine.ring.size == 41
+    rk, rv = state.engine.ring.peek()
+    assert torch.equal(rk[-1], k1[0]) and torch.equal(rv[-1], v1[0])
+    # hybrid mode without enough compressed history falls back to the backend's own attention
+    hooks.set_mode(hooks.MODE_HYBRID)
+    calls = impl.forward_calls
+    impl.forward(None, q1, k1, v1, None, FakeMeta(1, 1))
+    assert impl.forward_calls == calls + 1
+    # profiling pass (no metadata) is passed through, nothing is captured
+    size = state.engine.ring.size
+    impl.forward(None, q1, k1, v1, None, None)
+    assert state.engine.ring.size == size
+    # off: no capture at all
+    hooks.set_mode(hooks.MODE_OFF)
+    if separate_update:
+        impl.do_kv_cache_update(None, k1, v1, None, torch.arange(1))
+    impl.forward(None, q1, k1, v1, None, FakeMeta(1, 1))
+    assert state.engine.ring.size == size
+    stats = hooks.get_stats(r)
+    assert stats == {"num_layers": 1, "total_compressed_tokens": 0, "total_buffered_tokens": size,
+                     "total_memory_bytes": state.store.memory_bytes(), "mode": hooks.MODE_OFF}
+    state.reset()
+    assert state.engine.ring.size == 0
+
+
+def test_no_alloc_prefill_is_dense_causal_and_skips_backend():
+    dev = torch.device("cpu")
+    r = make_runner(dev, n_layers=1)
+    hooks.install_hooks(r, initial_layers_count=0, mode=hooks.MODE_HYBRID, no_alloc=True)
+    impl = r.compilation_config.static_forward_context["model.layers.0.attn"].impl
+    g = torch.Generator().manual_seed(1)
+    k, v = torch.randn(24, 2, 64, generator=g), torch.randn(24, 2, 64, generator=g)
+    q = torch.randn(24, 4, 64, generator=g)
+    impl.do_kv_cache_update(None, k, v, None, torch.arange(24))
+    assert impl.k == []                                   # the engine's own cache is not written in no_alloc mode
+    got = impl.forward(None, q, k, v, None, FakeMeta(24, 24))
+    assert impl.forward_calls == 0 and got.shape == (24, 4, 64)
+    impl.k, impl.v = [k], [v]
+    want = FakeImpl.forward(impl, None, q, k, v, None, FakeMeta(24, 24))
+    assert torch.allclose(got, want, atol=1e-5)
+    # decode with nothing compressed yet: zeros, as the reference does in no_alloc mode
+    z = impl.forward(None, q[:1].reshape(1, -1), k[:1], v[:1], None, FakeMeta(1, 1))
+    assert z.shape == (1, 256) and z.abs().sum() == 0
+
+
+def test_mla_layers_are_observed_only_and_free_kv_cache():
+    dev = torch.device("cpu")
+    r = make_runner(dev, n_layers=2, with_mla=True)
+    st = hooks.install_hooks(r, mode=hooks.MODE_HYBRID)
+    mla = r.compilation_config.static_forward_context["model.layers.9.mla"]
+    mla.impl.do_kv_cache_update(None, None, None, None, "auto", None)
+    assert mla.impl.updates == 1 and st["model.layers.9.mla"]._log_count == 1
+    x = torch.ones(2, 3)
+    assert mla.impl.forward_mqa(x, None, None, None) is x
+    per = 2 * 4 * 16 * 2 * 8 * 4
+    assert hooks.free_kv_cache(r) == 2 * per               # the MLA layer keeps its cache
+    ctx = r.compilation_config.static_forward_context
+    assert ctx["model.layers.0.attn"].kv_cache[0].numel() == 1 and mla.kv_cache[0].numel() == 2 * 4 * 16 * 2 * 8
+    assert [t.numel() for t in r.kv_caches] == [1, 1, 2 * 4 * 16 * 2 * 8]
+    assert hooks.free_kv_cache(types.SimpleNamespace()) == 0 and hooks.get_stats(types.SimpleNamespace()) == {}
+    assert legacy.free_kv_cache(types.SimpleNamespace()) == 0
+
+
+def test_enable_no_alloc_needs_vllm():
+    with pytest.raises(ImportError):
+        legacy.enable_no_alloc()
+
+
+@pytest.mark.gpu
+def test_hybrid_decode_through_the_hooks_matches_the_oracle(gpu):
+    from oracle import tq_oracle as O
+    from tests.helpers import cosine, key_code, params_of, value_code
+    dev = torch.device("cuda:0")
+    hq, hkv, d = 8, 2, 128
+    r = make_runner(dev, n_layers=2, hq=hq, hkv=hkv, d=d)
+    st = hooks.install_hooks(r, key_bits=3, value_bits=4, ring_capacity=128, initial_layers_count=1,
+                             mode=hooks.MODE_HYBRID)
+    g = torch.Generator(device=dev).manual_seed(5)
+    T = 500
+    for li, (name, state) in enumerate(st.items()):
+        impl = r.compilation_config.static_forward_context[name].impl
+        k = torch.randn(T, hkv, d, generator=g, device=dev).bfloat16()
+        v = torch.randn(T, hkv, d, generator=g, device=dev).bfloat16()
+        q = torch.randn(T, hq * d, generator=g, device=dev).bfloat16()
+        impl.do_kv_cache_update(None, k, v, None, torch.arange(T, device=dev))
+        impl.forward(None, q, k, v, None, FakeMeta(T, T))                 # prefill: backend's own attention
+        assert state.store.num_tokens == T - 128 and state.engine.ring.size == 128
+        assert state.config.key_bits == (4 if li == 0 else 3)
+        for step in range(3):
+            k1 = torch.randn(1, hkv, d, generator=g, device=dev).bfloat16()
+            v1 = torch.randn(1, hkv, d, generator=g, device=dev).bfloat16()
+            q1 = torch.randn(1, hq * d, generator=g, device=dev).bfloat16()
+            impl.do_kv_cache_update(None, k1, v1, None, torch.arange(1, device=dev))
+            calls = impl.forward_calls
+            out = torch.zeros(4, hq * d, dtype=torch.bfloat16, device=dev)
+            res = impl.forward(None, q1, k1, v1, None, FakeMeta(1, 1), output=out)
+            assert res is out and impl.forward_calls == calls             # answered from the compressed store
+            # oracle on the same store + ring
+            flat = state.store.get_flat_cache()
+            kc = key_code(flat.prod_q.mse_indices.cpu(), flat.prod_q.qjl_signs.cpu(), flat.prod_q.residual_norms.cpu(),
+                          flat.prod_q.norms.cpu(), state.config.key_bits - 1)
+            vc = value_code(flat.value_q.data.cpu(), flat.value_q.scales.cpu(), flat.value_q.zeros.cpu(), 4)
+            rk, rv = state.engine.ring.peek()
+            want = O.hybrid_attention(q1.view(1, hq, d).cpu(), kc, vc, flat.num_tokens,
+                                      params_of(state.store.quantizer), hkv, rk.cpu(), rv.cpu())
+            assert cosine(out[0].float().cpu(), want.flatten().float()) >= 0.9999
+            # and it stays close to the backend's exact attention over the same tokens
+            exact = FakeImpl.forward(impl, None, q1, k1, v1, None, FakeMeta(1, 1))
+            assert cosine(out[0].float().cpu(), exact[0].float().cpu()) > 0.9
+        # the ring spilled nothing yet (128 + 3 decode tokens -> one drain of 128 at the 129th)
+        assert state.engine.total_tokens == T + 3
