@@ -42,7 +42,7 @@ constexpr int MF_WAVES = 4;
 constexpr int BLK_TOK = 64;              // tokens per wavefront iteration
 constexpr float MF_NEG = -1.0e30f;
 constexpr int P_STRIDE = 20;             // floats per row of the LDS softmax-weight tile (16 + skew)
-constexpr int WAVE_LDS_FLOATS = 4 * 16 * P_STRIDE + 16 + 4 * 16 * 8;
+constexpr int WAVE_LDS_FLOATS = 4 * 16 * P_STRIDE + 16 + 4 * 16 * 16;
 
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
   f32x2 f = {lo, hi};
@@ -131,7 +131,7 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
   extern __shared__ __align__(16) unsigned char smem_raw[];
   float* s_p = (float*)smem_raw + wave * WAVE_LDS_FLOATS;   // [4 pages][16 rows][P_STRIDE]
   float* s_alpha = s_p + 4 * 16 * P_STRIDE;                 // [16]
-  uint32_t* s_scale = (uint32_t*)(s_alpha + 16);            // [4 pages][NG][8 dwords]
+  float* s_scale = s_alpha + 16;                            // [4 pages][NG][16 tokens] fp32, pre-scaled
   float* s_red = (float*)smem_raw;                          // after the loop: [MF_WAVES][G][D + 2]
 
   float cmax = 0.0f;
@@ -238,9 +238,13 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
     R.scale = *(const u32x4*)(pool_h + spid * page_stride + off_scale);
   };
 
-  const uint32_t base_pat = in_vgpr(VB == 2 ? 0x40804080u : 0x41804180u);   // bf16 pairs of 2^VB
-  const uint32_t code_mask = in_vgpr(VB == 2 ? 0x00600060u : 0x00780078u);  // top mantissa bits
-  const uint32_t neg_pat = VB == 2 ? 0xC080C080u : 0xC180C180u;             // bf16 pairs of -2^VB
+  // A value code sits in the low mantissa bits of bf16(128): B = 128 + code * 2^s exactly, where s
+  // is the bit position the code already has inside its packed word (0, 2 or 4 for 2-bit codes,
+  // 0 for 4-bit codes), so that most codes need no shift; the softmax weight carries 2^-s.
+  const uint32_t base_pat = in_vgpr(0x43004300u);                           // bf16 pairs of 128
+  const uint32_t m0 = in_vgpr(VB == 2 ? 0x00030003u : 0x000F000Fu);
+  const uint32_t m1 = in_vgpr(0x000C000Cu), m2 = in_vgpr(0x00300030u);
+  const uint32_t neg_pat = 0xC300C300u;                                     // bf16 pairs of -128
   const u32x4 neg_base = {neg_pat, neg_pat, neg_pat, neg_pat};
 
   // ---------------------------------------------------------------- one block of 64 tokens
@@ -307,8 +311,30 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
   // weights x (codes, scales, zeros) of block blk into the accumulators
   auto value_stage = [&](int blk, const ValRegs& V, bool rescale, auto partial_tag) {
     constexpr bool PARTIAL = decltype(partial_tag)::value;
-    // scales -> LDS ([page][group][16 tokens] bf16, as in the page); first use of the value loads
-    if (lane < 4 * PIECES) *(u32x4*)(s_scale + lane * 4) = V.scale;
+    // scales -> LDS as fp32 [page][group][16 tokens]; first use of the value loads.  The lane that
+    // holds a 16-byte piece widens it once (instead of all 16 row lanes later), folds in the
+    // 2^-s of its tokens' code position and zeroes tokens past the end of the sequence.
+    if (lane < 4 * PIECES) {
+      const int spage = lane / PIECES, pc = lane % PIECES;
+      float f[8];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        f[2 * i] = __uint_as_float(V.scale[i] << 16);
+        f[2 * i + 1] = __uint_as_float(V.scale[i] & 0xffff0000u);
+      }
+      if (VB == 2) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) f[e] *= (e % 3 == 0 ? 1.0f : (e % 3 == 1 ? 0.25f : 0.0625f));
+      }
+      if (PARTIAL) {
+        const int nv = seq_len - (blk * BLK_TOK + spage * 16 + 8 * (pc & 1));
+#pragma unroll
+        for (int e = 0; e < 8; ++e) f[e] = e < nv ? f[e] : 0.0f;
+      }
+      f32x4* dst = (f32x4*)(s_scale + (spage * NG + (pc >> 1)) * 16 + 8 * (pc & 1));
+      dst[0] = f32x4{f[0], f[1], f[2], f[3]};
+      dst[1] = f32x4{f[4], f[5], f[6], f[7]};
+    }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -351,20 +377,15 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
 #pragma unroll
     for (int grp = 0; grp < NG; ++grp) {
       // w = weight * scale for the 16 tokens of page kb, then the two A operands in the value token order
-      uint32_t sc[8];
-      {
-        const u32x4* sp = (const u32x4*)(s_scale + (kb * NG + grp) * 8);
-        const u32x4 s0 = sp[0], s1 = sp[1];
-        sc[0] = s0[0]; sc[1] = s0[1]; sc[2] = s0[2]; sc[3] = s0[3];
-        sc[4] = s1[0]; sc[5] = s1[1]; sc[6] = s1[2]; sc[7] = s1[3];
-      }
       float w[16];
+      {
+        const f32x4* sp = (const f32x4*)(s_scale + (kb * NG + grp) * 16);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        uint32_t sd = sc[i];
-        if (PARTIAL) sd &= keep[i];
-        w[2 * i] = pr[2 * i] * __uint_as_float(sd << 16);
-        w[2 * i + 1] = pr[2 * i + 1] * __uint_as_float(sd & 0xffff0000u);
+        for (int q4 = 0; q4 < 4; ++q4) {
+          const f32x4 sv = sp[q4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) w[4 * q4 + e] = pr[4 * q4 + e] * sv[e];
+        }
       }
       u32x4 aw[2];
 #pragma unroll
@@ -378,21 +399,15 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
         for (int u = 0; u < 2; ++u) {
           u32x4 bc;
           if (VB == 2) {
-            const uint32_t x = V.v[c];
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-              const int f = 4 * u + r, sh = 5 - 2 * f;
-              const uint32_t y = sh >= 0 ? (x << sh) : (x >> (-sh));
-              bc[r] = (y & code_mask) | base_pat;
-            }
+            // 16 two-bit fields; register r of MFMA u takes fields 4u+r (low half) and 4u+r+8 (high half)
+            const uint32_t x = V.v[c], x6 = x >> 6, x12 = x >> 12;
+            if (u == 0) bc = u32x4{(x & m0) | base_pat, (x & m1) | base_pat, (x & m2) | base_pat, (x6 & m0) | base_pat};
+            else bc = u32x4{(x6 & m1) | base_pat, (x6 & m2) | base_pat, (x12 & m0) | base_pat, (x12 & m1) | base_pat};
           } else {
+            // 8 four-bit fields; register r takes fields r (low half) and r+4 (high half)
             const uint32_t x = V.v[2 * c + u];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-              const int sh = 3 - 4 * r;
-              const uint32_t y = sh >= 0 ? (x << sh) : (x >> (-sh));
-              bc[r] = (y & code_mask) | base_pat;
-            }
+            for (int r = 0; r < 4; ++r) bc[r] = ((x >> (4 * r)) & m0) | base_pat;
           }
           acc[c] = mfma(aw[u], bc, acc[c]);
           acc[c] = mfma(aw[u], neg_base, acc[c]);
