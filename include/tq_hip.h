@@ -57,6 +57,11 @@ typedef struct tq_layer {
    * written as the exact sum of three bf16 matrices, stored [term][row][col] as raw
    * bf16 bit patterns (3*d*d each).  NULL selects the vector-ALU kernel.            */
   const uint16_t *Pi_split, *PiT_split, *S_split;
+  /* Optional constants of the fused query-preparation kernel of the decode path:
+   * Pi_colsum[i] = sum_j Pi[j][i], S_colsum[i] = sum_j S[j][i] (d floats each) and the
+   * largest row norm of S.  NULL selects the two-kernel preparation.                    */
+  const float *Pi_colsum, *S_colsum;
+  float S_rownorm_max;
   /* Walsh expansion of the codebook over the index bits, used by the decode
    * kernel: centroids[idx] = term_const + sum_t term_coef[t] * parity(idx & term_mask[t]).
    * Filled by tq_layer_fill_terms from the host copy of the centroids.          */
@@ -72,9 +77,9 @@ typedef struct tq_layer {
  *   keys   : key_bits = mse_bits+1 bit-planes (index bits high..low, then the QJL
  *            sign).  Word j of plane p of token n holds coordinates 32j..32j+31
  *            (bit i = coordinate 32j+i).  With key_lane_major != 0 (d a multiple
- *            of 128) the words are stored as [j%4][n][p][j/4], so that the
+ *            of 128) the words are stored as [j%4][n][j/4][p], so that the
  *            words one wavefront lane (token n, coordinate quarter j%4) consumes
- *            are contiguous; otherwise as [p][j][n].
+ *            are contiguous, 128 coordinates after 128; otherwise as [p][j][n].
  *   meta   : per token {float norm, float rnorm}: the key norm (a value of the
  *            input dtype, widened losslessly) and ||r||.
  *   vdata  : per channel c a little-endian field of 16*value_bits bits, token n's

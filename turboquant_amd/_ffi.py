@@ -33,6 +33,7 @@ class TqLayer(C.Structure):
         ("centroids", C.c_void_p), ("thresholds", C.c_void_p),
         ("qjl_scale", C.c_float),
         ("Pi_split", C.c_void_p), ("PiT_split", C.c_void_p), ("S_split", C.c_void_p),
+        ("Pi_colsum", C.c_void_p), ("S_colsum", C.c_void_p), ("S_rownorm_max", C.c_float),
         ("n_terms", C.c_int32),
         ("term_mask", C.c_int32 * TQ_MAX_TERMS),
         ("term_coef", C.c_float * TQ_MAX_TERMS),
@@ -138,7 +139,7 @@ def walsh_terms(centroids_host: torch.Tensor, mse_bits: int, layer: TqLayer):
 
 def make_layer(d: int, mse_bits: int, Pi: torch.Tensor, PiT: torch.Tensor, centroids: torch.Tensor,
                thresholds: torch.Tensor, S: Optional[torch.Tensor] = None, ST: Optional[torch.Tensor] = None,
-               centroids_host: Optional[torch.Tensor] = None, splits=None) -> TqLayer:
+               centroids_host: Optional[torch.Tensor] = None, splits=None, query_consts=None) -> TqLayer:
     """Describe a layer's constants to the library.  The tensors must stay alive
     while the struct is in use; they must be fp32, contiguous and on one GPU."""
     for name, t in (("Pi", Pi), ("PiT", PiT), ("centroids", centroids), ("thresholds", thresholds), ("S", S), ("ST", ST)):
@@ -158,6 +159,9 @@ def make_layer(d: int, mse_bits: int, Pi: torch.Tensor, PiT: torch.Tensor, centr
         pi_s, pit_s, s_s = splits
         ly.Pi_split, ly.PiT_split = pi_s.data_ptr(), pit_s.data_ptr()
         ly.S_split = None if s_s is None else s_s.data_ptr()
+    if query_consts is not None:
+        pi_cs, s_cs, s_max = query_consts
+        ly.Pi_colsum, ly.S_colsum, ly.S_rownorm_max = pi_cs.data_ptr(), s_cs.data_ptr(), float(s_max)
     walsh_terms(centroids_host if centroids_host is not None else centroids.detach().cpu(), mse_bits, ly)
     return ly
 

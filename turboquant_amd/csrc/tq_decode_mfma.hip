@@ -17,7 +17,12 @@
 //    operand, and a second MFMA with B = -2^vb removes the offset with the very
 //    same A.  The zero points go through one more MFMA (weights x zeros).
 //
-// One wavefront owns 64 tokens (4 pages) per iteration: lane (n, kb) = lane%16,
+// head_dim 256 is split over a pair of wavefronts (DS = 2): each scores half of the
+// coordinates, the halves of the scores meet in LDS once per block, both wavefronts
+// then compute the same softmax and each accumulates half of the channels.  That keeps
+// the per-wavefront register footprint of head_dim 128, so two wavefronts fit per SIMD.
+//
+// One wavefront (pair) owns 64 tokens (4 pages) per iteration: lane (n, kb) = lane%16,
 // lane/16 is token n and coordinate quarter kb in the score stage, and (row,
 // page kb) in the value stage.  The key words of the next 64 tokens are
 // requested before the current ones are consumed; the value words of the current
@@ -42,7 +47,10 @@ constexpr int MF_WAVES = 4;
 constexpr int BLK_TOK = 64;              // tokens per wavefront iteration
 constexpr float MF_NEG = -1.0e30f;
 constexpr int P_STRIDE = 20;             // floats per row of the LDS softmax-weight tile (16 + skew)
-constexpr int WAVE_LDS_FLOATS = 4 * 16 * P_STRIDE + 16 + 4 * 16 * 16;
+constexpr int X_FLOATS = 2 * 8 * 64;     // score-half exchange slot of a wavefront: [parity][8 values][64 lanes]
+__host__ __device__ constexpr int wave_lds_floats(int ng, int ds) {
+  return 4 * 16 * P_STRIDE + 16 + 4 * ng * 16 + (ds > 1 ? X_FLOATS : 0);
+}
 
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
   f32x2 f = {lo, hi};
@@ -108,23 +116,31 @@ __device__ __forceinline__ constexpr int v_token(int u, int r, int h) {
 }
 
 // D in {128, 256}; MB stored index bits; NX extra (multi-bit) Walsh terms; VB value bits;
-// GS value group size; WPS wavefronts per SIMD the register budget is sized for.
-template <int D, int MB, int NX, int VB, int GS, int WPS>
+// GS value group size; DS wavefronts that share one block (each takes D/DS coordinates and
+// channels); WPS wavefronts per SIMD the register budget is sized for.
+template <int D, int MB, int NX, int VB, int GS, int DS, int WPS>
 __global__ void __launch_bounds__(MF_WAVES * 64, WPS)
 decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict__ q_stat, int Hq, int Hkv, const uint8_t* __restrict__ pool, const int32_t* __restrict__ block_table,
                    int bt_stride, const int32_t* __restrict__ seq_lens, float sm_scale, tq_layer ly, tq_page_layout L,
                    float* __restrict__ parts, int n_parts, int n_split) {
-  constexpr int WPL = D / 128;                // plane words per lane per plane per page
+  constexpr int DW = D / DS;                  // coordinates / channels of one wavefront
+  constexpr int WPLT = D / 128;               // plane words per lane per plane per page, all wavefronts
+  constexpr int WPL = DW / 128;               // ... of one wavefront
   constexpr int NTP = MB + NX + 1;            // term planes fed to the MFMA (stored + XOR terms + sign)
   constexpr int NKW = (MB + 1) * WPL;         // key dwords per lane per page
-  constexpr int CT = D / 16;                  // channel tiles
+  constexpr int CT = DW / 16;                 // channel tiles of one wavefront
   constexpr int VW = CT * VB / 2;             // value dwords per lane per block
-  constexpr int NG = D / GS, CTG = GS / 16;   // groups, channel tiles per group
-  constexpr int PIECES = 2 * NG;              // 16-byte pieces of scales per page
+  constexpr int NG = DW / GS, CTG = GS / 16;  // groups of one wavefront, channel tiles per group
+  constexpr int NGT = D / GS;                 // groups of the whole head
+  constexpr int PIECES = 2 * NG;              // 16-byte pieces of this wavefront's scales per page
+  constexpr int NGRP = MF_WAVES / DS;         // wavefront groups (each walks its own blocks)
+  constexpr int WAVE_LDS_FLOATS = wave_lds_floats(NG, DS);
+  static_assert(WPL >= 1 && NG >= 1, "a wavefront takes at least 128 coordinates");
   const int G = Hq / Hkv;                     // <= 8
   const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wgrp = wave / DS, hf = wave % DS; // block walker this wavefront belongs to; its share of the head
   const int n = lane & 15, kb = lane >> 4;    // score stage: token / coordinate quarter; value stage: row / page
   const float LOG2E = 1.4426950408889634f;
 
@@ -132,7 +148,9 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
   float* s_p = (float*)smem_raw + wave * WAVE_LDS_FLOATS;   // [4 pages][16 rows][P_STRIDE]
   float* s_alpha = s_p + 4 * 16 * P_STRIDE;                 // [16]
   float* s_scale = s_alpha + 16;                            // [4 pages][NG][16 tokens] fp32, pre-scaled
-  float* s_red = (float*)smem_raw;                          // after the loop: [MF_WAVES][G][D + 2]
+  float* s_x = s_scale + 4 * NG * 16;                       // DS > 1: [parity][8][64] this wavefront's score halves
+  float* s_x_peer = (float*)smem_raw + (wave ^ 1) * WAVE_LDS_FLOATS + (4 * 16 * P_STRIDE + 16 + 4 * NG * 16);
+  float* s_red = (float*)smem_raw;                          // after the loop: [NGRP][G][D + 2]
 
   float cmax = 0.0f;
   for (int t = 0; t < ly.n_terms; ++t) cmax = fmaxf(cmax, fabsf(ly.term_coef[t]));
@@ -142,7 +160,7 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
   // kernel has stored them in register order, one coalesced 1 KB load per register quadruple
   u32x4 qa[NTP][WPL][4];
   {
-    const u32x4* src = (const u32x4*)qa_pack + ((int64_t)b * Hkv + h) * (NTP * WPL * 4 * 64) + lane;
+    const u32x4* src = (const u32x4*)qa_pack + ((int64_t)b * Hkv + h) * (NTP * WPLT * 4 * 64) + lane;
     const bool live = (n >> 1) < G;
 #pragma unroll
     for (int tp = 0; tp < NTP; ++tp)
@@ -150,7 +168,7 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
       for (int i = 0; i < WPL; ++i)
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-          u32x4 v = src[((tp * WPL + i) * 4 + u) * 64];
+          u32x4 v = src[((tp * WPLT + hf * WPL + i) * 4 + u) * 64];
           qa[tp][i][u] = live ? v : u32x4{0, 0, 0, 0};
         }
   }
@@ -191,9 +209,10 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
   const int32_t* bt = block_table + (int64_t)b * bt_stride;
   const uint8_t* pool_h = pool + (int64_t)h * L.page_bytes;
   const int64_t page_stride = (int64_t)Hkv * L.page_bytes;
-  const int off_keys = L.off_keys + lane * (NKW * 4), off_meta = L.off_meta + n * 8;
-  const int off_v = L.off_vdata + n * (VW * 4);
-  const int off_scale = L.off_vscale + (lane % PIECES) * 16;
+  // per lane the key words are [word i][plane], the value fields [channel tile]: a wavefront's share is contiguous
+  const int off_keys = L.off_keys + (lane * DS + hf) * (NKW * 4), off_meta = L.off_meta + n * 8;
+  const int off_v = L.off_vdata + (n * DS + hf) * (VW * 4);
+  const int off_scale = L.off_vscale + hf * (NG * 32) + (lane % PIECES) * 16;
 
   f32x4 acc[CT];
 #pragma unroll
@@ -223,7 +242,7 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
   // All loads below are unconditional (lanes without a group / piece of their own read a
   // neighbour's): a load inside a branch would make the wait counters at the join conservative
   // and serialise the prefetch.
-  const int off_zero_c = L.off_vzero + min(n, NG - 1) * 32;
+  const int off_zero_c = L.off_vzero + min(n, NGT - 1) * 32;
   const int spg = min(lane / PIECES, 3);
   auto load_vals = [&](const int (&pid)[4], ValRegs& R) {
     const int my_pid = kb == 0 ? pid[0] : (kb == 1 ? pid[1] : (kb == 2 ? pid[2] : pid[3]));
@@ -249,7 +268,7 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
 
   // ---------------------------------------------------------------- one block of 64 tokens
   // scores of the 4 pages of block blk, online softmax, weights -> LDS
-  auto score_stage = [&](int blk, const KeyRegs& K, auto partial_tag) -> bool {
+  auto score_stage = [&](int blk, int it, const KeyRegs& K, auto partial_tag) -> bool {
     constexpr bool PARTIAL = decltype(partial_tag)::value;
     float s2[2][4];
 #pragma unroll
@@ -260,12 +279,12 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
 #pragma unroll
         for (int tp = 0; tp < NTP; ++tp) {
           uint32_t x;
-          if (tp < MB) x = K.key[pg][tp * WPL + i];
-          else if (tp == NTP - 1) x = K.key[pg][MB * WPL + i];
+          if (tp < MB) x = K.key[pg][i * (MB + 1) + tp];
+          else if (tp == NTP - 1) x = K.key[pg][i * (MB + 1) + MB];
           else {
             x = 0;
 #pragma unroll
-            for (int p = 0; p < MB; ++p) x ^= ((xplanes[tp - MB] >> p) & 1) ? K.key[pg][p * WPL + i] : 0u;
+            for (int p = 0; p < MB; ++p) x ^= ((xplanes[tp - MB] >> p) & 1) ? K.key[pg][i * (MB + 1) + p] : 0u;
           }
           uint32_t bb[16];
           expand_plane_word(x, bb);
@@ -281,7 +300,32 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
         const float vm = dm[2 * j] + dm[2 * j + 1], vq = dq[2 * j] + dq[2 * j + 1];
-        float s = fmaf(nk, fmaf(am[j], vm, bm[j]), rk * fmaf(aq[j], vq, bq[j]));
+        // this wavefront's share of the score (the whole score when DS == 1); the constant
+        // terms are added after the shares have met
+        s2[j][pg] = fmaf(nk * am[j], vm, (rk * aq[j]) * vq);
+      }
+    }
+    if (DS > 1) {
+      // exchange with the wavefront that scored the other coordinates: own share -> LDS, workgroup
+      // barrier, partner's share <- LDS.  a + b == b + a, so both end with bit-identical scores.
+      float* mine = s_x + (it & 1) * (8 * 64);
+      const float* theirs = s_x_peer + (it & 1) * (8 * 64);
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int pg = 0; pg < 4; ++pg) mine[(j * 4 + pg) * 64 + lane] = s2[j][pg];
+      __syncthreads();
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int pg = 0; pg < 4; ++pg) s2[j][pg] += theirs[(j * 4 + pg) * 64 + lane];
+    }
+#pragma unroll
+    for (int pg = 0; pg < 4; ++pg) {
+      const float nk = K.meta[pg][0], rk = K.meta[pg][1];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        float s = s2[j][pg] + fmaf(nk, bm[j], rk * bq[j]);
         if (PARTIAL && (blk * BLK_TOK + pg * 16 + n >= seq_len)) s = MF_NEG;
         s2[j][pg] = s;
       }
@@ -417,29 +461,36 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
     __builtin_amdgcn_wave_barrier();
   };
 
-  // ---------------------------------------------------------------- pipeline over this wave's blocks
+  // ---------------------------------------------------------------- pipeline over this walker's blocks
   // Registers are reloaded as soon as their last reader is done: the key words of
   // the next block are requested right after the score stage, its value words
-  // right after the value stage.
+  // right after the value stage.  With DS > 1 the score stage contains a workgroup
+  // barrier, so every wavefront makes the same number of trips; a walker that has
+  // run out of blocks only attends the barrier.
   {
     KeyRegs K;
     ValRegs V;
     int pid[4];
-    int blk = blk_begin + wave;
+    const int trips = (max(blk_end - blk_begin, 0) + NGRP - 1) / NGRP;
+    int blk = blk_begin + wgrp;
     if (blk < blk_end) {
       page_ids(blk, pid);
       load_keys(pid, K);
       load_vals(pid, V);
     }
-    while (blk < blk_end) {
-      const int nxt = blk + MF_WAVES;
+    for (int it = 0; it < trips; ++it) {
+      if (blk >= blk_end) {                              // uniform per wavefront pair
+        if (DS > 1) __syncthreads();
+        continue;
+      }
+      const int nxt = blk + NGRP;
       const bool last = (blk + 1) * BLK_TOK > seq_len;
-      // the block after this wave's last one does not exist: re-request the current one instead,
+      // the block after this walker's last one does not exist: re-request the current one instead,
       // so that the loads stay outside any branch
       const int nxt_c = nxt < blk_end ? nxt : blk;
       int pid_n[4];
       page_ids(nxt_c, pid_n);                            // scalar loads, consumed after the score stage
-      const bool rescale = last ? score_stage(blk, K, std::true_type{}) : score_stage(blk, K, std::false_type{});
+      const bool rescale = last ? score_stage(blk, it, K, std::true_type{}) : score_stage(blk, it, K, std::false_type{});
       load_keys(pid_n, K);
       if (last) value_stage(blk, V, rescale, std::true_type{});
       else value_stage(blk, V, rescale, std::false_type{});
@@ -448,19 +499,21 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
     }
   }
 
-  // ---------------------------------------------------------------- merge the 4 waves, write the partial
+  // ---------------------------------------------------------------- merge the walkers, write the partial
   __syncthreads();      // every wave is done with its private LDS region
-  float* s_z = s_red + MF_WAVES * G * (D + 2);                 // [MF_WAVES][16 rows][16 groups]
+  float* s_z = s_red + NGRP * G * (D + 2);                     // [MF_WAVES][16 rows][16 groups]
 #pragma unroll
   for (int i = 0; i < 4; ++i) s_z[(wave * 16 + 4 * kb + i) * 16 + n] = zacc[i];
+  if (hf == 0) {                                               // the wavefronts of a pair hold the same (m, l)
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const float lsum = row_sum16(l_run[j]);
-    const int g = 2 * kb + j;
-    if (n == 0 && g < G) {
-      float* r = s_red + (wave * G + g) * (D + 2);
-      r[0] = m_run[j] * 0.6931471805599453f;     // back to the natural-log domain of the partials
-      r[1] = lsum;
+    for (int j = 0; j < 2; ++j) {
+      const float lsum = row_sum16(l_run[j]);
+      const int g = 2 * kb + j;
+      if (n == 0 && g < G) {
+        float* r = s_red + (wgrp * G + g) * (D + 2);
+        r[0] = m_run[j] * 0.6931471805599453f;     // back to the natural-log domain of the partials
+        r[1] = lsum;
+      }
     }
   }
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -472,8 +525,8 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
     for (int i = 0; i < 4; ++i) {
       const int g = 4 * kb + i;
       if (g < G) {
-        const float z = s_z[(wave * 16 + g) * 16 + c / CTG];
-        s_red[(wave * G + g) * (D + 2) + 2 + 16 * c + n] = acc[c][i] + z;
+        const float z = s_z[(wave * 16 + g) * 16 + hf * NG + c / CTG];
+        s_red[(wgrp * G + g) * (D + 2) + 2 + hf * DW + 16 * c + n] = acc[c][i] + z;
       }
     }
   }
@@ -481,9 +534,9 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
   for (int o = tid; o < G * D; o += blockDim.x) {
     const int g = o / D, ch = o - g * D;
     float mm = MF_NEG;
-    for (int w = 0; w < MF_WAVES; ++w) mm = fmaxf(mm, s_red[(w * G + g) * (D + 2)]);
+    for (int w = 0; w < NGRP; ++w) mm = fmaxf(mm, s_red[(w * G + g) * (D + 2)]);
     float ll = 0.0f, aa = 0.0f;
-    for (int w = 0; w < MF_WAVES; ++w) {
+    for (int w = 0; w < NGRP; ++w) {
       const float* r = s_red + (w * G + g) * (D + 2);
       const float wgt = __expf(r[0] - mm);
       ll += wgt * r[1];
@@ -495,16 +548,16 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
   }
 }
 
-template <int D, int MB, int NX, int VB, int GS, int WPS>
+template <int D, int MB, int NX, int VB, int GS, int DS, int WPS>
 static int launch_one(const uint32_t* qa_pack, const float* q_stat, int B, int Hq, int Hkv,
                       const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
                       float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts, int n_split,
                       hipStream_t st) {
   const int G = Hq / Hkv;
-  size_t per_wave = (size_t)WAVE_LDS_FLOATS * sizeof(float);
-  size_t merge = (size_t)(MF_WAVES * G * (D + 2) + MF_WAVES * 16 * 16) * sizeof(float);
+  size_t per_wave = (size_t)wave_lds_floats(D / DS / GS, DS) * sizeof(float);
+  size_t merge = (size_t)(MF_WAVES / DS * G * (D + 2) + MF_WAVES * 16 * 16) * sizeof(float);
   size_t smem = per_wave * MF_WAVES > merge ? per_wave * MF_WAVES : merge;
-  auto kern = decode_mfma_kernel<D, MB, NX, VB, GS, WPS>;
+  auto kern = decode_mfma_kernel<D, MB, NX, VB, GS, DS, WPS>;
   if (smem > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return (int)e;
@@ -530,14 +583,14 @@ int launch_decode_mfma(const uint32_t* qa_pack, const float* q_stat, int B, int 
   int nx = 0;
   for (int t = 0; t < ly.n_terms; ++t)
     if (__builtin_popcount(ly.term_mask[t]) > 1) ++nx;
-#define TQ_TRY(D_, MB_, NX_, VB_, GS_, WPS_)                                                                    \
+#define TQ_TRY(D_, MB_, NX_, VB_, GS_, DS_, WPS_)                                                               \
   if (d == D_ && mb == MB_ && nx == NX_ && vb == VB_ && gs == GS_)                                              \
-    return launch_one<D_, MB_, NX_, VB_, GS_, WPS_>(qa_pack, q_stat, B, Hq, Hkv, pool, block_table, bt_stride,    \
-                                                    seq_lens, sm_scale, ly, L, parts, n_parts, n_split, st);
-  TQ_TRY(128, 2, 0, 2, 32, 2) TQ_TRY(128, 2, 0, 4, 32, 2) TQ_TRY(256, 2, 0, 2, 32, 1) TQ_TRY(256, 2, 0, 4, 32, 1)
-  TQ_TRY(128, 1, 0, 2, 32, 2) TQ_TRY(128, 1, 0, 4, 32, 2) TQ_TRY(256, 1, 0, 2, 32, 1) TQ_TRY(256, 1, 0, 4, 32, 1)
-  TQ_TRY(128, 3, 1, 2, 32, 1) TQ_TRY(128, 3, 1, 4, 32, 1)
-  TQ_TRY(128, 2, 0, 2, 64, 2) TQ_TRY(128, 2, 0, 4, 64, 2) TQ_TRY(256, 2, 0, 2, 64, 1) TQ_TRY(256, 2, 0, 4, 64, 1)
+    return launch_one<D_, MB_, NX_, VB_, GS_, DS_, WPS_>(qa_pack, q_stat, B, Hq, Hkv, pool, block_table, bt_stride, \
+                                                         seq_lens, sm_scale, ly, L, parts, n_parts, n_split, st);
+  TQ_TRY(128, 2, 0, 2, 32, 1, 2) TQ_TRY(128, 2, 0, 4, 32, 1, 2) TQ_TRY(256, 2, 0, 2, 32, 2, 2) TQ_TRY(256, 2, 0, 4, 32, 2, 2)
+  TQ_TRY(128, 1, 0, 2, 32, 1, 2) TQ_TRY(128, 1, 0, 4, 32, 1, 2) TQ_TRY(256, 1, 0, 2, 32, 2, 2) TQ_TRY(256, 1, 0, 4, 32, 2, 2)
+  TQ_TRY(128, 3, 1, 2, 32, 1, 1) TQ_TRY(128, 3, 1, 4, 32, 1, 1)
+  TQ_TRY(128, 2, 0, 2, 64, 1, 2) TQ_TRY(128, 2, 0, 4, 64, 1, 2) TQ_TRY(256, 2, 0, 2, 64, 2, 2) TQ_TRY(256, 2, 0, 4, 64, 2, 2)
 #undef TQ_TRY
   return TQ_EUNSUPPORTED;
 }

@@ -473,7 +473,7 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
     }
   } else {
     // pages: a wavefront writes the bit-plane words of one tile, so the page lookup is uniform;
-    // lanes run over (word, token) in page order (lane-major: [w & 3][token][plane][w >> 2])
+    // lanes run over (word, token) in page order (lane-major: [w & 3][token][w >> 2][plane])
     const tq_page_layout& L = sink.L;
     constexpr int NSUB = KQ_WAVES / MT > 0 ? KQ_WAVES / MT : 1;   // wavefronts that share a tile
     const int planes = mb + 1;

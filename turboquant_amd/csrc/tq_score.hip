@@ -166,6 +166,160 @@ pack_query_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_s
   }
 }
 
+// Fused preparation of the matrix-core decode kernel: rotation, sketch, statistics and
+// operand packing in one launch.  A workgroup owns one GQA group (G query heads of one KV
+// head) and the 32 output coordinates of one plane word; PREP_SLICES threads share a
+// coordinate's contraction.  Nothing depends on another workgroup, because the operands
+// are normalised by bounds that every workgroup can compute from the raw query:
+// |q_rot_j| <= ||q|| (Pi is orthogonal) and |q_sk_j| <= ||q|| max_j ||S_j||, and the sums
+// over all coordinates that the decode kernel needs are q . colsum(Pi), q . colsum(S).
+// q_stat per row: {||q||, ||q|| max_j ||S_j||, sum_j q_rot_j, sum_j q_sk_j}.
+constexpr int PREP_COLS = 32, PREP_SLICES = 16;
+
+template <int PER>      // matrix rows per thread = d / PREP_SLICES
+__global__ void __launch_bounds__(PREP_COLS * PREP_SLICES)
+prep_query_kernel(const void* __restrict__ q, int dtype, int G, tq_layer ly, float* __restrict__ q_rot,
+                  float* __restrict__ q_sk, float* __restrict__ q_stat, uint32_t* __restrict__ qa_pack) {
+  extern __shared__ float sm[];
+  const int d = ly.d, tid = threadIdx.x, jl = tid % PREP_COLS, sl = tid / PREP_COLS;
+  const int word = blockIdx.y, j = word * PREP_COLS + jl;
+  // every global load of the kernel is issued here, before anything waits: the matrix slices
+  // do not depend on the query
+  float mp[PER], ms[PER];
+#pragma unroll
+  for (int k = 0; k < PER; ++k) {
+    mp[k] = ly.PiT[(int64_t)(sl * PER + k) * d + j];
+    ms[k] = ly.ST[(int64_t)(sl * PER + k) * d + j];
+  }
+  float cs1[4], cs2[4];                            // column sums at coordinates lane, lane + 64, ...
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int c = (tid & 63) + 64 * k;
+    cs1[k] = c < d ? ly.Pi_colsum[c] : 0.0f;
+    cs2[k] = c < d ? ly.S_colsum[c] : 0.0f;
+  }
+  float* sq = sm;                                   // [G][d] raw query
+  float* pa = sq + G * d;                           // [PREP_SLICES][G][PREP_COLS]
+  float* pb = pa + PREP_SLICES * G * PREP_COLS;
+  float* srot = pb + PREP_SLICES * G * PREP_COLS;   // [G][PREP_COLS]
+  float* ssk = srot + G * PREP_COLS;
+  float* stat = ssk + G * PREP_COLS;                // [G][4]
+  float* coefs = stat + 4 * ROT_MAX_ROWS;           // [16]
+  float* scale = coefs + 16;                        // [16]
+  const int64_t group = blockIdx.x, row0 = group * G;
+  for (int o = tid; o < G * d; o += blockDim.x) sq[o] = load_as_f32(q, row0 * d + o, dtype);
+  const int mb = ly.mse_bits;
+  int nx = 0;
+  float cmax = 0.0f;
+  for (int t = 0; t < ly.n_terms; ++t) {
+    cmax = fmaxf(cmax, fabsf(ly.term_coef[t]));
+    if (__builtin_popcount(ly.term_mask[t]) > 1) ++nx;
+  }
+  const int ntp = mb + nx + 1, wpl = d / 128;
+  if (tid < ntp) {
+    float coef = 1.0f;
+    if (tid < mb) {
+      coef = 0.0f;
+      for (int t = 0; t < ly.n_terms; ++t)
+        if (ly.term_mask[t] == (1 << (mb - 1 - tid))) coef = ly.term_coef[t];
+    } else if (tid < mb + nx) {
+      coef = 0.0f;
+      int seen = 0;
+      for (int t = 0; t < ly.n_terms; ++t) {
+        if (__builtin_popcount(ly.term_mask[t]) > 1) {
+          if (seen == tid - mb) coef = ly.term_coef[t];
+          ++seen;
+        }
+      }
+    }
+    coefs[tid] = coef;
+  }
+  if (tid >= 64 && tid < 80) scale[tid - 64] = ldexpf(1.0f, 127 - (1 << (qa_bit_slot(tid - 64) - 7)));
+  __syncthreads();
+  {  // row statistics: one wavefront per row
+    const int lane = tid & 63, wave = tid >> 6, n_wave = blockDim.x >> 6;
+    for (int r = wave; r < G; r += n_wave) {
+      float ss = 0.0f, s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const int c = lane + 64 * k;
+        const float x = c < d ? sq[r * d + c] : 0.0f;
+        ss = fmaf(x, x, ss);
+        s1 = fmaf(x, cs1[k], s1);
+        s2 = fmaf(x, cs2[k], s2);
+      }
+      ss = wave_sum(ss); s1 = wave_sum(s1); s2 = wave_sum(s2);
+      if (lane == 0) {
+        const float nq = sqrtf(ss);
+        stat[r * 4 + 0] = nq; stat[r * 4 + 1] = nq * ly.S_rownorm_max; stat[r * 4 + 2] = s1; stat[r * 4 + 3] = s2;
+        if (word == 0) {
+          q_stat[(row0 + r) * 4 + 0] = nq; q_stat[(row0 + r) * 4 + 1] = nq * ly.S_rownorm_max;
+          q_stat[(row0 + r) * 4 + 2] = s1; q_stat[(row0 + r) * 4 + 3] = s2;
+        }
+      }
+    }
+  }
+  // contraction over this thread's PER matrix rows
+  {
+    const int i0 = sl * PER;
+    float a[ROT_MAX_ROWS], b[ROT_MAX_ROWS];
+#pragma unroll
+    for (int r = 0; r < ROT_MAX_ROWS; ++r) a[r] = b[r] = 0.0f;
+#pragma unroll
+    for (int r = 0; r < ROT_MAX_ROWS; ++r) {
+      if (r < G) {
+#pragma unroll
+        for (int k = 0; k < PER; ++k) {
+          const float x = sq[r * d + i0 + k];
+          a[r] = fmaf(x, mp[k], a[r]);
+          b[r] = fmaf(x, ms[k], b[r]);
+        }
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < ROT_MAX_ROWS; ++r) {
+      if (r < G) {
+        pa[(sl * G + r) * PREP_COLS + jl] = a[r];
+        pb[(sl * G + r) * PREP_COLS + jl] = b[r];
+      }
+    }
+  }
+  __syncthreads();
+  for (int o = tid; o < G * PREP_COLS; o += blockDim.x) {
+    const int r = o / PREP_COLS, c = o - r * PREP_COLS;
+    float ra = 0.0f, rb = 0.0f;
+    for (int k = 0; k < PREP_SLICES; ++k) { ra += pa[(k * G + r) * PREP_COLS + c]; rb += pb[(k * G + r) * PREP_COLS + c]; }
+    srot[o] = ra;
+    ssk[o] = rb;
+    q_rot[(row0 + r) * d + word * PREP_COLS + c] = ra;
+    q_sk[(row0 + r) * d + word * PREP_COLS + c] = rb;
+  }
+  __syncthreads();
+  // operands of this plane word: [term plane][mfma u][16 lanes (2*g + part)][4 dwords]
+  const int i = word >> 2, kb = word & 3;
+  uint32_t* dst = qa_pack + group * (int64_t)(ntp * wpl * 4 * 64 * 4);
+  for (int o = tid; o < ntp * 256; o += blockDim.x) {
+    const int r = o & 3, n = (o >> 2) & 15, u = (o >> 6) & 3, tp = o >> 8;
+    const int g = n >> 1, part = n & 1;
+    uint32_t packed = 0;
+    if (g < G) {
+      const bool is_sign = tp == ntp - 1;
+      const float* src = (is_sign ? ssk : srot) + g * PREP_COLS;
+      const int bit = 4 * u + r;
+      const float inv = is_sign ? 1.0f / fmaxf(stat[g * 4 + 1], 1e-30f)
+                                : coefs[tp] / fmaxf(stat[g * 4 + 0] * cmax, 1e-30f);
+      const float mul = inv * scale[bit];
+      float v0 = src[bit] * mul, v1 = src[bit + 16] * mul;
+      if (part) {
+        v0 -= bf16_bits_to_f32(f32_to_bf16_bits(v0));
+        v1 -= bf16_bits_to_f32(f32_to_bf16_bits(v1));
+      }
+      packed = (uint32_t)f32_to_bf16_bits(v0) | ((uint32_t)f32_to_bf16_bits(v1) << 16);
+    }
+    dst[(((tp * wpl + i) * 4 + u) * 64 + n + 16 * kb) * 4 + r] = packed;
+  }
+}
+
 // scores[b, i, k] for a tile of QT queries and one key per thread.
 constexpr int QT = 8;
 
@@ -297,6 +451,16 @@ namespace tq {
 int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* layer, float* q_rot, float* q_sk,
                         float* q_stat, uint32_t* qa_pack, int G, hipStream_t st) {
   const int d = layer->d;
+  if (q_stat && qa_pack && layer->Pi_colsum && layer->S_colsum && G <= ROT_MAX_ROWS && rows % G == 0 &&
+      (d == 128 || d == 256)) {
+    size_t smem = (size_t)(G * d + 2 * PREP_SLICES * G * PREP_COLS + 2 * G * PREP_COLS + 4 * ROT_MAX_ROWS + 32) *
+                  sizeof(float);
+    const dim3 grid((unsigned)(rows / G), d / PREP_COLS), block(PREP_COLS * PREP_SLICES);
+    if (d == 128) prep_query_kernel<8><<<grid, block, smem, st>>>(q, dtype, G, *layer, q_rot, q_sk, q_stat, qa_pack);
+    else prep_query_kernel<16><<<grid, block, smem, st>>>(q, dtype, G, *layer, q_rot, q_sk, q_stat, qa_pack);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? TQ_OK : (int)e;
+  }
   // rows per workgroup: the GQA group when the decode operands are wanted, else up to 8
   const int R = (q_stat && G <= ROT_MAX_ROWS) ? G : (int)(rows < ROT_MAX_ROWS ? rows : ROT_MAX_ROWS);
   if (R < 1 || d % ROT_COLS || d % (8 * ROT_SLICES)) return TQ_EUNSUPPORTED;

@@ -111,10 +111,7 @@ class PagedKVPool:
         wavefront first builds its query operands."""
         blocks = max(1, (max_len + 63) // 64)
         pairs = max(1, B * self.num_kv_heads)
-        # head_dim 256 keeps one workgroup per CU resident (register budget), smaller heads two:
-        # a second round of workgroups would pay the per-workgroup set-up twice
-        resident = 256 if self.head_dim > 128 else 512
-        want = max(1, resident // pairs)
+        want = max(1, 512 // pairs)
         longest = max(1, blocks // 16)          # keep >= 4 blocks per wavefront
         return int(max(1, min(want, longest, 512)))
 

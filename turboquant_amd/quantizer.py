@@ -119,8 +119,14 @@ class TurboQuantMSE(torch.nn.Module):
             self._PiT = self.Pi.T.contiguous()
             self._splits = (key, (_ffi.split_bf16x3(self.Pi), _ffi.split_bf16x3(self._PiT),
                                   None if S is None else _ffi.split_bf16x3(S)))
+        qc = None
+        if S is not None:
+            if getattr(self, "_query_consts", None) is None or self._query_consts[0] != key:
+                self._query_consts = (key, (self.Pi.sum(dim=0).contiguous(), S.sum(dim=0).contiguous(),
+                                            float(S.norm(dim=1).max())))
+            qc = self._query_consts[1]
         return _ffi.make_layer(self.dim, self.bits, self.Pi, self._PiT, self.centroids, self.decision_boundaries,
-                               S, ST, centroids_host=self._centroids_host, splits=self._splits[1])
+                               S, ST, centroids_host=self._centroids_host, splits=self._splits[1], query_consts=qc)
 
     def quantize(self, x: torch.Tensor) -> MSEQuantized:
         """x (..., d) -> packed indices (..., d*eff/8) and norms (...) in x's dtype."""
