@@ -6,12 +6,12 @@
 //    of its index bits (Walsh expansion; for the symmetric codebooks simply of
 //    the individual index bits), so  sum_j q_rot[j] c[idx_j]  is a sum of
 //    "query . bit-plane" contractions, exactly like the QJL term
-//    sum_j q_sk[j] (2 bit_j - 1).  A bf16 whose only set bit is bit p (7..14) is
-//    the power of two 2^(2^(p-7)-127); one AND per pair of coordinates turns a
-//    32-bit plane word into MFMA B operands, and the query operand carries the
-//    inverse power of two, so the products are exact.  The query is split into
-//    bf16 hi + lo parts that occupy two rows of the 16-row A operand, which
-//    gives fp32-class scores.
+//    sum_j q_sk[j] (2 bit_j - 1).  The contraction runs on
+//    v_mfma_scale_f32_16x16x128_f8f6f4 with the bits as the fp4 operand: the nibble
+//    0001 is the fp4 number 0.5, so  (x >> s) & 0x11111111  for s = 0..3 turns a
+//    32-bit plane word into the four operand dwords (7 vector-ALU instructions for
+//    32 coordinates).  The query is the fp8 operand, split into three fp8 terms
+//    with per-row power-of-two scales (12 significant bits), prepared once per step.
 //  * values.  A code is OR-ed into the top mantissa bits of bf16(2^vb), i.e.
 //    B = 2^vb + code exactly; the softmax weight times the group scale is the A
 //    operand, and a second MFMA with B = -2^vb removes the offset with the very
@@ -42,6 +42,7 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef int i32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+typedef int i32x8 __attribute__((ext_vector_type(8)));
 
 constexpr int MF_WAVES = 4;
 constexpr int BLK_TOK = 64;              // tokens per wavefront iteration
@@ -93,20 +94,12 @@ __device__ __forceinline__ float row_sum16(float v) {
   return v;
 }
 
-// bit position p (inside each 16-bit half) that coordinate-pair `bit` of a plane
-// word occupies in the B operand of MFMA u = bit/4, register r = bit%4; the value
-// of that single-bit bf16 is 2^(2^(p-7) - 127)
-__host__ __device__ constexpr int bit_slot(int bit) { return bit <= 6 ? bit + 7 : (bit == 15 ? 14 : bit); }
-__host__ __device__ constexpr int slot_exponent(int p) { return (1 << (p - 7)) - 127; }
-
-// 32 coordinates of one plane word -> 16 dwords = B operands of 4 MFMAs
-__device__ __forceinline__ void expand_plane_word(uint32_t x, uint32_t (&b)[16]) {
-  const uint32_t xs = x << 7, xr = x >> 1;
-#pragma unroll
-  for (int bit = 0; bit < 16; ++bit) {
-    const uint32_t src = bit <= 6 ? xs : (bit == 15 ? xr : x);
-    b[bit] = src & (0x00010001u << bit_slot(bit));
-  }
+// fp8 (A: 16 rows x 128) x fp4 (B: 128 x 16) MFMA with per-lane power-of-two scales (E8M0 codes).
+// Only the first four dwords of the fp4 operand are read.
+__device__ __forceinline__ f32x4 mfma_f8f4(const i32x8& a, uint32_t b0, uint32_t b1, uint32_t b2, uint32_t b3,
+                                           f32x4 c, int scale_a, int scale_b) {
+  const i32x8 bv = {(int)b0, (int)b1, (int)b2, (int)b3, 0, 0, 0, 0};
+  return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, bv, c, 0 /*A: fp8 e4m3*/, 4 /*B: fp4*/, 0, scale_a, 0, scale_b);
 }
 
 // token held by element (r, h) of MFMA half u of the value stage
@@ -156,22 +149,21 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
   for (int t = 0; t < ly.n_terms; ++t) cmax = fmaxf(cmax, fabsf(ly.term_coef[t]));
 
   // ---------------------------------------------------------------- A operands of the score stage
-  // lane (row = n, kb): row -> (head g = row/2, part = row%2: bf16 hi / lo of the query); the query
-  // kernel has stored them in register order, one coalesced 1 KB load per register quadruple
-  u32x4 qa[NTP][WPL][4];
+  // fp8 query terms in register order (see the preparation kernel): row set 0 = terms 0, 1 of the 8
+  // heads (row 2g + t), row set 1 = term 2; rows of absent heads are zero
+  i32x8 qa[NTP][WPL][2];
   {
-    const u32x4* src = (const u32x4*)qa_pack + ((int64_t)b * Hkv + h) * (NTP * WPLT * 4 * 64) + lane;
-    const bool live = (n >> 1) < G;
+    const i32x8* src = (const i32x8*)qa_pack + ((int64_t)b * Hkv + h) * (NTP * WPLT * 2 * 64) + lane;
 #pragma unroll
     for (int tp = 0; tp < NTP; ++tp)
 #pragma unroll
       for (int i = 0; i < WPL; ++i)
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          u32x4 v = src[((tp * WPLT + hf * WPL + i) * 4 + u) * 64];
-          qa[tp][i][u] = live ? v : u32x4{0, 0, 0, 0};
-        }
+        for (int rs = 0; rs < 2; ++rs) qa[tp][i][rs] = src[((tp * WPLT + hf * WPL + i) * 2 + rs) * 64];
   }
+  // E8M0 scale codes: 64 v is stored, so term t carries 2^(-6 - 4t); the fp4 bit value 0.5 carries 2^1
+  const int sa01 = (n & 1) ? 127 - 10 : 127 - 6, sa2 = 127 - 14, sb = 127 + 1;
+  const uint32_t nib = in_vgpr(0x11111111u);
   // score constants of the two heads this lane sees in the MFMA output (rows 4kb..4kb+3 = heads 2kb, 2kb+1)
   float am[2], bm[2], aq[2], bq[2];
   int xplanes[NX > 0 ? NX : 1];                 // which stored planes each extra term XORs
@@ -273,7 +265,7 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
     float s2[2][4];
 #pragma unroll
     for (int pg = 0; pg < 4; ++pg) {
-      f32x4 dm = {0, 0, 0, 0}, dq = {0, 0, 0, 0};
+      f32x4 dm = {0, 0, 0, 0}, dq = {0, 0, 0, 0}, dm2 = {0, 0, 0, 0}, dq2 = {0, 0, 0, 0};
 #pragma unroll
       for (int i = 0; i < WPL; ++i) {
 #pragma unroll
@@ -286,20 +278,20 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
 #pragma unroll
             for (int p = 0; p < MB; ++p) x ^= ((xplanes[tp - MB] >> p) & 1) ? K.key[pg][i * (MB + 1) + p] : 0u;
           }
-          uint32_t bb[16];
-          expand_plane_word(x, bb);
-#pragma unroll
-          for (int u = 0; u < 4; ++u) {
-            u32x4 bv = {bb[4 * u], bb[4 * u + 1], bb[4 * u + 2], bb[4 * u + 3]};
-            if (tp == NTP - 1) dq = mfma(qa[tp][i][u], bv, dq);
-            else dm = mfma(qa[tp][i][u], bv, dm);
+          const uint32_t b0 = x & nib, b1 = (x >> 1) & nib, b2 = (x >> 2) & nib, b3 = (x >> 3) & nib;
+          if (tp == NTP - 1) {
+            dq = mfma_f8f4(qa[tp][i][0], b0, b1, b2, b3, dq, sa01, sb);
+            dq2 = mfma_f8f4(qa[tp][i][1], b0, b1, b2, b3, dq2, sa2, sb);
+          } else {
+            dm = mfma_f8f4(qa[tp][i][0], b0, b1, b2, b3, dm, sa01, sb);
+            dm2 = mfma_f8f4(qa[tp][i][1], b0, b1, b2, b3, dm2, sa2, sb);
           }
         }
       }
       const float nk = K.meta[pg][0], rk = K.meta[pg][1];
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
-        const float vm = dm[2 * j] + dm[2 * j + 1], vq = dq[2 * j] + dq[2 * j + 1];
+        const float vm = dm[2 * j] + dm[2 * j + 1] + dm2[j], vq = dq[2 * j] + dq[2 * j + 1] + dq2[j];
         // this wavefront's share of the score (the whole score when DS == 1); the constant
         // terms are added after the shares have met
         s2[j][pg] = fmaf(nk * am[j], vm, (rk * aq[j]) * vq);

@@ -67,105 +67,6 @@ rotate_query_kernel(const void* __restrict__ q, int dtype, int64_t rows, int R, 
   }
 }
 
-// Operands of the matrix-core decode kernel for one GQA group (G query heads of one
-// KV head), from the finished q_rot / q_sk rows.
-// q_stat receives per row {max|q_rot|, max|q_sk|, sum q_rot, sum q_sk}.
-// qa_pack receives the score-stage A operands in register order:
-// [kv head][term plane][word i][mfma u][lane 0..63][4 dwords], where lane
-// (n, kb) = (2*g + part, coordinate quarter), g the head within the group, part 0/1
-// the bf16 hi / lo half of the value, and element (r, h) of a register quadruple is
-// coordinate 32*(4i+kb) + 4u + r + 16h scaled by the inverse of the power of two its
-// bit occupies in the B operand.
-__host__ __device__ constexpr int qa_bit_slot(int bit) { return bit <= 6 ? bit + 7 : (bit == 15 ? 14 : bit); }
-
-__global__ void __launch_bounds__(1024)
-pack_query_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_sk, int G, tq_layer ly,
-                  float* __restrict__ q_stat, uint32_t* __restrict__ qa_pack) {
-  extern __shared__ float sm[];
-  const int d = ly.d, tid = threadIdx.x;
-  float* sq = sm;                 // [G][d]
-  float* sk = sq + G * d;         // [G][d]
-  float* stat = sk + G * d;       // [G][4]
-  const int64_t group = blockIdx.x, row0 = group * G;
-  for (int o = tid; o < G * d; o += blockDim.x) { sq[o] = q_rot[row0 * d + o]; sk[o] = q_sk[row0 * d + o]; }
-  __syncthreads();
-  {
-    const int lane = tid & 63, wave = tid >> 6, n_wave = blockDim.x >> 6;
-    for (int r = wave; r < G; r += n_wave) {
-      float m1 = 0.0f, m2 = 0.0f, s1 = 0.0f, s2 = 0.0f;
-      for (int c = lane; c < d; c += 64) {
-        const float x = sq[r * d + c], y = sk[r * d + c];
-        m1 = fmaxf(m1, fabsf(x)); m2 = fmaxf(m2, fabsf(y)); s1 += x; s2 += y;
-      }
-      m1 = wave_max(m1); m2 = wave_max(m2); s1 = wave_sum(s1); s2 = wave_sum(s2);
-      if (lane == 0) {
-        stat[r * 4 + 0] = m1; stat[r * 4 + 1] = m2; stat[r * 4 + 2] = s1; stat[r * 4 + 3] = s2;
-        q_stat[(row0 + r) * 4 + 0] = m1; q_stat[(row0 + r) * 4 + 1] = m2;
-        q_stat[(row0 + r) * 4 + 2] = s1; q_stat[(row0 + r) * 4 + 3] = s2;
-      }
-    }
-  }
-  if (!qa_pack) return;
-  const int mb = ly.mse_bits;
-  int nx = 0;
-  float cmax = 0.0f;
-  for (int t = 0; t < ly.n_terms; ++t) {
-    cmax = fmaxf(cmax, fabsf(ly.term_coef[t]));
-    if (__builtin_popcount(ly.term_mask[t]) > 1) ++nx;
-  }
-  const int ntp = mb + nx + 1, wpl = d / 128;
-  float* coefs = stat + 4 * G;          // [ntp] coefficient of each term plane (1 for the sign plane)
-  float* scale = coefs + 16;            // [16] inverse power of two of each bit slot
-  if (tid < ntp) {
-    float coef = 1.0f;
-    if (tid < mb) {
-      coef = 0.0f;
-      for (int t = 0; t < ly.n_terms; ++t)
-        if (ly.term_mask[t] == (1 << (mb - 1 - tid))) coef = ly.term_coef[t];
-    } else if (tid < mb + nx) {
-      coef = 0.0f;
-      int seen = 0;
-      for (int t = 0; t < ly.n_terms; ++t) {
-        if (__builtin_popcount(ly.term_mask[t]) > 1) {
-          if (seen == tid - mb) coef = ly.term_coef[t];
-          ++seen;
-        }
-      }
-    }
-    coefs[tid] = coef;
-  }
-  if (tid >= 64 && tid < 80) scale[tid - 64] = ldexpf(1.0f, 127 - (1 << (qa_bit_slot(tid - 64) - 7)));
-  __syncthreads();
-  if (tid < G) {                        // per head: 1 / normaliser of the rotated and of the sketched query
-    stat[tid * 4 + 2] = 1.0f / fmaxf(stat[tid * 4 + 0] * cmax, 1e-30f);
-    stat[tid * 4 + 3] = 1.0f / fmaxf(stat[tid * 4 + 1], 1e-30f);
-  }
-  __syncthreads();
-  // one thread per output word, in storage order (coalesced stores); lanes of absent heads get zeros
-  const int total = ntp * wpl * 4 * 64 * 4;
-  uint32_t* dst = qa_pack + group * (int64_t)total;
-  for (int o = tid; o < total; o += blockDim.x) {
-    const int r = o & 3, lane = (o >> 2) & 63, u = (o >> 8) & 3;
-    const int i = (o >> 10) % wpl, tp = (o >> 10) / wpl;
-    const int kb = lane >> 4, g = (lane & 15) >> 1, part = lane & 1;
-    uint32_t packed = 0;
-    if (g < G) {
-      const bool is_sign = tp == ntp - 1;
-      const float* src = (is_sign ? sk : sq) + g * d;
-      const int bit = 4 * u + r;
-      const float mul = (is_sign ? stat[g * 4 + 3] : coefs[tp] * stat[g * 4 + 2]) * scale[bit];
-      const int c0 = 32 * (4 * i + kb) + bit;
-      float v0 = src[c0] * mul, v1 = src[c0 + 16] * mul;
-      if (part) {
-        v0 -= bf16_bits_to_f32(f32_to_bf16_bits(v0));
-        v1 -= bf16_bits_to_f32(f32_to_bf16_bits(v1));
-      }
-      packed = (uint32_t)f32_to_bf16_bits(v0) | ((uint32_t)f32_to_bf16_bits(v1) << 16);
-    }
-    dst[o] = packed;
-  }
-}
-
 // Fused preparation of the matrix-core decode kernel: rotation, sketch, statistics and
 // operand packing in one launch.  A workgroup owns one GQA group (G query heads of one KV
 // head) and the 32 output coordinates of one plane word; PREP_SLICES threads share a
@@ -174,7 +75,22 @@ pack_query_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_s
 // |q_rot_j| <= ||q|| (Pi is orthogonal) and |q_sk_j| <= ||q|| max_j ||S_j||, and the sums
 // over all coordinates that the decode kernel needs are q . colsum(Pi), q . colsum(S).
 // q_stat per row: {||q||, ||q|| max_j ||S_j||, sum_j q_rot_j, sum_j q_sk_j}.
+//
+// qa_pack receives the score-stage A operands of v_mfma_scale_f32_16x16x128_f8f6f4 (A fp8 e4m3,
+// B fp4) in register order: [kv head][term plane][128-coordinate chunk i][row set][lane][8 dwords].
+// A value v (the normalised query coordinate times the plane's coefficient, |v| <= 1) is the sum
+// of three fp8 terms with per-row scales 2^-6, 2^-10, 2^-14: t0 = fp8(64 v), t1 = fp8(16 (64 v - t0)),
+// t2 = fp8(16 (16 (64 v - t0) - t1)).  Row set 0 holds terms 0 and 1 (row 2g + t for head g), row
+// set 1 holds term 2 in rows 4(g/2) + g%2 (the other rows are zero), so that a lane of the MFMA
+// output sees the same two heads in both.  The hardware takes, for lane (row, block b), bytes
+// 0..15 as contraction indices 16b..16b+15 and bytes 16..31 as 64+16b..64+16b+15, and the key
+// kernel puts coordinate c of plane word w at contraction index 32w + 8 (c % 4) + c / 4.
 constexpr int PREP_COLS = 32, PREP_SLICES = 16;
+
+__device__ __forceinline__ uint32_t f32_to_fp8(float v) {
+  return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(v, 0.0f, 0, false) & 0xffu;
+}
+__device__ __forceinline__ float fp8_to_f32(uint32_t b) { return __builtin_amdgcn_cvt_f32_fp8((int)b, 0); }
 
 template <int PER>      // matrix rows per thread = d / PREP_SLICES
 __global__ void __launch_bounds__(PREP_COLS * PREP_SLICES)
@@ -205,7 +121,6 @@ prep_query_kernel(const void* __restrict__ q, int dtype, int G, tq_layer ly, flo
   float* ssk = srot + G * PREP_COLS;
   float* stat = ssk + G * PREP_COLS;                // [G][4]
   float* coefs = stat + 4 * ROT_MAX_ROWS;           // [16]
-  float* scale = coefs + 16;                        // [16]
   const int64_t group = blockIdx.x, row0 = group * G;
   for (int o = tid; o < G * d; o += blockDim.x) sq[o] = load_as_f32(q, row0 * d + o, dtype);
   const int mb = ly.mse_bits;
@@ -234,7 +149,6 @@ prep_query_kernel(const void* __restrict__ q, int dtype, int G, tq_layer ly, flo
     }
     coefs[tid] = coef;
   }
-  if (tid >= 64 && tid < 80) scale[tid - 64] = ldexpf(1.0f, 127 - (1 << (qa_bit_slot(tid - 64) - 7)));
   __syncthreads();
   {  // row statistics: one wavefront per row
     const int lane = tid & 63, wave = tid >> 6, n_wave = blockDim.x >> 6;
@@ -295,28 +209,35 @@ prep_query_kernel(const void* __restrict__ q, int dtype, int G, tq_layer ly, flo
     q_sk[(row0 + r) * d + word * PREP_COLS + c] = rb;
   }
   __syncthreads();
-  // operands of this plane word: [term plane][mfma u][16 lanes (2*g + part)][4 dwords]
-  const int i = word >> 2, kb = word & 3;
-  uint32_t* dst = qa_pack + group * (int64_t)(ntp * wpl * 4 * 64 * 4);
+  // operands of this plane word: per (term plane, row set, row) two lanes x four dwords
+  const int i = word >> 2, kw = word & 3;
+  uint32_t* dst = qa_pack + group * (int64_t)(ntp * wpl * 2 * 64 * 8);
   for (int o = tid; o < ntp * 256; o += blockDim.x) {
-    const int r = o & 3, n = (o >> 2) & 15, u = (o >> 6) & 3, tp = o >> 8;
-    const int g = n >> 1, part = n & 1;
+    const int dw = o & 3, bsel = (o >> 2) & 1, n = (o >> 3) & 15, rs = (o >> 7) & 1, tp = o >> 8;
+    int g, term;
+    if (rs == 0) { g = n >> 1; term = n & 1; }
+    else { g = 2 * (n >> 2) + (n & 3); term = (n & 3) < 2 ? 2 : -1; }
     uint32_t packed = 0;
-    if (g < G) {
+    if (term >= 0 && g < G) {
       const bool is_sign = tp == ntp - 1;
       const float* src = (is_sign ? ssk : srot) + g * PREP_COLS;
-      const int bit = 4 * u + r;
-      const float inv = is_sign ? 1.0f / fmaxf(stat[g * 4 + 1], 1e-30f)
-                                : coefs[tp] / fmaxf(stat[g * 4 + 0] * cmax, 1e-30f);
-      const float mul = inv * scale[bit];
-      float v0 = src[bit] * mul, v1 = src[bit + 16] * mul;
-      if (part) {
-        v0 -= bf16_bits_to_f32(f32_to_bf16_bits(v0));
-        v1 -= bf16_bits_to_f32(f32_to_bf16_bits(v1));
+      const float mul = 64.0f * (is_sign ? 1.0f / fmaxf(stat[g * 4 + 1], 1e-30f)
+                                         : coefs[tp] / fmaxf(stat[g * 4 + 0] * cmax, 1e-30f));
+#pragma unroll
+      for (int by = 0; by < 4; ++by) {
+        const int kloc = 16 * bsel + 4 * dw + by;            // contraction index within the word's 32
+        const int c = 4 * (kloc & 7) + (kloc >> 3);          // coordinate within the word
+        float v = src[c] * mul;
+        uint32_t code = f32_to_fp8(v);
+        for (int t = 0; t < term; ++t) {
+          v = (v - fp8_to_f32(code)) * 16.0f;
+          code = f32_to_fp8(v);
+        }
+        packed |= code << (8 * by);
       }
-      packed = (uint32_t)f32_to_bf16_bits(v0) | ((uint32_t)f32_to_bf16_bits(v1) << 16);
     }
-    dst[(((tp * wpl + i) * 4 + u) * 64 + n + 16 * kb) * 4 + r] = packed;
+    const int lane = n + 16 * (2 * (kw & 1) + bsel), dword = 4 * (kw >> 1) + dw;
+    dst[(((tp * wpl + i) * 2 + rs) * 64 + lane) * 8 + dword] = packed;
   }
 }
 
@@ -451,8 +372,9 @@ namespace tq {
 int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* layer, float* q_rot, float* q_sk,
                         float* q_stat, uint32_t* qa_pack, int G, hipStream_t st) {
   const int d = layer->d;
-  if (q_stat && qa_pack && layer->Pi_colsum && layer->S_colsum && G <= ROT_MAX_ROWS && rows % G == 0 &&
-      (d == 128 || d == 256)) {
+  if (qa_pack) {       // operands of the matrix-core decode kernel wanted
+    if (!q_stat || !layer->Pi_colsum || !layer->S_colsum || G > ROT_MAX_ROWS || rows % G || (d != 128 && d != 256))
+      return TQ_EUNSUPPORTED;
     size_t smem = (size_t)(G * d + 2 * PREP_SLICES * G * PREP_COLS + 2 * G * PREP_COLS + 4 * ROT_MAX_ROWS + 32) *
                   sizeof(float);
     const dim3 grid((unsigned)(rows / G), d / PREP_COLS), block(PREP_COLS * PREP_SLICES);
@@ -461,21 +383,13 @@ int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* 
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? TQ_OK : (int)e;
   }
-  // rows per workgroup: the GQA group when the decode operands are wanted, else up to 8
-  const int R = (q_stat && G <= ROT_MAX_ROWS) ? G : (int)(rows < ROT_MAX_ROWS ? rows : ROT_MAX_ROWS);
+  const int R = (int)(rows < ROT_MAX_ROWS ? rows : ROT_MAX_ROWS);      // rows per workgroup
   if (R < 1 || d % ROT_COLS || d % (8 * ROT_SLICES)) return TQ_EUNSUPPORTED;
   size_t smem = (size_t)(R * d + 2 * ROT_SLICES * R * ROT_COLS) * sizeof(float);
   rotate_query_kernel<<<dim3((unsigned)((rows + R - 1) / R), d / ROT_COLS), dim3(ROT_COLS * ROT_SLICES), smem, st>>>(
       q, dtype, rows, R, *layer, q_rot, q_sk);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return (int)e;
-  if (q_stat) {
-    if (G > ROT_MAX_ROWS * 2 || rows % G) return TQ_EUNSUPPORTED;
-    size_t psm = (size_t)(2 * G * d + 4 * G + 32) * sizeof(float);
-    pack_query_kernel<<<dim3((unsigned)(rows / G)), dim3(1024), psm, st>>>(q_rot, q_sk, G, *layer, q_stat, qa_pack);
-    e = hipGetLastError();
-    if (e != hipSuccess) return (int)e;
-  }
   return TQ_OK;
 }
 }  // namespace tq
