@@ -305,6 +305,146 @@ value_tile_kernel(const void* __restrict__ v, Source src, int d, int gs, int bit
   }
 }
 
+// round to the input dtype and back with the hardware conversions (v_cvt_pk_bf16_f32 / v_cvt_f16_f32,
+// round to nearest even; NaN stays NaN)
+template <int DT>
+__device__ __forceinline__ float round_hw(float v) {
+  if constexpr (DT == TQ_BF16) {
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    const f32x2_t f = {v, 0.0f};
+    const bf16x2_t r = __builtin_convertvector(f, bf16x2_t);
+    uint32_t u;
+    __builtin_memcpy(&u, &r, 4);
+    return __uint_as_float(u << 16);
+  } else {
+    return Elem<DT>::round(v);
+  }
+}
+
+// Faster value kernel for 16-bit inputs, 2/4-bit codes and head_dim 64 / 128 / 256: a thread owns 8
+// consecutive channels of one token (one 16-byte load), a group's minimum / maximum meet through
+// cross-lane exchanges, and the codes pass through LDS only to be transposed into the page's
+// per-channel fields.  Arithmetic and rounding are those of value_tile_kernel.
+template <int DT, int VB, class Source, class Sink>
+__global__ void __launch_bounds__(512)
+value_chunk_kernel(const void* __restrict__ v, Source src, int d, int gs, Sink sink) {
+  using E = Elem<DT>;
+  static_assert(DT != TQ_F32, "16-bit inputs");
+  const int tid = threadIdx.x, tile = blockIdx.x;
+  const int cpt = d >> 3;                          // chunks (threads) per token
+  const int t = tid / cpt, ck = tid - t * cpt;     // token slot, chunk
+  const int tpg = gs >> 3;                         // threads per group (power of two, <= 16)
+  extern __shared__ __align__(16) unsigned char smem[];
+  uint8_t* scode = smem;                           // [TILE][d]
+  int* svalid = (int*)(smem + TILE * d);           // [TILE]
+
+  const typename Source::TileRef ref = src.tile_ref(tile);
+  int64_t off;
+  const bool ok = src.slot_off(ref, t, off);
+  // page lookup issued together with the input load (clamped into the table: a tile without a
+  // single existing slot may lie beyond it, and then nothing is stored anyway)
+  int64_t page = 0;
+  int head = 0;
+  if constexpr (!std::is_same<Sink, ValFlatSink>::value) {
+    int b, lpage;
+    src.decode(tile, b, lpage, head);
+    page = sink.block_table[(int64_t)b * sink.max_pages + min(lpage, sink.max_pages - 1)];
+  }
+  // unconditional load (slots that do not exist read the first vector)
+  const uint4 raw = *(const uint4*)((const uint16_t*)v + (ok ? off : 0) + ck * 8);
+  if (ck == 0) svalid[t] = ok;
+  // a tile none of whose slots exists may lie beyond the block table: leave before looking it up
+  if (!__syncthreads_or(ok)) return;
+  float x[8];
+  {
+    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      x[2 * i] = DT == TQ_BF16 ? __uint_as_float(w[i] << 16) : f16_bits_to_f32((uint16_t)(w[i] & 0xffffu));
+      x[2 * i + 1] = DT == TQ_BF16 ? __uint_as_float(w[i] & 0xffff0000u) : f16_bits_to_f32((uint16_t)(w[i] >> 16));
+    }
+  }
+  float lo = x[0], hi = x[0];
+  int has_nan = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    has_nan |= (x[i] != x[i]);
+    lo = fminf(lo, x[i]);
+    hi = fmaxf(hi, x[i]);
+  }
+  for (int o = 1; o < tpg; o <<= 1) {              // the threads of a group are neighbouring lanes
+    lo = fminf(lo, __shfl_xor(lo, o, 64));
+    hi = fmaxf(hi, __shfl_xor(hi, o, 64));
+    has_nan |= __shfl_xor(has_nan, o, 64);
+  }
+  if (has_nan) lo = hi = __uint_as_float(0x7fc00000u);       // torch min/max propagate NaN
+  const float levels = (float)((1 << VB) - 1);
+  float sc = round_hw<DT>(round_hw<DT>(hi - lo) / levels);
+  const float floor_v = round_hw<DT>(1e-10f);
+  sc = (sc != sc) ? sc : fmaxf(sc, floor_v);
+  const float z = lo;
+  uint32_t codes = 0;                              // 8 codes, VB bits each, channel order
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    float q = round_hw<DT>(round_hw<DT>(x[i] - z) / sc);
+    q = rintf(q);
+    q = fminf(fmaxf(q, 0.0f), levels);
+    const uint32_t c = (q != q) ? 0u : (uint32_t)q;
+    codes |= c << (VB * i);
+    if constexpr (!std::is_same<Sink, ValFlatSink>::value) scode[t * d + ck * 8 + i] = (uint8_t)c;
+  }
+  const int ng = d / gs, g = (ck * 8) / gs;
+  const bool leader = (ck & (tpg - 1)) == 0;
+
+  if constexpr (std::is_same<Sink, ValFlatSink>::value) {
+    if (ok) {
+      const int64_t vec = (int64_t)tile * TILE + t;
+      uint8_t* dst = sink.data + vec * (d * VB / 8) + ck * VB;           // 8 codes = VB bytes, little-end first
+      if (VB == 2) *(uint16_t*)dst = (uint16_t)codes;
+      else *(uint32_t*)dst = codes;
+      if (leader) {
+        E::store(sink.scale, vec * ng + g, sc);
+        E::store(sink.zero, vec * ng + g, z);
+      }
+    }
+  } else {
+    const tq_page_layout& L = sink.L;
+    uint8_t* pg = sink.pool + (page * src.H + head) * (int64_t)L.page_bytes;
+    if (ok && leader) {
+      E::store(pg + L.off_vscale, g * TILE + t, sc);
+      E::store(pg + L.off_vzero, g * TILE + t, z);
+    }
+    __syncthreads();
+    // channel c: a field of 16*VB bits, token n at bit VB*n; read-modify-write keeps the codes of
+    // slots this call does not touch
+    // every thread assembles half a field: 8 tokens of one channel (16 bits of 2-bit codes, 32 of 4-bit)
+    {
+      const int c = tid >> 1, half = tid & 1;
+      uint8_t* fbytes = pg + vfield_off(L, c) + half * VB;
+      uint32_t neu = 0, mask = 0;
+#pragma unroll
+      for (int s2 = 0; s2 < 8; ++s2) {
+        const int n = half * 8 + s2;
+        const uint32_t keep = svalid[n] ? (1u << VB) - 1u : 0u;
+        neu |= ((uint32_t)scode[n * d + c] & keep) << (VB * s2);
+        mask |= keep << (VB * s2);
+      }
+      if (mask != 0) {
+        if (VB == 2) {
+          uint16_t* f16p = (uint16_t*)fbytes;
+          const uint32_t old = (mask == 0xffffu) ? 0u : *f16p;
+          *f16p = (uint16_t)((old & ~mask) | neu);
+        } else {
+          uint32_t* f32p = (uint32_t*)fbytes;
+          const uint32_t old = (mask == 0xffffffffu) ? 0u : *f32p;
+          *f32p = (old & ~mask) | neu;
+        }
+      }
+    }
+  }
+}
+
 static size_t value_tile_smem(int d, int gs) { return (size_t)TILE * d * 5 + (size_t)TILE * (d / gs) * 8 + TILE * 4; }
 
 // ------------------------------------------------------------------------------------
@@ -488,9 +628,28 @@ static int launch_key(const void* x, int dtype, const Source& src, const tq_laye
   return TQ_OK;
 }
 
+static bool value_chunks_aligned(const void* v, const FlatSource& s) {
+  return (uintptr_t)v % 16 == 0 && s.row_stride % 8 == 0;
+}
+static bool value_chunks_aligned(const void* v, const PagedSource& s) {
+  return (uintptr_t)v % 16 == 0 && s.stride_b % 8 == 0 && s.stride_t % 8 == 0 && s.stride_h % 8 == 0;
+}
+
 template <class Source, class Sink>
 static int launch_value(const void* v, int dtype, const Source& src, int d, int gs, int bits, const Sink& sink,
                         int64_t tiles, hipStream_t st) {
+  // 16-bit inputs with 2/4-bit codes on the usual head sizes take the chunked kernel
+  if (dtype != TQ_F32 && (bits == 2 || bits == 4) && (d == 64 || d == 128 || d == 256) && gs >= 16 && gs <= 128 &&
+      (gs & (gs - 1)) == 0 && value_chunks_aligned(v, src)) {
+    const size_t sm = (size_t)TILE * d + TILE * sizeof(int);
+    const dim3 g2((unsigned)tiles), b2(TILE * d / 8);
+#define TQ_LAUNCH_VC(DT, VB) value_chunk_kernel<DT, VB, Source, Sink><<<g2, b2, sm, st>>>(v, src, d, gs, sink)
+    if (dtype == TQ_BF16) { if (bits == 2) TQ_LAUNCH_VC(TQ_BF16, 2); else TQ_LAUNCH_VC(TQ_BF16, 4); }
+    else { if (bits == 2) TQ_LAUNCH_VC(TQ_F16, 2); else TQ_LAUNCH_VC(TQ_F16, 4); }
+#undef TQ_LAUNCH_VC
+    TQ_CHECK_LAUNCH();
+    return TQ_OK;
+  }
   size_t smem = value_tile_smem(d, gs);
   dim3 grid((unsigned)tiles), block(d);
 #define TQ_LAUNCH_VAL(DT)                                                                              \

@@ -278,6 +278,17 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
   const int tr = tid / CPR, ck = tid % CPR;
   const int64_t tile0 = g * MT;
   lookup_x(g + gridDim.x);                                      // read long before issue_x needs it
+  // page of the tile this wavefront will write, looked up now so that the write phase does not
+  // wait for it (clamped into the table: a tile without a single existing slot may lie beyond it)
+  int64_t wpage = 0;
+  if constexpr (!std::is_same<Sink, KeyFlatSink>::value) {
+    const int64_t wt = tile0 + wave % MT;
+    if (wt < n_tiles) {
+      int b, lpage, h;
+      src.decode((int)wt, b, lpage, h);
+      wpage = sink.block_table[(int64_t)b * sink.max_pages + min(lpage, sink.max_pages - 1)];
+    }
+  }
 #pragma unroll
   for (int j = 0; j < PER; ++j) {
     const bool ok = (xok >> j) & 1;
@@ -480,10 +491,11 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
     for (int m = wave % MT; m < MT; m += KQ_WAVES) {
       const int64_t tile = tile0 + m;
       if (tile >= n_tiles) break;
+      // a tile none of whose slots exists may lie beyond the block table: do not look it up
+      if (__builtin_amdgcn_ballot_w64(lane < TILE && svalid[16 * m + lane]) == 0) continue;
       int b, lpage, h;
       src.decode((int)tile, b, lpage, h);
-      const int64_t page = sink.block_table[(int64_t)b * sink.max_pages + lpage];
-      uint8_t* pg = sink.pool + (page * src.H + h) * (int64_t)L.page_bytes;
+      uint8_t* pg = sink.pool + (wpage * src.H + h) * (int64_t)L.page_bytes;
       for (int p = wave / MT; p < planes; p += NSUB) {
 #pragma unroll
         for (int e = lane; e < W * TILE; e += 64) {
