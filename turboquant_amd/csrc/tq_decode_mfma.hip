@@ -263,6 +263,10 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
   auto score_stage = [&](int blk, int it, const KeyRegs& K, auto partial_tag) -> bool {
     constexpr bool PARTIAL = decltype(partial_tag)::value;
     float s2[2][4];
+    // The MFMA-dense parts run at raised wavefront priority (the value stage above the score
+    // stage): the SIMD's other wavefront then fills the gaps with its vector-ALU work instead of
+    // both alternating between the two kinds of instruction.
+    __builtin_amdgcn_s_setprio(1);
 #pragma unroll
     for (int pg = 0; pg < 4; ++pg) {
       f32x4 dm = {0, 0, 0, 0}, dq = {0, 0, 0, 0}, dm2 = {0, 0, 0, 0}, dq2 = {0, 0, 0, 0};
@@ -297,6 +301,7 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
         s2[j][pg] = fmaf(nk * am[j], vm, (rk * aq[j]) * vq);
       }
     }
+    __builtin_amdgcn_s_setprio(0);
     if (DS > 1) {
       // exchange with the wavefront that scored the other coordinates: own share -> LDS, workgroup
       // barrier, partner's share <- LDS.  a + b == b + a, so both end with bit-identical scores.
@@ -410,6 +415,7 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
       }
       zacc = mfma(ap, bz, zacc);
     }
+    __builtin_amdgcn_s_setprio(2);
 #pragma unroll
     for (int grp = 0; grp < NG; ++grp) {
       // w = weight * scale for the 16 tokens of page kb, then the two A operands in the value token order
@@ -450,6 +456,7 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
         }
       }
     }
+    __builtin_amdgcn_s_setprio(0);
     __builtin_amdgcn_wave_barrier();
   };
 
