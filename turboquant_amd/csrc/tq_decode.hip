@@ -269,7 +269,7 @@ using namespace tq;
 
 namespace tq {
 int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* layer, float* q_rot, float* q_sk,
-                        float* q_stat, uint32_t* qa_pack, int G, hipStream_t st);
+                        float* q_stat, uint32_t* qa_pack, int G, float sm_scale, hipStream_t st);
 size_t decode_mfma_pack_words(int B, int Hkv, int d);
 int launch_decode_mfma(const uint32_t* qa_pack, const float* q_stat, int B, int Hq, int Hkv,
                        const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
@@ -329,7 +329,7 @@ extern "C" int tq_decode_attn_paged_stages(const void* q, int dtype, int B, int 
     if (!layer->Pi || !layer->PiT || !layer->S || !layer->ST || !layer->centroids) return TQ_ENULL;
     if (dtype < TQ_F32 || dtype > TQ_BF16) return TQ_EINVAL;
     int rc = launch_rotate_query(q, dtype, (int64_t)B * Hq, layer, q_rot, q_sk, q_stat, mfma_shape ? qa_pack : nullptr,
-                                 G, st);
+                                 G, sm_scale, st);
     if (rc) return rc;
   }
   if (!(stages & 6)) return TQ_OK;

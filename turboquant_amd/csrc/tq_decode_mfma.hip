@@ -1,4 +1,4 @@
-// Page-streaming decode kernel on the matrix cores (gfx950, bf16 MFMA 16x16x32).
+// Page-streaming decode kernel on the matrix cores (gfx950).
 //
 // The packed bits feed the matrix cores almost directly:
 //
@@ -11,11 +11,15 @@
 //    0001 is the fp4 number 0.5, so  (x >> s) & 0x11111111  for s = 0..3 turns a
 //    32-bit plane word into the four operand dwords (7 vector-ALU instructions for
 //    32 coordinates).  The query is the fp8 operand, split into three fp8 terms
-//    with per-row power-of-two scales (12 significant bits), prepared once per step.
-//  * values.  A code is OR-ed into the top mantissa bits of bf16(2^vb), i.e.
-//    B = 2^vb + code exactly; the softmax weight times the group scale is the A
-//    operand, and a second MFMA with B = -2^vb removes the offset with the very
-//    same A.  The zero points go through one more MFMA (weights x zeros).
+//    with per-row power-of-two scales (12 significant bits), prepared once per step;
+//    every factor and constant of the score that belongs to a query head is folded
+//    into those operands, their block scales and the initial accumulator.
+//  * values.  A code masked out of its packed word IS a bf16 denormal (exponent
+//    field zero, the code in the low mantissa bits): B = code * 2^(s-133) exactly,
+//    s being the bit position the code has in its 16-bit half, and the bf16 MFMA
+//    (v_mfma_f32_16x16x32_bf16) keeps denormal inputs.  The softmax weight times the
+//    group scale times 2^(100-s) is the A operand; the accumulators carry 2^-33
+//    until the epilogue.  The zero points go through one more MFMA (weights x zeros).
 //
 // head_dim 256 is split over a pair of wavefronts (DS = 2): each scores half of the
 // coordinates, the halves of the scores meet in LDS once per block, both wavefronts
@@ -96,10 +100,12 @@ __device__ __forceinline__ float row_sum16(float v) {
 
 // fp8 (A: 16 rows x 128) x fp4 (B: 128 x 16) MFMA with per-lane power-of-two scales (E8M0 codes).
 // Only the first four dwords of the fp4 operand are read.
+// SEL picks the byte of scale_a that holds the code.
+template <int SEL>
 __device__ __forceinline__ f32x4 mfma_f8f4(const i32x8& a, uint32_t b0, uint32_t b1, uint32_t b2, uint32_t b3,
                                            f32x4 c, int scale_a, int scale_b) {
   const i32x8 bv = {(int)b0, (int)b1, (int)b2, (int)b3, 0, 0, 0, 0};
-  return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, bv, c, 0 /*A: fp8 e4m3*/, 4 /*B: fp4*/, 0, scale_a, 0, scale_b);
+  return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, bv, c, 0 /*A: fp8 e4m3*/, 4 /*B: fp4*/, SEL, scale_a, 0, scale_b);
 }
 
 // token held by element (r, h) of MFMA half u of the value stage
@@ -135,7 +141,6 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wgrp = wave / DS, hf = wave % DS; // block walker this wavefront belongs to; its share of the head
   const int n = lane & 15, kb = lane >> 4;    // score stage: token / coordinate quarter; value stage: row / page
-  const float LOG2E = 1.4426950408889634f;
 
   extern __shared__ __align__(16) unsigned char smem_raw[];
   float* s_p = (float*)smem_raw + wave * WAVE_LDS_FLOATS;   // [4 pages][16 rows][P_STRIDE]
@@ -145,12 +150,9 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
   float* s_x_peer = (float*)smem_raw + (wave ^ 1) * WAVE_LDS_FLOATS + (4 * 16 * P_STRIDE + 16 + 4 * NG * 16);
   float* s_red = (float*)smem_raw;                          // after the loop: [NGRP][G][D + 2]
 
-  float cmax = 0.0f;
-  for (int t = 0; t < ly.n_terms; ++t) cmax = fmaxf(cmax, fabsf(ly.term_coef[t]));
-
   // ---------------------------------------------------------------- A operands of the score stage
   // fp8 query terms in register order (see the preparation kernel): row set 0 = terms 0, 1 of the 8
-  // heads (row 2g + t), row set 1 = term 2; rows of absent heads are zero
+  // heads (row 2g + t), row set 1 = term 2 in row 2g; rows of absent heads are zero
   i32x8 qa[NTP][WPL][2];
   {
     const i32x8* src = (const i32x8*)qa_pack + ((int64_t)b * Hkv + h) * (NTP * WPLT * 2 * 64) + lane;
@@ -161,24 +163,31 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
 #pragma unroll
         for (int rs = 0; rs < 2; ++rs) qa[tp][i][rs] = src[((tp * WPLT + hf * WPL + i) * 2 + rs) * 64];
   }
-  // E8M0 scale codes: 64 v is stored, so term t carries 2^(-6 - 4t); the fp4 bit value 0.5 carries 2^1
-  const int sa01 = (n & 1) ? 127 - 10 : 127 - 6, sa2 = 127 - 14, sb = 127 + 1;
+  // E8M0 block-scale codes of this lane's operand row (head n / 2), one per byte: index planes row
+  // set 0, row set 1, sign plane row set 0, row set 1.  64 v / 2^E is stored, so term t carries
+  // 2^(E - 6 - 4t); the fp4 bit value 0.5 carries 2^1.
+  int sa;
+  {
+    const int g = n >> 1;
+    const int64_t qrow = (int64_t)b * Hq + h * G + (g < G ? g : 0);
+    const int e1 = 127 + (int)q_stat[qrow * 4 + 0], e2 = 127 + (int)q_stat[qrow * 4 + 1];
+    const int t01 = (n & 1) ? 10 : 6;
+    sa = (e1 - t01) | ((e1 - 14) << 8) | ((e2 - t01) << 16) | ((e2 - 14) << 24);
+  }
+  const int sb = 127 + 1;
   const uint32_t nib = in_vgpr(0x11111111u);
-  // score constants of the two heads this lane sees in the MFMA output (rows 4kb..4kb+3 = heads 2kb, 2kb+1)
-  float am[2], bm[2], aq[2], bq[2];
+  // constant parts of the scores of the two heads this lane sees in the MFMA output (rows 4kb..4kb+3
+  // = heads 2kb, 2kb+1), as the initial accumulators; only one wavefront of a pair adds them
+  f32x4 cm = {0, 0, 0, 0}, cq = {0, 0, 0, 0};
   int xplanes[NX > 0 ? NX : 1];                 // which stored planes each extra term XORs
   {
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       const int g = 2 * kb + j;
-      const bool live = g < G;
-      const int64_t qrow = (int64_t)b * Hq + h * G + (live ? g : 0);
-      const float m1 = fmaxf(q_stat[qrow * 4 + 0] * cmax, 1e-30f), m2 = fmaxf(q_stat[qrow * 4 + 1], 1e-30f);
-      const float k = live ? sm_scale * LOG2E : 0.0f;
-      am[j] = k * m1;
-      bm[j] = k * ly.term_const * q_stat[qrow * 4 + 2];
-      aq[j] = 2.0f * k * ly.qjl_scale * m2;
-      bq[j] = -k * ly.qjl_scale * q_stat[qrow * 4 + 3];
+      const bool live = g < G && hf == 0;
+      const int64_t qrow = (int64_t)b * Hq + h * G + (g < G ? g : 0);
+      cm[2 * j] = live ? q_stat[qrow * 4 + 2] : 0.0f;
+      cq[2 * j] = live ? q_stat[qrow * 4 + 3] : 0.0f;
     }
     int seen = 0;
     for (int t = 0; t < ly.n_terms; ++t) {
@@ -249,14 +258,11 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
     R.scale = *(const u32x4*)(pool_h + spid * page_stride + off_scale);
   };
 
-  // A value code sits in the low mantissa bits of bf16(128): B = 128 + code * 2^s exactly, where s
-  // is the bit position the code already has inside its packed word (0, 2 or 4 for 2-bit codes,
-  // 0 for 4-bit codes), so that most codes need no shift; the softmax weight carries 2^-s.
-  const uint32_t base_pat = in_vgpr(0x43004300u);                           // bf16 pairs of 128
+  // A value code masked in place is a bf16 denormal: B = code * 2^(s - 133) exactly, where s is the
+  // bit position the code already has inside its 16-bit half (0, 2 or 4 for 2-bit codes, 0 for
+  // 4-bit codes), so that most codes need no shift; the softmax weight carries 2^(100 - s).
   const uint32_t m0 = in_vgpr(VB == 2 ? 0x00030003u : 0x000F000Fu);
   const uint32_t m1 = in_vgpr(0x000C000Cu), m2 = in_vgpr(0x00300030u);
-  const uint32_t neg_pat = 0xC300C300u;                                     // bf16 pairs of -128
-  const u32x4 neg_base = {neg_pat, neg_pat, neg_pat, neg_pat};
 
   // ---------------------------------------------------------------- one block of 64 tokens
   // scores of the 4 pages of block blk, online softmax, weights -> LDS
@@ -269,7 +275,7 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
     __builtin_amdgcn_s_setprio(1);
 #pragma unroll
     for (int pg = 0; pg < 4; ++pg) {
-      f32x4 dm = {0, 0, 0, 0}, dq = {0, 0, 0, 0}, dm2 = {0, 0, 0, 0}, dq2 = {0, 0, 0, 0};
+      f32x4 dm = cm, dq = cq;
 #pragma unroll
       for (int i = 0; i < WPL; ++i) {
 #pragma unroll
@@ -284,21 +290,19 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
           }
           const uint32_t b0 = x & nib, b1 = (x >> 1) & nib, b2 = (x >> 2) & nib, b3 = (x >> 3) & nib;
           if (tp == NTP - 1) {
-            dq = mfma_f8f4(qa[tp][i][0], b0, b1, b2, b3, dq, sa01, sb);
-            dq2 = mfma_f8f4(qa[tp][i][1], b0, b1, b2, b3, dq2, sa2, sb);
+            dq = mfma_f8f4<2>(qa[tp][i][0], b0, b1, b2, b3, dq, sa, sb);
+            dq = mfma_f8f4<3>(qa[tp][i][1], b0, b1, b2, b3, dq, sa, sb);
           } else {
-            dm = mfma_f8f4(qa[tp][i][0], b0, b1, b2, b3, dm, sa01, sb);
-            dm2 = mfma_f8f4(qa[tp][i][1], b0, b1, b2, b3, dm2, sa2, sb);
+            dm = mfma_f8f4<0>(qa[tp][i][0], b0, b1, b2, b3, dm, sa, sb);
+            dm = mfma_f8f4<1>(qa[tp][i][1], b0, b1, b2, b3, dm, sa, sb);
           }
         }
       }
       const float nk = K.meta[pg][0], rk = K.meta[pg][1];
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
-        const float vm = dm[2 * j] + dm[2 * j + 1] + dm2[j], vq = dq[2 * j] + dq[2 * j + 1] + dq2[j];
-        // this wavefront's share of the score (the whole score when DS == 1); the constant
-        // terms are added after the shares have met
-        s2[j][pg] = fmaf(nk * am[j], vm, (rk * aq[j]) * vq);
+        // this wavefront's share of the score (the whole score when DS == 1)
+        s2[j][pg] = fmaf(nk, dm[2 * j] + dm[2 * j + 1], rk * (dq[2 * j] + dq[2 * j + 1]));
       }
     }
     __builtin_amdgcn_s_setprio(0);
@@ -317,15 +321,12 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
 #pragma unroll
         for (int pg = 0; pg < 4; ++pg) s2[j][pg] += theirs[(j * 4 + pg) * 64 + lane];
     }
+    if (PARTIAL) {
 #pragma unroll
-    for (int pg = 0; pg < 4; ++pg) {
-      const float nk = K.meta[pg][0], rk = K.meta[pg][1];
+      for (int pg = 0; pg < 4; ++pg)
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        float s = s2[j][pg] + fmaf(nk, bm[j], rk * bq[j]);
-        if (PARTIAL && (blk * BLK_TOK + pg * 16 + n >= seq_len)) s = MF_NEG;
-        s2[j][pg] = s;
-      }
+        for (int j = 0; j < 2; ++j)
+          if (blk * BLK_TOK + pg * 16 + n >= seq_len) s2[j][pg] = MF_NEG;
     }
     // ---- online softmax (log2 domain); every lane of a 16-lane row ends with the same maximum
     float alpha[2];
@@ -363,10 +364,8 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
         f[2 * i] = __uint_as_float(V.scale[i] << 16);
         f[2 * i + 1] = __uint_as_float(V.scale[i] & 0xffff0000u);
       }
-      if (VB == 2) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) f[e] *= (e % 3 == 0 ? 1.0f : (e % 3 == 1 ? 0.25f : 0.0625f));
-      }
+      for (int e = 0; e < 8; ++e) f[e] *= (VB == 4 || e % 3 == 0 ? 0x1p100f : (e % 3 == 1 ? 0x1p98f : 0x1p96f));
       if (PARTIAL) {
         const int nv = seq_len - (blk * BLK_TOK + spage * 16 + 8 * (pc & 1));
 #pragma unroll
@@ -443,16 +442,15 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
           if (VB == 2) {
             // 16 two-bit fields; register r of MFMA u takes fields 4u+r (low half) and 4u+r+8 (high half)
             const uint32_t x = V.v[c], x6 = x >> 6, x12 = x >> 12;
-            if (u == 0) bc = u32x4{(x & m0) | base_pat, (x & m1) | base_pat, (x & m2) | base_pat, (x6 & m0) | base_pat};
-            else bc = u32x4{(x6 & m1) | base_pat, (x6 & m2) | base_pat, (x12 & m0) | base_pat, (x12 & m1) | base_pat};
+            if (u == 0) bc = u32x4{x & m0, x & m1, x & m2, x6 & m0};
+            else bc = u32x4{x6 & m1, x6 & m2, x12 & m0, x12 & m1};
           } else {
             // 8 four-bit fields; register r takes fields r (low half) and r+4 (high half)
             const uint32_t x = V.v[2 * c + u];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) bc[r] = ((x >> (4 * r)) & m0) | base_pat;
+            for (int r = 0; r < 4; ++r) bc[r] = (x >> (4 * r)) & m0;
           }
           acc[c] = mfma(aw[u], bc, acc[c]);
-          acc[c] = mfma(aw[u], neg_base, acc[c]);
         }
       }
     }
@@ -525,7 +523,7 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
       const int g = 4 * kb + i;
       if (g < G) {
         const float z = s_z[(wave * 16 + g) * 16 + hf * NG + c / CTG];
-        s_red[(wgrp * G + g) * (D + 2) + 2 + hf * DW + 16 * c + n] = acc[c][i] + z;
+        s_red[(wgrp * G + g) * (D + 2) + 2 + hf * DW + 16 * c + n] = fmaf(acc[c][i], 0x1p33f, z);
       }
     }
   }

@@ -74,15 +74,21 @@ rotate_query_kernel(const void* __restrict__ q, int dtype, int64_t rows, int R, 
 // are normalised by bounds that every workgroup can compute from the raw query:
 // |q_rot_j| <= ||q|| (Pi is orthogonal) and |q_sk_j| <= ||q|| max_j ||S_j||, and the sums
 // over all coordinates that the decode kernel needs are q . colsum(Pi), q . colsum(S).
-// q_stat per row: {||q||, ||q|| max_j ||S_j||, sum_j q_rot_j, sum_j q_sk_j}.
+//
+// Everything that multiplies a whole score is folded into the operands: with k = sm_scale log2(e)
+// the index planes carry  k coef q_rot_j  and the sign plane  2 k qjl_scale q_sk_j, each divided
+// by a power of two 2^E >= its bound (E per query head and kind), which the decode kernel gives
+// back through the MFMA's per-row block scale.  q_stat per row:
+// {E_index, E_sign (as floats), k c0 sum_j q_rot_j, -k qjl_scale sum_j q_sk_j}: the last two
+// are the constant parts of the score and start the MFMA accumulators.
 //
 // qa_pack receives the score-stage A operands of v_mfma_scale_f32_16x16x128_f8f6f4 (A fp8 e4m3,
 // B fp4) in register order: [kv head][term plane][128-coordinate chunk i][row set][lane][8 dwords].
 // A value v (the normalised query coordinate times the plane's coefficient, |v| <= 1) is the sum
 // of three fp8 terms with per-row scales 2^-6, 2^-10, 2^-14: t0 = fp8(64 v), t1 = fp8(16 (64 v - t0)),
 // t2 = fp8(16 (16 (64 v - t0) - t1)).  Row set 0 holds terms 0 and 1 (row 2g + t for head g), row
-// set 1 holds term 2 in rows 4(g/2) + g%2 (the other rows are zero), so that a lane of the MFMA
-// output sees the same two heads in both.  The hardware takes, for lane (row, block b), bytes
+// set 1 holds term 2 in row 2g (the odd rows are zero), so that both accumulate into the same
+// MFMA output registers.  The hardware takes, for lane (row, block b), bytes
 // 0..15 as contraction indices 16b..16b+15 and bytes 16..31 as 64+16b..64+16b+15, and the key
 // kernel puts coordinate c of plane word w at contraction index 32w + 8 (c % 4) + c / 4.
 constexpr int PREP_COLS = 32, PREP_SLICES = 16;
@@ -94,8 +100,9 @@ __device__ __forceinline__ float fp8_to_f32(uint32_t b) { return __builtin_amdgc
 
 template <int PER>      // matrix rows per thread = d / PREP_SLICES
 __global__ void __launch_bounds__(PREP_COLS * PREP_SLICES)
-prep_query_kernel(const void* __restrict__ q, int dtype, int G, tq_layer ly, float* __restrict__ q_rot,
-                  float* __restrict__ q_sk, float* __restrict__ q_stat, uint32_t* __restrict__ qa_pack) {
+prep_query_kernel(const void* __restrict__ q, int dtype, int G, tq_layer ly, float sm_scale,
+                  float* __restrict__ q_rot, float* __restrict__ q_sk, float* __restrict__ q_stat,
+                  uint32_t* __restrict__ qa_pack) {
   extern __shared__ float sm[];
   const int d = ly.d, tid = threadIdx.x, jl = tid % PREP_COLS, sl = tid / PREP_COLS;
   const int word = blockIdx.y, j = word * PREP_COLS + jl;
@@ -164,11 +171,16 @@ prep_query_kernel(const void* __restrict__ q, int dtype, int G, tq_layer ly, flo
       }
       ss = wave_sum(ss); s1 = wave_sum(s1); s2 = wave_sum(s2);
       if (lane == 0) {
-        const float nq = sqrtf(ss);
-        stat[r * 4 + 0] = nq; stat[r * 4 + 1] = nq * ly.S_rownorm_max; stat[r * 4 + 2] = s1; stat[r * 4 + 3] = s2;
+        const float nq = sqrtf(ss), k = sm_scale * 1.4426950408889634f;
+        int e1, e2;      // bound < 2^e (frexp's mantissa is below 1); a zero query gives e = 0
+        frexpf(fminf(fabsf(k) * nq * cmax, 1e30f), &e1);
+        frexpf(fminf(2.0f * fabsf(k * ly.qjl_scale) * nq * ly.S_rownorm_max, 1e30f), &e2);
+        e1 = max(e1, -100); e2 = max(e2, -100);
+        stat[r * 4 + 0] = k * ldexpf(1.0f, -e1);                       // multiplier of coef q_rot_j
+        stat[r * 4 + 1] = 2.0f * k * ly.qjl_scale * ldexpf(1.0f, -e2); // multiplier of q_sk_j
         if (word == 0) {
-          q_stat[(row0 + r) * 4 + 0] = nq; q_stat[(row0 + r) * 4 + 1] = nq * ly.S_rownorm_max;
-          q_stat[(row0 + r) * 4 + 2] = s1; q_stat[(row0 + r) * 4 + 3] = s2;
+          q_stat[(row0 + r) * 4 + 0] = (float)e1; q_stat[(row0 + r) * 4 + 1] = (float)e2;
+          q_stat[(row0 + r) * 4 + 2] = k * ly.term_const * s1; q_stat[(row0 + r) * 4 + 3] = -k * ly.qjl_scale * s2;
         }
       }
     }
@@ -215,14 +227,14 @@ prep_query_kernel(const void* __restrict__ q, int dtype, int G, tq_layer ly, flo
   for (int o = tid; o < ntp * 256; o += blockDim.x) {
     const int dw = o & 3, bsel = (o >> 2) & 1, n = (o >> 3) & 15, rs = (o >> 7) & 1, tp = o >> 8;
     int g, term;
-    if (rs == 0) { g = n >> 1; term = n & 1; }
-    else { g = 2 * (n >> 2) + (n & 3); term = (n & 3) < 2 ? 2 : -1; }
+    g = n >> 1;
+    if (rs == 0) term = n & 1;
+    else term = (n & 1) ? -1 : 2;
     uint32_t packed = 0;
     if (term >= 0 && g < G) {
       const bool is_sign = tp == ntp - 1;
       const float* src = (is_sign ? ssk : srot) + g * PREP_COLS;
-      const float mul = 64.0f * (is_sign ? 1.0f / fmaxf(stat[g * 4 + 1], 1e-30f)
-                                         : coefs[tp] / fmaxf(stat[g * 4 + 0] * cmax, 1e-30f));
+      const float mul = 64.0f * (is_sign ? stat[g * 4 + 1] : coefs[tp] * stat[g * 4 + 0]);
 #pragma unroll
       for (int by = 0; by < 4; ++by) {
         const int kloc = 16 * bsel + 4 * dw + by;            // contraction index within the word's 32
@@ -370,7 +382,7 @@ static int check_layer_rd(const tq_layer* ly, bool need_sketch) {
 
 namespace tq {
 int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* layer, float* q_rot, float* q_sk,
-                        float* q_stat, uint32_t* qa_pack, int G, hipStream_t st) {
+                        float* q_stat, uint32_t* qa_pack, int G, float sm_scale, hipStream_t st) {
   const int d = layer->d;
   if (qa_pack) {       // operands of the matrix-core decode kernel wanted
     if (!q_stat || !layer->Pi_colsum || !layer->S_colsum || G > ROT_MAX_ROWS || rows % G || (d != 128 && d != 256))
@@ -378,8 +390,8 @@ int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* 
     size_t smem = (size_t)(G * d + 2 * PREP_SLICES * G * PREP_COLS + 2 * G * PREP_COLS + 4 * ROT_MAX_ROWS + 32) *
                   sizeof(float);
     const dim3 grid((unsigned)(rows / G), d / PREP_COLS), block(PREP_COLS * PREP_SLICES);
-    if (d == 128) prep_query_kernel<8><<<grid, block, smem, st>>>(q, dtype, G, *layer, q_rot, q_sk, q_stat, qa_pack);
-    else prep_query_kernel<16><<<grid, block, smem, st>>>(q, dtype, G, *layer, q_rot, q_sk, q_stat, qa_pack);
+    if (d == 128) prep_query_kernel<8><<<grid, block, smem, st>>>(q, dtype, G, *layer, sm_scale, q_rot, q_sk, q_stat, qa_pack);
+    else prep_query_kernel<16><<<grid, block, smem, st>>>(q, dtype, G, *layer, sm_scale, q_rot, q_sk, q_stat, qa_pack);
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? TQ_OK : (int)e;
   }
@@ -401,7 +413,7 @@ extern "C" int tq_rotate_query(const void* q, int dtype, int64_t rows, const tq_
   if (!q || !q_rot || !q_sk) return TQ_ENULL;
   if (rows < 0 || dtype < TQ_F32 || dtype > TQ_BF16) return TQ_EINVAL;
   if (rows == 0) return TQ_OK;
-  return launch_rotate_query(q, dtype, rows, layer, q_rot, q_sk, nullptr, nullptr, 1, (hipStream_t)stream);
+  return launch_rotate_query(q, dtype, rows, layer, q_rot, q_sk, nullptr, nullptr, 1, 0.0f, (hipStream_t)stream);
 }
 
 extern "C" int tq_score(const void* q, int dtype, int64_t batch, int64_t n_q, const uint8_t* idx, const uint8_t* signs,
