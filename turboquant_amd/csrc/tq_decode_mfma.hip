@@ -7,10 +7,11 @@
 //    the individual index bits), so  sum_j q_rot[j] c[idx_j]  is a sum of
 //    "query . bit-plane" contractions, exactly like the QJL term
 //    sum_j q_sk[j] (2 bit_j - 1).  The contraction runs on
-//    v_mfma_scale_f32_16x16x128_f8f6f4 with the bits as the fp4 operand: the nibble
-//    0001 is the fp4 number 0.5, so  (x >> s) & 0x11111111  for s = 0..3 turns a
-//    32-bit plane word into the four operand dwords (7 vector-ALU instructions for
-//    32 coordinates).  The query is the fp8 operand, split into three fp8 terms
+//    v_mfma_scale_f32_16x16x128_f8f6f4 with the bits as the fp4 operand: the nibbles
+//    0001, 0010, 0100 are the fp4 numbers 0.5, 1, 2, so  x & 0x11111111,
+//    x & 0x22222222, x & 0x44444444 and (x >> 3) & 0x11111111 turn a 32-bit plane
+//    word into the four operand dwords (5 vector-ALU instructions for 32
+//    coordinates); the query operand carries the inverse factors.  The query is the fp8 operand, split into three fp8 terms
 //    with per-row power-of-two scales (12 significant bits), prepared once per step;
 //    every factor and constant of the score that belongs to a query head is folded
 //    into those operands, their block scales and the initial accumulator.
@@ -19,7 +20,11 @@
 //    s being the bit position the code has in its 16-bit half, and the bf16 MFMA
 //    (v_mfma_f32_16x16x32_bf16) keeps denormal inputs.  The softmax weight times the
 //    group scale times 2^(100-s) is the A operand; the accumulators carry 2^-33
-//    until the epilogue.  The zero points go through one more MFMA (weights x zeros).
+//    until the epilogue.  At most 8 query heads share a KV head, so operand rows
+//    0..7 carry the heads weighted with the scales of an even group and rows 8..15
+//    the same heads with the scales of the next group: one set of weight products
+//    serves the channel tiles of two groups.  The zero points go through one more
+//    MFMA (weights x zeros).
 //
 // head_dim 256 is split over a pair of wavefronts (DS = 2): each scores half of the
 // coordinates, the halves of the scores meet in LDS once per block, both wavefronts
@@ -113,6 +118,11 @@ template <int VB>
 __device__ __forceinline__ constexpr int v_token(int u, int r, int h) {
   return VB == 2 ? 4 * u + r + 8 * h : 8 * u + r + 4 * h;
 }
+// bit position (inside its byte) of the code of token t: the weight of the token carries 2^-pos
+template <int VB>
+__device__ __forceinline__ constexpr int v_bitpos(int t) {
+  return VB == 2 ? 2 * (t & 3) : 4 * (t & 1);
+}
 
 // D in {128, 256}; MB stored index bits; NX extra (multi-bit) Walsh terms; VB value bits;
 // GS value group size; DS wavefronts that share one block (each takes D/DS coordinates and
@@ -134,7 +144,7 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
   constexpr int PIECES = 2 * NG;              // 16-byte pieces of this wavefront's scales per page
   constexpr int NGRP = MF_WAVES / DS;         // wavefront groups (each walks its own blocks)
   constexpr int WAVE_LDS_FLOATS = wave_lds_floats(NG, DS);
-  static_assert(WPL >= 1 && NG >= 1, "a wavefront takes at least 128 coordinates");
+  static_assert(WPL >= 1 && NG >= 2 && NG % 2 == 0, "a wavefront takes at least 128 coordinates and whole group pairs");
   const int G = Hq / Hkv;                     // <= 8
   const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
   const int tid = threadIdx.x, lane = tid & 63;
@@ -175,7 +185,7 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
     sa = (e1 - t01) | ((e1 - 14) << 8) | ((e2 - t01) << 16) | ((e2 - 14) << 24);
   }
   const int sb = 127 + 1;
-  const uint32_t nib = in_vgpr(0x11111111u);
+  const uint32_t nib = in_vgpr(0x11111111u), nib1 = in_vgpr(0x22222222u), nib2 = in_vgpr(0x44444444u);
   // constant parts of the scores of the two heads this lane sees in the MFMA output (rows 4kb..4kb+3
   // = heads 2kb, 2kb+1), as the initial accumulators; only one wavefront of a pair adds them
   f32x4 cm = {0, 0, 0, 0}, cq = {0, 0, 0, 0};
@@ -258,11 +268,12 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
     R.scale = *(const u32x4*)(pool_h + spid * page_stride + off_scale);
   };
 
-  // A value code masked in place is a bf16 denormal: B = code * 2^(s - 133) exactly, where s is the
-  // bit position the code already has inside its 16-bit half (0, 2 or 4 for 2-bit codes, 0 for
-  // 4-bit codes), so that most codes need no shift; the softmax weight carries 2^(100 - s).
+  // A value code masked in place is a bf16 number: a pattern n < 256 in a 16-bit half is n * 2^-133
+  // exactly (denormals, and the first binade continues them linearly), so B = code * 2^(s - 133)
+  // where s is the bit position the code has inside its byte; the softmax weight carries 2^(100 - s).
+  // Only the codes in the upper byte of each half need a shift.
   const uint32_t m0 = in_vgpr(VB == 2 ? 0x00030003u : 0x000F000Fu);
-  const uint32_t m1 = in_vgpr(0x000C000Cu), m2 = in_vgpr(0x00300030u);
+  const uint32_t m1 = in_vgpr(VB == 2 ? 0x000C000Cu : 0x00F000F0u), m2 = in_vgpr(0x00300030u), m3 = in_vgpr(0x00C000C0u);
 
   // ---------------------------------------------------------------- one block of 64 tokens
   // scores of the 4 pages of block blk, online softmax, weights -> LDS
@@ -288,7 +299,7 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
 #pragma unroll
             for (int p = 0; p < MB; ++p) x ^= ((xplanes[tp - MB] >> p) & 1) ? K.key[pg][i * (MB + 1) + p] : 0u;
           }
-          const uint32_t b0 = x & nib, b1 = (x >> 1) & nib, b2 = (x >> 2) & nib, b3 = (x >> 3) & nib;
+          const uint32_t b0 = x & nib, b1 = x & nib1, b2 = x & nib2, b3 = (x >> 3) & nib;
           if (tp == NTP - 1) {
             dq = mfma_f8f4<2>(qa[tp][i][0], b0, b1, b2, b3, dq, sa, sb);
             dq = mfma_f8f4<3>(qa[tp][i][1], b0, b1, b2, b3, dq, sa, sb);
@@ -365,7 +376,10 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
         f[2 * i + 1] = __uint_as_float(V.scale[i] & 0xffff0000u);
       }
 #pragma unroll
-      for (int e = 0; e < 8; ++e) f[e] *= (VB == 4 || e % 3 == 0 ? 0x1p100f : (e % 3 == 1 ? 0x1p98f : 0x1p96f));
+      for (int e = 0; e < 8; ++e) {
+        constexpr float k_pow[4] = {0x1p100f, 0x1p98f, 0x1p96f, 0x1p94f};
+        f[e] *= k_pow[v_bitpos<VB>(e) / 2];
+      }
       if (PARTIAL) {
         const int nv = seq_len - (blk * BLK_TOK + spage * 16 + 8 * (pc & 1));
 #pragma unroll
@@ -379,15 +393,15 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     if (rescale) {
-      const f32x4 a4 = *(const f32x4*)(s_alpha + 4 * kb);      // accumulator rows 4kb..4kb+3
+      const f32x4 a4 = *(const f32x4*)(s_alpha + 4 * (kb & 1)); // accumulator rows 4kb..4kb+3 = heads 4(kb%2)..
 #pragma unroll
       for (int c = 0; c < CT; ++c) acc[c] *= a4;
       zacc *= a4;
     }
-    // ---- value stage: lane = (row g = n, page kb)
+    // ---- value stage: lane = (row n = head n % 8 with the scales of group parity n / 8, page kb)
     float pr[16];
     {
-      const f32x4* pp = (const f32x4*)(s_p + (kb * 16 + n) * P_STRIDE);
+      const f32x4* pp = (const f32x4*)(s_p + (kb * 16 + (n & 7)) * P_STRIDE);
 #pragma unroll
       for (int q4 = 0; q4 < 4; ++q4) {
         f32x4 t = pp[q4];
@@ -416,11 +430,11 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
     }
     __builtin_amdgcn_s_setprio(2);
 #pragma unroll
-    for (int grp = 0; grp < NG; ++grp) {
+    for (int gp = 0; gp < NG / 2; ++gp) {
       // w = weight * scale for the 16 tokens of page kb, then the two A operands in the value token order
       float w[16];
       {
-        const f32x4* sp = (const f32x4*)(s_scale + (kb * NG + grp) * 16);
+        const f32x4* sp = (const f32x4*)(s_scale + (kb * NG + 2 * gp + (n >> 3)) * 16);
 #pragma unroll
         for (int q4 = 0; q4 < 4; ++q4) {
           const f32x4 sv = sp[q4];
@@ -434,21 +448,19 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
 #pragma unroll
         for (int r = 0; r < 4; ++r) aw[u][r] = pack_bf16(w[v_token<VB>(u, r, 0)], w[v_token<VB>(u, r, 1)]);
 #pragma unroll
-      for (int cc = 0; cc < CTG; ++cc) {
-        const int c = grp * CTG + cc;
+      for (int cc = 0; cc < 2 * CTG; ++cc) {
+        const int c = gp * 2 * CTG + cc;
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
           u32x4 bc;
           if (VB == 2) {
             // 16 two-bit fields; register r of MFMA u takes fields 4u+r (low half) and 4u+r+8 (high half)
-            const uint32_t x = V.v[c], x6 = x >> 6, x12 = x >> 12;
-            if (u == 0) bc = u32x4{x & m0, x & m1, x & m2, x6 & m0};
-            else bc = u32x4{x6 & m1, x6 & m2, x12 & m0, x12 & m1};
+            const uint32_t x = u == 0 ? V.v[c] : V.v[c] >> 8;
+            bc = u32x4{x & m0, x & m1, x & m2, x & m3};
           } else {
             // 8 four-bit fields; register r takes fields r (low half) and r+4 (high half)
-            const uint32_t x = V.v[2 * c + u];
-#pragma unroll
-            for (int r = 0; r < 4; ++r) bc[r] = (x >> (4 * r)) & m0;
+            const uint32_t x = V.v[2 * c + u], x8 = x >> 8;
+            bc = u32x4{x & m0, x & m1, x8 & m0, x8 & m1};
           }
           acc[c] = mfma(aw[u], bc, acc[c]);
         }
@@ -516,12 +528,13 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  // accumulator rows 0..7 are valid for the channel tiles of even groups, rows 8..15 for odd groups
 #pragma unroll
   for (int c = 0; c < CT; ++c) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int g = 4 * kb + i;
-      if (g < G) {
+      const int g = 4 * (kb & 1) + i;
+      if (g < G && (kb >> 1) == ((c / CTG) & 1)) {
         const float z = s_z[(wave * 16 + g) * 16 + hf * NG + c / CTG];
         s_red[(wgrp * G + g) * (D + 2) + 2 + hf * DW + 16 * c + n] = fmaf(acc[c][i], 0x1p33f, z);
       }

@@ -239,7 +239,10 @@ prep_query_kernel(const void* __restrict__ q, int dtype, int G, tq_layer ly, flo
       for (int by = 0; by < 4; ++by) {
         const int kloc = 16 * bsel + 4 * dw + by;            // contraction index within the word's 32
         const int c = 4 * (kloc & 7) + (kloc >> 3);          // coordinate within the word
-        float v = src[c] * mul;
+        // the decode kernel extracts three of the four bits of a nibble in place, where they are
+        // the fp4 numbers 1, 2 and 4 (after its block scale): the query side divides them out
+        const int t4 = kloc >> 3;
+        float v = src[c] * mul * (t4 == 1 ? 0.5f : (t4 == 2 ? 0.25f : 1.0f));
         uint32_t code = f32_to_fp8(v);
         for (int t = 0; t < term; ++t) {
           v = (v - fp8_to_f32(code)) * 16.0f;
