@@ -316,6 +316,15 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
         s2[j][pg] = fmaf(nk, dm[2 * j] + dm[2 * j + 1], rk * (dq[2 * j] + dq[2 * j + 1]));
       }
     }
+    // Wanted issue order of the section above: the bit expansion of the first page, then every MFMA
+    // followed by a few vector instructions (the next page's expansion, the previous page's score
+    // arithmetic), which run in the shadow of the matrix pipe.
+    __builtin_amdgcn_sched_group_barrier(0x002, 5 * NTP * WPL, 0);
+#pragma unroll
+    for (int k = 0; k < 4 * 2 * NTP * WPL; ++k) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+    }
     __builtin_amdgcn_s_setprio(0);
     if (DS > 1) {
       // exchange with the wavefront that scored the other coordinates: own share -> LDS, workgroup
