@@ -537,33 +537,57 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-  // accumulator rows 0..7 are valid for the channel tiles of even groups, rows 8..15 for odd groups
+  // Accumulator rows 0..7 are valid for the channel tiles of even groups, rows 8..15 for odd groups:
+  // a lane owns heads 4(kb%2)..+3 and the groups of parity kb/2.  Everything is read before the
+  // first conditional store, so that no memory latency sits inside a branch.
+  {
+    const int par = kb >> 1;
+    float zz[NG / 2][4];
 #pragma unroll
-  for (int c = 0; c < CT; ++c) {
+    for (int gpi = 0; gpi < NG / 2; ++gpi)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) zz[gpi][i] = s_z[(wave * 16 + 4 * (kb & 1) + i) * 16 + hf * NG + 2 * gpi + par];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int g = 4 * (kb & 1) + i;
-      if (g < G && (kb >> 1) == ((c / CTG) & 1)) {
-        const float z = s_z[(wave * 16 + g) * 16 + hf * NG + c / CTG];
-        s_red[(wgrp * G + g) * (D + 2) + 2 + hf * DW + 16 * c + n] = fmaf(acc[c][i], 0x1p33f, z);
+      if (g < G) {
+        float* row = s_red + (wgrp * G + g) * (D + 2) + 2 + hf * DW + par * (16 * CTG) + n;
+#pragma unroll
+        for (int gpi = 0; gpi < NG / 2; ++gpi)
+#pragma unroll
+          for (int cc = 0; cc < CTG; ++cc) {
+            const float v = par ? acc[(2 * gpi + 1) * CTG + cc][i] : acc[2 * gpi * CTG + cc][i];
+            row[16 * (2 * gpi * CTG + cc)] = fmaf(v, 0x1p33f, zz[gpi][i]);
+          }
       }
     }
   }
   __syncthreads();
-  for (int o = tid; o < G * D; o += blockDim.x) {
-    const int g = o / D, ch = o - g * D;
-    float mm = MF_NEG;
-    for (int w = 0; w < NGRP; ++w) mm = fmaxf(mm, s_red[(w * G + g) * (D + 2)]);
-    float ll = 0.0f, aa = 0.0f;
+  // merge of the walkers: thread -> (head, channel); loads are unconditional (clamped), stores guarded
+#pragma unroll
+  for (int k = 0; k < 8 * D / (MF_WAVES * 64); ++k) {
+    const int o = tid + k * (MF_WAVES * 64);
+    const bool live = o < G * D;
+    const int g = live ? o / D : 0, ch = o % D;
+    float m_w[NGRP], l_w[NGRP], a_w[NGRP], mm = MF_NEG;
+#pragma unroll
     for (int w = 0; w < NGRP; ++w) {
       const float* r = s_red + (w * G + g) * (D + 2);
-      const float wgt = __expf(r[0] - mm);
-      ll += wgt * r[1];
-      aa += wgt * r[2 + ch];
+      m_w[w] = r[0]; l_w[w] = r[1]; a_w[w] = r[2 + ch];
+      mm = fmaxf(mm, m_w[w]);
     }
-    float* out = parts + (((int64_t)b * Hq + h * G + g) * n_parts + split) * (D + 2);
-    if (ch == 0) { out[0] = mm; out[1] = ll; }
-    out[2 + ch] = aa;
+    float ll = 0.0f, aa = 0.0f;
+#pragma unroll
+    for (int w = 0; w < NGRP; ++w) {
+      const float wgt = __expf(m_w[w] - mm);
+      ll = fmaf(wgt, l_w[w], ll);
+      aa = fmaf(wgt, a_w[w], aa);
+    }
+    if (live) {
+      float* out = parts + (((int64_t)b * Hq + h * G + g) * n_parts + split) * (D + 2);
+      if (ch == 0) { out[0] = mm; out[1] = ll; }
+      out[2 + ch] = aa;
+    }
   }
 }
 
