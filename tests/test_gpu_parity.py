@@ -312,7 +312,8 @@ def _store_from_oracle_view(pool, table_row, n_tok):
     return key_code(idx, sgn, rnorms, norms, pool.quantizer.bits - 1), value_code(vdata, vsc, vz, pool.value_bits)
 
 
-def _decode_case(gpu, d, key_bits, vb, B, Hq, Hkv, lens, recent, seed, n_split=None, dtype=torch.bfloat16):
+def _decode_case(gpu, d, key_bits, vb, B, Hq, Hkv, lens, recent, seed, n_split=None, dtype=torch.bfloat16,
+                 shape_kq=None):
     g = torch.Generator().manual_seed(seed)
     max_len = max(max(lens), 1)
     pages_per_seq = (max_len + 15) // 16
@@ -322,8 +323,11 @@ def _decode_case(gpu, d, key_bits, vb, B, Hq, Hkv, lens, recent, seed, n_split=N
     table = perm.reshape(B, pages_per_seq).to(gpu)
     k = torch.randn(B, max_len, Hkv, d, generator=g).to(dtype)
     v = torch.randn(B, max_len, Hkv, d, generator=g).to(dtype)
-    pool.append(k.to(gpu), v.to(gpu), table)
     q = torch.randn(B, Hq, d, generator=g).to(dtype)
+    if shape_kq is not None:
+        k, q = shape_kq(k.float(), q.float())
+        k, q = k.to(dtype), q.to(dtype)
+    pool.append(k.to(gpu), v.to(gpu), table)
     rk = rv = rl = None
     if recent:
         rk = torch.randn(B, max(recent), Hkv, d, generator=g).to(dtype)
@@ -362,6 +366,52 @@ def test_decode_attention_matches_oracle_on_the_same_store(gpu, d, key_bits, vb,
     _progress(f"decode d={d} kb={key_bits} vb={vb} Hq={Hq} Hkv={Hkv}")
     worst = _decode_case(gpu, d, key_bits, vb, 3, Hq, Hkv, [200, 37, 512], None, seed=d + vb)
     _progress(f"   worst cosine {worst:.7f}")
+
+
+@pytest.mark.parametrize("trend", ["rising", "falling", "all_low", "spiky"])
+def test_decode_softmax_over_wide_score_ranges(gpu, trend):
+    # logits that climb or fall by hundreds over the context, sit far below zero everywhere, or jump
+    # at a few tokens: the running reference of the softmax has to follow without overflow, underflow
+    # or loss of the small weights that matter
+    d, Hkv, Hq = 256, 2, 16
+
+    def shape_kq(k, q):
+        B, N, H, _ = k.shape
+        u = torch.nn.functional.normalize(torch.ones(d), dim=0)
+        ramp = torch.linspace(-1.0, 1.0, N)[None, :, None, None]
+        if trend == "rising":
+            k = k + 60.0 * ramp * u
+        elif trend == "falling":
+            k = k - 60.0 * ramp * u
+        elif trend == "all_low":
+            k = k - 80.0 * u
+        else:
+            spikes = torch.zeros(N)
+            spikes[[3, N // 3, N // 2 + 1, N - 2]] = torch.tensor([20.0, 45.0, 70.0, 95.0])
+            k = k + spikes[None, :, None, None] * u
+        q = q + 40.0 * u                       # sm_scale * q.k swings by about +-150 along the ramp
+        return k, q
+
+    worst = _decode_case(gpu, d, 3, 2, 2, Hq, Hkv, [1500, 333], None, seed=11, shape_kq=shape_kq)
+    _progress(f"softmax range {trend}: worst cosine {worst:.7f}")
+    worst = _decode_case(gpu, 128, 3, 4, 2, 8, 2, [700, 64], [5, 0], seed=12, n_split=3,
+                         shape_kq=lambda k, q: (shape_kq_128(k, trend), q + 30.0 * torch.nn.functional.normalize(torch.ones(128), dim=0)))
+    _progress(f"softmax range {trend} (d=128, tail): worst cosine {worst:.7f}")
+
+
+def shape_kq_128(k, trend):
+    N = k.shape[1]
+    u = torch.nn.functional.normalize(torch.ones(128), dim=0)
+    ramp = torch.linspace(-1.0, 1.0, N)[None, :, None, None]
+    if trend == "rising":
+        return k + 50.0 * ramp * u
+    if trend == "falling":
+        return k - 50.0 * ramp * u
+    if trend == "all_low":
+        return k - 70.0 * u
+    spikes = torch.zeros(N)
+    spikes[[1, N // 2, N - 1]] = torch.tensor([30.0, 60.0, 90.0])
+    return k + spikes[None, :, None, None] * u
 
 
 def test_decode_attention_ragged_empty_and_hybrid_tail(gpu):

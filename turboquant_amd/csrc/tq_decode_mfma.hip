@@ -19,7 +19,7 @@
 //    field zero, the code in the low mantissa bits): B = code * 2^(s-133) exactly,
 //    s being the bit position the code has in its 16-bit half, and the bf16 MFMA
 //    (v_mfma_f32_16x16x32_bf16) keeps denormal inputs.  The softmax weight times the
-//    group scale times 2^(100-s) is the A operand; the accumulators carry 2^-33
+//    group scale times 2^(80-s) is the A operand; the accumulators carry 2^-53
 //    until the epilogue.  At most 8 query heads share a KV head, so operand rows
 //    0..7 carry the heads weighted with the scales of an even group and rows 8..15
 //    the same heads with the scales of the next group: one set of weight products
@@ -221,14 +221,17 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
   const uint8_t* pool_h = pool + (int64_t)h * L.page_bytes;
   const int64_t page_stride = (int64_t)Hkv * L.page_bytes;
   // per lane the key words are [word i][plane], the value fields [channel tile]: a wavefront's share is contiguous
-  const int off_keys = L.off_keys + (lane * DS + hf) * (NKW * 4), off_meta = L.off_meta + n * 8;
-  const int off_v = L.off_vdata + (n * DS + hf) * (VW * 4);
-  const int off_scale = L.off_vscale + hf * (NG * 32) + (lane % PIECES) * 16;
+  const uint32_t off_keys = L.off_keys + (lane * DS + hf) * (NKW * 4), off_meta = L.off_meta + n * 8;
+  const uint32_t off_v = L.off_vdata + (n * DS + hf) * (VW * 4);
+  const uint32_t off_scale = L.off_vscale + hf * (NG * 32) + (lane % PIECES) * 16;
 
   f32x4 acc[CT];
 #pragma unroll
   for (int c = 0; c < CT; ++c) acc[c] = f32x4{0, 0, 0, 0};
   f32x4 zacc = {0, 0, 0, 0};
+  // m_run is the reference the weights are taken against (exp2(score - m_run)); it only moves when
+  // a score exceeds it by more than REF_SLACK, so the usual block needs no row reduction
+  constexpr float REF_SLACK = 16.0f;
   float m_run[2] = {MF_NEG, MF_NEG}, l_run[2] = {0.0f, 0.0f};
 
   struct KeyRegs { uint32_t key[4][NKW]; f32x2 meta[4]; };
@@ -253,10 +256,12 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
   // All loads below are unconditional (lanes without a group / piece of their own read a
   // neighbour's): a load inside a branch would make the wait counters at the join conservative
   // and serialise the prefetch.
-  const int off_zero_c = L.off_vzero + min(n, NGT - 1) * 32;
+  const uint32_t off_zero_c = L.off_vzero + min(n, NGT - 1) * 32;
   const int spg = min(lane / PIECES, 3);
   auto load_vals = [&](const int (&pid)[4], ValRegs& R) {
-    const int my_pid = kb == 0 ? pid[0] : (kb == 1 ? pid[1] : (kb == 2 ? pid[2] : pid[3]));
+    // per-lane page: selected as a number (three conditional moves), not as one of four pointers
+    int my_pid = kb == 0 ? pid[0] : (kb == 1 ? pid[1] : (kb == 2 ? pid[2] : pid[3]));
+    asm volatile("" : "+v"(my_pid));
     const uint8_t* vbase = pool_h + my_pid * page_stride;
     const uint32_t* vp = (const uint32_t*)(vbase + off_v);
 #pragma unroll
@@ -264,13 +269,14 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
     const u32x4* zp = (const u32x4*)(vbase + off_zero_c);
     R.zero[0] = zp[0];
     R.zero[1] = zp[1];
-    const int spid = spg == 0 ? pid[0] : (spg == 1 ? pid[1] : (spg == 2 ? pid[2] : pid[3]));
+    int spid = spg == 0 ? pid[0] : (spg == 1 ? pid[1] : (spg == 2 ? pid[2] : pid[3]));
+    asm volatile("" : "+v"(spid));
     R.scale = *(const u32x4*)(pool_h + spid * page_stride + off_scale);
   };
 
   // A value code masked in place is a bf16 number: a pattern n < 256 in a 16-bit half is n * 2^-133
   // exactly (denormals, and the first binade continues them linearly), so B = code * 2^(s - 133)
-  // where s is the bit position the code has inside its byte; the softmax weight carries 2^(100 - s).
+  // where s is the bit position the code has inside its byte; the softmax weight carries 2^(80 - s).
   // Only the codes in the upper byte of each half need a shift.
   const uint32_t m0 = in_vgpr(VB == 2 ? 0x00030003u : 0x000F000Fu);
   const uint32_t m1 = in_vgpr(VB == 2 ? 0x000C000Cu : 0x00F000F0u), m2 = in_vgpr(0x00300030u), m3 = in_vgpr(0x00C000C0u);
@@ -280,6 +286,10 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
   auto score_stage = [&](int blk, int it, const KeyRegs& K, auto partial_tag) -> bool {
     constexpr bool PARTIAL = decltype(partial_tag)::value;
     float s2[2][4];
+    const bool first = it == 0;                 // first block of this walker: no reference yet
+    float mref[2];                              // only one wavefront of a pair subtracts it
+#pragma unroll
+    for (int j = 0; j < 2; ++j) mref[j] = (first || hf != 0) ? 0.0f : m_run[j];
     // The MFMA-dense parts run at raised wavefront priority (the value stage above the score
     // stage): the SIMD's other wavefront then fills the gaps with its vector-ALU work instead of
     // both alternating between the two kinds of instruction.
@@ -312,8 +322,8 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
       const float nk = K.meta[pg][0], rk = K.meta[pg][1];
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
-        // this wavefront's share of the score (the whole score when DS == 1)
-        s2[j][pg] = fmaf(nk, dm[2 * j] + dm[2 * j + 1], rk * (dq[2 * j] + dq[2 * j + 1]));
+        // this wavefront's share of the score (the whole score when DS == 1), relative to the reference
+        s2[j][pg] = fmaf(nk, dm[2 * j] + dm[2 * j + 1], fmaf(rk, dq[2 * j] + dq[2 * j + 1], -mref[j]));
       }
     }
     // Wanted issue order of the section above: the bit expansion of the first page, then every MFMA
@@ -348,26 +358,38 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
         for (int j = 0; j < 2; ++j)
           if (blk * BLK_TOK + pg * 16 + n >= seq_len) s2[j][pg] = MF_NEG;
     }
-    // ---- online softmax (log2 domain); every lane of a 16-lane row ends with the same maximum
-    float alpha[2];
+    // ---- online softmax (log2 domain) against a lazily updated reference
+    float mx = fmaxf(fmaxf(fmaxf(s2[0][0], s2[0][1]), fmaxf(s2[0][2], s2[0][3])),
+                     fmaxf(fmaxf(s2[1][0], s2[1][1]), fmaxf(s2[1][2], s2[1][3])));
+    const bool rescale = first || __builtin_amdgcn_ballot_w64(mx > REF_SLACK) != 0;
+    if (rescale) {
+      // move the reference to the row maximum (never down, except for the first block, where the
+      // accumulators are still empty and keep their scale); every lane of a row computes the same
+      float alpha[2];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        float mj = fmaxf(fmaxf(s2[j][0], s2[j][1]), fmaxf(s2[j][2], s2[j][3]));
+        mj = row_max16(mj);
+        const float delta = first ? mj : fmaxf(mj, 0.0f);
+        alpha[j] = first ? 1.0f : __builtin_amdgcn_exp2f(-delta);
+        m_run[j] = first ? delta : m_run[j] + delta;
+        l_run[j] *= alpha[j];
+#pragma unroll
+        for (int pg = 0; pg < 4; ++pg) s2[j][pg] -= delta;
+      }
+      if (n == 0) { s_alpha[2 * kb] = alpha[0]; s_alpha[2 * kb + 1] = alpha[1]; }
+    }
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      float mx = fmaxf(fmaxf(s2[j][0], s2[j][1]), fmaxf(s2[j][2], s2[j][3]));
-      mx = row_max16(mx);
-      const float m_new = fmaxf(m_run[j], mx);
-      alpha[j] = __builtin_amdgcn_exp2f(m_run[j] - m_new);
-      m_run[j] = m_new;
       float psum = 0.0f;
 #pragma unroll
       for (int pg = 0; pg < 4; ++pg) {
-        const float p = __builtin_amdgcn_exp2f(s2[j][pg] - m_new);
+        const float p = __builtin_amdgcn_exp2f(s2[j][pg]);
         psum += p;
         s_p[(pg * 16 + 2 * kb + j) * P_STRIDE + n] = p;
       }
-      l_run[j] = fmaf(l_run[j], alpha[j], psum);
+      l_run[j] += psum;
     }
-    const bool rescale = __builtin_amdgcn_ballot_w64(alpha[0] != 1.0f || alpha[1] != 1.0f) != 0;
-    if (rescale && n == 0) { s_alpha[2 * kb] = alpha[0]; s_alpha[2 * kb + 1] = alpha[1]; }
     return rescale;
   };
   // weights x (codes, scales, zeros) of block blk into the accumulators
@@ -386,7 +408,7 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
       }
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        constexpr float k_pow[4] = {0x1p100f, 0x1p98f, 0x1p96f, 0x1p94f};
+        constexpr float k_pow[4] = {0x1p80f, 0x1p78f, 0x1p76f, 0x1p74f};
         f[e] *= k_pow[v_bitpos<VB>(e) / 2];
       }
       if (PARTIAL) {
@@ -557,7 +579,7 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
 #pragma unroll
           for (int cc = 0; cc < CTG; ++cc) {
             const float v = par ? acc[(2 * gpi + 1) * CTG + cc][i] : acc[2 * gpi * CTG + cc][i];
-            row[16 * (2 * gpi * CTG + cc)] = fmaf(v, 0x1p33f, zz[gpi][i]);
+            row[16 * (2 * gpi * CTG + cc)] = fmaf(v, 0x1p53f, zz[gpi][i]);
           }
       }
     }
