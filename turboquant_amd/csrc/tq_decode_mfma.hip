@@ -11,8 +11,9 @@
 //    0001, 0010, 0100 are the fp4 numbers 0.5, 1, 2, so  x & 0x11111111,
 //    x & 0x22222222, x & 0x44444444 and (x >> 3) & 0x11111111 turn a 32-bit plane
 //    word into the four operand dwords (5 vector-ALU instructions for 32
-//    coordinates); the query operand carries the inverse factors.  The query is the fp8 operand, split into three fp8 terms
-//    with per-row power-of-two scales (12 significant bits), prepared once per step;
+//    coordinates); the query operand carries the inverse factors.  The query is the fp6 (e2m3) operand - the MFMA runs
+//    at twice the fp8 rate with it -, split into three fp6 terms with per-row
+//    power-of-two scales (good to 2^-15 of the row maximum), prepared once per step;
 //    every factor and constant of the score that belongs to a query head is folded
 //    into those operands, their block scales and the initial accumulator.
 //  * values.  A code masked out of its packed word IS a bf16 denormal (exponent
@@ -103,14 +104,14 @@ __device__ __forceinline__ float row_sum16(float v) {
   return v;
 }
 
-// fp8 (A: 16 rows x 128) x fp4 (B: 128 x 16) MFMA with per-lane power-of-two scales (E8M0 codes).
-// Only the first four dwords of the fp4 operand are read.
+// fp6 (A: 16 rows x 128) x fp4 (B: 128 x 16) MFMA with per-lane power-of-two scales (E8M0 codes).
+// Only the first six dwords of the fp6 operand and the first four of the fp4 operand are read.
 // SEL picks the byte of scale_a that holds the code.
 template <int SEL>
 __device__ __forceinline__ f32x4 mfma_f8f4(const i32x8& a, uint32_t b0, uint32_t b1, uint32_t b2, uint32_t b3,
                                            f32x4 c, int scale_a, int scale_b) {
   const i32x8 bv = {(int)b0, (int)b1, (int)b2, (int)b3, 0, 0, 0, 0};
-  return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, bv, c, 0 /*A: fp8 e4m3*/, 4 /*B: fp4*/, SEL, scale_a, 0, scale_b);
+  return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, bv, c, 2 /*A: fp6 e2m3*/, 4 /*B: fp4*/, SEL, scale_a, 0, scale_b);
 }
 
 // token held by element (r, h) of MFMA half u of the value stage
@@ -161,28 +162,34 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
   float* s_red = (float*)smem_raw;                          // after the loop: [NGRP][G][D + 2]
 
   // ---------------------------------------------------------------- A operands of the score stage
-  // fp8 query terms in register order (see the preparation kernel): row set 0 = terms 0, 1 of the 8
-  // heads (row 2g + t), row set 1 = term 2 in row 2g; rows of absent heads are zero
+  // fp6 query terms in register order (see the preparation kernel): row set 0 = terms 0, 1 of the 8
+  // heads (row 2g + t), row set 1 = term 2 in row 2g; rows of absent heads are zero.  Six dwords per
+  // lane are stored at a stride of eight.
   i32x8 qa[NTP][WPL][2];
   {
-    const i32x8* src = (const i32x8*)qa_pack + ((int64_t)b * Hkv + h) * (NTP * WPLT * 2 * 64) + lane;
+    const uint32_t* src = qa_pack + (((int64_t)b * Hkv + h) * (NTP * WPLT * 2 * 64) + lane) * 8;
 #pragma unroll
     for (int tp = 0; tp < NTP; ++tp)
 #pragma unroll
       for (int i = 0; i < WPL; ++i)
 #pragma unroll
-        for (int rs = 0; rs < 2; ++rs) qa[tp][i][rs] = src[((tp * WPLT + hf * WPL + i) * 2 + rs) * 64];
+        for (int rs = 0; rs < 2; ++rs) {
+          const uint32_t* p6 = src + ((tp * WPLT + hf * WPL + i) * 2 + rs) * (64 * 8);
+          const u32x4 lo = *(const u32x4*)p6;
+          const uint32_t d4 = p6[4], d5 = p6[5];
+          qa[tp][i][rs] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)d4, (int)d5, 0, 0};
+        }
   }
   // E8M0 block-scale codes of this lane's operand row (head n / 2), one per byte: index planes row
-  // set 0, row set 1, sign plane row set 0, row set 1.  64 v / 2^E is stored, so term t carries
-  // 2^(E - 6 - 4t); the fp4 bit value 0.5 carries 2^1.
+  // set 0, row set 1, sign plane row set 0, row set 1.  4 v / 2^E is stored, so term t carries
+  // 2^(E - 2 - 5t); the fp4 bit value 0.5 carries 2^1.
   int sa;
   {
     const int g = n >> 1;
     const int64_t qrow = (int64_t)b * Hq + h * G + (g < G ? g : 0);
     const int e1 = 127 + (int)q_stat[qrow * 4 + 0], e2 = 127 + (int)q_stat[qrow * 4 + 1];
-    const int t01 = (n & 1) ? 10 : 6;
-    sa = (e1 - t01) | ((e1 - 14) << 8) | ((e2 - t01) << 16) | ((e2 - 14) << 24);
+    const int t01 = (n & 1) ? 7 : 2;
+    sa = (e1 - t01) | ((e1 - 12) << 8) | ((e2 - t01) << 16) | ((e2 - 12) << 24);
   }
   const int sb = 127 + 1;
   const uint32_t nib = in_vgpr(0x11111111u), nib1 = in_vgpr(0x22222222u), nib2 = in_vgpr(0x44444444u);

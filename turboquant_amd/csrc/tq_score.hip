@@ -82,21 +82,30 @@ rotate_query_kernel(const void* __restrict__ q, int dtype, int64_t rows, int R, 
 // {E_index, E_sign (as floats), k c0 sum_j q_rot_j, -k qjl_scale sum_j q_sk_j}: the last two
 // are the constant parts of the score and start the MFMA accumulators.
 //
-// qa_pack receives the score-stage A operands of v_mfma_scale_f32_16x16x128_f8f6f4 (A fp8 e4m3,
-// B fp4) in register order: [kv head][term plane][128-coordinate chunk i][row set][lane][8 dwords].
-// A value v (the normalised query coordinate times the plane's coefficient, |v| <= 1) is the sum
-// of three fp8 terms with per-row scales 2^-6, 2^-10, 2^-14: t0 = fp8(64 v), t1 = fp8(16 (64 v - t0)),
-// t2 = fp8(16 (16 (64 v - t0) - t1)).  Row set 0 holds terms 0 and 1 (row 2g + t for head g), row
-// set 1 holds term 2 in row 2g (the odd rows are zero), so that both accumulate into the same
-// MFMA output registers.  The hardware takes, for lane (row, block b), bytes
-// 0..15 as contraction indices 16b..16b+15 and bytes 16..31 as 64+16b..64+16b+15, and the key
-// kernel puts coordinate c of plane word w at contraction index 32w + 8 (c % 4) + c / 4.
+// qa_pack receives the score-stage A operands of v_mfma_scale_f32_16x16x128_f8f6f4 (A fp6 e2m3, which
+// runs at twice the fp8 rate; B fp4) in register order: [kv head][term plane][128-coordinate chunk i]
+// [row set][lane][8 dwords, 6 used].  A value v (the normalised query coordinate times the plane's
+// coefficient, |v| <= 1) is the sum of three fp6 terms with per-row block scales 2^-2, 2^-7, 2^-12:
+// t0 = fp6(4 v), t1 = fp6(32 (4 v - t0)), t2 = fp6(32 (32 (4 v - t0) - t1)); a term's rounding error
+// is at most 1/8, so every product stays within the fp6 range and the sum is good to 2^-15.  Row set 0
+// holds terms 0 and 1 (row 2g + t for head g), row set 1 holds term 2 in row 2g (the odd rows are
+// zero), so that both accumulate into the same MFMA output registers.  For 6-bit operands lane
+// (row, block b) holds contraction indices 32b..32b+31, index j at bits 6j..6j+5 of its 192 bits, and
+// the key kernel puts coordinate c of plane word w at contraction index 32w + 8 (c % 4) + c / 4.
 constexpr int PREP_COLS = 32, PREP_SLICES = 16;
 
-__device__ __forceinline__ uint32_t f32_to_fp8(float v) {
-  return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(v, 0.0f, 0, false) & 0xffu;
+// round to the fp6 e2m3 grid (1 sign, 2 exponent, 3 mantissa bits; steps 1/8 below 2, 1/4 below 4,
+// 1/2 up to the maximum 7.5), nearest even; returns the rounded value and its 6-bit code
+__device__ __forceinline__ float round_fp6(float v, uint32_t& code) {
+  const float a = fminf(fabsf(v), 7.5f);
+  const float inv_step = a < 2.0f ? 8.0f : (a < 4.0f ? 4.0f : 2.0f);
+  const float r = rintf(a * inv_step) / inv_step;    // exact (powers of two); may land on the next binade
+  const int e = r < 1.0f ? 0 : (r < 2.0f ? 1 : (r < 4.0f ? 2 : 3));
+  const float inv_unit = e <= 1 ? 8.0f : (e == 2 ? 4.0f : 2.0f);
+  const int m = (int)(r * inv_unit) - (e == 0 ? 0 : 8);
+  code = (v < 0.0f && r != 0.0f ? 32u : 0u) | ((uint32_t)e << 3) | (uint32_t)m;
+  return v < 0.0f ? -r : r;
 }
-__device__ __forceinline__ float fp8_to_f32(uint32_t b) { return __builtin_amdgcn_cvt_f32_fp8((int)b, 0); }
 
 template <int PER>      // matrix rows per thread = d / PREP_SLICES
 __global__ void __launch_bounds__(PREP_COLS * PREP_SLICES)
@@ -221,38 +230,46 @@ prep_query_kernel(const void* __restrict__ q, int dtype, int G, tq_layer ly, flo
     q_sk[(row0 + r) * d + word * PREP_COLS + c] = rb;
   }
   __syncthreads();
-  // operands of this plane word: per (term plane, row set, row) two lanes x four dwords
+  // operands of this plane word.  First the three 6-bit codes of every (term plane, head, contraction
+  // index) into shared memory (the partial sums are no longer needed), then per (term plane, row set,
+  // row) one lane x six dwords, each gathered from the (up to seven) codes that overlap it.
+  uint32_t* codes = (uint32_t*)pa;                           // [ntp][G][3 terms][32]
+  for (int o = tid; o < ntp * G * PREP_COLS; o += blockDim.x) {
+    const int kloc = o % PREP_COLS, g = (o / PREP_COLS) % G, tp = o / (PREP_COLS * G);
+    const bool is_sign = tp == ntp - 1;
+    const int c = 4 * (kloc & 7) + (kloc >> 3);              // coordinate within the word
+    // the decode kernel extracts three of the four bits of a nibble in place, where they are the fp4
+    // numbers 1, 2 and 4 (after its block scale): the query side divides them out
+    const int t4 = kloc >> 3;
+    const float mul = 4.0f * (is_sign ? stat[g * 4 + 1] : coefs[tp] * stat[g * 4 + 0]) *
+                      (t4 == 1 ? 0.5f : (t4 == 2 ? 0.25f : 1.0f));
+    float v = (is_sign ? ssk : srot)[g * PREP_COLS + c] * mul;
+#pragma unroll
+    for (int t = 0; t < 3; ++t) {
+      uint32_t code;
+      const float r = round_fp6(v, code);
+      codes[((tp * G + g) * 3 + t) * PREP_COLS + kloc] = code;
+      v = (v - r) * 32.0f;
+    }
+  }
+  __syncthreads();
   const int i = word >> 2, kw = word & 3;
   uint32_t* dst = qa_pack + group * (int64_t)(ntp * wpl * 2 * 64 * 8);
   for (int o = tid; o < ntp * 256; o += blockDim.x) {
-    const int dw = o & 3, bsel = (o >> 2) & 1, n = (o >> 3) & 15, rs = (o >> 7) & 1, tp = o >> 8;
-    int g, term;
-    g = n >> 1;
-    if (rs == 0) term = n & 1;
-    else term = (n & 1) ? -1 : 2;
+    const int dwi = o & 7, n = (o >> 3) & 15, rs = (o >> 7) & 1, tp = o >> 8;
+    if (dwi >= 6) continue;
+    const int g = n >> 1;
+    const int term = rs == 0 ? (n & 1) : ((n & 1) ? -1 : 2);
     uint32_t packed = 0;
     if (term >= 0 && g < G) {
-      const bool is_sign = tp == ntp - 1;
-      const float* src = (is_sign ? ssk : srot) + g * PREP_COLS;
-      const float mul = 64.0f * (is_sign ? stat[g * 4 + 1] : coefs[tp] * stat[g * 4 + 0]);
-#pragma unroll
-      for (int by = 0; by < 4; ++by) {
-        const int kloc = 16 * bsel + 4 * dw + by;            // contraction index within the word's 32
-        const int c = 4 * (kloc & 7) + (kloc >> 3);          // coordinate within the word
-        // the decode kernel extracts three of the four bits of a nibble in place, where they are
-        // the fp4 numbers 1, 2 and 4 (after its block scale): the query side divides them out
-        const int t4 = kloc >> 3;
-        float v = src[c] * mul * (t4 == 1 ? 0.5f : (t4 == 2 ? 0.25f : 1.0f));
-        uint32_t code = f32_to_fp8(v);
-        for (int t = 0; t < term; ++t) {
-          v = (v - fp8_to_f32(code)) * 16.0f;
-          code = f32_to_fp8(v);
-        }
-        packed |= code << (8 * by);
+      const uint32_t* cd = codes + ((tp * G + g) * 3 + term) * PREP_COLS;
+      const int j0 = (32 * dwi) / 6, j1 = min((32 * dwi + 31) / 6, 31);
+      for (int kloc = j0; kloc <= j1; ++kloc) {
+        const int bit = 6 * kloc - 32 * dwi;                 // position of the code in this dword (may straddle)
+        packed |= bit >= 0 ? cd[kloc] << bit : cd[kloc] >> -bit;
       }
     }
-    const int lane = n + 16 * (2 * (kw & 1) + bsel), dword = 4 * (kw >> 1) + dw;
-    dst[(((tp * wpl + i) * 2 + rs) * 64 + lane) * 8 + dword] = packed;
+    dst[(((tp * wpl + i) * 2 + rs) * 64 + n + 16 * kw) * 8 + dwi] = packed;
   }
 }
 
