@@ -525,24 +525,32 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
       load_keys(pid, K);
       load_vals(pid, V);
     }
-    for (int it = 0; it < trips; ++it) {
-      if (blk >= blk_end) {                              // uniform per wavefront pair
-        if (DS > 1) __syncthreads();
-        continue;
-      }
-      const int nxt = blk + NGRP;
-      const bool last = (blk + 1) * BLK_TOK > seq_len;
+    // one trip of a walker that still has a block; PARTIAL: the block may reach past the sequence end
+    auto trip = [&](int it, auto partial_tag) {
       // the block after this walker's last one does not exist: re-request the current one instead,
       // so that the loads stay outside any branch
+      const int nxt = blk + NGRP;
       const int nxt_c = nxt < blk_end ? nxt : blk;
       int pid_n[4];
       page_ids(nxt_c, pid_n);                            // scalar loads, consumed after the score stage
-      const bool rescale = last ? score_stage(blk, it, K, std::true_type{}) : score_stage(blk, it, K, std::false_type{});
+      const bool rescale = score_stage(blk, it, K, partial_tag);
       load_keys(pid_n, K);
-      if (last) value_stage(blk, V, rescale, std::true_type{});
-      else value_stage(blk, V, rescale, std::false_type{});
+      value_stage(blk, V, rescale, partial_tag);
       load_vals(pid_n, V);
       blk = nxt;
+    };
+    // A walker takes every NGRP-th block of the workgroup's range, so it can only run out of blocks,
+    // and only meet the ragged end of the sequence, in the last trip: the loop before it is
+    // straight-line code.
+    for (int it = 0; it < trips - 1; ++it) trip(it, std::false_type{});
+    if (trips > 0) {
+      if (blk >= blk_end) {                              // uniform per wavefront pair
+        if (DS > 1) __syncthreads();
+      } else if ((blk + 1) * BLK_TOK > seq_len) {
+        trip(trips - 1, std::true_type{});
+      } else {
+        trip(trips - 1, std::false_type{});
+      }
     }
   }
 
