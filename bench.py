@@ -122,26 +122,27 @@ def time_steps(fn, steps, warmup):
 
 
 def time_kernel_stage(work, steps, warmup):
-    """Mean duration of the page-streaming kernel alone: events bracket each
-    stage-2 launch separately, the other stages run untimed in between."""
+    """Mean execution time of the page-streaming kernel alone, inside whole steps: every timed step
+    runs all three stages as usual, and the library attaches a HIP event pair to the dispatch of the
+    page kernel itself (tq_time_next_page_kernel), so that the elapsed time is the kernel's own
+    begin-to-end time - the quantity a profiler's kernel trace reports - without the dispatch gaps
+    that markers between launches would add."""
     import torch
+    from turboquant_amd import _ffi
+    lib = _ffi.lib()
     for i in range(warmup):
         work.step(i)
-    torch.cuda.synchronize()
-    total = 0.0
     evs = []
-    for i in range(steps):
-        work.step(warmup + i, stages=1)
+    for _ in range(steps):
         a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        a.record()
-        work.step(warmup + i, stages=2)
-        b.record()
-        work.step(warmup + i, stages=4)
+        a.record(); b.record()                      # creates the underlying events
         evs.append((a, b))
     torch.cuda.synchronize()
-    for a, b in evs:
-        total += a.elapsed_time(b)
-    return total / steps
+    for i, (a, b) in enumerate(evs):
+        lib.tq_time_next_page_kernel(a.cuda_event, b.cuda_event)
+        work.step(warmup + i)
+    torch.cuda.synchronize()
+    return sum(a.elapsed_time(b) for a, b in evs) / steps
 
 
 def cpu_decode_baseline(work):

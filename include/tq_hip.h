@@ -214,6 +214,14 @@ int tq_decode_attn_paged_stages(const void *q, int dtype, int B, int Hq, int Hkv
  * would use.                                                                      */
 int tq_decode_merge(const float *parts, int64_t rows, int n_parts, int d, int dtype, void *out, void *stream);
 
+/* Measurement aid (no counterpart in the reference).  Arms the calling thread: the next
+ * page-streaming kernel that tq_decode_attn_paged[_stages] launches from this thread (its matrix-core
+ * kernel) is launched with `start_event` / `stop_event` (hipEvent_t, created with timing enabled)
+ * attached to its own dispatch, so that hipEventElapsedTime(start, stop) is that kernel's execution
+ * time alone - what a profiler's kernel trace reports - and not the interval between two markers in the
+ * stream, which also contains the dispatch gap.  Pass NULLs to disarm.                             */
+void tq_time_next_page_kernel(void *start_event, void *stop_event);
+
 #ifdef __cplusplus
 }
 #endif

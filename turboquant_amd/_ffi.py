@@ -70,6 +70,7 @@ _SIGNATURES = {
                                               C.POINTER(TqPageLayout), _vp, _vp, _i, _i64, _i64, _i64, _vp, _vp, _vp, _i,
                                               _i, _vp]),
     "tq_decode_merge": (C.c_int, [_vp, _i64, _i, _i, _i, _vp, _vp]),
+    "tq_time_next_page_kernel": (None, [_vp, _vp]),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)

@@ -12,8 +12,8 @@
 //    x & 0x22222222, x & 0x44444444 and (x >> 3) & 0x11111111 turn a 32-bit plane
 //    word into the four operand dwords (5 vector-ALU instructions for 32
 //    coordinates); the query operand carries the inverse factors.  The query is the fp6 (e2m3) operand - the MFMA runs
-//    at twice the fp8 rate with it -, split into three fp6 terms with per-row
-//    power-of-two scales (good to 2^-15 of the row maximum), prepared once per step;
+//    at twice the fp8 rate with it -, split into four fp6 terms with per-row
+//    power-of-two scales (good to 2^-20 of the row bound), prepared once per step;
 //    every factor and constant of the score that belongs to a query head is folded
 //    into those operands, their block scales and the initial accumulator.
 //  * values.  A code masked out of its packed word IS a bf16 denormal (exponent
@@ -41,6 +41,8 @@
 // by another.
 
 #include <type_traits>
+
+#include <hip/hip_ext.h>
 
 #include "tq_common.h"
 
@@ -163,7 +165,7 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
 
   // ---------------------------------------------------------------- A operands of the score stage
   // fp6 query terms in register order (see the preparation kernel): row set 0 = terms 0, 1 of the 8
-  // heads (row 2g + t), row set 1 = term 2 in row 2g; rows of absent heads are zero.  Six dwords per
+  // heads (row 2g + t), row set 1 = terms 2, 3; rows of absent heads are zero.  Six dwords per
   // lane are stored at a stride of eight.
   i32x8 qa[NTP][WPL][2];
   {
@@ -188,8 +190,8 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
     const int g = n >> 1;
     const int64_t qrow = (int64_t)b * Hq + h * G + (g < G ? g : 0);
     const int e1 = 127 + (int)q_stat[qrow * 4 + 0], e2 = 127 + (int)q_stat[qrow * 4 + 1];
-    const int t01 = (n & 1) ? 7 : 2;
-    sa = (e1 - t01) | ((e1 - 12) << 8) | ((e2 - t01) << 16) | ((e2 - 12) << 24);
+    const int t01 = (n & 1) ? 7 : 2, t23 = t01 + 10;
+    sa = (e1 - t01) | ((e1 - t23) << 8) | ((e2 - t01) << 16) | ((e2 - t23) << 24);
   }
   const int sb = 127 + 1;
   const uint32_t nib = in_vgpr(0x11111111u), nib1 = in_vgpr(0x22222222u), nib2 = in_vgpr(0x44444444u);
@@ -237,8 +239,10 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
   for (int c = 0; c < CT; ++c) acc[c] = f32x4{0, 0, 0, 0};
   f32x4 zacc = {0, 0, 0, 0};
   // m_run is the reference the weights are taken against (exp2(score - m_run)); it only moves when
-  // a score exceeds it by more than REF_SLACK, so the usual block needs no row reduction
-  constexpr float REF_SLACK = 16.0f;
+  // a score exceeds it by more than REF_SLACK, so the usual block needs no row reduction.  The slack
+  // is small on purpose: a token that dominates its row should sit at (or near) the reference, where
+  // its weight 1.0 survives the bf16 rounding of the value-stage operands exactly.
+  constexpr float REF_SLACK = 4.0f;
   float m_run[2] = {MF_NEG, MF_NEG}, l_run[2] = {0.0f, 0.0f};
 
   struct KeyRegs { uint32_t key[4][NKW]; f32x2 meta[4]; };
@@ -628,6 +632,9 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
   }
 }
 
+// events the next launch of this thread attaches to its dispatch (see tq_time_next_page_kernel)
+static thread_local hipEvent_t t_start_event = nullptr, t_stop_event = nullptr;
+
 template <int D, int MB, int NX, int VB, int GS, int DS, int WPS>
 static int launch_one(const uint32_t* qa_pack, const float* q_stat, int B, int Hq, int Hkv,
                       const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
@@ -642,9 +649,16 @@ static int launch_one(const uint32_t* qa_pack, const float* q_stat, int B, int H
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return (int)e;
   }
-  kern<<<dim3(n_split, Hkv, B), dim3(MF_WAVES * 64), smem, st>>>(qa_pack, q_stat, Hq, Hkv, pool, block_table,
-                                                                 bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts,
-                                                                 n_split);
+  if (t_start_event || t_stop_event) {
+    hipExtLaunchKernelGGL(kern, dim3(n_split, Hkv, B), dim3(MF_WAVES * 64), smem, st, t_start_event, t_stop_event, 0,
+                          qa_pack, q_stat, Hq, Hkv, pool, block_table, bt_stride, seq_lens, sm_scale, ly, L, parts,
+                          n_parts, n_split);
+    t_start_event = t_stop_event = nullptr;
+  } else {
+    kern<<<dim3(n_split, Hkv, B), dim3(MF_WAVES * 64), smem, st>>>(qa_pack, q_stat, Hq, Hkv, pool, block_table,
+                                                                   bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts,
+                                                                   n_split);
+  }
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? TQ_OK : (int)e;
 }
@@ -676,3 +690,8 @@ int launch_decode_mfma(const uint32_t* qa_pack, const float* q_stat, int B, int 
 }
 
 }  // namespace tq
+
+extern "C" void tq_time_next_page_kernel(void* start_event, void* stop_event) {
+  tq::t_start_event = (hipEvent_t)start_event;
+  tq::t_stop_event = (hipEvent_t)stop_event;
+}

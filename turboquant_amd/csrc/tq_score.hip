@@ -85,11 +85,11 @@ rotate_query_kernel(const void* __restrict__ q, int dtype, int64_t rows, int R, 
 // qa_pack receives the score-stage A operands of v_mfma_scale_f32_16x16x128_f8f6f4 (A fp6 e2m3, which
 // runs at twice the fp8 rate; B fp4) in register order: [kv head][term plane][128-coordinate chunk i]
 // [row set][lane][8 dwords, 6 used].  A value v (the normalised query coordinate times the plane's
-// coefficient, |v| <= 1) is the sum of three fp6 terms with per-row block scales 2^-2, 2^-7, 2^-12:
-// t0 = fp6(4 v), t1 = fp6(32 (4 v - t0)), t2 = fp6(32 (32 (4 v - t0) - t1)); a term's rounding error
-// is at most 1/8, so every product stays within the fp6 range and the sum is good to 2^-15.  Row set 0
-// holds terms 0 and 1 (row 2g + t for head g), row set 1 holds term 2 in row 2g (the odd rows are
-// zero), so that both accumulate into the same MFMA output registers.  For 6-bit operands lane
+// coefficient, |v| <= 1) is the sum of four fp6 terms with per-row block scales 2^-2, 2^-7, 2^-12,
+// 2^-17: t0 = fp6(4 v), t1 = fp6(32 (4 v - t0)), t2 = fp6(32 (32 (4 v - t0) - t1)), ...; a term's
+// rounding error is at most 1/8, so every product stays within the fp6 range and the sum is good to
+// 2^-20.  Row set 0 holds terms 0 and 1 (row 2g + t for head g), row set 1 terms 2 and 3, so that
+// both accumulate into the same MFMA output registers (8 heads x 4 terms fill the 2 x 16 rows).  For 6-bit operands lane
 // (row, block b) holds contraction indices 32b..32b+31, index j at bits 6j..6j+5 of its 192 bits, and
 // the key kernel puts coordinate c of plane word w at contraction index 32w + 8 (c % 4) + c / 4.
 constexpr int PREP_COLS = 32, PREP_SLICES = 16;
@@ -230,10 +230,10 @@ prep_query_kernel(const void* __restrict__ q, int dtype, int G, tq_layer ly, flo
     q_sk[(row0 + r) * d + word * PREP_COLS + c] = rb;
   }
   __syncthreads();
-  // operands of this plane word.  First the three 6-bit codes of every (term plane, head, contraction
+  // operands of this plane word.  First the four 6-bit codes of every (term plane, head, contraction
   // index) into shared memory (the partial sums are no longer needed), then per (term plane, row set,
   // row) one lane x six dwords, each gathered from the (up to seven) codes that overlap it.
-  uint32_t* codes = (uint32_t*)pa;                           // [ntp][G][3 terms][32]
+  uint32_t* codes = (uint32_t*)pa;                           // [ntp][G][4 terms][32]
   for (int o = tid; o < ntp * G * PREP_COLS; o += blockDim.x) {
     const int kloc = o % PREP_COLS, g = (o / PREP_COLS) % G, tp = o / (PREP_COLS * G);
     const bool is_sign = tp == ntp - 1;
@@ -245,10 +245,10 @@ prep_query_kernel(const void* __restrict__ q, int dtype, int G, tq_layer ly, flo
                       (t4 == 1 ? 0.5f : (t4 == 2 ? 0.25f : 1.0f));
     float v = (is_sign ? ssk : srot)[g * PREP_COLS + c] * mul;
 #pragma unroll
-    for (int t = 0; t < 3; ++t) {
+    for (int t = 0; t < 4; ++t) {
       uint32_t code;
       const float r = round_fp6(v, code);
-      codes[((tp * G + g) * 3 + t) * PREP_COLS + kloc] = code;
+      codes[((tp * G + g) * 4 + t) * PREP_COLS + kloc] = code;
       v = (v - r) * 32.0f;
     }
   }
@@ -259,10 +259,10 @@ prep_query_kernel(const void* __restrict__ q, int dtype, int G, tq_layer ly, flo
     const int dwi = o & 7, n = (o >> 3) & 15, rs = (o >> 7) & 1, tp = o >> 8;
     if (dwi >= 6) continue;
     const int g = n >> 1;
-    const int term = rs == 0 ? (n & 1) : ((n & 1) ? -1 : 2);
+    const int term = 2 * rs + (n & 1);
     uint32_t packed = 0;
-    if (term >= 0 && g < G) {
-      const uint32_t* cd = codes + ((tp * G + g) * 3 + term) * PREP_COLS;
+    if (g < G) {
+      const uint32_t* cd = codes + ((tp * G + g) * 4 + term) * PREP_COLS;
       const int j0 = (32 * dwi) / 6, j1 = min((32 * dwi + 31) / 6, 31);
       for (int kloc = j0; kloc <= j1; ++kloc) {
         const int bit = 6 * kloc - 32 * dwi;                 // position of the code in this dword (may straddle)
