@@ -444,6 +444,39 @@ def test_decode_split_invariance_and_page_permutation(gpu):
     assert torch.equal(o2, outs[1])
 
 
+def test_page_kernel_timing_hook_times_one_dispatch_and_changes_nothing(gpu):
+    # tq_time_next_page_kernel attaches an event pair to the next page-kernel dispatch of this thread:
+    # the elapsed time is positive and below the bracketing stream markers', the hook disarms itself,
+    # and the result is bit-identical to an untimed call
+    from turboquant_amd import _ffi
+    g = torch.Generator().manual_seed(9)
+    d, Hkv, Hq, N = 256, 2, 16, 4096
+    pool, _ = _make_pool(gpu, d, 3, 2, Hkv, N // 16)
+    k = torch.randn(1, N, Hkv, d, generator=g).bfloat16().to(gpu)
+    v = torch.randn(1, N, Hkv, d, generator=g).bfloat16().to(gpu)
+    t = torch.arange(N // 16, dtype=torch.int32)[None].to(gpu)
+    pool.append(k, v, t)
+    q = torch.randn(1, Hq, d, generator=g).bfloat16().to(gpu)
+    seq = torch.tensor([N], dtype=torch.int32, device=gpu)
+    ref = pool.decode_attention(q, t, seq, max_len=N).clone()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
+    for e in ev:
+        e.record()                                   # creates the underlying events
+    torch.cuda.synchronize()
+    ev[0].record()
+    _ffi.lib().tq_time_next_page_kernel(ev[1].cuda_event, ev[2].cuda_event)
+    out = pool.decode_attention(q, t, seq, max_len=N).clone()
+    ev[3].record()
+    torch.cuda.synchronize()
+    inner, outer = ev[1].elapsed_time(ev[2]), ev[0].elapsed_time(ev[3])
+    _progress(f"page kernel {inner * 1e3:.1f} us inside a {outer * 1e3:.1f} us call")
+    assert 0.0 < inner < outer
+    assert torch.equal(out, ref)
+    again = pool.decode_attention(q, t, seq, max_len=N)          # hook disarmed: plain launch
+    torch.cuda.synchronize()
+    assert torch.equal(again, ref)
+
+
 def test_decode_constant_values_and_convexity(gpu):
     # softmax weights are a convex combination: constant V comes back exactly (up to value
     # quantisation of a constant group, which is exact) and outputs stay inside [min v, max v]
