@@ -107,6 +107,21 @@ __device__ __forceinline__ float round_fp6(float v, uint32_t& code) {
   return v < 0.0f ? -r : r;
 }
 
+// sum over the 64 lanes with DPP row operations and four lane reads (no shared-memory permutes)
+template <int CTRL>
+__device__ __forceinline__ float prep_dpp(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float wave_sum_dpp(float v) {
+  v += prep_dpp<0xB1>(v);      // quad_perm [1,0,3,2]
+  v += prep_dpp<0x4E>(v);      // quad_perm [2,3,0,1]
+  v += prep_dpp<0x141>(v);     // row_half_mirror
+  v += prep_dpp<0x140>(v);     // row_mirror: every lane holds its row's sum
+  const int b = __builtin_bit_cast(int, v);
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 0)) + __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 16)) +
+         __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 32)) + __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48));
+}
+
 template <int PER>      // matrix rows per thread = d / PREP_SLICES
 __global__ void __launch_bounds__(PREP_COLS * PREP_SLICES)
 prep_query_kernel(const void* __restrict__ q, int dtype, int G, tq_layer ly, float sm_scale,
@@ -115,8 +130,17 @@ prep_query_kernel(const void* __restrict__ q, int dtype, int G, tq_layer ly, flo
   extern __shared__ float sm[];
   const int d = ly.d, tid = threadIdx.x, jl = tid % PREP_COLS, sl = tid / PREP_COLS;
   const int word = blockIdx.y, j = word * PREP_COLS + jl;
-  // every global load of the kernel is issued here, before anything waits: the matrix slices
-  // do not depend on the query
+  // every global load of the kernel is issued here, before anything waits, the query first: loads
+  // return in order, so the query can go to shared memory (and its statistics be taken) while the
+  // matrix slices, which do not depend on it, are still on their way
+  const int64_t group = blockIdx.x, row0 = group * G;
+  constexpr int QPT = ROT_MAX_ROWS * 256 / (PREP_COLS * PREP_SLICES);   // query elements per thread, d <= 256
+  float qv[QPT];
+#pragma unroll
+  for (int k = 0; k < QPT; ++k) {
+    const int o = tid + k * (PREP_COLS * PREP_SLICES);
+    qv[k] = o < G * d ? load_as_f32(q, row0 * d + o, dtype) : 0.0f;
+  }
   float mp[PER], ms[PER];
 #pragma unroll
   for (int k = 0; k < PER; ++k) {
@@ -137,8 +161,11 @@ prep_query_kernel(const void* __restrict__ q, int dtype, int G, tq_layer ly, flo
   float* ssk = srot + G * PREP_COLS;
   float* stat = ssk + G * PREP_COLS;                // [G][4]
   float* coefs = stat + 4 * ROT_MAX_ROWS;           // [16]
-  const int64_t group = blockIdx.x, row0 = group * G;
-  for (int o = tid; o < G * d; o += blockDim.x) sq[o] = load_as_f32(q, row0 * d + o, dtype);
+#pragma unroll
+  for (int k = 0; k < QPT; ++k) {
+    const int o = tid + k * (PREP_COLS * PREP_SLICES);
+    if (o < G * d) sq[o] = qv[k];
+  }
   const int mb = ly.mse_bits;
   int nx = 0;
   float cmax = 0.0f;
@@ -178,15 +205,15 @@ prep_query_kernel(const void* __restrict__ q, int dtype, int G, tq_layer ly, flo
         s1 = fmaf(x, cs1[k], s1);
         s2 = fmaf(x, cs2[k], s2);
       }
-      ss = wave_sum(ss); s1 = wave_sum(s1); s2 = wave_sum(s2);
+      ss = wave_sum_dpp(ss); s1 = wave_sum_dpp(s1); s2 = wave_sum_dpp(s2);
       if (lane == 0) {
         const float nq = sqrtf(ss), k = sm_scale * 1.4426950408889634f;
-        int e1, e2;      // bound < 2^e (frexp's mantissa is below 1); a zero query gives e = 0
-        frexpf(fminf(fabsf(k) * nq * cmax, 1e30f), &e1);
-        frexpf(fminf(2.0f * fabsf(k * ly.qjl_scale) * nq * ly.S_rownorm_max, 1e30f), &e2);
-        e1 = max(e1, -100); e2 = max(e2, -100);
-        stat[r * 4 + 0] = k * ldexpf(1.0f, -e1);                       // multiplier of coef q_rot_j
-        stat[r * 4 + 1] = 2.0f * k * ly.qjl_scale * ldexpf(1.0f, -e2); // multiplier of q_sk_j
+        // bound < 2^e: e = exponent field - 126 (the mantissa of frexp is below 1), kept within
+        // +-100 (a zero, denormal or huge bound only has to stay finite)
+        const int e1 = min(max((int)((__float_as_uint(fabsf(k) * nq * cmax) >> 23) & 255u) - 126, -100), 100);
+        const int e2 = min(max((int)((__float_as_uint(2.0f * fabsf(k * ly.qjl_scale) * nq * ly.S_rownorm_max) >> 23) & 255u) - 126, -100), 100);
+        stat[r * 4 + 0] = k * __uint_as_float((uint32_t)(127 - e1) << 23);                       // multiplier of coef q_rot_j
+        stat[r * 4 + 1] = 2.0f * k * ly.qjl_scale * __uint_as_float((uint32_t)(127 - e2) << 23); // multiplier of q_sk_j
         if (word == 0) {
           q_stat[(row0 + r) * 4 + 0] = (float)e1; q_stat[(row0 + r) * 4 + 1] = (float)e2;
           q_stat[(row0 + r) * 4 + 2] = k * ly.term_const * s1; q_stat[(row0 + r) * 4 + 3] = -k * ly.qjl_scale * s2;
@@ -204,10 +231,14 @@ prep_query_kernel(const void* __restrict__ q, int dtype, int G, tq_layer ly, flo
     for (int r = 0; r < ROT_MAX_ROWS; ++r) {
       if (r < G) {
 #pragma unroll
-        for (int k = 0; k < PER; ++k) {
-          const float x = sq[r * d + i0 + k];
-          a[r] = fmaf(x, mp[k], a[r]);
-          b[r] = fmaf(x, ms[k], b[r]);
+        for (int k4 = 0; k4 < PER / 4; ++k4) {
+          const float4 x = *(const float4*)(sq + r * d + i0 + 4 * k4);
+          const float xs[4] = {x.x, x.y, x.z, x.w};
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            a[r] = fmaf(xs[k], mp[4 * k4 + k], a[r]);
+            b[r] = fmaf(xs[k], ms[4 * k4 + k], b[r]);
+          }
         }
       }
     }
@@ -220,22 +251,25 @@ prep_query_kernel(const void* __restrict__ q, int dtype, int G, tq_layer ly, flo
     }
   }
   __syncthreads();
-  for (int o = tid; o < G * PREP_COLS; o += blockDim.x) {
-    const int r = o / PREP_COLS, c = o - r * PREP_COLS;
-    float ra = 0.0f, rb = 0.0f;
-    for (int k = 0; k < PREP_SLICES; ++k) { ra += pa[(k * G + r) * PREP_COLS + c]; rb += pb[(k * G + r) * PREP_COLS + c]; }
-    srot[o] = ra;
-    ssk[o] = rb;
-    q_rot[(row0 + r) * d + word * PREP_COLS + c] = ra;
-    q_sk[(row0 + r) * d + word * PREP_COLS + c] = rb;
+  for (int o2 = tid; o2 < 2 * G * PREP_COLS; o2 += blockDim.x) {      // first half: rotation, second: sketch
+    const bool sk = o2 >= G * PREP_COLS;
+    const int o = sk ? o2 - G * PREP_COLS : o2, r = o / PREP_COLS, c = o - r * PREP_COLS;
+    const float* part = sk ? pb : pa;
+    float acc = 0.0f;
+#pragma unroll
+    for (int k = 0; k < PREP_SLICES; ++k) acc += part[(k * G + r) * PREP_COLS + c];
+    (sk ? ssk : srot)[o] = acc;
+    (sk ? q_sk : q_rot)[(row0 + r) * d + word * PREP_COLS + c] = acc;
   }
   __syncthreads();
   // operands of this plane word.  First the four 6-bit codes of every (term plane, head, contraction
   // index) into shared memory (the partial sums are no longer needed), then per (term plane, row set,
   // row) one lane x six dwords, each gathered from the (up to seven) codes that overlap it.
   uint32_t* codes = (uint32_t*)pa;                           // [ntp][G][4 terms][32]
-  for (int o = tid; o < ntp * G * PREP_COLS; o += blockDim.x) {
-    const int kloc = o % PREP_COLS, g = (o / PREP_COLS) % G, tp = o / (PREP_COLS * G);
+  // thread -> (contraction index, head, half of the workgroup); the halves take alternate term planes
+  for (int tp = tid >> 8; tp < ntp; tp += 2) {
+    const int kloc = tid & 31, g = (tid >> 5) & 7;
+    if (g >= G) break;
     const bool is_sign = tp == ntp - 1;
     const int c = 4 * (kloc & 7) + (kloc >> 3);              // coordinate within the word
     // the decode kernel extracts three of the four bits of a nibble in place, where they are the fp4
