@@ -269,20 +269,23 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
   // and serialise the prefetch.
   const uint32_t off_zero_c = L.off_vzero + min(n, NGT - 1) * 32;
   const int spg = min(lane / PIECES, 3);
+  // The page of a lane is picked among the four page numbers with conditional moves on vector
+  // registers (on scalar operands the compiler builds branches instead) and turned into an address
+  // with one unsigned 32 x 32 -> 64 bit multiply-add.
+  const uint32_t page_stride32 = (uint32_t)page_stride;
   auto load_vals = [&](const int (&pid)[4], ValRegs& R) {
-    // per-lane page: selected as a number (three conditional moves), not as one of four pointers
-    int my_pid = kb == 0 ? pid[0] : (kb == 1 ? pid[1] : (kb == 2 ? pid[2] : pid[3]));
-    asm volatile("" : "+v"(my_pid));
-    const uint8_t* vbase = pool_h + my_pid * page_stride;
+    const uint32_t p0 = in_vgpr((uint32_t)pid[0]), p1 = in_vgpr((uint32_t)pid[1]), p2 = in_vgpr((uint32_t)pid[2]),
+                   p3 = in_vgpr((uint32_t)pid[3]);
+    const uint32_t my_pid = kb == 0 ? p0 : (kb == 1 ? p1 : (kb == 2 ? p2 : p3));
+    const uint8_t* vbase = pool_h + (uint64_t)my_pid * page_stride32;
     const uint32_t* vp = (const uint32_t*)(vbase + off_v);
 #pragma unroll
     for (int w = 0; w < VW; ++w) R.v[w] = vp[w];
     const u32x4* zp = (const u32x4*)(vbase + off_zero_c);
     R.zero[0] = zp[0];
     R.zero[1] = zp[1];
-    int spid = spg == 0 ? pid[0] : (spg == 1 ? pid[1] : (spg == 2 ? pid[2] : pid[3]));
-    asm volatile("" : "+v"(spid));
-    R.scale = *(const u32x4*)(pool_h + spid * page_stride + off_scale);
+    const uint32_t spid = spg == 0 ? p0 : (spg == 1 ? p1 : (spg == 2 ? p2 : p3));
+    R.scale = *(const u32x4*)(pool_h + (uint64_t)spid * page_stride32 + off_scale);
   };
 
   // A value code masked in place is a bf16 number: a pattern n < 256 in a 16-bit half is n * 2^-133
