@@ -255,13 +255,16 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
     for (int pg = 0; pg < 4; ++pg) pid[pg] = bt[min(4 * blk + pg, n_pages - 1)];
   };
   auto load_keys = [&](const int (&pid)[4], KeyRegs& R) {
+    // the 32-bit lane offsets are re-materialised here, next to their use, so that the loads take
+    // the scalar page base plus a 32-bit vector offset instead of a 64-bit vector address
+    const uint32_t ok = in_vgpr(off_keys), om = in_vgpr(off_meta);
 #pragma unroll
     for (int pg = 0; pg < 4; ++pg) {
       const uint8_t* base = pool_h + pid[pg] * page_stride;
-      const uint32_t* kp = (const uint32_t*)(base + off_keys);
+      const uint32_t* kp = (const uint32_t*)(base + ok);
 #pragma unroll
       for (int w = 0; w < NKW; ++w) R.key[pg][w] = kp[w];
-      R.meta[pg] = *(const f32x2*)(base + off_meta);
+      R.meta[pg] = *(const f32x2*)(base + om);
     }
   };
   // All loads below are unconditional (lanes without a group / piece of their own read a
