@@ -161,7 +161,10 @@ int tq_rotate_query(const void *q, int dtype, int64_t rows, const tq_layer *laye
  * k, v: element (b, t, h, :) at  base + b*stride_b + t*stride_t + h*stride_h  (in
  * elements), innermost dimension contiguous.  Token t of sequence b goes to
  * logical position start_pos[b] + t, i.e. page block_table[b*max_pages + pos/16],
- * slot pos%16.  start_pos may be NULL (all zero).  pool is (num_pages, H, page_bytes). */
+ * slot pos%16.  start_pos may be NULL (all zero).  pool is (num_pages, H, page_bytes).
+ * Large appends run their value kernel on a side stream of the calling thread (created on
+ * first use, default priority) that is forked from and joined back into `stream` with
+ * events: the call is ordered on `stream` like any other and stays capturable.           */
 int tq_append_kv_paged(const void *k, const void *v, int dtype, int B, int T, int H, int64_t stride_b,
                        int64_t stride_t, int64_t stride_h, const int32_t *start_pos, const int32_t *block_table,
                        int max_pages, const tq_layer *layer, const tq_page_layout *layout, uint8_t *pool,

@@ -307,6 +307,30 @@ def test_paged_append_equals_flat_quantise(gpu, d, key_bits, vb, dtype):
     assert torch.equal(pool.data[used[:-1]], pool2.data[used[:-1]])
 
 
+def test_large_append_runs_values_beside_keys_and_stays_ordered(gpu):
+    # an append of >= 4096 tiles forks the value kernel onto a side stream and joins it back: the
+    # pages must equal those of two small appends (plain path), and a reader queued on the caller's
+    # stream right after the call must see finished pages
+    H, T, d = 8, 8192, 128
+    g = torch.Generator().manual_seed(21)
+    k = torch.randn(1, T, H, d, generator=g).bfloat16().to(gpu)
+    v = torch.randn(1, T, H, d, generator=g).bfloat16().to(gpu)
+    table = torch.randperm(T // 16, generator=g).to(torch.int32).to(gpu)[None, :]
+    big, _ = _make_pool(gpu, d, 3, 2, H, T // 16)
+    small, _ = _make_pool(gpu, d, 3, 2, H, T // 16)
+    for _ in range(3):                               # repeated so that a missing join would show as a race
+        big.data.zero_()
+        big.append(k, v, table)
+        seen = big.data.clone()                      # queued behind the append on the same stream
+    half = T // 2
+    small.append(k[:, :half], v[:, :half], table)
+    small.append(k[:, half:], v[:, half:], table, torch.tensor([half], dtype=torch.int32, device=gpu))
+    torch.cuda.synchronize()
+    used = table[0].long()
+    assert torch.equal(seen[used], small.data[used])
+    assert torch.equal(big.data[used], small.data[used])
+
+
 def _store_from_oracle_view(pool, table_row, n_tok):
     idx, sgn, norms, rnorms, vdata, vsc, vz = [t.cpu() for t in pool.export_flat(table_row, n_tok)]
     return key_code(idx, sgn, rnorms, norms, pool.quantizer.bits - 1), value_code(vdata, vsc, vz, pool.value_bits)

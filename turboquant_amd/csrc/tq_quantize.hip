@@ -698,6 +698,29 @@ extern "C" int tq_quantize_values(const void* v, int dtype, int64_t n_vec, int64
   return launch_value(v, dtype, src, d, group_size, bits, sink, (n_vec + TILE - 1) / TILE, (hipStream_t)stream);
 }
 
+// Side stream of the calling thread on the current device (created on first use, default priority,
+// kept until the process ends), with the two events of the fork / join.  nullptr when it cannot be
+// had: the caller then launches on its own stream.
+namespace {
+struct SideLane { hipStream_t stream = nullptr; hipEvent_t fork = nullptr, join = nullptr; bool tried = false; };
+constexpr int64_t SIDE_MIN_TILES = 4096;       // below this the fork / join costs more than it hides
+constexpr int SIDE_MAX_DEVICES = 16;
+SideLane* side_lane() {
+  static thread_local SideLane lanes[SIDE_MAX_DEVICES];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= SIDE_MAX_DEVICES) return nullptr;
+  SideLane& l = lanes[dev];
+  if (!l.tried) {
+    l.tried = true;
+    if (hipStreamCreateWithFlags(&l.stream, hipStreamNonBlocking) != hipSuccess) l.stream = nullptr;
+    if (l.stream && (hipEventCreateWithFlags(&l.fork, hipEventDisableTiming) != hipSuccess ||
+                     hipEventCreateWithFlags(&l.join, hipEventDisableTiming) != hipSuccess))
+      l.stream = nullptr;
+  }
+  return l.stream ? &l : nullptr;
+}
+}  // namespace
+
 extern "C" int tq_append_kv_paged(const void* k, const void* v, int dtype, int B, int T, int H, int64_t stride_b,
                                   int64_t stride_t, int64_t stride_h, const int32_t* start_pos,
                                   const int32_t* block_table, int max_pages, const tq_layer* layer,
@@ -714,9 +737,28 @@ extern "C" int tq_append_kv_paged(const void* k, const void* v, int dtype, int B
   PagedSource src{B, T, H, tiles_per_seq, stride_b, stride_t, stride_h, start_pos};
   int64_t tiles = (int64_t)B * tiles_per_seq * H;
   KeyPagedSink ks{pool, block_table, max_pages, *layout};
+  ValPagedSink vs{pool, block_table, max_pages, *layout};
+  // Large appends run the value kernel beside the key kernel: the key kernel leaves a quarter of the
+  // registers and issue slots of every SIMD free, which the small value wavefronts fill (the two
+  // kernels write disjoint bytes of the pages).  The value kernel goes to a side stream that is
+  // forked from and joined back into the caller's stream with events, so the call stays ordered
+  // on `stream` like any other.
+  if (tiles >= SIDE_MIN_TILES) {
+    if (SideLane* lane = side_lane()) {
+      hipStream_t st = (hipStream_t)stream;
+      if (hipEventRecord(lane->fork, st) == hipSuccess && hipStreamWaitEvent(lane->stream, lane->fork, 0) == hipSuccess) {
+        rc = launch_value(v, dtype, src, layer->d, layout->group_size, layout->value_bits, vs, tiles, lane->stream);
+        hipError_t e1 = hipEventRecord(lane->join, lane->stream);
+        int rc2 = launch_key(k, dtype, src, *layer, ks, 0, tiles, st);
+        hipError_t e2 = e1 == hipSuccess ? hipStreamWaitEvent(st, lane->join, 0) : e1;
+        if (rc) return rc;
+        if (rc2) return rc2;
+        return e2 == hipSuccess ? TQ_OK : (int)e2;
+      }
+    }
+  }
   rc = launch_key(k, dtype, src, *layer, ks, 0, tiles, (hipStream_t)stream);
   if (rc) return rc;
-  ValPagedSink vs{pool, block_table, max_pages, *layout};
   return launch_value(v, dtype, src, layer->d, layout->group_size, layout->value_bits, vs, tiles, (hipStream_t)stream);
 }
 
