@@ -438,6 +438,27 @@ def shape_kq_128(k, trend):
     return k + spikes[None, :, None, None] * u
 
 
+def test_decode_attention_random_shapes(gpu):
+    # seeded sweep over head dims, bit widths, GQA ratios, batch sizes, ragged lengths (block and page
+    # boundaries included), split counts and exact tails
+    import random
+    rnd = random.Random(1234)
+    boundary = [0, 1, 15, 16, 17, 63, 64, 65, 127, 128, 129, 255, 256, 257]
+    for case in range(14):
+        d = rnd.choice([64, 128, 128, 256, 256])
+        key_bits = rnd.choice([2, 3, 3, 4]) if d != 256 else rnd.choice([2, 3])
+        vb = rnd.choice([2, 4])
+        Hkv = rnd.choice([1, 2, 3])
+        G = rnd.choice([1, 2, 4, 8])
+        B = rnd.choice([1, 2, 4])
+        lens = [rnd.choice(boundary + [rnd.randrange(300, 900)]) for _ in range(B)]
+        recent = [rnd.choice([0, 0, 1, 7, 33]) for _ in range(B)] if rnd.random() < 0.4 else None
+        n_split = rnd.choice([None, 1, 2, 5, 16])
+        _progress(f"random case {case}: d={d} kb={key_bits} vb={vb} Hkv={Hkv} G={G} lens={lens} recent={recent} split={n_split}")
+        worst = _decode_case(gpu, d, key_bits, vb, B, Hkv * G, Hkv, lens, recent, seed=100 + case, n_split=n_split)
+        _progress(f"   worst cosine {worst:.7f}")
+
+
 def test_decode_attention_ragged_empty_and_hybrid_tail(gpu):
     # empty sequence, history shorter than a page, page-aligned history, ragged exact tails
     worst = _decode_case(gpu, 128, 3, 4, 5, 8, 2, [0, 5, 16, 33, 1000], [0, 3, 128, 0, 77], seed=77)
