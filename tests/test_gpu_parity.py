@@ -307,6 +307,40 @@ def test_paged_append_equals_flat_quantise(gpu, d, key_bits, vb, dtype):
     assert torch.equal(pool.data[used[:-1]], pool2.data[used[:-1]])
 
 
+def test_paged_append_random_chunks_equal_flat_quantise(gpu):
+    # seeded sweep: several sequences appended in ragged chunks (any start slot inside a page, chunk
+    # lengths across page boundaries, batched calls with per-sequence start positions); the exported
+    # pages must equal the flat quantisers' output bit for bit
+    import random
+    from turboquant_amd.kv_cache import quantize_values
+    rnd = random.Random(77)
+    for case in range(8):
+        d = rnd.choice([64, 128, 256])
+        key_bits = rnd.choice([2, 3, 4]) if d != 256 else rnd.choice([2, 3])
+        vb = rnd.choice([2, 4])
+        dtype = rnd.choice([torch.bfloat16, torch.bfloat16, torch.float16])
+        H, B = rnd.choice([1, 2, 4]), rnd.choice([1, 2, 3])
+        total = rnd.choice([16, 31, 64, 100, 177])
+        cuts = sorted(set([0, total] + [rnd.randrange(1, total) for _ in range(rnd.choice([0, 1, 2]))]))
+        pages = (total + 15) // 16
+        pool, tq = _make_pool(gpu, d, key_bits, vb, H, B * pages + 2, dtype, seed=5 + case)
+        g = torch.Generator().manual_seed(300 + case)
+        k = torch.randn(B, total, H, d, generator=g).to(dtype).to(gpu)
+        v = torch.randn(B, total, H, d, generator=g).to(dtype).to(gpu)
+        table = torch.randperm(B * pages + 2, generator=g)[: B * pages].to(torch.int32).reshape(B, pages).to(gpu)
+        _progress(f"append case {case}: d={d} kb={key_bits} vb={vb} {dtype} H={H} B={B} cuts={cuts}")
+        for a0, a1 in zip(cuts[:-1], cuts[1:]):
+            pool.append(k[:, a0:a1], v[:, a0:a1], table, torch.full((B,), a0, dtype=torch.int32, device=gpu))
+        for b in range(B):
+            idx, sgn, norms, rnorms, vdata, vsc, vz = pool.export_flat(table[b], total)
+            ref = tq.quantize(k[b].transpose(0, 1))
+            refv = quantize_values(v[b].transpose(0, 1), bits=vb, group_size=32)
+            torch.cuda.synchronize()
+            assert torch.equal(idx, ref.mse_indices) and torch.equal(sgn, ref.qjl_signs), (case, b)
+            assert torch.equal(norms, ref.norms) and torch.equal(rnorms, ref.residual_norms), (case, b)
+            assert torch.equal(vdata, refv.data) and torch.equal(vsc, refv.scales) and torch.equal(vz, refv.zeros), (case, b)
+
+
 def test_large_append_runs_values_beside_keys_and_stays_ordered(gpu):
     # an append of >= 4096 tiles forks the value kernel onto a side stream and joins it back: the
     # pages must equal those of two small appends (plain path), and a reader queued on the caller's
