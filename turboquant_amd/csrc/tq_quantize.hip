@@ -384,10 +384,25 @@ value_chunk_kernel(const void* __restrict__ v, Source src, int d, int gs, Sink s
   const float floor_v = round_hw<DT>(1e-10f);
   sc = (sc != sc) ? sc : fmaxf(sc, floor_v);
   const float z = lo;
+  // Quotients of bf16 numbers, rounded to bf16: a / s with 8-bit significands is either exactly a bf16
+  // rounding tie (a 9-bit quotient) or at least 2^-17 (relative) away from one, so any fp32 quotient good
+  // to an ulp rounds like the correctly rounded one, as long as ties come out exact.  q0 = a * (1/s)
+  // followed by one residual correction q0 + (a - q0 s)(1/s) does both (the fused residual is exact for
+  // a tie).  Used when the scale is an ordinary number; everything else takes the division.
+  const bool fast_div = DT == TQ_BF16 && sc > 0x1p-60f && sc < 0x1p60f;
+  const float rsc = 1.0f / sc;
   uint32_t codes = 0;                              // 8 codes, VB bits each, channel order
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    float q = round_hw<DT>(round_hw<DT>(x[i] - z) / sc);
+    const float a = round_hw<DT>(x[i] - z);
+    float quo;
+    if (fast_div && fabsf(a) < 0x1p60f) {
+      const float q0 = a * rsc;
+      quo = fmaf(fmaf(-q0, sc, a), rsc, q0);
+    } else {
+      quo = a / sc;
+    }
+    float q = round_hw<DT>(quo);
     q = rintf(q);
     q = fminf(fmaxf(q, 0.0f), levels);
     const uint32_t c = (q != q) ? 0u : (uint32_t)q;
