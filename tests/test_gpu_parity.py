@@ -472,6 +472,16 @@ def shape_kq_128(k, trend):
     return k + spikes[None, :, None, None] * u
 
 
+@pytest.mark.parametrize("d,key_bits,vb,Hq,Hkv,dtype", [(128, 3, 4, 8, 2, torch.float16), (128, 3, 2, 32, 2, torch.bfloat16),
+                                                         (64, 3, 4, 12, 1, torch.float16), (128, 4, 4, 4, 2, torch.float32)])
+def test_decode_attention_general_kernel_shapes(gpu, d, key_bits, vb, Hq, Hkv, dtype):
+    # shapes without a matrix-core kernel (fp16 / fp32 pools, more than 8 query heads per KV head)
+    # take the general page kernel and must meet the same gate
+    _progress(f"general decode d={d} kb={key_bits} vb={vb} Hq={Hq} Hkv={Hkv} {dtype}")
+    worst = _decode_case(gpu, d, key_bits, vb, 2, Hq, Hkv, [300, 77], [0, 9], seed=500 + d + Hq, dtype=dtype)
+    _progress(f"   worst cosine {worst:.7f}")
+
+
 def test_decode_attention_random_shapes(gpu):
     # seeded sweep over head dims, bit widths, GQA ratios, batch sizes, ragged lengths (block and page
     # boundaries included), split counts and exact tails
