@@ -223,42 +223,86 @@ exact_tail_kernel(const void* __restrict__ q, int dtype, int Hq, int Hkv, int d,
 }
 
 // n_parts partials are merged per row; consecutive rows are part_stride partials apart.
-// One workgroup per row: the weights exp(m_s - M) are computed once into LDS, then
-// thread ch sums its channel over the parts (coalesced across threads).
+// One workgroup per row.  A thread owns a pair of channels and every S-th part (S = 256 / (d/2)
+// subsets share the parts when a row has fewer than 256 channel pairs); its first MERGE_CHUNK
+// accumulator loads are issued before anything else, so that the (m, l) loads, the weights
+// exp(m_s - M) and their reductions all run under one memory latency.
+constexpr int MERGE_CHUNK = 16;
+static size_t merge_smem(int n_parts, int d) {
+  const int np = d >> 1, S = np >= 256 ? 1 : 256 / np;
+  return ((size_t)3 * n_parts + 8 + (size_t)S * d) * sizeof(float);
+}
+
 __global__ void __launch_bounds__(256)
 merge_kernel(const float* __restrict__ parts, int n_parts, int part_stride, int d, int dtype, void* __restrict__ out) {
-  extern __shared__ float s_w[];                 // [n_parts] weights, then [8] scratch
+  extern __shared__ float s_w[];                 // [n_parts] weights, [n_parts] m, [n_parts] l, [8] scratch, [S][d] sums
   const int64_t row = blockIdx.x;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const float* p = parts + row * part_stride * (int64_t)(d + 2);
-  float* scratch = s_w + n_parts;
+  float* s_m = s_w + n_parts;
+  float* s_l = s_m + n_parts;
+  float* scratch = s_l + n_parts;
+  float* s_sum = scratch + 8;
+  const int np = d >> 1;                                        // channel pairs of a row
+  const int S = np >= 256 ? 1 : 256 / np;                       // subsets of parts (d is a multiple of 64)
+  const int tps = 256 / S;                                      // threads per subset
+  const int sub = tid / tps, pr = tid - sub * tps;
+  typedef float f2 __attribute__((ext_vector_type(2)));
+  // first chunk of this thread's accumulator loads (pair pr; parts sub, sub + S, ...), clamped in range
+  f2 v[MERGE_CHUNK];
+#pragma unroll
+  for (int k = 0; k < MERGE_CHUNK; ++k) {
+    const int sp = min(sub + k * S, n_parts - 1);
+    v[k] = *(const f2*)(p + (int64_t)sp * (d + 2) + 2 + 2 * min(pr, np - 1));
+  }
   float mm = NEG_BIG;
-  for (int s = tid; s < n_parts; s += blockDim.x) {
-    const float* r = p + (int64_t)s * (d + 2);
-    if (r[1] > 0.0f) mm = fmaxf(mm, r[0]);
+  for (int sp = tid; sp < n_parts; sp += blockDim.x) {
+    const f2 ml = *(const f2*)(p + (int64_t)sp * (d + 2));
+    s_m[sp] = ml[0];
+    s_l[sp] = ml[1];
+    if (ml[1] > 0.0f) mm = fmaxf(mm, ml[0]);
   }
   mm = wave_max(mm);
   if (lane == 0) scratch[wave] = mm;
   __syncthreads();
   mm = fmaxf(fmaxf(scratch[0], scratch[1]), fmaxf(scratch[2], scratch[3]));
   float ll = 0.0f;
-  for (int s = tid; s < n_parts; s += blockDim.x) {
-    const float* r = p + (int64_t)s * (d + 2);
-    const float w = r[1] > 0.0f ? __expf(r[0] - mm) : 0.0f;
-    s_w[s] = w;
-    ll += w * r[1];
+  for (int sp = tid; sp < n_parts; sp += blockDim.x) {
+    const float w = s_l[sp] > 0.0f ? __expf(s_m[sp] - mm) : 0.0f;
+    s_w[sp] = w;
+    ll += w * s_l[sp];
   }
   ll = wave_sum(ll);
   if (lane == 0) scratch[4 + wave] = ll;
   __syncthreads();
   ll = scratch[4] + scratch[5] + scratch[6] + scratch[7];
   const float inv = ll > 0.0f ? 1.0f / ll : 0.0f;
+  // every part was written by its producer (empty ones as zeros), so the loads need no guard
+  for (int p0 = pr; p0 < np; p0 += tps) {
+    f2 acc = {0.0f, 0.0f};
+    for (int k0 = 0; sub + k0 * S < n_parts; k0 += MERGE_CHUNK) {
+      if (k0 > 0 || p0 != pr) {
+#pragma unroll
+        for (int k = 0; k < MERGE_CHUNK; ++k) {
+          const int sp = min(sub + (k0 + k) * S, n_parts - 1);
+          v[k] = *(const f2*)(p + (int64_t)sp * (d + 2) + 2 + 2 * p0);
+        }
+      }
+#pragma unroll
+      for (int k = 0; k < MERGE_CHUNK; ++k) {
+        const int sp = sub + (k0 + k) * S;
+        const float w = sp < n_parts ? s_w[sp] : 0.0f;
+        acc[0] = fmaf(w, v[k][0], acc[0]);
+        acc[1] = fmaf(w, v[k][1], acc[1]);
+      }
+    }
+    s_sum[sub * d + 2 * p0] = acc[0];
+    s_sum[sub * d + 2 * p0 + 1] = acc[1];
+  }
+  __syncthreads();
   for (int ch = tid; ch < d; ch += blockDim.x) {
     float aa = 0.0f;
-    // every part was written by its producer (empty ones as zeros), so the loads need no guard and
-    // stay independent of each other
-#pragma unroll 8
-    for (int s = 0; s < n_parts; ++s) aa = fmaf(s_w[s], p[(int64_t)s * (d + 2) + 2 + ch], aa);
+    for (int q = 0; q < S; ++q) aa += s_sum[q * d + ch];
     store_from_f32(out, row * d + ch, aa * inv, dtype);
   }
 }
@@ -292,7 +336,7 @@ extern "C" int tq_decode_merge(const float* parts, int64_t rows, int n_parts, in
   if (!parts || !out) return TQ_ENULL;
   if (rows < 0 || n_parts <= 0 || d <= 0 || dtype < TQ_F32 || dtype > TQ_BF16) return TQ_EINVAL;
   if (rows == 0) return TQ_OK;
-  merge_kernel<<<dim3((unsigned)rows), dim3(256), (n_parts + 8) * sizeof(float), (hipStream_t)stream>>>(
+  merge_kernel<<<dim3((unsigned)rows), dim3(256), merge_smem(n_parts, d), (hipStream_t)stream>>>(
       parts, n_parts, n_parts, d, dtype, out);
   TQ_CHECK_LAUNCH();
   return TQ_OK;
@@ -373,7 +417,7 @@ extern "C" int tq_decode_attn_paged_stages(const void* q, int dtype, int B, int 
   }
   if (!(stages & 4)) return TQ_OK;
   // without a tail the merge simply reads one part fewer
-  merge_kernel<<<dim3((unsigned)(B * Hq)), dim3(256), (n_parts + 8) * sizeof(float), st>>>(
+  merge_kernel<<<dim3((unsigned)(B * Hq)), dim3(256), merge_smem(n_parts, d), st>>>(
       parts, tail ? n_parts : n_split, n_parts, d, dtype, out);
   TQ_CHECK_LAUNCH();
   return TQ_OK;
