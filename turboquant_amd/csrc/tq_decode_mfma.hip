@@ -11,11 +11,15 @@
 //    0001, 0010, 0100 are the fp4 numbers 0.5, 1, 2, so  x & 0x11111111,
 //    x & 0x22222222, x & 0x44444444 and (x >> 3) & 0x11111111 turn a 32-bit plane
 //    word into the four operand dwords (5 vector-ALU instructions for 32
-//    coordinates); the query operand carries the inverse factors.  The query is the fp6 (e2m3) operand - the MFMA runs
-//    at twice the fp8 rate with it -, split into four fp6 terms with per-row
-//    power-of-two scales (good to 2^-20 of the row bound), prepared once per step;
-//    every factor and constant of the score that belongs to a query head is folded
-//    into those operands, their block scales and the initial accumulator.
+//    coordinates); the query operand carries the inverse factors.  The query is
+//    the fp6 (e2m3) operand - the MFMA runs at twice the fp8 rate with it -, split
+//    into four fp6 terms with per-row power-of-two scales (good to 2^-20 of the
+//    row bound), prepared once per step; every factor and constant of the score
+//    that belongs to a query head is folded into those operands, their block
+//    scales and the initial accumulator.
+//  * softmax.  Weights are exp2(score - reference); the reference of a row only
+//    moves when a score exceeds it by more than a small slack, so the usual block
+//    needs no row reduction and no rescaling.
 //  * values.  A code masked out of its packed word IS a bf16 denormal (exponent
 //    field zero, the code in the low mantissa bits): B = code * 2^(s-133) exactly,
 //    s being the bit position the code has in its 16-bit half, and the bf16 MFMA
@@ -35,10 +39,10 @@
 // One wavefront (pair) owns 64 tokens (4 pages) per iteration: lane (n, kb) = lane%16,
 // lane/16 is token n and coordinate quarter kb in the score stage, and (row,
 // page kb) in the value stage.  The key words of the next 64 tokens are
-// requested before the current ones are consumed; the value words of the current
-// 64 tokens are requested before its score stage.  Workgroups have 4 wavefronts;
-// WPS of them share a SIMD so that one wavefront's dependency stalls are filled
-// by another.
+// requested right after the current score stage, the value words right after the
+// current value stage, so each load has a whole stage to arrive.  Workgroups have 4
+// wavefronts; WPS of them share a SIMD so that one wavefront's dependency stalls
+// are filled by another.
 
 #include <type_traits>
 
