@@ -458,18 +458,31 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
   // (6) write
   if constexpr (std::is_same<Sink, KeyFlatSink>::value) {
     // flat format of the reference (quantizer.py:38-69): indices packed eff_bits apiece, signs 8 per byte
-    const int eff = eff_bits(mb), per = 8 / eff, row = idx_row_bytes(D, mb);
-    for (int o = tid; o < TT * row; o += KQ_THREADS) {
-      const int t = o / row, k = o - t * row;
+    // A thread builds one dword of a row: n = 32 / eff codes, code s at bit eff * s, plane 0 the top bit of a
+    // code.  The n bits a plane contributes are spread to a stride of eff bits with shift-and-mask steps.
+    const int eff = eff_bits(mb), n_per = 32 / eff, row_dw = idx_row_bytes(D, mb) >> 2;
+    for (int o = tid; o < TT * row_dw; o += KQ_THREADS) {
+      const int t = o / row_dw, k = o - t * row_dw;
       if (!svalid[t]) continue;
-      unsigned byte = 0;
-      for (int s = 0; s < per; ++s) {
-        const int c = k * per + s;
-        unsigned v = 0;
-        for (int p = 0; p < mb; ++p) v |= ((spl[(p * TT + t) * W + (c >> 5)] >> (c & 31)) & 1u) << (mb - 1 - p);
-        byte |= v << (eff * s);
+      const int c0 = k * n_per;                                  // first coordinate of this dword
+      uint32_t dw = 0;
+      for (int p = 0; p < mb; ++p) {
+        uint32_t x = spl[(p * TT + t) * W + (c0 >> 5)] >> (c0 & 31);
+        if (eff == 2) {
+          x &= 0xffffu;
+          x = (x | (x << 8)) & 0x00ff00ffu;
+          x = (x | (x << 4)) & 0x0f0f0f0fu;
+          x = (x | (x << 2)) & 0x33333333u;
+          x = (x | (x << 1)) & 0x55555555u;
+        } else if (eff == 4) {
+          x &= 0xffu;
+          x = (x | (x << 12)) & 0x000f000fu;
+          x = (x | (x << 6)) & 0x03030303u;
+          x = (x | (x << 3)) & 0x11111111u;
+        }                                                         // eff == 1: the plane word is the dword
+        dw |= x << (mb - 1 - p);
       }
-      sink.idx[(tile0 * TILE + t) * row + k] = (uint8_t)byte;
+      ((uint32_t*)sink.idx)[(tile0 * TILE + t) * row_dw + k] = dw;
     }
     if (!mse_only) {
       for (int o = tid; o < TT * W; o += KQ_THREADS) {
@@ -525,7 +538,8 @@ __host__ static bool aligned_for_chunks(const void* x, int dtype, const PagedSou
   return (uintptr_t)x % 16 == 0 && s.stride_b % ch == 0 && s.stride_t % ch == 0 && s.stride_h % ch == 0;
 }
 __host__ static bool sink_ok(const KeyFlatSink& s, int mse_only) {
-  return (uintptr_t)s.y_dbg % 16 == 0 && (uintptr_t)s.p_dbg % 16 == 0 && (mse_only || (uintptr_t)s.sign % 4 == 0);
+  return (uintptr_t)s.y_dbg % 16 == 0 && (uintptr_t)s.p_dbg % 16 == 0 && (uintptr_t)s.idx % 4 == 0 &&
+         (mse_only || (uintptr_t)s.sign % 4 == 0);
 }
 __host__ static bool sink_ok(const KeyPagedSink& s, int) { return s.L.key_lane_major != 0; }
 
