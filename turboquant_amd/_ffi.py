@@ -158,7 +158,8 @@ def make_layer(d: int, mse_bits: int, Pi: torch.Tensor, PiT: torch.Tensor, centr
     ly.qjl_scale = math.sqrt(math.pi / 2.0) / d
     if splits is not None:
         pi_s, pit_s, s_s = splits
-        ly.Pi_split, ly.PiT_split = pi_s.data_ptr(), pit_s.data_ptr()
+        ly.Pi_split = None if pi_s is None else pi_s.data_ptr()
+        ly.PiT_split = None if pit_s is None else pit_s.data_ptr()
         ly.S_split = None if s_s is None else s_s.data_ptr()
     if query_consts is not None:
         pi_cs, s_cs, s_max = query_consts
@@ -168,15 +169,22 @@ def make_layer(d: int, mse_bits: int, Pi: torch.Tensor, PiT: torch.Tensor, centr
 
 
 def split_bf16x3(m: torch.Tensor) -> torch.Tensor:
-    """fp32 matrix -> (3, rows, cols) int16 tensor of bf16 bit patterns whose three
-    terms sum to the matrix exactly (each term rounds the running remainder)."""
+    """fp32 (d, d) matrix -> int16 tensor of bf16 bit patterns of three terms that sum
+    to the matrix exactly (each term rounds the running remainder), in the operand order
+    of the matrix-core quantise kernel: [term][row // 16][col // 32][(col % 32) // 8]
+    [row % 16][col % 8], i.e. the 64 lanes' 16-byte MFMA operands of one (row tile,
+    32-column slice) are contiguous.  d must be a multiple of 32."""
     rest = m.float()
+    d = rest.shape[0]
+    if rest.dim() != 2 or rest.shape[1] != d or d % 32:
+        raise ValueError("split_bf16x3 needs a square matrix whose size is a multiple of 32")
     parts = []
     for _ in range(3):
         term = rest.to(torch.bfloat16)
         parts.append(term)
         rest = rest - term.float()
-    return torch.stack(parts).contiguous().view(torch.int16)
+    t = torch.stack(parts).view(3, d // 16, 16, d // 32, 4, 8)      # term, row tile, n, kblk, kb, j
+    return t.permute(0, 1, 3, 4, 2, 5).contiguous().view(torch.int16)
 
 
 def make_page_layout(d: int, mse_bits: int, value_bits: int, group_size: int, dtype: torch.dtype) -> TqPageLayout:

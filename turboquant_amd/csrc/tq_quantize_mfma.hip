@@ -6,8 +6,8 @@
 // exact sum of three bf16 numbers (8 + 8 + 8 significand bits), so each operand is
 // split into bf16 terms and the product is assembled from bf16 MFMAs whose partial
 // products are exact; terms (a, b) with a + b > 2 are below fp32 resolution and are
-// skipped.  The matrices are split once per layer on the host; inputs that already
-// are bf16 need a single term.
+// skipped.  The matrices are split once per layer on the host and stored in the order
+// the MFMA operands are loaded in; inputs that already are bf16 need a single term.
 //
 // Workgroups (4 wavefronts) are persistent: two per compute unit (about 75 KB of LDS
 // each), each looping over groups of TT = 8192/d vectors (TT/16 tiles of 16).  The next
@@ -135,17 +135,21 @@ struct MatRegs {
   u32x4 b[BUF][KeyGeom<D>::NPW][3];
 };
 
-// m_terms: [term][D][D] bf16 in global memory, row n holds the coefficients of output n
+// m_terms: the three bf16 term matrices in MFMA-operand order.  For term b, tile of 16 output rows ct
+// and slice of 32 contraction indices kblk, the 64 lanes' 16-byte operands lie one after the other
+// (lane n + 16 kb holds M[16 ct + n][32 kblk + 8 kb ..+8]), so a wavefront's load of one operand is one
+// contiguous kilobyte.  (Row-major storage would make every quarter-wavefront touch 16 cache lines.)
 template <int D>
 __device__ __forceinline__ void load_slice(const uint16_t* __restrict__ m_terms, int wave, int lane, int kblk,
                                            u32x4 (&dst)[KeyGeom<D>::NPW][3]) {
   // one 32-bit per-lane byte offset; everything else is a uniform constant added to the base pointer
-  const uint32_t lane_off = (uint32_t)(((16 * wave * KeyGeom<D>::NPW + (lane & 15)) * D + 8 * (lane >> 4)) * 2);
+  constexpr int KB = KeyGeom<D>::KB, NPW = KeyGeom<D>::NPW;
+  const uint32_t lane_off = (uint32_t)((wave * NPW * KB * 64 + lane) * 16);
 #pragma unroll
-  for (int c = 0; c < KeyGeom<D>::NPW; ++c) {
+  for (int c = 0; c < NPW; ++c) {
 #pragma unroll
     for (int b = 0; b < 3; ++b) {
-      const char* base = (const char*)m_terms + ((size_t)(b * D + 16 * c) * D + 32 * kblk) * 2;
+      const char* base = (const char*)m_terms + ((size_t)(b * (D / 16) + c) * KB + kblk) * 1024;
       dst[c][b] = *(const u32x4*)(base + lane_off);
     }
   }

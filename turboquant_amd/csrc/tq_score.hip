@@ -358,17 +358,20 @@ score_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_sk, in
   for (int i = 0; i < nq; ++i) scores[(b * n_q + q0 + i) * n_k + k] = __fadd_rn(__fmul_rn(am[i], nk), __fmul_rn(aq[i], rk));
 }
 
-// x_hat for a tile of 16 vectors: (c[idx] Pi) * norm + (sigma S) * (qjl_scale * rnorm)
-// (quantizer.py:151-165, 259-272).  d threads, thread i owns output coordinate i.
+// x_hat for a tile of TILE vectors: (c[idx] Pi) * norm + (sigma S) * (qjl_scale * rnorm)
+// (quantizer.py:151-165, 259-272).  d threads, thread i owns output coordinate i and
+// sums over j in ascending order.  The tile's centroid and sign values sit in LDS as
+// [j][TILE] rows (padded by 4 floats) so one 16-byte broadcast read feeds four FMAs.
+template <int TILE, bool QJL>
 __global__ void __launch_bounds__(1024)
 dequant_keys_kernel(const uint8_t* __restrict__ idx, const uint8_t* __restrict__ signs, const void* __restrict__ norms,
                     int norm_dtype, const float* __restrict__ rnorms, int64_t n_vec, tq_layer ly,
                     float* __restrict__ out) {
-  constexpr int TILE = 16;
+  constexpr int LD = TILE + 4;
   extern __shared__ float sm[];
   const int d = ly.d, mb = ly.mse_bits, i = threadIdx.x;
-  float* sc = sm;               // [TILE][d] centroid values
-  float* ss = sm + TILE * d;    // [TILE][d] +-1
+  float* sc = sm;             // [d][LD] centroid values
+  float* ss = sm + LD * d;    // [d][LD] +-1
   const int eff = eff_bits(mb), per = 8 / eff, row = idx_row_bytes(d, mb), srow = d >> 3;
   const unsigned mask = (1u << eff) - 1u;
   const int64_t v0 = (int64_t)blockIdx.x * TILE;
@@ -378,31 +381,62 @@ dequant_keys_kernel(const uint8_t* __restrict__ idx, const uint8_t* __restrict__
     if (v < n_vec) {
       unsigned byte = idx[v * row + i / per];
       cv = ly.centroids[(byte >> (eff * (i % per))) & mask];
-      if (signs) sg = ((signs[v * srow + (i >> 3)] >> (i & 7)) & 1u) ? 1.0f : -1.0f;
+      if (QJL) sg = ((signs[v * srow + (i >> 3)] >> (i & 7)) & 1u) ? 1.0f : -1.0f;
     }
-    sc[t * d + i] = cv;
-    ss[t * d + i] = sg;
+    sc[i * LD + t] = cv;
+    if (QJL) ss[i * LD + t] = sg;
   }
   __syncthreads();
-  float a[TILE], b[TILE];
+  float a[TILE], b[QJL ? TILE : 1];
 #pragma unroll
-  for (int t = 0; t < TILE; ++t) a[t] = b[t] = 0.0f;
+  for (int t = 0; t < TILE; ++t) a[t] = 0.0f;
+#pragma unroll
+  for (int t = 0; t < (QJL ? TILE : 1); ++t) b[t] = 0.0f;
+#pragma unroll 2
   for (int j = 0; j < d; ++j) {
-    float pv = ly.Pi[(int64_t)j * d + i];
-    float sv = signs ? ly.S[(int64_t)j * d + i] : 0.0f;
+    const float pv = ly.Pi[(int64_t)j * d + i];
+    const float sv = QJL ? ly.S[(int64_t)j * d + i] : 0.0f;
 #pragma unroll
-    for (int t = 0; t < TILE; ++t) {
-      a[t] = fmaf(sc[t * d + j], pv, a[t]);
-      b[t] = fmaf(ss[t * d + j], sv, b[t]);
+    for (int t4 = 0; t4 < TILE / 4; ++t4) {
+      const float4 c = *reinterpret_cast<const float4*>(sc + j * LD + 4 * t4);
+      a[4 * t4 + 0] = fmaf(c.x, pv, a[4 * t4 + 0]);
+      a[4 * t4 + 1] = fmaf(c.y, pv, a[4 * t4 + 1]);
+      a[4 * t4 + 2] = fmaf(c.z, pv, a[4 * t4 + 2]);
+      a[4 * t4 + 3] = fmaf(c.w, pv, a[4 * t4 + 3]);
+      if (QJL) {
+        const float4 g = *reinterpret_cast<const float4*>(ss + j * LD + 4 * t4);
+        b[4 * t4 + 0] = fmaf(g.x, sv, b[4 * t4 + 0]);
+        b[4 * t4 + 1] = fmaf(g.y, sv, b[4 * t4 + 1]);
+        b[4 * t4 + 2] = fmaf(g.z, sv, b[4 * t4 + 2]);
+        b[4 * t4 + 3] = fmaf(g.w, sv, b[4 * t4 + 3]);
+      }
     }
   }
+#pragma unroll
   for (int t = 0; t < TILE; ++t) {
     int64_t v = v0 + t;
-    if (v >= n_vec) break;
-    float r = __fmul_rn(a[t], load_as_f32(norms, v, norm_dtype));
-    if (signs) r = __fadd_rn(r, __fmul_rn(b[t], __fmul_rn(ly.qjl_scale, rnorms[v])));
-    out[v * d + i] = r;
+    if (v < n_vec) {
+      float r = __fmul_rn(a[t], load_as_f32(norms, v, norm_dtype));
+      if (QJL) r = __fadd_rn(r, __fmul_rn(b[t], __fmul_rn(ly.qjl_scale, rnorms[v])));
+      out[v * d + i] = r;
+    }
   }
+}
+
+template <int TILE, bool QJL>
+static int launch_dequant_keys(const uint8_t* idx, const uint8_t* signs, const void* norms, int norm_dtype,
+                               const float* rnorms, int64_t n_vec, const tq_layer* layer, float* out, hipStream_t st) {
+  const int d = layer->d;
+  const size_t smem = (size_t)(QJL ? 2 : 1) * (TILE + 4) * d * sizeof(float);
+  auto kern = dequant_keys_kernel<TILE, QJL>;
+  if (smem > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) return (int)e;
+  }
+  kern<<<dim3((unsigned)((n_vec + TILE - 1) / TILE)), dim3(d), smem, st>>>(idx, signs, norms, norm_dtype, rnorms, n_vec,
+                                                                            *layer, out);
+  TQ_CHECK_LAUNCH();
+  return TQ_OK;
 }
 
 // fp32(code) * scale + zero with separately rounded multiply and add (kv_cache.py:101-116)
@@ -500,17 +534,14 @@ extern "C" int tq_dequant_keys(const uint8_t* idx, const uint8_t* signs, const v
   if (signs && !rnorms) return TQ_ENULL;
   if (n_vec < 0 || norm_dtype < TQ_F32 || norm_dtype > TQ_BF16) return TQ_EINVAL;
   if (n_vec == 0) return TQ_OK;
-  const int d = layer->d;
-  size_t smem = (size_t)2 * 16 * d * sizeof(float);
-  auto kern = dequant_keys_kernel;
-  if (smem > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    if (e != hipSuccess) return (int)e;
-  }
-  kern<<<dim3((unsigned)((n_vec + 15) / 16)), dim3(d), smem, (hipStream_t)stream>>>(idx, signs, norms, norm_dtype,
-                                                                                    rnorms, n_vec, *layer, out);
-  TQ_CHECK_LAUNCH();
-  return TQ_OK;
+  // 32 vectors per workgroup while both LDS tiles fit (d <= 512), else 16
+  hipStream_t st = (hipStream_t)stream;
+  const bool wide = layer->d <= 512;
+  if (signs)
+    return wide ? launch_dequant_keys<32, true>(idx, signs, norms, norm_dtype, rnorms, n_vec, layer, out, st)
+                : launch_dequant_keys<16, true>(idx, signs, norms, norm_dtype, rnorms, n_vec, layer, out, st);
+  return wide ? launch_dequant_keys<32, false>(idx, signs, norms, norm_dtype, rnorms, n_vec, layer, out, st)
+              : launch_dequant_keys<16, false>(idx, signs, norms, norm_dtype, rnorms, n_vec, layer, out, st);
 }
 
 extern "C" int tq_dequant_values(const uint8_t* data, const void* scales, const void* zeros, int dtype, int64_t n_vec,

@@ -117,8 +117,9 @@ class TurboQuantMSE(torch.nn.Module):
         key = (self.Pi.data_ptr(), self.Pi._version, None if S is None else (S.data_ptr(), S._version))
         if self._splits is None or self._splits[0] != key:
             self._PiT = self.Pi.T.contiguous()
-            self._splits = (key, (_ffi.split_bf16x3(self.Pi), _ffi.split_bf16x3(self._PiT),
-                                  None if S is None else _ffi.split_bf16x3(S)))
+            # only head_dim 128 / 256 have a matrix-core kernel; other sizes pass no split operands
+            mk = _ffi.split_bf16x3 if self.dim in (128, 256) else (lambda m: None)
+            self._splits = (key, (mk(self.Pi), mk(self._PiT), None if S is None else mk(S)))
         qc = None
         if S is not None:
             if getattr(self, "_query_consts", None) is None or self._query_consts[0] != key:
