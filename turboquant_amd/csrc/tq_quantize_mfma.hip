@@ -12,8 +12,8 @@
 // Workgroups (4 wavefronts) are persistent: two per compute unit (about 75 KB of LDS
 // each), each looping over groups of TT = 8192/d vectors (TT/16 tiles of 16).  The next
 // group's vectors are fetched into registers while the current group is worked on, and
-// the matrix operand of a contraction is requested before the epilogue of the previous
-// one, so no global-memory latency sits on the critical path.  The vectors' operand terms sit in LDS (row
+// the matrix operand of a contraction is requested slice by slice while the previous
+// contraction runs, so no global-memory latency sits on the critical path.  The vectors' operand terms sit in LDS (row
 // stride padded so that the 16 rows of an MFMA operand fall into different banks);
 // a wavefront owns d/64 column tiles of the output for all TT vectors, keeps the
 // matrix terms of the current 32-wide slice of the contraction in registers (next
@@ -126,9 +126,8 @@ struct KeySmem {
 };
 
 // Register copy of the matrix operand: BUF slices of 32 contraction indices for the
-// wavefront's column tiles.  head_dim 128 holds a whole contraction (BUF = KB), so the
-// loads for the next contraction are issued before the current epilogue starts and their
-// latency hides behind it; head_dim 256 keeps a ring that runs BUF - 1 slices ahead.
+// wavefront's column tiles.  head_dim 128 holds a whole contraction (BUF = KB); head_dim 256
+// keeps a ring that runs BUF - 1 slices ahead.
 template <int D>
 struct MatRegs {
   static constexpr int BUF = D == 128 ? 4 : 2;
@@ -165,9 +164,14 @@ __device__ __forceinline__ void prefetch_matrix(const uint16_t* __restrict__ m_t
 // a_terms tiles in LDS ([term][TT][RS] bf16); the first BUF slices of M are in `mr` already.
 // NA vector terms, 3 matrix terms, pairs with a + b <= 2.
 // acc[m][c][i] = out[16 m + (lane & 15)][16 (wave NPW + c) + 4 (lane >> 4) + i].
+// As soon as a slice's registers are free they are refilled: with a later slice of M while
+// there is one, then with the first BUF slices of m_next, the matrix of the contraction that
+// follows.  Those loads have the rest of this contraction and the epilogue to arrive, and
+// the requests of a workgroup are spread out instead of coming in one burst.
 template <int D, int NA>
-__device__ __forceinline__ void contract(const uint16_t* a_terms, const uint16_t* __restrict__ m_terms, int wave,
-                                         int lane, MatRegs<D>& mr, f32x4 (&acc)[KeyGeom<D>::MT][KeyGeom<D>::NPW]) {
+__device__ __forceinline__ void contract(const uint16_t* a_terms, const uint16_t* __restrict__ m_terms,
+                                         const uint16_t* __restrict__ m_next, int wave, int lane, MatRegs<D>& mr,
+                                         f32x4 (&acc)[KeyGeom<D>::MT][KeyGeom<D>::NPW]) {
   using Gm = KeyGeom<D>;
   constexpr int MT = Gm::MT, NPW = Gm::NPW, KB = Gm::KB, RS = Gm::RS, BUF = MatRegs<D>::BUF;
   const int n = lane & 15, kb = lane >> 4;
@@ -194,6 +198,7 @@ __device__ __forceinline__ void contract(const uint16_t* a_terms, const uint16_t
         }
     }
     if (kblk + BUF < KB) load_slice<D>(m_terms, wave, lane, kblk + BUF, mr.b[kblk % BUF]);
+    else load_slice<D>(m_next, wave, lane, kblk + BUF - KB, mr.b[kblk % BUF]);
   }
 }
 
@@ -337,8 +342,7 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
 
   f32x4 acc[MT][NPW];
   // (3) y = u Pi^T, bucketise; index bit planes; centroid values as bf16 terms for the next contraction
-  contract<D, NA1>(terms, ly.Pi_split, wave, lane, mr, acc);
-  prefetch_matrix<D>(mse_only ? ly.Pi_split : ly.PiT_split, wave, lane, mr);   // lands during the epilogue
+  contract<D, NA1>(terms, ly.Pi_split, mse_only ? ly.Pi_split : ly.PiT_split, wave, lane, mr, acc);
   __syncthreads();                                              // every wavefront has read the unit-vector terms
   {
     uint32_t idx[MT][NPW][4];
@@ -396,8 +400,7 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
   if (mse_only) issue_x(g + gridDim.x, tr, ck);
   if (!mse_only) {
     // (4) x_hat = (c Pi) * norm ; r = x - x_hat ; ||r||^2 partial sums ; r as bf16 terms (quantizer.py:241-245)
-    contract<D, 3>(terms, ly.PiT_split, wave, lane, mr, acc);
-    prefetch_matrix<D>(ly.S_split, wave, lane, mr);
+    contract<D, 3>(terms, ly.PiT_split, ly.S_split, wave, lane, mr, acc);
     __syncthreads();                                            // every wavefront has read the centroid terms
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
@@ -434,8 +437,7 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
       srn[tid] = sqrtf(v);
     }
     // (5) p = r S^T ; sign bits (quantizer.py:248-249)
-    contract<D, 3>(terms, ly.S_split, wave, lane, mr, acc);
-    prefetch_matrix<D>(ly.Pi_split, wave, lane, mr);            // for the next group
+    contract<D, 3>(terms, ly.S_split, ly.Pi_split, wave, lane, mr, acc);    // Pi again for the next group
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
       const int t = 16 * m + n;
