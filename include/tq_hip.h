@@ -53,13 +53,14 @@ typedef struct tq_layer {
   const float *centroids;  /* 2^mse_bits                                                    */
   const float *thresholds; /* 2^mse_bits - 1 interior boundaries (quantizer.py:127)         */
   float qjl_scale;         /* sqrt(pi/2)/d (quantizer.py:212)                               */
-  /* Optional operands of the matrix-core quantise kernel: Pi, its transpose and S, each
+  /* Optional operands of the matrix-core quantise / de-quantise kernels: Pi, its transpose, S and its transpose, each
    * written as the exact sum of three bf16 matrices (term t rounds what terms < t left),
    * raw bf16 bit patterns, 3*d*d each, stored in the order the kernel loads its MFMA
    * operands: element (row, col) of term t sits at
    *   ((((t*(d/16) + row/16)*(d/32) + col/32)*4 + (col%32)/8)*16 + row%16)*8 + col%8.
-   * NULL selects the vector-ALU kernel.                                              */
-  const uint16_t *Pi_split, *PiT_split, *S_split;
+   * ST_split (the transpose of S) serves the de-quantiser.  NULL selects the vector-ALU
+   * kernels.                                                                           */
+  const uint16_t *Pi_split, *PiT_split, *S_split, *ST_split;
   /* Optional constants of the fused query-preparation kernel of the decode path:
    * Pi_colsum[i] = sum_j Pi[j][i], S_colsum[i] = sum_j S[j][i] (d floats each) and the
    * largest row norm of S.  NULL selects the two-kernel preparation.                    */

@@ -184,6 +184,52 @@ def test_prod_dequant_and_score_on_reference_bytes(gpu, golden):
         assert (sc - ref).abs().max() <= 2e-5 * rms, case      # fp32 kernels sit far inside the gate
 
 
+@pytest.mark.parametrize("d,key_bits,n,dtype", [(128, 3, 1000, torch.bfloat16), (128, 2, 64, torch.float32),
+                                               (128, 4, 77, torch.float16), (128, 5, 129, torch.bfloat16),
+                                               (256, 3, 333, torch.bfloat16), (256, 5, 31, torch.float32)])
+def test_matrix_core_dequantiser_vs_double_precision_and_vector_kernel(gpu, d, key_bits, n, dtype):
+    """head_dim 128 / 256 de-quantise on the matrix cores.  Random codes (every code and sign value
+    occurs), ragged vector counts, all index widths: the result must sit within fp32 product-sum
+    accuracy of the float64 value of quantizer.py:259-272, and agree with the vector-ALU kernel
+    (taken when the output is not 16-byte aligned) to the same accuracy."""
+    import ctypes as C
+    from turboquant_amd import _ffi
+    from turboquant_amd.quantizer import MSEQuantized, ProdQuantized, TurboQuantProd
+    tq = TurboQuantProd(d, bits=key_bits, device=gpu)
+    prm = params_of(tq)
+    mb = key_bits - 1
+    g = torch.Generator().manual_seed(7 * d + key_bits)
+    idx = torch.randint(0, 1 << mb, (n, d), generator=g)
+    packed = O.pack_indices(idx, mb)
+    signs = torch.randint(0, 256, (n, d // 8), generator=g, dtype=torch.uint8)
+    norms = (torch.rand(n, generator=g) * 8 + 0.05).to(dtype)
+    rnorms = torch.rand(n, generator=g) * 3
+    _progress(f"dequant d={d} bits={key_bits} n={n} {dtype}")
+    code = ProdQuantized(packed.to(gpu), signs.to(gpu), rnorms.to(gpu), norms.to(gpu), mb)
+    got = tq.dequantize(code).cpu().double()
+    cent = prm.centroids.double()[idx]
+    sg = O.unpack_signs(signs, d).double()
+    want = (cent @ prm.Pi.double()) * norms.double()[:, None] + \
+        (sg @ prm.S.double()) * (float(np.float32(prm.qjl_scale)) * rnorms.double())[:, None]
+    scale = want.abs().max()
+    assert (got - want).abs().max() <= 2e-6 * scale
+    got_mse = tq.mse_quantizer.dequantize(MSEQuantized(packed.to(gpu), norms.to(gpu), mb)).cpu().double()
+    want_mse = (cent @ prm.Pi.double()) * norms.double()[:, None]
+    assert (got_mse - want_mse).abs().max() <= 2e-6 * want_mse.abs().max()
+    # the same call with an output that is only 4-byte aligned runs the vector-ALU kernel
+    buf = torch.empty(n * d + 1, dtype=torch.float32, device=gpu)
+    out = buf[1:]
+    ly = tq._layer()
+    with torch.cuda.device(gpu):
+        _ffi.check(_ffi.lib().tq_dequant_keys(code.mse_indices.data_ptr(), code.qjl_signs.data_ptr(),
+                                              code.norms.data_ptr(), _ffi.dtype_tag(dtype),
+                                              code.residual_norms.data_ptr(), n, C.byref(ly), out.data_ptr(),
+                                              _ffi.stream_ptr(torch.device(gpu))), "tq_dequant_keys")
+    valu = out.cpu().double().reshape(n, d)
+    assert (valu - want).abs().max() <= 2e-6 * scale
+    assert (valu - got).abs().max() <= 2e-6 * scale
+
+
 def test_config1_scores_on_reference_bytes_and_round_trip(gpu, golden):
     from turboquant_amd.quantizer import ProdQuantized
     z = golden.npz("config1_full")

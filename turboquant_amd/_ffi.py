@@ -32,7 +32,7 @@ class TqLayer(C.Structure):
         ("Pi", C.c_void_p), ("PiT", C.c_void_p), ("S", C.c_void_p), ("ST", C.c_void_p),
         ("centroids", C.c_void_p), ("thresholds", C.c_void_p),
         ("qjl_scale", C.c_float),
-        ("Pi_split", C.c_void_p), ("PiT_split", C.c_void_p), ("S_split", C.c_void_p),
+        ("Pi_split", C.c_void_p), ("PiT_split", C.c_void_p), ("S_split", C.c_void_p), ("ST_split", C.c_void_p),
         ("Pi_colsum", C.c_void_p), ("S_colsum", C.c_void_p), ("S_rownorm_max", C.c_float),
         ("n_terms", C.c_int32),
         ("term_mask", C.c_int32 * TQ_MAX_TERMS),
@@ -157,10 +157,11 @@ def make_layer(d: int, mse_bits: int, Pi: torch.Tensor, PiT: torch.Tensor, centr
     ly.centroids, ly.thresholds = centroids.data_ptr(), thresholds.data_ptr()
     ly.qjl_scale = math.sqrt(math.pi / 2.0) / d
     if splits is not None:
-        pi_s, pit_s, s_s = splits
+        pi_s, pit_s, s_s, st_s = splits
         ly.Pi_split = None if pi_s is None else pi_s.data_ptr()
         ly.PiT_split = None if pit_s is None else pit_s.data_ptr()
         ly.S_split = None if s_s is None else s_s.data_ptr()
+        ly.ST_split = None if st_s is None else st_s.data_ptr()
     if query_consts is not None:
         pi_cs, s_cs, s_max = query_consts
         ly.Pi_colsum, ly.S_colsum, ly.S_rownorm_max = pi_cs.data_ptr(), s_cs.data_ptr(), float(s_max)

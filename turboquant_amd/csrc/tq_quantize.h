@@ -159,4 +159,8 @@ __device__ __forceinline__ void write_key_tile_paged(const KeyPagedSink& sink, c
   }
 }
 
+// matrix-core de-quantiser (tq_quantize_mfma.hip); TQ_EUNSUPPORTED = use the vector-ALU kernel
+int launch_dequant_mfma(const uint8_t* idx, const uint8_t* signs, const void* norms, int norm_dtype, const float* rnorms,
+                        int64_t n_vec, const tq_layer& ly, float* out, hipStream_t st);
+
 }  // namespace tq

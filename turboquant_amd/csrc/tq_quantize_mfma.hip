@@ -601,6 +601,183 @@ int launch_key_mfma(const void* x, int dtype, const Source& src, const tq_layer&
   return TQ_EUNSUPPORTED;
 }
 
+// ------------------------------------------------------------------------------------
+// De-quantiser on the matrix cores: x_hat = (c[idx] Pi) * norm + (sigma S) * (qjl_scale * rnorm)
+// (quantizer.py:151-165, 259-272) with the machinery of the quantiser.  The centroid values of a
+// group of TT vectors go to LDS as three bf16 terms (exact), the signs as one (+-1 is a bf16 number),
+// the matrices are the split Pi^T and S^T (a row of the operand = an output coordinate), and the
+// products are exact with fp32 accumulation, so the result has the accuracy of an fp32 product sum.
+// ------------------------------------------------------------------------------------
+template <int D>
+struct DeqSmem {
+  using G = KeyGeom<D>;
+  static constexpr size_t off_terms = 0;                                        // [3][TT][RS] centroid terms
+  static constexpr size_t off_sign = 3 * (size_t)G::TT * G::RS * 2;             // [TT][RS] +-1
+  static constexpr size_t off_small = off_sign + (size_t)G::TT * G::RS * 2;     // snorm[TT] srn[TT] slut[16]
+  static constexpr size_t bytes = off_small + (size_t)G::TT * 8 + 16 * 8;
+};
+
+template <int D, bool QJL>
+__global__ void __launch_bounds__(KQ_THREADS, 2)
+dequant_mfma_kernel(const uint8_t* __restrict__ idx, const uint8_t* __restrict__ signs, const void* __restrict__ norms,
+                    int norm_dtype, const float* __restrict__ rnorms, int64_t n_vec, tq_layer ly,
+                    float* __restrict__ out) {
+  using Gm = KeyGeom<D>;
+  using Sm = DeqSmem<D>;
+  constexpr int TT = Gm::TT, MT = Gm::MT, NPW = Gm::NPW, RS = Gm::RS, TPR = Gm::TPR, SEG = Gm::SEG;
+  static_assert(SEG == 32, "a thread fills 32 coordinates: one word of sign bits");
+  const int tid0 = threadIdx.x, wave0 = __builtin_amdgcn_readfirstlane(tid0 >> 6);
+  const int mb = ly.mse_bits, eff = eff_bits(mb), row = idx_row_bytes(D, mb);
+  const int64_t n_groups = (n_vec + TT - 1) / TT;
+  MatRegs<D> mr;
+  prefetch_matrix<D>(ly.PiT_split, wave0, tid0 & 63, mr);
+
+  extern __shared__ __align__(16) unsigned char smem[];
+  uint16_t* terms = (uint16_t*)(smem + Sm::off_terms);
+  uint16_t* sgn = (uint16_t*)(smem + Sm::off_sign);
+  float* snorm = (float*)(smem + Sm::off_small);
+  float* srn = snorm + TT;
+  u32x2* slut = (u32x2*)(srn + TT);                             // bf16 terms of a centroid: {t0 | t1 << 16, t2}
+  if (tid0 < (1 << mb)) {
+    uint32_t t[3];
+    split3_pk(ly.centroids[tid0], 0.0f, t);
+    slut[tid0] = u32x2{(t[0] & 0xffffu) | (t[1] << 16), t[2] & 0xffffu};
+  }
+  // a thread holds the packed codes of its 32 coordinates of the NEXT group: eff index words, one sign word
+  const int t = tid0 / TPR, seg = tid0 % TPR;
+  uint32_t iw[4] = {0, 0, 0, 0}, sw = 0;
+  float nv = 0.0f, rv = 0.0f;
+  auto fetch = [&](int64_t g) {
+    const int64_t v = g * TT + t;
+    const int64_t vv = v < n_vec ? v : 0;                       // vectors that do not exist read the first one
+    const uint32_t* ip = (const uint32_t*)(idx + vv * row) + seg * eff;
+    iw[0] = ip[0];
+    if (eff >= 2) iw[1] = ip[1];
+    if (eff == 4) { iw[2] = ip[2]; iw[3] = ip[3]; }
+    if (QJL) sw = ((const uint32_t*)(signs + vv * (D / 8)))[seg];
+    if (seg == 0) {
+      nv = load_as_f32(norms, vv, norm_dtype);
+      if (QJL) rv = rnorms[vv];
+    }
+  };
+  if ((int64_t)blockIdx.x < n_groups) fetch(blockIdx.x);
+  __syncthreads();
+
+  for (int64_t g = blockIdx.x; g < n_groups; g += gridDim.x) {
+    int tid = tid0, wave = wave0;
+    asm volatile("" : "+v"(tid), "+s"(wave));
+    const int lane = tid & 63, n = lane & 15, kb = lane >> 4;
+    // (1) codes -> centroid terms and +-1 in LDS
+    auto fill = [&](auto eff_c) {
+      constexpr int EFF = decltype(eff_c)::value;
+      constexpr uint32_t mask = (1u << EFF) - 1u;
+#pragma unroll
+      for (int c8 = 0; c8 < SEG; c8 += 8) {
+        u32x2 e[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const int bit = (c8 + i) * EFF;
+          e[i] = slut[(iw[bit >> 5] >> (bit & 31)) & mask];
+        }
+        uint32_t pk[3][4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const u32x2 a = e[2 * i], b = e[2 * i + 1];
+          pk[0][i] = (a.x & 0xffffu) | (b.x << 16);
+          pk[1][i] = (a.x >> 16) | (b.x & 0xffff0000u);
+          pk[2][i] = a.y | (b.y << 16);
+        }
+#pragma unroll
+        for (int a = 0; a < 3; ++a)
+          *(u32x4*)(terms + ((size_t)a * TT + t) * RS + seg * SEG + c8) = u32x4{pk[a][0], pk[a][1], pk[a][2], pk[a][3]};
+      }
+    };
+    if (eff == 4) fill(std::integral_constant<int, 4>{});
+    else if (eff == 2) fill(std::integral_constant<int, 2>{});
+    else fill(std::integral_constant<int, 1>{});
+    if (QJL) {
+#pragma unroll
+      for (int c8 = 0; c8 < SEG; c8 += 8) {
+        uint32_t w[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const uint32_t b2 = sw >> (c8 + 2 * i);               // bit set = +1 (0x3f80), clear = -1 (0xbf80)
+          w[i] = 0xbf80bf80u ^ ((b2 & 1u) << 15) ^ ((b2 & 2u) << 30);
+        }
+        *(u32x4*)(sgn + (size_t)t * RS + seg * SEG + c8) = u32x4{w[0], w[1], w[2], w[3]};
+      }
+    }
+    if (seg == 0) {
+      snorm[t] = nv;
+      if (QJL) srn[t] = __fmul_rn(ly.qjl_scale, rv);
+    }
+    __syncthreads();
+    if (g + gridDim.x < n_groups) fetch(g + gridDim.x);         // lands while this group is contracted
+    // (2) contractions
+    f32x4 acc[MT][NPW], acq[QJL ? MT : 1][QJL ? NPW : 1];
+    contract<D, 3>(terms, ly.PiT_split, QJL ? ly.ST_split : ly.PiT_split, wave, lane, mr, acc);
+    if constexpr (QJL) contract<D, 1>(sgn, ly.ST_split, ly.PiT_split, wave, lane, mr, acq);
+    // (3) scale and store: a lane holds four consecutive coordinates of a vector
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+      const int tt = 16 * m + n;
+      const int64_t v = g * TT + tt;
+      if (v < n_vec) {
+        const float nrm = snorm[tt];
+        const float rn = QJL ? srn[tt] : 0.0f;
+#pragma unroll
+        for (int c = 0; c < NPW; ++c) {
+          f32x4 r;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            r[i] = __fmul_rn(acc[m][c][i], nrm);
+            if constexpr (QJL) r[i] = __fadd_rn(r[i], __fmul_rn(acq[m][c][i], rn));
+          }
+          *(f32x4*)(out + v * D + 16 * (wave * NPW + c) + 4 * kb) = r;
+        }
+      }
+    }
+    __syncthreads();                                            // the next group overwrites the tiles
+  }
+}
+
+template <int D, bool QJL>
+static int launch_deq_d(const uint8_t* idx, const uint8_t* signs, const void* norms, int norm_dtype, const float* rnorms,
+                        int64_t n_vec, const tq_layer& ly, float* out, hipStream_t st) {
+  using Sm = DeqSmem<D>;
+  auto kern = dequant_mfma_kernel<D, QJL>;
+  static std::atomic<unsigned long long> configured{0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return TQ_EINVAL;
+  if (dev >= 64 || !(configured.load() >> dev & 1)) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)Sm::bytes);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 64) configured.fetch_or(1ull << dev);
+  }
+  int n_cu = 0;
+  if (hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n_cu <= 0) n_cu = 256;
+  const int64_t groups = (n_vec + KeyGeom<D>::TT - 1) / KeyGeom<D>::TT;
+  const int64_t resident = (int64_t)n_cu * 2;
+  const unsigned grid = (unsigned)(groups < resident ? groups : resident);
+  kern<<<dim3(grid), dim3(KQ_THREADS), Sm::bytes, st>>>(idx, signs, norms, norm_dtype, rnorms, n_vec, ly, out);
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? TQ_OK : (int)e;
+}
+
+// TQ_EUNSUPPORTED when there is no matrix-core kernel for this call (head_dim other than 128 / 256,
+// no split matrices, or operands not aligned for word / 16-byte accesses).
+int launch_dequant_mfma(const uint8_t* idx, const uint8_t* signs, const void* norms, int norm_dtype, const float* rnorms,
+                        int64_t n_vec, const tq_layer& ly, float* out, hipStream_t st) {
+  if (!ly.PiT_split || (signs && !ly.ST_split)) return TQ_EUNSUPPORTED;
+  if (ly.mse_bits < 1 || ly.mse_bits > 4 || (ly.d != 128 && ly.d != 256)) return TQ_EUNSUPPORTED;
+  if ((uintptr_t)idx % 4 || (uintptr_t)signs % 4 || (uintptr_t)out % 16) return TQ_EUNSUPPORTED;
+  if (ly.d == 128)
+    return signs ? launch_deq_d<128, true>(idx, signs, norms, norm_dtype, rnorms, n_vec, ly, out, st)
+                 : launch_deq_d<128, false>(idx, signs, norms, norm_dtype, rnorms, n_vec, ly, out, st);
+  return signs ? launch_deq_d<256, true>(idx, signs, norms, norm_dtype, rnorms, n_vec, ly, out, st)
+               : launch_deq_d<256, false>(idx, signs, norms, norm_dtype, rnorms, n_vec, ly, out, st);
+}
+
 template int launch_key_mfma<FlatSource, KeyFlatSink>(const void*, int, const FlatSource&, const tq_layer&,
                                                       const KeyFlatSink&, int, int64_t, hipStream_t);
 template int launch_key_mfma<PagedSource, KeyPagedSink>(const void*, int, const PagedSource&, const tq_layer&,

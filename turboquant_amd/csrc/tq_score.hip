@@ -469,6 +469,10 @@ static int check_layer_rd(const tq_layer* ly, bool need_sketch) {
 }
 
 namespace tq {
+// matrix-core de-quantiser (tq_quantize_mfma.hip); TQ_EUNSUPPORTED = use the vector-ALU kernel
+int launch_dequant_mfma(const uint8_t* idx, const uint8_t* signs, const void* norms, int norm_dtype, const float* rnorms,
+                        int64_t n_vec, const tq_layer& ly, float* out, hipStream_t st);
+
 int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* layer, float* q_rot, float* q_sk,
                         float* q_stat, uint32_t* qa_pack, int G, float sm_scale, hipStream_t st) {
   const int d = layer->d;
@@ -534,8 +538,10 @@ extern "C" int tq_dequant_keys(const uint8_t* idx, const uint8_t* signs, const v
   if (signs && !rnorms) return TQ_ENULL;
   if (n_vec < 0 || norm_dtype < TQ_F32 || norm_dtype > TQ_BF16) return TQ_EINVAL;
   if (n_vec == 0) return TQ_OK;
-  // 32 vectors per workgroup while both LDS tiles fit (d <= 512), else 16
   hipStream_t st = (hipStream_t)stream;
+  rc = tq::launch_dequant_mfma(idx, signs, norms, norm_dtype, rnorms, n_vec, *layer, out, st);
+  if (rc != TQ_EUNSUPPORTED) return rc;
+  // vector-ALU kernel: 32 vectors per workgroup while both LDS tiles fit (d <= 512), else 16
   const bool wide = layer->d <= 512;
   if (signs)
     return wide ? launch_dequant_keys<32, true>(idx, signs, norms, norm_dtype, rnorms, n_vec, layer, out, st)

@@ -105,7 +105,7 @@ class TurboQuantMSE(torch.nn.Module):
         # kernel-side companions (not part of the reference's state dict)
         self.register_buffer("_PiT", self.Pi.T.contiguous(), persistent=False)
         self._centroids_host = centroids.detach().float().cpu()
-        self._splits = None           # (Pi, Pi^T[, S]) as bf16 term triples, built on first GPU use
+        self._splits = None           # (Pi, Pi^T[, S, S^T]) as bf16 term triples, built on first GPU use
 
     # -- library plumbing ---------------------------------------------------------
     def _layer(self, S: Optional[torch.Tensor] = None, ST: Optional[torch.Tensor] = None) -> _ffi.TqLayer:
@@ -119,7 +119,8 @@ class TurboQuantMSE(torch.nn.Module):
             self._PiT = self.Pi.T.contiguous()
             # only head_dim 128 / 256 have a matrix-core kernel; other sizes pass no split operands
             mk = _ffi.split_bf16x3 if self.dim in (128, 256) else (lambda m: None)
-            self._splits = (key, (mk(self.Pi), mk(self._PiT), None if S is None else mk(S)))
+            self._splits = (key, (mk(self.Pi), mk(self._PiT), None if S is None else mk(S),
+                                  None if ST is None else mk(ST)))
         qc = None
         if S is not None:
             if getattr(self, "_query_consts", None) is None or self._query_consts[0] != key:
