@@ -230,6 +230,40 @@ def test_matrix_core_dequantiser_vs_double_precision_and_vector_kernel(gpu, d, k
     assert (valu - got).abs().max() <= 2e-6 * scale
 
 
+@pytest.mark.parametrize("d,key_bits,n_q", [(128, 3, 4), (64, 2, 9), (256, 4, 3), (192, 5, 8)])
+def test_score_word_and_byte_kernels_agree_bit_for_bit(gpu, d, key_bits, n_q):
+    """tq_score reads a key's codes a word at a time when the index / sign rows are 4-byte aligned and a
+    byte at a time otherwise; both sum over the coordinates in the same order, so the logits are equal."""
+    import ctypes as C
+    from turboquant_amd import _ffi
+    from turboquant_amd.quantizer import TurboQuantProd
+    tq = TurboQuantProd(d, bits=key_bits, device=gpu)
+    g = torch.Generator(device=gpu).manual_seed(d + key_bits)
+    n_k = 333
+    code = tq.quantize(torch.randn(n_k, d, generator=g, device=gpu))
+    q = torch.randn(n_q, d, generator=g, device=gpu)
+    _progress(f"score kernels d={d} bits={key_bits} n_q={n_q}")
+    aligned = tq.attention_score(q, code)
+    # the same call on copies of the index and sign rows that start one byte into an allocation
+    ib = torch.empty(code.mse_indices.numel() + 1, dtype=torch.uint8, device=gpu)
+    sb = torch.empty(code.qjl_signs.numel() + 1, dtype=torch.uint8, device=gpu)
+    ib[1:] = code.mse_indices.reshape(-1)
+    sb[1:] = code.qjl_signs.reshape(-1)
+    scores = torch.empty(n_q, n_k, dtype=torch.float32, device=gpu)
+    work = torch.empty(2 * n_q * d, dtype=torch.float32, device=gpu)
+    rn = code.residual_norms.float().contiguous()
+    ly = tq._layer()
+    with torch.cuda.device(gpu):
+        _ffi.check(_ffi.lib().tq_score(q.data_ptr(), _ffi.dtype_tag(q.dtype), 1, n_q, ib[1:].data_ptr(),
+                                       sb[1:].data_ptr(), code.norms.data_ptr(), _ffi.dtype_tag(code.norms.dtype),
+                                       rn.data_ptr(), n_k, C.byref(ly), scores.data_ptr(), work.data_ptr(),
+                                       _ffi.stream_ptr(torch.device(gpu))), "tq_score")
+    assert torch.equal(scores, aligned)
+    ref = O.attention_score(q.cpu(), O.KeyCode(code.mse_indices.cpu(), code.qjl_signs.cpu(), code.residual_norms.cpu(),
+                                               code.norms.cpu(), key_bits - 1, None, None), params_of(tq))
+    assert (aligned.cpu() - ref).abs().max() <= 2e-5 * ref.pow(2).mean().sqrt()
+
+
 def test_config1_scores_on_reference_bytes_and_round_trip(gpu, golden):
     from turboquant_amd.quantizer import ProdQuantized
     z = golden.npz("config1_full")

@@ -307,13 +307,91 @@ prep_query_kernel(const void* __restrict__ q, int dtype, int G, tq_layer ly, flo
   }
 }
 
-// scores[b, i, k] for a tile of QT queries and one key per thread.
+// scores[b, i, k] for a tile of QT queries and one key per thread.  The rotated and sketched queries sit
+// in LDS as [coordinate][QT] rows, so a 16-byte broadcast read feeds four queries; a thread reads its key's
+// packed codes 32 coordinates (eff index words, one sign word) at a time.  NQ = 4 serves tiles of at most four
+// queries with half the work.  Each (query, key) sum runs over the coordinates in ascending order.
 constexpr int QT = 8;
+
+template <int NQ>
+__device__ __forceinline__ void score_accumulate(const float* s_rot, const float* s_sk, const float* s_cent, int d,
+                                                 int eff, const uint32_t* ip, const uint32_t* sp, float (&am)[QT],
+                                                 float (&aq)[QT]) {
+  const unsigned mask = (1u << eff) - 1u;
+  for (int c0 = 0; c0 < d; c0 += 32) {
+    uint32_t iw[4] = {0, 0, 0, 0};
+    const uint32_t* w = ip + (c0 >> 5) * eff;
+    iw[0] = w[0];
+    if (eff >= 2) iw[1] = w[1];
+    if (eff == 4) { iw[2] = w[2]; iw[3] = w[3]; }
+    const uint32_t sb = sp[c0 >> 5];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {                    // index word j of this run: 32 / eff coordinates
+      const int per_w = 32 / eff;
+      if (j * per_w >= 32) break;
+      for (int s = 0; s < per_w; ++s) {
+        const int cl = j * per_w + s, c = c0 + cl;
+        const float cv = s_cent[(iw[j] >> (eff * s)) & mask];
+        const float sg = ((sb >> cl) & 1u) ? 1.0f : -1.0f;
+#pragma unroll
+        for (int i4 = 0; i4 < NQ / 4; ++i4) {
+          const float4 r = *reinterpret_cast<const float4*>(s_rot + c * QT + 4 * i4);
+          const float4 k = *reinterpret_cast<const float4*>(s_sk + c * QT + 4 * i4);
+          am[4 * i4 + 0] = fmaf(r.x, cv, am[4 * i4 + 0]);
+          am[4 * i4 + 1] = fmaf(r.y, cv, am[4 * i4 + 1]);
+          am[4 * i4 + 2] = fmaf(r.z, cv, am[4 * i4 + 2]);
+          am[4 * i4 + 3] = fmaf(r.w, cv, am[4 * i4 + 3]);
+          aq[4 * i4 + 0] = fmaf(k.x, sg, aq[4 * i4 + 0]);
+          aq[4 * i4 + 1] = fmaf(k.y, sg, aq[4 * i4 + 1]);
+          aq[4 * i4 + 2] = fmaf(k.z, sg, aq[4 * i4 + 2]);
+          aq[4 * i4 + 3] = fmaf(k.w, sg, aq[4 * i4 + 3]);
+        }
+      }
+    }
+  }
+}
 
 __global__ void __launch_bounds__(256)
 score_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_sk, int64_t n_q,
              const uint8_t* __restrict__ idx, const uint8_t* __restrict__ signs, const void* __restrict__ norms,
              int norm_dtype, const float* __restrict__ rnorms, int64_t n_k, tq_layer ly, float* __restrict__ scores) {
+  extern __shared__ __align__(16) float sm[];
+  const int d = ly.d, mb = ly.mse_bits;
+  float* s_rot = sm;              // [d][QT]
+  float* s_sk = sm + QT * d;      // [d][QT]
+  float* s_cent = s_sk + QT * d;  // [16]
+  const int64_t b = blockIdx.z;
+  const int64_t q0 = (int64_t)blockIdx.y * QT;
+  const int nq = (int)((n_q - q0) < QT ? (n_q - q0) : QT);
+  for (int o = threadIdx.x; o < QT * d; o += blockDim.x) {
+    int i = o / d, c = o - i * d;
+    bool ok = i < nq;
+    s_rot[c * QT + i] = ok ? q_rot[(b * n_q + q0) * d + o] : 0.0f;
+    s_sk[c * QT + i] = ok ? q_sk[(b * n_q + q0) * d + o] : 0.0f;
+  }
+  if (threadIdx.x < (1 << mb)) s_cent[threadIdx.x] = ly.centroids[threadIdx.x];
+  __syncthreads();
+  const int64_t k = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (k >= n_k) return;
+  const int eff = eff_bits(mb), row = idx_row_bytes(d, mb), srow = d >> 3;
+  const uint32_t* ip = (const uint32_t*)(idx + (b * n_k + k) * row);
+  const uint32_t* sp = (const uint32_t*)(signs + (b * n_k + k) * srow);
+  float am[QT], aq[QT];
+#pragma unroll
+  for (int i = 0; i < QT; ++i) am[i] = aq[i] = 0.0f;
+  if (nq <= 4) score_accumulate<4>(s_rot, s_sk, s_cent, d, eff, ip, sp, am, aq);
+  else score_accumulate<8>(s_rot, s_sk, s_cent, d, eff, ip, sp, am, aq);
+  const float nk = load_as_f32(norms, b * n_k + k, norm_dtype);
+  const float rk = __fmul_rn(ly.qjl_scale, rnorms[b * n_k + k]);
+  for (int i = 0; i < nq; ++i) scores[(b * n_q + q0 + i) * n_k + k] = __fadd_rn(__fmul_rn(am[i], nk), __fmul_rn(aq[i], rk));
+}
+
+// the same sums with byte loads, for index / sign rows that are not 4-byte aligned
+__global__ void __launch_bounds__(256)
+score_bytes_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_sk, int64_t n_q,
+                   const uint8_t* __restrict__ idx, const uint8_t* __restrict__ signs, const void* __restrict__ norms,
+                   int norm_dtype, const float* __restrict__ rnorms, int64_t n_k, tq_layer ly,
+                   float* __restrict__ scores) {
   extern __shared__ float sm[];
   const int d = ly.d, mb = ly.mse_bits;
   float* s_rot = sm;              // [QT][d]
@@ -455,6 +533,36 @@ __global__ void dequant_values_kernel(const uint8_t* __restrict__ data, const vo
   out[gid] = __fadd_rn(__fmul_rn(code, s), z);
 }
 
+// The same arithmetic, a thread per 8 consecutive channels (they share a group when the group size is a
+// multiple of 8): one load of the packed codes, scale and zero read once, two 16-byte stores.
+template <int BITS>
+__global__ void dequant_values8_kernel(const uint8_t* __restrict__ data, const void* __restrict__ scales,
+                                       const void* __restrict__ zeros, int dtype, int64_t n_vec, int d, int gs,
+                                       float* __restrict__ out) {
+  const int64_t gid = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;      // chunk of 8 channels
+  const int cpv = d >> 3;
+  if (gid >= n_vec * cpv) return;
+  const int64_t v = gid / cpv;
+  const int c0 = (int)(gid - v * cpv) * 8;
+  const int ng = d / gs;
+  const uint8_t* src = data + v * (d * BITS / 8) + c0 * BITS / 8;
+  uint64_t bits64;
+  if (BITS == 2) bits64 = *(const uint16_t*)src;
+  else if (BITS == 4) bits64 = *(const uint32_t*)src;
+  else bits64 = *(const uint64_t*)src;
+  const float sc = load_as_f32(scales, v * ng + c0 / gs, dtype);
+  const float z = load_as_f32(zeros, v * ng + c0 / gs, dtype);
+  float r[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float code = (float)(uint32_t)((bits64 >> (BITS * i)) & ((1u << BITS) - 1u));
+    r[i] = __fadd_rn(__fmul_rn(code, sc), z);
+  }
+  float4* dst = (float4*)(out + v * d + c0);
+  dst[0] = make_float4(r[0], r[1], r[2], r[3]);
+  dst[1] = make_float4(r[4], r[5], r[6], r[7]);
+}
+
 }  // namespace tq
 
 using namespace tq;
@@ -524,8 +632,12 @@ extern "C" int tq_score(const void* q, int dtype, int64_t batch, int64_t n_q, co
   if (rc) return rc;
   dim3 grid((unsigned)((n_k + 255) / 256), (unsigned)((n_q + QT - 1) / QT), (unsigned)batch);
   size_t smem = (2 * QT * d + 16) * sizeof(float);
-  score_kernel<<<grid, dim3(256), smem, (hipStream_t)stream>>>(q_rot, q_sk, n_q, idx, signs, norms, norm_dtype, rnorms,
-                                                              n_k, *layer, scores);
+  if ((uintptr_t)idx % 4 == 0 && (uintptr_t)signs % 4 == 0)
+    score_kernel<<<grid, dim3(256), smem, (hipStream_t)stream>>>(q_rot, q_sk, n_q, idx, signs, norms, norm_dtype,
+                                                                rnorms, n_k, *layer, scores);
+  else
+    score_bytes_kernel<<<grid, dim3(256), smem, (hipStream_t)stream>>>(q_rot, q_sk, n_q, idx, signs, norms,
+                                                                      norm_dtype, rnorms, n_k, *layer, scores);
   TQ_CHECK_LAUNCH();
   return TQ_OK;
 }
@@ -557,6 +669,18 @@ extern "C" int tq_dequant_values(const uint8_t* data, const void* scales, const 
   if (d <= 0 || group_size <= 0 || d % group_size || (d * bits) % 8 || n_vec < 0) return TQ_EINVAL;
   if (dtype < TQ_F32 || dtype > TQ_BF16) return TQ_EINVAL;
   if (n_vec == 0) return TQ_OK;
+  hipStream_t st = (hipStream_t)stream;
+  // chunks of 8 channels when they stay inside a group and the accesses are aligned
+  const int cb = bits;                                          // bytes of codes per chunk
+  if (d % 8 == 0 && group_size % 8 == 0 && (uintptr_t)data % cb == 0 && (uintptr_t)out % 16 == 0) {
+    const int64_t chunks = n_vec * (d / 8);
+    const dim3 grid((unsigned)((chunks + 255) / 256)), block(256);
+    if (bits == 2) dequant_values8_kernel<2><<<grid, block, 0, st>>>(data, scales, zeros, dtype, n_vec, d, group_size, out);
+    else if (bits == 4) dequant_values8_kernel<4><<<grid, block, 0, st>>>(data, scales, zeros, dtype, n_vec, d, group_size, out);
+    else dequant_values8_kernel<8><<<grid, block, 0, st>>>(data, scales, zeros, dtype, n_vec, d, group_size, out);
+    TQ_CHECK_LAUNCH();
+    return TQ_OK;
+  }
   int64_t total = n_vec * d;
   dequant_values_kernel<<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream>>>(
       data, scales, zeros, dtype, n_vec, d, group_size, bits, out);
