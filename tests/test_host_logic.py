@@ -33,6 +33,28 @@ def test_library_exports_every_declared_symbol():
     assert lib.tq_version() == _ffi.ABI_VERSION
 
 
+@pytest.mark.parametrize("d", [128, 256])
+def test_split_matrices_sum_exactly_and_follow_the_documented_operand_order(d):
+    """The three bf16 terms of a split matrix add up to the fp32 matrix bit for bit, and element
+    (row, col) of term t sits where include/tq_hip.h says the matrix-core kernels read it."""
+    g = torch.Generator().manual_seed(d)
+    m = torch.randn(d, d, generator=g) * torch.logspace(-6, 2, d)[None, :]
+    raw = _ffi.split_bf16x3(m)
+    assert raw.dtype == torch.int16 and raw.numel() == 3 * d * d
+    flat = raw.reshape(-1).view(torch.bfloat16).float()
+    t, r, c = torch.meshgrid(torch.arange(3), torch.arange(d), torch.arange(d), indexing="ij")
+    pos = ((((t * (d // 16) + r // 16) * (d // 32) + c // 32) * 4 + (c % 32) // 8) * 16 + r % 16) * 8 + c % 8
+    assert torch.equal(torch.sort(pos.reshape(-1)).values, torch.arange(3 * d * d))       # a permutation
+    terms = flat[pos]                                                                       # (3, d, d) row-major
+    want = m.clone()
+    for k in range(3):                       # each term is the bf16 rounding of what the terms before it left
+        assert torch.equal(terms[k], want.to(torch.bfloat16).float())
+        want = want - terms[k]
+    assert torch.equal(terms[0] + terms[1] + terms[2], m)
+    with pytest.raises(ValueError):
+        _ffi.split_bf16x3(torch.zeros(48, 48))
+
+
 def test_argument_errors_are_reported_before_any_launch():
     lib = _ffi.lib()
     assert lib.tq_bucketize_pack(None, 4, 128, None, 2, None, None) == -3
