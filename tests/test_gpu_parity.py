@@ -613,6 +613,39 @@ def test_decode_split_invariance_and_page_permutation(gpu):
     assert torch.equal(o2, outs[1])
 
 
+def test_decode_one_million_token_context_against_dense_attention_on_the_dequantised_cache(gpu):
+    """The largest context of the size table: one sequence of 2^20 tokens (65,536 pages, appended in four
+    chunks at growing start positions).  Size-independent checks: the result does not depend on the split
+    count, and it equals dense fp32 attention over the de-quantised keys and values (score.py:117-173),
+    which the flat entry points produce from the exported pages."""
+    from turboquant_amd.kv_cache import ValueQuantized, dequantize_values
+    from turboquant_amd.quantizer import ProdQuantized
+    g = torch.Generator(device=gpu).manual_seed(21)
+    d, Hkv, Hq, N = 128, 1, 4, 1 << 20
+    pool, tq = _make_pool(gpu, d, 3, 2, Hkv, N // 16)
+    table = torch.randperm(N // 16, generator=g, device=gpu).to(torch.int32)[None]
+    chunk = N // 4
+    for c in range(4):
+        _progress(f"1M context: append chunk {c}")
+        k = torch.randn(1, chunk, Hkv, d, generator=g, device=gpu).bfloat16()
+        v = torch.randn(1, chunk, Hkv, d, generator=g, device=gpu).bfloat16()
+        pool.append(k, v, table, start_pos=torch.tensor([c * chunk], dtype=torch.int32))
+    q = (torch.randn(1, Hq, d, generator=g, device=gpu) * 3).bfloat16()
+    seq = torch.tensor([N - 5], dtype=torch.int32, device=gpu)
+    outs = [pool.decode_attention(q, table, seq, n_split=s, max_len=N).float() for s in (64, 512, 7)]
+    for o in outs[1:]:
+        assert (o - outs[0]).abs().max() <= 2 ** -7 * outs[0].abs().max()
+    n = N - 5
+    idx, sgn, norms, rn, vd, vs, vz = pool.export_flat(table[0], n)
+    khat = tq.dequantize(ProdQuantized(idx[0], sgn[0], rn[0], norms[0], 2))             # (n, d) fp32
+    vhat = dequantize_values(ValueQuantized(vd[0], vs[0], vz[0], 2), 32).float()         # (n, d)
+    logits = (q[0].float() @ khat.T) / math.sqrt(d)                                      # (Hq, n)
+    want = torch.softmax(logits, dim=-1) @ vhat
+    cos = cosine(outs[0][0].cpu(), want.cpu())
+    _progress(f"1M context: cosine vs dense attention on the de-quantised cache {cos:.7f}")
+    assert cos >= 0.9999
+
+
 def test_page_kernel_timing_hook_times_one_dispatch_and_changes_nothing(gpu):
     # tq_time_next_page_kernel attaches an event pair to the next page-kernel dispatch of this thread:
     # the elapsed time is positive and below the bracketing stream markers', the hook disarms itself,
