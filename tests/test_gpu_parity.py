@@ -591,6 +591,34 @@ def test_decode_attention_ragged_empty_and_hybrid_tail(gpu):
     worst = _decode_case(gpu, 128, 3, 2, 2, 4, 2, [0, 64], None, seed=79)            # one row has nothing at all
 
 
+def test_pool_export_word_and_byte_kernels_agree(gpu):
+    """tq_pool_export writes the flat tensors a word at a time; outputs that are not 4-byte aligned take the
+    byte-wise kernel.  Both must give the same bytes (ragged token count, permuted pages, every value width)."""
+    import ctypes as C
+    from turboquant_amd import _ffi
+    for d, key_bits, vb in [(128, 3, 2), (256, 4, 4), (64, 2, 2), (128, 5, 4)]:
+        g = torch.Generator().manual_seed(d + vb)
+        H, n_tok = 2, 75
+        pool, tq = _make_pool(gpu, d, key_bits, vb, H, 8)
+        table = torch.randperm(8, generator=g).to(torch.int32)[None].to(gpu)
+        k = torch.randn(1, n_tok, H, d, generator=g).bfloat16().to(gpu)
+        v = torch.randn(1, n_tok, H, d, generator=g).bfloat16().to(gpu)
+        pool.append(k, v, table)
+        _progress(f"export kernels d={d} key_bits={key_bits} vb={vb}")
+        idx, sgn, norms, rn, vd, vs, vz = pool.export_flat(table[0], n_tok)
+        bufs = [torch.zeros(t.numel() + 1, dtype=torch.uint8, device=gpu) for t in (idx, sgn, vd)]
+        norms2, rn2, vs2, vz2 = [torch.zeros_like(t) for t in (norms, rn, vs, vz)]
+        with torch.cuda.device(gpu):
+            _ffi.check(_ffi.lib().tq_pool_export(
+                pool.data.data_ptr(), pool.num_pages, H, table[0].contiguous().data_ptr(), n_tok, C.byref(pool.layout),
+                bufs[0][1:].data_ptr(), bufs[1][1:].data_ptr(), norms2.data_ptr(), rn2.data_ptr(), bufs[2][1:].data_ptr(),
+                vs2.data_ptr(), vz2.data_ptr(), _ffi.stream_ptr(torch.device(gpu))), "tq_pool_export")
+        for got, want in zip(bufs, (idx, sgn, vd)):
+            assert torch.equal(got[1:], want.reshape(-1))
+        for got, want in ((norms2, norms), (rn2, rn), (vs2, vs), (vz2, vz)):
+            assert torch.equal(got.view(torch.uint8), want.view(torch.uint8))
+
+
 def test_decode_split_invariance_and_page_permutation(gpu):
     from turboquant_amd.paged import PagedKVPool
     g = torch.Generator().manual_seed(5)

@@ -471,6 +471,75 @@ __device__ __forceinline__ void copy_elem(void* dst, int64_t di, const void* src
   else ((uint16_t*)dst)[di] = ((const uint16_t*)src)[si];
 }
 
+// The same export a word at a time: a workgroup per (page, head); index words are assembled from the
+// bit planes with bit-spreading steps, sign words are copied, value codes are gathered from the page's
+// per-channel fields through LDS.  Needs 4-byte aligned outputs (rows are multiples of 4 bytes because
+// head_dim is a multiple of 64).
+__global__ void __launch_bounds__(256)
+pool_export_words_kernel(const uint8_t* __restrict__ pool, int H, const int32_t* __restrict__ block_table, int n_tok,
+                         tq_page_layout L, uint32_t* __restrict__ idx, uint32_t* __restrict__ signs, void* norms,
+                         float* rnorms, uint32_t* __restrict__ v_data, void* v_scales, void* v_zeros) {
+  extern __shared__ __align__(16) uint32_t s_fields[];          // the page's value section, d * 2 vb bytes
+  const int d = L.d, mb = L.mse_bits, vb = L.value_bits, ng = d / L.group_size, W = d >> 5;
+  const int lpage = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  const uint8_t* pg = pool + ((int64_t)block_table[lpage] * H + h) * (int64_t)L.page_bytes;
+  const int n_valid = min(TILE, n_tok - lpage * TILE);
+  const int64_t flat0 = (int64_t)h * n_tok + (int64_t)lpage * TILE;
+  const int field_dw = vb >> 1;                                  // dwords per channel field (16 * vb bits)
+  for (int o = tid; o < d * field_dw; o += blockDim.x) s_fields[o] = ((const uint32_t*)(pg + L.off_vdata))[o];
+  // keys: dword k of a row holds 32 / eff codes, code s at bit eff * s, plane 0 the top bit of a code
+  const int eff = eff_bits(mb), n_per = 32 / eff, row_dw = idx_row_bytes(d, mb) >> 2;
+  for (int o = tid; o < n_valid * row_dw; o += blockDim.x) {
+    const int t = o / row_dw, k = o - t * row_dw, c0 = k * n_per;
+    uint32_t dw = 0;
+    for (int p = 0; p < mb; ++p) {
+      uint32_t x = *(const uint32_t*)(pg + key_word_off(L, p, c0 >> 5, t)) >> (c0 & 31);
+      if (eff == 2) {
+        x &= 0xffffu;
+        x = (x | (x << 8)) & 0x00ff00ffu;
+        x = (x | (x << 4)) & 0x0f0f0f0fu;
+        x = (x | (x << 2)) & 0x33333333u;
+        x = (x | (x << 1)) & 0x55555555u;
+      } else if (eff == 4) {
+        x &= 0xffu;
+        x = (x | (x << 12)) & 0x000f000fu;
+        x = (x | (x << 6)) & 0x03030303u;
+        x = (x | (x << 3)) & 0x11111111u;
+      }
+      dw |= x << (mb - 1 - p);
+    }
+    idx[(flat0 + t) * row_dw + k] = dw;
+  }
+  for (int o = tid; o < n_valid * W; o += blockDim.x) {
+    const int t = o / W, w = o - t * W;
+    signs[(flat0 + t) * W + w] = *(const uint32_t*)(pg + key_word_off(L, mb, w, t));
+  }
+  for (int o = tid; o < n_valid * ng; o += blockDim.x) {
+    const int t = o / ng, g = o - t * ng;
+    copy_elem(v_scales, (flat0 + t) * ng + g, pg + L.off_vscale, g * TILE + t, L.dtype);
+    copy_elem(v_zeros, (flat0 + t) * ng + g, pg + L.off_vzero, g * TILE + t, L.dtype);
+  }
+  if (tid < n_valid) {
+    store_from_f32(norms, flat0 + tid, ((const float*)(pg + L.off_meta))[2 * tid], L.dtype);
+    rnorms[flat0 + tid] = ((const float*)(pg + L.off_meta))[2 * tid + 1];
+  }
+  __syncthreads();
+  // values: dword j of a token's row holds 32 / vb channels; channel c's code sits at bit vb * t of its field
+  const int cpd = 32 / vb, vrow_dw = (d * vb) >> 5;
+  const uint32_t vmask = vb == 8 ? 0xffu : (1u << vb) - 1u;
+  for (int o = tid; o < n_valid * vrow_dw; o += blockDim.x) {
+    const int t = o / vrow_dw, j = o - t * vrow_dw;
+    const int bit = vb * t;
+    uint32_t dw = 0;
+    for (int i = 0; i < cpd; ++i) {
+      const int c = j * cpd + i;
+      const int f = ((c & 15) * (d >> 4) + (c >> 4)) * field_dw;             // vfield_off in dwords
+      dw |= ((s_fields[f + (bit >> 5)] >> (bit & 31)) & vmask) << (vb * i);
+    }
+    v_data[(flat0 + t) * vrow_dw + j] = dw;
+  }
+}
+
 __global__ void pool_export_kernel(const uint8_t* __restrict__ pool, int H, const int32_t* __restrict__ block_table,
                                    int n_tok, tq_page_layout L, uint8_t* idx, uint8_t* signs, void* norms,
                                    float* rnorms, uint8_t* v_data, void* v_scales, void* v_zeros) {
@@ -784,6 +853,17 @@ extern "C" int tq_pool_export(const uint8_t* pool, int64_t num_pages, int H, con
     return TQ_ENULL;
   if (H <= 0 || n_tok < 0 || num_pages <= 0) return TQ_EINVAL;
   if (n_tok == 0) return TQ_OK;
+  const tq_page_layout& L = *layout;
+  if ((L.value_bits == 2 || L.value_bits == 4 || L.value_bits == 8) && L.d % 64 == 0 && L.off_vdata % 4 == 0 &&
+      (uintptr_t)idx % 4 == 0 && (uintptr_t)signs % 4 == 0 && (uintptr_t)v_data % 4 == 0) {
+    dim3 g2((n_tok + TILE - 1) / TILE, H), b2(256);
+    const size_t sm = (size_t)L.d * 2 * L.value_bits;
+    pool_export_words_kernel<<<g2, b2, sm, (hipStream_t)stream>>>(pool, H, block_table, n_tok, L, (uint32_t*)idx,
+                                                                 (uint32_t*)signs, norms, rnorms, (uint32_t*)v_data,
+                                                                 v_scales, v_zeros);
+    TQ_CHECK_LAUNCH();
+    return TQ_OK;
+  }
   dim3 grid((n_tok + TILE - 1) / TILE, H), block(64);
   pool_export_kernel<<<grid, block, 0, (hipStream_t)stream>>>(pool, H, block_table, n_tok, *layout, idx, signs, norms,
                                                              rnorms, v_data, v_scales, v_zeros);
