@@ -254,3 +254,118 @@ def test_hybrid_decode_through_the_hooks_matches_the_oracle(gpu):
             assert cosine(out[0].float().cpu(), exact[0].float().cpu()) > 0.9
         # the ring spilled nothing yet (128 + 3 decode tokens -> one drain of 128 at the 129th)
         assert state.engine.total_tokens == T + 3
+
+
+# ------------------------------------------------------------------ batch-aware hooks + minimal transformer
+def test_dense_backend_of_the_harness_is_plain_causal_attention():
+    """The harness' exact backend over a shuffled paged cache equals causal attention computed directly,
+    for a ragged batch fed in two chunks."""
+    from turboquant_amd.integration.harness import MinimalRunner
+    r = MinimalRunner(n_layers=1, hidden=64, num_heads=4, num_kv_heads=2, head_dim=16, ffn=64, vocab=50, batch=2,
+                      max_seq_len=64, device="cpu", dtype=torch.float32)
+    impl, cache = r.layers[0].attn.impl, r.layers[0].attn.kv_cache[0]
+    g = torch.Generator().manual_seed(0)
+    ks, vs, outs, qs = [[], []], [[], []], [[], []], [[], []]
+    for new in ([20, 7], [5, 30]):
+        meta = r.metadata(new)
+        T = sum(new)
+        q, k, v = torch.randn(T, 4 * 16, generator=g), torch.randn(T, 2, 16, generator=g), torch.randn(T, 2, 16, generator=g)
+        impl.do_kv_cache_update(None, k, v, cache, meta.slot_mapping)
+        o = impl.forward(None, q, k, v, cache, meta)
+        r.seq_lens = meta.seq_lens_cpu.tolist()
+        row = 0
+        for b, t in enumerate(new):
+            ks[b].append(k[row:row + t]); vs[b].append(v[row:row + t]); qs[b].append(q[row:row + t]); outs[b].append(o[row:row + t])
+            row += t
+    for b in range(2):
+        K, V = torch.cat(ks[b]).repeat_interleave(2, 1), torch.cat(vs[b]).repeat_interleave(2, 1)
+        Q = torch.cat(qs[b]).view(-1, 4, 16)
+        s = torch.einsum("thd,nhd->htn", Q, K) / 4.0
+        L = K.shape[0]
+        s = s.masked_fill((torch.arange(L)[None] > torch.arange(L)[:, None])[None], float("-inf"))
+        want = torch.einsum("htn,nhd->thd", s.softmax(-1), V).reshape(L, -1)
+        assert torch.allclose(torch.cat(outs[b]), want, atol=1e-5)
+
+
+@pytest.mark.gpu
+def test_batched_hooks_through_the_minimal_transformer(gpu):
+    """A ragged batch through every layer of the minimal transformer with the batch-aware hooks: the pools
+    hold exactly what quantising each sequence's K/V in one go gives (chunked prefill + decode appends),
+    decode attention from the pool matches the oracle on the exported pages (full and hybrid), and the
+    logits stay close to the exact model's."""
+    from oracle import tq_oracle as O
+    from tests.helpers import cosine, key_code, params_of, value_code
+    from turboquant_amd.integration import batched
+    from turboquant_amd.integration.harness import BLOCK, MinimalRunner
+    from turboquant_amd.kv_cache import quantize_values
+    dev = torch.device("cuda:0")
+    mk = lambda: MinimalRunner(n_layers=3, hidden=256, num_heads=8, num_kv_heads=2, head_dim=128, ffn=512, vocab=1000,
+                               batch=3, max_seq_len=400, device=dev, seed=3)
+    ra, rb = mk(), mk()                                   # rb: the same weights, no hooks
+    st = batched.install_batched_hooks(ra, num_blocks=ra.num_blocks, key_bits=3, value_bits=4, ring_capacity=32,
+                                       initial_layers_count=1, mode=hooks.MODE_CAPTURE_ONLY)
+    assert len(st) == 3 and [s.config.key_bits for s in st.values()] == [4, 3, 3]
+    g = torch.Generator().manual_seed(11)
+    for new in ([200, 45, 130], [100, 0, 0]):             # second step: sequence 0 continues, the others idle
+        toks = torch.randint(0, 1000, (sum(new),), generator=g).to(dev)
+        la = ra.step(toks, ra.metadata(new))
+        lb = rb.step(toks, rb.metadata(new))
+        assert torch.equal(la, lb)                        # capture mode: the backend answered
+    hooks.set_mode(hooks.MODE_FULL_TQ)
+    for step in range(3):
+        toks = torch.randint(0, 1000, (3,), generator=g).to(dev)
+        la, lb = ra.decode_step(toks), rb.decode_step(toks)
+        cos = min(cosine(la[b].float().cpu(), lb[b].float().cpu()) for b in range(3))
+        assert cos > 0.97, (step, cos)
+    assert ra.seq_lens == [303, 48, 133]
+    assert batched.get_batched_stats(ra)["decode_steps"] == 3
+    # pools == one-shot quantisation of every sequence's exact K/V (the exact cache of ra is kept current)
+    for li, (name, state) in enumerate(st.items()):
+        cache = ra.layers[li].attn.kv_cache[0]
+        for b, L in enumerate(ra.seq_lens):
+            pos = torch.arange(L, device=dev)
+            slot = ra.block_table[b].long()[pos // BLOCK] * BLOCK + pos % BLOCK
+            K = cache[0].view(-1, 2, 128)[slot].transpose(0, 1).contiguous()          # (H, L, d)
+            V = cache[1].view(-1, 2, 128)[slot].transpose(0, 1).contiguous()
+            idx, sgn, norms, rn, vd, vs, vz = state.pool.export_flat(ra.block_table[b], L)
+            code = state.quantizer.quantize(K)
+            vq = quantize_values(V, bits=4, group_size=32)
+            assert torch.equal(idx, code.mse_indices) and torch.equal(sgn, code.qjl_signs)
+            assert torch.equal(norms, code.norms) and torch.equal(rn, code.residual_norms)
+            assert torch.equal(vd, vq.data) and torch.equal(vs, vq.scales) and torch.equal(vz, vq.zeros)
+    # decode attention of layer 1 from the pool vs the oracle on the same pages, full and hybrid
+    state = list(st.values())[1]
+    cache = ra.layers[1].attn.kv_cache[0]
+    meta = ra.metadata([0, 0, 0])
+    q = torch.randn(3, 8, 128, generator=torch.Generator(device=dev).manual_seed(2), device=dev).bfloat16()
+    full = state.attend(q, meta, kv_cache=cache, hybrid=False)
+    hyb = state.attend(q, meta, kv_cache=cache, hybrid=True)
+    prm = params_of(state.quantizer)
+    for b, L in enumerate(ra.seq_lens):
+        idx, sgn, norms, rn, vd, vs, vz = [t.cpu() for t in state.pool.export_flat(ra.block_table[b], L)]
+        kc = key_code(idx, sgn, rn, norms, 2)
+        vc = value_code(vd, vs, vz, 4)
+        want = O.hybrid_attention(q[b:b + 1].cpu(), kc, vc, L, prm, 2, None, None)
+        assert cosine(full[b].float().cpu(), want.flatten().float()) >= 0.9999
+        R = 32
+        pos = torch.arange(L - R, L, device=dev)
+        slot = ra.block_table[b].long()[pos // BLOCK] * BLOCK + pos % BLOCK
+        rk, rv = cache[0].view(-1, 2, 128)[slot].cpu(), cache[1].view(-1, 2, 128)[slot].cpu()
+        kc_h = key_code(idx[:, :L - R], sgn[:, :L - R], rn[:, :L - R], norms[:, :L - R], 2)
+        vc_h = value_code(vd[:, :L - R], vs[:, :L - R], vz[:, :L - R], 4)
+        want_h = O.hybrid_attention(q[b:b + 1].cpu(), kc_h, vc_h, L - R, prm, 2, rk, rv)
+        assert cosine(hyb[b].float().cpu(), want_h.flatten().float()) >= 0.9999
+    # no exact cache at all: full_tq + no_alloc, prefill answered by dense causal attention over the step
+    rc = MinimalRunner(n_layers=2, hidden=256, num_heads=8, num_kv_heads=2, head_dim=128, ffn=512, vocab=1000,
+                       batch=2, max_seq_len=200, device=dev, seed=3, exact_cache=False)
+    rd = MinimalRunner(n_layers=2, hidden=256, num_heads=8, num_kv_heads=2, head_dim=128, ffn=512, vocab=1000,
+                       batch=2, max_seq_len=200, device=dev, seed=3)
+    batched.install_batched_hooks(rc, num_blocks=rc.num_blocks, key_bits=3, value_bits=4, initial_layers_count=0,
+                                  mode=hooks.MODE_FULL_TQ, no_alloc=True)
+    toks = torch.randint(0, 1000, (150,), generator=g).to(dev)
+    lc, ld = rc.step(toks, rc.metadata([90, 60])), rd.step(toks, rd.metadata([90, 60]))
+    assert min(cosine(lc[b].float().cpu(), ld[b].float().cpu()) for b in range(2)) > 0.999
+    toks = torch.randint(0, 1000, (2,), generator=g).to(dev)
+    lc, ld = rc.decode_step(toks), rd.decode_step(toks)
+    assert min(cosine(lc[b].float().cpu(), ld[b].float().cpu()) for b in range(2)) > 0.97
+    hooks.set_mode(hooks.MODE_CAPTURE_ONLY)
