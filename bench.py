@@ -1,7 +1,7 @@
 """Headline benchmark: compressed-KV decode attention GB/s (and % of HBM peak)
 plus quantize tokens/s, on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-backend-step]
 
 A step is one pass of the fused decode-attention path (query rotation, page
 streaming kernel, merge) over the long-context configuration: 4 sequences x
@@ -19,6 +19,9 @@ The same JSON line carries
   quantize     : tokens/s of the fused paged quantise call on the prefill
                  configuration (32 768 tokens x 8 KV heads, head_dim 128);
   decode_gqa   : the 16 x 8192-token GQA decode configuration;
+  backend_decode_step : a full decode step of a random-init 32-layer dense
+                 transformer (batch 32 x 32 768 context) whose attention layers run
+                 through the batch-aware backend hooks on compressed KV;
   cpu_baseline : the CPU oracle's de-quantise-everything attention (the
                  reference's production read path) timed on the host cores on
                  one of the four sequences.
@@ -206,6 +209,58 @@ def quantize_bench(device, steps, warmup):
                                  "against the 2500 TFLOP/s bf16 peak"}}, (pool, k, v, table, tq)
 
 
+def backend_step_bench(device, steps, warmup, n_layers=32, batch=32, context=32768):
+    """Full decode step through the attention-backend hooks: a random-init bf16 dense transformer (hidden 4096,
+    32 q / 8 KV heads of 128, SwiGLU 14336, vocabulary 128256) with compressed KV (3b keys, 4b values) in every
+    layer and no exact KV cache.  The prior tokens' K/V are drawn N(0,1) straight into the pools (running the
+    25-PFLOP prefill that would produce them is not part of the step being timed)."""
+    import torch
+    from turboquant_amd.integration import batched, vllm as hooks
+    from turboquant_amd.integration.harness import MinimalRunner
+    hidden, hq, hkv, d, ffn, vocab = 4096, 32, 8, 128, 14336, 128256
+    slack = 64 + warmup + steps
+    runner = MinimalRunner(n_layers, hidden, hq, hkv, d, ffn, vocab, batch, context + slack, device,
+                           exact_cache=False, seed=4)
+    states = batched.install_batched_hooks(runner, num_blocks=runner.num_blocks, key_bits=3, value_bits=4,
+                                           initial_layers_count=0, mode=hooks.MODE_FULL_TQ, no_alloc=True)
+    gen = torch.Generator(device=device).manual_seed(4)
+    chunk = 8192
+    zero = torch.zeros(batch, dtype=torch.int32)
+    for st in states.values():
+        for c0 in range(0, context, chunk):
+            k = torch.randn(batch, chunk, hkv, d, generator=gen, device=device, dtype=torch.bfloat16)
+            v = torch.randn(batch, chunk, hkv, d, generator=gen, device=device, dtype=torch.bfloat16)
+            st.pool.append(k, v, runner.block_table, start_pos=zero + c0)
+    del k, v
+    runner.seq_lens = [context] * batch
+    toks = torch.randint(0, vocab, (warmup + steps, batch), generator=gen, device=device)
+    ms, _ = time_steps(lambda i: runner.decode_step(toks[i]), steps, warmup)
+    # the compressed-KV part of a step alone: every layer's page write and fused decode attention
+    meta = runner.decode_metadata()
+    q1 = torch.randn(batch, hq, d, generator=gen, device=device, dtype=torch.bfloat16)
+    k1 = torch.randn(batch, hkv, d, generator=gen, device=device, dtype=torch.bfloat16)
+
+    def kv_part(i):
+        for st in states.values():
+            st.write(k1, k1, meta)
+            st.attend(q1, meta)
+    kv_ms, _ = time_steps(kv_part, steps, warmup)
+    attn_bytes = n_layers * batch * context * hkv * algorithmic_bytes_per_token_head(d, 2, 4, 32)
+    weight_bytes = 2 * (n_layers * (hidden * (hq + 2 * hkv) * d + hq * d * hidden + 3 * hidden * ffn) + hidden * vocab)
+    out = {"workload": f"full decode step through the attention-backend hooks: {n_layers} layers, hidden {hidden}, "
+                       f"{hq} q / {hkv} KV heads of {d}, SwiGLU {ffn}, batch {batch} x {context} context, "
+                       "compressed KV (3b keys, 4b values) in every layer, no exact KV cache; prior K/V synthetic",
+           "tokens_per_s": batch / (ms * 1e-3), "ms_per_step": ms, "steps": steps,
+           "compressed_kv_bytes_read_per_step": attn_bytes, "weight_bytes_read_per_step": weight_bytes,
+           "hbm_gbs": (attn_bytes + weight_bytes) / (ms * 1e-3) / 1e9,
+           "compressed_kv_ms_per_step": kv_ms, "compressed_kv_gbs": attn_bytes / (kv_ms * 1e-3) / 1e9,
+           "compressed_kv_gib": sum(s.memory_bytes() for s in states.values()) / 2 ** 30}
+    hooks.set_mode(hooks.MODE_CAPTURE_ONLY)
+    del runner, states
+    torch.cuda.empty_cache()
+    return out
+
+
 def cpu_quantize_baseline(k, v, tq, sample_tokens=4096):
     import torch
     from oracle import tq_oracle as O
@@ -230,6 +285,8 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    ap.add_argument("--no-backend-step", action="store_true",
+                    help="skip the full-decode-step leg (32-layer transformer through the backend hooks, ~60 GB)")
     ap.add_argument("--context", type=int, default=131072, help="context tokens per sequence of the main workload")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -265,6 +322,10 @@ def main():
 
     quant, (qpool, qk, qv, qtable, qtq) = quantize_bench(device, max(5, args.steps // 5), max(2, args.warmup // 5))
 
+    backend = None
+    if not args.no_backend_step:
+        backend = backend_step_bench(device, max(5, args.steps // 10), max(2, args.warmup // 10))
+
     cpu = None
     if not args.no_cpu:
         ref_out, cpu = cpu_decode_baseline(main_w)
@@ -294,6 +355,7 @@ def main():
                        "GBps": gqa_w.bytes / (gqa_ms * 1e-3) / 1e9, "ms_per_step": gqa_ms,
                        "kernel_GBps": gqa_w.bytes / (gqa_kern * 1e-3) / 1e9,
                        "pct_hbm_peak": 100.0 * gqa_w.bytes / (gqa_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
+        "backend_decode_step": backend,
         "cpu_baseline": cpu,
     }
     print(json.dumps(line))
