@@ -674,6 +674,62 @@ def test_decode_one_million_token_context_against_dense_attention_on_the_dequant
     assert cos >= 0.9999
 
 
+def test_decode_step_replays_from_a_captured_graph(gpu):
+    """A serving loop captures its decode step once and replays it.  One step = advance the lengths, append one
+    token per sequence, fused decode attention; the library allocates nothing and never synchronises, so the
+    step can be captured.  Every replay (inputs refilled in place, eager work and synchronisation between the
+    replays) must equal the same step run eagerly on a twin pool."""
+    g = torch.Generator(device=gpu).manual_seed(13)
+    d, Hkv, Hq, B, N0, cap = 128, 2, 8, 3, 200, 256
+    pools = [_make_pool(gpu, d, 3, 4, Hkv, B * (cap // 16))[0] for _ in range(2)]
+    table = torch.randperm(B * (cap // 16), generator=g, device=gpu).to(torch.int32).view(B, -1)
+    k0 = torch.randn(B, N0, Hkv, d, generator=g, device=gpu).bfloat16()
+    v0 = torch.randn(B, N0, Hkv, d, generator=g, device=gpu).bfloat16()
+    for p in pools:
+        p.append(k0, v0, table)
+    seqs = [torch.tensor([N0, N0 - 37, N0 - 150], dtype=torch.int32, device=gpu) for _ in range(2)]
+    k1, v1 = torch.zeros(B, 1, Hkv, d, dtype=torch.bfloat16, device=gpu), torch.zeros(B, 1, Hkv, d, dtype=torch.bfloat16, device=gpu)
+    q = torch.zeros(B, Hq, d, dtype=torch.bfloat16, device=gpu)
+    outs = [torch.zeros_like(q) for _ in range(2)]
+    ws = [p.workspace(B, Hq, 4) for p in pools]
+
+    def step(i):
+        seqs[i].add_(1)
+        pools[i].append(k1, v1, table, start_pos=seqs[i] - 1)
+        pools[i].decode_attention(q, table, seqs[i], n_split=4, workspace=ws[i], out=outs[i], max_len=cap)
+
+    def refill():
+        k1.copy_(torch.randn(k1.shape, generator=g, device=gpu).bfloat16())
+        v1.copy_(torch.randn(v1.shape, generator=g, device=gpu).bfloat16())
+        q.copy_(torch.randn(q.shape, generator=g, device=gpu).bfloat16())
+
+    refill()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):                      # warm-up outside the capture (launch attributes, allocator)
+        step(0)
+    torch.cuda.current_stream().wait_stream(side)
+    step(1)
+    torch.cuda.synchronize()
+    assert torch.equal(outs[0], outs[1])
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step(0)
+    step(1)                                            # the capture itself does not run the step: ...
+    graph.replay()                                     # ... this replay is step 2 of pool 0
+    torch.cuda.synchronize()
+    assert torch.equal(outs[0], outs[1]) and torch.equal(seqs[0], seqs[1])
+    for r in range(4):
+        refill()
+        _progress(f"graph replay {r}")
+        graph.replay()
+        step(1)
+        torch.cuda.synchronize()
+        assert torch.equal(seqs[0], seqs[1])
+        assert torch.equal(outs[0], outs[1]), r
+    assert torch.equal(pools[0].data, pools[1].data)
+
+
 def test_page_kernel_timing_hook_times_one_dispatch_and_changes_nothing(gpu):
     # tq_time_next_page_kernel attaches an event pair to the next page-kernel dispatch of this thread:
     # the elapsed time is positive and below the bracketing stream markers', the hook disarms itself,

@@ -368,4 +368,22 @@ def test_batched_hooks_through_the_minimal_transformer(gpu):
     toks = torch.randint(0, 1000, (2,), generator=g).to(dev)
     lc, ld = rc.decode_step(toks), rd.decode_step(toks)
     assert min(cosine(lc[b].float().cpu(), ld[b].float().cpu()) for b in range(2)) > 0.97
+    # the compressed decode step captured as a graph: replays equal the eager steps of a twin runner
+    twins = []
+    for _ in range(2):
+        r = MinimalRunner(n_layers=2, hidden=256, num_heads=8, num_kv_heads=2, head_dim=128, ffn=512, vocab=1000,
+                          batch=2, max_seq_len=200, device=dev, seed=3, exact_cache=False)
+        batched.install_batched_hooks(r, num_blocks=r.num_blocks, key_bits=3, value_bits=4, initial_layers_count=0,
+                                      mode=hooks.MODE_FULL_TQ, no_alloc=True)
+        r.step(torch.arange(150, device=dev) % 1000, r.metadata([90, 60]))
+        twins.append(r)
+    t0 = torch.tensor([5, 7], device=dev)
+    replay, first = twins[0].capture_decode_step(200, t0)
+    assert torch.equal(first, twins[1].decode_step(t0))
+    for i in range(4):
+        t = torch.randint(0, 1000, (2,), generator=g).to(dev)
+        got, want = replay(t), twins[1].decode_step(t)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), i
+        assert twins[0].seq_lens == twins[1].seq_lens
     hooks.set_mode(hooks.MODE_CAPTURE_ONLY)

@@ -205,3 +205,49 @@ class MinimalRunner:
         """tokens (B,): one new token per sequence."""
         meta = self.decode_metadata()
         return self.step(tokens, meta, positions=(meta.seq_lens - 1).long())
+
+    # ---- the decode step as a HIP graph ----------------------------------------------
+    def capture_decode_step(self, max_seq_len: int, first_tokens: torch.Tensor):
+        """Run one decode step eagerly on `first_tokens` (that settles launch attributes and the allocator),
+        capture the step (lengths advance on the device, slots and positions are derived from them inside
+        the graph) and return (replay, logits of the first step); replay(tokens) -> logits runs the next
+        step.  The sequences may grow up to `max_seq_len` tokens under this graph; it is meant for the
+        exact-cache-free compressed path (backends whose forward reads host copies of the metadata cannot
+        be captured)."""
+        dev = self.device
+        tokens = first_tokens.to(device=dev, dtype=torch.long).clone()
+        lens = torch.tensor(self.seq_lens, dtype=torch.int32, device=dev)
+        qsl = torch.arange(self.batch + 1, dtype=torch.int32)
+        meta = StepMetadata(num_actual_tokens=self.batch, max_query_len=1, max_seq_len=max_seq_len, seq_lens=lens,
+                            query_start_loc=qsl.to(dev), block_table=self.block_table,
+                            slot_mapping=torch.zeros(self.batch, dtype=torch.long, device=dev),
+                            seq_lens_cpu=torch.tensor(self.seq_lens, dtype=torch.int32), query_start_loc_cpu=qsl)
+
+        def body():
+            lens.add_(1)
+            pos = (lens - 1).long()
+            meta.slot_mapping.copy_(torch.gather(self.block_table.long(), 1, (pos // BLOCK)[:, None])[:, 0] * BLOCK
+                                    + pos % BLOCK)
+            return self.step(tokens, meta, positions=pos)
+
+        host_lens = list(self.seq_lens)
+        side = torch.cuda.Stream(device=dev)
+        side.wait_stream(torch.cuda.current_stream(dev))
+        with torch.cuda.stream(side):
+            first_logits = body().clone()
+        torch.cuda.current_stream(dev).wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            logits = body()
+        # the graph's kernels address `lens` and the metadata tensors directly: they must live as long as it does
+        state = {"steps": 1, "keep": (lens, meta, body)}
+
+        def replay(new_tokens: torch.Tensor) -> torch.Tensor:
+            tokens.copy_(new_tokens)
+            graph.replay()
+            state["steps"] += 1
+            self.seq_lens = [n + state["steps"] for n in host_lens]
+            return logits
+
+        self.seq_lens = [n + 1 for n in host_lens]
+        return replay, first_logits
