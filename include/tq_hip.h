@@ -174,6 +174,19 @@ int tq_append_kv_paged(const void *k, const void *v, int dtype, int B, int T, in
                        int max_pages, const tq_layer *layer, const tq_page_layout *layout, uint8_t *pool,
                        int64_t num_pages, void *stream);
 
+/* The same for tokens that already sit in a paged exact KV cache (gather + quantise in one pass;
+ * capture.py:187-217 ingest_prefill_from_paged_cache gathers the blocks with torch indexing first).
+ * k_cache, v_cache: blocks of 16 tokens, element (block, slot, h, :) at
+ * base + block*stride_blk + slot*stride_t + h*stride_h.  Sequence b's token at absolute position p
+ * is slot p%16 of block src_table[b*src_stride + p/16]; positions start_pos[b] .. start_pos[b] +
+ * min(run_len[b], T) - 1 are quantised (start_pos NULL = 0, run_len NULL = T for every sequence) and
+ * written to page block_table[b*max_pages + p/16], slot p%16, as by tq_append_kv_paged.             */
+int tq_append_kv_from_blocks(const void *k_cache, const void *v_cache, int dtype, int B, int T, int H,
+                             int64_t stride_blk, int64_t stride_t, int64_t stride_h, const int32_t *src_table,
+                             int src_stride, const int32_t *start_pos, const int32_t *run_len,
+                             const int32_t *block_table, int max_pages, const tq_layer *layer,
+                             const tq_page_layout *layout, uint8_t *pool, int64_t num_pages, void *stream);
+
 /* Gather a sequence's pages back into the reference's flat tensors
  * (store.py:92-114 get_flat_cache): idx (H, n_tok, d*eff/8), signs (H, n_tok, d/8),
  * norms (H, n_tok) input dtype, rnorms fp32, v_data (H, n_tok, d*vb/8),

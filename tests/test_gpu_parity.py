@@ -591,6 +591,61 @@ def test_decode_attention_ragged_empty_and_hybrid_tail(gpu):
     worst = _decode_case(gpu, 128, 3, 2, 2, 4, 2, [0, 64], None, seed=79)            # one row has nothing at all
 
 
+@pytest.mark.parametrize("d,key_bits,vb,dtype", [(128, 3, 4, torch.bfloat16), (256, 3, 2, torch.bfloat16),
+                                                   (64, 2, 2, torch.float16), (128, 4, 4, torch.float32)])
+def test_append_from_blocks_equals_gather_then_append(gpu, d, key_bits, vb, dtype):
+    """tq_append_kv_from_blocks reads the tokens in place from a paged exact cache; the pool it fills must be
+    byte-identical to gathering every sequence's tokens with torch indexing and appending them
+    (capture.py:187-217), for ragged run lengths and runs that start inside a page."""
+    from turboquant_amd.paged import PagedKVPool
+    g = torch.Generator().manual_seed(3 * d + vb)
+    H, B, n_blocks, per_seq = 2, 3, 40, 12
+    kc = torch.randn(n_blocks, 16, H, d, generator=g).to(dtype).to(gpu)
+    vc = torch.randn(n_blocks, 16, H, d, generator=g).to(dtype).to(gpu)
+    src = torch.randperm(n_blocks, generator=g)[: B * per_seq].view(B, per_seq).to(torch.int32).to(gpu)
+    dst = torch.randperm(B * per_seq, generator=g).view(B, per_seq).to(torch.int32).to(gpu)
+    for start, run in (([0, 0, 0], [70, 16, 133]), ([16, 5, 37], [100, 1, 90])):
+        _progress(f"append_from_blocks d={d} {dtype} start={start} run={run}")
+        pa, tq = _make_pool(gpu, d, key_bits, vb, H, B * per_seq, dtype=dtype)
+        pb = PagedKVPool(tq, H, B * per_seq, value_bits=vb, dtype=dtype, device=gpu)
+        sp = torch.tensor(start, dtype=torch.int32)
+        pa.append_from_blocks(kc, vc, src, dst, torch.tensor(run, dtype=torch.int32), start_pos=sp)
+        for b in range(B):
+            pos = torch.arange(start[b], start[b] + run[b], device=gpu)
+            blk = src[b].long()[pos // 16]
+            k = kc[blk, pos % 16][None]                       # (1, run, H, d)
+            v = vc[blk, pos % 16][None]
+            pb.append(k, v, dst[b:b + 1], start_pos=sp[b:b + 1])
+        assert torch.equal(pa.data, pb.data)
+
+
+def test_capture_engine_ingests_a_paged_cache_in_place(gpu):
+    """KVCaptureEngine.ingest_prefill_from_paged_cache (capture.py:187-217) with 16-token blocks quantises the
+    part to compress straight out of the paged cache; store and ring must equal the gather-then-ingest path."""
+    from turboquant_amd.capture import KVCaptureEngine
+    from turboquant_amd.store import CompressedKVStore
+    g = torch.Generator().manual_seed(17)
+    H, d, n_tok, n_blocks = 2, 128, 300, 32
+    cache = torch.randn(2, n_blocks, 16, H, d, generator=g).bfloat16().to(gpu)
+    table = torch.randperm(n_blocks, generator=g)[:19].to(torch.int32)
+    engines = []
+    for _ in range(2):
+        store = CompressedKVStore(head_dim=d, num_kv_heads=H, key_bits=3, value_bits=2, device=gpu)
+        engines.append(KVCaptureEngine(store=store, ring_capacity=128, device=gpu))
+    engines[0].ingest_prefill_from_paged_cache(cache, n_tok, table, 16)
+    phys = table.long().to(gpu)
+    k = cache[0].index_select(0, phys).reshape(-1, H, d)[:n_tok]
+    v = cache[1].index_select(0, phys).reshape(-1, H, d)[:n_tok]
+    engines[1].ingest_prefill(k, v, n_tok)
+    assert engines[0].store.num_tokens == engines[1].store.num_tokens == n_tok - 128
+    fa, fb = engines[0].store.get_flat_cache(), engines[1].store.get_flat_cache()
+    for a, b in zip(tuple(fa.prod_q)[:4] + tuple(fa.value_q)[:3], tuple(fb.prod_q)[:4] + tuple(fb.value_q)[:3]):
+        assert torch.equal(a, b)
+    for a, b in zip(engines[0].ring.peek(), engines[1].ring.peek()):
+        assert torch.equal(a, b)
+    assert engines[0].total_tokens == n_tok
+
+
 def test_pool_export_word_and_byte_kernels_agree(gpu):
     """tq_pool_export writes the flat tensors a word at a time; outputs that are not 4-byte aligned take the
     byte-wise kernel.  Both must give the same bytes (ragged token count, permuted pages, every value width)."""

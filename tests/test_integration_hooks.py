@@ -333,6 +333,18 @@ def test_batched_hooks_through_the_minimal_transformer(gpu):
             assert torch.equal(idx, code.mse_indices) and torch.equal(sgn, code.qjl_signs)
             assert torch.equal(norms, code.norms) and torch.equal(rn, code.residual_norms)
             assert torch.equal(vd, vq.data) and torch.equal(vs, vq.scales) and torch.equal(vz, vq.zeros)
+    # compressing rb's exact cache in place (gather-quantise through the block table) gives the same pools
+    for li, state in enumerate(st.values()):
+        fresh = batched.BatchedLayerState(config=state.config, quantizer=state.quantizer,
+                                          pool=type(state.pool)(state.quantizer, 2, ra.num_blocks, value_bits=4,
+                                                                dtype=torch.bfloat16, device=dev))
+        fresh.ingest_paged_cache(rb.layers[li].attn.kv_cache[0], rb.block_table,
+                                 torch.tensor(rb.seq_lens, dtype=torch.int32))
+        if li == 0:                                   # layer 0 saw the same K/V in both runners
+            assert torch.equal(fresh.pool.data, state.pool.data)
+        for b, L in enumerate(rb.seq_lens):
+            got = fresh.pool.export_flat(rb.block_table[b], L)
+            assert got[0].shape[1] == L
     # decode attention of layer 1 from the pool vs the oracle on the same pages, full and hybrid
     state = list(st.values())[1]
     cache = ra.layers[1].attn.kv_cache[0]

@@ -15,6 +15,8 @@ from typing import TYPE_CHECKING, Optional, Tuple
 
 import torch
 
+from .paged import PAGE_TOKENS
+
 if TYPE_CHECKING:
     from .store import CompressedKVStore
 
@@ -126,12 +128,26 @@ class KVCaptureEngine:
     def ingest_prefill_from_paged_cache(self, kv_cache_tensor: torch.Tensor, num_tokens: int,
                                         block_table: torch.Tensor, block_size: int):
         """Prefill from a paged exact cache (2, num_blocks, block_size, heads, dim)
-        through `block_table` (logical -> physical block)."""
+        through `block_table` (logical -> physical block).  With 16-token blocks and an empty
+        store the part to compress is quantised in place (gather and quantisation in one
+        kernel pass); only the ring's tail is gathered."""
         n_blocks = (num_tokens + block_size - 1) // block_size
         phys = block_table[:n_blocks].to(device=kv_cache_tensor.device, dtype=torch.long)
-        k = kv_cache_tensor[0].index_select(0, phys).reshape(n_blocks * block_size, *kv_cache_tensor.shape[3:])
-        v = kv_cache_tensor[1].index_select(0, phys).reshape(n_blocks * block_size, *kv_cache_tensor.shape[3:])
-        self.ingest_prefill(k[:num_tokens], v[:num_tokens], num_tokens)
+        cap = self.ring.capacity
+        in_place = (block_size == PAGE_TOKENS and num_tokens > cap and self.store.num_tokens == 0 and
+                    kv_cache_tensor.is_cuda and kv_cache_tensor.dim() == 5 and kv_cache_tensor[0].stride(-1) == 1 and
+                    kv_cache_tensor[0].stride() == kv_cache_tensor[1].stride())
+        if not in_place:
+            k = kv_cache_tensor[0].index_select(0, phys).reshape(n_blocks * block_size, *kv_cache_tensor.shape[3:])
+            v = kv_cache_tensor[1].index_select(0, phys).reshape(n_blocks * block_size, *kv_cache_tensor.shape[3:])
+            self.ingest_prefill(k[:num_tokens], v[:num_tokens], num_tokens)
+            return
+        head = num_tokens - cap
+        self.store.append_chunk_from_blocks(kv_cache_tensor[0], kv_cache_tensor[1], phys, head)
+        pos = torch.arange(head, num_tokens, device=kv_cache_tensor.device)
+        blk = phys[pos // block_size]
+        self.ring.write(kv_cache_tensor[0][blk, pos % block_size], kv_cache_tensor[1][blk, pos % block_size], cap)
+        self._prefill_done = True
 
     def ingest_decode(self, key: torch.Tensor, value: torch.Tensor, num_tokens: int):
         """Decode tokens go to the ring; what the ring drains is compressed."""

@@ -30,11 +30,20 @@ struct FlatSource {          // (n_vec, d) with a row stride
 };
 
 __device__ const int32_t k_zero_i32 = 0;
+__device__ const int32_t k_max_i32 = 0x7fffffff;
 
 struct PagedSource {         // (b, t, h, :) strided, tokens mapped onto 16-token pages
   int B, T, H, tiles_per_seq;
   int64_t stride_b, stride_t, stride_h;
   const int32_t* start_pos;
+  // Optional block-gather mode: the tokens sit in a paged exact cache (blocks of 16 tokens).  Token at
+  // absolute position p of sequence b is slot p % 16 of block src_table[b * src_stride + p / 16]; blocks
+  // are stride_blk elements apart and stride_b is unused.  run_len (optional) bounds the run of each
+  // sequence separately (<= T).
+  const int32_t* src_table = nullptr;
+  int src_stride = 0;
+  int64_t stride_blk = 0;
+  const int32_t* run_len = nullptr;
   // tile index -> (b, page slot window, head)
   __device__ void decode(int tile, int& b, int& lpage, int& h) const {
     h = tile % H;
@@ -45,29 +54,28 @@ struct PagedSource {         // (b, t, h, :) strided, tokens mapped onto 16-toke
     lpage = s0 / TILE + pg;
   }
   // the part of locate() that is the same for the 16 slots of a tile
-  struct TileRef { int64_t base; int t0; };
+  struct TileRef { int64_t base; int t0; int lim; };
   __device__ TileRef tile_ref(int64_t tile) const {
     int h = (int)tile % H;
     int r = (int)tile / H;
     int pg = r % tiles_per_seq;
     int b = r / tiles_per_seq;
-    // one unconditional load (no branch on the null pointer): a load under a branch makes the
+    // unconditional loads (no branch on the null pointers): a load under a branch makes the
     // compiler wait for every outstanding load at the join
     int s0 = *(start_pos ? start_pos + b : &k_zero_i32);
-    return TileRef{b * stride_b + h * stride_h, (s0 / TILE + pg) * TILE - s0};
+    const int lpage = s0 / TILE + pg, t0 = lpage * TILE - s0;
+    const int lim = min(*(run_len ? run_len + b : &k_max_i32), T);
+    const int64_t blk = *(src_table ? src_table + (int64_t)b * src_stride + min(lpage, src_stride - 1) : &k_zero_i32);
+    const int64_t base = src_table ? blk * stride_blk - (int64_t)t0 * stride_t : b * stride_b;
+    return TileRef{base + h * stride_h, t0, lim};
   }
   __device__ bool slot_off(const TileRef& r, int slot, int64_t& elem_off) const {
     int t = r.t0 + slot;
     elem_off = r.base + (int64_t)t * stride_t;
-    return t >= 0 && t < T;
+    return t >= 0 && t < r.lim;
   }
   __device__ bool locate(int tile, int slot, int64_t& elem_off) const {
-    int b, lpage, h;
-    decode(tile, b, lpage, h);
-    int s0 = start_pos ? start_pos[b] : 0;
-    int t = lpage * TILE + slot - s0;
-    elem_off = b * stride_b + (int64_t)t * stride_t + h * stride_h;
-    return t >= 0 && t < T;
+    return slot_off(tile_ref(tile), slot, elem_off);
   }
 };
 

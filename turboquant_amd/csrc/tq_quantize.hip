@@ -716,7 +716,8 @@ static bool value_chunks_aligned(const void* v, const FlatSource& s) {
   return (uintptr_t)v % 16 == 0 && s.row_stride % 8 == 0;
 }
 static bool value_chunks_aligned(const void* v, const PagedSource& s) {
-  return (uintptr_t)v % 16 == 0 && s.stride_b % 8 == 0 && s.stride_t % 8 == 0 && s.stride_h % 8 == 0;
+  return (uintptr_t)v % 16 == 0 && s.stride_b % 8 == 0 && s.stride_t % 8 == 0 && s.stride_h % 8 == 0 &&
+         s.stride_blk % 8 == 0;
 }
 
 template <class Source, class Sink>
@@ -805,23 +806,14 @@ SideLane* side_lane() {
 }
 }  // namespace
 
-extern "C" int tq_append_kv_paged(const void* k, const void* v, int dtype, int B, int T, int H, int64_t stride_b,
-                                  int64_t stride_t, int64_t stride_h, const int32_t* start_pos,
-                                  const int32_t* block_table, int max_pages, const tq_layer* layer,
-                                  const tq_page_layout* layout, uint8_t* pool, int64_t num_pages, void* stream) {
-  int rc = check_layer(layer, true);
-  if (rc) return rc;
-  if (!k || !v || !block_table || !layout || !pool) return TQ_ENULL;
-  if (dtype != layout->dtype || layout->d != layer->d || layout->mse_bits != layer->mse_bits) return TQ_EINVAL;
-  if (B < 0 || T < 0 || H <= 0 || max_pages <= 0 || num_pages <= 0) return TQ_EINVAL;
-  if (B == 0 || T == 0) return TQ_OK;
-  // a run of T tokens starting anywhere inside a page touches at most this many pages
-  // (the run may begin at any of the 16 slots of its first page when start_pos is given)
-  const int tiles_per_seq = start_pos ? (T + TILE - 2) / TILE + 1 : (T + TILE - 1) / TILE;
-  PagedSource src{B, T, H, tiles_per_seq, stride_b, stride_t, stride_h, start_pos};
-  int64_t tiles = (int64_t)B * tiles_per_seq * H;
+// keys and values of the runs described by `src` into the pages of `block_table`
+static int append_runs(const void* k, const void* v, int dtype, const PagedSource& src, const int32_t* block_table,
+                       int max_pages, const tq_layer* layer, const tq_page_layout* layout, uint8_t* pool,
+                       void* stream) {
+  int64_t tiles = (int64_t)src.B * src.tiles_per_seq * src.H;
   KeyPagedSink ks{pool, block_table, max_pages, *layout};
   ValPagedSink vs{pool, block_table, max_pages, *layout};
+  int rc;
   // Large appends run the value kernel beside the key kernel: the key kernel leaves a quarter of the
   // registers and issue slots of every SIMD free, which the small value wavefronts fill (the two
   // kernels write disjoint bytes of the pages).  The value kernel goes to a side stream that is
@@ -844,6 +836,44 @@ extern "C" int tq_append_kv_paged(const void* k, const void* v, int dtype, int B
   rc = launch_key(k, dtype, src, *layer, ks, 0, tiles, (hipStream_t)stream);
   if (rc) return rc;
   return launch_value(v, dtype, src, layer->d, layout->group_size, layout->value_bits, vs, tiles, (hipStream_t)stream);
+}
+
+extern "C" int tq_append_kv_paged(const void* k, const void* v, int dtype, int B, int T, int H, int64_t stride_b,
+                                  int64_t stride_t, int64_t stride_h, const int32_t* start_pos,
+                                  const int32_t* block_table, int max_pages, const tq_layer* layer,
+                                  const tq_page_layout* layout, uint8_t* pool, int64_t num_pages, void* stream) {
+  int rc = check_layer(layer, true);
+  if (rc) return rc;
+  if (!k || !v || !block_table || !layout || !pool) return TQ_ENULL;
+  if (dtype != layout->dtype || layout->d != layer->d || layout->mse_bits != layer->mse_bits) return TQ_EINVAL;
+  if (B < 0 || T < 0 || H <= 0 || max_pages <= 0 || num_pages <= 0) return TQ_EINVAL;
+  if (B == 0 || T == 0) return TQ_OK;
+  // a run of T tokens starting anywhere inside a page touches at most this many pages
+  // (the run may begin at any of the 16 slots of its first page when start_pos is given)
+  const int tiles_per_seq = start_pos ? (T + TILE - 2) / TILE + 1 : (T + TILE - 1) / TILE;
+  PagedSource src{B, T, H, tiles_per_seq, stride_b, stride_t, stride_h, start_pos};
+  return append_runs(k, v, dtype, src, block_table, max_pages, layer, layout, pool, stream);
+}
+
+extern "C" int tq_append_kv_from_blocks(const void* k_cache, const void* v_cache, int dtype, int B, int T, int H,
+                                        int64_t stride_blk, int64_t stride_t, int64_t stride_h,
+                                        const int32_t* src_table, int src_stride, const int32_t* start_pos,
+                                        const int32_t* run_len, const int32_t* block_table, int max_pages,
+                                        const tq_layer* layer, const tq_page_layout* layout, uint8_t* pool,
+                                        int64_t num_pages, void* stream) {
+  int rc = check_layer(layer, true);
+  if (rc) return rc;
+  if (!k_cache || !v_cache || !src_table || !block_table || !layout || !pool) return TQ_ENULL;
+  if (dtype != layout->dtype || layout->d != layer->d || layout->mse_bits != layer->mse_bits) return TQ_EINVAL;
+  if (B < 0 || T < 0 || H <= 0 || max_pages <= 0 || num_pages <= 0 || src_stride <= 0) return TQ_EINVAL;
+  if (B == 0 || T == 0) return TQ_OK;
+  const int tiles_per_seq = start_pos ? (T + TILE - 2) / TILE + 1 : (T + TILE - 1) / TILE;
+  PagedSource src{B, T, H, tiles_per_seq, 0, stride_t, stride_h, start_pos};
+  src.src_table = src_table;
+  src.src_stride = src_stride;
+  src.stride_blk = stride_blk;
+  src.run_len = run_len;
+  return append_runs(k_cache, v_cache, dtype, src, block_table, max_pages, layer, layout, pool, stream);
 }
 
 extern "C" int tq_pool_export(const uint8_t* pool, int64_t num_pages, int H, const int32_t* block_table, int n_tok,

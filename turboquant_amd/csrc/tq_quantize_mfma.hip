@@ -541,7 +541,8 @@ __host__ static bool aligned_for_chunks(const void* x, int dtype, const FlatSour
 }
 __host__ static bool aligned_for_chunks(const void* x, int dtype, const PagedSource& s) {
   const int64_t ch = 16 / elem_bytes(dtype);
-  return (uintptr_t)x % 16 == 0 && s.stride_b % ch == 0 && s.stride_t % ch == 0 && s.stride_h % ch == 0;
+  return (uintptr_t)x % 16 == 0 && s.stride_b % ch == 0 && s.stride_t % ch == 0 && s.stride_h % ch == 0 &&
+         s.stride_blk % ch == 0;
 }
 __host__ static bool sink_ok(const KeyFlatSink& s, int mse_only) {
   return (uintptr_t)s.y_dbg % 16 == 0 && (uintptr_t)s.p_dbg % 16 == 0 && (uintptr_t)s.idx % 4 == 0 &&

@@ -87,6 +87,16 @@ class BatchedLayerState:
                                      start_pos=torch.tensor([lens[b] - (r1 - r0)], dtype=torch.int32))
         self.tokens_written += n
 
+    def ingest_paged_cache(self, kv_cache: torch.Tensor, block_table: torch.Tensor, seq_lens: torch.Tensor,
+                           max_tokens: Optional[int] = None) -> None:
+        """Compress what the engine's exact paged cache (2, num_blocks, 16, H_kv, d) already holds for the
+        sequences of `block_table`: tokens [0, seq_lens[b]) of every sequence, read in place through the
+        block table and written to the pages of the same numbers (the batch counterpart of
+        capture.py:187-217, without the gather copy)."""
+        self.pool.append_from_blocks(kv_cache[0], kv_cache[1], block_table, block_table, seq_lens,
+                                     max_tokens=max_tokens)
+        self.tokens_written += int(seq_lens.sum())
+
     # ---- read --------------------------------------------------------------------
     def _exact_tail(self, kv_cache, meta):
         """The last `ring_capacity` tokens of every sequence from the engine's paged cache:

@@ -81,6 +81,41 @@ class PagedKVPool:
                 C.byref(self.layout), self.data.data_ptr(), self.num_pages, _ffi.stream_ptr(self.device)),
                 "tq_append_kv_paged")
 
+    def append_from_blocks(self, key_cache: torch.Tensor, value_cache: torch.Tensor, src_table: torch.Tensor,
+                           block_table: torch.Tensor, run_len: torch.Tensor, start_pos: Optional[torch.Tensor] = None,
+                           max_tokens: Optional[int] = None):
+        """Quantise tokens that sit in a paged exact cache, without gathering them first.
+        key_cache / value_cache (num_blocks, 16, H, d); sequence b's positions start_pos[b] ..
+        start_pos[b] + run_len[b] - 1 are read through src_table (B, n) (position p -> block
+        src_table[b, p // 16], slot p % 16) and written through block_table (B, max_pages)."""
+        _ffi.require_gpu(key_cache, "key_cache")
+        if key_cache.dim() != 4 or key_cache.shape != value_cache.shape or key_cache.shape[1] != PAGE_TOKENS:
+            raise ValueError("key_cache and value_cache must both be (num_blocks, 16, H, d)")
+        if key_cache.shape[2] != self.num_kv_heads or key_cache.shape[3] != self.head_dim:
+            raise ValueError(f"expected (num_blocks, 16, {self.num_kv_heads}, {self.head_dim})")
+        if key_cache.dtype != self.dtype or value_cache.dtype != self.dtype:
+            raise TypeError(f"pool was laid out for {self.dtype}")
+        if key_cache.stride(-1) != 1 or key_cache.stride() != value_cache.stride():
+            raise ValueError("key_cache and value_cache need the same strides and a contiguous last dimension")
+        B = src_table.shape[0]
+        for t in (src_table, block_table):
+            if t.dtype != torch.int32 or t.dim() != 2 or t.shape[0] != B:
+                raise ValueError("src_table and block_table must be int32 (B, n)")
+        src_table, block_table = src_table.contiguous(), block_table.contiguous()
+        run_len = run_len.to(device=self.device, dtype=torch.int32).contiguous()
+        if start_pos is not None:
+            start_pos = start_pos.to(device=self.device, dtype=torch.int32).contiguous()
+        if max_tokens is None:
+            max_tokens = int(run_len.max())
+        ly = self.quantizer._layer()
+        with torch.cuda.device(self.device):
+            _ffi.check(_ffi.lib().tq_append_kv_from_blocks(
+                key_cache.data_ptr(), value_cache.data_ptr(), _ffi.dtype_tag(self.dtype), B, int(max_tokens),
+                self.num_kv_heads, key_cache.stride(0), key_cache.stride(1), key_cache.stride(2), src_table.data_ptr(),
+                src_table.shape[1], _ffi.ptr(start_pos), run_len.data_ptr(), block_table.data_ptr(),
+                block_table.shape[1], C.byref(ly), C.byref(self.layout), self.data.data_ptr(), self.num_pages,
+                _ffi.stream_ptr(self.device)), "tq_append_kv_from_blocks")
+
     # ---- read -------------------------------------------------------------------
     def export_flat(self, block_table_row: torch.Tensor, n_tok: int):
         """Gather one sequence's pages into the reference's flat tensors

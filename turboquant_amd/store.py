@@ -90,6 +90,24 @@ class CompressedKVStore:
         self._chunk_lengths.append(chunk_len)
         self._flat = None
 
+    def append_chunk_from_blocks(self, key_cache: torch.Tensor, value_cache: torch.Tensor, src_blocks: torch.Tensor,
+                                 chunk_len: int):
+        """Quantise the first chunk_len tokens of a sequence straight out of a paged exact cache
+        ((num_blocks, 16, H, d) tensors, the sequence's blocks in src_blocks) into an EMPTY store:
+        the gather and the quantisation are one pass over the cache."""
+        if chunk_len == 0:
+            return
+        if self.num_tokens != 0:
+            raise RuntimeError("append_chunk_from_blocks fills an empty store (source and store positions coincide)")
+        pool = self.ensure_pool(key_cache.dtype, chunk_len)
+        if key_cache.dtype != pool.dtype:
+            raise TypeError(f"store holds {pool.dtype} pages; got a {key_cache.dtype} cache")
+        src = src_blocks.to(device=pool.device, dtype=torch.int32).reshape(1, -1).contiguous()
+        pool.append_from_blocks(key_cache, value_cache, src, self._block_table,
+                                torch.tensor([chunk_len], dtype=torch.int32), max_tokens=chunk_len)
+        self._chunk_lengths.append(chunk_len)
+        self._flat = None
+
     # ---- read ------------------------------------------------------------------------
     def get_flat_cache(self) -> Optional[FlatCache]:
         """The reference's flat tensors; None while the store is empty."""
