@@ -499,7 +499,8 @@ def _decode_case(gpu, d, key_bits, vb, B, Hq, Hkv, lens, recent, seed, n_split=N
 
 
 @pytest.mark.parametrize("d,key_bits,vb,Hq,Hkv", [(128, 3, 4, 8, 2), (256, 3, 2, 16, 2), (128, 3, 2, 4, 4),
-                                                   (64, 3, 4, 4, 1), (128, 4, 4, 8, 2), (128, 2, 2, 6, 2)])
+                                                   (64, 3, 4, 4, 1), (128, 4, 4, 8, 2), (128, 2, 2, 6, 2),
+                                                   (256, 4, 2, 16, 2), (256, 4, 4, 8, 4), (256, 2, 4, 6, 2)])
 def test_decode_attention_matches_oracle_on_the_same_store(gpu, d, key_bits, vb, Hq, Hkv):
     _progress(f"decode d={d} kb={key_bits} vb={vb} Hq={Hq} Hkv={Hkv}")
     worst = _decode_case(gpu, d, key_bits, vb, 3, Hq, Hkv, [200, 37, 512], None, seed=d + vb)
@@ -553,9 +554,12 @@ def shape_kq_128(k, trend):
 
 
 @pytest.mark.parametrize("d,key_bits,vb,Hq,Hkv,dtype", [(128, 3, 4, 8, 2, torch.float16), (128, 3, 2, 32, 2, torch.bfloat16),
-                                                         (64, 3, 4, 12, 1, torch.float16), (128, 4, 4, 4, 2, torch.float32)])
+                                                         (64, 3, 4, 12, 1, torch.float16), (128, 4, 4, 4, 2, torch.float32),
+                                                         (256, 3, 2, 16, 2, torch.float16), (128, 4, 2, 6, 2, torch.float16),
+                                                         (256, 4, 4, 8, 8, torch.float16), (128, 2, 4, 7, 1, torch.float16)])
 def test_decode_attention_general_kernel_shapes(gpu, d, key_bits, vb, Hq, Hkv, dtype):
-    # shapes without a matrix-core kernel (fp16 / fp32 pools, more than 8 query heads per KV head)
+    # fp16 pools (matrix-core kernel with the fp16 zero-point product), and shapes without a matrix-core
+    # kernel (fp32 pools, head_dim 64, more than 8 query heads per KV head)
     # take the general page kernel and must meet the same gate
     _progress(f"general decode d={d} kb={key_bits} vb={vb} Hq={Hq} Hkv={Hkv} {dtype}")
     worst = _decode_case(gpu, d, key_bits, vb, 2, Hq, Hkv, [300, 77], [0, 9], seed=500 + d + Hq, dtype=dtype)

@@ -366,7 +366,8 @@ extern "C" int tq_decode_attn_paged_stages(const void* q, int dtype, int B, int 
   float* q_sk = q_rot + (size_t)B * Hq * d;
   float* q_stat = q_sk + (size_t)B * Hq * d;
   uint32_t* qa_pack = (uint32_t*)(q_stat + (size_t)4 * B * Hq);
-  const bool mfma_shape = G <= 8 && (d == 128 || d == 256) && layout->dtype == TQ_BF16 && layer->Pi_colsum &&
+  const bool mfma_shape = G <= 8 && (d == 128 || d == 256) && (layout->dtype == TQ_BF16 || layout->dtype == TQ_F16) &&
+                          layer->Pi_colsum &&
                           layer->S_colsum;
 
   if (stages & 1) {

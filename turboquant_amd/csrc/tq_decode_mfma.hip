@@ -83,6 +83,32 @@ __device__ __forceinline__ f32x4 mfma(const u32x4& a, const u32x4& b, f32x4 c) {
   __builtin_memcpy(&bv, &b, 16);
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, bv, c, 0, 0, 0);
 }
+// fp16 pages: the zero points are fp16 numbers, so their product with the softmax weights runs on the
+// fp16 MFMA with the weights packed as fp16 (they are at most 2^REF_SLACK; weights below the fp16
+// denormal range belong to tokens whose share of the sum is below 2^-24)
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+__device__ __forceinline__ uint32_t pack_f16(float lo, float hi) {
+  f32x2 f = {lo, hi};
+  f16x2 r = __builtin_convertvector(f, f16x2);     // round to nearest even
+  uint32_t u;
+  __builtin_memcpy(&u, &r, 4);
+  return u;
+}
+__device__ __forceinline__ f32x4 mfma_f16(const u32x4& a, const u32x4& b, f32x4 c) {
+  f16x8 av, bv;
+  __builtin_memcpy(&av, &a, 16);
+  __builtin_memcpy(&bv, &b, 16);
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(av, bv, c, 0, 0, 0);
+}
+__device__ __forceinline__ float f16_lo(uint32_t w) {
+  const f16x2 h = __builtin_bit_cast(f16x2, w);
+  return (float)h[0];
+}
+__device__ __forceinline__ float f16_hi(uint32_t w) {
+  const f16x2 h = __builtin_bit_cast(f16x2, w);
+  return (float)h[1];
+}
 // keeps a loop-invariant constant in a vector register, so that three-operand
 // bit instructions do not need two scalar operands
 __device__ __forceinline__ uint32_t in_vgpr(uint32_t v) {
@@ -134,7 +160,7 @@ __device__ __forceinline__ constexpr int v_bitpos(int t) {
 // D in {128, 256}; MB stored index bits; NX extra (multi-bit) Walsh terms; VB value bits;
 // GS value group size; DS wavefronts that share one block (each takes D/DS coordinates and
 // channels); WPS wavefronts per SIMD the register budget is sized for.
-template <int D, int MB, int NX, int VB, int GS, int DS, int WPS>
+template <int D, int MB, int NX, int VB, int GS, int DS, int WPS, bool F16P>
 __global__ void __launch_bounds__(MF_WAVES * 64, WPS)
 decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict__ q_stat, int Hq, int Hkv, const uint8_t* __restrict__ pool, const int32_t* __restrict__ block_table,
                    int bt_stride, const int32_t* __restrict__ seq_lens, float sm_scale, tq_layer ly, tq_page_layout L,
@@ -424,8 +450,8 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
       float f[8];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        f[2 * i] = __uint_as_float(V.scale[i] << 16);
-        f[2 * i + 1] = __uint_as_float(V.scale[i] & 0xffff0000u);
+        f[2 * i] = F16P ? f16_lo(V.scale[i]) : __uint_as_float(V.scale[i] << 16);
+        f[2 * i + 1] = F16P ? f16_hi(V.scale[i]) : __uint_as_float(V.scale[i] & 0xffff0000u);
       }
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
@@ -475,10 +501,11 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
       u32x4 ap, bz = V.zero[u];
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        ap[r] = pack_bf16(pr[8 * u + 2 * r], pr[8 * u + 2 * r + 1]);
+        ap[r] = F16P ? pack_f16(pr[8 * u + 2 * r], pr[8 * u + 2 * r + 1])
+                     : pack_bf16(pr[8 * u + 2 * r], pr[8 * u + 2 * r + 1]);
         if (PARTIAL) bz[r] &= keep[4 * u + r];
       }
-      zacc = mfma(ap, bz, zacc);
+      zacc = F16P ? mfma_f16(ap, bz, zacc) : mfma(ap, bz, zacc);
     }
     __builtin_amdgcn_s_setprio(2);
 #pragma unroll
@@ -645,7 +672,7 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
 // events the next launch of this thread attaches to its dispatch (see tq_time_next_page_kernel)
 static thread_local hipEvent_t t_start_event = nullptr, t_stop_event = nullptr;
 
-template <int D, int MB, int NX, int VB, int GS, int DS, int WPS>
+template <int D, int MB, int NX, int VB, int GS, int DS, int WPS, bool F16P>
 static int launch_one(const uint32_t* qa_pack, const float* q_stat, int B, int Hq, int Hkv,
                       const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
                       float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts, int n_split,
@@ -654,7 +681,7 @@ static int launch_one(const uint32_t* qa_pack, const float* q_stat, int B, int H
   size_t per_wave = (size_t)wave_lds_floats(D / DS / GS, DS) * sizeof(float);
   size_t merge = (size_t)(MF_WAVES / DS * G * (D + 2) + MF_WAVES * 16 * 16) * sizeof(float);
   size_t smem = per_wave * MF_WAVES > merge ? per_wave * MF_WAVES : merge;
-  auto kern = decode_mfma_kernel<D, MB, NX, VB, GS, DS, WPS>;
+  auto kern = decode_mfma_kernel<D, MB, NX, VB, GS, DS, WPS, F16P>;
   if (smem > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return (int)e;
@@ -683,17 +710,24 @@ int launch_decode_mfma(const uint32_t* qa_pack, const float* q_stat, int B, int 
                        float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts,
                        int n_split, hipStream_t st) {
   const int G = Hq / Hkv, d = ly.d, mb = ly.mse_bits, vb = L.value_bits, gs = L.group_size;
-  if (G > 8 || L.dtype != TQ_BF16 || !L.key_lane_major) return TQ_EUNSUPPORTED;
+  if (G > 8 || (L.dtype != TQ_BF16 && L.dtype != TQ_F16) || !L.key_lane_major) return TQ_EUNSUPPORTED;
+  const bool f16p = L.dtype == TQ_F16;
   int nx = 0;
   for (int t = 0; t < ly.n_terms; ++t)
     if (__builtin_popcount(ly.term_mask[t]) > 1) ++nx;
 #define TQ_TRY(D_, MB_, NX_, VB_, GS_, DS_, WPS_)                                                               \
-  if (d == D_ && mb == MB_ && nx == NX_ && vb == VB_ && gs == GS_)                                              \
-    return launch_one<D_, MB_, NX_, VB_, GS_, DS_, WPS_>(qa_pack, q_stat, B, Hq, Hkv, pool, block_table, bt_stride, \
-                                                         seq_lens, sm_scale, ly, L, parts, n_parts, n_split, st);
+  if (d == D_ && mb == MB_ && nx == NX_ && vb == VB_ && gs == GS_) {                                            \
+    if (f16p)                                                                                                   \
+      return launch_one<D_, MB_, NX_, VB_, GS_, DS_, WPS_, true>(qa_pack, q_stat, B, Hq, Hkv, pool, block_table,  \
+                                                                 bt_stride, seq_lens, sm_scale, ly, L, parts,     \
+                                                                 n_parts, n_split, st);                          \
+    return launch_one<D_, MB_, NX_, VB_, GS_, DS_, WPS_, false>(qa_pack, q_stat, B, Hq, Hkv, pool, block_table,   \
+                                                                bt_stride, seq_lens, sm_scale, ly, L, parts,      \
+                                                                n_parts, n_split, st);                           \
+  }
   TQ_TRY(128, 2, 0, 2, 32, 1, 2) TQ_TRY(128, 2, 0, 4, 32, 1, 2) TQ_TRY(256, 2, 0, 2, 32, 2, 2) TQ_TRY(256, 2, 0, 4, 32, 2, 2)
   TQ_TRY(128, 1, 0, 2, 32, 1, 2) TQ_TRY(128, 1, 0, 4, 32, 1, 2) TQ_TRY(256, 1, 0, 2, 32, 2, 2) TQ_TRY(256, 1, 0, 4, 32, 2, 2)
-  TQ_TRY(128, 3, 1, 2, 32, 1, 1) TQ_TRY(128, 3, 1, 4, 32, 1, 1)
+  TQ_TRY(128, 3, 1, 2, 32, 1, 1) TQ_TRY(128, 3, 1, 4, 32, 1, 1) TQ_TRY(256, 3, 1, 2, 32, 2, 1) TQ_TRY(256, 3, 1, 4, 32, 2, 1)
   TQ_TRY(128, 2, 0, 2, 64, 1, 2) TQ_TRY(128, 2, 0, 4, 64, 1, 2) TQ_TRY(256, 2, 0, 2, 64, 2, 2) TQ_TRY(256, 2, 0, 4, 64, 2, 2)
 #undef TQ_TRY
   return TQ_EUNSUPPORTED;
