@@ -556,10 +556,13 @@ def shape_kq_128(k, trend):
 @pytest.mark.parametrize("d,key_bits,vb,Hq,Hkv,dtype", [(128, 3, 4, 8, 2, torch.float16), (128, 3, 2, 32, 2, torch.bfloat16),
                                                          (64, 3, 4, 12, 1, torch.float16), (128, 4, 4, 4, 2, torch.float32),
                                                          (256, 3, 2, 16, 2, torch.float16), (128, 4, 2, 6, 2, torch.float16),
-                                                         (256, 4, 4, 8, 8, torch.float16), (128, 2, 4, 7, 1, torch.float16)])
+                                                         (256, 4, 4, 8, 8, torch.float16), (128, 2, 4, 7, 1, torch.float16),
+                                                         (128, 3, 4, 12, 1, torch.bfloat16), (256, 3, 2, 18, 2, torch.bfloat16),
+                                                         (128, 3, 2, 11, 1, torch.bfloat16), (128, 4, 4, 32, 2, torch.float16)])
 def test_decode_attention_general_kernel_shapes(gpu, d, key_bits, vb, Hq, Hkv, dtype):
-    # fp16 pools (matrix-core kernel with the fp16 zero-point product), and shapes without a matrix-core
-    # kernel (fp32 pools, head_dim 64, more than 8 query heads per KV head)
+    # fp16 pools (matrix-core kernel with the fp16 zero-point product), more than 8 query heads per KV head
+    # (served as groups of at most 8: 16 = 2 x 8, 12 = 2 x 6, 9 = 3 x 3), and shapes without a
+    # matrix-core kernel (fp32 pools, head_dim 64, 11 query heads per KV head)
     # take the general page kernel and must meet the same gate
     _progress(f"general decode d={d} kb={key_bits} vb={vb} Hq={Hq} Hkv={Hkv} {dtype}")
     worst = _decode_case(gpu, d, key_bits, vb, 2, Hq, Hkv, [300, 77], [0, 9], seed=500 + d + Hq, dtype=dtype)

@@ -315,7 +315,7 @@ namespace tq {
 int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* layer, float* q_rot, float* q_sk,
                         float* q_stat, uint32_t* qa_pack, int G, float sm_scale, hipStream_t st);
 size_t decode_mfma_pack_words(int B, int Hkv, int d);
-int launch_decode_mfma(const uint32_t* qa_pack, const float* q_stat, int B, int Hq, int Hkv,
+int launch_decode_mfma(const uint32_t* qa_pack, const float* q_stat, int B, int Hq, int Hkv, int kv_div,
                        const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
                        float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts,
                        int n_split, hipStream_t st);
@@ -366,7 +366,13 @@ extern "C" int tq_decode_attn_paged_stages(const void* q, int dtype, int B, int 
   float* q_sk = q_rot + (size_t)B * Hq * d;
   float* q_stat = q_sk + (size_t)B * Hq * d;
   uint32_t* qa_pack = (uint32_t*)(q_stat + (size_t)4 * B * Hq);
-  const bool mfma_shape = G <= 8 && (d == 128 || d == 256) && (layout->dtype == TQ_BF16 || layout->dtype == TQ_F16) &&
+  // the matrix-core kernel takes up to 8 query heads per group: a KV head with more is served by kv_div
+  // groups of G / kv_div heads (0 = no such split, e.g. 11 heads)
+  int kv_div = 0;
+  for (int n = 1; n <= G && !kv_div; ++n)
+    if (G % n == 0 && G / n <= 8) kv_div = n;
+  const int Gq = kv_div ? G / kv_div : G;
+  const bool mfma_shape = kv_div && (d == 128 || d == 256) && (layout->dtype == TQ_BF16 || layout->dtype == TQ_F16) &&
                           layer->Pi_colsum &&
                           layer->S_colsum;
 
@@ -374,7 +380,7 @@ extern "C" int tq_decode_attn_paged_stages(const void* q, int dtype, int B, int 
     if (!layer->Pi || !layer->PiT || !layer->S || !layer->ST || !layer->centroids) return TQ_ENULL;
     if (dtype < TQ_F32 || dtype > TQ_BF16) return TQ_EINVAL;
     int rc = launch_rotate_query(q, dtype, (int64_t)B * Hq, layer, q_rot, q_sk, q_stat, mfma_shape ? qa_pack : nullptr,
-                                 G, sm_scale, st);
+                                 mfma_shape ? Gq : G, sm_scale, st);
     if (rc) return rc;
   }
   if (!(stages & 6)) return TQ_OK;
@@ -384,8 +390,9 @@ extern "C" int tq_decode_attn_paged_stages(const void* q, int dtype, int B, int 
   dim3 grid(n_split, Hkv, B), block(DEC_WAVES * 64);
   int mf = TQ_EUNSUPPORTED;
   if (stages & 2)
-    mf = launch_decode_mfma(qa_pack, q_stat, B, Hq, Hkv, pool, block_table, bt_stride, seq_lens, sm_scale, *layer,
-                            *layout, parts, n_parts, n_split, st);
+    mf = mfma_shape ? launch_decode_mfma(qa_pack, q_stat, B, Hq, Hkv * kv_div, kv_div, pool, block_table, bt_stride,
+                                         seq_lens, sm_scale, *layer, *layout, parts, n_parts, n_split, st)
+                    : TQ_EUNSUPPORTED;
   if (mf > 0) return mf;
   if ((stages & 2) && mf == TQ_EUNSUPPORTED) {      // no matrix-core kernel for this shape: general kernel
 #define TQ_LAUNCH_DEC(VB)                                                                                 \

@@ -162,7 +162,8 @@ __device__ __forceinline__ constexpr int v_bitpos(int t) {
 // channels); WPS wavefronts per SIMD the register budget is sized for.
 template <int D, int MB, int NX, int VB, int GS, int DS, int WPS, bool F16P>
 __global__ void __launch_bounds__(MF_WAVES * 64, WPS)
-decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict__ q_stat, int Hq, int Hkv, const uint8_t* __restrict__ pool, const int32_t* __restrict__ block_table,
+decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict__ q_stat, int Hq, int Hkv, int kv_div,
+                   const uint8_t* __restrict__ pool, const int32_t* __restrict__ block_table,
                    int bt_stride, const int32_t* __restrict__ seq_lens, float sm_scale, tq_layer ly, tq_page_layout L,
                    float* __restrict__ parts, int n_parts, int n_split) {
   constexpr int DW = D / DS;                  // coordinates / channels of one wavefront
@@ -178,7 +179,9 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
   constexpr int NGRP = MF_WAVES / DS;         // wavefront groups (each walks its own blocks)
   constexpr int WAVE_LDS_FLOATS = wave_lds_floats(NG, DS);
   static_assert(WPL >= 1 && NG >= 2 && NG % 2 == 0, "a wavefront takes at least 128 coordinates and whole group pairs");
-  const int G = Hq / Hkv;                     // <= 8
+  // Hkv counts query-head groups: a KV head with more than 8 query heads is served by kv_div groups
+  // of G <= 8 heads each (consecutive groups read the same pages)
+  const int G = Hq / Hkv;
   const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -257,8 +260,8 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
   const int blk_begin = split * per_split;
   const int blk_end = min(n_blocks, blk_begin + per_split);
   const int32_t* bt = block_table + (int64_t)b * bt_stride;
-  const uint8_t* pool_h = pool + (int64_t)h * L.page_bytes;
-  const int64_t page_stride = (int64_t)Hkv * L.page_bytes;
+  const uint8_t* pool_h = pool + (int64_t)(h / kv_div) * L.page_bytes;
+  const int64_t page_stride = (int64_t)(Hkv / kv_div) * L.page_bytes;
   // per lane the key words are [word i][plane], the value fields [channel tile]: a wavefront's share is contiguous
   const uint32_t off_keys = L.off_keys + (lane * DS + hf) * (NKW * 4), off_meta = L.off_meta + n * 8;
   const uint32_t off_v = L.off_vdata + (n * DS + hf) * (VW * 4);
@@ -673,7 +676,7 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
 static thread_local hipEvent_t t_start_event = nullptr, t_stop_event = nullptr;
 
 template <int D, int MB, int NX, int VB, int GS, int DS, int WPS, bool F16P>
-static int launch_one(const uint32_t* qa_pack, const float* q_stat, int B, int Hq, int Hkv,
+static int launch_one(const uint32_t* qa_pack, const float* q_stat, int B, int Hq, int Hkv, int kv_div,
                       const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
                       float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts, int n_split,
                       hipStream_t st) {
@@ -688,11 +691,11 @@ static int launch_one(const uint32_t* qa_pack, const float* q_stat, int B, int H
   }
   if (t_start_event || t_stop_event) {
     hipExtLaunchKernelGGL(kern, dim3(n_split, Hkv, B), dim3(MF_WAVES * 64), smem, st, t_start_event, t_stop_event, 0,
-                          qa_pack, q_stat, Hq, Hkv, pool, block_table, bt_stride, seq_lens, sm_scale, ly, L, parts,
+                          qa_pack, q_stat, Hq, Hkv, kv_div, pool, block_table, bt_stride, seq_lens, sm_scale, ly, L, parts,
                           n_parts, n_split);
     t_start_event = t_stop_event = nullptr;
   } else {
-    kern<<<dim3(n_split, Hkv, B), dim3(MF_WAVES * 64), smem, st>>>(qa_pack, q_stat, Hq, Hkv, pool, block_table,
+    kern<<<dim3(n_split, Hkv, B), dim3(MF_WAVES * 64), smem, st>>>(qa_pack, q_stat, Hq, Hkv, kv_div, pool, block_table,
                                                                    bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts,
                                                                    n_split);
   }
@@ -705,7 +708,7 @@ static int launch_one(const uint32_t* qa_pack, const float* q_stat, int B, int H
 // words of packed query operands tq_decode_attn_paged reserves in its workspace
 size_t decode_mfma_pack_words(int B, int Hq, int d) { return (size_t)B * Hq * 9 * (d / 128 + 1) * 1024; }
 
-int launch_decode_mfma(const uint32_t* qa_pack, const float* q_stat, int B, int Hq, int Hkv,
+int launch_decode_mfma(const uint32_t* qa_pack, const float* q_stat, int B, int Hq, int Hkv, int kv_div,
                        const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
                        float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts,
                        int n_split, hipStream_t st) {
@@ -718,10 +721,10 @@ int launch_decode_mfma(const uint32_t* qa_pack, const float* q_stat, int B, int 
 #define TQ_TRY(D_, MB_, NX_, VB_, GS_, DS_, WPS_)                                                               \
   if (d == D_ && mb == MB_ && nx == NX_ && vb == VB_ && gs == GS_) {                                            \
     if (f16p)                                                                                                   \
-      return launch_one<D_, MB_, NX_, VB_, GS_, DS_, WPS_, true>(qa_pack, q_stat, B, Hq, Hkv, pool, block_table,  \
+      return launch_one<D_, MB_, NX_, VB_, GS_, DS_, WPS_, true>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,  \
                                                                  bt_stride, seq_lens, sm_scale, ly, L, parts,     \
                                                                  n_parts, n_split, st);                          \
-    return launch_one<D_, MB_, NX_, VB_, GS_, DS_, WPS_, false>(qa_pack, q_stat, B, Hq, Hkv, pool, block_table,   \
+    return launch_one<D_, MB_, NX_, VB_, GS_, DS_, WPS_, false>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,   \
                                                                 bt_stride, seq_lens, sm_scale, ly, L, parts,      \
                                                                 n_parts, n_split, st);                           \
   }
