@@ -328,7 +328,11 @@ def main():
 
     backend = None
     if not args.no_backend_step:
-        backend = backend_step_bench(device, max(5, args.steps // 10), max(2, args.warmup // 10))
+        try:                     # a secondary leg (needs ~60 GB): its failure must not cost the headline line
+            backend = backend_step_bench(device, max(5, args.steps // 10), max(2, args.warmup // 10))
+        except Exception as exc:                                     # noqa: BLE001
+            backend = {"error": f"{type(exc).__name__}: {exc}"}
+            torch.cuda.empty_cache()
 
     cpu = None
     if not args.no_cpu:
