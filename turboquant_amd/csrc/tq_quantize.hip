@@ -396,7 +396,7 @@ value_chunk_kernel(const void* __restrict__ v, Source src, int d, int gs, Sink s
   for (int i = 0; i < 8; ++i) {
     const float a = round_hw<DT>(x[i] - z);
     float quo;
-    if (fast_div && fabsf(a) < 0x1p60f) {
+    if (fast_div) {              // every a of the group is finite and at most (levels + 1) * sc < 2^64 then
       const float q0 = a * rsc;
       quo = fmaf(fmaf(-q0, sc, a), rsc, q0);
     } else {
@@ -404,8 +404,10 @@ value_chunk_kernel(const void* __restrict__ v, Source src, int d, int gs, Sink s
     }
     float q = round_hw<DT>(quo);
     q = rintf(q);
-    q = fminf(fmaxf(q, 0.0f), levels);
-    const uint32_t c = (q != q) ? 0u : (uint32_t)q;
+    // clamp to [0, levels]; a NaN becomes code 0 (the median-of-three instruction returns the minimum of
+    // its operands when one of them is a NaN)
+    q = __builtin_amdgcn_fmed3f(q, 0.0f, levels);
+    const uint32_t c = (uint32_t)q;
     codes |= c << (VB * i);
     if constexpr (!std::is_same<Sink, ValFlatSink>::value) scode[t * d + ck * 8 + i] = (uint8_t)c;
   }
