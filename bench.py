@@ -95,7 +95,7 @@ class DecodeWorkload:
             self.pools.append(p)
         self.q = torch.randn(B, Hq, d, generator=gen, device=device).bfloat16()
         self.seq = torch.full((B,), N, dtype=torch.int32, device=device)
-        self.n_split = first.default_splits(B, N)
+        self.n_split = first.default_splits(B, N, Hq)
         self.ws = first.workspace(B, Hq, self.n_split)
         self.out = torch.empty_like(self.q)
         self.bytes = B * Hkv * N * algorithmic_bytes_per_token_head(d, key_bits - 1, value_bits, 32)

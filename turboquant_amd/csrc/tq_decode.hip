@@ -16,40 +16,65 @@
 namespace tq {
 
 constexpr int G_MAX = 16;      // query heads per KV head handled by one workgroup
-constexpr int DEC_WAVES = 4;
 constexpr float NEG_BIG = -1.0e30f;
 
-// index of coordinate c in the LDS query tile [d][G] with a 4-float skew per 32
-// coordinates so that the four coordinate quarters of a wave hit distinct banks
-__device__ __forceinline__ int qoff(int c, int G) { return c * G + (c >> 5) * 4; }
+// General page kernel (vector ALU) for the shapes without a matrix-core kernel: any head_dim that is a
+// multiple of 64, 1..4-bit indices, 2/4-bit values, fp16 / bf16 / fp32 pools, up to G_MAX query heads per
+// KV head.  A workgroup of 256 threads walks its pages in chunks of 256 tokens (16 pages):
+//   scores   a thread per token: the key's plane words are read a word at a time, the rotated / sketched
+//            queries sit in LDS as [coordinate][GP] rows (GP = query heads rounded up to 4) so that one
+//            16-byte broadcast read feeds four heads;
+//   softmax  online over chunks: the chunk maxima per head come from a [16 heads][16 lanes] reduction;
+//   values   a thread per channel (and per slice of the chunk's tokens while head_dim < 256): codes from the
+//            channel's field, scale / zero per (group, token), weights from LDS, four heads per read.
+constexpr int GEN_THREADS = 256, GEN_CHUNK = 256;
 
-template <int VB>
-__global__ void __launch_bounds__(DEC_WAVES * 64)
+// 16 consecutive elements of the pool's dtype (a 16-byte aligned row) as fp32
+__device__ __forceinline__ void load_row16(const uint8_t* p, int dtype, float (&out)[16]) {
+  if (dtype == TQ_F32) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const float4 v = reinterpret_cast<const float4*>(p)[q];
+      out[4 * q] = v.x; out[4 * q + 1] = v.y; out[4 * q + 2] = v.z; out[4 * q + 3] = v.w;
+    }
+  } else {
+    const uint4 a = reinterpret_cast<const uint4*>(p)[0], b = reinterpret_cast<const uint4*>(p)[1];
+    const uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      out[2 * q] = dtype == TQ_BF16 ? __uint_as_float(w[q] << 16) : f16_bits_to_f32((uint16_t)(w[q] & 0xffffu));
+      out[2 * q + 1] = dtype == TQ_BF16 ? __uint_as_float(w[q] & 0xffff0000u) : f16_bits_to_f32((uint16_t)(w[q] >> 16));
+    }
+  }
+}
+
+template <int VB, int GP4>      // GP4 = GP / 4
+__global__ void __launch_bounds__(GEN_THREADS)
 decode_pages_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_sk, int Hq, int Hkv,
                     const uint8_t* __restrict__ pool, const int32_t* __restrict__ block_table, int bt_stride,
                     const int32_t* __restrict__ seq_lens, float sm_scale, tq_layer ly, tq_page_layout L,
                     float* __restrict__ parts, int n_parts, int n_split) {
+  constexpr int GP = 4 * GP4;
   const int d = ly.d, mb = ly.mse_bits, G = Hq / Hkv, words = d >> 5;
   const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int n = lane & 15, kb = lane >> 4;
-  const int cpl = d >> 6;   // channels per lane in the value stage
+  const int tid = threadIdx.x;
 
   extern __shared__ __align__(16) float smem[];
-  const int qsz = d * G + (d >> 5) * 4;
-  float* s_rot = smem;                  // [d][G] skewed
-  float* s_sk = s_rot + qsz;
-  float* s_cent = s_sk + qsz;           // [16]
-  float* s_p = s_cent + 16;             // [DEC_WAVES][G][16] softmax weights of the current page
-  float* s_red = s_p + DEC_WAVES * G * 16;   // cross-wave reduction: [DEC_WAVES][G][d + 2]
+  float* s_rot = smem;                       // [d][GP]
+  float* s_sk = s_rot + d * GP;              // [d][GP]
+  float* s_m = s_sk + d * GP;                // [16] chunk maxima
+  float* s_cent = s_m + 16;                  // [16]
+  float* s_p = s_cent + 16;                  // [GEN_CHUNK][GP] scores, then softmax weights
+  float* s_red = s_p;                        // after the loop: [TG][GP][d] partial accumulators
+  float* s_ml = s_rot;                       // after the loop: [TG][GP] weight sums, then [GP] maxima
 
-  for (int o = tid; o < d * G; o += blockDim.x) {
-    int g = o / d, c = o - g * d;
-    int64_t row = (int64_t)b * Hq + h * G + g;
-    s_rot[qoff(c, G) + g] = q_rot[row * d + c];
-    s_sk[qoff(c, G) + g] = q_sk[row * d + c];
+  for (int o = tid; o < d * GP; o += GEN_THREADS) {
+    const int c = o / GP, g = o - c * GP;
+    const int64_t row = (int64_t)b * Hq + h * G + (g < G ? g : 0);
+    s_rot[o] = g < G ? q_rot[row * d + c] : 0.0f;
+    s_sk[o] = g < G ? q_sk[row * d + c] : 0.0f;
   }
-  if (tid < (1 << mb)) s_cent[tid] = ly.centroids[tid];
+  if (tid < 16) s_cent[tid] = tid < (1 << mb) ? ly.centroids[tid] : 0.0f;
   __syncthreads();
 
   const int seq_len = seq_lens[b];
@@ -57,117 +82,177 @@ decode_pages_kernel(const float* __restrict__ q_rot, const float* __restrict__ q
   const int per_split = (n_pages + n_split - 1) / n_split;
   const int pg_begin = split * per_split;
   const int pg_end = min(n_pages, pg_begin + per_split);
+  const int32_t* bt = block_table + (int64_t)b * bt_stride;
+  const int64_t head_off = (int64_t)h * L.page_bytes, page_stride = (int64_t)Hkv * L.page_bytes;
 
-  float m[G_MAX], l[G_MAX], acc[G_MAX][12];
+  // value stage geometry: TG slices of the chunk's tokens while head_dim < 256, else several channels a thread
+  const int TG = d < GEN_THREADS ? GEN_THREADS / d : 1;          // 4 (d = 64), 2 (d = 128), 1
+  const int vch = tid % (d < GEN_THREADS ? d : GEN_THREADS), vtg = d < GEN_THREADS ? tid / d : 0;
+  const bool vactive = vtg < TG;                                  // d = 192: 64 threads have no slice
+  const int NCH = (d + GEN_THREADS - 1) / GEN_THREADS;            // channels per thread: 1, or up to 3 (d = 768)
+  constexpr int MAXCH = 3;
+  const int tok_per_tg = GEN_CHUNK / TG;
+  const int es = L.dtype == TQ_F32 ? 4 : 2;
+
+  float m_run[GP], l_run[GP], acc[MAXCH][GP];
 #pragma unroll
-  for (int g = 0; g < G_MAX; ++g) {
-    m[g] = NEG_BIG;
-    l[g] = 0.0f;
+  for (int g = 0; g < GP; ++g) {
+    m_run[g] = NEG_BIG;
+    l_run[g] = 0.0f;
 #pragma unroll
-    for (int c = 0; c < 12; ++c) acc[g][c] = 0.0f;
+    for (int k = 0; k < MAXCH; ++k) acc[k][g] = 0.0f;
   }
 
-  const int32_t* bt = block_table + (int64_t)b * bt_stride;
-  float* my_p = s_p + wave * G * 16;
-
-  for (int pi = pg_begin + wave; pi < pg_end; pi += DEC_WAVES) {
-    const uint8_t* pg = pool + ((int64_t)bt[pi] * Hkv + h) * (int64_t)L.page_bytes;
-    const int n_valid = min(TQ_PAGE_TOKENS, seq_len - pi * TQ_PAGE_TOKENS);
-
-    // ---- scores: lane (n, kb) covers coordinate words kb, kb+4, ... of token n
-    float pm[G_MAX], pq[G_MAX];
+  for (int pc = pg_begin; pc < pg_end; pc += GEN_CHUNK / TQ_PAGE_TOKENS) {
+    // ---- scores: thread = token pc * 16 + tid
+    {
+      const int pi = pc + (tid >> 4), n = tid & 15;
+      const bool valid = pi < pg_end && pi * TQ_PAGE_TOKENS + n < seq_len;
+      const uint8_t* pg = pool + (int64_t)bt[valid ? pi : pg_begin] * page_stride + head_off;
+      float pm[GP], pq[GP];
 #pragma unroll
-    for (int g = 0; g < G_MAX; ++g) pm[g] = pq[g] = 0.0f;
-    for (int w = kb; w < words; w += 4) {
-      uint32_t pw[5];
-      for (int p = 0; p <= mb; ++p) pw[p] = *(const uint32_t*)(pg + key_word_off(L, p, w, n));
-      for (int i = 0; i < 32; ++i) {
-        unsigned id = 0;
-        for (int p = 0; p < mb; ++p) id = (id << 1) | ((pw[p] >> i) & 1u);
-        float cv = s_cent[id];
-        float sg = ((pw[mb] >> i) & 1u) ? 1.0f : -1.0f;
-        const float* qr = s_rot + qoff(w * 32 + i, G);
-        const float* qs = s_sk + qoff(w * 32 + i, G);
+      for (int g = 0; g < GP; ++g) pm[g] = pq[g] = 0.0f;
+      for (int w = 0; w < words; ++w) {
+        uint32_t pw[5] = {0, 0, 0, 0, 0};
+        for (int p = 0; p <= mb; ++p) pw[p] = *(const uint32_t*)(pg + key_word_off(L, p, w, n));
+        const uint32_t sgw = pw[mb];
+        for (int i = 0; i < 32; ++i) {
+          unsigned id = 0;
+          for (int p = 0; p < mb; ++p) id = (id << 1) | ((pw[p] >> i) & 1u);
+          const float cv = s_cent[id];
+          const float sg = ((sgw >> i) & 1u) ? 1.0f : -1.0f;
+          const float4* qr = reinterpret_cast<const float4*>(s_rot + (w * 32 + i) * GP);
+          const float4* qs = reinterpret_cast<const float4*>(s_sk + (w * 32 + i) * GP);
 #pragma unroll
-        for (int g = 0; g < G_MAX; ++g) {
-          if (g < G) {
-            pm[g] = fmaf(qr[g], cv, pm[g]);
-            pq[g] = fmaf(qs[g], sg, pq[g]);
+          for (int g4 = 0; g4 < GP4; ++g4) {
+            const float4 r = qr[g4], k = qs[g4];
+            pm[4 * g4 + 0] = fmaf(r.x, cv, pm[4 * g4 + 0]);
+            pm[4 * g4 + 1] = fmaf(r.y, cv, pm[4 * g4 + 1]);
+            pm[4 * g4 + 2] = fmaf(r.z, cv, pm[4 * g4 + 2]);
+            pm[4 * g4 + 3] = fmaf(r.w, cv, pm[4 * g4 + 3]);
+            pq[4 * g4 + 0] = fmaf(k.x, sg, pq[4 * g4 + 0]);
+            pq[4 * g4 + 1] = fmaf(k.y, sg, pq[4 * g4 + 1]);
+            pq[4 * g4 + 2] = fmaf(k.z, sg, pq[4 * g4 + 2]);
+            pq[4 * g4 + 3] = fmaf(k.w, sg, pq[4 * g4 + 3]);
+          }
+        }
+      }
+      const float nk = ((const float*)(pg + L.off_meta))[2 * n];
+      const float rk = ly.qjl_scale * ((const float*)(pg + L.off_meta))[2 * n + 1];
+#pragma unroll
+      for (int g = 0; g < GP; ++g) s_p[tid * GP + g] = valid ? sm_scale * (nk * pm[g] + rk * pq[g]) : NEG_BIG;
+    }
+    __syncthreads();
+    // ---- chunk maxima: thread (g, j) scans tokens j, j + 16, ... of head g, then the 16 lanes of a head combine
+    {
+      const int g = tid >> 4, j = tid & 15;
+      float mx = NEG_BIG;
+      if (g < GP)
+        for (int t = j; t < GEN_CHUNK; t += 16) mx = fmaxf(mx, s_p[t * GP + g]);
+      for (int o = 8; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+      if (j == 0) s_m[g] = mx;
+    }
+    __syncthreads();
+    // ---- weights of the chunk against the new running maxima; the accumulators follow the maxima
+    {
+      float alpha[GP];
+#pragma unroll
+      for (int g = 0; g < GP; ++g) {
+        const float m_new = fmaxf(m_run[g], s_m[g]);
+        alpha[g] = __expf(m_run[g] - m_new);
+        m_run[g] = m_new;
+        l_run[g] *= alpha[g];
+#pragma unroll
+        for (int k = 0; k < MAXCH; ++k) acc[k][g] *= alpha[g];
+      }
+      const int pi = pc + (tid >> 4), n = tid & 15;
+      const bool valid = pi < pg_end && pi * TQ_PAGE_TOKENS + n < seq_len;
+#pragma unroll
+      for (int g = 0; g < GP; ++g) {
+        const float sc = s_p[tid * GP + g];
+        s_p[tid * GP + g] = valid ? __expf(sc - m_run[g]) : 0.0f;
+      }
+    }
+    __syncthreads();
+    // ---- values: thread = channel (x slice of the chunk's tokens)
+    if (vactive) {
+      const int t_begin = vtg * tok_per_tg, t_end = t_begin + tok_per_tg;
+      for (int t0 = t_begin; t0 < t_end; t0 += TQ_PAGE_TOKENS) {
+        const int pi = pc + (t0 >> 4);
+        if (pi >= pg_end) break;
+        const uint8_t* pg = pool + (int64_t)bt[pi] * page_stride + head_off;
+        const int n_valid = min(TQ_PAGE_TOKENS, seq_len - pi * TQ_PAGE_TOKENS);
+#pragma unroll
+        for (int k = 0; k < MAXCH; ++k) {
+          if (k < NCH) {
+            const int ch = vch + GEN_THREADS * k;
+            if (ch < d) {
+              const int grp = ch / L.group_size;
+              const uint32_t* field = (const uint32_t*)(pg + vfield_off(L, ch));
+              const uint32_t f0 = field[0], f1 = (VB == 4) ? field[1] : 0u;
+              // scales and zeros of the 16 tokens of this (page, group): two rows of 16 elements
+              float sc[16], zr[16];
+              load_row16(pg + L.off_vscale + grp * TQ_PAGE_TOKENS * es, L.dtype, sc);
+              load_row16(pg + L.off_vzero + grp * TQ_PAGE_TOKENS * es, L.dtype, zr);
+#pragma unroll
+              for (int t = 0; t < TQ_PAGE_TOKENS; ++t) {
+                unsigned code;
+                if (VB == 2) code = (f0 >> (2 * t)) & 3u;
+                else code = ((t < 8 ? f0 : f1) >> (4 * (t & 7))) & 15u;
+                // slots past the end of the sequence may hold anything: they contribute an exact zero
+                const float val = t < n_valid ? fmaf((float)code, sc[t], zr[t]) : 0.0f;
+                const float4* pp = reinterpret_cast<const float4*>(s_p + (t0 + t) * GP);
+#pragma unroll
+                for (int g4 = 0; g4 < GP4; ++g4) {
+                  const float4 w4 = pp[g4];
+                  acc[k][4 * g4 + 0] = fmaf(w4.x, val, acc[k][4 * g4 + 0]);
+                  acc[k][4 * g4 + 1] = fmaf(w4.y, val, acc[k][4 * g4 + 1]);
+                  acc[k][4 * g4 + 2] = fmaf(w4.z, val, acc[k][4 * g4 + 2]);
+                  acc[k][4 * g4 + 3] = fmaf(w4.w, val, acc[k][4 * g4 + 3]);
+                  if (k == 0) {        // the sum of the weights rides along (the same in every thread of a slice)
+                    l_run[4 * g4 + 0] += w4.x;
+                    l_run[4 * g4 + 1] += w4.y;
+                    l_run[4 * g4 + 2] += w4.z;
+                    l_run[4 * g4 + 3] += w4.w;
+                  }
+                }
+              }
+            }
           }
         }
       }
     }
-    const float nk = (n < n_valid) ? ((const float*)(pg + L.off_meta))[2 * n] : 0.0f;
-    const float rk = (n < n_valid) ? ly.qjl_scale * ((const float*)(pg + L.off_meta))[2 * n + 1] : 0.0f;
-#pragma unroll
-    for (int g = 0; g < G_MAX; ++g) {
-      if (g < G) {
-        float a = pm[g], c = pq[g];
-        a += __shfl_xor(a, 16, 64); a += __shfl_xor(a, 32, 64);
-        c += __shfl_xor(c, 16, 64); c += __shfl_xor(c, 32, 64);
-        float s = (n < n_valid) ? sm_scale * (nk * a + rk * c) : NEG_BIG;
-        // online softmax over the 16 tokens of the page (all 64 lanes hold a copy)
-        float tmax = s;
-        for (int o = 8; o > 0; o >>= 1) tmax = fmaxf(tmax, __shfl_xor(tmax, o, 64));
-        float m_new = fmaxf(m[g], tmax);
-        float alpha = __expf(m[g] - m_new);
-        float p = (n < n_valid) ? __expf(s - m_new) : 0.0f;
-        float psum = p;
-        for (int o = 8; o > 0; o >>= 1) psum += __shfl_xor(psum, o, 64);
-        l[g] = l[g] * alpha + psum;
-        m[g] = m_new;
-#pragma unroll
-        for (int c2 = 0; c2 < 12; ++c2) acc[g][c2] *= alpha;
-        if (kb == 0) my_p[g * 16 + n] = p;
-      }
-    }
-    __builtin_amdgcn_wave_barrier();
-    __threadfence_block();
-
-    // ---- values: lane owns channels lane, lane+64, ...
-#pragma unroll
-    for (int c2 = 0; c2 < 12; ++c2) {
-      if (c2 < cpl) {
-        const int ch = lane + 64 * c2, grp = ch / L.group_size;
-        const uint32_t* field = (const uint32_t*)(pg + vfield_off(L, ch));
-        uint32_t f0 = field[0], f1 = (VB == 4) ? field[1] : 0u;
-        const int es = L.dtype == TQ_F32 ? 4 : 2;
-        const uint8_t* sc_p = pg + L.off_vscale + grp * TQ_PAGE_TOKENS * es;
-        const uint8_t* zr_p = pg + L.off_vzero + grp * TQ_PAGE_TOKENS * es;
-        for (int t = 0; t < n_valid; ++t) {
-          unsigned code;
-          if (VB == 2) code = (f0 >> (2 * t)) & 3u;
-          else code = ((t < 8 ? f0 : f1) >> (4 * (t & 7))) & 15u;
-          float val = fmaf((float)code, load_as_f32(sc_p, t, L.dtype), load_as_f32(zr_p, t, L.dtype));
-#pragma unroll
-          for (int g = 0; g < G_MAX; ++g)
-            if (g < G) acc[g][c2] = fmaf(my_p[g * 16 + t], val, acc[g][c2]);
-        }
-      }
-    }
-    __builtin_amdgcn_wave_barrier();
+    __syncthreads();                          // s_p is rewritten by the next chunk
   }
 
-  // ---- merge the four waves of the workgroup, then write the partial
-  for (int g = 0; g < G; ++g) {
-    float* r = s_red + ((wave * G) + g) * (d + 2);
-    if (lane == 0) { r[0] = m[g]; r[1] = l[g]; }
-    for (int c2 = 0; c2 < cpl; ++c2) r[2 + lane + 64 * c2] = acc[g][c2];
+  // ---- combine the token slices and write the partial (all threads share the same running maxima)
+  if (vactive) {
+#pragma unroll
+    for (int k = 0; k < MAXCH; ++k) {
+      if (k < NCH) {
+        const int ch = vch + GEN_THREADS * k;
+        if (ch < d)
+#pragma unroll
+          for (int g = 0; g < GP; ++g) s_red[(vtg * GP + g) * d + ch] = acc[k][g];
+      }
+    }
+    if (vch == 0)
+#pragma unroll
+      for (int g = 0; g < GP; ++g) s_ml[vtg * GP + g] = l_run[g];
   }
+  if (tid == 0)
+#pragma unroll
+    for (int g = 0; g < GP; ++g) s_ml[4 * GP + g] = m_run[g];
   __syncthreads();
-  for (int o = tid; o < G * d; o += blockDim.x) {
-    int g = o / d, ch = o - g * d;
-    float mm = NEG_BIG;
-    for (int w = 0; w < DEC_WAVES; ++w) mm = fmaxf(mm, s_red[((w * G) + g) * (d + 2)]);
-    float ll = 0.0f, aa = 0.0f;
-    for (int w = 0; w < DEC_WAVES; ++w) {
-      const float* r = s_red + ((w * G) + g) * (d + 2);
-      float wgt = __expf(r[0] - mm);
-      ll += wgt * r[1];
-      aa += wgt * r[2 + ch];
+  for (int o = tid; o < G * d; o += GEN_THREADS) {
+    const int g = o / d, ch = o - g * d;
+    float aa = 0.0f, ll = 0.0f;
+    for (int t = 0; t < TG; ++t) {
+      aa += s_red[(t * GP + g) * d + ch];
+      ll += s_ml[t * GP + g];
     }
     float* out = parts + (((int64_t)b * Hq + h * G + g) * n_parts + split) * (d + 2);
-    if (ch == 0) { out[0] = mm; out[1] = ll; }
+    if (ch == 0) { out[0] = s_ml[4 * GP + g]; out[1] = ll; }
     out[2 + ch] = aa;
   }
 }
@@ -385,9 +470,6 @@ extern "C" int tq_decode_attn_paged_stages(const void* q, int dtype, int B, int 
   }
   if (!(stages & 6)) return TQ_OK;
 
-  const int qsz = d * G + (d >> 5) * 4;
-  size_t smem = (size_t)(2 * qsz + 16 + DEC_WAVES * G * 16 + DEC_WAVES * G * (d + 2)) * sizeof(float);
-  dim3 grid(n_split, Hkv, B), block(DEC_WAVES * 64);
   int mf = TQ_EUNSUPPORTED;
   if (stages & 2)
     mf = mfma_shape ? launch_decode_mfma(qa_pack, q_stat, B, Hq, Hkv * kv_div, kv_div, pool, block_table, bt_stride,
@@ -395,9 +477,15 @@ extern "C" int tq_decode_attn_paged_stages(const void* q, int dtype, int B, int 
                     : TQ_EUNSUPPORTED;
   if (mf > 0) return mf;
   if ((stages & 2) && mf == TQ_EUNSUPPORTED) {      // no matrix-core kernel for this shape: general kernel
-#define TQ_LAUNCH_DEC(VB)                                                                                 \
+    if (dtype < TQ_F32 || dtype > TQ_BF16) return TQ_EINVAL;
+    const int gp4 = (G + 3) / 4, gp = 4 * gp4;      // query heads rounded up to a multiple of 4
+    const int tg = d < GEN_THREADS ? GEN_THREADS / d : 1;
+    const size_t work = (size_t)gp * (GEN_CHUNK > tg * d ? GEN_CHUNK : tg * d);    // weights, then slice partials
+    const size_t smem = ((size_t)2 * d * gp + 32 + work) * sizeof(float);
+    dim3 grid(n_split, Hkv, B), block(GEN_THREADS);
+#define TQ_LAUNCH_DEC(VB, GP4)                                                                            \
   {                                                                                                       \
-    auto kern = decode_pages_kernel<VB>;                                                                  \
+    auto kern = decode_pages_kernel<VB, GP4>;                                                             \
     if (smem > 48 * 1024) {                                                                               \
       hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem); \
       if (e != hipSuccess) return (int)e;                                                                 \
@@ -405,9 +493,16 @@ extern "C" int tq_decode_attn_paged_stages(const void* q, int dtype, int B, int 
     kern<<<grid, block, smem, st>>>(q_rot, q_sk, Hq, Hkv, pool, block_table, bt_stride, seq_lens, sm_scale, *layer,  \
                                     *layout, parts, n_parts, n_split);                                    \
   }
-  if (dtype < TQ_F32 || dtype > TQ_BF16) return TQ_EINVAL;
-  if (layout->value_bits == 2) TQ_LAUNCH_DEC(2)
-  else TQ_LAUNCH_DEC(4)
+#define TQ_LAUNCH_DEC_G(VB)                                                      \
+  {                                                                              \
+    if (gp4 == 1) TQ_LAUNCH_DEC(VB, 1)                                           \
+    else if (gp4 == 2) TQ_LAUNCH_DEC(VB, 2)                                      \
+    else if (gp4 == 3) TQ_LAUNCH_DEC(VB, 3)                                      \
+    else TQ_LAUNCH_DEC(VB, 4)                                                    \
+  }
+    if (layout->value_bits == 2) TQ_LAUNCH_DEC_G(2)
+    else TQ_LAUNCH_DEC_G(4)
+#undef TQ_LAUNCH_DEC_G
 #undef TQ_LAUNCH_DEC
   TQ_CHECK_LAUNCH();
   }

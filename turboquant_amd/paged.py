@@ -139,13 +139,29 @@ class PagedKVPool:
                 v_zeros.data_ptr(), _ffi.stream_ptr(dev)), "tq_pool_export")
         return idx, signs, norms, rnorms, v_data, v_scales, v_zeros
 
-    def default_splits(self, B: int, max_len: int) -> int:
-        """Split count of the page-streaming kernel.  Its workgroups (4 wavefronts,
-        one per SIMD, each walking 64-token blocks) should number about two per CU
-        (256 CUs) while every wavefront still gets several blocks, because each
-        wavefront first builds its query operands."""
-        blocks = max(1, (max_len + 63) // 64)
+    def _matrix_core_shape(self, Hq: Optional[int]) -> bool:
+        """Whether decode runs on the matrix-core page kernel (head_dim 128 / 256, 16-bit pools, up to 4-bit
+        keys, query heads that split into groups of at most 8); only the split heuristic depends on it."""
+        if self.head_dim not in (128, 256) or self.dtype not in (torch.bfloat16, torch.float16):
+            return False
+        if self.quantizer.bits - 1 > 3 or self.value_bits not in (2, 4) or self.value_group_size not in (32, 64):
+            return False
+        if Hq is None:
+            return True
+        G = max(1, Hq // self.num_kv_heads)
+        return any(G % n == 0 and G // n <= 8 for n in range(1, G + 1))
+
+    def default_splits(self, B: int, max_len: int, Hq: Optional[int] = None) -> int:
+        """Split count of the page-streaming kernel.  Matrix-core kernel: its workgroups (4 wavefronts,
+        one per SIMD, each walking 64-token blocks) should number about two per CU (256 CUs) while every
+        wavefront still gets several blocks, because each wavefront first builds its query operands.
+        General kernel: it hides its memory latency by occupancy, so about eight workgroups per CU, each
+        with at least one 256-token chunk."""
         pairs = max(1, B * self.num_kv_heads)
+        if not self._matrix_core_shape(Hq):
+            chunks = max(1, (max_len + 255) // 256)
+            return int(max(1, min(2048 // pairs, chunks, 512)))
+        blocks = max(1, (max_len + 63) // 64)
         want = max(1, 512 // pairs)
         longest = max(1, blocks // 16)          # keep >= 4 blocks per wavefront
         return int(max(1, min(want, longest, 512)))
@@ -179,7 +195,7 @@ class PagedKVPool:
         if n_split is None:
             if max_len is None:
                 max_len = (bt.shape[-1]) * PAGE_TOKENS
-            n_split = self.default_splits(B, max_len)
+            n_split = self.default_splits(B, max_len, Hq)
         if workspace is None:
             workspace = self.workspace(B, Hq, n_split)
         if out is None:
