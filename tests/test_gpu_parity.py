@@ -558,7 +558,9 @@ def shape_kq_128(k, trend):
                                                          (256, 3, 2, 16, 2, torch.float16), (128, 4, 2, 6, 2, torch.float16),
                                                          (256, 4, 4, 8, 8, torch.float16), (128, 2, 4, 7, 1, torch.float16),
                                                          (128, 3, 4, 12, 1, torch.bfloat16), (256, 3, 2, 18, 2, torch.bfloat16),
-                                                         (128, 3, 2, 11, 1, torch.bfloat16), (128, 4, 4, 32, 2, torch.float16)])
+                                                         (128, 3, 2, 11, 1, torch.bfloat16), (128, 4, 4, 32, 2, torch.float16),
+                                                         (576, 3, 2, 16, 1, torch.bfloat16), (768, 2, 4, 4, 2, torch.float32),
+                                                         (192, 3, 4, 6, 2, torch.float16), (64, 5, 2, 10, 2, torch.bfloat16)])
 def test_decode_attention_general_kernel_shapes(gpu, d, key_bits, vb, Hq, Hkv, dtype):
     # fp16 pools (matrix-core kernel with the fp16 zero-point product), more than 8 query heads per KV head
     # (served as groups of at most 8: 16 = 2 x 8, 12 = 2 x 6, 9 = 3 x 3), and shapes without a
