@@ -257,51 +257,158 @@ decode_pages_kernel(const float* __restrict__ q_rot, const float* __restrict__ q
   }
 }
 
-// Partial (m, l, acc) over exact recent tokens (score.py:99-111, 138-173): one
-// workgroup of 128 threads per (KV head, sequence).
-__global__ void __launch_bounds__(128)
-exact_tail_kernel(const void* __restrict__ q, int dtype, int Hq, int Hkv, int d, const void* __restrict__ rk,
+// Partial (m, l, acc) over exact recent tokens (score.py:99-111, 138-173): one workgroup of 512 threads
+// per (KV head, sequence, group of TAIL_GC query heads).  Key rows, then value rows, are staged through an
+// LDS tile a chunk of tokens at a time with every load of a chunk in flight at once (the rows come from HBM:
+// a loop that waits for one row per iteration costs a memory latency per token).  Scores: eight threads per
+// token, each over every eighth coordinate for the group's heads at once; values: a thread per channel and
+// slice of the chunk's tokens.
+constexpr int TAIL_THREADS = 512, TAIL_WAVES = TAIL_THREADS / 64, TAIL_GC = 4, TAIL_TILE_FLOATS = 64 * 260;
+
+static size_t tail_smem(int d, int recent_rows) {
+  return ((size_t)TAIL_GC * d + (size_t)TAIL_GC * recent_rows + 2 * TAIL_GC + TAIL_TILE_FLOATS) * sizeof(float);
+}
+
+// (the element type is a template parameter: a run-time switch inside the load would put every load of
+// the staging loop under a branch and serialise them)
+template <int DT>
+__global__ void __launch_bounds__(TAIL_THREADS)
+exact_tail_kernel(const void* __restrict__ q, int Hq, int Hkv, int d, const void* __restrict__ rk,
                   const void* __restrict__ rv, int recent_rows, int64_t rs_b, int64_t rs_r, int64_t rs_h,
                   const int32_t* __restrict__ recent_len, float sm_scale, float* __restrict__ parts, int n_parts,
                   int part_index) {
-  const int G = Hq / Hkv, h = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
-  const int R = recent_len ? min(recent_len[b], recent_rows) : recent_rows;
-  extern __shared__ float sm[];
-  float* sq = sm;              // [G][d]
-  float* ss = sq + G * d;      // [G][recent_rows]
-  float* sml = ss + G * recent_rows;  // [G][2]
-  for (int o = tid; o < G * d; o += blockDim.x) sq[o] = load_as_f32(q, ((int64_t)b * Hq + h * G) * d + o, dtype);
-  __syncthreads();
-  for (int t = tid; t < R; t += blockDim.x) {
-    const int64_t base = b * rs_b + (int64_t)t * rs_r + h * rs_h;
-    for (int g = 0; g < G; ++g) {
-      float a = 0.0f;
-      for (int i = 0; i < d; ++i) a = fmaf(sq[g * d + i], load_as_f32(rk, base + i, dtype), a);
-      ss[g * recent_rows + t] = a * sm_scale;
-    }
-  }
-  __syncthreads();
+  constexpr int GC = TAIL_GC;
+  const int G = Hq / Hkv, h = blockIdx.x, b = blockIdx.y, g0 = blockIdx.z * GC, tid = threadIdx.x;
+  const int Gc = min(GC, G - g0);                                   // query heads of this workgroup
   const int lane = tid & 63, wave = tid >> 6;
-  for (int g = wave; g < G; g += 2) {
+  const int R = recent_len ? min(recent_len[b], recent_rows) : recent_rows;
+  extern __shared__ __align__(16) float sm[];
+  float* sq = sm;                      // [d][GC]
+  float* ss = sq + GC * d;             // [recent_rows][GC] scores, then softmax weights
+  float* sml = ss + GC * recent_rows;  // [GC][2]
+  float* tile = sml + 2 * GC;          // [CH][d + 1] rows of the current chunk; at the end [TS][GC][d] partials
+  const int ld = d + 1;
+  const int CH = min(TAIL_TILE_FLOATS / ld, 32 * (d < TAIL_THREADS ? TAIL_THREADS / d : 1));   // 21 tokens (d = 768) .. 252 (d = 64)
+  // thread = column x row slice (rows ts, ts + TS, ...) for staging and for the value sums; a head
+  // dimension above 512 gives a thread two columns
+  const int TS = d < TAIL_THREADS ? TAIL_THREADS / d : 1;
+  const int ch0 = d < TAIL_THREADS ? tid % d : tid, ts = d < TAIL_THREADS ? tid / d : 0;
+  const bool active = ts < TS;
+  const int64_t base0 = b * rs_b + h * rs_h;
+  auto stage = [&](const void* src, int c0, int n) {                // rows c0 .. c0 + n - 1 -> tile
+    if (active) {
+#pragma unroll
+      for (int k = 0; k < 2; ++k) {
+        const int ch = ch0 + TAIL_THREADS * k;
+        if (ch < d) {
+          // a thread has at most 32 rows of a chunk (CH / TS): all of its loads are issued before the first store
+          float v[32];
+#pragma unroll
+          for (int i = 0; i < 32; ++i) {
+            const int t = ts + i * TS;
+            v[i] = Elem<DT>::load(src, base0 + (int64_t)(c0 + (t < n ? t : 0)) * rs_r + ch);
+          }
+#pragma unroll
+          for (int i = 0; i < 32; ++i) {
+            const int t = ts + i * TS;
+            if (t < n) tile[t * ld + ch] = v[i];
+          }
+        }
+      }
+    }
+  };
+  for (int o = tid; o < GC * d; o += TAIL_THREADS) {
+    const int g = o / d, c = o - g * d;
+    sq[c * GC + g] = g < Gc ? Elem<DT>::load(q, ((int64_t)b * Hq + h * G + g0) * d + o) : 0.0f;
+  }
+  // scores
+  for (int c0 = 0; c0 < R; c0 += CH) {
+    const int n = min(CH, R - c0);
+    stage(rk, c0, n);
+    __syncthreads();
+    const int seg = tid & 7;
+    for (int t0 = 0; t0 < n; t0 += TAIL_THREADS / 8) {              // uniform trip count: the shuffles need every lane
+      const int t = t0 + (tid >> 3);
+      const float* row = tile + (t < n ? t : 0) * ld;
+      float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
+      for (int c = seg; c < d; c += 8) {
+        const float kx = row[c];
+        const float4 q4 = *reinterpret_cast<const float4*>(sq + c * GC);
+        a0 = fmaf(kx, q4.x, a0);
+        a1 = fmaf(kx, q4.y, a1);
+        a2 = fmaf(kx, q4.z, a2);
+        a3 = fmaf(kx, q4.w, a3);
+      }
+#pragma unroll
+      for (int o = 4; o > 0; o >>= 1) {
+        a0 += __shfl_xor(a0, o, 64);
+        a1 += __shfl_xor(a1, o, 64);
+        a2 += __shfl_xor(a2, o, 64);
+        a3 += __shfl_xor(a3, o, 64);
+      }
+      if (seg == 0 && t < n)
+        *reinterpret_cast<float4*>(ss + (c0 + t) * GC) = make_float4(a0 * sm_scale, a1 * sm_scale, a2 * sm_scale, a3 * sm_scale);
+    }
+    __syncthreads();
+  }
+  // softmax statistics and weights, a wavefront per query head
+  for (int g = wave; g < GC; g += TAIL_WAVES) {
     float mx = NEG_BIG;
-    for (int t = lane; t < R; t += 64) mx = fmaxf(mx, ss[g * recent_rows + t]);
+    for (int t = lane; t < R; t += 64) mx = fmaxf(mx, ss[t * GC + g]);
     mx = wave_max(mx);
     float sum = 0.0f;
     for (int t = lane; t < R; t += 64) {
-      float p = __expf(ss[g * recent_rows + t] - mx);
-      ss[g * recent_rows + t] = p;
+      float p = __expf(ss[t * GC + g] - mx);
+      ss[t * GC + g] = p;
       sum += p;
     }
     sum = wave_sum(sum);
     if (lane == 0) { sml[g * 2] = mx; sml[g * 2 + 1] = sum; }
   }
   __syncthreads();
-  for (int o = tid; o < G * d; o += blockDim.x) {
-    int g = o / d, ch = o - g * d;
+  // values
+  float acc[2][GC];
+#pragma unroll
+  for (int k = 0; k < 2; ++k)
+#pragma unroll
+    for (int g = 0; g < GC; ++g) acc[k][g] = 0.0f;
+  for (int c0 = 0; c0 < R; c0 += CH) {
+    const int n = min(CH, R - c0);
+    stage(rv, c0, n);
+    __syncthreads();
+    if (active) {
+#pragma unroll
+      for (int k = 0; k < 2; ++k) {
+        const int ch = ch0 + TAIL_THREADS * k;
+        if (ch < d) {
+          for (int t = ts; t < n; t += TS) {
+            const float v = tile[t * ld + ch];
+            const float4 w4 = *reinterpret_cast<const float4*>(ss + (c0 + t) * GC);
+            acc[k][0] = fmaf(w4.x, v, acc[k][0]);
+            acc[k][1] = fmaf(w4.y, v, acc[k][1]);
+            acc[k][2] = fmaf(w4.z, v, acc[k][2]);
+            acc[k][3] = fmaf(w4.w, v, acc[k][3]);
+          }
+        }
+      }
+    }
+    __syncthreads();
+  }
+  if (active) {
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      const int ch = ch0 + TAIL_THREADS * k;
+      if (ch < d)
+#pragma unroll
+        for (int g = 0; g < GC; ++g) tile[(ts * GC + g) * d + ch] = acc[k][g];
+    }
+  }
+  __syncthreads();
+  for (int o = tid; o < Gc * d; o += TAIL_THREADS) {
+    const int g = o / d, ch = o - g * d;
     float a = 0.0f;
-    for (int t = 0; t < R; ++t)
-      a = fmaf(ss[g * recent_rows + t], load_as_f32(rv, b * rs_b + (int64_t)t * rs_r + h * rs_h + ch, dtype), a);
-    float* out = parts + (((int64_t)b * Hq + h * G + g) * n_parts + part_index) * (d + 2);
+    for (int s2 = 0; s2 < TS; ++s2) a += tile[(s2 * GC + g) * d + ch];
+    float* out = parts + (((int64_t)b * Hq + h * G + g0 + g) * n_parts + part_index) * (d + 2);
     if (ch == 0) { out[0] = sml[g * 2]; out[1] = sml[g * 2 + 1]; }
     out[2 + ch] = a;
   }
@@ -508,14 +615,22 @@ extern "C" int tq_decode_attn_paged_stages(const void* q, int dtype, int B, int 
   }
 
   if (tail && (stages & 2)) {
-    size_t tsm = (size_t)(G * d + G * recent_rows + 2 * G) * sizeof(float);
-    auto kern = exact_tail_kernel;
-    if (tsm > 48 * 1024) {
-      hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)tsm);
-      if (e != hipSuccess) return (int)e;
-    }
-    kern<<<dim3(Hkv, B), dim3(128), tsm, st>>>(q, dtype, Hq, Hkv, d, recent_k, recent_v, recent_rows, rs_b, rs_r, rs_h,
-                                               recent_len, sm_scale, parts, n_parts, n_split);
+    size_t tsm = tail_smem(d, recent_rows);
+    const dim3 tgrid(Hkv, B, (G + TAIL_GC - 1) / TAIL_GC);
+#define TQ_LAUNCH_TAIL(DT)                                                                                           \
+  {                                                                                                                  \
+    auto kern = exact_tail_kernel<DT>;                                                                               \
+    if (tsm > 48 * 1024) {                                                                                           \
+      hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)tsm);   \
+      if (e != hipSuccess) return (int)e;                                                                            \
+    }                                                                                                                \
+    kern<<<tgrid, dim3(TAIL_THREADS), tsm, st>>>(q, Hq, Hkv, d, recent_k, recent_v, recent_rows, rs_b, rs_r, rs_h,    \
+                                                 recent_len, sm_scale, parts, n_parts, n_split);                     \
+  }
+    if (dtype == TQ_BF16) TQ_LAUNCH_TAIL(TQ_BF16)
+    else if (dtype == TQ_F16) TQ_LAUNCH_TAIL(TQ_F16)
+    else TQ_LAUNCH_TAIL(TQ_F32)
+#undef TQ_LAUNCH_TAIL
     TQ_CHECK_LAUNCH();
   }
   if (!(stages & 4)) return TQ_OK;
