@@ -148,6 +148,32 @@ def time_kernel_stage(work, steps, warmup):
     return sum(a.elapsed_time(b) for a, b in evs) / steps
 
 
+def stream_read_peak(work, steps, warmup):
+    """Read bandwidth the card delivers to a kernel that only reads (GB/s): tq_stream_read over the same
+    rotating pools the decode workload streams, best of a few launch shapes, timed with events on the
+    stream of the launches."""
+    import torch
+    from turboquant_amd import _ffi
+    lib = _ffi.lib()
+    st = torch.cuda.current_stream().cuda_stream
+    best = None
+    for wg_per_cu, flight in ((4, 4), (8, 4), (8, 1), (16, 1), (4, 8)):
+        def one(i):
+            pool = work.pools[i % len(work.pools)].data
+            nbytes = pool.numel() * pool.element_size() // 16 * 16
+            rc = lib.tq_stream_read(pool.data_ptr(), nbytes, wg_per_cu, flight, None, st)
+            if rc:
+                raise RuntimeError(f"tq_stream_read failed: {rc}")
+            return nbytes
+        nbytes = one(0)
+        ms, _ = time_steps(one, steps, warmup)
+        gbs = nbytes / (ms * 1e-3) / 1e9
+        if best is None or gbs > best["GBps"]:
+            best = {"GBps": gbs, "workgroups_per_cu": wg_per_cu, "loads_in_flight": flight, "bytes": nbytes,
+                    "us_per_launch": ms * 1e3}
+    return best
+
+
 def cpu_decode_baseline(work):
     """The oracle's de-quantise-all + dense attention on one sequence of the
     workload, on the host cores."""
@@ -312,6 +338,8 @@ def main():
     value = main_w.bytes / (ms * 1e-3) / 1e9
     achieved = main_w.bytes / (kern_ms * 1e-3) / 1e9
 
+    stream = stream_read_peak(main_w, max(20, args.steps // 4), max(5, args.warmup // 5))
+
     traffic = None
     tpath = os.path.join(ROOT, "profiles", "decode_pages_traffic.json")
     if os.path.exists(tpath):
@@ -357,7 +385,8 @@ def main():
         "wall_ms_per_step": wall,
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": traffic, "kernel": "decode_mfma_kernel",
-                     "kernel_ms": kern_ms},
+                     "kernel_ms": kern_ms, "stream_read": stream,
+                     "frac_of_stream_read": achieved / stream["GBps"]},
         "quantize": quant,
         "decode_gqa": {"workload": "16 seq x 8192 ctx, 32 q heads / 8 KV heads, head_dim 128, keys 3b, values 4b",
                        "GBps": gqa_w.bytes / (gqa_ms * 1e-3) / 1e9, "ms_per_step": gqa_ms,

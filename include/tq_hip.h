@@ -242,6 +242,14 @@ int tq_decode_merge(const float *parts, int64_t rows, int n_parts, int d, int dt
  * stream, which also contains the dispatch gap.  Pass NULLs to disarm.                             */
 void tq_time_next_page_kernel(void *start_event, void *stop_event);
 
+/* Measurement aid (no counterpart in the reference).  Reads `bytes` (a multiple of 16) from `src`
+ * (16-byte aligned) with `workgroups_per_cu` workgroups of 256 lanes per compute unit, each lane keeping
+ * `loads_in_flight` (1, 4 or 8) 16-byte loads outstanding, and writes nothing (`sink`, 4 bytes, may be
+ * NULL).  Timed over a buffer larger than the caches it gives the read bandwidth the card really
+ * delivers, against which the page-streaming kernels are reported beside the vendor's peak.          */
+int tq_stream_read(const void *src, size_t bytes, int workgroups_per_cu, int loads_in_flight,
+                   uint32_t *sink, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

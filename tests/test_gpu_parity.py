@@ -938,3 +938,22 @@ def test_kv_cache_object_against_reference_golden(gpu, golden):
     assert cosine(out, torch.from_numpy(z["out"])) >= COS_GATE
     mem = cache.memory_bytes()
     assert [mem[n] for n in ("quantized_keys", "quantized_values", "buffer", "total")] == z["memory"].tolist()
+
+
+def test_stream_read_probe_runs_and_rejects_bad_arguments(gpu):
+    # the read-only probe behind the bench's "fraction of streaming-read bandwidth": argument checks and a
+    # launch that completes (it writes nothing, so there is no output to compare)
+    from turboquant_amd import _ffi
+    lib = _ffi.lib()
+    buf = torch.ones(1 << 22, dtype=torch.uint8, device=gpu)
+    st = torch.cuda.current_stream().cuda_stream
+    for flight in (1, 4, 8):
+        assert lib.tq_stream_read(buf.data_ptr(), buf.numel(), 4, flight, None, st) == 0
+    assert lib.tq_stream_read(buf.data_ptr(), 16 * 1000 + 16, 2, 4, None, st) == 0      # tail shorter than a round
+    assert lib.tq_stream_read(buf.data_ptr(), 0, 4, 4, None, st) == 0
+    torch.cuda.synchronize()
+    assert lib.tq_stream_read(None, 16, 4, 4, None, st) < 0
+    assert lib.tq_stream_read(buf.data_ptr() + 4, 16, 4, 4, None, st) < 0
+    assert lib.tq_stream_read(buf.data_ptr(), 24, 4, 4, None, st) < 0
+    assert lib.tq_stream_read(buf.data_ptr(), 16, 4, 3, None, st) < 0
+    assert lib.tq_stream_read(buf.data_ptr(), 16, 0, 4, None, st) < 0

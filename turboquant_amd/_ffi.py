@@ -73,6 +73,7 @@ _SIGNATURES = {
                                               _i, _vp]),
     "tq_decode_merge": (C.c_int, [_vp, _i64, _i, _i, _i, _vp, _vp]),
     "tq_time_next_page_kernel": (None, [_vp, _vp]),
+    "tq_stream_read": (C.c_int, [_vp, C.c_size_t, _i, _i, _vp, _vp]),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)

@@ -13,7 +13,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libtq_hip.so")
-SOURCES = ["tq_quantize.hip", "tq_quantize_mfma.hip", "tq_score.hip", "tq_decode.hip", "tq_decode_mfma.hip"]
+SOURCES = ["tq_quantize.hip", "tq_quantize_mfma.hip", "tq_score.hip", "tq_decode.hip", "tq_decode_mfma.hip", "tq_probe.hip"]
 
 # packed-fp32 instructions stay off: some of their forms have produced wrong
 # results on this hardware pool
