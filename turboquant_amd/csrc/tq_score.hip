@@ -122,9 +122,11 @@ __device__ __forceinline__ float wave_sum_dpp(float v) {
          __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 32)) + __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48));
 }
 
-template <int PER>      // matrix rows per thread = d / PREP_SLICES
+// PER = matrix rows per thread = d / PREP_SLICES; DT = element type of the query (a template parameter:
+// a run-time switch would put each query load under a branch, and the loads would wait for one another)
+template <int PER, int DT>
 __global__ void __launch_bounds__(PREP_COLS * PREP_SLICES)
-prep_query_kernel(const void* __restrict__ q, int dtype, int G, tq_layer ly, float sm_scale,
+prep_query_kernel(const void* __restrict__ q, int G, tq_layer ly, float sm_scale,
                   float* __restrict__ q_rot, float* __restrict__ q_sk, float* __restrict__ q_stat,
                   uint32_t* __restrict__ qa_pack) {
   extern __shared__ float sm[];
@@ -139,7 +141,8 @@ prep_query_kernel(const void* __restrict__ q, int dtype, int G, tq_layer ly, flo
 #pragma unroll
   for (int k = 0; k < QPT; ++k) {
     const int o = tid + k * (PREP_COLS * PREP_SLICES);
-    qv[k] = o < G * d ? load_as_f32(q, row0 * d + o, dtype) : 0.0f;
+    const float x = Elem<DT>::load(q, row0 * d + min(o, G * d - 1));      // unconditional, clamped
+    qv[k] = o < G * d ? x : 0.0f;
   }
   float mp[PER], ms[PER];
 #pragma unroll
@@ -590,8 +593,18 @@ int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* 
     size_t smem = (size_t)(G * d + 2 * PREP_SLICES * G * PREP_COLS + 2 * G * PREP_COLS + 4 * ROT_MAX_ROWS + 32) *
                   sizeof(float);
     const dim3 grid((unsigned)(rows / G), d / PREP_COLS), block(PREP_COLS * PREP_SLICES);
-    if (d == 128) prep_query_kernel<8><<<grid, block, smem, st>>>(q, dtype, G, *layer, sm_scale, q_rot, q_sk, q_stat, qa_pack);
-    else prep_query_kernel<16><<<grid, block, smem, st>>>(q, dtype, G, *layer, sm_scale, q_rot, q_sk, q_stat, qa_pack);
+#define TQ_PREP(PER, DT) prep_query_kernel<PER, DT><<<grid, block, smem, st>>>(q, G, *layer, sm_scale, q_rot, q_sk, q_stat, qa_pack)
+#define TQ_PREP_DT(PER)                              \
+  {                                                  \
+    if (dtype == TQ_BF16) TQ_PREP(PER, TQ_BF16);     \
+    else if (dtype == TQ_F16) TQ_PREP(PER, TQ_F16);  \
+    else if (dtype == TQ_F32) TQ_PREP(PER, TQ_F32);  \
+    else return TQ_EINVAL;                           \
+  }
+    if (d == 128) TQ_PREP_DT(8)
+    else TQ_PREP_DT(16)
+#undef TQ_PREP_DT
+#undef TQ_PREP
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? TQ_OK : (int)e;
   }
