@@ -451,7 +451,7 @@ def _store_from_oracle_view(pool, table_row, n_tok):
 
 
 def _decode_case(gpu, d, key_bits, vb, B, Hq, Hkv, lens, recent, seed, n_split=None, dtype=torch.bfloat16,
-                 shape_kq=None):
+                 shape_kq=None, recent_pad=0):
     g = torch.Generator().manual_seed(seed)
     max_len = max(max(lens), 1)
     pages_per_seq = (max_len + 15) // 16
@@ -472,8 +472,14 @@ def _decode_case(gpu, d, key_bits, vb, B, Hq, Hkv, lens, recent, seed, n_split=N
         rv = torch.randn(B, max(recent), Hkv, d, generator=g).to(dtype)
         rl = torch.tensor(recent, dtype=torch.int32)
     seq = torch.tensor(lens, dtype=torch.int32)
-    out = pool.decode_attention(q.to(gpu), table, seq.to(gpu), recent_k=None if rk is None else rk.to(gpu),
-                                recent_v=None if rv is None else rv.to(gpu),
+    rk_dev, rv_dev = (None, None) if rk is None else (rk.to(gpu), rv.to(gpu))
+    if rk is not None and recent_pad:
+        # rows inside a wider buffer, starting `recent_pad` elements in: strided, and not word-aligned when odd
+        wide = [torch.zeros(B, max(recent), Hkv, d + 2 * recent_pad, dtype=dtype, device=gpu) for _ in range(2)]
+        wide[0][..., recent_pad:recent_pad + d] = rk_dev
+        wide[1][..., recent_pad:recent_pad + d] = rv_dev
+        rk_dev, rv_dev = wide[0][..., recent_pad:recent_pad + d], wide[1][..., recent_pad:recent_pad + d]
+    out = pool.decode_attention(q.to(gpu), table, seq.to(gpu), recent_k=rk_dev, recent_v=rv_dev,
                                 recent_len=None if rl is None else rl.to(gpu), n_split=n_split, max_len=max_len)
     torch.cuda.synchronize()
     prm = params_of(tq)
@@ -598,6 +604,23 @@ def test_decode_attention_ragged_empty_and_hybrid_tail(gpu):
     _progress(f"ragged+tail worst cosine {worst:.7f}")
     worst = _decode_case(gpu, 128, 3, 2, 2, 8, 8, [0, 0], [40, 1], seed=78)          # exact tokens only
     worst = _decode_case(gpu, 128, 3, 2, 2, 4, 2, [0, 64], None, seed=79)            # one row has nothing at all
+
+
+@pytest.mark.parametrize("d,dtype,Hq,Hkv,recent,pad", [
+    (256, torch.bfloat16, 16, 2, [300, 129, 1], 0),       # three chunks of 128 rows, ragged
+    (256, torch.bfloat16, 16, 2, [128, 77, 0], 1),        # rows not word-aligned: row-staged kernel
+    (128, torch.float16, 8, 8, [200, 256, 13], 2),        # strided rows, still word-aligned; one head per KV head
+    (64, torch.float16, 6, 2, [520, 3, 64], 0),           # two chunks at the smallest head size, 3 heads per group
+    (128, torch.float32, 8, 2, [130, 64, 5], 0),          # fp32 rows
+    (576, torch.float32, 4, 1, [40, 17, 33], 0),          # fp32 rows wider than the workgroup: two columns per thread
+    (768, torch.bfloat16, 4, 2, [70, 32, 1], 0),
+])
+def test_exact_tail_shapes(gpu, d, dtype, Hq, Hkv, recent, pad):
+    """The exact recent tokens (score.py:99-111) at the tail kernels' corners: several chunks, rows that are
+    strided or not word-aligned, every element type, head sizes from 64 to 768."""
+    _progress(f"exact tail d={d} {dtype} Hq={Hq} Hkv={Hkv} recent={recent} pad={pad}")
+    worst = _decode_case(gpu, d, 3, 2, 3, Hq, Hkv, [100, 0, 33], recent, seed=300 + d + pad, dtype=dtype, recent_pad=pad)
+    _progress(f"  worst cosine {worst:.7f}")
 
 
 @pytest.mark.parametrize("d,key_bits,vb,dtype", [(128, 3, 4, torch.bfloat16), (256, 3, 2, torch.bfloat16),

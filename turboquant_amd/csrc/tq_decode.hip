@@ -5,7 +5,7 @@
 //            walks its share of the sequence's pages; all G query heads of the
 //            group are scored from one read of the page; online softmax and the
 //            value accumulation stay in registers; result = partial (m, l, acc)
-//            exact_tail_kernel: the same partial for the exact recent tokens
+//            exact_tail_words_kernel / exact_tail_kernel: the same partial for the exact recent tokens
 //   stage 2  merge_kernel: log-sum-exp merge of the partials, cast to q's dtype
 //
 // Score of a token (triton_kernels.py:49-53,138):
@@ -414,6 +414,221 @@ exact_tail_kernel(const void* __restrict__ q, int Hq, int Hkv, int d, const void
   }
 }
 
+// The same partial with the rows staged as 32-bit words (two 16-bit channels, or one fp32 channel, per
+// word): the key rows AND the value rows of the first chunk are requested before anything waits, so a
+// tail that fits one chunk (128 tokens at head size 256, 16-bit) costs a single memory latency.  Both
+// tiles stay in LDS in the cache's own element type and are converted where they are read.  Needs word
+// alignment: 16-bit rows whose strides are even and whose base is 4-byte aligned.
+constexpr int TAIL_TILE_WORDS = 128 * 130, TAIL_RPT = 32;     // words per tile (keys, values); rows per thread
+
+template <int DT> struct TailWord;
+template <> struct TailWord<TQ_F32> {
+  static constexpr int EPW = 1;
+  static __device__ __forceinline__ void unpack(uint32_t w, float (&x)[2]) { x[0] = __uint_as_float(w); x[1] = 0.0f; }
+};
+template <> struct TailWord<TQ_BF16> {
+  static constexpr int EPW = 2;
+  static __device__ __forceinline__ void unpack(uint32_t w, float (&x)[2]) {
+    x[0] = __uint_as_float(w << 16);
+    x[1] = __uint_as_float(w & 0xffff0000u);
+  }
+};
+template <> struct TailWord<TQ_F16> {
+  static constexpr int EPW = 2;
+  static __device__ __forceinline__ void unpack(uint32_t w, float (&x)[2]) {
+    x[0] = f16_bits_to_f32((uint16_t)(w & 0xffffu));
+    x[1] = f16_bits_to_f32((uint16_t)(w >> 16));
+  }
+};
+
+static size_t tail_words_smem(int d, int recent_rows) {
+  return ((size_t)TAIL_GC * d + (size_t)TAIL_GC * recent_rows + 2 * TAIL_GC + 2 * TAIL_TILE_WORDS) * sizeof(float);
+}
+
+// KC = word columns per thread (2 only for fp32 rows of more than 512 channels)
+template <int DT, int KC>
+__global__ void __launch_bounds__(TAIL_THREADS)
+exact_tail_words_kernel(const void* __restrict__ q, int Hq, int Hkv, int d, const uint32_t* __restrict__ rk,
+                        const uint32_t* __restrict__ rv, int recent_rows, int64_t ws_b, int64_t ws_r, int64_t ws_h,
+                        const int32_t* __restrict__ recent_len, float sm_scale, float* __restrict__ parts,
+                        int n_parts, int part_index) {
+  constexpr int GC = TAIL_GC, EPW = TailWord<DT>::EPW, RPT = TAIL_RPT / KC;
+  const int G = Hq / Hkv, h = blockIdx.x, b = blockIdx.y, g0 = blockIdx.z * GC, tid = threadIdx.x;
+  const int Gc = min(GC, G - g0);
+  const int lane = tid & 63, wave = tid >> 6;
+  const int R = recent_len ? min(recent_len[b], recent_rows) : recent_rows;
+  extern __shared__ __align__(16) float sm[];
+  float* sq = sm;                                   // [d][GC]
+  float* ss = sq + GC * d;                          // [recent_rows][GC] scores, then softmax weights
+  float* sml = ss + GC * recent_rows;               // [GC][2]
+  uint32_t* ktile = (uint32_t*)(sml + 2 * GC);      // [CH][W + 1] key rows of the chunk; at the end [TS][GC][d] partials
+  uint32_t* vtile = ktile + TAIL_TILE_WORDS;        // [CH][W + 1] value rows
+  const int W = d / EPW, ldw = W + 1;               // words per row (a multiple of 32), odd leading dimension
+  const int TS = W < TAIL_THREADS ? TAIL_THREADS / W : 1;          // row slices
+  const int CH = min(TAIL_TILE_WORDS / ldw, TS * RPT);             // rows per chunk
+  const int cw0 = W < TAIL_THREADS ? tid % W : tid, ts = W < TAIL_THREADS ? tid / W : 0;
+  const bool active = ts < TS;
+  const int64_t base0 = b * ws_b + h * ws_h;
+  // loads of rows c0 + ts, c0 + ts + TS, ... of this thread's columns, all issued before anything waits
+  auto request = [&](const uint32_t* src, int c0, int n, uint32_t (&reg)[KC][RPT]) {
+#pragma unroll
+    for (int k = 0; k < KC; ++k) {
+      const int cw = min(cw0 + TAIL_THREADS * k, W - 1);
+#pragma unroll
+      for (int i = 0; i < RPT; ++i) {
+        const int t = ts + i * TS;
+        reg[k][i] = src[base0 + (int64_t)(c0 + (t < n ? t : 0)) * ws_r + cw];
+      }
+    }
+  };
+  auto deposit = [&](uint32_t* tile, int n, const uint32_t (&reg)[KC][RPT]) {
+#pragma unroll
+    for (int k = 0; k < KC; ++k) {
+      const int cw = cw0 + TAIL_THREADS * k;
+#pragma unroll
+      for (int i = 0; i < RPT; ++i) {
+        const int t = ts + i * TS;
+        if (t < n && cw < W) tile[t * ldw + cw] = reg[k][i];
+      }
+    }
+  };
+  const int n_first = min(CH, R);
+  if (active) {
+    uint32_t kreg[KC][RPT], vreg[KC][RPT];
+    request(rk, 0, n_first, kreg);
+    request(rv, 0, n_first, vreg);
+    deposit(ktile, n_first, kreg);
+    deposit(vtile, n_first, vreg);
+  }
+  for (int o = tid; o < GC * d; o += TAIL_THREADS) {
+    const int g = o / d, c = o - g * d;
+    const float x = Elem<DT>::load(q, ((int64_t)b * Hq + h * G + g0) * d + min(o, Gc * d - 1));
+    sq[c * GC + g] = g < Gc ? x : 0.0f;
+  }
+  __syncthreads();
+  // scores: eight threads per token, each over every eighth word of the row, for the group's heads at once
+  for (int c0 = 0; c0 < R; c0 += CH) {
+    const int n = min(CH, R - c0);
+    if (c0 > 0) {
+      __syncthreads();
+      if (active) {
+        uint32_t kreg[KC][RPT];
+        request(rk, c0, n, kreg);
+        deposit(ktile, n, kreg);
+      }
+      __syncthreads();
+    }
+    const int seg = tid & 7;
+    for (int t0 = 0; t0 < n; t0 += TAIL_THREADS / 8) {              // uniform trip count: the shuffles need every lane
+      const int t = t0 + (tid >> 3);
+      const uint32_t* row = ktile + (t < n ? t : 0) * ldw;
+      float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
+      for (int cw = seg; cw < W; cw += 8) {
+        float x[2];
+        TailWord<DT>::unpack(row[cw], x);
+        const float4 qa = *reinterpret_cast<const float4*>(sq + (cw * EPW) * GC);
+        a0 = fmaf(x[0], qa.x, a0);
+        a1 = fmaf(x[0], qa.y, a1);
+        a2 = fmaf(x[0], qa.z, a2);
+        a3 = fmaf(x[0], qa.w, a3);
+        if (EPW == 2) {
+          const float4 qb = *reinterpret_cast<const float4*>(sq + (cw * EPW + 1) * GC);
+          a0 = fmaf(x[1], qb.x, a0);
+          a1 = fmaf(x[1], qb.y, a1);
+          a2 = fmaf(x[1], qb.z, a2);
+          a3 = fmaf(x[1], qb.w, a3);
+        }
+      }
+#pragma unroll
+      for (int o = 4; o > 0; o >>= 1) {
+        a0 += __shfl_xor(a0, o, 64);
+        a1 += __shfl_xor(a1, o, 64);
+        a2 += __shfl_xor(a2, o, 64);
+        a3 += __shfl_xor(a3, o, 64);
+      }
+      if (seg == 0 && t < n)
+        *reinterpret_cast<float4*>(ss + (c0 + t) * GC) = make_float4(a0 * sm_scale, a1 * sm_scale, a2 * sm_scale, a3 * sm_scale);
+    }
+  }
+  __syncthreads();
+  // softmax statistics and weights, a wavefront per query head
+  for (int g = wave; g < GC; g += TAIL_WAVES) {
+    float mx = NEG_BIG;
+    for (int t = lane; t < R; t += 64) mx = fmaxf(mx, ss[t * GC + g]);
+    mx = wave_max(mx);
+    float sum = 0.0f;
+    for (int t = lane; t < R; t += 64) {
+      float p = __expf(ss[t * GC + g] - mx);
+      ss[t * GC + g] = p;
+      sum += p;
+    }
+    sum = wave_sum(sum);
+    if (lane == 0) { sml[g * 2] = mx; sml[g * 2 + 1] = sum; }
+  }
+  __syncthreads();
+  // values: a thread per word column and row slice
+  float acc[KC][2][GC];
+#pragma unroll
+  for (int k = 0; k < KC; ++k)
+#pragma unroll
+    for (int e = 0; e < 2; ++e)
+#pragma unroll
+      for (int g = 0; g < GC; ++g) acc[k][e][g] = 0.0f;
+  for (int c0 = 0; c0 < R; c0 += CH) {
+    const int n = min(CH, R - c0);
+    if (c0 > 0) {
+      __syncthreads();
+      if (active) {
+        uint32_t vreg[KC][RPT];
+        request(rv, c0, n, vreg);
+        deposit(vtile, n, vreg);
+      }
+      __syncthreads();
+    }
+    if (active) {
+#pragma unroll
+      for (int k = 0; k < KC; ++k) {
+        const int cw = cw0 + TAIL_THREADS * k;
+        if (cw < W) {
+          for (int t = ts; t < n; t += TS) {
+            float x[2];
+            TailWord<DT>::unpack(vtile[t * ldw + cw], x);
+            const float4 w4 = *reinterpret_cast<const float4*>(ss + (c0 + t) * GC);
+#pragma unroll
+            for (int e = 0; e < EPW; ++e) {
+              acc[k][e][0] = fmaf(w4.x, x[e], acc[k][e][0]);
+              acc[k][e][1] = fmaf(w4.y, x[e], acc[k][e][1]);
+              acc[k][e][2] = fmaf(w4.z, x[e], acc[k][e][2]);
+              acc[k][e][3] = fmaf(w4.w, x[e], acc[k][e][3]);
+            }
+          }
+        }
+      }
+    }
+  }
+  float* ptile = (float*)ktile;                     // [TS][GC][d]: the key tile is no longer needed
+  if (active) {
+#pragma unroll
+    for (int k = 0; k < KC; ++k) {
+      const int cw = cw0 + TAIL_THREADS * k;
+      if (cw < W)
+#pragma unroll
+        for (int e = 0; e < EPW; ++e)
+#pragma unroll
+          for (int g = 0; g < GC; ++g) ptile[(ts * GC + g) * d + cw * EPW + e] = acc[k][e][g];
+    }
+  }
+  __syncthreads();
+  for (int o = tid; o < Gc * d; o += TAIL_THREADS) {
+    const int g = o / d, ch = o - g * d;
+    float a = 0.0f;
+    for (int s2 = 0; s2 < TS; ++s2) a += ptile[(s2 * GC + g) * d + ch];
+    float* out = parts + (((int64_t)b * Hq + h * G + g0 + g) * n_parts + part_index) * (d + 2);
+    if (ch == 0) { out[0] = sml[g * 2]; out[1] = sml[g * 2 + 1]; }
+    out[2 + ch] = a;
+  }
+}
+
 // n_parts partials are merged per row; consecutive rows are part_stride partials apart.
 // One workgroup per row.  A thread owns a pair of channels and every S-th part (S = 256 / (d/2)
 // subsets share the parts when a row has fewer than 256 channel pairs); its first MERGE_CHUNK
@@ -615,21 +830,33 @@ extern "C" int tq_decode_attn_paged_stages(const void* q, int dtype, int B, int 
   }
 
   if (tail && (stages & 2)) {
-    size_t tsm = tail_smem(d, recent_rows);
     const dim3 tgrid(Hkv, B, (G + TAIL_GC - 1) / TAIL_GC);
-#define TQ_LAUNCH_TAIL(DT)                                                                                           \
+    const int epw = dtype == TQ_F32 ? 1 : 2;
+    const bool words = epw == 1 || (((((uintptr_t)recent_k | (uintptr_t)recent_v) & 3) == 0) && !((rs_b | rs_r | rs_h) & 1));
+    size_t tsm = words ? tail_words_smem(d, recent_rows) : tail_smem(d, recent_rows);
+#define TQ_LAUNCH_TAIL(KERN, ...)                                                                                    \
   {                                                                                                                  \
-    auto kern = exact_tail_kernel<DT>;                                                                               \
+    auto kern = KERN;                                                                                                \
     if (tsm > 48 * 1024) {                                                                                           \
       hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)tsm);   \
       if (e != hipSuccess) return (int)e;                                                                            \
     }                                                                                                                \
-    kern<<<tgrid, dim3(TAIL_THREADS), tsm, st>>>(q, Hq, Hkv, d, recent_k, recent_v, recent_rows, rs_b, rs_r, rs_h,    \
-                                                 recent_len, sm_scale, parts, n_parts, n_split);                     \
+    kern<<<tgrid, dim3(TAIL_THREADS), tsm, st>>>(__VA_ARGS__);                                                       \
   }
-    if (dtype == TQ_BF16) TQ_LAUNCH_TAIL(TQ_BF16)
-    else if (dtype == TQ_F16) TQ_LAUNCH_TAIL(TQ_F16)
-    else TQ_LAUNCH_TAIL(TQ_F32)
+#define TQ_TAIL_ROWS_ARGS q, Hq, Hkv, d, recent_k, recent_v, recent_rows, rs_b, rs_r, rs_h, recent_len, sm_scale, parts, n_parts, n_split
+#define TQ_TAIL_WORD_ARGS q, Hq, Hkv, d, (const uint32_t*)recent_k, (const uint32_t*)recent_v, recent_rows, rs_b / epw, rs_r / epw, \
+                          rs_h / epw, recent_len, sm_scale, parts, n_parts, n_split
+    if (words) {
+      if (dtype == TQ_BF16) TQ_LAUNCH_TAIL((exact_tail_words_kernel<TQ_BF16, 1>), TQ_TAIL_WORD_ARGS)
+      else if (dtype == TQ_F16) TQ_LAUNCH_TAIL((exact_tail_words_kernel<TQ_F16, 1>), TQ_TAIL_WORD_ARGS)
+      else if (d <= TAIL_THREADS) TQ_LAUNCH_TAIL((exact_tail_words_kernel<TQ_F32, 1>), TQ_TAIL_WORD_ARGS)
+      else TQ_LAUNCH_TAIL((exact_tail_words_kernel<TQ_F32, 2>), TQ_TAIL_WORD_ARGS)
+    } else {      // 16-bit rows that are not word-aligned
+      if (dtype == TQ_BF16) TQ_LAUNCH_TAIL(exact_tail_kernel<TQ_BF16>, TQ_TAIL_ROWS_ARGS)
+      else TQ_LAUNCH_TAIL(exact_tail_kernel<TQ_F16>, TQ_TAIL_ROWS_ARGS)
+    }
+#undef TQ_TAIL_WORD_ARGS
+#undef TQ_TAIL_ROWS_ARGS
 #undef TQ_LAUNCH_TAIL
     TQ_CHECK_LAUNCH();
   }
