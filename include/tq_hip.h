@@ -228,6 +228,21 @@ int tq_decode_attn_paged_stages(const void *q, int dtype, int B, int Hq, int Hkv
                                 const int32_t *recent_len, void *out, void *workspace, int n_split, int stages,
                                 void *stream);
 
+/* Hybrid decode step straight from the engine's paged exact cache (the reference keeps the exact recent
+ * tokens in a ring of its own, capture.py:75-131, and concatenates them in score.py:99-111; here they are
+ * read in place).  seq_lens[b] counts ALL tokens of sequence b.  The newest min(seq_lens[b], ring_rows) of
+ * them are attended to exactly, from k_cache / v_cache: blocks of 16 tokens, token p of sequence b in slot
+ * p % 16 of block block_table[b*bt_stride + p/16], element strides cs_blk (block), cs_t (token), cs_h (KV
+ * head), channels contiguous, `dtype`; 16-bit caches need even strides and 4-byte aligned bases
+ * (TQ_EUNSUPPORTED otherwise).  The tokens before them come from the compressed pages of the same block
+ * numbers.  Result as tq_decode_attn_paged with recent_k / recent_v = those rows and seq_lens reduced by
+ * their count, bit for bit.  ring_rows <= 1024.                                                         */
+int tq_decode_attn_paged_ring(const void *q, int dtype, int B, int Hq, int Hkv, const uint8_t *pool,
+                              int64_t num_pages, const int32_t *block_table, int bt_stride, const int32_t *seq_lens,
+                              float sm_scale, const tq_layer *layer, const tq_page_layout *layout,
+                              const void *k_cache, const void *v_cache, int64_t cs_blk, int64_t cs_t, int64_t cs_h,
+                              int ring_rows, void *out, void *workspace, int n_split, void *stream);
+
 /* Log-sum-exp merge of n_parts partial results per (b, query head):
  * parts (B*Hq, n_parts, d+2) fp32 = [running max, sum of exp, un-normalised acc];
  * out (B*Hq, d) `dtype`.  The same operator a context-parallel shard exchange

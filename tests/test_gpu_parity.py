@@ -980,3 +980,52 @@ def test_stream_read_probe_runs_and_rejects_bad_arguments(gpu):
     assert lib.tq_stream_read(buf.data_ptr(), 24, 4, 4, None, st) < 0
     assert lib.tq_stream_read(buf.data_ptr(), 16, 4, 3, None, st) < 0
     assert lib.tq_stream_read(buf.data_ptr(), 16, 0, 4, None, st) < 0
+
+
+@pytest.mark.parametrize("d,dtype,Hq,Hkv,ring", [(128, torch.bfloat16, 16, 4, 128), (256, torch.bfloat16, 16, 2, 128),
+                                                   (64, torch.float16, 8, 2, 200), (128, torch.float32, 4, 2, 48)])
+def test_ring_entry_reads_the_exact_cache_in_place(gpu, d, dtype, Hq, Hkv, ring):
+    """tq_decode_attn_paged_ring takes the exact recent tokens (score.py:99-111) straight from a paged exact
+    cache through the block table; it must equal, bit for bit, gathering those rows with torch indexing and
+    passing them as recent_k / recent_v with the history lengths reduced by their count."""
+    g = torch.Generator().manual_seed(5 * d + ring)
+    lens = [0, 7, ring, ring + 1, 333, 16 * 40]
+    B, per_seq = len(lens), 40
+    n_blocks = B * per_seq + 5
+    pool, _ = _make_pool(gpu, d, 3, 2, Hkv, n_blocks, dtype)
+    perm = torch.randperm(n_blocks, generator=g)[: B * per_seq].view(B, per_seq).to(torch.int32)
+    used = (torch.tensor(lens)[:, None] + 15) // 16 > torch.arange(per_seq)[None]
+    table = torch.where(used, perm, torch.zeros_like(perm)).to(gpu)        # unused entries padded with block 0
+    cache = torch.zeros(2, n_blocks, 16, Hkv, d, dtype=dtype, device=gpu)
+    k = torch.randn(B, max(lens), Hkv, d, generator=g).to(dtype).to(gpu)
+    v = torch.randn(B, max(lens), Hkv, d, generator=g).to(dtype).to(gpu)
+    seq = torch.tensor(lens, dtype=torch.int32, device=gpu)
+    for b, n in enumerate(lens):
+        if n == 0:
+            continue
+        pos = torch.arange(n, device=gpu)
+        blk = table[b].long()[pos // 16]
+        cache[0, blk, pos % 16] = k[b, :n]
+        cache[1, blk, pos % 16] = v[b, :n]
+        pool.append(k[b:b + 1, :n], v[b:b + 1, :n], table[b:b + 1])
+    q = torch.randn(B, Hq, d, generator=g).to(dtype).to(gpu)
+    _progress(f"ring entry d={d} {dtype} ring={ring} lens={lens}")
+    got = pool.decode_attention_ring(q, table, seq, cache[0], cache[1], ring, max_len=max(lens)).clone()
+    # the same step with the rows gathered on the host side
+    tail = torch.clamp(seq.long(), max=ring)
+    pos = (seq.long() - tail)[:, None] + torch.arange(ring, device=gpu)[None]
+    pos = torch.minimum(pos, (seq.long() - 1).clamp_min(0)[:, None])
+    slot = torch.gather(table.long(), 1, pos // 16) * 16 + pos % 16
+    rk = cache[0].reshape(-1, Hkv, d)[slot]
+    rv = cache[1].reshape(-1, Hkv, d)[slot]
+    want = pool.decode_attention(q, table, (seq.long() - tail).to(torch.int32), recent_k=rk, recent_v=rv,
+                                 recent_len=tail.to(torch.int32), max_len=max(lens))
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+    assert torch.count_nonzero(got[0]) == 0                         # the empty sequence
+    # and against the oracle on one sequence that has both parts
+    b = 4
+    kc, vc = _store_from_oracle_view(pool, table[b], lens[b] - ring)
+    ref = O.hybrid_attention(q[b:b + 1].cpu(), kc, vc, max(lens[b] - ring, O.MIN_HISTORY), params_of(pool.quantizer), Hkv,
+                             k[b, lens[b] - ring:lens[b]].cpu(), v[b, lens[b] - ring:lens[b]].cpu())
+    assert cosine(got[b:b + 1].cpu(), ref) >= COS_GATE

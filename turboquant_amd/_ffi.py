@@ -71,6 +71,8 @@ _SIGNATURES = {
     "tq_decode_attn_paged_stages": (C.c_int, [_vp, _i, _i, _i, _i, _vp, _i64, _vp, _i, _vp, _f, C.POINTER(TqLayer),
                                               C.POINTER(TqPageLayout), _vp, _vp, _i, _i64, _i64, _i64, _vp, _vp, _vp, _i,
                                               _i, _vp]),
+    "tq_decode_attn_paged_ring": (C.c_int, [_vp, _i, _i, _i, _i, _vp, _i64, _vp, _i, _vp, _f, C.POINTER(TqLayer),
+                                            C.POINTER(TqPageLayout), _vp, _vp, _i64, _i64, _i64, _i, _vp, _vp, _i, _vp]),
     "tq_decode_merge": (C.c_int, [_vp, _i64, _i, _i, _i, _vp, _vp]),
     "tq_time_next_page_kernel": (None, [_vp, _vp]),
     "tq_stream_read": (C.c_int, [_vp, C.c_size_t, _i, _i, _vp, _vp]),

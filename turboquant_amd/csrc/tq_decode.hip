@@ -53,7 +53,7 @@ __global__ void __launch_bounds__(GEN_THREADS)
 decode_pages_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_sk, int Hq, int Hkv,
                     const uint8_t* __restrict__ pool, const int32_t* __restrict__ block_table, int bt_stride,
                     const int32_t* __restrict__ seq_lens, float sm_scale, tq_layer ly, tq_page_layout L,
-                    float* __restrict__ parts, int n_parts, int n_split) {
+                    float* __restrict__ parts, int n_parts, int n_split, int len_sub) {
   constexpr int GP = 4 * GP4;
   const int d = ly.d, mb = ly.mse_bits, G = Hq / Hkv, words = d >> 5;
   const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
@@ -77,7 +77,7 @@ decode_pages_kernel(const float* __restrict__ q_rot, const float* __restrict__ q
   if (tid < 16) s_cent[tid] = tid < (1 << mb) ? ly.centroids[tid] : 0.0f;
   __syncthreads();
 
-  const int seq_len = seq_lens[b];
+  const int seq_len = max(seq_lens[b] - len_sub, 0);      // len_sub: newest tokens that are attended to exactly
   const int n_pages = (seq_len + TQ_PAGE_TOKENS - 1) / TQ_PAGE_TOKENS;
   const int per_split = (n_pages + n_split - 1) / n_split;
   const int pg_begin = split * per_split;
@@ -445,18 +445,26 @@ static size_t tail_words_smem(int d, int recent_rows) {
   return ((size_t)TAIL_GC * d + (size_t)TAIL_GC * recent_rows + 2 * TAIL_GC + 2 * TAIL_TILE_WORDS) * sizeof(float);
 }
 
-// KC = word columns per thread (2 only for fp32 rows of more than 512 channels)
-template <int DT, int KC>
+// KC = word columns per thread (2 only for fp32 rows of more than 512 channels).
+// PAGED: the exact tokens are the newest min(seq_len, recent_rows) tokens of the sequence in a paged
+// exact cache of 16-token blocks (rk / rv its base, ws_blk / ws_r / ws_h its block, token and head
+// strides in words); token p of sequence b sits in slot p % 16 of block block_table[b][p / 16].
+// Otherwise rk / rv are (B, recent_rows, H, d) rows with strides ws_b / ws_r / ws_h and recent_len valid rows.
+template <int DT, int KC, bool PAGED>
 __global__ void __launch_bounds__(TAIL_THREADS)
 exact_tail_words_kernel(const void* __restrict__ q, int Hq, int Hkv, int d, const uint32_t* __restrict__ rk,
                         const uint32_t* __restrict__ rv, int recent_rows, int64_t ws_b, int64_t ws_r, int64_t ws_h,
-                        const int32_t* __restrict__ recent_len, float sm_scale, float* __restrict__ parts,
-                        int n_parts, int part_index) {
+                        const int32_t* __restrict__ recent_len, const int32_t* __restrict__ block_table, int bt_stride,
+                        const int32_t* __restrict__ seq_lens, int64_t ws_blk, float sm_scale,
+                        float* __restrict__ parts, int n_parts, int part_index) {
   constexpr int GC = TAIL_GC, EPW = TailWord<DT>::EPW, RPT = TAIL_RPT / KC;
   const int G = Hq / Hkv, h = blockIdx.x, b = blockIdx.y, g0 = blockIdx.z * GC, tid = threadIdx.x;
   const int Gc = min(GC, G - g0);
   const int lane = tid & 63, wave = tid >> 6;
-  const int R = recent_len ? min(recent_len[b], recent_rows) : recent_rows;
+  const int seq = PAGED ? seq_lens[b] : 0;
+  const int R = PAGED ? max(min(seq, recent_rows), 0) : (recent_len ? min(recent_len[b], recent_rows) : recent_rows);
+  const int first = PAGED ? seq - R : 0;            // position of the first exact token
+  const int32_t* bt = block_table + (PAGED ? (int64_t)b * bt_stride : 0);
   extern __shared__ __align__(16) float sm[];
   float* sq = sm;                                   // [d][GC]
   float* ss = sq + GC * d;                          // [recent_rows][GC] scores, then softmax weights
@@ -468,17 +476,29 @@ exact_tail_words_kernel(const void* __restrict__ q, int Hq, int Hkv, int d, cons
   const int CH = min(TAIL_TILE_WORDS / ldw, TS * RPT);             // rows per chunk
   const int cw0 = W < TAIL_THREADS ? tid % W : tid, ts = W < TAIL_THREADS ? tid / W : 0;
   const bool active = ts < TS;
-  const int64_t base0 = b * ws_b + h * ws_h;
+  const int64_t base0 = (PAGED ? 0 : b * ws_b) + h * ws_h;
+  // word offset of exact row `row` (< R) of this (sequence, head)
+  auto row_base = [&](int row) -> int64_t {
+    if (PAGED) {
+      const int p = first + row;
+      return base0 + (int64_t)bt[p >> 4] * ws_blk + (int64_t)(p & 15) * ws_r;
+    }
+    return base0 + (int64_t)row * ws_r;
+  };
   // loads of rows c0 + ts, c0 + ts + TS, ... of this thread's columns, all issued before anything waits
+  // (n >= 1: callers skip empty chunks, so the clamped row exists)
   auto request = [&](const uint32_t* src, int c0, int n, uint32_t (&reg)[KC][RPT]) {
+    int64_t rb[RPT];
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) {
+      const int t = ts + i * TS;
+      rb[i] = row_base(c0 + (t < n ? t : 0));
+    }
 #pragma unroll
     for (int k = 0; k < KC; ++k) {
       const int cw = min(cw0 + TAIL_THREADS * k, W - 1);
 #pragma unroll
-      for (int i = 0; i < RPT; ++i) {
-        const int t = ts + i * TS;
-        reg[k][i] = src[base0 + (int64_t)(c0 + (t < n ? t : 0)) * ws_r + cw];
-      }
+      for (int i = 0; i < RPT; ++i) reg[k][i] = src[rb[i] + cw];
     }
   };
   auto deposit = [&](uint32_t* tile, int n, const uint32_t (&reg)[KC][RPT]) {
@@ -493,7 +513,7 @@ exact_tail_words_kernel(const void* __restrict__ q, int Hq, int Hkv, int d, cons
     }
   };
   const int n_first = min(CH, R);
-  if (active) {
+  if (active && n_first > 0) {
     uint32_t kreg[KC][RPT], vreg[KC][RPT];
     request(rk, 0, n_first, kreg);
     request(rv, 0, n_first, vreg);
@@ -725,7 +745,7 @@ size_t decode_mfma_pack_words(int B, int Hkv, int d);
 int launch_decode_mfma(const uint32_t* qa_pack, const float* q_stat, int B, int Hq, int Hkv, int kv_div,
                        const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
                        float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts,
-                       int n_split, hipStream_t st);
+                       int n_split, int len_sub, hipStream_t st);
 }  // namespace tq
 
 static size_t parts_floats(int B, int Hq, int d, int n_parts) { return (size_t)B * Hq * n_parts * (d + 2); }
@@ -749,13 +769,29 @@ extern "C" int tq_decode_merge(const float* parts, int64_t rows, int n_parts, in
   return TQ_OK;
 }
 
-extern "C" int tq_decode_attn_paged_stages(const void* q, int dtype, int B, int Hq, int Hkv, const uint8_t* pool,
-                                           int64_t num_pages, const int32_t* block_table, int bt_stride,
-                                           const int32_t* seq_lens, float sm_scale, const tq_layer* layer,
-                                           const tq_page_layout* layout, const void* recent_k, const void* recent_v,
-                                           int recent_rows, int64_t rs_b, int64_t rs_r, int64_t rs_h,
-                                           const int32_t* recent_len, void* out, void* workspace, int n_split,
-                                           int stages, void* stream) {
+namespace {
+// The exact tokens of a step.  Rows: (B, rows, H, d) tensors with element strides s_b / s_r / s_h and `len`
+// valid rows per sequence.  Paged: the newest min(seq_len, rows) tokens of every sequence, read in place
+// from a paged exact cache (block stride s_blk, token stride s_r, head stride s_h) through the step's
+// block table; the compressed pages then cover the tokens before them.
+struct TailSpec {
+  const void* k = nullptr;
+  const void* v = nullptr;
+  int rows = 0;
+  int64_t s_b = 0, s_r = 0, s_h = 0, s_blk = 0;
+  const int32_t* len = nullptr;
+  bool paged = false;
+};
+}  // namespace
+
+static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const uint8_t* pool, int64_t num_pages,
+                         const int32_t* block_table, int bt_stride, const int32_t* seq_lens, float sm_scale,
+                         const tq_layer* layer, const tq_page_layout* layout, const TailSpec& ts, void* out,
+                         void* workspace, int n_split, int stages, void* stream) {
+  const void *recent_k = ts.k, *recent_v = ts.v;
+  const int recent_rows = ts.rows;
+  const int64_t rs_b = ts.s_b, rs_r = ts.s_r, rs_h = ts.s_h;
+  const int32_t* recent_len = ts.len;
   if (!q || !pool || !block_table || !seq_lens || !layer || !layout || !out || !workspace) return TQ_ENULL;
   if (B <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || n_split <= 0 || num_pages <= 0 || bt_stride < 0) return TQ_EINVAL;
   if (B > 65535 || Hkv > 65535) return TQ_EUNSUPPORTED;
@@ -766,6 +802,7 @@ extern "C" int tq_decode_attn_paged_stages(const void* q, int dtype, int B, int 
   const bool tail = recent_k != nullptr && recent_rows > 0;
   if (tail && !recent_v) return TQ_ENULL;
   if (tail && recent_rows > 1024) return TQ_EUNSUPPORTED;
+  const int len_sub = tail && ts.paged ? recent_rows : 0;       // newest tokens the pages do not cover
   hipStream_t st = (hipStream_t)stream;
   const int n_parts = n_split + 1;
   float* parts = (float*)workspace;
@@ -795,7 +832,7 @@ extern "C" int tq_decode_attn_paged_stages(const void* q, int dtype, int B, int 
   int mf = TQ_EUNSUPPORTED;
   if (stages & 2)
     mf = mfma_shape ? launch_decode_mfma(qa_pack, q_stat, B, Hq, Hkv * kv_div, kv_div, pool, block_table, bt_stride,
-                                         seq_lens, sm_scale, *layer, *layout, parts, n_parts, n_split, st)
+                                         seq_lens, sm_scale, *layer, *layout, parts, n_parts, n_split, len_sub, st)
                     : TQ_EUNSUPPORTED;
   if (mf > 0) return mf;
   if ((stages & 2) && mf == TQ_EUNSUPPORTED) {      // no matrix-core kernel for this shape: general kernel
@@ -813,7 +850,7 @@ extern "C" int tq_decode_attn_paged_stages(const void* q, int dtype, int B, int 
       if (e != hipSuccess) return (int)e;                                                                 \
     }                                                                                                     \
     kern<<<grid, block, smem, st>>>(q_rot, q_sk, Hq, Hkv, pool, block_table, bt_stride, seq_lens, sm_scale, *layer,  \
-                                    *layout, parts, n_parts, n_split);                                    \
+                                    *layout, parts, n_parts, n_split, len_sub);                           \
   }
 #define TQ_LAUNCH_DEC_G(VB)                                                      \
   {                                                                              \
@@ -832,7 +869,9 @@ extern "C" int tq_decode_attn_paged_stages(const void* q, int dtype, int B, int 
   if (tail && (stages & 2)) {
     const dim3 tgrid(Hkv, B, (G + TAIL_GC - 1) / TAIL_GC);
     const int epw = dtype == TQ_F32 ? 1 : 2;
-    const bool words = epw == 1 || (((((uintptr_t)recent_k | (uintptr_t)recent_v) & 3) == 0) && !((rs_b | rs_r | rs_h) & 1));
+    const bool words = epw == 1 || (((((uintptr_t)recent_k | (uintptr_t)recent_v) & 3) == 0) &&
+                                    !((rs_b | rs_r | rs_h | ts.s_blk) & 1));
+    if (ts.paged && !words) return TQ_EUNSUPPORTED;             // a paged exact cache has to be word-aligned
     size_t tsm = words ? tail_words_smem(d, recent_rows) : tail_smem(d, recent_rows);
 #define TQ_LAUNCH_TAIL(KERN, ...)                                                                                    \
   {                                                                                                                  \
@@ -845,16 +884,22 @@ extern "C" int tq_decode_attn_paged_stages(const void* q, int dtype, int B, int 
   }
 #define TQ_TAIL_ROWS_ARGS q, Hq, Hkv, d, recent_k, recent_v, recent_rows, rs_b, rs_r, rs_h, recent_len, sm_scale, parts, n_parts, n_split
 #define TQ_TAIL_WORD_ARGS q, Hq, Hkv, d, (const uint32_t*)recent_k, (const uint32_t*)recent_v, recent_rows, rs_b / epw, rs_r / epw, \
-                          rs_h / epw, recent_len, sm_scale, parts, n_parts, n_split
+                          rs_h / epw, recent_len, block_table, bt_stride, seq_lens, ts.s_blk / epw, sm_scale, parts, n_parts, n_split
+#define TQ_TAIL_WORDS(PAGED)                                                                                   \
+  {                                                                                                            \
+    if (dtype == TQ_BF16) TQ_LAUNCH_TAIL((exact_tail_words_kernel<TQ_BF16, 1, PAGED>), TQ_TAIL_WORD_ARGS)      \
+    else if (dtype == TQ_F16) TQ_LAUNCH_TAIL((exact_tail_words_kernel<TQ_F16, 1, PAGED>), TQ_TAIL_WORD_ARGS)   \
+    else if (d <= TAIL_THREADS) TQ_LAUNCH_TAIL((exact_tail_words_kernel<TQ_F32, 1, PAGED>), TQ_TAIL_WORD_ARGS) \
+    else TQ_LAUNCH_TAIL((exact_tail_words_kernel<TQ_F32, 2, PAGED>), TQ_TAIL_WORD_ARGS)                        \
+  }
     if (words) {
-      if (dtype == TQ_BF16) TQ_LAUNCH_TAIL((exact_tail_words_kernel<TQ_BF16, 1>), TQ_TAIL_WORD_ARGS)
-      else if (dtype == TQ_F16) TQ_LAUNCH_TAIL((exact_tail_words_kernel<TQ_F16, 1>), TQ_TAIL_WORD_ARGS)
-      else if (d <= TAIL_THREADS) TQ_LAUNCH_TAIL((exact_tail_words_kernel<TQ_F32, 1>), TQ_TAIL_WORD_ARGS)
-      else TQ_LAUNCH_TAIL((exact_tail_words_kernel<TQ_F32, 2>), TQ_TAIL_WORD_ARGS)
+      if (ts.paged) TQ_TAIL_WORDS(true)
+      else TQ_TAIL_WORDS(false)
     } else {      // 16-bit rows that are not word-aligned
       if (dtype == TQ_BF16) TQ_LAUNCH_TAIL(exact_tail_kernel<TQ_BF16>, TQ_TAIL_ROWS_ARGS)
       else TQ_LAUNCH_TAIL(exact_tail_kernel<TQ_F16>, TQ_TAIL_ROWS_ARGS)
     }
+#undef TQ_TAIL_WORDS
 #undef TQ_TAIL_WORD_ARGS
 #undef TQ_TAIL_ROWS_ARGS
 #undef TQ_LAUNCH_TAIL
@@ -866,6 +911,35 @@ extern "C" int tq_decode_attn_paged_stages(const void* q, int dtype, int B, int 
       parts, tail ? n_parts : n_split, n_parts, d, dtype, out);
   TQ_CHECK_LAUNCH();
   return TQ_OK;
+}
+
+extern "C" int tq_decode_attn_paged_stages(const void* q, int dtype, int B, int Hq, int Hkv, const uint8_t* pool,
+                                           int64_t num_pages, const int32_t* block_table, int bt_stride,
+                                           const int32_t* seq_lens, float sm_scale, const tq_layer* layer,
+                                           const tq_page_layout* layout, const void* recent_k, const void* recent_v,
+                                           int recent_rows, int64_t rs_b, int64_t rs_r, int64_t rs_h,
+                                           const int32_t* recent_len, void* out, void* workspace, int n_split,
+                                           int stages, void* stream) {
+  TailSpec ts;
+  ts.k = recent_k; ts.v = recent_v; ts.rows = recent_rows;
+  ts.s_b = rs_b; ts.s_r = rs_r; ts.s_h = rs_h; ts.len = recent_len;
+  return decode_stages(q, dtype, B, Hq, Hkv, pool, num_pages, block_table, bt_stride, seq_lens, sm_scale, layer, layout,
+                       ts, out, workspace, n_split, stages, stream);
+}
+
+extern "C" int tq_decode_attn_paged_ring(const void* q, int dtype, int B, int Hq, int Hkv, const uint8_t* pool,
+                                         int64_t num_pages, const int32_t* block_table, int bt_stride,
+                                         const int32_t* seq_lens, float sm_scale, const tq_layer* layer,
+                                         const tq_page_layout* layout, const void* k_cache, const void* v_cache,
+                                         int64_t cs_blk, int64_t cs_t, int64_t cs_h, int ring_rows, void* out,
+                                         void* workspace, int n_split, void* stream) {
+  if (!k_cache || !v_cache) return TQ_ENULL;
+  if (ring_rows <= 0 || cs_blk <= 0 || cs_t <= 0 || cs_h <= 0) return TQ_EINVAL;
+  TailSpec ts;
+  ts.k = k_cache; ts.v = v_cache; ts.rows = ring_rows;
+  ts.s_blk = cs_blk; ts.s_r = cs_t; ts.s_h = cs_h; ts.paged = true;
+  return decode_stages(q, dtype, B, Hq, Hkv, pool, num_pages, block_table, bt_stride, seq_lens, sm_scale, layer, layout,
+                       ts, out, workspace, n_split, 7, stream);
 }
 
 extern "C" int tq_decode_attn_paged(const void* q, int dtype, int B, int Hq, int Hkv, const uint8_t* pool,

@@ -165,7 +165,7 @@ __global__ void __launch_bounds__(MF_WAVES * 64, WPS)
 decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict__ q_stat, int Hq, int Hkv, int kv_div,
                    const uint8_t* __restrict__ pool, const int32_t* __restrict__ block_table,
                    int bt_stride, const int32_t* __restrict__ seq_lens, float sm_scale, tq_layer ly, tq_page_layout L,
-                   float* __restrict__ parts, int n_parts, int n_split) {
+                   float* __restrict__ parts, int n_parts, int n_split, int len_sub) {
   constexpr int DW = D / DS;                  // coordinates / channels of one wavefront
   constexpr int WPLT = D / 128;               // plane words per lane per plane per page, all wavefronts
   constexpr int WPL = DW / 128;               // ... of one wavefront
@@ -253,7 +253,7 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
   }
 
   // ---------------------------------------------------------------- work range (all scalar)
-  const int seq_len = seq_lens[b];
+  const int seq_len = max(seq_lens[b] - len_sub, 0);      // len_sub: newest tokens that are attended to exactly
   const int n_pages = (seq_len + TQ_PAGE_TOKENS - 1) / TQ_PAGE_TOKENS;
   const int n_blocks = (seq_len + BLK_TOK - 1) / BLK_TOK;
   const int per_split = (n_blocks + n_split - 1) / n_split;
@@ -679,7 +679,7 @@ template <int D, int MB, int NX, int VB, int GS, int DS, int WPS, bool F16P>
 static int launch_one(const uint32_t* qa_pack, const float* q_stat, int B, int Hq, int Hkv, int kv_div,
                       const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
                       float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts, int n_split,
-                      hipStream_t st) {
+                      int len_sub, hipStream_t st) {
   const int G = Hq / Hkv;
   size_t per_wave = (size_t)wave_lds_floats(D / DS / GS, DS) * sizeof(float);
   size_t merge = (size_t)(MF_WAVES / DS * G * (D + 2) + MF_WAVES * 16 * 16) * sizeof(float);
@@ -692,12 +692,12 @@ static int launch_one(const uint32_t* qa_pack, const float* q_stat, int B, int H
   if (t_start_event || t_stop_event) {
     hipExtLaunchKernelGGL(kern, dim3(n_split, Hkv, B), dim3(MF_WAVES * 64), smem, st, t_start_event, t_stop_event, 0,
                           qa_pack, q_stat, Hq, Hkv, kv_div, pool, block_table, bt_stride, seq_lens, sm_scale, ly, L, parts,
-                          n_parts, n_split);
+                          n_parts, n_split, len_sub);
     t_start_event = t_stop_event = nullptr;
   } else {
     kern<<<dim3(n_split, Hkv, B), dim3(MF_WAVES * 64), smem, st>>>(qa_pack, q_stat, Hq, Hkv, kv_div, pool, block_table,
                                                                    bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts,
-                                                                   n_split);
+                                                                   n_split, len_sub);
   }
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? TQ_OK : (int)e;
@@ -711,7 +711,7 @@ size_t decode_mfma_pack_words(int B, int Hq, int d) { return (size_t)B * Hq * 9 
 int launch_decode_mfma(const uint32_t* qa_pack, const float* q_stat, int B, int Hq, int Hkv, int kv_div,
                        const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
                        float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts,
-                       int n_split, hipStream_t st) {
+                       int n_split, int len_sub, hipStream_t st) {
   const int G = Hq / Hkv, d = ly.d, mb = ly.mse_bits, vb = L.value_bits, gs = L.group_size;
   if (G > 8 || (L.dtype != TQ_BF16 && L.dtype != TQ_F16) || !L.key_lane_major) return TQ_EUNSUPPORTED;
   const bool f16p = L.dtype == TQ_F16;
@@ -723,10 +723,10 @@ int launch_decode_mfma(const uint32_t* qa_pack, const float* q_stat, int B, int 
     if (f16p)                                                                                                   \
       return launch_one<D_, MB_, NX_, VB_, GS_, DS_, WPS_, true>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,  \
                                                                  bt_stride, seq_lens, sm_scale, ly, L, parts,     \
-                                                                 n_parts, n_split, st);                          \
+                                                                 n_parts, n_split, len_sub, st);                 \
     return launch_one<D_, MB_, NX_, VB_, GS_, DS_, WPS_, false>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,   \
                                                                 bt_stride, seq_lens, sm_scale, ly, L, parts,      \
-                                                                n_parts, n_split, st);                           \
+                                                                n_parts, n_split, len_sub, st);                  \
   }
   TQ_TRY(128, 2, 0, 2, 32, 1, 2) TQ_TRY(128, 2, 0, 4, 32, 1, 2) TQ_TRY(256, 2, 0, 2, 32, 2, 2) TQ_TRY(256, 2, 0, 4, 32, 2, 2)
   TQ_TRY(128, 1, 0, 2, 32, 1, 2) TQ_TRY(128, 1, 0, 4, 32, 1, 2) TQ_TRY(256, 1, 0, 2, 32, 2, 2) TQ_TRY(256, 1, 0, 4, 32, 2, 2)

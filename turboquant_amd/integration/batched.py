@@ -121,8 +121,17 @@ class BatchedLayerState:
     def attend(self, query: torch.Tensor, meta, scale: Optional[float] = None, kv_cache=None,
                hybrid: bool = False) -> torch.Tensor:
         """One query token per sequence, (B, H_q, d) -> (B, H_q, d)."""
-        recent = self._exact_tail(kv_cache, meta) if hybrid else None
         self.decode_steps += 1
+        cfg = self.config
+        if (hybrid and cfg.ring_capacity > 0 and torch.is_tensor(kv_cache) and kv_cache.dim() == 5 and
+                kv_cache.shape[0] == 2 and tuple(kv_cache.shape[2:]) == (PAGE_TOKENS, cfg.num_kv_heads, cfg.head_dim) and
+                kv_cache.dtype == query.dtype and cfg.ring_capacity <= 1024 and
+                self.pool.ring_cache_ok(kv_cache[0], kv_cache[1])):
+            # the exact tokens are read in place from the engine's cache, through the step's block table
+            return self.pool.decode_attention_ring(query, meta.block_table, meta.seq_lens, kv_cache[0], kv_cache[1],
+                                                   cfg.ring_capacity, scale=scale,
+                                                   max_len=getattr(meta, "max_seq_len", None))
+        recent = self._exact_tail(kv_cache, meta) if hybrid else None
         if recent is None:
             return self.pool.decode_attention(query, meta.block_table, meta.seq_lens, scale=scale,
                                               max_len=getattr(meta, "max_seq_len", None))

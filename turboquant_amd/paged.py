@@ -222,3 +222,59 @@ class PagedKVPool:
                 C.byref(self.layout), rk_ptr, rv_ptr, rows, rs[0], rs[1], rs[2], rl_ptr, out.data_ptr(),
                 workspace.data_ptr(), n_split, stages, _ffi.stream_ptr(self.device)), "tq_decode_attn_paged")
         return out
+
+    @staticmethod
+    def ring_cache_ok(key_cache: torch.Tensor, value_cache: torch.Tensor) -> bool:
+        """Whether decode_attention_ring can read this paged exact cache in place: (blocks, 16, H, d) with
+        contiguous channels, equal strides, and (16-bit types) even strides and 4-byte aligned bases."""
+        if key_cache.dim() != 4 or key_cache.shape != value_cache.shape or key_cache.shape[1] != PAGE_TOKENS:
+            return False
+        if key_cache.stride() != value_cache.stride() or key_cache.stride(-1) != 1 or key_cache.dtype != value_cache.dtype:
+            return False
+        if key_cache.element_size() == 2:
+            if any(st % 2 for st in key_cache.stride()[:3]) or key_cache.data_ptr() % 4 or value_cache.data_ptr() % 4:
+                return False
+        return True
+
+    def decode_attention_ring(self, query: torch.Tensor, block_table: torch.Tensor, seq_lens: torch.Tensor,
+                              key_cache: torch.Tensor, value_cache: torch.Tensor, ring_rows: int,
+                              scale: Optional[float] = None, n_split: Optional[int] = None,
+                              workspace: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
+                              max_len: Optional[int] = None) -> torch.Tensor:
+        """Hybrid attention of one query token per sequence (score.py:99-111) with the exact tokens read in
+        place: the newest min(seq_lens[b], ring_rows) tokens of sequence b come from the engine's paged exact
+        cache key_cache / value_cache (blocks, 16, H, d) through `block_table`, the tokens before them from
+        this pool's pages of the same numbers.  seq_lens counts all tokens.  Same result as decode_attention
+        with those rows gathered into recent_k / recent_v."""
+        _ffi.require_gpu(query, "query")
+        B, Hq, d = query.shape
+        if d != self.head_dim or Hq % self.num_kv_heads:
+            raise ValueError(f"Incompatible GQA shapes: Q={Hq}, H_kv={self.num_kv_heads}, d={d}")
+        if key_cache.dtype != query.dtype:
+            raise TypeError("the exact cache must have the query's dtype")
+        if tuple(key_cache.shape[2:]) != (self.num_kv_heads, d) or not self.ring_cache_ok(key_cache, value_cache):
+            raise ValueError("decode_attention_ring needs a (blocks, 16, H_kv, d) cache with contiguous channels, "
+                             "equal key / value strides and word-aligned rows")
+        query = query.contiguous()
+        if scale is None:
+            scale = 1.0 / math.sqrt(d)
+        bt = block_table.contiguous()
+        bt_stride = 0 if bt.dim() == 1 else bt.shape[1]
+        seq_lens = seq_lens.to(device=self.device, dtype=torch.int32).contiguous()
+        if n_split is None:
+            if max_len is None:
+                max_len = (bt.shape[-1]) * PAGE_TOKENS
+            n_split = self.default_splits(B, max_len, Hq)
+        if workspace is None:
+            workspace = self.workspace(B, Hq, n_split)
+        if out is None:
+            out = torch.empty_like(query)
+        ly = self.quantizer._layer()
+        with torch.cuda.device(self.device):
+            _ffi.check(_ffi.lib().tq_decode_attn_paged_ring(
+                query.data_ptr(), _ffi.dtype_tag(query.dtype), B, Hq, self.num_kv_heads, self.data.data_ptr(),
+                self.num_pages, bt.data_ptr(), bt_stride, seq_lens.data_ptr(), float(scale), C.byref(ly),
+                C.byref(self.layout), key_cache.data_ptr(), value_cache.data_ptr(), key_cache.stride(0),
+                key_cache.stride(1), key_cache.stride(2), int(ring_rows), out.data_ptr(), workspace.data_ptr(),
+                n_split, _ffi.stream_ptr(self.device)), "tq_decode_attn_paged_ring")
+        return out
