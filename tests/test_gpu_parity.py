@@ -1029,3 +1029,76 @@ def test_ring_entry_reads_the_exact_cache_in_place(gpu, d, dtype, Hq, Hkv, ring)
     ref = O.hybrid_attention(q[b:b + 1].cpu(), kc, vc, max(lens[b] - ring, O.MIN_HISTORY), params_of(pool.quantizer), Hkv,
                              k[b, lens[b] - ring:lens[b]].cpu(), v[b, lens[b] - ring:lens[b]].cpu())
     assert cosine(got[b:b + 1].cpu(), ref) >= COS_GATE
+
+
+def test_config2_full_size_prefill_quantise(gpu):
+    """The prefill-quantise workload at its full size (32768 tokens x 8 KV heads, head size 128, four outlier
+    channels x20 per tensor and head, bf16; 3-bit keys, 2-bit values in groups of 32, 2048 pages per head):
+    a sample of tokens against the oracle, and over all tokens what does not depend on the size - chunked
+    appends give the same pages, every value is within half a step of its code, the key estimator
+    (quantizer.py:274-302) is unbiased, the MSE stage's distortion is the codebook's."""
+    from turboquant_amd.codebook import get_codebook
+    from turboquant_amd.quantizer import MSEQuantized, ProdQuantized
+    H, T, d = 8, 32768, 128
+    g = torch.Generator().manual_seed(1)
+    K = torch.randn(1, H, T, d, generator=g)
+    V = torch.randn(1, H, T, d, generator=g)
+    for X in (K, V):
+        for h in range(H):
+            X[0, h][:, torch.randperm(d, generator=g)[:4]] *= 20.0
+    k = K[0].transpose(0, 1)[None].bfloat16().contiguous()             # (1, T, H, d)
+    v = V[0].transpose(0, 1)[None].bfloat16().contiguous()
+    table = torch.randperm(T // 16, generator=g).to(torch.int32)[None].to(gpu)
+    pool, tq = _make_pool(gpu, d, 3, 2, H, T // 16)
+    _progress("config 2 full size: one append of 32768 tokens x 8 heads")
+    kd, vd = k.to(gpu), v.to(gpu)
+    pool.append(kd, vd, table)
+    idx, sgn, norms, rnorms, vdata, vsc, vz = pool.export_flat(table[0], T)
+    torch.cuda.synchronize()
+    # (1) the same tokens in four chunks with ragged boundaries
+    pool2, _ = _make_pool(gpu, d, 3, 2, H, T // 16)
+    for a, b in ((0, 5000), (5000, 5001), (5001, 20000), (20000, T)):
+        pool2.append(kd[:, a:b], vd[:, a:b], table, torch.tensor([a], dtype=torch.int32, device=gpu))
+    torch.cuda.synchronize()
+    assert torch.equal(pool.data, pool2.data)
+    # (2) 1024 sampled tokens against the oracle
+    prm = params_of(tq)
+    pick = torch.randperm(T, generator=g)[:1024].sort().values
+    ks = k[0, pick].transpose(0, 1).contiguous()                        # (H, 1024, d)
+    vs = v[0, pick].transpose(0, 1).contiguous()
+    want = O.prod_quantize(ks, prm)
+    n_coord = ks.numel()
+    pk = pick.to(gpu)
+    idx_flips = byte_mismatch(idx[:, pk].cpu(), want.mse_indices)
+    sgn_flips = bit_mismatch(sgn[:, pk].cpu(), want.qjl_signs)
+    _progress(f"   sample: index bytes differing {idx_flips}, sign bits differing {sgn_flips} of {n_coord}")
+    assert idx_flips <= max(1, FLIP_RATE * n_coord)
+    assert sgn_flips <= max(2, FLIP_RATE * n_coord)
+    got_norm, ref_norm = norms[:, pk].float().cpu(), want.norms.float()
+    assert torch.all((got_norm - ref_norm).abs() <= 2.0 ** -7 * ref_norm.abs())
+    assert torch.allclose(rnorms[:, pk].cpu(), want.residual_norms, rtol=2e-5, atol=1e-6)
+    wv = O.quantize_values(vs, 2, 32)
+    assert torch.equal(vdata[:, pk].cpu(), wv.data)
+    assert torch.equal(vsc[:, pk].cpu(), wv.scales) and torch.equal(vz[:, pk].cpu(), wv.zeros)
+    # (3) every value within half a quantisation step (plus the bf16 rounding of the per-op arithmetic)
+    vt = vd[0].transpose(0, 1).float()                                  # (H, T, d)
+    codes = torch.stack([(vdata >> s) & 3 for s in (0, 2, 4, 6)], dim=-1).reshape(H, T, d).float()
+    sc = vsc.float().repeat_interleave(32, dim=-1)
+    zr = vz.float().repeat_interleave(32, dim=-1)
+    err = (codes * sc + zr - vt).abs()
+    assert torch.all(err <= 0.5 * sc + 2.0 ** -6 * (vt.abs() + zr.abs() + sc) + 1e-6)
+    # (4) MSE stage: relative distortion of the de-quantised unit vectors = the codebook's (within 5 %)
+    kt = kd[0].transpose(0, 1).float()
+    mse_hat = tq.mse_quantizer.dequantize(MSEQuantized(idx, norms, 2))
+    rel = ((mse_hat - kt) ** 2).sum(-1) / (kt ** 2).sum(-1)
+    theory = float(get_codebook(d, 2)["mse_total"])
+    _progress(f"   relative MSE distortion {rel.mean().item():.5f}, codebook {theory:.5f}")
+    assert abs(rel.mean().item() - theory) <= 0.05 * theory
+    # (5) the inner-product estimator is unbiased: the slope of estimate on truth over all tokens is 1
+    q = torch.randn(H, 4, d, generator=g).to(gpu)
+    code = ProdQuantized(idx, sgn, rnorms, norms, 2)
+    est = tq.attention_score(q, code)                                   # (H, 4, T)
+    true = torch.einsum("hqd,htd->hqt", q, kt)
+    slope = (est * true).sum() / (true * true).sum()
+    _progress(f"   estimator slope {slope.item():.5f}")
+    assert abs(slope.item() - 1.0) < 0.01
