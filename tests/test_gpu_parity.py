@@ -1102,3 +1102,14 @@ def test_config2_full_size_prefill_quantise(gpu):
     slope = (est * true).sum() / (true * true).sum()
     _progress(f"   estimator slope {slope.item():.5f}")
     assert abs(slope.item() - 1.0) < 0.01
+
+
+def test_config3_full_size_decode_against_the_oracle(gpu):
+    """The GQA decode workload at its full size (16 sequences x 8192 tokens, 32 query / 8 KV heads of 128,
+    3-bit keys, 4-bit values in groups of 32, physical pages a random permutation): every sequence against
+    the oracle on the same store (score.py:84-173), and the split count must not matter."""
+    _progress("config 3 full size: 16 x 8192, 32 / 8 heads of 128")
+    worst = _decode_case(gpu, 128, 3, 4, 16, 32, 8, [8192] * 16, None, seed=2)
+    _progress(f"   worst cosine over 16 sequences {worst:.7f}")
+    worst = _decode_case(gpu, 128, 3, 4, 4, 32, 8, [8192, 8191, 4097, 8192], [128, 0, 5, 64], seed=3, n_split=7)
+    _progress(f"   ragged, hybrid, 7 splits: worst cosine {worst:.7f}")
