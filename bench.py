@@ -107,6 +107,25 @@ class DecodeWorkload:
                               max_len=self.N, stages=stages)
 
 
+def hybrid_step_bench(work, steps, warmup, ring=128):
+    """The same decode step in hybrid mode: the newest `ring` tokens of every sequence attended to exactly,
+    read in place from a paged exact cache (synthetic bf16 rows) through the block table, the tokens before
+    them from the compressed pages."""
+    import torch
+    dev = work.q.device
+    n_blocks = work.pools[0].num_pages
+    gen = torch.Generator(device=dev).manual_seed(11)
+    cache = torch.randn(2, n_blocks, 16, work.Hkv, work.d, generator=gen, device=dev, dtype=torch.float32).bfloat16()
+
+    def step(i):
+        pool = work.pools[i % len(work.pools)]
+        pool.decode_attention_ring(work.q, work.table, work.seq, cache[0], cache[1], ring, n_split=work.n_split,
+                                   workspace=work.ws, out=work.out, max_len=work.N)
+    ms, _ = time_steps(step, steps, warmup)
+    del cache
+    return {"exact_tokens": ring, "ms_per_step": ms}
+
+
 def time_steps(fn, steps, warmup):
     """(mean ms per step, wall ms per step) with HIP events on the launch stream."""
     import torch
@@ -341,6 +360,8 @@ def main():
 
     stream = stream_read_peak(main_w, max(20, args.steps // 4), max(5, args.warmup // 5))
 
+    hybrid_main = hybrid_step_bench(main_w, max(20, args.steps // 4), max(5, args.warmup // 5))
+
     traffic = None
     tpath = os.path.join(ROOT, "profiles", "decode_pages_traffic.json")
     if os.path.exists(tpath):
@@ -352,6 +373,8 @@ def main():
     gqa_w = DecodeWorkload("gqa decode", 16, 8192, 32, 8, 128, 3, 4, n_pools=4, seed=2, dist="normal", device=device)
     gqa_ms, _ = time_steps(gqa_w.step, args.steps, args.warmup)
     gqa_kern = time_kernel_stage(gqa_w, args.steps, args.warmup)
+
+    hybrid_gqa = hybrid_step_bench(gqa_w, max(20, args.steps // 4), max(5, args.warmup // 5))
 
     quant, (qpool, qk, qv, qtable, qtq) = quantize_bench(device, max(5, args.steps // 5), max(2, args.warmup // 5))
 
@@ -393,6 +416,9 @@ def main():
                        "GBps": gqa_w.bytes / (gqa_ms * 1e-3) / 1e9, "ms_per_step": gqa_ms,
                        "kernel_GBps": gqa_w.bytes / (gqa_kern * 1e-3) / 1e9,
                        "pct_hbm_peak": 100.0 * gqa_w.bytes / (gqa_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
+        "decode_hybrid": {"note": "whole step with the newest 128 tokens exact, read in place from a paged bf16 cache "
+                                  "(tq_decode_attn_paged_ring); compare ms_per_step of the compressed-only steps",
+                          "long_context": hybrid_main, "gqa": hybrid_gqa},
         "backend_decode_step": backend,
         "cpu_baseline": cpu,
     }
