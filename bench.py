@@ -152,14 +152,14 @@ def time_kernel_stage(work, steps, warmup):
     import torch
     from turboquant_amd import _ffi
     lib = _ffi.lib()
-    for i in range(warmup):
-        work.step(i)
     evs = []
     for _ in range(steps):
         a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         a.record(); b.record()                      # creates the underlying events
         evs.append((a, b))
     torch.cuda.synchronize()
+    for i in range(warmup):                         # the timed steps follow the warm-up without a pause
+        work.step(i)
     for i, (a, b) in enumerate(evs):
         lib.tq_time_next_page_kernel(a.cuda_event, b.cuda_event)
         work.step(warmup + i)
