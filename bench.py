@@ -126,9 +126,27 @@ def hybrid_step_bench(work, steps, warmup, ring=128):
     return {"exact_tokens": ring, "ms_per_step": ms}
 
 
-def time_steps(fn, steps, warmup):
+RAMP_SECONDS = 0.25      # --ramp-seconds
+
+
+def clock_ramp(fn, n_indices):
+    """Untimed: keeps the card busy with the leg's own step for RAMP_SECONDS, so that the W warm-up and K timed
+    steps that follow run at the steady clocks of a serving loop whatever W is (a card that has idled needs
+    ~0.2 s of sustained work to get there)."""
+    import torch
+    t0, i = time.perf_counter(), 0
+    while RAMP_SECONDS > 0 and time.perf_counter() - t0 < RAMP_SECONDS:
+        for _ in range(50):
+            fn(i % max(n_indices, 1))
+            i += 1
+        torch.cuda.synchronize()
+
+
+def time_steps(fn, steps, warmup, ramp=True):
     """(mean ms per step, wall ms per step) with HIP events on the launch stream."""
     import torch
+    if ramp:
+        clock_ramp(fn, warmup + steps)
     for i in range(warmup):
         fn(i)
     torch.cuda.synchronize()
@@ -158,6 +176,7 @@ def time_kernel_stage(work, steps, warmup):
         a.record(); b.record()                      # creates the underlying events
         evs.append((a, b))
     torch.cuda.synchronize()
+    clock_ramp(work.step, warmup + steps)
     for i in range(warmup):                         # the timed steps follow the warm-up without a pause
         work.step(i)
     for i, (a, b) in enumerate(evs):
@@ -280,10 +299,10 @@ def backend_step_bench(device, steps, warmup, n_layers=32, batch=32, context=327
     del k, v
     runner.seq_lens = [context] * batch
     toks = torch.randint(0, vocab, (warmup + steps, batch), generator=gen, device=device)
-    ms, _ = time_steps(lambda i: runner.decode_step(toks[i]), steps, warmup)
+    ms, _ = time_steps(lambda i: runner.decode_step(toks[i]), steps, warmup, ramp=False)
     # the same step captured once as a HIP graph and replayed (what a serving loop does)
     replay, _ = runner.capture_decode_step(context + slack, toks[0])
-    graph_ms, _ = time_steps(lambda i: replay(toks[i]), steps, warmup)
+    graph_ms, _ = time_steps(lambda i: replay(toks[i]), steps, warmup, ramp=False)
     # the compressed-KV part of a step alone: every layer's page write and fused decode attention
     meta = runner.decode_metadata()
     q1 = torch.randn(batch, hq, d, generator=gen, device=device, dtype=torch.bfloat16)
@@ -337,6 +356,8 @@ def main():
                     help="untimed steps before the timed ones; the card needs ~0.2 s of sustained work to reach its "
                          "steady clocks (with 50 steps the same build measures 5 %% slower decode steps and 17 %% "
                          "slower quantise passes)")
+    ap.add_argument("--ramp-seconds", type=float, default=0.25,
+                    help="untimed busy time before each leg's warm-up (clock ramp); 0 disables it")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--no-backend-step", action="store_true",
                     help="skip the full-decode-step leg (32-layer transformer through the backend hooks, ~60 GB)")
@@ -347,6 +368,8 @@ def main():
               "use --gpus 1", file=sys.stderr)
         sys.exit(2)
 
+    global RAMP_SECONDS
+    RAMP_SECONDS = max(0.0, args.ramp_seconds)
     import torch
     from turboquant_amd import _ffi
     if not os.path.exists(_ffi.library_path()):
@@ -409,7 +432,7 @@ def main():
                    "algorithmic_bytes_per_step": main_w.bytes, "stored_bytes_per_step": main_w.stored_bytes,
                    "n_split": main_w.n_split, "kv_pools_rotated": len(main_w.pools)},
         "pct_hbm_peak": 100.0 * value / HBM_PEAK_GBS,
-        "wall_ms_per_step": wall,
+        "wall_ms_per_step": wall, "clock_ramp_s": RAMP_SECONDS,
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": traffic, "kernel": "decode_mfma_kernel",
                      "kernel_ms": kern_ms, "stream_read": stream,
