@@ -11,7 +11,10 @@
 // Score of a token (triton_kernels.py:49-53,138):
 //   s = sm_scale * ( norm * sum_j q_rot[j] c[idx_j] + qjl_scale * rnorm * sum_j q_sk[j] sigma_j )
 
+#include <atomic>
+
 #include "tq_common.h"
+#include "tq_prep.h"
 
 namespace tq {
 
@@ -450,22 +453,45 @@ static size_t tail_words_smem(int d, int recent_rows) {
 // exact cache of 16-token blocks (rk / rv its base, ws_blk / ws_r / ws_h its block, token and head
 // strides in words); token p of sequence b sits in slot p % 16 of block block_table[b][p / 16].
 // Otherwise rk / rv are (B, recent_rows, H, d) rows with strides ws_b / ws_r / ws_h and recent_len valid rows.
+struct TailArgs {
+  const void* q;
+  int Hq, Hkv, d;
+  const uint32_t *rk, *rv;
+  int recent_rows;
+  int64_t ws_b, ws_r, ws_h;
+  const int32_t* recent_len;
+  const int32_t* block_table;
+  int bt_stride;
+  const int32_t* seq_lens;
+  int64_t ws_blk;
+  float sm_scale;
+  float* parts;
+  int n_parts, part_index;
+};
+
+// (a device function: the stand-alone kernel and the launch that shares its grid with the query
+// preparation both run it; h / b / gz are the workgroup's KV head, sequence and head group, `sm` its LDS)
 template <int DT, int KC, bool PAGED>
-__global__ void __launch_bounds__(TAIL_THREADS)
-exact_tail_words_kernel(const void* __restrict__ q, int Hq, int Hkv, int d, const uint32_t* __restrict__ rk,
-                        const uint32_t* __restrict__ rv, int recent_rows, int64_t ws_b, int64_t ws_r, int64_t ws_h,
-                        const int32_t* __restrict__ recent_len, const int32_t* __restrict__ block_table, int bt_stride,
-                        const int32_t* __restrict__ seq_lens, int64_t ws_blk, float sm_scale,
-                        float* __restrict__ parts, int n_parts, int part_index) {
+__device__ __forceinline__ void exact_tail_words_body(const TailArgs& A, int h, int b, int gz, float* sm) {
+  const void* __restrict__ q = A.q;
+  const int Hq = A.Hq, Hkv = A.Hkv, d = A.d, recent_rows = A.recent_rows, bt_stride = A.bt_stride;
+  const uint32_t* __restrict__ rk = A.rk;
+  const uint32_t* __restrict__ rv = A.rv;
+  const int64_t ws_b = A.ws_b, ws_r = A.ws_r, ws_h = A.ws_h, ws_blk = A.ws_blk;
+  const int32_t* __restrict__ recent_len = A.recent_len;
+  const int32_t* __restrict__ block_table = A.block_table;
+  const int32_t* __restrict__ seq_lens = A.seq_lens;
+  const float sm_scale = A.sm_scale;
+  float* __restrict__ parts = A.parts;
+  const int n_parts = A.n_parts, part_index = A.part_index;
   constexpr int GC = TAIL_GC, EPW = TailWord<DT>::EPW, RPT = TAIL_RPT / KC;
-  const int G = Hq / Hkv, h = blockIdx.x, b = blockIdx.y, g0 = blockIdx.z * GC, tid = threadIdx.x;
+  const int G = Hq / Hkv, g0 = gz * GC, tid = threadIdx.x;
   const int Gc = min(GC, G - g0);
   const int lane = tid & 63, wave = tid >> 6;
   const int seq = PAGED ? seq_lens[b] : 0;
   const int R = PAGED ? max(min(seq, recent_rows), 0) : (recent_len ? min(recent_len[b], recent_rows) : recent_rows);
   const int first = PAGED ? seq - R : 0;            // position of the first exact token
   const int32_t* bt = block_table + (PAGED ? (int64_t)b * bt_stride : 0);
-  extern __shared__ __align__(16) float sm[];
   float* sq = sm;                                   // [d][GC]
   float* ss = sq + GC * d;                          // [recent_rows][GC] scores, then softmax weights
   float* sml = ss + GC * recent_rows;               // [GC][2]
@@ -649,6 +675,34 @@ exact_tail_words_kernel(const void* __restrict__ q, int Hq, int Hkv, int d, cons
   }
 }
 
+template <int DT, int KC, bool PAGED>
+__global__ void __launch_bounds__(TAIL_THREADS)
+exact_tail_words_kernel(TailArgs A) {
+  extern __shared__ __align__(16) float sm[];
+  exact_tail_words_body<DT, KC, PAGED>(A, blockIdx.x, blockIdx.y, blockIdx.z, sm);
+}
+
+// One launch for the two things a hybrid step does before its page kernel: the exact-tail workgroups
+// (the first n_tail, so that the longer-running ones start first) and the query preparation of the
+// matrix-core kernel.  They are independent of each other, both have 512 lanes, and together they are
+// far fewer workgroups than the card has compute units, so the launch takes as long as the slower of
+// the two instead of their sum plus a dispatch gap.
+static_assert(TAIL_THREADS == PREP_COLS * PREP_SLICES, "the two roles share a workgroup size");
+template <int PER, int DT, bool PAGED>
+__global__ void __launch_bounds__(TAIL_THREADS)
+prep_tail_kernel(TailArgs A, int n_tail, int B, int Gq, tq_layer ly, float* __restrict__ q_rot, float* __restrict__ q_sk,
+                 float* __restrict__ q_stat, uint32_t* __restrict__ qa_pack) {
+  extern __shared__ __align__(16) float sm[];
+  const int id = blockIdx.x;
+  if (id < n_tail) {
+    const int per_z = A.Hkv * B;
+    exact_tail_words_body<DT, 1, PAGED>(A, id % A.Hkv, (id / A.Hkv) % B, id / per_z, sm);
+  } else {
+    const int words = ly.d / PREP_COLS, p = id - n_tail;
+    prep_query_body<PER, DT>(A.q, Gq, ly, A.sm_scale, q_rot, q_sk, q_stat, qa_pack, p / words, p % words, sm);
+  }
+}
+
 // n_parts partials are merged per row; consecutive rows are part_stride partials apart.
 // One workgroup per row.  A thread owns a pair of channels and every S-th part (S = 256 / (d/2)
 // subsets share the parts when a row has fewer than 256 channel pairs); its first MERGE_CHUNK
@@ -770,6 +824,19 @@ extern "C" int tq_decode_merge(const float* parts, int64_t rows, int n_parts, in
 }
 
 namespace {
+int compute_units() {
+  static std::atomic<int> cached{0};
+  int v = cached.load();
+  if (!v) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0)
+      v = 1;
+    cached.store(v);
+  }
+  return v;
+}
+
 // The exact tokens of a step.  Rows: (B, rows, H, d) tensors with element strides s_b / s_r / s_h and `len`
 // valid rows per sequence.  Paged: the newest min(seq_len, rows) tokens of every sequence, read in place
 // from a paged exact cache (block stride s_blk, token stride s_r, head stride s_h) through the step's
@@ -820,12 +887,61 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
                           layer->Pi_colsum &&
                           layer->S_colsum;
 
+  if (dtype < TQ_F32 || dtype > TQ_BF16) return TQ_EINVAL;
+  // the exact tail as 32-bit words: always for fp32, for 16-bit rows when they are word-aligned
+  const int epw = dtype == TQ_F32 ? 1 : 2;
+  const bool words = epw == 1 || (((((uintptr_t)recent_k | (uintptr_t)recent_v) & 3) == 0) &&
+                                  !((rs_b | rs_r | rs_h | ts.s_blk) & 1));
+  if (tail && ts.paged && !words) return TQ_EUNSUPPORTED;       // a paged exact cache has to be word-aligned
+  TailArgs ta;
+  ta.q = q; ta.Hq = Hq; ta.Hkv = Hkv; ta.d = d;
+  ta.rk = (const uint32_t*)recent_k; ta.rv = (const uint32_t*)recent_v; ta.recent_rows = recent_rows;
+  ta.ws_b = rs_b / epw; ta.ws_r = rs_r / epw; ta.ws_h = rs_h / epw; ta.recent_len = recent_len;
+  ta.block_table = block_table; ta.bt_stride = bt_stride; ta.seq_lens = seq_lens; ta.ws_blk = ts.s_blk / epw;
+  ta.sm_scale = sm_scale; ta.parts = parts; ta.n_parts = n_parts; ta.part_index = n_split;
+  const int n_tail = Hkv * B * ((G + TAIL_GC - 1) / TAIL_GC);
+  bool tail_done = false;
+
   if (stages & 1) {
     if (!layer->Pi || !layer->PiT || !layer->S || !layer->ST || !layer->centroids) return TQ_ENULL;
-    if (dtype < TQ_F32 || dtype > TQ_BF16) return TQ_EINVAL;
-    int rc = launch_rotate_query(q, dtype, (int64_t)B * Hq, layer, q_rot, q_sk, q_stat, mfma_shape ? qa_pack : nullptr,
-                                 mfma_shape ? Gq : G, sm_scale, st);
-    if (rc) return rc;
+    const int n_prep = (B * Hq / Gq) * (d / PREP_COLS);
+    // Whole hybrid step on the matrix-core path: the exact tail shares the preparation's launch, as long as
+    // every workgroup of the two gets a compute unit of its own at once (a tail workgroup's LDS fills one).
+    if (tail && words && mfma_shape && stages == 7 && n_tail + n_prep <= compute_units()) {
+      size_t fsm = tail_words_smem(d, recent_rows);
+      if (prep_smem_bytes(Gq, d) > fsm) fsm = prep_smem_bytes(Gq, d);
+#define TQ_LAUNCH_PT(PER, DT, PAGED)                                                                                 \
+  {                                                                                                                  \
+    auto kern = prep_tail_kernel<PER, DT, PAGED>;                                                                    \
+    if (fsm > 48 * 1024) {                                                                                           \
+      hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)fsm);   \
+      if (e != hipSuccess) return (int)e;                                                                            \
+    }                                                                                                                \
+    kern<<<dim3((unsigned)(n_tail + n_prep)), dim3(TAIL_THREADS), fsm, st>>>(ta, n_tail, B, Gq, *layer, q_rot, q_sk,  \
+                                                                            q_stat, qa_pack);                        \
+  }
+#define TQ_LAUNCH_PT_DT(PER, PAGED)                                \
+  {                                                                \
+    if (dtype == TQ_BF16) TQ_LAUNCH_PT(PER, TQ_BF16, PAGED)        \
+    else if (dtype == TQ_F16) TQ_LAUNCH_PT(PER, TQ_F16, PAGED)     \
+    else TQ_LAUNCH_PT(PER, TQ_F32, PAGED)                          \
+  }
+      if (d == 128) {
+        if (ts.paged) TQ_LAUNCH_PT_DT(8, true)
+        else TQ_LAUNCH_PT_DT(8, false)
+      } else {
+        if (ts.paged) TQ_LAUNCH_PT_DT(16, true)
+        else TQ_LAUNCH_PT_DT(16, false)
+      }
+#undef TQ_LAUNCH_PT_DT
+#undef TQ_LAUNCH_PT
+      TQ_CHECK_LAUNCH();
+      tail_done = true;
+    } else {
+      int rc = launch_rotate_query(q, dtype, (int64_t)B * Hq, layer, q_rot, q_sk, q_stat,
+                                   mfma_shape ? qa_pack : nullptr, mfma_shape ? Gq : G, sm_scale, st);
+      if (rc) return rc;
+    }
   }
   if (!(stages & 6)) return TQ_OK;
 
@@ -866,12 +982,8 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   TQ_CHECK_LAUNCH();
   }
 
-  if (tail && (stages & 2)) {
+  if (tail && (stages & 2) && !tail_done) {
     const dim3 tgrid(Hkv, B, (G + TAIL_GC - 1) / TAIL_GC);
-    const int epw = dtype == TQ_F32 ? 1 : 2;
-    const bool words = epw == 1 || (((((uintptr_t)recent_k | (uintptr_t)recent_v) & 3) == 0) &&
-                                    !((rs_b | rs_r | rs_h | ts.s_blk) & 1));
-    if (ts.paged && !words) return TQ_EUNSUPPORTED;             // a paged exact cache has to be word-aligned
     size_t tsm = words ? tail_words_smem(d, recent_rows) : tail_smem(d, recent_rows);
 #define TQ_LAUNCH_TAIL(KERN, ...)                                                                                    \
   {                                                                                                                  \
@@ -883,8 +995,7 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
     kern<<<tgrid, dim3(TAIL_THREADS), tsm, st>>>(__VA_ARGS__);                                                       \
   }
 #define TQ_TAIL_ROWS_ARGS q, Hq, Hkv, d, recent_k, recent_v, recent_rows, rs_b, rs_r, rs_h, recent_len, sm_scale, parts, n_parts, n_split
-#define TQ_TAIL_WORD_ARGS q, Hq, Hkv, d, (const uint32_t*)recent_k, (const uint32_t*)recent_v, recent_rows, rs_b / epw, rs_r / epw, \
-                          rs_h / epw, recent_len, block_table, bt_stride, seq_lens, ts.s_blk / epw, sm_scale, parts, n_parts, n_split
+#define TQ_TAIL_WORD_ARGS ta
 #define TQ_TAIL_WORDS(PAGED)                                                                                   \
   {                                                                                                            \
     if (dtype == TQ_BF16) TQ_LAUNCH_TAIL((exact_tail_words_kernel<TQ_BF16, 1, PAGED>), TQ_TAIL_WORD_ARGS)      \

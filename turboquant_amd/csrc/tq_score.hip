@@ -2,6 +2,7 @@
 // sketch, the asymmetric score estimator, and key / value de-quantisation.
 
 #include "tq_common.h"
+#include "tq_prep.h"
 
 namespace tq {
 
@@ -11,7 +12,7 @@ namespace tq {
 // ROT_COLS x ROT_SLICES threads: thread (j, s) sums slice s of the contraction for
 // its column of every row, so each matrix element is read once per workgroup; the
 // slices meet in LDS.
-constexpr int ROT_MAX_ROWS = 8, ROT_COLS = 32, ROT_SLICES = 8;
+constexpr int ROT_COLS = 32, ROT_SLICES = 8;
 
 __global__ void __launch_bounds__(ROT_COLS * ROT_SLICES)
 rotate_query_kernel(const void* __restrict__ q, int dtype, int64_t rows, int R, tq_layer ly, float* __restrict__ q_rot,
@@ -67,247 +68,13 @@ rotate_query_kernel(const void* __restrict__ q, int dtype, int64_t rows, int R, 
   }
 }
 
-// Fused preparation of the matrix-core decode kernel: rotation, sketch, statistics and
-// operand packing in one launch.  A workgroup owns one GQA group (G query heads of one KV
-// head) and the 32 output coordinates of one plane word; PREP_SLICES threads share a
-// coordinate's contraction.  Nothing depends on another workgroup, because the operands
-// are normalised by bounds that every workgroup can compute from the raw query:
-// |q_rot_j| <= ||q|| (Pi is orthogonal) and |q_sk_j| <= ||q|| max_j ||S_j||, and the sums
-// over all coordinates that the decode kernel needs are q . colsum(Pi), q . colsum(S).
-//
-// Everything that multiplies a whole score is folded into the operands: with k = sm_scale log2(e)
-// the index planes carry  k coef q_rot_j  and the sign plane  2 k qjl_scale q_sk_j, each divided
-// by a power of two 2^E >= its bound (E per query head and kind), which the decode kernel gives
-// back through the MFMA's per-row block scale.  q_stat per row:
-// {E_index, E_sign (as floats), k c0 sum_j q_rot_j, -k qjl_scale sum_j q_sk_j}: the last two
-// are the constant parts of the score and start the MFMA accumulators.
-//
-// qa_pack receives the score-stage A operands of v_mfma_scale_f32_16x16x128_f8f6f4 (A fp6 e2m3, which
-// runs at twice the fp8 rate; B fp4) in register order: [kv head][term plane][128-coordinate chunk i]
-// [row set][lane][8 dwords, 6 used].  A value v (the normalised query coordinate times the plane's
-// coefficient, |v| <= 1) is the sum of four fp6 terms with per-row block scales 2^-2, 2^-7, 2^-12,
-// 2^-17: t0 = fp6(4 v), t1 = fp6(32 (4 v - t0)), t2 = fp6(32 (32 (4 v - t0) - t1)), ...; a term's
-// rounding error is at most 1/8, so every product stays within the fp6 range and the sum is good to
-// 2^-20.  Row set 0 holds terms 0 and 1 (row 2g + t for head g), row set 1 terms 2 and 3, so that
-// both accumulate into the same MFMA output registers (8 heads x 4 terms fill the 2 x 16 rows).  For 6-bit operands lane
-// (row, block b) holds contraction indices 32b..32b+31, index j at bits 6j..6j+5 of its 192 bits, and
-// the key kernel puts coordinate c of plane word w at contraction index 32w + 8 (c % 4) + c / 4.
-constexpr int PREP_COLS = 32, PREP_SLICES = 16;
-
-// round to the fp6 e2m3 grid (1 sign, 2 exponent, 3 mantissa bits; steps 1/8 below 2, 1/4 below 4,
-// 1/2 up to the maximum 7.5), nearest even; returns the rounded value and its 6-bit code
-__device__ __forceinline__ float round_fp6(float v, uint32_t& code) {
-  const float a = fminf(fabsf(v), 7.5f);
-  const float inv_step = a < 2.0f ? 8.0f : (a < 4.0f ? 4.0f : 2.0f);
-  const float r = rintf(a * inv_step) / inv_step;    // exact (powers of two); may land on the next binade
-  const int e = r < 1.0f ? 0 : (r < 2.0f ? 1 : (r < 4.0f ? 2 : 3));
-  const float inv_unit = e <= 1 ? 8.0f : (e == 2 ? 4.0f : 2.0f);
-  const int m = (int)(r * inv_unit) - (e == 0 ? 0 : 8);
-  code = (v < 0.0f && r != 0.0f ? 32u : 0u) | ((uint32_t)e << 3) | (uint32_t)m;
-  return v < 0.0f ? -r : r;
-}
-
-// sum over the 64 lanes with DPP row operations and four lane reads (no shared-memory permutes)
-template <int CTRL>
-__device__ __forceinline__ float prep_dpp(float v) {
-  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
-}
-__device__ __forceinline__ float wave_sum_dpp(float v) {
-  v += prep_dpp<0xB1>(v);      // quad_perm [1,0,3,2]
-  v += prep_dpp<0x4E>(v);      // quad_perm [2,3,0,1]
-  v += prep_dpp<0x141>(v);     // row_half_mirror
-  v += prep_dpp<0x140>(v);     // row_mirror: every lane holds its row's sum
-  const int b = __builtin_bit_cast(int, v);
-  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 0)) + __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 16)) +
-         __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 32)) + __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48));
-}
-
-// PER = matrix rows per thread = d / PREP_SLICES; DT = element type of the query (a template parameter:
-// a run-time switch would put each query load under a branch, and the loads would wait for one another)
 template <int PER, int DT>
 __global__ void __launch_bounds__(PREP_COLS * PREP_SLICES)
 prep_query_kernel(const void* __restrict__ q, int G, tq_layer ly, float sm_scale,
                   float* __restrict__ q_rot, float* __restrict__ q_sk, float* __restrict__ q_stat,
                   uint32_t* __restrict__ qa_pack) {
   extern __shared__ float sm[];
-  const int d = ly.d, tid = threadIdx.x, jl = tid % PREP_COLS, sl = tid / PREP_COLS;
-  const int word = blockIdx.y, j = word * PREP_COLS + jl;
-  // every global load of the kernel is issued here, before anything waits, the query first: loads
-  // return in order, so the query can go to shared memory (and its statistics be taken) while the
-  // matrix slices, which do not depend on it, are still on their way
-  const int64_t group = blockIdx.x, row0 = group * G;
-  constexpr int QPT = ROT_MAX_ROWS * 256 / (PREP_COLS * PREP_SLICES);   // query elements per thread, d <= 256
-  float qv[QPT];
-#pragma unroll
-  for (int k = 0; k < QPT; ++k) {
-    const int o = tid + k * (PREP_COLS * PREP_SLICES);
-    const float x = Elem<DT>::load(q, row0 * d + min(o, G * d - 1));      // unconditional, clamped
-    qv[k] = o < G * d ? x : 0.0f;
-  }
-  float mp[PER], ms[PER];
-#pragma unroll
-  for (int k = 0; k < PER; ++k) {
-    mp[k] = ly.PiT[(int64_t)(sl * PER + k) * d + j];
-    ms[k] = ly.ST[(int64_t)(sl * PER + k) * d + j];
-  }
-  float cs1[4], cs2[4];                            // column sums at coordinates lane, lane + 64, ...
-#pragma unroll
-  for (int k = 0; k < 4; ++k) {
-    const int c = (tid & 63) + 64 * k;
-    cs1[k] = c < d ? ly.Pi_colsum[c] : 0.0f;
-    cs2[k] = c < d ? ly.S_colsum[c] : 0.0f;
-  }
-  float* sq = sm;                                   // [G][d] raw query
-  float* pa = sq + G * d;                           // [PREP_SLICES][G][PREP_COLS]
-  float* pb = pa + PREP_SLICES * G * PREP_COLS;
-  float* srot = pb + PREP_SLICES * G * PREP_COLS;   // [G][PREP_COLS]
-  float* ssk = srot + G * PREP_COLS;
-  float* stat = ssk + G * PREP_COLS;                // [G][4]
-  float* coefs = stat + 4 * ROT_MAX_ROWS;           // [16]
-#pragma unroll
-  for (int k = 0; k < QPT; ++k) {
-    const int o = tid + k * (PREP_COLS * PREP_SLICES);
-    if (o < G * d) sq[o] = qv[k];
-  }
-  const int mb = ly.mse_bits;
-  int nx = 0;
-  float cmax = 0.0f;
-  for (int t = 0; t < ly.n_terms; ++t) {
-    cmax = fmaxf(cmax, fabsf(ly.term_coef[t]));
-    if (__builtin_popcount(ly.term_mask[t]) > 1) ++nx;
-  }
-  const int ntp = mb + nx + 1, wpl = d / 128;
-  if (tid < ntp) {
-    float coef = 1.0f;
-    if (tid < mb) {
-      coef = 0.0f;
-      for (int t = 0; t < ly.n_terms; ++t)
-        if (ly.term_mask[t] == (1 << (mb - 1 - tid))) coef = ly.term_coef[t];
-    } else if (tid < mb + nx) {
-      coef = 0.0f;
-      int seen = 0;
-      for (int t = 0; t < ly.n_terms; ++t) {
-        if (__builtin_popcount(ly.term_mask[t]) > 1) {
-          if (seen == tid - mb) coef = ly.term_coef[t];
-          ++seen;
-        }
-      }
-    }
-    coefs[tid] = coef;
-  }
-  __syncthreads();
-  {  // row statistics: one wavefront per row
-    const int lane = tid & 63, wave = tid >> 6, n_wave = blockDim.x >> 6;
-    for (int r = wave; r < G; r += n_wave) {
-      float ss = 0.0f, s1 = 0.0f, s2 = 0.0f;
-#pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        const int c = lane + 64 * k;
-        const float x = c < d ? sq[r * d + c] : 0.0f;
-        ss = fmaf(x, x, ss);
-        s1 = fmaf(x, cs1[k], s1);
-        s2 = fmaf(x, cs2[k], s2);
-      }
-      ss = wave_sum_dpp(ss); s1 = wave_sum_dpp(s1); s2 = wave_sum_dpp(s2);
-      if (lane == 0) {
-        const float nq = sqrtf(ss), k = sm_scale * 1.4426950408889634f;
-        // bound < 2^e: e = exponent field - 126 (the mantissa of frexp is below 1), kept within
-        // +-100 (a zero, denormal or huge bound only has to stay finite)
-        const int e1 = min(max((int)((__float_as_uint(fabsf(k) * nq * cmax) >> 23) & 255u) - 126, -100), 100);
-        const int e2 = min(max((int)((__float_as_uint(2.0f * fabsf(k * ly.qjl_scale) * nq * ly.S_rownorm_max) >> 23) & 255u) - 126, -100), 100);
-        stat[r * 4 + 0] = k * __uint_as_float((uint32_t)(127 - e1) << 23);                       // multiplier of coef q_rot_j
-        stat[r * 4 + 1] = 2.0f * k * ly.qjl_scale * __uint_as_float((uint32_t)(127 - e2) << 23); // multiplier of q_sk_j
-        if (word == 0) {
-          q_stat[(row0 + r) * 4 + 0] = (float)e1; q_stat[(row0 + r) * 4 + 1] = (float)e2;
-          q_stat[(row0 + r) * 4 + 2] = k * ly.term_const * s1; q_stat[(row0 + r) * 4 + 3] = -k * ly.qjl_scale * s2;
-        }
-      }
-    }
-  }
-  // contraction over this thread's PER matrix rows
-  {
-    const int i0 = sl * PER;
-    float a[ROT_MAX_ROWS], b[ROT_MAX_ROWS];
-#pragma unroll
-    for (int r = 0; r < ROT_MAX_ROWS; ++r) a[r] = b[r] = 0.0f;
-#pragma unroll
-    for (int r = 0; r < ROT_MAX_ROWS; ++r) {
-      if (r < G) {
-#pragma unroll
-        for (int k4 = 0; k4 < PER / 4; ++k4) {
-          const float4 x = *(const float4*)(sq + r * d + i0 + 4 * k4);
-          const float xs[4] = {x.x, x.y, x.z, x.w};
-#pragma unroll
-          for (int k = 0; k < 4; ++k) {
-            a[r] = fmaf(xs[k], mp[4 * k4 + k], a[r]);
-            b[r] = fmaf(xs[k], ms[4 * k4 + k], b[r]);
-          }
-        }
-      }
-    }
-#pragma unroll
-    for (int r = 0; r < ROT_MAX_ROWS; ++r) {
-      if (r < G) {
-        pa[(sl * G + r) * PREP_COLS + jl] = a[r];
-        pb[(sl * G + r) * PREP_COLS + jl] = b[r];
-      }
-    }
-  }
-  __syncthreads();
-  for (int o2 = tid; o2 < 2 * G * PREP_COLS; o2 += blockDim.x) {      // first half: rotation, second: sketch
-    const bool sk = o2 >= G * PREP_COLS;
-    const int o = sk ? o2 - G * PREP_COLS : o2, r = o / PREP_COLS, c = o - r * PREP_COLS;
-    const float* part = sk ? pb : pa;
-    float acc = 0.0f;
-#pragma unroll
-    for (int k = 0; k < PREP_SLICES; ++k) acc += part[(k * G + r) * PREP_COLS + c];
-    (sk ? ssk : srot)[o] = acc;
-    (sk ? q_sk : q_rot)[(row0 + r) * d + word * PREP_COLS + c] = acc;
-  }
-  __syncthreads();
-  // operands of this plane word.  First the four 6-bit codes of every (term plane, head, contraction
-  // index) into shared memory (the partial sums are no longer needed), then per (term plane, row set,
-  // row) one lane x six dwords, each gathered from the (up to seven) codes that overlap it.
-  uint32_t* codes = (uint32_t*)pa;                           // [ntp][G][4 terms][32]
-  // thread -> (contraction index, head, half of the workgroup); the halves take alternate term planes
-  for (int tp = tid >> 8; tp < ntp; tp += 2) {
-    const int kloc = tid & 31, g = (tid >> 5) & 7;
-    if (g >= G) break;
-    const bool is_sign = tp == ntp - 1;
-    const int c = 4 * (kloc & 7) + (kloc >> 3);              // coordinate within the word
-    // the decode kernel extracts three of the four bits of a nibble in place, where they are the fp4
-    // numbers 1, 2 and 4 (after its block scale): the query side divides them out
-    const int t4 = kloc >> 3;
-    const float mul = 4.0f * (is_sign ? stat[g * 4 + 1] : coefs[tp] * stat[g * 4 + 0]) *
-                      (t4 == 1 ? 0.5f : (t4 == 2 ? 0.25f : 1.0f));
-    float v = (is_sign ? ssk : srot)[g * PREP_COLS + c] * mul;
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      uint32_t code;
-      const float r = round_fp6(v, code);
-      codes[((tp * G + g) * 4 + t) * PREP_COLS + kloc] = code;
-      v = (v - r) * 32.0f;
-    }
-  }
-  __syncthreads();
-  const int i = word >> 2, kw = word & 3;
-  uint32_t* dst = qa_pack + group * (int64_t)(ntp * wpl * 2 * 64 * 8);
-  for (int o = tid; o < ntp * 256; o += blockDim.x) {
-    const int dwi = o & 7, n = (o >> 3) & 15, rs = (o >> 7) & 1, tp = o >> 8;
-    if (dwi >= 6) continue;
-    const int g = n >> 1;
-    const int term = 2 * rs + (n & 1);
-    uint32_t packed = 0;
-    if (g < G) {
-      const uint32_t* cd = codes + ((tp * G + g) * 4 + term) * PREP_COLS;
-      const int j0 = (32 * dwi) / 6, j1 = min((32 * dwi + 31) / 6, 31);
-      for (int kloc = j0; kloc <= j1; ++kloc) {
-        const int bit = 6 * kloc - 32 * dwi;                 // position of the code in this dword (may straddle)
-        packed |= bit >= 0 ? cd[kloc] << bit : cd[kloc] >> -bit;
-      }
-    }
-    dst[(((tp * wpl + i) * 2 + rs) * 64 + n + 16 * kw) * 8 + dwi] = packed;
-  }
+  prep_query_body<PER, DT>(q, G, ly, sm_scale, q_rot, q_sk, q_stat, qa_pack, blockIdx.x, blockIdx.y, sm);
 }
 
 // scores[b, i, k] for a tile of QT queries and one key per thread.  The rotated and sketched queries sit
@@ -590,8 +357,7 @@ int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* 
   if (qa_pack) {       // operands of the matrix-core decode kernel wanted
     if (!q_stat || !layer->Pi_colsum || !layer->S_colsum || G > ROT_MAX_ROWS || rows % G || (d != 128 && d != 256))
       return TQ_EUNSUPPORTED;
-    size_t smem = (size_t)(G * d + 2 * PREP_SLICES * G * PREP_COLS + 2 * G * PREP_COLS + 4 * ROT_MAX_ROWS + 32) *
-                  sizeof(float);
+    size_t smem = prep_smem_bytes(G, d);
     const dim3 grid((unsigned)(rows / G), d / PREP_COLS), block(PREP_COLS * PREP_SLICES);
 #define TQ_PREP(PER, DT) prep_query_kernel<PER, DT><<<grid, block, smem, st>>>(q, G, *layer, sm_scale, q_rot, q_sk, q_stat, qa_pack)
 #define TQ_PREP_DT(PER)                              \
