@@ -6,6 +6,7 @@
 //            group are scored from one read of the page; online softmax and the
 //            value accumulation stay in registers; result = partial (m, l, acc)
 //            exact_tail_words_kernel / exact_tail_kernel: the same partial for the exact recent tokens
+//            (prep_tail_kernel: stage 0 and the exact tail in one launch, for small grids)
 //   stage 2  merge_kernel: log-sum-exp merge of the partials, cast to q's dtype
 //
 // Score of a token (triton_kernels.py:49-53,138):
