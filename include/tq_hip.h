@@ -174,6 +174,17 @@ int tq_append_kv_paged(const void *k, const void *v, int dtype, int B, int T, in
                        int max_pages, const tq_layer *layer, const tq_page_layout *layout, uint8_t *pool,
                        int64_t num_pages, void *stream);
 
+/* Ragged batch of runs (the batch counterpart of CompressedKVStore.append_chunk, store.py:73-90, for an
+ * engine step that carries several sequences): k / v are (rows, H, d) `dtype` with element strides
+ * stride_t / stride_h, the run of sequence b is rows row0[b] .. row0[b] + run_len[b] - 1 (run_len[b] <=
+ * T_max, 0 = nothing) and lands at token positions start_pos[b] .. of the pages block_table[b*max_pages + i].
+ * All three arrays are device int32 (B,): row0 = query_start_loc[:-1], run_len = its differences,
+ * start_pos = seq_lens - run_len for an engine's step metadata.  Pages as tq_append_kv_paged writes them. */
+int tq_append_kv_ragged(const void *k, const void *v, int dtype, int B, int T_max, int H, int64_t stride_t,
+                        int64_t stride_h, const int32_t *row0, const int32_t *run_len, const int32_t *start_pos,
+                        const int32_t *block_table, int max_pages, const tq_layer *layer,
+                        const tq_page_layout *layout, uint8_t *pool, int64_t num_pages, void *stream);
+
 /* The same for tokens that already sit in a paged exact KV cache (gather + quantise in one pass;
  * capture.py:187-217 ingest_prefill_from_paged_cache gathers the blocks with torch indexing first).
  * k_cache, v_cache: blocks of 16 tokens, element (block, slot, h, :) at

@@ -1113,3 +1113,34 @@ def test_config3_full_size_decode_against_the_oracle(gpu):
     _progress(f"   worst cosine over 16 sequences {worst:.7f}")
     worst = _decode_case(gpu, 128, 3, 4, 4, 32, 8, [8192, 8191, 4097, 8192], [128, 0, 5, 64], seed=3, n_split=7)
     _progress(f"   ragged, hybrid, 7 splits: worst cosine {worst:.7f}")
+
+
+@pytest.mark.parametrize("d,key_bits,vb,dtype", [(128, 3, 4, torch.bfloat16), (256, 3, 2, torch.bfloat16),
+                                                   (64, 2, 2, torch.float16)])
+def test_append_ragged_equals_one_append_per_sequence(gpu, d, key_bits, vb, dtype):
+    """tq_append_kv_ragged writes a step's ragged rows (several sequences, each continuing at its own
+    position, store.py:73-90 per sequence) in one call; the pages must equal, byte for byte, one
+    tq_append_kv_paged call per sequence."""
+    g = torch.Generator().manual_seed(7 * d + vb)
+    H, per_seq = 2, 12
+    runs = [37, 0, 1, 150, 16, 5]
+    starts = [0, 20, 33, 7, 16, 170]
+    B, n_pages = len(runs), len(runs) * per_seq
+    rows = sum(runs) + 9                                               # a few rows that belong to nobody
+    k = torch.randn(rows, H, d, generator=g).to(dtype).to(gpu)
+    v = torch.randn(rows, H, d, generator=g).to(dtype).to(gpu)
+    table = torch.randperm(n_pages, generator=g).view(B, per_seq).to(torch.int32).to(gpu)
+    row0 = [3]                                                         # the first run does not start at row 0
+    for r in runs[:-1]:
+        row0.append(row0[-1] + r)
+    _progress(f"append_ragged d={d} {dtype} runs={runs} starts={starts}")
+    pa, _ = _make_pool(gpu, d, key_bits, vb, H, n_pages, dtype)
+    pb, _ = _make_pool(gpu, d, key_bits, vb, H, n_pages, dtype)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=gpu)
+    pa.append_ragged(k, v, i32(row0), i32(runs), i32(starts), table, max_run=max(runs))
+    for b in range(B):
+        if runs[b]:
+            pb.append(k[None, row0[b]:row0[b] + runs[b]], v[None, row0[b]:row0[b] + runs[b]], table[b:b + 1],
+                      start_pos=i32([starts[b]]))
+    torch.cuda.synchronize()
+    assert torch.equal(pa.data, pb.data)

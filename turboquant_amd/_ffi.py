@@ -62,6 +62,8 @@ _SIGNATURES = {
     "tq_rotate_query": (C.c_int, [_vp, _i, _i64, C.POINTER(TqLayer), _vp, _vp, _vp]),
     "tq_append_kv_paged": (C.c_int, [_vp, _vp, _i, _i, _i, _i, _i64, _i64, _i64, _vp, _vp, _i,
                                      C.POINTER(TqLayer), C.POINTER(TqPageLayout), _vp, _i64, _vp]),
+    "tq_append_kv_ragged": (C.c_int, [_vp, _vp, _i, _i, _i, _i, _i64, _i64, _vp, _vp, _vp, _vp, _i,
+                                      C.POINTER(TqLayer), C.POINTER(TqPageLayout), _vp, _i64, _vp]),
     "tq_append_kv_from_blocks": (C.c_int, [_vp, _vp, _i, _i, _i, _i, _i64, _i64, _i64, _vp, _i, _vp, _vp, _vp, _i,
                                            C.POINTER(TqLayer), C.POINTER(TqPageLayout), _vp, _i64, _vp]),
     "tq_pool_export": (C.c_int, [_vp, _i64, _i, _vp, _i, C.POINTER(TqPageLayout), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),

@@ -44,6 +44,9 @@ struct PagedSource {         // (b, t, h, :) strided, tokens mapped onto 16-toke
   int src_stride = 0;
   int64_t stride_blk = 0;
   const int32_t* run_len = nullptr;
+  // Optional ragged mode: the rows of all sequences lie one after another in one (rows, H, :) tensor; the
+  // run of sequence b begins at row row0[b] (stride_b is unused, run_len gives its length).
+  const int32_t* row0 = nullptr;
   // tile index -> (b, page slot window, head)
   __device__ void decode(int tile, int& b, int& lpage, int& h) const {
     h = tile % H;
@@ -66,7 +69,8 @@ struct PagedSource {         // (b, t, h, :) strided, tokens mapped onto 16-toke
     const int lpage = s0 / TILE + pg, t0 = lpage * TILE - s0;
     const int lim = min(*(run_len ? run_len + b : &k_max_i32), T);
     const int64_t blk = *(src_table ? src_table + (int64_t)b * src_stride + min(lpage, src_stride - 1) : &k_zero_i32);
-    const int64_t base = src_table ? blk * stride_blk - (int64_t)t0 * stride_t : b * stride_b;
+    const int64_t r0 = *(row0 ? row0 + b : &k_zero_i32);
+    const int64_t base = src_table ? blk * stride_blk - (int64_t)t0 * stride_t : (row0 ? r0 * stride_t : b * stride_b);
     return TileRef{base + h * stride_h, t0, lim};
   }
   __device__ bool slot_off(const TileRef& r, int slot, int64_t& elem_off) const {

@@ -857,6 +857,24 @@ extern "C" int tq_append_kv_paged(const void* k, const void* v, int dtype, int B
   return append_runs(k, v, dtype, src, block_table, max_pages, layer, layout, pool, stream);
 }
 
+extern "C" int tq_append_kv_ragged(const void* k, const void* v, int dtype, int B, int T_max, int H, int64_t stride_t,
+                                   int64_t stride_h, const int32_t* row0, const int32_t* run_len,
+                                   const int32_t* start_pos, const int32_t* block_table, int max_pages,
+                                   const tq_layer* layer, const tq_page_layout* layout, uint8_t* pool,
+                                   int64_t num_pages, void* stream) {
+  int rc = check_layer(layer, true);
+  if (rc) return rc;
+  if (!k || !v || !row0 || !run_len || !start_pos || !block_table || !layout || !pool) return TQ_ENULL;
+  if (dtype != layout->dtype || layout->d != layer->d || layout->mse_bits != layer->mse_bits) return TQ_EINVAL;
+  if (B < 0 || T_max < 0 || H <= 0 || max_pages <= 0 || num_pages <= 0) return TQ_EINVAL;
+  if (B == 0 || T_max == 0) return TQ_OK;
+  const int tiles_per_seq = (T_max + TILE - 2) / TILE + 1;      // a run may begin at any slot of its first page
+  PagedSource src{B, T_max, H, tiles_per_seq, 0, stride_t, stride_h, start_pos};
+  src.run_len = run_len;
+  src.row0 = row0;
+  return append_runs(k, v, dtype, src, block_table, max_pages, layer, layout, pool, stream);
+}
+
 extern "C" int tq_append_kv_from_blocks(const void* k_cache, const void* v_cache, int dtype, int B, int T, int H,
                                         int64_t stride_blk, int64_t stride_t, int64_t stride_h,
                                         const int32_t* src_table, int src_stride, const int32_t* start_pos,

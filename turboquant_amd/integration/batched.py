@@ -78,13 +78,11 @@ class BatchedLayerState:
         if int(meta.max_query_len) == 1:                       # one token per sequence: a single batched append
             start = meta.seq_lens.to(torch.int32) - 1
             self.pool.append(k[:, None], v[:, None], table, start_pos=start)
-        else:                                                  # ragged rows: one append per sequence
-            lens, qsl = _host_list(meta, "seq_lens"), _host_list(meta, "query_start_loc")
-            for b in range(len(lens)):
-                r0, r1 = qsl[b], qsl[b + 1]
-                if r1 > r0:
-                    self.pool.append(k[None, r0:r1], v[None, r0:r1], table[b:b + 1],
-                                     start_pos=torch.tensor([lens[b] - (r1 - r0)], dtype=torch.int32))
+        else:                                                  # ragged rows: still one call, nothing read back
+            qsl = meta.query_start_loc.to(device=k.device, dtype=torch.int32)
+            run = qsl[1:] - qsl[:-1]
+            start = meta.seq_lens.to(device=k.device, dtype=torch.int32) - run
+            self.pool.append_ragged(k, v, qsl[:-1], run, start, table, max_run=int(meta.max_query_len))
         self.tokens_written += n
 
     def ingest_paged_cache(self, kv_cache: torch.Tensor, block_table: torch.Tensor, seq_lens: torch.Tensor,

@@ -116,6 +116,34 @@ class PagedKVPool:
                 block_table.shape[1], C.byref(ly), C.byref(self.layout), self.data.data_ptr(), self.num_pages,
                 _ffi.stream_ptr(self.device)), "tq_append_kv_from_blocks")
 
+    def append_ragged(self, key: torch.Tensor, value: torch.Tensor, row0: torch.Tensor, run_len: torch.Tensor,
+                      start_pos: torch.Tensor, block_table: torch.Tensor, max_run: int):
+        """Quantise a ragged batch of runs in one call: key / value (rows, H, d) hold the rows of all
+        sequences one after another; sequence b owns rows row0[b] .. row0[b] + run_len[b] - 1, which become
+        its tokens start_pos[b] .. in the pages of block_table[b].  row0 / run_len / start_pos are (B,) device
+        tensors (nothing is read back to the host); max_run bounds every run_len."""
+        _ffi.require_gpu(key, "key")
+        if key.dim() != 3 or key.shape != value.shape or tuple(key.shape[1:]) != (self.num_kv_heads, self.head_dim):
+            raise ValueError(f"expected key and value of shape (rows, {self.num_kv_heads}, {self.head_dim})")
+        if key.dtype != self.dtype or value.dtype != self.dtype:
+            raise TypeError(f"pool was laid out for {self.dtype}")
+        if key.stride(-1) != 1 or key.stride() != value.stride():
+            key, value = key.contiguous(), value.contiguous()
+        if block_table.dtype != torch.int32 or block_table.dim() != 2:
+            raise ValueError("block_table must be int32 (B, max_pages)")
+        B = block_table.shape[0]
+        block_table = block_table.contiguous()
+        arrs = [t.to(device=self.device, dtype=torch.int32).contiguous() for t in (row0, run_len, start_pos)]
+        if any(t.shape != (B,) for t in arrs):
+            raise ValueError("row0, run_len and start_pos must have one entry per row of block_table")
+        ly = self.quantizer._layer()
+        with torch.cuda.device(self.device):
+            _ffi.check(_ffi.lib().tq_append_kv_ragged(
+                key.data_ptr(), value.data_ptr(), _ffi.dtype_tag(self.dtype), B, int(max_run), self.num_kv_heads,
+                key.stride(0), key.stride(1), arrs[0].data_ptr(), arrs[1].data_ptr(), arrs[2].data_ptr(),
+                block_table.data_ptr(), block_table.shape[1], C.byref(ly), C.byref(self.layout),
+                self.data.data_ptr(), self.num_pages, _ffi.stream_ptr(self.device)), "tq_append_kv_ragged")
+
     # ---- read -------------------------------------------------------------------
     def export_flat(self, block_table_row: torch.Tensor, n_tok: int):
         """Gather one sequence's pages into the reference's flat tensors
