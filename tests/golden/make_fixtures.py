@@ -3,7 +3,7 @@
 Run from the repository root, in the build container only (the reference does
 not exist anywhere else):
 
-    python tests/golden/make_fixtures.py [/root/reference]
+    python tests/golden/make_fixtures.py [/root/reference [step ...]]
 
 The script imports the reference package from the given checkout, feeds it
 seeded synthetic inputs and stores inputs + outputs as .npz / .json data.  The
@@ -164,6 +164,46 @@ def key_cases():
         out[f"{name}.meta"] = np.array([d, bits, 42 + 7 * (seed % 3)])
     np.savez_compressed(os.path.join(HERE, "key_cases.npz"), **out)
     print("key_cases:", len(out), "arrays")
+
+
+# ---------------------------------------------------------------- keys, wide heads and the zero-coordinate bucket
+def key_cases_wide():
+    """head_dim 576 with 4-bit keys (the only d = 576 table the reference ships is the 3-bit one) and
+    head_dim 128 with 5-bit keys: the two shipped tables whose middle threshold is a tiny negative number
+    instead of 0, so that the all-zero vector in each case lands in the upper middle bucket.  The sketch
+    matrix S is not stored for d = 576 (1.3 MB): it is torch.randn of seed + 1000, which is bit-stable."""
+    out = {}
+    for name, d, bits, dt, seed, n_tok in (("bf16_d576_b4", 576, 4, torch.bfloat16, 17, 24),
+                                           ("bf16_d128_b5", 128, 5, torch.bfloat16, 18, 48)):
+        seed_codebook_cache(d, bits - 1)
+        g = torch.Generator(device="cpu").manual_seed(seed)
+        x = torch.randn(2, n_tok, d, generator=g, dtype=torch.float32)
+        ch = torch.randperm(d, generator=g)[:4]
+        x[..., ch] *= 20.0
+        x[0, 0] = 0.0
+        x[1, 3] = 0.0
+        x = x.to(dt)
+        q = torch.randn(2, 5, d, generator=g, dtype=torch.float32).to(dt)
+        tq = TurboQuantProd(d, bits=bits, device=CPU, seed=42 + 7 * (seed % 3))
+        code, y, p = key_trace(tq, x)
+        store_float(out, f"{name}.x", x)
+        store_float(out, f"{name}.q", q)
+        out[f"{name}.Pi"] = tq.mse_quantizer.Pi.numpy()
+        if d <= 256:
+            out[f"{name}.S"] = tq.S.numpy()
+        out[f"{name}.centroids"] = tq.mse_quantizer.centroids.numpy()
+        out[f"{name}.thresholds"] = tq.mse_quantizer.decision_boundaries.numpy()
+        out[f"{name}.y"] = y.numpy()
+        out[f"{name}.p"] = p.numpy()
+        out[f"{name}.mse_indices"] = code.mse_indices.numpy()
+        out[f"{name}.qjl_signs"] = code.qjl_signs.numpy()
+        store_float(out, f"{name}.norms", code.norms)
+        out[f"{name}.residual_norms"] = code.residual_norms.numpy()
+        out[f"{name}.dequant"] = tq.dequantize(code).numpy()
+        out[f"{name}.scores"] = tq.attention_score(q, code).numpy()
+        out[f"{name}.meta"] = np.array([d, bits, 42 + 7 * (seed % 3)])
+    np.savez_compressed(os.path.join(HERE, "key_cases_wide.npz"), **out)
+    print("key_cases_wide:", len(out), "arrays")
 
 
 # ---------------------------------------------------------------- packing
@@ -352,13 +392,11 @@ def kv_cache_object():
 
 if __name__ == "__main__":
     torch.manual_seed(0)
-    config1()
-    key_cases()
-    packing()
-    values()
-    codebooks_d256()
-    hybrid()
-    capture_trace()
-    kv_cache_object()
+    steps = {"config1": config1, "key_cases": key_cases, "key_cases_wide": key_cases_wide, "packing": packing,
+             "values": values, "codebooks_d256": codebooks_d256, "hybrid": hybrid, "capture_trace": capture_trace,
+             "kv_cache_object": kv_cache_object}
+    # python tests/golden/make_fixtures.py /root/reference [step ...]   (no step names = all of them)
+    for name in (sys.argv[2:] or list(steps)):
+        steps[name]()
     for f in sorted(os.listdir(HERE)):
         print(f, os.path.getsize(os.path.join(HERE, f)))

@@ -48,9 +48,17 @@ class Golden:
     def codebook(self, d, bits):
         return self.json(f"ref_codebook_d{d}_b{bits}.json")
 
+    def key_case_list(self):
+        """(file, case) of every golden key-quantiser case."""
+        return [(f, c) for f in ("key_cases", "key_cases_wide") for c in self.cases(f)]
+
     def key_params(self, file, case) -> O.KeyParams:
-        d, bits, _ = [int(v) for v in self.npz(file)[case + ".meta"]]
-        return O.KeyParams(self.tensor(file, case + ".Pi"), self.tensor(file, case + ".S"),
+        d, bits, seed = [int(v) for v in self.npz(file)[case + ".meta"]]
+        if self.has(file, case + ".S"):
+            S = self.tensor(file, case + ".S")
+        else:       # not stored for the widest case: S is torch.randn of seed + 1000, which is bit-stable
+            S = torch.randn(d, d, generator=torch.Generator().manual_seed(seed + 1000))
+        return O.KeyParams(self.tensor(file, case + ".Pi"), S,
                            self.tensor(file, case + ".centroids"), self.tensor(file, case + ".thresholds"), bits - 1)
 
 

@@ -42,8 +42,8 @@ def test_bucketize_and_sign_pack_bit_exact_on_reference_tensors(gpu, golden):
     z = golden.npz("config1_full")
     jobs = [("config1", torch.from_numpy(z["y_head"]), torch.from_numpy(z["p_head"]), torch.from_numpy(z["thresholds"]),
              2, z["mse_indices"][:256], z["qjl_signs"][:256])]
-    kc = golden.npz("key_cases")
-    for case in golden.cases("key_cases"):
+    for file, case in golden.key_case_list():
+        kc = golden.npz(file)
         d, bits, _ = [int(v) for v in kc[case + ".meta"]]
         y = torch.from_numpy(kc[case + ".y"]).reshape(-1, d)
         p = torch.from_numpy(kc[case + ".p"]).reshape(-1, d)
@@ -97,15 +97,15 @@ def _quantizer_for(prm, key_bits, gpu):
 
 
 def test_key_quantiser_end_to_end_vs_reference_vectors(gpu, golden):
-    kc = golden.npz("key_cases")
-    for case in golden.cases("key_cases"):
+    for file, case in golden.key_case_list():
+        kc = golden.npz(file)
         d, bits, _ = [int(v) for v in kc[case + ".meta"]]
         if bits - 1 > 4:
             continue
         _progress(f"quantize_keys {case}")
-        prm = golden.key_params("key_cases", case)
+        prm = golden.key_params(file, case)
         tq = _quantizer_for(prm, bits, gpu)
-        x = golden.tensor("key_cases", case + ".x")
+        x = golden.tensor(file, case + ".x")
         code, y, p = tq.quantize_traced(x.to(gpu))
         torch.cuda.synchronize()
         n_coord = x.numel()
@@ -119,7 +119,7 @@ def test_key_quantiser_end_to_end_vs_reference_vectors(gpu, golden):
         _progress(f"   index bytes differing {idx_flips}, sign bits differing {sgn_flips} of {n_coord}")
         assert idx_flips <= max(1, FLIP_RATE * n_coord), case
         assert sgn_flips <= max(2, FLIP_RATE * n_coord), case
-        ref_norm = golden.tensor("key_cases", case + ".norms").float()
+        ref_norm = golden.tensor(file, case + ".norms").float()
         got_norm = code.norms.float().cpu()
         ulp = 2.0 ** -7 if x.dtype == torch.bfloat16 else (2.0 ** -10 if x.dtype == torch.float16 else 2.0 ** -22)
         assert torch.all((got_norm - ref_norm).abs() <= ulp * ref_norm.abs() + 1e-30), case
@@ -160,22 +160,22 @@ def test_mse_only_quantiser_and_dequant(gpu, golden):
 
 def test_prod_dequant_and_score_on_reference_bytes(gpu, golden):
     from turboquant_amd.quantizer import ProdQuantized
-    kc = golden.npz("key_cases")
-    for case in golden.cases("key_cases"):
+    for file, case in golden.key_case_list():
+        kc = golden.npz(file)
         d, bits, _ = [int(v) for v in kc[case + ".meta"]]
         if bits - 1 > 4:
             continue
         _progress(f"dequant+score {case}")
-        prm = golden.key_params("key_cases", case)
+        prm = golden.key_params(file, case)
         tq = _quantizer_for(prm, bits, gpu)
         code = ProdQuantized(torch.from_numpy(kc[case + ".mse_indices"]).to(gpu),
                              torch.from_numpy(kc[case + ".qjl_signs"]).to(gpu),
                              torch.from_numpy(kc[case + ".residual_norms"]).to(gpu),
-                             golden.tensor("key_cases", case + ".norms").to(gpu), bits - 1)
+                             golden.tensor(file, case + ".norms").to(gpu), bits - 1)
         deq = tq.dequantize(code).cpu()
         want = torch.from_numpy(kc[case + ".dequant"])
         assert (deq - want).abs().max() <= 4e-6 * want.abs().max(), case
-        q = golden.tensor("key_cases", case + ".q").to(gpu)
+        q = golden.tensor(file, case + ".q").to(gpu)
         sc = tq.attention_score(q, code).cpu()
         ref = torch.from_numpy(kc[case + ".scores"])
         assert sc.shape == ref.shape and sc.dtype == torch.float32

@@ -1,0 +1,179 @@
+"""GPU: the scores the page-streaming kernels compute in flight, the long-context workload at its full
+size, and the wide-head (576) quantiser - each through the C ABI against the pinned oracle.
+
+The fused decode kernels never write a score; what they do write per (sequence, query head, split) is the
+partial (running maximum m, sum l of exp(score - m), accumulator).  m + log l is the log-sum-exp of the
+scores of the sequence's tokens, so a family of sequences that share one block table and have lengths
+1, 2, 3, ... gives every token's score as a difference of neighbouring sums."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import tq_oracle as O
+from tests.helpers import bit_mismatch, byte_mismatch, cosine, key_code, params_of, value_code
+from tests.test_gpu_parity import COS_GATE, FLIP_RATE, SCORE_TOL, _decode_case, _make_pool, _progress, _store_from_oracle_view
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("d,key_bits,vb,G,dtype", [(128, 3, 4, 8, torch.bfloat16), (128, 2, 2, 8, torch.bfloat16),
+                                                   (128, 4, 4, 8, torch.bfloat16), (256, 3, 2, 8, torch.bfloat16),
+                                                   (256, 4, 2, 8, torch.bfloat16), (256, 2, 4, 5, torch.float16),
+                                                   (128, 3, 2, 3, torch.float16), (64, 3, 2, 4, torch.bfloat16),
+                                                   (128, 5, 4, 8, torch.bfloat16)])
+def test_scores_inside_the_decode_kernels_meet_the_score_gate(gpu, d, key_bits, vb, G, dtype):
+    """sm_scale * TurboQuantProd.attention_score (quantizer.py:274-302) as the page kernels compute it
+    from the packed pages: matrix-core kernel (head_dim 128 / 256, up to 4-bit keys) and the general kernel
+    (head_dim 64, 5-bit keys).  Gate: |delta| <= 1e-3 * rms(scores) on the same stored bytes."""
+    Hkv, N = 2, 192
+    Hq = Hkv * G
+    pool, tq = _make_pool(gpu, d, key_bits, vb, Hkv, N // 16 + 2, dtype, seed=42 + 7 * key_bits)
+    g = torch.Generator().manual_seed(1000 + d + key_bits)
+    k = torch.randn(1, N, Hkv, d, generator=g).to(dtype)
+    k = k * (0.25 + 1.5 * torch.rand(1, N, Hkv, 1, generator=g)).to(dtype)       # norms that differ per token
+    v = torch.randn(1, N, Hkv, d, generator=g).to(dtype)
+    q0 = torch.randn(Hq, d, generator=g).to(dtype)
+    table = torch.randperm(N // 16 + 2, generator=g)[: N // 16].to(torch.int32).to(gpu)
+    pool.append(k.to(gpu), v.to(gpu), table[None, :])
+    # sequence b = the first b + 1 tokens of the same pages; scores with a spread of about 0.4, so that
+    # no token is a negligible share of a sum it has to be recovered from
+    sm_scale = 0.4 / math.sqrt(d)
+    B = N
+    q = q0[None].expand(B, Hq, d).contiguous().to(gpu)
+    seq = torch.arange(1, B + 1, dtype=torch.int32, device=gpu)
+    ws = pool.workspace(B, Hq, 1)
+    _progress(f"in-kernel scores d={d} kb={key_bits} vb={vb} G={G} {dtype}")
+    pool.decode_attention(q, table, seq, scale=sm_scale, n_split=1, workspace=ws, stages=3)
+    torch.cuda.synchronize()
+    parts = ws[: B * Hq * 2 * (d + 2)].view(B, Hq, 2, d + 2)[:, :, 0, :2].double().cpu()
+    lse = parts[..., 0] + parts[..., 1].log()                                       # (B, Hq)
+    rel = (lse - lse[-1:]).exp()                                                   # prefix sums / the total
+    w = torch.cat([rel[:1], rel[1:] - rel[:-1]], dim=0)                            # share of token t
+    assert torch.all(w > 0)
+    got = (w.log() + lse[-1:]).transpose(0, 1)                                     # (Hq, N) scaled scores
+    kc, _ = _store_from_oracle_view(pool, table, N)
+    want = sm_scale * O.attention_score(q0.view(Hkv, G, d), kc, params_of(tq)).double().reshape(Hq, N)
+    rms = want.pow(2).mean().sqrt()
+    err = (got - want).abs().max()
+    _progress(f"   max |delta| {err:.3e} = {err / rms:.2e} x rms(scores)")
+    assert err <= SCORE_TOL * rms
+
+
+def _student_t(shape, nu, gen):
+    """z / sqrt(chi2_nu / nu) element-wise, chi2 as the sum of nu squared normals."""
+    z = torch.randn(shape, generator=gen)
+    c = torch.zeros(shape)
+    for _ in range(nu):
+        c.add_(torch.randn(shape, generator=gen).square_())
+    return z.div_(c.div_(nu).sqrt_())
+
+
+def test_config4_full_size_decode_against_the_oracle(gpu):
+    """The long-context decode workload at its full size: 4 sequences x 131072 tokens, 16 query / 2 KV heads
+    of 256, 3-bit keys, 2-bit values in groups of 32, bf16 Student-t (nu = 5) keys and values from a CPU
+    generator seeded 3, physical pages a random permutation, default split count.  Every sequence against
+    the oracle's de-quantise-everything attention on the same store (score.py:84-173)."""
+    B, Hq, Hkv, d, N = 4, 16, 2, 256, 131072
+    pages = N // 16
+    pool, tq = _make_pool(gpu, d, 3, 2, Hkv, B * pages, torch.bfloat16, seed=42)
+    g = torch.Generator().manual_seed(3)
+    table = torch.randperm(B * pages, generator=g).to(torch.int32).view(B, pages).to(gpu)
+    for b in range(B):
+        _progress(f"config 4: sequence {b}: Student-t keys / values, quantise")
+        k = _student_t((1, N, Hkv, d), 5, g).bfloat16().to(gpu)
+        v = _student_t((1, N, Hkv, d), 5, g).bfloat16().to(gpu)
+        pool.append(k, v, table[b:b + 1])
+        del k, v
+    q = torch.randn(B, Hq, d, generator=g).bfloat16()
+    seq = torch.full((B,), N, dtype=torch.int32, device=gpu)
+    out = pool.decode_attention(q.to(gpu), table, seq, max_len=N).cpu()
+    torch.cuda.synchronize()
+    prm = params_of(tq)
+    for b in range(B):
+        kc, vc = _store_from_oracle_view(pool, table[b], N)
+        want = O.hybrid_attention(q[b:b + 1], kc, vc, N, prm, Hkv, None, None)
+        c = cosine(out[b:b + 1], want)
+        _progress(f"config 4: sequence {b} cosine {c:.8f}")
+        assert c >= COS_GATE, (b, c)
+        assert (out[b:b + 1].float() - want.float()).abs().max() <= 2 ** -7 * want.float().abs().max() + 1e-3, b
+
+
+@pytest.mark.parametrize("d,key_bits,dtype", [(576, 4, torch.bfloat16), (576, 3, torch.float32), (192, 4, torch.float16)])
+def test_wide_head_quantiser_against_the_oracle(gpu, d, key_bits, dtype):
+    """Head sizes without a matrix-core quantiser (the fp32 vector-ALU kernel): 576 with 4-bit keys is the shape
+    the reference ships a codebook for (codebook_d576_b3.json; integration/vllm.py:378-379 sizes a layer from
+    kv_lora_rank).  Bytes against the oracle on the same Pi / S (quantizer.py:231-257): a coordinate that
+    sits on a threshold may flip with the fp32 summation order, bounded at 1e-4 per coordinate; norms and
+    residual norms to rounding; all-zero vectors byte for byte."""
+    from turboquant_amd.quantizer import TurboQuantProd
+    tq = TurboQuantProd(d, bits=key_bits, device=gpu, seed=49)
+    prm = params_of(tq)
+    g = torch.Generator().manual_seed(d + key_bits)
+    n = 300
+    x = torch.randn(n, d, generator=g)
+    x[:, torch.randperm(d, generator=g)[:4]] *= 20.0
+    x[7] = 0.0
+    x[n - 1] = 0.0
+    x = x.to(dtype)
+    _progress(f"wide quantiser d={d} kb={key_bits} {dtype}")
+    code = tq.quantize(x.to(gpu))
+    torch.cuda.synchronize()
+    want = O.prod_quantize(x, prm)
+    n_coord = x.numel()
+    idx_flips = byte_mismatch(code.mse_indices, want.mse_indices)
+    sgn_flips = bit_mismatch(code.qjl_signs, want.qjl_signs)
+    _progress(f"   index bytes differing {idx_flips}, sign bits differing {sgn_flips} of {n_coord}")
+    assert idx_flips <= max(1, FLIP_RATE * n_coord) and sgn_flips <= max(2, FLIP_RATE * n_coord)
+    for row in (7, n - 1):
+        assert torch.equal(code.mse_indices[row].cpu(), want.mse_indices[row])
+        assert torch.equal(code.qjl_signs[row].cpu(), want.qjl_signs[row])
+    ulp = 2.0 ** -7 if dtype == torch.bfloat16 else (2.0 ** -10 if dtype == torch.float16 else 2.0 ** -22)
+    assert torch.all((code.norms.float().cpu() - want.norms.float()).abs() <= ulp * want.norms.float().abs() + 1e-30)
+    assert torch.allclose(code.residual_norms.cpu(), want.residual_norms, rtol=3e-5, atol=1e-6)
+    # the paged sink of the same kernel writes the same codes
+    pool, _ = _make_pool(gpu, d, key_bits, 2, 1, n // 16 + 2, dtype if dtype != torch.float32 else torch.float32, seed=49)
+    table = torch.arange(n // 16 + 1, dtype=torch.int32, device=gpu)[None, :]
+    pool.append(x.to(gpu)[None, :, None, :], x.to(gpu)[None, :, None, :], table)
+    idx, sgn, norms, rnorms, _, _, _ = pool.export_flat(table[0], n)
+    torch.cuda.synchronize()
+    assert torch.equal(idx[0], code.mse_indices) and torch.equal(sgn[0], code.qjl_signs)
+    assert torch.equal(norms[0], code.norms) and torch.equal(rnorms[0], code.residual_norms)
+
+
+@pytest.mark.parametrize("d,key_bits", [(128, 5), (576, 4)])
+def test_all_zero_vectors_land_in_the_reference_bucket(gpu, golden, d, key_bits):
+    """Two of the reference's tables (codebook_d128_b4.json, codebook_d576_b3.json) hold a tiny negative
+    middle threshold instead of 0, so a coordinate that is exactly 0 - every coordinate of an all-zero key,
+    e.g. a padding row - belongs to the bucket above the middle (searchsorted, quantizer.py:144).  Flat and
+    paged quantisers must pack exactly those bytes."""
+    from turboquant_amd.quantizer import TurboQuantProd
+    mb = key_bits - 1
+    ref_thr = torch.tensor(golden.codebook(d, mb)["boundaries"][1:-1], dtype=torch.float32)
+    assert ref_thr[len(ref_thr) // 2] < 0
+    for dtype in (torch.bfloat16, torch.float32):
+        tq = TurboQuantProd(d, bits=key_bits, device=gpu)
+        assert torch.equal(tq.mse_quantizer.decision_boundaries.cpu(), ref_thr)
+        x = torch.zeros(20, d, dtype=dtype)
+        code = tq.quantize(x.to(gpu))
+        want = O.prod_quantize(x, params_of(tq))
+        assert int(want.mse_indices[0, 0]) == (1 << (mb - 1)) * 0x11           # both nibbles: upper middle bucket
+        assert torch.equal(code.mse_indices.cpu(), want.mse_indices)
+        assert torch.equal(code.qjl_signs.cpu(), want.qjl_signs)
+        assert torch.count_nonzero(code.norms) == 0 and torch.count_nonzero(code.residual_norms) == 0
+        pool, _ = _make_pool(gpu, d, key_bits, 2, 1, 4, dtype)
+        table = torch.arange(2, dtype=torch.int32, device=gpu)[None, :]
+        pool.append(x.to(gpu)[None, :, None, :], x.to(gpu)[None, :, None, :], table)
+        idx, sgn, _, _, _, _, _ = pool.export_flat(table[0], 20)
+        assert torch.equal(idx[0].cpu(), want.mse_indices) and torch.equal(sgn[0].cpu(), want.qjl_signs)
+
+
+@pytest.mark.parametrize("vb,Hq,Hkv,dtype", [(2, 16, 1, torch.bfloat16), (4, 8, 2, torch.float16)])
+def test_decode_head_dim_576_with_4_bit_keys(gpu, vb, Hq, Hkv, dtype):
+    """head_dim 576 with 4-bit keys (3-bit indices in nibbles): the shape of the only 576 table the reference
+    ships, through the page kernel against the oracle on the same store."""
+    _progress(f"decode d=576 kb=4 vb={vb} Hq={Hq} Hkv={Hkv} {dtype}")
+    worst = _decode_case(gpu, 576, 4, vb, 2, Hq, Hkv, [300, 77], [0, 9], seed=900 + vb, dtype=dtype)
+    _progress(f"   worst cosine {worst:.7f}")

@@ -126,11 +126,38 @@ def test_shipped_codebooks_equal_reference_files(golden):
         # the fp32 tensors handed to the kernels are identical
         c, e = get_codebook_tensors(d, b, "cpu")
         assert torch.equal(c, torch.tensor(ref["centroids"], dtype=torch.float32))
-        # the middle boundary is 0 by symmetry; two of the reference's files hold -4e-17 / -3e-18 there
-        # (rounding noise of the machine that wrote them), everything else is identical in fp32
-        ref_e = torch.tensor(ref["boundaries"], dtype=torch.float32)
-        differs = (e != ref_e)
-        assert int(differs.sum()) <= 1 and torch.all(ref_e[differs].abs() < 1e-15) and torch.all(e[differs] == 0)
+        # ... and so are the thresholds, the middle one included: two of the reference's tables hold
+        # -4e-17 / -3e-18 there instead of 0, which decides the bucket of a coordinate that is exactly 0
+        # (every coordinate of an all-zero vector), so the shipped tables carry the published values
+        assert torch.equal(e, torch.tensor(ref["boundaries"], dtype=torch.float32)), (d, b)
+
+
+def test_rotation_and_sketch_matrices_equal_the_reference_ones(golden):
+    """generate_rotation_matrix / generate_qjl_matrix (rotation.py:17-56) against the matrices the
+    reference produced for config 1 (seed 42, sketch seed 42 + 1000) and for the other golden cases.
+    torch.randn from a seeded CPU generator is bit-stable, so S must match bit for bit; Pi goes
+    through LAPACK's QR, whose summation order depends on the BLAS thread count (differences of 1e-6
+    between 1 and 8 threads were observed), hence 2e-6."""
+    from turboquant_amd.rotation import generate_qjl_matrix, generate_rotation_matrix
+    z = golden.npz("config1_full")
+    S = generate_qjl_matrix(128, "cpu", seed=42 + 1000)
+    assert S.dtype == torch.float32 and torch.equal(S, torch.from_numpy(z["S"]))
+    Pi = generate_rotation_matrix(128, "cpu", seed=42)
+    ref = torch.from_numpy(z["Pi"])
+    assert Pi.shape == ref.shape and (Pi - ref).abs().max() <= 2e-6
+    assert (Pi @ Pi.T - torch.eye(128)).abs().max() < 1e-5
+    # a wrong sign convention, a transposed factor or a different seed rule would be off by O(1)
+    assert (Pi.T - ref).abs().max() > 0.1
+    for file, case in golden.key_case_list():
+        kc = golden.npz(file)
+        d, bits, seed = [int(v) for v in kc[case + ".meta"]]
+        if golden.has(file, case + ".S"):
+            assert torch.equal(generate_qjl_matrix(d, "cpu", seed=seed + 1000), torch.from_numpy(kc[case + ".S"])), case
+        assert (generate_rotation_matrix(d, "cpu", seed=seed) - torch.from_numpy(kc[case + ".Pi"])).abs().max() <= 2e-6, case
+    # the quantiser objects draw their matrices through the same two functions, seeds as quantizer.py:107,208
+    tq = TurboQuantProd(128, bits=3, device="cpu", seed=42)
+    assert torch.equal(tq.S, torch.from_numpy(z["S"]))
+    assert (tq.mse_quantizer.Pi - ref).abs().max() <= 2e-6
 
 
 def test_codebook_solver_known_answer(golden):

@@ -118,16 +118,16 @@ def test_rotation_is_orthogonal_with_positive_r_diagonal(d, seed):
 
 # ---------------------------------------------------------------- key quantiser vs reference vectors
 def test_key_cases_match_reference(golden):
-    for case in golden.cases("key_cases"):
-        prm = golden.key_params("key_cases", case)
-        x = golden.tensor("key_cases", case + ".x")
-        q = golden.tensor("key_cases", case + ".q")
+    for file, case in golden.key_case_list():
+        prm = golden.key_params(file, case)
+        x = golden.tensor(file, case + ".x")
+        q = golden.tensor(file, case + ".q")
         code = O.prod_quantize(x, prm)
-        z = golden.npz("key_cases")
+        z = golden.npz(file)
         assert np.array_equal(code.mse_indices.numpy(), z[case + ".mse_indices"]), case
         assert np.array_equal(code.qjl_signs.numpy(), z[case + ".qjl_signs"]), case
         assert code.norms.dtype == x.dtype
-        assert torch.equal(code.norms, golden.tensor("key_cases", case + ".norms")), case
+        assert torch.equal(code.norms, golden.tensor(file, case + ".norms")), case
         assert np.array_equal(code.residual_norms.numpy(), z[case + ".residual_norms"]), case
         assert np.array_equal(code.y.numpy(), z[case + ".y"], equal_nan=True), case
         assert np.array_equal(code.p.numpy(), z[case + ".p"], equal_nan=True), case
