@@ -11,9 +11,14 @@
  *   - `stream` is a hipStream_t passed as void* (NULL = the null stream);
  *   - `dtype` tags the element type of floating inputs: TQ_F32 / TQ_F16 / TQ_BF16;
  *   - the caller allocates every output and the decode workspace; no entry
- *     point allocates, frees or synchronises;
- *   - the library keeps no mutable global state: calls on different streams
- *     may overlap;
+ *     point allocates device memory, frees or synchronises;
+ *   - calls on different streams may overlap.  The only state the library keeps is per
+ *     host thread and per device: a side stream with two events that tq_append_kv_paged and
+ *     its siblings create on first use for large appends, the per-kernel launch attributes
+ *     set on first use, and the pair of events armed by tq_time_next_page_kernel;
+ *   - block tables are device data the host cannot inspect, so the kernels bound them:
+ *     a logical page beyond the table row, or a table entry outside [0, num_pages), is
+ *     never written through (append) and contributes no token (decode); see each entry;
  *   - return value: 0 on success, a negative TQ_E* code for a rejected argument
  *     (nothing was launched), or a positive hipError_t from the launch.
  */
@@ -166,6 +171,9 @@ int tq_rotate_query(const void *q, int dtype, int64_t rows, const tq_layer *laye
  * elements), innermost dimension contiguous.  Token t of sequence b goes to
  * logical position start_pos[b] + t, i.e. page block_table[b*max_pages + pos/16],
  * slot pos%16.  start_pos may be NULL (all zero).  pool is (num_pages, H, page_bytes).
+ * Tokens whose logical page lies beyond the table row (pos/16 >= max_pages) or whose table entry is not
+ * in [0, num_pages) are dropped: nothing outside the pool is written.  Without start_pos the run length is
+ * known on the host and T > 16*max_pages is TQ_EINVAL.
  * Large appends run their value kernel on a side stream of the calling thread (created on
  * first use, default priority) that is forked from and joined back into `stream` with
  * events: the call is ordered on `stream` like any other and stays capturable.           */
@@ -201,7 +209,8 @@ int tq_append_kv_from_blocks(const void *k_cache, const void *v_cache, int dtype
 /* Gather a sequence's pages back into the reference's flat tensors
  * (store.py:92-114 get_flat_cache): idx (H, n_tok, d*eff/8), signs (H, n_tok, d/8),
  * norms (H, n_tok) input dtype, rnorms fp32, v_data (H, n_tok, d*vb/8),
- * v_scales / v_zeros (H, n_tok, d/group).  block_table is this sequence's row.    */
+ * v_scales / v_zeros (H, n_tok, d/group).  block_table is this sequence's row
+ * (at least ceil(n_tok/16) entries); an entry outside [0, num_pages) is read as page 0. */
 int tq_pool_export(const uint8_t *pool, int64_t num_pages, int H, const int32_t *block_table, int n_tok,
                    const tq_page_layout *layout, uint8_t *idx, uint8_t *signs, void *norms, float *rnorms,
                    uint8_t *v_data, void *v_scales, void *v_zeros, void *stream);
@@ -214,8 +223,10 @@ size_t tq_decode_workspace_bytes(int B, int Hq, int d, int n_split);
  * triton_kernels.py:209-356 with GQA sharing, paging and split-K added).
  * q (B, Hq, d) `dtype` contiguous (it need not be the pages' dtype); query head h
  * reads KV head h / (Hq/Hkv).
- * seq_lens[b] compressed tokens of sequence b sit in block_table[b*bt_stride + i]
- * (bt_stride = 0 shares one table among all b).  recent_k / recent_v (nullable)
+ * seq_lens[b] compressed tokens of sequence b sit in block_table[b*bt_stride + i]:
+ * bt_stride > 0 is a row of that many entries per sequence; bt_stride < 0 one row of -bt_stride entries
+ * shared by all sequences; 0 one shared row of unchecked length.  A length beyond the row is cut to
+ * 16 entries per row entry, and the tokens of a page whose entry is not in [0, num_pages) get no weight.  recent_k / recent_v (nullable)
  * hold exact tokens (b, r, h, :) `dtype`, element strides rs_b, rs_r, rs_h, with
  * recent_len[b] valid rows (NULL = recent_rows for all).  out (B, Hq, d) `dtype`:
  * softmax(sm_scale * [scores_hist ; q k_recent^T]) [v_hist ; v_recent]; all-empty

@@ -177,3 +177,105 @@ def test_decode_head_dim_576_with_4_bit_keys(gpu, vb, Hq, Hkv, dtype):
     _progress(f"decode d=576 kb=4 vb={vb} Hq={Hq} Hkv={Hkv} {dtype}")
     worst = _decode_case(gpu, 576, 4, vb, 2, Hq, Hkv, [300, 77], [0, 9], seed=900 + vb, dtype=dtype)
     _progress(f"   worst cosine {worst:.7f}")
+
+
+# ------------------------------------------------------------------ block tables are bounded on the device
+@pytest.mark.parametrize("d,key_bits,vb,dtype,T", [(128, 3, 4, torch.bfloat16, 70), (256, 3, 2, torch.bfloat16, 5000),
+                                                     (64, 2, 2, torch.float16, 70), (128, 3, 2, torch.float32, 40),
+                                                     (128, 3, 4, torch.bfloat16, 8192)])
+def test_append_never_writes_through_a_bad_table_entry(gpu, d, key_bits, vb, dtype, T):
+    """A block table is device data the host cannot check.  Entries outside [0, num_pages) (stale, poisoned or
+    negative) and runs that continue past the end of the table row must leave every byte of the pool as it
+    was and return normally; the tokens of the good pages are written as usual.  (Small and large appends:
+    the tile kernels, the chunk kernels, the matrix-core key kernel and the side-stream path.)"""
+    H = 8 if T >= 8192 else 2                      # 8192 tokens x 8 heads: large enough for the side-stream path
+    n_log = (T + 15) // 16
+    n_pages = n_log + 3
+    g = torch.Generator().manual_seed(T + d)
+    k = torch.randn(1, T, H, d, generator=g).to(dtype).to(gpu)
+    v = torch.randn(1, T, H, d, generator=g).to(dtype).to(gpu)
+    good = torch.randperm(n_pages, generator=g)[:n_log].to(torch.int32)
+    ref, _ = _make_pool(gpu, d, key_bits, vb, H, n_pages, dtype)
+    ref.data.fill_(0xA5)                           # (padding bytes of a page are never written)
+    ref.append(k, v, good[None].to(gpu))
+    _progress(f"append with bad table entries d={d} {dtype} T={T}")
+    bad_slots = sorted({0, n_log // 2, n_log - 1})
+    for poison in (n_pages, 2 ** 31 - 1, -1, -2 ** 31):
+        table = good.clone()
+        table[bad_slots] = poison
+        pool, _ = _make_pool(gpu, d, key_bits, vb, H, n_pages, dtype)
+        pool.data.fill_(0xA5)
+        refp = ref.data.clone()
+        pool.append(k, v, table[None].to(gpu))
+        torch.cuda.synchronize()
+        touched = torch.zeros(n_pages, dtype=torch.bool)
+        ok_slots = [i for i in range(n_log) if i not in bad_slots]
+        touched[good[ok_slots].long()] = True
+        assert torch.all(pool.data[~touched] == 0xA5), poison                       # nothing else was written
+        # full pages written through good entries equal the reference pool's (the last page may be partial)
+        full = [i for i in ok_slots if (i + 1) * 16 <= T]
+        assert torch.equal(pool.data[good[full].long()], refp[good[full].long()]), poison
+    # a run that starts near the end of the table row and continues past it: the overflow is dropped
+    pool, _ = _make_pool(gpu, d, key_bits, vb, H, n_pages, dtype)
+    pool.data.fill_(0x5A)
+    short = good[:2].clone()
+    start = torch.tensor([20], dtype=torch.int32, device=gpu)
+    pool.append(k, v, short[None].to(gpu), start)                                   # positions 20 .. 20 + T - 1, row of 2
+    torch.cuda.synchronize()
+    touched = torch.zeros(n_pages, dtype=torch.bool)
+    touched[short.long()] = True
+    assert torch.all(pool.data[~touched] == 0x5A)
+    # without start positions the host knows the run and refuses it
+    if T > 32:
+        with pytest.raises((ValueError, RuntimeError)):
+            pool.append(k, v, short[None].to(gpu))
+
+
+@pytest.mark.parametrize("d,key_bits,vb,Hq,Hkv,dtype", [(128, 3, 4, 8, 2, torch.bfloat16), (256, 3, 2, 16, 2, torch.bfloat16),
+                                                         (64, 3, 2, 4, 1, torch.bfloat16), (128, 3, 2, 4, 2, torch.float32)])
+def test_decode_gives_no_weight_to_pages_outside_the_pool(gpu, d, key_bits, vb, Hq, Hkv, dtype):
+    """Decode with table entries outside [0, num_pages): those pages' tokens get no weight, so the result is
+    the attention over the remaining tokens - checked against the oracle on exactly those tokens
+    (score.py:84-173) - and sequence lengths beyond the table row are cut to the row."""
+    N, B = 390, 2
+    n_log = (N + 15) // 16
+    n_pages = B * n_log + 2
+    pool, tq = _make_pool(gpu, d, key_bits, vb, Hkv, n_pages, dtype, seed=42)
+    g = torch.Generator().manual_seed(31 * d + vb)
+    k = torch.randn(B, N, Hkv, d, generator=g).to(dtype)
+    v = torch.randn(B, N, Hkv, d, generator=g).to(dtype)
+    q = torch.randn(B, Hq, d, generator=g).to(dtype)
+    table = torch.randperm(n_pages, generator=g)[: B * n_log].to(torch.int32).view(B, n_log)
+    pool.append(k.to(gpu), v.to(gpu), table.to(gpu))
+    prm = params_of(tq)
+    _progress(f"decode with bad table entries d={d} kb={key_bits} vb={vb} {dtype}")
+    # sequence 0 loses its whole first 64-token block, a page in the middle and its last (partial) page;
+    # sequence 1 loses one page
+    lost = {0: [0, 1, 2, 3, 9, n_log - 1], 1: [5]}
+    bad = table.clone()
+    for b, slots in lost.items():
+        bad[b, slots] = torch.tensor([n_pages, -1, 2 ** 31 - 1, -7, n_pages + 5, 2 ** 30][: len(slots)], dtype=torch.int32)
+    seq = torch.tensor([N, N], dtype=torch.int32, device=gpu)
+    for n_split in (1, 3, None):
+        out = pool.decode_attention(q.to(gpu), bad.to(gpu), seq, n_split=n_split, max_len=N).cpu()
+        torch.cuda.synchronize()
+        for b in range(B):
+            keep = [i for i in range(n_log) if i not in lost[b]]
+            tok = torch.cat([torch.arange(16 * i, min(16 * i + 16, N)) for i in keep])
+            idx, sgn, norms, rn, vd, vs, vz = [t.cpu()[:, tok] for t in pool.export_flat(table[b], N)]
+            want = O.hybrid_attention(q[b:b + 1], key_code(idx, sgn, rn, norms, key_bits - 1), value_code(vd, vs, vz, vb),
+                                      len(tok), prm, Hkv, None, None)
+            c = cosine(out[b:b + 1], want)
+            assert c >= COS_GATE, (n_split, b, c)
+    # a sequence length beyond the table row is cut to the row: same result as the full row
+    over = pool.decode_attention(q.to(gpu), table.to(gpu), torch.tensor([N + 4000, 10 ** 9], dtype=torch.int32, device=gpu),
+                                 n_split=2, max_len=N)
+    row_full = pool.decode_attention(q.to(gpu), table.to(gpu), torch.tensor([n_log * 16] * 2, dtype=torch.int32, device=gpu),
+                                     n_split=2, max_len=N)
+    torch.cuda.synchronize()
+    assert torch.equal(over, row_full)
+    # every table entry bad: nothing to attend to, zeros
+    allbad = torch.full_like(table, -1)
+    z = pool.decode_attention(q.to(gpu), allbad.to(gpu), seq, n_split=2, max_len=N)
+    torch.cuda.synchronize()
+    assert torch.count_nonzero(z) == 0

@@ -27,19 +27,41 @@ FLAGS = [
 ]
 
 
-def build_library(verbose: bool = False) -> str:
-    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc] + FLAGS + [os.path.join(CSRC, s) for s in SOURCES] + ["-o", LIB]
-    if verbose:
-        print(" ".join(cmd))
+def _run(cmd):
     res = subprocess.run(cmd, capture_output=True, text=True)
     # the host pass warns that it does not know the packed-fp32 feature; that is harmless
-    noise = "packed-fp32-ops"
-    err = "\n".join(l for l in res.stderr.splitlines() if noise not in l)
-    if res.returncode != 0:
-        raise RuntimeError(f"hipcc failed ({res.returncode}):\n{err}")
-    if verbose and err.strip():
-        print(err, file=sys.stderr)
+    err = "\n".join(l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l)
+    return res.returncode, err
+
+
+def build_library(verbose: bool = False) -> str:
+    """Compile every source to an object file (in parallel: the files are independent translation units)
+    and link them into libtq_hip.so."""
+    from concurrent.futures import ThreadPoolExecutor
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    objdir = os.path.join(HERE, "build")
+    os.makedirs(objdir, exist_ok=True)
+    compile_flags = [f for f in FLAGS if f != "-shared"]
+    jobs = []
+    for src in SOURCES:
+        obj = os.path.join(objdir, src.replace(".hip", ".o"))
+        jobs.append((obj, [hipcc] + compile_flags + ["-c", os.path.join(CSRC, src), "-o", obj]))
+    if verbose:
+        for _, cmd in jobs:
+            print(" ".join(cmd))
+    with ThreadPoolExecutor(max_workers=min(len(jobs), os.cpu_count() or 1)) as pool:
+        results = list(pool.map(lambda j: _run(j[1]), jobs))
+    for (obj, _), (rc, err) in zip(jobs, results):
+        if rc != 0:
+            raise RuntimeError(f"hipcc failed ({rc}) for {obj}:\n{err}")
+        if verbose and err.strip():
+            print(err, file=sys.stderr)
+    link = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc"] + [obj for obj, _ in jobs] + ["-o", LIB]
+    if verbose:
+        print(" ".join(link))
+    rc, err = _run(link)
+    if rc != 0:
+        raise RuntimeError(f"hipcc link failed ({rc}):\n{err}")
     return LIB
 
 

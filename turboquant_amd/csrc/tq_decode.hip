@@ -57,7 +57,7 @@ __global__ void __launch_bounds__(GEN_THREADS)
 decode_pages_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_sk, int Hq, int Hkv,
                     const uint8_t* __restrict__ pool, const int32_t* __restrict__ block_table, int bt_stride,
                     const int32_t* __restrict__ seq_lens, float sm_scale, tq_layer ly, tq_page_layout L,
-                    float* __restrict__ parts, int n_parts, int n_split, int len_sub) {
+                    float* __restrict__ parts, int n_parts, int n_split, int len_sub, int max_pages, int num_pages) {
   constexpr int GP = 4 * GP4;
   const int d = ly.d, mb = ly.mse_bits, G = Hq / Hkv, words = d >> 5;
   const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
@@ -81,7 +81,8 @@ decode_pages_kernel(const float* __restrict__ q_rot, const float* __restrict__ q
   if (tid < 16) s_cent[tid] = tid < (1 << mb) ? ly.centroids[tid] : 0.0f;
   __syncthreads();
 
-  const int seq_len = max(seq_lens[b] - len_sub, 0);      // len_sub: newest tokens that are attended to exactly
+  // len_sub: newest tokens that are attended to exactly.  A length beyond the block table is cut to the table.
+  const int seq_len = max(min(seq_lens[b], max_pages * TQ_PAGE_TOKENS) - len_sub, 0);
   const int n_pages = (seq_len + TQ_PAGE_TOKENS - 1) / TQ_PAGE_TOKENS;
   const int per_split = (n_pages + n_split - 1) / n_split;
   const int pg_begin = split * per_split;
@@ -111,8 +112,11 @@ decode_pages_kernel(const float* __restrict__ q_rot, const float* __restrict__ q
     // ---- scores: thread = token pc * 16 + tid
     {
       const int pi = pc + (tid >> 4), n = tid & 15;
-      const bool valid = pi < pg_end && pi * TQ_PAGE_TOKENS + n < seq_len;
-      const uint8_t* pg = pool + (int64_t)bt[valid ? pi : pg_begin] * page_stride + head_off;
+      // a table entry outside the pool (stale or poisoned) is read as page 0 and its tokens get no weight
+      const int raw = bt[pi < pg_end ? pi : pg_begin];
+      const bool in_pool = (unsigned)raw < (unsigned)num_pages;
+      const bool valid = pi < pg_end && pi * TQ_PAGE_TOKENS + n < seq_len && in_pool;
+      const uint8_t* pg = pool + (int64_t)(in_pool ? raw : 0) * page_stride + head_off;
       float pm[GP], pq[GP];
 #pragma unroll
       for (int g = 0; g < GP; ++g) pm[g] = pq[g] = 0.0f;
@@ -170,7 +174,8 @@ decode_pages_kernel(const float* __restrict__ q_rot, const float* __restrict__ q
         for (int k = 0; k < MAXCH; ++k) acc[k][g] *= alpha[g];
       }
       const int pi = pc + (tid >> 4), n = tid & 15;
-      const bool valid = pi < pg_end && pi * TQ_PAGE_TOKENS + n < seq_len;
+      const bool valid = pi < pg_end && pi * TQ_PAGE_TOKENS + n < seq_len &&
+                         (unsigned)bt[pi < pg_end ? pi : pg_begin] < (unsigned)num_pages;
 #pragma unroll
       for (int g = 0; g < GP; ++g) {
         const float sc = s_p[tid * GP + g];
@@ -184,6 +189,7 @@ decode_pages_kernel(const float* __restrict__ q_rot, const float* __restrict__ q
       for (int t0 = t_begin; t0 < t_end; t0 += TQ_PAGE_TOKENS) {
         const int pi = pc + (t0 >> 4);
         if (pi >= pg_end) break;
+        if ((unsigned)bt[pi] >= (unsigned)num_pages) continue;        // its tokens have weight 0
         const uint8_t* pg = pool + (int64_t)bt[pi] * page_stride + head_off;
         const int n_valid = min(TQ_PAGE_TOKENS, seq_len - pi * TQ_PAGE_TOKENS);
 #pragma unroll
@@ -463,6 +469,7 @@ struct TailArgs {
   const int32_t* recent_len;
   const int32_t* block_table;
   int bt_stride;
+  int max_pages, num_blocks;       // entries of a block-table row; blocks of the paged exact cache
   const int32_t* seq_lens;
   int64_t ws_blk;
   float sm_scale;
@@ -489,7 +496,8 @@ __device__ __forceinline__ void exact_tail_words_body(const TailArgs& A, int h, 
   const int G = Hq / Hkv, g0 = gz * GC, tid = threadIdx.x;
   const int Gc = min(GC, G - g0);
   const int lane = tid & 63, wave = tid >> 6;
-  const int seq = PAGED ? seq_lens[b] : 0;
+  const int seq = PAGED ? min(seq_lens[b], A.max_pages * TQ_PAGE_TOKENS) : 0;     // cut to the block table
+  const int num_blocks = A.num_blocks;
   const int R = PAGED ? max(min(seq, recent_rows), 0) : (recent_len ? min(recent_len[b], recent_rows) : recent_rows);
   const int first = PAGED ? seq - R : 0;            // position of the first exact token
   const int32_t* bt = block_table + (PAGED ? (int64_t)b * bt_stride : 0);
@@ -508,7 +516,8 @@ __device__ __forceinline__ void exact_tail_words_body(const TailArgs& A, int h, 
   auto row_base = [&](int row) -> int64_t {
     if (PAGED) {
       const int p = first + row;
-      return base0 + (int64_t)bt[p >> 4] * ws_blk + (int64_t)(p & 15) * ws_r;
+      const int raw = bt[p >> 4];                       // an entry outside the cache is read as block 0
+      return base0 + (int64_t)((unsigned)raw < (unsigned)num_blocks ? raw : 0) * ws_blk + (int64_t)(p & 15) * ws_r;
     }
     return base0 + (int64_t)row * ws_r;
   };
@@ -800,7 +809,7 @@ size_t decode_mfma_pack_words(int B, int Hkv, int d);
 int launch_decode_mfma(const uint32_t* qa_pack, const float* q_stat, int B, int Hq, int Hkv, int kv_div,
                        const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
                        float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts,
-                       int n_split, int len_sub, hipStream_t st);
+                       int n_split, int len_sub, int max_pages, int num_pages, hipStream_t st);
 }  // namespace tq
 
 static size_t parts_floats(int B, int Hq, int d, int n_parts) { return (size_t)B * Hq * n_parts * (d + 2); }
@@ -861,8 +870,15 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   const int64_t rs_b = ts.s_b, rs_r = ts.s_r, rs_h = ts.s_h;
   const int32_t* recent_len = ts.len;
   if (!q || !pool || !block_table || !seq_lens || !layer || !layout || !out || !workspace) return TQ_ENULL;
-  if (B <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || n_split <= 0 || num_pages <= 0 || bt_stride < 0) return TQ_EINVAL;
+  if (B <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || n_split <= 0 || num_pages <= 0) return TQ_EINVAL;
   if (B > 65535 || Hkv > 65535) return TQ_EUNSUPPORTED;
+  // bt_stride > 0: a table row per sequence, that many entries; 0: one row shared by all sequences, length
+  // unknown; < 0: one shared row of -bt_stride entries.  Lengths beyond the row are cut to it in the kernels.
+  const int k_max_rows = 0x7fffffff / TQ_PAGE_TOKENS;
+  const int max_pages = bt_stride == 0 ? k_max_rows : (bt_stride > 0 ? bt_stride : -bt_stride) < k_max_rows
+                                                          ? (bt_stride > 0 ? bt_stride : -bt_stride) : k_max_rows;
+  if (bt_stride < 0) bt_stride = 0;
+  const int pool_pages = (int)(num_pages < 0x7fffffff ? num_pages : 0x7fffffff);
   const int d = layer->d, G = Hq / Hkv;
   if (d != layout->d || layer->mse_bits != layout->mse_bits) return TQ_EINVAL;
   if (d < 64 || d > 768 || (d & 63) || G > G_MAX) return TQ_EUNSUPPORTED;
@@ -899,6 +915,7 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   ta.rk = (const uint32_t*)recent_k; ta.rv = (const uint32_t*)recent_v; ta.recent_rows = recent_rows;
   ta.ws_b = rs_b / epw; ta.ws_r = rs_r / epw; ta.ws_h = rs_h / epw; ta.recent_len = recent_len;
   ta.block_table = block_table; ta.bt_stride = bt_stride; ta.seq_lens = seq_lens; ta.ws_blk = ts.s_blk / epw;
+  ta.max_pages = max_pages; ta.num_blocks = pool_pages;       // the exact cache shares the pool's block numbers
   ta.sm_scale = sm_scale; ta.parts = parts; ta.n_parts = n_parts; ta.part_index = n_split;
   const int n_tail = Hkv * B * ((G + TAIL_GC - 1) / TAIL_GC);
   bool tail_done = false;
@@ -949,7 +966,8 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   int mf = TQ_EUNSUPPORTED;
   if (stages & 2)
     mf = mfma_shape ? launch_decode_mfma(qa_pack, q_stat, B, Hq, Hkv * kv_div, kv_div, pool, block_table, bt_stride,
-                                         seq_lens, sm_scale, *layer, *layout, parts, n_parts, n_split, len_sub, st)
+                                         seq_lens, sm_scale, *layer, *layout, parts, n_parts, n_split, len_sub,
+                                         max_pages, pool_pages, st)
                     : TQ_EUNSUPPORTED;
   if (mf > 0) return mf;
   if ((stages & 2) && mf == TQ_EUNSUPPORTED) {      // no matrix-core kernel for this shape: general kernel
@@ -967,7 +985,7 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
       if (e != hipSuccess) return (int)e;                                                                 \
     }                                                                                                     \
     kern<<<grid, block, smem, st>>>(q_rot, q_sk, Hq, Hkv, pool, block_table, bt_stride, seq_lens, sm_scale, *layer,  \
-                                    *layout, parts, n_parts, n_split, len_sub);                           \
+                                    *layout, parts, n_parts, n_split, len_sub, max_pages, pool_pages);     \
   }
 #define TQ_LAUNCH_DEC_G(VB)                                                      \
   {                                                                              \

@@ -165,7 +165,7 @@ __global__ void __launch_bounds__(MF_WAVES * 64, WPS)
 decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict__ q_stat, int Hq, int Hkv, int kv_div,
                    const uint8_t* __restrict__ pool, const int32_t* __restrict__ block_table,
                    int bt_stride, const int32_t* __restrict__ seq_lens, float sm_scale, tq_layer ly, tq_page_layout L,
-                   float* __restrict__ parts, int n_parts, int n_split, int len_sub) {
+                   float* __restrict__ parts, int n_parts, int n_split, int len_sub, int max_pages, int num_pages) {
   constexpr int DW = D / DS;                  // coordinates / channels of one wavefront
   constexpr int WPLT = D / 128;               // plane words per lane per plane per page, all wavefronts
   constexpr int WPL = DW / 128;               // ... of one wavefront
@@ -253,7 +253,8 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
   }
 
   // ---------------------------------------------------------------- work range (all scalar)
-  const int seq_len = max(seq_lens[b] - len_sub, 0);      // len_sub: newest tokens that are attended to exactly
+  // len_sub: newest tokens that are attended to exactly.  A length beyond the block table is cut to the table.
+  const int seq_len = max(min(seq_lens[b], max_pages * TQ_PAGE_TOKENS) - len_sub, 0);
   const int n_pages = (seq_len + TQ_PAGE_TOKENS - 1) / TQ_PAGE_TOKENS;
   const int n_blocks = (seq_len + BLK_TOK - 1) / BLK_TOK;
   const int per_split = (n_blocks + n_split - 1) / n_split;
@@ -282,10 +283,20 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
   struct ValRegs { uint32_t v[VW]; u32x4 zero[2]; u32x4 scale; };
 
   // page ids of block `blk` -> 4 scalars; a page past the end of the sequence (last block only) is
-  // replaced by the block's first page, which always exists
-  auto page_ids = [&](int blk, int (&pid)[4]) {
+  // replaced by the block's first page, which always exists.  CHECK: a table entry outside the pool (a
+  // stale or poisoned entry) is replaced by page 0 and reported in the returned mask (bit pg); the block
+  // then takes the masking path, where those tokens get no weight.
+  auto page_ids = [&](int blk, int (&pid)[4], auto check_tag) -> int {
+    constexpr bool CHECK = decltype(check_tag)::value;
+    int bad = 0;
 #pragma unroll
-    for (int pg = 0; pg < 4; ++pg) pid[pg] = bt[min(4 * blk + pg, n_pages - 1)];
+    for (int pg = 0; pg < 4; ++pg) {
+      const int raw = bt[min(4 * blk + pg, n_pages - 1)];
+      const bool ok = !CHECK || (unsigned)raw < (unsigned)num_pages;
+      pid[pg] = ok ? raw : 0;
+      bad |= ok ? 0 : 1 << pg;
+    }
+    return bad;
   };
   auto load_keys = [&](const int (&pid)[4], KeyRegs& R) {
     // the 32-bit lane offsets are re-materialised here, next to their use, so that the loads take
@@ -333,10 +344,14 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
 
   // ---------------------------------------------------------------- one block of 64 tokens
   // scores of the 4 pages of block blk, online softmax, weights -> LDS
-  auto score_stage = [&](int blk, int it, const KeyRegs& K, auto partial_tag) -> bool {
+  // PARTIAL: some tokens of the block do not exist (the ragged end of the sequence, pages named in `bad`)
+  auto tokens_of_page = [&](int blk, int pg, int bad) -> int {          // existing tokens of page pg: a prefix
+    return ((bad >> pg) & 1) ? 0 : min(max(seq_len - (blk * BLK_TOK + pg * 16), 0), 16);
+  };
+  bool fresh = true;                            // this walker has not seen a token yet: no reference
+  auto score_stage = [&](int blk, int it, bool first, const KeyRegs& K, int bad, auto partial_tag) -> bool {
     constexpr bool PARTIAL = decltype(partial_tag)::value;
     float s2[2][4];
-    const bool first = it == 0;                 // first block of this walker: no reference yet
     float mref[2];                              // only one wavefront of a pair subtracts it
 #pragma unroll
     for (int j = 0; j < 2; ++j) mref[j] = (first || hf != 0) ? 0.0f : m_run[j];
@@ -401,12 +416,19 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
 #pragma unroll
         for (int pg = 0; pg < 4; ++pg) s2[j][pg] += theirs[(j * 4 + pg) * 64 + lane];
     }
+    bool gone[4] = {false, false, false, false};
     if (PARTIAL) {
+      bool any = false;
 #pragma unroll
-      for (int pg = 0; pg < 4; ++pg)
+      for (int pg = 0; pg < 4; ++pg) {
+        gone[pg] = n >= tokens_of_page(blk, pg, bad);
+        any |= !gone[pg];
 #pragma unroll
         for (int j = 0; j < 2; ++j)
-          if (blk * BLK_TOK + pg * 16 + n >= seq_len) s2[j][pg] = MF_NEG;
+          if (gone[pg]) s2[j][pg] = MF_NEG;
+      }
+      // a block without a single token leaves the walker as it was (the next block is still its first)
+      fresh = fresh && __builtin_amdgcn_ballot_w64(any) == 0;
     }
     // ---- online softmax (log2 domain) against a lazily updated reference
     float mx = fmaxf(fmaxf(fmaxf(s2[0][0], s2[0][1]), fmaxf(s2[0][2], s2[0][3])),
@@ -434,7 +456,9 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
       float psum = 0.0f;
 #pragma unroll
       for (int pg = 0; pg < 4; ++pg) {
-        const float p = __builtin_amdgcn_exp2f(s2[j][pg]);
+        // (a token that does not exist has weight 0 even when the whole block is empty and the
+        // reference therefore sits at the masking value itself)
+        const float p = PARTIAL && gone[pg] ? 0.0f : __builtin_amdgcn_exp2f(s2[j][pg]);
         psum += p;
         s_p[(pg * 16 + 2 * kb + j) * P_STRIDE + n] = p;
       }
@@ -443,7 +467,7 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
     return rescale;
   };
   // weights x (codes, scales, zeros) of block blk into the accumulators
-  auto value_stage = [&](int blk, const ValRegs& V, bool rescale, auto partial_tag) {
+  auto value_stage = [&](int blk, const ValRegs& V, bool rescale, int bad, auto partial_tag) {
     constexpr bool PARTIAL = decltype(partial_tag)::value;
     // scales -> LDS as fp32 [page][group][16 tokens]; first use of the value loads.  The lane that
     // holds a 16-byte piece widens it once (instead of all 16 row lanes later), folds in the
@@ -462,7 +486,7 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
         f[e] *= k_pow[v_bitpos<VB>(e) / 2];
       }
       if (PARTIAL) {
-        const int nv = seq_len - (blk * BLK_TOK + spage * 16 + 8 * (pc & 1));
+        const int nv = tokens_of_page(blk, spage, bad) - 8 * (pc & 1);
 #pragma unroll
         for (int e = 0; e < 8; ++e) f[e] = e < nv ? f[e] : 0.0f;
       }
@@ -492,7 +516,7 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
     // validity of this lane's page tokens (last block only): bit t set = token t of page kb exists
     uint32_t keep[8];
     if (PARTIAL) {
-      const int nv = min(max(seq_len - (blk * BLK_TOK + kb * 16), 0), 16);
+      const int nv = tokens_of_page(blk, kb, bad);
       const uint32_t tokmask = (1u << nv) - 1u;
 #pragma unroll
       for (int i = 0; i < 8; ++i)
@@ -564,38 +588,57 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
     int pid[4];
     const int trips = (max(blk_end - blk_begin, 0) + NGRP - 1) / NGRP;
     int blk = blk_begin + wgrp;
+    // Block tables are device data nobody has checked: every wavefront looks once at the table entries of its
+    // workgroup's blocks (a lane per entry; requested first, used after the first block's loads are on
+    // their way).  Only a workgroup that finds an entry outside the pool runs the checking loop.
+    bool entry_bad = false;
+    {
+      const int e0 = 4 * blk_begin, e1 = min(4 * blk_end, n_pages);
+      for (int e = e0 + lane; e < e1; e += 4 * 64) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) entry_bad |= (unsigned)bt[min(e + 64 * i, e1 - 1)] >= (unsigned)num_pages;
+      }
+    }
+    int bad = 0;                                          // pages of the current block that lie outside the pool
     if (blk < blk_end) {
-      page_ids(blk, pid);
+      bad = page_ids(blk, pid, std::true_type{});
       load_keys(pid, K);
       load_vals(pid, V);
     }
-    // one trip of a walker that still has a block; PARTIAL: the block may reach past the sequence end
-    auto trip = [&](int it, auto partial_tag) {
-      // the block after this walker's last one does not exist: re-request the current one instead,
-      // so that the loads stay outside any branch
-      const int nxt = blk + NGRP;
-      const int nxt_c = nxt < blk_end ? nxt : blk;
-      int pid_n[4];
-      page_ids(nxt_c, pid_n);                            // scalar loads, consumed after the score stage
-      const bool rescale = score_stage(blk, it, K, partial_tag);
-      load_keys(pid_n, K);
-      value_stage(blk, V, rescale, partial_tag);
-      load_vals(pid_n, V);
-      blk = nxt;
-    };
-    // A walker takes every NGRP-th block of the workgroup's range, so it can only run out of blocks,
-    // and only meet the ragged end of the sequence, in the last trip: the loop before it is
-    // straight-line code.
-    for (int it = 0; it < trips - 1; ++it) trip(it, std::false_type{});
-    if (trips > 0) {
-      if (blk >= blk_end) {                              // uniform per wavefront pair
-        if (DS > 1) __syncthreads();
-      } else if ((blk + 1) * BLK_TOK > seq_len) {
-        trip(trips - 1, std::true_type{});
-      } else {
-        trip(trips - 1, std::false_type{});
+    // CHECKED: page ids are validated and every trip takes the masking (PARTIAL) path
+    auto run = [&](auto checked_tag) {
+      constexpr bool CHECKED = decltype(checked_tag)::value;
+      // one trip of a walker that still has a block; PARTIAL: some tokens of the block may not exist
+      auto trip = [&](int it, auto partial_tag) {
+        // the block after this walker's last one does not exist: re-request the current one instead,
+        // so that the loads stay outside any branch
+        const int nxt = blk + NGRP;
+        const int nxt_c = nxt < blk_end ? nxt : blk;
+        int pid_n[4];
+        const int bad_n = page_ids(nxt_c, pid_n, checked_tag);   // scalar loads, consumed after the score stage
+        const bool rescale = score_stage(blk, it, CHECKED ? fresh : it == 0, K, bad, partial_tag);
+        load_keys(pid_n, K);
+        value_stage(blk, V, rescale, bad, partial_tag);
+        load_vals(pid_n, V);
+        blk = nxt;
+        bad = bad_n;
+      };
+      // A walker takes every NGRP-th block of the workgroup's range, so it can only run out of blocks,
+      // and only meet the ragged end of the sequence, in the last trip: the loop before it is
+      // straight-line code.
+      for (int it = 0; it < trips - 1; ++it) trip(it, std::integral_constant<bool, CHECKED>{});
+      if (trips > 0) {
+        if (blk >= blk_end) {                              // uniform per wavefront pair
+          if (DS > 1) __syncthreads();
+        } else if (CHECKED || (blk + 1) * BLK_TOK > seq_len) {
+          trip(trips - 1, std::true_type{});
+        } else {
+          trip(trips - 1, std::false_type{});
+        }
       }
-    }
+    };
+    if (__builtin_amdgcn_ballot_w64(entry_bad) != 0) run(std::true_type{});
+    else run(std::false_type{});
   }
 
   // ---------------------------------------------------------------- merge the walkers, write the partial
@@ -679,7 +722,7 @@ template <int D, int MB, int NX, int VB, int GS, int DS, int WPS, bool F16P>
 static int launch_one(const uint32_t* qa_pack, const float* q_stat, int B, int Hq, int Hkv, int kv_div,
                       const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
                       float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts, int n_split,
-                      int len_sub, hipStream_t st) {
+                      int len_sub, int max_pages, int num_pages, hipStream_t st) {
   const int G = Hq / Hkv;
   size_t per_wave = (size_t)wave_lds_floats(D / DS / GS, DS) * sizeof(float);
   size_t merge = (size_t)(MF_WAVES / DS * G * (D + 2) + MF_WAVES * 16 * 16) * sizeof(float);
@@ -692,12 +735,12 @@ static int launch_one(const uint32_t* qa_pack, const float* q_stat, int B, int H
   if (t_start_event || t_stop_event) {
     hipExtLaunchKernelGGL(kern, dim3(n_split, Hkv, B), dim3(MF_WAVES * 64), smem, st, t_start_event, t_stop_event, 0,
                           qa_pack, q_stat, Hq, Hkv, kv_div, pool, block_table, bt_stride, seq_lens, sm_scale, ly, L, parts,
-                          n_parts, n_split, len_sub);
+                          n_parts, n_split, len_sub, max_pages, num_pages);
     t_start_event = t_stop_event = nullptr;
   } else {
     kern<<<dim3(n_split, Hkv, B), dim3(MF_WAVES * 64), smem, st>>>(qa_pack, q_stat, Hq, Hkv, kv_div, pool, block_table,
                                                                    bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts,
-                                                                   n_split, len_sub);
+                                                                   n_split, len_sub, max_pages, num_pages);
   }
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? TQ_OK : (int)e;
@@ -711,7 +754,7 @@ size_t decode_mfma_pack_words(int B, int Hq, int d) { return (size_t)B * Hq * 9 
 int launch_decode_mfma(const uint32_t* qa_pack, const float* q_stat, int B, int Hq, int Hkv, int kv_div,
                        const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
                        float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts,
-                       int n_split, int len_sub, hipStream_t st) {
+                       int n_split, int len_sub, int max_pages, int num_pages, hipStream_t st) {
   const int G = Hq / Hkv, d = ly.d, mb = ly.mse_bits, vb = L.value_bits, gs = L.group_size;
   if (G > 8 || (L.dtype != TQ_BF16 && L.dtype != TQ_F16) || !L.key_lane_major) return TQ_EUNSUPPORTED;
   const bool f16p = L.dtype == TQ_F16;
@@ -723,10 +766,10 @@ int launch_decode_mfma(const uint32_t* qa_pack, const float* q_stat, int B, int 
     if (f16p)                                                                                                   \
       return launch_one<D_, MB_, NX_, VB_, GS_, DS_, WPS_, true>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,  \
                                                                  bt_stride, seq_lens, sm_scale, ly, L, parts,     \
-                                                                 n_parts, n_split, len_sub, st);                 \
+                                                                 n_parts, n_split, len_sub, max_pages, num_pages, st); \
     return launch_one<D_, MB_, NX_, VB_, GS_, DS_, WPS_, false>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,   \
                                                                 bt_stride, seq_lens, sm_scale, ly, L, parts,      \
-                                                                n_parts, n_split, len_sub, st);                  \
+                                                                n_parts, n_split, len_sub, max_pages, num_pages, st); \
   }
   TQ_TRY(128, 2, 0, 2, 32, 1, 2) TQ_TRY(128, 2, 0, 4, 32, 1, 2) TQ_TRY(256, 2, 0, 2, 32, 2, 2) TQ_TRY(256, 2, 0, 4, 32, 2, 2)
   TQ_TRY(128, 1, 0, 2, 32, 1, 2) TQ_TRY(128, 1, 0, 4, 32, 1, 2) TQ_TRY(256, 1, 0, 2, 32, 2, 2) TQ_TRY(256, 1, 0, 4, 32, 2, 2)

@@ -100,8 +100,18 @@ struct KeyPagedSink {
   uint8_t* pool;
   const int32_t* block_table;
   int max_pages;
+  int num_pages;           // pages of the pool: a table entry outside [0, num_pages) is never written through
   tq_page_layout L;
 };
+
+// Physical page of logical page `lpage` of sequence b, or -1 when the logical page lies outside the block
+// table or the table entry outside the pool (a stale or poisoned entry): the writers then store nothing.
+// The table load itself is unconditional and clamped into the table.
+__device__ __forceinline__ int64_t checked_page(const int32_t* block_table, int max_pages, int num_pages, int b,
+                                                int lpage) {
+  const int raw = block_table[(int64_t)b * max_pages + min(max(lpage, 0), max_pages - 1)];
+  return (lpage >= 0 && lpage < max_pages && (unsigned)raw < (unsigned)num_pages) ? (int64_t)raw : (int64_t)-1;
+}
 
 
 // ------------------------------------------------------------------------------------
@@ -149,7 +159,8 @@ __device__ __forceinline__ void write_key_tile_paged(const KeyPagedSink& sink, c
   int b, lpage, h;
   src.decode(tile, b, lpage, h);
   const tq_page_layout& L = sink.L;
-  int64_t page = sink.block_table[(int64_t)b * sink.max_pages + lpage];
+  const int64_t page = checked_page(sink.block_table, sink.max_pages, sink.num_pages, b, lpage);
+  if (page < 0) return;                                   // the same for every thread of the tile
   uint8_t* pg = sink.pool + (page * src.H + h) * (int64_t)L.page_bytes;
   const int words = d >> 5, planes = mb + 1;
   for (int o = tid; o < planes * words * TILE; o += nthreads) {

@@ -191,6 +191,7 @@ struct ValPagedSink {
   uint8_t* pool;
   const int32_t* block_table;
   int max_pages;
+  int num_pages;           // pages of the pool (see checked_page)
   tq_page_layout L;
 };
 
@@ -277,7 +278,8 @@ value_tile_kernel(const void* __restrict__ v, Source src, int d, int gs, int bit
     int b, lpage, h;
     src.decode(tile, b, lpage, h);
     const tq_page_layout& L = sink.L;
-    int64_t page = sink.block_table[(int64_t)b * sink.max_pages + lpage];
+    const int64_t page = checked_page(sink.block_table, sink.max_pages, sink.num_pages, b, lpage);
+    if (page < 0) return;                              // outside the table or the pool: nothing is stored
     uint8_t* pg = sink.pool + (page * src.H + h) * (int64_t)L.page_bytes;
     // channel j: a field of 16*bits bits, token n at bit bits*n; read-modify-write keeps
     // the codes of slots this call does not touch
@@ -349,8 +351,9 @@ value_chunk_kernel(const void* __restrict__ v, Source src, int d, int gs, Sink s
   if constexpr (!std::is_same<Sink, ValFlatSink>::value) {
     int b, lpage;
     src.decode(tile, b, lpage, head);
-    page = sink.block_table[(int64_t)b * sink.max_pages + min(lpage, sink.max_pages - 1)];
+    page = checked_page(sink.block_table, sink.max_pages, sink.num_pages, b, lpage);
   }
+  const bool page_ok = page >= 0;                    // uniform over the workgroup; false: nothing is stored
   // unconditional load (slots that do not exist read the first vector)
   const uint4 raw = *(const uint4*)((const uint16_t*)v + (ok ? off : 0) + ck * 8);
   if (ck == 0) svalid[t] = ok;
@@ -428,7 +431,7 @@ value_chunk_kernel(const void* __restrict__ v, Source src, int d, int gs, Sink s
   } else {
     const tq_page_layout& L = sink.L;
     uint8_t* pg = sink.pool + (page * src.H + head) * (int64_t)L.page_bytes;
-    if (ok && leader) {
+    if (ok && leader && page_ok) {
       E::store(pg + L.off_vscale, g * TILE + t, sc);
       E::store(pg + L.off_vzero, g * TILE + t, z);
     }
@@ -447,7 +450,7 @@ value_chunk_kernel(const void* __restrict__ v, Source src, int d, int gs, Sink s
         neu |= ((uint32_t)scode[n * d + c] & keep) << (VB * s2);
         mask |= keep << (VB * s2);
       }
-      if (mask != 0) {
+      if (mask != 0 && page_ok) {
         if (VB == 2) {
           uint16_t* f16p = (uint16_t*)fbytes;
           const uint32_t old = (mask == 0xffffu) ? 0u : *f16p;
@@ -468,6 +471,10 @@ static size_t value_tile_smem(int d, int gs) { return (size_t)TILE * d * 5 + (si
 // page -> flat export (store.py:92-114)
 // ------------------------------------------------------------------------------------
 
+// a table entry outside the pool (stale or poisoned) is read as page 0: the export then holds that page's
+// bytes for those tokens, and nothing outside the pool is touched
+__device__ __forceinline__ int export_page(int raw, int num_pages) { return (unsigned)raw < (unsigned)num_pages ? raw : 0; }
+
 __device__ __forceinline__ void copy_elem(void* dst, int64_t di, const void* src, int64_t si, int dt) {
   if (dt == TQ_F32) ((uint32_t*)dst)[di] = ((const uint32_t*)src)[si];
   else ((uint16_t*)dst)[di] = ((const uint16_t*)src)[si];
@@ -478,13 +485,13 @@ __device__ __forceinline__ void copy_elem(void* dst, int64_t di, const void* src
 // per-channel fields through LDS.  Needs 4-byte aligned outputs (rows are multiples of 4 bytes because
 // head_dim is a multiple of 64).
 __global__ void __launch_bounds__(256)
-pool_export_words_kernel(const uint8_t* __restrict__ pool, int H, const int32_t* __restrict__ block_table, int n_tok,
+pool_export_words_kernel(const uint8_t* __restrict__ pool, int num_pages, int H, const int32_t* __restrict__ block_table, int n_tok,
                          tq_page_layout L, uint32_t* __restrict__ idx, uint32_t* __restrict__ signs, void* norms,
                          float* rnorms, uint32_t* __restrict__ v_data, void* v_scales, void* v_zeros) {
   extern __shared__ __align__(16) uint32_t s_fields[];          // the page's value section, d * 2 vb bytes
   const int d = L.d, mb = L.mse_bits, vb = L.value_bits, ng = d / L.group_size, W = d >> 5;
   const int lpage = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
-  const uint8_t* pg = pool + ((int64_t)block_table[lpage] * H + h) * (int64_t)L.page_bytes;
+  const uint8_t* pg = pool + ((int64_t)export_page(block_table[lpage], num_pages) * H + h) * (int64_t)L.page_bytes;
   const int n_valid = min(TILE, n_tok - lpage * TILE);
   const int64_t flat0 = (int64_t)h * n_tok + (int64_t)lpage * TILE;
   const int field_dw = vb >> 1;                                  // dwords per channel field (16 * vb bits)
@@ -542,12 +549,12 @@ pool_export_words_kernel(const uint8_t* __restrict__ pool, int H, const int32_t*
   }
 }
 
-__global__ void pool_export_kernel(const uint8_t* __restrict__ pool, int H, const int32_t* __restrict__ block_table,
+__global__ void pool_export_kernel(const uint8_t* __restrict__ pool, int num_pages, int H, const int32_t* __restrict__ block_table,
                                    int n_tok, tq_page_layout L, uint8_t* idx, uint8_t* signs, void* norms,
                                    float* rnorms, uint8_t* v_data, void* v_scales, void* v_zeros) {
   const int d = L.d, mb = L.mse_bits, vb = L.value_bits, ng = d / L.group_size;
   const int lpage = blockIdx.x, h = blockIdx.y, j = threadIdx.x;
-  const uint8_t* pg = pool + ((int64_t)block_table[lpage] * H + h) * (int64_t)L.page_bytes;
+  const uint8_t* pg = pool + ((int64_t)export_page(block_table[lpage], num_pages) * H + h) * (int64_t)L.page_bytes;
   const int eff = eff_bits(mb), per = 8 / eff, row = idx_row_bytes(d, mb), srow = d >> 3;
   const int vrow = d * vb / 8, vper = 8 / vb;
   for (int n = 0; n < TILE; ++n) {
@@ -811,10 +818,11 @@ SideLane* side_lane() {
 // keys and values of the runs described by `src` into the pages of `block_table`
 static int append_runs(const void* k, const void* v, int dtype, const PagedSource& src, const int32_t* block_table,
                        int max_pages, const tq_layer* layer, const tq_page_layout* layout, uint8_t* pool,
-                       void* stream) {
+                       int64_t num_pages, void* stream) {
   int64_t tiles = (int64_t)src.B * src.tiles_per_seq * src.H;
-  KeyPagedSink ks{pool, block_table, max_pages, *layout};
-  ValPagedSink vs{pool, block_table, max_pages, *layout};
+  const int pool_pages = (int)(num_pages < 0x7fffffff ? num_pages : 0x7fffffff);    // page numbers are int32
+  KeyPagedSink ks{pool, block_table, max_pages, pool_pages, *layout};
+  ValPagedSink vs{pool, block_table, max_pages, pool_pages, *layout};
   int rc;
   // Large appends run the value kernel beside the key kernel: the key kernel leaves a quarter of the
   // registers and issue slots of every SIMD free, which the small value wavefronts fill (the two
@@ -850,11 +858,14 @@ extern "C" int tq_append_kv_paged(const void* k, const void* v, int dtype, int B
   if (dtype != layout->dtype || layout->d != layer->d || layout->mse_bits != layer->mse_bits) return TQ_EINVAL;
   if (B < 0 || T < 0 || H <= 0 || max_pages <= 0 || num_pages <= 0) return TQ_EINVAL;
   if (B == 0 || T == 0) return TQ_OK;
+  // without start positions the run is known on the host: it has to fit the block table (with start
+  // positions, the kernels skip whatever falls outside the table)
+  if (!start_pos && T > (int64_t)max_pages * TILE) return TQ_EINVAL;
   // a run of T tokens starting anywhere inside a page touches at most this many pages
   // (the run may begin at any of the 16 slots of its first page when start_pos is given)
   const int tiles_per_seq = start_pos ? (T + TILE - 2) / TILE + 1 : (T + TILE - 1) / TILE;
   PagedSource src{B, T, H, tiles_per_seq, stride_b, stride_t, stride_h, start_pos};
-  return append_runs(k, v, dtype, src, block_table, max_pages, layer, layout, pool, stream);
+  return append_runs(k, v, dtype, src, block_table, max_pages, layer, layout, pool, num_pages, stream);
 }
 
 extern "C" int tq_append_kv_ragged(const void* k, const void* v, int dtype, int B, int T_max, int H, int64_t stride_t,
@@ -872,7 +883,7 @@ extern "C" int tq_append_kv_ragged(const void* k, const void* v, int dtype, int 
   PagedSource src{B, T_max, H, tiles_per_seq, 0, stride_t, stride_h, start_pos};
   src.run_len = run_len;
   src.row0 = row0;
-  return append_runs(k, v, dtype, src, block_table, max_pages, layer, layout, pool, stream);
+  return append_runs(k, v, dtype, src, block_table, max_pages, layer, layout, pool, num_pages, stream);
 }
 
 extern "C" int tq_append_kv_from_blocks(const void* k_cache, const void* v_cache, int dtype, int B, int T, int H,
@@ -887,13 +898,14 @@ extern "C" int tq_append_kv_from_blocks(const void* k_cache, const void* v_cache
   if (dtype != layout->dtype || layout->d != layer->d || layout->mse_bits != layer->mse_bits) return TQ_EINVAL;
   if (B < 0 || T < 0 || H <= 0 || max_pages <= 0 || num_pages <= 0 || src_stride <= 0) return TQ_EINVAL;
   if (B == 0 || T == 0) return TQ_OK;
+  if (!start_pos && !run_len && T > (int64_t)max_pages * TILE) return TQ_EINVAL;
   const int tiles_per_seq = start_pos ? (T + TILE - 2) / TILE + 1 : (T + TILE - 1) / TILE;
   PagedSource src{B, T, H, tiles_per_seq, 0, stride_t, stride_h, start_pos};
   src.src_table = src_table;
   src.src_stride = src_stride;
   src.stride_blk = stride_blk;
   src.run_len = run_len;
-  return append_runs(k_cache, v_cache, dtype, src, block_table, max_pages, layer, layout, pool, stream);
+  return append_runs(k_cache, v_cache, dtype, src, block_table, max_pages, layer, layout, pool, num_pages, stream);
 }
 
 extern "C" int tq_pool_export(const uint8_t* pool, int64_t num_pages, int H, const int32_t* block_table, int n_tok,
@@ -904,18 +916,19 @@ extern "C" int tq_pool_export(const uint8_t* pool, int64_t num_pages, int H, con
   if (H <= 0 || n_tok < 0 || num_pages <= 0) return TQ_EINVAL;
   if (n_tok == 0) return TQ_OK;
   const tq_page_layout& L = *layout;
+  const int pool_pages = (int)(num_pages < 0x7fffffff ? num_pages : 0x7fffffff);
   if ((L.value_bits == 2 || L.value_bits == 4 || L.value_bits == 8) && L.d % 64 == 0 && L.off_vdata % 4 == 0 &&
       (uintptr_t)idx % 4 == 0 && (uintptr_t)signs % 4 == 0 && (uintptr_t)v_data % 4 == 0) {
     dim3 g2((n_tok + TILE - 1) / TILE, H), b2(256);
     const size_t sm = (size_t)L.d * 2 * L.value_bits;
-    pool_export_words_kernel<<<g2, b2, sm, (hipStream_t)stream>>>(pool, H, block_table, n_tok, L, (uint32_t*)idx,
+    pool_export_words_kernel<<<g2, b2, sm, (hipStream_t)stream>>>(pool, pool_pages, H, block_table, n_tok, L, (uint32_t*)idx,
                                                                  (uint32_t*)signs, norms, rnorms, (uint32_t*)v_data,
                                                                  v_scales, v_zeros);
     TQ_CHECK_LAUNCH();
     return TQ_OK;
   }
   dim3 grid((n_tok + TILE - 1) / TILE, H), block(64);
-  pool_export_kernel<<<grid, block, 0, (hipStream_t)stream>>>(pool, H, block_table, n_tok, *layout, idx, signs, norms,
+  pool_export_kernel<<<grid, block, 0, (hipStream_t)stream>>>(pool, pool_pages, H, block_table, n_tok, *layout, idx, signs, norms,
                                                              rnorms, v_data, v_scales, v_zeros);
   TQ_CHECK_LAUNCH();
   return TQ_OK;

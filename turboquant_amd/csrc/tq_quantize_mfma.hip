@@ -295,7 +295,7 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
     if (wt < n_tiles) {
       int b, lpage, h;
       src.decode((int)wt, b, lpage, h);
-      wpage = sink.block_table[(int64_t)b * sink.max_pages + min(lpage, sink.max_pages - 1)];
+      wpage = checked_page(sink.block_table, sink.max_pages, sink.num_pages, b, lpage);
     }
   }
 #pragma unroll
@@ -511,7 +511,8 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
       const int64_t tile = tile0 + m;
       if (tile >= n_tiles) break;
       // a tile none of whose slots exists may lie beyond the block table: do not look it up
-      if (__builtin_amdgcn_ballot_w64(lane < TILE && svalid[16 * m + lane]) == 0) continue;
+      // (and a page outside the table or the pool is not written)
+      if (__builtin_amdgcn_ballot_w64(lane < TILE && svalid[16 * m + lane]) == 0 || wpage < 0) continue;
       int b, lpage, h;
       src.decode((int)tile, b, lpage, h);
       uint8_t* pg = sink.pool + (wpage * src.H + h) * (int64_t)L.page_bytes;

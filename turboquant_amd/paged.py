@@ -218,7 +218,7 @@ class PagedKVPool:
         if scale is None:
             scale = 1.0 / math.sqrt(d)
         bt = block_table.contiguous()
-        bt_stride = 0 if bt.dim() == 1 else bt.shape[1]
+        bt_stride = -bt.shape[0] if bt.dim() == 1 else bt.shape[1]      # negative: one shared row of that length
         seq_lens = seq_lens.to(device=self.device, dtype=torch.int32).contiguous()
         if n_split is None:
             if max_len is None:
@@ -287,7 +287,7 @@ class PagedKVPool:
         if scale is None:
             scale = 1.0 / math.sqrt(d)
         bt = block_table.contiguous()
-        bt_stride = 0 if bt.dim() == 1 else bt.shape[1]
+        bt_stride = -bt.shape[0] if bt.dim() == 1 else bt.shape[1]      # negative: one shared row of that length
         seq_lens = seq_lens.to(device=self.device, dtype=torch.int32).contiguous()
         if n_split is None:
             if max_len is None:
