@@ -40,7 +40,8 @@ enum {
   TQ_OK = 0,
   TQ_EINVAL = -1,       /* a size, stride or enum is out of range                */
   TQ_EUNSUPPORTED = -2, /* a legal request this build has no kernel for          */
-  TQ_ENULL = -3         /* a required pointer is NULL                            */
+  TQ_ENULL = -3,        /* a required pointer is NULL                            */
+  TQ_ETOOBIG = -4       /* the call needs more scratch than the library's static area holds */
 };
 
 #define TQ_PAGE_TOKENS 16
@@ -264,6 +265,23 @@ int tq_decode_attn_paged_ring(const void *q, int dtype, int B, int Hq, int Hkv, 
                               float sm_scale, const tq_layer *layer, const tq_page_layout *layout,
                               const void *k_cache, const void *v_cache, int64_t cs_blk, int64_t cs_t, int64_t cs_h,
                               int ring_rows, void *out, void *workspace, int n_split, void *stream);
+
+/* tq_decode_attn_paged for callers that cannot allocate or pass a workspace (code under HIP graph capture
+ * that owns no buffers, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the
+ * reference.  Same arguments and result, bit for bit, as tq_decode_attn_paged with the same n_split, minus the
+ * workspace: partials, rotated queries and query operands live in a file-scope device array of
+ * TQ_NOALLOC_SCRATCH_BYTES inside the library (one copy per GPU, held until the process ends; its address is
+ * looked up with hipGetSymbolAddress the first time a device is used).  The call allocates nothing and
+ * frees nothing.  A call that needs more than the array holds - roughly 4*B*Hq*(n_split+1)*(d+2) bytes of
+ * partials plus 8*B*Hq*d - returns TQ_ETOOBIG and launches nothing.  All calls on one GPU share the array:
+ * calls that overlap on one GPU (different streams or threads) race; serialise them or use the workspace form. */
+#define TQ_NOALLOC_SCRATCH_BYTES (16u << 20)
+int tq_decode_attn_paged_noalloc(const void *q, int dtype, int B, int Hq, int Hkv, const uint8_t *pool,
+                                 int64_t num_pages, const int32_t *block_table, int bt_stride, const int32_t *seq_lens,
+                                 float sm_scale, const tq_layer *layer, const tq_page_layout *layout,
+                                 const void *recent_k, const void *recent_v, int recent_rows, int64_t rs_b,
+                                 int64_t rs_r, int64_t rs_h, const int32_t *recent_len, void *out, int n_split,
+                                 void *stream);
 
 /* Log-sum-exp merge of n_parts partial results per (b, query head):
  * parts (B*Hq, n_parts, d+2) fp32 = [running max, sum of exp, un-normalised acc];

@@ -23,7 +23,8 @@ _lib: Optional[C.CDLL] = None
 
 _ERR = {-1: "TQ_EINVAL (a size, stride or enum is out of range)",
         -2: "TQ_EUNSUPPORTED (no kernel for this shape / bit-width)",
-        -3: "TQ_ENULL (a required pointer is NULL)"}
+        -3: "TQ_ENULL (a required pointer is NULL)",
+        -4: "TQ_ETOOBIG (the call needs more scratch than the library's static area holds; use the workspace form)"}
 
 
 class TqLayer(C.Structure):
@@ -75,6 +76,8 @@ _SIGNATURES = {
                                               _i, _vp]),
     "tq_decode_attn_paged_ring": (C.c_int, [_vp, _i, _i, _i, _i, _vp, _i64, _vp, _i, _vp, _f, C.POINTER(TqLayer),
                                             C.POINTER(TqPageLayout), _vp, _vp, _i64, _i64, _i64, _i, _vp, _vp, _i, _vp]),
+    "tq_decode_attn_paged_noalloc": (C.c_int, [_vp, _i, _i, _i, _i, _vp, _i64, _vp, _i, _vp, _f, C.POINTER(TqLayer),
+                                               C.POINTER(TqPageLayout), _vp, _vp, _i, _i64, _i64, _i64, _vp, _vp, _i, _vp]),
     "tq_decode_merge": (C.c_int, [_vp, _i64, _i, _i, _i, _vp, _vp]),
     "tq_time_next_page_kernel": (None, [_vp, _vp]),
     "tq_stream_read": (C.c_int, [_vp, C.c_size_t, _i, _i, _vp, _vp]),

@@ -17,6 +17,12 @@
 #include "tq_common.h"
 #include "tq_prep.h"
 
+// Device memory of the entry point that allocates nothing (tq_decode_attn_paged_noalloc): the split partials,
+// the rotated queries and the packed query operands of one decode call.  One copy per GPU the library's code
+// is loaded on, held until the process ends.  In host code this name is only a handle for
+// hipGetSymbolAddress; kernels receive the address that call returned.
+static __device__ __align__(256) unsigned char scratch[TQ_NOALLOC_SCRATCH_BYTES];
+
 namespace tq {
 
 constexpr int G_MAX = 16;      // query heads per KV head handled by one workgroup
@@ -1081,4 +1087,69 @@ extern "C" int tq_decode_attn_paged(const void* q, int dtype, int B, int Hq, int
   return tq_decode_attn_paged_stages(q, dtype, B, Hq, Hkv, pool, num_pages, block_table, bt_stride, seq_lens, sm_scale,
                                      layer, layout, recent_k, recent_v, recent_rows, rs_b, rs_r, rs_h, recent_len, out,
                                      workspace, n_split, 7, stream);
+}
+
+// ---- the entry point that allocates nothing -----------------------------------------------------------
+namespace {
+constexpr int SCRATCH_MAX_DEVICES = 64;
+std::atomic<void*> g_scratch_ptr[SCRATCH_MAX_DEVICES];      // device address of `scratch`, per device
+
+// Address of the current device's copy of `scratch` (looked up once per device; two threads that race
+// here ask for the same address).
+int scratch_address(void** out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= SCRATCH_MAX_DEVICES) return TQ_EUNSUPPORTED;
+  void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (!p) return TQ_EINVAL;
+    g_scratch_ptr[dev].store(p, std::memory_order_release);
+  }
+  *out = p;
+  return TQ_OK;
+}
+
+// Bytes of workspace decode_stages really touches for this call (tq_decode_workspace_bytes reserves
+// room for the largest operand set instead): partials, rotated / sketched queries, statistics, and the
+// packed operands of the matrix-core kernel, (index planes + multi-bit terms + sign plane) x d/128 KiB-words
+// per group of query heads.
+size_t decode_scratch_need(int B, int Hq, int Hkv, int n_split, const tq_layer& ly) {
+  const int d = ly.d, G = Hq / Hkv;
+  int kv_div = 0;
+  for (int n = 1; n <= G && !kv_div; ++n)
+    if (G % n == 0 && G / n <= 8) kv_div = n;
+  size_t floats = parts_floats(B, Hq, d, n_split + 1) + (size_t)2 * B * Hq * d + (size_t)4 * B * Hq;
+  size_t words = 0;
+  if (kv_div && (d == 128 || d == 256)) {
+    int planes = ly.mse_bits + 1;
+    for (int t = 0; t < ly.n_terms; ++t)
+      if (__builtin_popcount(ly.term_mask[t]) > 1) ++planes;
+    words = (size_t)B * Hkv * kv_div * planes * (d / 128) * 2 * 64 * 8;
+  }
+  return (floats + words) * 4;
+}
+}  // namespace
+
+extern "C" int tq_decode_attn_paged_noalloc(const void* q, int dtype, int B, int Hq, int Hkv, const uint8_t* pool,
+                                            int64_t num_pages, const int32_t* block_table, int bt_stride,
+                                            const int32_t* seq_lens, float sm_scale, const tq_layer* layer,
+                                            const tq_page_layout* layout, const void* recent_k, const void* recent_v,
+                                            int recent_rows, int64_t rs_b, int64_t rs_r, int64_t rs_h,
+                                            const int32_t* recent_len, void* out, int n_split, void* stream) {
+  if (!layer) return TQ_ENULL;
+  if (B <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || n_split <= 0 || layer->d <= 0 || layer->n_terms < 0 ||
+      layer->n_terms > TQ_MAX_TERMS)
+    return TQ_EINVAL;
+  if (decode_scratch_need(B, Hq, Hkv, n_split, *layer) > (size_t)TQ_NOALLOC_SCRATCH_BYTES) return TQ_ETOOBIG;
+  void* ws = nullptr;
+  const int rc = scratch_address(&ws);
+  if (rc) return rc;
+  // Every byte of the scratch area that a stage reads was written by an earlier stage of the same call,
+  // so nothing has to be cleared between calls.
+  return tq_decode_attn_paged_stages(q, dtype, B, Hq, Hkv, pool, num_pages, block_table, bt_stride, seq_lens, sm_scale,
+                                     layer, layout, recent_k, recent_v, recent_rows, rs_b, rs_r, rs_h, recent_len, out,
+                                     ws, n_split, 7, stream);
 }

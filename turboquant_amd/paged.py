@@ -203,13 +203,16 @@ class PagedKVPool:
                          recent_v: Optional[torch.Tensor] = None, recent_len: Optional[torch.Tensor] = None,
                          n_split: Optional[int] = None, workspace: Optional[torch.Tensor] = None,
                          out: Optional[torch.Tensor] = None, max_len: Optional[int] = None,
-                         stages: int = 7) -> torch.Tensor:
+                         stages: int = 7, static_scratch: bool = False) -> torch.Tensor:
         """softmax(scale * [scores_hist ; q k_recent^T]) [v_hist ; v_recent] for one
         query token per sequence.  query (B, Hq, d);
         block_table (B, max_pages) or (max_pages,) shared; seq_lens (B,) int32;
         recent_k / recent_v (B, R, H, d) exact tokens, recent_len (B,) valid rows.
         `stages` (bit 0 query rotation, bit 1 page kernel, bit 2 merge) exists for
-        timing the stages apart; 7 runs the whole thing."""
+        timing the stages apart; 7 runs the whole thing.  `static_scratch` runs the library's entry
+        point that allocates nothing (tq_decode_attn_paged_noalloc): no workspace tensor, the partials live
+        in a fixed device array inside the library (16 MiB; larger calls raise), shared by all calls on
+        this GPU - pass `out` as well and the call touches no allocator at all."""
         _ffi.require_gpu(query, "query")
         B, Hq, d = query.shape
         if d != self.head_dim or Hq % self.num_kv_heads:
@@ -224,7 +227,10 @@ class PagedKVPool:
             if max_len is None:
                 max_len = (bt.shape[-1]) * PAGE_TOKENS
             n_split = self.default_splits(B, max_len, Hq)
-        if workspace is None:
+        if static_scratch:
+            if workspace is not None or stages != 7:
+                raise ValueError("static_scratch takes no workspace and runs all stages")
+        elif workspace is None:
             workspace = self.workspace(B, Hq, n_split)
         if out is None:
             out = torch.empty_like(query)
@@ -243,6 +249,14 @@ class PagedKVPool:
                 recent_len = recent_len.to(device=self.device, dtype=torch.int32).contiguous()
                 rl_ptr = recent_len.data_ptr()
         ly = self.quantizer._layer()
+        if static_scratch:
+            with torch.cuda.device(self.device):
+                _ffi.check(_ffi.lib().tq_decode_attn_paged_noalloc(
+                    query.data_ptr(), _ffi.dtype_tag(query.dtype), B, Hq, self.num_kv_heads, self.data.data_ptr(),
+                    self.num_pages, bt.data_ptr(), bt_stride, seq_lens.data_ptr(), float(scale), C.byref(ly),
+                    C.byref(self.layout), rk_ptr, rv_ptr, rows, rs[0], rs[1], rs[2], rl_ptr, out.data_ptr(),
+                    n_split, _ffi.stream_ptr(self.device)), "tq_decode_attn_paged_noalloc")
+            return out
         with torch.cuda.device(self.device):
             _ffi.check(_ffi.lib().tq_decode_attn_paged_stages(
                 query.data_ptr(), _ffi.dtype_tag(query.dtype), B, Hq, self.num_kv_heads, self.data.data_ptr(),
