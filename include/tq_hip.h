@@ -297,6 +297,20 @@ int tq_decode_merge(const float *parts, int64_t rows, int n_parts, int d, int dt
  * stream, which also contains the dispatch gap.  Pass NULLs to disarm.                             */
 void tq_time_next_page_kernel(void *start_event, void *stop_event);
 
+/* Tuning and test knobs (no counterpart in the reference); process-wide, take effect at the next call.
+ *   "prep_units"       0 (default): the query preparation of the matrix-core decode path runs as one workgroup
+ *                      per 32-coordinate plane word for all heads of a group; 1: one small workgroup per (few
+ *                      query heads, plane word).  Same operands bit for bit.
+ *   "fuse_prep"        0 (default): a decode step is three launches (query preparation, page kernel, merge);
+ *                      1: a compressed-only step on the matrix-core path prepares its query operands inside
+ *                      the page kernel's launch (two launches; the workgroups of a (sequence, KV head) share
+ *                      the work and hand the operands to each other).  Same result bit for bit.  Only in a
+ *                      library built with -DTQ_FUSED_PREP (TQ_EUNSUPPORTED otherwise): it measured slower.
+ *   "prep_spin_limit"  with fuse_prep: how often a workgroup polls for the other workgroups' share of the
+ *                      operands before it computes them itself (default 20000; 0 = never wait).
+ * Returns TQ_EINVAL for an unknown name or a value out of range.                                        */
+int tq_set_option(const char *name, int64_t value);
+
 /* Measurement aid (no counterpart in the reference).  Reads `bytes` (a multiple of 16) from `src`
  * (16-byte aligned) with `workgroups_per_cu` workgroups of 256 lanes per compute unit, each lane keeping
  * `loads_in_flight` (1, 4 or 8) 16-byte loads outstanding, and writes nothing (`sink`, 4 bytes, may be

@@ -279,3 +279,76 @@ def test_decode_gives_no_weight_to_pages_outside_the_pool(gpu, d, key_bits, vb, 
     z = pool.decode_attention(q.to(gpu), allbad.to(gpu), seq, n_split=2, max_len=N)
     torch.cuda.synchronize()
     assert torch.count_nonzero(z) == 0
+
+
+# ------------------------------------------------------------------ query preparation inside the page kernel's launch
+def _set_option(name, value):
+    from turboquant_amd import _ffi
+    _ffi.check(_ffi.lib().tq_set_option(name.encode(), int(value)), "tq_set_option")
+
+
+def _has_fused_prep():
+    from turboquant_amd import _ffi
+    rc = _ffi.lib().tq_set_option(b"fuse_prep", 1)
+    _ffi.lib().tq_set_option(b"fuse_prep", 0)
+    return rc == 0
+
+
+@pytest.mark.parametrize("d,key_bits,vb,Hq,Hkv,B,lens,n_split", [
+    (256, 3, 2, 16, 2, 2, [5000, 777], 64),        # one head per unit, 64 units
+    (256, 3, 2, 16, 2, 2, [5000, 777], 5),         # fewer workgroups than units: several units each
+    (128, 3, 4, 32, 8, 3, [900, 64, 300], 4),      # 4 of 8 heads exist, one unit per plane word
+    (128, 4, 4, 8, 2, 2, [700, 1], 9),             # 4-bit keys (an extra term plane), odd split count
+    (256, 2, 4, 10, 2, 1, [2000], 33),             # 5 heads per group
+    (128, 3, 2, 32, 2, 2, [400, 900], 16),         # 16 heads per KV head = two groups of 8
+    (128, 3, 2, 3, 1, 1, [130], 1)])               # a single workgroup does everything
+def test_decode_step_with_the_preparation_inside_the_page_kernel(gpu, d, key_bits, vb, Hq, Hkv, B, lens, n_split):
+    """The query operands of the matrix-core page kernel (triton_kernels.py:527-528: q Pi^T, q S^T, here also
+    their fp6 operand form) can be prepared three ways: a workgroup per plane word, a workgroup per (few heads,
+    plane word) unit, or inside the page kernel's own launch with the workgroups of a (sequence, KV head)
+    sharing the units.  The operands are the same numbers whoever computes them, so all three must give the
+    same output bit for bit - also when no workgroup of the fused launch waits for the others at all (every
+    workgroup then computes every unit itself), and for fp16 / fp32 queries."""
+    g = torch.Generator().manual_seed(d + Hq + n_split)
+    pages = (max(lens) + 15) // 16
+    pool, tq = _make_pool(gpu, d, key_bits, vb, Hkv, B * pages + 1, torch.bfloat16, seed=42)
+    table = torch.randperm(B * pages + 1, generator=g)[: B * pages].to(torch.int32).view(B, pages).to(gpu)
+    k = torch.randn(B, max(lens), Hkv, d, generator=g).bfloat16().to(gpu)
+    v = torch.randn(B, max(lens), Hkv, d, generator=g).bfloat16().to(gpu)
+    pool.append(k, v, table)
+    seq = torch.tensor(lens, dtype=torch.int32, device=gpu)
+    _progress(f"fused preparation d={d} kb={key_bits} vb={vb} Hq={Hq} Hkv={Hkv} lens={lens} splits={n_split}")
+    try:
+        for qdt in (torch.bfloat16, torch.float16, torch.float32):
+            q = torch.randn(B, Hq, d, generator=g).to(qdt).to(gpu)
+            _set_option("fuse_prep", 0)
+            _set_option("prep_units", 0)
+            want = pool.decode_attention(q, table, seq, n_split=n_split)
+            _set_option("prep_units", 1)
+            units = pool.decode_attention(q, table, seq, n_split=n_split)
+            torch.cuda.synchronize()
+            assert torch.equal(units, want), qdt
+            if not _has_fused_prep():       # the in-launch preparation is a build option (-DTQ_FUSED_PREP)
+                continue
+            _set_option("fuse_prep", 1)
+            got = pool.decode_attention(q, table, seq, n_split=n_split)
+            again = pool.decode_attention(q, table, seq, n_split=n_split)
+            _set_option("prep_spin_limit", 0)
+            alone = pool.decode_attention(q, table, seq, n_split=n_split)
+            _set_option("prep_spin_limit", 20000)
+            torch.cuda.synchronize()
+            assert torch.equal(got, want), qdt
+            assert torch.equal(again, want), qdt
+            assert torch.equal(alone, want), qdt
+        # and against the oracle, like every other decode test
+        q = torch.randn(B, Hq, d, generator=g).bfloat16()
+        out = pool.decode_attention(q.to(gpu), table, seq, n_split=n_split).cpu()
+    finally:
+        _set_option("fuse_prep", 0)
+        _set_option("prep_units", 0)
+        _set_option("prep_spin_limit", 20000)
+    prm = params_of(tq)
+    for b in range(B):
+        kc, vc = _store_from_oracle_view(pool, table[b], lens[b])
+        want = O.hybrid_attention(q[b:b + 1], kc, vc, max(lens[b], O.MIN_HISTORY), prm, Hkv, None, None)
+        assert cosine(out[b:b + 1], want) >= COS_GATE, b

@@ -18,7 +18,8 @@ TQ_PAGE_TOKENS = 16
 TQ_MAX_TERMS = 15
 ABI_VERSION = 1
 
-_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libtq_hip.so")
+# TQ_HIP_LIBRARY overrides the in-tree library (e.g. to compare two builds)
+_LIB_PATH = os.environ.get("TQ_HIP_LIBRARY") or os.path.join(os.path.dirname(os.path.abspath(__file__)), "libtq_hip.so")
 _lib: Optional[C.CDLL] = None
 
 _ERR = {-1: "TQ_EINVAL (a size, stride or enum is out of range)",
@@ -80,6 +81,7 @@ _SIGNATURES = {
                                                C.POINTER(TqPageLayout), _vp, _vp, _i, _i64, _i64, _i64, _vp, _vp, _i, _vp]),
     "tq_decode_merge": (C.c_int, [_vp, _i64, _i, _i, _i, _vp, _vp]),
     "tq_time_next_page_kernel": (None, [_vp, _vp]),
+    "tq_set_option": (C.c_int, [C.c_char_p, _i64]),
     "tq_stream_read": (C.c_int, [_vp, C.c_size_t, _i, _i, _vp, _vp]),
 }
 

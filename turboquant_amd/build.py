@@ -41,7 +41,8 @@ def build_library(verbose: bool = False) -> str:
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     objdir = os.path.join(HERE, "build")
     os.makedirs(objdir, exist_ok=True)
-    compile_flags = [f for f in FLAGS if f != "-shared"]
+    # TQ_EXTRA_HIPCC_FLAGS: extra compile flags, e.g. -DTQ_FUSED_PREP for the in-launch query preparation
+    compile_flags = [f for f in FLAGS if f != "-shared"] + os.environ.get("TQ_EXTRA_HIPCC_FLAGS", "").split()
     jobs = []
     for src in SOURCES:
         obj = os.path.join(objdir, src.replace(".hip", ".o"))

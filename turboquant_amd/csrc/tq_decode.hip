@@ -14,8 +14,13 @@
 
 #include <atomic>
 
+#include <chrono>
+#include <cstring>
+
 #include "tq_common.h"
 #include "tq_prep.h"
+#include "tq_decode_mfma.h"
+#include "tq_options.h"
 
 // Device memory of the entry point that allocates nothing (tq_decode_attn_paged_noalloc): the split partials,
 // the rotated queries and the packed query operands of one decode call.  One copy per GPU the library's code
@@ -731,7 +736,18 @@ static size_t merge_smem(int n_parts, int d) {
 }
 
 __global__ void __launch_bounds__(256)
-merge_kernel(const float* __restrict__ parts, int n_parts, int part_stride, int d, int dtype, void* __restrict__ out) {
+merge_kernel(const float* __restrict__ parts, int n_parts, int part_stride, int d, int dtype, void* __restrict__ out,
+             unsigned long long* __restrict__ flags, int n_flags) {
+  // the flags under which the page kernel's workgroups published their query-preparation units are
+  // cleared here, after that kernel has ended: the next call (or the next replay of a captured one,
+  // which carries the same nonce) starts without a published unit
+  {
+    const int per_row = (n_flags + (int)gridDim.x - 1) / (int)gridDim.x;
+    for (int i = threadIdx.x; i < per_row; i += blockDim.x) {
+      const int64_t at = (int64_t)blockIdx.x * per_row + i;
+      if (at < n_flags) flags[at] = 0ull;
+    }
+  }
   extern __shared__ float s_w[];                 // [n_parts] weights, [n_parts] m, [n_parts] l, [8] scratch, [S][d] sums
   const int64_t row = blockIdx.x;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -810,22 +826,57 @@ using namespace tq;
 
 namespace tq {
 int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* layer, float* q_rot, float* q_sk,
-                        float* q_stat, uint32_t* qa_pack, int G, float sm_scale, hipStream_t st);
-size_t decode_mfma_pack_words(int B, int Hkv, int d);
-int launch_decode_mfma(const uint32_t* qa_pack, const float* q_stat, int B, int Hq, int Hkv, int kv_div,
-                       const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
-                       float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts,
-                       int n_split, int len_sub, int max_pages, int num_pages, hipStream_t st);
+                        float* q_stat, uint32_t* qa_pack, int G, float sm_scale, hipStream_t st, bool q_rot_unused);
 }  // namespace tq
 
 static size_t parts_floats(int B, int Hq, int d, int n_parts) { return (size_t)B * Hq * n_parts * (d + 2); }
+// publication flags of the in-kernel query preparation: 64 per group of query heads, at most B * Hq groups
+static size_t flag_words(int B, int Hq) { return (size_t)B * Hq * 64; }
+
+// ---- knobs (tq_set_option) -----------------------------------------------------------------------------
+namespace tq {
+std::atomic<int> opt_fuse_prep{0};
+std::atomic<int> opt_prep_spin_limit{20000};
+std::atomic<int> opt_prep_units{0};
+}  // namespace tq
+
+namespace {
+std::atomic<unsigned long long> g_nonce{0};
+
+unsigned long long next_nonce() {
+  unsigned long long v = g_nonce.load();
+  if (v == 0) {       // first use in this process: start somewhere unpredictable, far from small numbers
+    const unsigned long long seed =
+        ((unsigned long long)std::chrono::steady_clock::now().time_since_epoch().count() * 0x9E3779B97F4A7C15ull) | (1ull << 62);
+    g_nonce.compare_exchange_strong(v, seed);
+  }
+  v = g_nonce.fetch_add(1) + 1;
+  return v ? v : g_nonce.fetch_add(1) + 1;
+}
+}  // namespace
+
+extern "C" int tq_set_option(const char* name, int64_t value) {
+  if (!name) return TQ_ENULL;
+  if (!std::strcmp(name, "fuse_prep")) {
+    if (value != 0 && !decode_mfma_has_fused_prep()) return TQ_EUNSUPPORTED;     // not compiled into this build
+    opt_fuse_prep.store(value != 0);
+    return TQ_OK;
+  }
+  if (!std::strcmp(name, "prep_units")) { opt_prep_units.store(value != 0); return TQ_OK; }
+  if (!std::strcmp(name, "prep_spin_limit")) {
+    if (value < 0 || value > 100000000) return TQ_EINVAL;
+    opt_prep_spin_limit.store((int)value);
+    return TQ_OK;
+  }
+  return TQ_EINVAL;
+}
 
 extern "C" size_t tq_decode_workspace_bytes(int B, int Hq, int d, int n_split) {
   if (B <= 0 || Hq <= 0 || d <= 0 || n_split <= 0) return 0;
   // partials for n_split history splits + 1 exact tail, then q_rot, q_sk, 4 statistics per query row and
   // the packed query operands of the matrix-core kernel (sized for the largest kernel: 9 term planes, 8 heads)
   return (parts_floats(B, Hq, d, n_split + 1) + (size_t)2 * B * Hq * d + (size_t)4 * B * Hq) * sizeof(float) +
-         decode_mfma_pack_words(B, Hq, d) * sizeof(uint32_t);
+         flag_words(B, Hq) * sizeof(unsigned long long) + decode_mfma_pack_words(B, Hq, d) * sizeof(uint32_t);
 }
 
 extern "C" int tq_decode_merge(const float* parts, int64_t rows, int n_parts, int d, int dtype, void* out,
@@ -834,7 +885,7 @@ extern "C" int tq_decode_merge(const float* parts, int64_t rows, int n_parts, in
   if (rows < 0 || n_parts <= 0 || d <= 0 || dtype < TQ_F32 || dtype > TQ_BF16) return TQ_EINVAL;
   if (rows == 0) return TQ_OK;
   merge_kernel<<<dim3((unsigned)rows), dim3(256), merge_smem(n_parts, d), (hipStream_t)stream>>>(
-      parts, n_parts, n_parts, d, dtype, out);
+      parts, n_parts, n_parts, d, dtype, out, nullptr, 0);
   TQ_CHECK_LAUNCH();
   return TQ_OK;
 }
@@ -899,7 +950,8 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   float* q_rot = parts + parts_floats(B, Hq, d, n_parts);
   float* q_sk = q_rot + (size_t)B * Hq * d;
   float* q_stat = q_sk + (size_t)B * Hq * d;
-  uint32_t* qa_pack = (uint32_t*)(q_stat + (size_t)4 * B * Hq);
+  unsigned long long* flags = (unsigned long long*)(q_stat + (size_t)4 * B * Hq);       // 8-byte aligned: every term above is even
+  uint32_t* qa_pack = (uint32_t*)(flags + flag_words(B, Hq));
   // the matrix-core kernel takes up to 8 query heads per group: a KV head with more is served by kv_div
   // groups of G / kv_div heads (0 = no such split, e.g. 11 heads)
   int kv_div = 0;
@@ -926,7 +978,32 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   const int n_tail = Hkv * B * ((G + TAIL_GC - 1) / TAIL_GC);
   bool tail_done = false;
 
-  if (stages & 1) {
+  // Whole compressed-only step on the matrix-core path: the query preparation runs as a prologue of the
+  // page kernel's own launch (its workgroups share the work and hand the operands to each other), so the
+  // step is two launches, page kernel and merge.
+  bool fused = false;
+  const int n_flags = B * Hkv * (kv_div ? kv_div : 1) * 64;
+  if (stages == 7 && mfma_shape && !tail && opt_fuse_prep.load()) {
+    if (!layer->PiT || !layer->ST || !layer->centroids) return TQ_ENULL;
+    FusedPrep fz;
+    fz.q = q;
+    fz.q_dtype = dtype;
+    const int words = d / PREP_COLS;
+    int hp = 8;                      // as few heads per unit as still gives every unit a workgroup of its own
+    while (hp > 1 && ((Gq + hp / 2 - 1) / (hp / 2)) * words <= n_split) hp /= 2;
+    fz.hp = hp;
+    fz.n_units = (8 / hp) * words;
+    fz.spin_limit = opt_prep_spin_limit.load();
+    fz.flags = flags;
+    fz.nonce = next_nonce();
+    const int mf = launch_decode_mfma(qa_pack, q_stat, B, Hq, Hkv * kv_div, kv_div, pool, block_table, bt_stride, seq_lens,
+                                      sm_scale, *layer, *layout, parts, n_parts, n_split, len_sub, max_pages, pool_pages,
+                                      fz, st);
+    if (mf > 0) return mf;
+    fused = mf == TQ_OK;             // TQ_EUNSUPPORTED: nothing was launched, the separate launches below run
+  }
+
+  if ((stages & 1) && !fused) {
     if (!layer->Pi || !layer->PiT || !layer->S || !layer->ST || !layer->centroids) return TQ_ENULL;
     const int n_prep = (B * Hq / Gq) * (d / PREP_COLS);
     // Whole hybrid step on the matrix-core path: the exact tail shares the preparation's launch, as long as
@@ -963,17 +1040,17 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
       tail_done = true;
     } else {
       int rc = launch_rotate_query(q, dtype, (int64_t)B * Hq, layer, q_rot, q_sk, q_stat,
-                                   mfma_shape ? qa_pack : nullptr, mfma_shape ? Gq : G, sm_scale, st);
+                                   mfma_shape ? qa_pack : nullptr, mfma_shape ? Gq : G, sm_scale, st, mfma_shape);
       if (rc) return rc;
     }
   }
   if (!(stages & 6)) return TQ_OK;
 
-  int mf = TQ_EUNSUPPORTED;
-  if (stages & 2)
+  int mf = fused ? TQ_OK : TQ_EUNSUPPORTED;
+  if ((stages & 2) && !fused)
     mf = mfma_shape ? launch_decode_mfma(qa_pack, q_stat, B, Hq, Hkv * kv_div, kv_div, pool, block_table, bt_stride,
                                          seq_lens, sm_scale, *layer, *layout, parts, n_parts, n_split, len_sub,
-                                         max_pages, pool_pages, st)
+                                         max_pages, pool_pages, FusedPrep{}, st)
                     : TQ_EUNSUPPORTED;
   if (mf > 0) return mf;
   if ((stages & 2) && mf == TQ_EUNSUPPORTED) {      // no matrix-core kernel for this shape: general kernel
@@ -1044,7 +1121,7 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   if (!(stages & 4)) return TQ_OK;
   // without a tail the merge simply reads one part fewer
   merge_kernel<<<dim3((unsigned)(B * Hq)), dim3(256), merge_smem(n_parts, d), st>>>(
-      parts, tail ? n_parts : n_split, n_parts, d, dtype, out);
+      parts, tail ? n_parts : n_split, n_parts, d, dtype, out, fused ? flags : nullptr, fused ? n_flags : 0);
   TQ_CHECK_LAUNCH();
   return TQ_OK;
 }
@@ -1121,7 +1198,8 @@ size_t decode_scratch_need(int B, int Hq, int Hkv, int n_split, const tq_layer& 
   int kv_div = 0;
   for (int n = 1; n <= G && !kv_div; ++n)
     if (G % n == 0 && G / n <= 8) kv_div = n;
-  size_t floats = parts_floats(B, Hq, d, n_split + 1) + (size_t)2 * B * Hq * d + (size_t)4 * B * Hq;
+  size_t floats = parts_floats(B, Hq, d, n_split + 1) + (size_t)2 * B * Hq * d + (size_t)4 * B * Hq +
+                  2 * flag_words(B, Hq);
   size_t words = 0;
   if (kv_div && (d == 128 || d == 256)) {
     int planes = ly.mse_bits + 1;

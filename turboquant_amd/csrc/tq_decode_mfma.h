@@ -1,0 +1,34 @@
+// Interface between the host side of the decode path (tq_decode.hip) and the matrix-core page kernel
+// (tq_decode_mfma.hip).
+#pragma once
+
+#include "tq_common.h"
+
+namespace tq {
+
+// Query preparation as a prologue of the page kernel's own launch (q == nullptr: the operands in
+// qa_pack / q_stat were prepared by an earlier launch).
+struct FusedPrep {
+  const void* q = nullptr;           // (B, Hq, d) raw queries
+  int q_dtype = 0;
+  int n_units = 0;                   // units per group of query heads (<= 64): (8 / hp) head sets x d / 32 plane words
+  int hp = 8;                        // heads per unit: 1, 2, 4 or 8
+  int spin_limit = 0;                // polls before a workgroup stops waiting for the others' units
+  unsigned long long* flags = nullptr;   // 64 words per group
+  unsigned long long nonce = 0;      // value of a published flag in this call (never 0)
+};
+
+// whether the library was built with the in-launch preparation (-DTQ_FUSED_PREP)
+bool decode_mfma_has_fused_prep();
+
+// words of packed query operands tq_decode_workspace_bytes reserves
+size_t decode_mfma_pack_words(int B, int Hq, int d);
+
+// Returns TQ_EUNSUPPORTED when the shape has no matrix-core kernel (nothing was launched); the caller then
+// uses the general vector-ALU kernel.
+int launch_decode_mfma(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, int kv_div, const uint8_t* pool,
+                       const int32_t* block_table, int bt_stride, const int32_t* seq_lens, float sm_scale,
+                       const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts, int n_split, int len_sub,
+                       int max_pages, int num_pages, const FusedPrep& fz, hipStream_t st);
+
+}  // namespace tq

@@ -49,6 +49,8 @@
 #include <hip/hip_ext.h>
 
 #include "tq_common.h"
+#include "tq_prep.h"
+#include "tq_decode_mfma.h"
 
 namespace tq {
 
@@ -59,6 +61,16 @@ typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef int i32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
 typedef int i32x8 __attribute__((ext_vector_type(8)));
+
+// The query preparation as a prologue of the page kernel's launch is compiled in with -DTQ_FUSED_PREP only:
+// it measured slower than the separate launch (see the kernel), and its mere presence costs the page
+// kernel half a microsecond.
+#ifdef TQ_FUSED_PREP
+constexpr bool fused_build = true;
+#else
+constexpr bool fused_build = false;
+#endif
+bool decode_mfma_has_fused_prep() { return fused_build; }
 
 constexpr int MF_WAVES = 4;
 constexpr int BLK_TOK = 64;              // tokens per wavefront iteration
@@ -162,10 +174,11 @@ __device__ __forceinline__ constexpr int v_bitpos(int t) {
 // channels); WPS wavefronts per SIMD the register budget is sized for.
 template <int D, int MB, int NX, int VB, int GS, int DS, int WPS, bool F16P>
 __global__ void __launch_bounds__(MF_WAVES * 64, WPS)
-decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict__ q_stat, int Hq, int Hkv, int kv_div,
+decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div,
                    const uint8_t* __restrict__ pool, const int32_t* __restrict__ block_table,
                    int bt_stride, const int32_t* __restrict__ seq_lens, float sm_scale, tq_layer ly, tq_page_layout L,
-                   float* __restrict__ parts, int n_parts, int n_split, int len_sub, int max_pages, int num_pages) {
+                   float* __restrict__ parts, int n_parts, int n_split, int len_sub, int max_pages, int num_pages,
+                   FusedPrep fz) {
   constexpr int DW = D / DS;                  // coordinates / channels of one wavefront
   constexpr int WPLT = D / 128;               // plane words per lane per plane per page, all wavefronts
   constexpr int WPL = DW / 128;               // ... of one wavefront
@@ -196,6 +209,49 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
   float* s_x_peer = (float*)smem_raw + (wave ^ 1) * WAVE_LDS_FLOATS + (4 * 16 * P_STRIDE + 16 + 4 * NG * 16);
   float* s_red = (float*)smem_raw;                          // after the loop: [NGRP][G][D + 2]
 
+  // ---------------------------------------------------------------- query preparation inside this launch
+  // fz.q != nullptr: nobody has prepared the query operands; the workgroups that share a group of query
+  // heads (the n_split workgroups of a (sequence, KV head)) do it together.  The work is cut into
+  // fz.n_units units (some heads x one plane word, prep_unit256); workgroup `split` computes units split,
+  // split + n_split, ..., writes them to qa_pack / q_stat, and publishes each under a flag that carries
+  // this call's nonce.  Then every workgroup waits until all units of its group are published.  The wait
+  // is bounded: after fz.spin_limit polls a workgroup stops waiting and computes every unit itself (the
+  // values are the same whoever computes them), so the kernel ends whatever the other workgroups do.
+  // Flags are 64-bit words that never hold a call's nonce by accident (the nonce changes with every call;
+  // the merge kernel that follows clears them, which also covers replays of a captured launch).
+#ifdef TQ_FUSED_PREP
+  if (fz.q != nullptr) {
+    float* sm = (float*)smem_raw;
+    const int words = D / PREP_COLS;
+    const int64_t grp = (int64_t)b * Hkv + h;
+    unsigned long long* gflags = fz.flags + grp * 64;
+    // first pass: this workgroup's own units, published; second pass (only after a wait that ran out): all units
+    for (bool everything = false;; everything = true) {
+      const int u0 = everything ? 0 : split, du = everything ? 1 : n_split;
+      for (int u = u0; u < fz.n_units; u += du)
+        prep_unit256<D / PREP_SLICES, true>(fz.q, fz.q_dtype, G, ly, sm_scale, q_stat, qa_pack, grp, u % words,
+                                            (u / words) * fz.hp, fz.hp, sm);
+      // The units were written with device-coherent stores; once they have completed (the barrier waits
+      // for every wavefront's outstanding stores) their flags may follow.
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+      __syncthreads();
+      if (everything) break;
+      if (tid == 0)
+        for (int u = split; u < fz.n_units; u += n_split)
+          __hip_atomic_store(gflags + u, fz.nonce, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      bool have = lane >= fz.n_units;
+      for (int spin = 0; spin < fz.spin_limit; ++spin) {
+        if (!have) have = load_coherent(gflags + lane) == fz.nonce;
+        if (__builtin_amdgcn_ballot_w64(!have) == 0) break;
+        __builtin_amdgcn_s_sleep(4);
+      }
+      if (!have) have = load_coherent(gflags + min(lane, fz.n_units - 1)) == fz.nonce;
+      if (__syncthreads_and(__builtin_amdgcn_ballot_w64(!have) == 0)) break;       // every unit of the group is there
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");      // the (device-coherent) operand loads stay below the wait
+  }
+#endif
+
   // ---------------------------------------------------------------- A operands of the score stage
   // fp6 query terms in register order (see the preparation kernel): row set 0 = terms 0, 1 of the 8
   // heads (row 2g + t), row set 1 = terms 2, 3; rows of absent heads are zero.  Six dwords per
@@ -210,9 +266,16 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
 #pragma unroll
         for (int rs = 0; rs < 2; ++rs) {
           const uint32_t* p6 = src + ((tp * WPLT + hf * WPL + i) * 2 + rs) * (64 * 8);
-          const u32x4 lo = *(const u32x4*)p6;
-          const uint32_t d4 = p6[4], d5 = p6[5];
-          qa[tp][i][rs] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)d4, (int)d5, 0, 0};
+          if (fused_build && fz.q != nullptr) {       // written by other workgroups of this launch: device-coherent loads
+            const unsigned long long* p64 = (const unsigned long long*)p6;
+            const unsigned long long x0 = load_coherent(p64), x1 = load_coherent(p64 + 1), x2 = load_coherent(p64 + 2);
+            qa[tp][i][rs] = i32x8{(int)(uint32_t)x0, (int)(x0 >> 32), (int)(uint32_t)x1, (int)(x1 >> 32),
+                                  (int)(uint32_t)x2, (int)(x2 >> 32), 0, 0};
+          } else {
+            const u32x4 lo = *(const u32x4*)p6;
+            const uint32_t d4 = p6[4], d5 = p6[5];
+            qa[tp][i][rs] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)d4, (int)d5, 0, 0};
+          }
         }
   }
   // E8M0 block-scale codes of this lane's operand row (head n / 2), one per byte: index planes row
@@ -222,7 +285,9 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
   {
     const int g = n >> 1;
     const int64_t qrow = (int64_t)b * Hq + h * G + (g < G ? g : 0);
-    const int e1 = 127 + (int)q_stat[qrow * 4 + 0], e2 = 127 + (int)q_stat[qrow * 4 + 1];
+    const bool coh = fused_build && fz.q != nullptr;
+    const int e1 = 127 + (int)(coh ? load_coherent(q_stat + qrow * 4 + 0) : q_stat[qrow * 4 + 0]);
+    const int e2 = 127 + (int)(coh ? load_coherent(q_stat + qrow * 4 + 1) : q_stat[qrow * 4 + 1]);
     const int t01 = (n & 1) ? 7 : 2, t23 = t01 + 10;
     sa = (e1 - t01) | ((e1 - t23) << 8) | ((e2 - t01) << 16) | ((e2 - t23) << 24);
   }
@@ -238,8 +303,11 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
       const int g = 2 * kb + j;
       const bool live = g < G && hf == 0;
       const int64_t qrow = (int64_t)b * Hq + h * G + (g < G ? g : 0);
-      cm[2 * j] = live ? q_stat[qrow * 4 + 2] : 0.0f;
-      cq[2 * j] = live ? q_stat[qrow * 4 + 3] : 0.0f;
+      const bool coh = fused_build && fz.q != nullptr;
+      const float c2 = coh ? load_coherent(q_stat + qrow * 4 + 2) : q_stat[qrow * 4 + 2];
+      const float c3 = coh ? load_coherent(q_stat + qrow * 4 + 3) : q_stat[qrow * 4 + 3];
+      cm[2 * j] = live ? c2 : 0.0f;
+      cq[2 * j] = live ? c3 : 0.0f;
     }
     int seen = 0;
     for (int t = 0; t < ly.n_terms; ++t) {
@@ -592,6 +660,7 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
     // workgroup's blocks (a lane per entry; requested first, used after the first block's loads are on
     // their way).  Only a workgroup that finds an entry outside the pool runs the checking loop.
     bool entry_bad = false;
+#ifndef TQ_EXP_NO_TABLE_SCAN
     {
       const int e0 = 4 * blk_begin, e1 = min(4 * blk_end, n_pages);
       for (int e = e0 + lane; e < e1; e += 4 * 64) {
@@ -599,6 +668,7 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
         for (int i = 0; i < 4; ++i) entry_bad |= (unsigned)bt[min(e + 64 * i, e1 - 1)] >= (unsigned)num_pages;
       }
     }
+#endif
     int bad = 0;                                          // pages of the current block that lie outside the pool
     if (blk < blk_end) {
       bad = page_ids(blk, pid, std::true_type{});
@@ -719,14 +789,18 @@ decode_mfma_kernel(const uint32_t* __restrict__ qa_pack, const float* __restrict
 static thread_local hipEvent_t t_start_event = nullptr, t_stop_event = nullptr;
 
 template <int D, int MB, int NX, int VB, int GS, int DS, int WPS, bool F16P>
-static int launch_one(const uint32_t* qa_pack, const float* q_stat, int B, int Hq, int Hkv, int kv_div,
+static int launch_one(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, int kv_div,
                       const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
                       float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts, int n_split,
-                      int len_sub, int max_pages, int num_pages, hipStream_t st) {
+                      int len_sub, int max_pages, int num_pages, const FusedPrep& fz, hipStream_t st) {
   const int G = Hq / Hkv;
   size_t per_wave = (size_t)wave_lds_floats(D / DS / GS, DS) * sizeof(float);
   size_t merge = (size_t)(MF_WAVES / DS * G * (D + 2) + MF_WAVES * 16 * 16) * sizeof(float);
   size_t smem = per_wave * MF_WAVES > merge ? per_wave * MF_WAVES : merge;
+  if (fz.q) {
+    const size_t prep = (size_t)prep_unit_smem_floats(fz.hp, D) * sizeof(float);
+    if (prep > smem) smem = prep;
+  }
   auto kern = decode_mfma_kernel<D, MB, NX, VB, GS, DS, WPS, F16P>;
   if (smem > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
@@ -735,12 +809,12 @@ static int launch_one(const uint32_t* qa_pack, const float* q_stat, int B, int H
   if (t_start_event || t_stop_event) {
     hipExtLaunchKernelGGL(kern, dim3(n_split, Hkv, B), dim3(MF_WAVES * 64), smem, st, t_start_event, t_stop_event, 0,
                           qa_pack, q_stat, Hq, Hkv, kv_div, pool, block_table, bt_stride, seq_lens, sm_scale, ly, L, parts,
-                          n_parts, n_split, len_sub, max_pages, num_pages);
+                          n_parts, n_split, len_sub, max_pages, num_pages, fz);
     t_start_event = t_stop_event = nullptr;
   } else {
     kern<<<dim3(n_split, Hkv, B), dim3(MF_WAVES * 64), smem, st>>>(qa_pack, q_stat, Hq, Hkv, kv_div, pool, block_table,
                                                                    bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts,
-                                                                   n_split, len_sub, max_pages, num_pages);
+                                                                   n_split, len_sub, max_pages, num_pages, fz);
   }
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? TQ_OK : (int)e;
@@ -751,10 +825,10 @@ static int launch_one(const uint32_t* qa_pack, const float* q_stat, int B, int H
 // words of packed query operands tq_decode_attn_paged reserves in its workspace
 size_t decode_mfma_pack_words(int B, int Hq, int d) { return (size_t)B * Hq * 9 * (d / 128 + 1) * 1024; }
 
-int launch_decode_mfma(const uint32_t* qa_pack, const float* q_stat, int B, int Hq, int Hkv, int kv_div,
+int launch_decode_mfma(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, int kv_div,
                        const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
                        float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts,
-                       int n_split, int len_sub, int max_pages, int num_pages, hipStream_t st) {
+                       int n_split, int len_sub, int max_pages, int num_pages, const FusedPrep& fz, hipStream_t st) {
   const int G = Hq / Hkv, d = ly.d, mb = ly.mse_bits, vb = L.value_bits, gs = L.group_size;
   if (G > 8 || (L.dtype != TQ_BF16 && L.dtype != TQ_F16) || !L.key_lane_major) return TQ_EUNSUPPORTED;
   const bool f16p = L.dtype == TQ_F16;
@@ -766,10 +840,10 @@ int launch_decode_mfma(const uint32_t* qa_pack, const float* q_stat, int B, int 
     if (f16p)                                                                                                   \
       return launch_one<D_, MB_, NX_, VB_, GS_, DS_, WPS_, true>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,  \
                                                                  bt_stride, seq_lens, sm_scale, ly, L, parts,     \
-                                                                 n_parts, n_split, len_sub, max_pages, num_pages, st); \
+                                                                 n_parts, n_split, len_sub, max_pages, num_pages, fz, st); \
     return launch_one<D_, MB_, NX_, VB_, GS_, DS_, WPS_, false>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,   \
                                                                 bt_stride, seq_lens, sm_scale, ly, L, parts,      \
-                                                                n_parts, n_split, len_sub, max_pages, num_pages, st); \
+                                                                n_parts, n_split, len_sub, max_pages, num_pages, fz, st); \
   }
   TQ_TRY(128, 2, 0, 2, 32, 1, 2) TQ_TRY(128, 2, 0, 4, 32, 1, 2) TQ_TRY(256, 2, 0, 2, 32, 2, 2) TQ_TRY(256, 2, 0, 4, 32, 2, 2)
   TQ_TRY(128, 1, 0, 2, 32, 1, 2) TQ_TRY(128, 1, 0, 4, 32, 1, 2) TQ_TRY(256, 1, 0, 2, 32, 2, 2) TQ_TRY(256, 1, 0, 4, 32, 2, 2)

@@ -1,0 +1,10 @@
+// Process-wide knobs set through tq_set_option (defined in tq_decode.hip).
+#pragma once
+
+#include <atomic>
+
+namespace tq {
+extern std::atomic<int> opt_fuse_prep;         // query preparation inside the page kernel's launch
+extern std::atomic<int> opt_prep_spin_limit;   // polls before a workgroup of that launch stops waiting for the others
+extern std::atomic<int> opt_prep_units;        // stand-alone preparation: one workgroup per (few heads, plane word) unit
+}  // namespace tq

@@ -3,6 +3,7 @@
 
 #include "tq_common.h"
 #include "tq_prep.h"
+#include "tq_options.h"
 
 namespace tq {
 
@@ -75,6 +76,18 @@ prep_query_kernel(const void* __restrict__ q, int G, tq_layer ly, float sm_scale
                   uint32_t* __restrict__ qa_pack) {
   extern __shared__ float sm[];
   prep_query_body<PER, DT>(q, G, ly, sm_scale, q_rot, q_sk, q_stat, qa_pack, blockIdx.x, blockIdx.y, sm);
+}
+
+// The same preparation cut into more, smaller workgroups: one per unit = (hp consecutive heads of a group,
+// plane word), 256 threads (prep_unit256).  The launch is latency-bound, and a unit of one or two heads has
+// a shorter dependent chain than one workgroup per plane word doing all eight heads.
+template <int PER>
+__global__ void __launch_bounds__(PREP_UNIT_THREADS)
+prep_units_kernel(const void* __restrict__ q, int dtype, int G, tq_layer ly, float sm_scale, float* __restrict__ q_stat,
+                  uint32_t* __restrict__ qa_pack, int hp) {
+  extern __shared__ float sm[];
+  const int words = ly.d / PREP_COLS, u = blockIdx.x;
+  prep_unit256<PER, false>(q, dtype, G, ly, sm_scale, q_stat, qa_pack, blockIdx.y, u % words, (u / words) * hp, hp, sm);
 }
 
 // scores[b, i, k] for a tile of QT queries and one key per thread.  The rotated and sketched queries sit
@@ -351,12 +364,28 @@ namespace tq {
 int launch_dequant_mfma(const uint8_t* idx, const uint8_t* signs, const void* norms, int norm_dtype, const float* rnorms,
                         int64_t n_vec, const tq_layer& ly, float* out, hipStream_t st);
 
+// q_rot_unused: the caller only needs the packed operands and statistics (the page kernel on the matrix
+// cores), not the fp32 rotated / sketched queries
 int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* layer, float* q_rot, float* q_sk,
-                        float* q_stat, uint32_t* qa_pack, int G, float sm_scale, hipStream_t st) {
+                        float* q_stat, uint32_t* qa_pack, int G, float sm_scale, hipStream_t st, bool q_rot_unused) {
   const int d = layer->d;
   if (qa_pack) {       // operands of the matrix-core decode kernel wanted
     if (!q_stat || !layer->Pi_colsum || !layer->S_colsum || G > ROT_MAX_ROWS || rows % G || (d != 128 && d != 256))
       return TQ_EUNSUPPORTED;
+    if (opt_prep_units.load() && q_rot_unused) {
+      // heads per unit: as few as keep the launch at about a thousand workgroups
+      const int64_t groups = rows / G;
+      const int words = d / PREP_COLS;
+      int hp = 1;
+      while (hp < 8 && groups * ((G + hp - 1) / hp) * words > 1024) hp *= 2;
+      const dim3 ugrid((unsigned)((8 / hp) * words), (unsigned)groups);
+      const size_t usm = (size_t)prep_unit_smem_floats(hp, d) * sizeof(float);
+      if (groups > 65535) return TQ_EUNSUPPORTED;
+      if (d == 128) prep_units_kernel<8><<<ugrid, dim3(PREP_UNIT_THREADS), usm, st>>>(q, dtype, G, *layer, sm_scale, q_stat, qa_pack, hp);
+      else prep_units_kernel<16><<<ugrid, dim3(PREP_UNIT_THREADS), usm, st>>>(q, dtype, G, *layer, sm_scale, q_stat, qa_pack, hp);
+      hipError_t e = hipGetLastError();
+      return e == hipSuccess ? TQ_OK : (int)e;
+    }
     size_t smem = prep_smem_bytes(G, d);
     const dim3 grid((unsigned)(rows / G), d / PREP_COLS), block(PREP_COLS * PREP_SLICES);
 #define TQ_PREP(PER, DT) prep_query_kernel<PER, DT><<<grid, block, smem, st>>>(q, G, *layer, sm_scale, q_rot, q_sk, q_stat, qa_pack)
@@ -392,7 +421,7 @@ extern "C" int tq_rotate_query(const void* q, int dtype, int64_t rows, const tq_
   if (!q || !q_rot || !q_sk) return TQ_ENULL;
   if (rows < 0 || dtype < TQ_F32 || dtype > TQ_BF16) return TQ_EINVAL;
   if (rows == 0) return TQ_OK;
-  return launch_rotate_query(q, dtype, rows, layer, q_rot, q_sk, nullptr, nullptr, 1, 0.0f, (hipStream_t)stream);
+  return launch_rotate_query(q, dtype, rows, layer, q_rot, q_sk, nullptr, nullptr, 1, 0.0f, (hipStream_t)stream, false);
 }
 
 extern "C" int tq_score(const void* q, int dtype, int64_t batch, int64_t n_q, const uint8_t* idx, const uint8_t* signs,
