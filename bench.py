@@ -17,14 +17,19 @@ The same JSON line carries
   roofline     : the page-streaming kernel alone (hipEvents around that stage),
                  algorithmic bytes / its mean duration, against 8 TB/s;
   quantize     : tokens/s of the fused paged quantise call on the prefill
-                 configuration (32 768 tokens x 8 KV heads, head_dim 128);
-  decode_gqa   : the 16 x 8192-token GQA decode configuration;
+                 configuration (32 768 tokens x 8 KV heads, head_dim 128), with the
+                 paged key kernel's own time against the bf16 matrix peak and
+                 the whole append against the HBM peak;
+  decode_gqa   : the 16 x 8192-token GQA decode configuration (and the same with
+                 4-bit keys, the reference's default for the first four layers);
+  round_trip   : the 4096-key x 32-query round trip (quantise + all scores);
   backend_decode_step : a full decode step of a random-init 32-layer dense
                  transformer (batch 32 x 32 768 context) whose attention layers run
                  through the batch-aware backend hooks on compressed KV;
   cpu_baseline : the CPU oracle's de-quantise-everything attention (the
                  reference's production read path) timed on the host cores on
-                 one of the four sequences.
+                 one of the four sequences; every sequence's GPU output is checked
+                 against it (cosine).
 """
 
 from __future__ import annotations
@@ -43,13 +48,14 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 
 
-def student_t(shape, nu, gen, device):
+def student_t(shape, nu, gen):
+    """z / sqrt(chi2_nu / nu) element-wise on the CPU generator, chi2 as the sum of nu squared normals."""
     import torch
-    z = torch.randn(*shape, generator=gen, device=device)
-    chi = torch.zeros(shape, device=device)
+    z = torch.randn(*shape, generator=gen)
+    chi = torch.zeros(shape)
     for _ in range(nu):
-        chi += torch.randn(*shape, generator=gen, device=device) ** 2
-    return z / torch.sqrt(chi / nu)
+        chi.add_(torch.randn(*shape, generator=gen).square_())
+    return z.div_(chi.div_(nu).sqrt_())
 
 
 def algorithmic_bytes_per_token_head(d, mse_bits, value_bits, group):
@@ -66,26 +72,26 @@ class DecodeWorkload:
         from turboquant_amd.quantizer import TurboQuantProd
         self.name, self.B, self.N, self.Hq, self.Hkv, self.d = name, B, N, Hq, Hkv, d
         self.key_bits, self.value_bits = key_bits, value_bits
-        gen = torch.Generator(device=device).manual_seed(seed)
+        gen = torch.Generator().manual_seed(seed)            # a CPU generator: the same data on every machine
         self.tq = TurboQuantProd(d, bits=key_bits, device=device)
         pages_per_seq = (N + 15) // 16
         n_pages = B * pages_per_seq
         self.pools = []
-        perm = torch.randperm(n_pages, generator=gen, device=device).to(torch.int32)
+        perm = torch.randperm(n_pages, generator=gen).to(torch.int32).to(device)
         self.table = perm.reshape(B, pages_per_seq).contiguous()
         first = PagedKVPool(self.tq, Hkv, n_pages, value_bits=value_bits, value_group_size=32,
                             dtype=torch.bfloat16, device=device)
-        chunk = 16384
+        chunk = 32768
         for b in range(B):                      # sequence by sequence, in chunks, to bound the bf16 staging memory
             for t0 in range(0, N, chunk):
                 t1 = min(N, t0 + chunk)
                 shape = (1, t1 - t0, Hkv, d)
                 if dist == "student_t5":
-                    k, v = student_t(shape, 5, gen, device), student_t(shape, 5, gen, device)
+                    k, v = student_t(shape, 5, gen), student_t(shape, 5, gen)
                 else:
-                    k = torch.randn(*shape, generator=gen, device=device)
-                    v = torch.randn(*shape, generator=gen, device=device)
-                first.append(k.bfloat16(), v.bfloat16(), self.table[b:b + 1],
+                    k = torch.randn(*shape, generator=gen)
+                    v = torch.randn(*shape, generator=gen)
+                first.append(k.bfloat16().to(device), v.bfloat16().to(device), self.table[b:b + 1],
                              torch.tensor([t0], dtype=torch.int32, device=device))
         self.pools.append(first)
         for _ in range(n_pools - 1):
@@ -93,7 +99,7 @@ class DecodeWorkload:
                             dtype=torch.bfloat16, device=device)
             p.data.copy_(first.data)
             self.pools.append(p)
-        self.q = torch.randn(B, Hq, d, generator=gen, device=device).bfloat16()
+        self.q = torch.randn(B, Hq, d, generator=gen).bfloat16().to(device)
         self.seq = torch.full((B,), N, dtype=torch.int32, device=device)
         self.n_split = first.default_splits(B, N, Hq)
         self.ws = first.workspace(B, Hq, self.n_split)
@@ -123,7 +129,10 @@ def hybrid_step_bench(work, steps, warmup, ring=128):
                                    workspace=work.ws, out=work.out, max_len=work.N)
     ms, _ = time_steps(step, steps, warmup)
     del cache
-    return {"exact_tokens": ring, "ms_per_step": ms}
+    per_tok = algorithmic_bytes_per_token_head(work.d, work.key_bits - 1, work.value_bits, 32)
+    nbytes = work.B * work.Hkv * ((work.N - ring) * per_tok + ring * 2 * work.d * 2)     # pages + exact bf16 K and V rows
+    return {"exact_tokens": ring, "ms_per_step": ms, "bytes_per_step": nbytes, "GBps": nbytes / (ms * 1e-3) / 1e9,
+            "pct_hbm_peak": 100.0 * nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
 
 
 RAMP_SECONDS = 0.25      # --ramp-seconds
@@ -212,30 +221,62 @@ def stream_read_peak(work, steps, warmup):
     return best
 
 
-def cpu_decode_baseline(work):
-    """The oracle's de-quantise-all + dense attention on one sequence of the
-    workload, on the host cores."""
+def cpu_decode_baseline(work, n_seq=None, runs=3):
+    """The oracle's de-quantise-all + dense attention (the reference's production read path, score.py:84-173)
+    on the host cores: every sequence of the workload once (so that the GPU result of every sequence is
+    checked), the first one `runs` times for the timing."""
     import torch
     from oracle import tq_oracle as O
     from tests.helpers import key_code, value_code, params_of
     pool = work.pools[0]
-    idx, sgn, norms, rn, vd, vs, vz = [t.cpu() for t in pool.export_flat(work.table[0], work.N)]
-    kc = key_code(idx, sgn, rn, norms, work.key_bits - 1)
-    vc = value_code(vd, vs, vz, work.value_bits)
     prm = params_of(work.tq)
-    q = work.q[:1].cpu()
-    times = []
-    out = None
-    for _ in range(5):
-        t0 = time.perf_counter()
-        out = O.hybrid_attention(q, kc, vc, work.N, prm, work.Hkv, None, None)
-        times.append(time.perf_counter() - t0)
+    n_seq = work.B if n_seq is None else n_seq
+    work.step(0)
+    torch.cuda.synchronize()
+    gpu_out = work.out.float().cpu()
+    times, cosines = [], []
+    for b in range(n_seq):
+        idx, sgn, norms, rn, vd, vs, vz = [t.cpu() for t in pool.export_flat(work.table[b], work.N)]
+        kc = key_code(idx, sgn, rn, norms, work.key_bits - 1)
+        vc = value_code(vd, vs, vz, work.value_bits)
+        q = work.q[b:b + 1].cpu()
+        for _ in range(runs if b == 0 else 1):
+            t0 = time.perf_counter()
+            out = O.hybrid_attention(q, kc, vc, work.N, prm, work.Hkv, None, None)
+            if b == 0:
+                times.append(time.perf_counter() - t0)
+        got, want = gpu_out[b].flatten(), out.float().flatten()
+        cosines.append(float((got @ want) / (got.norm() * want.norm())))
     sec = sorted(times)[len(times) // 2]
     sample_bytes = work.bytes // work.B
-    return out, {"value": sample_bytes / sec / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(),
-                 "kind": "port", "seconds": sec,
-                 "sample": f"1 of {work.B} sequences ({work.N} tokens x {work.Hkv} KV heads), median of 5 runs, "
-                           f"full-job time = x{work.B}"}
+    return {"value": sample_bytes / sec / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(),
+            "kind": "port", "seconds": sec,
+            "sample": f"1 of {work.B} sequences ({work.N} tokens x {work.Hkv} KV heads), median of {runs} runs, "
+                      f"full-job time = x{work.B}",
+            "gpu_vs_oracle_cosine": min(cosines), "gpu_vs_oracle_cosine_per_sequence": cosines,
+            "sequences_checked": n_seq}
+
+
+def time_key_kernel(step, steps, warmup):
+    """Mean execution time of the paged matrix-core key-quantise kernel alone, inside whole appends (the
+    library attaches a HIP event pair to that kernel's own dispatch, tq_time_next_key_kernel)."""
+    import torch
+    from turboquant_amd import _ffi
+    lib = _ffi.lib()
+    evs = []
+    for _ in range(steps):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record(); b.record()
+        evs.append((a, b))
+    torch.cuda.synchronize()
+    clock_ramp(step, warmup + steps)
+    for i in range(warmup):
+        step(i)
+    for i, (a, b) in enumerate(evs):
+        lib.tq_time_next_key_kernel(a.cuda_event, b.cuda_event)
+        step(warmup + i)
+    torch.cuda.synchronize()
+    return sum(a.elapsed_time(b) for a, b in evs) / steps
 
 
 def quantize_bench(device, steps, warmup):
@@ -255,23 +296,70 @@ def quantize_bench(device, steps, warmup):
     pool = PagedKVPool(tq, H, T // 16, value_bits=2, value_group_size=32, dtype=torch.bfloat16, device=device)
     table = torch.arange(T // 16, dtype=torch.int32, device=device)[None]
     ms, _ = time_steps(lambda i: pool.append(k, v, table), steps, warmup)
-    # the key kernel alone (same kernel body, flat output): its three d x d contractions are the
-    # matrix-core part of the path
-    kflat = k.reshape(-1, d)
-    key_ms, _ = time_steps(lambda i: tq.quantize(kflat), steps, warmup)
+    # the paged key kernel alone, timed inside whole appends: its three d x d contractions are the
+    # matrix-core part of the path.  The kernel issues them as 15 exact bf16 term products (5 per
+    # contraction instead of one fp32 product), so the matrix-core work it issues is 5 x the algorithmic FLOP,
+    # and the roofline that bounds it is the bf16 matrix peak.
+    key_ms = time_key_kernel(lambda i: pool.append(k, v, table), steps, warmup)
     flops = 3 * 2 * d * d * T * H
+    issued = 5 * flops / (key_ms * 1e-3) / 1e12
+    nbytes = T * (2 * H * d * 2 + H * 100)
     return {"tokens_per_s": T / (ms * 1e-3), "ms": ms, "tokens": T, "kv_heads": H, "head_dim": d,
             "workload": "prefill quantize, 32768 tok x 8 KV heads, d=128, 3b keys + 2b values, pages of 16",
-            "hbm_gbs": (T * (2 * H * d * 2 + H * 100)) / (ms * 1e-3) / 1e9,
-            "roofline": {"bound": "mfma", "kernel": "key_mfma_kernel", "kernel_ms": key_ms,
-                         "achieved": flops / (key_ms * 1e-3) / 1e12, "peak": 157.3, "unit": "TFLOP/s",
-                         "frac": flops / (key_ms * 1e-3) / 1e12 / 157.3,
-                         "mfma_issued": 5 * flops / (key_ms * 1e-3) / 1e12, "mfma_issued_peak": 2500.0,
-                         "mfma_issued_frac": 5 * flops / (key_ms * 1e-3) / 1e12 / 2500.0,
-                         "note": "achieved = algorithmic FLOP (3 contractions x 2 d^2 per vector, fp32 accuracy) "
-                                 "against the fp32 matrix peak; it can pass 1 because the kernel issues the work as "
-                                 "15 exact bf16 MFMA term products: mfma_issued is that bf16 work in TFLOP/s "
-                                 "against the 2500 TFLOP/s bf16 peak"}}, (pool, k, v, table, tq)
+            "hbm_gbs": nbytes / (ms * 1e-3) / 1e9, "hbm_bytes": nbytes,
+            "hbm_frac": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "roofline": {"bound": "mfma", "kernel": "key_mfma_kernel (paged sink)", "kernel_ms": key_ms,
+                         "achieved": issued, "peak": 2500.0, "unit": "TFLOP/s", "frac": issued / 2500.0,
+                         "algorithmic_tflops": flops / (key_ms * 1e-3) / 1e12,
+                         "note": "achieved = bf16 matrix-core work the kernel issues (15 exact bf16 term products for "
+                                 "the 3 fp32-accurate d x d contractions per vector = 5 x the algorithmic 6 d^2 FLOP) "
+                                 "against the 2500 TFLOP/s bf16 peak; algorithmic_tflops is the 6 d^2 figure"}}, (pool, k, v, table, tq)
+
+
+def round_trip_bench(device, steps, warmup, with_cpu):
+    """The CPU-runnable round trip (4096 keys x 128, 32 queries, 3-bit keys, seed 0): quantise the keys and
+    estimate all 32 x 4096 inner products, on the GPU and (oracle) on the host cores."""
+    import torch
+    from turboquant_amd.quantizer import TurboQuantProd
+    g = torch.Generator().manual_seed(0)
+    K = torch.randn(4096, 128, generator=g)
+    K = K / K.norm(dim=-1, keepdim=True) * (0.5 + 1.5 * torch.rand(4096, generator=g)).unsqueeze(-1)
+    Q = torch.randn(32, 128, generator=g)
+    Q = Q / Q.norm(dim=-1, keepdim=True) * (0.5 + 1.5 * torch.rand(32, generator=g)).unsqueeze(-1)
+    tq = TurboQuantProd(128, bits=3, device=device)
+    Kd, Qd = K.to(device), Q.to(device)
+
+    def step(i):
+        code = tq.quantize(Kd)
+        return tq.attention_score(Qd, code)
+    ms, _ = time_steps(step, steps, warmup)
+    out = {"workload": "4096 keys x 128 fp32, 32 queries, 3-bit keys: quantise + all 32 x 4096 estimates",
+           "ms": ms, "keys_per_s": 4096 / (ms * 1e-3)}
+    if with_cpu:
+        from oracle import tq_oracle as O
+        from tests.helpers import params_of
+        prm = params_of(tq)
+        times = []
+        for _ in range(5):
+            t0 = time.perf_counter()
+            code = O.prod_quantize(K, prm)
+            ref = O.attention_score(Q, code, prm)
+            times.append(time.perf_counter() - t0)
+        sec = sorted(times)[2]
+        out["cpu_baseline"] = {"seconds": sec, "keys_per_s": 4096 / sec, "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": "the whole workload, median of 5 runs"}
+        # end to end the GPU quantiser may flip a coordinate that sits on a threshold (fp32 summation order);
+        # the score gate itself is taken on identical bytes in the tests
+        gcode = tq.quantize(Kd)
+        got = tq.attention_score(Qd, gcode)
+        torch.cuda.synchronize()
+        out["index_bytes_differing"] = int((gcode.mse_indices.cpu() != code.mse_indices).sum())
+        out["sign_bytes_differing"] = int((gcode.qjl_signs.cpu() != code.qjl_signs).sum())
+        rms = float(ref.pow(2).mean().sqrt())
+        same = (gcode.mse_indices.cpu() == code.mse_indices).all(dim=-1) & (gcode.qjl_signs.cpu() == code.qjl_signs).all(dim=-1)
+        diff = (got.float().cpu() - ref).abs()
+        out["scores_max_abs_over_rms_on_keys_with_identical_bytes"] = float(diff[:, same].max()) / rms
+    return out
 
 
 def backend_step_bench(device, steps, warmup, n_layers=32, batch=32, context=32768):
@@ -388,21 +476,40 @@ def main():
 
     hybrid_main = hybrid_step_bench(main_w, max(20, args.steps // 4), max(5, args.warmup // 5))
 
-    traffic = None
+    traffic, traffic_source = None, None
     tpath = os.path.join(ROOT, "profiles", "decode_pages_traffic.json")
     if os.path.exists(tpath):
         with open(tpath) as f:
             t = json.load(f)
         if t.get("context") == args.context:
             traffic = t.get("hbm_bytes_per_launch")
+            traffic_source = ("stored profile figure, not measured in this run: profiles/decode_pages_traffic.json "
+                              "(rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command, scaled by a copy kernel)")
 
     gqa_w = DecodeWorkload("gqa decode", 16, 8192, 32, 8, 128, 3, 4, n_pools=4, seed=2, dist="normal", device=device)
     gqa_ms, _ = time_steps(gqa_w.step, args.steps, args.warmup)
     gqa_kern = time_kernel_stage(gqa_w, args.steps, args.warmup)
-
     hybrid_gqa = hybrid_step_bench(gqa_w, max(20, args.steps // 4), max(5, args.warmup // 5))
+    gqa_cpu = None
+    if not args.no_cpu:
+        gqa_cpu = cpu_decode_baseline(gqa_w, runs=3)
+
+    # the same shape with 4-bit keys (3-bit indices in nibbles + sign plane): the reference's default for the
+    # first four layers (integration/vllm.py:358-359)
+    kb4_w = DecodeWorkload("gqa decode, 4-bit keys", 16, 8192, 32, 8, 128, 4, 4, n_pools=4, seed=2, dist="normal",
+                           device=device)
+    kb4_ms, _ = time_steps(kb4_w.step, args.steps, args.warmup)
+    kb4_kern = time_kernel_stage(kb4_w, args.steps, args.warmup)
+    kb4 = {"workload": "16 seq x 8192 ctx, 32 q heads / 8 KV heads, head_dim 128, keys 4b, values 4b",
+           "bytes_per_step": kb4_w.bytes, "GBps": kb4_w.bytes / (kb4_ms * 1e-3) / 1e9, "ms_per_step": kb4_ms,
+           "pct_hbm_peak": 100.0 * kb4_w.bytes / (kb4_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+           "kernel_ms": kb4_kern, "kernel_GBps": kb4_w.bytes / (kb4_kern * 1e-3) / 1e9,
+           "kernel_frac": kb4_w.bytes / (kb4_kern * 1e-3) / 1e9 / HBM_PEAK_GBS}
+    del kb4_w
+    torch.cuda.empty_cache()
 
     quant, (qpool, qk, qv, qtable, qtq) = quantize_bench(device, max(5, args.steps // 5), max(2, args.warmup // 5))
+    round_trip = round_trip_bench(device, max(5, args.steps // 5), max(2, args.warmup // 5), not args.no_cpu)
 
     backend = None
     if not args.no_backend_step:
@@ -414,36 +521,39 @@ def main():
 
     cpu = None
     if not args.no_cpu:
-        ref_out, cpu = cpu_decode_baseline(main_w)
-        main_w.step(0)
-        torch.cuda.synchronize()
-        got = main_w.out[:1].float().cpu().flatten()
-        want = ref_out.float().flatten()
-        cpu["gpu_vs_oracle_cosine"] = float((got @ want) / (got.norm() * want.norm()))
+        cpu = cpu_decode_baseline(main_w, runs=3)
         quant["cpu_baseline"] = cpu_quantize_baseline(qk, qv, qtq)
 
     line = {
         "metric": "compressed-KV decode attn GB/s (% HBM peak) + quantize tokens/s, 1 GPU",
         "value": value, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "u8 codes, fp32 accumulate", "data": "synthetic (seeded GPU generator; Student-t nu=5 K/V, bf16)",
+        "dtype": "u8 packed codes; scores: 4-term fp6 (e2m3) query x fp4 bit planes on the matrix cores, fp32 accumulate; "
+                 "values: bf16-rounded weight x scale operands x exact bf16-denormal codes on the matrix cores, "
+                 "fp32 accumulate; softmax fp32",
+        "data": "synthetic (CPU generator seed 3; Student-t nu=5 K/V, N(0,1) queries, bf16; pages in a random permutation)",
         "config": {"workload": f"long-context decode: 4 seq x {args.context} ctx, 16 q heads / 2 KV heads, head_dim 256, "
                                "keys 3b (2b Lloyd-Max + 1b QJL, m=256), values 2b group 32, pages of 16, bf16 query",
                    "algorithmic_bytes_per_step": main_w.bytes, "stored_bytes_per_step": main_w.stored_bytes,
-                   "n_split": main_w.n_split, "kv_pools_rotated": len(main_w.pools)},
+                   "n_split": main_w.n_split, "kv_pools_rotated": len(main_w.pools),
+                   "launches_per_step": 3},
         "pct_hbm_peak": 100.0 * value / HBM_PEAK_GBS,
         "wall_ms_per_step": wall, "clock_ramp_s": RAMP_SECONDS,
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic, "kernel": "decode_mfma_kernel",
-                     "kernel_ms": kern_ms, "stream_read": stream,
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic, "traffic_source": traffic_source,
+                     "kernel": "decode_mfma_kernel", "kernel_ms": kern_ms, "stream_read": stream,
                      "frac_of_stream_read": achieved / stream["GBps"]},
         "quantize": quant,
+        "round_trip": round_trip,
         "decode_gqa": {"workload": "16 seq x 8192 ctx, 32 q heads / 8 KV heads, head_dim 128, keys 3b, values 4b",
-                       "GBps": gqa_w.bytes / (gqa_ms * 1e-3) / 1e9, "ms_per_step": gqa_ms,
-                       "kernel_GBps": gqa_w.bytes / (gqa_kern * 1e-3) / 1e9,
-                       "pct_hbm_peak": 100.0 * gqa_w.bytes / (gqa_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
+                       "bytes_per_step": gqa_w.bytes, "GBps": gqa_w.bytes / (gqa_ms * 1e-3) / 1e9, "ms_per_step": gqa_ms,
+                       "kernel_ms": gqa_kern, "kernel_GBps": gqa_w.bytes / (gqa_kern * 1e-3) / 1e9,
+                       "kernel_frac": gqa_w.bytes / (gqa_kern * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                       "pct_hbm_peak": 100.0 * gqa_w.bytes / (gqa_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                       "cpu_baseline": gqa_cpu},
+        "decode_gqa_kb4": kb4,
         "decode_hybrid": {"note": "whole step with the newest 128 tokens exact, read in place from a paged bf16 cache "
-                                  "(tq_decode_attn_paged_ring); compare ms_per_step of the compressed-only steps",
+                                  "(tq_decode_attn_paged_ring); bytes = pages of the older tokens + the exact rows",
                           "long_context": hybrid_main, "gqa": hybrid_gqa},
         "backend_decode_step": backend,
         "cpu_baseline": cpu,

@@ -108,7 +108,7 @@ int tq_version(void);
 int tq_layer_fill_terms(tq_layer *layer /*host*/, const float *centroids_host);
 
 /* Host helper: computes the page geometry for inputs of `dtype`;
- * value_bits 2 or 4, d a multiple of 64 and of group_size (>= 16).                     */
+ * value_bits 2, 4 or 8, d a multiple of 64 and of group_size (>= 16).                  */
 int tq_page_layout_init(tq_page_layout *out /*host*/, int d, int mse_bits, int value_bits,
                         int group_size, int dtype);
 
@@ -296,6 +296,11 @@ int tq_decode_merge(const float *parts, int64_t rows, int n_parts, int d, int dt
  * time alone - what a profiler's kernel trace reports - and not the interval between two markers in the
  * stream, which also contains the dispatch gap.  Pass NULLs to disarm.                             */
 void tq_time_next_page_kernel(void *start_event, void *stop_event);
+
+/* The same for the next matrix-core key-quantise kernel that tq_append_kv_paged and its siblings launch from
+ * this thread (head_dim 128 / 256, 16-byte aligned inputs): its execution time alone, without the value
+ * kernel that runs beside it.                                                                        */
+void tq_time_next_key_kernel(void *start_event, void *stop_event);
 
 /* Tuning and test knobs (no counterpart in the reference); process-wide, take effect at the next call.
  *   "prep_units"       0 (default): the query preparation of the matrix-core decode path runs as one workgroup

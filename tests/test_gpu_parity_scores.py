@@ -352,3 +352,66 @@ def test_decode_step_with_the_preparation_inside_the_page_kernel(gpu, d, key_bit
         kc, vc = _store_from_oracle_view(pool, table[b], lens[b])
         want = O.hybrid_attention(q[b:b + 1], kc, vc, max(lens[b], O.MIN_HISTORY), prm, Hkv, None, None)
         assert cosine(out[b:b + 1], want) >= COS_GATE, b
+
+
+# ------------------------------------------------------------------ 8-bit values in the paged store
+@pytest.mark.parametrize("d,key_bits,dtype,gs", [(128, 3, torch.bfloat16, 32), (256, 3, torch.float16, 32),
+                                                 (64, 4, torch.float32, 32), (128, 3, torch.bfloat16, 64)])
+def test_eight_bit_values_in_pages(gpu, golden, d, key_bits, dtype, gs):
+    """quantize_values(bits=8) (kv_cache.py:89-98: one code per byte) through the paged store: the exported flat
+    tensors equal the flat quantiser's (which is bit-exact against the reference's *_b8_* vectors), and decode
+    attention over those pages matches the oracle on the same store."""
+    from turboquant_amd.kv_cache import quantize_values
+    H, T = 2, 75
+    pool, tq = _make_pool(gpu, d, key_bits, 8, H, 16, dtype, gs=gs)
+    g = torch.Generator().manual_seed(8 * d + key_bits)
+    k = torch.randn(1, T, H, d, generator=g).to(dtype).to(gpu)
+    v = torch.randn(1, T, H, d, generator=g).to(dtype).to(gpu)
+    table = torch.randperm(16, generator=g).to(torch.int32).to(gpu)[None, :]
+    for a, b in ((0, 20), (20, 21), (21, 75)):             # ragged appends: codes of earlier slots must survive
+        pool.append(k[:, a:b], v[:, a:b], table, torch.tensor([a], dtype=torch.int32, device=gpu))
+    idx, sgn, norms, rnorms, vdata, vsc, vz = pool.export_flat(table[0], T)
+    ref = tq.quantize(k[0].transpose(0, 1))
+    refv = quantize_values(v[0].transpose(0, 1), bits=8, group_size=gs)
+    torch.cuda.synchronize()
+    assert vdata.shape == (H, T, d) and torch.equal(vdata, refv.data)
+    assert torch.equal(vsc, refv.scales) and torch.equal(vz, refv.zeros)
+    assert torch.equal(idx, ref.mse_indices) and torch.equal(sgn, ref.qjl_signs)
+    # the oracle's value quantiser gives the same bytes (kv_cache.py:45-98)
+    want = O.quantize_values(v[0].transpose(0, 1).cpu(), 8, gs)
+    assert torch.equal(vdata.cpu(), want.data) and torch.equal(vsc.cpu(), want.scales)
+    # decode over 8-bit pages
+    _progress(f"decode over 8-bit values d={d} {dtype}")
+    Hq = 4 * H
+    q = torch.randn(1, Hq, d, generator=g).to(dtype)
+    out = pool.decode_attention(q.to(gpu), table, torch.tensor([T], dtype=torch.int32, device=gpu), max_len=T).cpu()
+    kc, vc = _store_from_oracle_view(pool, table[0], T)
+    if gs == 32:            # (the reference's read path de-quantises values with group size 32, score.py:94,127)
+        ref_out = O.hybrid_attention(q, kc, vc, T, params_of(tq), H, None, None)
+        assert cosine(out, ref_out) >= COS_GATE
+
+
+def test_compressed_store_with_eight_bit_values(gpu):
+    """CompressedKVStore(value_bits=8) (store.py:34-48 passes value_bits straight to quantize_values): chunks
+    in, flat cache out, and the hybrid attention on it."""
+    from turboquant_amd.score import compute_hybrid_attention
+    from turboquant_amd.store import CompressedKVStore
+    g = torch.Generator().manual_seed(88)
+    H, d, T = 2, 128, 100
+    store = CompressedKVStore(d, H, key_bits=3, value_bits=8, device=gpu, layer_idx=1)
+    k = torch.randn(T, H, d, generator=g).bfloat16().to(gpu)
+    v = torch.randn(T, H, d, generator=g).bfloat16().to(gpu)
+    store.append_chunk(k[:40], v[:40])
+    store.append_chunk(k[40:], v[40:])
+    flat = store.get_flat_cache()
+    assert flat.value_q.bits == 8 and flat.value_q.data.shape == (H, T, d)
+    want = O.quantize_values(v.transpose(0, 1).cpu(), 8, 32)
+    assert torch.equal(flat.value_q.data.cpu(), want.data)
+    q = torch.randn(1, 4 * H, d, generator=g).bfloat16().to(gpu)
+    out = compute_hybrid_attention(q, store, None, None, num_query_heads=4 * H).cpu()
+    kc = key_code(flat.prod_q.mse_indices.cpu(), flat.prod_q.qjl_signs.cpu(), flat.prod_q.residual_norms.cpu(),
+                  flat.prod_q.norms.cpu(), 2)
+    vc = value_code(flat.value_q.data.cpu(), flat.value_q.scales.cpu(), flat.value_q.zeros.cpu(), 8)
+    ref = O.hybrid_attention(q.cpu(), kc, vc, T, params_of(store.quantizer), H, None, None)
+    assert cosine(out, ref) >= COS_GATE
+    assert store.memory_bytes() > 0

@@ -81,6 +81,7 @@ _SIGNATURES = {
                                                C.POINTER(TqPageLayout), _vp, _vp, _i, _i64, _i64, _i64, _vp, _vp, _i, _vp]),
     "tq_decode_merge": (C.c_int, [_vp, _i64, _i, _i, _i, _vp, _vp]),
     "tq_time_next_page_kernel": (None, [_vp, _vp]),
+    "tq_time_next_key_kernel": (None, [_vp, _vp]),
     "tq_set_option": (C.c_int, [C.c_char_p, _i64]),
     "tq_stream_read": (C.c_int, [_vp, C.c_size_t, _i, _i, _vp, _vp]),
 }

@@ -210,7 +210,8 @@ decode_pages_kernel(const float* __restrict__ q_rot, const float* __restrict__ q
             if (ch < d) {
               const int grp = ch / L.group_size;
               const uint32_t* field = (const uint32_t*)(pg + vfield_off(L, ch));
-              const uint32_t f0 = field[0], f1 = (VB == 4) ? field[1] : 0u;
+              const uint32_t f0 = field[0], f1 = (VB >= 4) ? field[1] : 0u;
+              const uint32_t f2 = (VB == 8) ? field[2] : 0u, f3 = (VB == 8) ? field[3] : 0u;
               // scales and zeros of the 16 tokens of this (page, group): two rows of 16 elements
               float sc[16], zr[16];
               load_row16(pg + L.off_vscale + grp * TQ_PAGE_TOKENS * es, L.dtype, sc);
@@ -219,7 +220,8 @@ decode_pages_kernel(const float* __restrict__ q_rot, const float* __restrict__ q
               for (int t = 0; t < TQ_PAGE_TOKENS; ++t) {
                 unsigned code;
                 if (VB == 2) code = (f0 >> (2 * t)) & 3u;
-                else code = ((t < 8 ? f0 : f1) >> (4 * (t & 7))) & 15u;
+                else if (VB == 4) code = ((t < 8 ? f0 : f1) >> (4 * (t & 7))) & 15u;
+                else code = ((t < 4 ? f0 : (t < 8 ? f1 : (t < 12 ? f2 : f3))) >> (8 * (t & 3))) & 255u;
                 // slots past the end of the sequence may hold anything: they contribute an exact zero
                 const float val = t < n_valid ? fmaf((float)code, sc[t], zr[t]) : 0.0f;
                 const float4* pp = reinterpret_cast<const float4*>(s_p + (t0 + t) * GP);
@@ -939,7 +941,7 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   const int d = layer->d, G = Hq / Hkv;
   if (d != layout->d || layer->mse_bits != layout->mse_bits) return TQ_EINVAL;
   if (d < 64 || d > 768 || (d & 63) || G > G_MAX) return TQ_EUNSUPPORTED;
-  if (layout->value_bits != 2 && layout->value_bits != 4) return TQ_EUNSUPPORTED;
+  if (layout->value_bits != 2 && layout->value_bits != 4 && layout->value_bits != 8) return TQ_EUNSUPPORTED;
   const bool tail = recent_k != nullptr && recent_rows > 0;
   if (tail && !recent_v) return TQ_ENULL;
   if (tail && recent_rows > 1024) return TQ_EUNSUPPORTED;
@@ -959,7 +961,7 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
     if (G % n == 0 && G / n <= 8) kv_div = n;
   const int Gq = kv_div ? G / kv_div : G;
   const bool mfma_shape = kv_div && (d == 128 || d == 256) && (layout->dtype == TQ_BF16 || layout->dtype == TQ_F16) &&
-                          layer->Pi_colsum &&
+                          layout->value_bits != 8 && layer->Pi_colsum &&
                           layer->S_colsum;
 
   if (dtype < TQ_F32 || dtype > TQ_BF16) return TQ_EINVAL;
@@ -1078,7 +1080,8 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
     else TQ_LAUNCH_DEC(VB, 4)                                                    \
   }
     if (layout->value_bits == 2) TQ_LAUNCH_DEC_G(2)
-    else TQ_LAUNCH_DEC_G(4)
+    else if (layout->value_bits == 4) TQ_LAUNCH_DEC_G(4)
+    else TQ_LAUNCH_DEC_G(8)
 #undef TQ_LAUNCH_DEC_G
 #undef TQ_LAUNCH_DEC
   TQ_CHECK_LAUNCH();

@@ -18,6 +18,10 @@ struct FusedPrep {
   unsigned long long nonce = 0;      // value of a published flag in this call (never 0)
 };
 
+// Events armed by tq_time_next_page_kernel (which = 0) / tq_time_next_key_kernel (which = 1) on this thread:
+// returns them and disarms; false when none is armed.
+bool take_time_hook(int which, hipEvent_t& start, hipEvent_t& stop);
+
 // whether the library was built with the in-launch preparation (-DTQ_FUSED_PREP)
 bool decode_mfma_has_fused_prep();
 

@@ -785,8 +785,16 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   }
 }
 
-// events the next launch of this thread attaches to its dispatch (see tq_time_next_page_kernel)
-static thread_local hipEvent_t t_start_event = nullptr, t_stop_event = nullptr;
+// events the next launch of this thread attaches to its dispatch (see tq_time_next_page_kernel /
+// tq_time_next_key_kernel): [0] the page kernel of the decode path, [1] the paged key-quantise kernel
+static thread_local hipEvent_t t_hook_events[2][2] = {{nullptr, nullptr}, {nullptr, nullptr}};
+
+bool take_time_hook(int which, hipEvent_t& start, hipEvent_t& stop) {
+  start = t_hook_events[which][0];
+  stop = t_hook_events[which][1];
+  t_hook_events[which][0] = t_hook_events[which][1] = nullptr;
+  return start != nullptr || stop != nullptr;
+}
 
 template <int D, int MB, int NX, int VB, int GS, int DS, int WPS, bool F16P>
 static int launch_one(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, int kv_div,
@@ -806,11 +814,11 @@ static int launch_one(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, 
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return (int)e;
   }
-  if (t_start_event || t_stop_event) {
+  hipEvent_t t_start_event = nullptr, t_stop_event = nullptr;
+  if (take_time_hook(0, t_start_event, t_stop_event)) {
     hipExtLaunchKernelGGL(kern, dim3(n_split, Hkv, B), dim3(MF_WAVES * 64), smem, st, t_start_event, t_stop_event, 0,
                           qa_pack, q_stat, Hq, Hkv, kv_div, pool, block_table, bt_stride, seq_lens, sm_scale, ly, L, parts,
                           n_parts, n_split, len_sub, max_pages, num_pages, fz);
-    t_start_event = t_stop_event = nullptr;
   } else {
     kern<<<dim3(n_split, Hkv, B), dim3(MF_WAVES * 64), smem, st>>>(qa_pack, q_stat, Hq, Hkv, kv_div, pool, block_table,
                                                                    bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts,
@@ -856,6 +864,11 @@ int launch_decode_mfma(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv,
 }  // namespace tq
 
 extern "C" void tq_time_next_page_kernel(void* start_event, void* stop_event) {
-  tq::t_start_event = (hipEvent_t)start_event;
-  tq::t_stop_event = (hipEvent_t)stop_event;
+  tq::t_hook_events[0][0] = (hipEvent_t)start_event;
+  tq::t_hook_events[0][1] = (hipEvent_t)stop_event;
+}
+
+extern "C" void tq_time_next_key_kernel(void* start_event, void* stop_event) {
+  tq::t_hook_events[1][0] = (hipEvent_t)start_event;
+  tq::t_hook_events[1][1] = (hipEvent_t)stop_event;
 }

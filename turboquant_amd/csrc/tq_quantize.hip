@@ -648,7 +648,7 @@ extern "C" int tq_page_layout_init(tq_page_layout* L, int d, int mse_bits, int v
   if (!L) return TQ_ENULL;
   if (d < 64 || d > 768 || (d & 63)) return TQ_EUNSUPPORTED;
   if (mse_bits < 1 || mse_bits > 4) return TQ_EUNSUPPORTED;
-  if (value_bits != 2 && value_bits != 4) return TQ_EUNSUPPORTED;
+  if (value_bits != 2 && value_bits != 4 && value_bits != 8) return TQ_EUNSUPPORTED;
   if (group_size < 16 || d % group_size) return TQ_EINVAL;
   if (dtype < TQ_F32 || dtype > TQ_BF16) return TQ_EINVAL;
   const int es = dtype == TQ_F32 ? 4 : 2;

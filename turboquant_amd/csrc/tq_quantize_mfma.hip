@@ -27,6 +27,8 @@
 #include <atomic>
 
 #include "tq_quantize.h"
+#include "tq_decode_mfma.h"
+#include <hip/hip_ext.h>
 
 namespace tq {
 
@@ -576,7 +578,12 @@ static int launch_dt_d(const void* x, const Source& src, const tq_layer& ly, con
   const int64_t groups = (tiles + Gm::MT - 1) / Gm::MT;
   const int64_t resident = (int64_t)n_cu.load() * (per_cu > 0 ? per_cu : 1);
   const unsigned grid = (unsigned)(groups < resident ? groups : resident);
-  kern<<<dim3(grid), dim3(KQ_THREADS), Sm::bytes, st>>>(x, src, ly, sink, tiles);
+  hipEvent_t ev_start = nullptr, ev_stop = nullptr;
+  if (std::is_same<Sink, KeyPagedSink>::value && take_time_hook(1, ev_start, ev_stop)) {
+    hipExtLaunchKernelGGL(kern, dim3(grid), dim3(KQ_THREADS), Sm::bytes, st, ev_start, ev_stop, 0, x, src, ly, sink, tiles);
+  } else {
+    kern<<<dim3(grid), dim3(KQ_THREADS), Sm::bytes, st>>>(x, src, ly, sink, tiles);
+  }
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? TQ_OK : (int)e;
 }
