@@ -87,9 +87,10 @@ typedef struct tq_layer {
  *   keys   : key_bits = mse_bits+1 bit-planes (index bits high..low, then the QJL
  *            sign).  Word j of plane p of token n holds coordinates 32j..32j+31
  *            (bit i = coordinate 32j+i).  With key_lane_major != 0 (d a multiple
- *            of 128) the words are stored as [j%4][n][j/4][p], so that the
+ *            of 128, or 64) the words are stored as [j%4][n][j/4][p], so that the
  *            words one wavefront lane (token n, coordinate quarter j%4) consumes
- *            are contiguous, 128 coordinates after 128; otherwise as [p][j][n].
+ *            are contiguous, 128 coordinates after 128 (d = 64: [j][n][p]);
+ *            otherwise as [p][j][n].
  *   meta   : per token {float norm, float rnorm}: the key norm (a value of the
  *            input dtype, widened losslessly) and ||r||.
  *   vdata  : per channel c a little-endian field of 16*value_bits bits, token n's

@@ -415,3 +415,19 @@ def test_compressed_store_with_eight_bit_values(gpu):
     ref = O.hybrid_attention(q.cpu(), kc, vc, T, params_of(store.quantizer), H, None, None)
     assert cosine(out, ref) >= COS_GATE
     assert store.memory_bytes() > 0
+
+
+# ------------------------------------------------------------------ head_dim 64 on the matrix-core page kernel
+@pytest.mark.parametrize("key_bits,vb,Hq,Hkv,dtype", [(3, 4, 8, 2, torch.bfloat16), (3, 2, 32, 4, torch.bfloat16),
+                                                       (2, 2, 6, 2, torch.float16), (4, 4, 16, 2, torch.bfloat16),
+                                                       (3, 4, 1, 1, torch.float16), (4, 2, 12, 1, torch.bfloat16)])
+def test_decode_head_dim_64_on_the_matrix_cores(gpu, key_bits, vb, Hq, Hkv, dtype):
+    """head_dim 64 (the reference ships codebook_d64_b1..4.json) runs the matrix-core page kernel: the score
+    contraction still takes 128 coordinates per instruction, half of them zeros.  Ragged lengths, block and
+    page boundaries, exact tails, several split counts, against the oracle on the same store."""
+    _progress(f"decode d=64 kb={key_bits} vb={vb} Hq={Hq} Hkv={Hkv} {dtype}")
+    worst = _decode_case(gpu, 64, key_bits, vb, 4, Hq, Hkv, [513, 64, 1, 200], [0, 7, 33, 0], seed=640 + Hq, dtype=dtype)
+    for n_split in (1, 3, 8):
+        worst = min(worst, _decode_case(gpu, 64, key_bits, vb, 2, Hq, Hkv, [1000, 17], None, seed=650 + n_split,
+                                        n_split=n_split, dtype=dtype))
+    _progress(f"   worst cosine {worst:.7f}")

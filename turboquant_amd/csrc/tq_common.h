@@ -104,7 +104,9 @@ __host__ __device__ __forceinline__ int idx_row_bytes(int d, int mse_bits) {
 // byte offset of word j (coordinates 32j..32j+31) of plane p of token n
 __host__ __device__ __forceinline__ int key_word_off(const tq_page_layout& L, int p, int j, int n) {
   const int W = L.d >> 5, planes = L.mse_bits + 1;
-  if (L.key_lane_major) return L.off_keys + (((((j & 3) * TQ_PAGE_TOKENS + n) * (W >> 2)) + (j >> 2)) * planes + p) * 4;
+  // (head_dim 64 has two words per plane: [j][n][p])
+  if (L.key_lane_major)
+    return L.off_keys + (((((j & 3) * TQ_PAGE_TOKENS + n) * (W >= 4 ? W >> 2 : 1)) + (j >> 2)) * planes + p) * 4;
   return L.off_keys + ((p * W + j) * TQ_PAGE_TOKENS + n) * 4;
 }
 

@@ -960,7 +960,7 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   for (int n = 1; n <= G && !kv_div; ++n)
     if (G % n == 0 && G / n <= 8) kv_div = n;
   const int Gq = kv_div ? G / kv_div : G;
-  const bool mfma_shape = kv_div && (d == 128 || d == 256) && (layout->dtype == TQ_BF16 || layout->dtype == TQ_F16) &&
+  const bool mfma_shape = kv_div && (d == 64 || d == 128 || d == 256) && (layout->dtype == TQ_BF16 || layout->dtype == TQ_F16) &&
                           layout->value_bits != 8 && layer->Pi_colsum &&
                           layer->S_colsum;
 
@@ -1029,7 +1029,10 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
     else if (dtype == TQ_F16) TQ_LAUNCH_PT(PER, TQ_F16, PAGED)     \
     else TQ_LAUNCH_PT(PER, TQ_F32, PAGED)                          \
   }
-      if (d == 128) {
+      if (d == 64) {
+        if (ts.paged) TQ_LAUNCH_PT_DT(4, true)
+        else TQ_LAUNCH_PT_DT(4, false)
+      } else if (d == 128) {
         if (ts.paged) TQ_LAUNCH_PT_DT(8, true)
         else TQ_LAUNCH_PT_DT(8, false)
       } else {
@@ -1204,11 +1207,11 @@ size_t decode_scratch_need(int B, int Hq, int Hkv, int n_split, const tq_layer& 
   size_t floats = parts_floats(B, Hq, d, n_split + 1) + (size_t)2 * B * Hq * d + (size_t)4 * B * Hq +
                   2 * flag_words(B, Hq);
   size_t words = 0;
-  if (kv_div && (d == 128 || d == 256)) {
+  if (kv_div && (d == 64 || d == 128 || d == 256)) {
     int planes = ly.mse_bits + 1;
     for (int t = 0; t < ly.n_terms; ++t)
       if (__builtin_popcount(ly.term_mask[t]) > 1) ++planes;
-    words = (size_t)B * Hkv * kv_div * planes * (d / 128) * 2 * 64 * 8;
+    words = (size_t)B * Hkv * kv_div * planes * (d >= 128 ? d / 128 : 1) * 2 * 64 * 8;
   }
   return (floats + words) * 4;
 }

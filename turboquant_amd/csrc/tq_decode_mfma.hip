@@ -180,8 +180,8 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
                    float* __restrict__ parts, int n_parts, int n_split, int len_sub, int max_pages, int num_pages,
                    FusedPrep fz) {
   constexpr int DW = D / DS;                  // coordinates / channels of one wavefront
-  constexpr int WPLT = D / 128;               // plane words per lane per plane per page, all wavefronts
-  constexpr int WPL = DW / 128;               // ... of one wavefront
+  constexpr int WPLT = (D + 127) / 128;       // plane words per lane per plane per page, all wavefronts
+  constexpr int WPL = (DW + 127) / 128;       // ... of one wavefront (head_dim 64: one, with half of the lanes idle)
   constexpr int NTP = MB + NX + 1;            // term planes fed to the MFMA (stored + XOR terms + sign)
   constexpr int NKW = (MB + 1) * WPL;         // key dwords per lane per page
   constexpr int CT = DW / 16;                 // channel tiles of one wavefront
@@ -191,7 +191,8 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   constexpr int PIECES = 2 * NG;              // 16-byte pieces of this wavefront's scales per page
   constexpr int NGRP = MF_WAVES / DS;         // wavefront groups (each walks its own blocks)
   constexpr int WAVE_LDS_FLOATS = wave_lds_floats(NG, DS);
-  static_assert(WPL >= 1 && NG >= 2 && NG % 2 == 0, "a wavefront takes at least 128 coordinates and whole group pairs");
+  static_assert(NG >= 2 && NG % 2 == 0 && (DW % 128 == 0 || (D == 64 && DS == 1)),
+                "a wavefront takes whole 128-coordinate chunks (or a whole head of 64) and whole group pairs");
   // Hkv counts query-head groups: a KV head with more than 8 query heads is served by kv_div groups
   // of G <= 8 heads each (consecutive groups read the same pages)
   const int G = Hq / Hkv;
@@ -292,7 +293,11 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
     sa = (e1 - t01) | ((e1 - t23) << 8) | ((e2 - t01) << 16) | ((e2 - t23) << 24);
   }
   const int sb = 127 + 1;
-  const uint32_t nib = in_vgpr(0x11111111u), nib1 = in_vgpr(0x22222222u), nib2 = in_vgpr(0x44444444u);
+  // head_dim 64: the score MFMA still contracts 128 coordinates; the lanes of the upper two coordinate
+  // quarters feed zeros (their masks are zero, whatever their loads return)
+  const bool kq_live = D >= 128 || kb < D / 32;
+  const uint32_t nib = in_vgpr(kq_live ? 0x11111111u : 0u), nib1 = in_vgpr(kq_live ? 0x22222222u : 0u),
+                 nib2 = in_vgpr(kq_live ? 0x44444444u : 0u);
   // constant parts of the scores of the two heads this lane sees in the MFMA output (rows 4kb..4kb+3
   // = heads 2kb, 2kb+1), as the initial accumulators; only one wavefront of a pair adds them
   f32x4 cm = {0, 0, 0, 0}, cq = {0, 0, 0, 0};
@@ -332,7 +337,9 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   const uint8_t* pool_h = pool + (int64_t)(h / kv_div) * L.page_bytes;
   const int64_t page_stride = (int64_t)(Hkv / kv_div) * L.page_bytes;
   // per lane the key words are [word i][plane], the value fields [channel tile]: a wavefront's share is contiguous
-  const uint32_t off_keys = L.off_keys + (lane * DS + hf) * (NKW * 4), off_meta = L.off_meta + n * 8;
+  // (head_dim 64: the idle lanes re-read the last live lane's words)
+  const int klane = D >= 128 ? lane : min(lane, D / 2 - 1);
+  const uint32_t off_keys = L.off_keys + (klane * DS + hf) * (NKW * 4), off_meta = L.off_meta + n * 8;
   const uint32_t off_v = L.off_vdata + (n * DS + hf) * (VW * 4);
   const uint32_t off_scale = L.off_vscale + hf * (NG * 32) + (lane % PIECES) * 16;
 
@@ -656,24 +663,29 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
     int pid[4];
     const int trips = (max(blk_end - blk_begin, 0) + NGRP - 1) / NGRP;
     int blk = blk_begin + wgrp;
-    // Block tables are device data nobody has checked: every wavefront looks once at the table entries of its
-    // workgroup's blocks (a lane per entry; requested first, used after the first block's loads are on
-    // their way).  Only a workgroup that finds an entry outside the pool runs the checking loop.
-    bool entry_bad = false;
-#ifndef TQ_EXP_NO_TABLE_SCAN
-    {
-      const int e0 = 4 * blk_begin, e1 = min(4 * blk_end, n_pages);
-      for (int e = e0 + lane; e < e1; e += 4 * 64) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) entry_bad |= (unsigned)bt[min(e + 64 * i, e1 - 1)] >= (unsigned)num_pages;
-      }
-    }
-#endif
     int bad = 0;                                          // pages of the current block that lie outside the pool
     if (blk < blk_end) {
       bad = page_ids(blk, pid, std::true_type{});
       load_keys(pid, K);
       load_vals(pid, V);
+    }
+    // Block tables are device data nobody has checked: every wavefront looks once at the table entries of its
+    // workgroup's blocks, a lane per entry: up to 256 entries in straight-line code (all loads unconditional
+    // and inside the table row, requested behind the first block's loads so that nothing waits for them
+    // alone), a loop for longer ranges.  Only a workgroup that finds an entry outside the pool runs the
+    // checking loop.
+    bool entry_bad = false;
+    {
+      const int e0 = 4 * blk_begin, e1 = min(4 * blk_end, n_pages), last = max(e1 - 1, 0);
+      uint32_t raw[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) raw[i] = (uint32_t)bt[min(max(e0 + lane + 64 * i, 0), last)];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) entry_bad |= e0 + lane + 64 * i < e1 && raw[i] >= (unsigned)num_pages;
+      for (int e = e0 + 4 * 64 + lane; e < e1; e += 4 * 64) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) entry_bad |= (unsigned)bt[min(e + 64 * i, e1 - 1)] >= (unsigned)num_pages;
+      }
     }
     // CHECKED: page ids are validated and every trip takes the masking (PARTIAL) path
     auto run = [&](auto checked_tag) {
@@ -831,7 +843,7 @@ static int launch_one(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, 
 // Returns TQ_EUNSUPPORTED when the shape has no matrix-core kernel; the caller then
 // uses the general vector-ALU kernel.
 // words of packed query operands tq_decode_attn_paged reserves in its workspace
-size_t decode_mfma_pack_words(int B, int Hq, int d) { return (size_t)B * Hq * 9 * (d / 128 + 1) * 1024; }
+size_t decode_mfma_pack_words(int B, int Hq, int d) { return (size_t)B * Hq * 9 * (d / 128 + 1) * 1024; }   // d = 64: one chunk
 
 int launch_decode_mfma(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, int kv_div,
                        const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
@@ -857,6 +869,8 @@ int launch_decode_mfma(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv,
   TQ_TRY(128, 1, 0, 2, 32, 1, 2) TQ_TRY(128, 1, 0, 4, 32, 1, 2) TQ_TRY(256, 1, 0, 2, 32, 2, 2) TQ_TRY(256, 1, 0, 4, 32, 2, 2)
   TQ_TRY(128, 3, 1, 2, 32, 1, 1) TQ_TRY(128, 3, 1, 4, 32, 1, 1) TQ_TRY(256, 3, 1, 2, 32, 2, 1) TQ_TRY(256, 3, 1, 4, 32, 2, 1)
   TQ_TRY(128, 2, 0, 2, 64, 1, 2) TQ_TRY(128, 2, 0, 4, 64, 1, 2) TQ_TRY(256, 2, 0, 2, 64, 2, 2) TQ_TRY(256, 2, 0, 4, 64, 2, 2)
+  TQ_TRY(64, 2, 0, 2, 32, 1, 2) TQ_TRY(64, 2, 0, 4, 32, 1, 2) TQ_TRY(64, 1, 0, 2, 32, 1, 2) TQ_TRY(64, 1, 0, 4, 32, 1, 2)
+  TQ_TRY(64, 3, 1, 2, 32, 1, 2) TQ_TRY(64, 3, 1, 4, 32, 1, 2)
 #undef TQ_TRY
   return TQ_EUNSUPPORTED;
 }

@@ -117,7 +117,7 @@ __device__ __forceinline__ void prep_query_body(const void* __restrict__ q, int 
     cmax = fmaxf(cmax, fabsf(ly.term_coef[t]));
     if (__builtin_popcount(ly.term_mask[t]) > 1) ++nx;
   }
-  const int ntp = mb + nx + 1, wpl = d / 128;
+  const int ntp = mb + nx + 1, wpl = d >= 128 ? d / 128 : 1;      // head_dim 64: one chunk of 128 with its upper half unused
   if (tid < ntp) {
     float coef = 1.0f;
     if (tid < mb) {
@@ -337,7 +337,7 @@ __device__ __forceinline__ void prep_unit256(const void* __restrict__ q, int dty
     cmax = fmaxf(cmax, fabsf(ly.term_coef[t]));
     if (__builtin_popcount(ly.term_mask[t]) > 1) ++nx;
   }
-  const int ntp = mb + nx + 1, wpl = d / 128;
+  const int ntp = mb + nx + 1, wpl = d >= 128 ? d / 128 : 1;      // head_dim 64: one chunk of 128 with its upper half unused
   if (tid < ntp) {
     float coef = 1.0f;
     if (tid < mb) {

@@ -653,7 +653,7 @@ extern "C" int tq_page_layout_init(tq_page_layout* L, int d, int mse_bits, int v
   if (dtype < TQ_F32 || dtype > TQ_BF16) return TQ_EINVAL;
   const int es = dtype == TQ_F32 ? 4 : 2;
   L->d = d; L->mse_bits = mse_bits; L->value_bits = value_bits; L->group_size = group_size; L->dtype = dtype;
-  L->key_lane_major = (d % 128 == 0) ? 1 : 0;
+  L->key_lane_major = (d % 128 == 0 || d == 64) ? 1 : 0;
   int off = 0;
   L->off_keys = off;   off += (mse_bits + 1) * (d / 8) * TQ_PAGE_TOKENS;
   L->off_meta = off;   off += 8 * TQ_PAGE_TOKENS;

@@ -370,7 +370,7 @@ int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* 
                         float* q_stat, uint32_t* qa_pack, int G, float sm_scale, hipStream_t st, bool q_rot_unused) {
   const int d = layer->d;
   if (qa_pack) {       // operands of the matrix-core decode kernel wanted
-    if (!q_stat || !layer->Pi_colsum || !layer->S_colsum || G > ROT_MAX_ROWS || rows % G || (d != 128 && d != 256))
+    if (!q_stat || !layer->Pi_colsum || !layer->S_colsum || G > ROT_MAX_ROWS || rows % G || (d != 64 && d != 128 && d != 256))
       return TQ_EUNSUPPORTED;
     if (opt_prep_units.load() && q_rot_unused) {
       // heads per unit: as few as keep the launch at about a thousand workgroups
@@ -381,7 +381,8 @@ int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* 
       const dim3 ugrid((unsigned)((8 / hp) * words), (unsigned)groups);
       const size_t usm = (size_t)prep_unit_smem_floats(hp, d) * sizeof(float);
       if (groups > 65535) return TQ_EUNSUPPORTED;
-      if (d == 128) prep_units_kernel<8><<<ugrid, dim3(PREP_UNIT_THREADS), usm, st>>>(q, dtype, G, *layer, sm_scale, q_stat, qa_pack, hp);
+      if (d == 64) prep_units_kernel<4><<<ugrid, dim3(PREP_UNIT_THREADS), usm, st>>>(q, dtype, G, *layer, sm_scale, q_stat, qa_pack, hp);
+      else if (d == 128) prep_units_kernel<8><<<ugrid, dim3(PREP_UNIT_THREADS), usm, st>>>(q, dtype, G, *layer, sm_scale, q_stat, qa_pack, hp);
       else prep_units_kernel<16><<<ugrid, dim3(PREP_UNIT_THREADS), usm, st>>>(q, dtype, G, *layer, sm_scale, q_stat, qa_pack, hp);
       hipError_t e = hipGetLastError();
       return e == hipSuccess ? TQ_OK : (int)e;
@@ -396,7 +397,8 @@ int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* 
     else if (dtype == TQ_F32) TQ_PREP(PER, TQ_F32);  \
     else return TQ_EINVAL;                           \
   }
-    if (d == 128) TQ_PREP_DT(8)
+    if (d == 64) TQ_PREP_DT(4)
+    else if (d == 128) TQ_PREP_DT(8)
     else TQ_PREP_DT(16)
 #undef TQ_PREP_DT
 #undef TQ_PREP

@@ -168,9 +168,9 @@ class PagedKVPool:
         return idx, signs, norms, rnorms, v_data, v_scales, v_zeros
 
     def _matrix_core_shape(self, Hq: Optional[int]) -> bool:
-        """Whether decode runs on the matrix-core page kernel (head_dim 128 / 256, 16-bit pools, up to 4-bit
+        """Whether decode runs on the matrix-core page kernel (head_dim 64 / 128 / 256, 16-bit pools, up to 4-bit
         keys, query heads that split into groups of at most 8); only the split heuristic depends on it."""
-        if self.head_dim not in (128, 256) or self.dtype not in (torch.bfloat16, torch.float16):
+        if self.head_dim not in (64, 128, 256) or self.dtype not in (torch.bfloat16, torch.float16):
             return False
         if self.quantizer.bits - 1 > 3 or self.value_bits not in (2, 4) or self.value_group_size not in (32, 64):
             return False
