@@ -867,7 +867,7 @@ int launch_decode_mfma(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv,
   }
   TQ_TRY(128, 2, 0, 2, 32, 1, 2) TQ_TRY(128, 2, 0, 4, 32, 1, 2) TQ_TRY(256, 2, 0, 2, 32, 2, 2) TQ_TRY(256, 2, 0, 4, 32, 2, 2)
   TQ_TRY(128, 1, 0, 2, 32, 1, 2) TQ_TRY(128, 1, 0, 4, 32, 1, 2) TQ_TRY(256, 1, 0, 2, 32, 2, 2) TQ_TRY(256, 1, 0, 4, 32, 2, 2)
-  TQ_TRY(128, 3, 1, 2, 32, 1, 1) TQ_TRY(128, 3, 1, 4, 32, 1, 1) TQ_TRY(256, 3, 1, 2, 32, 2, 1) TQ_TRY(256, 3, 1, 4, 32, 2, 1)
+  TQ_TRY(128, 3, 1, 2, 32, 1, 2) TQ_TRY(128, 3, 1, 4, 32, 1, 2) TQ_TRY(256, 3, 1, 2, 32, 2, 2) TQ_TRY(256, 3, 1, 4, 32, 2, 2)
   TQ_TRY(128, 2, 0, 2, 64, 1, 2) TQ_TRY(128, 2, 0, 4, 64, 1, 2) TQ_TRY(256, 2, 0, 2, 64, 2, 2) TQ_TRY(256, 2, 0, 4, 64, 2, 2)
   TQ_TRY(64, 2, 0, 2, 32, 1, 2) TQ_TRY(64, 2, 0, 4, 32, 1, 2) TQ_TRY(64, 1, 0, 2, 32, 1, 2) TQ_TRY(64, 1, 0, 4, 32, 1, 2)
   TQ_TRY(64, 3, 1, 2, 32, 1, 2) TQ_TRY(64, 3, 1, 4, 32, 1, 2)
