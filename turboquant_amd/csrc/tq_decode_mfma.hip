@@ -336,6 +336,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   const int32_t* bt = block_table + (int64_t)b * bt_stride;
   const uint8_t* pool_h = pool + (int64_t)(h / kv_div) * L.page_bytes;
   const int64_t page_stride = (int64_t)(Hkv / kv_div) * L.page_bytes;
+  const uint32_t page_stride32 = (uint32_t)page_stride;
   // per lane the key words are [word i][plane], the value fields [channel tile]: a wavefront's share is contiguous
   // (head_dim 64: the idle lanes re-read the last live lane's words)
   const int klane = D >= 128 ? lane : min(lane, D / 2 - 1);
@@ -364,9 +365,12 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   auto page_ids = [&](int blk, int (&pid)[4], auto check_tag) -> int {
     constexpr bool CHECK = decltype(check_tag)::value;
     int bad = 0;
+    // one 64-bit address per block; the four entries are read at 32-bit scalar offsets from it
+    const int32_t* row = bt + 4 * blk;
+    const int last = n_pages - 1 - 4 * blk;               // >= 0: the block has at least one page
 #pragma unroll
     for (int pg = 0; pg < 4; ++pg) {
-      const int raw = bt[min(4 * blk + pg, n_pages - 1)];
+      const int raw = row[min(pg, last)];
       const bool ok = !CHECK || (unsigned)raw < (unsigned)num_pages;
       pid[pg] = ok ? raw : 0;
       bad |= ok ? 0 : 1 << pg;
@@ -379,7 +383,8 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
     const uint32_t ok = in_vgpr(off_keys), om = in_vgpr(off_meta);
 #pragma unroll
     for (int pg = 0; pg < 4; ++pg) {
-      const uint8_t* base = pool_h + pid[pg] * page_stride;
+      // (page numbers are non-negative and the stride fits 32 bits: an unsigned 32 x 32 -> 64 bit product)
+      const uint8_t* base = pool_h + (uint64_t)(uint32_t)pid[pg] * page_stride32;
       const uint32_t* kp = (const uint32_t*)(base + ok);
 #pragma unroll
       for (int w = 0; w < NKW; ++w) R.key[pg][w] = kp[w];
@@ -394,7 +399,6 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   // The page of a lane is picked among the four page numbers with conditional moves on vector
   // registers (on scalar operands the compiler builds branches instead) and turned into an address
   // with one unsigned 32 x 32 -> 64 bit multiply-add.
-  const uint32_t page_stride32 = (uint32_t)page_stride;
   auto load_vals = [&](const int (&pid)[4], ValRegs& R) {
     const uint32_t p0 = in_vgpr((uint32_t)pid[0]), p1 = in_vgpr((uint32_t)pid[1]), p2 = in_vgpr((uint32_t)pid[2]),
                    p3 = in_vgpr((uint32_t)pid[3]);
