@@ -296,24 +296,28 @@ def quantize_bench(device, steps, warmup):
     pool = PagedKVPool(tq, H, T // 16, value_bits=2, value_group_size=32, dtype=torch.bfloat16, device=device)
     table = torch.arange(T // 16, dtype=torch.int32, device=device)[None]
     ms, _ = time_steps(lambda i: pool.append(k, v, table), steps, warmup)
-    # the paged key kernel alone, timed inside whole appends: its three d x d contractions are the
-    # matrix-core part of the path.  The kernel issues them as 15 exact bf16 term products (5 per
-    # contraction instead of one fp32 product), so the matrix-core work it issues is 5 x the algorithmic FLOP,
-    # and the roofline that bounds it is the bf16 matrix peak.
+    # The three d x d contractions of the key quantiser are the matrix-core part of the path.  The kernel issues
+    # them as 15 exact bf16 term products (5 per contraction instead of one fp32 product), so the matrix-core work
+    # it issues is 5 x the algorithmic FLOP, and the roofline that bounds it is the bf16 matrix peak.  The key
+    # kernel runs beside the value kernel (a second stream), and an event pair around it inside such an append
+    # also covers time it spends waiting for its share of the machine, so the fraction is taken over the WHOLE
+    # append (both kernels, fork and join); the event-pair figure is reported next to it.
     key_ms = time_key_kernel(lambda i: pool.append(k, v, table), steps, warmup)
     flops = 3 * 2 * d * d * T * H
-    issued = 5 * flops / (key_ms * 1e-3) / 1e12
+    issued = 5 * flops / (ms * 1e-3) / 1e12
     nbytes = T * (2 * H * d * 2 + H * 100)
     return {"tokens_per_s": T / (ms * 1e-3), "ms": ms, "tokens": T, "kv_heads": H, "head_dim": d,
             "workload": "prefill quantize, 32768 tok x 8 KV heads, d=128, 3b keys + 2b values, pages of 16",
             "hbm_gbs": nbytes / (ms * 1e-3) / 1e9, "hbm_bytes": nbytes,
             "hbm_frac": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-            "roofline": {"bound": "mfma", "kernel": "key_mfma_kernel (paged sink)", "kernel_ms": key_ms,
+            "roofline": {"bound": "mfma", "kernel": "key_mfma_kernel (paged sink) beside value_chunk_kernel",
+                         "append_ms": ms, "key_kernel_event_ms": key_ms,
                          "achieved": issued, "peak": 2500.0, "unit": "TFLOP/s", "frac": issued / 2500.0,
-                         "algorithmic_tflops": flops / (key_ms * 1e-3) / 1e12,
-                         "note": "achieved = bf16 matrix-core work the kernel issues (15 exact bf16 term products for "
-                                 "the 3 fp32-accurate d x d contractions per vector = 5 x the algorithmic 6 d^2 FLOP) "
-                                 "against the 2500 TFLOP/s bf16 peak; algorithmic_tflops is the 6 d^2 figure"}}, (pool, k, v, table, tq)
+                         "algorithmic_tflops": flops / (ms * 1e-3) / 1e12,
+                         "note": "achieved = bf16 matrix-core work the key kernel issues (15 exact bf16 term products "
+                                 "for the 3 fp32-accurate d x d contractions per vector = 5 x the algorithmic 6 d^2 "
+                                 "FLOP) over the whole append time, against the 2500 TFLOP/s bf16 peak; "
+                                 "algorithmic_tflops is the 6 d^2 figure over the same time"}}, (pool, k, v, table, tq)
 
 
 def round_trip_bench(device, steps, warmup, with_cpu):

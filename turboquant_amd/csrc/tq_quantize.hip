@@ -337,9 +337,14 @@ value_chunk_kernel(const void* __restrict__ v, Source src, int d, int gs, Sink s
   const int cpt = d >> 3;                          // chunks (threads) per token
   const int t = tid / cpt, ck = tid - t * cpt;     // token slot, chunk
   const int tpg = gs >> 3;                         // threads per group (power of two, <= 16)
+  // a thread's 8 codes are one word of 8 * VB bits; the words of a chunk's 16 tokens lie together
+  // (rows padded by 16 bytes), so that the thread that assembles half a channel field reads the
+  // words of its 8 tokens with one or two 16-byte loads
+  using CodeWord = typename std::conditional<VB == 2, uint16_t, uint32_t>::type;
+  constexpr int CROW = TILE * (int)sizeof(CodeWord) + 16;      // bytes per chunk row
   extern __shared__ __align__(16) unsigned char smem[];
-  uint8_t* scode = smem;                           // [TILE][d]
-  int* svalid = (int*)(smem + TILE * d);           // [TILE]
+  unsigned char* scode = smem;                     // [d / 8] rows of CROW bytes
+  int* svalid = (int*)(smem + (size_t)cpt * CROW); // [TILE]
 
   const typename Source::TileRef ref = src.tile_ref(tile);
   int64_t off;
@@ -358,7 +363,9 @@ value_chunk_kernel(const void* __restrict__ v, Source src, int d, int gs, Sink s
   const uint4 raw = *(const uint4*)((const uint16_t*)v + (ok ? off : 0) + ck * 8);
   if (ck == 0) svalid[t] = ok;
   // a tile none of whose slots exists may lie beyond the block table: leave before looking it up
-  if (!__syncthreads_or(ok)) return;
+  const int n_ok = __syncthreads_count(ok);
+  if (n_ok == 0) return;
+  const bool full_tile = n_ok == (int)blockDim.x;
   float x[8];
   {
     const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
@@ -395,25 +402,28 @@ value_chunk_kernel(const void* __restrict__ v, Source src, int d, int gs, Sink s
   const bool fast_div = DT == TQ_BF16 && sc > 0x1p-60f && sc < 0x1p60f;
   const float rsc = 1.0f / sc;
   uint32_t codes = 0;                              // 8 codes, VB bits each, channel order
+  float quo[8];
+  if (fast_div) {                // every a of the group is finite and at most (levels + 1) * sc < 2^64 then
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float a = round_hw<DT>(x[i] - z);
+      const float q0 = a * rsc;
+      quo[i] = fmaf(fmaf(-q0, sc, a), rsc, q0);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) quo[i] = round_hw<DT>(x[i] - z) / sc;
+  }
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    const float a = round_hw<DT>(x[i] - z);
-    float quo;
-    if (fast_div) {              // every a of the group is finite and at most (levels + 1) * sc < 2^64 then
-      const float q0 = a * rsc;
-      quo = fmaf(fmaf(-q0, sc, a), rsc, q0);
-    } else {
-      quo = a / sc;
-    }
-    float q = round_hw<DT>(quo);
+    float q = round_hw<DT>(quo[i]);
     q = rintf(q);
     // clamp to [0, levels]; a NaN becomes code 0 (the median-of-three instruction returns the minimum of
     // its operands when one of them is a NaN)
     q = __builtin_amdgcn_fmed3f(q, 0.0f, levels);
-    const uint32_t c = (uint32_t)q;
-    codes |= c << (VB * i);
-    if constexpr (!std::is_same<Sink, ValFlatSink>::value) scode[t * d + ck * 8 + i] = (uint8_t)c;
+    codes |= (uint32_t)q << (VB * i);
   }
+  if constexpr (!std::is_same<Sink, ValFlatSink>::value) *(CodeWord*)(scode + ck * CROW + t * sizeof(CodeWord)) = (CodeWord)codes;
   const int ng = d / gs, g = (ck * 8) / gs;
   const bool leader = (ck & (tpg - 1)) == 0;
 
@@ -442,13 +452,28 @@ value_chunk_kernel(const void* __restrict__ v, Source src, int d, int gs, Sink s
     {
       const int c = tid >> 1, half = tid & 1;
       uint8_t* fbytes = pg + vfield_off(L, c) + half * VB;
-      uint32_t neu = 0, mask = 0;
+      const unsigned char* row = scode + (c >> 3) * CROW + half * 8 * sizeof(CodeWord);
+      const int sh = (c & 7) * VB;                   // the channel's code inside a word
+      uint32_t neu = 0, mask = VB == 2 ? 0xffffu : 0xffffffffu;
+      if constexpr (VB == 2) {
+        const uint4 w = *(const uint4*)row;          // 8 tokens, two to a dword
+        const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
-      for (int s2 = 0; s2 < 8; ++s2) {
-        const int n = half * 8 + s2;
-        const uint32_t keep = svalid[n] ? (1u << VB) - 1u : 0u;
-        neu |= ((uint32_t)scode[n * d + c] & keep) << (VB * s2);
-        mask |= keep << (VB * s2);
+        for (int k = 0; k < 4; ++k) {
+          const uint32_t pr = (ww[k] >> sh) & 0x00030003u;
+          neu |= ((pr | (pr >> 14)) & 0xfu) << (4 * k);
+        }
+      } else {
+        const uint4 w0 = *(const uint4*)row, w1 = *(const uint4*)(row + 16);
+        const uint32_t ww[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+#pragma unroll
+        for (int k = 0; k < 8; ++k) neu |= ((ww[k] >> sh) & 0xfu) << (4 * k);
+      }
+      if (!full_tile) {                              // uniform over the workgroup
+        mask = 0;
+#pragma unroll
+        for (int s2 = 0; s2 < 8; ++s2) mask |= (svalid[half * 8 + s2] ? (1u << VB) - 1u : 0u) << (VB * s2);
+        neu &= mask;
       }
       if (mask != 0 && page_ok) {
         if (VB == 2) {
@@ -735,7 +760,7 @@ static int launch_value(const void* v, int dtype, const Source& src, int d, int 
   // 16-bit inputs with 2/4-bit codes on the usual head sizes take the chunked kernel
   if (dtype != TQ_F32 && (bits == 2 || bits == 4) && (d == 64 || d == 128 || d == 256) && gs >= 16 && gs <= 128 &&
       (gs & (gs - 1)) == 0 && value_chunks_aligned(v, src)) {
-    const size_t sm = (size_t)TILE * d + TILE * sizeof(int);
+    const size_t sm = (size_t)(d / 8) * (TILE * (bits == 2 ? 2 : 4) + 16) + TILE * sizeof(int);
     const dim3 g2((unsigned)tiles), b2(TILE * d / 8);
 #define TQ_LAUNCH_VC(DT, VB) value_chunk_kernel<DT, VB, Source, Sink><<<g2, b2, sm, st>>>(v, src, d, gs, sink)
     if (dtype == TQ_BF16) { if (bits == 2) TQ_LAUNCH_VC(TQ_BF16, 2); else TQ_LAUNCH_VC(TQ_BF16, 4); }

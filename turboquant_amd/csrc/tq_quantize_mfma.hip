@@ -321,13 +321,31 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
     const float nrm = E::round(sqrtf(ss));
     const float den = E::round(nrm + 1e-10f);
     if (seg == 0) snorm[t] = nrm;
+    if constexpr (DT == TQ_BF16) {
+      // Quotients of bf16 numbers, rounded to bf16: a / den is either exactly a rounding tie or at least
+      // 2^-17 (relative) away from one, so q0 = a (1/den) with one residual correction, which is exact
+      // for a tie, rounds like the correctly rounded quotient.  (Compared with the division over every
+      // pair of bf16 numbers with |a| <= 2 den and den in the range below: the only difference is that
+      // a = -0 gives +0, which no product sum can tell apart.)  |x_i| <= 2 den holds for any finite norm.
+      if (den > 0x1p-60f && den < 0x1p60f) {
+        const float rden = 1.0f / den;
+#pragma unroll
+        for (int c = 0; c < SEG; ++c) {
+          const float q0 = xs[c] * rden;
+          xs[c] = fmaf(fmaf(-q0, den, xs[c]), rden, q0);
+        }
+      } else {
+#pragma unroll
+        for (int c = 0; c < SEG; ++c) xs[c] = xs[c] / den;
+      }
+    }
 #pragma unroll
     for (int c8 = 0; c8 < SEG; c8 += 8) {
       uint32_t pk[3][4];
 #pragma unroll
       for (int c = 0; c < 8; c += 2) {
         if constexpr (DT == TQ_BF16) {                          // the rounded quotient is its own single term
-          pk[0][c >> 1] = cvt_pk_bf16(xs[c8 + c] / den, xs[c8 + c + 1] / den);
+          pk[0][c >> 1] = cvt_pk_bf16(xs[c8 + c], xs[c8 + c + 1]);
         } else {
           uint32_t tm[3];
           split3_pk(E::round(xs[c8 + c] / den), E::round(xs[c8 + c + 1] / den), tm);
