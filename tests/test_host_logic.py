@@ -82,7 +82,7 @@ def test_argument_errors_are_reported_before_any_launch():
 ])
 def test_page_layout_geometry(d, mb, vb, gs, dt, per_token):
     L = _ffi.make_page_layout(d, mb, vb, gs, dt)
-    assert L.off_keys == 0 and L.key_lane_major == (1 if d % 128 == 0 else 0)
+    assert L.off_keys == 0 and L.key_lane_major == (1 if d % 128 == 0 or d == 64 else 0)
     offs = [L.off_keys, L.off_meta, L.off_vdata, L.off_vscale, L.off_vzero]
     assert offs == sorted(offs) and all(o % 16 == 0 for o in offs)
     used = L.off_vzero + (d // gs) * 16 * (4 if dt == torch.float32 else 2)
