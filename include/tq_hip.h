@@ -314,6 +314,9 @@ void tq_time_next_key_kernel(void *start_event, void *stop_event);
  *                      library built with -DTQ_FUSED_PREP (TQ_EUNSUPPORTED otherwise): it measured slower.
  *   "prep_spin_limit"  with fuse_prep: how often a workgroup polls for the other workgroups' share of the
  *                      operands before it computes them itself (default 20000; 0 = never wait).
+ *   "append_parts"     measurement only: 3 (default) = the append entry points quantise keys and values,
+ *                      1 = keys only, 2 = values only (the other half of every page is left as it was), so
+ *                      that either kernel can be timed without the other running beside it.
  * Returns TQ_EINVAL for an unknown name or a value out of range.                                        */
 int tq_set_option(const char *name, int64_t value);
 

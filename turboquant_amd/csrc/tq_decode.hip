@@ -840,6 +840,7 @@ namespace tq {
 std::atomic<int> opt_fuse_prep{0};
 std::atomic<int> opt_prep_spin_limit{20000};
 std::atomic<int> opt_prep_units{0};
+std::atomic<int> opt_append_parts{3};
 }  // namespace tq
 
 namespace {
@@ -868,6 +869,11 @@ extern "C" int tq_set_option(const char* name, int64_t value) {
   if (!std::strcmp(name, "prep_spin_limit")) {
     if (value < 0 || value > 100000000) return TQ_EINVAL;
     opt_prep_spin_limit.store((int)value);
+    return TQ_OK;
+  }
+  if (!std::strcmp(name, "append_parts")) {
+    if (value < 1 || value > 3) return TQ_EINVAL;
+    opt_append_parts.store((int)value);
     return TQ_OK;
   }
   return TQ_EINVAL;

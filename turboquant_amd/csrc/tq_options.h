@@ -7,4 +7,5 @@ namespace tq {
 extern std::atomic<int> opt_fuse_prep;         // query preparation inside the page kernel's launch
 extern std::atomic<int> opt_prep_spin_limit;   // polls before a workgroup of that launch stops waiting for the others
 extern std::atomic<int> opt_prep_units;        // stand-alone preparation: one workgroup per (few heads, plane word) unit
+extern std::atomic<int> opt_append_parts;      // measurement: 3 keys and values (the product), 1 keys only, 2 values only
 }  // namespace tq

@@ -14,8 +14,41 @@ constexpr int TILE = TQ_PAGE_TOKENS;
 // tile sources: where the 16 vectors of a tile come from and which are valid
 // ------------------------------------------------------------------------------------
 
+// What the staging code of the matrix-core kernels needs to know about a tile, all of it uniform: slot s
+// of the tile exists iff lo <= s < hi, and its row starts `base + s * slot_stride()` elements into the
+// tensor.  A source hands it out for consecutive tiles through a walk (begin at a tile, step to the next),
+// so that the index arithmetic of a tile number (divisions by run-time sizes) is done once per group.
+struct TileAddr { int64_t base; int lo, hi; };
+
+// N uniform 32-bit loads p[at[k]] through the scalar cache with one wait (read-only inputs only: the
+// scalar cache does not see what vector stores of the same launch write)
+template <int N>
+__device__ __forceinline__ void sload(const int32_t* p, const int (&at)[N], int32_t (&v)[N]) {
+  static_assert(N == 2 || N == 4, "two or four at a time");
+  const int32_t* q[N];
+#pragma unroll
+  for (int k = 0; k < N; ++k) q[k] = p + __builtin_amdgcn_readfirstlane(at[k]);
+  if constexpr (N == 4) {
+    asm volatile("s_load_dword %0, %4, 0x0\n\ts_load_dword %1, %5, 0x0\n\ts_load_dword %2, %6, 0x0\n\t"
+                 "s_load_dword %3, %7, 0x0\n\ts_waitcnt lgkmcnt(0)"
+                 : "=&s"(v[0]), "=&s"(v[1]), "=&s"(v[2]), "=&s"(v[3])
+                 : "s"(q[0]), "s"(q[1]), "s"(q[2]), "s"(q[3])
+                 : "memory");
+  } else {
+    asm volatile("s_load_dword %0, %2, 0x0\n\ts_load_dword %1, %3, 0x0\n\ts_waitcnt lgkmcnt(0)"
+                 : "=&s"(v[0]), "=&s"(v[1])
+                 : "s"(q[0]), "s"(q[1])
+                 : "memory");
+  }
+}
+
 struct FlatSource {          // (n_vec, d) with a row stride
   int64_t n_vec, row_stride;
+  __device__ int64_t slot_stride() const { return row_stride; }
+  __device__ TileAddr tile_addr(int64_t tile) const {
+    const int64_t left = n_vec - tile * TILE;
+    return TileAddr{tile * TILE * row_stride, 0, (int)(left < 0 ? 0 : (left > TILE ? TILE : left))};
+  }
   struct TileRef { int64_t v0; };
   __device__ TileRef tile_ref(int64_t tile) const { return TileRef{tile * TILE}; }
   __device__ bool slot_off(const TileRef& r, int slot, int64_t& elem_off) const {
@@ -47,6 +80,49 @@ struct PagedSource {         // (b, t, h, :) strided, tokens mapped onto 16-toke
   // Optional ragged mode: the rows of all sequences lie one after another in one (rows, H, :) tensor; the
   // run of sequence b begins at row row0[b] (stride_b is unused, run_len gives its length).
   const int32_t* row0 = nullptr;
+  // (sequence, page slot window, head) of a tile, and of the tile after it (a walk that leaves the last
+  // sequence stays on its last tile): the divisions by run-time sizes are done once per group of tiles
+  struct Coord { int b, pg, h; };
+  __device__ Coord coord(int64_t tile) const {
+    Coord c;
+    c.h = (int)tile % H;
+    const int r = (int)tile / H;
+    c.pg = r % tiles_per_seq;
+    c.b = r / tiles_per_seq;
+    return c;
+  }
+  __device__ void next(Coord& c) const {
+    if (c.h + 1 < H) ++c.h;
+    else if (c.pg + 1 < tiles_per_seq) { c.h = 0; ++c.pg; }
+    else if (c.b + 1 < B) { c.h = 0; c.pg = 0; ++c.b; }
+  }
+  __device__ int64_t slot_stride() const { return stride_t; }
+  // Addresses of N tiles.  The per-sequence words come through the scalar cache, N at a time (they are
+  // inputs of the launch that no kernel writes; as ordinary loads they would be vector-memory loads with
+  // a full wait each, one after the other, in every pass of a persistent workgroup).
+  template <int N>
+  __device__ void tile_addrs(const Coord (&c)[N], TileAddr (&ta)[N], int (&lpage)[N]) const {
+    int32_t s0[N], lim[N], r0[N], blk[N], at[N];
+#pragma unroll
+    for (int m = 0; m < N; ++m) { at[m] = c[m].b; s0[m] = 0; lim[m] = k_max_i32; r0[m] = 0; blk[m] = 0; }
+    if (start_pos) sload<N>(start_pos, at, s0);
+    if (run_len) sload<N>(run_len, at, lim);
+    if (row0) sload<N>(row0, at, r0);
+#pragma unroll
+    for (int m = 0; m < N; ++m) {
+      lpage[m] = s0[m] / TILE + c[m].pg;
+      at[m] = c[m].b * src_stride + min(lpage[m], src_stride - 1);
+    }
+    if (src_table) sload<N>(src_table, at, blk);
+#pragma unroll
+    for (int m = 0; m < N; ++m) {
+      const int t0 = lpage[m] * TILE - s0[m];
+      const int64_t base = src_table ? (int64_t)blk[m] * stride_blk - (int64_t)t0 * stride_t
+                                     : (row0 ? (int64_t)r0[m] * stride_t : c[m].b * stride_b);
+      // slot s is token t0 + s of the run: it exists iff 0 <= t0 + s < min(run length, T)
+      ta[m] = TileAddr{base + c[m].h * stride_h + (int64_t)t0 * stride_t, -t0, min(lim[m], T) - t0};
+    }
+  }
   // tile index -> (b, page slot window, head)
   __device__ void decode(int tile, int& b, int& lpage, int& h) const {
     h = tile % H;

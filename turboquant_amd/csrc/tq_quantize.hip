@@ -8,6 +8,7 @@
 // in LDS; matrices are read column-coalesced from their row-major transposes.
 
 #include "tq_quantize.h"
+#include "tq_options.h"
 
 namespace tq {
 
@@ -854,6 +855,11 @@ static int append_runs(const void* k, const void* v, int dtype, const PagedSourc
   // kernels write disjoint bytes of the pages).  The value kernel goes to a side stream that is
   // forked from and joined back into the caller's stream with events, so the call stays ordered
   // on `stream` like any other.
+  // (measurement knob: one of the two kernels alone, to time it without the other beside it)
+  const int parts = opt_append_parts.load();
+  if (parts == 1) return launch_key(k, dtype, src, *layer, ks, 0, tiles, (hipStream_t)stream);
+  if (parts == 2)
+    return launch_value(v, dtype, src, layer->d, layout->group_size, layout->value_bits, vs, tiles, (hipStream_t)stream);
   if (tiles >= SIDE_MIN_TILES) {
     if (SideLane* lane = side_lane()) {
       hipStream_t st = (hipStream_t)stream;

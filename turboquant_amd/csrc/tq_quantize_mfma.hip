@@ -11,7 +11,8 @@
 //
 // Workgroups (4 wavefronts) are persistent: two per compute unit (about 75 KB of LDS
 // each), each looping over groups of TT = 8192/d vectors (TT/16 tiles of 16).  The next
-// group's vectors are fetched into registers while the current group is worked on, and
+// group's vectors are fetched into registers while the current group is worked on (the
+// tile lookups behind their addresses are uniform and go through the scalar cache), and
 // the matrix operand of a contraction is requested slice by slice while the previous
 // contraction runs, so no global-memory latency sits on the critical path.  The vectors' operand terms sit in LDS (row
 // stride padded so that the 16 rows of an MFMA operand fall into different banks);
@@ -21,7 +22,7 @@
 // the MFMA's row operand, so a lane ends up with four consecutive output columns
 // of one vector: terms for the next contraction go back to LDS as 8-byte writes and
 // the index / sign bits of a vector are gathered into 32-bit plane words with two
-// cross-lane exchanges.  The three contractions are separated by workgroup barriers
+// lane-swap instructions.  The three contractions are separated by workgroup barriers
 // because each needs complete rows of the previous result.
 
 #include <atomic>
@@ -204,12 +205,111 @@ __device__ __forceinline__ void contract(const uint16_t* a_terms, const uint16_t
   }
 }
 
-// OR a value over the four lanes that hold the same vector (lane & 15 equal)
+// OR / sum of a value over the four lanes that hold the same vector (lane & 15 equal); the result is valid in
+// the first of them (lanes 0..15).  The lane-swap instructions move rows of 16 / halves of 32 lanes through
+// the vector ALU: no LDS round trip and nothing to wait for.
 __device__ __forceinline__ uint32_t or_over_kb(uint32_t v) {
-  v |= (uint32_t)__shfl_xor((int)v, 16, 64);
-  v |= (uint32_t)__shfl_xor((int)v, 32, 64);
+  v |= (uint32_t)__builtin_amdgcn_permlane32_swap(v, v, false, false)[1];       // lanes 0..31: | lane + 32
+  v |= (uint32_t)__builtin_amdgcn_permlane16_swap(v, v, false, false)[1];       // lanes 0..15: | lane + 16
   return v;
 }
+// sum over groups of N neighbouring lanes (N = 4, 8 or 16, inside a row of 16) with DPP moves: quad swaps,
+// then half-row / row mirrors (every lane of a quad already holds the quad's sum, so a mirror pairs the quads)
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+template <int N>
+__device__ __forceinline__ float sum_lanes(float v) {
+  static_assert(N == 4 || N == 8 || N == 16, "4, 8 or 16 lanes");
+  v += dpp_mov<0xB1>(v);
+  v += dpp_mov<0x4E>(v);
+  if (N >= 8) v += dpp_mov<0x141>(v);
+  if (N >= 16) v += dpp_mov<0x140>(v);
+  return v;
+}
+__device__ __forceinline__ float sum_over_kb(float f) {
+  f += __uint_as_float(__builtin_amdgcn_permlane32_swap(__float_as_uint(f), __float_as_uint(f), false, false)[1]);
+  f += __uint_as_float(__builtin_amdgcn_permlane16_swap(__float_as_uint(f), __float_as_uint(f), false, false)[1]);
+  return f;
+}
+
+// Staging of a group's vectors: a thread holds its 16-byte chunks of the NEXT group in registers while the
+// current group is worked on, so the latency of the loads is never waited for.  The KQ_THREADS chunks of
+// one round lie in one tile.  Everything that depends on the tile number is uniform and comes from one
+// walk over the group's MT consecutive tiles (TileAddr); a lane only adds its own offset, which is the
+// same for every group (slot * row stride + chunk, kept in registers on purpose).
+template <int DT, int D, class Source>
+struct XStage {
+  using S = typename Elem<DT>::storage;
+  using Gm = KeyGeom<D>;
+  static constexpr int CH = 16 / (int)sizeof(S);                // elements per 16-byte chunk
+  static constexpr int CPR = D / CH;                            // chunks per vector
+  static constexpr int PER = Gm::TT * CPR / KQ_THREADS;         // rounds
+  static constexpr int RPR = KQ_THREADS / CPR;                  // vectors per round (<= 16)
+  static constexpr int NSL = TILE / RPR;                        // rounds per tile = slots a thread serves
+  static_assert(RPR <= TILE && TILE % RPR == 0 && PER == Gm::MT * NSL, "a round of chunks stays inside one tile");
+  u32x4 xbuf[PER];
+  unsigned xok = 0;
+  TileAddr ta[Gm::MT];                                          // tiles of the group looked up last
+  bool live[Gm::MT];
+  int w_b = 0, w_lpage = 0, w_h = 0;                            // (paged) where the tile this wavefront writes goes
+  int64_t lane_off[NSL];
+  int slot[NSL];
+
+  __device__ __forceinline__ void init(const Source& src, int tid) {
+    const int tr = tid / CPR, ck = tid % CPR;
+#pragma unroll
+    for (int k = 0; k < NSL; ++k) {
+      slot[k] = tr + RPR * k;
+      lane_off[k] = (int64_t)slot[k] * src.slot_stride() + ck * CH;
+    }
+  }
+  // uniform part for `group`: tile addresses, and (paged sources) the coordinates of tile group * MT + wtile
+  __device__ __forceinline__ void lookup(const Source& src, int64_t group, int64_t n_tiles, int wtile) {
+    const int64_t tile0 = group * Gm::MT;
+    const int64_t first = tile0 < n_tiles ? tile0 : 0;
+#pragma unroll
+    for (int m = 0; m < Gm::MT; ++m) live[m] = tile0 + m < n_tiles;
+    if constexpr (std::is_same<Source, PagedSource>::value) {
+      PagedSource::Coord c[Gm::MT];
+      int lpage[Gm::MT];
+      c[0] = src.coord(first);
+#pragma unroll
+      for (int m = 1; m < Gm::MT; ++m) { c[m] = c[m - 1]; src.next(c[m]); }
+      src.template tile_addrs<Gm::MT>(c, ta, lpage);
+#pragma unroll
+      for (int m = 0; m < Gm::MT; ++m)
+        if (m == wtile) { w_b = c[m].b; w_lpage = lpage[m]; w_h = c[m].h; }
+    } else {
+#pragma unroll
+      for (int m = 0; m < Gm::MT; ++m) ta[m] = src.tile_addr(first + m);
+    }
+  }
+  // request the chunks of the group looked up last (unconditional loads: a load under a branch makes every
+  // later wait a wait for all loads; slots that do not exist read the first vector and are zeroed when stored)
+  __device__ __forceinline__ void issue(const void* x) {
+    xok = 0;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int m = j / NSL, k = j % NSL;
+      const bool ok = live[m] && slot[k] >= ta[m].lo && slot[k] < ta[m].hi;
+      xbuf[j] = *(const u32x4*)((const S*)x + (ok ? ta[m].base + lane_off[k] : 0));
+      xok |= (unsigned)ok << j;
+    }
+  }
+  // registers -> the LDS tile [TT][XRS], validity flags
+  template <int XRS>
+  __device__ __forceinline__ void store(S* sx, int* svalid, int tid) const {
+    const int tr = tid / CPR, ck = tid % CPR;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const bool ok = (xok >> j) & 1;
+      *(u32x4*)(sx + (RPR * j + tr) * XRS + ck * CH) = ok ? xbuf[j] : u32x4{0, 0, 0, 0};
+      if (ck == 0) svalid[RPR * j + tr] = ok;
+    }
+  }
+};
 
 // MSE_ONLY (the stage-1 quantiser alone: no residual, no signs) is a template parameter: as a
 // run-time flag it adds control flow that costs the register allocator its footing.
@@ -223,7 +323,6 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
   using Sm = KeySmem<DT, D>;
   constexpr int TT = Gm::TT, MT = Gm::MT, NPW = Gm::NPW, RS = Gm::RS, W = Gm::W, NA1 = InTerms<DT>::N;
   constexpr int XRS = Sm::XRS, TPR = Gm::TPR, SEG = Gm::SEG;
-  constexpr int CH = 16 / (int)sizeof(S);                       // elements per 16-byte chunk of the input
   const int tid0 = threadIdx.x, wave0 = __builtin_amdgcn_readfirstlane(tid0 >> 6);
   const int mb = ly.mse_bits, n_thr = (1 << mb) - 1;
   const int64_t n_groups = (n_tiles + MT - 1) / MT;             // a group = the TT vectors of one pass
@@ -247,38 +346,11 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
     split3_pk(ly.centroids[tid0], 0.0f, t);
     slut[tid0] = u32x2{(t[0] & 0xffffu) | (t[1] << 16), t[2] & 0xffffu};
   }
-  // (1) staging: a thread holds its 16-byte chunks of the NEXT group in registers while the
-  //     current group is worked on, so the latency of the loads is never waited for.  The
-  //     KQ_THREADS chunks of one round lie in one tile, so the tile lookup is wavefront-uniform.
-  constexpr int CPR = D / CH;                                   // chunks per vector
-  constexpr int PER = TT * CPR / KQ_THREADS;                    // rounds
-  constexpr int RPR = KQ_THREADS / CPR;                         // vectors per round (<= 16)
-  static_assert(RPR <= TILE && TILE % RPR == 0, "a round of chunks stays inside one tile");
-  u32x4 xbuf[PER];
-  unsigned xok = 0;
-  typename Source::TileRef xref[PER];                           // tile lookups of the group to fetch next
-  auto lookup_x = [&](int64_t group) {
-#pragma unroll
-    for (int j = 0; j < PER; ++j) {
-      const int64_t tile = group * MT + (RPR * j) / TILE;
-      xref[j] = src.tile_ref(tile < n_tiles ? tile : 0);
-    }
-  };
-  auto issue_x = [&](int64_t group, int tr, int ck) {
-    xok = 0;
-#pragma unroll
-    for (int j = 0; j < PER; ++j) {
-      const int64_t tile = group * MT + (RPR * j) / TILE;
-      int64_t off = 0;
-      const bool ok = src.slot_off(xref[j], (RPR * j + tr) % TILE, off) && tile < n_tiles;
-      // unconditional load (a load under a branch makes every later wait a wait for all loads);
-      // slots that do not exist read the first vector and are zeroed when they are stored
-      xbuf[j] = *(const u32x4*)((const S*)x + (ok ? off : 0) + ck * CH);
-      xok |= (unsigned)ok << j;
-    }
-  };
-  lookup_x(blockIdx.x);
-  issue_x(blockIdx.x, tid0 / CPR, tid0 % CPR);
+  // (1) staging (XStage): the next group's chunks wait in registers while the current group is worked on
+  XStage<DT, D, Source> stg;
+  stg.init(src, tid0);
+  stg.lookup(src, blockIdx.x, n_tiles, wave0 % MT);
+  stg.issue(x);
 
   for (int64_t g = blockIdx.x; g < n_groups; g += gridDim.x) {
   // The thread index is re-read through an opaque copy in every pass: otherwise the compiler
@@ -286,26 +358,18 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
   int tid = tid0, wave = wave0;
   asm volatile("" : "+v"(tid), "+s"(wave));
   const int lane = tid & 63, n = lane & 15, kb = lane >> 4;
-  const int tr = tid / CPR, ck = tid % CPR;
   const int64_t tile0 = g * MT;
-  lookup_x(g + gridDim.x);                                      // read long before issue_x needs it
-  // page of the tile this wavefront will write, looked up now so that the write phase does not
-  // wait for it (clamped into the table: a tile without a single existing slot may lie beyond it)
+  // coordinates of the tile this wavefront writes: looked up one pass ago together with this group's loads;
+  // then the lookups of the group to fetch next (long before issue() needs them)
+  const int wr_b = stg.w_b, wr_lpage = stg.w_lpage, wr_h = stg.w_h;
+  stg.lookup(src, g + gridDim.x, n_tiles, wave % MT);
+  // page of that tile, read now so that the write phase does not wait for it (a page outside the table or
+  // the pool comes back as -1 and is not written)
   int64_t wpage = 0;
   if constexpr (!std::is_same<Sink, KeyFlatSink>::value) {
-    const int64_t wt = tile0 + wave % MT;
-    if (wt < n_tiles) {
-      int b, lpage, h;
-      src.decode((int)wt, b, lpage, h);
-      wpage = checked_page(sink.block_table, sink.max_pages, sink.num_pages, b, lpage);
-    }
+    if (tile0 + wave % MT < n_tiles) wpage = checked_page(sink.block_table, sink.max_pages, sink.num_pages, wr_b, wr_lpage);
   }
-#pragma unroll
-  for (int j = 0; j < PER; ++j) {
-    const bool ok = (xok >> j) & 1;
-    *(u32x4*)(sx + (RPR * j + tr) * XRS + ck * CH) = ok ? xbuf[j] : u32x4{0, 0, 0, 0};
-    if (ck == 0) svalid[RPR * j + tr] = ok;
-  }
+  stg.template store<XRS>(sx, svalid, tid);
   __syncthreads();
   // (2) norm, unit vector in the input dtype (quantizer.py:136-138), its bf16 terms.
   //     TPR neighbouring threads share a vector, 32 coordinates each.
@@ -316,8 +380,7 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
     float ss = 0.0f;
 #pragma unroll
     for (int c = 0; c < SEG; ++c) ss += xs[c] * xs[c];
-#pragma unroll
-    for (int o = 1; o < TPR; o <<= 1) ss += __shfl_xor(ss, o, 64);
+    ss = sum_lanes<TPR>(ss);
     const float nrm = E::round(sqrtf(ss));
     const float den = E::round(nrm + 1e-10f);
     if (seg == 0) snorm[t] = nrm;
@@ -417,7 +480,7 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
     }
   }
   __syncthreads();
-  if (mse_only) issue_x(g + gridDim.x, tr, ck);
+  if (mse_only) stg.issue(x);
   if (!mse_only) {
     // (4) x_hat = (c Pi) * norm ; r = x - x_hat ; ||r||^2 partial sums ; r as bf16 terms (quantizer.py:241-245)
     contract<D, 3>(terms, ly.PiT_split, ly.S_split, wave, lane, mr, acc);
@@ -444,12 +507,11 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
 #pragma unroll
         for (int a = 0; a < 3; ++a) *(u32x2*)(terms + ((size_t)a * TT + t) * RS + col0) = u32x2{lo[a], hi[a]};
       }
-      rs += __shfl_xor(rs, 16, 64);
-      rs += __shfl_xor(rs, 32, 64);
+      rs = sum_over_kb(rs);
       if (kb == 0) spart[wave * TT + t] = rs;
     }
     __syncthreads();
-    issue_x(g + gridDim.x, tr, ck);                                     // the input tile is free: fetch the next group
+    stg.issue(x);                                               // the input tile is free: fetch the next group
     if (tid < TT) {
       float v = 0.0f;
 #pragma unroll
@@ -533,9 +595,7 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
       // a tile none of whose slots exists may lie beyond the block table: do not look it up
       // (and a page outside the table or the pool is not written)
       if (__builtin_amdgcn_ballot_w64(lane < TILE && svalid[16 * m + lane]) == 0 || wpage < 0) continue;
-      int b, lpage, h;
-      src.decode((int)tile, b, lpage, h);
-      uint8_t* pg = sink.pool + (wpage * src.H + h) * (int64_t)L.page_bytes;
+      uint8_t* pg = sink.pool + (wpage * src.H + wr_h) * (int64_t)L.page_bytes;
       for (int p = wave / MT; p < planes; p += NSUB) {
 #pragma unroll
         for (int e = lane; e < W * TILE; e += 64) {
@@ -555,6 +615,7 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
   __syncthreads();                                              // the next group overwrites what the writers read
   }
 }
+
 
 __host__ static bool aligned_for_chunks(const void* x, int dtype, const FlatSource& s) {
   const int64_t ch = 16 / elem_bytes(dtype);
