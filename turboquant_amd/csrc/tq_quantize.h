@@ -24,7 +24,7 @@ struct TileAddr { int64_t base; int lo, hi; };
 // scalar cache does not see what vector stores of the same launch write)
 template <int N>
 __device__ __forceinline__ void sload(const int32_t* p, const int (&at)[N], int32_t (&v)[N]) {
-  static_assert(N == 2 || N == 4, "two or four at a time");
+  static_assert(N == 1 || N == 2 || N == 4, "one, two or four at a time");
   const int32_t* q[N];
 #pragma unroll
   for (int k = 0; k < N; ++k) q[k] = p + __builtin_amdgcn_readfirstlane(at[k]);
@@ -34,6 +34,8 @@ __device__ __forceinline__ void sload(const int32_t* p, const int (&at)[N], int3
                  : "=&s"(v[0]), "=&s"(v[1]), "=&s"(v[2]), "=&s"(v[3])
                  : "s"(q[0]), "s"(q[1]), "s"(q[2]), "s"(q[3])
                  : "memory");
+  } else if constexpr (N == 1) {
+    asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=&s"(v[0]) : "s"(q[0]) : "memory");
   } else {
     asm volatile("s_load_dword %0, %2, 0x0\n\ts_load_dword %1, %3, 0x0\n\ts_waitcnt lgkmcnt(0)"
                  : "=&s"(v[0]), "=&s"(v[1])

@@ -336,7 +336,7 @@ value_chunk_kernel(const void* __restrict__ v, Source src, int d, int gs, Sink s
   static_assert(DT != TQ_F32, "16-bit inputs");
   const int tid = threadIdx.x, tile = blockIdx.x;
   const int cpt = d >> 3;                          // chunks (threads) per token
-  const int t = tid / cpt, ck = tid - t * cpt;     // token slot, chunk
+  const int t = tid >> (31 - __builtin_clz(cpt)), ck = tid & (cpt - 1);     // token slot, chunk (head_dim 64 / 128 / 256)
   const int tpg = gs >> 3;                         // threads per group (power of two, <= 16)
   // a thread's 8 codes are one word of 8 * VB bits; the words of a chunk's 16 tokens lie together
   // (rows padded by 16 bytes), so that the thread that assembles half a channel field reads the
@@ -347,18 +347,26 @@ value_chunk_kernel(const void* __restrict__ v, Source src, int d, int gs, Sink s
   unsigned char* scode = smem;                     // [d / 8] rows of CROW bytes
   int* svalid = (int*)(smem + (size_t)cpt * CROW); // [TILE]
 
-  const typename Source::TileRef ref = src.tile_ref(tile);
-  int64_t off;
-  const bool ok = src.slot_off(ref, t, off);
+  // where the tile's rows are and which of its slots exist: uniform, looked up through the scalar cache
+  TileAddr ta;
   // page lookup issued together with the input load (clamped into the table: a tile without a
   // single existing slot may lie beyond it, and then nothing is stored anyway)
   int64_t page = 0;
   int head = 0;
-  if constexpr (!std::is_same<Sink, ValFlatSink>::value) {
-    int b, lpage;
-    src.decode(tile, b, lpage, head);
-    page = checked_page(sink.block_table, sink.max_pages, sink.num_pages, b, lpage);
+  if constexpr (std::is_same<Source, PagedSource>::value) {
+    PagedSource::Coord c[1] = {src.coord(tile)};
+    TileAddr ta1[1];
+    int lpage[1];
+    src.template tile_addrs<1>(c, ta1, lpage);
+    ta = ta1[0];
+    head = c[0].h;
+    if constexpr (!std::is_same<Sink, ValFlatSink>::value)
+      page = checked_page(sink.block_table, sink.max_pages, sink.num_pages, c[0].b, lpage[0]);
+  } else {
+    ta = src.tile_addr(tile);
   }
+  const bool ok = t >= ta.lo && t < ta.hi;
+  const int64_t off = ta.base + (int64_t)t * src.slot_stride();
   const bool page_ok = page >= 0;                    // uniform over the workgroup; false: nothing is stored
   // unconditional load (slots that do not exist read the first vector)
   const uint4 raw = *(const uint4*)((const uint16_t*)v + (ok ? off : 0) + ck * 8);
@@ -384,11 +392,18 @@ value_chunk_kernel(const void* __restrict__ v, Source src, int d, int gs, Sink s
     lo = fminf(lo, x[i]);
     hi = fmaxf(hi, x[i]);
   }
-  for (int o = 1; o < tpg; o <<= 1) {              // the threads of a group are neighbouring lanes
-    lo = fminf(lo, __shfl_xor(lo, o, 64));
-    hi = fmaxf(hi, __shfl_xor(hi, o, 64));
-    has_nan |= __shfl_xor(has_nan, o, 64);
-  }
+  // the threads of a group are neighbouring lanes inside a row of 16: DPP moves (quad swaps, then half-row and
+  // row mirrors, which pair quads that already agree) instead of shuffles through the LDS
+  auto reduce_step = [&](auto ctrl_c) {
+    constexpr int CTRL = decltype(ctrl_c)::value;
+    lo = fminf(lo, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, lo), CTRL, 0xF, 0xF, true)));
+    hi = fmaxf(hi, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, hi), CTRL, 0xF, 0xF, true)));
+    has_nan |= __builtin_amdgcn_update_dpp(0, has_nan, CTRL, 0xF, 0xF, true);
+  };
+  if (tpg >= 2) reduce_step(std::integral_constant<int, 0xB1>{});
+  if (tpg >= 4) reduce_step(std::integral_constant<int, 0x4E>{});
+  if (tpg >= 8) reduce_step(std::integral_constant<int, 0x141>{});
+  if (tpg >= 16) reduce_step(std::integral_constant<int, 0x140>{});
   if (has_nan) lo = hi = __uint_as_float(0x7fc00000u);       // torch min/max propagate NaN
   const float levels = (float)((1 << VB) - 1);
   float sc = round_hw<DT>(round_hw<DT>(hi - lo) / levels);
@@ -401,7 +416,7 @@ value_chunk_kernel(const void* __restrict__ v, Source src, int d, int gs, Sink s
   // followed by one residual correction q0 + (a - q0 s)(1/s) does both (the fused residual is exact for
   // a tie).  Used when the scale is an ordinary number; everything else takes the division.
   const bool fast_div = DT == TQ_BF16 && sc > 0x1p-60f && sc < 0x1p60f;
-  const float rsc = 1.0f / sc;
+  const float rsc = __builtin_amdgcn_rcpf(sc);     // any reciprocal good to an ulp will do (checked over all bf16 pairs)
   uint32_t codes = 0;                              // 8 codes, VB bits each, channel order
   float quo[8];
   if (fast_div) {                // every a of the group is finite and at most (levels + 1) * sc < 2^64 then

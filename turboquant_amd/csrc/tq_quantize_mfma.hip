@@ -388,10 +388,10 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
       // Quotients of bf16 numbers, rounded to bf16: a / den is either exactly a rounding tie or at least
       // 2^-17 (relative) away from one, so q0 = a (1/den) with one residual correction, which is exact
       // for a tie, rounds like the correctly rounded quotient.  (Compared with the division over every
-      // pair of bf16 numbers with |a| <= 2 den and den in the range below: the only difference is that
-      // a = -0 gives +0, which no product sum can tell apart.)  |x_i| <= 2 den holds for any finite norm.
+      // pair of bf16 numbers with |a| <= 2 den and den in the range below, also with the reciprocal an ulp
+      // off either way: the only difference is that a = -0 gives +0, which no product sum can tell apart.)  |x_i| <= 2 den holds for any finite norm.
       if (den > 0x1p-60f && den < 0x1p60f) {
-        const float rden = 1.0f / den;
+        const float rden = __builtin_amdgcn_rcpf(den);          // any reciprocal good to an ulp will do
 #pragma unroll
         for (int c = 0; c < SEG; ++c) {
           const float q0 = xs[c] * rden;
