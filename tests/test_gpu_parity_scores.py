@@ -101,6 +101,39 @@ def test_config4_full_size_decode_against_the_oracle(gpu):
         assert (out[b:b + 1].float() - want.float()).abs().max() <= 2 ** -7 * want.float().abs().max() + 1e-3, b
 
 
+def test_config5_layer_at_full_size_against_the_oracle(gpu):
+    """One attention layer of the 32-layer serving step at its full size: batch 32 x 32768 context tokens, 32
+    query / 8 KV heads of 128, 3-bit keys, 4-bit values in groups of 32 (the shape every layer of the
+    backend decode-step benchmark runs), pages a random permutation, default split count, sequences of
+    unequal length.  Four of the 32 sequences (the shortest, the longest and two in between) against the
+    oracle's de-quantise-everything attention on the same store (score.py:84-173)."""
+    B, Hq, Hkv, d, N = 32, 32, 8, 128, 32768
+    pages = N // 16
+    pool, tq = _make_pool(gpu, d, 3, 4, Hkv, B * pages, torch.bfloat16, seed=42 + 7 * 5)
+    g = torch.Generator().manual_seed(5)
+    table = torch.randperm(B * pages, generator=g).to(torch.int32).view(B, pages).to(gpu)
+    gg = torch.Generator(device=gpu).manual_seed(5)         # keys and values straight on the card (1 GB of them)
+    for b0 in range(0, B, 4):
+        _progress(f"config 5 layer: sequences {b0}..{b0 + 3}: quantise")
+        k = torch.randn(4, N, Hkv, d, generator=gg, device=gpu).bfloat16()
+        v = torch.randn(4, N, Hkv, d, generator=gg, device=gpu).bfloat16()
+        pool.append(k, v, table[b0:b0 + 4])
+        del k, v
+    q = torch.randn(B, Hq, d, generator=g).bfloat16()
+    lens = torch.randint(N // 2, N + 1, (B,), generator=g).to(torch.int32)
+    lens[0], lens[B - 1] = N, N // 2 + 3
+    out = pool.decode_attention(q.to(gpu), table, lens.to(gpu), max_len=N).cpu()
+    torch.cuda.synchronize()
+    prm = params_of(tq)
+    for b in (0, 9, 20, B - 1):
+        n = int(lens[b])
+        kc, vc = _store_from_oracle_view(pool, table[b], n)
+        want = O.hybrid_attention(q[b:b + 1], kc, vc, n, prm, Hkv, None, None)
+        c = cosine(out[b:b + 1], want)
+        _progress(f"config 5 layer: sequence {b} ({n} tokens) cosine {c:.8f}")
+        assert c >= COS_GATE, (b, c)
+
+
 @pytest.mark.parametrize("d,key_bits,dtype", [(576, 4, torch.bfloat16), (576, 3, torch.float32), (192, 4, torch.float16)])
 def test_wide_head_quantiser_against_the_oracle(gpu, d, key_bits, dtype):
     """Head sizes without a matrix-core quantiser (the fp32 vector-ALU kernel): 576 with 4-bit keys is the shape
