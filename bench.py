@@ -463,6 +463,8 @@ def main():
     ap.add_argument("--no-backend-step", action="store_true",
                     help="skip the full-decode-step leg (32-layer transformer through the backend hooks, ~60 GB)")
     ap.add_argument("--context", type=int, default=131072, help="context tokens per sequence of the main workload")
+    ap.add_argument("--quantize-only", action="store_true",
+                    help="run the prefill-quantize leg alone and print its object (for profiles of its kernels)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the path has no cross-GPU step and this build runs on a single MI355X; "
@@ -477,6 +479,11 @@ def main():
         raise SystemExit("turboquant_amd/libtq_hip.so is missing; run `python -m turboquant_amd.build` first")
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
+
+    if args.quantize_only:
+        quant, _keep = quantize_bench(device, args.steps, args.warmup)
+        print(json.dumps({"quantize": quant}))
+        return
 
     main_w = DecodeWorkload("long-context decode", 4, args.context, 16, 2, 256, 3, 2, n_pools=4, seed=3,
                             dist="student_t5", device=device)
