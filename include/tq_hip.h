@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define TQ_ABI_VERSION 1
+#define TQ_ABI_VERSION 2
 
 enum { TQ_F32 = 0, TQ_F16 = 1, TQ_BF16 = 2 };
 
@@ -72,6 +72,20 @@ typedef struct tq_layer {
    * largest row norm of S.  NULL selects the two-kernel preparation.                    */
   const float *Pi_colsum, *S_colsum;
   float S_rownorm_max;
+  /* Optional operands of the centroid contraction x_hat = c[idx] Pi (quantizer.py:160) of the matrix-core
+   * key quantiser, head_dim 128, codebooks whose Walsh expansion has only single-bit terms (the symmetric
+   * 1- and 2-bit Lloyd-Max codebooks).  The index bit planes are the fp4 operand of the block-scaled
+   * 16x16x128 MFMA; Pi^T is its fp6 operand, five fp6 (e2m3) digits per value:
+   *   PiT_fp6       uint32 [d/16 row tiles][d/128][5 terms][64 lanes][6]: lane (row % 16, block b) holds the
+   *                 32 six-bit codes of (row, contraction indices 32 b ..), index s at bits 6 s .. 6 s + 5;
+   *                 contraction index 32 w + 8 (c % 4) + c / 4 is coordinate c of plane word w, and the value is
+   *                 Pi^T[row][coordinate] divided by 0.5, 1, 2, 0.5 for c % 4 = 0..3 (the fp4 values of a set
+   *                 bit at that position): v = 2^E sum_t digit_t 2^(-2 - 5 t), 2^E >= the block's largest |v|;
+   *   PiT_fp6_scale uint32 [d/16][d/128][64 lanes][2]: E8M0 codes 127 + E - 2 - 5 t, terms 0..3 in the bytes of
+   *                 the first word, term 4 in the lowest byte of the second.
+   * Needs Pi_colsum.  NULL selects the bf16 term products for this contraction too.  (turboquant_amd._ffi
+   * .split_fp6x5 builds both.)                                                                            */
+  const uint32_t *PiT_fp6, *PiT_fp6_scale;
   /* Walsh expansion of the codebook over the index bits, used by the decode
    * kernel: centroids[idx] = term_const + sum_t term_coef[t] * parity(idx & term_mask[t]).
    * Filled by tq_layer_fill_terms from the host copy of the centroids.          */
@@ -314,6 +328,8 @@ void tq_time_next_key_kernel(void *start_event, void *stop_event);
  *                      library built with -DTQ_FUSED_PREP (TQ_EUNSUPPORTED otherwise): it measured slower.
  *   "prep_spin_limit"  with fuse_prep: how often a workgroup polls for the other workgroups' share of the
  *                      operands before it computes them itself (default 20000; 0 = never wait).
+ *   "fp6_centroids"    1 (default): the key quantiser takes the fp6 x fp4 centroid contraction when the layer
+ *                      carries PiT_fp6; 0: always the bf16 term products (for A/B runs).
  *   "append_parts"     measurement only: 3 (default) = the append entry points quantise keys and values,
  *                      1 = keys only, 2 = values only (the other half of every page is left as it was), so
  *                      that either kernel can be timed without the other running beside it.

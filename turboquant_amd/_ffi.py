@@ -16,7 +16,7 @@ import torch
 TQ_F32, TQ_F16, TQ_BF16 = 0, 1, 2
 TQ_PAGE_TOKENS = 16
 TQ_MAX_TERMS = 15
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 # TQ_HIP_LIBRARY overrides the in-tree library (e.g. to compare two builds)
 _LIB_PATH = os.environ.get("TQ_HIP_LIBRARY") or os.path.join(os.path.dirname(os.path.abspath(__file__)), "libtq_hip.so")
@@ -36,6 +36,7 @@ class TqLayer(C.Structure):
         ("qjl_scale", C.c_float),
         ("Pi_split", C.c_void_p), ("PiT_split", C.c_void_p), ("S_split", C.c_void_p), ("ST_split", C.c_void_p),
         ("Pi_colsum", C.c_void_p), ("S_colsum", C.c_void_p), ("S_rownorm_max", C.c_float),
+        ("PiT_fp6", C.c_void_p), ("PiT_fp6_scale", C.c_void_p),
         ("n_terms", C.c_int32),
         ("term_mask", C.c_int32 * TQ_MAX_TERMS),
         ("term_coef", C.c_float * TQ_MAX_TERMS),
@@ -170,7 +171,9 @@ def make_layer(d: int, mse_bits: int, Pi: torch.Tensor, PiT: torch.Tensor, centr
     ly.centroids, ly.thresholds = centroids.data_ptr(), thresholds.data_ptr()
     ly.qjl_scale = math.sqrt(math.pi / 2.0) / d
     if splits is not None:
-        pi_s, pit_s, s_s, st_s = splits
+        pi_s, pit_s, s_s, st_s = splits[:4]
+        if len(splits) > 4 and splits[4] is not None:
+            ly.PiT_fp6, ly.PiT_fp6_scale = splits[4][0].data_ptr(), splits[4][1].data_ptr()
         ly.Pi_split = None if pi_s is None else pi_s.data_ptr()
         ly.PiT_split = None if pit_s is None else pit_s.data_ptr()
         ly.S_split = None if s_s is None else s_s.data_ptr()
@@ -199,6 +202,70 @@ def split_bf16x3(m: torch.Tensor) -> torch.Tensor:
         rest = rest - term.float()
     t = torch.stack(parts).view(3, d // 16, 16, d // 32, 4, 8)      # term, row tile, n, kblk, kb, j
     return t.permute(0, 1, 3, 4, 2, 5).contiguous().view(torch.int16)
+
+
+FP6_TERMS = 5
+
+
+def split_fp6x5(m: torch.Tensor):
+    """fp32 (d, d) matrix (row = output coordinate, column = contraction index), d a multiple of 128 -> the
+    operands of the block-scaled fp6 x fp4 MFMA (16x16x128) whose other operand is a bit-plane word turned
+    into fp4 codes in place: (codes, scales).
+
+    The 32 coordinates of plane word w reach the MFMA at contraction index 32 w + 8 (c % 4) + c // 4
+    (c = coordinate inside the word) with the fp4 values 0.5, 1, 2, 0.5 for c % 4 = 0, 1, 2, 3, so the
+    matrix is permuted the same way and divided by those factors.  Each row's 32 values of a block are
+    written as v = 2^E * sum_t digit_t * 2^(-2 - 5 t) with 2^E >= max |v| and FP6_TERMS fp6 (e2m3) digits
+    (each rounds what the digits before it left, to nearest even; good to 2^-23 of the block maximum).
+
+    codes  int32 [d // 16][d // 128][FP6_TERMS][64 lanes][6]: lane (row % 16, block b) holds its 32 six-bit
+           codes, contraction index s of the block at bits 6 s .. 6 s + 5 of the lane's 192 bits;
+    scales int32 [d // 16][d // 128][64 lanes][2]: the E8M0 codes 127 + E - 2 - 5 t of the lane's (row,
+           block), terms 0..3 in the bytes of the first word, term 4 in the lowest byte of the second."""
+    import numpy as np
+    a = m.detach().double().cpu().numpy()
+    d = a.shape[0]
+    if a.ndim != 2 or a.shape[1] != d or d % 128:
+        raise ValueError("split_fp6x5 needs a square matrix whose size is a multiple of 128")
+    s_idx = np.arange(32)
+    coord = 4 * (s_idx % 8) + s_idx // 8                       # coordinate inside the word at contraction index s
+    factor = np.array([0.5, 1.0, 2.0, 0.5])[coord % 4]
+    blocks = a.reshape(d, d // 32, 32)[:, :, coord] / factor    # [row][block][s]
+    mx = np.abs(blocks).max(-1)
+    e = np.where(mx > 0, np.ceil(np.log2(np.maximum(mx, 1e-300))), -60.0)
+    e = np.where(np.abs(blocks).max(-1) > 2.0 ** e, e + 1, e).astype(np.int64)       # guard against log2 rounding
+    x = 4.0 * blocks / (2.0 ** e)[..., None]
+    codes = np.zeros((FP6_TERMS,) + blocks.shape, dtype=np.uint64)
+    for t in range(FP6_TERMS):
+        mag = np.minimum(np.abs(x), 7.5)
+        inv = np.where(mag < 2.0, 8.0, np.where(mag < 4.0, 4.0, 2.0))
+        r = np.rint(mag * inv) / inv
+        ex = np.where(r < 1.0, 0, np.where(r < 2.0, 1, np.where(r < 4.0, 2, 3)))
+        unit = np.where(ex <= 1, 8.0, np.where(ex == 2, 4.0, 2.0))
+        man = (r * unit).astype(np.int64) - np.where(ex == 0, 0, 8)
+        neg = (x < 0) & (r != 0)
+        codes[t] = (neg.astype(np.uint64) << np.uint64(5)) | (ex.astype(np.uint64) << np.uint64(3)) | man.astype(np.uint64)
+        x = 32.0 * (x - np.where(x < 0, -r, r))
+    # 32 six-bit codes -> 192 bits -> 6 little-endian dwords
+    bits = np.zeros((FP6_TERMS,) + blocks.shape[:2] + (6,), dtype=np.uint64)
+    for s_ in range(32):
+        lo = 6 * s_
+        w, sh = lo // 32, lo % 32
+        bits[..., w] |= (codes[..., s_] << np.uint64(sh)) & np.uint64(0xFFFFFFFF)
+        if sh > 26:
+            bits[..., w + 1] |= codes[..., s_] >> np.uint64(32 - sh)
+    # [t][row][block][6] -> [row tile][chunk of 128][t][lane = (row % 16) + 16 (block % 4)][6]
+    bits = bits.reshape(FP6_TERMS, d // 16, 16, d // 128, 4, 6).transpose(1, 3, 0, 4, 2, 5)
+    packed = np.ascontiguousarray(bits).reshape(d // 16, d // 128, FP6_TERMS, 64, 6).astype(np.uint32)
+    sc = 127 + e[..., None] - 2 - 5 * np.arange(FP6_TERMS)                             # [row][block][t]
+    if sc.min() < 0 or sc.max() > 254:
+        raise ValueError("matrix values out of the range of the block scales")
+    sc = sc.astype(np.uint32)
+    words = np.stack([sc[..., 0] | (sc[..., 1] << 8) | (sc[..., 2] << 16) | (sc[..., 3] << 24), sc[..., 4]], axis=-1)
+    words = words.reshape(d // 16, 16, d // 128, 4, 2).transpose(0, 2, 3, 1, 4)
+    scales = np.ascontiguousarray(words).reshape(d // 16, d // 128, 64, 2).astype(np.uint32)
+    dev = m.device
+    return (torch.from_numpy(packed.view(np.int32)).to(dev), torch.from_numpy(scales.view(np.int32)).to(dev))
 
 
 def make_page_layout(d: int, mse_bits: int, value_bits: int, group_size: int, dtype: torch.dtype) -> TqPageLayout:

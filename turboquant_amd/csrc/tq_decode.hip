@@ -841,6 +841,7 @@ std::atomic<int> opt_fuse_prep{0};
 std::atomic<int> opt_prep_spin_limit{20000};
 std::atomic<int> opt_prep_units{0};
 std::atomic<int> opt_append_parts{3};
+std::atomic<int> opt_fp6_centroids{1};
 }  // namespace tq
 
 namespace {
@@ -871,6 +872,7 @@ extern "C" int tq_set_option(const char* name, int64_t value) {
     opt_prep_spin_limit.store((int)value);
     return TQ_OK;
   }
+  if (!std::strcmp(name, "fp6_centroids")) { opt_fp6_centroids.store(value != 0); return TQ_OK; }
   if (!std::strcmp(name, "append_parts")) {
     if (value < 1 || value > 3) return TQ_EINVAL;
     opt_append_parts.store((int)value);

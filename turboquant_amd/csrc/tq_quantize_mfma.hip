@@ -29,6 +29,7 @@
 
 #include "tq_quantize.h"
 #include "tq_decode_mfma.h"
+#include "tq_options.h"
 #include <hip/hip_ext.h>
 
 namespace tq {
@@ -39,12 +40,21 @@ typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x8 __attribute__((ext_vector_type(8)));
 
 __device__ __forceinline__ f32x4 mfma_bf16(const u32x4& rows, const u32x4& cols, f32x4 c) {
   bf16x8 av, bv;
   __builtin_memcpy(&av, &rows, 16);
   __builtin_memcpy(&bv, &cols, 16);
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, bv, c, 0, 0, 0);
+}
+
+// fp6 (A: 16 rows x 128) x fp4 (B: 128 x 16) MFMA with per-lane power-of-two block scales (E8M0 codes); SEL
+// picks the byte of scale_a that holds the code.  Only six dwords of `a` and the four of `b` are read.
+template <int SEL>
+__device__ __forceinline__ f32x4 mfma_fp6_fp4(const i32x8& a, const u32x4& b, f32x4 c, int scale_a, int scale_b) {
+  const i32x8 bv = {(int)b[0], (int)b[1], (int)b[2], (int)b[3], 0, 0, 0, 0};
+  return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, bv, c, 2 /*A: fp6 e2m3*/, 4 /*B: fp4*/, SEL, scale_a, 0, scale_b);
 }
 
 // two fp32 -> packed bf16 (first value in the low half), round to nearest even
@@ -171,7 +181,7 @@ __device__ __forceinline__ void prefetch_matrix(const uint16_t* __restrict__ m_t
 // there is one, then with the first BUF slices of m_next, the matrix of the contraction that
 // follows.  Those loads have the rest of this contraction and the epilogue to arrive, and
 // the requests of a workgroup are spread out instead of coming in one burst.
-template <int D, int NA>
+template <int D, int NA, bool REFILL = true>
 __device__ __forceinline__ void contract(const uint16_t* a_terms, const uint16_t* __restrict__ m_terms,
                                          const uint16_t* __restrict__ m_next, int wave, int lane, MatRegs<D>& mr,
                                          f32x4 (&acc)[KeyGeom<D>::MT][KeyGeom<D>::NPW]) {
@@ -201,7 +211,7 @@ __device__ __forceinline__ void contract(const uint16_t* a_terms, const uint16_t
         }
     }
     if (kblk + BUF < KB) load_slice<D>(m_terms, wave, lane, kblk + BUF, mr.b[kblk % BUF]);
-    else load_slice<D>(m_next, wave, lane, kblk + BUF - KB, mr.b[kblk % BUF]);
+    else if (REFILL) load_slice<D>(m_next, wave, lane, kblk + BUF - KB, mr.b[kblk % BUF]);
   }
 }
 
@@ -313,9 +323,17 @@ struct XStage {
 
 // MSE_ONLY (the stage-1 quantiser alone: no residual, no signs) is a template parameter: as a
 // run-time flag it adds control flow that costs the register allocator its footing.
-template <int DT, int D, bool MSE_ONLY, class Source, class Sink>
+//
+// FX (head_dim 128, codebooks with single-bit Walsh terms): the centroid contraction x_hat = c[idx] Pi runs on
+// the block-scaled fp6 x fp4 MFMA (16x16x128, four times the bf16 rate).  c[idx] = c0 + sum_p k_p bit_p(idx), so
+// x_hat = c0 colsum(Pi) + sum_p k_p (plane_p Pi): the index bit planes, which are being built anyway, are the fp4
+// operand (a plane word turns into fp4 codes with four ANDs), and Pi^T is the fp6 operand, cut into five
+// fp6 digits per value on the host (good to 2^-23 of a block's largest value: below the rounding noise of an
+// fp32 product sum).  10 MFMAs per 16 x 16 tile instead of 24, and no centroid terms go through the LDS.
+template <int DT, int D, bool MSE_ONLY, bool FX, class Source, class Sink>
 __global__ void __launch_bounds__(KQ_THREADS, 2)
 key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, int64_t n_tiles) {
+  static_assert(!FX || (D == 128 && !MSE_ONLY), "the fp6 centroid contraction: head_dim 128, full quantiser");
   constexpr int mse_only = MSE_ONLY;
   using E = Elem<DT>;
   using S = typename E::storage;
@@ -345,6 +363,26 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
     uint32_t t[3];
     split3_pk(ly.centroids[tid0], 0.0f, t);
     slut[tid0] = u32x2{(t[0] & 0xffffu) | (t[1] << 16), t[2] & 0xffffu};
+  }
+  // FX: Pi^T as fp6 digits (this wavefront's column tiles, resident), their block scales, the plane
+  // coefficients and the constant part c0 colsum(Pi) of this lane's output columns
+  constexpr int FXT = 5;
+  int fs0[FX ? KeyGeom<D>::NPW : 1], fs1[FX ? KeyGeom<D>::NPW : 1];
+  float fk[2] = {0.0f, 0.0f};
+  f32x4 fconst[FX ? KeyGeom<D>::NPW : 1];
+  if constexpr (FX) {
+    const int lane0 = tid0 & 63;
+#pragma unroll
+    for (int c = 0; c < NPW; ++c) {
+      const int ct = wave0 * NPW + c;
+      fs0[c] = (int)ly.PiT_fp6_scale[((size_t)ct * 64 + lane0) * 2];
+      fs1[c] = (int)ly.PiT_fp6_scale[((size_t)ct * 64 + lane0) * 2 + 1];
+      const float* cs = ly.Pi_colsum + 16 * ct + 4 * (lane0 >> 4);
+      fconst[c] = f32x4{ly.term_const * cs[0], ly.term_const * cs[1], ly.term_const * cs[2], ly.term_const * cs[3]};
+    }
+    for (int t = 0; t < ly.n_terms; ++t)                          // plane p holds index bit mb - 1 - p
+      for (int p = 0; p < 2; ++p)
+        if (p < mb && ly.term_mask[t] == (1 << (mb - 1 - p))) fk[p] = ly.term_coef[t];
   }
   // (1) staging (XStage): the next group's chunks wait in registers while the current group is worked on
   XStage<DT, D, Source> stg;
@@ -425,7 +463,19 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
 
   f32x4 acc[MT][NPW];
   // (3) y = u Pi^T, bucketise; index bit planes; centroid values as bf16 terms for the next contraction
-  contract<D, NA1>(terms, ly.Pi_split, mse_only ? ly.Pi_split : ly.PiT_split, wave, lane, mr, acc);
+  // (FX: the matrix registers stay free after this contraction; the fp6 digits of Pi^T take their place until
+  // the centroid contraction is done, then S is requested and has the residual pass to arrive)
+  contract<D, NA1, !FX>(terms, ly.Pi_split, mse_only ? ly.Pi_split : ly.PiT_split, wave, lane, mr, acc);
+  i32x8 fa[FX ? NPW : 1][FX ? FXT : 1];
+  if constexpr (FX) {
+#pragma unroll
+    for (int c = 0; c < NPW; ++c)
+#pragma unroll
+      for (int t = 0; t < FXT; ++t) {
+        const uint32_t* p6 = ly.PiT_fp6 + ((size_t)((wave * NPW + c) * FXT + t) * 64 + lane) * 6;
+        fa[c][t] = i32x8{(int)p6[0], (int)p6[1], (int)p6[2], (int)p6[3], (int)p6[4], (int)p6[5], 0, 0};
+      }
+  }
   __syncthreads();                                              // every wavefront has read the unit-vector terms
   {
     uint32_t idx[MT][NPW][4];
@@ -463,16 +513,18 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
 #pragma unroll
       for (int c = 0; c < NPW; ++c) {
         const int col0 = 16 * (wave * NPW + c) + 4 * kb;
-        u32x2 e[4];
+        if constexpr (!FX) {
+          u32x2 e[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) e[i] = slut[idx[m][c][i]];
-        // term 0: low halves of .x, term 1: high halves of .x, term 2: low halves of .y
-        const u32x2 t0{(e[0].x & 0xffffu) | (e[1].x << 16), (e[2].x & 0xffffu) | (e[3].x << 16)};
-        const u32x2 t1{(e[0].x >> 16) | (e[1].x & 0xffff0000u), (e[2].x >> 16) | (e[3].x & 0xffff0000u)};
-        const u32x2 t2{e[0].y | (e[1].y << 16), e[2].y | (e[3].y << 16)};
-        *(u32x2*)(terms + ((size_t)0 * TT + t) * RS + col0) = t0;
-        *(u32x2*)(terms + ((size_t)1 * TT + t) * RS + col0) = t1;
-        *(u32x2*)(terms + ((size_t)2 * TT + t) * RS + col0) = t2;
+          for (int i = 0; i < 4; ++i) e[i] = slut[idx[m][c][i]];
+          // term 0: low halves of .x, term 1: high halves of .x, term 2: low halves of .y
+          const u32x2 t0{(e[0].x & 0xffffu) | (e[1].x << 16), (e[2].x & 0xffffu) | (e[3].x << 16)};
+          const u32x2 t1{(e[0].x >> 16) | (e[1].x & 0xffff0000u), (e[2].x >> 16) | (e[3].x & 0xffff0000u)};
+          const u32x2 t2{e[0].y | (e[1].y << 16), e[2].y | (e[3].y << 16)};
+          *(u32x2*)(terms + ((size_t)0 * TT + t) * RS + col0) = t0;
+          *(u32x2*)(terms + ((size_t)1 * TT + t) * RS + col0) = t1;
+          *(u32x2*)(terms + ((size_t)2 * TT + t) * RS + col0) = t2;
+        }
         if constexpr (std::is_same<Sink, KeyFlatSink>::value) {
           if (sink.y_dbg && svalid[t]) *(f32x4*)(sink.y_dbg + (tile0 * TILE + t) * D + col0) = acc[m][c];
         }
@@ -483,8 +535,59 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
   if (mse_only) stg.issue(x);
   if (!mse_only) {
     // (4) x_hat = (c Pi) * norm ; r = x - x_hat ; ||r||^2 partial sums ; r as bf16 terms (quantizer.py:241-245)
-    contract<D, 3>(terms, ly.PiT_split, ly.S_split, wave, lane, mr, acc);
-    __syncthreads();                                            // every wavefront has read the centroid terms
+    if constexpr (FX) {
+      // lane (n, kb) feeds plane word kb of vector 16 m + n: coordinate c of the word sits at contraction
+      // index 32 kb + 8 (c % 4) + c / 4 with the fp4 value 0.5, 1, 2, 0.5 (the matrix digits carry the inverse)
+#pragma unroll
+      for (int m = 0; m < MT; ++m)
+#pragma unroll
+        for (int c = 0; c < NPW; ++c) acc[m][c] = fconst[c];
+#pragma unroll
+      for (int p = 0; p < 2; ++p) {
+        if (p < mb) {
+          u32x4 b[MT];
+          f32x4 part[MT][NPW];
+#pragma unroll
+          for (int m = 0; m < MT; ++m) {
+            const uint32_t w = spl[(p * TT + 16 * m + n) * W + kb];
+            b[m] = u32x4{w & 0x11111111u, w & 0x22222222u, w & 0x44444444u, (w >> 3) & 0x11111111u};
+#pragma unroll
+            for (int c = 0; c < NPW; ++c) part[m][c] = f32x4{0, 0, 0, 0};
+          }
+          // digit by digit over all tiles: consecutive MFMAs go to different accumulators
+#pragma unroll
+          for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int c = 0; c < NPW; ++c) part[m][c] = mfma_fp6_fp4<0>(fa[c][0], b[m], part[m][c], fs0[c], 127);
+#pragma unroll
+          for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int c = 0; c < NPW; ++c) part[m][c] = mfma_fp6_fp4<1>(fa[c][1], b[m], part[m][c], fs0[c], 127);
+#pragma unroll
+          for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int c = 0; c < NPW; ++c) part[m][c] = mfma_fp6_fp4<2>(fa[c][2], b[m], part[m][c], fs0[c], 127);
+#pragma unroll
+          for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int c = 0; c < NPW; ++c) part[m][c] = mfma_fp6_fp4<3>(fa[c][3], b[m], part[m][c], fs0[c], 127);
+#pragma unroll
+          for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int c = 0; c < NPW; ++c) part[m][c] = mfma_fp6_fp4<0>(fa[c][4], b[m], part[m][c], fs1[c], 127);
+#pragma unroll
+          for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int c = 0; c < NPW; ++c)
+#pragma unroll
+              for (int i = 0; i < 4; ++i) acc[m][c][i] = fmaf(fk[p], part[m][c][i], acc[m][c][i]);
+        }
+      }
+      prefetch_matrix<D>(ly.S_split, wave, lane, mr);
+    } else {
+      contract<D, 3>(terms, ly.PiT_split, ly.S_split, wave, lane, mr, acc);
+      __syncthreads();                                          // every wavefront has read the centroid terms
+    }
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
       const int t = 16 * m + n;
@@ -632,12 +735,12 @@ __host__ static bool sink_ok(const KeyFlatSink& s, int mse_only) {
 }
 __host__ static bool sink_ok(const KeyPagedSink& s, int) { return s.L.key_lane_major != 0; }
 
-template <int DT, int D, bool MSE_ONLY, class Source, class Sink>
+template <int DT, int D, bool MSE_ONLY, bool FX, class Source, class Sink>
 static int launch_dt_d(const void* x, const Source& src, const tq_layer& ly, const Sink& sink, int64_t tiles,
                        hipStream_t st) {
   using Gm = KeyGeom<D>;
   using Sm = KeySmem<DT, D>;
-  auto kern = key_mfma_kernel<DT, D, MSE_ONLY, Source, Sink>;
+  auto kern = key_mfma_kernel<DT, D, MSE_ONLY, FX, Source, Sink>;
   static std::atomic<uint64_t> configured{0};           // per instantiation, one bit per device; the attribute is sticky
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return TQ_EINVAL;
@@ -678,11 +781,18 @@ int launch_key_mfma(const void* x, int dtype, const Source& src, const tq_layer&
   if (!aligned_for_chunks(x, dtype, src) || !sink_ok(sink, mse_only)) return TQ_EUNSUPPORTED;
   constexpr bool paged = std::is_same<Sink, KeyPagedSink>::value;     // pages always hold the full code
   if (paged && mse_only) return TQ_EUNSUPPORTED;
+  // head_dim 128 with the fp6 digits of Pi^T and a codebook whose Walsh expansion has single-bit terms only:
+  // the centroid contraction on the block-scaled MFMA
+  bool fx = ly.d == 128 && !mse_only && ly.PiT_fp6 && ly.PiT_fp6_scale && ly.Pi_colsum && ly.mse_bits <= 2 &&
+            opt_fp6_centroids.load() != 0;
+  for (int t = 0; t < ly.n_terms; ++t) fx = fx && __builtin_popcount((unsigned)ly.term_mask[t]) == 1;
 #define TQ_KQ(DT_, D_)                                                                                     \
   if (dtype == DT_ && ly.d == D_) {                                                                        \
     if constexpr (!paged)                                                                                  \
-      if (mse_only) return launch_dt_d<DT_, D_, true, Source, Sink>(x, src, ly, sink, tiles, st);          \
-    return launch_dt_d<DT_, D_, false, Source, Sink>(x, src, ly, sink, tiles, st);                         \
+      if (mse_only) return launch_dt_d<DT_, D_, true, false, Source, Sink>(x, src, ly, sink, tiles, st);   \
+    if constexpr (D_ == 128)                                                                               \
+      if (fx) return launch_dt_d<DT_, D_, false, true, Source, Sink>(x, src, ly, sink, tiles, st);         \
+    return launch_dt_d<DT_, D_, false, false, Source, Sink>(x, src, ly, sink, tiles, st);                  \
   }
   TQ_KQ(TQ_BF16, 128) TQ_KQ(TQ_BF16, 256) TQ_KQ(TQ_F16, 128) TQ_KQ(TQ_F16, 256) TQ_KQ(TQ_F32, 128) TQ_KQ(TQ_F32, 256)
 #undef TQ_KQ

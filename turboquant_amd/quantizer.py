@@ -119,8 +119,10 @@ class TurboQuantMSE(torch.nn.Module):
             self._PiT = self.Pi.T.contiguous()
             # only head_dim 128 / 256 have a matrix-core kernel; other sizes pass no split operands
             mk = _ffi.split_bf16x3 if self.dim in (128, 256) else (lambda m: None)
+            # head_dim 128: Pi^T also as fp6 terms, for the centroid contraction on the block-scaled MFMA
+            fp6 = _ffi.split_fp6x5(self._PiT) if (self.dim == 128 and S is not None) else None
             self._splits = (key, (mk(self.Pi), mk(self._PiT), None if S is None else mk(S),
-                                  None if ST is None else mk(ST)))
+                                  None if ST is None else mk(ST), fp6))
         qc = None
         if S is not None:
             if getattr(self, "_query_consts", None) is None or self._query_consts[0] != key:
