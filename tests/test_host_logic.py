@@ -283,3 +283,39 @@ def test_paged_cache_ingest_gathers_blocks_in_table_order():
     eng.ingest_prefill_from_paged_cache(cache, 10, table, 4)
     assert st.chunks == [[0, 1, 2, 3, 4, 5]]
     assert eng.ring.peek()[0][:, 0, 0].tolist() == [6, 7, 8, 9]
+
+
+def test_fp6_digits_of_the_rotation_decode_back_to_it():
+    """_ffi.split_fp6x5: the five fp6 (e2m3) digits and block scales of Pi^T, in the lane order of the block-scaled
+    MFMA, decode back to the matrix within 2^-22 of each (row, 32-coordinate block)'s largest value (the permuted
+    contraction index and the 0.5 / 1 / 2 / 0.5 position factors of the fp4 bit operand included)."""
+    from turboquant_amd import _ffi
+    from turboquant_amd.rotation import generate_rotation_matrix
+    d = 128
+    m = generate_rotation_matrix(d, "cpu", seed=42).T.contiguous()
+    codes, scales = _ffi.split_fp6x5(m)
+    assert tuple(codes.shape) == (d // 16, 1, 5, 64, 6) and tuple(scales.shape) == (d // 16, 1, 64, 2)
+    c = codes.numpy().view(np.uint32).astype(np.uint64)
+    sc = scales.numpy().view(np.uint32)
+    s_idx = np.arange(32)
+    coord = 4 * (s_idx % 8) + s_idx // 8
+    factor = np.array([0.5, 1.0, 2.0, 0.5])[coord % 4]
+    rec = np.zeros((d, d))
+    for t in range(5):
+        word = sc[:, 0, :, 0] if t < 4 else sc[:, 0, :, 1]                   # [tile][lane]
+        e8 = ((word >> (8 * (t % 4))) & 0xFF).astype(np.int64) - 127
+        for s_ in range(32):
+            lo = 6 * s_
+            w, sh = lo // 32, lo % 32
+            code = (c[:, 0, t, :, w] >> np.uint64(sh)) & np.uint64(63)
+            if sh > 26:
+                code |= (c[:, 0, t, :, w + 1] << np.uint64(32 - sh)) & np.uint64(63)
+            code = code.astype(np.int64)
+            ex, man = (code >> 3) & 3, code & 7
+            mag = np.where(ex == 0, man / 8.0, (1 + man / 8.0) * 2.0 ** (ex - 1))
+            val = np.where(code & 32, -mag, mag) * 2.0 ** e8 * factor[s_]    # [tile][lane]
+            for lane in range(64):
+                rec[16 * np.arange(d // 16) + (lane & 15), 32 * (lane >> 4) + coord[s_]] += val[:, lane]
+    ref = m.double().numpy()
+    blockmax = np.abs(ref).reshape(d, d // 32, 32).max(-1).repeat(32, axis=1)
+    assert np.all(np.abs(rec - ref) <= 2.0 ** -22 * 2.0 * blockmax)
