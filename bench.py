@@ -297,12 +297,15 @@ def quantize_bench(device, steps, warmup):
     table = torch.arange(T // 16, dtype=torch.int32, device=device)[None]
     ms, _ = time_steps(lambda i: pool.append(k, v, table), steps, warmup)
     # The three d x d contractions of the key quantiser are the matrix-core part of the path.  The kernel issues
-    # them as 15 exact bf16 term products (5 per contraction instead of one fp32 product), so the matrix-core work
-    # it issues is 5 x the algorithmic FLOP, and the roofline that bounds it is the bf16 matrix peak.  In the
-    # product the key kernel runs beside the value kernel (a second stream); an event pair around it inside such
-    # an append also covers time it spends waiting for its share of the machine.  So: `frac` is taken over the
-    # WHOLE append (both kernels, fork and join), and the kernel's own duration is measured with the value kernel
-    # switched off (tq_set_option "append_parts" = 1, events attached to the kernel's dispatch).
+    # y = u Pi^T as 3 and p = r S^T as 6 exact bf16 term products (one fp32-accurate product each), and the centroid
+    # contraction x_hat = c[idx] Pi as 2 bit planes x 5 fp6 digits on the block-scaled fp6 x fp4 MFMA.  The roofline
+    # that bounds it is the matrix pipe: `frac` = the time the issued work takes at the peaks of its instruction
+    # types (bf16 2500 TFLOP/s, fp6 / fp4 10100 TFLOP/s) over the measured time; `achieved` / `peak` are the issued
+    # FLOP rate and the blend of the two peaks that this mix could reach.  In the product the key kernel runs beside
+    # the value kernel (a second stream); an event pair around it inside such an append also covers time it spends
+    # waiting for its share of the machine.  So: `frac` is taken over the WHOLE append (both kernels, fork and
+    # join), and the kernel's own duration is measured with the value kernel switched off (tq_set_option
+    # "append_parts" = 1, events attached to the kernel's dispatch).
     from turboquant_amd import _ffi
     lib = _ffi.lib()
     _ffi.check(lib.tq_set_option(b"append_parts", 1), "tq_set_option")
@@ -311,22 +314,25 @@ def quantize_bench(device, steps, warmup):
     finally:
         _ffi.check(lib.tq_set_option(b"append_parts", 3), "tq_set_option")
     flops = 3 * 2 * d * d * T * H
-    issued = 5 * flops / (ms * 1e-3) / 1e12
+    bf16_flop = (3 + 6) * 2 * d * d * T * H                     # term products of the first and the third contraction
+    fp6_flop = 2 * 5 * 2 * d * d * T * H                        # planes x digits of the centroid contraction
+    at_peak_s = bf16_flop / 2500e12 + fp6_flop / 10100e12
+    issued = (bf16_flop + fp6_flop) / (ms * 1e-3) / 1e12
+    blend_peak = (bf16_flop + fp6_flop) / at_peak_s / 1e12
     nbytes = T * (2 * H * d * 2 + H * 100)
     return {"tokens_per_s": T / (ms * 1e-3), "ms": ms, "tokens": T, "kv_heads": H, "head_dim": d,
             "workload": "prefill quantize, 32768 tok x 8 KV heads, d=128, 3b keys + 2b values, pages of 16",
             "hbm_gbs": nbytes / (ms * 1e-3) / 1e9, "hbm_bytes": nbytes,
             "hbm_frac": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
             "roofline": {"bound": "mfma", "kernel": "key_mfma_kernel (paged sink) beside value_chunk_kernel",
-                         "append_ms": ms, "achieved": issued, "peak": 2500.0, "unit": "TFLOP/s",
-                         "frac": issued / 2500.0, "algorithmic_tflops": flops / (ms * 1e-3) / 1e12,
-                         "key_kernel_alone_ms": key_ms,
-                         "key_kernel_alone_frac": 5 * flops / (key_ms * 1e-3) / 1e12 / 2500.0,
-                         "note": "achieved = bf16 matrix-core work the key kernel issues (15 exact bf16 term products "
-                                 "for the 3 fp32-accurate d x d contractions per vector = 5 x the algorithmic 6 d^2 "
-                                 "FLOP) over the whole append time, against the 2500 TFLOP/s bf16 peak; "
-                                 "key_kernel_alone_* = the same work over the kernel's own duration when the value "
-                                 "kernel does not run beside it"}}, (pool, k, v, table, tq)
+                         "append_ms": ms, "achieved": issued, "peak": blend_peak, "unit": "TFLOP/s",
+                         "frac": at_peak_s / (ms * 1e-3), "algorithmic_tflops": flops / (ms * 1e-3) / 1e12,
+                         "issued_bf16_gflop": bf16_flop / 1e9, "issued_fp6_fp4_gflop": fp6_flop / 1e9,
+                         "key_kernel_alone_ms": key_ms, "key_kernel_alone_frac": at_peak_s / (key_ms * 1e-3),
+                         "note": "issued matrix work of the key kernel (9 bf16 term products + 10 fp6 x fp4 plane/digit "
+                                 "products per vector and d x d contraction size) over the whole append time, against "
+                                 "the peaks of the two instruction types; key_kernel_alone_* = the same work over the "
+                                 "kernel's own duration when the value kernel does not run beside it"}}, (pool, k, v, table, tq)
 
 
 def round_trip_bench(device, steps, warmup, with_cpu):

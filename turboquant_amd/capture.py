@@ -24,9 +24,9 @@ KVPair = Tuple[torch.Tensor, torch.Tensor]
 
 
 class RingBuffer:
-    """`capacity` exact tokens, (capacity, num_kv_heads, head_dim) per tensor."""
-
-    __slots__ = ("capacity", "num_kv_heads", "head_dim", "device", "dtype", "_k", "_v", "_pos", "_total_written")
+    """The newest exact tokens of one layer: one (2, capacity, num_kv_heads, head_dim) tensor, keys in plane 0
+    and values in plane 1, filled from the front.  Same interface and token routing as the reference's ring
+    (capture.py:21-131): a write that needs room while the ring is full first hands back everything in it."""
 
     def __init__(self, capacity: int, num_kv_heads: int, head_dim: int, device, dtype: torch.dtype = torch.bfloat16):
         self.capacity = capacity
@@ -34,59 +34,60 @@ class RingBuffer:
         self.head_dim = head_dim
         self.device = device
         self.dtype = dtype
-        self._k = torch.zeros(capacity, num_kv_heads, head_dim, device=device, dtype=dtype)
-        self._v = torch.zeros(capacity, num_kv_heads, head_dim, device=device, dtype=dtype)
-        self._pos = 0
-        self._total_written = 0
+        self._rows = torch.zeros(2, capacity, num_kv_heads, head_dim, device=device, dtype=dtype)
+        self._fill = 0          # tokens held
+        self._seen = 0          # tokens ever written
 
     @property
     def size(self) -> int:
-        return self._pos
+        return self._fill
 
     @property
     def is_full(self) -> bool:
-        return self._pos >= self.capacity
+        return self._fill >= self.capacity
 
     @property
     def total_written(self) -> int:
-        return self._total_written
+        return self._seen
+
+    def _take_all(self) -> torch.Tensor:
+        held = self._rows[:, : self._fill].clone()
+        self._fill = 0
+        return held
 
     def write(self, key: torch.Tensor, value: torch.Tensor, num_tokens: int) -> Optional[KVPair]:
-        """Append num_tokens tokens.  Whenever the ring is full at the moment a
-        token needs room, everything in it is drained first; the drained tokens
-        come back (oldest first) as (k, v), or None if nothing was drained."""
-        spilled_k, spilled_v = [], []
-        done = 0
-        while done < num_tokens:
-            if self._pos >= self.capacity:
-                spilled_k.append(self._k[: self._pos].clone())
-                spilled_v.append(self._v[: self._pos].clone())
-                self._pos = 0
-            take = min(num_tokens - done, self.capacity - self._pos)
-            self._k[self._pos: self._pos + take] = key[done: done + take]
-            self._v[self._pos: self._pos + take] = value[done: done + take]
-            self._pos += take
-            done += take
-        self._total_written += num_tokens
-        if not spilled_k:
+        """Append num_tokens tokens; returns what had to leave the ring on the way (oldest first) as (k, v),
+        or None.  The ring is emptied, completely, each time a token arrives while it is full."""
+        handed_back = []
+        src = 0
+        while src < num_tokens:
+            if self.is_full:
+                handed_back.append(self._take_all())
+            n = min(num_tokens - src, self.capacity - self._fill)
+            self._rows[0, self._fill: self._fill + n] = key[src: src + n]
+            self._rows[1, self._fill: self._fill + n] = value[src: src + n]
+            self._fill += n
+            src += n
+        self._seen += num_tokens
+        if not handed_back:
             return None
-        return torch.cat(spilled_k, dim=0), torch.cat(spilled_v, dim=0)
+        out = handed_back[0] if len(handed_back) == 1 else torch.cat(handed_back, dim=1)
+        return out[0], out[1]
 
     def drain(self) -> Optional[KVPair]:
-        if self._pos == 0:
+        if self._fill == 0:
             return None
-        pair = (self._k[: self._pos].clone(), self._v[: self._pos].clone())
-        self._pos = 0
-        return pair
+        held = self._take_all()
+        return held[0], held[1]
 
     def peek(self) -> Optional[KVPair]:
-        if self._pos == 0:
+        if self._fill == 0:
             return None
-        return self._k[: self._pos], self._v[: self._pos]
+        return self._rows[0, : self._fill], self._rows[1, : self._fill]
 
     def reset(self):
-        self._pos = 0
-        self._total_written = 0
+        self._fill = 0
+        self._seen = 0
 
 
 class KVCaptureEngine:
