@@ -328,6 +328,9 @@ void tq_time_next_key_kernel(void *start_event, void *stop_event);
  *                      library built with -DTQ_FUSED_PREP (TQ_EUNSUPPORTED otherwise): it measured slower.
  *   "prep_spin_limit"  with fuse_prep: how often a workgroup polls for the other workgroups' share of the
  *                      operands before it computes them itself (default 20000; 0 = never wait).
+ *   "merge_in_kernel"  1 (default): a compressed-only decode step on the matrix-core kernel with at most 8 context
+ *                      splits has its splits merged by the last workgroup of the page kernel (two launches per
+ *                      step); 0: always the separate merge kernel.
  *   "fp6_centroids"    1 (default): the key quantiser takes the fp6 x fp4 centroid contraction when the layer
  *                      carries PiT_fp6; 0: always the bf16 term products (for A/B runs).
  *   "append_parts"     measurement only: 3 (default) = the append entry points quantise keys and values,

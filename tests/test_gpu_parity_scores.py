@@ -464,3 +464,48 @@ def test_decode_head_dim_64_on_the_matrix_cores(gpu, key_bits, vb, Hq, Hkv, dtyp
         worst = min(worst, _decode_case(gpu, 64, key_bits, vb, 2, Hq, Hkv, [1000, 17], None, seed=650 + n_split,
                                         n_split=n_split, dtype=dtype))
     _progress(f"   worst cosine {worst:.7f}")
+
+
+@pytest.mark.parametrize("d,key_bits,vb,Hq,Hkv,lens,n_split", [
+    (128, 3, 4, 32, 8, [900, 1, 16, 0, 517], 4),
+    (128, 3, 2, 8, 1, [2100], 8),
+    (256, 3, 2, 16, 2, [1500, 700], 5),
+    (256, 4, 4, 10, 2, [333, 64], 2),              # 5 heads per group
+    (64, 3, 4, 8, 2, [800, 130, 65], 3),
+    (128, 3, 4, 32, 2, [640], 1)])                 # 16 heads per KV head = two groups of 8, a single split
+def test_splits_merged_inside_the_page_kernel(gpu, d, key_bits, vb, Hq, Hkv, lens, n_split):
+    """With at most eight context splits the workgroup that finishes last among the splits of a (sequence, group
+    of query heads) merges them inside the page kernel's launch (the log-sum-exp merge of score.py:84-173's
+    segments), instead of a merge kernel: same result up to the order of the sums, for ragged and empty
+    sequences, on consecutive calls (the arrival counters are reset by each step's preparation), and against the
+    oracle."""
+    B = len(lens)
+    g = torch.Generator().manual_seed(d + Hq + n_split)
+    pages = (max(lens) + 15) // 16
+    pool, tq = _make_pool(gpu, d, key_bits, vb, Hkv, B * pages + 1, torch.bfloat16, seed=42)
+    table = torch.randperm(B * pages + 1, generator=g)[: B * pages].to(torch.int32).view(B, pages).to(gpu)
+    k = torch.randn(B, max(lens), Hkv, d, generator=g).bfloat16().to(gpu)
+    v = torch.randn(B, max(lens), Hkv, d, generator=g).bfloat16().to(gpu)
+    pool.append(k, v, table)
+    seq = torch.tensor(lens, dtype=torch.int32, device=gpu)
+    q = torch.randn(B, Hq, d, generator=g).bfloat16()
+    _progress(f"in-launch merge d={d} kb={key_bits} vb={vb} Hq={Hq} Hkv={Hkv} lens={lens} splits={n_split}")
+    try:
+        _set_option("merge_in_kernel", 0)
+        want = pool.decode_attention(q.to(gpu), table, seq, n_split=n_split).float().cpu()
+        _set_option("merge_in_kernel", 1)
+        got = pool.decode_attention(q.to(gpu), table, seq, n_split=n_split).float().cpu()
+        again = pool.decode_attention(q.to(gpu), table, seq, n_split=n_split).float().cpu()
+        torch.cuda.synchronize()
+    finally:
+        _set_option("merge_in_kernel", 1)
+    assert torch.equal(got, again)
+    assert (got - want).abs().max() <= 2 ** -7 * want.abs().max() + 1e-6        # one bf16 step of the largest value
+    prm = params_of(tq)
+    for b in range(B):
+        if lens[b] == 0:
+            assert torch.count_nonzero(got[b]) == 0
+            continue
+        kc, vc = _store_from_oracle_view(pool, table[b], lens[b])
+        ref = O.hybrid_attention(q[b:b + 1], kc, vc, max(lens[b], O.MIN_HISTORY), prm, Hkv, None, None)
+        assert cosine(got[b:b + 1], ref) >= COS_GATE, b

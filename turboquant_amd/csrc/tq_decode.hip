@@ -828,7 +828,8 @@ using namespace tq;
 
 namespace tq {
 int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* layer, float* q_rot, float* q_sk,
-                        float* q_stat, uint32_t* qa_pack, int G, float sm_scale, hipStream_t st, bool q_rot_unused);
+                        float* q_stat, uint32_t* qa_pack, int G, float sm_scale, hipStream_t st, bool q_rot_unused,
+                        unsigned long long* arrivals);
 }  // namespace tq
 
 static size_t parts_floats(int B, int Hq, int d, int n_parts) { return (size_t)B * Hq * n_parts * (d + 2); }
@@ -842,6 +843,7 @@ std::atomic<int> opt_prep_spin_limit{20000};
 std::atomic<int> opt_prep_units{0};
 std::atomic<int> opt_append_parts{3};
 std::atomic<int> opt_fp6_centroids{1};
+std::atomic<int> opt_merge_in_kernel{1};
 }  // namespace tq
 
 namespace {
@@ -872,6 +874,7 @@ extern "C" int tq_set_option(const char* name, int64_t value) {
     opt_prep_spin_limit.store((int)value);
     return TQ_OK;
   }
+  if (!std::strcmp(name, "merge_in_kernel")) { opt_merge_in_kernel.store(value != 0); return TQ_OK; }
   if (!std::strcmp(name, "fp6_centroids")) { opt_fp6_centroids.store(value != 0); return TQ_OK; }
   if (!std::strcmp(name, "append_parts")) {
     if (value < 1 || value > 3) return TQ_EINVAL;
@@ -1008,11 +1011,21 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
     fz.nonce = next_nonce();
     const int mf = launch_decode_mfma(qa_pack, q_stat, B, Hq, Hkv * kv_div, kv_div, pool, block_table, bt_stride, seq_lens,
                                       sm_scale, *layer, *layout, parts, n_parts, n_split, len_sub, max_pages, pool_pages,
-                                      fz, st);
+                                      fz, FusedMerge{}, st);
     if (mf > 0) return mf;
     fused = mf == TQ_OK;             // TQ_EUNSUPPORTED: nothing was launched, the separate launches below run
   }
 
+  // A whole compressed-only step with few context splits: the workgroup that finishes last among the splits of a
+  // (sequence, group of query heads) merges them inside the page kernel's launch, and no merge kernel follows
+  // (with many splits that workgroup would read more than the separate launch costs).  The preparation kernel
+  // zeroes the arrival counters of its groups.
+  FusedMerge fm;
+  if (stages == 7 && mfma_shape && !tail && !fused && n_split <= MERGE_IN_KERNEL_MAX_SPLITS && opt_merge_in_kernel.load()) {
+    fm.out = out;
+    fm.out_dtype = dtype;
+    fm.counters = flags;
+  }
   if ((stages & 1) && !fused) {
     if (!layer->Pi || !layer->PiT || !layer->S || !layer->ST || !layer->centroids) return TQ_ENULL;
     const int n_prep = (B * Hq / Gq) * (d / PREP_COLS);
@@ -1053,7 +1066,8 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
       tail_done = true;
     } else {
       int rc = launch_rotate_query(q, dtype, (int64_t)B * Hq, layer, q_rot, q_sk, q_stat,
-                                   mfma_shape ? qa_pack : nullptr, mfma_shape ? Gq : G, sm_scale, st, mfma_shape);
+                                   mfma_shape ? qa_pack : nullptr, mfma_shape ? Gq : G, sm_scale, st, mfma_shape,
+                                   fm.counters);
       if (rc) return rc;
     }
   }
@@ -1063,9 +1077,10 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   if ((stages & 2) && !fused)
     mf = mfma_shape ? launch_decode_mfma(qa_pack, q_stat, B, Hq, Hkv * kv_div, kv_div, pool, block_table, bt_stride,
                                          seq_lens, sm_scale, *layer, *layout, parts, n_parts, n_split, len_sub,
-                                         max_pages, pool_pages, FusedPrep{}, st)
+                                         max_pages, pool_pages, FusedPrep{}, fm, st)
                     : TQ_EUNSUPPORTED;
   if (mf > 0) return mf;
+  if (mf == TQ_OK && fm.out != nullptr) return TQ_OK;         // merged in the launch
   if ((stages & 2) && mf == TQ_EUNSUPPORTED) {      // no matrix-core kernel for this shape: general kernel
     if (dtype < TQ_F32 || dtype > TQ_BF16) return TQ_EINVAL;
     const int gp4 = (G + 3) / 4, gp = 4 * gp4;      // query heads rounded up to a multiple of 4

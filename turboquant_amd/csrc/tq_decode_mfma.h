@@ -18,6 +18,17 @@ struct FusedPrep {
   unsigned long long nonce = 0;      // value of a published flag in this call (never 0)
 };
 
+// Merge of the context splits inside the page kernel's launch (out == nullptr: a merge kernel follows).  The
+// workgroup that finishes last among the n_split workgroups of a (sequence, group of query heads) reads the
+// others' partials and writes the attention output; nobody waits for anybody.  `counters` holds one arrival
+// counter per group, zeroed by the query preparation kernel of the same step.
+struct FusedMerge {
+  void* out = nullptr;               // (B, Hq, d) in out_dtype
+  int out_dtype = 0;
+  unsigned long long* counters = nullptr;
+};
+constexpr int MERGE_IN_KERNEL_MAX_SPLITS = 8;
+
 // Events armed by tq_time_next_page_kernel (which = 0) / tq_time_next_key_kernel (which = 1) on this thread:
 // returns them and disarms; false when none is armed.
 bool take_time_hook(int which, hipEvent_t& start, hipEvent_t& stop);
@@ -33,6 +44,6 @@ size_t decode_mfma_pack_words(int B, int Hq, int d);
 int launch_decode_mfma(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, int kv_div, const uint8_t* pool,
                        const int32_t* block_table, int bt_stride, const int32_t* seq_lens, float sm_scale,
                        const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts, int n_split, int len_sub,
-                       int max_pages, int num_pages, const FusedPrep& fz, hipStream_t st);
+                       int max_pages, int num_pages, const FusedPrep& fz, const FusedMerge& fm, hipStream_t st);
 
 }  // namespace tq

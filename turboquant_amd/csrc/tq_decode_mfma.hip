@@ -178,7 +178,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
                    const uint8_t* __restrict__ pool, const int32_t* __restrict__ block_table,
                    int bt_stride, const int32_t* __restrict__ seq_lens, float sm_scale, tq_layer ly, tq_page_layout L,
                    float* __restrict__ parts, int n_parts, int n_split, int len_sub, int max_pages, int num_pages,
-                   FusedPrep fz) {
+                   FusedPrep fz, FusedMerge fm) {
   constexpr int DW = D / DS;                  // coordinates / channels of one wavefront
   constexpr int WPLT = (D + 127) / 128;       // plane words per lane per plane per page, all wavefronts
   constexpr int WPL = (DW + 127) / 128;       // ... of one wavefront (head_dim 64: one, with half of the lanes idle)
@@ -795,8 +795,57 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
     }
     if (live) {
       float* out = parts + (((int64_t)b * Hq + h * G + g) * n_parts + split) * (D + 2);
-      if (ch == 0) { out[0] = mm; out[1] = ll; }
-      out[2 + ch] = aa;
+      if (fm.out != nullptr) {                 // read by another workgroup of this launch: device-coherent stores
+        if (ch == 0) { store_coherent(out, mm); store_coherent(out + 1, ll); }
+        store_coherent(out + 2 + ch, aa);
+      } else {
+        if (ch == 0) { out[0] = mm; out[1] = ll; }
+        out[2 + ch] = aa;
+      }
+    }
+  }
+  // ---------------------------------------------------------------- merge of the splits inside this launch
+  // Every workgroup counts itself in after its partial has been written (one atomic increment of the group's
+  // counter, which the preparation kernel of this step has zeroed); the one that counts last merges.
+  if (fm.out != nullptr) {
+    __shared__ int s_last;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");      // the partial's stores have completed ...
+    __syncthreads();                                            // ... in every wavefront
+    if (tid == 0) {
+      const unsigned long long before = __hip_atomic_fetch_add(fm.counters + ((int64_t)b * Hkv + h), 1ull, __ATOMIC_RELAXED,
+                                                               __HIP_MEMORY_SCOPE_AGENT);
+      s_last = before + 1ull == (unsigned long long)n_split;
+    }
+    __syncthreads();
+    if (s_last) {
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+#pragma unroll
+      for (int k = 0; k < 8 * D / (MF_WAVES * 64); ++k) {
+        const int o = tid + k * (MF_WAVES * 64);
+        const bool live = o < G * D;
+        const int g = live ? o / D : 0, ch = o % D;
+        const float* row = parts + ((int64_t)b * Hq + h * G + g) * n_parts * (D + 2);
+        // all loads first (clamped to an existing split), then the log-sum-exp merge
+        float m_s[MERGE_IN_KERNEL_MAX_SPLITS], l_s[MERGE_IN_KERNEL_MAX_SPLITS], a_s[MERGE_IN_KERNEL_MAX_SPLITS];
+#pragma unroll
+        for (int sp = 0; sp < MERGE_IN_KERNEL_MAX_SPLITS; ++sp) {
+          const float* r = row + (int64_t)min(sp, n_split - 1) * (D + 2);
+          m_s[sp] = load_coherent(r); l_s[sp] = load_coherent(r + 1); a_s[sp] = load_coherent(r + 2 + ch);
+        }
+        float mm = MF_NEG;
+#pragma unroll
+        for (int sp = 0; sp < MERGE_IN_KERNEL_MAX_SPLITS; ++sp)
+          if (sp < n_split && l_s[sp] > 0.0f) mm = fmaxf(mm, m_s[sp]);
+        float ll = 0.0f, aa = 0.0f;
+#pragma unroll
+        for (int sp = 0; sp < MERGE_IN_KERNEL_MAX_SPLITS; ++sp) {
+          const float wgt = (sp < n_split && l_s[sp] > 0.0f) ? __expf(m_s[sp] - mm) : 0.0f;
+          ll = fmaf(wgt, l_s[sp], ll);
+          aa = fmaf(wgt, a_s[sp], aa);
+        }
+        const float inv = ll > 0.0f ? 1.0f / ll : 0.0f;
+        if (live) store_from_f32(fm.out, ((int64_t)b * Hq + h * G + g) * D + ch, aa * inv, fm.out_dtype);
+      }
     }
   }
 }
@@ -816,7 +865,7 @@ template <int D, int MB, int NX, int VB, int GS, int DS, int WPS, bool F16P>
 static int launch_one(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, int kv_div,
                       const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
                       float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts, int n_split,
-                      int len_sub, int max_pages, int num_pages, const FusedPrep& fz, hipStream_t st) {
+                      int len_sub, int max_pages, int num_pages, const FusedPrep& fz, const FusedMerge& fm, hipStream_t st) {
   const int G = Hq / Hkv;
   size_t per_wave = (size_t)wave_lds_floats(D / DS / GS, DS) * sizeof(float);
   size_t merge = (size_t)(MF_WAVES / DS * G * (D + 2) + MF_WAVES * 16 * 16) * sizeof(float);
@@ -834,11 +883,11 @@ static int launch_one(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, 
   if (take_time_hook(0, t_start_event, t_stop_event)) {
     hipExtLaunchKernelGGL(kern, dim3(n_split, Hkv, B), dim3(MF_WAVES * 64), smem, st, t_start_event, t_stop_event, 0,
                           qa_pack, q_stat, Hq, Hkv, kv_div, pool, block_table, bt_stride, seq_lens, sm_scale, ly, L, parts,
-                          n_parts, n_split, len_sub, max_pages, num_pages, fz);
+                          n_parts, n_split, len_sub, max_pages, num_pages, fz, fm);
   } else {
     kern<<<dim3(n_split, Hkv, B), dim3(MF_WAVES * 64), smem, st>>>(qa_pack, q_stat, Hq, Hkv, kv_div, pool, block_table,
                                                                    bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts,
-                                                                   n_split, len_sub, max_pages, num_pages, fz);
+                                                                   n_split, len_sub, max_pages, num_pages, fz, fm);
   }
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? TQ_OK : (int)e;
@@ -852,7 +901,8 @@ size_t decode_mfma_pack_words(int B, int Hq, int d) { return (size_t)B * Hq * 9 
 int launch_decode_mfma(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, int kv_div,
                        const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
                        float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts,
-                       int n_split, int len_sub, int max_pages, int num_pages, const FusedPrep& fz, hipStream_t st) {
+                       int n_split, int len_sub, int max_pages, int num_pages, const FusedPrep& fz, const FusedMerge& fm,
+                       hipStream_t st) {
   const int G = Hq / Hkv, d = ly.d, mb = ly.mse_bits, vb = L.value_bits, gs = L.group_size;
   if (G > 8 || (L.dtype != TQ_BF16 && L.dtype != TQ_F16) || !L.key_lane_major) return TQ_EUNSUPPORTED;
   const bool f16p = L.dtype == TQ_F16;
@@ -864,10 +914,10 @@ int launch_decode_mfma(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv,
     if (f16p)                                                                                                   \
       return launch_one<D_, MB_, NX_, VB_, GS_, DS_, WPS_, true>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,  \
                                                                  bt_stride, seq_lens, sm_scale, ly, L, parts,     \
-                                                                 n_parts, n_split, len_sub, max_pages, num_pages, fz, st); \
+                                                                 n_parts, n_split, len_sub, max_pages, num_pages, fz, fm, st); \
     return launch_one<D_, MB_, NX_, VB_, GS_, DS_, WPS_, false>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,   \
                                                                 bt_stride, seq_lens, sm_scale, ly, L, parts,      \
-                                                                n_parts, n_split, len_sub, max_pages, num_pages, fz, st); \
+                                                                n_parts, n_split, len_sub, max_pages, num_pages, fz, fm, st); \
   }
   TQ_TRY(128, 2, 0, 2, 32, 1, 2) TQ_TRY(128, 2, 0, 4, 32, 1, 2) TQ_TRY(256, 2, 0, 2, 32, 2, 2) TQ_TRY(256, 2, 0, 4, 32, 2, 2)
   TQ_TRY(128, 1, 0, 2, 32, 1, 2) TQ_TRY(128, 1, 0, 4, 32, 1, 2) TQ_TRY(256, 1, 0, 2, 32, 2, 2) TQ_TRY(256, 1, 0, 4, 32, 2, 2)

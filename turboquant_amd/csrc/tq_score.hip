@@ -73,8 +73,10 @@ template <int PER, int DT>
 __global__ void __launch_bounds__(PREP_COLS * PREP_SLICES)
 prep_query_kernel(const void* __restrict__ q, int G, tq_layer ly, float sm_scale,
                   float* __restrict__ q_rot, float* __restrict__ q_sk, float* __restrict__ q_stat,
-                  uint32_t* __restrict__ qa_pack) {
+                  uint32_t* __restrict__ qa_pack, unsigned long long* __restrict__ arrivals) {
   extern __shared__ float sm[];
+  // the arrival counter of this group of query heads, for the page kernel that merges its splits itself
+  if (arrivals != nullptr && blockIdx.y == 0 && threadIdx.x == 0) arrivals[blockIdx.x] = 0ull;
   prep_query_body<PER, DT>(q, G, ly, sm_scale, q_rot, q_sk, q_stat, qa_pack, blockIdx.x, blockIdx.y, sm);
 }
 
@@ -367,12 +369,13 @@ int launch_dequant_mfma(const uint8_t* idx, const uint8_t* signs, const void* no
 // q_rot_unused: the caller only needs the packed operands and statistics (the page kernel on the matrix
 // cores), not the fp32 rotated / sketched queries
 int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* layer, float* q_rot, float* q_sk,
-                        float* q_stat, uint32_t* qa_pack, int G, float sm_scale, hipStream_t st, bool q_rot_unused) {
+                        float* q_stat, uint32_t* qa_pack, int G, float sm_scale, hipStream_t st, bool q_rot_unused,
+                        unsigned long long* arrivals) {
   const int d = layer->d;
   if (qa_pack) {       // operands of the matrix-core decode kernel wanted
     if (!q_stat || !layer->Pi_colsum || !layer->S_colsum || G > ROT_MAX_ROWS || rows % G || (d != 64 && d != 128 && d != 256))
       return TQ_EUNSUPPORTED;
-    if (opt_prep_units.load() && q_rot_unused) {
+    if (opt_prep_units.load() && q_rot_unused && !arrivals) {
       // heads per unit: as few as keep the launch at about a thousand workgroups
       const int64_t groups = rows / G;
       const int words = d / PREP_COLS;
@@ -389,7 +392,7 @@ int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* 
     }
     size_t smem = prep_smem_bytes(G, d);
     const dim3 grid((unsigned)(rows / G), d / PREP_COLS), block(PREP_COLS * PREP_SLICES);
-#define TQ_PREP(PER, DT) prep_query_kernel<PER, DT><<<grid, block, smem, st>>>(q, G, *layer, sm_scale, q_rot, q_sk, q_stat, qa_pack)
+#define TQ_PREP(PER, DT) prep_query_kernel<PER, DT><<<grid, block, smem, st>>>(q, G, *layer, sm_scale, q_rot, q_sk, q_stat, qa_pack, arrivals)
 #define TQ_PREP_DT(PER)                              \
   {                                                  \
     if (dtype == TQ_BF16) TQ_PREP(PER, TQ_BF16);     \
@@ -423,7 +426,7 @@ extern "C" int tq_rotate_query(const void* q, int dtype, int64_t rows, const tq_
   if (!q || !q_rot || !q_sk) return TQ_ENULL;
   if (rows < 0 || dtype < TQ_F32 || dtype > TQ_BF16) return TQ_EINVAL;
   if (rows == 0) return TQ_OK;
-  return launch_rotate_query(q, dtype, rows, layer, q_rot, q_sk, nullptr, nullptr, 1, 0.0f, (hipStream_t)stream, false);
+  return launch_rotate_query(q, dtype, rows, layer, q_rot, q_sk, nullptr, nullptr, 1, 0.0f, (hipStream_t)stream, false, nullptr);
 }
 
 extern "C" int tq_score(const void* q, int dtype, int64_t batch, int64_t n_q, const uint8_t* idx, const uint8_t* signs,
