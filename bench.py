@@ -572,6 +572,9 @@ def main():
         "quantize": quant,
         "round_trip": round_trip,
         "decode_gqa": {"workload": "16 seq x 8192 ctx, 32 q heads / 8 KV heads, head_dim 128, keys 3b, values 4b",
+                       "launches_per_step": 2 if gqa_w.n_split <= 8 else 3,
+                       "note": "with at most 8 context splits the page kernel merges them itself (its last-arriving "
+                               "workgroups), so kernel_ms includes that merge and no merge kernel follows",
                        "bytes_per_step": gqa_w.bytes, "GBps": gqa_w.bytes / (gqa_ms * 1e-3) / 1e9, "ms_per_step": gqa_ms,
                        "kernel_ms": gqa_kern, "kernel_GBps": gqa_w.bytes / (gqa_kern * 1e-3) / 1e9,
                        "kernel_frac": gqa_w.bytes / (gqa_kern * 1e-3) / 1e9 / HBM_PEAK_GBS,
