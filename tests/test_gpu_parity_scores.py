@@ -501,6 +501,20 @@ def test_splits_merged_inside_the_page_kernel(gpu, d, key_bits, vb, Hq, Hkv, len
         _set_option("merge_in_kernel", 1)
     assert torch.equal(got, again)
     assert (got - want).abs().max() <= 2 ** -7 * want.abs().max() + 1e-6        # one bf16 step of the largest value
+    # the same with an exact tail (its partial is one more part of the in-launch merge)
+    R = 40
+    rk = torch.randn(B, R, Hkv, d, generator=g).bfloat16().to(gpu)
+    rv = torch.randn(B, R, Hkv, d, generator=g).bfloat16().to(gpu)
+    rl = torch.tensor([R if i % 2 == 0 else 7 for i in range(B)], dtype=torch.int32, device=gpu)
+    try:
+        _set_option("merge_in_kernel", 0)
+        want_h = pool.decode_attention(q.to(gpu), table, seq, recent_k=rk, recent_v=rv, recent_len=rl, n_split=n_split).float().cpu()
+        _set_option("merge_in_kernel", 1)
+        got_h = pool.decode_attention(q.to(gpu), table, seq, recent_k=rk, recent_v=rv, recent_len=rl, n_split=n_split).float().cpu()
+        torch.cuda.synchronize()
+    finally:
+        _set_option("merge_in_kernel", 1)
+    assert (got_h - want_h).abs().max() <= 2 ** -7 * want_h.abs().max() + 1e-6
     prm = params_of(tq)
     for b in range(B):
         if lens[b] == 0:

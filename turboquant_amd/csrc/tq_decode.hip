@@ -714,7 +714,7 @@ static_assert(TAIL_THREADS == PREP_COLS * PREP_SLICES, "the two roles share a wo
 template <int PER, int DT, bool PAGED>
 __global__ void __launch_bounds__(TAIL_THREADS)
 prep_tail_kernel(TailArgs A, int n_tail, int B, int Gq, tq_layer ly, float* __restrict__ q_rot, float* __restrict__ q_sk,
-                 float* __restrict__ q_stat, uint32_t* __restrict__ qa_pack) {
+                 float* __restrict__ q_stat, uint32_t* __restrict__ qa_pack, unsigned long long* __restrict__ arrivals) {
   extern __shared__ __align__(16) float sm[];
   const int id = blockIdx.x;
   if (id < n_tail) {
@@ -722,6 +722,8 @@ prep_tail_kernel(TailArgs A, int n_tail, int B, int Gq, tq_layer ly, float* __re
     exact_tail_words_body<DT, 1, PAGED>(A, id % A.Hkv, (id / A.Hkv) % B, id / per_z, sm);
   } else {
     const int words = ly.d / PREP_COLS, p = id - n_tail;
+    // (the arrival counter of this group of query heads, for a page kernel that merges its splits itself)
+    if (arrivals != nullptr && p % words == 0 && threadIdx.x == 0) arrivals[p / words] = 0ull;
     prep_query_body<PER, DT>(A.q, Gq, ly, A.sm_scale, q_rot, q_sk, q_stat, qa_pack, p / words, p % words, sm);
   }
 }
@@ -1021,10 +1023,11 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   // (with many splits that workgroup would read more than the separate launch costs).  The preparation kernel
   // zeroes the arrival counters of its groups.
   FusedMerge fm;
-  if (stages == 7 && mfma_shape && !tail && !fused && n_split <= MERGE_IN_KERNEL_MAX_SPLITS && opt_merge_in_kernel.load()) {
+  if (stages == 7 && mfma_shape && !fused && n_split <= MERGE_IN_KERNEL_MAX_SPLITS && opt_merge_in_kernel.load()) {
     fm.out = out;
     fm.out_dtype = dtype;
     fm.counters = flags;
+    fm.n_extra = tail ? 1 : 0;          // the exact tail's partial, written by an earlier launch of this step
   }
   if ((stages & 1) && !fused) {
     if (!layer->Pi || !layer->PiT || !layer->S || !layer->ST || !layer->centroids) return TQ_ENULL;
@@ -1042,7 +1045,7 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
       if (e != hipSuccess) return (int)e;                                                                            \
     }                                                                                                                \
     kern<<<dim3((unsigned)(n_tail + n_prep)), dim3(TAIL_THREADS), fsm, st>>>(ta, n_tail, B, Gq, *layer, q_rot, q_sk,  \
-                                                                            q_stat, qa_pack);                        \
+                                                                            q_stat, qa_pack, fm.counters);           \
   }
 #define TQ_LAUNCH_PT_DT(PER, PAGED)                                \
   {                                                                \
@@ -1073,6 +1076,42 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   }
   if (!(stages & 6)) return TQ_OK;
 
+  // the exact tail's partial first (it depends on nothing the page kernel does), so that a page kernel that merges
+  // its splits itself finds it written
+  if (tail && (stages & 2) && !tail_done) {
+    const dim3 tgrid(Hkv, B, (G + TAIL_GC - 1) / TAIL_GC);
+    size_t tsm = words ? tail_words_smem(d, recent_rows) : tail_smem(d, recent_rows);
+#define TQ_LAUNCH_TAIL(KERN, ...)                                                                                    \
+  {                                                                                                                  \
+    auto kern = KERN;                                                                                                \
+    if (tsm > 48 * 1024) {                                                                                           \
+      hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)tsm);   \
+      if (e != hipSuccess) return (int)e;                                                                            \
+    }                                                                                                                \
+    kern<<<tgrid, dim3(TAIL_THREADS), tsm, st>>>(__VA_ARGS__);                                                       \
+  }
+#define TQ_TAIL_ROWS_ARGS q, Hq, Hkv, d, recent_k, recent_v, recent_rows, rs_b, rs_r, rs_h, recent_len, sm_scale, parts, n_parts, n_split
+#define TQ_TAIL_WORD_ARGS ta
+#define TQ_TAIL_WORDS(PAGED)                                                                                   \
+  {                                                                                                            \
+    if (dtype == TQ_BF16) TQ_LAUNCH_TAIL((exact_tail_words_kernel<TQ_BF16, 1, PAGED>), TQ_TAIL_WORD_ARGS)      \
+    else if (dtype == TQ_F16) TQ_LAUNCH_TAIL((exact_tail_words_kernel<TQ_F16, 1, PAGED>), TQ_TAIL_WORD_ARGS)   \
+    else if (d <= TAIL_THREADS) TQ_LAUNCH_TAIL((exact_tail_words_kernel<TQ_F32, 1, PAGED>), TQ_TAIL_WORD_ARGS) \
+    else TQ_LAUNCH_TAIL((exact_tail_words_kernel<TQ_F32, 2, PAGED>), TQ_TAIL_WORD_ARGS)                        \
+  }
+    if (words) {
+      if (ts.paged) TQ_TAIL_WORDS(true)
+      else TQ_TAIL_WORDS(false)
+    } else {      // 16-bit rows that are not word-aligned
+      if (dtype == TQ_BF16) TQ_LAUNCH_TAIL(exact_tail_kernel<TQ_BF16>, TQ_TAIL_ROWS_ARGS)
+      else TQ_LAUNCH_TAIL(exact_tail_kernel<TQ_F16>, TQ_TAIL_ROWS_ARGS)
+    }
+#undef TQ_TAIL_WORDS
+#undef TQ_TAIL_WORD_ARGS
+#undef TQ_TAIL_ROWS_ARGS
+#undef TQ_LAUNCH_TAIL
+    TQ_CHECK_LAUNCH();
+  }
   int mf = fused ? TQ_OK : TQ_EUNSUPPORTED;
   if ((stages & 2) && !fused)
     mf = mfma_shape ? launch_decode_mfma(qa_pack, q_stat, B, Hq, Hkv * kv_div, kv_div, pool, block_table, bt_stride,
@@ -1113,40 +1152,6 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   TQ_CHECK_LAUNCH();
   }
 
-  if (tail && (stages & 2) && !tail_done) {
-    const dim3 tgrid(Hkv, B, (G + TAIL_GC - 1) / TAIL_GC);
-    size_t tsm = words ? tail_words_smem(d, recent_rows) : tail_smem(d, recent_rows);
-#define TQ_LAUNCH_TAIL(KERN, ...)                                                                                    \
-  {                                                                                                                  \
-    auto kern = KERN;                                                                                                \
-    if (tsm > 48 * 1024) {                                                                                           \
-      hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)tsm);   \
-      if (e != hipSuccess) return (int)e;                                                                            \
-    }                                                                                                                \
-    kern<<<tgrid, dim3(TAIL_THREADS), tsm, st>>>(__VA_ARGS__);                                                       \
-  }
-#define TQ_TAIL_ROWS_ARGS q, Hq, Hkv, d, recent_k, recent_v, recent_rows, rs_b, rs_r, rs_h, recent_len, sm_scale, parts, n_parts, n_split
-#define TQ_TAIL_WORD_ARGS ta
-#define TQ_TAIL_WORDS(PAGED)                                                                                   \
-  {                                                                                                            \
-    if (dtype == TQ_BF16) TQ_LAUNCH_TAIL((exact_tail_words_kernel<TQ_BF16, 1, PAGED>), TQ_TAIL_WORD_ARGS)      \
-    else if (dtype == TQ_F16) TQ_LAUNCH_TAIL((exact_tail_words_kernel<TQ_F16, 1, PAGED>), TQ_TAIL_WORD_ARGS)   \
-    else if (d <= TAIL_THREADS) TQ_LAUNCH_TAIL((exact_tail_words_kernel<TQ_F32, 1, PAGED>), TQ_TAIL_WORD_ARGS) \
-    else TQ_LAUNCH_TAIL((exact_tail_words_kernel<TQ_F32, 2, PAGED>), TQ_TAIL_WORD_ARGS)                        \
-  }
-    if (words) {
-      if (ts.paged) TQ_TAIL_WORDS(true)
-      else TQ_TAIL_WORDS(false)
-    } else {      // 16-bit rows that are not word-aligned
-      if (dtype == TQ_BF16) TQ_LAUNCH_TAIL(exact_tail_kernel<TQ_BF16>, TQ_TAIL_ROWS_ARGS)
-      else TQ_LAUNCH_TAIL(exact_tail_kernel<TQ_F16>, TQ_TAIL_ROWS_ARGS)
-    }
-#undef TQ_TAIL_WORDS
-#undef TQ_TAIL_WORD_ARGS
-#undef TQ_TAIL_ROWS_ARGS
-#undef TQ_LAUNCH_TAIL
-    TQ_CHECK_LAUNCH();
-  }
   if (!(stages & 4)) return TQ_OK;
   // without a tail the merge simply reads one part fewer
   merge_kernel<<<dim3((unsigned)(B * Hq)), dim3(256), merge_smem(n_parts, d), st>>>(

@@ -26,6 +26,7 @@ struct FusedMerge {
   void* out = nullptr;               // (B, Hq, d) in out_dtype
   int out_dtype = 0;
   unsigned long long* counters = nullptr;
+  int n_extra = 0;                   // parts after the n_split splits that an earlier launch has written (the exact tail)
 };
 constexpr int MERGE_IN_KERNEL_MAX_SPLITS = 8;
 

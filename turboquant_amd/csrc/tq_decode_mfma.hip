@@ -825,21 +825,23 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
         const bool live = o < G * D;
         const int g = live ? o / D : 0, ch = o % D;
         const float* row = parts + ((int64_t)b * Hq + h * G + g) * n_parts * (D + 2);
-        // all loads first (clamped to an existing split), then the log-sum-exp merge
-        float m_s[MERGE_IN_KERNEL_MAX_SPLITS], l_s[MERGE_IN_KERNEL_MAX_SPLITS], a_s[MERGE_IN_KERNEL_MAX_SPLITS];
+        // all loads first (clamped to an existing part), then the log-sum-exp merge
+        constexpr int NP = MERGE_IN_KERNEL_MAX_SPLITS + 1;
+        const int n_merge = n_split + fm.n_extra;
+        float m_s[NP], l_s[NP], a_s[NP];
 #pragma unroll
-        for (int sp = 0; sp < MERGE_IN_KERNEL_MAX_SPLITS; ++sp) {
-          const float* r = row + (int64_t)min(sp, n_split - 1) * (D + 2);
+        for (int sp = 0; sp < NP; ++sp) {
+          const float* r = row + (int64_t)min(sp, n_merge - 1) * (D + 2);
           m_s[sp] = load_coherent(r); l_s[sp] = load_coherent(r + 1); a_s[sp] = load_coherent(r + 2 + ch);
         }
         float mm = MF_NEG;
 #pragma unroll
-        for (int sp = 0; sp < MERGE_IN_KERNEL_MAX_SPLITS; ++sp)
-          if (sp < n_split && l_s[sp] > 0.0f) mm = fmaxf(mm, m_s[sp]);
+        for (int sp = 0; sp < NP; ++sp)
+          if (sp < n_merge && l_s[sp] > 0.0f) mm = fmaxf(mm, m_s[sp]);
         float ll = 0.0f, aa = 0.0f;
 #pragma unroll
-        for (int sp = 0; sp < MERGE_IN_KERNEL_MAX_SPLITS; ++sp) {
-          const float wgt = (sp < n_split && l_s[sp] > 0.0f) ? __expf(m_s[sp] - mm) : 0.0f;
+        for (int sp = 0; sp < NP; ++sp) {
+          const float wgt = (sp < n_merge && l_s[sp] > 0.0f) ? __expf(m_s[sp] - mm) : 0.0f;
           ll = fmaf(wgt, l_s[sp], ll);
           aa = fmaf(wgt, a_s[sp], aa);
         }
