@@ -331,6 +331,9 @@ void tq_time_next_key_kernel(void *start_event, void *stop_event);
  *   "merge_in_kernel"  1 (default): a compressed-only decode step on the matrix-core kernel with at most 8 context
  *                      splits has its splits merged by the last workgroup of the page kernel (two launches per
  *                      step); 0: always the separate merge kernel.
+ *   "page_pairs"       1 (default): head_dim 64 with at most 4 query heads per KV head scores two pages per
+ *                      matrix instruction (block-diagonal query operand); 0: one page per instruction, half
+ *                      of the contraction idle (the kernel of more than 4 heads per KV head).
  *   "fp6_centroids"    1 (default): the key quantiser takes the fp6 x fp4 centroid contraction when the layer
  *                      carries PiT_fp6; 0: always the bf16 term products (for A/B runs).
  *   "append_parts"     measurement only: 3 (default) = the append entry points quantise keys and values,

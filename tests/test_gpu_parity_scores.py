@@ -466,6 +466,50 @@ def test_decode_head_dim_64_on_the_matrix_cores(gpu, key_bits, vb, Hq, Hkv, dtyp
     _progress(f"   worst cosine {worst:.7f}")
 
 
+@pytest.mark.parametrize("key_bits,vb,Hq,Hkv,dtype", [(3, 4, 8, 2, torch.bfloat16), (4, 2, 3, 1, torch.float16),
+                                                       (2, 2, 2, 2, torch.bfloat16)])
+def test_head_dim_64_two_pages_per_score_instruction(gpu, key_bits, vb, Hq, Hkv, dtype):
+    """With at most four query heads per KV head the head_dim 64 kernel scores two pages per matrix instruction
+    (block-diagonal query operand).  The sums are the same ones in the same order, so the output must equal,
+    bit for bit, that of the one-page-per-instruction kernel (option "page_pairs" = 0, itself checked against
+    the oracle above) - for ragged ends inside either page of a pair, table entries outside the pool in either
+    half, and several split counts; and it is checked against the oracle (score.py:84-173) directly."""
+    d, B = 64, 4
+    lens = [1000, 17, 16 * 37 + 1, 16 * 6]          # ends in the 1st / 2nd page of a pair, on a pair boundary
+    n_log = max((n + 15) // 16 for n in lens)
+    n_pages = B * n_log + 1
+    pool, tq = _make_pool(gpu, d, key_bits, vb, Hkv, n_pages, dtype, seed=77)
+    g = torch.Generator().manual_seed(640 + key_bits)
+    k = torch.randn(B, max(lens), Hkv, d, generator=g).to(dtype)
+    v = torch.randn(B, max(lens), Hkv, d, generator=g).to(dtype)
+    q = torch.randn(B, Hq, d, generator=g).to(dtype)
+    table = torch.randperm(n_pages, generator=g)[: B * n_log].to(torch.int32).view(B, n_log)
+    pool.append(k.to(gpu), v.to(gpu), table.to(gpu))
+    seq = torch.tensor(lens, dtype=torch.int32, device=gpu)
+    bad = table.clone()
+    bad[0, [4, 7, 20, 21]] = torch.tensor([n_pages, -1, 2 ** 31 - 1, -9], dtype=torch.int32)
+    prm = params_of(tq)
+    _progress(f"page pairs d=64 kb={key_bits} vb={vb} Hq={Hq} Hkv={Hkv} {dtype}")
+    try:
+        for tab in (table, bad):
+            for n_split in (1, 3, 8, 11):
+                outs = []
+                for on in (1, 0):
+                    _set_option("page_pairs", on)
+                    outs.append(pool.decode_attention(q.to(gpu), tab.to(gpu), seq, n_split=n_split, max_len=max(lens)).cpu())
+                torch.cuda.synchronize()
+                assert torch.equal(outs[0], outs[1]), (n_split, tab is bad)
+        _set_option("page_pairs", 1)
+        out = pool.decode_attention(q.to(gpu), table.to(gpu), seq, n_split=2, max_len=max(lens)).cpu()
+        for b in range(B):
+            idx, sgn, norms, rn, vd, vs, vz = [t.cpu() for t in pool.export_flat(table[b], lens[b])]
+            want = O.hybrid_attention(q[b:b + 1], key_code(idx, sgn, rn, norms, key_bits - 1), value_code(vd, vs, vz, vb),
+                                      lens[b], prm, Hkv, None, None)
+            assert cosine(out[b:b + 1], want) >= COS_GATE, b
+    finally:
+        _set_option("page_pairs", 1)
+
+
 @pytest.mark.parametrize("d,key_bits,vb,Hq,Hkv,lens,n_split", [
     (128, 3, 4, 32, 8, [900, 1, 16, 0, 517], 4),
     (128, 3, 2, 8, 1, [2100], 8),

@@ -846,6 +846,7 @@ std::atomic<int> opt_prep_units{0};
 std::atomic<int> opt_append_parts{3};
 std::atomic<int> opt_fp6_centroids{1};
 std::atomic<int> opt_merge_in_kernel{1};
+std::atomic<int> opt_page_pairs{1};
 }  // namespace tq
 
 namespace {
@@ -876,6 +877,7 @@ extern "C" int tq_set_option(const char* name, int64_t value) {
     opt_prep_spin_limit.store((int)value);
     return TQ_OK;
   }
+  if (!std::strcmp(name, "page_pairs")) { opt_page_pairs.store(value != 0); return TQ_OK; }
   if (!std::strcmp(name, "merge_in_kernel")) { opt_merge_in_kernel.store(value != 0); return TQ_OK; }
   if (!std::strcmp(name, "fp6_centroids")) { opt_fp6_centroids.store(value != 0); return TQ_OK; }
   if (!std::strcmp(name, "append_parts")) {

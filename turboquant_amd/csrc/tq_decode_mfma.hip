@@ -51,6 +51,7 @@
 #include "tq_common.h"
 #include "tq_prep.h"
 #include "tq_decode_mfma.h"
+#include "tq_options.h"
 
 namespace tq {
 
@@ -140,6 +141,16 @@ __device__ __forceinline__ float row_max16(float v) {
   v = fmaxf(v, dpp<0x140>(v));
   return v;
 }
+// all-reduce over the two lanes 32 apart (the half-swap instruction of gfx950: no LDS round trip)
+__device__ __forceinline__ float max_xor32(float v) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(fmaxf(v, __uint_as_float(r[0])), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float sum_xor32(float v) {
+  // r[0] holds the lower half's values in both halves, r[1] the upper half's
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
 __device__ __forceinline__ float row_sum16(float v) {
   v += dpp<0xB1>(v);
   v += dpp<0x4E>(v);
@@ -172,7 +183,13 @@ __device__ __forceinline__ constexpr int v_bitpos(int t) {
 // D in {128, 256}; MB stored index bits; NX extra (multi-bit) Walsh terms; VB value bits;
 // GS value group size; DS wavefronts that share one block (each takes D/DS coordinates and
 // channels); WPS wavefronts per SIMD the register budget is sized for.
-template <int D, int MB, int NX, int VB, int GS, int DS, int WPS, bool F16P>
+// PP (head_dim 64, at most 4 query heads per KV head): one score MFMA serves two pages.  The contraction is
+// 128 long and a head has 64 coordinates, so the lanes of the upper two coordinate quarters hold the key
+// words of a second page, and the query operand is block-diagonal: rows 0..7 (4 heads x 2 terms) carry the
+// query in coordinates 0..63 and score the first page, rows 8..15 carry the same terms in coordinates
+// 64..127 and score the second.  Lane (n, kb) then sees heads 2(kb%2), 2(kb%2)+1 of token n of page
+// 2 * pair + kb/2; the value stage is the same as without PP.
+template <int D, int MB, int NX, int VB, int GS, int DS, int WPS, bool F16P, bool PP>
 __global__ void __launch_bounds__(MF_WAVES * 64, WPS)
 decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div,
                    const uint8_t* __restrict__ pool, const int32_t* __restrict__ block_table,
@@ -191,8 +208,10 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   constexpr int PIECES = 2 * NG;              // 16-byte pieces of this wavefront's scales per page
   constexpr int NGRP = MF_WAVES / DS;         // wavefront groups (each walks its own blocks)
   constexpr int WAVE_LDS_FLOATS = wave_lds_floats(NG, DS);
+  constexpr int NPG = PP ? 2 : 4;             // score MFMA groups per block: pages, or pairs of pages
   static_assert(NG >= 2 && NG % 2 == 0 && (DW % 128 == 0 || (D == 64 && DS == 1)),
                 "a wavefront takes whole 128-coordinate chunks (or a whole head of 64) and whole group pairs");
+  static_assert(!PP || (D == 64 && DS == 1), "page pairs are for head_dim 64");
   // Hkv counts query-head groups: a KV head with more than 8 query heads is served by kv_div groups
   // of G <= 8 heads each (consecutive groups read the same pages)
   const int G = Hq / Hkv;
@@ -259,7 +278,10 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   // lane are stored at a stride of eight.
   i32x8 qa[NTP][WPL][2];
   {
-    const uint32_t* src = qa_pack + (((int64_t)b * Hkv + h) * (NTP * WPLT * 2 * 64) + lane) * 8;
+    // PP: rows 8..15 / coordinates 64..127 repeat rows 0..7 / coordinates 0..63; the off-diagonal blocks are zero
+    const int slane = PP ? (n & 7) + 16 * (kb & 1) : lane;
+    const bool a_live = !PP || ((n < 8) == (kb < 2));
+    const uint32_t* src = qa_pack + (((int64_t)b * Hkv + h) * (NTP * WPLT * 2 * 64) + slane) * 8;
 #pragma unroll
     for (int tp = 0; tp < NTP; ++tp)
 #pragma unroll
@@ -277,6 +299,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
             const uint32_t d4 = p6[4], d5 = p6[5];
             qa[tp][i][rs] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)d4, (int)d5, 0, 0};
           }
+          if (!a_live) qa[tp][i][rs] = i32x8{0, 0, 0, 0, 0, 0, 0, 0};
         }
   }
   // E8M0 block-scale codes of this lane's operand row (head n / 2), one per byte: index planes row
@@ -284,7 +307,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   // 2^(E - 2 - 5t); the fp4 bit value 0.5 carries 2^1.
   int sa;
   {
-    const int g = n >> 1;
+    const int g = PP ? (n & 7) >> 1 : n >> 1;
     const int64_t qrow = (int64_t)b * Hq + h * G + (g < G ? g : 0);
     const bool coh = fused_build && fz.q != nullptr;
     const int e1 = 127 + (int)(coh ? load_coherent(q_stat + qrow * 4 + 0) : q_stat[qrow * 4 + 0]);
@@ -295,7 +318,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   const int sb = 127 + 1;
   // head_dim 64: the score MFMA still contracts 128 coordinates; the lanes of the upper two coordinate
   // quarters feed zeros (their masks are zero, whatever their loads return)
-  const bool kq_live = D >= 128 || kb < D / 32;
+  const bool kq_live = D >= 128 || PP || kb < D / 32;
   const uint32_t nib = in_vgpr(kq_live ? 0x11111111u : 0u), nib1 = in_vgpr(kq_live ? 0x22222222u : 0u),
                  nib2 = in_vgpr(kq_live ? 0x44444444u : 0u);
   // constant parts of the scores of the two heads this lane sees in the MFMA output (rows 4kb..4kb+3
@@ -305,7 +328,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   {
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      const int g = 2 * kb + j;
+      const int g = PP ? 2 * (kb & 1) + j : 2 * kb + j;
       const bool live = g < G && hf == 0;
       const int64_t qrow = (int64_t)b * Hq + h * G + (g < G ? g : 0);
       const bool coh = fused_build && fz.q != nullptr;
@@ -325,6 +348,11 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
     }
   }
 
+  if (PP) {
+    // rows of heads 4..7 are never written with page pairs; the value stage reads them as operand rows
+    // whose results nobody uses: keep them finite
+    for (int i = lane; i < 4 * 16 * P_STRIDE + 16; i += 64) s_p[i] = 0.0f;
+  }
   // ---------------------------------------------------------------- work range (all scalar)
   // len_sub: newest tokens that are attended to exactly.  A length beyond the block table is cut to the table.
   const int seq_len = max(min(seq_lens[b], max_pages * TQ_PAGE_TOKENS) - len_sub, 0);
@@ -339,7 +367,8 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   const uint32_t page_stride32 = (uint32_t)page_stride;
   // per lane the key words are [word i][plane], the value fields [channel tile]: a wavefront's share is contiguous
   // (head_dim 64: the idle lanes re-read the last live lane's words)
-  const int klane = D >= 128 ? lane : min(lane, D / 2 - 1);
+  // (PP: every lane is live: word kb % 2 of token n, of the pair's first page for kb < 2, else of its second)
+  const int klane = D >= 128 ? lane : (PP ? (kb & 1) * 16 + n : min(lane, D / 2 - 1));
   const uint32_t off_keys = L.off_keys + (klane * DS + hf) * (NKW * 4), off_meta = L.off_meta + n * 8;
   const uint32_t off_v = L.off_vdata + (n * DS + hf) * (VW * 4);
   const uint32_t off_scale = L.off_vscale + hf * (NG * 32) + (lane % PIECES) * 16;
@@ -355,7 +384,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   constexpr float REF_SLACK = 4.0f;
   float m_run[2] = {MF_NEG, MF_NEG}, l_run[2] = {0.0f, 0.0f};
 
-  struct KeyRegs { uint32_t key[4][NKW]; f32x2 meta[4]; };
+  struct KeyRegs { uint32_t key[NPG][NKW]; f32x2 meta[NPG]; };
   struct ValRegs { uint32_t v[VW]; u32x4 zero[2]; u32x4 scale; };
 
   // page ids of block `blk` -> 4 scalars; a page past the end of the sequence (last block only) is
@@ -381,6 +410,19 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
     // the 32-bit lane offsets are re-materialised here, next to their use, so that the loads take
     // the scalar page base plus a 32-bit vector offset instead of a 64-bit vector address
     const uint32_t ok = in_vgpr(off_keys), om = in_vgpr(off_meta);
+    if constexpr (PP) {
+      const uint32_t p0 = in_vgpr((uint32_t)pid[0]), p1 = in_vgpr((uint32_t)pid[1]), p2 = in_vgpr((uint32_t)pid[2]),
+                     p3 = in_vgpr((uint32_t)pid[3]);
+#pragma unroll
+      for (int pr = 0; pr < 2; ++pr) {
+        const uint32_t my_pid = kb < 2 ? (pr == 0 ? p0 : p2) : (pr == 0 ? p1 : p3);
+        const uint8_t* base = pool_h + (uint64_t)my_pid * page_stride32;
+        const uint32_t* kp = (const uint32_t*)(base + ok);
+#pragma unroll
+        for (int w = 0; w < NKW; ++w) R.key[pr][w] = kp[w];
+        R.meta[pr] = *(const f32x2*)(base + om);
+      }
+    } else
 #pragma unroll
     for (int pg = 0; pg < 4; ++pg) {
       // (page numbers are non-negative and the stride fits 32 bits: an unsigned 32 x 32 -> 64 bit product)
@@ -430,7 +472,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   bool fresh = true;                            // this walker has not seen a token yet: no reference
   auto score_stage = [&](int blk, int it, bool first, const KeyRegs& K, int bad, auto partial_tag) -> bool {
     constexpr bool PARTIAL = decltype(partial_tag)::value;
-    float s2[2][4];
+    float s2[2][NPG];
     float mref[2];                              // only one wavefront of a pair subtracts it
 #pragma unroll
     for (int j = 0; j < 2; ++j) mref[j] = (first || hf != 0) ? 0.0f : m_run[j];
@@ -439,7 +481,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
     // both alternating between the two kinds of instruction.
     __builtin_amdgcn_s_setprio(1);
 #pragma unroll
-    for (int pg = 0; pg < 4; ++pg) {
+    for (int pg = 0; pg < NPG; ++pg) {
       f32x4 dm = cm, dq = cq;
 #pragma unroll
       for (int i = 0; i < WPL; ++i) {
@@ -475,12 +517,12 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
     // arithmetic), which run in the shadow of the matrix pipe.
     __builtin_amdgcn_sched_group_barrier(0x002, 5 * NTP * WPL, 0);
 #pragma unroll
-    for (int k = 0; k < 4 * 2 * NTP * WPL; ++k) {
+    for (int k = 0; k < NPG * 2 * NTP * WPL; ++k) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
     }
     __builtin_amdgcn_s_setprio(0);
-    if (DS > 1) {
+    if constexpr (DS > 1) {
       // exchange with the wavefront that scored the other coordinates: own share -> LDS, workgroup
       // barrier, partner's share <- LDS.  a + b == b + a, so both end with bit-identical scores.
       float* mine = s_x + (it & 1) * (8 * 64);
@@ -495,12 +537,14 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
 #pragma unroll
         for (int pg = 0; pg < 4; ++pg) s2[j][pg] += theirs[(j * 4 + pg) * 64 + lane];
     }
-    bool gone[4] = {false, false, false, false};
+    bool gone[NPG];
+#pragma unroll
+    for (int pg = 0; pg < NPG; ++pg) gone[pg] = false;
     if (PARTIAL) {
       bool any = false;
 #pragma unroll
-      for (int pg = 0; pg < 4; ++pg) {
-        gone[pg] = n >= tokens_of_page(blk, pg, bad);
+      for (int pg = 0; pg < NPG; ++pg) {
+        gone[pg] = n >= tokens_of_page(blk, PP ? 2 * pg + (kb >> 1) : pg, bad);
         any |= !gone[pg];
 #pragma unroll
         for (int j = 0; j < 2; ++j)
@@ -510,8 +554,9 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
       fresh = fresh && __builtin_amdgcn_ballot_w64(any) == 0;
     }
     // ---- online softmax (log2 domain) against a lazily updated reference
-    float mx = fmaxf(fmaxf(fmaxf(s2[0][0], s2[0][1]), fmaxf(s2[0][2], s2[0][3])),
-                     fmaxf(fmaxf(s2[1][0], s2[1][1]), fmaxf(s2[1][2], s2[1][3])));
+    float mx = fmaxf(s2[0][0], s2[1][0]);
+#pragma unroll
+    for (int pg = 1; pg < NPG; ++pg) mx = fmaxf(mx, fmaxf(s2[0][pg], s2[1][pg]));
     const bool rescale = first || __builtin_amdgcn_ballot_w64(mx > REF_SLACK) != 0;
     if (rescale) {
       // move the reference to the row maximum (never down, except for the first block, where the
@@ -519,27 +564,31 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
       float alpha[2];
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
-        float mj = fmaxf(fmaxf(s2[j][0], s2[j][1]), fmaxf(s2[j][2], s2[j][3]));
+        float mj = s2[j][0];
+#pragma unroll
+        for (int pg = 1; pg < NPG; ++pg) mj = fmaxf(mj, s2[j][pg]);
         mj = row_max16(mj);
+        if (PP) mj = max_xor32(mj);                 // the lanes 32 apart hold the same heads
         const float delta = first ? mj : fmaxf(mj, 0.0f);
         alpha[j] = first ? 1.0f : __builtin_amdgcn_exp2f(-delta);
         m_run[j] = first ? delta : m_run[j] + delta;
         l_run[j] *= alpha[j];
 #pragma unroll
-        for (int pg = 0; pg < 4; ++pg) s2[j][pg] -= delta;
+        for (int pg = 0; pg < NPG; ++pg) s2[j][pg] -= delta;
       }
-      if (n == 0) { s_alpha[2 * kb] = alpha[0]; s_alpha[2 * kb + 1] = alpha[1]; }
+      if (n == 0 && (!PP || kb < 2)) { s_alpha[2 * kb] = alpha[0]; s_alpha[2 * kb + 1] = alpha[1]; }
     }
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       float psum = 0.0f;
 #pragma unroll
-      for (int pg = 0; pg < 4; ++pg) {
+      for (int pg = 0; pg < NPG; ++pg) {
         // (a token that does not exist has weight 0 even when the whole block is empty and the
         // reference therefore sits at the masking value itself)
         const float p = PARTIAL && gone[pg] ? 0.0f : __builtin_amdgcn_exp2f(s2[j][pg]);
         psum += p;
-        s_p[(pg * 16 + 2 * kb + j) * P_STRIDE + n] = p;
+        if (PP) s_p[((2 * pg + (kb >> 1)) * 16 + 2 * (kb & 1) + j) * P_STRIDE + n] = p;
+        else s_p[(pg * 16 + 2 * kb + j) * P_STRIDE + n] = p;
       }
       l_run[j] += psum;
     }
@@ -735,9 +784,10 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   if (hf == 0) {                                               // the wavefronts of a pair hold the same (m, l)
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      const float lsum = row_sum16(l_run[j]);
-      const int g = 2 * kb + j;
-      if (n == 0 && g < G) {
+      float lsum = row_sum16(l_run[j]);
+      if (PP) lsum = sum_xor32(lsum);
+      const int g = PP ? 2 * (kb & 1) + j : 2 * kb + j;
+      if (n == 0 && g < G && (!PP || kb < 2)) {
         float* r = s_red + (wgrp * G + g) * (D + 2);
         r[0] = m_run[j] * 0.6931471805599453f;     // back to the natural-log domain of the partials
         r[1] = lsum;
@@ -863,7 +913,7 @@ bool take_time_hook(int which, hipEvent_t& start, hipEvent_t& stop) {
   return start != nullptr || stop != nullptr;
 }
 
-template <int D, int MB, int NX, int VB, int GS, int DS, int WPS, bool F16P>
+template <int D, int MB, int NX, int VB, int GS, int DS, int WPS, bool F16P, bool PP = false>
 static int launch_one(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, int kv_div,
                       const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
                       float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts, int n_split,
@@ -876,7 +926,11 @@ static int launch_one(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, 
     const size_t prep = (size_t)prep_unit_smem_floats(fz.hp, D) * sizeof(float);
     if (prep > smem) smem = prep;
   }
-  auto kern = decode_mfma_kernel<D, MB, NX, VB, GS, DS, WPS, F16P>;
+  if (D == 64 && !PP && G <= 4 && opt_page_pairs.load(std::memory_order_relaxed) != 0)
+    return launch_one<D, MB, NX, VB, GS, DS, WPS, F16P, D == 64>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,
+                                                                 bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts,
+                                                                 n_split, len_sub, max_pages, num_pages, fz, fm, st);
+  auto kern = decode_mfma_kernel<D, MB, NX, VB, GS, DS, WPS, F16P, PP>;
   if (smem > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return (int)e;

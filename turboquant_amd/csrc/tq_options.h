@@ -9,5 +9,6 @@ extern std::atomic<int> opt_prep_spin_limit;   // polls before a workgroup of th
 extern std::atomic<int> opt_prep_units;        // stand-alone preparation: one workgroup per (few heads, plane word) unit
 extern std::atomic<int> opt_append_parts;      // measurement: 3 keys and values (the product), 1 keys only, 2 values only
 extern std::atomic<int> opt_fp6_centroids;     // key quantiser, head_dim 128: centroid contraction on the fp6 x fp4 MFMA
+extern std::atomic<int> opt_page_pairs;        // decode, head_dim 64 with at most 4 query heads per KV head: one score MFMA per two pages
 extern std::atomic<int> opt_merge_in_kernel;    // decode: few context splits are merged by the last workgroup of the page kernel
 }  // namespace tq
