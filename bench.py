@@ -520,19 +520,24 @@ def main():
     if not args.no_cpu:
         gqa_cpu = cpu_decode_baseline(gqa_w, runs=3)
 
+    def side_leg(d, key_bits, text):
+        w = DecodeWorkload(text, 16, 8192, 32, 8, d, key_bits, 4, n_pools=4, seed=2, dist="normal", device=device)
+        ms_, _ = time_steps(w.step, args.steps, args.warmup)
+        kern_ = time_kernel_stage(w, args.steps, args.warmup)
+        leg = {"workload": text, "launches_per_step": 2 if w.n_split <= 8 else 3,
+               "bytes_per_step": w.bytes, "GBps": w.bytes / (ms_ * 1e-3) / 1e9, "ms_per_step": ms_,
+               "pct_hbm_peak": 100.0 * w.bytes / (ms_ * 1e-3) / 1e9 / HBM_PEAK_GBS,
+               "kernel_ms": kern_, "kernel_GBps": w.bytes / (kern_ * 1e-3) / 1e9,
+               "kernel_frac": w.bytes / (kern_ * 1e-3) / 1e9 / HBM_PEAK_GBS}
+        del w
+        torch.cuda.empty_cache()
+        return leg
     # the same shape with 4-bit keys (3-bit indices in nibbles + sign plane): the reference's default for the
     # first four layers (integration/vllm.py:358-359)
-    kb4_w = DecodeWorkload("gqa decode, 4-bit keys", 16, 8192, 32, 8, 128, 4, 4, n_pools=4, seed=2, dist="normal",
-                           device=device)
-    kb4_ms, _ = time_steps(kb4_w.step, args.steps, args.warmup)
-    kb4_kern = time_kernel_stage(kb4_w, args.steps, args.warmup)
-    kb4 = {"workload": "16 seq x 8192 ctx, 32 q heads / 8 KV heads, head_dim 128, keys 4b, values 4b",
-           "bytes_per_step": kb4_w.bytes, "GBps": kb4_w.bytes / (kb4_ms * 1e-3) / 1e9, "ms_per_step": kb4_ms,
-           "pct_hbm_peak": 100.0 * kb4_w.bytes / (kb4_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-           "kernel_ms": kb4_kern, "kernel_GBps": kb4_w.bytes / (kb4_kern * 1e-3) / 1e9,
-           "kernel_frac": kb4_w.bytes / (kb4_kern * 1e-3) / 1e9 / HBM_PEAK_GBS}
-    del kb4_w
-    torch.cuda.empty_cache()
+    kb4 = side_leg(128, 4, "16 seq x 8192 ctx, 32 q heads / 8 KV heads, head_dim 128, keys 4b, values 4b")
+    # the smallest head size the reference ships codebooks for (codebooks/codebook_d64_b*.json); with 4 query heads
+    # per KV head the kernel scores two pages per matrix instruction
+    d64 = side_leg(64, 3, "16 seq x 8192 ctx, 32 q heads / 8 KV heads, head_dim 64, keys 3b, values 4b")
 
     quant, (qpool, qk, qv, qtable, qtq) = quantize_bench(device, max(5, args.steps // 5), max(2, args.warmup // 5))
     round_trip = round_trip_bench(device, max(5, args.steps // 5), max(2, args.warmup // 5), not args.no_cpu)
@@ -581,6 +586,7 @@ def main():
                        "pct_hbm_peak": 100.0 * gqa_w.bytes / (gqa_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
                        "cpu_baseline": gqa_cpu},
         "decode_gqa_kb4": kb4,
+        "decode_gqa_d64": d64,
         "decode_hybrid": {"note": "whole step with the newest 128 tokens exact, read in place from a paged bf16 cache "
                                   "(tq_decode_attn_paged_ring); bytes = pages of the older tokens + the exact rows",
                           "long_context": hybrid_main, "gqa": hybrid_gqa},

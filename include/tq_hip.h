@@ -334,6 +334,10 @@ void tq_time_next_key_kernel(void *start_event, void *stop_event);
  *   "page_pairs"       1 (default): head_dim 64 with at most 4 query heads per KV head scores two pages per
  *                      matrix instruction (block-diagonal query operand); 0: one page per instruction, half
  *                      of the contraction idle (the kernel of more than 4 heads per KV head).
+ *   "narrow_rows"      1 (default): head_dim 128 / 256 with at most 4 query heads per KV head puts the four fp6
+ *                      terms of a head into one score operand (one matrix instruction per plane word); 0: two.
+ *   "lds_stage"        1 (default): the 4-bit-key kernels of head_dim 128 / 256 bring the next block's page data
+ *                      into LDS with LDS-direct loads instead of holding it in registers; 0: registers (spills).
  *   "fp6_centroids"    1 (default): the key quantiser takes the fp6 x fp4 centroid contraction when the layer
  *                      carries PiT_fp6; 0: always the bf16 term products (for A/B runs).
  *   "append_parts"     measurement only: 3 (default) = the append entry points quantise keys and values,

@@ -847,6 +847,8 @@ std::atomic<int> opt_append_parts{3};
 std::atomic<int> opt_fp6_centroids{1};
 std::atomic<int> opt_merge_in_kernel{1};
 std::atomic<int> opt_page_pairs{1};
+std::atomic<int> opt_narrow_rows{1};
+std::atomic<int> opt_lds_stage{1};
 }  // namespace tq
 
 namespace {
@@ -877,6 +879,8 @@ extern "C" int tq_set_option(const char* name, int64_t value) {
     opt_prep_spin_limit.store((int)value);
     return TQ_OK;
   }
+  if (!std::strcmp(name, "lds_stage")) { opt_lds_stage.store(value != 0); return TQ_OK; }
+  if (!std::strcmp(name, "narrow_rows")) { opt_narrow_rows.store(value != 0); return TQ_OK; }
   if (!std::strcmp(name, "page_pairs")) { opt_page_pairs.store(value != 0); return TQ_OK; }
   if (!std::strcmp(name, "merge_in_kernel")) { opt_merge_in_kernel.store(value != 0); return TQ_OK; }
   if (!std::strcmp(name, "fp6_centroids")) { opt_fp6_centroids.store(value != 0); return TQ_OK; }

@@ -79,8 +79,34 @@ constexpr float MF_NEG = -1.0e30f;
 constexpr int P_STRIDE = 20;             // floats per row of the LDS softmax-weight tile (16 + skew)
 constexpr int X_FLOATS = 2 * 8 * 64;     // score-half exchange slot of a wavefront: [parity][8 values][64 lanes]
 __host__ __device__ constexpr int wave_lds_floats(int ng, int ds) {
-  return 4 * 16 * P_STRIDE + 16 + 4 * ng * 16 + (ds > 1 ? X_FLOATS : 0);
+  return 4 * 8 * P_STRIDE + 16 + 4 * ng * 16 + (ds > 1 ? X_FLOATS : 0);
 }
+// Staging area of a wavefront for page data that travels HBM -> LDS without passing through registers
+// (SG kernels): every piece is what one LDS-direct load instruction writes, 16 bytes per lane:
+// [4 pages] key words, [32 lanes] norms, [VW / 4] value words, [2] zero points, [1] scales.
+__host__ __device__ constexpr int stage_bytes(int vw) { return 4 * 1024 + 512 + (vw / 4) * 1024 + 2 * 1024 + 1024; }
+
+// LDS-direct loads (gfx950: 12 and 16 bytes per lane): lane l's bytes land at m0 + OFF + 16 l, read from
+// its address + OFF.  The compiler does not see these instructions: it neither counts them in vmcnt nor
+// orders LDS accesses against them; the kernel waits for them itself (stage_wait) before it reads the area.
+template <int OFF>
+__device__ __forceinline__ void dma16(const void* vaddr, uint32_t m0) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off offset:%2"
+               :: "v"(vaddr), "s"(m0), "n"(OFF) : "memory", "m0");
+}
+template <int BYTES>
+__device__ __forceinline__ void dma_so(uint32_t voff, const void* sbase, uint32_t m0) {
+  // (12 bytes: three dwords per lane; anything else is taken as four)
+  if (BYTES == 12)
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx3 %0, %1" :: "v"(voff), "s"(sbase), "s"(m0) : "memory", "m0");
+  else
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" :: "v"(voff), "s"(sbase), "s"(m0) : "memory", "m0");
+}
+// wait until at most N vector-memory instructions of this wavefront are outstanding (they complete in order)
+template <int N>
+__device__ __forceinline__ void stage_wait() { asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory"); }
+// the LDS reads issued so far have returned: their area may be overwritten
+__device__ __forceinline__ void stage_release() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
   f32x2 f = {lo, hi};
@@ -189,7 +215,13 @@ __device__ __forceinline__ constexpr int v_bitpos(int t) {
 // query in coordinates 0..63 and score the first page, rows 8..15 carry the same terms in coordinates
 // 64..127 and score the second.  Lane (n, kb) then sees heads 2(kb%2), 2(kb%2)+1 of token n of page
 // 2 * pair + kb/2; the value stage is the same as without PP.
-template <int D, int MB, int NX, int VB, int GS, int DS, int WPS, bool F16P, bool PP>
+// NR (at most 4 query heads per KV head, head_dim 128 / 256): the four fp6 terms of a head fill four rows of
+// ONE operand (row 4g + t) instead of two rows in each of two, so a plane word takes one score MFMA, the
+// query operands half the registers, and lane (n, kb) sees a single head (kb) of token n.
+// SG: the page data of the next block goes HBM -> LDS with LDS-direct loads, requested when the current
+// block's copy has been taken out of LDS, so every load has a whole trip to arrive (instead of one stage)
+// and no register holds data in flight.
+template <int D, int MB, int NX, int VB, int GS, int DS, int WPS, bool F16P, bool PP, bool NR, bool SG>
 __global__ void __launch_bounds__(MF_WAVES * 64, WPS)
 decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div,
                    const uint8_t* __restrict__ pool, const int32_t* __restrict__ block_table,
@@ -212,6 +244,11 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   static_assert(NG >= 2 && NG % 2 == 0 && (DW % 128 == 0 || (D == 64 && DS == 1)),
                 "a wavefront takes whole 128-coordinate chunks (or a whole head of 64) and whole group pairs");
   static_assert(!PP || (D == 64 && DS == 1), "page pairs are for head_dim 64");
+  static_assert(!(PP && NR), "page pairs use both row sets");
+  static_assert(!SG || (NKW >= 3 && !PP), "staged loads take 12 or 16 key bytes per lane");
+  constexpr int STAGE_BYTES = stage_bytes(VW);
+  constexpr int NRS = NR ? 1 : 2;             // fp6 operands (row sets) per plane word
+  constexpr int NJ = NR ? 1 : 2;              // heads a lane sees in the score MFMA's output
   // Hkv counts query-head groups: a KV head with more than 8 query heads is served by kv_div groups
   // of G <= 8 heads each (consecutive groups read the same pages)
   const int G = Hq / Hkv;
@@ -222,12 +259,18 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   const int n = lane & 15, kb = lane >> 4;    // score stage: token / coordinate quarter; value stage: row / page
 
   extern __shared__ __align__(16) unsigned char smem_raw[];
-  float* s_p = (float*)smem_raw + wave * WAVE_LDS_FLOATS;   // [4 pages][16 rows][P_STRIDE]
-  float* s_alpha = s_p + 4 * 16 * P_STRIDE;                 // [16]
+  float* s_p = (float*)smem_raw + wave * WAVE_LDS_FLOATS;   // [4 pages][8 heads][P_STRIDE]
+  float* s_alpha = s_p + 4 * 8 * P_STRIDE;                 // [16]
   float* s_scale = s_alpha + 16;                            // [4 pages][NG][16 tokens] fp32, pre-scaled
   float* s_x = s_scale + 4 * NG * 16;                       // DS > 1: [parity][8][64] this wavefront's score halves
-  float* s_x_peer = (float*)smem_raw + (wave ^ 1) * WAVE_LDS_FLOATS + (4 * 16 * P_STRIDE + 16 + 4 * NG * 16);
+  float* s_x_peer = (float*)smem_raw + (wave ^ 1) * WAVE_LDS_FLOATS + (4 * 8 * P_STRIDE + 16 + 4 * NG * 16);
   float* s_red = (float*)smem_raw;                          // after the loop: [NGRP][G][D + 2]
+  // SG: this wavefront's staging area behind the wavefronts' private regions
+  unsigned char* stage = smem_raw + MF_WAVES * WAVE_LDS_FLOATS * sizeof(float) + wave * STAGE_BYTES;
+  unsigned char* stage_m = stage + 4 * 1024;
+  unsigned char* stage_v = stage_m + 512;
+  unsigned char* stage_z = stage_v + (VW / 4) * 1024;
+  unsigned char* stage_s = stage_z + 2 * 1024;
 
   // ---------------------------------------------------------------- query preparation inside this launch
   // fz.q != nullptr: nobody has prepared the query operands; the workgroups that share a group of query
@@ -276,18 +319,20 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   // fp6 query terms in register order (see the preparation kernel): row set 0 = terms 0, 1 of the 8
   // heads (row 2g + t), row set 1 = terms 2, 3; rows of absent heads are zero.  Six dwords per
   // lane are stored at a stride of eight.
-  i32x8 qa[NTP][WPL][2];
+  i32x8 qa[NTP][WPL][NRS];
   {
     // PP: rows 8..15 / coordinates 64..127 repeat rows 0..7 / coordinates 0..63; the off-diagonal blocks are zero
-    const int slane = PP ? (n & 7) + 16 * (kb & 1) : lane;
+    // NR: row 4g + t is row 2g + t % 2 of row set t / 2
+    const int slane = PP ? (n & 7) + 16 * (kb & 1) : (NR ? 2 * (n >> 2) + (n & 1) + 16 * kb : lane);
     const bool a_live = !PP || ((n < 8) == (kb < 2));
-    const uint32_t* src = qa_pack + (((int64_t)b * Hkv + h) * (NTP * WPLT * 2 * 64) + slane) * 8;
+    const uint32_t* src = qa_pack + (((int64_t)b * Hkv + h) * (NTP * WPLT * 2 * 64) + slane) * 8 +
+                          (NR ? ((n >> 1) & 1) * (64 * 8) : 0);
 #pragma unroll
     for (int tp = 0; tp < NTP; ++tp)
 #pragma unroll
       for (int i = 0; i < WPL; ++i)
 #pragma unroll
-        for (int rs = 0; rs < 2; ++rs) {
+        for (int rs = 0; rs < NRS; ++rs) {
           const uint32_t* p6 = src + ((tp * WPLT + hf * WPL + i) * 2 + rs) * (64 * 8);
           if (fused_build && fz.q != nullptr) {       // written by other workgroups of this launch: device-coherent loads
             const unsigned long long* p64 = (const unsigned long long*)p6;
@@ -307,13 +352,17 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   // 2^(E - 2 - 5t); the fp4 bit value 0.5 carries 2^1.
   int sa;
   {
-    const int g = PP ? (n & 7) >> 1 : n >> 1;
+    const int g = PP ? (n & 7) >> 1 : (NR ? n >> 2 : n >> 1);
     const int64_t qrow = (int64_t)b * Hq + h * G + (g < G ? g : 0);
     const bool coh = fused_build && fz.q != nullptr;
     const int e1 = 127 + (int)(coh ? load_coherent(q_stat + qrow * 4 + 0) : q_stat[qrow * 4 + 0]);
     const int e2 = 127 + (int)(coh ? load_coherent(q_stat + qrow * 4 + 1) : q_stat[qrow * 4 + 1]);
     const int t01 = (n & 1) ? 7 : 2, t23 = t01 + 10;
     sa = (e1 - t01) | ((e1 - t23) << 8) | ((e2 - t01) << 16) | ((e2 - t23) << 24);
+    if (NR) {                                    // one row set: byte 0 index planes, byte 2 sign plane
+      const int tn = 2 + 5 * (n & 3);
+      sa = (e1 - tn) | ((e2 - tn) << 16);
+    }
   }
   const int sb = 127 + 1;
   // head_dim 64: the score MFMA still contracts 128 coordinates; the lanes of the upper two coordinate
@@ -327,8 +376,8 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   int xplanes[NX > 0 ? NX : 1];                 // which stored planes each extra term XORs
   {
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int g = PP ? 2 * (kb & 1) + j : 2 * kb + j;
+    for (int j = 0; j < NJ; ++j) {
+      const int g = PP ? 2 * (kb & 1) + j : (NR ? kb : 2 * kb + j);
       const bool live = g < G && hf == 0;
       const int64_t qrow = (int64_t)b * Hq + h * G + (g < G ? g : 0);
       const bool coh = fused_build && fz.q != nullptr;
@@ -348,10 +397,10 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
     }
   }
 
-  if (PP) {
-    // rows of heads 4..7 are never written with page pairs; the value stage reads them as operand rows
+  if (PP || NR) {
+    // rows of heads 4..7 are never written with at most four heads; the value stage reads them as operand rows
     // whose results nobody uses: keep them finite
-    for (int i = lane; i < 4 * 16 * P_STRIDE + 16; i += 64) s_p[i] = 0.0f;
+    for (int i = lane; i < 4 * 8 * P_STRIDE + 16; i += 64) s_p[i] = 0.0f;
   }
   // ---------------------------------------------------------------- work range (all scalar)
   // len_sub: newest tokens that are attended to exactly.  A length beyond the block table is cut to the table.
@@ -382,7 +431,9 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   // is small on purpose: a token that dominates its row should sit at (or near) the reference, where
   // its weight 1.0 survives the bf16 rounding of the value-stage operands exactly.
   constexpr float REF_SLACK = 4.0f;
-  float m_run[2] = {MF_NEG, MF_NEG}, l_run[2] = {0.0f, 0.0f};
+  float m_run[NJ], l_run[NJ];
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) { m_run[j] = MF_NEG; l_run[j] = 0.0f; }
 
   struct KeyRegs { uint32_t key[NPG][NKW]; f32x2 meta[NPG]; };
   struct ValRegs { uint32_t v[VW]; u32x4 zero[2]; u32x4 scale; };
@@ -456,6 +507,69 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
     R.scale = *(const u32x4*)(pool_h + (uint64_t)spid * page_stride32 + off_scale);
   };
 
+  // SG: requests for a block's page data (fixed numbers of instructions: the waits below count them) and the
+  // copies LDS -> registers
+  constexpr int K_OPS = 5, V_OPS = VW / 4 + 3;
+  auto dma_keys = [&](const int (&pid)[4]) {
+    const uint32_t ok = in_vgpr(off_keys);
+    const uint32_t m0k = (uint32_t)(uintptr_t)stage;
+#pragma unroll
+    for (int pg = 0; pg < 4; ++pg)
+      dma_so<NKW * 4>(ok, pool_h + (uint64_t)(uint32_t)pid[pg] * page_stride32, m0k + pg * 1024);
+    // norms: lane l < 32 takes the (norm, residual norm) pairs of tokens 2 (l % 8), 2 (l % 8) + 1 of page l / 8
+    const uint32_t p0 = in_vgpr((uint32_t)pid[0]), p1 = in_vgpr((uint32_t)pid[1]), p2 = in_vgpr((uint32_t)pid[2]),
+                   p3 = in_vgpr((uint32_t)pid[3]);
+    const int mp = (lane >> 3) & 3;
+    const uint32_t mpid = mp == 0 ? p0 : (mp == 1 ? p1 : (mp == 2 ? p2 : p3));
+    const uint8_t* ma = pool_h + (uint64_t)mpid * page_stride32 + (L.off_meta + (lane & 7) * 16);
+    if (lane < 32) dma16<0>(ma, (uint32_t)(uintptr_t)stage_m);
+  };
+  auto fetch_keys = [&](KeyRegs& R) {
+#pragma unroll
+    for (int pg = 0; pg < 4; ++pg) {
+      const uint32_t* kp = (const uint32_t*)(stage + pg * 1024 + lane * 16);
+      if (NKW == 4) {
+        const u32x4 t = *(const u32x4*)kp;
+#pragma unroll
+        for (int w = 0; w < NKW; ++w) R.key[pg][w] = t[w];
+      } else {
+#pragma unroll
+        for (int w = 0; w < NKW; ++w) R.key[pg][w] = kp[w];
+      }
+      R.meta[pg] = *(const f32x2*)(stage_m + (pg * 16 + n) * 8);
+    }
+  };
+  auto dma_vals = [&](const int (&pid)[4]) {
+    const uint32_t p0 = in_vgpr((uint32_t)pid[0]), p1 = in_vgpr((uint32_t)pid[1]), p2 = in_vgpr((uint32_t)pid[2]),
+                   p3 = in_vgpr((uint32_t)pid[3]);
+    const uint32_t my_pid = kb == 0 ? p0 : (kb == 1 ? p1 : (kb == 2 ? p2 : p3));
+    const uint8_t* vbase = pool_h + (uint64_t)my_pid * page_stride32;
+    const uint32_t m0v = (uint32_t)(uintptr_t)stage_v, m0z = (uint32_t)(uintptr_t)stage_z;
+    // (the instruction offset moves the LDS address as well as the memory address)
+    static_assert(!SG || VW == 8 || VW == 16, "two or four pieces of value words");
+    dma16<0>(vbase + off_v, m0v);
+    dma16<16>(vbase + off_v, m0v + 1 * (1024 - 16));
+    if (VW == 16) {
+      dma16<32>(vbase + off_v, m0v + 2 * (1024 - 16));
+      dma16<48>(vbase + off_v, m0v + 3 * (1024 - 16));
+    }
+    dma16<0>(vbase + off_zero_c, m0z);
+    dma16<16>(vbase + off_zero_c, m0z + (1024 - 16));
+    const uint32_t spid = spg == 0 ? p0 : (spg == 1 ? p1 : (spg == 2 ? p2 : p3));
+    dma16<0>(pool_h + (uint64_t)spid * page_stride32 + off_scale, (uint32_t)(uintptr_t)stage_s);
+  };
+  auto fetch_vals = [&](ValRegs& R) {
+#pragma unroll
+    for (int j = 0; j < VW / 4; ++j) {
+      const u32x4 t = *(const u32x4*)(stage_v + (j * 64 + lane) * 16);
+#pragma unroll
+      for (int w = 0; w < 4; ++w) R.v[4 * j + w] = t[w];
+    }
+    R.zero[0] = *(const u32x4*)(stage_z + lane * 16);
+    R.zero[1] = *(const u32x4*)(stage_z + (64 + lane) * 16);
+    R.scale = *(const u32x4*)(stage_s + lane * 16);
+  };
+
   // A value code masked in place is a bf16 number: a pattern n < 256 in a 16-bit half is n * 2^-133
   // exactly (denormals, and the first binade continues them linearly), so B = code * 2^(s - 133)
   // where s is the bit position the code has inside its byte; the softmax weight carries 2^(80 - s).
@@ -472,10 +586,10 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   bool fresh = true;                            // this walker has not seen a token yet: no reference
   auto score_stage = [&](int blk, int it, bool first, const KeyRegs& K, int bad, auto partial_tag) -> bool {
     constexpr bool PARTIAL = decltype(partial_tag)::value;
-    float s2[2][NPG];
-    float mref[2];                              // only one wavefront of a pair subtracts it
+    float s2[NJ][NPG];
+    float mref[NJ];                             // only one wavefront of a pair subtracts it
 #pragma unroll
-    for (int j = 0; j < 2; ++j) mref[j] = (first || hf != 0) ? 0.0f : m_run[j];
+    for (int j = 0; j < NJ; ++j) mref[j] = (first || hf != 0) ? 0.0f : m_run[j];
     // The MFMA-dense parts run at raised wavefront priority (the value stage above the score
     // stage): the SIMD's other wavefront then fills the gaps with its vector-ALU work instead of
     // both alternating between the two kinds of instruction.
@@ -498,18 +612,21 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
           const uint32_t b0 = x & nib, b1 = x & nib1, b2 = x & nib2, b3 = (x >> 3) & nib;
           if (tp == NTP - 1) {
             dq = mfma_f8f4<2>(qa[tp][i][0], b0, b1, b2, b3, dq, sa, sb);
-            dq = mfma_f8f4<3>(qa[tp][i][1], b0, b1, b2, b3, dq, sa, sb);
+            if (!NR) dq = mfma_f8f4<3>(qa[tp][i][NRS - 1], b0, b1, b2, b3, dq, sa, sb);
           } else {
             dm = mfma_f8f4<0>(qa[tp][i][0], b0, b1, b2, b3, dm, sa, sb);
-            dm = mfma_f8f4<1>(qa[tp][i][1], b0, b1, b2, b3, dm, sa, sb);
+            if (!NR) dm = mfma_f8f4<1>(qa[tp][i][NRS - 1], b0, b1, b2, b3, dm, sa, sb);
           }
         }
       }
       const float nk = K.meta[pg][0], rk = K.meta[pg][1];
+      // this wavefront's share of the score (the whole score when DS == 1), relative to the reference
+      if (NR) {
+        s2[0][pg] = fmaf(nk, (dm[0] + dm[1]) + (dm[2] + dm[3]), fmaf(rk, (dq[0] + dq[1]) + (dq[2] + dq[3]), -mref[0]));
+      } else {
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        // this wavefront's share of the score (the whole score when DS == 1), relative to the reference
-        s2[j][pg] = fmaf(nk, dm[2 * j] + dm[2 * j + 1], fmaf(rk, dq[2 * j] + dq[2 * j + 1], -mref[j]));
+        for (int j = 0; j < NJ; ++j)
+          s2[j][pg] = fmaf(nk, dm[2 * j] + dm[2 * j + 1], fmaf(rk, dq[2 * j] + dq[2 * j + 1], -mref[j]));
       }
     }
     // Wanted issue order of the section above: the bit expansion of the first page, then every MFMA
@@ -517,7 +634,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
     // arithmetic), which run in the shadow of the matrix pipe.
     __builtin_amdgcn_sched_group_barrier(0x002, 5 * NTP * WPL, 0);
 #pragma unroll
-    for (int k = 0; k < NPG * 2 * NTP * WPL; ++k) {
+    for (int k = 0; k < NPG * NRS * NTP * WPL; ++k) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
     }
@@ -528,12 +645,12 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
       float* mine = s_x + (it & 1) * (8 * 64);
       const float* theirs = s_x_peer + (it & 1) * (8 * 64);
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
+      for (int j = 0; j < NJ; ++j)
 #pragma unroll
         for (int pg = 0; pg < 4; ++pg) mine[(j * 4 + pg) * 64 + lane] = s2[j][pg];
       __syncthreads();
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
+      for (int j = 0; j < NJ; ++j)
 #pragma unroll
         for (int pg = 0; pg < 4; ++pg) s2[j][pg] += theirs[(j * 4 + pg) * 64 + lane];
     }
@@ -547,23 +664,23 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
         gone[pg] = n >= tokens_of_page(blk, PP ? 2 * pg + (kb >> 1) : pg, bad);
         any |= !gone[pg];
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < NJ; ++j)
           if (gone[pg]) s2[j][pg] = MF_NEG;
       }
       // a block without a single token leaves the walker as it was (the next block is still its first)
       fresh = fresh && __builtin_amdgcn_ballot_w64(any) == 0;
     }
     // ---- online softmax (log2 domain) against a lazily updated reference
-    float mx = fmaxf(s2[0][0], s2[1][0]);
+    float mx = fmaxf(s2[0][0], s2[NJ - 1][0]);
 #pragma unroll
-    for (int pg = 1; pg < NPG; ++pg) mx = fmaxf(mx, fmaxf(s2[0][pg], s2[1][pg]));
+    for (int pg = 1; pg < NPG; ++pg) mx = fmaxf(mx, fmaxf(s2[0][pg], s2[NJ - 1][pg]));
     const bool rescale = first || __builtin_amdgcn_ballot_w64(mx > REF_SLACK) != 0;
     if (rescale) {
       // move the reference to the row maximum (never down, except for the first block, where the
       // accumulators are still empty and keep their scale); every lane of a row computes the same
-      float alpha[2];
+      float alpha[NJ];
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
+      for (int j = 0; j < NJ; ++j) {
         float mj = s2[j][0];
 #pragma unroll
         for (int pg = 1; pg < NPG; ++pg) mj = fmaxf(mj, s2[j][pg]);
@@ -576,10 +693,15 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
 #pragma unroll
         for (int pg = 0; pg < NPG; ++pg) s2[j][pg] -= delta;
       }
-      if (n == 0 && (!PP || kb < 2)) { s_alpha[2 * kb] = alpha[0]; s_alpha[2 * kb + 1] = alpha[1]; }
+      if (NR) {
+        if (n == 0) s_alpha[kb] = alpha[0];
+      } else if (n == 0 && (!PP || kb < 2)) {
+        s_alpha[2 * kb] = alpha[0];
+        s_alpha[2 * kb + 1] = alpha[NJ - 1];
+      }
     }
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < NJ; ++j) {
       float psum = 0.0f;
 #pragma unroll
       for (int pg = 0; pg < NPG; ++pg) {
@@ -587,8 +709,9 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
         // reference therefore sits at the masking value itself)
         const float p = PARTIAL && gone[pg] ? 0.0f : __builtin_amdgcn_exp2f(s2[j][pg]);
         psum += p;
-        if (PP) s_p[((2 * pg + (kb >> 1)) * 16 + 2 * (kb & 1) + j) * P_STRIDE + n] = p;
-        else s_p[(pg * 16 + 2 * kb + j) * P_STRIDE + n] = p;
+        if (PP) s_p[((2 * pg + (kb >> 1)) * 8 + 2 * (kb & 1) + j) * P_STRIDE + n] = p;
+        else if (NR) s_p[(pg * 8 + kb) * P_STRIDE + n] = p;
+        else s_p[(pg * 8 + 2 * kb + j) * P_STRIDE + n] = p;
       }
       l_run[j] += psum;
     }
@@ -634,7 +757,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
     // ---- value stage: lane = (row n = head n % 8 with the scales of group parity n / 8, page kb)
     float pr[16];
     {
-      const f32x4* pp = (const f32x4*)(s_p + (kb * 16 + (n & 7)) * P_STRIDE);
+      const f32x4* pp = (const f32x4*)(s_p + (kb * 8 + (n & 7)) * P_STRIDE);
 #pragma unroll
       for (int q4 = 0; q4 < 4; ++q4) {
         f32x4 t = pp[q4];
@@ -719,8 +842,13 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
     int bad = 0;                                          // pages of the current block that lie outside the pool
     if (blk < blk_end) {
       bad = page_ids(blk, pid, std::true_type{});
-      load_keys(pid, K);
-      load_vals(pid, V);
+      if constexpr (SG) {
+        dma_keys(pid);
+        dma_vals(pid);
+      } else {
+        load_keys(pid, K);
+        load_vals(pid, V);
+      }
     }
     // Block tables are device data nobody has checked: every wavefront looks once at the table entries of its
     // workgroup's blocks, a lane per entry: up to 256 entries in straight-line code (all loads unconditional
@@ -751,10 +879,25 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
         const int nxt_c = nxt < blk_end ? nxt : blk;
         int pid_n[4];
         const int bad_n = page_ids(nxt_c, pid_n, checked_tag);   // scalar loads, consumed after the score stage
-        const bool rescale = score_stage(blk, it, CHECKED ? fresh : it == 0, K, bad, partial_tag);
-        load_keys(pid_n, K);
-        value_stage(blk, V, rescale, bad, partial_tag);
-        load_vals(pid_n, V);
+        if constexpr (SG) {
+          // outstanding, oldest first: this block's keys, this block's values
+          stage_wait<V_OPS>();
+          fetch_keys(K);
+          stage_release();
+          dma_keys(pid_n);
+          const bool rescale = score_stage(blk, it, CHECKED ? fresh : it == 0, K, bad, partial_tag);
+          // outstanding: this block's values, the next block's keys
+          stage_wait<K_OPS>();
+          fetch_vals(V);
+          stage_release();
+          dma_vals(pid_n);
+          value_stage(blk, V, rescale, bad, partial_tag);
+        } else {
+          const bool rescale = score_stage(blk, it, CHECKED ? fresh : it == 0, K, bad, partial_tag);
+          load_keys(pid_n, K);
+          value_stage(blk, V, rescale, bad, partial_tag);
+          load_vals(pid_n, V);
+        }
         blk = nxt;
         bad = bad_n;
       };
@@ -777,16 +920,17 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   }
 
   // ---------------------------------------------------------------- merge the walkers, write the partial
+  if (SG) stage_wait<0>();   // the last trip's requests (a repeat of its own block) have landed
   __syncthreads();      // every wave is done with its private LDS region
   float* s_z = s_red + NGRP * G * (D + 2);                     // [MF_WAVES][16 rows][16 groups]
 #pragma unroll
   for (int i = 0; i < 4; ++i) s_z[(wave * 16 + 4 * kb + i) * 16 + n] = zacc[i];
   if (hf == 0) {                                               // the wavefronts of a pair hold the same (m, l)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < NJ; ++j) {
       float lsum = row_sum16(l_run[j]);
       if (PP) lsum = sum_xor32(lsum);
-      const int g = PP ? 2 * (kb & 1) + j : 2 * kb + j;
+      const int g = PP ? 2 * (kb & 1) + j : (NR ? kb : 2 * kb + j);
       if (n == 0 && g < G && (!PP || kb < 2)) {
         float* r = s_red + (wgrp * G + g) * (D + 2);
         r[0] = m_run[j] * 0.6931471805599453f;     // back to the natural-log domain of the partials
@@ -913,7 +1057,7 @@ bool take_time_hook(int which, hipEvent_t& start, hipEvent_t& stop) {
   return start != nullptr || stop != nullptr;
 }
 
-template <int D, int MB, int NX, int VB, int GS, int DS, int WPS, bool F16P, bool PP = false>
+template <int D, int MB, int NX, int VB, int GS, int DS, int WPS, bool F16P, bool PP = false, bool NR = false, bool SG = false>
 static int launch_one(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, int kv_div,
                       const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
                       float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts, int n_split,
@@ -921,6 +1065,7 @@ static int launch_one(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, 
   const int G = Hq / Hkv;
   size_t per_wave = (size_t)wave_lds_floats(D / DS / GS, DS) * sizeof(float);
   size_t merge = (size_t)(MF_WAVES / DS * G * (D + 2) + MF_WAVES * 16 * 16) * sizeof(float);
+  if (SG) per_wave += stage_bytes((D / DS / 16) * VB / 2);
   size_t smem = per_wave * MF_WAVES > merge ? per_wave * MF_WAVES : merge;
   if (fz.q) {
     const size_t prep = (size_t)prep_unit_smem_floats(fz.hp, D) * sizeof(float);
@@ -930,7 +1075,17 @@ static int launch_one(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, 
     return launch_one<D, MB, NX, VB, GS, DS, WPS, F16P, D == 64>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,
                                                                  bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts,
                                                                  n_split, len_sub, max_pages, num_pages, fz, fm, st);
-  auto kern = decode_mfma_kernel<D, MB, NX, VB, GS, DS, WPS, F16P, PP>;
+  if (D >= 128 && !NR && G <= 4 && opt_narrow_rows.load(std::memory_order_relaxed) != 0)
+    return launch_one<D, MB, NX, VB, GS, DS, WPS, F16P, false, D >= 128>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,
+                                                                         bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts,
+                                                                         n_split, len_sub, max_pages, num_pages, fz, fm, st);
+  // (measured: the staged variant only pays where the register-held variant spills, i.e. with three index planes)
+  constexpr bool can_stage = D >= 128 && MB == 3;
+  if (can_stage && !SG && opt_lds_stage.load(std::memory_order_relaxed) != 0)
+    return launch_one<D, MB, NX, VB, GS, DS, WPS, F16P, PP, NR, can_stage>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,
+                                                                           bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts,
+                                                                           n_split, len_sub, max_pages, num_pages, fz, fm, st);
+  auto kern = decode_mfma_kernel<D, MB, NX, VB, GS, DS, WPS, F16P, PP, NR, SG>;
   if (smem > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return (int)e;
