@@ -325,6 +325,27 @@ __device__ __forceinline__ float round_hw(float v) {
   }
 }
 
+// out[i] = in[i] - sub rounded to the input dtype, i < 8; bf16 rounds two numbers per conversion instruction
+template <int DT>
+__device__ __forceinline__ void round_pairs(const float (&in)[8], float sub, float (&out)[8]) {
+  if constexpr (DT == TQ_BF16) {
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const f32x2_t f = {in[2 * i] - sub, in[2 * i + 1] - sub};
+      const bf16x2_t r = __builtin_convertvector(f, bf16x2_t);
+      uint32_t u;
+      __builtin_memcpy(&u, &r, 4);
+      out[2 * i] = __uint_as_float(u << 16);
+      out[2 * i + 1] = __uint_as_float(u & 0xffff0000u);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) out[i] = round_hw<DT>(in[i] - sub);
+  }
+}
+
 // Faster value kernel for 16-bit inputs, 2/4-bit codes and head_dim 64 / 128 / 256: a thread owns 8
 // consecutive channels of one token (one 16-byte load), a group's minimum / maximum meet through
 // cross-lane exchanges, and the codes pass through LDS only to be transposed into the page's
@@ -385,12 +406,21 @@ value_chunk_kernel(const void* __restrict__ v, Source src, int d, int gs, Sink s
     }
   }
   float lo = x[0], hi = x[0];
-  int has_nan = 0;
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    has_nan |= (x[i] != x[i]);
+  for (int i = 1; i < 8; ++i) {
     lo = fminf(lo, x[i]);
     hi = fmaxf(hi, x[i]);
+  }
+  // a NaN among the 8 inputs, on the packed 16-bit patterns: magnitude bits above those of infinity
+  int has_nan;
+  {
+    typedef uint16_t u16x2_t __attribute__((ext_vector_type(2)));
+    u16x2_t m = __builtin_bit_cast(u16x2_t, raw.x & 0x7fff7fffu);
+    m = __builtin_elementwise_max(m, __builtin_bit_cast(u16x2_t, raw.y & 0x7fff7fffu));
+    m = __builtin_elementwise_max(m, __builtin_bit_cast(u16x2_t, raw.z & 0x7fff7fffu));
+    m = __builtin_elementwise_max(m, __builtin_bit_cast(u16x2_t, raw.w & 0x7fff7fffu));
+    constexpr uint16_t inf_bits = DT == TQ_BF16 ? 0x7f80 : 0x7c00;
+    has_nan = (m[0] > inf_bits) | (m[1] > inf_bits);
   }
   // the threads of a group are neighbouring lanes inside a row of 16: DPP moves (quad swaps, then half-row and
   // row mirrors, which pair quads that already agree) instead of shuffles through the LDS
@@ -406,38 +436,46 @@ value_chunk_kernel(const void* __restrict__ v, Source src, int d, int gs, Sink s
   if (tpg >= 16) reduce_step(std::integral_constant<int, 0x140>{});
   if (has_nan) lo = hi = __uint_as_float(0x7fc00000u);       // torch min/max propagate NaN
   const float levels = (float)((1 << VB) - 1);
-  float sc = round_hw<DT>(round_hw<DT>(hi - lo) / levels);
+  // (hi - lo) / levels as a product: both are numbers of at most 8 significant bits, so is the divisor of every
+  // quotient below, and such a quotient is never a rounding tie of the 16-bit format and at least 2^-17
+  // (relative) away from one: a product with a reciprocal good to an ulp rounds like the division (checked
+  // over all pairs of significands and the three nearest reciprocals).  fp16 keeps the division.
+  const float range = round_hw<DT>(hi - lo);
+  float sc = round_hw<DT>(DT == TQ_BF16 ? range * (1.0f / levels) : range / levels);
   const float floor_v = round_hw<DT>(1e-10f);
   sc = (sc != sc) ? sc : fmaxf(sc, floor_v);
   const float z = lo;
-  // Quotients of bf16 numbers, rounded to bf16: a / s with 8-bit significands is either exactly a bf16
-  // rounding tie (a 9-bit quotient) or at least 2^-17 (relative) away from one, so any fp32 quotient good
-  // to an ulp rounds like the correctly rounded one, as long as ties come out exact.  q0 = a * (1/s)
-  // followed by one residual correction q0 + (a - q0 s)(1/s) does both (the fused residual is exact for
-  // a tie).  Used when the scale is an ordinary number; everything else takes the division.
+  // Quotients of bf16 numbers, rounded to bf16: a * (1/s) with any reciprocal good to an ulp (see above).
+  // Used when the scale is an ordinary number; everything else takes the division.
   const bool fast_div = DT == TQ_BF16 && sc > 0x1p-60f && sc < 0x1p60f;
-  const float rsc = __builtin_amdgcn_rcpf(sc);     // any reciprocal good to an ulp will do (checked over all bf16 pairs)
-  uint32_t codes = 0;                              // 8 codes, VB bits each, channel order
+  const float rsc = __builtin_amdgcn_rcpf(sc);
   float quo[8];
   if (fast_div) {                // every a of the group is finite and at most (levels + 1) * sc < 2^64 then
+    float a[8];
+    round_pairs<DT>(x, z, a);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const float a = round_hw<DT>(x[i] - z);
-      const float q0 = a * rsc;
-      quo[i] = fmaf(fmaf(-q0, sc, a), rsc, q0);
-    }
+    for (int i = 0; i < 8; ++i) quo[i] = a[i] * rsc;
   } else {
 #pragma unroll
     for (int i = 0; i < 8; ++i) quo[i] = round_hw<DT>(x[i] - z) / sc;
   }
+  // 8 codes, VB bits each, channel order.  The codes are small integers held in floats: 16 bits' worth of
+  // them are put together with exact multiply-adds and converted once.
+  float qr[8];
+  round_pairs<DT>(quo, 0.0f, qr);
+  uint32_t codes = 0;
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    float q = round_hw<DT>(quo[i]);
-    q = rintf(q);
-    // clamp to [0, levels]; a NaN becomes code 0 (the median-of-three instruction returns the minimum of
-    // its operands when one of them is a NaN)
-    q = __builtin_amdgcn_fmed3f(q, 0.0f, levels);
-    codes |= (uint32_t)q << (VB * i);
+  for (int hw = 0; hw < (VB == 2 ? 1 : 2); ++hw) {
+    constexpr int PER = 16 / VB;                   // codes per 16 bits
+    float acc = 0.0f;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      // clamp to [0, levels]; a NaN becomes code 0 (the median-of-three instruction returns the minimum of
+      // its operands when one of them is a NaN)
+      const float q = __builtin_amdgcn_fmed3f(rintf(qr[hw * PER + i]), 0.0f, levels);
+      acc = fmaf(q, (float)(1 << (VB * i)), acc);
+    }
+    codes |= (uint32_t)acc << (16 * hw);
   }
   if constexpr (!std::is_same<Sink, ValFlatSink>::value) *(CodeWord*)(scode + ck * CROW + t * sizeof(CodeWord)) = (CodeWord)codes;
   const int ng = d / gs, g = (ck * 8) / gs;
