@@ -319,3 +319,23 @@ def test_fp6_digits_of_the_rotation_decode_back_to_it():
     ref = m.double().numpy()
     blockmax = np.abs(ref).reshape(d, d // 32, 32).max(-1).repeat(32, axis=1)
     assert np.all(np.abs(rec - ref) <= 2.0 ** -22 * 2.0 * blockmax)
+
+
+def test_quotient_of_bf16_numbers_rounds_like_its_product_with_a_reciprocal():
+    """The value quantiser (kv_cache.py:53-99 divides bf16 numbers and rounds to bf16) replaces a / s by
+    a * r, r an fp32 reciprocal of s good to one ulp.  Both operands have at most 8 significant bits, so the
+    quotient is never a rounding tie of bf16 and never closer than 2^-17 (relative) to one, far more than the
+    product's error: the two round to the same bf16 number.  Exhaustive over all pairs of significands, the
+    exponent offsets the quantiser can meet, and the three reciprocals nearest to 1 / s."""
+    def bf16_bits(f):
+        u = f.view(np.uint32).astype(np.uint64)
+        return ((u + 0x7fff + ((u >> 16) & 1)) >> 16).astype(np.uint32)
+    ms = np.arange(128, 256, dtype=np.float32)[:, None, None]
+    ma = np.arange(128, 256, dtype=np.float32)[None, :, None]
+    a = ma * np.exp2(np.arange(-30, 9, dtype=np.float32))[None, None, :]
+    ref = bf16_bits((a / ms).astype(np.float32))
+    r0 = (np.float32(1.0) / ms).astype(np.float32)
+    for step in (-1, 0, 1):
+        r = (r0.view(np.int32) + step).view(np.float32)
+        got = bf16_bits((a * r).astype(np.float32))
+        assert np.array_equal(got, np.broadcast_to(ref, got.shape)), step
