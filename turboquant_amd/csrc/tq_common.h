@@ -91,6 +91,43 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
+// The same reductions with DPP row operations and four lane reads instead of shared-memory permutes (no LDS
+// round trip per step).  The sum adds in a different order than wave_sum.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+// sum / maximum over groups of 4, 8 or 16 neighbouring lanes (quad swaps, half-row mirror, row mirror); every
+// lane of a group ends with the group's result
+template <int N>
+__device__ __forceinline__ float lanes_sum_dpp(float v) {
+  static_assert(N == 4 || N == 8 || N == 16, "4, 8 or 16 lanes");
+  v += dpp_f32<0xB1>(v);
+  v += dpp_f32<0x4E>(v);
+  if (N >= 8) v += dpp_f32<0x141>(v);
+  if (N >= 16) v += dpp_f32<0x140>(v);
+  return v;
+}
+template <int N>
+__device__ __forceinline__ float lanes_max_dpp(float v) {
+  static_assert(N == 4 || N == 8 || N == 16, "4, 8 or 16 lanes");
+  v = fmaxf(v, dpp_f32<0xB1>(v));
+  v = fmaxf(v, dpp_f32<0x4E>(v));
+  if (N >= 8) v = fmaxf(v, dpp_f32<0x141>(v));
+  if (N >= 16) v = fmaxf(v, dpp_f32<0x140>(v));
+  return v;
+}
+__device__ __forceinline__ float wave_sum_fast(float v) {
+  const int b = __builtin_bit_cast(int, lanes_sum_dpp<16>(v));
+  return (__builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 0)) + __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 16))) +
+         (__builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 32)) + __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48)));
+}
+__device__ __forceinline__ float wave_max_fast(float v) {
+  const int b = __builtin_bit_cast(int, lanes_max_dpp<16>(v));
+  return fmaxf(fmaxf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 0)), __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 16))),
+               fmaxf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 32)), __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48))));
+}
+
 // ---- index packing of the reference's flat layout (quantizer.py:38-69) --------------
 
 __host__ __device__ __forceinline__ int eff_bits(int mse_bits) { return mse_bits == 1 ? 1 : (mse_bits == 2 ? 2 : (mse_bits <= 4 ? 4 : 8)); }

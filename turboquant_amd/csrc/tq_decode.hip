@@ -168,7 +168,7 @@ decode_pages_kernel(const float* __restrict__ q_rot, const float* __restrict__ q
       float mx = NEG_BIG;
       if (g < GP)
         for (int t = j; t < GEN_CHUNK; t += 16) mx = fmaxf(mx, s_p[t * GP + g]);
-      for (int o = 8; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+      mx = lanes_max_dpp<16>(mx);
       if (j == 0) s_m[g] = mx;
     }
     __syncthreads();
@@ -362,13 +362,10 @@ exact_tail_kernel(const void* __restrict__ q, int Hq, int Hkv, int d, const void
         a2 = fmaf(kx, q4.z, a2);
         a3 = fmaf(kx, q4.w, a3);
       }
-#pragma unroll
-      for (int o = 4; o > 0; o >>= 1) {
-        a0 += __shfl_xor(a0, o, 64);
-        a1 += __shfl_xor(a1, o, 64);
-        a2 += __shfl_xor(a2, o, 64);
-        a3 += __shfl_xor(a3, o, 64);
-      }
+      a0 = lanes_sum_dpp<8>(a0);
+      a1 = lanes_sum_dpp<8>(a1);
+      a2 = lanes_sum_dpp<8>(a2);
+      a3 = lanes_sum_dpp<8>(a3);
       if (seg == 0 && t < n)
         *reinterpret_cast<float4*>(ss + (c0 + t) * GC) = make_float4(a0 * sm_scale, a1 * sm_scale, a2 * sm_scale, a3 * sm_scale);
     }
@@ -378,14 +375,14 @@ exact_tail_kernel(const void* __restrict__ q, int Hq, int Hkv, int d, const void
   for (int g = wave; g < GC; g += TAIL_WAVES) {
     float mx = NEG_BIG;
     for (int t = lane; t < R; t += 64) mx = fmaxf(mx, ss[t * GC + g]);
-    mx = wave_max(mx);
+    mx = wave_max_fast(mx);
     float sum = 0.0f;
     for (int t = lane; t < R; t += 64) {
       float p = __expf(ss[t * GC + g] - mx);
       ss[t * GC + g] = p;
       sum += p;
     }
-    sum = wave_sum(sum);
+    sum = wave_sum_fast(sum);
     if (lane == 0) { sml[g * 2] = mx; sml[g * 2 + 1] = sum; }
   }
   __syncthreads();
@@ -608,13 +605,10 @@ __device__ __forceinline__ void exact_tail_words_body(const TailArgs& A, int h, 
           a3 = fmaf(x[1], qb.w, a3);
         }
       }
-#pragma unroll
-      for (int o = 4; o > 0; o >>= 1) {
-        a0 += __shfl_xor(a0, o, 64);
-        a1 += __shfl_xor(a1, o, 64);
-        a2 += __shfl_xor(a2, o, 64);
-        a3 += __shfl_xor(a3, o, 64);
-      }
+      a0 = lanes_sum_dpp<8>(a0);
+      a1 = lanes_sum_dpp<8>(a1);
+      a2 = lanes_sum_dpp<8>(a2);
+      a3 = lanes_sum_dpp<8>(a3);
       if (seg == 0 && t < n)
         *reinterpret_cast<float4*>(ss + (c0 + t) * GC) = make_float4(a0 * sm_scale, a1 * sm_scale, a2 * sm_scale, a3 * sm_scale);
     }
@@ -624,14 +618,14 @@ __device__ __forceinline__ void exact_tail_words_body(const TailArgs& A, int h, 
   for (int g = wave; g < GC; g += TAIL_WAVES) {
     float mx = NEG_BIG;
     for (int t = lane; t < R; t += 64) mx = fmaxf(mx, ss[t * GC + g]);
-    mx = wave_max(mx);
+    mx = wave_max_fast(mx);
     float sum = 0.0f;
     for (int t = lane; t < R; t += 64) {
       float p = __expf(ss[t * GC + g] - mx);
       ss[t * GC + g] = p;
       sum += p;
     }
-    sum = wave_sum(sum);
+    sum = wave_sum_fast(sum);
     if (lane == 0) { sml[g * 2] = mx; sml[g * 2 + 1] = sum; }
   }
   __syncthreads();
@@ -779,7 +773,7 @@ merge_kernel(const float* __restrict__ parts, int n_parts, int part_stride, int 
     s_l[sp] = ml[1];
     if (ml[1] > 0.0f) mm = fmaxf(mm, ml[0]);
   }
-  mm = wave_max(mm);
+  mm = wave_max_fast(mm);
   if (lane == 0) scratch[wave] = mm;
   __syncthreads();
   mm = fmaxf(fmaxf(scratch[0], scratch[1]), fmaxf(scratch[2], scratch[3]));
@@ -789,7 +783,7 @@ merge_kernel(const float* __restrict__ parts, int n_parts, int part_stride, int 
     s_w[sp] = w;
     ll += w * s_l[sp];
   }
-  ll = wave_sum(ll);
+  ll = wave_sum_fast(ll);
   if (lane == 0) scratch[4 + wave] = ll;
   __syncthreads();
   ll = scratch[4] + scratch[5] + scratch[6] + scratch[7];
