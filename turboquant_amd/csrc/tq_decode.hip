@@ -439,7 +439,8 @@ exact_tail_kernel(const void* __restrict__ q, int Hq, int Hkv, int d, const void
 // tail that fits one chunk (128 tokens at head size 256, 16-bit) costs a single memory latency.  Both
 // tiles stay in LDS in the cache's own element type and are converted where they are read.  Needs word
 // alignment: 16-bit rows whose strides are even and whose base is 4-byte aligned.
-constexpr int TAIL_TILE_WORDS = 128 * 130, TAIL_RPT = 32;     // words per tile (keys, values); rows per thread
+constexpr int TAIL_TILE_WORDS = 128 * 136, TAIL_RPT = 32;     // words per tile (keys, values); rows per thread
+constexpr int TAIL_WIDE_LOADS = 8;                            // 16-byte loads a thread has in flight per tile
 
 template <int DT> struct TailWord;
 template <> struct TailWord<TQ_F32> {
@@ -482,6 +483,7 @@ struct TailArgs {
   int max_pages, num_blocks;       // entries of a block-table row; blocks of the paged exact cache
   const int32_t* seq_lens;
   int64_t ws_blk;
+  int wide;                        // rows and strides are 16-byte aligned: four words per load
   float sm_scale;
   float* parts;
   int n_parts, part_index;
@@ -516,9 +518,15 @@ __device__ __forceinline__ void exact_tail_words_body(const TailArgs& A, int h, 
   float* sml = ss + GC * recent_rows;               // [GC][2]
   uint32_t* ktile = (uint32_t*)(sml + 2 * GC);      // [CH][W + 1] key rows of the chunk; at the end [TS][GC][d] partials
   uint32_t* vtile = ktile + TAIL_TILE_WORDS;        // [CH][W + 1] value rows
-  const int W = d / EPW, ldw = W + 1;               // words per row (a multiple of 32), odd leading dimension
+  // words per row (a multiple of 32); leading dimension: odd, or (16-byte loads) W + 8, which keeps rows
+  // 16-byte aligned and spreads the 8 tokens x 8 segments a wavefront reads in the score stage over all banks
+  const bool wide = A.wide != 0;
+  const int W = d / EPW, ldw = wide ? W + 8 : W + 1;
   const int TS = W < TAIL_THREADS ? TAIL_THREADS / W : 1;          // row slices
-  const int CH = min(TAIL_TILE_WORDS / ldw, TS * RPT);             // rows per chunk
+  const int QW = W >> 2, RP = TAIL_THREADS / QW;                   // wide: 4-word pieces per row, rows per round of loads
+  const int wq = tid % QW, wr = tid / QW;                          // wide: this thread's piece and row slot
+  const int CH = wide ? min(TAIL_TILE_WORDS / ldw, TAIL_WIDE_LOADS * RP)
+                      : min(TAIL_TILE_WORDS / ldw, TS * RPT);      // rows per chunk
   const int cw0 = W < TAIL_THREADS ? tid % W : tid, ts = W < TAIL_THREADS ? tid / W : 0;
   const bool active = ts < TS;
   const int64_t base0 = (PAGED ? 0 : b * ws_b) + h * ws_h;
@@ -558,18 +566,71 @@ __device__ __forceinline__ void exact_tail_words_body(const TailArgs& A, int h, 
       }
     }
   };
+  // the query first (it is the oldest request, so it can go to LDS while the rows are still on their way)
+  constexpr int QPT = (GC * 768 + TAIL_THREADS - 1) / TAIL_THREADS;      // query elements per thread, d <= 768
+  float qreg[QPT];
+#pragma unroll
+  for (int i = 0; i < QPT; ++i) {
+    const int o = tid + i * TAIL_THREADS;
+    qreg[i] = Elem<DT>::load(q, ((int64_t)b * Hq + h * G + g0) * d + min(o, Gc * d - 1));
+  }
+  auto deposit_query = [&]() {
+#pragma unroll
+    for (int i = 0; i < QPT; ++i) {
+      const int o = tid + i * TAIL_THREADS;
+      if (o < GC * d) {
+        const int g = o / d, c = o - g * d;
+        sq[c * GC + g] = g < Gc ? qreg[i] : 0.0f;
+      }
+    }
+  };
+  // the same with 16-byte pieces: round i takes rows wr + i RP; a round none of whose rows exists is skipped
+  // (uniformly), a row that does not exist inside a live round re-reads the chunk's first row
+  typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+  // (the row offsets first, all of them - they hold the block-table loads of a paged cache -, and once for
+  // keys and values: a table load between two row loads would have to wait for the row load before it)
+  auto row_bases4 = [&](int c0, int n, int64_t (&rb)[TAIL_WIDE_LOADS]) {
+#pragma unroll
+    for (int i = 0; i < TAIL_WIDE_LOADS; ++i) {
+      const int t = wr + i * RP;
+      rb[i] = row_base(c0 + (t < n ? t : 0)) + 4 * wq;
+    }
+  };
+  auto request4 = [&](const uint32_t* src, const int64_t (&rb)[TAIL_WIDE_LOADS], int n, u32x4_t (&reg)[TAIL_WIDE_LOADS]) {
+#pragma unroll
+    for (int i = 0; i < TAIL_WIDE_LOADS; ++i)
+      if (i * RP < n) reg[i] = *(const u32x4_t*)(src + rb[i]);
+  };
+  auto deposit4 = [&](uint32_t* tile, int n, const u32x4_t (&reg)[TAIL_WIDE_LOADS]) {
+#pragma unroll
+    for (int i = 0; i < TAIL_WIDE_LOADS; ++i) {
+      const int t = wr + i * RP;
+      if (i * RP < n && t < n) *(u32x4_t*)(tile + t * ldw + 4 * wq) = reg[i];
+    }
+  };
   const int n_first = min(CH, R);
-  if (active && n_first > 0) {
+  if (wide) {
+    if (wr < RP && n_first > 0) {
+      u32x4_t kreg[TAIL_WIDE_LOADS], vreg[TAIL_WIDE_LOADS];
+      int64_t rb[TAIL_WIDE_LOADS];
+      row_bases4(0, n_first, rb);
+      request4(rk, rb, n_first, kreg);
+      request4(rv, rb, n_first, vreg);
+      deposit_query();
+      deposit4(ktile, n_first, kreg);
+      deposit4(vtile, n_first, vreg);
+    } else {
+      deposit_query();
+    }
+  } else if (active && n_first > 0) {
     uint32_t kreg[KC][RPT], vreg[KC][RPT];
     request(rk, 0, n_first, kreg);
     request(rv, 0, n_first, vreg);
+    deposit_query();
     deposit(ktile, n_first, kreg);
     deposit(vtile, n_first, vreg);
-  }
-  for (int o = tid; o < GC * d; o += TAIL_THREADS) {
-    const int g = o / d, c = o - g * d;
-    const float x = Elem<DT>::load(q, ((int64_t)b * Hq + h * G + g0) * d + min(o, Gc * d - 1));
-    sq[c * GC + g] = g < Gc ? x : 0.0f;
+  } else {
+    deposit_query();
   }
   __syncthreads();
   // scores: eight threads per token, each over every eighth word of the row, for the group's heads at once
@@ -577,40 +638,53 @@ __device__ __forceinline__ void exact_tail_words_body(const TailArgs& A, int h, 
     const int n = min(CH, R - c0);
     if (c0 > 0) {
       __syncthreads();
-      if (active) {
+      if (wide) {
+        if (wr < RP) {
+          u32x4_t kreg[TAIL_WIDE_LOADS];
+          int64_t rb[TAIL_WIDE_LOADS];
+          row_bases4(c0, n, rb);
+          request4(rk, rb, n, kreg);
+          deposit4(ktile, n, kreg);
+        }
+      } else if (active) {
         uint32_t kreg[KC][RPT];
         request(rk, c0, n, kreg);
         deposit(ktile, n, kreg);
       }
       __syncthreads();
     }
+    // (a thread takes two tokens per trip, 64 apart, against one read of the query values)
     const int seg = tid & 7;
-    for (int t0 = 0; t0 < n; t0 += TAIL_THREADS / 8) {              // uniform trip count: the shuffles need every lane
-      const int t = t0 + (tid >> 3);
-      const uint32_t* row = ktile + (t < n ? t : 0) * ldw;
-      float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
+    constexpr int TPT = TAIL_THREADS / 8;
+    for (int t0 = 0; t0 < n; t0 += 2 * TPT) {                        // uniform trip count: the lane exchanges need every lane
+      const int t[2] = {t0 + (tid >> 3), t0 + (tid >> 3) + TPT};
+      const uint32_t* row0 = ktile + (t[0] < n ? t[0] : 0) * ldw;
+      const uint32_t* row1 = ktile + (t[1] < n ? t[1] : 0) * ldw;
+      float a[2][4] = {{0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}};
       for (int cw = seg; cw < W; cw += 8) {
-        float x[2];
-        TailWord<DT>::unpack(row[cw], x);
-        const float4 qa = *reinterpret_cast<const float4*>(sq + (cw * EPW) * GC);
-        a0 = fmaf(x[0], qa.x, a0);
-        a1 = fmaf(x[0], qa.y, a1);
-        a2 = fmaf(x[0], qa.z, a2);
-        a3 = fmaf(x[0], qa.w, a3);
-        if (EPW == 2) {
-          const float4 qb = *reinterpret_cast<const float4*>(sq + (cw * EPW + 1) * GC);
-          a0 = fmaf(x[1], qb.x, a0);
-          a1 = fmaf(x[1], qb.y, a1);
-          a2 = fmaf(x[1], qb.z, a2);
-          a3 = fmaf(x[1], qb.w, a3);
+        float x[2][2];
+        TailWord<DT>::unpack(row0[cw], x[0]);
+        TailWord<DT>::unpack(row1[cw], x[1]);
+#pragma unroll
+        for (int e = 0; e < EPW; ++e) {
+          const float4 q4 = *reinterpret_cast<const float4*>(sq + (cw * EPW + e) * GC);
+#pragma unroll
+          for (int u = 0; u < 2; ++u) {
+            a[u][0] = fmaf(x[u][e], q4.x, a[u][0]);
+            a[u][1] = fmaf(x[u][e], q4.y, a[u][1]);
+            a[u][2] = fmaf(x[u][e], q4.z, a[u][2]);
+            a[u][3] = fmaf(x[u][e], q4.w, a[u][3]);
+          }
         }
       }
-      a0 = lanes_sum_dpp<8>(a0);
-      a1 = lanes_sum_dpp<8>(a1);
-      a2 = lanes_sum_dpp<8>(a2);
-      a3 = lanes_sum_dpp<8>(a3);
-      if (seg == 0 && t < n)
-        *reinterpret_cast<float4*>(ss + (c0 + t) * GC) = make_float4(a0 * sm_scale, a1 * sm_scale, a2 * sm_scale, a3 * sm_scale);
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) a[u][g] = lanes_sum_dpp<8>(a[u][g]);
+        if (seg == 0 && t[u] < n)
+          *reinterpret_cast<float4*>(ss + (c0 + t[u]) * GC) =
+              make_float4(a[u][0] * sm_scale, a[u][1] * sm_scale, a[u][2] * sm_scale, a[u][3] * sm_scale);
+      }
     }
   }
   __syncthreads();
@@ -641,7 +715,15 @@ __device__ __forceinline__ void exact_tail_words_body(const TailArgs& A, int h, 
     const int n = min(CH, R - c0);
     if (c0 > 0) {
       __syncthreads();
-      if (active) {
+      if (wide) {
+        if (wr < RP) {
+          u32x4_t vreg[TAIL_WIDE_LOADS];
+          int64_t rb[TAIL_WIDE_LOADS];
+          row_bases4(c0, n, rb);
+          request4(rv, rb, n, vreg);
+          deposit4(vtile, n, vreg);
+        }
+      } else if (active) {
         uint32_t vreg[KC][RPT];
         request(rv, c0, n, vreg);
         deposit(vtile, n, vreg);
@@ -988,6 +1070,9 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   ta.rk = (const uint32_t*)recent_k; ta.rv = (const uint32_t*)recent_v; ta.recent_rows = recent_rows;
   ta.ws_b = rs_b / epw; ta.ws_r = rs_r / epw; ta.ws_h = rs_h / epw; ta.recent_len = recent_len;
   ta.block_table = block_table; ta.bt_stride = bt_stride; ta.seq_lens = seq_lens; ta.ws_blk = ts.s_blk / epw;
+  // 16-byte pieces when every row starts on a 16-byte boundary and a row's pieces fit the workgroup
+  ta.wide = words && ((((uintptr_t)recent_k | (uintptr_t)recent_v) & 15) == 0) &&
+            !((ta.ws_b | ta.ws_r | ta.ws_h | ta.ws_blk) & 3) && (d / epw) / 4 <= TAIL_THREADS;
   ta.max_pages = max_pages; ta.num_blocks = pool_pages;       // the exact cache shares the pool's block numbers
   ta.sm_scale = sm_scale; ta.parts = parts; ta.n_parts = n_parts; ta.part_index = n_split;
   const int n_tail = Hkv * B * ((G + TAIL_GC - 1) / TAIL_GC);
