@@ -462,8 +462,17 @@ template <> struct TailWord<TQ_F16> {
   }
 };
 
-static size_t tail_words_smem(int d, int recent_rows) {
-  return ((size_t)TAIL_GC * d + (size_t)TAIL_GC * recent_rows + 2 * TAIL_GC + 2 * TAIL_TILE_WORDS) * sizeof(float);
+// words of one row tile (keys, values): room for every exact row when that is less than the largest tile
+// (W words per row: d for fp32 rows, d / 2 for 16-bit rows)
+static int tail_tile_words(int W, int recent_rows, bool wide) {
+  const int64_t ldw = wide ? W + 8 : W + 1;
+  // (at least 4096 words: at the end the key tile holds the row slices' partial sums, [<= 8][4 heads][d])
+  int64_t need = ((recent_rows + 15) / 16 * 16) * ldw;
+  if (need < 4096) need = 4096;
+  return (int)(need < TAIL_TILE_WORDS ? (need + 3) / 4 * 4 : TAIL_TILE_WORDS);
+}
+static size_t tail_words_smem(int d, int recent_rows, int tile_words) {
+  return ((size_t)TAIL_GC * d + (size_t)TAIL_GC * recent_rows + 2 * TAIL_GC + 2 * (size_t)tile_words) * sizeof(float);
 }
 
 // KC = word columns per thread (2 only for fp32 rows of more than 512 channels).
@@ -484,6 +493,7 @@ struct TailArgs {
   const int32_t* seq_lens;
   int64_t ws_blk;
   int wide;                        // rows and strides are 16-byte aligned: four words per load
+  int tile_words;                  // LDS words of one row tile (tail_tile_words)
   float sm_scale;
   float* parts;
   int n_parts, part_index;
@@ -491,7 +501,7 @@ struct TailArgs {
 
 // (a device function: the stand-alone kernel and the launch that shares its grid with the query
 // preparation both run it; h / b / gz are the workgroup's KV head, sequence and head group, `sm` its LDS)
-template <int DT, int KC, bool PAGED>
+template <int DT, int KC, bool PAGED, bool WIDE>
 __device__ __forceinline__ void exact_tail_words_body(const TailArgs& A, int h, int b, int gz, float* sm) {
   const void* __restrict__ q = A.q;
   const int Hq = A.Hq, Hkv = A.Hkv, d = A.d, recent_rows = A.recent_rows, bt_stride = A.bt_stride;
@@ -517,16 +527,16 @@ __device__ __forceinline__ void exact_tail_words_body(const TailArgs& A, int h, 
   float* ss = sq + GC * d;                          // [recent_rows][GC] scores, then softmax weights
   float* sml = ss + GC * recent_rows;               // [GC][2]
   uint32_t* ktile = (uint32_t*)(sml + 2 * GC);      // [CH][W + 1] key rows of the chunk; at the end [TS][GC][d] partials
-  uint32_t* vtile = ktile + TAIL_TILE_WORDS;        // [CH][W + 1] value rows
+  uint32_t* vtile = ktile + A.tile_words;           // [CH][W + 1] value rows
   // words per row (a multiple of 32); leading dimension: odd, or (16-byte loads) W + 8, which keeps rows
   // 16-byte aligned and spreads the 8 tokens x 8 segments a wavefront reads in the score stage over all banks
-  const bool wide = A.wide != 0;
+  constexpr bool wide = WIDE;
   const int W = d / EPW, ldw = wide ? W + 8 : W + 1;
   const int TS = W < TAIL_THREADS ? TAIL_THREADS / W : 1;          // row slices
   const int QW = W >> 2, RP = TAIL_THREADS / QW;                   // wide: 4-word pieces per row, rows per round of loads
   const int wq = tid % QW, wr = tid / QW;                          // wide: this thread's piece and row slot
-  const int CH = wide ? min(TAIL_TILE_WORDS / ldw, TAIL_WIDE_LOADS * RP)
-                      : min(TAIL_TILE_WORDS / ldw, TS * RPT);      // rows per chunk
+  const int CH = wide ? min(A.tile_words / ldw, TAIL_WIDE_LOADS * RP)
+                      : min(A.tile_words / ldw, TS * RPT);         // rows per chunk
   const int cw0 = W < TAIL_THREADS ? tid % W : tid, ts = W < TAIL_THREADS ? tid / W : 0;
   const bool active = ts < TS;
   const int64_t base0 = (PAGED ? 0 : b * ws_b) + h * ws_h;
@@ -609,7 +619,7 @@ __device__ __forceinline__ void exact_tail_words_body(const TailArgs& A, int h, 
     }
   };
   const int n_first = min(CH, R);
-  if (wide) {
+  if constexpr (wide) {
     if (wr < RP && n_first > 0) {
       u32x4_t kreg[TAIL_WIDE_LOADS], vreg[TAIL_WIDE_LOADS];
       int64_t rb[TAIL_WIDE_LOADS];
@@ -622,15 +632,17 @@ __device__ __forceinline__ void exact_tail_words_body(const TailArgs& A, int h, 
     } else {
       deposit_query();
     }
-  } else if (active && n_first > 0) {
-    uint32_t kreg[KC][RPT], vreg[KC][RPT];
-    request(rk, 0, n_first, kreg);
-    request(rv, 0, n_first, vreg);
-    deposit_query();
-    deposit(ktile, n_first, kreg);
-    deposit(vtile, n_first, vreg);
   } else {
-    deposit_query();
+    if (active && n_first > 0) {
+      uint32_t kreg[KC][RPT], vreg[KC][RPT];
+      request(rk, 0, n_first, kreg);
+      request(rv, 0, n_first, vreg);
+      deposit_query();
+      deposit(ktile, n_first, kreg);
+      deposit(vtile, n_first, vreg);
+    } else {
+      deposit_query();
+    }
   }
   __syncthreads();
   // scores: eight threads per token, each over every eighth word of the row, for the group's heads at once
@@ -638,7 +650,7 @@ __device__ __forceinline__ void exact_tail_words_body(const TailArgs& A, int h, 
     const int n = min(CH, R - c0);
     if (c0 > 0) {
       __syncthreads();
-      if (wide) {
+      if constexpr (wide) {
         if (wr < RP) {
           u32x4_t kreg[TAIL_WIDE_LOADS];
           int64_t rb[TAIL_WIDE_LOADS];
@@ -646,10 +658,12 @@ __device__ __forceinline__ void exact_tail_words_body(const TailArgs& A, int h, 
           request4(rk, rb, n, kreg);
           deposit4(ktile, n, kreg);
         }
-      } else if (active) {
-        uint32_t kreg[KC][RPT];
-        request(rk, c0, n, kreg);
-        deposit(ktile, n, kreg);
+      } else {
+        if (active) {
+          uint32_t kreg[KC][RPT];
+          request(rk, c0, n, kreg);
+          deposit(ktile, n, kreg);
+        }
       }
       __syncthreads();
     }
@@ -715,7 +729,7 @@ __device__ __forceinline__ void exact_tail_words_body(const TailArgs& A, int h, 
     const int n = min(CH, R - c0);
     if (c0 > 0) {
       __syncthreads();
-      if (wide) {
+      if constexpr (wide) {
         if (wr < RP) {
           u32x4_t vreg[TAIL_WIDE_LOADS];
           int64_t rb[TAIL_WIDE_LOADS];
@@ -723,10 +737,12 @@ __device__ __forceinline__ void exact_tail_words_body(const TailArgs& A, int h, 
           request4(rv, rb, n, vreg);
           deposit4(vtile, n, vreg);
         }
-      } else if (active) {
-        uint32_t vreg[KC][RPT];
-        request(rv, c0, n, vreg);
-        deposit(vtile, n, vreg);
+      } else {
+        if (active) {
+          uint32_t vreg[KC][RPT];
+          request(rv, c0, n, vreg);
+          deposit(vtile, n, vreg);
+        }
       }
       __syncthreads();
     }
@@ -774,11 +790,11 @@ __device__ __forceinline__ void exact_tail_words_body(const TailArgs& A, int h, 
   }
 }
 
-template <int DT, int KC, bool PAGED>
+template <int DT, int KC, bool PAGED, bool WIDE>
 __global__ void __launch_bounds__(TAIL_THREADS)
 exact_tail_words_kernel(TailArgs A) {
   extern __shared__ __align__(16) float sm[];
-  exact_tail_words_body<DT, KC, PAGED>(A, blockIdx.x, blockIdx.y, blockIdx.z, sm);
+  exact_tail_words_body<DT, KC, PAGED, WIDE>(A, blockIdx.x, blockIdx.y, blockIdx.z, sm);
 }
 
 // One launch for the two things a hybrid step does before its page kernel: the exact-tail workgroups
@@ -788,14 +804,14 @@ exact_tail_words_kernel(TailArgs A) {
 // the two instead of their sum plus a dispatch gap.
 static_assert(TAIL_THREADS == PREP_COLS * PREP_SLICES, "the two roles share a workgroup size");
 template <int PER, int DT, bool PAGED>
-__global__ void __launch_bounds__(TAIL_THREADS)
+__global__ void __launch_bounds__(TAIL_THREADS, 4)
 prep_tail_kernel(TailArgs A, int n_tail, int B, int Gq, tq_layer ly, float* __restrict__ q_rot, float* __restrict__ q_sk,
                  float* __restrict__ q_stat, uint32_t* __restrict__ qa_pack, unsigned long long* __restrict__ arrivals) {
   extern __shared__ __align__(16) float sm[];
   const int id = blockIdx.x;
   if (id < n_tail) {
     const int per_z = A.Hkv * B;
-    exact_tail_words_body<DT, 1, PAGED>(A, id % A.Hkv, (id / A.Hkv) % B, id / per_z, sm);
+    exact_tail_words_body<DT, 1, PAGED, true>(A, id % A.Hkv, (id / A.Hkv) % B, id / per_z, sm);
   } else {
     const int words = ly.d / PREP_COLS, p = id - n_tail;
     // (the arrival counter of this group of query heads, for a page kernel that merges its splits itself)
@@ -1073,6 +1089,7 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   // 16-byte pieces when every row starts on a 16-byte boundary and a row's pieces fit the workgroup
   ta.wide = words && ((((uintptr_t)recent_k | (uintptr_t)recent_v) & 15) == 0) &&
             !((ta.ws_b | ta.ws_r | ta.ws_h | ta.ws_blk) & 3) && (d / epw) / 4 <= TAIL_THREADS;
+  ta.tile_words = tail_tile_words(d / epw, recent_rows, ta.wide != 0);
   ta.max_pages = max_pages; ta.num_blocks = pool_pages;       // the exact cache shares the pool's block numbers
   ta.sm_scale = sm_scale; ta.parts = parts; ta.n_parts = n_parts; ta.part_index = n_split;
   const int n_tail = Hkv * B * ((G + TAIL_GC - 1) / TAIL_GC);
@@ -1118,10 +1135,12 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
     if (!layer->Pi || !layer->PiT || !layer->S || !layer->ST || !layer->centroids) return TQ_ENULL;
     const int n_prep = (B * Hq / Gq) * (d / PREP_COLS);
     // Whole hybrid step on the matrix-core path: the exact tail shares the preparation's launch, as long as
-    // every workgroup of the two gets a compute unit of its own at once (a tail workgroup's LDS fills one).
-    if (tail && words && mfma_shape && stages == 7 && n_tail + n_prep <= compute_units()) {
-      size_t fsm = tail_words_smem(d, recent_rows);
-      if (prep_smem_bytes(Gq, d) > fsm) fsm = prep_smem_bytes(Gq, d);
+    // all workgroups of the two are resident at once (two per compute unit when their LDS allows it: the
+    // kernel is built for 128 registers per lane).
+    size_t fsm = tail_words_smem(d, recent_rows, ta.tile_words);
+    if (prep_smem_bytes(Gq, d) > fsm) fsm = prep_smem_bytes(Gq, d);
+    const int per_cu = 2 * fsm + 2048 <= 160 * 1024 ? 2 : 1;
+    if (tail && ta.wide && mfma_shape && stages == 7 && n_tail + n_prep <= per_cu * compute_units()) {
 #define TQ_LAUNCH_PT(PER, DT, PAGED)                                                                                 \
   {                                                                                                                  \
     auto kern = prep_tail_kernel<PER, DT, PAGED>;                                                                    \
@@ -1165,7 +1184,7 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   // its splits itself finds it written
   if (tail && (stages & 2) && !tail_done) {
     const dim3 tgrid(Hkv, B, (G + TAIL_GC - 1) / TAIL_GC);
-    size_t tsm = words ? tail_words_smem(d, recent_rows) : tail_smem(d, recent_rows);
+    size_t tsm = words ? tail_words_smem(d, recent_rows, ta.tile_words) : tail_smem(d, recent_rows);
 #define TQ_LAUNCH_TAIL(KERN, ...)                                                                                    \
   {                                                                                                                  \
     auto kern = KERN;                                                                                                \
@@ -1177,16 +1196,21 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   }
 #define TQ_TAIL_ROWS_ARGS q, Hq, Hkv, d, recent_k, recent_v, recent_rows, rs_b, rs_r, rs_h, recent_len, sm_scale, parts, n_parts, n_split
 #define TQ_TAIL_WORD_ARGS ta
-#define TQ_TAIL_WORDS(PAGED)                                                                                   \
-  {                                                                                                            \
-    if (dtype == TQ_BF16) TQ_LAUNCH_TAIL((exact_tail_words_kernel<TQ_BF16, 1, PAGED>), TQ_TAIL_WORD_ARGS)      \
-    else if (dtype == TQ_F16) TQ_LAUNCH_TAIL((exact_tail_words_kernel<TQ_F16, 1, PAGED>), TQ_TAIL_WORD_ARGS)   \
-    else if (d <= TAIL_THREADS) TQ_LAUNCH_TAIL((exact_tail_words_kernel<TQ_F32, 1, PAGED>), TQ_TAIL_WORD_ARGS) \
-    else TQ_LAUNCH_TAIL((exact_tail_words_kernel<TQ_F32, 2, PAGED>), TQ_TAIL_WORD_ARGS)                        \
+#define TQ_TAIL_WORDS(PAGED, WIDE)                                                                                   \
+  {                                                                                                                  \
+    if (dtype == TQ_BF16) TQ_LAUNCH_TAIL((exact_tail_words_kernel<TQ_BF16, 1, PAGED, WIDE>), TQ_TAIL_WORD_ARGS)      \
+    else if (dtype == TQ_F16) TQ_LAUNCH_TAIL((exact_tail_words_kernel<TQ_F16, 1, PAGED, WIDE>), TQ_TAIL_WORD_ARGS)   \
+    else if (d <= TAIL_THREADS) TQ_LAUNCH_TAIL((exact_tail_words_kernel<TQ_F32, 1, PAGED, WIDE>), TQ_TAIL_WORD_ARGS) \
+    else TQ_LAUNCH_TAIL((exact_tail_words_kernel<TQ_F32, 2, PAGED, WIDE>), TQ_TAIL_WORD_ARGS)                        \
   }
     if (words) {
-      if (ts.paged) TQ_TAIL_WORDS(true)
-      else TQ_TAIL_WORDS(false)
+      if (ts.paged) {
+        if (ta.wide) TQ_TAIL_WORDS(true, true)
+        else TQ_TAIL_WORDS(true, false)
+      } else {
+        if (ta.wide) TQ_TAIL_WORDS(false, true)
+        else TQ_TAIL_WORDS(false, false)
+      }
     } else {      // 16-bit rows that are not word-aligned
       if (dtype == TQ_BF16) TQ_LAUNCH_TAIL(exact_tail_kernel<TQ_BF16>, TQ_TAIL_ROWS_ARGS)
       else TQ_LAUNCH_TAIL(exact_tail_kernel<TQ_F16>, TQ_TAIL_ROWS_ARGS)
