@@ -1004,19 +1004,6 @@ extern "C" int tq_decode_merge(const float* parts, int64_t rows, int n_parts, in
 }
 
 namespace {
-int compute_units() {
-  static std::atomic<int> cached{0};
-  int v = cached.load();
-  if (!v) {
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0)
-      v = 1;
-    cached.store(v);
-  }
-  return v;
-}
-
 // The exact tokens of a step.  Rows: (B, rows, H, d) tensors with element strides s_b / s_r / s_h and `len`
 // valid rows per sequence.  Paged: the newest min(seq_len, rows) tokens of every sequence, read in place
 // from a paged exact cache (block stride s_blk, token stride s_r, head stride s_h) through the step's
@@ -1134,13 +1121,14 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   if ((stages & 1) && !fused) {
     if (!layer->Pi || !layer->PiT || !layer->S || !layer->ST || !layer->centroids) return TQ_ENULL;
     const int n_prep = (B * Hq / Gq) * (d / PREP_COLS);
-    // Whole hybrid step on the matrix-core path: the exact tail shares the preparation's launch, as long as
-    // all workgroups of the two are resident at once (two per compute unit when their LDS allows it: the
-    // kernel is built for 128 registers per lane).
+    // Whole hybrid step on the matrix-core path: the exact tail shares the preparation's launch (the tail
+    // workgroups first, so that the longer-running ones start first).  The kernel is built for 128 registers
+    // per lane and the tail's LDS is sized by the rows it holds, so two workgroups fit a compute unit; with more
+    // workgroups than that the rest follow as slots free up, which still measured faster than a launch each
+    // (16 x 8192: 48.9 -> 45.2 us per step, 32 x 32768: 223.6 -> 221.5 us).
     size_t fsm = tail_words_smem(d, recent_rows, ta.tile_words);
     if (prep_smem_bytes(Gq, d) > fsm) fsm = prep_smem_bytes(Gq, d);
-    const int per_cu = 2 * fsm + 2048 <= 160 * 1024 ? 2 : 1;
-    if (tail && ta.wide && mfma_shape && stages == 7 && n_tail + n_prep <= per_cu * compute_units()) {
+    if (tail && ta.wide && mfma_shape && stages == 7) {
 #define TQ_LAUNCH_PT(PER, DT, PAGED)                                                                                 \
   {                                                                                                                  \
     auto kern = prep_tail_kernel<PER, DT, PAGED>;                                                                    \
