@@ -39,7 +39,8 @@ constexpr int PREP_COLS = 32, PREP_SLICES = 16;
 __device__ __forceinline__ float round_fp6(float v, uint32_t& code) {
   const float a = fminf(fabsf(v), 7.5f);
   const float inv_step = a < 2.0f ? 8.0f : (a < 4.0f ? 4.0f : 2.0f);
-  const float r = rintf(a * inv_step) / inv_step;    // exact (powers of two); may land on the next binade
+  const float step = a < 2.0f ? 0.125f : (a < 4.0f ? 0.25f : 0.5f);
+  const float r = rintf(a * inv_step) * step;        // exact (powers of two); may land on the next binade
   const int e = r < 1.0f ? 0 : (r < 2.0f ? 1 : (r < 4.0f ? 2 : 3));
   const float inv_unit = e <= 1 ? 8.0f : (e == 2 ? 4.0f : 2.0f);
   const int m = (int)(r * inv_unit) - (e == 0 ? 0 : 8);
