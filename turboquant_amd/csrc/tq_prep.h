@@ -207,48 +207,58 @@ __device__ __forceinline__ void prep_query_body(const void* __restrict__ q, int 
     (sk ? q_sk : q_rot)[(row0 + r) * d + word * PREP_COLS + c] = acc;
   }
   __syncthreads();
-  // operands of this plane word.  First the four 6-bit codes of every (term plane, head, contraction
-  // index) into shared memory (the partial sums are no longer needed), then per (term plane, row set,
-  // row) one lane x six dwords, each gathered from the (up to seven) codes that overlap it.
-  uint32_t* codes = (uint32_t*)pa;                           // [ntp][G][4 terms][32]
-  // thread -> (contraction index, head, half of the workgroup); the halves take alternate term planes
-  for (int tp = tid >> 8; tp < ntp; tp += 2) {
-    const int kloc = tid & 31, g = (tid >> 5) & 7;
-    if (g >= G) break;
-    const bool is_sign = tp == ntp - 1;
-    const int c = 4 * (kloc & 7) + (kloc >> 3);              // coordinate within the word
+  // Operands of this plane word: one lane per (term plane, head) turns the 32 values of its row block into
+  // the four fp6 terms with the packing conversion of gfx950 (v_cvt_scalef32_2xpk16_fp6_f32: 32 floats ->
+  // 32 six-bit codes in six dwords, round to nearest even, saturating - the grid and rounding of round_fp6,
+  // except that a small negative value keeps its sign on the zero code, which adds nothing in the MFMA) and
+  // gets the rounded values back for the residual with its inverse (v_cvt_scalef32_pk32_f32_fp6).
+  // Code j of a conversion comes from element j / 2 of its first (j even) or second (j odd) operand.
+  if (tid < ntp * 8) {
+    typedef float f32x16_t __attribute__((ext_vector_type(16)));
+    typedef float f32x32_t __attribute__((ext_vector_type(32)));
+    typedef uint32_t u32x6_t __attribute__((ext_vector_type(6)));
+    const int tp = tid >> 3, g = tid & 7;
+    const bool is_sign = tp == ntp - 1, live = g < G;
+    const int gs = live ? g : 0;
     // the decode kernel extracts three of the four bits of a nibble in place, where they are the fp4
     // numbers 1, 2 and 4 (after its block scale): the query side divides them out
-    const int t4 = kloc >> 3;
-    const float mul = 4.0f * (is_sign ? stat[g * 4 + 1] : coefs[tp] * stat[g * 4 + 0]) *
-                      (t4 == 1 ? 0.5f : (t4 == 2 ? 0.25f : 1.0f));
-    float v = (is_sign ? ssk : srot)[g * PREP_COLS + c] * mul;
+    const float base = live ? 4.0f * (is_sign ? stat[gs * 4 + 1] : coefs[tp] * stat[gs * 4 + 0]) : 0.0f;
+    const float4* src = (const float4*)((is_sign ? ssk : srot) + gs * PREP_COLS);
+    float x[PREP_COLS];
+#pragma unroll
+    for (int k = 0; k < PREP_COLS / 4; ++k) {
+      const float4 v4 = src[k];
+      x[4 * k] = v4.x; x[4 * k + 1] = v4.y; x[4 * k + 2] = v4.z; x[4 * k + 3] = v4.w;
+    }
+    f32x16_t va, vb;                      // contraction indices 0, 2, 4, ... and 1, 3, 5, ...
+#pragma unroll
+    for (int kloc = 0; kloc < 32; ++kloc) {
+      const int c = 4 * (kloc & 7) + (kloc >> 3), t4 = kloc >> 3;      // coordinate within the word
+      const float v = x[c] * (base * (t4 == 1 ? 0.5f : (t4 == 2 ? 0.25f : 1.0f)));
+      if (kloc & 1) vb[kloc >> 1] = v;
+      else va[kloc >> 1] = v;
+    }
+    const int i = word >> 2, kw = word & 3;
+    uint32_t* dst = qa_pack + group * (int64_t)(ntp * wpl * 2 * 64 * 8);
+    const float one = 1.0f;
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-      uint32_t code;
-      const float r = round_fp6(v, code);
-      codes[((tp * G + g) * 4 + t) * PREP_COLS + kloc] = code;
-      v = (v - r) * 32.0f;
-    }
-  }
-  __syncthreads();
-  const int i = word >> 2, kw = word & 3;
-  uint32_t* dst = qa_pack + group * (int64_t)(ntp * wpl * 2 * 64 * 8);
-  for (int o = tid; o < ntp * 256; o += blockDim.x) {
-    const int dwi = o & 7, n = (o >> 3) & 15, rs = (o >> 7) & 1, tp = o >> 8;
-    if (dwi >= 6) continue;
-    const int g = n >> 1;
-    const int term = 2 * rs + (n & 1);
-    uint32_t packed = 0;
-    if (g < G) {
-      const uint32_t* cd = codes + ((tp * G + g) * 4 + term) * PREP_COLS;
-      const int j0 = (32 * dwi) / 6, j1 = min((32 * dwi + 31) / 6, 31);
-      for (int kloc = j0; kloc <= j1; ++kloc) {
-        const int bit = 6 * kloc - 32 * dwi;                 // position of the code in this dword (may straddle)
-        packed |= bit >= 0 ? cd[kloc] << bit : cd[kloc] >> -bit;
+      u32x6_t code;
+      // (inline assembly with early-clobber results: the conversions read their sources over several passes)
+      asm volatile("v_cvt_scalef32_2xpk16_fp6_f32 %0, %1, %2, %3" : "=&v"(code) : "v"(va), "v"(vb), "v"(one));
+      uint32_t* o = dst + (((tp * wpl + i) * 2 + (t >> 1)) * 64 + 2 * g + (t & 1) + 16 * kw) * 8;
+      *(uint4*)o = make_uint4(code[0], code[1], code[2], code[3]);
+      *(uint2*)(o + 4) = make_uint2(code[4], code[5]);
+      if (t < 3) {
+        f32x32_t r;
+        asm volatile("v_cvt_scalef32_pk32_f32_fp6 %0, %1, %2" : "=&v"(r) : "v"(code), "v"(one));
+#pragma unroll
+        for (int k = 0; k < 16; ++k) {
+          va[k] = (va[k] - r[2 * k]) * 32.0f;
+          vb[k] = (vb[k] - r[2 * k + 1]) * 32.0f;
+        }
       }
     }
-    dst[(((tp * wpl + i) * 2 + rs) * 64 + n + 16 * kw) * 8 + dwi] = packed;
   }
 }
 

@@ -74,7 +74,7 @@ __global__ void __launch_bounds__(PREP_COLS * PREP_SLICES)
 prep_query_kernel(const void* __restrict__ q, int G, tq_layer ly, float sm_scale,
                   float* __restrict__ q_rot, float* __restrict__ q_sk, float* __restrict__ q_stat,
                   uint32_t* __restrict__ qa_pack, unsigned long long* __restrict__ arrivals) {
-  extern __shared__ float sm[];
+  extern __shared__ __align__(16) float sm[];
   // the arrival counter of this group of query heads, for the page kernel that merges its splits itself
   if (arrivals != nullptr && blockIdx.y == 0 && threadIdx.x == 0) arrivals[blockIdx.x] = 0ull;
   prep_query_body<PER, DT>(q, G, ly, sm_scale, q_rot, q_sk, q_stat, qa_pack, blockIdx.x, blockIdx.y, sm);
