@@ -477,7 +477,53 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
       }
   }
   __syncthreads();                                              // every wavefront has read the unit-vector terms
-  {
+  if constexpr (FX) {
+    // The index bit planes straight from the comparisons (no index is formed): with the count of thresholds
+    // below y as the index (searchsorted; a NaN counts all), the low bit is the parity of the comparisons and,
+    // for two bits, the high bit the comparison with the middle threshold.  The comparison results are lane
+    // masks, so the parity costs scalar instructions only.
+    uint32_t bitc[2][4];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) bitc[h][i] = 1u << (16 * h + 4 * kb + i);
+    const float t0 = sthr[0], t1 = mb == 2 ? sthr[1] : 0.0f, t2 = mb == 2 ? sthr[2] : 0.0f;
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+      const int t = 16 * m + n;
+#pragma unroll
+      for (int wl = 0; wl < NPW / 2; ++wl) {
+        uint32_t hi = 0, lo = 0;
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float y = acc[m][2 * wl + h][i];
+            const bool c0 = !(y <= t0);
+            if (mb == 2) {
+              const bool c1 = !(y <= t1), c2 = !(y <= t2);
+              hi |= c1 ? bitc[h][i] : 0u;
+              lo |= (c0 != c1) != c2 ? bitc[h][i] : 0u;
+            } else {
+              hi |= c0 ? bitc[h][i] : 0u;
+            }
+          }
+        hi = or_over_kb(hi);
+        if (mb == 2) lo = or_over_kb(lo);
+        if (kb == 0) {
+          spl[(0 * TT + t) * W + (wave * NPW) / 2 + wl] = hi;
+          if (mb == 2) spl[(1 * TT + t) * W + (wave * NPW) / 2 + wl] = lo;
+        }
+      }
+      if constexpr (std::is_same<Sink, KeyFlatSink>::value) {
+#pragma unroll
+        for (int c = 0; c < NPW; ++c) {
+          const int col0 = 16 * (wave * NPW + c) + 4 * kb;
+          if (sink.y_dbg && svalid[t]) *(f32x4*)(sink.y_dbg + (tile0 * TILE + t) * D + col0) = acc[m][c];
+        }
+      }
+    }
+  } else {
     uint32_t idx[MT][NPW][4];
 #pragma unroll
     for (int m = 0; m < MT; ++m)
