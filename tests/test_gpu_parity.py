@@ -610,6 +610,8 @@ def test_decode_attention_ragged_empty_and_hybrid_tail(gpu):
     (256, torch.bfloat16, 16, 2, [300, 129, 1], 0),       # three chunks of 128 rows, ragged
     (256, torch.bfloat16, 16, 2, [128, 77, 0], 1),        # rows not word-aligned: row-staged kernel
     (128, torch.float16, 8, 8, [200, 256, 13], 2),        # strided rows, still word-aligned; one head per KV head
+    (128, torch.bfloat16, 8, 2, [150, 128, 1], 8),        # 16-byte aligned rows in a wider buffer, two chunks' worth
+    (256, torch.bfloat16, 16, 2, [128, 40, 0], 6),        # word-aligned but not 16-byte aligned: 4-byte loads
     (64, torch.float16, 6, 2, [520, 3, 64], 0),           # two chunks at the smallest head size, 3 heads per group
     (128, torch.float32, 8, 2, [130, 64, 5], 0),          # fp32 rows
     (576, torch.float32, 4, 1, [40, 17, 33], 0),          # fp32 rows wider than the workgroup: two columns per thread
