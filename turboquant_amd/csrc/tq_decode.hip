@@ -941,6 +941,7 @@ std::atomic<int> opt_merge_in_kernel{1};
 std::atomic<int> opt_page_pairs{1};
 std::atomic<int> opt_narrow_rows{1};
 std::atomic<int> opt_lds_stage{1};
+std::atomic<int> opt_wide_workgroups{1};
 }  // namespace tq
 
 namespace {
@@ -971,6 +972,7 @@ extern "C" int tq_set_option(const char* name, int64_t value) {
     opt_prep_spin_limit.store((int)value);
     return TQ_OK;
   }
+  if (!std::strcmp(name, "wide_workgroups")) { opt_wide_workgroups.store(value != 0); return TQ_OK; }
   if (!std::strcmp(name, "lds_stage")) { opt_lds_stage.store(value != 0); return TQ_OK; }
   if (!std::strcmp(name, "narrow_rows")) { opt_narrow_rows.store(value != 0); return TQ_OK; }
   if (!std::strcmp(name, "page_pairs")) { opt_page_pairs.store(value != 0); return TQ_OK; }
@@ -1045,13 +1047,6 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   if (tail && recent_rows > 1024) return TQ_EUNSUPPORTED;
   const int len_sub = tail && ts.paged ? recent_rows : 0;       // newest tokens the pages do not cover
   hipStream_t st = (hipStream_t)stream;
-  const int n_parts = n_split + 1;
-  float* parts = (float*)workspace;
-  float* q_rot = parts + parts_floats(B, Hq, d, n_parts);
-  float* q_sk = q_rot + (size_t)B * Hq * d;
-  float* q_stat = q_sk + (size_t)B * Hq * d;
-  unsigned long long* flags = (unsigned long long*)(q_stat + (size_t)4 * B * Hq);       // 8-byte aligned: every term above is even
-  uint32_t* qa_pack = (uint32_t*)(flags + flag_words(B, Hq));
   // the matrix-core kernel takes up to 8 query heads per group: a KV head with more is served by kv_div
   // groups of G / kv_div heads (0 = no such split, e.g. 11 heads)
   int kv_div = 0;
@@ -1061,6 +1056,18 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   const bool mfma_shape = kv_div && (d == 64 || d == 128 || d == 256) && (layout->dtype == TQ_BF16 || layout->dtype == TQ_F16) &&
                           layout->value_bits != 8 && layer->Pi_colsum &&
                           layer->S_colsum;
+  // Short contexts with at most four query heads per group run workgroups of eight wavefronts on half as many
+  // splits (the same number of wavefronts): everything below - partials, merge, the workspace's carving - then
+  // uses the halved count, for every stage of the step alike.
+  const bool wide_wg = mfma_shape && layout->key_lane_major && decode_mfma_wide_workgroups(d, Gq, n_split, max_pages);
+  if (wide_wg) n_split /= 2;
+  const int n_parts = n_split + 1;
+  float* parts = (float*)workspace;
+  float* q_rot = parts + parts_floats(B, Hq, d, n_parts);
+  float* q_sk = q_rot + (size_t)B * Hq * d;
+  float* q_stat = q_sk + (size_t)B * Hq * d;
+  unsigned long long* flags = (unsigned long long*)(q_stat + (size_t)4 * B * Hq);       // 8-byte aligned: every term above is even
+  uint32_t* qa_pack = (uint32_t*)(flags + flag_words(B, Hq));
 
   if (dtype < TQ_F32 || dtype > TQ_BF16) return TQ_EINVAL;
   // the exact tail as 32-bit words: always for fp32, for 16-bit rows when they are word-aligned
@@ -1102,7 +1109,7 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
     fz.nonce = next_nonce();
     const int mf = launch_decode_mfma(qa_pack, q_stat, B, Hq, Hkv * kv_div, kv_div, pool, block_table, bt_stride, seq_lens,
                                       sm_scale, *layer, *layout, parts, n_parts, n_split, len_sub, max_pages, pool_pages,
-                                      fz, FusedMerge{}, st);
+                                      fz, FusedMerge{}, wide_wg, st);
     if (mf > 0) return mf;
     fused = mf == TQ_OK;             // TQ_EUNSUPPORTED: nothing was launched, the separate launches below run
   }
@@ -1213,7 +1220,7 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   if ((stages & 2) && !fused)
     mf = mfma_shape ? launch_decode_mfma(qa_pack, q_stat, B, Hq, Hkv * kv_div, kv_div, pool, block_table, bt_stride,
                                          seq_lens, sm_scale, *layer, *layout, parts, n_parts, n_split, len_sub,
-                                         max_pages, pool_pages, FusedPrep{}, fm, st)
+                                         max_pages, pool_pages, FusedPrep{}, fm, wide_wg, st)
                     : TQ_EUNSUPPORTED;
   if (mf > 0) return mf;
   if (mf == TQ_OK && fm.out != nullptr) return TQ_OK;         // merged in the launch

@@ -45,6 +45,11 @@ size_t decode_mfma_pack_words(int B, int Hq, int d);
 int launch_decode_mfma(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, int kv_div, const uint8_t* pool,
                        const int32_t* block_table, int bt_stride, const int32_t* seq_lens, float sm_scale,
                        const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts, int n_split, int len_sub,
-                       int max_pages, int num_pages, const FusedPrep& fz, const FusedMerge& fm, hipStream_t st);
+                       int max_pages, int num_pages, const FusedPrep& fz, const FusedMerge& fm, bool wide_wg,
+                       hipStream_t st);
+
+// Whether a step of this shape runs workgroups of eight wavefronts: the caller then passes HALF its split count
+// (and wide_wg = true) to launch_decode_mfma and uses that count for everything that follows.
+bool decode_mfma_wide_workgroups(int d, int G, int n_split, int max_pages);
 
 }  // namespace tq

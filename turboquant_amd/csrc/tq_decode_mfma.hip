@@ -221,8 +221,10 @@ __device__ __forceinline__ constexpr int v_bitpos(int t) {
 // SG: the page data of the next block goes HBM -> LDS with LDS-direct loads, requested when the current
 // block's copy has been taken out of LDS, so every load has a whole trip to arrive (instead of one stage)
 // and no register holds data in flight.
-template <int D, int MB, int NX, int VB, int GS, int DS, int WPS, bool F16P, bool PP, bool NR, bool SG>
-__global__ void __launch_bounds__(MF_WAVES * 64, WPS)
+// NW: wavefronts per workgroup, 4 (two workgroups per compute unit) or 8 (one): with few blocks per
+// wavefront the larger workgroup wins - half as many workgroups to dispatch, prologues and partials.
+template <int D, int MB, int NX, int VB, int GS, int DS, int WPS, bool F16P, bool PP, bool NR, bool SG, int NW>
+__global__ void __launch_bounds__(NW * 64, WPS)
 decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div,
                    const uint8_t* __restrict__ pool, const int32_t* __restrict__ block_table,
                    int bt_stride, const int32_t* __restrict__ seq_lens, float sm_scale, tq_layer ly, tq_page_layout L,
@@ -238,6 +240,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   constexpr int NG = DW / GS, CTG = GS / 16;  // groups of one wavefront, channel tiles per group
   constexpr int NGT = D / GS;                 // groups of the whole head
   constexpr int PIECES = 2 * NG;              // 16-byte pieces of this wavefront's scales per page
+  constexpr int MF_WAVES = NW;
   constexpr int NGRP = MF_WAVES / DS;         // wavefront groups (each walks its own blocks)
   constexpr int WAVE_LDS_FLOATS = wave_lds_floats(NG, DS);
   constexpr int NPG = PP ? 2 : 4;             // score MFMA groups per block: pages, or pairs of pages
@@ -1057,16 +1060,18 @@ bool take_time_hook(int which, hipEvent_t& start, hipEvent_t& stop) {
   return start != nullptr || stop != nullptr;
 }
 
-template <int D, int MB, int NX, int VB, int GS, int DS, int WPS, bool F16P, bool PP = false, bool NR = false, bool SG = false>
+template <int D, int MB, int NX, int VB, int GS, int DS, int WPS, bool F16P, bool PP = false, bool NR = false, bool SG = false,
+          int NW = MF_WAVES>
 static int launch_one(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, int kv_div,
                       const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
                       float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts, int n_split,
-                      int len_sub, int max_pages, int num_pages, const FusedPrep& fz, const FusedMerge& fm, hipStream_t st) {
+                      int len_sub, int max_pages, int num_pages, const FusedPrep& fz, const FusedMerge& fm, bool wide_wg,
+                      hipStream_t st) {
   const int G = Hq / Hkv;
   size_t per_wave = (size_t)wave_lds_floats(D / DS / GS, DS) * sizeof(float);
-  size_t merge = (size_t)(MF_WAVES / DS * G * (D + 2) + MF_WAVES * 16 * 16) * sizeof(float);
+  size_t merge = (size_t)(NW / DS * G * (D + 2) + NW * 16 * 16) * sizeof(float);
   if (SG) per_wave += stage_bytes((D / DS / 16) * VB / 2);
-  size_t smem = per_wave * MF_WAVES > merge ? per_wave * MF_WAVES : merge;
+  size_t smem = per_wave * NW > merge ? per_wave * NW : merge;
   if (fz.q) {
     const size_t prep = (size_t)prep_unit_smem_floats(fz.hp, D) * sizeof(float);
     if (prep > smem) smem = prep;
@@ -1074,34 +1079,53 @@ static int launch_one(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, 
   if (D == 64 && !PP && G <= 4 && opt_page_pairs.load(std::memory_order_relaxed) != 0)
     return launch_one<D, MB, NX, VB, GS, DS, WPS, F16P, D == 64>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,
                                                                  bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts,
-                                                                 n_split, len_sub, max_pages, num_pages, fz, fm, st);
+                                                                 n_split, len_sub, max_pages, num_pages, fz, fm, wide_wg, st);
   if (D >= 128 && !NR && G <= 4 && opt_narrow_rows.load(std::memory_order_relaxed) != 0)
     return launch_one<D, MB, NX, VB, GS, DS, WPS, F16P, false, D >= 128>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,
                                                                          bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts,
-                                                                         n_split, len_sub, max_pages, num_pages, fz, fm, st);
+                                                                         n_split, len_sub, max_pages, num_pages, fz, fm, wide_wg, st);
   // (measured: the staged variant only pays where the register-held variant spills, i.e. with three index planes)
   constexpr bool can_stage = D >= 128 && MB == 3;
   if (can_stage && !SG && opt_lds_stage.load(std::memory_order_relaxed) != 0)
     return launch_one<D, MB, NX, VB, GS, DS, WPS, F16P, PP, NR, can_stage>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,
                                                                            bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts,
-                                                                           n_split, len_sub, max_pages, num_pages, fz, fm, st);
-  auto kern = decode_mfma_kernel<D, MB, NX, VB, GS, DS, WPS, F16P, PP, NR, SG>;
+                                                                           n_split, len_sub, max_pages, num_pages, fz, fm, wide_wg, st);
+  // eight wavefronts per workgroup (one workgroup per compute unit) for the kernels of at most four query heads
+  constexpr bool can_widen = DS == 1 && (PP || NR) && NW == MF_WAVES;
+  if (can_widen && wide_wg)
+    return launch_one<D, MB, NX, VB, GS, DS, WPS, F16P, PP, NR, SG, can_widen ? 2 * MF_WAVES : NW>(
+        qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table, bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts, n_split,
+        len_sub, max_pages, num_pages, fz, fm, false, st);
+  auto kern = decode_mfma_kernel<D, MB, NX, VB, GS, DS, WPS, F16P, PP, NR, SG, NW>;
   if (smem > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return (int)e;
   }
   hipEvent_t t_start_event = nullptr, t_stop_event = nullptr;
   if (take_time_hook(0, t_start_event, t_stop_event)) {
-    hipExtLaunchKernelGGL(kern, dim3(n_split, Hkv, B), dim3(MF_WAVES * 64), smem, st, t_start_event, t_stop_event, 0,
+    hipExtLaunchKernelGGL(kern, dim3(n_split, Hkv, B), dim3(NW * 64), smem, st, t_start_event, t_stop_event, 0,
                           qa_pack, q_stat, Hq, Hkv, kv_div, pool, block_table, bt_stride, seq_lens, sm_scale, ly, L, parts,
                           n_parts, n_split, len_sub, max_pages, num_pages, fz, fm);
   } else {
-    kern<<<dim3(n_split, Hkv, B), dim3(MF_WAVES * 64), smem, st>>>(qa_pack, q_stat, Hq, Hkv, kv_div, pool, block_table,
+    kern<<<dim3(n_split, Hkv, B), dim3(NW * 64), smem, st>>>(qa_pack, q_stat, Hq, Hkv, kv_div, pool, block_table,
                                                                    bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts,
                                                                    n_split, len_sub, max_pages, num_pages, fz, fm);
   }
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? TQ_OK : (int)e;
+}
+
+// Whether a step of this shape should run workgroups of eight wavefronts (the caller then halves its split
+// count: the launch keeps its number of wavefronts).  Taken when a wavefront would walk at most 16 blocks of
+// the longest sequence the block table can hold: 16 x 8192 tokens at 32 q / 8 KV heads 39.7 -> 38.2 us per
+// step, but 32 x 32768 (64 blocks per wavefront) 212 -> 216 us.
+bool decode_mfma_wide_workgroups(int d, int G, int n_split, int max_pages) {
+  if (!(d == 64 || d == 128) || G > 4 || n_split < 2 || (n_split & 1)) return false;
+  if (opt_wide_workgroups.load(std::memory_order_relaxed) == 0) return false;
+  if (d == 64 ? opt_page_pairs.load(std::memory_order_relaxed) == 0 : opt_narrow_rows.load(std::memory_order_relaxed) == 0)
+    return false;
+  const int64_t blocks = ((int64_t)max_pages * TQ_PAGE_TOKENS + BLK_TOK - 1) / BLK_TOK;
+  return blocks <= (int64_t)16 * MF_WAVES * n_split;
 }
 
 // Returns TQ_EUNSUPPORTED when the shape has no matrix-core kernel; the caller then
@@ -1113,7 +1137,7 @@ int launch_decode_mfma(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv,
                        const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
                        float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts,
                        int n_split, int len_sub, int max_pages, int num_pages, const FusedPrep& fz, const FusedMerge& fm,
-                       hipStream_t st) {
+                       bool wide_wg, hipStream_t st) {
   const int G = Hq / Hkv, d = ly.d, mb = ly.mse_bits, vb = L.value_bits, gs = L.group_size;
   if (G > 8 || (L.dtype != TQ_BF16 && L.dtype != TQ_F16) || !L.key_lane_major) return TQ_EUNSUPPORTED;
   const bool f16p = L.dtype == TQ_F16;
@@ -1125,10 +1149,10 @@ int launch_decode_mfma(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv,
     if (f16p)                                                                                                   \
       return launch_one<D_, MB_, NX_, VB_, GS_, DS_, WPS_, true>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,  \
                                                                  bt_stride, seq_lens, sm_scale, ly, L, parts,     \
-                                                                 n_parts, n_split, len_sub, max_pages, num_pages, fz, fm, st); \
+                                                                 n_parts, n_split, len_sub, max_pages, num_pages, fz, fm, wide_wg, st); \
     return launch_one<D_, MB_, NX_, VB_, GS_, DS_, WPS_, false>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,   \
                                                                 bt_stride, seq_lens, sm_scale, ly, L, parts,      \
-                                                                n_parts, n_split, len_sub, max_pages, num_pages, fz, fm, st); \
+                                                                n_parts, n_split, len_sub, max_pages, num_pages, fz, fm, wide_wg, st); \
   }
   TQ_TRY(128, 2, 0, 2, 32, 1, 2) TQ_TRY(128, 2, 0, 4, 32, 1, 2) TQ_TRY(256, 2, 0, 2, 32, 2, 2) TQ_TRY(256, 2, 0, 4, 32, 2, 2)
   TQ_TRY(128, 1, 0, 2, 32, 1, 2) TQ_TRY(128, 1, 0, 4, 32, 1, 2) TQ_TRY(256, 1, 0, 2, 32, 2, 2) TQ_TRY(256, 1, 0, 4, 32, 2, 2)
