@@ -336,8 +336,8 @@ void tq_time_next_key_kernel(void *start_event, void *stop_event);
  *                      of the contraction idle (the kernel of more than 4 heads per KV head).
  *   "narrow_rows"      1 (default): head_dim 128 / 256 with at most 4 query heads per KV head puts the four fp6
  *                      terms of a head into one score operand (one matrix instruction per plane word); 0: two.
- *   "wide_workgroups"  1 (default): with at most 4 query heads per KV head (head_dim 64 / 128) and at most 16 blocks of
- *                      64 tokens per wavefront (judged by the width of the block table), a step runs workgroups of 8
+ *   "wide_workgroups"  1 (default): at head_dim 64 / 128, with an even split count and at most 16 blocks of 64 tokens
+ *                      per wavefront (judged by the width of the block table), a step runs workgroups of 8
  *                      wavefronts on half the split count it was given; 0: always 4 wavefronts per workgroup.
  *   "lds_stage"        1 (default): the 4-bit-key kernels of head_dim 128 / 256 bring the next block's page data
  *                      into LDS with LDS-direct loads instead of holding it in registers; 0: registers (spills).

@@ -536,9 +536,10 @@ def test_four_fp6_terms_in_one_operand(gpu, d, key_bits, vb, Hq, Hkv, dtype):
 
 
 @pytest.mark.parametrize("d,key_bits,vb,Hq,Hkv,dtype", [(128, 3, 4, 8, 2, torch.bfloat16), (64, 3, 2, 3, 1, torch.float16),
-                                                         (128, 4, 2, 4, 2, torch.bfloat16), (64, 2, 4, 8, 2, torch.bfloat16)])
+                                                         (128, 4, 2, 4, 2, torch.bfloat16), (64, 2, 4, 8, 2, torch.bfloat16),
+                                                         (128, 3, 2, 16, 2, torch.bfloat16), (64, 4, 4, 7, 1, torch.float16)])
 def test_eight_wavefronts_per_workgroup_on_half_the_splits(gpu, d, key_bits, vb, Hq, Hkv, dtype):
-    """Short contexts with at most four query heads per KV head run workgroups of eight wavefronts on half the
+    """Short contexts at head_dim 64 / 128 run workgroups of eight wavefronts on half the
     split count they were given (option "wide_workgroups"; even split counts only): another partition of the same
     tokens, so the result agrees with the four-wavefront kernel to rounding and with the oracle to the usual
     gate - ragged ends, table entries outside the pool and the in-launch merge included.  (The two partitions

@@ -1090,8 +1090,8 @@ static int launch_one(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, 
     return launch_one<D, MB, NX, VB, GS, DS, WPS, F16P, PP, NR, can_stage>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,
                                                                            bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts,
                                                                            n_split, len_sub, max_pages, num_pages, fz, fm, wide_wg, st);
-  // eight wavefronts per workgroup (one workgroup per compute unit) for the kernels of at most four query heads
-  constexpr bool can_widen = DS == 1 && (PP || NR) && NW == MF_WAVES;
+  // eight wavefronts per workgroup (one workgroup per compute unit) for the kernels whose wavefronts work alone
+  constexpr bool can_widen = DS == 1 && NW == MF_WAVES;
   if (can_widen && wide_wg)
     return launch_one<D, MB, NX, VB, GS, DS, WPS, F16P, PP, NR, SG, can_widen ? 2 * MF_WAVES : NW>(
         qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table, bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts, n_split,
@@ -1118,12 +1118,10 @@ static int launch_one(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, 
 // Whether a step of this shape should run workgroups of eight wavefronts (the caller then halves its split
 // count: the launch keeps its number of wavefronts).  Taken when a wavefront would walk at most 16 blocks of
 // the longest sequence the block table can hold: 16 x 8192 tokens at 32 q / 8 KV heads 39.7 -> 38.2 us per
-// step, but 32 x 32768 (64 blocks per wavefront) 212 -> 216 us.
+// step, at 64 q / 8 KV heads 42.9 -> 40.5 us, but 32 x 32768 (64 blocks per wavefront) 212 -> 216 us.
 bool decode_mfma_wide_workgroups(int d, int G, int n_split, int max_pages) {
-  if (!(d == 64 || d == 128) || G > 4 || n_split < 2 || (n_split & 1)) return false;
+  if (!(d == 64 || d == 128) || G > 8 || n_split < 2 || (n_split & 1)) return false;
   if (opt_wide_workgroups.load(std::memory_order_relaxed) == 0) return false;
-  if (d == 64 ? opt_page_pairs.load(std::memory_order_relaxed) == 0 : opt_narrow_rows.load(std::memory_order_relaxed) == 0)
-    return false;
   const int64_t blocks = ((int64_t)max_pages * TQ_PAGE_TOKENS + BLK_TOK - 1) / BLK_TOK;
   return blocks <= (int64_t)16 * MF_WAVES * n_split;
 }
