@@ -13,7 +13,9 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libtq_hip.so")
-SOURCES = ["tq_quantize.hip", "tq_quantize_mfma.hip", "tq_score.hip", "tq_decode.hip", "tq_decode_mfma.hip", "tq_probe.hip"]
+# (the matrix-core page kernel is instantiated by one file per head size, so that they compile side by side)
+SOURCES = ["tq_decode_mfma_d128.hip", "tq_decode_mfma_d64.hip", "tq_decode_mfma_d256.hip", "tq_quantize_mfma.hip",
+           "tq_quantize.hip", "tq_score.hip", "tq_decode.hip", "tq_decode_mfma.hip", "tq_probe.hip"]
 
 # packed-fp32 instructions stay off: some of their forms have produced wrong
 # results on this hardware pool
@@ -24,6 +26,8 @@ FLAGS = [
     # the kernels call fmaf() explicitly wherever a fused multiply-add is wanted
     "-ffp-contract=off",
     "-fno-gpu-rdc", "-Wall", "-Wno-unused-function",
+    # the LDS-direct loads name m0 in their clobber lists, which the compiler reports as a reserved register
+    "-Wno-inline-asm",
 ]
 
 
