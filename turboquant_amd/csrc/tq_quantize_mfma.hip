@@ -584,49 +584,55 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
     if constexpr (FX) {
       // lane (n, kb) feeds plane word kb of vector 16 m + n: coordinate c of the word sits at contraction
       // index 32 kb + 8 (c % 4) + c / 4 with the fp4 value 0.5, 1, 2, 0.5 (the matrix digits carry the inverse)
+      // (the first plane's sum starts from the constant term: no separate initialisation of the accumulators)
+      auto plane = [&](int p, f32x4 (&part)[MT][NPW]) {
+        u32x4 b[MT];
 #pragma unroll
-      for (int m = 0; m < MT; ++m)
+        for (int m = 0; m < MT; ++m) {
+          const uint32_t w = spl[(p * TT + 16 * m + n) * W + kb];
+          b[m] = u32x4{w & 0x11111111u, w & 0x22222222u, w & 0x44444444u, (w >> 3) & 0x11111111u};
 #pragma unroll
-        for (int c = 0; c < NPW; ++c) acc[m][c] = fconst[c];
+          for (int c = 0; c < NPW; ++c) part[m][c] = f32x4{0, 0, 0, 0};
+        }
+        // digit by digit over all tiles: consecutive MFMAs go to different accumulators
 #pragma unroll
-      for (int p = 0; p < 2; ++p) {
-        if (p < mb) {
-          u32x4 b[MT];
-          f32x4 part[MT][NPW];
+        for (int m = 0; m < MT; ++m)
 #pragma unroll
-          for (int m = 0; m < MT; ++m) {
-            const uint32_t w = spl[(p * TT + 16 * m + n) * W + kb];
-            b[m] = u32x4{w & 0x11111111u, w & 0x22222222u, w & 0x44444444u, (w >> 3) & 0x11111111u};
+          for (int c = 0; c < NPW; ++c) part[m][c] = mfma_fp6_fp4<0>(fa[c][0], b[m], part[m][c], fs0[c], 127);
 #pragma unroll
-            for (int c = 0; c < NPW; ++c) part[m][c] = f32x4{0, 0, 0, 0};
-          }
-          // digit by digit over all tiles: consecutive MFMAs go to different accumulators
+        for (int m = 0; m < MT; ++m)
 #pragma unroll
-          for (int m = 0; m < MT; ++m)
+          for (int c = 0; c < NPW; ++c) part[m][c] = mfma_fp6_fp4<1>(fa[c][1], b[m], part[m][c], fs0[c], 127);
 #pragma unroll
-            for (int c = 0; c < NPW; ++c) part[m][c] = mfma_fp6_fp4<0>(fa[c][0], b[m], part[m][c], fs0[c], 127);
+        for (int m = 0; m < MT; ++m)
 #pragma unroll
-          for (int m = 0; m < MT; ++m)
+          for (int c = 0; c < NPW; ++c) part[m][c] = mfma_fp6_fp4<2>(fa[c][2], b[m], part[m][c], fs0[c], 127);
 #pragma unroll
-            for (int c = 0; c < NPW; ++c) part[m][c] = mfma_fp6_fp4<1>(fa[c][1], b[m], part[m][c], fs0[c], 127);
+        for (int m = 0; m < MT; ++m)
 #pragma unroll
-          for (int m = 0; m < MT; ++m)
+          for (int c = 0; c < NPW; ++c) part[m][c] = mfma_fp6_fp4<3>(fa[c][3], b[m], part[m][c], fs0[c], 127);
 #pragma unroll
-            for (int c = 0; c < NPW; ++c) part[m][c] = mfma_fp6_fp4<2>(fa[c][2], b[m], part[m][c], fs0[c], 127);
+        for (int m = 0; m < MT; ++m)
 #pragma unroll
-          for (int m = 0; m < MT; ++m)
+          for (int c = 0; c < NPW; ++c) part[m][c] = mfma_fp6_fp4<0>(fa[c][4], b[m], part[m][c], fs1[c], 127);
+      };
+      {
+        f32x4 part[MT][NPW];
+        plane(0, part);
 #pragma unroll
-            for (int c = 0; c < NPW; ++c) part[m][c] = mfma_fp6_fp4<3>(fa[c][3], b[m], part[m][c], fs0[c], 127);
+        for (int m = 0; m < MT; ++m)
 #pragma unroll
-          for (int m = 0; m < MT; ++m)
+          for (int c = 0; c < NPW; ++c)
 #pragma unroll
-            for (int c = 0; c < NPW; ++c) part[m][c] = mfma_fp6_fp4<0>(fa[c][4], b[m], part[m][c], fs1[c], 127);
+            for (int i = 0; i < 4; ++i) acc[m][c][i] = fmaf(fk[0], part[m][c][i], fconst[c][i]);
+        if (mb == 2) {
+          plane(1, part);
 #pragma unroll
           for (int m = 0; m < MT; ++m)
 #pragma unroll
             for (int c = 0; c < NPW; ++c)
 #pragma unroll
-              for (int i = 0; i < 4; ++i) acc[m][c][i] = fmaf(fk[p], part[m][c][i], acc[m][c][i]);
+              for (int i = 0; i < 4; ++i) acc[m][c][i] = fmaf(fk[1], part[m][c][i], acc[m][c][i]);
         }
       }
       prefetch_matrix<D>(ly.S_split, wave, lane, mr);
