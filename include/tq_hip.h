@@ -339,6 +339,10 @@ void tq_time_next_key_kernel(void *start_event, void *stop_event);
  *   "wide_workgroups"  1 (default): at head_dim 64 / 128, with an even split count and at most 16 blocks of 64 tokens
  *                      per wavefront (judged by the width of the block table), a step runs workgroups of 8
  *                      wavefronts on half the split count it was given; 0: always 4 wavefronts per workgroup.
+ *   "split_skew"       0..8, default 1: at head_dim 256, when a launch of 4-wavefront workgroups fills (nearly) every
+ *                      compute unit twice and the split count is even, the workgroups of the first half of the grid
+ *                      (dispatched first, served first by their SIMDs) take the even splits and this many sixteenths
+ *                      of a split's trips over from the odd splits of the second half; 0: equal shares.
  *   "lds_stage"        1 (default): the 4-bit-key kernels of head_dim 128 / 256 bring the next block's page data
  *                      into LDS with LDS-direct loads instead of holding it in registers; 0: registers (spills).
  *   "fp6_centroids"    1 (default): the key quantiser takes the fp6 x fp4 centroid contraction when the layer

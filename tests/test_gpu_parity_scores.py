@@ -548,6 +548,51 @@ def test_eight_wavefronts_per_workgroup_on_half_the_splits(gpu, d, key_bits, vb,
     _variant_against_default(gpu, "wide_workgroups", d, key_bits, vb, Hq, Hkv, dtype, exact=False, rel=2.0 ** -8)
 
 
+@pytest.mark.parametrize("key_bits,vb,Hq,Hkv,n_split", [(3, 2, 16, 2, 64), (4, 4, 4, 2, 60), (2, 2, 8, 2, 62)])
+def test_unequal_shares_for_the_two_workgroups_of_a_compute_unit(gpu, key_bits, vb, Hq, Hkv, n_split):
+    """Head_dim 256 with a launch that fills the compute units twice (here 480 - 512 workgroups on 256 units): the
+    workgroups of the first half of the grid take the even splits and a part of their odd neighbours' trips (option
+    "split_skew", in sixteenths; 8 moves half of them, which with one or two trips per split leaves odd splits empty).
+    Another partition of the same tokens: the result agrees with equal shares to rounding (one unit in the last place
+    of a 16-bit output) and with the oracle (score.py:84-173) to the usual gate - ragged ends, a sequence shorter than
+    the split count, and table entries outside the pool included."""
+    d, B, dtype = 256, 4, torch.bfloat16
+    lens = [64 * 130 + 5, 17, 64 * 64, 64 * 301 + 33]
+    n_log = max((n + 15) // 16 for n in lens)
+    n_pages = B * n_log + 1
+    pool, tq = _make_pool(gpu, d, key_bits, vb, Hkv, n_pages, dtype, seed=78)
+    g = torch.Generator().manual_seed(911 + key_bits)
+    k = torch.randn(B, max(lens), Hkv, d, generator=g).to(dtype)
+    v = torch.randn(B, max(lens), Hkv, d, generator=g).to(dtype)
+    q = torch.randn(B, Hq, d, generator=g).to(dtype)
+    table = torch.randperm(n_pages, generator=g)[: B * n_log].to(torch.int32).view(B, n_log)
+    pool.append(k.to(gpu), v.to(gpu), table.to(gpu))
+    seq = torch.tensor(lens, dtype=torch.int32, device=gpu)
+    bad = table.clone()
+    bad[0, [4, 7, 200, 201]] = torch.tensor([n_pages, -1, 2 ** 31 - 1, -9], dtype=torch.int32)
+    prm = params_of(tq)
+    _progress(f"split_skew kb={key_bits} vb={vb} Hq={Hq} Hkv={Hkv} n_split={n_split}")
+    try:
+        for tab in (table, bad):
+            outs = {}
+            for skew in (0, 1, 3, 8):
+                _set_option("split_skew", skew)
+                outs[skew] = pool.decode_attention(q.to(gpu), tab.to(gpu), seq, n_split=n_split, max_len=max(lens)).cpu()
+            torch.cuda.synchronize()
+            tol = 2.0 ** -8 * float(outs[0].float().abs().max()) + 1e-6
+            for skew in (1, 3, 8):
+                assert float((outs[skew].float() - outs[0].float()).abs().max()) <= tol, (skew, tab is bad)
+            if tab is table:
+                for skew in (1, 8):
+                    for b in range(B):
+                        idx, sgn, norms, rn, vd, vs, vz = [t.cpu() for t in pool.export_flat(table[b], lens[b])]
+                        want = O.hybrid_attention(q[b:b + 1], key_code(idx, sgn, rn, norms, key_bits - 1),
+                                                  value_code(vd, vs, vz, vb), lens[b], prm, Hkv, None, None)
+                        assert cosine(outs[skew][b:b + 1], want) >= COS_GATE, (skew, b)
+    finally:
+        _set_option("split_skew", 1)
+
+
 @pytest.mark.parametrize("d,vb,Hq,Hkv,dtype", [(128, 4, 16, 2, torch.bfloat16), (128, 2, 4, 1, torch.float16),
                                                (256, 2, 16, 2, torch.bfloat16), (256, 4, 6, 2, torch.bfloat16)])
 def test_four_bit_keys_staged_through_lds(gpu, d, vb, Hq, Hkv, dtype):

@@ -942,6 +942,7 @@ std::atomic<int> opt_page_pairs{1};
 std::atomic<int> opt_narrow_rows{1};
 std::atomic<int> opt_lds_stage{1};
 std::atomic<int> opt_wide_workgroups{1};
+std::atomic<int> opt_split_skew{1};
 }  // namespace tq
 
 namespace {
@@ -973,6 +974,11 @@ extern "C" int tq_set_option(const char* name, int64_t value) {
     return TQ_OK;
   }
   if (!std::strcmp(name, "wide_workgroups")) { opt_wide_workgroups.store(value != 0); return TQ_OK; }
+  if (!std::strcmp(name, "split_skew")) {
+    if (value < 0 || value > 8) return TQ_EINVAL;
+    opt_split_skew.store((int)value);
+    return TQ_OK;
+  }
   if (!std::strcmp(name, "lds_stage")) { opt_lds_stage.store(value != 0); return TQ_OK; }
   if (!std::strcmp(name, "narrow_rows")) { opt_narrow_rows.store(value != 0); return TQ_OK; }
   if (!std::strcmp(name, "page_pairs")) { opt_page_pairs.store(value != 0); return TQ_OK; }

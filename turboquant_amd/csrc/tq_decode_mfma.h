@@ -52,4 +52,8 @@ int launch_decode_mfma(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv,
 // (and wide_wg = true) to launch_decode_mfma and uses that count for everything that follows.
 bool decode_mfma_wide_workgroups(int d, int G, int n_split, int max_pages);
 
+// Sixteenths of a split that every even split takes over from its odd neighbour (0: equal shares), for a launch of
+// n_split x rows workgroups of four wavefronts that sit two to a compute unit.
+int decode_mfma_split_skew(int n_split, int rows);
+
 }  // namespace tq

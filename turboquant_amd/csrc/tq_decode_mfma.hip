@@ -43,6 +43,25 @@ bool decode_mfma_wide_workgroups(int d, int G, int n_split, int max_pages) {
   return blocks <= (int64_t)16 * MF_WAVES * n_split;
 }
 
+// Unequal shares for the two workgroups of a compute unit.  Workgroups are dispatched in grid order and spread
+// over the compute units, so when the launch fills (nearly) every compute unit twice, the first half of the grid
+// holds the older workgroup of every unit; a SIMD serves its older wavefronts first, and with equal shares those
+// finish about a tenth of the kernel's time before the younger ones.  4 x 131072 tokens, 16 q / 2 KV heads,
+// head_dim 256 (512 workgroups of 16 trips): one trip moved.  If the dispatch order were another one the shares
+// would merely be as unequal as they are unlucky: results do not depend on it.
+int decode_mfma_split_skew(int n_split, int rows) {
+  const int skew = opt_split_skew.load(std::memory_order_relaxed);
+  if (skew <= 0 || n_split < 2 || (n_split & 1)) return 0;
+  static const int units = [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) n = 0;
+    return n;
+  }();
+  const int64_t groups = (int64_t)n_split * rows;
+  return units > 0 && groups <= 2 * (int64_t)units && groups * 16 >= 30 * (int64_t)units ? skew : 0;
+}
+
 // words of packed query operands tq_decode_attn_paged reserves in its workspace
 size_t decode_mfma_pack_words(int B, int Hq, int d) { return (size_t)B * Hq * 9 * (d / 128 + 1) * 1024; }   // d = 64: one chunk
 

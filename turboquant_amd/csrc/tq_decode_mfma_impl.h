@@ -230,7 +230,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
                    const uint8_t* __restrict__ pool, const int32_t* __restrict__ block_table,
                    int bt_stride, const int32_t* __restrict__ seq_lens, float sm_scale, tq_layer ly, tq_page_layout L,
                    float* __restrict__ parts, int n_parts, int n_split, int len_sub, int max_pages, int num_pages,
-                   FusedPrep fz, FusedMerge fm) {
+                   int skew16, FusedPrep fz, FusedMerge fm) {
   constexpr int DW = D / DS;                  // coordinates / channels of one wavefront
   constexpr int WPLT = (D + 127) / 128;       // plane words per lane per plane per page, all wavefronts
   constexpr int WPL = (DW + 127) / 128;       // ... of one wavefront (head_dim 64: one, with half of the lanes idle)
@@ -256,7 +256,18 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   // Hkv counts query-head groups: a KV head with more than 8 query heads is served by kv_div groups
   // of G <= 8 heads each (consecutive groups read the same pages)
   const int G = Hq / Hkv;
-  const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  // skew16 > 0 (an even number of splits; the grid is (n_split / 2, Hkv, 2 B)): the workgroups of the first half
+  // of the grid take the even splits, those of the second half the odd ones, and every even split takes
+  // skew16 sixteenths of a split's trips over from its odd neighbour.  Workgroups are dispatched in grid order, two
+  // to a compute unit, and a SIMD serves its older wavefronts first: with equal shares the first half of the grid
+  // finishes early and the second half runs on alone.
+  int split = blockIdx.x, b = blockIdx.z;
+  const int h = blockIdx.y;
+  if (skew16 > 0) {
+    const int seqs = (int)gridDim.z >> 1, late = b >= seqs;
+    b -= late ? seqs : 0;
+    split = 2 * split + late;
+  }
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wgrp = wave / DS, hf = wave % DS; // block walker this wavefront belongs to; its share of the head
@@ -412,8 +423,13 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   const int n_pages = (seq_len + TQ_PAGE_TOKENS - 1) / TQ_PAGE_TOKENS;
   const int n_blocks = (seq_len + BLK_TOK - 1) / BLK_TOK;
   const int per_split = (n_blocks + n_split - 1) / n_split;
-  const int blk_begin = split * per_split;
-  const int blk_end = min(n_blocks, blk_begin + per_split);
+  int blk_begin = split * per_split;
+  int blk_end = min(n_blocks, blk_begin + per_split);
+  if (skew16 > 0) {
+    const int moved = min(NGRP * ((((per_split + NGRP - 1) / NGRP) * skew16 + 8) >> 4), per_split);
+    if (split & 1) blk_begin = min(blk_begin + moved, blk_end);
+    else blk_end = min(blk_end + moved, n_blocks);
+  }
   const int32_t* bt = block_table + (int64_t)b * bt_stride;
   const uint8_t* pool_h = pool + (int64_t)(h / kv_div) * L.page_bytes;
   const int64_t page_stride = (int64_t)(Hkv / kv_div) * L.page_bytes;
@@ -1086,6 +1102,12 @@ static int launch_one(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, 
     return launch_one<D, MB, NX, VB, GS, DS, WPS, F16P, PP, NR, SG, can_widen ? 2 * MF_WAVES : NW>(
         qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table, bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts, n_split,
         len_sub, max_pages, num_pages, fz, fm, false, st);
+  // two workgroups of four wavefronts share a compute unit: see the kernel's comment on skew16.  Only the
+  // head_dim 256 kernels, which are bound by instruction issue, gain (4 x 131072: 46.4 -> 45.5 us); the head_dim 128
+  // kernels wait for memory, their workgroups advance side by side whatever their age, and unequal shares cost
+  // what they move (32 x 32768: 203 -> 208 us).
+  const int skew16 = NW == MF_WAVES && WPS == 2 && DS == 2 ? decode_mfma_split_skew(n_split, Hkv * B) : 0;
+  const dim3 grid = skew16 > 0 ? dim3(n_split / 2, Hkv, 2 * B) : dim3(n_split, Hkv, B);
   auto kern = decode_mfma_kernel<D, MB, NX, VB, GS, DS, WPS, F16P, PP, NR, SG, NW>;
   if (smem > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
@@ -1093,13 +1115,13 @@ static int launch_one(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, 
   }
   hipEvent_t t_start_event = nullptr, t_stop_event = nullptr;
   if (take_time_hook(0, t_start_event, t_stop_event)) {
-    hipExtLaunchKernelGGL(kern, dim3(n_split, Hkv, B), dim3(NW * 64), smem, st, t_start_event, t_stop_event, 0,
+    hipExtLaunchKernelGGL(kern, grid, dim3(NW * 64), smem, st, t_start_event, t_stop_event, 0,
                           qa_pack, q_stat, Hq, Hkv, kv_div, pool, block_table, bt_stride, seq_lens, sm_scale, ly, L, parts,
-                          n_parts, n_split, len_sub, max_pages, num_pages, fz, fm);
+                          n_parts, n_split, len_sub, max_pages, num_pages, skew16, fz, fm);
   } else {
-    kern<<<dim3(n_split, Hkv, B), dim3(NW * 64), smem, st>>>(qa_pack, q_stat, Hq, Hkv, kv_div, pool, block_table,
-                                                                   bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts,
-                                                                   n_split, len_sub, max_pages, num_pages, fz, fm);
+    kern<<<grid, dim3(NW * 64), smem, st>>>(qa_pack, q_stat, Hq, Hkv, kv_div, pool, block_table, bt_stride, seq_lens,
+                                            sm_scale, ly, L, parts, n_parts, n_split, len_sub, max_pages, num_pages, skew16,
+                                            fz, fm);
   }
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? TQ_OK : (int)e;

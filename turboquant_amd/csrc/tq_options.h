@@ -13,5 +13,6 @@ extern std::atomic<int> opt_page_pairs;        // decode, head_dim 64 with at mo
 extern std::atomic<int> opt_narrow_rows;       // decode, head_dim 128 / 256 with at most 4 query heads per KV head: one score MFMA per plane word
 extern std::atomic<int> opt_lds_stage;         // decode: page data through LDS-direct loads, a whole trip ahead
 extern std::atomic<int> opt_wide_workgroups;   // decode, head_dim 64 / 128, short contexts: workgroups of 8 wavefronts
+extern std::atomic<int> opt_split_skew;        // decode, two workgroups per compute unit: sixteenths of a split moved to the workgroup dispatched first (0: none)
 extern std::atomic<int> opt_merge_in_kernel;    // decode: few context splits are merged by the last workgroup of the page kernel
 }  // namespace tq
