@@ -343,6 +343,8 @@ void tq_time_next_key_kernel(void *start_event, void *stop_event);
  *                      compute unit twice and the split count is even, the workgroups of the first half of the grid
  *                      (dispatched first, served first by their SIMDs) take the even splits and this many sixteenths
  *                      of a split's trips over from the odd splits of the second half; 0: equal shares.
+ *   "merge_row_groups" 1 (default): the merge kernel gives a row of partials to 2 or 4 workgroups (a share of the
+ *                      channels each) when there are fewer rows than compute units; 0: one workgroup per row.
  *   "lds_stage"        1 (default): the 4-bit-key kernels of head_dim 128 / 256 bring the next block's page data
  *                      into LDS with LDS-direct loads instead of holding it in registers; 0: registers (spills).
  *   "fp6_centroids"    1 (default): the key quantiser takes the fp6 x fp4 centroid contraction when the layer

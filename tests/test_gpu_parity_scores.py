@@ -603,6 +603,58 @@ def test_four_bit_keys_staged_through_lds(gpu, d, vb, Hq, Hkv, dtype):
     _variant_against_default(gpu, "lds_stage", d, 4, vb, Hq, Hkv, dtype, exact=True)
 
 
+@pytest.mark.parametrize("rows,n_parts,d,dtype", [(64, 64, 256, torch.bfloat16), (64, 65, 256, torch.float16),
+                                                  (3, 9, 256, torch.float32), (100, 33, 128, torch.bfloat16),
+                                                  (7, 5, 128, torch.float32), (129, 17, 128, torch.float16),
+                                                  (5, 40, 64, torch.bfloat16), (2, 19, 576, torch.float32),
+                                                  (300, 3, 256, torch.bfloat16), (1, 1, 128, torch.float32)])
+def test_merge_of_split_partials(gpu, rows, n_parts, d, dtype):
+    """tq_decode_merge on its own: the log-sum-exp merge of per-split partials (m, l, acc[d]) - the segments of
+    score.py:84-173 - against a float64 computation of the same formula, with empty parts (l = 0, which carry no
+    weight whatever their m says), maxima of very different size, and row counts on both sides of what makes the
+    kernel give a row to several workgroups (option "merge_row_groups": both settings are run and must agree)."""
+    from turboquant_amd import _ffi
+    g = torch.Generator().manual_seed(rows * 1000 + n_parts * 10 + d)
+    parts = torch.empty(rows, n_parts, d + 2, dtype=torch.float32)
+    parts[..., 0] = torch.randn(rows, n_parts, generator=g) * 20.0                       # m
+    parts[..., 1] = torch.rand(rows, n_parts, generator=g) * 50.0 + 0.5                  # l
+    parts[..., 2:] = torch.randn(rows, n_parts, d, generator=g) * parts[..., 1:2]        # acc
+    empty = torch.rand(rows, n_parts, generator=g) < 0.2
+    empty[0, :] = n_parts > 1                                                            # a row without any token
+    empty[0, 0] = False
+    if rows > 1:
+        empty[1, :] = True                                                               # ... and one that is all empty
+    parts[..., 1][empty] = 0.0
+    parts[..., 2:][empty] = 0.0
+    parts[..., 0][empty] = 1e30                                                          # must not count
+    p64 = parts.double()
+    live = p64[..., 1] > 0
+    m = torch.where(live, p64[..., 0], torch.full_like(p64[..., 0], -1e300))
+    M = m.max(dim=1, keepdim=True).values
+    w = torch.where(live, torch.exp(m - M), torch.zeros_like(m))
+    den = (w * p64[..., 1]).sum(dim=1, keepdim=True)
+    want = torch.where(den > 0, (w[..., None] * p64[..., 2:]).sum(dim=1) / den.clamp_min(1e-300), torch.zeros(rows, d, dtype=torch.float64))
+    dt = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dtype]
+    dev_parts = parts.to(gpu)
+    outs = []
+    _progress(f"merge rows={rows} n_parts={n_parts} d={d} {dtype}")
+    try:
+        for on in (1, 0):
+            _set_option("merge_row_groups", on)
+            out = torch.full((rows, d), float("nan"), dtype=dtype, device=gpu)
+            _ffi.check(_ffi.lib().tq_decode_merge(dev_parts.data_ptr(), rows, n_parts, d, dt, out.data_ptr(),
+                                                  torch.cuda.current_stream().cuda_stream), "tq_decode_merge")
+            torch.cuda.synchronize()
+            outs.append(out.cpu())
+    finally:
+        _set_option("merge_row_groups", 1)
+    eps = {torch.float32: 2.0 ** -20, torch.float16: 2.0 ** -10, torch.bfloat16: 2.0 ** -7}[dtype]
+    for out in outs:
+        err = (out.double() - want).abs()
+        assert bool((err <= eps * want.abs() + 1e-5).all()), float(err.max())
+    assert float((outs[0].double() - outs[1].double()).abs().max()) <= 2 * eps * float(want.abs().max())
+
+
 @pytest.mark.parametrize("d,key_bits,vb,Hq,Hkv,lens,n_split", [
     (128, 3, 4, 32, 8, [900, 1, 16, 0, 517], 4),
     (128, 3, 2, 8, 1, [2100], 8),
