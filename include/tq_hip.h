@@ -287,7 +287,7 @@ int tq_decode_attn_paged_ring(const void *q, int dtype, int B, int Hq, int Hkv, 
  * workspace: partials, rotated queries and query operands live in a file-scope device array of
  * TQ_NOALLOC_SCRATCH_BYTES inside the library (one copy per GPU, held until the process ends; its address is
  * looked up with hipGetSymbolAddress the first time a device is used).  The call allocates nothing and
- * frees nothing.  A call that needs more than the array holds - roughly 4*B*Hq*(n_split+1)*(d+2) bytes of
+ * frees nothing.  A call that needs more than the array holds - roughly 4*B*Hq*(n_split+4)*(d+2) bytes of
  * partials plus 8*B*Hq*d - returns TQ_ETOOBIG and launches nothing.  All calls on one GPU share the array:
  * calls that overlap on one GPU (different streams or threads) race; serialise them or use the workspace form. */
 #define TQ_NOALLOC_SCRATCH_BYTES (16u << 20)
@@ -343,6 +343,9 @@ void tq_time_next_key_kernel(void *start_event, void *stop_event);
  *                      compute unit twice and the split count is even, the workgroups of the first half of the grid
  *                      (dispatched first, served first by their SIMDs) take the even splits and this many sixteenths
  *                      of a split's trips over from the odd splits of the second half; 0: equal shares.
+ *   "tail_chunks"      1 (default): a hybrid step with more than 8 context splits and few (sequence, KV head)
+ *                      pairs lets 2 or 4 workgroups share the exact tokens of a group of query heads, each with
+ *                      a partial of its own for the merge kernel; 0: one workgroup and one partial.
  *   "merge_row_groups" 1 (default): the merge kernel gives a row of partials to 2 or 4 workgroups (a share of the
  *                      channels each) when there are fewer rows than compute units; 0: one workgroup per row.
  *   "lds_stage"        1 (default): the 4-bit-key kernels of head_dim 128 / 256 bring the next block's page data

@@ -451,7 +451,7 @@ def _store_from_oracle_view(pool, table_row, n_tok):
 
 
 def _decode_case(gpu, d, key_bits, vb, B, Hq, Hkv, lens, recent, seed, n_split=None, dtype=torch.bfloat16,
-                 shape_kq=None, recent_pad=0):
+                 shape_kq=None, recent_pad=0, return_out=False):
     g = torch.Generator().manual_seed(seed)
     max_len = max(max(lens), 1)
     pages_per_seq = (max_len + 15) // 16
@@ -501,7 +501,7 @@ def _decode_case(gpu, d, key_bits, vb, B, Hq, Hkv, lens, recent, seed, n_split=N
         worst = min(worst, c)
         assert c >= COS_GATE, (b, c)
         assert (got.float() - want.float()).abs().max() <= 2 ** -7 * want.float().abs().max() + 1e-3, b
-    return worst
+    return out.cpu() if return_out else worst
 
 
 @pytest.mark.parametrize("d,key_bits,vb,Hq,Hkv", [(128, 3, 4, 8, 2), (256, 3, 2, 16, 2), (128, 3, 2, 4, 4),
@@ -623,6 +623,35 @@ def test_exact_tail_shapes(gpu, d, dtype, Hq, Hkv, recent, pad):
     _progress(f"exact tail d={d} {dtype} Hq={Hq} Hkv={Hkv} recent={recent} pad={pad}")
     worst = _decode_case(gpu, d, 3, 2, 3, Hq, Hkv, [100, 0, 33], recent, seed=300 + d + pad, dtype=dtype, recent_pad=pad)
     _progress(f"  worst cosine {worst:.7f}")
+
+
+@pytest.mark.parametrize("d,dtype,Hq,Hkv,recent,n_split,pad", [
+    (256, torch.bfloat16, 16, 2, [128, 3, 0], 12, 0),      # four workgroups per head group; shares of 32, of 0 / 1 tokens, of none
+    (128, torch.float16, 8, 1, [300, 77, 1], 9, 8),        # several load rounds per share, rows inside a wider buffer
+    (128, torch.float32, 4, 4, [64, 33, 2], 16, 0),        # 64 rows: two workgroups
+    (64, torch.bfloat16, 3, 1, [130, 5, 129], 11, 6),      # 4-byte loads
+    (576, torch.float32, 4, 1, [40, 17, 33], 10, 0),       # a head size of the general page kernel
+])
+def test_exact_tail_shared_by_several_workgroups(gpu, d, dtype, Hq, Hkv, recent, n_split, pad):
+    """A hybrid step (score.py:99-173) with more than eight context splits and few (sequence, KV head) pairs gives
+    the exact tokens of a group of query heads to 2 or 4 workgroups, a share of the tokens and a partial each
+    (option "tail_chunks"): against the oracle, and against the one-workgroup tail to rounding."""
+    from turboquant_amd import _ffi
+
+    def _set_option(name, value):
+        _ffi.check(_ffi.lib().tq_set_option(name.encode(), int(value)), "tq_set_option")
+
+    _progress(f"shared exact tail d={d} {dtype} Hq={Hq} Hkv={Hkv} recent={recent} n_split={n_split} pad={pad}")
+    outs = []
+    try:
+        for on in (1, 0):
+            _set_option("tail_chunks", on)
+            outs.append(_decode_case(gpu, d, 3, 2, 3, Hq, Hkv, [400, 0, 33], recent, seed=500 + d + pad, dtype=dtype,
+                                     recent_pad=pad, n_split=n_split, return_out=True))
+    finally:
+        _set_option("tail_chunks", 1)
+    eps = 2.0 ** -20 if dtype == torch.float32 else 2.0 ** -8
+    assert float((outs[0].float() - outs[1].float()).abs().max()) <= eps * float(outs[1].float().abs().max()) + 1e-6
 
 
 @pytest.mark.parametrize("d,key_bits,vb,dtype", [(128, 3, 4, torch.bfloat16), (256, 3, 2, torch.bfloat16),
@@ -984,9 +1013,11 @@ def test_stream_read_probe_runs_and_rejects_bad_arguments(gpu):
     assert lib.tq_stream_read(buf.data_ptr(), 16, 0, 4, None, st) < 0
 
 
-@pytest.mark.parametrize("d,dtype,Hq,Hkv,ring", [(128, torch.bfloat16, 16, 4, 128), (256, torch.bfloat16, 16, 2, 128),
-                                                   (64, torch.float16, 8, 2, 200), (128, torch.float32, 4, 2, 48)])
-def test_ring_entry_reads_the_exact_cache_in_place(gpu, d, dtype, Hq, Hkv, ring):
+@pytest.mark.parametrize("d,dtype,Hq,Hkv,ring,n_split", [(128, torch.bfloat16, 16, 4, 128, None), (256, torch.bfloat16, 16, 2, 128, None),
+                                                           (64, torch.float16, 8, 2, 200, None), (128, torch.float32, 4, 2, 48, None),
+                                                           (256, torch.bfloat16, 16, 2, 128, 12),       # many splits: the exact tokens
+                                                           (128, torch.float16, 4, 1, 100, 9)])         # are shared by 2 / 4 workgroups
+def test_ring_entry_reads_the_exact_cache_in_place(gpu, d, dtype, Hq, Hkv, ring, n_split):
     """tq_decode_attn_paged_ring takes the exact recent tokens (score.py:99-111) straight from a paged exact
     cache through the block table; it must equal, bit for bit, gathering those rows with torch indexing and
     passing them as recent_k / recent_v with the history lengths reduced by their count."""
@@ -1012,7 +1043,7 @@ def test_ring_entry_reads_the_exact_cache_in_place(gpu, d, dtype, Hq, Hkv, ring)
         pool.append(k[b:b + 1, :n], v[b:b + 1, :n], table[b:b + 1])
     q = torch.randn(B, Hq, d, generator=g).to(dtype).to(gpu)
     _progress(f"ring entry d={d} {dtype} ring={ring} lens={lens}")
-    got = pool.decode_attention_ring(q, table, seq, cache[0], cache[1], ring, max_len=max(lens)).clone()
+    got = pool.decode_attention_ring(q, table, seq, cache[0], cache[1], ring, n_split=n_split, max_len=max(lens)).clone()
     # the same step with the rows gathered on the host side
     tail = torch.clamp(seq.long(), max=ring)
     pos = (seq.long() - tail)[:, None] + torch.arange(ring, device=gpu)[None]
@@ -1021,7 +1052,7 @@ def test_ring_entry_reads_the_exact_cache_in_place(gpu, d, dtype, Hq, Hkv, ring)
     rk = cache[0].reshape(-1, Hkv, d)[slot]
     rv = cache[1].reshape(-1, Hkv, d)[slot]
     want = pool.decode_attention(q, table, (seq.long() - tail).to(torch.int32), recent_k=rk, recent_v=rv,
-                                 recent_len=tail.to(torch.int32), max_len=max(lens))
+                                 recent_len=tail.to(torch.int32), n_split=n_split, max_len=max(lens))
     torch.cuda.synchronize()
     assert torch.equal(got, want)
     assert torch.count_nonzero(got[0]) == 0                         # the empty sequence

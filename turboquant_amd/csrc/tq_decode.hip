@@ -286,6 +286,7 @@ decode_pages_kernel(const float* __restrict__ q_rot, const float* __restrict__ q
 // a loop that waits for one row per iteration costs a memory latency per token).  Scores: eight threads per
 // token, each over every eighth coordinate for the group's heads at once; values: a thread per channel and
 // slice of the chunk's tokens.
+constexpr int TAIL_MAX_CHUNKS = 4;      // workgroups that may share the exact tokens of one (sequence, head group)
 constexpr int TAIL_THREADS = 512, TAIL_WAVES = TAIL_THREADS / 64, TAIL_GC = 4, TAIL_TILE_FLOATS = 64 * 260;
 
 static size_t tail_smem(int d, int recent_rows) {
@@ -497,10 +498,12 @@ struct TailArgs {
   float sm_scale;
   float* parts;
   int n_parts, part_index;
+  int t_chunks;                    // workgroups that share the exact tokens of a (sequence, head group); chunk c writes part part_index + c
 };
 
 // (a device function: the stand-alone kernel and the launch that shares its grid with the query
-// preparation both run it; h / b / gz are the workgroup's KV head, sequence and head group, `sm` its LDS)
+// preparation both run it; h / b are the workgroup's KV head and sequence, gz = head group + number of head
+// groups x token chunk, `sm` its LDS)
 template <int DT, int KC, bool PAGED, bool WIDE>
 __device__ __forceinline__ void exact_tail_words_body(const TailArgs& A, int h, int b, int gz, float* sm) {
   const void* __restrict__ q = A.q;
@@ -513,15 +516,19 @@ __device__ __forceinline__ void exact_tail_words_body(const TailArgs& A, int h, 
   const int32_t* __restrict__ seq_lens = A.seq_lens;
   const float sm_scale = A.sm_scale;
   float* __restrict__ parts = A.parts;
-  const int n_parts = A.n_parts, part_index = A.part_index;
+  const int n_parts = A.n_parts;
   constexpr int GC = TAIL_GC, EPW = TailWord<DT>::EPW, RPT = TAIL_RPT / KC;
-  const int G = Hq / Hkv, g0 = gz * GC, tid = threadIdx.x;
+  const int G = Hq / Hkv, tid = threadIdx.x;
+  const int n_gz = (G + GC - 1) / GC, chunk = gz / n_gz, g0 = (gz - chunk * n_gz) * GC;
+  const int part_index = A.part_index + chunk;
   const int Gc = min(GC, G - g0);
   const int lane = tid & 63, wave = tid >> 6;
   const int seq = PAGED ? min(seq_lens[b], A.max_pages * TQ_PAGE_TOKENS) : 0;     // cut to the block table
   const int num_blocks = A.num_blocks;
-  const int R = PAGED ? max(min(seq, recent_rows), 0) : (recent_len ? min(recent_len[b], recent_rows) : recent_rows);
-  const int first = PAGED ? seq - R : 0;            // position of the first exact token
+  const int R_all = PAGED ? max(min(seq, recent_rows), 0) : (recent_len ? min(recent_len[b], recent_rows) : recent_rows);
+  // this workgroup's share of the exact tokens (all of them with one chunk); it may be empty
+  const int r_lo = (int)((int64_t)R_all * chunk / A.t_chunks), R = (int)((int64_t)R_all * (chunk + 1) / A.t_chunks) - r_lo;
+  const int first = (PAGED ? seq - R_all : 0) + r_lo;   // position (row, when not paged) of the first exact token of the share
   const int32_t* bt = block_table + (PAGED ? (int64_t)b * bt_stride : 0);
   float* sq = sm;                                   // [d][GC]
   float* ss = sq + GC * d;                          // [recent_rows][GC] scores, then softmax weights
@@ -547,7 +554,7 @@ __device__ __forceinline__ void exact_tail_words_body(const TailArgs& A, int h, 
       const int raw = bt[p >> 4];                       // an entry outside the cache is read as block 0
       return base0 + (int64_t)((unsigned)raw < (unsigned)num_blocks ? raw : 0) * ws_blk + (int64_t)(p & 15) * ws_r;
     }
-    return base0 + (int64_t)row * ws_r;
+    return base0 + (int64_t)(first + row) * ws_r;
   };
   // loads of rows c0 + ts, c0 + ts + TS, ... of this thread's columns, all issued before anything waits
   // (n >= 1: callers skip empty chunks, so the clamped row exists)
@@ -957,6 +964,7 @@ std::atomic<int> opt_lds_stage{1};
 std::atomic<int> opt_wide_workgroups{1};
 std::atomic<int> opt_split_skew{1};
 std::atomic<int> opt_merge_row_groups{1};
+std::atomic<int> opt_tail_chunks{1};
 }  // namespace tq
 
 namespace {
@@ -993,6 +1001,7 @@ extern "C" int tq_set_option(const char* name, int64_t value) {
     opt_split_skew.store((int)value);
     return TQ_OK;
   }
+  if (!std::strcmp(name, "tail_chunks")) { opt_tail_chunks.store(value != 0); return TQ_OK; }
   if (!std::strcmp(name, "merge_row_groups")) { opt_merge_row_groups.store(value != 0); return TQ_OK; }
   if (!std::strcmp(name, "lds_stage")) { opt_lds_stage.store(value != 0); return TQ_OK; }
   if (!std::strcmp(name, "narrow_rows")) { opt_narrow_rows.store(value != 0); return TQ_OK; }
@@ -1009,9 +1018,9 @@ extern "C" int tq_set_option(const char* name, int64_t value) {
 
 extern "C" size_t tq_decode_workspace_bytes(int B, int Hq, int d, int n_split) {
   if (B <= 0 || Hq <= 0 || d <= 0 || n_split <= 0) return 0;
-  // partials for n_split history splits + 1 exact tail, then q_rot, q_sk, 4 statistics per query row and
+  // partials for n_split history splits + up to TAIL_MAX_CHUNKS of the exact tail, then q_rot, q_sk, 4 statistics per query row and
   // the packed query operands of the matrix-core kernel (sized for the largest kernel: 9 term planes, 8 heads)
-  return (parts_floats(B, Hq, d, n_split + 1) + (size_t)2 * B * Hq * d + (size_t)4 * B * Hq) * sizeof(float) +
+  return (parts_floats(B, Hq, d, n_split + TAIL_MAX_CHUNKS) + (size_t)2 * B * Hq * d + (size_t)4 * B * Hq) * sizeof(float) +
          flag_words(B, Hq) * sizeof(unsigned long long) + decode_mfma_pack_words(B, Hq, d) * sizeof(uint32_t);
 }
 
@@ -1083,7 +1092,22 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   // uses the halved count, for every stage of the step alike.
   const bool wide_wg = mfma_shape && layout->key_lane_major && decode_mfma_wide_workgroups(d, Gq, n_split, max_pages);
   if (wide_wg) n_split /= 2;
-  const int n_parts = n_split + 1;
+  if (dtype < TQ_F32 || dtype > TQ_BF16) return TQ_EINVAL;
+  // the exact tail as 32-bit words: always for fp32, for 16-bit rows when they are word-aligned
+  const int epw = dtype == TQ_F32 ? 1 : 2;
+  const bool words = epw == 1 || (((((uintptr_t)recent_k | (uintptr_t)recent_v) & 3) == 0) &&
+                                  !((rs_b | rs_r | rs_h | ts.s_blk) & 1));
+  // Workgroups per (sequence, KV head, group of TAIL_GC query heads) of the exact tail, each with a share of the
+  // exact tokens and a partial of its own.  One such workgroup pulls 2 x recent_rows rows into one compute unit
+  // and is the longest-running part of its launch; with few of them and a merge kernel behind (many splits - the
+  // in-launch merge takes exactly one partial of the tail) up to TAIL_MAX_CHUNKS share the rows
+  // (4 x 131072, 16 q / 2 KV heads, 128 exact tokens: 16 -> 64 workgroups).
+  int t_chunks = 1;
+  if (tail && words && n_split > MERGE_IN_KERNEL_MAX_SPLITS && opt_tail_chunks.load(std::memory_order_relaxed) != 0) {
+    const int64_t groups = (int64_t)Hkv * B * ((G + TAIL_GC - 1) / TAIL_GC);
+    while (t_chunks < TAIL_MAX_CHUNKS && groups * t_chunks * 2 <= 128 && recent_rows / (t_chunks * 2) >= 16) t_chunks *= 2;
+  }
+  const int n_parts = n_split + t_chunks;
   float* parts = (float*)workspace;
   float* q_rot = parts + parts_floats(B, Hq, d, n_parts);
   float* q_sk = q_rot + (size_t)B * Hq * d;
@@ -1091,11 +1115,6 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   unsigned long long* flags = (unsigned long long*)(q_stat + (size_t)4 * B * Hq);       // 8-byte aligned: every term above is even
   uint32_t* qa_pack = (uint32_t*)(flags + flag_words(B, Hq));
 
-  if (dtype < TQ_F32 || dtype > TQ_BF16) return TQ_EINVAL;
-  // the exact tail as 32-bit words: always for fp32, for 16-bit rows when they are word-aligned
-  const int epw = dtype == TQ_F32 ? 1 : 2;
-  const bool words = epw == 1 || (((((uintptr_t)recent_k | (uintptr_t)recent_v) & 3) == 0) &&
-                                  !((rs_b | rs_r | rs_h | ts.s_blk) & 1));
   if (tail && ts.paged && !words) return TQ_EUNSUPPORTED;       // a paged exact cache has to be word-aligned
   TailArgs ta;
   ta.q = q; ta.Hq = Hq; ta.Hkv = Hkv; ta.d = d;
@@ -1108,7 +1127,8 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   ta.tile_words = tail_tile_words(d / epw, recent_rows, ta.wide != 0);
   ta.max_pages = max_pages; ta.num_blocks = pool_pages;       // the exact cache shares the pool's block numbers
   ta.sm_scale = sm_scale; ta.parts = parts; ta.n_parts = n_parts; ta.part_index = n_split;
-  const int n_tail = Hkv * B * ((G + TAIL_GC - 1) / TAIL_GC);
+  ta.t_chunks = t_chunks;
+  const int n_tail = Hkv * B * ((G + TAIL_GC - 1) / TAIL_GC) * t_chunks;
   bool tail_done = false;
 
   // Whole compressed-only step on the matrix-core path: the query preparation runs as a prologue of the
@@ -1200,7 +1220,7 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   // the exact tail's partial first (it depends on nothing the page kernel does), so that a page kernel that merges
   // its splits itself finds it written
   if (tail && (stages & 2) && !tail_done) {
-    const dim3 tgrid(Hkv, B, (G + TAIL_GC - 1) / TAIL_GC);
+    const dim3 tgrid(Hkv, B, ((G + TAIL_GC - 1) / TAIL_GC) * (words ? t_chunks : 1));
     size_t tsm = words ? tail_words_smem(d, recent_rows, ta.tile_words) : tail_smem(d, recent_rows);
 #define TQ_LAUNCH_TAIL(KERN, ...)                                                                                    \
   {                                                                                                                  \
@@ -1359,7 +1379,7 @@ size_t decode_scratch_need(int B, int Hq, int Hkv, int n_split, const tq_layer& 
   int kv_div = 0;
   for (int n = 1; n <= G && !kv_div; ++n)
     if (G % n == 0 && G / n <= 8) kv_div = n;
-  size_t floats = parts_floats(B, Hq, d, n_split + 1) + (size_t)2 * B * Hq * d + (size_t)4 * B * Hq +
+  size_t floats = parts_floats(B, Hq, d, n_split + TAIL_MAX_CHUNKS) + (size_t)2 * B * Hq * d + (size_t)4 * B * Hq +
                   2 * flag_words(B, Hq);
   size_t words = 0;
   if (kv_div && (d == 64 || d == 128 || d == 256)) {
