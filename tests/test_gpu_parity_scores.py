@@ -607,7 +607,9 @@ def test_four_bit_keys_staged_through_lds(gpu, d, vb, Hq, Hkv, dtype):
                                                   (3, 9, 256, torch.float32), (100, 33, 128, torch.bfloat16),
                                                   (7, 5, 128, torch.float32), (129, 17, 128, torch.float16),
                                                   (5, 40, 64, torch.bfloat16), (2, 19, 576, torch.float32),
-                                                  (300, 3, 256, torch.bfloat16), (1, 1, 128, torch.float32)])
+                                                  (300, 3, 256, torch.bfloat16), (1, 1, 128, torch.float32),
+                                                  (16, 20, 512, torch.float32), (8, 12, 192, torch.bfloat16),
+                                                  (4, 70, 384, torch.float16), (33, 66, 768, torch.bfloat16)])
 def test_merge_of_split_partials(gpu, rows, n_parts, d, dtype):
     """tq_decode_merge on its own: the log-sum-exp merge of per-split partials (m, l, acc[d]) - the segments of
     score.py:84-173 - against a float64 computation of the same formula, with empty parts (l = 0, which carry no
