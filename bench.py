@@ -66,13 +66,15 @@ def algorithmic_bytes_per_token_head(d, mse_bits, value_bits, group):
 class DecodeWorkload:
     """B sequences of N compressed tokens in `n_pools` separate pools."""
 
-    def __init__(self, name, B, N, Hq, Hkv, d, key_bits, value_bits, n_pools, seed, dist, device):
+    def __init__(self, name, B, N, Hq, Hkv, d, key_bits, value_bits, n_pools, seed, dist, device, device_data=False):
         import torch
         from turboquant_amd.paged import PagedKVPool
         from turboquant_amd.quantizer import TurboQuantProd
         self.name, self.B, self.N, self.Hq, self.Hkv, self.d = name, B, N, Hq, Hkv, d
         self.key_bits, self.value_bits = key_bits, value_bits
         gen = torch.Generator().manual_seed(seed)            # a CPU generator: the same data on every machine
+        # (device_data: the bulk of the keys and values from the card's generator instead - timing-only tables)
+        dgen = torch.Generator(device=device).manual_seed(seed) if device_data else None
         self.tq = TurboQuantProd(d, bits=key_bits, device=device)
         pages_per_seq = (N + 15) // 16
         n_pages = B * pages_per_seq
@@ -88,6 +90,9 @@ class DecodeWorkload:
                 shape = (1, t1 - t0, Hkv, d)
                 if dist == "student_t5":
                     k, v = student_t(shape, 5, gen), student_t(shape, 5, gen)
+                elif dgen is not None:
+                    k = torch.randn(*shape, generator=dgen, device=device)
+                    v = torch.randn(*shape, generator=dgen, device=device)
                 else:
                     k = torch.randn(*shape, generator=gen)
                     v = torch.randn(*shape, generator=gen)
@@ -191,6 +196,7 @@ def time_kernel_stage(work, steps, warmup):
     for i, (a, b) in enumerate(evs):
         lib.tq_time_next_page_kernel(a.cuda_event, b.cuda_event)
         work.step(warmup + i)
+    lib.tq_time_next_page_kernel(None, None)        # (nothing is left armed once the events go away)
     torch.cuda.synchronize()
     return sum(a.elapsed_time(b) for a, b in evs) / steps
 
@@ -455,6 +461,46 @@ def cpu_quantize_baseline(k, v, tq, sample_tokens=32768):
             "sample": f"{sample_tokens} of 32768 tokens x 8 KV heads, median of 3 runs"}
 
 
+# (sequences, context, query heads, KV heads, head_dim, key bits, value bits): every family of decode kernels -
+# head_dim 64 / 128 / 256 on the matrix cores with 2- / 3- / 4-bit keys and 2- / 4-bit values, 1 to 16 query heads
+# per KV head, short and long contexts - and the general kernel's shapes (head_dim 576, 5-bit keys, 8-bit values)
+SHAPE_TABLE = [
+    (4, 131072, 16, 2, 256, 3, 2), (4, 131072, 16, 2, 256, 2, 2), (4, 131072, 16, 2, 256, 4, 2),
+    (4, 131072, 16, 2, 256, 3, 4), (4, 131072, 8, 2, 256, 3, 2), (4, 131072, 2, 2, 256, 3, 2),
+    (8, 65536, 16, 2, 256, 3, 2), (4, 65536, 32, 4, 256, 3, 2), (32, 8192, 16, 2, 256, 3, 2), (1, 524288, 16, 2, 256, 3, 2),
+    (16, 8192, 32, 8, 128, 3, 4), (16, 8192, 32, 8, 128, 2, 4), (16, 8192, 32, 8, 128, 4, 4), (16, 8192, 32, 8, 128, 3, 2),
+    (16, 8192, 64, 8, 128, 3, 4), (16, 8192, 8, 8, 128, 3, 4), (16, 8192, 128, 8, 128, 3, 4),
+    (32, 32768, 32, 8, 128, 3, 4), (8, 131072, 32, 8, 128, 3, 4), (64, 2048, 32, 8, 128, 3, 4), (256, 1024, 32, 8, 128, 3, 4),
+    (1, 131072, 32, 8, 128, 3, 4),
+    (16, 8192, 32, 8, 64, 3, 4), (16, 8192, 32, 8, 64, 2, 2), (16, 8192, 32, 8, 64, 4, 4), (16, 8192, 64, 8, 64, 3, 4),
+    (32, 32768, 32, 8, 64, 3, 4),
+    (16, 8192, 8, 1, 576, 4, 4), (16, 8192, 32, 8, 128, 5, 4), (16, 8192, 32, 8, 128, 3, 8), (16, 8192, 88, 8, 128, 3, 4),
+]
+
+
+def shape_table(device, steps, warmup):
+    """Whole-step and page-kernel times of SHAPE_TABLE's decode shapes (timing only; N(0,1) data from the card's
+    generator), compressed-only and with the newest 128 tokens exact."""
+    import torch
+    rows = []
+    for (B, N, Hq, Hkv, d, kb, vb) in SHAPE_TABLE:
+        w = DecodeWorkload("shape", B, N, Hq, Hkv, d, kb, vb, n_pools=2 if B * N * Hkv >= 1 << 22 else 4, seed=5,
+                           dist="normal", device=device, device_data=True)
+        ms, _ = time_steps(w.step, steps, warmup)
+        kern = time_kernel_stage(w, steps, warmup)
+        hyb = hybrid_step_bench(w, steps, warmup)
+        rows.append({"sequences": B, "context": N, "q_heads": Hq, "kv_heads": Hkv, "head_dim": d, "key_bits": kb,
+                     "value_bits": vb, "n_split": w.n_split, "bytes_per_step": w.bytes,
+                     "step_us": round(ms * 1e3, 2), "step_pct_hbm_peak": round(100.0 * w.bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 1),
+                     "page_kernel_us": round(kern * 1e3, 2),
+                     "page_kernel_pct_hbm_peak": round(100.0 * w.bytes / (kern * 1e-3) / 1e9 / HBM_PEAK_GBS, 1),
+                     "hybrid_step_us": round(hyb["ms_per_step"] * 1e3, 2)})
+        print(json.dumps(rows[-1]), file=sys.stderr, flush=True)
+        del w
+        torch.cuda.empty_cache()
+    return rows
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -469,6 +515,9 @@ def main():
     ap.add_argument("--no-backend-step", action="store_true",
                     help="skip the full-decode-step leg (32-layer transformer through the backend hooks, ~60 GB)")
     ap.add_argument("--context", type=int, default=131072, help="context tokens per sequence of the main workload")
+    ap.add_argument("--shapes", action="store_true",
+                    help="time the decode step over SHAPE_TABLE instead (one JSON line with a row per shape; rows also "
+                         "go to stderr as they finish)")
     ap.add_argument("--quantize-only", action="store_true",
                     help="run the prefill-quantize leg alone and print its object (for profiles of its kernels)")
     args = ap.parse_args()
@@ -485,6 +534,11 @@ def main():
         raise SystemExit("turboquant_amd/libtq_hip.so is missing; run `python -m turboquant_amd.build` first")
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
+
+    if args.shapes:
+        print(json.dumps({"metric": "decode step over a table of shapes, 1 GPU", "steps": args.steps, "warmup": args.warmup,
+                          "shapes": shape_table(device, args.steps, args.warmup)}))
+        return
 
     if args.quantize_only:
         quant, _keep = quantize_bench(device, args.steps, args.warmup)

@@ -305,8 +305,8 @@ int tq_decode_attn_paged_noalloc(const void *q, int dtype, int B, int Hq, int Hk
 int tq_decode_merge(const float *parts, int64_t rows, int n_parts, int d, int dtype, void *out, void *stream);
 
 /* Measurement aid (no counterpart in the reference).  Arms the calling thread: the next
- * page-streaming kernel that tq_decode_attn_paged[_stages] launches from this thread (its matrix-core
- * kernel) is launched with `start_event` / `stop_event` (hipEvent_t, created with timing enabled)
+ * page-streaming kernel that tq_decode_attn_paged[_stages] launches from this thread (matrix-core or
+ * general) is launched with `start_event` / `stop_event` (hipEvent_t, created with timing enabled)
  * attached to its own dispatch, so that hipEventElapsedTime(start, stop) is that kernel's execution
  * time alone - what a profiler's kernel trace reports - and not the interval between two markers in the
  * stream, which also contains the dispatch gap.  Pass NULLs to disarm.                             */
@@ -343,6 +343,9 @@ void tq_time_next_key_kernel(void *start_event, void *stop_event);
  *                      compute unit twice and the split count is even, the workgroups of the first half of the grid
  *                      (dispatched first, served first by their SIMDs) take the even splits and this many sixteenths
  *                      of a split's trips over from the odd splits of the second half; 0: equal shares.
+ *   "prep_workgroups"  default 1024: the query preparation launches one workgroup per (group of query heads, 32
+ *                      coordinates) up to this many; with more units a workgroup prepares several groups in turn,
+ *                      keeping its slices of the matrices in registers; 0: always one workgroup per unit.
  *   "tail_chunks"      1 (default): a hybrid step with more than 8 context splits and few (sequence, KV head)
  *                      pairs lets 2 or 4 workgroups share the exact tokens of a group of query heads, each with
  *                      a partial of its own for the merge kernel; 0: one workgroup and one partial.

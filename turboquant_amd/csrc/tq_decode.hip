@@ -17,6 +17,8 @@
 #include <chrono>
 #include <cstring>
 
+#include <hip/hip_ext.h>
+
 #include "tq_common.h"
 #include "tq_prep.h"
 #include "tq_decode_mfma.h"
@@ -813,7 +815,8 @@ static_assert(TAIL_THREADS == PREP_COLS * PREP_SLICES, "the two roles share a wo
 template <int PER, int DT, bool PAGED>
 __global__ void __launch_bounds__(TAIL_THREADS, 4)
 prep_tail_kernel(TailArgs A, int n_tail, int B, int Gq, tq_layer ly, float* __restrict__ q_rot, float* __restrict__ q_sk,
-                 float* __restrict__ q_stat, uint32_t* __restrict__ qa_pack, unsigned long long* __restrict__ arrivals) {
+                 float* __restrict__ q_stat, uint32_t* __restrict__ qa_pack, unsigned long long* __restrict__ arrivals,
+                 int n_prep_x, int n_groups) {
   extern __shared__ __align__(16) float sm[];
   const int id = blockIdx.x;
   if (id < n_tail) {
@@ -821,9 +824,10 @@ prep_tail_kernel(TailArgs A, int n_tail, int B, int Gq, tq_layer ly, float* __re
     exact_tail_words_body<DT, 1, PAGED, true>(A, id % A.Hkv, (id / A.Hkv) % B, id / per_z, sm);
   } else {
     const int words = ly.d / PREP_COLS, p = id - n_tail;
-    // (the arrival counter of this group of query heads, for a page kernel that merges its splits itself)
-    if (arrivals != nullptr && p % words == 0 && threadIdx.x == 0) arrivals[p / words] = 0ull;
-    prep_query_body<PER, DT>(A.q, Gq, ly, A.sm_scale, q_rot, q_sk, q_stat, qa_pack, p / words, p % words, sm);
+    // (n_prep_x workgroups per plane word share the n_groups groups of query heads; arrivals: the groups' arrival
+    // counters, zeroed for a page kernel that merges its splits itself)
+    prep_query_body<PER, DT>(A.q, Gq, ly, A.sm_scale, q_rot, q_sk, q_stat, qa_pack, p / words, n_prep_x, n_groups, p % words,
+                             arrivals, sm);
   }
 }
 
@@ -965,6 +969,7 @@ std::atomic<int> opt_wide_workgroups{1};
 std::atomic<int> opt_split_skew{1};
 std::atomic<int> opt_merge_row_groups{1};
 std::atomic<int> opt_tail_chunks{1};
+std::atomic<int> opt_prep_workgroups{1024};
 }  // namespace tq
 
 namespace {
@@ -999,6 +1004,11 @@ extern "C" int tq_set_option(const char* name, int64_t value) {
   if (!std::strcmp(name, "split_skew")) {
     if (value < 0 || value > 8) return TQ_EINVAL;
     opt_split_skew.store((int)value);
+    return TQ_OK;
+  }
+  if (!std::strcmp(name, "prep_workgroups")) {
+    if (value < 0 || value > (1 << 20)) return TQ_EINVAL;
+    opt_prep_workgroups.store((int)value);
     return TQ_OK;
   }
   if (!std::strcmp(name, "tail_chunks")) { opt_tail_chunks.store(value != 0); return TQ_OK; }
@@ -1169,7 +1179,11 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   }
   if ((stages & 1) && !fused) {
     if (!layer->Pi || !layer->PiT || !layer->S || !layer->ST || !layer->centroids) return TQ_ENULL;
-    const int n_prep = (B * Hq / Gq) * (d / PREP_COLS);
+    const int n_groups = B * Hq / Gq, prep_words = d / PREP_COLS;
+    const int prep_limit = opt_prep_workgroups.load(std::memory_order_relaxed);
+    const int prep_cap = prep_limit > 0 ? (prep_limit / prep_words > 0 ? prep_limit / prep_words : 1) : 0;
+    const int n_prep_x = prep_cap > 0 && n_groups > prep_cap ? prep_cap : n_groups;     // see launch_rotate_query
+    const int n_prep = n_prep_x * prep_words;
     // Whole hybrid step on the matrix-core path: the exact tail shares the preparation's launch (the tail
     // workgroups first, so that the longer-running ones start first).  The kernel is built for 128 registers
     // per lane and the tail's LDS is sized by the rows it holds, so two workgroups fit a compute unit; with more
@@ -1186,7 +1200,8 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
       if (e != hipSuccess) return (int)e;                                                                            \
     }                                                                                                                \
     kern<<<dim3((unsigned)(n_tail + n_prep)), dim3(TAIL_THREADS), fsm, st>>>(ta, n_tail, B, Gq, *layer, q_rot, q_sk,  \
-                                                                            q_stat, qa_pack, fm.counters);           \
+                                                                            q_stat, qa_pack, fm.counters, n_prep_x,  \
+                                                                            n_groups);                               \
   }
 #define TQ_LAUNCH_PT_DT(PER, PAGED)                                \
   {                                                                \
@@ -1273,6 +1288,9 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
     const size_t work = (size_t)gp * (GEN_CHUNK > tg * d ? GEN_CHUNK : tg * d);    // weights, then slice partials
     const size_t smem = ((size_t)2 * d * gp + 32 + work) * sizeof(float);
     dim3 grid(n_split, Hkv, B), block(GEN_THREADS);
+    // an armed pair of timing events goes to this kernel's dispatch as it would to the matrix-core kernel's
+    hipEvent_t t_start = nullptr, t_stop = nullptr;
+    const bool timed = take_time_hook(0, t_start, t_stop);
 #define TQ_LAUNCH_DEC(VB, GP4)                                                                            \
   {                                                                                                       \
     auto kern = decode_pages_kernel<VB, GP4>;                                                             \
@@ -1280,8 +1298,13 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
       hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem); \
       if (e != hipSuccess) return (int)e;                                                                 \
     }                                                                                                     \
-    kern<<<grid, block, smem, st>>>(q_rot, q_sk, Hq, Hkv, pool, block_table, bt_stride, seq_lens, sm_scale, *layer,  \
-                                    *layout, parts, n_parts, n_split, len_sub, max_pages, pool_pages);     \
+    if (timed)                                                                                            \
+      hipExtLaunchKernelGGL(kern, grid, block, smem, st, t_start, t_stop, 0, q_rot, q_sk, Hq, Hkv, pool, block_table,  \
+                            bt_stride, seq_lens, sm_scale, *layer, *layout, parts, n_parts, n_split, len_sub,          \
+                            max_pages, pool_pages);                                                                      \
+    else                                                                                                  \
+      kern<<<grid, block, smem, st>>>(q_rot, q_sk, Hq, Hkv, pool, block_table, bt_stride, seq_lens, sm_scale, *layer,  \
+                                      *layout, parts, n_parts, n_split, len_sub, max_pages, pool_pages);   \
   }
 #define TQ_LAUNCH_DEC_G(VB)                                                      \
   {                                                                              \
