@@ -625,6 +625,19 @@ def test_exact_tail_shapes(gpu, d, dtype, Hq, Hkv, recent, pad):
     _progress(f"  worst cosine {worst:.7f}")
 
 
+def test_hybrid_step_of_many_sequences_at_head_dim_256(gpu):
+    """Twenty sequences at head_dim 256 with 128 exact tokens each: the exact tail's tiles fill a compute unit's
+    LDS, the grid is larger than the card, and the tail and the query preparation run as two launches instead of
+    one (score.py:99-173 against the oracle, ragged histories and tails, few and many splits)."""
+    B = 20
+    lens = [64 * (b % 5) + 17 * b for b in range(B)]
+    recent = [128 if b % 3 else 7 * b % 128 for b in range(B)]
+    for n_split in (2, 9):
+        _progress(f"many sequences d=256 n_split={n_split}")
+        worst = _decode_case(gpu, 256, 3, 2, B, 16, 2, lens, recent, seed=4242, n_split=n_split)
+        _progress(f"  worst cosine {worst:.7f}")
+
+
 @pytest.mark.parametrize("d,dtype,Hq,Hkv,recent,n_split,pad", [
     (256, torch.bfloat16, 16, 2, [128, 3, 0], 12, 0),      # four workgroups per head group; shares of 32, of 0 / 1 tokens, of none
     (128, torch.float16, 8, 1, [300, 77, 1], 9, 8),        # several load rounds per share, rows inside a wider buffer

@@ -1191,7 +1191,11 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
     // (16 x 8192: 48.9 -> 45.2 us per step, 32 x 32768: 223.6 -> 221.5 us).
     size_t fsm = tail_words_smem(d, recent_rows, ta.tile_words);
     if (prep_smem_bytes(Gq, d) > fsm) fsm = prep_smem_bytes(Gq, d);
-    if (tail && ta.wide && mfma_shape && stages == 7) {
+    // ... unless the tail's tiles leave room for one workgroup per compute unit only (head_dim 256 with 128 exact
+    // tokens: 139 KB) and the grid is larger than the card: the preparation workgroups would queue behind that
+    // LDS size too (128 x 2048, 16 q / 2 KV heads: 109.7 us per step fused, 88.1 as two launches)
+    const bool one_per_unit = fsm > (size_t)80 * 1024;
+    if (tail && ta.wide && mfma_shape && stages == 7 && !(one_per_unit && n_tail + n_prep > device_compute_units())) {
 #define TQ_LAUNCH_PT(PER, DT, PAGED)                                                                                 \
   {                                                                                                                  \
     auto kern = prep_tail_kernel<PER, DT, PAGED>;                                                                    \

@@ -56,4 +56,7 @@ bool decode_mfma_wide_workgroups(int d, int G, int n_split, int max_pages);
 // n_split x rows workgroups of four wavefronts that sit two to a compute unit.
 int decode_mfma_split_skew(int n_split, int rows);
 
+// Compute units of the device (looked up once); 0 if unknown.
+int device_compute_units();
+
 }  // namespace tq

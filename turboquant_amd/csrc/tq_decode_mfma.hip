@@ -43,6 +43,17 @@ bool decode_mfma_wide_workgroups(int d, int G, int n_split, int max_pages) {
   return blocks <= (int64_t)16 * MF_WAVES * n_split;
 }
 
+// Compute units of the device that is current at the first call (the cards of one machine are alike); 0 if unknown.
+int device_compute_units() {
+  static const int units = [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) n = 0;
+    return n;
+  }();
+  return units;
+}
+
 // Unequal shares for the two workgroups of a compute unit.  Workgroups are dispatched in grid order and spread
 // over the compute units, so when the launch fills (nearly) every compute unit twice, the first half of the grid
 // holds the older workgroup of every unit; a SIMD serves its older wavefronts first, and with equal shares those
@@ -52,12 +63,7 @@ bool decode_mfma_wide_workgroups(int d, int G, int n_split, int max_pages) {
 int decode_mfma_split_skew(int n_split, int rows) {
   const int skew = opt_split_skew.load(std::memory_order_relaxed);
   if (skew <= 0 || n_split < 2 || (n_split & 1)) return 0;
-  static const int units = [] {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) n = 0;
-    return n;
-  }();
+  const int units = device_compute_units();
   const int64_t groups = (int64_t)n_split * rows;
   return units > 0 && groups <= 2 * (int64_t)units && groups * 16 >= 30 * (int64_t)units ? skew : 0;
 }
