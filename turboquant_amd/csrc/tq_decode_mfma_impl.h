@@ -262,7 +262,14 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   // to a compute unit, and a SIMD serves its older wavefronts first: with equal shares the first half of the grid
   // finishes early and the second half runs on alone.
   int split = blockIdx.x, b = blockIdx.z;
-  const int h = blockIdx.y;
+  // The groups of a KV head are (splits x KV heads) workgroups apart in the grid, not next to each other: workgroups
+  // go to the card's eight dies in turn, each die has its own L2, and a distance that is a multiple of eight puts the
+  // groups that read the same pages at the same time on the same die.
+  int h = blockIdx.y;
+  if (kv_div > 1) {
+    const int kv_heads = Hkv / kv_div, grp = h / kv_heads;
+    h = (h - grp * kv_heads) * kv_div + grp;
+  }
   if (skew16 > 0) {
     const int seqs = (int)gridDim.z >> 1, late = b >= seqs;
     b -= late ? seqs : 0;
