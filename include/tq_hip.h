@@ -343,9 +343,6 @@ void tq_time_next_key_kernel(void *start_event, void *stop_event);
  *                      compute unit twice and the split count is even, the workgroups of the first half of the grid
  *                      (dispatched first, served first by their SIMDs) take the even splits and this many sixteenths
  *                      of a split's trips over from the odd splits of the second half; 0: equal shares.
- *   "prep_workgroups"  default 1024: the query preparation launches one workgroup per (group of query heads, 32
- *                      coordinates) up to this many; with more units a workgroup prepares several groups in turn,
- *                      keeping its slices of the matrices in registers; 0: always one workgroup per unit.
  *   "tail_chunks"      1 (default): a hybrid step with more than 8 context splits and few (sequence, KV head)
  *                      pairs lets 2 or 4 workgroups share the exact tokens of a group of query heads, each with
  *                      a partial of its own for the merge kernel; 0: one workgroup and one partial.

@@ -603,56 +603,6 @@ def test_four_bit_keys_staged_through_lds(gpu, d, vb, Hq, Hkv, dtype):
     _variant_against_default(gpu, "lds_stage", d, 4, vb, Hq, Hkv, dtype, exact=True)
 
 
-@pytest.mark.parametrize("d,key_bits,vb,Hq,Hkv,dtype", [(128, 3, 4, 8, 2, torch.bfloat16), (256, 3, 2, 16, 2, torch.bfloat16),
-                                                         (64, 4, 2, 6, 2, torch.float16), (128, 2, 4, 32, 2, torch.bfloat16)])
-def test_preparation_workgroups_that_take_several_groups_of_heads(gpu, d, key_bits, vb, Hq, Hkv, dtype):
-    """With more (group of query heads, plane word) units than option "prep_workgroups" allows, a preparation
-    workgroup takes several groups in turn (matrix slices kept in registers, the next query requested early).  The
-    arithmetic per group is the same: compressed-only and hybrid steps, with the in-launch merge (few splits, whose
-    arrival counters the preparation zeroes) and with the merge kernel, must equal the one-workgroup-per-unit launch
-    bit for bit - here with limits that leave one, two and three workgroups per plane word for 14 groups."""
-    B = 7
-    lens = [700, 17, 16 * 37 + 1, 96, 0, 333, 64]
-    ring = 40
-    n_log = max((n + 15) // 16 for n in lens)
-    n_pages = B * n_log + 1
-    pool, tq = _make_pool(gpu, d, key_bits, vb, Hkv, n_pages, dtype, seed=79)
-    g = torch.Generator().manual_seed(77 + key_bits + d)
-    k = torch.randn(B, max(lens), Hkv, d, generator=g).to(dtype)
-    v = torch.randn(B, max(lens), Hkv, d, generator=g).to(dtype)
-    q = torch.randn(B, Hq, d, generator=g).to(dtype).to(gpu)
-    table = torch.randperm(n_pages, generator=g)[: B * n_log].to(torch.int32).view(B, n_log).to(gpu)
-    pool.append(k.to(gpu), v.to(gpu), table)
-    seq = torch.tensor(lens, dtype=torch.int32, device=gpu)
-    cache = torch.randn(2, n_pages, 16, Hkv, d, generator=g).to(dtype).to(gpu)
-    words = d // 32
-    _progress(f"prep_workgroups d={d} kb={key_bits} vb={vb} Hq={Hq} Hkv={Hkv} {dtype}")
-
-    def run():
-        outs = []
-        for n_split in (2, 12):
-            outs.append(pool.decode_attention(q, table, seq, n_split=n_split, max_len=max(lens)).clone())
-            outs.append(pool.decode_attention_ring(q, table, seq, cache[0], cache[1], ring, n_split=n_split,
-                                                   max_len=max(lens)).clone())
-        torch.cuda.synchronize()
-        return outs
-    try:
-        _set_option("prep_workgroups", 0)
-        want = run()
-        for limit in (1, 2 * words, 3 * words):
-            _set_option("prep_workgroups", limit)
-            got = run()
-            for i, (a, b) in enumerate(zip(got, want)):
-                assert torch.equal(a, b), (limit, i)
-    finally:
-        _set_option("prep_workgroups", 1024)
-    b = 0
-    idx, sgn, norms, rn, vd, vs, vz = [t.cpu() for t in pool.export_flat(table[b], lens[b])]
-    ref = O.hybrid_attention(q[b:b + 1].cpu(), key_code(idx, sgn, rn, norms, key_bits - 1), value_code(vd, vs, vz, vb),
-                             lens[b], params_of(tq), Hkv, None, None)
-    assert cosine(want[0][b:b + 1].cpu(), ref) >= COS_GATE
-
-
 @pytest.mark.parametrize("rows,n_parts,d,dtype", [(64, 64, 256, torch.bfloat16), (64, 65, 256, torch.float16),
                                                   (3, 9, 256, torch.float32), (100, 33, 128, torch.bfloat16),
                                                   (7, 5, 128, torch.float32), (129, 17, 128, torch.float16),

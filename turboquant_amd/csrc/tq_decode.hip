@@ -815,8 +815,7 @@ static_assert(TAIL_THREADS == PREP_COLS * PREP_SLICES, "the two roles share a wo
 template <int PER, int DT, bool PAGED>
 __global__ void __launch_bounds__(TAIL_THREADS, 4)
 prep_tail_kernel(TailArgs A, int n_tail, int B, int Gq, tq_layer ly, float* __restrict__ q_rot, float* __restrict__ q_sk,
-                 float* __restrict__ q_stat, uint32_t* __restrict__ qa_pack, unsigned long long* __restrict__ arrivals,
-                 int n_prep_x, int n_groups) {
+                 float* __restrict__ q_stat, uint32_t* __restrict__ qa_pack, unsigned long long* __restrict__ arrivals) {
   extern __shared__ __align__(16) float sm[];
   const int id = blockIdx.x;
   if (id < n_tail) {
@@ -824,10 +823,9 @@ prep_tail_kernel(TailArgs A, int n_tail, int B, int Gq, tq_layer ly, float* __re
     exact_tail_words_body<DT, 1, PAGED, true>(A, id % A.Hkv, (id / A.Hkv) % B, id / per_z, sm);
   } else {
     const int words = ly.d / PREP_COLS, p = id - n_tail;
-    // (n_prep_x workgroups per plane word share the n_groups groups of query heads; arrivals: the groups' arrival
-    // counters, zeroed for a page kernel that merges its splits itself)
-    prep_query_body<PER, DT>(A.q, Gq, ly, A.sm_scale, q_rot, q_sk, q_stat, qa_pack, p / words, n_prep_x, n_groups, p % words,
-                             arrivals, sm);
+    // (the arrival counter of this group of query heads, for a page kernel that merges its splits itself)
+    if (arrivals != nullptr && p % words == 0 && threadIdx.x == 0) arrivals[p / words] = 0ull;
+    prep_query_body<PER, DT>(A.q, Gq, ly, A.sm_scale, q_rot, q_sk, q_stat, qa_pack, p / words, p % words, sm);
   }
 }
 
@@ -969,7 +967,6 @@ std::atomic<int> opt_wide_workgroups{1};
 std::atomic<int> opt_split_skew{1};
 std::atomic<int> opt_merge_row_groups{1};
 std::atomic<int> opt_tail_chunks{1};
-std::atomic<int> opt_prep_workgroups{1024};
 }  // namespace tq
 
 namespace {
@@ -1004,11 +1001,6 @@ extern "C" int tq_set_option(const char* name, int64_t value) {
   if (!std::strcmp(name, "split_skew")) {
     if (value < 0 || value > 8) return TQ_EINVAL;
     opt_split_skew.store((int)value);
-    return TQ_OK;
-  }
-  if (!std::strcmp(name, "prep_workgroups")) {
-    if (value < 0 || value > (1 << 20)) return TQ_EINVAL;
-    opt_prep_workgroups.store((int)value);
     return TQ_OK;
   }
   if (!std::strcmp(name, "tail_chunks")) { opt_tail_chunks.store(value != 0); return TQ_OK; }
@@ -1179,11 +1171,7 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   }
   if ((stages & 1) && !fused) {
     if (!layer->Pi || !layer->PiT || !layer->S || !layer->ST || !layer->centroids) return TQ_ENULL;
-    const int n_groups = B * Hq / Gq, prep_words = d / PREP_COLS;
-    const int prep_limit = opt_prep_workgroups.load(std::memory_order_relaxed);
-    const int prep_cap = prep_limit > 0 ? (prep_limit / prep_words > 0 ? prep_limit / prep_words : 1) : 0;
-    const int n_prep_x = prep_cap > 0 && n_groups > prep_cap ? prep_cap : n_groups;     // see launch_rotate_query
-    const int n_prep = n_prep_x * prep_words;
+    const int n_prep = (B * Hq / Gq) * (d / PREP_COLS);
     // Whole hybrid step on the matrix-core path: the exact tail shares the preparation's launch (the tail
     // workgroups first, so that the longer-running ones start first).  The kernel is built for 128 registers
     // per lane and the tail's LDS is sized by the rows it holds, so two workgroups fit a compute unit; with more
@@ -1204,8 +1192,7 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
       if (e != hipSuccess) return (int)e;                                                                            \
     }                                                                                                                \
     kern<<<dim3((unsigned)(n_tail + n_prep)), dim3(TAIL_THREADS), fsm, st>>>(ta, n_tail, B, Gq, *layer, q_rot, q_sk,  \
-                                                                            q_stat, qa_pack, fm.counters, n_prep_x,  \
-                                                                            n_groups);                               \
+                                                                            q_stat, qa_pack, fm.counters);           \
   }
 #define TQ_LAUNCH_PT_DT(PER, PAGED)                                \
   {                                                                \

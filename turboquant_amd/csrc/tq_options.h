@@ -14,7 +14,6 @@ extern std::atomic<int> opt_narrow_rows;       // decode, head_dim 128 / 256 wit
 extern std::atomic<int> opt_lds_stage;         // decode: page data through LDS-direct loads, a whole trip ahead
 extern std::atomic<int> opt_wide_workgroups;   // decode, head_dim 64 / 128, short contexts: workgroups of 8 wavefronts
 extern std::atomic<int> opt_split_skew;        // decode, two workgroups per compute unit: sixteenths of a split moved to the workgroup dispatched first (0: none)
-extern std::atomic<int> opt_prep_workgroups;    // query preparation: workgroups per launch beyond which a workgroup takes several groups of heads (0: no limit)
 extern std::atomic<int> opt_tail_chunks;        // hybrid decode with many splits: up to 4 workgroups share the exact tokens of a head group
 extern std::atomic<int> opt_merge_row_groups;  // merge kernel: with few rows, several workgroups share a row's channels
 extern std::atomic<int> opt_merge_in_kernel;    // decode: few context splits are merged by the last workgroup of the page kernel

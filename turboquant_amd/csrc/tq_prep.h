@@ -66,33 +66,26 @@ __device__ __forceinline__ float wave_sum_dpp(float v) {
 // PER = matrix rows per thread = d / PREP_SLICES; DT = element type of the query (a template parameter:
 // a run-time switch would put each query load under a branch, and the loads would wait for one another)
 // (a device function: the stand-alone kernel and the launch that shares its grid with the exact-tail
-// workgroups both run it; `word` is the workgroup's plane word, `sm` its dynamic LDS.  The workgroup prepares
-// the groups of query heads group0, group0 + group_step, ... below n_groups one after the other: its matrix
-// slices stay in registers, and the query of the next group is requested while the current one is worked on,
-// so a further group costs the LDS phases only - with thousands of groups (hundreds of sequences) a workgroup
-// per group spent its time on launches and matrix loads.  `arrivals`: see the stand-alone kernel.)
+// workgroups both run it; `group` / `word` are the workgroup's coordinates, `sm` its dynamic LDS)
 template <int PER, int DT>
 __device__ __forceinline__ void prep_query_body(const void* __restrict__ q, int G, const tq_layer& ly, float sm_scale,
                                                 float* __restrict__ q_rot, float* __restrict__ q_sk,
                                                 float* __restrict__ q_stat, uint32_t* __restrict__ qa_pack,
-                                                int64_t group0, int64_t group_step, int64_t n_groups, int word,
-                                                unsigned long long* __restrict__ arrivals, float* sm) {
+                                                int64_t group, int word, float* sm) {
   const int d = ly.d, tid = threadIdx.x, jl = tid % PREP_COLS, sl = tid / PREP_COLS;
   const int j = word * PREP_COLS + jl;
   // every global load of the kernel is issued here, before anything waits, the query first: loads
   // return in order, so the query can go to shared memory (and its statistics be taken) while the
   // matrix slices, which do not depend on it, are still on their way
+  const int64_t row0 = group * G;
   constexpr int QPT = ROT_MAX_ROWS * 256 / (PREP_COLS * PREP_SLICES);   // query elements per thread, d <= 256
   float qv[QPT];
-  auto request_query = [&](int64_t group) {
 #pragma unroll
-    for (int k = 0; k < QPT; ++k) {
-      const int o = tid + k * (PREP_COLS * PREP_SLICES);
-      const float x = Elem<DT>::load(q, group * G * d + min(o, G * d - 1));      // unconditional, clamped
-      qv[k] = o < G * d ? x : 0.0f;
-    }
-  };
-  request_query(group0);
+  for (int k = 0; k < QPT; ++k) {
+    const int o = tid + k * (PREP_COLS * PREP_SLICES);
+    const float x = Elem<DT>::load(q, row0 * d + min(o, G * d - 1));      // unconditional, clamped
+    qv[k] = o < G * d ? x : 0.0f;
+  }
   float mp[PER], ms[PER];
 #pragma unroll
   for (int k = 0; k < PER; ++k) {
@@ -113,6 +106,11 @@ __device__ __forceinline__ void prep_query_body(const void* __restrict__ q, int 
   float* ssk = srot + G * PREP_COLS;
   float* stat = ssk + G * PREP_COLS;                // [G][4]
   float* coefs = stat + 4 * ROT_MAX_ROWS;           // [16]
+#pragma unroll
+  for (int k = 0; k < QPT; ++k) {
+    const int o = tid + k * (PREP_COLS * PREP_SLICES);
+    if (o < G * d) sq[o] = qv[k];
+  }
   const int mb = ly.mse_bits;
   int nx = 0;
   float cmax = 0.0f;
@@ -139,17 +137,7 @@ __device__ __forceinline__ void prep_query_body(const void* __restrict__ q, int 
     }
     coefs[tid] = coef;
   }
-  for (int64_t group = group0; group < n_groups; group += group_step) {
-  const int64_t row0 = group * G;
-  if (arrivals != nullptr && word == 0 && tid == 0) arrivals[group] = 0ull;
-  // (the previous group's last readers of the query were two barriers ago)
-#pragma unroll
-  for (int k = 0; k < QPT; ++k) {
-    const int o = tid + k * (PREP_COLS * PREP_SLICES);
-    if (o < G * d) sq[o] = qv[k];
-  }
-  __syncthreads();       // also: every lane has left the previous group's pack stage, which read stat / srot / ssk
-  if (group + group_step < n_groups) request_query(group + group_step);
+  __syncthreads();
   {  // row statistics: one wavefront per row
     const int lane = tid & 63, wave = tid >> 6, n_wave = blockDim.x >> 6;
     for (int r = wave; r < G; r += n_wave) {
@@ -272,7 +260,6 @@ __device__ __forceinline__ void prep_query_body(const void* __restrict__ q, int 
       }
     }
   }
-  }       // groups
 }
 
 // ------------------------------------------------------------------------------------------------------

@@ -73,12 +73,11 @@ template <int PER, int DT>
 __global__ void __launch_bounds__(PREP_COLS * PREP_SLICES)
 prep_query_kernel(const void* __restrict__ q, int G, tq_layer ly, float sm_scale,
                   float* __restrict__ q_rot, float* __restrict__ q_sk, float* __restrict__ q_stat,
-                  uint32_t* __restrict__ qa_pack, unsigned long long* __restrict__ arrivals, int64_t n_groups) {
+                  uint32_t* __restrict__ qa_pack, unsigned long long* __restrict__ arrivals) {
   extern __shared__ __align__(16) float sm[];
-  // arrivals: the arrival counter of every group of query heads, zeroed here for the page kernel that merges
-  // its splits itself.  Workgroup x takes the groups x, x + gridDim.x, ...
-  prep_query_body<PER, DT>(q, G, ly, sm_scale, q_rot, q_sk, q_stat, qa_pack, blockIdx.x, gridDim.x, n_groups, blockIdx.y,
-                           arrivals, sm);
+  // the arrival counter of this group of query heads, for the page kernel that merges its splits itself
+  if (arrivals != nullptr && blockIdx.y == 0 && threadIdx.x == 0) arrivals[blockIdx.x] = 0ull;
+  prep_query_body<PER, DT>(q, G, ly, sm_scale, q_rot, q_sk, q_stat, qa_pack, blockIdx.x, blockIdx.y, sm);
 }
 
 // The same preparation cut into more, smaller workgroups: one per unit = (hp consecutive heads of a group,
@@ -392,14 +391,8 @@ int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* 
       return e == hipSuccess ? TQ_OK : (int)e;
     }
     size_t smem = prep_smem_bytes(G, d);
-    // one workgroup per (group of heads, plane word) up to about four workgroups per compute unit; beyond that a
-    // workgroup takes several groups in turn (256 sequences x 1024 tokens, 32 q / 8 KV heads: 8192 units)
-    const int64_t n_groups = rows / G;
-    const int64_t limit = opt_prep_workgroups.load(std::memory_order_relaxed);
-    const int64_t cap = limit > 0 ? (limit / (d / PREP_COLS) > 0 ? limit / (d / PREP_COLS) : 1) : 0;
-    const int64_t gx = cap > 0 && n_groups > cap ? cap : n_groups;
-    const dim3 grid((unsigned)gx, d / PREP_COLS), block(PREP_COLS * PREP_SLICES);
-#define TQ_PREP(PER, DT) prep_query_kernel<PER, DT><<<grid, block, smem, st>>>(q, G, *layer, sm_scale, q_rot, q_sk, q_stat, qa_pack, arrivals, n_groups)
+    const dim3 grid((unsigned)(rows / G), d / PREP_COLS), block(PREP_COLS * PREP_SLICES);
+#define TQ_PREP(PER, DT) prep_query_kernel<PER, DT><<<grid, block, smem, st>>>(q, G, *layer, sm_scale, q_rot, q_sk, q_stat, qa_pack, arrivals)
 #define TQ_PREP_DT(PER)                              \
   {                                                  \
     if (dtype == TQ_BF16) TQ_PREP(PER, TQ_BF16);     \
