@@ -854,7 +854,7 @@ static size_t merge_smem(int n_parts, int d, int ny) {
 
 __global__ void __launch_bounds__(256)
 merge_kernel(const float* __restrict__ parts, int n_parts, int part_stride, int d, int dtype, void* __restrict__ out,
-             unsigned long long* __restrict__ flags, int n_flags) {
+             unsigned long long* __restrict__ flags, int n_flags, int row_groups) {
   // the flags under which the page kernel's workgroups published their query-preparation units are
   // cleared here, after that kernel has ended: the next call (or the next replay of a captured one,
   // which carries the same nonce) starts without a published unit
@@ -868,7 +868,8 @@ merge_kernel(const float* __restrict__ parts, int n_parts, int part_stride, int 
   extern __shared__ float s_w[];                 // [n_parts] weights, [n_parts] m, [n_parts] l, [8] scratch, [S][dw] sums
   const int64_t row = blockIdx.x;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int dw = d / (int)gridDim.y, c0 = (int)blockIdx.y * dw;   // this workgroup's channels: c0 .. c0 + dw - 1
+  // (row_groups = gridDim.y, as an argument: the grid's size would have to be read from the dispatch packet first)
+  const int dw = d / row_groups, c0 = (int)blockIdx.y * dw;       // this workgroup's channels: c0 .. c0 + dw - 1
   const float* p = parts + row * part_stride * (int64_t)(d + 2);
   float* s_m = s_w + n_parts;
   float* s_l = s_m + n_parts;
@@ -1033,7 +1034,7 @@ extern "C" int tq_decode_merge(const float* parts, int64_t rows, int n_parts, in
   if (rows == 0) return TQ_OK;
   const int ny = merge_row_groups(rows, n_parts, d);
   merge_kernel<<<dim3((unsigned)rows, ny), dim3(256), merge_smem(n_parts, d, ny), (hipStream_t)stream>>>(
-      parts, n_parts, n_parts, d, dtype, out, nullptr, 0);
+      parts, n_parts, n_parts, d, dtype, out, nullptr, 0, ny);
   TQ_CHECK_LAUNCH();
   return TQ_OK;
 }
@@ -1316,7 +1317,7 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   // without a tail the merge simply reads one part fewer
   const int merged = tail ? n_parts : n_split, ny = merge_row_groups((int64_t)B * Hq, merged, d);
   merge_kernel<<<dim3((unsigned)(B * Hq), ny), dim3(256), merge_smem(n_parts, d, ny), st>>>(
-      parts, merged, n_parts, d, dtype, out, fused ? flags : nullptr, fused ? n_flags : 0);
+      parts, merged, n_parts, d, dtype, out, fused ? flags : nullptr, fused ? n_flags : 0, ny);
   TQ_CHECK_LAUNCH();
   return TQ_OK;
 }

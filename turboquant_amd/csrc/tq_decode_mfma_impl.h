@@ -230,7 +230,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
                    const uint8_t* __restrict__ pool, const int32_t* __restrict__ block_table,
                    int bt_stride, const int32_t* __restrict__ seq_lens, float sm_scale, tq_layer ly, tq_page_layout L,
                    float* __restrict__ parts, int n_parts, int n_split, int len_sub, int max_pages, int num_pages,
-                   int skew16, FusedPrep fz, FusedMerge fm) {
+                   int skew16, int n_seq, FusedPrep fz, FusedMerge fm) {
   constexpr int DW = D / DS;                  // coordinates / channels of one wavefront
   constexpr int WPLT = (D + 127) / 128;       // plane words per lane per plane per page, all wavefronts
   constexpr int WPL = (DW + 127) / 128;       // ... of one wavefront (head_dim 64: one, with half of the lanes idle)
@@ -256,7 +256,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   // Hkv counts query-head groups: a KV head with more than 8 query heads is served by kv_div groups
   // of G <= 8 heads each (consecutive groups read the same pages)
   const int G = Hq / Hkv;
-  // skew16 > 0 (an even number of splits; the grid is (n_split / 2, Hkv, 2 B)): the workgroups of the first half
+  // skew16 > 0 (an even number of splits; the grid is (n_split / 2, Hkv, 2 n_seq)): the workgroups of the first half
   // of the grid take the even splits, those of the second half the odd ones, and every even split takes
   // skew16 sixteenths of a split's trips over from its odd neighbour.  Workgroups are dispatched in grid order, two
   // to a compute unit, and a SIMD serves its older wavefronts first: with equal shares the first half of the grid
@@ -271,8 +271,9 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
     h = (h - grp * kv_heads) * kv_div + grp;
   }
   if (skew16 > 0) {
-    const int seqs = (int)gridDim.z >> 1, late = b >= seqs;
-    b -= late ? seqs : 0;
+    // (n_seq is a kernel argument: the grid's size would have to be read from the dispatch packet)
+    const int late = b >= n_seq;
+    b -= late ? n_seq : 0;
     split = 2 * split + late;
   }
   const int tid = threadIdx.x, lane = tid & 63;
@@ -1124,11 +1125,11 @@ static int launch_one(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, 
   if (take_time_hook(0, t_start_event, t_stop_event)) {
     hipExtLaunchKernelGGL(kern, grid, dim3(NW * 64), smem, st, t_start_event, t_stop_event, 0,
                           qa_pack, q_stat, Hq, Hkv, kv_div, pool, block_table, bt_stride, seq_lens, sm_scale, ly, L, parts,
-                          n_parts, n_split, len_sub, max_pages, num_pages, skew16, fz, fm);
+                          n_parts, n_split, len_sub, max_pages, num_pages, skew16, B, fz, fm);
   } else {
     kern<<<grid, dim3(NW * 64), smem, st>>>(qa_pack, q_stat, Hq, Hkv, kv_div, pool, block_table, bt_stride, seq_lens,
                                             sm_scale, ly, L, parts, n_parts, n_split, len_sub, max_pages, num_pages, skew16,
-                                            fz, fm);
+                                            B, fz, fm);
   }
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? TQ_OK : (int)e;
