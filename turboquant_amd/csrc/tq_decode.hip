@@ -868,7 +868,8 @@ merge_kernel(const float* __restrict__ parts, int n_parts, int part_stride, int 
   extern __shared__ float s_w[];                 // [n_parts] weights, [n_parts] m, [n_parts] l, [8] scratch, [S][dw] sums
   const int64_t row = blockIdx.x;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  // (row_groups = gridDim.y, as an argument: the grid's size would have to be read from the dispatch packet first)
+  // (row_groups = gridDim.y, as an argument: it arrives with the others instead of through one more scalar load
+  // of the launch's implicit data in front of the first accumulator loads)
   const int dw = d / row_groups, c0 = (int)blockIdx.y * dw;       // this workgroup's channels: c0 .. c0 + dw - 1
   const float* p = parts + row * part_stride * (int64_t)(d + 2);
   float* s_m = s_w + n_parts;

@@ -271,7 +271,8 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
     h = (h - grp * kv_heads) * kv_div + grp;
   }
   if (skew16 > 0) {
-    // (n_seq is a kernel argument: the grid's size would have to be read from the dispatch packet)
+    // (n_seq arrives with the other kernel arguments; the grid's size would be one more scalar load of the
+    // launch's implicit data in front of everything that depends on the sequence)
     const int late = b >= n_seq;
     b -= late ? n_seq : 0;
     split = 2 * split + late;
