@@ -142,8 +142,33 @@ def ptr(t: Optional[torch.Tensor]) -> Optional[int]:
     return None if t is None else t.data_ptr()
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def stream_ptr(device) -> int:
+    """hipStream_t of torch's current stream on `device` (the raw accessor when this torch has it: no Stream object)."""
+    if _raw_stream is not None and device.index is not None:
+        return _raw_stream(device.index)
     return torch.cuda.current_stream(device).cuda_stream
+
+
+class on_device:
+    """`with on_device(dev):` - makes `dev` the current device for the library call inside, and costs nothing
+    when it already is (the usual case: one process per GPU)."""
+    __slots__ = ("dev", "ctx")
+
+    def __init__(self, dev):
+        self.dev, self.ctx = dev, None
+
+    def __enter__(self):
+        if self.dev.index is None or torch.cuda.current_device() != self.dev.index:
+            self.ctx = torch.cuda.device(self.dev)
+            self.ctx.__enter__()
+
+    def __exit__(self, *exc):
+        if self.ctx is not None:
+            self.ctx.__exit__(*exc)
+        return False
 
 
 def walsh_terms(centroids_host: torch.Tensor, mse_bits: int, layer: TqLayer):

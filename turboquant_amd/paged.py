@@ -74,7 +74,7 @@ class PagedKVPool:
         if start_pos is not None:
             start_pos = start_pos.to(device=self.device, dtype=torch.int32).contiguous()
         ly = self.quantizer._layer()
-        with torch.cuda.device(self.device):
+        with _ffi.on_device(self.device):
             _ffi.check(_ffi.lib().tq_append_kv_paged(
                 key.data_ptr(), value.data_ptr(), _ffi.dtype_tag(self.dtype), B, T, H, key.stride(0), key.stride(1),
                 key.stride(2), _ffi.ptr(start_pos), block_table.data_ptr(), block_table.shape[1], C.byref(ly),
@@ -108,7 +108,7 @@ class PagedKVPool:
         if max_tokens is None:
             max_tokens = int(run_len.max())
         ly = self.quantizer._layer()
-        with torch.cuda.device(self.device):
+        with _ffi.on_device(self.device):
             _ffi.check(_ffi.lib().tq_append_kv_from_blocks(
                 key_cache.data_ptr(), value_cache.data_ptr(), _ffi.dtype_tag(self.dtype), B, int(max_tokens),
                 self.num_kv_heads, key_cache.stride(0), key_cache.stride(1), key_cache.stride(2), src_table.data_ptr(),
@@ -137,7 +137,7 @@ class PagedKVPool:
         if any(t.shape != (B,) for t in arrs):
             raise ValueError("row0, run_len and start_pos must have one entry per row of block_table")
         ly = self.quantizer._layer()
-        with torch.cuda.device(self.device):
+        with _ffi.on_device(self.device):
             _ffi.check(_ffi.lib().tq_append_kv_ragged(
                 key.data_ptr(), value.data_ptr(), _ffi.dtype_tag(self.dtype), B, int(max_run), self.num_kv_heads,
                 key.stride(0), key.stride(1), arrs[0].data_ptr(), arrs[1].data_ptr(), arrs[2].data_ptr(),
@@ -250,14 +250,14 @@ class PagedKVPool:
                 rl_ptr = recent_len.data_ptr()
         ly = self.quantizer._layer()
         if static_scratch:
-            with torch.cuda.device(self.device):
+            with _ffi.on_device(self.device):
                 _ffi.check(_ffi.lib().tq_decode_attn_paged_noalloc(
                     query.data_ptr(), _ffi.dtype_tag(query.dtype), B, Hq, self.num_kv_heads, self.data.data_ptr(),
                     self.num_pages, bt.data_ptr(), bt_stride, seq_lens.data_ptr(), float(scale), C.byref(ly),
                     C.byref(self.layout), rk_ptr, rv_ptr, rows, rs[0], rs[1], rs[2], rl_ptr, out.data_ptr(),
                     n_split, _ffi.stream_ptr(self.device)), "tq_decode_attn_paged_noalloc")
             return out
-        with torch.cuda.device(self.device):
+        with _ffi.on_device(self.device):
             _ffi.check(_ffi.lib().tq_decode_attn_paged_stages(
                 query.data_ptr(), _ffi.dtype_tag(query.dtype), B, Hq, self.num_kv_heads, self.data.data_ptr(),
                 self.num_pages, bt.data_ptr(), bt_stride, seq_lens.data_ptr(), float(scale), C.byref(ly),
@@ -312,7 +312,7 @@ class PagedKVPool:
         if out is None:
             out = torch.empty_like(query)
         ly = self.quantizer._layer()
-        with torch.cuda.device(self.device):
+        with _ffi.on_device(self.device):
             _ffi.check(_ffi.lib().tq_decode_attn_paged_ring(
                 query.data_ptr(), _ffi.dtype_tag(query.dtype), B, Hq, self.num_kv_heads, self.data.data_ptr(),
                 self.num_pages, bt.data_ptr(), bt_stride, seq_lens.data_ptr(), float(scale), C.byref(ly),

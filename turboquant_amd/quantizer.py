@@ -106,9 +106,23 @@ class TurboQuantMSE(torch.nn.Module):
         self.register_buffer("_PiT", self.Pi.T.contiguous(), persistent=False)
         self._centroids_host = centroids.detach().float().cpu()
         self._splits = None           # (Pi, Pi^T[, S, S^T]) as bf16 term triples, built on first GPU use
+        self._layer_cache = None      # (key, TqLayer): the descriptor of the buffers as they are now
 
     # -- library plumbing ---------------------------------------------------------
     def _layer(self, S: Optional[torch.Tensor] = None, ST: Optional[torch.Tensor] = None) -> _ffi.TqLayer:
+        # One descriptor per state of the buffers: building it costs more host time than a decode call has to
+        # spare (a dozen buffer look-ups and a library call), so it is kept until a buffer moves or is written.
+        Pi, cen, thr = self.Pi, self.centroids, self.decision_boundaries
+        state = (Pi.data_ptr(), Pi._version, cen.data_ptr(), cen._version, thr.data_ptr(), thr._version,
+                 None if S is None else (S.data_ptr(), S._version, None if ST is None else ST.data_ptr()))
+        cached = self._layer_cache
+        if cached is not None and cached[0] == state:
+            return cached[1]
+        ly = self._build_layer(S, ST)
+        self._layer_cache = (state, ly)
+        return ly
+
+    def _build_layer(self, S: Optional[torch.Tensor] = None, ST: Optional[torch.Tensor] = None) -> _ffi.TqLayer:
         if self.Pi.dtype != torch.float32:
             raise TypeError("the kernels need float32 rotation / codebook buffers")
         if self._PiT.device != self.Pi.device or self._PiT.data_ptr() == 0:
