@@ -603,6 +603,47 @@ def test_four_bit_keys_staged_through_lds(gpu, d, vb, Hq, Hkv, dtype):
     _variant_against_default(gpu, "lds_stage", d, 4, vb, Hq, Hkv, dtype, exact=True)
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,d,key_bits,vb,dtype", [(201, 4, 1, 128, 3, 4, torch.bfloat16), (201, 2, 1, 128, 4, 2, torch.bfloat16),
+                                                           (101, 3, 1, 256, 3, 2, torch.float16), (401, 1, 1, 64, 3, 4, torch.bfloat16),
+                                                           (70, 12, 2, 128, 2, 4, torch.bfloat16)])
+def test_preparation_with_several_groups_of_heads_per_workgroup(gpu, B, Hq, Hkv, d, key_bits, vb, dtype):
+    """A launch of more (group of query heads, 32 coordinates) units than the card holds at once packs as many whole
+    groups as fit eight rows into one preparation workgroup (two groups of 4 heads, four of 2, eight of 1; an odd
+    number of groups leaves the last workgroup partly empty).  The operands of a group do not depend on its
+    neighbours: the batch must equal, bit for bit, the same sequences decoded 32 at a time (one group per workgroup),
+    compressed-only and with exact recent tokens, and a sequence of it the oracle (score.py:84-173)."""
+    g = torch.Generator().manual_seed(B + 7 * Hq + d)
+    lens = [int(x) for x in torch.randint(20, 90, (B,), generator=g)]
+    lens[3] = 0
+    ring = 24
+    n_log = 6
+    n_pages = B * n_log + 1
+    pool, tq = _make_pool(gpu, d, key_bits, vb, Hkv, n_pages, dtype, seed=81)
+    k = torch.randn(B, max(lens), Hkv, d, generator=g).to(dtype)
+    v = torch.randn(B, max(lens), Hkv, d, generator=g).to(dtype)
+    q = torch.randn(B, Hq, d, generator=g).to(dtype).to(gpu)
+    table = torch.randperm(n_pages, generator=g)[: B * n_log].to(torch.int32).view(B, n_log).to(gpu)
+    pool.append(k.to(gpu), v.to(gpu), table)
+    seq = torch.tensor(lens, dtype=torch.int32, device=gpu)
+    cache = torch.randn(2, n_pages, 16, Hkv, d, generator=g).to(dtype).to(gpu)
+    _progress(f"packed preparation B={B} Hq={Hq} Hkv={Hkv} d={d} kb={key_bits} {dtype}")
+    whole = pool.decode_attention(q, table, seq, n_split=2, max_len=max(lens)).clone()
+    whole_h = pool.decode_attention_ring(q, table, seq, cache[0], cache[1], ring, n_split=2, max_len=max(lens)).clone()
+    for b0 in range(0, B, 32):
+        sl = slice(b0, min(B, b0 + 32))
+        part = pool.decode_attention(q[sl], table[sl], seq[sl], n_split=2, max_len=max(lens))
+        part_h = pool.decode_attention_ring(q[sl], table[sl], seq[sl], cache[0], cache[1], ring, n_split=2, max_len=max(lens))
+        torch.cuda.synchronize()
+        assert torch.equal(whole[sl], part), b0
+        assert torch.equal(whole_h[sl], part_h), b0
+    assert torch.count_nonzero(whole[3]) == 0
+    for b in (0, B - 1):
+        idx, sgn, norms, rn, vd, vs, vz = [t.cpu() for t in pool.export_flat(table[b], lens[b])]
+        ref = O.hybrid_attention(q[b:b + 1].cpu(), key_code(idx, sgn, rn, norms, key_bits - 1), value_code(vd, vs, vz, vb),
+                                 lens[b], params_of(tq), Hkv, None, None)
+        assert cosine(whole[b:b + 1].cpu(), ref) >= COS_GATE, b
+
+
 @pytest.mark.parametrize("rows,n_parts,d,dtype", [(64, 64, 256, torch.bfloat16), (64, 65, 256, torch.float16),
                                                   (3, 9, 256, torch.float32), (100, 33, 128, torch.bfloat16),
                                                   (7, 5, 128, torch.float32), (129, 17, 128, torch.float16),

@@ -815,7 +815,8 @@ static_assert(TAIL_THREADS == PREP_COLS * PREP_SLICES, "the two roles share a wo
 template <int PER, int DT, bool PAGED>
 __global__ void __launch_bounds__(TAIL_THREADS, 4)
 prep_tail_kernel(TailArgs A, int n_tail, int B, int Gq, tq_layer ly, float* __restrict__ q_rot, float* __restrict__ q_sk,
-                 float* __restrict__ q_stat, uint32_t* __restrict__ qa_pack, unsigned long long* __restrict__ arrivals) {
+                 float* __restrict__ q_stat, uint32_t* __restrict__ qa_pack, unsigned long long* __restrict__ arrivals,
+                 int prep_gpw) {
   extern __shared__ __align__(16) float sm[];
   const int id = blockIdx.x;
   if (id < n_tail) {
@@ -823,9 +824,9 @@ prep_tail_kernel(TailArgs A, int n_tail, int B, int Gq, tq_layer ly, float* __re
     exact_tail_words_body<DT, 1, PAGED, true>(A, id % A.Hkv, (id / A.Hkv) % B, id / per_z, sm);
   } else {
     const int words = ly.d / PREP_COLS, p = id - n_tail;
-    // (the arrival counter of this group of query heads, for a page kernel that merges its splits itself)
-    if (arrivals != nullptr && p % words == 0 && threadIdx.x == 0) arrivals[p / words] = 0ull;
-    prep_query_body<PER, DT>(A.q, Gq, ly, A.sm_scale, q_rot, q_sk, q_stat, qa_pack, p / words, p % words, sm);
+    // (arrivals: the arrival counters of the groups of query heads, zeroed for a page kernel that merges its splits itself)
+    prep_query_body<PER, DT>(A.q, Gq, prep_gpw, (int64_t)B * A.Hq, ly, A.sm_scale, q_rot, q_sk, q_stat, qa_pack, arrivals,
+                             p / words, p % words, sm);
   }
 }
 
@@ -1173,14 +1174,19 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   }
   if ((stages & 1) && !fused) {
     if (!layer->Pi || !layer->PiT || !layer->S || !layer->ST || !layer->centroids) return TQ_ENULL;
-    const int n_prep = (B * Hq / Gq) * (d / PREP_COLS);
+    // (in the launch shared with the tail a compute unit holds two workgroups: beyond that the preparation
+    // workgroups take several groups of heads each, see prep_query_body)
+    const int prep_gpw = prep_groups_per_workgroup(Gq, n_tail + (int64_t)(B * Hq / Gq) * (d / PREP_COLS),
+                                                   2 * (int64_t)device_compute_units());
+    const int prep_rows = Gq * prep_gpw;                          // query rows of a preparation workgroup
+    const int n_prep = (B * Hq + prep_rows - 1) / prep_rows * (d / PREP_COLS);
     // Whole hybrid step on the matrix-core path: the exact tail shares the preparation's launch (the tail
     // workgroups first, so that the longer-running ones start first).  The kernel is built for 128 registers
     // per lane and the tail's LDS is sized by the rows it holds, so two workgroups fit a compute unit; with more
     // workgroups than that the rest follow as slots free up, which still measured faster than a launch each
     // (16 x 8192: 48.9 -> 45.2 us per step, 32 x 32768: 223.6 -> 221.5 us).
     size_t fsm = tail_words_smem(d, recent_rows, ta.tile_words);
-    if (prep_smem_bytes(Gq, d) > fsm) fsm = prep_smem_bytes(Gq, d);
+    if (prep_smem_bytes(prep_rows, d) > fsm) fsm = prep_smem_bytes(prep_rows, d);
     // ... unless the tail's tiles leave room for one workgroup per compute unit only (head_dim 256 with 128 exact
     // tokens: 139 KB) and the grid is larger than the card: the preparation workgroups would queue behind that
     // LDS size too (128 x 2048, 16 q / 2 KV heads: 109.7 us per step fused, 88.1 as two launches)
@@ -1194,7 +1200,7 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
       if (e != hipSuccess) return (int)e;                                                                            \
     }                                                                                                                \
     kern<<<dim3((unsigned)(n_tail + n_prep)), dim3(TAIL_THREADS), fsm, st>>>(ta, n_tail, B, Gq, *layer, q_rot, q_sk,  \
-                                                                            q_stat, qa_pack, fm.counters);           \
+                                                                            q_stat, qa_pack, fm.counters, prep_gpw); \
   }
 #define TQ_LAUNCH_PT_DT(PER, PAGED)                                \
   {                                                                \

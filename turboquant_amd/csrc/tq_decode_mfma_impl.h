@@ -270,7 +270,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
     const int kv_heads = Hkv / kv_div, grp = h / kv_heads;
     h = (h - grp * kv_heads) * kv_div + grp;
   }
-  if (skew16 > 0) {
+  if (DS == 2 && skew16 > 0) {                                  // (only the launcher of DS == 2 kernels passes a skew)
     // (n_seq arrives with the other kernel arguments; the grid's size would be one more scalar load of the
     // launch's implicit data in front of everything that depends on the sequence)
     const int late = b >= n_seq;
@@ -434,7 +434,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   const int per_split = (n_blocks + n_split - 1) / n_split;
   int blk_begin = split * per_split;
   int blk_end = min(n_blocks, blk_begin + per_split);
-  if (skew16 > 0) {
+  if (DS == 2 && skew16 > 0) {
     const int moved = min(NGRP * ((((per_split + NGRP - 1) / NGRP) * skew16 + 8) >> 4), per_split);
     if (split & 1) blk_begin = min(blk_begin + moved, blk_end);
     else blk_end = min(blk_end + moved, n_blocks);

@@ -66,25 +66,40 @@ __device__ __forceinline__ float wave_sum_dpp(float v) {
 // PER = matrix rows per thread = d / PREP_SLICES; DT = element type of the query (a template parameter:
 // a run-time switch would put each query load under a branch, and the loads would wait for one another)
 // (a device function: the stand-alone kernel and the launch that shares its grid with the exact-tail
-// workgroups both run it; `group` / `word` are the workgroup's coordinates, `sm` its dynamic LDS)
+// workgroups both run it; `unit` / `word` are the workgroup's coordinates, `sm` its dynamic LDS.)
+// A workgroup works on gpw consecutive groups of G heads (gpw x G <= ROT_MAX_ROWS rows; rows of consecutive
+// groups are consecutive), the last workgroup possibly on fewer (n_rows = all rows = groups x G).  One group per
+// workgroup is the shortest chain and what a launch that fits the card at once wants; a launch of thousands of
+// units is bound by how many workgroups it takes, and then two groups of 4 heads, four of 2, ... share one
+// (prep_groups_per_workgroup).  `arrivals`: the groups' arrival counters, zeroed here for a page kernel that
+// merges its splits itself.
+// units = workgroups of the launch with one group each, slots = workgroups the card holds at once
+__host__ __device__ inline int prep_groups_per_workgroup(int G, int64_t units, int64_t slots) {
+  return units > slots && G >= 1 && G <= ROT_MAX_ROWS ? ROT_MAX_ROWS / G : 1;
+}
+
 template <int PER, int DT>
-__device__ __forceinline__ void prep_query_body(const void* __restrict__ q, int G, const tq_layer& ly, float sm_scale,
-                                                float* __restrict__ q_rot, float* __restrict__ q_sk,
+__device__ __forceinline__ void prep_query_body(const void* __restrict__ q, int G, int gpw, int64_t n_rows, const tq_layer& ly,
+                                                float sm_scale, float* __restrict__ q_rot, float* __restrict__ q_sk,
                                                 float* __restrict__ q_stat, uint32_t* __restrict__ qa_pack,
-                                                int64_t group, int word, float* sm) {
+                                                unsigned long long* __restrict__ arrivals, int64_t unit, int word,
+                                                float* sm) {
   const int d = ly.d, tid = threadIdx.x, jl = tid % PREP_COLS, sl = tid / PREP_COLS;
   const int j = word * PREP_COLS + jl;
+  const int RG = G * gpw;                                              // rows a workgroup has room for
+  const int64_t row0 = unit * RG, group0 = unit * gpw;
+  const int R = (int)(n_rows - row0 < RG ? n_rows - row0 : RG);        // rows of this workgroup (a multiple of G)
+  if (arrivals != nullptr && word == 0 && tid < gpw && tid * G < R) arrivals[group0 + tid] = 0ull;
   // every global load of the kernel is issued here, before anything waits, the query first: loads
   // return in order, so the query can go to shared memory (and its statistics be taken) while the
   // matrix slices, which do not depend on it, are still on their way
-  const int64_t row0 = group * G;
   constexpr int QPT = ROT_MAX_ROWS * 256 / (PREP_COLS * PREP_SLICES);   // query elements per thread, d <= 256
   float qv[QPT];
 #pragma unroll
   for (int k = 0; k < QPT; ++k) {
     const int o = tid + k * (PREP_COLS * PREP_SLICES);
-    const float x = Elem<DT>::load(q, row0 * d + min(o, G * d - 1));      // unconditional, clamped
-    qv[k] = o < G * d ? x : 0.0f;
+    const float x = Elem<DT>::load(q, row0 * d + min(o, R * d - 1));      // unconditional, clamped
+    qv[k] = o < R * d ? x : 0.0f;
   }
   float mp[PER], ms[PER];
 #pragma unroll
@@ -99,17 +114,17 @@ __device__ __forceinline__ void prep_query_body(const void* __restrict__ q, int 
     cs1[k] = c < d ? ly.Pi_colsum[c] : 0.0f;
     cs2[k] = c < d ? ly.S_colsum[c] : 0.0f;
   }
-  float* sq = sm;                                   // [G][d] raw query
-  float* pa = sq + G * d;                           // [PREP_SLICES][G][PREP_COLS]
-  float* pb = pa + PREP_SLICES * G * PREP_COLS;
-  float* srot = pb + PREP_SLICES * G * PREP_COLS;   // [G][PREP_COLS]
-  float* ssk = srot + G * PREP_COLS;
-  float* stat = ssk + G * PREP_COLS;                // [G][4]
+  float* sq = sm;                                   // [RG][d] raw query
+  float* pa = sq + RG * d;                          // [PREP_SLICES][RG][PREP_COLS]
+  float* pb = pa + PREP_SLICES * RG * PREP_COLS;
+  float* srot = pb + PREP_SLICES * RG * PREP_COLS;  // [RG][PREP_COLS]
+  float* ssk = srot + RG * PREP_COLS;
+  float* stat = ssk + RG * PREP_COLS;               // [RG][4]
   float* coefs = stat + 4 * ROT_MAX_ROWS;           // [16]
 #pragma unroll
   for (int k = 0; k < QPT; ++k) {
     const int o = tid + k * (PREP_COLS * PREP_SLICES);
-    if (o < G * d) sq[o] = qv[k];
+    if (o < R * d) sq[o] = qv[k];
   }
   const int mb = ly.mse_bits;
   int nx = 0;
@@ -140,7 +155,7 @@ __device__ __forceinline__ void prep_query_body(const void* __restrict__ q, int 
   __syncthreads();
   {  // row statistics: one wavefront per row
     const int lane = tid & 63, wave = tid >> 6, n_wave = blockDim.x >> 6;
-    for (int r = wave; r < G; r += n_wave) {
+    for (int r = wave; r < R; r += n_wave) {
       float ss = 0.0f, s1 = 0.0f, s2 = 0.0f;
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
@@ -174,7 +189,7 @@ __device__ __forceinline__ void prep_query_body(const void* __restrict__ q, int 
     for (int r = 0; r < ROT_MAX_ROWS; ++r) a[r] = b[r] = 0.0f;
 #pragma unroll
     for (int r = 0; r < ROT_MAX_ROWS; ++r) {
-      if (r < G) {
+      if (r < R) {
 #pragma unroll
         for (int k4 = 0; k4 < PER / 4; ++k4) {
           const float4 x = *(const float4*)(sq + r * d + i0 + 4 * k4);
@@ -189,20 +204,20 @@ __device__ __forceinline__ void prep_query_body(const void* __restrict__ q, int 
     }
 #pragma unroll
     for (int r = 0; r < ROT_MAX_ROWS; ++r) {
-      if (r < G) {
-        pa[(sl * G + r) * PREP_COLS + jl] = a[r];
-        pb[(sl * G + r) * PREP_COLS + jl] = b[r];
+      if (r < R) {
+        pa[(sl * RG + r) * PREP_COLS + jl] = a[r];
+        pb[(sl * RG + r) * PREP_COLS + jl] = b[r];
       }
     }
   }
   __syncthreads();
-  for (int o2 = tid; o2 < 2 * G * PREP_COLS; o2 += blockDim.x) {      // first half: rotation, second: sketch
-    const bool sk = o2 >= G * PREP_COLS;
-    const int o = sk ? o2 - G * PREP_COLS : o2, r = o / PREP_COLS, c = o - r * PREP_COLS;
+  for (int o2 = tid; o2 < 2 * R * PREP_COLS; o2 += blockDim.x) {      // first half: rotation, second: sketch
+    const bool sk = o2 >= R * PREP_COLS;
+    const int o = sk ? o2 - R * PREP_COLS : o2, r = o / PREP_COLS, c = o - r * PREP_COLS;
     const float* part = sk ? pb : pa;
     float acc = 0.0f;
 #pragma unroll
-    for (int k = 0; k < PREP_SLICES; ++k) acc += part[(k * G + r) * PREP_COLS + c];
+    for (int k = 0; k < PREP_SLICES; ++k) acc += part[(k * RG + r) * PREP_COLS + c];
     (sk ? ssk : srot)[o] = acc;
     (sk ? q_sk : q_rot)[(row0 + r) * d + word * PREP_COLS + c] = acc;
   }
@@ -213,12 +228,16 @@ __device__ __forceinline__ void prep_query_body(const void* __restrict__ q, int 
   // except that a small negative value keeps its sign on the zero code, which adds nothing in the MFMA) and
   // gets the rounded values back for the residual with its inverse (v_cvt_scalef32_pk32_f32_fp6).
   // Code j of a conversion comes from element j / 2 of its first (j even) or second (j odd) operand.
-  if (tid < ntp * 8) {
+  // Lane (term plane, row g) belongs to head g % G of the workgroup's group g / G.  The operand rows of the heads
+  // a group does not have are zero: with one group per workgroup the lanes beyond its heads write them (lane g
+  // the rows of head g), with several groups the lane of head h writes those of h + G, h + 2 G, ... below 8.
+  if (tid < ntp * 8 && ((tid & 7) < R || gpw == 1)) {
     typedef float f32x16_t __attribute__((ext_vector_type(16)));
     typedef float f32x32_t __attribute__((ext_vector_type(32)));
     typedef uint32_t u32x6_t __attribute__((ext_vector_type(6)));
     const int tp = tid >> 3, g = tid & 7;
-    const bool is_sign = tp == ntp - 1, live = g < G;
+    const bool is_sign = tp == ntp - 1, live = g < R;
+    const int gi = live ? g / G : 0, hg = g - gi * G;      // (not live: head g of the workgroup's only group)
     const int gs = live ? g : 0;
     // the decode kernel extracts three of the four bits of a nibble in place, where they are the fp4
     // numbers 1, 2 and 4 (after its block scale): the query side divides them out
@@ -239,16 +258,21 @@ __device__ __forceinline__ void prep_query_body(const void* __restrict__ q, int 
       else va[kloc >> 1] = v;
     }
     const int i = word >> 2, kw = word & 3;
-    uint32_t* dst = qa_pack + group * (int64_t)(ntp * wpl * 2 * 64 * 8);
+    uint32_t* dst = qa_pack + (group0 + gi) * (int64_t)(ntp * wpl * 2 * 64 * 8);
     const float one = 1.0f;
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
       u32x6_t code;
       // (inline assembly with early-clobber results: the conversions read their sources over several passes)
       asm volatile("v_cvt_scalef32_2xpk16_fp6_f32 %0, %1, %2, %3" : "=&v"(code) : "v"(va), "v"(vb), "v"(one));
-      uint32_t* o = dst + (((tp * wpl + i) * 2 + (t >> 1)) * 64 + 2 * g + (t & 1) + 16 * kw) * 8;
+      uint32_t* o = dst + (((tp * wpl + i) * 2 + (t >> 1)) * 64 + 2 * hg + (t & 1) + 16 * kw) * 8;
       *(uint4*)o = make_uint4(code[0], code[1], code[2], code[3]);
       *(uint2*)(o + 4) = make_uint2(code[4], code[5]);
+      for (int ha = hg + G; gpw > 1 && ha < 8; ha += G) {        // heads the group does not have
+        uint32_t* z = o + (2 * (ha - hg)) * 8;
+        *(uint4*)z = make_uint4(0u, 0u, 0u, 0u);
+        *(uint2*)(z + 4) = make_uint2(0u, 0u);
+      }
       if (t < 3) {
         f32x32_t r;
         asm volatile("v_cvt_scalef32_pk32_f32_fp6 %0, %1, %2" : "=&v"(r) : "v"(code), "v"(one));
@@ -481,8 +505,8 @@ __device__ __forceinline__ void prep_unit256(const void* __restrict__ q, int dty
 }
 
 // LDS bytes of a preparation workgroup
-static inline size_t prep_smem_bytes(int G, int d) {
-  return (size_t)(G * d + 2 * PREP_SLICES * G * PREP_COLS + 2 * G * PREP_COLS + 4 * ROT_MAX_ROWS + 32) * sizeof(float);
+static inline size_t prep_smem_bytes(int RG, int d) {       // RG: query rows of a workgroup
+  return (size_t)(RG * d + 2 * PREP_SLICES * RG * PREP_COLS + 2 * RG * PREP_COLS + 4 * ROT_MAX_ROWS + 32) * sizeof(float);
 }
 
 }  // namespace tq
