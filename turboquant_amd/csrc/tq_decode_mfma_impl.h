@@ -997,6 +997,9 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   }
   __syncthreads();
   // merge of the walkers: thread -> (head, channel); loads are unconditional (clamped), stores guarded
+  // A launch that merges its splits itself and has a single split and no other partial is done here: the walkers'
+  // sum is the result (what the merge below would compute from the one partial, without the trip through memory).
+  const bool direct = fm.out != nullptr && n_split == 1 && fm.n_extra == 0;
 #pragma unroll
   for (int k = 0; k < 8 * D / (MF_WAVES * 64); ++k) {
     const int o = tid + k * (MF_WAVES * 64);
@@ -1016,7 +1019,10 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
       ll = fmaf(wgt, l_w[w], ll);
       aa = fmaf(wgt, a_w[w], aa);
     }
-    if (live) {
+    if (live && direct) {
+      const float inv = ll > 0.0f ? 1.0f / ll : 0.0f;
+      store_from_f32(fm.out, ((int64_t)b * Hq + h * G + g) * D + ch, aa * inv, fm.out_dtype);
+    } else if (live) {
       float* out = parts + (((int64_t)b * Hq + h * G + g) * n_parts + split) * (D + 2);
       if (fm.out != nullptr) {                 // read by another workgroup of this launch: device-coherent stores
         if (ch == 0) { store_coherent(out, mm); store_coherent(out + 1, ll); }
@@ -1030,7 +1036,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   // ---------------------------------------------------------------- merge of the splits inside this launch
   // Every workgroup counts itself in after its partial has been written (one atomic increment of the group's
   // counter, which the preparation kernel of this step has zeroed); the one that counts last merges.
-  if (fm.out != nullptr) {
+  if (fm.out != nullptr && !direct) {
     __shared__ int s_last;
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");      // the partial's stores have completed ...
     __syncthreads();                                            // ... in every wavefront
