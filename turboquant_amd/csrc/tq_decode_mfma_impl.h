@@ -997,9 +997,10 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   }
   __syncthreads();
   // merge of the walkers: thread -> (head, channel); loads are unconditional (clamped), stores guarded
-  // A launch that merges its splits itself and has a single split and no other partial is done here: the walkers'
-  // sum is the result (what the merge below would compute from the one partial, without the trip through memory).
-  const bool direct = fm.out != nullptr && n_split == 1 && fm.n_extra == 0;
+  // A launch that merges its splits itself and has a single split is done here: the walkers' sum, merged with the
+  // exact tail's partial if there is one (an earlier launch wrote it: plain loads), is the result - what the merge
+  // below would compute from the same parts in the same order, without the trip through memory and the counting.
+  const bool direct = fm.out != nullptr && n_split == 1 && fm.n_extra <= 1;
 #pragma unroll
   for (int k = 0; k < 8 * D / (MF_WAVES * 64); ++k) {
     const int o = tid + k * (MF_WAVES * 64);
@@ -1019,9 +1020,19 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
       ll = fmaf(wgt, l_w[w], ll);
       aa = fmaf(wgt, a_w[w], aa);
     }
-    if (live && direct) {
+    if (live && direct && fm.n_extra == 0) {
       const float inv = ll > 0.0f ? 1.0f / ll : 0.0f;
       store_from_f32(fm.out, ((int64_t)b * Hq + h * G + g) * D + ch, aa * inv, fm.out_dtype);
+    } else if (live && direct) {
+      const float* x = parts + (((int64_t)b * Hq + h * G + g) * n_parts + 1) * (D + 2);     // the exact tail's part
+      const float m_x = x[0], l_x = x[1], a_x = x[2 + ch];
+      float top = MF_NEG;
+      if (ll > 0.0f) top = fmaxf(top, mm);
+      if (l_x > 0.0f) top = fmaxf(top, m_x);
+      const float w0 = ll > 0.0f ? __expf(mm - top) : 0.0f, w1 = l_x > 0.0f ? __expf(m_x - top) : 0.0f;
+      const float l_all = fmaf(w1, l_x, fmaf(w0, ll, 0.0f)), a_all = fmaf(w1, a_x, fmaf(w0, aa, 0.0f));
+      const float inv = l_all > 0.0f ? 1.0f / l_all : 0.0f;
+      store_from_f32(fm.out, ((int64_t)b * Hq + h * G + g) * D + ch, a_all * inv, fm.out_dtype);
     } else if (live) {
       float* out = parts + (((int64_t)b * Hq + h * G + g) * n_parts + split) * (D + 2);
       if (fm.out != nullptr) {                 // read by another workgroup of this launch: device-coherent stores
