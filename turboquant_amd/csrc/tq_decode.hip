@@ -812,7 +812,7 @@ exact_tail_words_kernel(TailArgs A) {
 // far fewer workgroups than the card has compute units, so the launch takes as long as the slower of
 // the two instead of their sum plus a dispatch gap.
 static_assert(TAIL_THREADS == PREP_COLS * PREP_SLICES, "the two roles share a workgroup size");
-template <int PER, int DT, bool PAGED>
+template <int PER, int DT, bool PAGED, bool PACKED>
 __global__ void __launch_bounds__(TAIL_THREADS, 4)
 prep_tail_kernel(TailArgs A, int n_tail, int B, int Gq, tq_layer ly, float* __restrict__ q_rot, float* __restrict__ q_sk,
                  float* __restrict__ q_stat, uint32_t* __restrict__ qa_pack, unsigned long long* __restrict__ arrivals,
@@ -825,8 +825,8 @@ prep_tail_kernel(TailArgs A, int n_tail, int B, int Gq, tq_layer ly, float* __re
   } else {
     const int words = ly.d / PREP_COLS, p = id - n_tail;
     // (arrivals: the arrival counters of the groups of query heads, zeroed for a page kernel that merges its splits itself)
-    prep_query_body<PER, DT>(A.q, Gq, prep_gpw, (int64_t)B * A.Hq, ly, A.sm_scale, q_rot, q_sk, q_stat, qa_pack, arrivals,
-                             p / words, p % words, sm);
+    prep_query_body<PER, DT, PACKED>(A.q, Gq, prep_gpw, (int64_t)B * A.Hq, ly, A.sm_scale, q_rot, q_sk, q_stat, qa_pack,
+                                     arrivals, p / words, p % words, sm);
   }
 }
 
@@ -1194,7 +1194,7 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
     if (tail && ta.wide && mfma_shape && stages == 7 && !(one_per_unit && n_tail + n_prep > device_compute_units())) {
 #define TQ_LAUNCH_PT(PER, DT, PAGED)                                                                                 \
   {                                                                                                                  \
-    auto kern = prep_tail_kernel<PER, DT, PAGED>;                                                                    \
+    auto kern = prep_gpw > 1 ? prep_tail_kernel<PER, DT, PAGED, true> : prep_tail_kernel<PER, DT, PAGED, false>;     \
     if (fsm > 48 * 1024) {                                                                                           \
       hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)fsm);   \
       if (e != hipSuccess) return (int)e;                                                                            \

@@ -997,43 +997,60 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   }
   __syncthreads();
   // merge of the walkers: thread -> (head, channel); loads are unconditional (clamped), stores guarded
-  // A launch that merges its splits itself and has a single split is done here: the walkers' sum, merged with the
-  // exact tail's partial if there is one (an earlier launch wrote it: plain loads), is the result - what the merge
-  // below would compute from the same parts in the same order, without the trip through memory and the counting.
-  const bool direct = fm.out != nullptr && n_split == 1 && fm.n_extra <= 1;
-#pragma unroll
-  for (int k = 0; k < 8 * D / (MF_WAVES * 64); ++k) {
-    const int o = tid + k * (MF_WAVES * 64);
-    const bool live = o < G * D;
-    const int g = live ? o / D : 0, ch = o % D;
-    float m_w[NGRP], l_w[NGRP], a_w[NGRP], mm = MF_NEG;
+  auto walkers_sum = [&](int g, int ch, float& mm, float& ll, float& aa) {
+    float m_w[NGRP], l_w[NGRP], a_w[NGRP];
+    mm = MF_NEG;
 #pragma unroll
     for (int w = 0; w < NGRP; ++w) {
       const float* r = s_red + (w * G + g) * (D + 2);
       m_w[w] = r[0]; l_w[w] = r[1]; a_w[w] = r[2 + ch];
       mm = fmaxf(mm, m_w[w]);
     }
-    float ll = 0.0f, aa = 0.0f;
+    ll = 0.0f; aa = 0.0f;
 #pragma unroll
     for (int w = 0; w < NGRP; ++w) {
       const float wgt = __expf(m_w[w] - mm);
       ll = fmaf(wgt, l_w[w], ll);
       aa = fmaf(wgt, a_w[w], aa);
     }
-    if (live && direct && fm.n_extra == 0) {
-      const float inv = ll > 0.0f ? 1.0f / ll : 0.0f;
-      store_from_f32(fm.out, ((int64_t)b * Hq + h * G + g) * D + ch, aa * inv, fm.out_dtype);
-    } else if (live && direct) {
-      const float* x = parts + (((int64_t)b * Hq + h * G + g) * n_parts + 1) * (D + 2);     // the exact tail's part
-      const float m_x = x[0], l_x = x[1], a_x = x[2 + ch];
-      float top = MF_NEG;
-      if (ll > 0.0f) top = fmaxf(top, mm);
-      if (l_x > 0.0f) top = fmaxf(top, m_x);
-      const float w0 = ll > 0.0f ? __expf(mm - top) : 0.0f, w1 = l_x > 0.0f ? __expf(m_x - top) : 0.0f;
-      const float l_all = fmaf(w1, l_x, fmaf(w0, ll, 0.0f)), a_all = fmaf(w1, a_x, fmaf(w0, aa, 0.0f));
-      const float inv = l_all > 0.0f ? 1.0f / l_all : 0.0f;
-      store_from_f32(fm.out, ((int64_t)b * Hq + h * G + g) * D + ch, a_all * inv, fm.out_dtype);
-    } else if (live) {
+  };
+  // A launch that merges its splits itself and has a single split is done here (the kernels whose wavefronts work
+  // alone; a path of its own, so that the others' epilogue stays what it was): the walkers' sum, merged with the
+  // exact tail's partial if there is one (an earlier launch wrote it: plain loads), is the result - what the merge
+  // further down would compute from the same parts in the same order, without the trip through memory and the counting.
+  if (DS == 1 && fm.out != nullptr && n_split == 1 && fm.n_extra <= 1) {
+#pragma unroll
+    for (int k = 0; k < 8 * D / (MF_WAVES * 64); ++k) {
+      const int o = tid + k * (MF_WAVES * 64);
+      const bool live = o < G * D;
+      const int g = live ? o / D : 0, ch = o % D;
+      float mm, ll, aa;
+      walkers_sum(g, ch, mm, ll, aa);
+      if (live && fm.n_extra == 0) {
+        const float inv = ll > 0.0f ? 1.0f / ll : 0.0f;
+        store_from_f32(fm.out, ((int64_t)b * Hq + h * G + g) * D + ch, aa * inv, fm.out_dtype);
+      } else if (live) {
+        const float* x = parts + (((int64_t)b * Hq + h * G + g) * n_parts + 1) * (D + 2);     // the exact tail's part
+        const float m_x = x[0], l_x = x[1], a_x = x[2 + ch];
+        float top = MF_NEG;
+        if (ll > 0.0f) top = fmaxf(top, mm);
+        if (l_x > 0.0f) top = fmaxf(top, m_x);
+        const float w0 = ll > 0.0f ? __expf(mm - top) : 0.0f, w1 = l_x > 0.0f ? __expf(m_x - top) : 0.0f;
+        const float l_all = fmaf(w1, l_x, fmaf(w0, ll, 0.0f)), a_all = fmaf(w1, a_x, fmaf(w0, aa, 0.0f));
+        const float inv = l_all > 0.0f ? 1.0f / l_all : 0.0f;
+        store_from_f32(fm.out, ((int64_t)b * Hq + h * G + g) * D + ch, a_all * inv, fm.out_dtype);
+      }
+    }
+    return;
+  }
+#pragma unroll
+  for (int k = 0; k < 8 * D / (MF_WAVES * 64); ++k) {
+    const int o = tid + k * (MF_WAVES * 64);
+    const bool live = o < G * D;
+    const int g = live ? o / D : 0, ch = o % D;
+    float mm, ll, aa;
+    walkers_sum(g, ch, mm, ll, aa);
+    if (live) {
       float* out = parts + (((int64_t)b * Hq + h * G + g) * n_parts + split) * (D + 2);
       if (fm.out != nullptr) {                 // read by another workgroup of this launch: device-coherent stores
         if (ch == 0) { store_coherent(out, mm); store_coherent(out + 1, ll); }
@@ -1047,7 +1064,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   // ---------------------------------------------------------------- merge of the splits inside this launch
   // Every workgroup counts itself in after its partial has been written (one atomic increment of the group's
   // counter, which the preparation kernel of this step has zeroed); the one that counts last merges.
-  if (fm.out != nullptr && !direct) {
+  if (fm.out != nullptr) {
     __shared__ int s_last;
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");      // the partial's stores have completed ...
     __syncthreads();                                            // ... in every wavefront

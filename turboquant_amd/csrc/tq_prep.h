@@ -78,7 +78,9 @@ __host__ __device__ inline int prep_groups_per_workgroup(int G, int64_t units, i
   return units > slots && G >= 1 && G <= ROT_MAX_ROWS ? ROT_MAX_ROWS / G : 1;
 }
 
-template <int PER, int DT>
+// PACKED: gpw may exceed 1.  One group per workgroup is a build of its own (no row bounds, no head / group
+// arithmetic in the packing lanes): it is the one the latency-bound launches take, and half a microsecond shorter.
+template <int PER, int DT, bool PACKED>
 __device__ __forceinline__ void prep_query_body(const void* __restrict__ q, int G, int gpw, int64_t n_rows, const tq_layer& ly,
                                                 float sm_scale, float* __restrict__ q_rot, float* __restrict__ q_sk,
                                                 float* __restrict__ q_stat, uint32_t* __restrict__ qa_pack,
@@ -86,10 +88,10 @@ __device__ __forceinline__ void prep_query_body(const void* __restrict__ q, int 
                                                 float* sm) {
   const int d = ly.d, tid = threadIdx.x, jl = tid % PREP_COLS, sl = tid / PREP_COLS;
   const int j = word * PREP_COLS + jl;
-  const int RG = G * gpw;                                              // rows a workgroup has room for
-  const int64_t row0 = unit * RG, group0 = unit * gpw;
-  const int R = (int)(n_rows - row0 < RG ? n_rows - row0 : RG);        // rows of this workgroup (a multiple of G)
-  if (arrivals != nullptr && word == 0 && tid < gpw && tid * G < R) arrivals[group0 + tid] = 0ull;
+  const int RG = PACKED ? G * gpw : G;                                 // rows a workgroup has room for
+  const int64_t row0 = unit * RG, group0 = PACKED ? unit * gpw : unit;
+  const int R = PACKED ? (int)(n_rows - row0 < RG ? n_rows - row0 : RG) : G;      // rows of this workgroup (a multiple of G)
+  if (arrivals != nullptr && word == 0 && tid < (PACKED ? gpw : 1) && tid * G < R) arrivals[group0 + tid] = 0ull;
   // every global load of the kernel is issued here, before anything waits, the query first: loads
   // return in order, so the query can go to shared memory (and its statistics be taken) while the
   // matrix slices, which do not depend on it, are still on their way
@@ -231,13 +233,13 @@ __device__ __forceinline__ void prep_query_body(const void* __restrict__ q, int 
   // Lane (term plane, row g) belongs to head g % G of the workgroup's group g / G.  The operand rows of the heads
   // a group does not have are zero: with one group per workgroup the lanes beyond its heads write them (lane g
   // the rows of head g), with several groups the lane of head h writes those of h + G, h + 2 G, ... below 8.
-  if (tid < ntp * 8 && ((tid & 7) < R || gpw == 1)) {
+  if (tid < ntp * 8 && ((tid & 7) < R || !PACKED || gpw == 1)) {
     typedef float f32x16_t __attribute__((ext_vector_type(16)));
     typedef float f32x32_t __attribute__((ext_vector_type(32)));
     typedef uint32_t u32x6_t __attribute__((ext_vector_type(6)));
     const int tp = tid >> 3, g = tid & 7;
     const bool is_sign = tp == ntp - 1, live = g < R;
-    const int gi = live ? g / G : 0, hg = g - gi * G;      // (not live: head g of the workgroup's only group)
+    const int gi = PACKED && live ? g / G : 0, hg = g - gi * G;      // (not live: head g of the workgroup's only group)
     const int gs = live ? g : 0;
     // the decode kernel extracts three of the four bits of a nibble in place, where they are the fp4
     // numbers 1, 2 and 4 (after its block scale): the query side divides them out
@@ -268,7 +270,7 @@ __device__ __forceinline__ void prep_query_body(const void* __restrict__ q, int 
       uint32_t* o = dst + (((tp * wpl + i) * 2 + (t >> 1)) * 64 + 2 * hg + (t & 1) + 16 * kw) * 8;
       *(uint4*)o = make_uint4(code[0], code[1], code[2], code[3]);
       *(uint2*)(o + 4) = make_uint2(code[4], code[5]);
-      for (int ha = hg + G; gpw > 1 && ha < 8; ha += G) {        // heads the group does not have
+      for (int ha = hg + G; PACKED && gpw > 1 && ha < 8; ha += G) {        // heads the group does not have
         uint32_t* z = o + (2 * (ha - hg)) * 8;
         *(uint4*)z = make_uint4(0u, 0u, 0u, 0u);
         *(uint2*)(z + 4) = make_uint2(0u, 0u);

@@ -70,13 +70,13 @@ rotate_query_kernel(const void* __restrict__ q, int dtype, int64_t rows, int R, 
   }
 }
 
-template <int PER, int DT>
+template <int PER, int DT, bool PACKED>
 __global__ void __launch_bounds__(PREP_COLS * PREP_SLICES)
 prep_query_kernel(const void* __restrict__ q, int G, int gpw, int64_t n_rows, tq_layer ly, float sm_scale,
                   float* __restrict__ q_rot, float* __restrict__ q_sk, float* __restrict__ q_stat,
                   uint32_t* __restrict__ qa_pack, unsigned long long* __restrict__ arrivals) {
   extern __shared__ __align__(16) float sm[];
-  prep_query_body<PER, DT>(q, G, gpw, n_rows, ly, sm_scale, q_rot, q_sk, q_stat, qa_pack, arrivals, blockIdx.x, blockIdx.y, sm);
+  prep_query_body<PER, DT, PACKED>(q, G, gpw, n_rows, ly, sm_scale, q_rot, q_sk, q_stat, qa_pack, arrivals, blockIdx.x, blockIdx.y, sm);
 }
 
 // The same preparation cut into more, smaller workgroups: one per unit = (hp consecutive heads of a group,
@@ -396,12 +396,20 @@ int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* 
     const int64_t rows_per_wg = (int64_t)G * gpw;
     size_t smem = prep_smem_bytes(G * gpw, d);
     const dim3 grid((unsigned)((rows + rows_per_wg - 1) / rows_per_wg), d / PREP_COLS), block(PREP_COLS * PREP_SLICES);
-#define TQ_PREP(PER, DT) prep_query_kernel<PER, DT><<<grid, block, smem, st>>>(q, G, gpw, rows, *layer, sm_scale, q_rot, q_sk, q_stat, qa_pack, arrivals)
+#define TQ_PREP(PER, DT)                                                                                               \
+  {                                                                                                                    \
+    if (gpw > 1)                                                                                                       \
+      prep_query_kernel<PER, DT, true><<<grid, block, smem, st>>>(q, G, gpw, rows, *layer, sm_scale, q_rot, q_sk, q_stat, \
+                                                                  qa_pack, arrivals);                                   \
+    else                                                                                                               \
+      prep_query_kernel<PER, DT, false><<<grid, block, smem, st>>>(q, G, gpw, rows, *layer, sm_scale, q_rot, q_sk, q_stat, \
+                                                                   qa_pack, arrivals);                                  \
+  }
 #define TQ_PREP_DT(PER)                              \
   {                                                  \
-    if (dtype == TQ_BF16) TQ_PREP(PER, TQ_BF16);     \
-    else if (dtype == TQ_F16) TQ_PREP(PER, TQ_F16);  \
-    else if (dtype == TQ_F32) TQ_PREP(PER, TQ_F32);  \
+    if (dtype == TQ_BF16) TQ_PREP(PER, TQ_BF16)      \
+    else if (dtype == TQ_F16) TQ_PREP(PER, TQ_F16)   \
+    else if (dtype == TQ_F32) TQ_PREP(PER, TQ_F32)   \
     else return TQ_EINVAL;                           \
   }
     if (d == 64) TQ_PREP_DT(4)
