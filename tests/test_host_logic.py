@@ -339,3 +339,24 @@ def test_quotient_of_bf16_numbers_rounds_like_its_product_with_a_reciprocal():
         r = (r0.view(np.int32) + step).view(np.float32)
         got = bf16_bits((a * r).astype(np.float32))
         assert np.array_equal(got, np.broadcast_to(ref, got.shape)), step
+
+
+def test_bench_refuses_more_than_one_gpu_and_its_shape_table_is_well_formed():
+    """bench.py measures one GPU: --gpus 2 exits with a message instead of running; the shapes of its table mode
+    are ones the entry points accept (query heads a multiple of KV heads, head sizes a multiple of 64 up to 768,
+    key bits 2 - 5, value bits 2 / 4 / 8) and the byte count per token and head follows the page layout."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    res = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert res.returncode == 2 and "one GPU" in res.stderr and res.stdout.strip() == ""
+    sys.path.insert(0, root)
+    import bench
+    assert len(set(bench.SHAPE_TABLE)) == len(bench.SHAPE_TABLE)
+    for (B, N, Hq, Hkv, d, kb, vb) in bench.SHAPE_TABLE:
+        assert B > 0 and N > 0 and Hq % Hkv == 0 and d % 64 == 0 and 64 <= d <= 768
+        assert 2 <= kb <= 5 and vb in (2, 4, 8)
+    # 3-bit keys (2-bit indices), 2-bit values in groups of 32 at head_dim 256: 64 + 32 + 2 + 2 + 64 + 32 bytes
+    assert bench.algorithmic_bytes_per_token_head(256, 2, 2, 32) == 196
+    assert bench.algorithmic_bytes_per_token_head(128, 2, 4, 32) == 132
