@@ -637,6 +637,26 @@ def test_preparation_with_several_groups_of_heads_per_workgroup(gpu, B, Hq, Hkv,
         assert torch.equal(whole[sl], part), b0
         assert torch.equal(whole_h[sl], part_h), b0
     assert torch.count_nonzero(whole[3]) == 0
+    # the kernels that read the operand rows of all eight heads (the variants for few heads switched off) must find
+    # zeros in the rows of the heads a group does not have, whichever workgroup shape wrote the operands: a
+    # workspace filled with NaN bit patterns first
+    try:
+        _set_option("narrow_rows", 0)
+        _set_option("page_pairs", 0)
+        ws = pool.workspace(B, Hq, 2)
+        ws.view(torch.int32).fill_(0x7fc00000)
+        wide_rows = pool.decode_attention(q, table, seq, n_split=2, workspace=ws, max_len=max(lens)).clone()
+        ws32 = pool.workspace(32, Hq, 2)
+        for b0 in range(0, B, 32):
+            sl = slice(b0, min(B, b0 + 32))
+            ws32.view(torch.int32).fill_(0x7fc00000)
+            part = pool.decode_attention(q[sl], table[sl], seq[sl], n_split=2, workspace=ws32, max_len=max(lens))
+            torch.cuda.synchronize()
+            assert torch.equal(wide_rows[sl], part), b0
+        assert not torch.isnan(wide_rows.float()).any()
+    finally:
+        _set_option("narrow_rows", 1)
+        _set_option("page_pairs", 1)
     for b in (0, B - 1):
         idx, sgn, norms, rn, vd, vs, vz = [t.cpu() for t in pool.export_flat(table[b], lens[b])]
         ref = O.hybrid_attention(q[b:b + 1].cpu(), key_code(idx, sgn, rn, norms, key_bits - 1), value_code(vd, vs, vz, vb),
