@@ -12,10 +12,16 @@
  *   - `dtype` tags the element type of floating inputs: TQ_F32 / TQ_F16 / TQ_BF16;
  *   - the caller allocates every output and the decode workspace; no entry
  *     point allocates device memory, frees or synchronises;
- *   - calls on different streams may overlap.  The only state the library keeps is per
- *     host thread and per device: a side stream with two events that tq_append_kv_paged and
- *     its siblings create on first use for large appends, the per-kernel launch attributes
- *     set on first use, and the pair of events armed by tq_time_next_page_kernel;
+ *   - calls on different streams may overlap (tq_decode_attn_paged_noalloc excepted, see there).  State the
+ *     library keeps, all of it listed here:
+ *       per host thread and device - a side stream with two events that tq_append_kv_paged and its siblings
+ *         create on first use for large appends, and the pair of events armed by tq_time_next_*_kernel;
+ *       per process - the launch attributes set on a kernel's first use, the compute-unit count of the first
+ *         device used (the cards of one machine are taken to be alike), and the knobs of tq_set_option, which
+ *         select grid shapes and the carving of the workspace: they must not change between the `stages`
+ *         calls of one step, nor while another thread is inside a decode or append call;
+ *       per device - the static scratch array of tq_decode_attn_paged_noalloc (TQ_NOALLOC_SCRATCH_BYTES),
+ *         shared by every caller of that entry point on the device;
  *   - block tables are device data the host cannot inspect, so the kernels bound them:
  *     a logical page beyond the table row, or a table entry outside [0, num_pages), is
  *     never written through (append) and contributes no token (decode); see each entry;
@@ -286,10 +292,13 @@ int tq_decode_attn_paged_ring(const void *q, int dtype, int B, int Hq, int Hkv, 
  * reference.  Same arguments and result, bit for bit, as tq_decode_attn_paged with the same n_split, minus the
  * workspace: partials, rotated queries and query operands live in a file-scope device array of
  * TQ_NOALLOC_SCRATCH_BYTES inside the library (one copy per GPU, held until the process ends; its address is
- * looked up with hipGetSymbolAddress the first time a device is used).  The call allocates nothing and
- * frees nothing.  A call that needs more than the array holds - roughly 4*B*Hq*(n_split+4)*(d+2) bytes of
- * partials plus 8*B*Hq*d - returns TQ_ETOOBIG and launches nothing.  All calls on one GPU share the array:
- * calls that overlap on one GPU (different streams or threads) race; serialise them or use the workspace form. */
+ * looked up with hipGetSymbolAddress by tq_noalloc_init, or by the first call on a device).  The call
+ * allocates nothing and frees nothing.  A call that needs more than the array holds returns TQ_ETOOBIG and
+ * launches nothing; tq_decode_noalloc_bytes gives the exact requirement of a shape.  All calls on one GPU share
+ * the array: calls that overlap on one GPU (different streams or threads) race; serialise them or use the
+ * workspace form.  The device that is current must be the stream's device.  Under stream capture, call
+ * tq_noalloc_init (or make one un-captured call) on the device first: the symbol lookup is not a stream
+ * operation and should not happen while a capture is open.                                              */
 #define TQ_NOALLOC_SCRATCH_BYTES (16u << 20)
 int tq_decode_attn_paged_noalloc(const void *q, int dtype, int B, int Hq, int Hkv, const uint8_t *pool,
                                  int64_t num_pages, const int32_t *block_table, int bt_stride, const int32_t *seq_lens,
@@ -297,6 +306,15 @@ int tq_decode_attn_paged_noalloc(const void *q, int dtype, int B, int Hq, int Hk
                                  const void *recent_k, const void *recent_v, int recent_rows, int64_t rs_b,
                                  int64_t rs_r, int64_t rs_h, const int32_t *recent_len, void *out, int n_split,
                                  void *stream);
+
+/* Bytes of the static scratch array a tq_decode_attn_paged_noalloc call of this shape uses (no counterpart in
+ * the reference); the call returns TQ_ETOOBIG exactly when this exceeds TQ_NOALLOC_SCRATCH_BYTES.  `layer` is
+ * read on the host (head_dim, index bits, codebook terms).  0 for a NULL layer or sizes that are not positive. */
+size_t tq_decode_noalloc_bytes(int B, int Hq, int Hkv, int n_split, const tq_layer *layer);
+
+/* Resolves the address of the current device's scratch array (hipGetSymbolAddress, once per device), so that
+ * the first tq_decode_attn_paged_noalloc call on that device does nothing but launch.  Idempotent.         */
+int tq_noalloc_init(void);
 
 /* Log-sum-exp merge of n_parts partial results per (b, query head):
  * parts (B*Hq, n_parts, d+2) fp32 = [running max, sum of exp, un-normalised acc];
@@ -318,16 +336,6 @@ void tq_time_next_page_kernel(void *start_event, void *stop_event);
 void tq_time_next_key_kernel(void *start_event, void *stop_event);
 
 /* Tuning and test knobs (no counterpart in the reference); process-wide, take effect at the next call.
- *   "prep_units"       0 (default): the query preparation of the matrix-core decode path runs as one workgroup
- *                      per 32-coordinate plane word for all heads of a group; 1: one small workgroup per (few
- *                      query heads, plane word).  Same operands bit for bit.
- *   "fuse_prep"        0 (default): a decode step is three launches (query preparation, page kernel, merge);
- *                      1: a compressed-only step on the matrix-core path prepares its query operands inside
- *                      the page kernel's launch (two launches; the workgroups of a (sequence, KV head) share
- *                      the work and hand the operands to each other).  Same result bit for bit.  Only in a
- *                      library built with -DTQ_FUSED_PREP (TQ_EUNSUPPORTED otherwise): it measured slower.
- *   "prep_spin_limit"  with fuse_prep: how often a workgroup polls for the other workgroups' share of the
- *                      operands before it computes them itself (default 20000; 0 = never wait).
  *   "merge_in_kernel"  1 (default): a compressed-only decode step on the matrix-core kernel with at most 8 context
  *                      splits has its splits merged by the last workgroup of the page kernel (two launches per
  *                      step); 0: always the separate merge kernel.

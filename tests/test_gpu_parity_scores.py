@@ -314,34 +314,24 @@ def test_decode_gives_no_weight_to_pages_outside_the_pool(gpu, d, key_bits, vb, 
     assert torch.count_nonzero(z) == 0
 
 
-# ------------------------------------------------------------------ query preparation inside the page kernel's launch
+# ------------------------------------------------------------------ query preparation for every query dtype
 def _set_option(name, value):
     from turboquant_amd import _ffi
     _ffi.check(_ffi.lib().tq_set_option(name.encode(), int(value)), "tq_set_option")
 
 
-def _has_fused_prep():
-    from turboquant_amd import _ffi
-    rc = _ffi.lib().tq_set_option(b"fuse_prep", 1)
-    _ffi.lib().tq_set_option(b"fuse_prep", 0)
-    return rc == 0
-
-
 @pytest.mark.parametrize("d,key_bits,vb,Hq,Hkv,B,lens,n_split", [
-    (256, 3, 2, 16, 2, 2, [5000, 777], 64),        # one head per unit, 64 units
-    (256, 3, 2, 16, 2, 2, [5000, 777], 5),         # fewer workgroups than units: several units each
-    (128, 3, 4, 32, 8, 3, [900, 64, 300], 4),      # 4 of 8 heads exist, one unit per plane word
+    (256, 3, 2, 16, 2, 2, [5000, 777], 64),
+    (256, 3, 2, 16, 2, 2, [5000, 777], 5),
+    (128, 3, 4, 32, 8, 3, [900, 64, 300], 4),      # 4 of 8 operand heads exist
     (128, 4, 4, 8, 2, 2, [700, 1], 9),             # 4-bit keys (an extra term plane), odd split count
     (256, 2, 4, 10, 2, 1, [2000], 33),             # 5 heads per group
     (128, 3, 2, 32, 2, 2, [400, 900], 16),         # 16 heads per KV head = two groups of 8
     (128, 3, 2, 3, 1, 1, [130], 1)])               # a single workgroup does everything
-def test_decode_step_with_the_preparation_inside_the_page_kernel(gpu, d, key_bits, vb, Hq, Hkv, B, lens, n_split):
+def test_decode_step_for_every_query_dtype(gpu, d, key_bits, vb, Hq, Hkv, B, lens, n_split):
     """The query operands of the matrix-core page kernel (triton_kernels.py:527-528: q Pi^T, q S^T, here also
-    their fp6 operand form) can be prepared three ways: a workgroup per plane word, a workgroup per (few heads,
-    plane word) unit, or inside the page kernel's own launch with the workgroups of a (sequence, KV head)
-    sharing the units.  The operands are the same numbers whoever computes them, so all three must give the
-    same output bit for bit - also when no workgroup of the fused launch waits for the others at all (every
-    workgroup then computes every unit itself), and for fp16 / fp32 queries."""
+    their fp6 operand form) are prepared by one launch per step for bf16, fp16 and fp32 queries; each must meet
+    the oracle (score.py:138-173) on the same store, whatever the split count."""
     g = torch.Generator().manual_seed(d + Hq + n_split)
     pages = (max(lens) + 15) // 16
     pool, tq = _make_pool(gpu, d, key_bits, vb, Hkv, B * pages + 1, torch.bfloat16, seed=42)
@@ -350,41 +340,16 @@ def test_decode_step_with_the_preparation_inside_the_page_kernel(gpu, d, key_bit
     v = torch.randn(B, max(lens), Hkv, d, generator=g).bfloat16().to(gpu)
     pool.append(k, v, table)
     seq = torch.tensor(lens, dtype=torch.int32, device=gpu)
-    _progress(f"fused preparation d={d} kb={key_bits} vb={vb} Hq={Hq} Hkv={Hkv} lens={lens} splits={n_split}")
-    try:
-        for qdt in (torch.bfloat16, torch.float16, torch.float32):
-            q = torch.randn(B, Hq, d, generator=g).to(qdt).to(gpu)
-            _set_option("fuse_prep", 0)
-            _set_option("prep_units", 0)
-            want = pool.decode_attention(q, table, seq, n_split=n_split)
-            _set_option("prep_units", 1)
-            units = pool.decode_attention(q, table, seq, n_split=n_split)
-            torch.cuda.synchronize()
-            assert torch.equal(units, want), qdt
-            if not _has_fused_prep():       # the in-launch preparation is a build option (-DTQ_FUSED_PREP)
-                continue
-            _set_option("fuse_prep", 1)
-            got = pool.decode_attention(q, table, seq, n_split=n_split)
-            again = pool.decode_attention(q, table, seq, n_split=n_split)
-            _set_option("prep_spin_limit", 0)
-            alone = pool.decode_attention(q, table, seq, n_split=n_split)
-            _set_option("prep_spin_limit", 20000)
-            torch.cuda.synchronize()
-            assert torch.equal(got, want), qdt
-            assert torch.equal(again, want), qdt
-            assert torch.equal(alone, want), qdt
-        # and against the oracle, like every other decode test
-        q = torch.randn(B, Hq, d, generator=g).bfloat16()
-        out = pool.decode_attention(q.to(gpu), table, seq, n_split=n_split).cpu()
-    finally:
-        _set_option("fuse_prep", 0)
-        _set_option("prep_units", 0)
-        _set_option("prep_spin_limit", 20000)
+    _progress(f"query dtypes d={d} kb={key_bits} vb={vb} Hq={Hq} Hkv={Hkv} lens={lens} splits={n_split}")
     prm = params_of(tq)
-    for b in range(B):
-        kc, vc = _store_from_oracle_view(pool, table[b], lens[b])
-        want = O.hybrid_attention(q[b:b + 1], kc, vc, max(lens[b], O.MIN_HISTORY), prm, Hkv, None, None)
-        assert cosine(out[b:b + 1], want) >= COS_GATE, b
+    stores = [_store_from_oracle_view(pool, table[b], lens[b]) for b in range(B)]
+    for qdt in (torch.bfloat16, torch.float16, torch.float32):
+        q = torch.randn(B, Hq, d, generator=g).to(qdt)
+        out = pool.decode_attention(q.to(gpu), table, seq, n_split=n_split).cpu()
+        for b in range(B):
+            kc, vc = stores[b]
+            want = O.hybrid_attention(q[b:b + 1], kc, vc, max(lens[b], O.MIN_HISTORY), prm, Hkv, None, None)
+            assert cosine(out[b:b + 1], want) >= COS_GATE, (qdt, b)
 
 
 # ------------------------------------------------------------------ 8-bit values in the paged store
@@ -775,3 +740,49 @@ def test_splits_merged_inside_the_page_kernel(gpu, d, key_bits, vb, Hq, Hkv, len
         kc, vc = _store_from_oracle_view(pool, table[b], lens[b])
         ref = O.hybrid_attention(q[b:b + 1], kc, vc, max(lens[b], O.MIN_HISTORY), prm, Hkv, None, None)
         assert cosine(got[b:b + 1], ref) >= COS_GATE, b
+
+
+def test_in_launch_merge_over_thousands_of_consecutive_steps(gpu):
+    """The hand-off of the in-launch merge (every workgroup's partial, then the arrival counter, then the last
+    arriver's reads) over 3,000 consecutive decode steps of the 16 x 8192, 32 q / 8 KV head shape on ONE
+    workspace.  The queries rotate among four, so a partial that the merging workgroup read before its producer's
+    stores had landed would be the previous step's, a different query's.  The in-launch merge sums in a fixed
+    order, so every step must reproduce its query's first result bit for bit; that first result is held to the
+    merge kernel's (merge_in_kernel 0) at one bf16 step.  Stops at the first mismatch (checked every 50 steps)."""
+    d, Hq, Hkv, B, N = 128, 32, 8, 16, 8192
+    g = torch.Generator().manual_seed(77)
+    pages = N // 16
+    pool, tq = _make_pool(gpu, d, 3, 4, Hkv, B * pages, torch.bfloat16, seed=42)
+    table = torch.randperm(B * pages, generator=g).to(torch.int32).view(B, pages).to(gpu)
+    for b0 in range(0, B, 4):
+        k = torch.randn(4, N, Hkv, d, generator=g).bfloat16().to(gpu)
+        v = torch.randn(4, N, Hkv, d, generator=g).bfloat16().to(gpu)
+        pool.append(k, v, table[b0:b0 + 4])
+    seq = torch.full((B,), N, dtype=torch.int32, device=gpu)
+    qs = [torch.randn(B, Hq, d, generator=g).bfloat16().to(gpu) for _ in range(4)]
+    n_split = pool.default_splits(B, N, Hq)
+    ws = pool.workspace(B, Hq, n_split)
+    _progress(f"in-launch merge soak: {B} x {N}, {Hq} q / {Hkv} KV heads, {n_split} splits, 3000 steps")
+    try:
+        _set_option("merge_in_kernel", 0)
+        sep = [pool.decode_attention(q, table, seq, n_split=n_split, workspace=ws).clone() for q in qs]
+        _set_option("merge_in_kernel", 1)
+        first = [pool.decode_attention(q, table, seq, n_split=n_split, workspace=ws).clone() for q in qs]
+        torch.cuda.synchronize()
+        for a, b_ in zip(first, sep):
+            assert (a.float() - b_.float()).abs().max() <= 2 ** -7 * b_.float().abs().max() + 1e-6
+        assert not torch.equal(first[0], first[1])
+        out = torch.empty_like(qs[0])
+        bad = torch.zeros((), dtype=torch.int64, device=gpu)
+        steps = torch.arange(1, 3001, device=gpu)
+        for step in range(3000):
+            i = step % 4
+            pool.decode_attention(qs[i], table, seq, n_split=n_split, workspace=ws, out=out)
+            # step number of the first mismatch (0 = none so far), kept on the card
+            differs = (out != first[i]).any()
+            bad = torch.where((bad == 0) & differs, steps[step], bad)
+            if step % 50 == 49:
+                at = int(bad.item())
+                assert at == 0, f"in-launch merge differs from its first result at step {at - 1}"
+    finally:
+        _set_option("merge_in_kernel", 1)

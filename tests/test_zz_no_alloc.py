@@ -40,7 +40,8 @@ def _both(gpu, pool, tq, q, table, seq, n_split, rk=None, rv=None, rl=None):
     return want, got
 
 
-@pytest.mark.parametrize("d,key_bits,vb,Hq,Hkv", [(128, 3, 4, 8, 2), (256, 3, 2, 16, 2), (64, 3, 2, 4, 1)])
+# (the last case has 8-bit values: no matrix-core kernel, the general page kernel runs on the static area)
+@pytest.mark.parametrize("d,key_bits,vb,Hq,Hkv", [(128, 3, 4, 8, 2), (256, 3, 2, 16, 2), (64, 3, 2, 4, 1), (128, 3, 8, 8, 2)])
 def test_static_scratch_decode_equals_the_workspace_form_on_consecutive_calls(gpu, d, key_bits, vb, Hq, Hkv):
     g = torch.Generator().manual_seed(d + Hq)
     B, N = 3, 900
@@ -86,6 +87,11 @@ def test_static_scratch_decode_rejects_what_does_not_fit(gpu):
                             out.data_ptr(), n_split, _ffi.stream_ptr(gpu))
     need = 4 * B * Hq * 33 * (d + 2)
     assert need > 16 << 20
+    # the exported size rule is what the entry point applies: refused exactly when it exceeds the area
+    assert lib.tq_noalloc_init() == 0
+    assert lib.tq_decode_noalloc_bytes(B, Hq, Hkv, 32, C.byref(ly)) > 16 << 20 >= lib.tq_decode_noalloc_bytes(B, Hq, Hkv, 1, C.byref(ly))
+    assert lib.tq_decode_noalloc_bytes(B, Hq, Hkv, 32, C.byref(ly)) >= need
+    assert lib.tq_decode_noalloc_bytes(B, Hq, Hkv, 0, C.byref(ly)) == 0
     assert lib.tq_decode_attn_paged_noalloc(*args(32)) == -4
     torch.cuda.synchronize()
     assert torch.all(out == 7.0)                                   # nothing ran

@@ -80,6 +80,8 @@ _SIGNATURES = {
                                             C.POINTER(TqPageLayout), _vp, _vp, _i64, _i64, _i64, _i, _vp, _vp, _i, _vp]),
     "tq_decode_attn_paged_noalloc": (C.c_int, [_vp, _i, _i, _i, _i, _vp, _i64, _vp, _i, _vp, _f, C.POINTER(TqLayer),
                                                C.POINTER(TqPageLayout), _vp, _vp, _i, _i64, _i64, _i64, _vp, _vp, _i, _vp]),
+    "tq_decode_noalloc_bytes": (C.c_size_t, [_i, _i, _i, _i, C.POINTER(TqLayer)]),
+    "tq_noalloc_init": (C.c_int, []),
     "tq_decode_merge": (C.c_int, [_vp, _i64, _i, _i, _i, _vp, _vp]),
     "tq_time_next_page_kernel": (None, [_vp, _vp]),
     "tq_time_next_key_kernel": (None, [_vp, _vp]),

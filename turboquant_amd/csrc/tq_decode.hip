@@ -855,17 +855,7 @@ static size_t merge_smem(int n_parts, int d, int ny) {
 
 __global__ void __launch_bounds__(256)
 merge_kernel(const float* __restrict__ parts, int n_parts, int part_stride, int d, int dtype, void* __restrict__ out,
-             unsigned long long* __restrict__ flags, int n_flags, int row_groups) {
-  // the flags under which the page kernel's workgroups published their query-preparation units are
-  // cleared here, after that kernel has ended: the next call (or the next replay of a captured one,
-  // which carries the same nonce) starts without a published unit
-  if (blockIdx.y == 0) {
-    const int per_row = (n_flags + (int)gridDim.x - 1) / (int)gridDim.x;
-    for (int i = threadIdx.x; i < per_row; i += blockDim.x) {
-      const int64_t at = (int64_t)blockIdx.x * per_row + i;
-      if (at < n_flags) flags[at] = 0ull;
-    }
-  }
+             int row_groups) {
   extern __shared__ float s_w[];                 // [n_parts] weights, [n_parts] m, [n_parts] l, [8] scratch, [S][dw] sums
   const int64_t row = blockIdx.x;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -952,14 +942,11 @@ int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* 
 }  // namespace tq
 
 static size_t parts_floats(int B, int Hq, int d, int n_parts) { return (size_t)B * Hq * n_parts * (d + 2); }
-// publication flags of the in-kernel query preparation: 64 per group of query heads, at most B * Hq groups
-static size_t flag_words(int B, int Hq) { return (size_t)B * Hq * 64; }
+// arrival counters of the in-launch merge: one 64-bit word per group of query heads, at most B * Hq groups
+static size_t counter_words(int B, int Hq) { return (size_t)B * Hq; }
 
 // ---- knobs (tq_set_option) -----------------------------------------------------------------------------
 namespace tq {
-std::atomic<int> opt_fuse_prep{0};
-std::atomic<int> opt_prep_spin_limit{20000};
-std::atomic<int> opt_prep_units{0};
 std::atomic<int> opt_append_parts{3};
 std::atomic<int> opt_fp6_centroids{1};
 std::atomic<int> opt_merge_in_kernel{1};
@@ -972,34 +959,8 @@ std::atomic<int> opt_merge_row_groups{1};
 std::atomic<int> opt_tail_chunks{1};
 }  // namespace tq
 
-namespace {
-std::atomic<unsigned long long> g_nonce{0};
-
-unsigned long long next_nonce() {
-  unsigned long long v = g_nonce.load();
-  if (v == 0) {       // first use in this process: start somewhere unpredictable, far from small numbers
-    const unsigned long long seed =
-        ((unsigned long long)std::chrono::steady_clock::now().time_since_epoch().count() * 0x9E3779B97F4A7C15ull) | (1ull << 62);
-    g_nonce.compare_exchange_strong(v, seed);
-  }
-  v = g_nonce.fetch_add(1) + 1;
-  return v ? v : g_nonce.fetch_add(1) + 1;
-}
-}  // namespace
-
 extern "C" int tq_set_option(const char* name, int64_t value) {
   if (!name) return TQ_ENULL;
-  if (!std::strcmp(name, "fuse_prep")) {
-    if (value != 0 && !decode_mfma_has_fused_prep()) return TQ_EUNSUPPORTED;     // not compiled into this build
-    opt_fuse_prep.store(value != 0);
-    return TQ_OK;
-  }
-  if (!std::strcmp(name, "prep_units")) { opt_prep_units.store(value != 0); return TQ_OK; }
-  if (!std::strcmp(name, "prep_spin_limit")) {
-    if (value < 0 || value > 100000000) return TQ_EINVAL;
-    opt_prep_spin_limit.store((int)value);
-    return TQ_OK;
-  }
   if (!std::strcmp(name, "wide_workgroups")) { opt_wide_workgroups.store(value != 0); return TQ_OK; }
   if (!std::strcmp(name, "split_skew")) {
     if (value < 0 || value > 8) return TQ_EINVAL;
@@ -1026,7 +987,7 @@ extern "C" size_t tq_decode_workspace_bytes(int B, int Hq, int d, int n_split) {
   // partials for n_split history splits + up to TAIL_MAX_CHUNKS of the exact tail, then q_rot, q_sk, 4 statistics per query row and
   // the packed query operands of the matrix-core kernel (sized for the largest kernel: 9 term planes, 8 heads)
   return (parts_floats(B, Hq, d, n_split + TAIL_MAX_CHUNKS) + (size_t)2 * B * Hq * d + (size_t)4 * B * Hq) * sizeof(float) +
-         flag_words(B, Hq) * sizeof(unsigned long long) + decode_mfma_pack_words(B, Hq, d) * sizeof(uint32_t);
+         counter_words(B, Hq) * sizeof(unsigned long long) + decode_mfma_pack_words(B, Hq, d) * sizeof(uint32_t);
 }
 
 extern "C" int tq_decode_merge(const float* parts, int64_t rows, int n_parts, int d, int dtype, void* out,
@@ -1036,7 +997,7 @@ extern "C" int tq_decode_merge(const float* parts, int64_t rows, int n_parts, in
   if (rows == 0) return TQ_OK;
   const int ny = merge_row_groups(rows, n_parts, d);
   merge_kernel<<<dim3((unsigned)rows, ny), dim3(256), merge_smem(n_parts, d, ny), (hipStream_t)stream>>>(
-      parts, n_parts, n_parts, d, dtype, out, nullptr, 0, ny);
+      parts, n_parts, n_parts, d, dtype, out, ny);
   TQ_CHECK_LAUNCH();
   return TQ_OK;
 }
@@ -1089,9 +1050,9 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   for (int n = 1; n <= G && !kv_div; ++n)
     if (G % n == 0 && G / n <= 8) kv_div = n;
   const int Gq = kv_div ? G / kv_div : G;
-  const bool mfma_shape = kv_div && (d == 64 || d == 128 || d == 256) && (layout->dtype == TQ_BF16 || layout->dtype == TQ_F16) &&
-                          layout->value_bits != 8 && layer->Pi_colsum &&
-                          layer->S_colsum;
+  // (the same table the launchers dispatch over: a shape without an instantiation keeps its split count and takes
+  // the general kernel's preparation, which writes the fp32 rotated / sketched queries that kernel reads)
+  const bool mfma_shape = kv_div && layer->Pi_colsum && layer->S_colsum && decode_mfma_has_kernel(*layer, *layout);
   // Short contexts with at most four query heads per group run workgroups of eight wavefronts on half as many
   // splits (the same number of wavefronts): everything below - partials, merge, the workspace's carving - then
   // uses the halved count, for every stage of the step alike.
@@ -1117,8 +1078,8 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   float* q_rot = parts + parts_floats(B, Hq, d, n_parts);
   float* q_sk = q_rot + (size_t)B * Hq * d;
   float* q_stat = q_sk + (size_t)B * Hq * d;
-  unsigned long long* flags = (unsigned long long*)(q_stat + (size_t)4 * B * Hq);       // 8-byte aligned: every term above is even
-  uint32_t* qa_pack = (uint32_t*)(flags + flag_words(B, Hq));
+  unsigned long long* arrivals = (unsigned long long*)(q_stat + (size_t)4 * B * Hq);    // 8-byte aligned: every term above is even
+  uint32_t* qa_pack = (uint32_t*)(arrivals + counter_words(B, Hq));
 
   if (tail && ts.paged && !words) return TQ_EUNSUPPORTED;       // a paged exact cache has to be word-aligned
   TailArgs ta;
@@ -1136,43 +1097,18 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   const int n_tail = Hkv * B * ((G + TAIL_GC - 1) / TAIL_GC) * t_chunks;
   bool tail_done = false;
 
-  // Whole compressed-only step on the matrix-core path: the query preparation runs as a prologue of the
-  // page kernel's own launch (its workgroups share the work and hand the operands to each other), so the
-  // step is two launches, page kernel and merge.
-  bool fused = false;
-  const int n_flags = B * Hkv * (kv_div ? kv_div : 1) * 64;
-  if (stages == 7 && mfma_shape && !tail && opt_fuse_prep.load()) {
-    if (!layer->PiT || !layer->ST || !layer->centroids) return TQ_ENULL;
-    FusedPrep fz;
-    fz.q = q;
-    fz.q_dtype = dtype;
-    const int words = d / PREP_COLS;
-    int hp = 8;                      // as few heads per unit as still gives every unit a workgroup of its own
-    while (hp > 1 && ((Gq + hp / 2 - 1) / (hp / 2)) * words <= n_split) hp /= 2;
-    fz.hp = hp;
-    fz.n_units = (8 / hp) * words;
-    fz.spin_limit = opt_prep_spin_limit.load();
-    fz.flags = flags;
-    fz.nonce = next_nonce();
-    const int mf = launch_decode_mfma(qa_pack, q_stat, B, Hq, Hkv * kv_div, kv_div, pool, block_table, bt_stride, seq_lens,
-                                      sm_scale, *layer, *layout, parts, n_parts, n_split, len_sub, max_pages, pool_pages,
-                                      fz, FusedMerge{}, wide_wg, st);
-    if (mf > 0) return mf;
-    fused = mf == TQ_OK;             // TQ_EUNSUPPORTED: nothing was launched, the separate launches below run
-  }
-
   // A whole compressed-only step with few context splits: the workgroup that finishes last among the splits of a
   // (sequence, group of query heads) merges them inside the page kernel's launch, and no merge kernel follows
   // (with many splits that workgroup would read more than the separate launch costs).  The preparation kernel
   // zeroes the arrival counters of its groups.
   FusedMerge fm;
-  if (stages == 7 && mfma_shape && !fused && n_split <= MERGE_IN_KERNEL_MAX_SPLITS && opt_merge_in_kernel.load()) {
+  if (stages == 7 && mfma_shape && n_split <= MERGE_IN_KERNEL_MAX_SPLITS && opt_merge_in_kernel.load()) {
     fm.out = out;
     fm.out_dtype = dtype;
-    fm.counters = flags;
+    fm.counters = arrivals;
     fm.n_extra = tail ? 1 : 0;          // the exact tail's partial, written by an earlier launch of this step
   }
-  if ((stages & 1) && !fused) {
+  if (stages & 1) {
     if (!layer->Pi || !layer->PiT || !layer->S || !layer->ST || !layer->centroids) return TQ_ENULL;
     // (in the launch shared with the tail a compute unit holds two workgroups: beyond that the preparation
     // workgroups take several groups of heads each, see prep_query_body)
@@ -1272,11 +1208,11 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
 #undef TQ_LAUNCH_TAIL
     TQ_CHECK_LAUNCH();
   }
-  int mf = fused ? TQ_OK : TQ_EUNSUPPORTED;
-  if ((stages & 2) && !fused)
+  int mf = TQ_EUNSUPPORTED;
+  if (stages & 2)
     mf = mfma_shape ? launch_decode_mfma(qa_pack, q_stat, B, Hq, Hkv * kv_div, kv_div, pool, block_table, bt_stride,
                                          seq_lens, sm_scale, *layer, *layout, parts, n_parts, n_split, len_sub,
-                                         max_pages, pool_pages, FusedPrep{}, fm, wide_wg, st)
+                                         max_pages, pool_pages, fm, wide_wg, st)
                     : TQ_EUNSUPPORTED;
   if (mf > 0) return mf;
   if (mf == TQ_OK && fm.out != nullptr) return TQ_OK;         // merged in the launch
@@ -1324,7 +1260,7 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   // without a tail the merge simply reads one part fewer
   const int merged = tail ? n_parts : n_split, ny = merge_row_groups((int64_t)B * Hq, merged, d);
   merge_kernel<<<dim3((unsigned)(B * Hq), ny), dim3(256), merge_smem(n_parts, d, ny), st>>>(
-      parts, merged, n_parts, d, dtype, out, fused ? flags : nullptr, fused ? n_flags : 0, ny);
+      parts, merged, n_parts, d, dtype, out, ny);
   TQ_CHECK_LAUNCH();
   return TQ_OK;
 }
@@ -1402,7 +1338,7 @@ size_t decode_scratch_need(int B, int Hq, int Hkv, int n_split, const tq_layer& 
   for (int n = 1; n <= G && !kv_div; ++n)
     if (G % n == 0 && G / n <= 8) kv_div = n;
   size_t floats = parts_floats(B, Hq, d, n_split + TAIL_MAX_CHUNKS) + (size_t)2 * B * Hq * d + (size_t)4 * B * Hq +
-                  2 * flag_words(B, Hq);
+                  2 * counter_words(B, Hq);
   size_t words = 0;
   if (kv_div && (d == 64 || d == 128 || d == 256)) {
     int planes = ly.mse_bits + 1;
@@ -1413,6 +1349,18 @@ size_t decode_scratch_need(int B, int Hq, int Hkv, int n_split, const tq_layer& 
   return (floats + words) * 4;
 }
 }  // namespace
+
+extern "C" size_t tq_decode_noalloc_bytes(int B, int Hq, int Hkv, int n_split, const tq_layer* layer) {
+  if (!layer || B <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || n_split <= 0 || layer->d <= 0 || layer->n_terms < 0 ||
+      layer->n_terms > TQ_MAX_TERMS)
+    return 0;
+  return decode_scratch_need(B, Hq, Hkv, n_split, *layer);
+}
+
+extern "C" int tq_noalloc_init(void) {
+  void* ws = nullptr;
+  return scratch_address(&ws);
+}
 
 extern "C" int tq_decode_attn_paged_noalloc(const void* q, int dtype, int B, int Hq, int Hkv, const uint8_t* pool,
                                             int64_t num_pages, const int32_t* block_table, int bt_stride,

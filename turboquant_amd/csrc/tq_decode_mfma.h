@@ -6,18 +6,6 @@
 
 namespace tq {
 
-// Query preparation as a prologue of the page kernel's own launch (q == nullptr: the operands in
-// qa_pack / q_stat were prepared by an earlier launch).
-struct FusedPrep {
-  const void* q = nullptr;           // (B, Hq, d) raw queries
-  int q_dtype = 0;
-  int n_units = 0;                   // units per group of query heads (<= 64): (8 / hp) head sets x d / 32 plane words
-  int hp = 8;                        // heads per unit: 1, 2, 4 or 8
-  int spin_limit = 0;                // polls before a workgroup stops waiting for the others' units
-  unsigned long long* flags = nullptr;   // 64 words per group
-  unsigned long long nonce = 0;      // value of a published flag in this call (never 0)
-};
-
 // Merge of the context splits inside the page kernel's launch (out == nullptr: a merge kernel follows).  The
 // workgroup that finishes last among the n_split workgroups of a (sequence, group of query heads) reads the
 // others' partials and writes the attention output; nobody waits for anybody.  `counters` holds one arrival
@@ -34,18 +22,42 @@ constexpr int MERGE_IN_KERNEL_MAX_SPLITS = 8;
 // returns them and disarms; false when none is armed.
 bool take_time_hook(int which, hipEvent_t& start, hipEvent_t& stop);
 
-// whether the library was built with the in-launch preparation (-DTQ_FUSED_PREP)
-bool decode_mfma_has_fused_prep();
-
 // words of packed query operands tq_decode_workspace_bytes reserves
 size_t decode_mfma_pack_words(int B, int Hq, int d);
+
+// The instantiations of the matrix-core page kernel, one list per head size: X(head_dim, index bits, multi-bit
+// Walsh terms, value bits, value group size, wavefronts per block, wavefronts per SIMD).  The launchers and the
+// host-side predicate below both expand these lists, so they cannot disagree.
+#define TQ_MFMA_SHAPES_D64(X) \
+  X(64, 2, 0, 2, 32, 1, 2) X(64, 2, 0, 4, 32, 1, 2) X(64, 1, 0, 2, 32, 1, 2) X(64, 1, 0, 4, 32, 1, 2) \
+  X(64, 3, 1, 2, 32, 1, 2) X(64, 3, 1, 4, 32, 1, 2)
+#define TQ_MFMA_SHAPES_D128(X) \
+  X(128, 2, 0, 2, 32, 1, 2) X(128, 2, 0, 4, 32, 1, 2) X(128, 1, 0, 2, 32, 1, 2) X(128, 1, 0, 4, 32, 1, 2) \
+  X(128, 3, 1, 2, 32, 1, 2) X(128, 3, 1, 4, 32, 1, 2) X(128, 2, 0, 2, 64, 1, 2) X(128, 2, 0, 4, 64, 1, 2)
+#define TQ_MFMA_SHAPES_D256(X) \
+  X(256, 2, 0, 2, 32, 2, 2) X(256, 2, 0, 4, 32, 2, 2) X(256, 1, 0, 2, 32, 2, 2) X(256, 1, 0, 4, 32, 2, 2) \
+  X(256, 3, 1, 2, 32, 2, 2) X(256, 3, 1, 4, 32, 2, 2) X(256, 2, 0, 2, 64, 2, 2) X(256, 2, 0, 4, 64, 2, 2)
+
+// the parameters of a layer that pick an instantiation
+struct MfmaShape { int d, mb, nx, vb, gs; bool f16p; };
+inline MfmaShape mfma_shape_of(const tq_layer& ly, const tq_page_layout& L) {
+  MfmaShape s{ly.d, ly.mse_bits, 0, L.value_bits, L.group_size, L.dtype == TQ_F16};
+  for (int t = 0; t < ly.n_terms; ++t)
+    if (__builtin_popcount(ly.term_mask[t]) > 1) ++s.nx;
+  return s;
+}
+
+// Whether launch_decode_mfma has a kernel for this layer and page layout (head size, bit widths, codebook terms,
+// group size, page dtype and key order); the host side decides the step's shape - split count, operand packing,
+// workspace carving - from this, before anything is launched.
+bool decode_mfma_has_kernel(const tq_layer& ly, const tq_page_layout& L);
 
 // Returns TQ_EUNSUPPORTED when the shape has no matrix-core kernel (nothing was launched); the caller then
 // uses the general vector-ALU kernel.
 int launch_decode_mfma(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, int kv_div, const uint8_t* pool,
                        const int32_t* block_table, int bt_stride, const int32_t* seq_lens, float sm_scale,
                        const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts, int n_split, int len_sub,
-                       int max_pages, int num_pages, const FusedPrep& fz, const FusedMerge& fm, bool wide_wg,
+                       int max_pages, int num_pages, const FusedMerge& fm, bool wide_wg,
                        hipStream_t st);
 
 // Whether a step of this shape runs workgroups of eight wavefronts: the caller then passes HALF its split count

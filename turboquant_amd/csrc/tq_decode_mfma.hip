@@ -11,13 +11,6 @@
 
 namespace tq {
 
-// The query preparation as a prologue of the page kernel's launch is compiled in with -DTQ_FUSED_PREP only.
-#ifdef TQ_FUSED_PREP
-bool decode_mfma_has_fused_prep() { return true; }
-#else
-bool decode_mfma_has_fused_prep() { return false; }
-#endif
-
 constexpr int MF_WAVES = 4;              // wavefronts of the (smaller) workgroup, as in tq_decode_mfma_impl.h
 constexpr int BLK_TOK = 64;              // tokens per wavefront iteration
 
@@ -71,21 +64,31 @@ int decode_mfma_split_skew(int n_split, int rows) {
 // words of packed query operands tq_decode_attn_paged reserves in its workspace
 size_t decode_mfma_pack_words(int B, int Hq, int d) { return (size_t)B * Hq * 9 * (d / 128 + 1) * 1024; }   // d = 64: one chunk
 
+bool decode_mfma_has_kernel(const tq_layer& ly, const tq_page_layout& L) {
+  if ((L.dtype != TQ_BF16 && L.dtype != TQ_F16) || !L.key_lane_major) return false;
+  const MfmaShape sh = mfma_shape_of(ly, L);
+#define TQ_HAS(D_, MB_, NX_, VB_, GS_, DS_, WPS_) \
+  if (sh.d == D_ && sh.mb == MB_ && sh.nx == NX_ && sh.vb == VB_ && sh.gs == GS_) return true;
+  TQ_MFMA_SHAPES_D64(TQ_HAS) TQ_MFMA_SHAPES_D128(TQ_HAS) TQ_MFMA_SHAPES_D256(TQ_HAS)
+#undef TQ_HAS
+  return false;
+}
+
 // the launchers of the three head sizes (tq_decode_mfma_d64 / _d128 / _d256.hip)
 int launch_decode_mfma_d64(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, int kv_div,
                        const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
                        float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts,
-                       int n_split, int len_sub, int max_pages, int num_pages, const FusedPrep& fz, const FusedMerge& fm,
+                       int n_split, int len_sub, int max_pages, int num_pages, const FusedMerge& fm,
                        bool wide_wg, hipStream_t st);
 int launch_decode_mfma_d128(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, int kv_div,
                        const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
                        float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts,
-                       int n_split, int len_sub, int max_pages, int num_pages, const FusedPrep& fz, const FusedMerge& fm,
+                       int n_split, int len_sub, int max_pages, int num_pages, const FusedMerge& fm,
                        bool wide_wg, hipStream_t st);
 int launch_decode_mfma_d256(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, int kv_div,
                        const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
                        float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts,
-                       int n_split, int len_sub, int max_pages, int num_pages, const FusedPrep& fz, const FusedMerge& fm,
+                       int n_split, int len_sub, int max_pages, int num_pages, const FusedMerge& fm,
                        bool wide_wg, hipStream_t st);
 
 // Returns TQ_EUNSUPPORTED when the shape has no matrix-core kernel; the caller then
@@ -93,16 +96,16 @@ int launch_decode_mfma_d256(uint32_t* qa_pack, float* q_stat, int B, int Hq, int
 int launch_decode_mfma(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, int kv_div,
                        const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
                        float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts,
-                       int n_split, int len_sub, int max_pages, int num_pages, const FusedPrep& fz, const FusedMerge& fm,
+                       int n_split, int len_sub, int max_pages, int num_pages, const FusedMerge& fm,
                        bool wide_wg, hipStream_t st) {
   const int G = Hq / Hkv, d = ly.d;
   if (G > 8 || (L.dtype != TQ_BF16 && L.dtype != TQ_F16) || !L.key_lane_major) return TQ_EUNSUPPORTED;
   if (d == 64) return launch_decode_mfma_d64(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table, bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts, n_split,
-                                   len_sub, max_pages, num_pages, fz, fm, wide_wg, st);
+                                   len_sub, max_pages, num_pages, fm, wide_wg, st);
   if (d == 128) return launch_decode_mfma_d128(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table, bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts, n_split,
-                                   len_sub, max_pages, num_pages, fz, fm, wide_wg, st);
+                                   len_sub, max_pages, num_pages, fm, wide_wg, st);
   if (d == 256) return launch_decode_mfma_d256(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table, bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts, n_split,
-                                   len_sub, max_pages, num_pages, fz, fm, wide_wg, st);
+                                   len_sub, max_pages, num_pages, fm, wide_wg, st);
   return TQ_EUNSUPPORTED;
 }
 

@@ -7,10 +7,10 @@ namespace tq {
 int launch_decode_mfma_d128(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, int kv_div,
                        const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
                        float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts,
-                       int n_split, int len_sub, int max_pages, int num_pages, const FusedPrep& fz, const FusedMerge& fm,
+                       int n_split, int len_sub, int max_pages, int num_pages, const FusedMerge& fm,
                        bool wide_wg, hipStream_t st) {
   const MfmaShape sh = mfma_shape_of(ly, L);
-  TQ_TRY(128, 2, 0, 2, 32, 1, 2) TQ_TRY(128, 2, 0, 4, 32, 1, 2) TQ_TRY(128, 1, 0, 2, 32, 1, 2) TQ_TRY(128, 1, 0, 4, 32, 1, 2) TQ_TRY(128, 3, 1, 2, 32, 1, 2) TQ_TRY(128, 3, 1, 4, 32, 1, 2) TQ_TRY(128, 2, 0, 2, 64, 1, 2) TQ_TRY(128, 2, 0, 4, 64, 1, 2)
+  TQ_MFMA_SHAPES_D128(TQ_TRY)
   return TQ_EUNSUPPORTED;
 }
 

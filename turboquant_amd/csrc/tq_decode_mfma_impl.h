@@ -65,15 +65,6 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef int i32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
 typedef int i32x8 __attribute__((ext_vector_type(8)));
 
-// The query preparation as a prologue of the page kernel's launch is compiled in with -DTQ_FUSED_PREP only:
-// it measured slower than the separate launch (see the kernel), and its mere presence costs the page
-// kernel half a microsecond.
-#ifdef TQ_FUSED_PREP
-constexpr bool fused_build = true;
-#else
-constexpr bool fused_build = false;
-#endif
-
 constexpr int MF_WAVES = 4;
 constexpr int BLK_TOK = 64;              // tokens per wavefront iteration
 constexpr float MF_NEG = -1.0e30f;
@@ -230,7 +221,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
                    const uint8_t* __restrict__ pool, const int32_t* __restrict__ block_table,
                    int bt_stride, const int32_t* __restrict__ seq_lens, float sm_scale, tq_layer ly, tq_page_layout L,
                    float* __restrict__ parts, int n_parts, int n_split, int len_sub, int max_pages, int num_pages,
-                   int skew16, int n_seq, FusedPrep fz, FusedMerge fm) {
+                   int skew16, int n_seq, FusedMerge fm) {
   constexpr int DW = D / DS;                  // coordinates / channels of one wavefront
   constexpr int WPLT = (D + 127) / 128;       // plane words per lane per plane per page, all wavefronts
   constexpr int WPL = (DW + 127) / 128;       // ... of one wavefront (head_dim 64: one, with half of the lanes idle)
@@ -296,49 +287,6 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   unsigned char* stage_z = stage_v + (VW / 4) * 1024;
   unsigned char* stage_s = stage_z + 2 * 1024;
 
-  // ---------------------------------------------------------------- query preparation inside this launch
-  // fz.q != nullptr: nobody has prepared the query operands; the workgroups that share a group of query
-  // heads (the n_split workgroups of a (sequence, KV head)) do it together.  The work is cut into
-  // fz.n_units units (some heads x one plane word, prep_unit256); workgroup `split` computes units split,
-  // split + n_split, ..., writes them to qa_pack / q_stat, and publishes each under a flag that carries
-  // this call's nonce.  Then every workgroup waits until all units of its group are published.  The wait
-  // is bounded: after fz.spin_limit polls a workgroup stops waiting and computes every unit itself (the
-  // values are the same whoever computes them), so the kernel ends whatever the other workgroups do.
-  // Flags are 64-bit words that never hold a call's nonce by accident (the nonce changes with every call;
-  // the merge kernel that follows clears them, which also covers replays of a captured launch).
-#ifdef TQ_FUSED_PREP
-  if (fz.q != nullptr) {
-    float* sm = (float*)smem_raw;
-    const int words = D / PREP_COLS;
-    const int64_t grp = (int64_t)b * Hkv + h;
-    unsigned long long* gflags = fz.flags + grp * 64;
-    // first pass: this workgroup's own units, published; second pass (only after a wait that ran out): all units
-    for (bool everything = false;; everything = true) {
-      const int u0 = everything ? 0 : split, du = everything ? 1 : n_split;
-      for (int u = u0; u < fz.n_units; u += du)
-        prep_unit256<D / PREP_SLICES, true>(fz.q, fz.q_dtype, G, ly, sm_scale, q_stat, qa_pack, grp, u % words,
-                                            (u / words) * fz.hp, fz.hp, sm);
-      // The units were written with device-coherent stores; once they have completed (the barrier waits
-      // for every wavefront's outstanding stores) their flags may follow.
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-      __syncthreads();
-      if (everything) break;
-      if (tid == 0)
-        for (int u = split; u < fz.n_units; u += n_split)
-          __hip_atomic_store(gflags + u, fz.nonce, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      bool have = lane >= fz.n_units;
-      for (int spin = 0; spin < fz.spin_limit; ++spin) {
-        if (!have) have = load_coherent(gflags + lane) == fz.nonce;
-        if (__builtin_amdgcn_ballot_w64(!have) == 0) break;
-        __builtin_amdgcn_s_sleep(4);
-      }
-      if (!have) have = load_coherent(gflags + min(lane, fz.n_units - 1)) == fz.nonce;
-      if (__syncthreads_and(__builtin_amdgcn_ballot_w64(!have) == 0)) break;       // every unit of the group is there
-    }
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");      // the (device-coherent) operand loads stay below the wait
-  }
-#endif
-
   // ---------------------------------------------------------------- A operands of the score stage
   // fp6 query terms in register order (see the preparation kernel): row set 0 = terms 0, 1 of the 8
   // heads (row 2g + t), row set 1 = terms 2, 3; rows of absent heads are zero.  Six dwords per
@@ -358,16 +306,9 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
 #pragma unroll
         for (int rs = 0; rs < NRS; ++rs) {
           const uint32_t* p6 = src + ((tp * WPLT + hf * WPL + i) * 2 + rs) * (64 * 8);
-          if (fused_build && fz.q != nullptr) {       // written by other workgroups of this launch: device-coherent loads
-            const unsigned long long* p64 = (const unsigned long long*)p6;
-            const unsigned long long x0 = load_coherent(p64), x1 = load_coherent(p64 + 1), x2 = load_coherent(p64 + 2);
-            qa[tp][i][rs] = i32x8{(int)(uint32_t)x0, (int)(x0 >> 32), (int)(uint32_t)x1, (int)(x1 >> 32),
-                                  (int)(uint32_t)x2, (int)(x2 >> 32), 0, 0};
-          } else {
-            const u32x4 lo = *(const u32x4*)p6;
-            const uint32_t d4 = p6[4], d5 = p6[5];
-            qa[tp][i][rs] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)d4, (int)d5, 0, 0};
-          }
+          const u32x4 lo = *(const u32x4*)p6;
+          const uint32_t d4 = p6[4], d5 = p6[5];
+          qa[tp][i][rs] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)d4, (int)d5, 0, 0};
           if (!a_live) qa[tp][i][rs] = i32x8{0, 0, 0, 0, 0, 0, 0, 0};
         }
   }
@@ -378,9 +319,8 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   {
     const int g = PP ? (n & 7) >> 1 : (NR ? n >> 2 : n >> 1);
     const int64_t qrow = (int64_t)b * Hq + h * G + (g < G ? g : 0);
-    const bool coh = fused_build && fz.q != nullptr;
-    const int e1 = 127 + (int)(coh ? load_coherent(q_stat + qrow * 4 + 0) : q_stat[qrow * 4 + 0]);
-    const int e2 = 127 + (int)(coh ? load_coherent(q_stat + qrow * 4 + 1) : q_stat[qrow * 4 + 1]);
+    const int e1 = 127 + (int)q_stat[qrow * 4 + 0];
+    const int e2 = 127 + (int)q_stat[qrow * 4 + 1];
     const int t01 = (n & 1) ? 7 : 2, t23 = t01 + 10;
     sa = (e1 - t01) | ((e1 - t23) << 8) | ((e2 - t01) << 16) | ((e2 - t23) << 24);
     if (NR) {                                    // one row set: byte 0 index planes, byte 2 sign plane
@@ -404,9 +344,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
       const int g = PP ? 2 * (kb & 1) + j : (NR ? kb : 2 * kb + j);
       const bool live = g < G && hf == 0;
       const int64_t qrow = (int64_t)b * Hq + h * G + (g < G ? g : 0);
-      const bool coh = fused_build && fz.q != nullptr;
-      const float c2 = coh ? load_coherent(q_stat + qrow * 4 + 2) : q_stat[qrow * 4 + 2];
-      const float c3 = coh ? load_coherent(q_stat + qrow * 4 + 3) : q_stat[qrow * 4 + 3];
+      const float c2 = q_stat[qrow * 4 + 2], c3 = q_stat[qrow * 4 + 3];
       cm[2 * j] = live ? c2 : 0.0f;
       cq[2 * j] = live ? c3 : 0.0f;
     }
@@ -1066,8 +1004,13 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   // counter, which the preparation kernel of this step has zeroed); the one that counts last merges.
   if (fm.out != nullptr) {
     __shared__ int s_last;
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");      // the partial's stores have completed ...
-    __syncthreads();                                            // ... in every wavefront
+    // Release: the partial was written with device-coherent (agent-scope, write-through) stores, so there is
+    // nothing to write back; what the hand-off needs is that every one of them has been acknowledged before
+    // the counter moves.  Each wavefront therefore waits for its own outstanding stores (s_waitcnt vmcnt(0):
+    // on this target stores count in vmcnt, and a workgroup-scope fence does not wait for them), the barrier
+    // collects all wavefronts, and only then does thread 0 count the workgroup in.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
     if (tid == 0) {
       const unsigned long long before = __hip_atomic_fetch_add(fm.counters + ((int64_t)b * Hkv + h), 1ull, __ATOMIC_RELAXED,
                                                                __HIP_MEMORY_SCOPE_AGENT);
@@ -1075,6 +1018,8 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
     }
     __syncthreads();
     if (s_last) {
+      // Acquire: the loads below are device-coherent loads issued after the counter's value has come back
+      // (s_last depends on it), and every other workgroup's stores were acknowledged before its increment.
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
 #pragma unroll
       for (int k = 0; k < 8 * D / (MF_WAVES * 64); ++k) {
@@ -1114,37 +1059,33 @@ template <int D, int MB, int NX, int VB, int GS, int DS, int WPS, bool F16P, boo
 static int launch_one(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, int kv_div,
                       const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
                       float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts, int n_split,
-                      int len_sub, int max_pages, int num_pages, const FusedPrep& fz, const FusedMerge& fm, bool wide_wg,
+                      int len_sub, int max_pages, int num_pages, const FusedMerge& fm, bool wide_wg,
                       hipStream_t st) {
   const int G = Hq / Hkv;
   size_t per_wave = (size_t)wave_lds_floats(D / DS / GS, DS) * sizeof(float);
   size_t merge = (size_t)(NW / DS * G * (D + 2) + NW * 16 * 16) * sizeof(float);
   if (SG) per_wave += stage_bytes((D / DS / 16) * VB / 2);
   size_t smem = per_wave * NW > merge ? per_wave * NW : merge;
-  if (fz.q) {
-    const size_t prep = (size_t)prep_unit_smem_floats(fz.hp, D) * sizeof(float);
-    if (prep > smem) smem = prep;
-  }
   if (D == 64 && !PP && G <= 4 && opt_page_pairs.load(std::memory_order_relaxed) != 0)
     return launch_one<D, MB, NX, VB, GS, DS, WPS, F16P, D == 64>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,
                                                                  bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts,
-                                                                 n_split, len_sub, max_pages, num_pages, fz, fm, wide_wg, st);
+                                                                 n_split, len_sub, max_pages, num_pages, fm, wide_wg, st);
   if (D >= 128 && !NR && G <= 4 && opt_narrow_rows.load(std::memory_order_relaxed) != 0)
     return launch_one<D, MB, NX, VB, GS, DS, WPS, F16P, false, D >= 128>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,
                                                                          bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts,
-                                                                         n_split, len_sub, max_pages, num_pages, fz, fm, wide_wg, st);
+                                                                         n_split, len_sub, max_pages, num_pages, fm, wide_wg, st);
   // (measured: the staged variant only pays where the register-held variant spills, i.e. with three index planes)
   constexpr bool can_stage = D >= 128 && MB == 3;
   if (can_stage && !SG && opt_lds_stage.load(std::memory_order_relaxed) != 0)
     return launch_one<D, MB, NX, VB, GS, DS, WPS, F16P, PP, NR, can_stage>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,
                                                                            bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts,
-                                                                           n_split, len_sub, max_pages, num_pages, fz, fm, wide_wg, st);
+                                                                           n_split, len_sub, max_pages, num_pages, fm, wide_wg, st);
   // eight wavefronts per workgroup (one workgroup per compute unit) for the kernels whose wavefronts work alone
   constexpr bool can_widen = DS == 1 && NW == MF_WAVES;
   if (can_widen && wide_wg)
     return launch_one<D, MB, NX, VB, GS, DS, WPS, F16P, PP, NR, SG, can_widen ? 2 * MF_WAVES : NW>(
         qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table, bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts, n_split,
-        len_sub, max_pages, num_pages, fz, fm, false, st);
+        len_sub, max_pages, num_pages, fm, false, st);
   // two workgroups of four wavefronts share a compute unit: see the kernel's comment on skew16.  Only the
   // head_dim 256 kernels, which are bound by instruction issue, gain (4 x 131072: 46.4 -> 45.5 us); the head_dim 128
   // kernels wait for memory, their workgroups advance side by side whatever their age, and unequal shares cost
@@ -1160,35 +1101,26 @@ static int launch_one(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, 
   if (take_time_hook(0, t_start_event, t_stop_event)) {
     hipExtLaunchKernelGGL(kern, grid, dim3(NW * 64), smem, st, t_start_event, t_stop_event, 0,
                           qa_pack, q_stat, Hq, Hkv, kv_div, pool, block_table, bt_stride, seq_lens, sm_scale, ly, L, parts,
-                          n_parts, n_split, len_sub, max_pages, num_pages, skew16, B, fz, fm);
+                          n_parts, n_split, len_sub, max_pages, num_pages, skew16, B, fm);
   } else {
     kern<<<grid, dim3(NW * 64), smem, st>>>(qa_pack, q_stat, Hq, Hkv, kv_div, pool, block_table, bt_stride, seq_lens,
                                             sm_scale, ly, L, parts, n_parts, n_split, len_sub, max_pages, num_pages, skew16,
-                                            B, fz, fm);
+                                            B, fm);
   }
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? TQ_OK : (int)e;
 }
 
 
-// the parameters of a layer that pick an instantiation (shared by the per-head-size launchers)
-struct MfmaShape { int d, mb, nx, vb, gs; bool f16p; };
-inline MfmaShape mfma_shape_of(const tq_layer& ly, const tq_page_layout& L) {
-  MfmaShape s{ly.d, ly.mse_bits, 0, L.value_bits, L.group_size, L.dtype == TQ_F16};
-  for (int t = 0; t < ly.n_terms; ++t)
-    if (__builtin_popcount(ly.term_mask[t]) > 1) ++s.nx;
-  return s;
-}
-
 #define TQ_TRY(D_, MB_, NX_, VB_, GS_, DS_, WPS_)                                                               \
   if (sh.d == D_ && sh.mb == MB_ && sh.nx == NX_ && sh.vb == VB_ && sh.gs == GS_) {                                            \
     if (sh.f16p)                                                                                                   \
       return launch_one<D_, MB_, NX_, VB_, GS_, DS_, WPS_, true>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,  \
                                                                  bt_stride, seq_lens, sm_scale, ly, L, parts,     \
-                                                                 n_parts, n_split, len_sub, max_pages, num_pages, fz, fm, wide_wg, st); \
+                                                                 n_parts, n_split, len_sub, max_pages, num_pages, fm, wide_wg, st); \
     return launch_one<D_, MB_, NX_, VB_, GS_, DS_, WPS_, false>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,   \
                                                                 bt_stride, seq_lens, sm_scale, ly, L, parts,      \
-                                                                n_parts, n_split, len_sub, max_pages, num_pages, fz, fm, wide_wg, st); \
+                                                                n_parts, n_split, len_sub, max_pages, num_pages, fm, wide_wg, st); \
   }
 
 }  // namespace tq

@@ -4,9 +4,6 @@
 #include <atomic>
 
 namespace tq {
-extern std::atomic<int> opt_fuse_prep;         // query preparation inside the page kernel's launch
-extern std::atomic<int> opt_prep_spin_limit;   // polls before a workgroup of that launch stops waiting for the others
-extern std::atomic<int> opt_prep_units;        // stand-alone preparation: one workgroup per (few heads, plane word) unit
 extern std::atomic<int> opt_append_parts;      // measurement: 3 keys and values (the product), 1 keys only, 2 values only
 extern std::atomic<int> opt_fp6_centroids;     // key quantiser, head_dim 128: centroid contraction on the fp6 x fp4 MFMA
 extern std::atomic<int> opt_page_pairs;        // decode, head_dim 64 with at most 4 query heads per KV head: one score MFMA per two pages

@@ -288,16 +288,6 @@ __device__ __forceinline__ void prep_query_body(const void* __restrict__ q, int 
   }
 }
 
-// ------------------------------------------------------------------------------------------------------
-// The same preparation as a prologue of the page kernel itself (256 threads): the work of a group of query
-// heads is cut into units = (up to `hp` consecutive heads g0.., plane word), and the workgroups that share
-// the group's pages each take some units, publish them, and wait for the others (see the page kernel).
-// The arithmetic - partial sums over 16 row slices, their order of summation, the statistics, the fp6
-// terms - is that of prep_query_body, so both give the same operands bit for bit.
-// PER = d / PREP_SLICES.  `sm`: prep_unit_smem_floats(hp, d) floats of LDS.  Ends with a barrier.
-// COH: the results are written with device-coherent stores (for readers in the same launch).
-constexpr int PREP_UNIT_THREADS = 256;
-
 // Stores / loads that are coherent across the whole device on their own (agent-scope atomics: they go
 // through the per-XCD L2 to the memory side), so that handing data from one workgroup to another needs no
 // cache write-back or invalidation, which cost tens of microseconds when hundreds of wavefronts issue them.
@@ -315,195 +305,6 @@ __device__ __forceinline__ float load_coherent(const float* p) {
 }
 __device__ __forceinline__ unsigned long long load_coherent(const unsigned long long* p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
-__host__ __device__ inline int prep_unit_smem_floats(int hp, int d) {
-  return hp * d + 2 * PREP_SLICES * hp * PREP_COLS + 2 * hp * PREP_COLS + 4 * ROT_MAX_ROWS + 16;
-}
-
-template <int PER, bool COH>
-__device__ __forceinline__ void prep_unit256(const void* __restrict__ q, int dtype, int G, const tq_layer& ly,
-                                             float sm_scale, float* __restrict__ q_stat,
-                                             uint32_t* __restrict__ qa_pack, int64_t group, int word, int g0, int hp,
-                                             float* sm) {
-  const int d = ly.d, tid = threadIdx.x, jl = tid % PREP_COLS, sl2 = tid / PREP_COLS;     // sl2 = 0..7
-  const int j = word * PREP_COLS + jl;
-  const int gn = max(min(G - g0, hp), 0);                // heads of this unit that exist
-  const int64_t row0 = group * G + (gn > 0 ? g0 : 0);    // (a unit of absent heads only writes zero rows)
-  // every global load of the unit is issued here, before anything waits
-  constexpr int QPT = ROT_MAX_ROWS;                      // query elements per thread (hp * d <= 8 * 256)
-  float qv[QPT];
-#pragma unroll
-  for (int k = 0; k < QPT; ++k) {
-    const int o = tid + k * PREP_UNIT_THREADS;
-    const float x = load_as_f32(q, row0 * d + min(o, max(gn * d - 1, 0)), dtype);
-    qv[k] = o < gn * d ? x : 0.0f;
-  }
-  float mp[2][PER], ms[2][PER];                          // the thread's two row slices: sl2 and sl2 + 8
-#pragma unroll
-  for (int half = 0; half < 2; ++half)
-#pragma unroll
-    for (int k = 0; k < PER; ++k) {
-      const int64_t r = (int64_t)((sl2 + 8 * half) * PER + k) * d + j;
-      mp[half][k] = ly.PiT[r];
-      ms[half][k] = ly.ST[r];
-    }
-  float cs1[4], cs2[4];
-#pragma unroll
-  for (int k = 0; k < 4; ++k) {
-    const int c = (tid & 63) + 64 * k;
-    cs1[k] = c < d ? ly.Pi_colsum[c] : 0.0f;
-    cs2[k] = c < d ? ly.S_colsum[c] : 0.0f;
-  }
-  float* sq = sm;                                          // [hp][d] raw query
-  float* pa = sq + hp * d;                                 // [PREP_SLICES][hp][PREP_COLS]
-  float* pb = pa + PREP_SLICES * hp * PREP_COLS;
-  float* srot = pb + PREP_SLICES * hp * PREP_COLS;         // [hp][PREP_COLS]
-  float* ssk = srot + hp * PREP_COLS;
-  float* stat = ssk + hp * PREP_COLS;                      // [hp][4]
-  float* coefs = stat + 4 * ROT_MAX_ROWS;                  // [16]
-#pragma unroll
-  for (int k = 0; k < QPT; ++k) {
-    const int o = tid + k * PREP_UNIT_THREADS;
-    if (o < gn * d) sq[o] = qv[k];
-  }
-  const int mb = ly.mse_bits;
-  int nx = 0;
-  float cmax = 0.0f;
-  for (int t = 0; t < ly.n_terms; ++t) {
-    cmax = fmaxf(cmax, fabsf(ly.term_coef[t]));
-    if (__builtin_popcount(ly.term_mask[t]) > 1) ++nx;
-  }
-  const int ntp = mb + nx + 1, wpl = d >= 128 ? d / 128 : 1;      // head_dim 64: one chunk of 128 with its upper half unused
-  if (tid < ntp) {
-    float coef = 1.0f;
-    if (tid < mb) {
-      coef = 0.0f;
-      for (int t = 0; t < ly.n_terms; ++t)
-        if (ly.term_mask[t] == (1 << (mb - 1 - tid))) coef = ly.term_coef[t];
-    } else if (tid < mb + nx) {
-      coef = 0.0f;
-      int seen = 0;
-      for (int t = 0; t < ly.n_terms; ++t) {
-        if (__builtin_popcount(ly.term_mask[t]) > 1) {
-          if (seen == tid - mb) coef = ly.term_coef[t];
-          ++seen;
-        }
-      }
-    }
-    coefs[tid] = coef;
-  }
-  __syncthreads();
-  {  // row statistics: one wavefront per row
-    const int lane = tid & 63, wave = tid >> 6;
-    for (int r = wave; r < gn; r += PREP_UNIT_THREADS / 64) {
-      float ss = 0.0f, s1 = 0.0f, s2 = 0.0f;
-#pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        const int c = lane + 64 * k;
-        const float x = c < d ? sq[r * d + c] : 0.0f;
-        ss = fmaf(x, x, ss);
-        s1 = fmaf(x, cs1[k], s1);
-        s2 = fmaf(x, cs2[k], s2);
-      }
-      ss = wave_sum_dpp(ss); s1 = wave_sum_dpp(s1); s2 = wave_sum_dpp(s2);
-      if (lane == 0) {
-        const float nq = sqrtf(ss), k = sm_scale * 1.4426950408889634f;
-        const int e1 = min(max((int)((__float_as_uint(fabsf(k) * nq * cmax) >> 23) & 255u) - 126, -100), 100);
-        const int e2 = min(max((int)((__float_as_uint(2.0f * fabsf(k * ly.qjl_scale) * nq * ly.S_rownorm_max) >> 23) & 255u) - 126, -100), 100);
-        stat[r * 4 + 0] = k * __uint_as_float((uint32_t)(127 - e1) << 23);
-        stat[r * 4 + 1] = 2.0f * k * ly.qjl_scale * __uint_as_float((uint32_t)(127 - e2) << 23);
-        if (word == 0) {
-          const float st4[4] = {(float)e1, (float)e2, k * ly.term_const * s1, -k * ly.qjl_scale * s2};
-#pragma unroll
-          for (int z = 0; z < 4; ++z) {
-            if (COH) store_coherent(q_stat + (row0 + r) * 4 + z, st4[z]);
-            else q_stat[(row0 + r) * 4 + z] = st4[z];
-          }
-        }
-      }
-    }
-  }
-  // contraction over this thread's two row slices
-#pragma unroll
-  for (int half = 0; half < 2; ++half) {
-    const int sl = sl2 + 8 * half, i0 = sl * PER;
-    float a[ROT_MAX_ROWS], b[ROT_MAX_ROWS];
-#pragma unroll
-    for (int r = 0; r < ROT_MAX_ROWS; ++r) a[r] = b[r] = 0.0f;
-#pragma unroll
-    for (int r = 0; r < ROT_MAX_ROWS; ++r) {
-      if (r < gn) {
-#pragma unroll
-        for (int k4 = 0; k4 < PER / 4; ++k4) {
-          const float4 x = *(const float4*)(sq + r * d + i0 + 4 * k4);
-          const float xs[4] = {x.x, x.y, x.z, x.w};
-#pragma unroll
-          for (int k = 0; k < 4; ++k) {
-            a[r] = fmaf(xs[k], mp[half][4 * k4 + k], a[r]);
-            b[r] = fmaf(xs[k], ms[half][4 * k4 + k], b[r]);
-          }
-        }
-      }
-    }
-#pragma unroll
-    for (int r = 0; r < ROT_MAX_ROWS; ++r) {
-      if (r < gn) {
-        pa[(sl * hp + r) * PREP_COLS + jl] = a[r];
-        pb[(sl * hp + r) * PREP_COLS + jl] = b[r];
-      }
-    }
-  }
-  __syncthreads();
-  for (int o2 = tid; o2 < 2 * gn * PREP_COLS; o2 += PREP_UNIT_THREADS) {     // first half: rotation, second: sketch
-    const bool sk = o2 >= gn * PREP_COLS;
-    const int o = sk ? o2 - gn * PREP_COLS : o2, r = o / PREP_COLS, c = o - r * PREP_COLS;
-    const float* part = sk ? pb : pa;
-    float acc = 0.0f;
-#pragma unroll
-    for (int k = 0; k < PREP_SLICES; ++k) acc += part[(k * hp + r) * PREP_COLS + c];
-    (sk ? ssk : srot)[o] = acc;
-  }
-  __syncthreads();
-  uint32_t* codes = (uint32_t*)pa;                           // [ntp][hp][4 terms][32]
-  for (int o = tid; o < ntp * gn * PREP_COLS; o += PREP_UNIT_THREADS) {
-    const int kloc = o & 31, g = (o >> 5) % gn, tp = (o >> 5) / gn;
-    const bool is_sign = tp == ntp - 1;
-    const int c = 4 * (kloc & 7) + (kloc >> 3);              // coordinate within the word
-    const int t4 = kloc >> 3;
-    const float mul = 4.0f * (is_sign ? stat[g * 4 + 1] : coefs[tp] * stat[g * 4 + 0]) *
-                      (t4 == 1 ? 0.5f : (t4 == 2 ? 0.25f : 1.0f));
-    float v = (is_sign ? ssk : srot)[g * PREP_COLS + c] * mul;
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      uint32_t code;
-      const float r = round_fp6(v, code);
-      codes[((tp * hp + g) * 4 + t) * PREP_COLS + kloc] = code;
-      v = (v - r) * 32.0f;
-    }
-  }
-  __syncthreads();
-  const int i = word >> 2, kw = word & 3;
-  uint32_t* dst = qa_pack + group * (int64_t)(ntp * wpl * 2 * 64 * 8);
-  // rows of this unit's heads, absent ones (zeros) included: (term plane, row set, head, term in the set, dword)
-  for (int o = tid; o < ntp * 2 * hp * 2 * 8; o += PREP_UNIT_THREADS) {
-    const int dwi = o & 7, tl = (o >> 3) & 1, g = (o >> 4) % hp, rs = ((o >> 4) / hp) & 1, tp = (o >> 4) / (2 * hp);
-    if (dwi >= 6) continue;
-    const int term = 2 * rs + tl, n = 2 * (g0 + g) + tl;
-    uint32_t packed = 0;
-    if (g < gn) {
-      const uint32_t* cd = codes + ((tp * hp + g) * 4 + term) * PREP_COLS;
-      const int j0 = (32 * dwi) / 6, j1 = min((32 * dwi + 31) / 6, 31);
-      for (int kloc = j0; kloc <= j1; ++kloc) {
-        const int bit = 6 * kloc - 32 * dwi;                 // position of the code in this dword (may straddle)
-        packed |= bit >= 0 ? cd[kloc] << bit : cd[kloc] >> -bit;
-      }
-    }
-    uint32_t* at = dst + (((tp * wpl + i) * 2 + rs) * 64 + n + 16 * kw) * 8 + dwi;
-    if (COH) store_coherent(at, packed);       // handed to other workgroups of the same launch
-    else *at = packed;
-  }
-  __syncthreads();
 }
 
 // LDS bytes of a preparation workgroup

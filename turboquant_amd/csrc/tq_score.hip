@@ -79,18 +79,6 @@ prep_query_kernel(const void* __restrict__ q, int G, int gpw, int64_t n_rows, tq
   prep_query_body<PER, DT, PACKED>(q, G, gpw, n_rows, ly, sm_scale, q_rot, q_sk, q_stat, qa_pack, arrivals, blockIdx.x, blockIdx.y, sm);
 }
 
-// The same preparation cut into more, smaller workgroups: one per unit = (hp consecutive heads of a group,
-// plane word), 256 threads (prep_unit256).  The launch is latency-bound, and a unit of one or two heads has
-// a shorter dependent chain than one workgroup per plane word doing all eight heads.
-template <int PER>
-__global__ void __launch_bounds__(PREP_UNIT_THREADS)
-prep_units_kernel(const void* __restrict__ q, int dtype, int G, tq_layer ly, float sm_scale, float* __restrict__ q_stat,
-                  uint32_t* __restrict__ qa_pack, int hp) {
-  extern __shared__ float sm[];
-  const int words = ly.d / PREP_COLS, u = blockIdx.x;
-  prep_unit256<PER, false>(q, dtype, G, ly, sm_scale, q_stat, qa_pack, blockIdx.y, u % words, (u / words) * hp, hp, sm);
-}
-
 // scores[b, i, k] for a tile of QT queries and one key per thread.  The rotated and sketched queries sit
 // in LDS as [coordinate][QT] rows, so a 16-byte broadcast read feeds four queries; a thread reads its key's
 // packed codes 32 coordinates (eff index words, one sign word) at a time.  NQ = 4 serves tiles of at most four
@@ -374,21 +362,6 @@ int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* 
   if (qa_pack) {       // operands of the matrix-core decode kernel wanted
     if (!q_stat || !layer->Pi_colsum || !layer->S_colsum || G > ROT_MAX_ROWS || rows % G || (d != 64 && d != 128 && d != 256))
       return TQ_EUNSUPPORTED;
-    if (opt_prep_units.load() && q_rot_unused && !arrivals) {
-      // heads per unit: as few as keep the launch at about a thousand workgroups
-      const int64_t groups = rows / G;
-      const int words = d / PREP_COLS;
-      int hp = 1;
-      while (hp < 8 && groups * ((G + hp - 1) / hp) * words > 1024) hp *= 2;
-      const dim3 ugrid((unsigned)((8 / hp) * words), (unsigned)groups);
-      const size_t usm = (size_t)prep_unit_smem_floats(hp, d) * sizeof(float);
-      if (groups > 65535) return TQ_EUNSUPPORTED;
-      if (d == 64) prep_units_kernel<4><<<ugrid, dim3(PREP_UNIT_THREADS), usm, st>>>(q, dtype, G, *layer, sm_scale, q_stat, qa_pack, hp);
-      else if (d == 128) prep_units_kernel<8><<<ugrid, dim3(PREP_UNIT_THREADS), usm, st>>>(q, dtype, G, *layer, sm_scale, q_stat, qa_pack, hp);
-      else prep_units_kernel<16><<<ugrid, dim3(PREP_UNIT_THREADS), usm, st>>>(q, dtype, G, *layer, sm_scale, q_stat, qa_pack, hp);
-      hipError_t e = hipGetLastError();
-      return e == hipSuccess ? TQ_OK : (int)e;
-    }
     // one group of heads per workgroup while the card holds all of them at once (three workgroups of 74 registers
     // per lane on each compute unit); beyond that, as many whole groups as fit a workgroup's eight rows
     // (64 x 2048 tokens at 32 q / 8 KV heads: 45.9 -> 42.2 us per step, 256 x 1024: 134 -> 121)
