@@ -336,6 +336,10 @@ void tq_time_next_page_kernel(void *start_event, void *stop_event);
 void tq_time_next_key_kernel(void *start_event, void *stop_event);
 
 /* Tuning and test knobs (no counterpart in the reference); process-wide, take effect at the next call.
+ *   "prefetch_trips"   0..64, default 1: the preparation launch of a step on the matrix-core path carries extra
+ *                      workgroups that read the pages every page-kernel workgroup asks for first (this many trips
+ *                      of each of its block walkers, at most 96 KB per workgroup) into the caches ahead of it;
+ *                      0: none.  Same result bit for bit.
  *   "merge_in_kernel"  1 (default): a compressed-only decode step on the matrix-core kernel with at most 8 context
  *                      splits has its splits merged by the last workgroup of the page kernel (two launches per
  *                      step); 0: always the separate merge kernel.

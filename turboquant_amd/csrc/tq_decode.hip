@@ -816,12 +816,14 @@ template <int PER, int DT, bool PAGED, bool PACKED>
 __global__ void __launch_bounds__(TAIL_THREADS, 4)
 prep_tail_kernel(TailArgs A, int n_tail, int B, int Gq, tq_layer ly, float* __restrict__ q_rot, float* __restrict__ q_sk,
                  float* __restrict__ q_stat, uint32_t* __restrict__ qa_pack, unsigned long long* __restrict__ arrivals,
-                 int prep_gpw) {
+                 int prep_gpw, int n_front, PagePrefetch pf) {
   extern __shared__ __align__(16) float sm[];
   const int id = blockIdx.x;
   if (id < n_tail) {
     const int per_z = A.Hkv * B;
     exact_tail_words_body<DT, 1, PAGED, true>(A, id % A.Hkv, (id / A.Hkv) % B, id / per_z, sm);
+  } else if (id >= n_front) {      // behind the tail and the preparation: the page kernel's first pages, read ahead of it
+    prefetch_pages_body(pf, id - n_front);
   } else {
     const int words = ly.d / PREP_COLS, p = id - n_tail;
     // (arrivals: the arrival counters of the groups of query heads, zeroed for a page kernel that merges its splits itself)
@@ -938,7 +940,7 @@ using namespace tq;
 namespace tq {
 int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* layer, float* q_rot, float* q_sk,
                         float* q_stat, uint32_t* qa_pack, int G, float sm_scale, hipStream_t st, bool q_rot_unused,
-                        unsigned long long* arrivals);
+                        unsigned long long* arrivals, const PagePrefetch* prefetch);
 }  // namespace tq
 
 static size_t parts_floats(int B, int Hq, int d, int n_parts) { return (size_t)B * Hq * n_parts * (d + 2); }
@@ -957,6 +959,7 @@ std::atomic<int> opt_wide_workgroups{1};
 std::atomic<int> opt_split_skew{1};
 std::atomic<int> opt_merge_row_groups{1};
 std::atomic<int> opt_tail_chunks{1};
+std::atomic<int> opt_prefetch_trips{1};
 }  // namespace tq
 
 extern "C" int tq_set_option(const char* name, int64_t value) {
@@ -965,6 +968,11 @@ extern "C" int tq_set_option(const char* name, int64_t value) {
   if (!std::strcmp(name, "split_skew")) {
     if (value < 0 || value > 8) return TQ_EINVAL;
     opt_split_skew.store((int)value);
+    return TQ_OK;
+  }
+  if (!std::strcmp(name, "prefetch_trips")) {
+    if (value < 0 || value > 64) return TQ_EINVAL;
+    opt_prefetch_trips.store((int)value);
     return TQ_OK;
   }
   if (!std::strcmp(name, "tail_chunks")) { opt_tail_chunks.store(value != 0); return TQ_OK; }
@@ -1110,6 +1118,18 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   }
   if (stages & 1) {
     if (!layer->Pi || !layer->PiT || !layer->S || !layer->ST || !layer->centroids) return TQ_ENULL;
+    // Workgroups added to the preparation launch read the first pages of every page-kernel workgroup's range
+    // ahead of it (the preparation leaves most of the card idle): prefetch_trips trips of each block walker.
+    PagePrefetch pf;
+    const int pf_trips = mfma_shape ? opt_prefetch_trips.load(std::memory_order_relaxed) : 0;
+    if (pf_trips > 0 && (int64_t)n_split * Hkv * kv_div * B <= 4096) {
+      decode_mfma_plan(pf, d, B, Hkv * kv_div, kv_div, n_split, wide_wg);
+      pf.pool = pool; pf.block_table = block_table; pf.seq_lens = seq_lens;
+      pf.bt_stride = bt_stride; pf.max_pages = max_pages; pf.num_pages = pool_pages; pf.len_sub = len_sub;
+      pf.page_bytes = (uint32_t)layout->page_bytes;
+      pf.page_stride = (uint32_t)((int64_t)Hkv * layout->page_bytes);
+      pf.blocks = pf_trips * pf.ngrp;
+    }
     // (in the launch shared with the tail a compute unit holds two workgroups: beyond that the preparation
     // workgroups take several groups of heads each, see prep_query_body)
     const int prep_gpw = prep_groups_per_workgroup(Gq, n_tail + (int64_t)(B * Hq / Gq) * (d / PREP_COLS),
@@ -1135,8 +1155,10 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
       hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)fsm);   \
       if (e != hipSuccess) return (int)e;                                                                            \
     }                                                                                                                \
-    kern<<<dim3((unsigned)(n_tail + n_prep)), dim3(TAIL_THREADS), fsm, st>>>(ta, n_tail, B, Gq, *layer, q_rot, q_sk,  \
-                                                                            q_stat, qa_pack, fm.counters, prep_gpw); \
+    pf.front = n_tail + n_prep;                                                                                      \
+    if (pf.front > 2 * device_compute_units()) pf.blocks = 0;                                                        \
+    kern<<<dim3((unsigned)(n_tail + n_prep + (pf.blocks > 0 ? pf.n_wg : 0))), dim3(TAIL_THREADS), fsm, st>>>(        \
+        ta, n_tail, B, Gq, *layer, q_rot, q_sk, q_stat, qa_pack, fm.counters, prep_gpw, n_tail + n_prep, pf);        \
   }
 #define TQ_LAUNCH_PT_DT(PER, PAGED)                                \
   {                                                                \
@@ -1161,7 +1183,7 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
     } else {
       int rc = launch_rotate_query(q, dtype, (int64_t)B * Hq, layer, q_rot, q_sk, q_stat,
                                    mfma_shape ? qa_pack : nullptr, mfma_shape ? Gq : G, sm_scale, st, mfma_shape,
-                                   fm.counters);
+                                   fm.counters, &pf);
       if (rc) return rc;
     }
   }

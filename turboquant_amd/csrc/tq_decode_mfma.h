@@ -18,6 +18,47 @@ struct FusedMerge {
 };
 constexpr int MERGE_IN_KERNEL_MAX_SPLITS = 8;
 
+// The blocks (64 tokens) a page-kernel workgroup walks: split `split` of n_split over a sequence of seq_len
+// compressed tokens.  skew16 > 0 (head_dim 256, two workgroups per compute unit): every even split takes skew16
+// sixteenths of a split's trips over from its odd neighbour; ngrp = block walkers of a workgroup.  The page kernel
+// and the page prefetch of the preparation launch both call this, so they agree on who reads what.
+__host__ __device__ inline void decode_block_range(int seq_len, int n_split, int split, int skew16, int ngrp,
+                                                   int& blk_begin, int& blk_end) {
+  const int n_blocks = (seq_len + 63) / 64;
+  const int per_split = (n_blocks + n_split - 1) / n_split;
+  blk_begin = split * per_split;
+  blk_end = blk_begin + per_split < n_blocks ? blk_begin + per_split : n_blocks;
+  if (skew16 > 0) {
+    int moved = ngrp * ((((per_split + ngrp - 1) / ngrp) * skew16 + 8) >> 4);
+    moved = moved < per_split ? moved : per_split;
+    if (split & 1) blk_begin = blk_begin + moved < blk_end ? blk_begin + moved : blk_end;
+    else blk_end = blk_end + moved < n_blocks ? blk_end + moved : n_blocks;
+  }
+}
+
+// Page prefetch inside the preparation launch of a decode step.  The preparation is a short, latency-bound
+// launch that leaves most compute units and the whole memory system idle; workgroups added to its grid read
+// the pages that every page-kernel workgroup will ask for first (the first `blocks` blocks of its range), so
+// that they sit in the cache hierarchy (the die's L2 when the reader shares the die, the memory-side cache
+// otherwise) when the page kernel starts.  Nothing depends on it: with blocks = 0 the step is the same minus
+// the head start.  The fields mirror the page kernel's launch (launch_one) so that the same ranges come out.
+struct PagePrefetch {
+  const uint8_t* pool = nullptr;
+  const int32_t* block_table = nullptr;
+  const int32_t* seq_lens = nullptr;
+  int bt_stride = 0, max_pages = 0, num_pages = 0, len_sub = 0;
+  int n_split = 0, groups = 0, kv_div = 1, n_seq = 0, skew16 = 0, ngrp = 1;
+  int gx = 1;                        // x extent of the page kernel's grid (n_split, or n_split / 2 with a skew)
+  uint32_t page_bytes = 0, page_stride = 0;
+  int blocks = 0;                    // blocks to read per page-kernel workgroup (0: no prefetch workgroups)
+  int n_wg = 0;                      // page-kernel workgroups = prefetch workgroups
+  int front = 0;                     // workgroups of this launch in front of the prefetch ones
+};
+
+// Shape of the page kernel's launch for a step (what launch_one will decide), for the prefetch: fills n_split,
+// groups, kv_div, n_seq, skew16, ngrp, gx, n_wg.
+void decode_mfma_plan(PagePrefetch& pf, int d, int B, int groups, int kv_div, int n_split, bool wide_wg);
+
 // Events armed by tq_time_next_page_kernel (which = 0) / tq_time_next_key_kernel (which = 1) on this thread:
 // returns them and disarms; false when none is armed.
 bool take_time_hook(int which, hipEvent_t& start, hipEvent_t& stop);

@@ -61,6 +61,15 @@ int decode_mfma_split_skew(int n_split, int rows) {
   return units > 0 && groups <= 2 * (int64_t)units && groups * 16 >= 30 * (int64_t)units ? skew : 0;
 }
 
+void decode_mfma_plan(PagePrefetch& pf, int d, int B, int groups, int kv_div, int n_split, bool wide_wg) {
+  const int ds = d == 256 ? 2 : 1, nw = wide_wg ? 2 * MF_WAVES : MF_WAVES;
+  pf.n_split = n_split; pf.groups = groups; pf.kv_div = kv_div; pf.n_seq = B;
+  pf.ngrp = nw / ds;
+  pf.skew16 = !wide_wg && ds == 2 ? decode_mfma_split_skew(n_split, groups * B) : 0;
+  pf.gx = pf.skew16 > 0 ? n_split / 2 : n_split;
+  pf.n_wg = n_split * groups * B;
+}
+
 // words of packed query operands tq_decode_attn_paged reserves in its workspace
 size_t decode_mfma_pack_words(int B, int Hq, int d) { return (size_t)B * Hq * 9 * (d / 128 + 1) * 1024; }   // d = 64: one chunk
 

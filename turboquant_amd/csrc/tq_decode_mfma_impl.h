@@ -368,15 +368,8 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   // len_sub: newest tokens that are attended to exactly.  A length beyond the block table is cut to the table.
   const int seq_len = max(min(seq_lens[b], max_pages * TQ_PAGE_TOKENS) - len_sub, 0);
   const int n_pages = (seq_len + TQ_PAGE_TOKENS - 1) / TQ_PAGE_TOKENS;
-  const int n_blocks = (seq_len + BLK_TOK - 1) / BLK_TOK;
-  const int per_split = (n_blocks + n_split - 1) / n_split;
-  int blk_begin = split * per_split;
-  int blk_end = min(n_blocks, blk_begin + per_split);
-  if (DS == 2 && skew16 > 0) {
-    const int moved = min(NGRP * ((((per_split + NGRP - 1) / NGRP) * skew16 + 8) >> 4), per_split);
-    if (split & 1) blk_begin = min(blk_begin + moved, blk_end);
-    else blk_end = min(blk_end + moved, n_blocks);
-  }
+  int blk_begin, blk_end;
+  decode_block_range(seq_len, n_split, split, DS == 2 ? skew16 : 0, NGRP, blk_begin, blk_end);
   const int32_t* bt = block_table + (int64_t)b * bt_stride;
   const uint8_t* pool_h = pool + (int64_t)(h / kv_div) * L.page_bytes;
   const int64_t page_stride = (int64_t)(Hkv / kv_div) * L.page_bytes;

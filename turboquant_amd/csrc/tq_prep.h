@@ -2,6 +2,7 @@
 #pragma once
 
 #include "tq_common.h"
+#include "tq_decode_mfma.h"
 
 namespace tq {
 
@@ -305,6 +306,63 @@ __device__ __forceinline__ float load_coherent(const float* p) {
 }
 __device__ __forceinline__ unsigned long long load_coherent(const unsigned long long* p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Prefetch workgroup p of a preparation launch (see PagePrefetch): reads, and discards, the pages that one
+// page-kernel workgroup will ask for first.  Workgroups go to the card's dies in turn, so the page-kernel
+// workgroup picked is the one whose position in its grid is congruent to this workgroup's position in this
+// grid: when the counts are multiples of eight the reader and the prefetcher share a die and its L2.
+__device__ __forceinline__ void prefetch_pages_body(const PagePrefetch& P, int p) {
+  int lin = p + P.front;
+  lin -= lin >= P.n_wg ? (lin / P.n_wg) * P.n_wg : 0;
+  int split = lin % P.gx;
+  const int rest = lin / P.gx;
+  int h = rest % P.groups, b = rest / P.groups;
+  if (P.kv_div > 1) {                                 // the groups of a KV head read the same pages: the first one's twin fetches
+    const int kv_heads = P.groups / P.kv_div;
+    if (h >= kv_heads) return;
+  }
+  if (P.skew16 > 0) {
+    const int late = b >= P.n_seq;
+    b -= late ? P.n_seq : 0;
+    split = 2 * split + late;
+  }
+  int seq_len = P.seq_lens[b];
+  seq_len = (seq_len < P.max_pages * TQ_PAGE_TOKENS ? seq_len : P.max_pages * TQ_PAGE_TOKENS) - P.len_sub;
+  seq_len = seq_len > 0 ? seq_len : 0;
+  const int n_pages = (seq_len + TQ_PAGE_TOKENS - 1) / TQ_PAGE_TOKENS;
+  int blk_begin, blk_end;
+  decode_block_range(seq_len, P.n_split, split, P.skew16, P.ngrp, blk_begin, blk_end);
+  const int blk_stop = blk_begin + P.blocks < blk_end ? blk_begin + P.blocks : blk_end;
+  const int pg0 = 4 * blk_begin, pg1 = 4 * blk_stop < n_pages ? 4 * blk_stop : n_pages;
+  const int32_t* bt = P.block_table + (int64_t)b * P.bt_stride;
+  const uint8_t* base = P.pool + (uint64_t)h * P.page_bytes;
+  // 16 bytes per lane; piece i of the range = piece i % pieces of page i / pieces.  Every table load is issued
+  // before the first page load and every page load before anything waits: the workgroup costs two memory
+  // latencies, whatever its share.  Slots beyond the range re-read the head's page 0 (in the pool, cached).
+  constexpr int SLOTS = 12;                            // per lane: 512 lanes x 12 x 16 bytes = 96 KB per workgroup
+  const int tid = threadIdx.x, pieces = (int)(P.page_bytes >> 4), total = (pg1 > pg0 ? pg1 - pg0 : 0) * pieces;
+  if (total <= 0) return;
+  const float inv_pieces = 1.0f / (float)pieces;
+  typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+  uint32_t pid[SLOTS], off[SLOTS];
+#pragma unroll
+  for (int k = 0; k < SLOTS; ++k) {
+    const int i = tid + 512 * k;
+    const int pg = (int)(((float)i + 0.5f) * inv_pieces);       // exact for the few thousand pieces of a range
+    const bool live = i < total;
+    off[k] = live ? (uint32_t)(i - pg * pieces) * 16u : 0u;
+    pid[k] = (uint32_t)bt[live ? pg0 + pg : pg0];              // (unconditional: a load under a branch would be waited for)
+  }
+  u32x4_t keep = {0u, 0u, 0u, 0u}, got[SLOTS];
+#pragma unroll
+  for (int k = 0; k < SLOTS; ++k) {
+    const uint32_t page = pid[k] < (uint32_t)P.num_pages ? pid[k] : 0u;
+    got[k] = *(const u32x4_t*)(base + (uint64_t)page * P.page_stride + off[k]);
+  }
+#pragma unroll
+  for (int k = 0; k < SLOTS; ++k) keep ^= got[k];
+  asm volatile("" :: "v"(keep));                      // the loads are wanted for their side effect
 }
 
 // LDS bytes of a preparation workgroup
