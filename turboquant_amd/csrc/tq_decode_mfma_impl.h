@@ -65,6 +65,16 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef int i32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
 typedef int i32x8 __attribute__((ext_vector_type(8)));
 
+// -DTQ_STAMPS (a profiling build, never the shipped one): lane 0 of every wavefront of the first 1024 workgroups
+// records the 100 MHz real-time counter at the kernel's phase boundaries - 0 start, 1 operands loaded, 2 first block
+// requested and table scanned, 3 loop done, 6 / 7 inside the epilogue, 4 partial stores issued, 5 stores acknowledged;
+// tq_debug_stamps copies them out.  The per-phase times quoted for the page kernels come from such a build.
+#ifdef TQ_STAMPS
+__device__ unsigned long long tq_stamps[4096 * 8];
+#define TQ_STAMP(k) do { if (lane == 0) tq_stamps[((blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z)) * 4 + wave) * 8 + (k)] = __builtin_amdgcn_s_memrealtime(); } while (0)
+#else
+#define TQ_STAMP(k)
+#endif
 constexpr int MF_WAVES = 4;
 constexpr int BLK_TOK = 64;              // tokens per wavefront iteration
 constexpr float MF_NEG = -1.0e30f;
@@ -272,6 +282,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wgrp = wave / DS, hf = wave % DS; // block walker this wavefront belongs to; its share of the head
   const int n = lane & 15, kb = lane >> 4;    // score stage: token / coordinate quarter; value stage: row / page
+  TQ_STAMP(0);
 
   extern __shared__ __align__(16) unsigned char smem_raw[];
   float* s_p = (float*)smem_raw + wave * WAVE_LDS_FLOATS;   // [4 pages][8 heads][P_STRIDE]
@@ -292,6 +303,9 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   // heads (row 2g + t), row set 1 = terms 2, 3; rows of absent heads are zero.  Six dwords per
   // lane are stored at a stride of eight.
   i32x8 qa[NTP][WPL][NRS];
+  int sa = 0;
+  f32x4 cm = {0, 0, 0, 0}, cq = {0, 0, 0, 0};
+  auto load_operands = [&]() {
   {
     // PP: rows 8..15 / coordinates 64..127 repeat rows 0..7 / coordinates 0..63; the off-diagonal blocks are zero
     // NR: row 4g + t is row 2g + t % 2 of row set t / 2
@@ -315,7 +329,6 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   // E8M0 block-scale codes of this lane's operand row (head n / 2), one per byte: index planes row
   // set 0, row set 1, sign plane row set 0, row set 1.  4 v / 2^E is stored, so term t carries
   // 2^(E - 2 - 5t); the fp4 bit value 0.5 carries 2^1.
-  int sa;
   {
     const int g = PP ? (n & 7) >> 1 : (NR ? n >> 2 : n >> 1);
     const int64_t qrow = (int64_t)b * Hq + h * G + (g < G ? g : 0);
@@ -328,26 +341,27 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
       sa = (e1 - tn) | ((e2 - tn) << 16);
     }
   }
+  // constant parts of the scores of the two heads this lane sees in the MFMA output (rows 4kb..4kb+3
+  // = heads 2kb, 2kb+1), as the initial accumulators; only one wavefront of a pair adds them
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) {
+    const int g = PP ? 2 * (kb & 1) + j : (NR ? kb : 2 * kb + j);
+    const bool live = g < G && hf == 0;
+    const int64_t qrow = (int64_t)b * Hq + h * G + (g < G ? g : 0);
+    const float c2 = q_stat[qrow * 4 + 2], c3 = q_stat[qrow * 4 + 3];
+    cm[2 * j] = live ? c2 : 0.0f;
+    cq[2 * j] = live ? c3 : 0.0f;
+  }
+  };
+  load_operands();
   const int sb = 127 + 1;
   // head_dim 64: the score MFMA still contracts 128 coordinates; the lanes of the upper two coordinate
   // quarters feed zeros (their masks are zero, whatever their loads return)
   const bool kq_live = D >= 128 || PP || kb < D / 32;
   const uint32_t nib = in_vgpr(kq_live ? 0x11111111u : 0u), nib1 = in_vgpr(kq_live ? 0x22222222u : 0u),
                  nib2 = in_vgpr(kq_live ? 0x44444444u : 0u);
-  // constant parts of the scores of the two heads this lane sees in the MFMA output (rows 4kb..4kb+3
-  // = heads 2kb, 2kb+1), as the initial accumulators; only one wavefront of a pair adds them
-  f32x4 cm = {0, 0, 0, 0}, cq = {0, 0, 0, 0};
   int xplanes[NX > 0 ? NX : 1];                 // which stored planes each extra term XORs
   {
-#pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-      const int g = PP ? 2 * (kb & 1) + j : (NR ? kb : 2 * kb + j);
-      const bool live = g < G && hf == 0;
-      const int64_t qrow = (int64_t)b * Hq + h * G + (g < G ? g : 0);
-      const float c2 = q_stat[qrow * 4 + 2], c3 = q_stat[qrow * 4 + 3];
-      cm[2 * j] = live ? c2 : 0.0f;
-      cq[2 * j] = live ? c3 : 0.0f;
-    }
     int seen = 0;
     for (int t = 0; t < ly.n_terms; ++t) {
       if (__builtin_popcount(ly.term_mask[t]) > 1 && seen < NX) {
@@ -364,6 +378,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
     // whose results nobody uses: keep them finite
     for (int i = lane; i < 4 * 8 * P_STRIDE + 16; i += 64) s_p[i] = 0.0f;
   }
+  TQ_STAMP(1);
   // ---------------------------------------------------------------- work range (all scalar)
   // len_sub: newest tokens that are attended to exactly.  A length beyond the block table is cut to the table.
   const int seq_len = max(min(seq_lens[b], max_pages * TQ_PAGE_TOKENS) - len_sub, 0);
@@ -832,14 +847,27 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
     auto run = [&](auto checked_tag) {
       constexpr bool CHECKED = decltype(checked_tag)::value;
       // one trip of a walker that still has a block; PARTIAL: some tokens of the block may not exist
-      auto trip = [&](int it, auto partial_tag) {
+      // LAST: the walker's last trip (a code instance of its own behind the loop): nothing is requested
+      auto trip = [&](int it, auto partial_tag, auto last_tag) {
+        constexpr bool LAST = decltype(last_tag)::value;
         // the block after this walker's last one does not exist: re-request the current one instead,
         // so that the loads stay outside any branch
         const int nxt = blk + NGRP;
         const int nxt_c = nxt < blk_end ? nxt : blk;
-        int pid_n[4];
-        const int bad_n = page_ids(nxt_c, pid_n, checked_tag);   // scalar loads, consumed after the score stage
-        if constexpr (SG) {
+        int pid_n[4] = {0, 0, 0, 0};
+        int bad_n = 0;
+        if constexpr (!LAST) bad_n = page_ids(nxt_c, pid_n, checked_tag);   // scalar loads, consumed after the score stage
+        if constexpr (LAST && !SG) {
+          const bool rescale = score_stage(blk, it, CHECKED ? fresh : it == 0, K, bad, partial_tag);
+          value_stage(blk, V, rescale, bad, partial_tag);
+        } else if constexpr (LAST) {
+          stage_wait<0>();                                  // this block's keys and values are all that is outstanding
+          fetch_keys(K);
+          const bool rescale = score_stage(blk, it, CHECKED ? fresh : it == 0, K, bad, partial_tag);
+          fetch_vals(V);
+          stage_release();
+          value_stage(blk, V, rescale, bad, partial_tag);
+        } else if constexpr (SG) {
           // outstanding, oldest first: this block's keys, this block's values
           stage_wait<V_OPS>();
           fetch_keys(K);
@@ -864,24 +892,27 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
       // A walker takes every NGRP-th block of the workgroup's range, so it can only run out of blocks,
       // and only meet the ragged end of the sequence, in the last trip: the loop before it is
       // straight-line code.
-      for (int it = 0; it < trips - 1; ++it) trip(it, std::integral_constant<bool, CHECKED>{});
+      for (int it = 0; it < trips - 1; ++it) trip(it, std::integral_constant<bool, CHECKED>{}, std::false_type{});
       if (trips > 0) {
         if (blk >= blk_end) {                              // uniform per wavefront pair
           if (DS > 1) __syncthreads();
         } else if (CHECKED || (blk + 1) * BLK_TOK > seq_len) {
-          trip(trips - 1, std::true_type{});
+          trip(trips - 1, std::true_type{}, std::true_type{});
         } else {
-          trip(trips - 1, std::false_type{});
+          trip(trips - 1, std::false_type{}, std::true_type{});
         }
       }
     };
+    TQ_STAMP(2);
     if (__builtin_amdgcn_ballot_w64(entry_bad) != 0) run(std::true_type{});
     else run(std::false_type{});
   }
 
   // ---------------------------------------------------------------- merge the walkers, write the partial
+  TQ_STAMP(3);
   if (SG) stage_wait<0>();   // the last trip's requests (a repeat of its own block) have landed
   __syncthreads();      // every wave is done with its private LDS region
+  TQ_STAMP(6);
   float* s_z = s_red + NGRP * G * (D + 2);                     // [MF_WAVES][16 rows][16 groups]
 #pragma unroll
   for (int i = 0; i < 4; ++i) s_z[(wave * 16 + 4 * kb + i) * 16 + n] = zacc[i];
@@ -927,6 +958,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
     }
   }
   __syncthreads();
+  TQ_STAMP(7);
   // merge of the walkers: thread -> (head, channel); loads are unconditional (clamped), stores guarded
   auto walkers_sum = [&](int g, int ch, float& mm, float& ll, float& aa) {
     float m_w[NGRP], l_w[NGRP], a_w[NGRP];
@@ -974,24 +1006,61 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
     }
     return;
   }
+  // The partial of this workgroup: a thread owns a pair of channels of HPP heads in turn.  All LDS reads of all
+  // passes are issued first and all stores last, so the epilogue pays one LDS latency and no wait inside a branch.
+  {
+    constexpr int PAIRS = D / 2, THREADS = MF_WAVES * 64;
+    constexpr int HPP = THREADS / PAIRS, NPASS = (8 + HPP - 1) / HPP;
+    const int pr = tid % PAIRS, hsub = tid / PAIRS;
+    float m_w[NPASS][NGRP], l_w[NPASS][NGRP];
+    f32x2 a_w[NPASS][NGRP];
 #pragma unroll
-  for (int k = 0; k < 8 * D / (MF_WAVES * 64); ++k) {
-    const int o = tid + k * (MF_WAVES * 64);
-    const bool live = o < G * D;
-    const int g = live ? o / D : 0, ch = o % D;
-    float mm, ll, aa;
-    walkers_sum(g, ch, mm, ll, aa);
-    if (live) {
-      float* out = parts + (((int64_t)b * Hq + h * G + g) * n_parts + split) * (D + 2);
-      if (fm.out != nullptr) {                 // read by another workgroup of this launch: device-coherent stores
-        if (ch == 0) { store_coherent(out, mm); store_coherent(out + 1, ll); }
-        store_coherent(out + 2 + ch, aa);
-      } else {
-        if (ch == 0) { out[0] = mm; out[1] = ll; }
-        out[2 + ch] = aa;
+    for (int ps = 0; ps < NPASS; ++ps) {
+      const int g = min(ps * HPP + hsub, G - 1);
+#pragma unroll
+      for (int w = 0; w < NGRP; ++w) {
+        const float* r = s_red + (w * G + g) * (D + 2);
+        const f32x2 ml = *(const f32x2*)r;
+        m_w[ps][w] = ml[0]; l_w[ps][w] = ml[1];
+        a_w[ps][w] = *(const f32x2*)(r + 2 + 2 * pr);
+      }
+    }
+    f32x2 res[NPASS], ml_out[NPASS];
+#pragma unroll
+    for (int ps = 0; ps < NPASS; ++ps) {
+      float mm = MF_NEG;
+#pragma unroll
+      for (int w = 0; w < NGRP; ++w) mm = fmaxf(mm, m_w[ps][w]);
+      float ll = 0.0f, a0 = 0.0f, a1 = 0.0f;
+#pragma unroll
+      for (int w = 0; w < NGRP; ++w) {
+        const float wgt = __expf(m_w[ps][w] - mm);
+        ll = fmaf(wgt, l_w[ps][w], ll);
+        a0 = fmaf(wgt, a_w[ps][w][0], a0);
+        a1 = fmaf(wgt, a_w[ps][w][1], a1);
+      }
+      res[ps] = f32x2{a0, a1};
+      ml_out[ps] = f32x2{mm, ll};
+    }
+    // Write-through (device-coherent) stores in every case.  A merging workgroup of this launch needs them
+    // (it reads the partial from another compute die); and with a merge kernel behind, partials that left the
+    // L2 as they were produced are not waiting for the write-back at the end of the kernel, which every
+    // launch pays before the next one starts (4 x 131072, 64 splits: page kernel 42.6 -> 42.2 us, step -0.45).
+#pragma unroll
+    for (int ps = 0; ps < NPASS; ++ps) {
+      const int g = ps * HPP + hsub;
+      if (g < G) {
+        float* out = parts + (((int64_t)b * Hq + h * G + g) * n_parts + split) * (D + 2);
+        store_coherent2(out + 2 + 2 * pr, res[ps]);
+        if (pr == 0) store_coherent2(out, ml_out[ps]);
       }
     }
   }
+  TQ_STAMP(4);
+#ifdef TQ_STAMPS
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  TQ_STAMP(5);
+#endif
   // ---------------------------------------------------------------- merge of the splits inside this launch
   // Every workgroup counts itself in after its partial has been written (one atomic increment of the group's
   // counter, which the preparation kernel of this step has zeroed); the one that counts last merges.

@@ -298,6 +298,11 @@ __device__ __forceinline__ void store_coherent(uint32_t* p, uint32_t v) {
 __device__ __forceinline__ void store_coherent(float* p, float v) {
   __hip_atomic_store((uint32_t*)p, __float_as_uint(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+// two floats at an 8-byte aligned address, as one 64-bit store
+__device__ __forceinline__ void store_coherent2(float* p, float __attribute__((ext_vector_type(2))) v) {
+  __hip_atomic_store((unsigned long long*)p, __builtin_bit_cast(unsigned long long, v), __ATOMIC_RELAXED,
+                     __HIP_MEMORY_SCOPE_AGENT);
+}
 __device__ __forceinline__ uint32_t load_coherent(const uint32_t* p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
