@@ -105,8 +105,8 @@ def test_config5_layer_at_full_size_against_the_oracle(gpu):
     """One attention layer of the 32-layer serving step at its full size: batch 32 x 32768 context tokens, 32
     query / 8 KV heads of 128, 3-bit keys, 4-bit values in groups of 32 (the shape every layer of the
     backend decode-step benchmark runs), pages a random permutation, default split count, sequences of
-    unequal length.  Four of the 32 sequences (the shortest, the longest and two in between) against the
-    oracle's de-quantise-everything attention on the same store (score.py:84-173)."""
+    unequal length.  Every sequence against the oracle's de-quantise-everything attention on the same store
+    (score.py:84-173)."""
     B, Hq, Hkv, d, N = 32, 32, 8, 128, 32768
     pages = N // 16
     pool, tq = _make_pool(gpu, d, 3, 4, Hkv, B * pages, torch.bfloat16, seed=42 + 7 * 5)
@@ -125,13 +125,15 @@ def test_config5_layer_at_full_size_against_the_oracle(gpu):
     out = pool.decode_attention(q.to(gpu), table, lens.to(gpu), max_len=N).cpu()
     torch.cuda.synchronize()
     prm = params_of(tq)
-    for b in (0, 9, 20, B - 1):
+    worst = 1.0
+    for b in range(B):
         n = int(lens[b])
         kc, vc = _store_from_oracle_view(pool, table[b], n)
         want = O.hybrid_attention(q[b:b + 1], kc, vc, n, prm, Hkv, None, None)
         c = cosine(out[b:b + 1], want)
-        _progress(f"config 5 layer: sequence {b} ({n} tokens) cosine {c:.8f}")
+        worst = min(worst, c)
         assert c >= COS_GATE, (b, c)
+    _progress(f"config 5 layer: all {B} sequences, worst cosine {worst:.8f} (1 - cos = {1 - worst:.2e})")
 
 
 @pytest.mark.parametrize("d,key_bits,dtype", [(576, 4, torch.bfloat16), (576, 3, torch.float32), (192, 4, torch.float16)])
@@ -786,3 +788,49 @@ def test_in_launch_merge_over_thousands_of_consecutive_steps(gpu):
                 assert at == 0, f"in-launch merge differs from its first result at step {at - 1}"
     finally:
         _set_option("merge_in_kernel", 1)
+
+
+@pytest.mark.parametrize("d,Hq,Hkv,vb,key_bits", [(128, 32, 8, 2, 3), (128, 32, 8, 4, 3), (128, 16, 2, 4, 4), (256, 16, 2, 2, 3)])
+def test_decode_over_a_store_with_outlier_channels(gpu, d, Hq, Hkv, vb, key_bits):
+    """Decode over a store built from the prefill workload's kind of data: bf16 N(0,1) keys and values with four
+    channels per (tensor, head) scaled by 20 (CPU generator seed 1, picked by randperm as in that workload), so
+    that a value group's scale and zero point are dominated by its outlier channel and the weight x scale and
+    weight x zero operands of the value stage carry large numbers.  Queries of three kinds per sequence - diffuse
+    (small norm: near-uniform weights over 4096 tokens), ordinary N(0,1), and peaked (aligned with one stored
+    key, so that a single token takes nearly all the weight) - against the oracle's de-quantise-everything
+    attention on the same store (score.py:138-173): cosine >= 0.9999 over a sequence's output, as everywhere.
+    Per query head the gate is 0.9995: the kernel rounds weight x scale and weight to bf16 (relative 2^-9 per
+    token), and in a group with an outlier channel sum(w zero) and sum(w scale code) are sixty times the value
+    they add up to, so a head whose mean value happens to be small shows 1 - cos of 1e-4 (measured worst head
+    1.4e-4 with 2-bit values and diffuse weights; the sequence's output is at 3e-5).  The margins are printed."""
+    g = torch.Generator().manual_seed(1)
+    B, N = 3, 4096
+    pages = N // 16
+    pool, tq = _make_pool(gpu, d, key_bits, vb, Hkv, B * pages + 2, torch.bfloat16, seed=42)
+    table = torch.randperm(B * pages + 2, generator=g)[: B * pages].to(torch.int32).view(B, pages).to(gpu)
+    k = torch.randn(B, N, Hkv, d, generator=g)
+    v = torch.randn(B, N, Hkv, d, generator=g)
+    for t in (k, v):
+        for h in range(Hkv):
+            t[:, :, h, torch.randperm(d, generator=g)[:4]] *= 20.0
+    k, v = k.bfloat16(), v.bfloat16()
+    pool.append(k.to(gpu), v.to(gpu), table)
+    G = Hq // Hkv
+    q = torch.randn(B, Hq, d, generator=g)
+    q[0] *= 0.02                                                       # diffuse
+    for hq in range(Hq):                                               # peaked: along key 1000 + hq of the head's KV head
+        kk = k[2, 1000 + hq, hq // G].float()
+        q[2, hq] = 6.0 * kk / kk.norm() * (d ** 0.5) / 8.0
+    q = q.bfloat16()
+    seq = torch.full((B,), N, dtype=torch.int32, device=gpu)
+    _progress(f"outlier store d={d} Hq={Hq} Hkv={Hkv} vb={vb} kb={key_bits}")
+    out = pool.decode_attention(q.to(gpu), table, seq).cpu()
+    prm = params_of(tq)
+    for b, kind in enumerate(("diffuse", "ordinary", "peaked")):
+        kc, vc = _store_from_oracle_view(pool, table[b], N)
+        want = O.hybrid_attention(q[b:b + 1], kc, vc, N, prm, Hkv, None, None)
+        per_head = [cosine(out[b, hq:hq + 1], want[0, hq:hq + 1]) for hq in range(Hq)]
+        c = cosine(out[b:b + 1], want)
+        _progress(f"   {kind}: cosine {c:.8f} (1 - cos = {1 - c:.2e}), worst head {min(per_head):.8f}")
+        assert c >= COS_GATE, (kind, c)
+        assert min(per_head) >= 0.9995, (kind, min(per_head))

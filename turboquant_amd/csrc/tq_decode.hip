@@ -1127,6 +1127,7 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
       pf.pool = pool; pf.block_table = block_table; pf.seq_lens = seq_lens;
       pf.bt_stride = bt_stride; pf.max_pages = max_pages; pf.num_pages = pool_pages; pf.len_sub = len_sub;
       pf.page_bytes = (uint32_t)layout->page_bytes;
+      pf.fetch_bytes = pf.page_bytes;       // (keys and norms alone, half the bytes, measured the same)
       pf.page_stride = (uint32_t)((int64_t)Hkv * layout->page_bytes);
       pf.blocks = pf_trips * pf.ngrp;
     }

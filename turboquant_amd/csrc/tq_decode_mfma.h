@@ -50,6 +50,7 @@ struct PagePrefetch {
   int n_split = 0, groups = 0, kv_div = 1, n_seq = 0, skew16 = 0, ngrp = 1;
   int gx = 1;                        // x extent of the page kernel's grid (n_split, or n_split / 2 with a skew)
   uint32_t page_bytes = 0, page_stride = 0;
+  uint32_t fetch_bytes = 0;          // leading bytes of a page that are read ahead (a multiple of 16, <= page_bytes)
   int blocks = 0;                    // blocks to read per page-kernel workgroup (0: no prefetch workgroups)
   int n_wg = 0;                      // page-kernel workgroups = prefetch workgroups
   int front = 0;                     // workgroups of this launch in front of the prefetch ones

@@ -15,3 +15,9 @@ int launch_decode_mfma_d128(uint32_t* qa_pack, float* q_stat, int B, int Hq, int
 }
 
 }  // namespace tq
+
+#ifdef TQ_STAMPS
+extern "C" int tq_debug_stamps_d128(unsigned long long* host, int n) {
+  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(tq::tq_stamps), (size_t)n * 8);
+}
+#endif

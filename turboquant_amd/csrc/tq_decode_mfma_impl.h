@@ -71,7 +71,7 @@ typedef int i32x8 __attribute__((ext_vector_type(8)));
 // tq_debug_stamps copies them out.  The per-phase times quoted for the page kernels come from such a build.
 #ifdef TQ_STAMPS
 __device__ unsigned long long tq_stamps[4096 * 8];
-#define TQ_STAMP(k) do { if (lane == 0) tq_stamps[((blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z)) * 4 + wave) * 8 + (k)] = __builtin_amdgcn_s_memrealtime(); } while (0)
+#define TQ_STAMP(k) do { if (lane == 0) tq_stamps[(((blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z)) * 8 + wave) * 8 + (k)) & 32767] = __builtin_amdgcn_s_memrealtime(); } while (0)
 #else
 #define TQ_STAMP(k)
 #endif

@@ -346,7 +346,7 @@ __device__ __forceinline__ void prefetch_pages_body(const PagePrefetch& P, int p
   // before the first page load and every page load before anything waits: the workgroup costs two memory
   // latencies, whatever its share.  Slots beyond the range re-read the head's page 0 (in the pool, cached).
   constexpr int SLOTS = 12;                            // per lane: 512 lanes x 12 x 16 bytes = 96 KB per workgroup
-  const int tid = threadIdx.x, pieces = (int)(P.page_bytes >> 4), total = (pg1 > pg0 ? pg1 - pg0 : 0) * pieces;
+  const int tid = threadIdx.x, pieces = (int)(P.fetch_bytes >> 4), total = (pg1 > pg0 ? pg1 - pg0 : 0) * pieces;
   if (total <= 0) return;
   const float inv_pieces = 1.0f / (float)pieces;
   typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
