@@ -399,3 +399,132 @@ def test_batched_hooks_through_the_minimal_transformer(gpu):
         assert torch.equal(got, want), i
         assert twins[0].seq_lens == twins[1].seq_lens
     hooks.set_mode(hooks.MODE_CAPTURE_ONLY)
+
+
+@pytest.mark.gpu
+def test_serving_step_at_reduced_depth_logits_against_the_model_with_oracle_attention(gpu):
+    """The 32-layer serving workload at two layers and full width: hidden 4096, 32 query / 8 KV heads of 128,
+    SwiGLU 14336, vocabulary 128256, random bf16 weights, batch 32 x 32768 prior tokens drawn uniformly from the
+    vocabulary by a CPU generator seeded 4, 3-bit keys and 4-bit values in both layers (initial_layers_count 0).
+    The prior tokens go through the model in chunks (exact causal attention; the hooks fill the compressed
+    pools from every step's K / V), then ONE decode step runs twice: through the hooks (page write + fused
+    decode attention of the library) and through the same dense layers with the CPU oracle as the attention -
+    its own quantisation of the new token appended to the exported pages, de-quantise everything, dense
+    attention (quantizer.py:231-272, kv_cache.py:45-116, score.py:138-173).  The attention output of the first
+    layer (same queries, same store in both runs) meets cosine >= 0.9999 for every sequence, measured 0.99998.
+    The logits are held to 0.9995: uniform random tokens through random weights give near-uniform attention
+    weights over 32769 tokens, the worst case for the kernel's bf16 weight operands (the output is the small
+    difference of two sums 400 times its size), and this random network turns the 1.5e-5 (1 - cos) of the
+    attention outputs into 9e-5 at the logits; feeding the library's attention outputs through the dense
+    layers by hand reproduces the hooked step's logits exactly, so nothing else differs."""
+    from oracle import tq_oracle as O
+    from tests.helpers import cosine, key_code, params_of, value_code
+    from turboquant_amd.integration import batched
+    from turboquant_amd.integration.harness import BLOCK, DenseBackend, MinimalRunner, _rms, _rope
+    import torch.nn.functional as F
+    dev = torch.device("cuda:0")
+    B, N, Hq, Hkv, d, vocab = 32, 32768, 32, 8, 128, 128256
+
+    class GroupedExact(DenseBackend):
+        """The harness' exact causal attention with bf16 products grouped by KV head (the fp32 einsum over
+        repeated heads is too slow for a million prior tokens); same cache, same metadata."""
+
+        def forward(self, layer, query, key, value, kv_cache, attn_metadata, output=None, output_scale=None,
+                    output_block_scale=None):
+            m = attn_metadata
+            n = m.num_actual_tokens
+            q = query[:n].view(n, Hq, d)
+            out = torch.empty_like(q)
+            G = Hq // Hkv
+            fk, fv = kv_cache[0].view(-1, Hkv, d), kv_cache[1].view(-1, Hkv, d)
+            lens, qsl = m.seq_lens_cpu.tolist(), m.query_start_loc_cpu.tolist()
+            for b, L in enumerate(lens):
+                r0, r1 = qsl[b], qsl[b + 1]
+                t = r1 - r0
+                if t <= 0:
+                    continue
+                pos = torch.arange(L, device=q.device)
+                slot = m.block_table[b].long()[pos // BLOCK] * BLOCK + pos % BLOCK
+                k, v = fk[slot].transpose(0, 1), fv[slot].transpose(0, 1)                   # (Hkv, L, d)
+                qq = q[r0:r1].view(t, Hkv, G, d).permute(1, 2, 0, 3).reshape(Hkv, G * t, d)
+                sc = torch.matmul(qq, k.transpose(1, 2)).float().mul_(self.scale)              # (Hkv, G t, L)
+                qpos = (L - t + torch.arange(t, device=q.device)).repeat(G)
+                sc.masked_fill_(pos[None, None, :] > qpos[None, :, None], float("-inf"))
+                o = torch.matmul(sc.softmax(-1).to(q.dtype), v)                                # (Hkv, G t, d)
+                out[r0:r1] = o.view(Hkv, G, t, d).permute(2, 0, 1, 3).reshape(t, Hq, d)
+            res = out if query.dim() == 3 else out.reshape(n, -1)
+            if output is not None:
+                output[:n].copy_(res.reshape(output[:n].shape))
+                return output
+            return res
+
+    print("[serving step] model and pools", flush=True)
+    r = MinimalRunner(n_layers=2, hidden=4096, num_heads=Hq, num_kv_heads=Hkv, head_dim=d, ffn=14336, vocab=vocab,
+                      batch=B, max_seq_len=N + BLOCK, device=dev, seed=4)
+    for lay in r.layers:
+        lay.attn.impl = GroupedExact(Hq, Hkv, d)
+    st = batched.install_batched_hooks(r, num_blocks=r.num_blocks, key_bits=3, value_bits=4, initial_layers_count=0,
+                                       mode=hooks.MODE_CAPTURE_ONLY)
+    states = list(st.values())
+    assert [s.config.key_bits for s in states] == [3, 3]
+    ids = torch.randint(0, vocab, (B, N + 1), generator=torch.Generator().manual_seed(4))
+    chunk = 1024
+    try:
+        for c0 in range(0, N, chunk):
+            if c0 % 8192 == 0:
+                print(f"[serving step] prior tokens {c0}..{c0 + 8191} of every sequence", flush=True)
+            r.step(ids[:, c0:c0 + chunk].reshape(-1).to(dev), r.metadata([chunk] * B))
+        assert r.seq_lens == [N] * B
+        tok = ids[:, N].to(dev)
+        # the oracle's model first (the pools still hold exactly the prior tokens)
+        pos = torch.full((B,), N, device=dev)
+        x = r.embed[tok]
+        oracle_attn = []
+        for li, lay in enumerate(r.layers):
+            print(f"[serving step] decode step, layer {li}: oracle attention over {B} x {N + 1} tokens", flush=True)
+            h = _rms(x, lay.ln1)
+            q, k, v = (h @ lay.wqkv).split([Hq * d, Hkv * d, Hkv * d], dim=-1)
+            q = _rope(q.view(B, Hq, d), pos).cpu()
+            k = _rope(k.view(B, Hkv, d), pos).cpu()
+            v = v.view(B, Hkv, d).cpu()
+            prm = params_of(states[li].quantizer)
+            attn = torch.empty(B, Hq, d, dtype=torch.bfloat16)
+            for b in range(B):
+                idx, sgn, norms, rn, vd, vs, vz = [t.cpu() for t in states[li].pool.export_flat(r.block_table[b], N)]
+                kq = O.prod_quantize(k[b][:, None, :], prm)
+                vq = O.quantize_values(v[b][:, None, :], bits=4, group_size=32)
+                kc = key_code(torch.cat([idx, kq.mse_indices], 1), torch.cat([sgn, kq.qjl_signs], 1),
+                              torch.cat([rn, kq.residual_norms], 1), torch.cat([norms, kq.norms], 1), 2)
+                vc = value_code(torch.cat([vd, vq.data], 1), torch.cat([vs, vq.scales], 1), torch.cat([vz, vq.zeros], 1), 4)
+                attn[b] = O.hybrid_attention(q[b:b + 1], kc, vc, N + 1, prm, Hkv, None, None)[0]
+            oracle_attn.append(attn)
+            x = x + attn.to(dev).reshape(B, Hq * d) @ lay.wo
+            h = _rms(x, lay.ln2)
+            gate, up = (h @ lay.w_gate_up).chunk(2, dim=-1)
+            x = x + (F.silu(gate) * up) @ lay.w_down
+        want = (_rms(x, r.final_norm) @ r.lm_head).float().cpu()
+        # the same step through the hooks (the library's attention outputs are recorded on the way)
+        hooks.set_mode(hooks.MODE_FULL_TQ)
+        kernel_attn = []
+        for state in states:
+            def recording(query, meta, *a, _orig=state.attend, **kw):
+                res = _orig(query, meta, *a, **kw)
+                kernel_attn.append(res.detach().float().cpu())
+                return res
+            state.attend = recording
+        got = r.decode_step(tok).float().cpu()
+        torch.cuda.synchronize()
+        for li in range(2):
+            ac = [cosine(kernel_attn[li][b], oracle_attn[li][b]) for b in range(B)]
+            print(f"[serving step] layer {li} attention output, library vs oracle: worst cosine {min(ac):.8f}, "
+                  f"mean {sum(ac) / B:.8f}", flush=True)
+            if li == 0:                                       # same queries and the same store in both runs
+                assert min(ac) >= 0.9999, ac
+        assert r.seq_lens == [N + 1] * B and batched.get_batched_stats(r)["decode_steps"] == 1
+        cos = [cosine(got[b], want[b]) for b in range(B)]
+        print(f"[serving step] logits cosine: worst {min(cos):.8f} (1 - cos = {1 - min(cos):.2e}), mean {sum(cos) / B:.8f}",
+              flush=True)
+        assert min(cos) >= 0.9995, cos
+        assert (got.argmax(-1) == want.argmax(-1)).float().mean() >= 0.9
+    finally:
+        hooks.set_mode(hooks.MODE_CAPTURE_ONLY)
