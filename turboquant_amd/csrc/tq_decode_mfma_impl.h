@@ -200,12 +200,14 @@ __device__ __forceinline__ f32x4 mfma_f8f4(const i32x8& a, uint32_t b0, uint32_t
 // token held by element (r, h) of MFMA half u of the value stage
 template <int VB>
 __device__ __forceinline__ constexpr int v_token(int u, int r, int h) {
-  return VB == 2 ? 4 * u + r + 8 * h : 8 * u + r + 4 * h;
+  // (8-bit codes: dword j of a channel's field holds tokens 4j..4j+3, a byte each; its even bytes are one operand
+  // dword, its odd bytes the next)
+  return VB == 2 ? 4 * u + r + 8 * h : (VB == 4 ? 8 * u + r + 4 * h : 8 * u + 4 * (r >> 1) + (r & 1) + 2 * h);
 }
 // bit position (inside its byte) of the code of token t: the weight of the token carries 2^-pos
 template <int VB>
 __device__ __forceinline__ constexpr int v_bitpos(int t) {
-  return VB == 2 ? 2 * (t & 3) : 4 * (t & 1);
+  return VB == 2 ? 2 * (t & 3) : (VB == 4 ? 4 * (t & 1) : 0);
 }
 
 // D in {128, 256}; MB stored index bits; NX extra (multi-bit) Walsh terms; VB value bits;
@@ -549,7 +551,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   // exactly (denormals, and the first binade continues them linearly), so B = code * 2^(s - 133)
   // where s is the bit position the code has inside its byte; the softmax weight carries 2^(80 - s).
   // Only the codes in the upper byte of each half need a shift.
-  const uint32_t m0 = in_vgpr(VB == 2 ? 0x00030003u : 0x000F000Fu);
+  const uint32_t m0 = in_vgpr(VB == 2 ? 0x00030003u : (VB == 4 ? 0x000F000Fu : 0x00FF00FFu));
   const uint32_t m1 = in_vgpr(VB == 2 ? 0x000C000Cu : 0x00F000F0u), m2 = in_vgpr(0x00300030u), m3 = in_vgpr(0x00C000C0u);
 
   // ---------------------------------------------------------------- one block of 64 tokens
@@ -789,10 +791,15 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
             // 16 two-bit fields; register r of MFMA u takes fields 4u+r (low half) and 4u+r+8 (high half)
             const uint32_t x = u == 0 ? V.v[c] : V.v[c] >> 8;
             bc = u32x4{x & m0, x & m1, x & m2, x & m3};
-          } else {
+          } else if (VB == 4) {
             // 8 four-bit fields; register r takes fields r (low half) and r+4 (high half)
             const uint32_t x = V.v[2 * c + u], x8 = x >> 8;
             bc = u32x4{x & m0, x & m1, x8 & m0, x8 & m1};
+          } else {
+            // four bytes per dword: the even bytes are one register (a code in the low byte of each half is a bf16
+            // denormal as it stands), the odd bytes, shifted down, the next
+            const uint32_t x = V.v[4 * c + 2 * u], y = V.v[4 * c + 2 * u + 1];
+            bc = u32x4{x & m0, (x >> 8) & m0, y & m0, (y >> 8) & m0};
           }
           acc[c] = mfma(aw[u], bc, acc[c]);
         }

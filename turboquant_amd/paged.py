@@ -172,7 +172,9 @@ class PagedKVPool:
         keys, query heads that split into groups of at most 8); only the split heuristic depends on it."""
         if self.head_dim not in (64, 128, 256) or self.dtype not in (torch.bfloat16, torch.float16):
             return False
-        if self.quantizer.bits - 1 > 3 or self.value_bits not in (2, 4) or self.value_group_size not in (32, 64):
+        if self.quantizer.bits - 1 > 3 or self.value_bits not in (2, 4, 8) or self.value_group_size not in (32, 64):
+            return False
+        if self.value_bits == 8 and (self.quantizer.bits != 3 or self.value_group_size != 32):
             return False
         if Hq is None:
             return True
