@@ -566,12 +566,16 @@ def shape_kq_128(k, trend):
                                                          (128, 3, 4, 12, 1, torch.bfloat16), (256, 3, 2, 18, 2, torch.bfloat16),
                                                          (128, 3, 2, 11, 1, torch.bfloat16), (128, 4, 4, 32, 2, torch.float16),
                                                          (576, 3, 2, 16, 1, torch.bfloat16), (768, 2, 4, 4, 2, torch.float32),
-                                                         (192, 3, 4, 6, 2, torch.float16), (64, 5, 2, 10, 2, torch.bfloat16)])
+                                                         (192, 3, 4, 6, 2, torch.float16), (64, 5, 2, 10, 2, torch.bfloat16),
+                                                         (128, 3, 4, 22, 2, torch.bfloat16), (256, 3, 2, 26, 2, torch.bfloat16),
+                                                         (64, 3, 4, 9, 1, torch.float16), (128, 3, 4, 15, 1, torch.bfloat16),
+                                                         (128, 3, 8, 20, 2, torch.bfloat16)])
 def test_decode_attention_general_kernel_shapes(gpu, d, key_bits, vb, Hq, Hkv, dtype):
     # fp16 pools (matrix-core kernel with the fp16 zero-point product), more than 8 query heads per KV head
-    # (served as groups of at most 8: 16 = 2 x 8, 12 = 2 x 6, 9 = 3 x 3), and shapes without a
-    # matrix-core kernel (fp32 pools, head_dim 64, 11 query heads per KV head)
-    # take the general page kernel and must meet the same gate
+    # (served as ceil(G / 8) groups of at most 8 that read the same pages: 16 = 8 + 8, 12 = 6 + 6, and unequal ones
+    # where G does not divide: 9 = 5 + 4, 11 = 6 + 5, 13 = 7 + 6, 15 = 8 + 7), and shapes without a matrix-core
+    # kernel (fp32 pools, head sizes other than 64 / 128 / 256, 5-bit keys), which take the general page kernel:
+    # all must meet the same gate
     _progress(f"general decode d={d} kb={key_bits} vb={vb} Hq={Hq} Hkv={Hkv} {dtype}")
     worst = _decode_case(gpu, d, key_bits, vb, 2, Hq, Hkv, [300, 77], [0, 9], seed=500 + d + Hq, dtype=dtype)
     _progress(f"   worst cosine {worst:.7f}")

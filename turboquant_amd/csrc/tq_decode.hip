@@ -816,7 +816,7 @@ template <int PER, int DT, bool PAGED, bool PACKED>
 __global__ void __launch_bounds__(TAIL_THREADS, 4)
 prep_tail_kernel(TailArgs A, int n_tail, int B, int Gq, tq_layer ly, float* __restrict__ q_rot, float* __restrict__ q_sk,
                  float* __restrict__ q_stat, uint32_t* __restrict__ qa_pack, unsigned long long* __restrict__ arrivals,
-                 int prep_gpw, int n_front, PagePrefetch pf) {
+                 int prep_gpw, int n_front, PagePrefetch pf, int g_tot) {
   extern __shared__ __align__(16) float sm[];
   const int id = blockIdx.x;
   if (id < n_tail) {
@@ -827,7 +827,7 @@ prep_tail_kernel(TailArgs A, int n_tail, int B, int Gq, tq_layer ly, float* __re
   } else {
     const int words = ly.d / PREP_COLS, p = id - n_tail;
     // (arrivals: the arrival counters of the groups of query heads, zeroed for a page kernel that merges its splits itself)
-    prep_query_body<PER, DT, PACKED>(A.q, Gq, prep_gpw, (int64_t)B * A.Hq, ly, A.sm_scale, q_rot, q_sk, q_stat, qa_pack,
+    prep_query_body<PER, DT, PACKED>(A.q, Gq, prep_gpw, (int64_t)B * A.Hq, g_tot, ly, A.sm_scale, q_rot, q_sk, q_stat, qa_pack,
                                      arrivals, p / words, p % words, sm);
   }
 }
@@ -940,7 +940,7 @@ using namespace tq;
 namespace tq {
 int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* layer, float* q_rot, float* q_sk,
                         float* q_stat, uint32_t* qa_pack, int G, float sm_scale, hipStream_t st, bool q_rot_unused,
-                        unsigned long long* arrivals, const PagePrefetch* prefetch);
+                        unsigned long long* arrivals, const PagePrefetch* prefetch, int g_tot);
 }  // namespace tq
 
 static size_t parts_floats(int B, int Hq, int d, int n_parts) { return (size_t)B * Hq * n_parts * (d + 2); }
@@ -1053,11 +1053,9 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   const int len_sub = tail && ts.paged ? recent_rows : 0;       // newest tokens the pages do not cover
   hipStream_t st = (hipStream_t)stream;
   // the matrix-core kernel takes up to 8 query heads per group: a KV head with more is served by kv_div
-  // groups of G / kv_div heads (0 = no such split, e.g. 11 heads)
-  int kv_div = 0;
-  for (int n = 1; n <= G && !kv_div; ++n)
-    if (G % n == 0 && G / n <= 8) kv_div = n;
-  const int Gq = kv_div ? G / kv_div : G;
+  // groups of Gq = ceil(G / kv_div) heads, the last one of fewer when G does not divide (11 heads: 6 + 5)
+  const int kv_div = (G + 7) / 8;
+  const int Gq = (G + kv_div - 1) / kv_div;
   // (the same table the launchers dispatch over: a shape without an instantiation keeps its split count and takes
   // the general kernel's preparation, which writes the fp32 rotated / sketched queries that kernel reads)
   const bool mfma_shape = kv_div && layer->Pi_colsum && layer->S_colsum && decode_mfma_has_kernel(*layer, *layout);
@@ -1133,10 +1131,12 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
     }
     // (in the launch shared with the tail a compute unit holds two workgroups: beyond that the preparation
     // workgroups take several groups of heads each, see prep_query_body)
-    const int prep_gpw = prep_groups_per_workgroup(Gq, n_tail + (int64_t)(B * Hq / Gq) * (d / PREP_COLS),
-                                                   2 * (int64_t)device_compute_units());
+    // (groups of unequal size - the heads of a KV head do not divide into kv_div groups - take one workgroup each)
+    const int g_tot = kv_div > 1 && G % kv_div ? G : 0;
+    const int prep_gpw = g_tot ? 1 : prep_groups_per_workgroup(Gq, n_tail + (int64_t)(B * Hq / Gq) * (d / PREP_COLS),
+                                                               2 * (int64_t)device_compute_units());
     const int prep_rows = Gq * prep_gpw;                          // query rows of a preparation workgroup
-    const int n_prep = (B * Hq + prep_rows - 1) / prep_rows * (d / PREP_COLS);
+    const int n_prep = (g_tot ? B * Hkv * kv_div : (B * Hq + prep_rows - 1) / prep_rows) * (d / PREP_COLS);
     // Whole hybrid step on the matrix-core path: the exact tail shares the preparation's launch (the tail
     // workgroups first, so that the longer-running ones start first).  The kernel is built for 128 registers
     // per lane and the tail's LDS is sized by the rows it holds, so two workgroups fit a compute unit; with more
@@ -1159,7 +1159,7 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
     pf.front = n_tail + n_prep;                                                                                      \
     if (pf.front > 2 * device_compute_units()) pf.blocks = 0;                                                        \
     kern<<<dim3((unsigned)(n_tail + n_prep + (pf.blocks > 0 ? pf.n_wg : 0))), dim3(TAIL_THREADS), fsm, st>>>(        \
-        ta, n_tail, B, Gq, *layer, q_rot, q_sk, q_stat, qa_pack, fm.counters, prep_gpw, n_tail + n_prep, pf);        \
+        ta, n_tail, B, Gq, *layer, q_rot, q_sk, q_stat, qa_pack, fm.counters, prep_gpw, n_tail + n_prep, pf, g_tot); \
   }
 #define TQ_LAUNCH_PT_DT(PER, PAGED)                                \
   {                                                                \
@@ -1184,7 +1184,7 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
     } else {
       int rc = launch_rotate_query(q, dtype, (int64_t)B * Hq, layer, q_rot, q_sk, q_stat,
                                    mfma_shape ? qa_pack : nullptr, mfma_shape ? Gq : G, sm_scale, st, mfma_shape,
-                                   fm.counters, &pf);
+                                   fm.counters, &pf, mfma_shape ? g_tot : 0);
       if (rc) return rc;
     }
   }
@@ -1357,9 +1357,7 @@ int scratch_address(void** out) {
 // per group of query heads.
 size_t decode_scratch_need(int B, int Hq, int Hkv, int n_split, const tq_layer& ly) {
   const int d = ly.d, G = Hq / Hkv;
-  int kv_div = 0;
-  for (int n = 1; n <= G && !kv_div; ++n)
-    if (G % n == 0 && G / n <= 8) kv_div = n;
+  const int kv_div = (G + 7) / 8;
   size_t floats = parts_floats(B, Hq, d, n_split + TAIL_MAX_CHUNKS) + (size_t)2 * B * Hq * d + (size_t)4 * B * Hq +
                   2 * counter_words(B, Hq);
   size_t words = 0;

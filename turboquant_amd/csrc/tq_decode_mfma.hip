@@ -107,7 +107,7 @@ int launch_decode_mfma(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv,
                        float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts,
                        int n_split, int len_sub, int max_pages, int num_pages, const FusedMerge& fm,
                        bool wide_wg, hipStream_t st) {
-  const int G = Hq / Hkv, d = ly.d;
+  const int G = kv_div > 1 ? (Hq / (Hkv / kv_div) + kv_div - 1) / kv_div : Hq / Hkv, d = ly.d;
   if (G > 8 || (L.dtype != TQ_BF16 && L.dtype != TQ_F16) || !L.key_lane_major) return TQ_EUNSUPPORTED;
   if (d == 64) return launch_decode_mfma_d64(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table, bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts, n_split,
                                    len_sub, max_pages, num_pages, fm, wide_wg, st);

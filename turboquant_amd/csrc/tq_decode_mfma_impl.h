@@ -256,9 +256,10 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   constexpr int STAGE_BYTES = stage_bytes(VW);
   constexpr int NRS = NR ? 1 : 2;             // fp6 operands (row sets) per plane word
   constexpr int NJ = NR ? 1 : 2;              // heads a lane sees in the score MFMA's output
-  // Hkv counts query-head groups: a KV head with more than 8 query heads is served by kv_div groups
-  // of G <= 8 heads each (consecutive groups read the same pages)
-  const int G = Hq / Hkv;
+  // Hkv counts query-head groups: a KV head with more than 8 query heads is served by kv_div groups of at most 8
+  // heads each (consecutive groups read the same pages); when the heads do not divide evenly the last group of
+  // a KV head has fewer (11 heads: 6 + 5).  G = heads of this workgroup's group, qbase = its first query head.
+  int G = Hq / Hkv;
   // skew16 > 0 (an even number of splits; the grid is (n_split / 2, Hkv, 2 n_seq)): the workgroups of the first half
   // of the grid take the even splits, those of the second half the odd ones, and every even split takes
   // skew16 sixteenths of a split's trips over from its odd neighbour.  Workgroups are dispatched in grid order, two
@@ -268,10 +269,15 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   // The groups of a KV head are (splits x KV heads) workgroups apart in the grid, not next to each other: workgroups
   // go to the card's eight dies in turn, each die has its own L2, and a distance that is a multiple of eight puts the
   // groups that read the same pages at the same time on the same die.
-  int h = blockIdx.y;
+  int h = blockIdx.y, qbase;
   if (kv_div > 1) {
-    const int kv_heads = Hkv / kv_div, grp = h / kv_heads;
-    h = (h - grp * kv_heads) * kv_div + grp;
+    const int kv_heads = Hkv / kv_div, grp = h / kv_heads, kvh = h - grp * kv_heads;
+    const int g_tot = Hq / kv_heads, g_max = (g_tot + kv_div - 1) / kv_div;
+    h = kvh * kv_div + grp;
+    qbase = kvh * g_tot + grp * g_max;
+    G = min(g_max, g_tot - grp * g_max);
+  } else {
+    qbase = h * G;
   }
   if (DS == 2 && skew16 > 0) {                                  // (only the launcher of DS == 2 kernels passes a skew)
     // (n_seq arrives with the other kernel arguments; the grid's size would be one more scalar load of the
@@ -333,7 +339,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   // 2^(E - 2 - 5t); the fp4 bit value 0.5 carries 2^1.
   {
     const int g = PP ? (n & 7) >> 1 : (NR ? n >> 2 : n >> 1);
-    const int64_t qrow = (int64_t)b * Hq + h * G + (g < G ? g : 0);
+    const int64_t qrow = (int64_t)b * Hq + qbase + (g < G ? g : 0);
     const int e1 = 127 + (int)q_stat[qrow * 4 + 0];
     const int e2 = 127 + (int)q_stat[qrow * 4 + 1];
     const int t01 = (n & 1) ? 7 : 2, t23 = t01 + 10;
@@ -349,7 +355,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   for (int j = 0; j < NJ; ++j) {
     const int g = PP ? 2 * (kb & 1) + j : (NR ? kb : 2 * kb + j);
     const bool live = g < G && hf == 0;
-    const int64_t qrow = (int64_t)b * Hq + h * G + (g < G ? g : 0);
+    const int64_t qrow = (int64_t)b * Hq + qbase + (g < G ? g : 0);
     const float c2 = q_stat[qrow * 4 + 2], c3 = q_stat[qrow * 4 + 3];
     cm[2 * j] = live ? c2 : 0.0f;
     cq[2 * j] = live ? c3 : 0.0f;
@@ -998,9 +1004,9 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
       walkers_sum(g, ch, mm, ll, aa);
       if (live && fm.n_extra == 0) {
         const float inv = ll > 0.0f ? 1.0f / ll : 0.0f;
-        store_from_f32(fm.out, ((int64_t)b * Hq + h * G + g) * D + ch, aa * inv, fm.out_dtype);
+        store_from_f32(fm.out, ((int64_t)b * Hq + qbase + g) * D + ch, aa * inv, fm.out_dtype);
       } else if (live) {
-        const float* x = parts + (((int64_t)b * Hq + h * G + g) * n_parts + 1) * (D + 2);     // the exact tail's part
+        const float* x = parts + (((int64_t)b * Hq + qbase + g) * n_parts + 1) * (D + 2);     // the exact tail's part
         const float m_x = x[0], l_x = x[1], a_x = x[2 + ch];
         float top = MF_NEG;
         if (ll > 0.0f) top = fmaxf(top, mm);
@@ -1008,7 +1014,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
         const float w0 = ll > 0.0f ? __expf(mm - top) : 0.0f, w1 = l_x > 0.0f ? __expf(m_x - top) : 0.0f;
         const float l_all = fmaf(w1, l_x, fmaf(w0, ll, 0.0f)), a_all = fmaf(w1, a_x, fmaf(w0, aa, 0.0f));
         const float inv = l_all > 0.0f ? 1.0f / l_all : 0.0f;
-        store_from_f32(fm.out, ((int64_t)b * Hq + h * G + g) * D + ch, a_all * inv, fm.out_dtype);
+        store_from_f32(fm.out, ((int64_t)b * Hq + qbase + g) * D + ch, a_all * inv, fm.out_dtype);
       }
     }
     return;
@@ -1057,7 +1063,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
     for (int ps = 0; ps < NPASS; ++ps) {
       const int g = ps * HPP + hsub;
       if (g < G) {
-        float* out = parts + (((int64_t)b * Hq + h * G + g) * n_parts + split) * (D + 2);
+        float* out = parts + (((int64_t)b * Hq + qbase + g) * n_parts + split) * (D + 2);
         store_coherent2(out + 2 + 2 * pr, res[ps]);
         if (pr == 0) store_coherent2(out, ml_out[ps]);
       }
@@ -1095,7 +1101,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
         const int o = tid + k * (MF_WAVES * 64);
         const bool live = o < G * D;
         const int g = live ? o / D : 0, ch = o % D;
-        const float* row = parts + ((int64_t)b * Hq + h * G + g) * n_parts * (D + 2);
+        const float* row = parts + ((int64_t)b * Hq + qbase + g) * n_parts * (D + 2);
         // all loads first (clamped to an existing part), then the log-sum-exp merge
         constexpr int NP = MERGE_IN_KERNEL_MAX_SPLITS + 1;
         const int n_merge = n_split + fm.n_extra;
@@ -1117,7 +1123,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
           aa = fmaf(wgt, a_s[sp], aa);
         }
         const float inv = ll > 0.0f ? 1.0f / ll : 0.0f;
-        if (live) store_from_f32(fm.out, ((int64_t)b * Hq + h * G + g) * D + ch, aa * inv, fm.out_dtype);
+        if (live) store_from_f32(fm.out, ((int64_t)b * Hq + qbase + g) * D + ch, aa * inv, fm.out_dtype);
       }
     }
   }
@@ -1130,7 +1136,8 @@ static int launch_one(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, 
                       float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts, int n_split,
                       int len_sub, int max_pages, int num_pages, const FusedMerge& fm, bool wide_wg,
                       hipStream_t st) {
-  const int G = Hq / Hkv;
+  // (heads of the largest group of a KV head; kv_div groups share a KV head's heads, the last one may have fewer)
+  const int G = kv_div > 1 ? (Hq / (Hkv / kv_div) + kv_div - 1) / kv_div : Hq / Hkv;
   size_t per_wave = (size_t)wave_lds_floats(D / DS / GS, DS) * sizeof(float);
   size_t merge = (size_t)(NW / DS * G * (D + 2) + NW * 16 * 16) * sizeof(float);
   if (SG) per_wave += stage_bytes((D / DS / 16) * VB / 2);

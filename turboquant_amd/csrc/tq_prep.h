@@ -81,8 +81,11 @@ __host__ __device__ inline int prep_groups_per_workgroup(int G, int64_t units, i
 
 // PACKED: gpw may exceed 1.  One group per workgroup is a build of its own (no row bounds, no head / group
 // arithmetic in the packing lanes): it is the one the latency-bound launches take, and half a microsecond shorter.
+// g_tot > 0 (one group per workgroup only): the groups tile runs of g_tot consecutive rows - the query heads of one
+// KV head - instead of the whole row range: group i of a run has rows i G .. min((i + 1) G, g_tot) - 1, so the last
+// group of every run is shorter when G does not divide g_tot (11 heads per KV head: groups of 6 and 5).
 template <int PER, int DT, bool PACKED>
-__device__ __forceinline__ void prep_query_body(const void* __restrict__ q, int G, int gpw, int64_t n_rows, const tq_layer& ly,
+__device__ __forceinline__ void prep_query_body(const void* __restrict__ q, int G, int gpw, int64_t n_rows, int g_tot, const tq_layer& ly,
                                                 float sm_scale, float* __restrict__ q_rot, float* __restrict__ q_sk,
                                                 float* __restrict__ q_stat, uint32_t* __restrict__ qa_pack,
                                                 unsigned long long* __restrict__ arrivals, int64_t unit, int word,
@@ -90,8 +93,16 @@ __device__ __forceinline__ void prep_query_body(const void* __restrict__ q, int 
   const int d = ly.d, tid = threadIdx.x, jl = tid % PREP_COLS, sl = tid / PREP_COLS;
   const int j = word * PREP_COLS + jl;
   const int RG = PACKED ? G * gpw : G;                                 // rows a workgroup has room for
-  const int64_t row0 = unit * RG, group0 = PACKED ? unit * gpw : unit;
-  const int R = PACKED ? (int)(n_rows - row0 < RG ? n_rows - row0 : RG) : G;      // rows of this workgroup (a multiple of G)
+  int64_t row0 = unit * RG;
+  const int64_t group0 = PACKED ? unit * gpw : unit;
+  int R = PACKED ? (int)(n_rows - row0 < RG ? n_rows - row0 : RG) : G;      // rows of this workgroup (PACKED: a multiple of G)
+  if (!PACKED && g_tot > 0) {
+    const int per = (g_tot + G - 1) / G;
+    const int64_t run = unit / per;
+    const int i = (int)(unit - run * per);
+    row0 = run * g_tot + (int64_t)i * G;
+    R = g_tot - i * G < G ? g_tot - i * G : G;
+  }
   if (arrivals != nullptr && word == 0 && tid < (PACKED ? gpw : 1) && tid * G < R) arrivals[group0 + tid] = 0ull;
   // every global load of the kernel is issued here, before anything waits, the query first: loads
   // return in order, so the query can go to shared memory (and its statistics be taken) while the

@@ -72,7 +72,7 @@ rotate_query_kernel(const void* __restrict__ q, int dtype, int64_t rows, int R, 
 
 template <int PER, int DT, bool PACKED>
 __global__ void __launch_bounds__(PREP_COLS * PREP_SLICES)
-prep_query_kernel(const void* __restrict__ q, int G, int gpw, int64_t n_rows, tq_layer ly, float sm_scale,
+prep_query_kernel(const void* __restrict__ q, int G, int gpw, int64_t n_rows, int g_tot, tq_layer ly, float sm_scale,
                   float* __restrict__ q_rot, float* __restrict__ q_sk, float* __restrict__ q_stat,
                   uint32_t* __restrict__ qa_pack, unsigned long long* __restrict__ arrivals, int n_units, int n_prep,
                   PagePrefetch pf) {
@@ -81,7 +81,7 @@ prep_query_kernel(const void* __restrict__ q, int G, int gpw, int64_t n_rows, tq
   // workgroups that read the page kernel's first pages ahead of it
   const int id = blockIdx.x;
   if (id < n_prep)
-    prep_query_body<PER, DT, PACKED>(q, G, gpw, n_rows, ly, sm_scale, q_rot, q_sk, q_stat, qa_pack, arrivals, id % n_units,
+    prep_query_body<PER, DT, PACKED>(q, G, gpw, n_rows, g_tot, ly, sm_scale, q_rot, q_sk, q_stat, qa_pack, arrivals, id % n_units,
                                      id / n_units, sm);
   else
     prefetch_pages_body(pf, id - n_prep);
@@ -365,18 +365,22 @@ int launch_dequant_mfma(const uint8_t* idx, const uint8_t* signs, const void* no
 // cores), not the fp32 rotated / sketched queries
 int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* layer, float* q_rot, float* q_sk,
                         float* q_stat, uint32_t* qa_pack, int G, float sm_scale, hipStream_t st, bool q_rot_unused,
-                        unsigned long long* arrivals, const PagePrefetch* prefetch) {
+                        unsigned long long* arrivals, const PagePrefetch* prefetch, int g_tot) {
   const int d = layer->d;
   if (qa_pack) {       // operands of the matrix-core decode kernel wanted
-    if (!q_stat || !layer->Pi_colsum || !layer->S_colsum || G > ROT_MAX_ROWS || rows % G || (d != 64 && d != 128 && d != 256))
+    // g_tot: query heads per KV head when its groups of G are unequal (0: the rows are whole groups of G)
+    if (g_tot > 0 && g_tot % G == 0) g_tot = 0;
+    if (!q_stat || !layer->Pi_colsum || !layer->S_colsum || G > ROT_MAX_ROWS || (g_tot > 0 ? rows % g_tot : rows % G) ||
+        (d != 64 && d != 128 && d != 256))
       return TQ_EUNSUPPORTED;
     // one group of heads per workgroup while the card holds all of them at once (three workgroups of 74 registers
     // per lane on each compute unit); beyond that, as many whole groups as fit a workgroup's eight rows
     // (64 x 2048 tokens at 32 q / 8 KV heads: 45.9 -> 42.2 us per step, 256 x 1024: 134 -> 121)
-    const int gpw = prep_groups_per_workgroup(G, (rows / G) * (d / PREP_COLS), 3 * (int64_t)device_compute_units());
+    const int gpw = g_tot > 0 ? 1 : prep_groups_per_workgroup(G, (rows / G) * (d / PREP_COLS), 3 * (int64_t)device_compute_units());
     const int64_t rows_per_wg = (int64_t)G * gpw;
     size_t smem = prep_smem_bytes(G * gpw, d);
-    const int n_units = (int)((rows + rows_per_wg - 1) / rows_per_wg), n_prep = n_units * (d / PREP_COLS);
+    const int n_units = g_tot > 0 ? (int)(rows / g_tot) * ((g_tot + G - 1) / G) : (int)((rows + rows_per_wg - 1) / rows_per_wg);
+    const int n_prep = n_units * (d / PREP_COLS);
     PagePrefetch pf;
     // (a preparation that already fills the card - hundreds of sequences - gains nothing from more workgroups:
     // 64 x 2048 tokens at 32 q / 8 KV heads measured 44.6 -> 46.3 us per step with them)
@@ -386,10 +390,10 @@ int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* 
 #define TQ_PREP(PER, DT)                                                                                               \
   {                                                                                                                    \
     if (gpw > 1)                                                                                                       \
-      prep_query_kernel<PER, DT, true><<<grid, block, smem, st>>>(q, G, gpw, rows, *layer, sm_scale, q_rot, q_sk, q_stat, \
+      prep_query_kernel<PER, DT, true><<<grid, block, smem, st>>>(q, G, gpw, rows, g_tot, *layer, sm_scale, q_rot, q_sk, q_stat, \
                                                                   qa_pack, arrivals, n_units, n_prep, pf);              \
     else                                                                                                               \
-      prep_query_kernel<PER, DT, false><<<grid, block, smem, st>>>(q, G, gpw, rows, *layer, sm_scale, q_rot, q_sk, q_stat, \
+      prep_query_kernel<PER, DT, false><<<grid, block, smem, st>>>(q, G, gpw, rows, g_tot, *layer, sm_scale, q_rot, q_sk, q_stat, \
                                                                    qa_pack, arrivals, n_units, n_prep, pf);             \
   }
 #define TQ_PREP_DT(PER)                              \
@@ -425,7 +429,7 @@ extern "C" int tq_rotate_query(const void* q, int dtype, int64_t rows, const tq_
   if (!q || !q_rot || !q_sk) return TQ_ENULL;
   if (rows < 0 || dtype < TQ_F32 || dtype > TQ_BF16) return TQ_EINVAL;
   if (rows == 0) return TQ_OK;
-  return launch_rotate_query(q, dtype, rows, layer, q_rot, q_sk, nullptr, nullptr, 1, 0.0f, (hipStream_t)stream, false, nullptr, nullptr);
+  return launch_rotate_query(q, dtype, rows, layer, q_rot, q_sk, nullptr, nullptr, 1, 0.0f, (hipStream_t)stream, false, nullptr, nullptr, 0);
 }
 
 extern "C" int tq_score(const void* q, int dtype, int64_t batch, int64_t n_q, const uint8_t* idx, const uint8_t* signs,
