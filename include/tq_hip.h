@@ -340,6 +340,10 @@ void tq_time_next_key_kernel(void *start_event, void *stop_event);
  *                      workgroups that read the pages every page-kernel workgroup asks for first (this many trips
  *                      of each of its block walkers, at most 96 KB per workgroup) into the caches ahead of it;
  *                      0: none.  Same result bit for bit.
+ *   "prep_mfma"        1 (default): bf16 queries at head_dim 128, and at head_dim 256 from 64 (row tile, plane word)
+ *                      workgroups on, are rotated, sketched and packed on the matrix cores (three-term bf16 products
+ *                      with Pi_split / S_split: fp32-accurate, summed in another order than the vector-ALU kernel,
+ *                      so outputs agree to rounding, not bit for bit); 2: wherever the kernel applies; 0: never.
  *   "merge_in_kernel"  1 (default): a compressed-only decode step on the matrix-core kernel with at most 8 context
  *                      splits has its splits merged by the last workgroup of the page kernel (two launches per
  *                      step); 0: always the separate merge kernel.

@@ -834,3 +834,52 @@ def test_decode_over_a_store_with_outlier_channels(gpu, d, Hq, Hkv, vb, key_bits
         _progress(f"   {kind}: cosine {c:.8f} (1 - cos = {1 - c:.2e}), worst head {min(per_head):.8f}")
         assert c >= COS_GATE, (kind, c)
         assert min(per_head) >= 0.9995, (kind, min(per_head))
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,d,key_bits,vb", [(5, 8, 2, 128, 3, 4), (3, 21, 3, 128, 3, 2), (7, 10, 2, 128, 4, 4),
+                                                      (2, 6, 1, 256, 3, 2), (9, 12, 4, 128, 2, 4), (33, 16, 2, 256, 3, 2),
+                                                      (4, 1, 1, 128, 3, 4), (3, 16, 1, 128, 3, 8)])
+def test_query_preparation_on_the_matrix_cores(gpu, B, Hq, Hkv, d, key_bits, vb):
+    """bf16 queries are rotated (q Pi^T), sketched (q S^T; triton_kernels.py:527-528) and packed into the page
+    kernel's fp6 operands by a matrix-core kernel: three-term bf16 products that are fp32-accurate but summed in
+    another order than the vector-ALU preparation.  On the same store the two preparations must agree to the
+    rounding of the bf16 output (group sizes 1 to 8, a last row tile that is partly empty, 16 heads per KV head as
+    two groups), both with the page kernels that read all eight operand rows of a group on a workspace poisoned
+    with NaN patterns, and each must meet the oracle (score.py:138-173)."""
+    g = torch.Generator().manual_seed(B + 7 * Hq + d)
+    lens = [int(x) for x in torch.randint(40, 400, (B,), generator=g)]
+    pages = (max(lens) + 15) // 16
+    pool, tq = _make_pool(gpu, d, key_bits, vb, Hkv, B * pages + 1, torch.bfloat16, seed=42)
+    table = torch.randperm(B * pages + 1, generator=g)[: B * pages].to(torch.int32).view(B, pages).to(gpu)
+    k = torch.randn(B, max(lens), Hkv, d, generator=g).bfloat16().to(gpu)
+    v = torch.randn(B, max(lens), Hkv, d, generator=g).bfloat16().to(gpu)
+    pool.append(k, v, table)
+    seq = torch.tensor(lens, dtype=torch.int32, device=gpu)
+    q = torch.randn(B, Hq, d, generator=g).bfloat16()
+    _progress(f"matrix-core preparation B={B} Hq={Hq} Hkv={Hkv} d={d} kb={key_bits} vb={vb}")
+    outs = {}
+    try:
+        for narrow in (1, 0):
+            _set_option("narrow_rows", narrow)
+            _set_option("page_pairs", narrow)
+            for mode in (2, 0):
+                _set_option("prep_mfma", mode)
+                ws = pool.workspace(B, Hq, 3)
+                ws.view(torch.int32).fill_(0x7fc00000)
+                outs[(narrow, mode)] = pool.decode_attention(q.to(gpu), table, seq, n_split=3, workspace=ws).float().cpu()
+        torch.cuda.synchronize()
+    finally:
+        _set_option("prep_mfma", 1)
+        _set_option("narrow_rows", 1)
+        _set_option("page_pairs", 1)
+    for narrow in (1, 0):
+        a, b = outs[(narrow, 2)], outs[(narrow, 0)]
+        assert not torch.isnan(a).any() and not torch.isnan(b).any()
+        assert (a - b).abs().max() <= 2 ** -7 * b.abs().max() + 1e-6, narrow
+    assert torch.equal(outs[(1, 2)], outs[(0, 2)]) or (outs[(1, 2)] - outs[(0, 2)]).abs().max() <= 2 ** -7 * outs[(0, 2)].abs().max()
+    prm = params_of(tq)
+    for b in (0, B - 1):
+        kc, vc = _store_from_oracle_view(pool, table[b], lens[b])
+        want = O.hybrid_attention(q[b:b + 1], kc, vc, lens[b], prm, Hkv, None, None)
+        assert cosine(outs[(1, 2)][b:b + 1], want) >= COS_GATE, b
+        assert cosine(outs[(1, 0)][b:b + 1], want) >= COS_GATE, b

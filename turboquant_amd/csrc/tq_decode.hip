@@ -823,7 +823,7 @@ prep_tail_kernel(TailArgs A, int n_tail, int B, int Gq, tq_layer ly, float* __re
     const int per_z = A.Hkv * B;
     exact_tail_words_body<DT, 1, PAGED, true>(A, id % A.Hkv, (id / A.Hkv) % B, id / per_z, sm);
   } else if (id >= n_front) {      // behind the tail and the preparation: the page kernel's first pages, read ahead of it
-    prefetch_pages_body(pf, id - n_front);
+    prefetch_pages_body<TAIL_THREADS>(pf, id - n_front);
   } else {
     const int words = ly.d / PREP_COLS, p = id - n_tail;
     // (arrivals: the arrival counters of the groups of query heads, zeroed for a page kernel that merges its splits itself)
@@ -960,6 +960,7 @@ std::atomic<int> opt_split_skew{1};
 std::atomic<int> opt_merge_row_groups{1};
 std::atomic<int> opt_tail_chunks{1};
 std::atomic<int> opt_prefetch_trips{1};
+std::atomic<int> opt_prep_mfma{1};
 }  // namespace tq
 
 extern "C" int tq_set_option(const char* name, int64_t value) {
@@ -973,6 +974,11 @@ extern "C" int tq_set_option(const char* name, int64_t value) {
   if (!std::strcmp(name, "prefetch_trips")) {
     if (value < 0 || value > 64) return TQ_EINVAL;
     opt_prefetch_trips.store((int)value);
+    return TQ_OK;
+  }
+  if (!std::strcmp(name, "prep_mfma")) {
+    if (value < 0 || value > 2) return TQ_EINVAL;
+    opt_prep_mfma.store((int)value);
     return TQ_OK;
   }
   if (!std::strcmp(name, "tail_chunks")) { opt_tail_chunks.store(value != 0); return TQ_OK; }

@@ -328,6 +328,7 @@ __device__ __forceinline__ unsigned long long load_coherent(const unsigned long 
 // page-kernel workgroup will ask for first.  Workgroups go to the card's dies in turn, so the page-kernel
 // workgroup picked is the one whose position in its grid is congruent to this workgroup's position in this
 // grid: when the counts are multiples of eight the reader and the prefetcher share a die and its L2.
+template <int THREADS>
 __device__ __forceinline__ void prefetch_pages_body(const PagePrefetch& P, int p) {
   int lin = p + P.front;
   lin -= lin >= P.n_wg ? (lin / P.n_wg) * P.n_wg : 0;
@@ -356,7 +357,7 @@ __device__ __forceinline__ void prefetch_pages_body(const PagePrefetch& P, int p
   // 16 bytes per lane; piece i of the range = piece i % pieces of page i / pieces.  Every table load is issued
   // before the first page load and every page load before anything waits: the workgroup costs two memory
   // latencies, whatever its share.  Slots beyond the range re-read the head's page 0 (in the pool, cached).
-  constexpr int SLOTS = 12;                            // per lane: 512 lanes x 12 x 16 bytes = 96 KB per workgroup
+  constexpr int SLOTS = 6144 / THREADS;                // 16-byte pieces per lane: 96 KB per workgroup
   const int tid = threadIdx.x, pieces = (int)(P.fetch_bytes >> 4), total = (pg1 > pg0 ? pg1 - pg0 : 0) * pieces;
   if (total <= 0) return;
   const float inv_pieces = 1.0f / (float)pieces;
@@ -364,7 +365,7 @@ __device__ __forceinline__ void prefetch_pages_body(const PagePrefetch& P, int p
   uint32_t pid[SLOTS], off[SLOTS];
 #pragma unroll
   for (int k = 0; k < SLOTS; ++k) {
-    const int i = tid + 512 * k;
+    const int i = tid + THREADS * k;
     const int pg = (int)(((float)i + 0.5f) * inv_pieces);       // exact for the few thousand pieces of a range
     const bool live = i < total;
     off[k] = live ? (uint32_t)(i - pg * pieces) * 16u : 0u;
@@ -379,6 +380,179 @@ __device__ __forceinline__ void prefetch_pages_body(const PagePrefetch& P, int p
 #pragma unroll
   for (int k = 0; k < SLOTS; ++k) keep ^= got[k];
   asm volatile("" :: "v"(keep));                      // the loads are wanted for their side effect
+}
+
+// ------------------------------------------------------------------------------------------------------
+// The same preparation on the matrix cores, for bf16 queries at head_dim 128 / 256: q Pi^T and q S^T are
+// (rows x d) x (d x d) products, a bf16 query is an exact single term, and Pi and S already exist as three
+// bf16 terms each in MFMA operand order (tq_layer::Pi_split / S_split, built for the key quantiser), so
+// v_mfma_f32_16x16x32_bf16 gives the fp32-accurate products with the matrix as the row operand and sixteen
+// query rows as the column operand.  A workgroup of four wavefronts owns a tile of up to 16 rows - as many whole
+// groups of G heads as fit - and one plane word (32 coordinates); each wavefront owns one of the word's two
+// 16-coordinate halves of one of the two products: d / 32 x 3 MFMAs whose matrix operands are all requested before
+// the first is used (one memory latency).  The 16 x 32 results meet in LDS and one lane per (term plane, row) packs
+// the four fp6 terms exactly as prep_query_body does.  Nothing is read from another workgroup.
+typedef uint32_t prep_u32x4 __attribute__((ext_vector_type(4)));
+typedef float prep_f32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 prep_bf16x8 __attribute__((ext_vector_type(8)));
+constexpr int PREP_MFMA_THREADS = 256, PREP_MFMA_LD = 36;          // LDS row stride of a wavefront's 16 x 32 tile
+__host__ __device__ inline int prep_mfma_smem_floats() { return 2 * 16 * PREP_MFMA_LD + 32; }
+
+template <int D>
+__device__ __forceinline__ void prep_mfma_body(const uint16_t* __restrict__ q, int G, int64_t n_rows, const tq_layer& ly,
+                                               float sm_scale, float* __restrict__ q_stat, uint32_t* __restrict__ qa_pack,
+                                               unsigned long long* __restrict__ arrivals, int64_t tile, int word,
+                                               float* sm) {
+  constexpr int KS = D / 32;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n = lane & 15, kb = lane >> 4;
+  const int gpt = 16 / G, rows_tile = gpt * G;                     // whole groups per tile
+  const int64_t row0 = tile * rows_tile, group0 = tile * gpt;
+  const int R = (int)(n_rows - row0 < rows_tile ? n_rows - row0 : rows_tile);
+  const int chunk = word >> 2, kw = word & 3;                       // the word's place in the operand layout
+  const int jt = wave & 1, m = wave >> 1;                           // this wavefront's half of the word, and its product
+  if (arrivals != nullptr && word == 0 && tid < gpt && tid * G < R) arrivals[group0 + tid] = 0ull;
+  float* s_rot = sm;                                                // [16 rows][32 coordinates], stride PREP_MFMA_LD
+  float* s_sk = s_rot + 16 * PREP_MFMA_LD;
+  float* stat = s_sk + 16 * PREP_MFMA_LD;                           // [16 rows][2]: multipliers of coef q_rot_j and q_sk_j
+  // column operands: lane (row n, block kb) holds q[n][32 ks + 8 kb .. + 7]; rows beyond the tile are zero
+  prep_u32x4 qb[KS];
+  {
+    const uint16_t* qrow = q + (row0 + (n < R ? n : R - 1)) * D + kb * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qb[ks] = *(const prep_u32x4*)(qrow + ks * 32);
+    if (n >= R) {
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) qb[ks] = prep_u32x4{0u, 0u, 0u, 0u};
+    }
+  }
+  // row operands: the three bf16 terms of this wavefront's 16 matrix rows, all requested before anything waits
+  prep_u32x4 ma[3][KS];
+  {
+    const uint16_t* mat = m ? ly.S_split : ly.Pi_split;
+#pragma unroll
+    for (int t = 0; t < 3; ++t) {
+      const uint16_t* base = mat + (((int64_t)(t * (D / 16) + word * 2 + jt) * KS) * 64 + lane) * 8;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) ma[t][ks] = *(const prep_u32x4*)(base + ks * (64 * 8));
+    }
+  }
+  // row statistics from the same registers: the four lanes of a row each hold a quarter of its coordinates
+  {
+    float ss = 0.0f, s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const prep_f32x4* c1 = (const prep_f32x4*)(ly.Pi_colsum + ks * 32 + kb * 8);
+      const prep_f32x4* c2 = (const prep_f32x4*)(ly.S_colsum + ks * 32 + kb * 8);
+      const prep_f32x4 a0 = c1[0], a1 = c1[1], b0 = c2[0], b1 = c2[1];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float xl = __uint_as_float(qb[ks][e] << 16), xh = __uint_as_float(qb[ks][e] & 0xffff0000u);
+        const float cl1 = e < 2 ? a0[2 * e] : a1[2 * e - 4], ch1 = e < 2 ? a0[2 * e + 1] : a1[2 * e - 3];
+        const float cl2 = e < 2 ? b0[2 * e] : b1[2 * e - 4], ch2 = e < 2 ? b0[2 * e + 1] : b1[2 * e - 3];
+        ss = fmaf(xl, xl, fmaf(xh, xh, ss));
+        s1 = fmaf(xl, cl1, fmaf(xh, ch1, s1));
+        s2 = fmaf(xl, cl2, fmaf(xh, ch2, s2));
+      }
+    }
+    ss += __shfl_xor(ss, 16, 64); s1 += __shfl_xor(s1, 16, 64); s2 += __shfl_xor(s2, 16, 64);
+    ss += __shfl_xor(ss, 32, 64); s1 += __shfl_xor(s1, 32, 64); s2 += __shfl_xor(s2, 32, 64);
+    float cmax = 0.0f;
+    for (int t = 0; t < ly.n_terms; ++t) cmax = fmaxf(cmax, fabsf(ly.term_coef[t]));
+    const float nq = sqrtf(ss), k = sm_scale * 1.4426950408889634f;
+    const int e1 = min(max((int)((__float_as_uint(fabsf(k) * nq * cmax) >> 23) & 255u) - 126, -100), 100);
+    const int e2 = min(max((int)((__float_as_uint(2.0f * fabsf(k * ly.qjl_scale) * nq * ly.S_rownorm_max) >> 23) & 255u) - 126, -100), 100);
+    if (kb == 0 && wave == 0) {
+      stat[n * 2 + 0] = k * __uint_as_float((uint32_t)(127 - e1) << 23);
+      stat[n * 2 + 1] = 2.0f * k * ly.qjl_scale * __uint_as_float((uint32_t)(127 - e2) << 23);
+      if (word == 0 && n < R) {
+        float* st = q_stat + (row0 + n) * 4;
+        st[0] = (float)e1; st[1] = (float)e2;
+        st[2] = k * ly.term_const * s1; st[3] = -k * ly.qjl_scale * s2;
+      }
+    }
+  }
+  prep_f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+  for (int t = 2; t >= 0; --t)                                       // the small terms first
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(prep_bf16x8, ma[t][ks]),
+                                                    __builtin_bit_cast(prep_bf16x8, qb[ks]), acc, 0, 0, 0);
+  // result register i of lane (row n, quarter kb) is coordinate 16 jt + 4 kb + i of query row n
+  *(prep_f32x4*)((m ? s_sk : s_rot) + n * PREP_MFMA_LD + jt * 16 + 4 * kb) = acc;
+  __syncthreads();
+  // operands of this plane word: one lane per (term plane, row), as in prep_query_body
+  const int mb = ly.mse_bits;
+  int nx = 0;
+  for (int t = 0; t < ly.n_terms; ++t)
+    if (__builtin_popcount(ly.term_mask[t]) > 1) ++nx;
+  const int ntp = mb + nx + 1;
+  constexpr int wpl = D / 128;
+  for (int idx = tid; idx < ntp * 16; idx += PREP_MFMA_THREADS) {
+    const int tp = idx >> 4, r = idx & 15;
+    if (r >= R) continue;
+    typedef float f32x16_t __attribute__((ext_vector_type(16)));
+    typedef float f32x32_t __attribute__((ext_vector_type(32)));
+    typedef uint32_t u32x6_t __attribute__((ext_vector_type(6)));
+    const bool is_sign = tp == ntp - 1;
+    float coef = 1.0f;
+    if (tp < mb) {
+      coef = 0.0f;
+      for (int t = 0; t < ly.n_terms; ++t)
+        if (ly.term_mask[t] == (1 << (mb - 1 - tp))) coef = ly.term_coef[t];
+    } else if (!is_sign) {
+      coef = 0.0f;
+      int seen = 0;
+      for (int t = 0; t < ly.n_terms; ++t) {
+        if (__builtin_popcount(ly.term_mask[t]) > 1) {
+          if (seen == tp - mb) coef = ly.term_coef[t];
+          ++seen;
+        }
+      }
+    }
+    const int gi = r / G, hg = r - gi * G;
+    const float base = 4.0f * (is_sign ? stat[r * 2 + 1] : coef * stat[r * 2 + 0]);
+    const prep_f32x4* src = (const prep_f32x4*)((is_sign ? s_sk : s_rot) + r * PREP_MFMA_LD);
+    float x[32];
+#pragma unroll
+    for (int k4 = 0; k4 < 8; ++k4) {
+      const prep_f32x4 v4 = src[k4];
+      x[4 * k4] = v4[0]; x[4 * k4 + 1] = v4[1]; x[4 * k4 + 2] = v4[2]; x[4 * k4 + 3] = v4[3];
+    }
+    f32x16_t va, vb;
+#pragma unroll
+    for (int kloc = 0; kloc < 32; ++kloc) {
+      const int c = 4 * (kloc & 7) + (kloc >> 3), t4 = kloc >> 3;
+      const float v = x[c] * (base * (t4 == 1 ? 0.5f : (t4 == 2 ? 0.25f : 1.0f)));
+      if (kloc & 1) vb[kloc >> 1] = v;
+      else va[kloc >> 1] = v;
+    }
+    uint32_t* dst = qa_pack + (group0 + gi) * (int64_t)(ntp * wpl * 2 * 64 * 8);
+    const float one = 1.0f;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      u32x6_t code;
+      asm volatile("v_cvt_scalef32_2xpk16_fp6_f32 %0, %1, %2, %3" : "=&v"(code) : "v"(va), "v"(vb), "v"(one));
+      uint32_t* o = dst + (((tp * wpl + chunk) * 2 + (t >> 1)) * 64 + 2 * hg + (t & 1) + 16 * kw) * 8;
+      *(uint4*)o = make_uint4(code[0], code[1], code[2], code[3]);
+      *(uint2*)(o + 4) = make_uint2(code[4], code[5]);
+      for (int ha = hg + G; ha < 8; ha += G) {                       // operand rows of heads the group does not have
+        uint32_t* z = o + (2 * (ha - hg)) * 8;
+        *(uint4*)z = make_uint4(0u, 0u, 0u, 0u);
+        *(uint2*)(z + 4) = make_uint2(0u, 0u);
+      }
+      if (t < 3) {
+        f32x32_t rr;
+        asm volatile("v_cvt_scalef32_pk32_f32_fp6 %0, %1, %2" : "=&v"(rr) : "v"(code), "v"(one));
+#pragma unroll
+        for (int k = 0; k < 16; ++k) {
+          va[k] = (va[k] - rr[2 * k]) * 32.0f;
+          vb[k] = (vb[k] - rr[2 * k + 1]) * 32.0f;
+        }
+      }
+    }
+  }
 }
 
 // LDS bytes of a preparation workgroup

@@ -84,7 +84,20 @@ prep_query_kernel(const void* __restrict__ q, int G, int gpw, int64_t n_rows, in
     prep_query_body<PER, DT, PACKED>(q, G, gpw, n_rows, g_tot, ly, sm_scale, q_rot, q_sk, q_stat, qa_pack, arrivals, id % n_units,
                                      id / n_units, sm);
   else
-    prefetch_pages_body(pf, id - n_prep);
+    prefetch_pages_body<PREP_COLS * PREP_SLICES>(pf, id - n_prep);
+}
+
+// The preparation on the matrix cores (bf16 queries, head_dim 128 / 256): a workgroup per (tile of up to 16 query
+// rows, plane word), then the page-prefetch workgroups.
+template <int D>
+__global__ void __launch_bounds__(PREP_MFMA_THREADS)
+prep_mfma_kernel(const uint16_t* __restrict__ q, int G, int64_t n_rows, tq_layer ly, float sm_scale,
+                 float* __restrict__ q_stat, uint32_t* __restrict__ qa_pack, unsigned long long* __restrict__ arrivals,
+                 int n_tiles, int n_prep, PagePrefetch pf) {
+  extern __shared__ __align__(16) float sm[];
+  const int id = blockIdx.x;
+  if (id < n_prep) prep_mfma_body<D>(q, G, n_rows, ly, sm_scale, q_stat, qa_pack, arrivals, id % n_tiles, id / n_tiles, sm);
+  else prefetch_pages_body<PREP_MFMA_THREADS>(pf, id - n_prep);
 }
 
 // scores[b, i, k] for a tile of QT queries and one key per thread.  The rotated and sketched queries sit
@@ -373,6 +386,29 @@ int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* 
     if (!q_stat || !layer->Pi_colsum || !layer->S_colsum || G > ROT_MAX_ROWS || (g_tot > 0 ? rows % g_tot : rows % G) ||
         (d != 64 && d != 128 && d != 256))
       return TQ_EUNSUPPORTED;
+    // bf16 queries at head_dim 128 / 256 with the split matrices at hand: the products run on the matrix cores
+    // (head_dim 256 with few rows keeps the vector-ALU kernel: 64 rows - 32 workgroups here, each pulling 96 KB of
+    // matrix terms - measured 1 us slower per step; from 64 workgroups on the two are level or this one ahead:
+    // 16 x 8192 at 32 q heads 35.0 -> 34.5 us per step, 64 x 2048 40.2 -> 36.4, 256 x 1024 107.6 -> 86.2)
+    const int rows_tile = (16 / G) * G;
+    const int n_tiles = (int)((rows + rows_tile - 1) / rows_tile), n_prep = n_tiles * (d / 32);
+    const int mfma_opt = opt_prep_mfma.load(std::memory_order_relaxed);
+    if (dtype == TQ_BF16 && (d == 128 || d == 256) && layer->Pi_split && layer->S_split && g_tot == 0 && q_rot_unused &&
+        (((uintptr_t)q) & 15) == 0 && mfma_opt != 0 && (d == 128 || n_prep >= 64 || mfma_opt > 1)) {
+      PagePrefetch pf;
+      if (prefetch && prefetch->blocks > 0 && prefetch->n_wg > 0 && n_prep <= 2 * device_compute_units()) pf = *prefetch;
+      pf.front = n_prep;
+      const dim3 grid((unsigned)(n_prep + (pf.blocks > 0 ? pf.n_wg : 0))), block(PREP_MFMA_THREADS);
+      const size_t smem = (size_t)prep_mfma_smem_floats() * sizeof(float);
+      if (d == 128)
+        prep_mfma_kernel<128><<<grid, block, smem, st>>>((const uint16_t*)q, G, rows, *layer, sm_scale, q_stat, qa_pack,
+                                                         arrivals, n_tiles, n_prep, pf);
+      else
+        prep_mfma_kernel<256><<<grid, block, smem, st>>>((const uint16_t*)q, G, rows, *layer, sm_scale, q_stat, qa_pack,
+                                                         arrivals, n_tiles, n_prep, pf);
+      hipError_t e = hipGetLastError();
+      return e == hipSuccess ? TQ_OK : (int)e;
+    }
     // one group of heads per workgroup while the card holds all of them at once (three workgroups of 74 registers
     // per lane on each compute unit); beyond that, as many whole groups as fit a workgroup's eight rows
     // (64 x 2048 tokens at 32 q / 8 KV heads: 45.9 -> 42.2 us per step, 256 x 1024: 134 -> 121)
