@@ -519,6 +519,54 @@ def shape_table(device, steps, warmup):
     return rows
 
 
+def phase_stamps(device, reps=40):
+    """Mean time (microseconds after the first wavefront's start) at which the wavefronts of the page kernel reach
+    its phase boundaries, with and without the page prefetch of the preparation launch.  Needs a library built
+    with -DTQ_STAMPS: lane 0 of every wavefront then stores the 100 MHz real-time counter at each boundary."""
+    import ctypes
+    import numpy as np
+    import torch
+    from turboquant_amd import _ffi
+    lib = _ffi.lib()
+    if not hasattr(lib, "tq_debug_stamps"):
+        raise SystemExit("this libtq_hip.so has no stamps: build it with TQ_EXTRA_HIPCC_FLAGS=-DTQ_STAMPS")
+    names = ["start", "operands loaded", "first block requested, table scanned", "loop done", "epilogue barrier",
+             "walkers in LDS", "partial stores issued", "partial stores acknowledged"]
+    order = [0, 1, 2, 3, 6, 7, 4, 5]
+    out = []
+    for label, shape, fn_name, n_wg, nw in (("4 x 131072, head_dim 256", (4, 131072, 16, 2, 256, 3, 2), "tq_debug_stamps", 512, 4),
+                                            ("16 x 8192, head_dim 128", (16, 8192, 32, 8, 128, 3, 4), "tq_debug_stamps_d128", 256, 8)):
+        B, N, Hq, Hkv, d, kb, vb = shape
+        w = DecodeWorkload(label, B, N, Hq, Hkv, d, kb, vb, n_pools=4, seed=3, dist="normal", device=device, device_data=True)
+        fn = getattr(lib, fn_name)
+        fn.argtypes = [ctypes.c_void_p, ctypes.c_int]
+        for trips in (1, 0):
+            _ffi.check(lib.tq_set_option(b"prefetch_trips", trips), "tq_set_option")
+            for i in range(600):
+                w.step(i)
+            torch.cuda.synchronize()
+            acc = []
+            for r in range(reps):
+                w.step(r)
+                torch.cuda.synchronize()
+                buf = (ctypes.c_ulonglong * (n_wg * 64))()
+                if fn(buf, n_wg * 64) != 0:
+                    raise SystemExit("reading the stamps failed")
+                a = np.frombuffer(buf, dtype=np.uint64).reshape(n_wg, 8, 8).astype(np.int64)[:, :nw, :]
+                acc.append((a - a[:, :, 0].min()) / 100.0)
+            a = np.mean(acc, axis=0)
+            out.append({"workload": label, "prefetch_trips": trips,
+                        "reached_us": {names[i]: round(float(a[:, :, k].mean()), 2) for i, k in enumerate(order)},
+                        "last_wavefront_done_us": round(float(a[:, :, 5].max()), 2),
+                        "loop_done_first_half_of_grid_us": round(float(a[: n_wg // 2, :, 3].mean()), 2),
+                        "loop_done_second_half_of_grid_us": round(float(a[n_wg // 2:, :, 3].mean()), 2)})
+            print(json.dumps(out[-1]), file=sys.stderr, flush=True)
+        _ffi.check(lib.tq_set_option(b"prefetch_trips", 1), "tq_set_option")
+        del w
+        torch.cuda.empty_cache()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -536,6 +584,10 @@ def main():
     ap.add_argument("--shapes", action="store_true",
                     help="time the decode step over SHAPE_TABLE instead (one JSON line with a row per shape; rows also "
                          "go to stderr as they finish)")
+    ap.add_argument("--phase-stamps", action="store_true",
+                    help="per-phase times inside the page kernel of the long-context and the 16 x 8192 workloads, from "
+                         "the real-time counter stamps of a library built with TQ_EXTRA_HIPCC_FLAGS=-DTQ_STAMPS "
+                         "(a profiling build; the shipped one has no stamps and this mode then exits)")
     ap.add_argument("--quantize-only", action="store_true",
                     help="run the prefill-quantize leg alone and print its object (for profiles of its kernels)")
     args = ap.parse_args()
@@ -556,6 +608,10 @@ def main():
     if args.shapes:
         print(json.dumps({"metric": "decode step over a table of shapes, 1 GPU", "steps": args.steps, "warmup": args.warmup,
                           "shapes": shape_table(device, args.steps, args.warmup)}))
+        return
+
+    if args.phase_stamps:
+        print(json.dumps({"metric": "page kernel phases, 1 GPU", "phases": phase_stamps(device)}))
         return
 
     if args.quantize_only:

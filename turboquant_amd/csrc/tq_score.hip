@@ -391,21 +391,21 @@ int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* 
     // matrix terms - measured 1 us slower per step; from 64 workgroups on the two are level or this one ahead:
     // 16 x 8192 at 32 q heads 35.0 -> 34.5 us per step, 64 x 2048 40.2 -> 36.4, 256 x 1024 107.6 -> 86.2)
     const int rows_tile = (16 / G) * G;
-    const int n_tiles = (int)((rows + rows_tile - 1) / rows_tile), n_prep = n_tiles * (d / 32);
+    const int n_tiles = (int)((rows + rows_tile - 1) / rows_tile), n_mprep = n_tiles * (d / 32);
     const int mfma_opt = opt_prep_mfma.load(std::memory_order_relaxed);
     if (dtype == TQ_BF16 && (d == 128 || d == 256) && layer->Pi_split && layer->S_split && g_tot == 0 && q_rot_unused &&
-        (((uintptr_t)q) & 15) == 0 && mfma_opt != 0 && (d == 128 || n_prep >= 64 || mfma_opt > 1)) {
+        (((uintptr_t)q) & 15) == 0 && mfma_opt != 0 && (d == 128 || n_mprep >= 64 || mfma_opt > 1)) {
       PagePrefetch pf;
-      if (prefetch && prefetch->blocks > 0 && prefetch->n_wg > 0 && n_prep <= 2 * device_compute_units()) pf = *prefetch;
-      pf.front = n_prep;
-      const dim3 grid((unsigned)(n_prep + (pf.blocks > 0 ? pf.n_wg : 0))), block(PREP_MFMA_THREADS);
+      if (prefetch && prefetch->blocks > 0 && prefetch->n_wg > 0 && n_mprep <= 2 * device_compute_units()) pf = *prefetch;
+      pf.front = n_mprep;
+      const dim3 grid((unsigned)(n_mprep + (pf.blocks > 0 ? pf.n_wg : 0))), block(PREP_MFMA_THREADS);
       const size_t smem = (size_t)prep_mfma_smem_floats() * sizeof(float);
       if (d == 128)
         prep_mfma_kernel<128><<<grid, block, smem, st>>>((const uint16_t*)q, G, rows, *layer, sm_scale, q_stat, qa_pack,
-                                                         arrivals, n_tiles, n_prep, pf);
+                                                         arrivals, n_tiles, n_mprep, pf);
       else
         prep_mfma_kernel<256><<<grid, block, smem, st>>>((const uint16_t*)q, G, rows, *layer, sm_scale, q_stat, qa_pack,
-                                                         arrivals, n_tiles, n_prep, pf);
+                                                         arrivals, n_tiles, n_mprep, pf);
       hipError_t e = hipGetLastError();
       return e == hipSuccess ? TQ_OK : (int)e;
     }
