@@ -336,10 +336,11 @@ void tq_time_next_page_kernel(void *start_event, void *stop_event);
 void tq_time_next_key_kernel(void *start_event, void *stop_event);
 
 /* Tuning and test knobs (no counterpart in the reference); process-wide, take effect at the next call.
- *   "prefetch_trips"   0..64, default 1: the preparation launch of a step on the matrix-core path carries extra
- *                      workgroups that read the pages every page-kernel workgroup asks for first (this many trips
- *                      of each of its block walkers, at most 96 KB per workgroup) into the caches ahead of it;
- *                      0: none.  Same result bit for bit.
+ *   "prefetch_trips"   -1..64: the preparation launch of a step on the matrix-core path carries extra workgroups
+ *                      that read the pages every page-kernel workgroup asks for first (this many trips of each of
+ *                      its block walkers, at most 96 KB per workgroup) into the caches ahead of it; 0: none;
+ *                      -1 (default): one trip at head_dim 256, none at the other head sizes (where the read-ahead
+ *                      moves as much time into the preparation launch as it saves).  Same result bit for bit.
  *   "prep_mfma"        1 (default): bf16 queries at head_dim 128, and at head_dim 256 from 64 (row tile, plane word)
  *                      workgroups on, are rotated, sketched and packed on the matrix cores (three-term bf16 products
  *                      with Pi_split / S_split: fp32-accurate, summed in another order than the vector-ALU kernel,

@@ -464,7 +464,13 @@ def _variant_against_default(gpu, option, d, key_bits, vb, Hq, Hkv, dtype, exact
                 outs = []
                 for on in (1, 0):
                     _set_option(option, on)
-                    outs.append(pool.decode_attention(q.to(gpu), tab.to(gpu), seq, n_split=n_split, max_len=max(lens)).cpu())
+                    # every byte of the workspace poisoned first: the preparation only writes the operand rows its page
+                    # kernel reads (those of heads 0..3 for the variants of at most four heads), and nothing may
+                    # depend on what the other rows, or an earlier call, left behind
+                    ws = pool.workspace(B, Hq, n_split)
+                    ws.view(torch.uint8).fill_(0xFF)
+                    outs.append(pool.decode_attention(q.to(gpu), tab.to(gpu), seq, n_split=n_split, max_len=max(lens),
+                                                      workspace=ws).cpu())
                 torch.cuda.synchronize()
                 if exact:
                     assert torch.equal(outs[0], outs[1]), (n_split, tab is bad)

@@ -45,7 +45,7 @@ def build_library(verbose: bool = False) -> str:
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     objdir = os.path.join(HERE, "build")
     os.makedirs(objdir, exist_ok=True)
-    # TQ_EXTRA_HIPCC_FLAGS: extra compile flags, e.g. -DTQ_FUSED_PREP for the in-launch query preparation
+    # TQ_EXTRA_HIPCC_FLAGS: extra compile flags, e.g. -DTQ_STAMPS for the page kernel's phase time stamps
     compile_flags = [f for f in FLAGS if f != "-shared"] + os.environ.get("TQ_EXTRA_HIPCC_FLAGS", "").split()
     jobs = []
     for src in SOURCES:

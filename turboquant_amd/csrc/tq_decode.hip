@@ -816,7 +816,7 @@ template <int PER, int DT, bool PAGED, bool PACKED>
 __global__ void __launch_bounds__(TAIL_THREADS, 4)
 prep_tail_kernel(TailArgs A, int n_tail, int B, int Gq, tq_layer ly, float* __restrict__ q_rot, float* __restrict__ q_sk,
                  float* __restrict__ q_stat, uint32_t* __restrict__ qa_pack, unsigned long long* __restrict__ arrivals,
-                 int prep_gpw, int n_front, PagePrefetch pf, int g_tot) {
+                 int prep_gpw, int n_front, PagePrefetch pf, int g_tot, int head_rows) {
   extern __shared__ __align__(16) float sm[];
   const int id = blockIdx.x;
   if (id < n_tail) {
@@ -828,7 +828,7 @@ prep_tail_kernel(TailArgs A, int n_tail, int B, int Gq, tq_layer ly, float* __re
     const int words = ly.d / PREP_COLS, p = id - n_tail;
     // (arrivals: the arrival counters of the groups of query heads, zeroed for a page kernel that merges its splits itself)
     prep_query_body<PER, DT, PACKED>(A.q, Gq, prep_gpw, (int64_t)B * A.Hq, g_tot, ly, A.sm_scale, q_rot, q_sk, q_stat, qa_pack,
-                                     arrivals, p / words, p % words, sm);
+                                     arrivals, head_rows, p / words, p % words, sm);
   }
 }
 
@@ -959,7 +959,7 @@ std::atomic<int> opt_wide_workgroups{1};
 std::atomic<int> opt_split_skew{1};
 std::atomic<int> opt_merge_row_groups{1};
 std::atomic<int> opt_tail_chunks{1};
-std::atomic<int> opt_prefetch_trips{1};
+std::atomic<int> opt_prefetch_trips{-1};
 std::atomic<int> opt_prep_mfma{1};
 }  // namespace tq
 
@@ -972,7 +972,7 @@ extern "C" int tq_set_option(const char* name, int64_t value) {
     return TQ_OK;
   }
   if (!std::strcmp(name, "prefetch_trips")) {
-    if (value < 0 || value > 64) return TQ_EINVAL;
+    if (value < -1 || value > 64) return TQ_EINVAL;
     opt_prefetch_trips.store((int)value);
     return TQ_OK;
   }
@@ -1125,7 +1125,11 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
     // Workgroups added to the preparation launch read the first pages of every page-kernel workgroup's range
     // ahead of it (the preparation leaves most of the card idle): prefetch_trips trips of each block walker.
     PagePrefetch pf;
-    const int pf_trips = mfma_shape ? opt_prefetch_trips.load(std::memory_order_relaxed) : 0;
+    // By default (-1) only at head_dim 256: there the read-ahead takes 1.5 us off the page kernel and adds 0.7 - 1.1 us to the
+    // preparation launch (4 x 131072: step 54.8 -> 54.0 us); at head_dim 128 / 64 it moves as much time as it saves
+    // (16 x 8192: page kernel 33.1 -> 31.4 us, step 38.1 -> 38.7 us; 64 x 2048: step 35.3 -> 36.4 us).
+    const int pf_opt = opt_prefetch_trips.load(std::memory_order_relaxed);
+    const int pf_trips = mfma_shape ? (pf_opt < 0 ? (d == 256 ? 1 : 0) : pf_opt) : 0;
     if (pf_trips > 0 && (int64_t)n_split * Hkv * kv_div * B <= 4096) {
       decode_mfma_plan(pf, d, B, Hkv * kv_div, kv_div, n_split, wide_wg);
       pf.pool = pool; pf.block_table = block_table; pf.seq_lens = seq_lens;
@@ -1165,7 +1169,8 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
     pf.front = n_tail + n_prep;                                                                                      \
     if (pf.front > 2 * device_compute_units()) pf.blocks = 0;                                                        \
     kern<<<dim3((unsigned)(n_tail + n_prep + (pf.blocks > 0 ? pf.n_wg : 0))), dim3(TAIL_THREADS), fsm, st>>>(        \
-        ta, n_tail, B, Gq, *layer, q_rot, q_sk, q_stat, qa_pack, fm.counters, prep_gpw, n_tail + n_prep, pf, g_tot); \
+        ta, n_tail, B, Gq, *layer, q_rot, q_sk, q_stat, qa_pack, fm.counters, prep_gpw, n_tail + n_prep, pf, g_tot, \
+        decode_mfma_head_rows(d, Gq));                                                                               \
   }
 #define TQ_LAUNCH_PT_DT(PER, PAGED)                                \
   {                                                                \

@@ -3,6 +3,7 @@
 #pragma once
 
 #include "tq_common.h"
+#include "tq_options.h"
 
 namespace tq {
 
@@ -17,6 +18,15 @@ struct FusedMerge {
   int n_extra = 0;                   // parts after the n_split splits that an earlier launch has written (the exact tail)
 };
 constexpr int MERGE_IN_KERNEL_MAX_SPLITS = 8;
+
+// Operand rows (query heads) of a group that the page kernel reads from the packed query operands: with at most four
+// heads per group the kernels that take them (two pages per score instruction at head_dim 64, one operand per plane
+// word at head_dim 128 / 256) only touch the rows of heads 0..3, so the preparation need not write zeros into the rest.
+inline int decode_mfma_head_rows(int d, int G) {
+  const bool four = G <= 4 && (d == 64 ? opt_page_pairs.load(std::memory_order_relaxed) != 0
+                                       : opt_narrow_rows.load(std::memory_order_relaxed) != 0);
+  return four ? 4 : 8;
+}
 
 // The blocks (64 tokens) a page-kernel workgroup walks: split `split` of n_split over a sequence of seq_len
 // compressed tokens.  skew16 > 0 (head_dim 256, two workgroups per compute unit): every even split takes skew16

@@ -1142,11 +1142,11 @@ static int launch_one(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, 
   size_t merge = (size_t)(NW / DS * G * (D + 2) + NW * 16 * 16) * sizeof(float);
   if (SG) per_wave += stage_bytes((D / DS / 16) * VB / 2);
   size_t smem = per_wave * NW > merge ? per_wave * NW : merge;
-  if (D == 64 && !PP && G <= 4 && opt_page_pairs.load(std::memory_order_relaxed) != 0)
+  if (D == 64 && !PP && decode_mfma_head_rows(D, G) == 4)
     return launch_one<D, MB, NX, VB, GS, DS, WPS, F16P, D == 64>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,
                                                                  bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts,
                                                                  n_split, len_sub, max_pages, num_pages, fm, wide_wg, st);
-  if (D >= 128 && !NR && G <= 4 && opt_narrow_rows.load(std::memory_order_relaxed) != 0)
+  if (D >= 128 && !NR && decode_mfma_head_rows(D, G) == 4)
     return launch_one<D, MB, NX, VB, GS, DS, WPS, F16P, false, D >= 128>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,
                                                                          bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts,
                                                                          n_split, len_sub, max_pages, num_pages, fm, wide_wg, st);

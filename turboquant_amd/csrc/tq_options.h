@@ -13,7 +13,7 @@ extern std::atomic<int> opt_wide_workgroups;   // decode, head_dim 64 / 128, sho
 extern std::atomic<int> opt_split_skew;        // decode, two workgroups per compute unit: sixteenths of a split moved to the workgroup dispatched first (0: none)
 extern std::atomic<int> opt_tail_chunks;        // hybrid decode with many splits: up to 4 workgroups share the exact tokens of a head group
 extern std::atomic<int> opt_merge_row_groups;  // merge kernel: with few rows, several workgroups share a row's channels
-extern std::atomic<int> opt_prefetch_trips;     // decode: trips of every block walker whose pages the preparation launch reads ahead (0: none)
+extern std::atomic<int> opt_prefetch_trips;     // decode: trips of every block walker whose pages the preparation launch reads ahead (0: none, -1: one at head_dim 256)
 extern std::atomic<int> opt_prep_mfma;           // decode: bf16 queries at head_dim 128 / 256 are prepared on the matrix cores
 extern std::atomic<int> opt_merge_in_kernel;    // decode: few context splits are merged by the last workgroup of the page kernel
 }  // namespace tq

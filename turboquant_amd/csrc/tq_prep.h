@@ -88,8 +88,8 @@ template <int PER, int DT, bool PACKED>
 __device__ __forceinline__ void prep_query_body(const void* __restrict__ q, int G, int gpw, int64_t n_rows, int g_tot, const tq_layer& ly,
                                                 float sm_scale, float* __restrict__ q_rot, float* __restrict__ q_sk,
                                                 float* __restrict__ q_stat, uint32_t* __restrict__ qa_pack,
-                                                unsigned long long* __restrict__ arrivals, int64_t unit, int word,
-                                                float* sm) {
+                                                unsigned long long* __restrict__ arrivals, int head_rows, int64_t unit,
+                                                int word, float* sm) {
   const int d = ly.d, tid = threadIdx.x, jl = tid % PREP_COLS, sl = tid / PREP_COLS;
   const int j = word * PREP_COLS + jl;
   const int RG = PACKED ? G * gpw : G;                                 // rows a workgroup has room for
@@ -243,9 +243,10 @@ __device__ __forceinline__ void prep_query_body(const void* __restrict__ q, int 
   // gets the rounded values back for the residual with its inverse (v_cvt_scalef32_pk32_f32_fp6).
   // Code j of a conversion comes from element j / 2 of its first (j even) or second (j odd) operand.
   // Lane (term plane, row g) belongs to head g % G of the workgroup's group g / G.  The operand rows of the heads
-  // a group does not have are zero: with one group per workgroup the lanes beyond its heads write them (lane g
-  // the rows of head g), with several groups the lane of head h writes those of h + G, h + 2 G, ... below 8.
-  if (tid < ntp * 8 && ((tid & 7) < R || !PACKED || gpw == 1)) {
+  // a group does not have are zero, as far as the page kernel reads them (head_rows: 4 or 8): with one group per
+  // workgroup the lanes beyond its heads write them (lane g the rows of head g), with several groups the lane of
+  // head h writes those of h + G, h + 2 G, ... below head_rows.
+  if (tid < ntp * 8 && ((tid & 7) < R || ((!PACKED || gpw == 1) && (tid & 7) < head_rows))) {
     typedef float f32x16_t __attribute__((ext_vector_type(16)));
     typedef float f32x32_t __attribute__((ext_vector_type(32)));
     typedef uint32_t u32x6_t __attribute__((ext_vector_type(6)));
@@ -280,12 +281,13 @@ __device__ __forceinline__ void prep_query_body(const void* __restrict__ q, int 
       // (inline assembly with early-clobber results: the conversions read their sources over several passes)
       asm volatile("v_cvt_scalef32_2xpk16_fp6_f32 %0, %1, %2, %3" : "=&v"(code) : "v"(va), "v"(vb), "v"(one));
       uint32_t* o = dst + (((tp * wpl + i) * 2 + (t >> 1)) * 64 + 2 * hg + (t & 1) + 16 * kw) * 8;
+      // (whole 32-byte slots, the two unused dwords included: full sectors reach memory without a merge)
       *(uint4*)o = make_uint4(code[0], code[1], code[2], code[3]);
-      *(uint2*)(o + 4) = make_uint2(code[4], code[5]);
-      for (int ha = hg + G; PACKED && gpw > 1 && ha < 8; ha += G) {        // heads the group does not have
+      *(uint4*)(o + 4) = make_uint4(code[4], code[5], 0u, 0u);
+      for (int ha = hg + G; PACKED && gpw > 1 && ha < head_rows; ha += G) {   // heads the group does not have
         uint32_t* z = o + (2 * (ha - hg)) * 8;
         *(uint4*)z = make_uint4(0u, 0u, 0u, 0u);
-        *(uint2*)(z + 4) = make_uint2(0u, 0u);
+        *(uint4*)(z + 4) = make_uint4(0u, 0u, 0u, 0u);
       }
       if (t < 3) {
         f32x32_t r;
@@ -401,8 +403,8 @@ __host__ __device__ inline int prep_mfma_smem_floats() { return 2 * 16 * PREP_MF
 template <int D>
 __device__ __forceinline__ void prep_mfma_body(const uint16_t* __restrict__ q, int G, int64_t n_rows, const tq_layer& ly,
                                                float sm_scale, float* __restrict__ q_stat, uint32_t* __restrict__ qa_pack,
-                                               unsigned long long* __restrict__ arrivals, int64_t tile, int word,
-                                               float* sm) {
+                                               unsigned long long* __restrict__ arrivals, int head_rows, int64_t tile,
+                                               int word, float* sm) {
   constexpr int KS = D / 32;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n = lane & 15, kb = lane >> 4;
@@ -535,12 +537,13 @@ __device__ __forceinline__ void prep_mfma_body(const uint16_t* __restrict__ q, i
       u32x6_t code;
       asm volatile("v_cvt_scalef32_2xpk16_fp6_f32 %0, %1, %2, %3" : "=&v"(code) : "v"(va), "v"(vb), "v"(one));
       uint32_t* o = dst + (((tp * wpl + chunk) * 2 + (t >> 1)) * 64 + 2 * hg + (t & 1) + 16 * kw) * 8;
+      // (whole 32-byte slots, the two unused dwords included: full sectors reach memory without a merge)
       *(uint4*)o = make_uint4(code[0], code[1], code[2], code[3]);
-      *(uint2*)(o + 4) = make_uint2(code[4], code[5]);
-      for (int ha = hg + G; ha < 8; ha += G) {                       // operand rows of heads the group does not have
+      *(uint4*)(o + 4) = make_uint4(code[4], code[5], 0u, 0u);
+      for (int ha = hg + G; ha < head_rows; ha += G) {               // operand rows of heads the group does not have
         uint32_t* z = o + (2 * (ha - hg)) * 8;
         *(uint4*)z = make_uint4(0u, 0u, 0u, 0u);
-        *(uint2*)(z + 4) = make_uint2(0u, 0u);
+        *(uint4*)(z + 4) = make_uint4(0u, 0u, 0u, 0u);
       }
       if (t < 3) {
         f32x32_t rr;

@@ -74,15 +74,15 @@ template <int PER, int DT, bool PACKED>
 __global__ void __launch_bounds__(PREP_COLS * PREP_SLICES)
 prep_query_kernel(const void* __restrict__ q, int G, int gpw, int64_t n_rows, int g_tot, tq_layer ly, float sm_scale,
                   float* __restrict__ q_rot, float* __restrict__ q_sk, float* __restrict__ q_stat,
-                  uint32_t* __restrict__ qa_pack, unsigned long long* __restrict__ arrivals, int n_units, int n_prep,
-                  PagePrefetch pf) {
+                  uint32_t* __restrict__ qa_pack, unsigned long long* __restrict__ arrivals, int head_rows, int n_units,
+                  int n_prep, PagePrefetch pf) {
   extern __shared__ __align__(16) float sm[];
   // the preparation workgroups first (unit fastest, as a two-dimensional grid would order them), then the
   // workgroups that read the page kernel's first pages ahead of it
   const int id = blockIdx.x;
   if (id < n_prep)
-    prep_query_body<PER, DT, PACKED>(q, G, gpw, n_rows, g_tot, ly, sm_scale, q_rot, q_sk, q_stat, qa_pack, arrivals, id % n_units,
-                                     id / n_units, sm);
+    prep_query_body<PER, DT, PACKED>(q, G, gpw, n_rows, g_tot, ly, sm_scale, q_rot, q_sk, q_stat, qa_pack, arrivals, head_rows,
+                                     id % n_units, id / n_units, sm);
   else
     prefetch_pages_body<PREP_COLS * PREP_SLICES>(pf, id - n_prep);
 }
@@ -93,11 +93,13 @@ template <int D>
 __global__ void __launch_bounds__(PREP_MFMA_THREADS)
 prep_mfma_kernel(const uint16_t* __restrict__ q, int G, int64_t n_rows, tq_layer ly, float sm_scale,
                  float* __restrict__ q_stat, uint32_t* __restrict__ qa_pack, unsigned long long* __restrict__ arrivals,
-                 int n_tiles, int n_prep, PagePrefetch pf) {
+                 int head_rows, int n_tiles, int n_prep, PagePrefetch pf) {
   extern __shared__ __align__(16) float sm[];
   const int id = blockIdx.x;
-  if (id < n_prep) prep_mfma_body<D>(q, G, n_rows, ly, sm_scale, q_stat, qa_pack, arrivals, id % n_tiles, id / n_tiles, sm);
-  else prefetch_pages_body<PREP_MFMA_THREADS>(pf, id - n_prep);
+  if (id < n_prep)
+    prep_mfma_body<D>(q, G, n_rows, ly, sm_scale, q_stat, qa_pack, arrivals, head_rows, id % n_tiles, id / n_tiles, sm);
+  else
+    prefetch_pages_body<PREP_MFMA_THREADS>(pf, id - n_prep);
 }
 
 // scores[b, i, k] for a tile of QT queries and one key per thread.  The rotated and sketched queries sit
@@ -390,8 +392,12 @@ int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* 
     // (head_dim 256 with few rows keeps the vector-ALU kernel: 64 rows - 32 workgroups here, each pulling 96 KB of
     // matrix terms - measured 1 us slower per step; from 64 workgroups on the two are level or this one ahead:
     // 16 x 8192 at 32 q heads 35.0 -> 34.5 us per step, 64 x 2048 40.2 -> 36.4, 256 x 1024 107.6 -> 86.2)
+    const int head_rows = decode_mfma_head_rows(d, G);      // rows of a group's operands the page kernel reads
     const int rows_tile = (16 / G) * G;
-    const int n_tiles = (int)((rows + rows_tile - 1) / rows_tile), n_mprep = n_tiles * (d / 32);
+    const int n_tiles = (int)((rows + rows_tile - 1) / rows_tile);
+    // (several tiles per workgroup - in turn, or their products first and then all four wavefronts packing - measured
+    // slower at every size: 256 x 1024 tokens 83.0 -> 83.9 us per step with four, 64 x 2048 33.8 -> 38.6)
+    const int n_mprep = n_tiles * (d / 32);
     const int mfma_opt = opt_prep_mfma.load(std::memory_order_relaxed);
     if (dtype == TQ_BF16 && (d == 128 || d == 256) && layer->Pi_split && layer->S_split && g_tot == 0 && q_rot_unused &&
         (((uintptr_t)q) & 15) == 0 && mfma_opt != 0 && (d == 128 || n_mprep >= 64 || mfma_opt > 1)) {
@@ -402,10 +408,10 @@ int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* 
       const size_t smem = (size_t)prep_mfma_smem_floats() * sizeof(float);
       if (d == 128)
         prep_mfma_kernel<128><<<grid, block, smem, st>>>((const uint16_t*)q, G, rows, *layer, sm_scale, q_stat, qa_pack,
-                                                         arrivals, n_tiles, n_mprep, pf);
+                                                         arrivals, head_rows, n_tiles, n_mprep, pf);
       else
         prep_mfma_kernel<256><<<grid, block, smem, st>>>((const uint16_t*)q, G, rows, *layer, sm_scale, q_stat, qa_pack,
-                                                         arrivals, n_tiles, n_mprep, pf);
+                                                         arrivals, head_rows, n_tiles, n_mprep, pf);
       hipError_t e = hipGetLastError();
       return e == hipSuccess ? TQ_OK : (int)e;
     }
@@ -427,10 +433,10 @@ int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* 
   {                                                                                                                    \
     if (gpw > 1)                                                                                                       \
       prep_query_kernel<PER, DT, true><<<grid, block, smem, st>>>(q, G, gpw, rows, g_tot, *layer, sm_scale, q_rot, q_sk, q_stat, \
-                                                                  qa_pack, arrivals, n_units, n_prep, pf);              \
+                                                                  qa_pack, arrivals, head_rows, n_units, n_prep, pf);              \
     else                                                                                                               \
       prep_query_kernel<PER, DT, false><<<grid, block, smem, st>>>(q, G, gpw, rows, g_tot, *layer, sm_scale, q_rot, q_sk, q_stat, \
-                                                                   qa_pack, arrivals, n_units, n_prep, pf);             \
+                                                                   qa_pack, arrivals, head_rows, n_units, n_prep, pf);             \
   }
 #define TQ_PREP_DT(PER)                              \
   {                                                  \
