@@ -642,6 +642,26 @@ def test_hybrid_step_of_many_sequences_at_head_dim_256(gpu):
         _progress(f"  worst cosine {worst:.7f}")
 
 
+def test_hybrid_step_of_many_sequences_with_the_preparation_on_the_matrix_cores(gpu):
+    """A hybrid step whose query preparation alone is more workgroups than the card holds at once (here 80 sequences
+    x 32 query heads at head_dim 128, bf16): the exact tail and the preparation run as a launch each, the latter on the
+    matrix cores, instead of sharing the launch of the vector-ALU preparation (score.py:99-173 against the oracle,
+    ragged histories and tails; and against the shared launch, which sums the rotation in another order)."""
+    from turboquant_amd import _ffi
+    B = 80
+    lens = [48 * (b % 7) + 5 * b for b in range(B)]
+    recent = [128 if b % 3 else (11 * b) % 128 for b in range(B)]
+    outs = []
+    try:
+        for on in (1, 0):
+            _ffi.check(_ffi.lib().tq_set_option(b"prep_mfma", on), "tq_set_option")
+            _progress(f"many sequences d=128 prep_mfma={on}")
+            outs.append(_decode_case(gpu, 128, 3, 4, B, 32, 8, lens, recent, seed=977, n_split=1, return_out=True))
+    finally:
+        _ffi.check(_ffi.lib().tq_set_option(b"prep_mfma", 1), "tq_set_option")
+    assert float((outs[0].float() - outs[1].float()).abs().max()) <= 2.0 ** -7 * float(outs[1].float().abs().max()) + 1e-6
+
+
 @pytest.mark.parametrize("d,dtype,Hq,Hkv,recent,n_split,pad", [
     (256, torch.bfloat16, 16, 2, [128, 3, 0], 12, 0),      # four workgroups per head group; shares of 32, of 0 / 1 tokens, of none
     (128, torch.float16, 8, 1, [300, 77, 1], 9, 8),        # several load rounds per share, rows inside a wider buffer

@@ -941,6 +941,7 @@ namespace tq {
 int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* layer, float* q_rot, float* q_sk,
                         float* q_stat, uint32_t* qa_pack, int G, float sm_scale, hipStream_t st, bool q_rot_unused,
                         unsigned long long* arrivals, const PagePrefetch* prefetch, int g_tot);
+bool prep_on_matrix_cores(const void* q, int dtype, int64_t rows, const tq_layer* layer, int G, int g_tot);
 }  // namespace tq
 
 static size_t parts_floats(int B, int Hq, int d, int n_parts) { return (size_t)B * Hq * n_parts * (d + 2); }
@@ -1158,7 +1159,12 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
     // tokens: 139 KB) and the grid is larger than the card: the preparation workgroups would queue behind that
     // LDS size too (128 x 2048, 16 q / 2 KV heads: 109.7 us per step fused, 88.1 as two launches)
     const bool one_per_unit = fsm > (size_t)80 * 1024;
-    if (tail && ta.wide && mfma_shape && stages == 7 && !(one_per_unit && n_tail + n_prep > device_compute_units())) {
+    // ... or the preparation alone is more than the card holds at once and can run on the matrix cores, which the
+    // shared launch (vector-ALU preparation body) cannot: then a launch each
+    const bool mfma_prep_ahead = mfma_shape && n_prep > 2 * device_compute_units() &&
+                                 prep_on_matrix_cores(q, dtype, (int64_t)B * Hq, layer, Gq, g_tot);
+    if (tail && ta.wide && mfma_shape && stages == 7 && !mfma_prep_ahead &&
+        !(one_per_unit && n_tail + n_prep > device_compute_units())) {
 #define TQ_LAUNCH_PT(PER, DT, PAGED)                                                                                 \
   {                                                                                                                  \
     auto kern = prep_gpw > 1 ? prep_tail_kernel<PER, DT, PAGED, true> : prep_tail_kernel<PER, DT, PAGED, false>;     \

@@ -376,6 +376,22 @@ namespace tq {
 int launch_dequant_mfma(const uint8_t* idx, const uint8_t* signs, const void* norms, int norm_dtype, const float* rnorms,
                         int64_t n_vec, const tq_layer& ly, float* out, hipStream_t st);
 
+// Whether launch_rotate_query prepares these rows on the matrix cores (bf16 queries at head_dim 128 / 256 with the
+// split matrices at hand; whole groups of G heads; operands only).
+// (head_dim 256 with few rows keeps the vector-ALU kernel: 64 rows - 32 workgroups here, each pulling 96 KB of
+// matrix terms - measured 1 us slower per step; from 64 workgroups on the two are level or this one ahead:
+// 16 x 8192 at 32 q heads 35.0 -> 34.5 us per step, 64 x 2048 40.2 -> 36.4, 256 x 1024 107.6 -> 86.2)
+bool prep_on_matrix_cores(const void* q, int dtype, int64_t rows, const tq_layer* layer, int G, int g_tot) {
+  const int d = layer->d;
+  if (g_tot > 0 && g_tot % G == 0) g_tot = 0;
+  const int rows_tile = (16 / G) * G;
+  const int64_t n_mprep = ((rows + rows_tile - 1) / rows_tile) * (d / 32);
+  const int mfma_opt = opt_prep_mfma.load(std::memory_order_relaxed);
+  return dtype == TQ_BF16 && (d == 128 || d == 256) && layer->Pi_split && layer->S_split && layer->Pi_colsum &&
+         layer->S_colsum && g_tot == 0 && G <= ROT_MAX_ROWS && rows % G == 0 && (((uintptr_t)q) & 15) == 0 &&
+         mfma_opt != 0 && (d == 128 || n_mprep >= 64 || mfma_opt > 1);
+}
+
 // q_rot_unused: the caller only needs the packed operands and statistics (the page kernel on the matrix
 // cores), not the fp32 rotated / sketched queries
 int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* layer, float* q_rot, float* q_sk,
@@ -388,19 +404,13 @@ int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* 
     if (!q_stat || !layer->Pi_colsum || !layer->S_colsum || G > ROT_MAX_ROWS || (g_tot > 0 ? rows % g_tot : rows % G) ||
         (d != 64 && d != 128 && d != 256))
       return TQ_EUNSUPPORTED;
-    // bf16 queries at head_dim 128 / 256 with the split matrices at hand: the products run on the matrix cores
-    // (head_dim 256 with few rows keeps the vector-ALU kernel: 64 rows - 32 workgroups here, each pulling 96 KB of
-    // matrix terms - measured 1 us slower per step; from 64 workgroups on the two are level or this one ahead:
-    // 16 x 8192 at 32 q heads 35.0 -> 34.5 us per step, 64 x 2048 40.2 -> 36.4, 256 x 1024 107.6 -> 86.2)
     const int head_rows = decode_mfma_head_rows(d, G);      // rows of a group's operands the page kernel reads
-    const int rows_tile = (16 / G) * G;
-    const int n_tiles = (int)((rows + rows_tile - 1) / rows_tile);
-    // (several tiles per workgroup - in turn, or their products first and then all four wavefronts packing - measured
-    // slower at every size: 256 x 1024 tokens 83.0 -> 83.9 us per step with four, 64 x 2048 33.8 -> 38.6)
-    const int n_mprep = n_tiles * (d / 32);
-    const int mfma_opt = opt_prep_mfma.load(std::memory_order_relaxed);
-    if (dtype == TQ_BF16 && (d == 128 || d == 256) && layer->Pi_split && layer->S_split && g_tot == 0 && q_rot_unused &&
-        (((uintptr_t)q) & 15) == 0 && mfma_opt != 0 && (d == 128 || n_mprep >= 64 || mfma_opt > 1)) {
+    if (q_rot_unused && prep_on_matrix_cores(q, dtype, rows, layer, G, g_tot)) {
+      const int rows_tile = (16 / G) * G;
+      const int n_tiles = (int)((rows + rows_tile - 1) / rows_tile);
+      // (several tiles per workgroup - in turn, or their products first and then all four wavefronts packing - measured
+      // slower at every size: 256 x 1024 tokens 83.0 -> 83.9 us per step with four, 64 x 2048 33.8 -> 38.6)
+      const int n_mprep = n_tiles * (d / 32);
       PagePrefetch pf;
       if (prefetch && prefetch->blocks > 0 && prefetch->n_wg > 0 && n_mprep <= 2 * device_compute_units()) pf = *prefetch;
       pf.front = n_mprep;
