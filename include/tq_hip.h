@@ -365,8 +365,6 @@ void tq_time_next_key_kernel(void *start_event, void *stop_event);
  *                      a partial of its own for the merge kernel; 0: one workgroup and one partial.
  *   "merge_row_groups" 1 (default): the merge kernel gives a row of partials to 2 or 4 workgroups (a share of the
  *                      channels each) when there are fewer rows than compute units; 0: one workgroup per row.
- *   "lds_stage"        1 (default): the 4-bit-key kernels of head_dim 128 / 256 bring the next block's page data
- *                      into LDS with LDS-direct loads instead of holding it in registers; 0: registers (spills).
  *   "fp6_centroids"    1 (default): the key quantiser takes the fp6 x fp4 centroid contraction when the layer
  *                      carries PiT_fp6; 0: always the bf16 term products (for A/B runs).
  *   "append_parts"     measurement only: 3 (default) = the append entry points quantise keys and values,

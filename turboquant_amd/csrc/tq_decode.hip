@@ -955,7 +955,6 @@ std::atomic<int> opt_fp6_centroids{1};
 std::atomic<int> opt_merge_in_kernel{1};
 std::atomic<int> opt_page_pairs{1};
 std::atomic<int> opt_narrow_rows{1};
-std::atomic<int> opt_lds_stage{1};
 std::atomic<int> opt_wide_workgroups{1};
 std::atomic<int> opt_split_skew{1};
 std::atomic<int> opt_merge_row_groups{1};
@@ -984,7 +983,6 @@ extern "C" int tq_set_option(const char* name, int64_t value) {
   }
   if (!std::strcmp(name, "tail_chunks")) { opt_tail_chunks.store(value != 0); return TQ_OK; }
   if (!std::strcmp(name, "merge_row_groups")) { opt_merge_row_groups.store(value != 0); return TQ_OK; }
-  if (!std::strcmp(name, "lds_stage")) { opt_lds_stage.store(value != 0); return TQ_OK; }
   if (!std::strcmp(name, "narrow_rows")) { opt_narrow_rows.store(value != 0); return TQ_OK; }
   if (!std::strcmp(name, "page_pairs")) { opt_page_pairs.store(value != 0); return TQ_OK; }
   if (!std::strcmp(name, "merge_in_kernel")) { opt_merge_in_kernel.store(value != 0); return TQ_OK; }

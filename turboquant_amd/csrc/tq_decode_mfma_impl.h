@@ -1150,12 +1150,15 @@ static int launch_one(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, 
     return launch_one<D, MB, NX, VB, GS, DS, WPS, F16P, false, D >= 128>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,
                                                                          bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts,
                                                                          n_split, len_sub, max_pages, num_pages, fm, wide_wg, st);
-  // (measured: the staged variant only pays where the register-held variant spills, i.e. with three index planes)
+  // Three index planes (4-bit keys) at head_dim 128 / 256: always the variant that stages the next block's page data in
+  // LDS.  With that data in registers these kernels spill 21 - 98 of them (16 x 8192: 63.3 vs 46.6 us per step), so the
+  // register variant is not built; for fewer planes the staged variant measured 2 - 5 % slower and is not built either.
   constexpr bool can_stage = D >= 128 && MB == 3;
-  if (can_stage && !SG && opt_lds_stage.load(std::memory_order_relaxed) != 0)
-    return launch_one<D, MB, NX, VB, GS, DS, WPS, F16P, PP, NR, can_stage>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,
-                                                                           bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts,
-                                                                           n_split, len_sub, max_pages, num_pages, fm, wide_wg, st);
+  if constexpr (can_stage && !SG) {
+    return launch_one<D, MB, NX, VB, GS, DS, WPS, F16P, PP, NR, true>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,
+                                                                      bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts,
+                                                                      n_split, len_sub, max_pages, num_pages, fm, wide_wg, st);
+  } else {
   // eight wavefronts per workgroup (one workgroup per compute unit) for the kernels whose wavefronts work alone
   constexpr bool can_widen = DS == 1 && NW == MF_WAVES;
   if (can_widen && wide_wg)
@@ -1185,6 +1188,7 @@ static int launch_one(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, 
   }
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? TQ_OK : (int)e;
+  }
 }
 
 

@@ -8,7 +8,6 @@ extern std::atomic<int> opt_append_parts;      // measurement: 3 keys and values
 extern std::atomic<int> opt_fp6_centroids;     // key quantiser, head_dim 128: centroid contraction on the fp6 x fp4 MFMA
 extern std::atomic<int> opt_page_pairs;        // decode, head_dim 64 with at most 4 query heads per KV head: one score MFMA per two pages
 extern std::atomic<int> opt_narrow_rows;       // decode, head_dim 128 / 256 with at most 4 query heads per KV head: one score MFMA per plane word
-extern std::atomic<int> opt_lds_stage;         // decode: page data through LDS-direct loads, a whole trip ahead
 extern std::atomic<int> opt_wide_workgroups;   // decode, head_dim 64 / 128, short contexts: workgroups of 8 wavefronts
 extern std::atomic<int> opt_split_skew;        // decode, two workgroups per compute unit: sixteenths of a split moved to the workgroup dispatched first (0: none)
 extern std::atomic<int> opt_tail_chunks;        // hybrid decode with many splits: up to 4 workgroups share the exact tokens of a head group
