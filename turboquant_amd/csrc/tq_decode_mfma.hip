@@ -4,6 +4,8 @@
 
 #include <hip/hip_ext.h>
 
+#include <atomic>
+
 #include "tq_common.h"
 #include "tq_prep.h"
 #include "tq_decode_mfma.h"
@@ -37,14 +39,18 @@ bool decode_mfma_wide_workgroups(int d, int G, int n_split, int max_pages) {
 }
 
 // Compute units of the device that is current at the first call (the cards of one machine are alike); 0 if unknown.
+// compute units of the current device (looked up once per device)
 int device_compute_units() {
-  static const int units = [] {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) n = 0;
-    return n;
-  }();
-  return units;
+  static std::atomic<int> units[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 0;
+  const bool cached = dev >= 0 && dev < 64;
+  int n = cached ? units[dev].load(std::memory_order_relaxed) : 0;
+  if (n <= 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) n = 0;
+    if (cached && n > 0) units[dev].store(n, std::memory_order_relaxed);
+  }
+  return n;
 }
 
 // Unequal shares for the two workgroups of a compute unit.  Workgroups are dispatched in grid order and spread

@@ -802,15 +802,15 @@ static int launch_dt_d(const void* x, const Source& src, const tq_layer& ly, con
     if (dev < 64) configured.fetch_or(1ull << dev);
   }
   // persistent workgroups: as many as stay resident (LDS allows 160 KB / bytes per compute unit)
-  static std::atomic<int> n_cu{0};
-  if (!n_cu.load()) {
-    int v = 0;
-    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) v = 256;
-    n_cu.store(v);
+  static std::atomic<int> n_cu[64];                       // per device
+  int cus = dev < 64 ? n_cu[dev].load(std::memory_order_relaxed) : 0;
+  if (cus <= 0) {
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+    if (dev < 64) n_cu[dev].store(cus, std::memory_order_relaxed);
   }
   const int per_cu = (int)(160 * 1024 / Sm::bytes) > 2 ? 2 : (int)(160 * 1024 / Sm::bytes);
   const int64_t groups = (tiles + Gm::MT - 1) / Gm::MT;
-  const int64_t resident = (int64_t)n_cu.load() * (per_cu > 0 ? per_cu : 1);
+  const int64_t resident = (int64_t)cus * (per_cu > 0 ? per_cu : 1);
   const unsigned grid = (unsigned)(groups < resident ? groups : resident);
   hipEvent_t ev_start = nullptr, ev_stop = nullptr;
   if (std::is_same<Sink, KeyPagedSink>::value && take_time_hook(1, ev_start, ev_stop)) {
