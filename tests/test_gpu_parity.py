@@ -574,7 +574,8 @@ def test_decode_attention_general_kernel_shapes(gpu, d, key_bits, vb, Hq, Hkv, d
     # fp16 pools (matrix-core kernel with the fp16 zero-point product), more than 8 query heads per KV head
     # (served as ceil(G / 8) groups of at most 8 that read the same pages: 16 = 8 + 8, 12 = 6 + 6, and unequal ones
     # where G does not divide: 9 = 5 + 4, 11 = 6 + 5, 13 = 7 + 6, 15 = 8 + 7), and shapes without a matrix-core
-    # kernel (fp32 pools, head sizes other than 64 / 128 / 256, 5-bit keys), which take the general page kernel:
+    # kernel (fp32 pools, head sizes other than 64 / 128 / 256, 5-bit keys at head_dim 64), which take the general page
+    # kernel:
     # all must meet the same gate
     _progress(f"general decode d={d} kb={key_bits} vb={vb} Hq={Hq} Hkv={Hkv} {dtype}")
     worst = _decode_case(gpu, d, key_bits, vb, 2, Hq, Hkv, [300, 77], [0, 9], seed=500 + d + Hq, dtype=dtype)

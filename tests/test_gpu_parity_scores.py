@@ -577,6 +577,19 @@ def test_four_bit_keys_staged_through_lds(gpu, d, vb, Hq, Hkv, dtype):
     _variant_against_default(gpu, "merge_in_kernel", d, 4, vb, Hq, Hkv, dtype, exact=False, rel=2.0 ** -8)
 
 
+@pytest.mark.parametrize("option", ["merge_in_kernel", "narrow_rows", "wide_workgroups"])
+@pytest.mark.parametrize("vb,Hq,Hkv,dtype", [(4, 16, 2, torch.bfloat16), (2, 3, 1, torch.float16), (4, 32, 2, torch.bfloat16),
+                                             (2, 18, 2, torch.bfloat16)])
+def test_five_bit_keys_with_the_query_operands_in_lds(gpu, option, vb, Hq, Hkv, dtype):
+    """5-bit keys at head_dim 128 (four index planes + the sign plane, nine fp6 terms per query row): the query's
+    matrix-core operands do not fit in registers beside the page data, so each workgroup copies its group's
+    operands to LDS once and the score stage reads one term plane at a time for all pages of the block.  Groups of
+    8, 3 (four-row operands), 16 (two groups of 8) and 9 (5 + 4) query heads per KV head; ragged lengths, a
+    poisoned block table and 1 - 11 context splits against the oracle (score.py:84-173), with each of the merge,
+    row-count and workgroup-width variants on and off."""
+    _variant_against_default(gpu, option, 128, 5, vb, Hq, Hkv, dtype, exact=False, rel=2.0 ** -8)
+
+
 @pytest.mark.parametrize("B,Hq,Hkv,d,key_bits,vb,dtype", [(201, 4, 1, 128, 3, 4, torch.bfloat16), (201, 2, 1, 128, 4, 2, torch.bfloat16),
                                                            (101, 3, 1, 256, 3, 2, torch.float16), (401, 1, 1, 64, 3, 4, torch.bfloat16),
                                                            (70, 12, 2, 128, 2, 4, torch.bfloat16)])

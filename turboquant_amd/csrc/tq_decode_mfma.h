@@ -86,7 +86,7 @@ size_t decode_mfma_pack_words(int B, int Hq, int d);
 #define TQ_MFMA_SHAPES_D128(X) \
   X(128, 2, 0, 2, 32, 1, 2) X(128, 2, 0, 4, 32, 1, 2) X(128, 1, 0, 2, 32, 1, 2) X(128, 1, 0, 4, 32, 1, 2) \
   X(128, 3, 1, 2, 32, 1, 2) X(128, 3, 1, 4, 32, 1, 2) X(128, 2, 0, 2, 64, 1, 2) X(128, 2, 0, 4, 64, 1, 2) \
-  X(128, 2, 0, 8, 32, 1, 2)
+  X(128, 2, 0, 8, 32, 1, 2) X(128, 4, 4, 4, 32, 1, 2) X(128, 4, 4, 2, 32, 1, 2)
 #define TQ_MFMA_SHAPES_D256(X) \
   X(256, 2, 0, 2, 32, 2, 2) X(256, 2, 0, 4, 32, 2, 2) X(256, 1, 0, 2, 32, 2, 2) X(256, 1, 0, 4, 32, 2, 2) \
   X(256, 3, 1, 2, 32, 2, 2) X(256, 3, 1, 4, 32, 2, 2) X(256, 2, 0, 2, 64, 2, 2) X(256, 2, 0, 4, 64, 2, 2) \

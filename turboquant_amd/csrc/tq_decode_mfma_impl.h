@@ -255,6 +255,11 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   static_assert(!SG || (NKW >= 3 && !PP), "staged loads take 12 or 16 key bytes per lane");
   constexpr int STAGE_BYTES = stage_bytes(VW);
   constexpr int NRS = NR ? 1 : 2;             // fp6 operands (row sets) per plane word
+  // Four stored index planes (5-bit keys: nine term planes with the multi-bit terms and the signs): the query
+  // operands - 72 to 144 registers - stay in LDS, one copy per workgroup, and the score stage walks a block plane
+  // by plane so that an operand is read once for its four pages.
+  constexpr bool QL = MB >= 4;
+  static_assert(!QL || (!PP && !SG && DS == 1), "operands in LDS: head_dim 128, page data in registers");
   constexpr int NJ = NR ? 1 : 2;              // heads a lane sees in the score MFMA's output
   // Hkv counts query-head groups: a KV head with more than 8 query heads is served by kv_div groups of at most 8
   // heads each (consecutive groups read the same pages); when the heads do not divide evenly the last group of
@@ -300,6 +305,8 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   float* s_x_peer = (float*)smem_raw + (wave ^ 1) * WAVE_LDS_FLOATS + (4 * 8 * P_STRIDE + 16 + 4 * NG * 16);
   float* s_red = (float*)smem_raw;                          // after the loop: [NGRP][G][D + 2]
   // SG: this wavefront's staging area behind the wavefronts' private regions
+  // QL: the group's packed query operands behind the wavefronts' private regions
+  uint32_t* qa_lds = (uint32_t*)(smem_raw + MF_WAVES * WAVE_LDS_FLOATS * sizeof(float));
   unsigned char* stage = smem_raw + MF_WAVES * WAVE_LDS_FLOATS * sizeof(float) + wave * STAGE_BYTES;
   unsigned char* stage_m = stage + 4 * 1024;
   unsigned char* stage_v = stage_m + 512;
@@ -310,8 +317,9 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   // fp6 query terms in register order (see the preparation kernel): row set 0 = terms 0, 1 of the 8
   // heads (row 2g + t), row set 1 = terms 2, 3; rows of absent heads are zero.  Six dwords per
   // lane are stored at a stride of eight.
-  i32x8 qa[NTP][WPL][NRS];
+  i32x8 qa[QL ? 1 : NTP][WPL][NRS];
   int sa = 0;
+  int qa_lane = 0;                             // QL: dword offset of this lane's slot inside an operand of 64 slots
   f32x4 cm = {0, 0, 0, 0}, cq = {0, 0, 0, 0};
   auto load_operands = [&]() {
   {
@@ -321,6 +329,14 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
     const bool a_live = !PP || ((n < 8) == (kb < 2));
     const uint32_t* src = qa_pack + (((int64_t)b * Hkv + h) * (NTP * WPLT * 2 * 64) + slane) * 8 +
                           (NR ? ((n >> 1) & 1) * (64 * 8) : 0);
+    if constexpr (QL) {
+      // the whole block of the group, 16 bytes per lane and step, as it lies in memory
+      const uint32_t* blk = qa_pack + ((int64_t)b * Hkv + h) * (NTP * WPLT * 2 * 64 * 8);
+      for (int o = tid * 4; o < NTP * WPLT * 2 * 64 * 8; o += MF_WAVES * 64 * 4)
+        *(u32x4*)(qa_lds + o) = *(const u32x4*)(blk + o);
+      qa_lane = slane * 8 + (NR ? ((n >> 1) & 1) * (64 * 8) : 0);
+      __syncthreads();
+    } else
 #pragma unroll
     for (int tp = 0; tp < NTP; ++tp)
 #pragma unroll
@@ -440,7 +456,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
     }
     return bad;
   };
-  auto load_keys = [&](const int (&pid)[4], KeyRegs& R) {
+  auto load_keys = [&](const int (&pid)[4], KeyRegs& R) __attribute__((always_inline)) {
     // the 32-bit lane offsets are re-materialised here, next to their use, so that the loads take
     // the scalar page base plus a 32-bit vector offset instead of a 64-bit vector address
     const uint32_t ok = in_vgpr(off_keys), om = in_vgpr(off_meta);
@@ -475,7 +491,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   // The page of a lane is picked among the four page numbers with conditional moves on vector
   // registers (on scalar operands the compiler builds branches instead) and turned into an address
   // with one unsigned 32 x 32 -> 64 bit multiply-add.
-  auto load_vals = [&](const int (&pid)[4], ValRegs& R) {
+  auto load_vals = [&](const int (&pid)[4], ValRegs& R) __attribute__((always_inline)) {
     const uint32_t p0 = in_vgpr((uint32_t)pid[0]), p1 = in_vgpr((uint32_t)pid[1]), p2 = in_vgpr((uint32_t)pid[2]),
                    p3 = in_vgpr((uint32_t)pid[3]);
     const uint32_t my_pid = kb == 0 ? p0 : (kb == 1 ? p1 : (kb == 2 ? p2 : p3));
@@ -567,7 +583,9 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
     return ((bad >> pg) & 1) ? 0 : min(max(seq_len - (blk * BLK_TOK + pg * 16), 0), 16);
   };
   bool fresh = true;                            // this walker has not seen a token yet: no reference
-  auto score_stage = [&](int blk, int it, bool first, const KeyRegs& K, int bad, auto partial_tag) -> bool {
+  // (always inlined: an outlined stage would pass the block's page data through memory)
+  auto score_stage = [&](int blk, int it, bool first, const KeyRegs& K, int bad, auto partial_tag)
+                         __attribute__((always_inline)) -> bool {
     constexpr bool PARTIAL = decltype(partial_tag)::value;
     float s2[NJ][NPG];
     float mref[NJ];                             // only one wavefront of a pair subtracts it
@@ -577,6 +595,58 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
     // stage): the SIMD's other wavefront then fills the gaps with its vector-ALU work instead of
     // both alternating between the two kinds of instruction.
     __builtin_amdgcn_s_setprio(1);
+    if constexpr (QL) {
+      f32x4 dmp[NPG], dqp[NPG];
+#pragma unroll
+      for (int pg = 0; pg < NPG; ++pg) { dmp[pg] = cm; dqp[pg] = cq; }
+#pragma unroll
+      for (int i = 0; i < WPL; ++i) {
+#pragma unroll
+        for (int tp = 0; tp < NTP; ++tp) {
+          i32x8 a[NRS];
+#pragma unroll
+          for (int rs = 0; rs < NRS; ++rs) {
+            const uint32_t* p6 = qa_lds + ((tp * WPLT + hf * WPL + i) * 2 + rs) * (64 * 8) + qa_lane;
+            const u32x4 lo = *(const u32x4*)p6;
+            const uint32_t d4 = p6[4], d5 = p6[5];
+            a[rs] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)d4, (int)d5, 0, 0};
+          }
+#pragma unroll
+          for (int pg = 0; pg < NPG; ++pg) {
+            uint32_t x;
+            if (tp < MB) x = K.key[pg][i * (MB + 1) + tp];
+            else if (tp == NTP - 1) x = K.key[pg][i * (MB + 1) + MB];
+            else {
+              x = 0;
+#pragma unroll
+              for (int p = 0; p < MB; ++p) x ^= ((xplanes[tp - MB] >> p) & 1) ? K.key[pg][i * (MB + 1) + p] : 0u;
+            }
+            const uint32_t b0 = x & nib, b1 = x & nib1, b2 = x & nib2, b3 = (x >> 3) & nib;
+            if (tp == NTP - 1) {
+              dqp[pg] = mfma_f8f4<2>(a[0], b0, b1, b2, b3, dqp[pg], sa, sb);
+              if (!NR) dqp[pg] = mfma_f8f4<3>(a[NRS - 1], b0, b1, b2, b3, dqp[pg], sa, sb);
+            } else {
+              dmp[pg] = mfma_f8f4<0>(a[0], b0, b1, b2, b3, dmp[pg], sa, sb);
+              if (!NR) dmp[pg] = mfma_f8f4<1>(a[NRS - 1], b0, b1, b2, b3, dmp[pg], sa, sb);
+            }
+          }
+          // (the next plane's operands are not to be read before this plane is done: all nine at once do not fit)
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+#pragma unroll
+      for (int pg = 0; pg < NPG; ++pg) {
+        const f32x4 dm = dmp[pg], dq = dqp[pg];
+        const float nk = K.meta[pg][0], rk = K.meta[pg][1];
+        if (NR) {
+          s2[0][pg] = fmaf(nk, (dm[0] + dm[1]) + (dm[2] + dm[3]), fmaf(rk, (dq[0] + dq[1]) + (dq[2] + dq[3]), -mref[0]));
+        } else {
+#pragma unroll
+          for (int j = 0; j < NJ; ++j)
+            s2[j][pg] = fmaf(nk, dm[2 * j] + dm[2 * j + 1], fmaf(rk, dq[2 * j] + dq[2 * j + 1], -mref[j]));
+        }
+      }
+    } else {
 #pragma unroll
     for (int pg = 0; pg < NPG; ++pg) {
       f32x4 dm = cm, dq = cq;
@@ -620,6 +690,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
     for (int k = 0; k < NPG * NRS * NTP * WPL; ++k) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+    }
     }
     __builtin_amdgcn_s_setprio(0);
     if constexpr (DS > 1) {
@@ -701,7 +772,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
     return rescale;
   };
   // weights x (codes, scales, zeros) of block blk into the accumulators
-  auto value_stage = [&](int blk, const ValRegs& V, bool rescale, int bad, auto partial_tag) {
+  auto value_stage = [&](int blk, const ValRegs& V, bool rescale, int bad, auto partial_tag) __attribute__((always_inline)) {
     constexpr bool PARTIAL = decltype(partial_tag)::value;
     // scales -> LDS as fp32 [page][group][16 tokens]; first use of the value loads.  The lane that
     // holds a 16-byte piece widens it once (instead of all 16 row lanes later), folds in the
@@ -857,11 +928,11 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
       }
     }
     // CHECKED: page ids are validated and every trip takes the masking (PARTIAL) path
-    auto run = [&](auto checked_tag) {
+    auto run = [&](auto checked_tag) __attribute__((always_inline)) {
       constexpr bool CHECKED = decltype(checked_tag)::value;
       // one trip of a walker that still has a block; PARTIAL: some tokens of the block may not exist
       // LAST: the walker's last trip (a code instance of its own behind the loop): nothing is requested
-      auto trip = [&](int it, auto partial_tag, auto last_tag) {
+      auto trip = [&](int it, auto partial_tag, auto last_tag) __attribute__((always_inline)) {
         constexpr bool LAST = decltype(last_tag)::value;
         // the block after this walker's last one does not exist: re-request the current one instead,
         // so that the loads stay outside any branch
@@ -1142,6 +1213,9 @@ static int launch_one(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, 
   size_t merge = (size_t)(NW / DS * G * (D + 2) + NW * 16 * 16) * sizeof(float);
   if (SG) per_wave += stage_bytes((D / DS / 16) * VB / 2);
   size_t smem = per_wave * NW > merge ? per_wave * NW : merge;
+  // four index planes: the group's packed query operands in LDS, behind the wavefronts' regions
+  if (MB >= 4) smem = per_wave * NW + (size_t)(MB + NX + 1) * ((D + 127) / 128) * 2 * 64 * 8 * sizeof(uint32_t);
+  if (MB >= 4 && smem < merge) smem = merge;
   if (D == 64 && !PP && decode_mfma_head_rows(D, G) == 4)
     return launch_one<D, MB, NX, VB, GS, DS, WPS, F16P, D == 64>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,
                                                                  bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts,
