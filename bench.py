@@ -481,7 +481,8 @@ def cpu_quantize_baseline(k, v, tq, sample_tokens=32768):
 
 # (sequences, context, query heads, KV heads, head_dim, key bits, value bits): every family of decode kernels -
 # head_dim 64 / 128 / 256 on the matrix cores with 2- / 3- / 4-bit keys and 2- / 4- / 8-bit values, 1 to 16 query
-# heads per KV head (11 as 6 + 5), short and long contexts - and the general kernel's shapes (head_dim 576, 5-bit keys)
+# heads per KV head (11 as 6 + 5), 5-bit keys at head_dim 128, short and long contexts - and the general kernel's shape
+# (head_dim 576)
 SHAPE_TABLE = [
     (4, 131072, 16, 2, 256, 3, 2), (4, 131072, 16, 2, 256, 2, 2), (4, 131072, 16, 2, 256, 4, 2),
     (4, 131072, 16, 2, 256, 3, 4), (4, 131072, 8, 2, 256, 3, 2), (4, 131072, 2, 2, 256, 3, 2),
@@ -492,7 +493,8 @@ SHAPE_TABLE = [
     (1, 131072, 32, 8, 128, 3, 4),
     (16, 8192, 32, 8, 64, 3, 4), (16, 8192, 32, 8, 64, 2, 2), (16, 8192, 32, 8, 64, 4, 4), (16, 8192, 64, 8, 64, 3, 4),
     (32, 32768, 32, 8, 64, 3, 4),
-    (16, 8192, 8, 1, 576, 4, 4), (16, 8192, 32, 8, 128, 5, 4), (16, 8192, 32, 8, 128, 3, 8), (16, 8192, 88, 8, 128, 3, 4),
+    (16, 8192, 8, 1, 576, 4, 4), (16, 8192, 32, 8, 128, 5, 4), (16, 8192, 64, 8, 128, 5, 4), (16, 8192, 32, 8, 128, 3, 8),
+    (16, 8192, 88, 8, 128, 3, 4),
 ]
 
 

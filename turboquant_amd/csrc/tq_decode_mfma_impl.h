@@ -307,6 +307,10 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   // SG: this wavefront's staging area behind the wavefronts' private regions
   // QL: the group's packed query operands behind the wavefronts' private regions
   uint32_t* qa_lds = (uint32_t*)(smem_raw + MF_WAVES * WAVE_LDS_FLOATS * sizeof(float));
+  // QL: behind the operands, the constant parts of the scores of the heads a lane sees (the same for every wavefront;
+  // indexed like the operands, so that the reads share their address register):
+  // [64 operand slots][index part of head 0, 1, sign part of head 0, 1]
+  float* c_lds = (float*)(qa_lds + (MB + NX + 1) * WPLT * 2 * (64 * 6));
   unsigned char* stage = smem_raw + MF_WAVES * WAVE_LDS_FLOATS * sizeof(float) + wave * STAGE_BYTES;
   unsigned char* stage_m = stage + 4 * 1024;
   unsigned char* stage_v = stage_m + 512;
@@ -319,7 +323,10 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   // lane are stored at a stride of eight.
   i32x8 qa[QL ? 1 : NTP][WPL][NRS];
   int sa = 0;
-  int qa_lane = 0;                             // QL: dword offset of this lane's slot inside an operand of 64 slots
+  // QL: an operand in LDS is [64 lanes][4 dwords] followed by [64 lanes][2 dwords] (QA_OP dwords), so that both reads of
+  // a lane, 16 and 8 bytes, are contiguous across the lanes; qa_lane = this lane's slot, qa_sel = (NR) its row set's operand
+  constexpr int QA_OP = 64 * 6;
+  int qa_lane = 0, qa_sel = 0;
   f32x4 cm = {0, 0, 0, 0}, cq = {0, 0, 0, 0};
   auto load_operands = [&]() {
   {
@@ -332,9 +339,15 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
     if constexpr (QL) {
       // the whole block of the group, 16 bytes per lane and step, as it lies in memory
       const uint32_t* blk = qa_pack + ((int64_t)b * Hkv + h) * (NTP * WPLT * 2 * 64 * 8);
-      for (int o = tid * 4; o < NTP * WPLT * 2 * 64 * 8; o += MF_WAVES * 64 * 4)
-        *(u32x4*)(qa_lds + o) = *(const u32x4*)(blk + o);
-      qa_lane = slane * 8 + (NR ? ((n >> 1) & 1) * (64 * 8) : 0);
+      for (int o = tid; o < NTP * WPLT * 2 * 64 * 2; o += MF_WAVES * 64) {       // o: 16-byte piece, two per lane slot
+        const u32x4 v = *(const u32x4*)(blk + o * 4);
+        uint32_t* op = qa_lds + (o >> 7) * QA_OP;
+        const int sl = (o >> 1) & 63;
+        if (o & 1) *(uint2*)(op + 64 * 4 + sl * 2) = make_uint2(v[0], v[1]);
+        else *(u32x4*)(op + sl * 4) = v;
+      }
+      qa_lane = slane;
+      qa_sel = NR ? ((n >> 1) & 1) * QA_OP : 0;
       __syncthreads();
     } else
 #pragma unroll
@@ -375,6 +388,10 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
     const float c2 = q_stat[qrow * 4 + 2], c3 = q_stat[qrow * 4 + 3];
     cm[2 * j] = live ? c2 : 0.0f;
     cq[2 * j] = live ? c3 : 0.0f;
+    if (QL) {                                     // (lanes that share an operand slot see the same heads)
+      c_lds[qa_lane * 4 + j] = live ? c2 : 0.0f;
+      c_lds[qa_lane * 4 + 2 + j] = live ? c3 : 0.0f;
+    }
   }
   };
   load_operands();
@@ -598,7 +615,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
     if constexpr (QL) {
       f32x4 dmp[NPG], dqp[NPG];
 #pragma unroll
-      for (int pg = 0; pg < NPG; ++pg) { dmp[pg] = cm; dqp[pg] = cq; }
+      for (int pg = 0; pg < NPG; ++pg) { dmp[pg] = f32x4{0, 0, 0, 0}; dqp[pg] = f32x4{0, 0, 0, 0}; }
 #pragma unroll
       for (int i = 0; i < WPL; ++i) {
 #pragma unroll
@@ -606,10 +623,10 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
           i32x8 a[NRS];
 #pragma unroll
           for (int rs = 0; rs < NRS; ++rs) {
-            const uint32_t* p6 = qa_lds + ((tp * WPLT + hf * WPL + i) * 2 + rs) * (64 * 8) + qa_lane;
-            const u32x4 lo = *(const u32x4*)p6;
-            const uint32_t d4 = p6[4], d5 = p6[5];
-            a[rs] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)d4, (int)d5, 0, 0};
+            const uint32_t* op = qa_lds + ((tp * WPLT + hf * WPL + i) * 2 + rs) * QA_OP + qa_sel;
+            const u32x4 lo = *(const u32x4*)(op + qa_lane * 4);
+            const uint2 hi = *(const uint2*)(op + 64 * 4 + qa_lane * 2);
+            a[rs] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi.x, (int)hi.y, 0, 0};
           }
 #pragma unroll
           for (int pg = 0; pg < NPG; ++pg) {
@@ -634,16 +651,22 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
           __builtin_amdgcn_sched_barrier(0);
         }
       }
+      // The constant parts of the scores are added here, from LDS.  As initial accumulators they would sit in eight
+      // registers through the whole loop, the register allocator would keep them in scratch memory instead, and a
+      // reload from scratch inside the loop is the worst there is: vector memory instructions return in order, so
+      // waiting for it means waiting for the page data requested just before, which has the whole stage to arrive.
+      const f32x4 cc = *(const f32x4*)(c_lds + qa_lane * 4);
 #pragma unroll
       for (int pg = 0; pg < NPG; ++pg) {
         const f32x4 dm = dmp[pg], dq = dqp[pg];
         const float nk = K.meta[pg][0], rk = K.meta[pg][1];
         if (NR) {
-          s2[0][pg] = fmaf(nk, (dm[0] + dm[1]) + (dm[2] + dm[3]), fmaf(rk, (dq[0] + dq[1]) + (dq[2] + dq[3]), -mref[0]));
+          s2[0][pg] = fmaf(nk, ((dm[0] + cc[0]) + dm[1]) + (dm[2] + dm[3]),
+                           fmaf(rk, ((dq[0] + cc[2]) + dq[1]) + (dq[2] + dq[3]), -mref[0]));
         } else {
 #pragma unroll
           for (int j = 0; j < NJ; ++j)
-            s2[j][pg] = fmaf(nk, dm[2 * j] + dm[2 * j + 1], fmaf(rk, dq[2 * j] + dq[2 * j + 1], -mref[j]));
+            s2[j][pg] = fmaf(nk, (dm[2 * j] + cc[j]) + dm[2 * j + 1], fmaf(rk, (dq[2 * j] + cc[2 + j]) + dq[2 * j + 1], -mref[j]));
         }
       }
     } else {
@@ -1214,7 +1237,8 @@ static int launch_one(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, 
   if (SG) per_wave += stage_bytes((D / DS / 16) * VB / 2);
   size_t smem = per_wave * NW > merge ? per_wave * NW : merge;
   // four index planes: the group's packed query operands in LDS, behind the wavefronts' regions
-  if (MB >= 4) smem = per_wave * NW + (size_t)(MB + NX + 1) * ((D + 127) / 128) * 2 * 64 * 8 * sizeof(uint32_t);
+  if (MB >= 4)
+    smem = per_wave * NW + (size_t)(MB + NX + 1) * ((D + 127) / 128) * 2 * 64 * 6 * sizeof(uint32_t) + (size_t)64 * 4 * sizeof(float);
   if (MB >= 4 && smem < merge) smem = merge;
   if (D == 64 && !PP && decode_mfma_head_rows(D, G) == 4)
     return launch_one<D, MB, NX, VB, GS, DS, WPS, F16P, D == 64>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,
