@@ -356,6 +356,10 @@ void tq_time_next_key_kernel(void *start_event, void *stop_event);
  *   "wide_workgroups"  1 (default): at head_dim 64 / 128, with an even split count and at most 16 blocks of 64 tokens
  *                      per wavefront (judged by the width of the block table), a step runs workgroups of 8
  *                      wavefronts on half the split count it was given; 0: always 4 wavefronts per workgroup.
+ *   "sequence_per_wave" -1 (default), 0 or a count: at head_dim 64 / 128 a step with a single context split and at
+ *                      least this many (sequence, group of query heads) pairs - -1: eight per compute unit, 0: never -
+ *                      gives every wavefront of a workgroup a pair of its own, walked from the first block to the last,
+ *                      instead of four wavefronts sharing one (a quarter of the workgroups, no walkers to merge).
  *   "split_skew"       0..8, default 1: at head_dim 256, when a launch of 4-wavefront workgroups fills (nearly) every
  *                      compute unit twice and the split count is even, the workgroups of the first half of the grid
  *                      (dispatched first, served first by their SIMDs) take the even splits and this many sixteenths

@@ -317,6 +317,9 @@ def test_decode_gives_no_weight_to_pages_outside_the_pool(gpu, d, key_bits, vb, 
 
 
 # ------------------------------------------------------------------ query preparation for every query dtype
+_OPTION_DEFAULTS = {"sequence_per_wave": -1}     # every other option: 1
+
+
 def _set_option(name, value):
     from turboquant_amd import _ffi
     _ffi.check(_ffi.lib().tq_set_option(name.encode(), int(value)), "tq_set_option")
@@ -485,7 +488,7 @@ def _variant_against_default(gpu, option, d, key_bits, vb, Hq, Hkv, dtype, exact
                                       lens[b], prm, Hkv, None, None)
             assert cosine(out[b:b + 1], want) >= COS_GATE, b
     finally:
-        _set_option(option, 1)
+        _set_option(option, _OPTION_DEFAULTS.get(option, 1))
         _set_option("wide_workgroups", 1)
 
 
@@ -588,6 +591,70 @@ def test_five_bit_keys_with_the_query_operands_in_lds(gpu, option, vb, Hq, Hkv, 
     poisoned block table and 1 - 11 context splits against the oracle (score.py:84-173), with each of the merge,
     row-count and workgroup-width variants on and off."""
     _variant_against_default(gpu, option, 128, 5, vb, Hq, Hkv, dtype, exact=False, rel=2.0 ** -8)
+
+
+@pytest.mark.parametrize("d,key_bits,vb,Hq,Hkv,dtype", [(128, 3, 4, 8, 2, torch.bfloat16), (128, 3, 4, 16, 2, torch.bfloat16),
+                                                        (128, 4, 2, 3, 1, torch.float16), (64, 3, 4, 4, 1, torch.bfloat16),
+                                                        (64, 3, 2, 16, 2, torch.float16), (128, 3, 4, 22, 2, torch.bfloat16),
+                                                        (128, 3, 8, 5, 1, torch.bfloat16), (128, 2, 2, 7, 1, torch.bfloat16)])
+def test_a_sequence_per_wavefront(gpu, d, key_bits, vb, Hq, Hkv, dtype):
+    """Many short sequences in one split: every wavefront of a page-kernel workgroup walks a (sequence, group of
+    heads) of its own (run-time option "sequence_per_wave": from how many pairs on; 1 = always, 0 = never) instead of
+    four wavefronts sharing one.  Five sequences - so that the last workgroup has wavefronts without a pair - of
+    ragged and zero length, a poisoned block table, head groups of unequal size (22 heads on 2 KV heads: 6 + 5), all
+    three endings of the step (output written by the page kernel, partials for the merge kernel, an exact tail's
+    partial merged in) against the four-wavefront form and the oracle (score.py:84-173)."""
+    lens = [700, 0, 16 * 9 + 1, 64, 333]
+    B = len(lens)
+    g = torch.Generator().manual_seed(d + Hq + key_bits)
+    pages = (max(lens) + 15) // 16
+    pool, tq = _make_pool(gpu, d, key_bits, vb, Hkv, B * pages + 1, dtype, seed=43)
+    table = torch.randperm(B * pages + 1, generator=g)[: B * pages].to(torch.int32).view(B, pages)
+    k = torch.randn(B, max(lens), Hkv, d, generator=g).to(dtype).to(gpu)
+    v = torch.randn(B, max(lens), Hkv, d, generator=g).to(dtype).to(gpu)
+    pool.append(k, v, table.to(gpu))
+    seq = torch.tensor(lens, dtype=torch.int32, device=gpu)
+    q = torch.randn(B, Hq, d, generator=g).to(dtype)
+    bad = table.clone()
+    bad[0, [3, 8, 20]] = torch.tensor([B * pages + 1, -1, 2 ** 31 - 1], dtype=torch.int32)
+    R = 24
+    rk = torch.randn(B, R, Hkv, d, generator=g).to(dtype).to(gpu)
+    rv = torch.randn(B, R, Hkv, d, generator=g).to(dtype).to(gpu)
+    rl = torch.tensor([R, 3, 0, R, 11], dtype=torch.int32, device=gpu)
+    _progress(f"a sequence per wavefront d={d} kb={key_bits} vb={vb} Hq={Hq} Hkv={Hkv} {dtype}")
+
+    def runs():
+        outs = []
+        for tab in (table, bad):
+            for merge_in_kernel in (1, 0):
+                _set_option("merge_in_kernel", merge_in_kernel)
+                ws = pool.workspace(B, Hq, 1)
+                ws.view(torch.uint8).fill_(0xFF)
+                outs.append(pool.decode_attention(q.to(gpu), tab.to(gpu), seq, n_split=1, workspace=ws).float().cpu())
+            outs.append(pool.decode_attention(q.to(gpu), tab.to(gpu), seq, recent_k=rk, recent_v=rv, recent_len=rl,
+                                              n_split=1).float().cpu())
+        torch.cuda.synchronize()
+        return outs
+
+    try:
+        _set_option("sequence_per_wave", 0)
+        want = runs()
+        _set_option("sequence_per_wave", 1)
+        got = runs()
+    finally:
+        _set_option("sequence_per_wave", -1)
+        _set_option("merge_in_kernel", 1)
+    for i, (a, b_) in enumerate(zip(got, want)):
+        assert torch.isfinite(a).all(), i
+        assert (a - b_).abs().max() <= 2 ** -7 * b_.abs().max() + 1e-6, i        # one bf16 step of the largest value
+    prm = params_of(tq)
+    for b in range(B):
+        if lens[b] == 0:
+            assert torch.count_nonzero(got[0][b]) == 0
+            continue
+        kc, vc = _store_from_oracle_view(pool, table[b].to(gpu), lens[b])
+        ref = O.hybrid_attention(q[b:b + 1], kc, vc, max(lens[b], O.MIN_HISTORY), prm, Hkv, None, None)
+        assert cosine(got[0][b:b + 1], ref) >= COS_GATE, b
 
 
 @pytest.mark.parametrize("B,Hq,Hkv,d,key_bits,vb,dtype", [(201, 4, 1, 128, 3, 4, torch.bfloat16), (201, 2, 1, 128, 4, 2, torch.bfloat16),

@@ -89,13 +89,24 @@ bool decode_mfma_has_kernel(const tq_layer& ly, const tq_page_layout& L) {
   return false;
 }
 
-// the launchers of the three head sizes (tq_decode_mfma_d64 / _d128 / _d256.hip)
+// the launchers of the three head sizes (tq_decode_mfma_d64 / _d128 / _d256.hip; head_dim 64 / 128: bf16 and fp16
+// pools in units of their own, _f16)
 int launch_decode_mfma_d64(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, int kv_div,
                        const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
                        float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts,
                        int n_split, int len_sub, int max_pages, int num_pages, const FusedMerge& fm,
                        bool wide_wg, hipStream_t st);
 int launch_decode_mfma_d128(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, int kv_div,
+                       const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
+                       float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts,
+                       int n_split, int len_sub, int max_pages, int num_pages, const FusedMerge& fm,
+                       bool wide_wg, hipStream_t st);
+int launch_decode_mfma_d64_f16(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, int kv_div,
+                       const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
+                       float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts,
+                       int n_split, int len_sub, int max_pages, int num_pages, const FusedMerge& fm,
+                       bool wide_wg, hipStream_t st);
+int launch_decode_mfma_d128_f16(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, int kv_div,
                        const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
                        float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts,
                        int n_split, int len_sub, int max_pages, int num_pages, const FusedMerge& fm,
@@ -115,8 +126,14 @@ int launch_decode_mfma(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv,
                        bool wide_wg, hipStream_t st) {
   const int G = kv_div > 1 ? (Hq / (Hkv / kv_div) + kv_div - 1) / kv_div : Hq / Hkv, d = ly.d;
   if (G > 8 || (L.dtype != TQ_BF16 && L.dtype != TQ_F16) || !L.key_lane_major) return TQ_EUNSUPPORTED;
+  if (d == 64 && L.dtype == TQ_F16)
+    return launch_decode_mfma_d64_f16(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table, bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts,
+                                      n_split, len_sub, max_pages, num_pages, fm, wide_wg, st);
   if (d == 64) return launch_decode_mfma_d64(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table, bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts, n_split,
                                    len_sub, max_pages, num_pages, fm, wide_wg, st);
+  if (d == 128 && L.dtype == TQ_F16)
+    return launch_decode_mfma_d128_f16(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table, bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts,
+                                       n_split, len_sub, max_pages, num_pages, fm, wide_wg, st);
   if (d == 128) return launch_decode_mfma_d128(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table, bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts, n_split,
                                    len_sub, max_pages, num_pages, fm, wide_wg, st);
   if (d == 256) return launch_decode_mfma_d256(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table, bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts, n_split,

@@ -1,5 +1,6 @@
-// Instantiations of the matrix-core page kernel for head_dim 64 (see tq_decode_mfma_impl.h).
+// Instantiations of the matrix-core page kernel for head_dim 64, bf16 pools (see tq_decode_mfma_impl.h).
 
+#define TQ_POOL_F16 0
 #include "tq_decode_mfma_impl.h"
 
 namespace tq {

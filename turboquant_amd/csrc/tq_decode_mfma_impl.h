@@ -227,7 +227,11 @@ __device__ __forceinline__ constexpr int v_bitpos(int t) {
 // and no register holds data in flight.
 // NW: wavefronts per workgroup, 4 (two workgroups per compute unit) or 8 (one): with few blocks per
 // wavefront the larger workgroup wins - half as many workgroups to dispatch, prologues and partials.
-template <int D, int MB, int NX, int VB, int GS, int DS, int WPS, bool F16P, bool PP, bool NR, bool SG, int NW>
+// IW (many short sequences, one split): every wavefront of a workgroup walks a (sequence, group of heads) of its own
+// from the first block to the last, instead of the workgroup's wavefronts sharing one.  A wavefront then makes four
+// times the trips after one prologue, a launch has a quarter of the workgroups (256 sequences x 8 KV heads: one
+// resident round instead of four), and the epilogue has no walkers to merge.  The grid is (1, ceil(items / 4), 1).
+template <int D, int MB, int NX, int VB, int GS, int DS, int WPS, bool F16P, bool PP, bool NR, bool SG, int NW, bool IW>
 __global__ void __launch_bounds__(NW * 64, WPS)
 decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div,
                    const uint8_t* __restrict__ pool, const int32_t* __restrict__ block_table,
@@ -260,6 +264,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   // by plane so that an operand is read once for its four pages.
   constexpr bool QL = MB >= 4;
   static_assert(!QL || (!PP && !SG && DS == 1), "operands in LDS: head_dim 128, page data in registers");
+  static_assert(!IW || (DS == 1 && !QL), "a (sequence, head group) per wavefront: wavefronts that work alone, operands in registers");
   constexpr int NJ = NR ? 1 : 2;              // heads a lane sees in the score MFMA's output
   // Hkv counts query-head groups: a KV head with more than 8 query heads is served by kv_div groups of at most 8
   // heads each (consecutive groups read the same pages); when the heads do not divide evenly the last group of
@@ -271,10 +276,21 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   // to a compute unit, and a SIMD serves its older wavefronts first: with equal shares the first half of the grid
   // finishes early and the second half runs on alone.
   int split = blockIdx.x, b = blockIdx.z;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wgrp = wave / DS, hf = wave % DS; // block walker this wavefront belongs to; its share of the head
   // The groups of a KV head are (splits x KV heads) workgroups apart in the grid, not next to each other: workgroups
   // go to the card's eight dies in turn, each die has its own L2, and a distance that is a multiple of eight puts the
   // groups that read the same pages at the same time on the same die.
   int h = blockIdx.y, qbase;
+  bool item_live = true;                        // IW: this wavefront has a (sequence, head group) of its own
+  if constexpr (IW) {
+    const int item = blockIdx.y * (NW / DS) + wgrp, items = Hkv * n_seq;
+    item_live = item < items;
+    const int item_c = item_live ? item : items - 1;          // (a wavefront without an item repeats the last one and stores nothing)
+    h = item_c % Hkv;
+    b = item_c / Hkv;
+  }
   if (kv_div > 1) {
     const int kv_heads = Hkv / kv_div, grp = h / kv_heads, kvh = h - grp * kv_heads;
     const int g_tot = Hq / kv_heads, g_max = (g_tot + kv_div - 1) / kv_div;
@@ -291,9 +307,6 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
     b -= late ? n_seq : 0;
     split = 2 * split + late;
   }
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wgrp = wave / DS, hf = wave % DS; // block walker this wavefront belongs to; its share of the head
   const int n = lane & 15, kb = lane >> 4;    // score stage: token / coordinate quarter; value stage: row / page
   TQ_STAMP(0);
 
@@ -422,7 +435,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   TQ_STAMP(1);
   // ---------------------------------------------------------------- work range (all scalar)
   // len_sub: newest tokens that are attended to exactly.  A length beyond the block table is cut to the table.
-  const int seq_len = max(min(seq_lens[b], max_pages * TQ_PAGE_TOKENS) - len_sub, 0);
+  const int seq_len = item_live ? max(min(seq_lens[b], max_pages * TQ_PAGE_TOKENS) - len_sub, 0) : 0;
   const int n_pages = (seq_len + TQ_PAGE_TOKENS - 1) / TQ_PAGE_TOKENS;
   int blk_begin, blk_end;
   decode_block_range(seq_len, n_split, split, DS == 2 ? skew16 : 0, NGRP, blk_begin, blk_end);
@@ -919,8 +932,9 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
     KeyRegs K;
     ValRegs V;
     int pid[4];
-    const int trips = (max(blk_end - blk_begin, 0) + NGRP - 1) / NGRP;
-    int blk = blk_begin + wgrp;
+    constexpr int WSTEP = IW ? 1 : NGRP;                   // distance of a walker's consecutive blocks
+    const int trips = (max(blk_end - blk_begin, 0) + WSTEP - 1) / WSTEP;
+    int blk = blk_begin + (IW ? 0 : wgrp);
     int bad = 0;                                          // pages of the current block that lie outside the pool
     if (blk < blk_end) {
       bad = page_ids(blk, pid, std::true_type{});
@@ -959,7 +973,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
         constexpr bool LAST = decltype(last_tag)::value;
         // the block after this walker's last one does not exist: re-request the current one instead,
         // so that the loads stay outside any branch
-        const int nxt = blk + NGRP;
+        const int nxt = blk + WSTEP;
         const int nxt_c = nxt < blk_end ? nxt : blk;
         int pid_n[4] = {0, 0, 0, 0};
         int bad_n = 0;
@@ -1020,7 +1034,8 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   if (SG) stage_wait<0>();   // the last trip's requests (a repeat of its own block) have landed
   __syncthreads();      // every wave is done with its private LDS region
   TQ_STAMP(6);
-  float* s_z = s_red + NGRP * G * (D + 2);                     // [MF_WAVES][16 rows][16 groups]
+  const int g_rows = IW ? 8 : G;                               // rows of a walker in s_red (IW: the walkers' groups may differ in size)
+  float* s_z = s_red + NGRP * g_rows * (D + 2);                // [MF_WAVES][16 rows][16 groups]
 #pragma unroll
   for (int i = 0; i < 4; ++i) s_z[(wave * 16 + 4 * kb + i) * 16 + n] = zacc[i];
   if (hf == 0) {                                               // the wavefronts of a pair hold the same (m, l)
@@ -1030,7 +1045,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
       if (PP) lsum = sum_xor32(lsum);
       const int g = PP ? 2 * (kb & 1) + j : (NR ? kb : 2 * kb + j);
       if (n == 0 && g < G && (!PP || kb < 2)) {
-        float* r = s_red + (wgrp * G + g) * (D + 2);
+        float* r = s_red + (wgrp * g_rows + g) * (D + 2);
         r[0] = m_run[j] * 0.6931471805599453f;     // back to the natural-log domain of the partials
         r[1] = lsum;
       }
@@ -1053,7 +1068,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
     for (int i = 0; i < 4; ++i) {
       const int g = 4 * (kb & 1) + i;
       if (g < G) {
-        float* row = s_red + (wgrp * G + g) * (D + 2) + 2 + hf * DW + par * (16 * CTG) + n;
+        float* row = s_red + (wgrp * g_rows + g) * (D + 2) + 2 + hf * DW + par * (16 * CTG) + n;
 #pragma unroll
         for (int gpi = 0; gpi < NG / 2; ++gpi)
 #pragma unroll
@@ -1066,6 +1081,47 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   }
   __syncthreads();
   TQ_STAMP(7);
+  if constexpr (IW) {
+    // Every wavefront finishes the (sequence, head group) it walked alone: its rows of s_red are the result.
+    if (fm.out != nullptr && fm.n_extra <= 1) {
+      // the attention output, merged with the exact tail's partial if there is one (an earlier launch wrote it)
+#pragma unroll
+      for (int k = 0; k < 8 * D / 64; ++k) {
+        const int o = lane + k * 64;
+        const int g_o = o / D, ch = o % D;
+        const bool live = item_live && g_o < G;
+        const int g = live ? g_o : 0;
+        const float* r = s_red + (wgrp * g_rows + g) * (D + 2);
+        const float mm = r[0], ll = r[1], aa = r[2 + ch];
+        if (live && fm.n_extra == 0) {
+          const float inv = ll > 0.0f ? 1.0f / ll : 0.0f;
+          store_from_f32(fm.out, ((int64_t)b * Hq + qbase + g) * D + ch, aa * inv, fm.out_dtype);
+        } else if (live) {
+          const float* x = parts + (((int64_t)b * Hq + qbase + g) * n_parts + 1) * (D + 2);     // the exact tail's part
+          const float m_x = x[0], l_x = x[1], a_x = x[2 + ch];
+          float top = MF_NEG;
+          if (ll > 0.0f) top = fmaxf(top, mm);
+          if (l_x > 0.0f) top = fmaxf(top, m_x);
+          const float w0 = ll > 0.0f ? __expf(mm - top) : 0.0f, w1 = l_x > 0.0f ? __expf(m_x - top) : 0.0f;
+          const float l_all = fmaf(w1, l_x, fmaf(w0, ll, 0.0f)), a_all = fmaf(w1, a_x, fmaf(w0, aa, 0.0f));
+          const float inv = l_all > 0.0f ? 1.0f / l_all : 0.0f;
+          store_from_f32(fm.out, ((int64_t)b * Hq + qbase + g) * D + ch, a_all * inv, fm.out_dtype);
+        }
+      }
+    } else {
+      // the partial (m, l, acc[D]) of every head, for the merge kernel
+      constexpr int PAIRS = (D + 2) / 2;
+      for (int o = lane; o < 8 * PAIRS; o += 64) {
+        const int g = o / PAIRS, pr = o % PAIRS;
+        if (item_live && g < G) {
+          const float* r = s_red + (wgrp * g_rows + g) * (D + 2);
+          float* out = parts + (((int64_t)b * Hq + qbase + g) * n_parts + split) * (D + 2);
+          store_coherent2(out + 2 * pr, f32x2{r[2 * pr], r[2 * pr + 1]});
+        }
+      }
+    }
+    return;
+  }
   // merge of the walkers: thread -> (head, channel); loads are unconditional (clamped), stores guarded
   auto walkers_sum = [&](int g, int ch, float& mm, float& ll, float& aa) {
     float m_w[NGRP], l_w[NGRP], a_w[NGRP];
@@ -1224,7 +1280,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
 }
 
 template <int D, int MB, int NX, int VB, int GS, int DS, int WPS, bool F16P, bool PP = false, bool NR = false, bool SG = false,
-          int NW = MF_WAVES>
+          int NW = MF_WAVES, bool IW = false>
 static int launch_one(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, int kv_div,
                       const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
                       float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts, int n_split,
@@ -1233,7 +1289,7 @@ static int launch_one(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, 
   // (heads of the largest group of a KV head; kv_div groups share a KV head's heads, the last one may have fewer)
   const int G = kv_div > 1 ? (Hq / (Hkv / kv_div) + kv_div - 1) / kv_div : Hq / Hkv;
   size_t per_wave = (size_t)wave_lds_floats(D / DS / GS, DS) * sizeof(float);
-  size_t merge = (size_t)(NW / DS * G * (D + 2) + NW * 16 * 16) * sizeof(float);
+  size_t merge = (size_t)(NW / DS * (IW ? 8 : G) * (D + 2) + NW * 16 * 16) * sizeof(float);
   if (SG) per_wave += stage_bytes((D / DS / 16) * VB / 2);
   size_t smem = per_wave * NW > merge ? per_wave * NW : merge;
   // four index planes: the group's packed query operands in LDS, behind the wavefronts' regions
@@ -1241,11 +1297,11 @@ static int launch_one(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, 
     smem = per_wave * NW + (size_t)(MB + NX + 1) * ((D + 127) / 128) * 2 * 64 * 6 * sizeof(uint32_t) + (size_t)64 * 4 * sizeof(float);
   if (MB >= 4 && smem < merge) smem = merge;
   if (D == 64 && !PP && decode_mfma_head_rows(D, G) == 4)
-    return launch_one<D, MB, NX, VB, GS, DS, WPS, F16P, D == 64>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,
+    return launch_one<D, MB, NX, VB, GS, DS, WPS, F16P, D == 64, false, false, MF_WAVES, IW>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,
                                                                  bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts,
                                                                  n_split, len_sub, max_pages, num_pages, fm, wide_wg, st);
   if (D >= 128 && !NR && decode_mfma_head_rows(D, G) == 4)
-    return launch_one<D, MB, NX, VB, GS, DS, WPS, F16P, false, D >= 128>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,
+    return launch_one<D, MB, NX, VB, GS, DS, WPS, F16P, false, D >= 128, false, MF_WAVES, IW>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,
                                                                          bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts,
                                                                          n_split, len_sub, max_pages, num_pages, fm, wide_wg, st);
   // Three index planes (4-bit keys) at head_dim 128 / 256: always the variant that stages the next block's page data in
@@ -1253,12 +1309,25 @@ static int launch_one(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, 
   // register variant is not built; for fewer planes the staged variant measured 2 - 5 % slower and is not built either.
   constexpr bool can_stage = D >= 128 && MB == 3;
   if constexpr (can_stage && !SG) {
-    return launch_one<D, MB, NX, VB, GS, DS, WPS, F16P, PP, NR, true>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,
+    return launch_one<D, MB, NX, VB, GS, DS, WPS, F16P, PP, NR, true, MF_WAVES, IW>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,
                                                                       bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts,
                                                                       n_split, len_sub, max_pages, num_pages, fm, wide_wg, st);
   } else {
   // eight wavefronts per workgroup (one workgroup per compute unit) for the kernels whose wavefronts work alone
-  constexpr bool can_widen = DS == 1 && NW == MF_WAVES;
+  // Many short sequences in one split: a (sequence, head group) per wavefront once there are enough of them to give
+  // every wavefront slot of the card one (8 per compute unit).  256 x 1024 tokens, 32 q / 8 KV heads: page kernel
+  // 66.8 -> 57.8 us; with half as many sequences the wavefronts left without one cost more than the prologues saved
+  // (128 x 2048: 60.5 -> 69.8 us), so not below that number.
+  constexpr bool can_iw = DS == 1 && MB < 4 && NW == MF_WAVES;
+  if constexpr (can_iw && !IW) {
+    const int opt = opt_sequence_per_wave.load(std::memory_order_relaxed);
+    const int64_t from = opt < 0 ? (int64_t)8 * device_compute_units() : opt;
+    if (n_split == 1 && !wide_wg && from > 0 && (int64_t)Hkv * B >= from)
+      return launch_one<D, MB, NX, VB, GS, DS, WPS, F16P, PP, NR, SG, NW, true>(
+          qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table, bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts, n_split,
+          len_sub, max_pages, num_pages, fm, false, st);
+  }
+  constexpr bool can_widen = DS == 1 && NW == MF_WAVES && !IW;
   if (can_widen && wide_wg)
     return launch_one<D, MB, NX, VB, GS, DS, WPS, F16P, PP, NR, SG, can_widen ? 2 * MF_WAVES : NW>(
         qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table, bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts, n_split,
@@ -1268,8 +1337,9 @@ static int launch_one(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, 
   // kernels wait for memory, their workgroups advance side by side whatever their age, and unequal shares cost
   // what they move (32 x 32768: 203 -> 208 us).
   const int skew16 = NW == MF_WAVES && WPS == 2 && DS == 2 ? decode_mfma_split_skew(n_split, Hkv * B) : 0;
-  const dim3 grid = skew16 > 0 ? dim3(n_split / 2, Hkv, 2 * B) : dim3(n_split, Hkv, B);
-  auto kern = decode_mfma_kernel<D, MB, NX, VB, GS, DS, WPS, F16P, PP, NR, SG, NW>;
+  const dim3 grid = IW ? dim3(1, (unsigned)(((int64_t)Hkv * B + NW / DS - 1) / (NW / DS)), 1)
+                       : (skew16 > 0 ? dim3(n_split / 2, Hkv, 2 * B) : dim3(n_split, Hkv, B));
+  auto kern = decode_mfma_kernel<D, MB, NX, VB, GS, DS, WPS, F16P, PP, NR, SG, NW, IW>;
   if (smem > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return (int)e;
@@ -1290,15 +1360,27 @@ static int launch_one(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, 
 }
 
 
+// TQ_POOL_F16, defined by a translation unit before it includes this file: 0 = it holds the kernels for bf16 pools only,
+// 1 = those for fp16 pools only (head_dim 64 / 128: two units each, so that they compile side by side); else both.
+#ifndef TQ_POOL_F16
+#define TQ_POOL_F16 -1
+#endif
+#define TQ_LAUNCH_POOL(F16P_, D_, MB_, NX_, VB_, GS_, DS_, WPS_)                                                \
+  if (sh.f16p == F16P_)                                                                                            \
+    return launch_one<D_, MB_, NX_, VB_, GS_, DS_, WPS_, F16P_>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,     \
+                                                                bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts,      \
+                                                                n_split, len_sub, max_pages, num_pages, fm, wide_wg, st);
+#if TQ_POOL_F16 == 0
+#define TQ_LAUNCH_POOLS(...) TQ_LAUNCH_POOL(false, __VA_ARGS__)
+#elif TQ_POOL_F16 == 1
+#define TQ_LAUNCH_POOLS(...) TQ_LAUNCH_POOL(true, __VA_ARGS__)
+#else
+#define TQ_LAUNCH_POOLS(...) TQ_LAUNCH_POOL(true, __VA_ARGS__) TQ_LAUNCH_POOL(false, __VA_ARGS__)
+#endif
 #define TQ_TRY(D_, MB_, NX_, VB_, GS_, DS_, WPS_)                                                               \
   if (sh.d == D_ && sh.mb == MB_ && sh.nx == NX_ && sh.vb == VB_ && sh.gs == GS_) {                                            \
-    if (sh.f16p)                                                                                                   \
-      return launch_one<D_, MB_, NX_, VB_, GS_, DS_, WPS_, true>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,  \
-                                                                 bt_stride, seq_lens, sm_scale, ly, L, parts,     \
-                                                                 n_parts, n_split, len_sub, max_pages, num_pages, fm, wide_wg, st); \
-    return launch_one<D_, MB_, NX_, VB_, GS_, DS_, WPS_, false>(qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table,   \
-                                                                bt_stride, seq_lens, sm_scale, ly, L, parts,      \
-                                                                n_parts, n_split, len_sub, max_pages, num_pages, fm, wide_wg, st); \
+    TQ_LAUNCH_POOLS(D_, MB_, NX_, VB_, GS_, DS_, WPS_)                                                              \
+    return TQ_EUNSUPPORTED;                                                                                        \
   }
 
 }  // namespace tq
