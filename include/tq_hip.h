@@ -356,10 +356,11 @@ void tq_time_next_key_kernel(void *start_event, void *stop_event);
  *   "wide_workgroups"  1 (default): at head_dim 64 / 128, with an even split count and at most 16 blocks of 64 tokens
  *                      per wavefront (judged by the width of the block table), a step runs workgroups of 8
  *                      wavefronts on half the split count it was given; 0: always 4 wavefronts per workgroup.
- *   "sequence_per_wave" -1 (default), 0 or a count: at head_dim 64 / 128 a step with a single context split and at
- *                      least this many (sequence, group of query heads) pairs - -1: eight per compute unit, 0: never -
- *                      gives every wavefront of a workgroup a pair of its own, walked from the first block to the last,
- *                      instead of four wavefronts sharing one (a quarter of the workgroups, no walkers to merge).
+ *   "sequence_walkers" -1 (default), 4, 2 or 1: at head_dim 64 / 128 a step with a single context split lets 4, 2 or 1
+ *                      wavefronts of a workgroup walk a (sequence, group of query heads), so a workgroup serves 1, 2 or
+ *                      4 of those pairs (fewer workgroups, more trips after each prologue, fewer walkers to merge);
+ *                      -1: the largest of the three with which all wavefronts of the launch are resident at once
+ *                      (8 per compute unit), one if there are more pairs than that.
  *   "split_skew"       0..8, default 1: at head_dim 256, when a launch of 4-wavefront workgroups fills (nearly) every
  *                      compute unit twice and the split count is even, the workgroups of the first half of the grid
  *                      (dispatched first, served first by their SIMDs) take the even splits and this many sixteenths

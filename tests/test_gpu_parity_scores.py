@@ -317,7 +317,7 @@ def test_decode_gives_no_weight_to_pages_outside_the_pool(gpu, d, key_bits, vb, 
 
 
 # ------------------------------------------------------------------ query preparation for every query dtype
-_OPTION_DEFAULTS = {"sequence_per_wave": -1}     # every other option: 1
+_OPTION_DEFAULTS = {"sequence_walkers": -1}     # every other option: 1
 
 
 def _set_option(name, value):
@@ -597,10 +597,10 @@ def test_five_bit_keys_with_the_query_operands_in_lds(gpu, option, vb, Hq, Hkv, 
                                                         (128, 4, 2, 3, 1, torch.float16), (64, 3, 4, 4, 1, torch.bfloat16),
                                                         (64, 3, 2, 16, 2, torch.float16), (128, 3, 4, 22, 2, torch.bfloat16),
                                                         (128, 3, 8, 5, 1, torch.bfloat16), (128, 2, 2, 7, 1, torch.bfloat16)])
-def test_a_sequence_per_wavefront(gpu, d, key_bits, vb, Hq, Hkv, dtype):
-    """Many short sequences in one split: every wavefront of a page-kernel workgroup walks a (sequence, group of
-    heads) of its own (run-time option "sequence_per_wave": from how many pairs on; 1 = always, 0 = never) instead of
-    four wavefronts sharing one.  Five sequences - so that the last workgroup has wavefronts without a pair - of
+def test_one_or_two_wavefronts_per_sequence(gpu, d, key_bits, vb, Hq, Hkv, dtype):
+    """Many short sequences in one split: one or two wavefronts of a page-kernel workgroup walk a (sequence, group
+    of heads) (run-time option "sequence_walkers": 1, 2, or 4 = all of them; by default chosen from the number of
+    pairs) instead of all four.  Five sequences - so that the last workgroup has wavefronts without a pair - of
     ragged and zero length, a poisoned block table, head groups of unequal size (22 heads on 2 KV heads: 6 + 5), all
     three endings of the step (output written by the page kernel, partials for the merge kernel, an exact tail's
     partial merged in) against the four-wavefront form and the oracle (score.py:84-173)."""
@@ -621,7 +621,7 @@ def test_a_sequence_per_wavefront(gpu, d, key_bits, vb, Hq, Hkv, dtype):
     rk = torch.randn(B, R, Hkv, d, generator=g).to(dtype).to(gpu)
     rv = torch.randn(B, R, Hkv, d, generator=g).to(dtype).to(gpu)
     rl = torch.tensor([R, 3, 0, R, 11], dtype=torch.int32, device=gpu)
-    _progress(f"a sequence per wavefront d={d} kb={key_bits} vb={vb} Hq={Hq} Hkv={Hkv} {dtype}")
+    _progress(f"one or two wavefronts per sequence d={d} kb={key_bits} vb={vb} Hq={Hq} Hkv={Hkv} {dtype}")
 
     def runs():
         outs = []
@@ -637,16 +637,19 @@ def test_a_sequence_per_wavefront(gpu, d, key_bits, vb, Hq, Hkv, dtype):
         return outs
 
     try:
-        _set_option("sequence_per_wave", 0)
+        _set_option("sequence_walkers", 4)
         want = runs()
-        _set_option("sequence_per_wave", 1)
+        _set_option("sequence_walkers", 1)
         got = runs()
+        _set_option("sequence_walkers", 2)
+        got2 = runs()
     finally:
-        _set_option("sequence_per_wave", -1)
+        _set_option("sequence_walkers", -1)
         _set_option("merge_in_kernel", 1)
-    for i, (a, b_) in enumerate(zip(got, want)):
-        assert torch.isfinite(a).all(), i
+    for i, (a, a2, b_) in enumerate(zip(got, got2, want)):
+        assert torch.isfinite(a).all() and torch.isfinite(a2).all(), i
         assert (a - b_).abs().max() <= 2 ** -7 * b_.abs().max() + 1e-6, i        # one bf16 step of the largest value
+        assert (a2 - b_).abs().max() <= 2 ** -7 * b_.abs().max() + 1e-6, i
     prm = params_of(tq)
     for b in range(B):
         if lens[b] == 0:

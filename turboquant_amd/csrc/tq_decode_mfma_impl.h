@@ -227,11 +227,12 @@ __device__ __forceinline__ constexpr int v_bitpos(int t) {
 // and no register holds data in flight.
 // NW: wavefronts per workgroup, 4 (two workgroups per compute unit) or 8 (one): with few blocks per
 // wavefront the larger workgroup wins - half as many workgroups to dispatch, prologues and partials.
-// IW (many short sequences, one split): every wavefront of a workgroup walks a (sequence, group of heads) of its own
-// from the first block to the last, instead of the workgroup's wavefronts sharing one.  A wavefront then makes four
-// times the trips after one prologue, a launch has a quarter of the workgroups (256 sequences x 8 KV heads: one
-// resident round instead of four), and the epilogue has no walkers to merge.  The grid is (1, ceil(items / 4), 1).
-template <int D, int MB, int NX, int VB, int GS, int DS, int WPS, bool F16P, bool PP, bool NR, bool SG, int NW, bool IW>
+// IW > 0 (many short sequences, one split): a (sequence, group of heads) is walked by IW wavefronts (1 or 2) of a
+// workgroup instead of all four, from the first block to the last, so a workgroup serves 4 / IW of them.  A wavefront
+// then makes 4 / IW times the trips after one prologue, a launch has IW / 4 of the workgroups (256 sequences x 8 KV
+// heads: one resident round instead of four), and the epilogue merges IW walkers instead of four (IW = 1: none).
+// The grid is (1, ceil(items IW / 4), 1).
+template <int D, int MB, int NX, int VB, int GS, int DS, int WPS, bool F16P, bool PP, bool NR, bool SG, int NW, int IW>
 __global__ void __launch_bounds__(NW * 64, WPS)
 decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div,
                    const uint8_t* __restrict__ pool, const int32_t* __restrict__ block_table,
@@ -264,7 +265,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   // by plane so that an operand is read once for its four pages.
   constexpr bool QL = MB >= 4;
   static_assert(!QL || (!PP && !SG && DS == 1), "operands in LDS: head_dim 128, page data in registers");
-  static_assert(!IW || (DS == 1 && !QL), "a (sequence, head group) per wavefront: wavefronts that work alone, operands in registers");
+  static_assert(IW == 0 || (DS == 1 && !QL && (IW == 1 || IW == 2)), "a (sequence, head group) per wavefront: wavefronts that work alone, operands in registers");
   constexpr int NJ = NR ? 1 : 2;              // heads a lane sees in the score MFMA's output
   // Hkv counts query-head groups: a KV head with more than 8 query heads is served by kv_div groups of at most 8
   // heads each (consecutive groups read the same pages); when the heads do not divide evenly the last group of
@@ -283,9 +284,11 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   // go to the card's eight dies in turn, each die has its own L2, and a distance that is a multiple of eight puts the
   // groups that read the same pages at the same time on the same die.
   int h = blockIdx.y, qbase;
-  bool item_live = true;                        // IW: this wavefront has a (sequence, head group) of its own
-  if constexpr (IW) {
-    const int item = blockIdx.y * (NW / DS) + wgrp, items = Hkv * n_seq;
+  bool item_live = true;                        // IW: this wavefront has a (sequence, head group) to walk
+  constexpr int IWC = IW > 0 ? IW : 1;
+  const int wsub = IW > 0 ? wgrp % IWC : wgrp;  // this walker's number among those of its (sequence, head group)
+  if constexpr (IW > 0) {
+    const int item = blockIdx.y * (NW / DS / IWC) + wgrp / IWC, items = Hkv * n_seq;
     item_live = item < items;
     const int item_c = item_live ? item : items - 1;          // (a wavefront without an item repeats the last one and stores nothing)
     h = item_c % Hkv;
@@ -932,9 +935,9 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
     KeyRegs K;
     ValRegs V;
     int pid[4];
-    constexpr int WSTEP = IW ? 1 : NGRP;                   // distance of a walker's consecutive blocks
+    constexpr int WSTEP = IW > 0 ? IW : NGRP;              // distance of a walker's consecutive blocks
     const int trips = (max(blk_end - blk_begin, 0) + WSTEP - 1) / WSTEP;
-    int blk = blk_begin + (IW ? 0 : wgrp);
+    int blk = blk_begin + wsub;
     int bad = 0;                                          // pages of the current block that lie outside the pool
     if (blk < blk_end) {
       bad = page_ids(blk, pid, std::true_type{});
@@ -1034,7 +1037,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   if (SG) stage_wait<0>();   // the last trip's requests (a repeat of its own block) have landed
   __syncthreads();      // every wave is done with its private LDS region
   TQ_STAMP(6);
-  const int g_rows = IW ? 8 : G;                               // rows of a walker in s_red (IW: the walkers' groups may differ in size)
+ const int g_rows = IW > 0 ? 8 : G;                              // rows of a walker in s_red (IW: the walkers' groups may differ in size)
   float* s_z = s_red + NGRP * g_rows * (D + 2);                // [MF_WAVES][16 rows][16 groups]
 #pragma unroll
   for (int i = 0; i < 4; ++i) s_z[(wave * 16 + 4 * kb + i) * 16 + n] = zacc[i];
@@ -1081,18 +1084,40 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
   }
   __syncthreads();
   TQ_STAMP(7);
-  if constexpr (IW) {
-    // Every wavefront finishes the (sequence, head group) it walked alone: its rows of s_red are the result.
+  if constexpr (IW > 0) {
+    // The IW wavefronts of a (sequence, head group) finish it among themselves: their rows of s_red hold its walkers.
+    constexpr int TP = 64 * IWC;                 // threads of a (sequence, head group)
+    const int tsub = wsub * 64 + lane, w0 = wgrp - wsub;
+    // log-sum-exp merge of the walkers' element e (0: the maximum itself, 1: the sum of weights, 2 + ch: a channel)
+    auto merged = [&](int g, int e, float& mm, float& ll) -> float {
+      float m_w[IWC], l_w[IWC], a_w[IWC];
+      mm = MF_NEG;
+#pragma unroll
+      for (int w = 0; w < IWC; ++w) {
+        const float* r = s_red + ((w0 + w) * g_rows + g) * (D + 2);
+        m_w[w] = r[0]; l_w[w] = r[1]; a_w[w] = r[e];
+        mm = fmaxf(mm, m_w[w]);
+      }
+      ll = 0.0f;
+      float aa = 0.0f;
+#pragma unroll
+      for (int w = 0; w < IWC; ++w) {
+        const float wgt = __expf(m_w[w] - mm);
+        ll = fmaf(wgt, l_w[w], ll);
+        aa = fmaf(wgt, a_w[w], aa);
+      }
+      return aa;
+    };
     if (fm.out != nullptr && fm.n_extra <= 1) {
       // the attention output, merged with the exact tail's partial if there is one (an earlier launch wrote it)
 #pragma unroll
-      for (int k = 0; k < 8 * D / 64; ++k) {
-        const int o = lane + k * 64;
+      for (int k = 0; k < 8 * D / TP; ++k) {
+        const int o = tsub + k * TP;
         const int g_o = o / D, ch = o % D;
         const bool live = item_live && g_o < G;
         const int g = live ? g_o : 0;
-        const float* r = s_red + (wgrp * g_rows + g) * (D + 2);
-        const float mm = r[0], ll = r[1], aa = r[2 + ch];
+        float mm, ll;
+        const float aa = merged(g, 2 + ch, mm, ll);
         if (live && fm.n_extra == 0) {
           const float inv = ll > 0.0f ? 1.0f / ll : 0.0f;
           store_from_f32(fm.out, ((int64_t)b * Hq + qbase + g) * D + ch, aa * inv, fm.out_dtype);
@@ -1102,8 +1127,8 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
           float top = MF_NEG;
           if (ll > 0.0f) top = fmaxf(top, mm);
           if (l_x > 0.0f) top = fmaxf(top, m_x);
-          const float w0 = ll > 0.0f ? __expf(mm - top) : 0.0f, w1 = l_x > 0.0f ? __expf(m_x - top) : 0.0f;
-          const float l_all = fmaf(w1, l_x, fmaf(w0, ll, 0.0f)), a_all = fmaf(w1, a_x, fmaf(w0, aa, 0.0f));
+          const float w0x = ll > 0.0f ? __expf(mm - top) : 0.0f, w1x = l_x > 0.0f ? __expf(m_x - top) : 0.0f;
+          const float l_all = fmaf(w1x, l_x, fmaf(w0x, ll, 0.0f)), a_all = fmaf(w1x, a_x, fmaf(w0x, aa, 0.0f));
           const float inv = l_all > 0.0f ? 1.0f / l_all : 0.0f;
           store_from_f32(fm.out, ((int64_t)b * Hq + qbase + g) * D + ch, a_all * inv, fm.out_dtype);
         }
@@ -1111,12 +1136,13 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
     } else {
       // the partial (m, l, acc[D]) of every head, for the merge kernel
       constexpr int PAIRS = (D + 2) / 2;
-      for (int o = lane; o < 8 * PAIRS; o += 64) {
+      for (int o = tsub; o < 8 * PAIRS; o += TP) {
         const int g = o / PAIRS, pr = o % PAIRS;
         if (item_live && g < G) {
-          const float* r = s_red + (wgrp * g_rows + g) * (D + 2);
+          float mm, ll, m2, l2;
+          const float a0 = merged(g, 2 * pr, mm, ll), a1 = merged(g, 2 * pr + 1, m2, l2);
           float* out = parts + (((int64_t)b * Hq + qbase + g) * n_parts + split) * (D + 2);
-          store_coherent2(out + 2 * pr, f32x2{r[2 * pr], r[2 * pr + 1]});
+          store_coherent2(out + 2 * pr, pr == 0 ? f32x2{mm, ll} : f32x2{a0, a1});
         }
       }
     }
@@ -1280,7 +1306,7 @@ decode_mfma_kernel(uint32_t* qa_pack, float* q_stat, int Hq, int Hkv, int kv_div
 }
 
 template <int D, int MB, int NX, int VB, int GS, int DS, int WPS, bool F16P, bool PP = false, bool NR = false, bool SG = false,
-          int NW = MF_WAVES, bool IW = false>
+          int NW = MF_WAVES, int IW = 0>
 static int launch_one(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, int kv_div,
                       const uint8_t* pool, const int32_t* block_table, int bt_stride, const int32_t* seq_lens,
                       float sm_scale, const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts, int n_split,
@@ -1289,7 +1315,7 @@ static int launch_one(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, 
   // (heads of the largest group of a KV head; kv_div groups share a KV head's heads, the last one may have fewer)
   const int G = kv_div > 1 ? (Hq / (Hkv / kv_div) + kv_div - 1) / kv_div : Hq / Hkv;
   size_t per_wave = (size_t)wave_lds_floats(D / DS / GS, DS) * sizeof(float);
-  size_t merge = (size_t)(NW / DS * (IW ? 8 : G) * (D + 2) + NW * 16 * 16) * sizeof(float);
+  size_t merge = (size_t)(NW / DS * (IW > 0 ? 8 : G) * (D + 2) + NW * 16 * 16) * sizeof(float);
   if (SG) per_wave += stage_bytes((D / DS / 16) * VB / 2);
   size_t smem = per_wave * NW > merge ? per_wave * NW : merge;
   // four index planes: the group's packed query operands in LDS, behind the wavefronts' regions
@@ -1314,20 +1340,31 @@ static int launch_one(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, 
                                                                       n_split, len_sub, max_pages, num_pages, fm, wide_wg, st);
   } else {
   // eight wavefronts per workgroup (one workgroup per compute unit) for the kernels whose wavefronts work alone
-  // Many short sequences in one split: a (sequence, head group) per wavefront once there are enough of them to give
-  // every wavefront slot of the card one (8 per compute unit).  256 x 1024 tokens, 32 q / 8 KV heads: page kernel
-  // 66.8 -> 57.8 us; with half as many sequences the wavefronts left without one cost more than the prologues saved
-  // (128 x 2048: 60.5 -> 69.8 us), so not below that number.
+  // Many short sequences in one split: the fewer wavefronts walk a (sequence, head group), the fewer workgroups the
+  // launch has and the more trips follow each prologue; the most wavefronts per pair (4, 2 or 1) with which all of the
+  // launch's wavefronts are resident at once (8 per compute unit) wins at every size measured (page kernel, 32 q / 8 KV
+  // heads, four / two / one wavefront per pair: 64 x 2048 28.1 / 37.2 / 63.5 us, 96 x 2048 51.9 / 45.6 / 67.0,
+  // 128 x 2048 60.4 / 56.0 / 69.7, 128 x 512 21.7 / 18.8 / 22.2, 160 x 1024 46.6 / 48.9 / 44.1, 192 x 1024 51.4 / 52.7 /
+  // 47.0, 256 x 1024 66.7 / 61.5 / 58.0); with more pairs than wavefront slots, one.
   constexpr bool can_iw = DS == 1 && MB < 4 && NW == MF_WAVES;
-  if constexpr (can_iw && !IW) {
-    const int opt = opt_sequence_per_wave.load(std::memory_order_relaxed);
-    const int64_t from = opt < 0 ? (int64_t)8 * device_compute_units() : opt;
-    if (n_split == 1 && !wide_wg && from > 0 && (int64_t)Hkv * B >= from)
-      return launch_one<D, MB, NX, VB, GS, DS, WPS, F16P, PP, NR, SG, NW, true>(
-          qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table, bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts, n_split,
-          len_sub, max_pages, num_pages, fm, false, st);
+  if constexpr (can_iw && IW == 0) {
+    if (n_split == 1 && !wide_wg) {
+      int walkers = opt_sequence_walkers.load(std::memory_order_relaxed);
+      if (walkers < 0) {
+        const int64_t slots = (int64_t)8 * device_compute_units(), items = (int64_t)Hkv * B;
+        walkers = slots <= 0 || 4 * items <= slots ? 4 : (2 * items <= slots ? 2 : 1);
+      }
+      if (walkers == 1)
+        return launch_one<D, MB, NX, VB, GS, DS, WPS, F16P, PP, NR, SG, NW, 1>(
+            qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table, bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts, n_split,
+            len_sub, max_pages, num_pages, fm, false, st);
+      if (walkers == 2)
+        return launch_one<D, MB, NX, VB, GS, DS, WPS, F16P, PP, NR, SG, NW, 2>(
+            qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table, bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts, n_split,
+            len_sub, max_pages, num_pages, fm, false, st);
+    }
   }
-  constexpr bool can_widen = DS == 1 && NW == MF_WAVES && !IW;
+  constexpr bool can_widen = DS == 1 && NW == MF_WAVES && IW == 0;
   if (can_widen && wide_wg)
     return launch_one<D, MB, NX, VB, GS, DS, WPS, F16P, PP, NR, SG, can_widen ? 2 * MF_WAVES : NW>(
         qa_pack, q_stat, B, Hq, Hkv, kv_div, pool, block_table, bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts, n_split,
@@ -1337,7 +1374,8 @@ static int launch_one(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv, 
   // kernels wait for memory, their workgroups advance side by side whatever their age, and unequal shares cost
   // what they move (32 x 32768: 203 -> 208 us).
   const int skew16 = NW == MF_WAVES && WPS == 2 && DS == 2 ? decode_mfma_split_skew(n_split, Hkv * B) : 0;
-  const dim3 grid = IW ? dim3(1, (unsigned)(((int64_t)Hkv * B + NW / DS - 1) / (NW / DS)), 1)
+  constexpr int IPW = NW / DS / (IW > 0 ? IW : 1);          // (sequence, head group) pairs of a workgroup with IW > 0
+  const dim3 grid = IW > 0 ? dim3(1, (unsigned)(((int64_t)Hkv * B + IPW - 1) / IPW), 1)
                        : (skew16 > 0 ? dim3(n_split / 2, Hkv, 2 * B) : dim3(n_split, Hkv, B));
   auto kern = decode_mfma_kernel<D, MB, NX, VB, GS, DS, WPS, F16P, PP, NR, SG, NW, IW>;
   if (smem > 48 * 1024) {

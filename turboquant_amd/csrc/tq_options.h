@@ -14,6 +14,6 @@ extern std::atomic<int> opt_tail_chunks;        // hybrid decode with many split
 extern std::atomic<int> opt_merge_row_groups;  // merge kernel: with few rows, several workgroups share a row's channels
 extern std::atomic<int> opt_prefetch_trips;     // decode: trips of every block walker whose pages the preparation launch reads ahead (0: none, -1: one at head_dim 256)
 extern std::atomic<int> opt_prep_mfma;           // decode: bf16 queries at head_dim 128 / 256 are prepared on the matrix cores
-extern std::atomic<int> opt_sequence_per_wave;     // decode, one split: from this many (sequence, head group) pairs on, a wavefront walks one alone (0: never, -1: 8 per compute unit)
+extern std::atomic<int> opt_sequence_walkers;     // decode, one split, head_dim 64 / 128: wavefronts that walk a (sequence, head group): 4, 2, 1, or -1 = as many of those as keep the whole launch resident
 extern std::atomic<int> opt_merge_in_kernel;    // decode: few context splits are merged by the last workgroup of the page kernel
 }  // namespace tq
