@@ -317,7 +317,7 @@ def test_decode_gives_no_weight_to_pages_outside_the_pool(gpu, d, key_bits, vb, 
 
 
 # ------------------------------------------------------------------ query preparation for every query dtype
-_OPTION_DEFAULTS = {"sequence_walkers": -1}     # every other option: 1
+_OPTION_DEFAULTS = {"sequence_walkers": -1, "prep_words": -1}     # every other option: 1
 
 
 def _set_option(name, value):
@@ -658,6 +658,16 @@ def test_one_or_two_wavefronts_per_sequence(gpu, d, key_bits, vb, Hq, Hkv, dtype
         kc, vc = _store_from_oracle_view(pool, table[b].to(gpu), lens[b])
         ref = O.hybrid_attention(q[b:b + 1], kc, vc, max(lens[b], O.MIN_HISTORY), prm, Hkv, None, None)
         assert cosine(got[0][b:b + 1], ref) >= COS_GATE, b
+
+
+@pytest.mark.parametrize("d,key_bits,vb,Hq,Hkv", [(128, 3, 4, 8, 2), (128, 4, 2, 3, 1), (256, 3, 2, 16, 2), (256, 2, 4, 5, 1),
+                                                  (128, 3, 4, 22, 2), (128, 5, 4, 4, 1)])
+def test_preparation_with_a_plane_word_per_wavefront(gpu, d, key_bits, vb, Hq, Hkv):
+    """Large matrix-core preparations run a workgroup per tile of query rows whose wavefronts take a plane word each
+    (run-time option "prep_words" 1), small ones a workgroup per (tile, word) (0): the same products in the same order,
+    so the packed operands, and with them the step's output, are the same bits (score.py:84-173 through the oracle
+    for the first form)."""
+    _variant_against_default(gpu, "prep_words", d, key_bits, vb, Hq, Hkv, torch.bfloat16, exact=True)
 
 
 @pytest.mark.parametrize("B,Hq,Hkv,d,key_bits,vb,dtype", [(201, 4, 1, 128, 3, 4, torch.bfloat16), (201, 2, 1, 128, 4, 2, torch.bfloat16),

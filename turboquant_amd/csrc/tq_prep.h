@@ -394,27 +394,30 @@ __device__ __forceinline__ void prefetch_pages_body(const PagePrefetch& P, int p
 // 16-coordinate halves of one of the two products: d / 32 x 3 MFMAs whose matrix operands are all requested before
 // the first is used (one memory latency).  The 16 x 32 results meet in LDS and one lane per (term plane, row) packs
 // the four fp6 terms exactly as prep_query_body does.  Nothing is read from another workgroup.
+// WW (large preparations): a workgroup owns a tile and ALL its plane words - wavefront w takes words w, w + 4, ...,
+// computes the four 16 x 16 pieces of a word (two halves x two products) one after the other and packs the word
+// itself, so the launch has a quarter (head_dim 128) or an eighth (256) of the workgroups, all four wavefronts pack
+// instead of one, and nothing waits for another wavefront.  The operands are the same bits either way.
 typedef uint32_t prep_u32x4 __attribute__((ext_vector_type(4)));
 typedef float prep_f32x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 prep_bf16x8 __attribute__((ext_vector_type(8)));
 constexpr int PREP_MFMA_THREADS = 256, PREP_MFMA_LD = 36;          // LDS row stride of a wavefront's 16 x 32 tile
 __host__ __device__ inline int prep_mfma_smem_floats() { return 2 * 16 * PREP_MFMA_LD + 32; }
 
-template <int D>
+template <int D, bool WW>
 __device__ __forceinline__ void prep_mfma_body(const uint16_t* __restrict__ q, int G, int64_t n_rows, const tq_layer& ly,
                                                float sm_scale, float* __restrict__ q_stat, uint32_t* __restrict__ qa_pack,
                                                unsigned long long* __restrict__ arrivals, int head_rows, int64_t tile,
-                                               int word, float* sm) {
+                                               int word_of_wg, float* sm) {
   constexpr int KS = D / 32;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = lane & 15, kb = lane >> 4;
   const int gpt = 16 / G, rows_tile = gpt * G;                     // whole groups per tile
   const int64_t row0 = tile * rows_tile, group0 = tile * gpt;
   const int R = (int)(n_rows - row0 < rows_tile ? n_rows - row0 : rows_tile);
-  const int chunk = word >> 2, kw = word & 3;                       // the word's place in the operand layout
-  const int jt = wave & 1, m = wave >> 1;                           // this wavefront's half of the word, and its product
-  if (arrivals != nullptr && word == 0 && tid < gpt && tid * G < R) arrivals[group0 + tid] = 0ull;
-  float* s_rot = sm;                                                // [16 rows][32 coordinates], stride PREP_MFMA_LD
+  if (arrivals != nullptr && (WW || word_of_wg == 0) && tid < gpt && tid * G < R) arrivals[group0 + tid] = 0ull;
+  // (WW: a region per wavefront)
+  float* s_rot = sm + (WW ? wave * prep_mfma_smem_floats() : 0);    // [16 rows][32 coordinates], stride PREP_MFMA_LD
   float* s_sk = s_rot + 16 * PREP_MFMA_LD;
   float* stat = s_sk + 16 * PREP_MFMA_LD;                           // [16 rows][2]: multipliers of coef q_rot_j and q_sk_j
   // column operands: lane (row n, block kb) holds q[n][32 ks + 8 kb .. + 7]; rows beyond the tile are zero
@@ -428,9 +431,10 @@ __device__ __forceinline__ void prep_mfma_body(const uint16_t* __restrict__ q, i
       for (int ks = 0; ks < KS; ++ks) qb[ks] = prep_u32x4{0u, 0u, 0u, 0u};
     }
   }
-  // row operands: the three bf16 terms of this wavefront's 16 matrix rows, all requested before anything waits
-  prep_u32x4 ma[3][KS];
-  {
+  // one 16 x 16 piece: half jt of plane word `word`, product m (0: q Pi^T, 1: q S^T).  Row operands: the three bf16
+  // terms of 16 matrix rows, all requested before anything waits.
+  auto piece = [&](int word, int jt, int m) __attribute__((always_inline)) {
+    prep_u32x4 ma[3][KS];
     const uint16_t* mat = m ? ly.S_split : ly.Pi_split;
 #pragma unroll
     for (int t = 0; t < 3; ++t) {
@@ -438,7 +442,16 @@ __device__ __forceinline__ void prep_mfma_body(const uint16_t* __restrict__ q, i
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) ma[t][ks] = *(const prep_u32x4*)(base + ks * (64 * 8));
     }
-  }
+    prep_f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int t = 2; t >= 0; --t)                                       // the small terms first
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(prep_bf16x8, ma[t][ks]),
+                                                      __builtin_bit_cast(prep_bf16x8, qb[ks]), acc, 0, 0, 0);
+    // result register i of lane (row n, quarter kb) is coordinate 16 jt + 4 kb + i of query row n
+    *(prep_f32x4*)((m ? s_sk : s_rot) + n * PREP_MFMA_LD + jt * 16 + 4 * kb) = acc;
+  };
   // row statistics from the same registers: the four lanes of a row each hold a quarter of its coordinates
   {
     float ss = 0.0f, s1 = 0.0f, s2 = 0.0f;
@@ -464,34 +477,43 @@ __device__ __forceinline__ void prep_mfma_body(const uint16_t* __restrict__ q, i
     const float nq = sqrtf(ss), k = sm_scale * 1.4426950408889634f;
     const int e1 = min(max((int)((__float_as_uint(fabsf(k) * nq * cmax) >> 23) & 255u) - 126, -100), 100);
     const int e2 = min(max((int)((__float_as_uint(2.0f * fabsf(k * ly.qjl_scale) * nq * ly.S_rownorm_max) >> 23) & 255u) - 126, -100), 100);
-    if (kb == 0 && wave == 0) {
+    if (kb == 0 && (WW || wave == 0)) {
       stat[n * 2 + 0] = k * __uint_as_float((uint32_t)(127 - e1) << 23);
       stat[n * 2 + 1] = 2.0f * k * ly.qjl_scale * __uint_as_float((uint32_t)(127 - e2) << 23);
-      if (word == 0 && n < R) {
+      if ((WW ? wave == 0 : word_of_wg == 0) && n < R) {
         float* st = q_stat + (row0 + n) * 4;
         st[0] = (float)e1; st[1] = (float)e2;
         st[2] = k * ly.term_const * s1; st[3] = -k * ly.qjl_scale * s2;
       }
     }
   }
-  prep_f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-  for (int t = 2; t >= 0; --t)                                       // the small terms first
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(prep_bf16x8, ma[t][ks]),
-                                                    __builtin_bit_cast(prep_bf16x8, qb[ks]), acc, 0, 0, 0);
-  // result register i of lane (row n, quarter kb) is coordinate 16 jt + 4 kb + i of query row n
-  *(prep_f32x4*)((m ? s_sk : s_rot) + n * PREP_MFMA_LD + jt * 16 + 4 * kb) = acc;
-  __syncthreads();
-  // operands of this plane word: one lane per (term plane, row), as in prep_query_body
   const int mb = ly.mse_bits;
   int nx = 0;
   for (int t = 0; t < ly.n_terms; ++t)
     if (__builtin_popcount(ly.term_mask[t]) > 1) ++nx;
   const int ntp = mb + nx + 1;
   constexpr int wpl = D / 128;
-  for (int idx = tid; idx < ntp * 16; idx += PREP_MFMA_THREADS) {
+  constexpr int NPASS = WW ? (D / 32) / 4 : 1;
+#pragma unroll 1
+  for (int pass = 0; pass < NPASS; ++pass) {
+  const int word = WW ? wave + 4 * pass : word_of_wg;
+  const int chunk = word >> 2, kw = word & 3;                       // the word's place in the operand layout
+  if constexpr (WW) {
+    // (the tile of the last word has been read by this wavefront's packing lanes)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int c = 0; c < 4; ++c) piece(word, c & 1, c >> 1);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  } else {
+    piece(word, wave & 1, wave >> 1);                               // this wavefront's half of the word, and its product
+    __syncthreads();
+  }
+  // operands of this plane word: one lane per (term plane, row), as in prep_query_body
+  for (int idx = WW ? lane : tid; idx < ntp * 16; idx += WW ? 64 : PREP_MFMA_THREADS) {
     const int tp = idx >> 4, r = idx & 15;
     if (r >= R) continue;
     typedef float f32x16_t __attribute__((ext_vector_type(16)));
@@ -555,6 +577,7 @@ __device__ __forceinline__ void prep_mfma_body(const uint16_t* __restrict__ q, i
         }
       }
     }
+  }
   }
 }
 

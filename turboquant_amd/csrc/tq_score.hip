@@ -89,7 +89,8 @@ prep_query_kernel(const void* __restrict__ q, int G, int gpw, int64_t n_rows, in
 
 // The preparation on the matrix cores (bf16 queries, head_dim 128 / 256): a workgroup per (tile of up to 16 query
 // rows, plane word), then the page-prefetch workgroups.
-template <int D>
+// WW: a workgroup per tile, its wavefronts each taking a plane word at a time.
+template <int D, bool WW>
 __global__ void __launch_bounds__(PREP_MFMA_THREADS)
 prep_mfma_kernel(const uint16_t* __restrict__ q, int G, int64_t n_rows, tq_layer ly, float sm_scale,
                  float* __restrict__ q_stat, uint32_t* __restrict__ qa_pack, unsigned long long* __restrict__ arrivals,
@@ -97,7 +98,7 @@ prep_mfma_kernel(const uint16_t* __restrict__ q, int G, int64_t n_rows, tq_layer
   extern __shared__ __align__(16) float sm[];
   const int id = blockIdx.x;
   if (id < n_prep)
-    prep_mfma_body<D>(q, G, n_rows, ly, sm_scale, q_stat, qa_pack, arrivals, head_rows, id % n_tiles, id / n_tiles, sm);
+    prep_mfma_body<D, WW>(q, G, n_rows, ly, sm_scale, q_stat, qa_pack, arrivals, head_rows, id % n_tiles, id / n_tiles, sm);
   else
     prefetch_pages_body<PREP_MFMA_THREADS>(pf, id - n_prep);
 }
@@ -410,18 +411,30 @@ int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* 
       const int n_tiles = (int)((rows + rows_tile - 1) / rows_tile);
       // (several tiles per workgroup - in turn, or their products first and then all four wavefronts packing - measured
       // slower at every size: 256 x 1024 tokens 83.0 -> 83.9 us per step with four, 64 x 2048 33.8 -> 38.6)
-      const int n_mprep = n_tiles * (d / 32);
+      // Head_dim 128 with more (tile, word) pairs than the card holds workgroups of this kernel at once (four per compute
+      // unit): a workgroup per tile, its wavefronts taking a plane word each (256 x 1024 tokens, 32 q / 8 KV heads:
+      // preparation 16.5 -> 12.3 us; smaller ones lose 1 - 2 us, and at head_dim 256, where a wavefront takes two words in
+      // turn, 128 x 2048 at 16 q / 2 KV heads goes from 44.6 to 54.5 us per step).
+      const int opt_ww = opt_prep_words.load(std::memory_order_relaxed);
+      const bool ww = opt_ww < 0 ? d == 128 && (int64_t)n_tiles * (d / 32) > (int64_t)4 * device_compute_units() : opt_ww != 0;
+      const int n_mprep = ww ? n_tiles : n_tiles * (d / 32);
       PagePrefetch pf;
       if (prefetch && prefetch->blocks > 0 && prefetch->n_wg > 0 && n_mprep <= 2 * device_compute_units()) pf = *prefetch;
       pf.front = n_mprep;
       const dim3 grid((unsigned)(n_mprep + (pf.blocks > 0 ? pf.n_wg : 0))), block(PREP_MFMA_THREADS);
-      const size_t smem = (size_t)prep_mfma_smem_floats() * sizeof(float);
-      if (d == 128)
-        prep_mfma_kernel<128><<<grid, block, smem, st>>>((const uint16_t*)q, G, rows, *layer, sm_scale, q_stat, qa_pack,
-                                                         arrivals, head_rows, n_tiles, n_mprep, pf);
+      const size_t smem = (size_t)prep_mfma_smem_floats() * sizeof(float) * (ww ? 4 : 1);
+      if (d == 128 && ww)
+        prep_mfma_kernel<128, true><<<grid, block, smem, st>>>((const uint16_t*)q, G, rows, *layer, sm_scale, q_stat, qa_pack,
+                                                               arrivals, head_rows, n_tiles, n_mprep, pf);
+      else if (d == 128)
+        prep_mfma_kernel<128, false><<<grid, block, smem, st>>>((const uint16_t*)q, G, rows, *layer, sm_scale, q_stat, qa_pack,
+                                                                arrivals, head_rows, n_tiles, n_mprep, pf);
+      else if (ww)
+        prep_mfma_kernel<256, true><<<grid, block, smem, st>>>((const uint16_t*)q, G, rows, *layer, sm_scale, q_stat, qa_pack,
+                                                               arrivals, head_rows, n_tiles, n_mprep, pf);
       else
-        prep_mfma_kernel<256><<<grid, block, smem, st>>>((const uint16_t*)q, G, rows, *layer, sm_scale, q_stat, qa_pack,
-                                                         arrivals, head_rows, n_tiles, n_mprep, pf);
+        prep_mfma_kernel<256, false><<<grid, block, smem, st>>>((const uint16_t*)q, G, rows, *layer, sm_scale, q_stat, qa_pack,
+                                                                arrivals, head_rows, n_tiles, n_mprep, pf);
       hipError_t e = hipGetLastError();
       return e == hipSuccess ? TQ_OK : (int)e;
     }
