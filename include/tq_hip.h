@@ -356,6 +356,9 @@ void tq_time_next_key_kernel(void *start_event, void *stop_event);
  *   "wide_workgroups"  1 (default): at head_dim 64 / 128, with an even split count and at most 16 blocks of 64 tokens
  *                      per wavefront (judged by the width of the block table), a step runs workgroups of 8
  *                      wavefronts on half the split count it was given; 0: always 4 wavefronts per workgroup.
+ *   "append_small"     -1 (default), 0, or a tile count: an append to pages of at most this many 16-vector tiles (-1: two
+ *                      per compute unit) gives every tile a workgroup that computes that tile only - the page write of
+ *                      a decode step, a token per sequence; 0: always workgroups over groups of tiles.  Same bytes.
  *   "prep_words"       -1 (default), 0 or 1: the matrix-core query preparation runs a workgroup per (tile of up to 16 query
  *                      rows, 32-coordinate plane word) (0) or a workgroup per tile whose four wavefronts take a word each
  *                      (1: a quarter or an eighth of the workgroups); -1: the second at head_dim 128 when the first would not

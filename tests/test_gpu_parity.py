@@ -387,6 +387,35 @@ def test_paged_append_equals_flat_quantise(gpu, d, key_bits, vb, dtype):
     assert torch.equal(pool.data[used[:-1]], pool2.data[used[:-1]])
 
 
+@pytest.mark.parametrize("d,key_bits,vb,dtype,B,H", [(128, 3, 4, torch.bfloat16, 32, 8), (256, 3, 2, torch.bfloat16, 5, 2),
+                                                       (64, 2, 2, torch.float16, 40, 4), (128, 4, 4, torch.float32, 7, 8)])
+def test_single_token_append_with_a_workgroup_per_tile(gpu, d, key_bits, vb, dtype, B, H):
+    """The page write of a decode step: a token per sequence at ragged positions.  Few 16-vector tiles get a
+    workgroup each that computes its tile only (option "append_small", the default); the pages must equal,
+    byte for byte, those of the kernel whose workgroups compute groups of tiles (option 0)."""
+    from turboquant_amd import _ffi
+    pages = 8
+    g = torch.Generator().manual_seed(11 * d + B)
+    k = torch.randn(B, 1, H, d, generator=g).to(dtype).to(gpu)
+    v = torch.randn(B, 1, H, d, generator=g).to(dtype).to(gpu)
+    table = torch.randperm(B * pages, generator=g).to(torch.int32).view(B, pages).to(gpu)
+    pos = torch.randint(0, pages * 16, (B,), generator=g).to(torch.int32).to(gpu)
+    got = {}
+    try:
+        for mode in (0, -1, 3):                      # 3: only appends of up to three tiles take the small kernel
+            _ffi.check(_ffi.lib().tq_set_option(b"append_small", mode), "tq_set_option")
+            pool, _ = _make_pool(gpu, d, key_bits, vb, H, B * pages, dtype)
+            pool.data.fill_(0x3C)
+            _progress(f"single-token append d={d} {dtype} B={B} append_small={mode}")
+            pool.append(k, v, table, pos)
+            torch.cuda.synchronize()
+            got[mode] = pool.data.clone()
+    finally:
+        _ffi.check(_ffi.lib().tq_set_option(b"append_small", -1), "tq_set_option")
+    assert torch.equal(got[0], got[-1]) and torch.equal(got[0], got[3])
+    assert not torch.all(got[0] == 0x3C)
+
+
 def test_paged_append_random_chunks_equal_flat_quantise(gpu):
     # seeded sweep: several sequences appended in ragged chunks (any start slot inside a page, chunk
     # lengths across page boundaries, batched calls with per-sequence start positions); the exported

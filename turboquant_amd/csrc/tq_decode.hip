@@ -963,6 +963,7 @@ std::atomic<int> opt_prefetch_trips{-1};
 std::atomic<int> opt_prep_mfma{1};
 std::atomic<int> opt_sequence_walkers{-1};
 std::atomic<int> opt_prep_words{-1};
+std::atomic<int> opt_append_small{-1};
 }  // namespace tq
 
 extern "C" int tq_set_option(const char* name, int64_t value) {
@@ -985,6 +986,11 @@ extern "C" int tq_set_option(const char* name, int64_t value) {
   }
   if (!std::strcmp(name, "tail_chunks")) { opt_tail_chunks.store(value != 0); return TQ_OK; }
   if (!std::strcmp(name, "merge_row_groups")) { opt_merge_row_groups.store(value != 0); return TQ_OK; }
+  if (!std::strcmp(name, "append_small")) {
+    if (value < -1 || value > (1 << 24)) return TQ_EINVAL;
+    opt_append_small.store((int)value);
+    return TQ_OK;
+  }
   if (!std::strcmp(name, "prep_words")) {
     if (value < -1 || value > 1) return TQ_EINVAL;
     opt_prep_words.store((int)value);

@@ -181,7 +181,8 @@ __device__ __forceinline__ void prefetch_matrix(const uint16_t* __restrict__ m_t
 // there is one, then with the first BUF slices of m_next, the matrix of the contraction that
 // follows.  Those loads have the rest of this contraction and the epilogue to arrive, and
 // the requests of a workgroup are spread out instead of coming in one burst.
-template <int D, int NA, bool REFILL = true>
+// (ML: the group's first ML tiles hold vectors; the others are not computed)
+template <int D, int NA, bool REFILL = true, int ML = KeyGeom<D>::MT>
 __device__ __forceinline__ void contract(const uint16_t* a_terms, const uint16_t* __restrict__ m_terms,
                                          const uint16_t* __restrict__ m_next, int wave, int lane, MatRegs<D>& mr,
                                          f32x4 (&acc)[KeyGeom<D>::MT][KeyGeom<D>::NPW]) {
@@ -189,7 +190,7 @@ __device__ __forceinline__ void contract(const uint16_t* a_terms, const uint16_t
   constexpr int MT = Gm::MT, NPW = Gm::NPW, KB = Gm::KB, RS = Gm::RS, BUF = MatRegs<D>::BUF;
   const int n = lane & 15, kb = lane >> 4;
 #pragma unroll
-  for (int m = 0; m < MT; ++m)
+  for (int m = 0; m < ML; ++m)
 #pragma unroll
     for (int c = 0; c < NPW; ++c) acc[m][c] = f32x4{0, 0, 0, 0};
 #pragma unroll
@@ -199,13 +200,13 @@ __device__ __forceinline__ void contract(const uint16_t* a_terms, const uint16_t
     for (int a = 0; a < NA; ++a) {
       u32x4 av[MT];
 #pragma unroll
-      for (int m = 0; m < MT; ++m)
+      for (int m = 0; m < ML; ++m)
         av[m] = *(const u32x4*)(a_terms + ((size_t)a * Gm::TT + 16 * m + n) * RS + 32 * kblk + 8 * kb);
 #pragma unroll
       for (int b = 0; b < 3; ++b)
         if (a + b <= 2) {
 #pragma unroll
-          for (int m = 0; m < MT; ++m)
+          for (int m = 0; m < ML; ++m)
 #pragma unroll
             for (int c = 0; c < NPW; ++c) acc[m][c] = mfma_bf16(mr.b[kblk % BUF][c][b], av[m], acc[m][c]);
         }
@@ -276,11 +277,13 @@ struct XStage {
     }
   }
   // uniform part for `group`: tile addresses, and (paged sources) the coordinates of tile group * MT + wtile
+  // (ML: tiles of a group that hold vectors - groups are ML tiles apart; the other MT - ML are not loaded)
+  template <int ML = Gm::MT>
   __device__ __forceinline__ void lookup(const Source& src, int64_t group, int64_t n_tiles, int wtile) {
-    const int64_t tile0 = group * Gm::MT;
+    const int64_t tile0 = group * ML;
     const int64_t first = tile0 < n_tiles ? tile0 : 0;
 #pragma unroll
-    for (int m = 0; m < Gm::MT; ++m) live[m] = tile0 + m < n_tiles;
+    for (int m = 0; m < Gm::MT; ++m) live[m] = m < ML && tile0 + m < n_tiles;
     if constexpr (std::is_same<Source, PagedSource>::value) {
       PagedSource::Coord c[Gm::MT];
       int lpage[Gm::MT];
@@ -330,7 +333,9 @@ struct XStage {
 // operand (a plane word turns into fp4 codes with four ANDs), and Pi^T is the fp6 operand, cut into five
 // fp6 digits per value on the host (good to 2^-23 of a block's largest value: below the rounding noise of an
 // fp32 product sum).  10 MFMAs per 16 x 16 tile instead of 24, and no centroid terms go through the LDS.
-template <int DT, int D, bool MSE_ONLY, bool FX, class Source, class Sink>
+// ML (1 or the MT tiles of a group): small appends - the page write of a decode step - give every 16-vector tile a
+// workgroup of its own that computes one tile instead of four, a quarter of the instructions behind one another.
+template <int DT, int D, bool MSE_ONLY, bool FX, class Source, class Sink, int ML = KeyGeom<D>::MT>
 __global__ void __launch_bounds__(KQ_THREADS, 2)
 key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, int64_t n_tiles) {
   static_assert(!FX || (D == 128 && !MSE_ONLY), "the fp6 centroid contraction: head_dim 128, full quantiser");
@@ -343,7 +348,7 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
   constexpr int XRS = Sm::XRS, TPR = Gm::TPR, SEG = Gm::SEG;
   const int tid0 = threadIdx.x, wave0 = __builtin_amdgcn_readfirstlane(tid0 >> 6);
   const int mb = ly.mse_bits, n_thr = (1 << mb) - 1;
-  const int64_t n_groups = (n_tiles + MT - 1) / MT;             // a group = the TT vectors of one pass
+  const int64_t n_groups = (n_tiles + ML - 1) / ML;             // a group = the TT vectors of one pass
   MatRegs<D> mr;
   prefetch_matrix<D>(ly.Pi_split, wave0, tid0 & 63, mr);        // in flight while the vectors are staged
 
@@ -387,7 +392,7 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
   // (1) staging (XStage): the next group's chunks wait in registers while the current group is worked on
   XStage<DT, D, Source> stg;
   stg.init(src, tid0);
-  stg.lookup(src, blockIdx.x, n_tiles, wave0 % MT);
+  stg.template lookup<ML>(src, blockIdx.x, n_tiles, wave0 % ML);
   stg.issue(x);
 
   for (int64_t g = blockIdx.x; g < n_groups; g += gridDim.x) {
@@ -396,16 +401,16 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
   int tid = tid0, wave = wave0;
   asm volatile("" : "+v"(tid), "+s"(wave));
   const int lane = tid & 63, n = lane & 15, kb = lane >> 4;
-  const int64_t tile0 = g * MT;
+  const int64_t tile0 = g * ML;
   // coordinates of the tile this wavefront writes: looked up one pass ago together with this group's loads;
   // then the lookups of the group to fetch next (long before issue() needs them)
   const int wr_b = stg.w_b, wr_lpage = stg.w_lpage, wr_h = stg.w_h;
-  stg.lookup(src, g + gridDim.x, n_tiles, wave % MT);
+  stg.template lookup<ML>(src, g + gridDim.x, n_tiles, wave % ML);
   // page of that tile, read now so that the write phase does not wait for it (a page outside the table or
   // the pool comes back as -1 and is not written)
   int64_t wpage = 0;
   if constexpr (!std::is_same<Sink, KeyFlatSink>::value) {
-    if (tile0 + wave % MT < n_tiles) wpage = checked_page(sink.block_table, sink.max_pages, sink.num_pages, wr_b, wr_lpage);
+    if (tile0 + wave % ML < n_tiles) wpage = checked_page(sink.block_table, sink.max_pages, sink.num_pages, wr_b, wr_lpage);
   }
   stg.template store<XRS>(sx, svalid, tid);
   __syncthreads();
@@ -465,7 +470,7 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
   // (3) y = u Pi^T, bucketise; index bit planes; centroid values as bf16 terms for the next contraction
   // (FX: the matrix registers stay free after this contraction; the fp6 digits of Pi^T take their place until
   // the centroid contraction is done, then S is requested and has the residual pass to arrive)
-  contract<D, NA1, !FX>(terms, ly.Pi_split, mse_only ? ly.Pi_split : ly.PiT_split, wave, lane, mr, acc);
+  contract<D, NA1, !FX, ML>(terms, ly.Pi_split, mse_only ? ly.Pi_split : ly.PiT_split, wave, lane, mr, acc);
   i32x8 fa[FX ? NPW : 1][FX ? FXT : 1];
   if constexpr (FX) {
 #pragma unroll
@@ -489,7 +494,7 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
       for (int i = 0; i < 4; ++i) bitc[h][i] = 1u << (16 * h + 4 * kb + i);
     const float t0 = sthr[0], t1 = mb == 2 ? sthr[1] : 0.0f, t2 = mb == 2 ? sthr[2] : 0.0f;
 #pragma unroll
-    for (int m = 0; m < MT; ++m) {
+    for (int m = 0; m < ML; ++m) {
       const int t = 16 * m + n;
 #pragma unroll
       for (int wl = 0; wl < NPW / 2; ++wl) {
@@ -526,7 +531,7 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
   } else {
     uint32_t idx[MT][NPW][4];
 #pragma unroll
-    for (int m = 0; m < MT; ++m)
+    for (int m = 0; m < ML; ++m)
 #pragma unroll
       for (int c = 0; c < NPW; ++c)
 #pragma unroll
@@ -534,14 +539,14 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
     for (int k = 0; k < n_thr; ++k) {                           // searchsorted: count thresholds below y (NaN counts all)
       const float th = sthr[k];
 #pragma unroll
-      for (int m = 0; m < MT; ++m)
+      for (int m = 0; m < ML; ++m)
 #pragma unroll
         for (int c = 0; c < NPW; ++c)
 #pragma unroll
           for (int i = 0; i < 4; ++i) idx[m][c][i] += !(acc[m][c][i] <= th);
     }
 #pragma unroll
-    for (int m = 0; m < MT; ++m) {
+    for (int m = 0; m < ML; ++m) {
       const int t = 16 * m + n;
       for (int p = 0; p < mb; ++p) {
         const int sh = mb - 1 - p;
@@ -588,7 +593,7 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
       auto plane = [&](int p, f32x4 (&part)[MT][NPW]) {
         u32x4 b[MT];
 #pragma unroll
-        for (int m = 0; m < MT; ++m) {
+        for (int m = 0; m < ML; ++m) {
           const uint32_t w = spl[(p * TT + 16 * m + n) * W + kb];
           b[m] = u32x4{w & 0x11111111u, w & 0x22222222u, w & 0x44444444u, (w >> 3) & 0x11111111u};
 #pragma unroll
@@ -596,23 +601,23 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
         }
         // digit by digit over all tiles: consecutive MFMAs go to different accumulators
 #pragma unroll
-        for (int m = 0; m < MT; ++m)
+        for (int m = 0; m < ML; ++m)
 #pragma unroll
           for (int c = 0; c < NPW; ++c) part[m][c] = mfma_fp6_fp4<0>(fa[c][0], b[m], part[m][c], fs0[c], 127);
 #pragma unroll
-        for (int m = 0; m < MT; ++m)
+        for (int m = 0; m < ML; ++m)
 #pragma unroll
           for (int c = 0; c < NPW; ++c) part[m][c] = mfma_fp6_fp4<1>(fa[c][1], b[m], part[m][c], fs0[c], 127);
 #pragma unroll
-        for (int m = 0; m < MT; ++m)
+        for (int m = 0; m < ML; ++m)
 #pragma unroll
           for (int c = 0; c < NPW; ++c) part[m][c] = mfma_fp6_fp4<2>(fa[c][2], b[m], part[m][c], fs0[c], 127);
 #pragma unroll
-        for (int m = 0; m < MT; ++m)
+        for (int m = 0; m < ML; ++m)
 #pragma unroll
           for (int c = 0; c < NPW; ++c) part[m][c] = mfma_fp6_fp4<3>(fa[c][3], b[m], part[m][c], fs0[c], 127);
 #pragma unroll
-        for (int m = 0; m < MT; ++m)
+        for (int m = 0; m < ML; ++m)
 #pragma unroll
           for (int c = 0; c < NPW; ++c) part[m][c] = mfma_fp6_fp4<0>(fa[c][4], b[m], part[m][c], fs1[c], 127);
       };
@@ -620,7 +625,7 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
         f32x4 part[MT][NPW];
         plane(0, part);
 #pragma unroll
-        for (int m = 0; m < MT; ++m)
+        for (int m = 0; m < ML; ++m)
 #pragma unroll
           for (int c = 0; c < NPW; ++c)
 #pragma unroll
@@ -628,7 +633,7 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
         if (mb == 2) {
           plane(1, part);
 #pragma unroll
-          for (int m = 0; m < MT; ++m)
+          for (int m = 0; m < ML; ++m)
 #pragma unroll
             for (int c = 0; c < NPW; ++c)
 #pragma unroll
@@ -637,11 +642,11 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
       }
       prefetch_matrix<D>(ly.S_split, wave, lane, mr);
     } else {
-      contract<D, 3>(terms, ly.PiT_split, ly.S_split, wave, lane, mr, acc);
+      contract<D, 3, true, ML>(terms, ly.PiT_split, ly.S_split, wave, lane, mr, acc);
       __syncthreads();                                          // every wavefront has read the centroid terms
     }
 #pragma unroll
-    for (int m = 0; m < MT; ++m) {
+    for (int m = 0; m < ML; ++m) {
       const int t = 16 * m + n;
       const float nrm = snorm[t];
       float rs = 0.0f;
@@ -674,9 +679,9 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
       srn[tid] = sqrtf(v);
     }
     // (5) p = r S^T ; sign bits (quantizer.py:248-249)
-    contract<D, 3>(terms, ly.S_split, ly.Pi_split, wave, lane, mr, acc);    // Pi again for the next group
+    contract<D, 3, true, ML>(terms, ly.S_split, ly.Pi_split, wave, lane, mr, acc);    // Pi again for the next group
 #pragma unroll
-    for (int m = 0; m < MT; ++m) {
+    for (int m = 0; m < ML; ++m) {
       const int t = 16 * m + n;
 #pragma unroll
       for (int wl = 0; wl < NPW / 2; ++wl) {
@@ -742,16 +747,16 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
     // pages: a wavefront writes the bit-plane words of one tile, so the page lookup is uniform;
     // lanes run over (word, token) in page order (lane-major: [w & 3][token][w >> 2][plane])
     const tq_page_layout& L = sink.L;
-    constexpr int NSUB = KQ_WAVES / MT > 0 ? KQ_WAVES / MT : 1;   // wavefronts that share a tile
+    constexpr int NSUB = KQ_WAVES / ML > 0 ? KQ_WAVES / ML : 1;   // wavefronts that share a tile
     const int planes = mb + 1;
-    for (int m = wave % MT; m < MT; m += KQ_WAVES) {
+    for (int m = wave % ML; m < ML; m += KQ_WAVES) {
       const int64_t tile = tile0 + m;
       if (tile >= n_tiles) break;
       // a tile none of whose slots exists may lie beyond the block table: do not look it up
       // (and a page outside the table or the pool is not written)
       if (__builtin_amdgcn_ballot_w64(lane < TILE && svalid[16 * m + lane]) == 0 || wpage < 0) continue;
       uint8_t* pg = sink.pool + (wpage * src.H + wr_h) * (int64_t)L.page_bytes;
-      for (int p = wave / MT; p < planes; p += NSUB) {
+      for (int p = wave / ML; p < planes; p += NSUB) {
 #pragma unroll
         for (int e = lane; e < W * TILE; e += 64) {
           const int jh = e % (W / 4), nn = (e / (W / 4)) % TILE, jl = e / (W / 4) / TILE;
@@ -760,7 +765,7 @@ key_mfma_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
             *(uint32_t*)(pg + key_word_off(L, p, w, nn)) = (p == mb && mse_only) ? 0u : spl[(p * TT + 16 * m + nn) * W + w];
         }
       }
-      if (wave / MT == 0 && lane < TILE && svalid[16 * m + lane]) {
+      if (wave / ML == 0 && lane < TILE && svalid[16 * m + lane]) {
         float* meta = (float*)(pg + L.off_meta);
         meta[2 * lane] = snorm[16 * m + lane];
         meta[2 * lane + 1] = mse_only ? 0.0f : srn[16 * m + lane];
@@ -787,12 +792,19 @@ __host__ static bool sink_ok(const KeyFlatSink& s, int mse_only) {
 }
 __host__ static bool sink_ok(const KeyPagedSink& s, int) { return s.L.key_lane_major != 0; }
 
-template <int DT, int D, bool MSE_ONLY, bool FX, class Source, class Sink>
+template <int DT, int D, bool MSE_ONLY, bool FX, class Source, class Sink, int ML = KeyGeom<D>::MT>
 static int launch_dt_d(const void* x, const Source& src, const tq_layer& ly, const Sink& sink, int64_t tiles,
                        hipStream_t st) {
   using Gm = KeyGeom<D>;
   using Sm = KeySmem<DT, D>;
-  auto kern = key_mfma_kernel<DT, D, MSE_ONLY, FX, Source, Sink>;
+  // Few tiles, written to pages (the page write of a decode step: a token per sequence): a workgroup per tile, which
+  // then computes that tile only, while they all fit the card at once
+  if constexpr (ML == Gm::MT && std::is_same<Sink, KeyPagedSink>::value && !MSE_ONLY) {
+    const int opt = opt_append_small.load(std::memory_order_relaxed);
+    if (opt != 0 && tiles <= (opt < 0 ? 2 * (int64_t)device_compute_units() : (int64_t)opt))
+      return launch_dt_d<DT, D, MSE_ONLY, FX, Source, Sink, 1>(x, src, ly, sink, tiles, st);
+  }
+  auto kern = key_mfma_kernel<DT, D, MSE_ONLY, FX, Source, Sink, ML>;
   static std::atomic<uint64_t> configured{0};           // per instantiation, one bit per device; the attribute is sticky
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return TQ_EINVAL;
@@ -809,7 +821,7 @@ static int launch_dt_d(const void* x, const Source& src, const tq_layer& ly, con
     if (dev < 64) n_cu[dev].store(cus, std::memory_order_relaxed);
   }
   const int per_cu = (int)(160 * 1024 / Sm::bytes) > 2 ? 2 : (int)(160 * 1024 / Sm::bytes);
-  const int64_t groups = (tiles + Gm::MT - 1) / Gm::MT;
+  const int64_t groups = (tiles + ML - 1) / ML;
   const int64_t resident = (int64_t)cus * (per_cu > 0 ? per_cu : 1);
   const unsigned grid = (unsigned)(groups < resident ? groups : resident);
   hipEvent_t ev_start = nullptr, ev_stop = nullptr;
