@@ -237,6 +237,12 @@ int tq_pool_export(const uint8_t *pool, int64_t num_pages, int H, const int32_t 
                    const tq_page_layout *layout, uint8_t *idx, uint8_t *signs, void *norms, float *rnorms,
                    uint8_t *v_data, void *v_scales, void *v_zeros, void *stream);
 
+/* No counterpart in the reference: which page kernel a decode step over this layer and page layout runs (with at
+ * most 8 query heads per group of a KV head; the current options applied): 0 the general vector-ALU kernel,
+ * 1 the matrix-core kernel of head_dim 64 / 128 / 256 (a block of 64 tokens per wavefront), 2 the matrix-core
+ * kernel of the head sizes 320 .. 704 (a block of 32 tokens per workgroup).  Negative: an error code.           */
+int tq_decode_page_kernel(const tq_layer *layer /*host*/, const tq_page_layout *layout /*host*/);
+
 /* Bytes of workspace tq_decode_attn_paged needs for these sizes.                   */
 size_t tq_decode_workspace_bytes(int B, int Hq, int d, int n_split);
 

@@ -214,6 +214,39 @@ def test_decode_head_dim_576_with_4_bit_keys(gpu, vb, Hq, Hkv, dtype):
     _progress(f"   worst cosine {worst:.7f}")
 
 
+# ------------------------------------------------------------------ head sizes above 256 on the matrix cores
+@pytest.mark.parametrize("d,key_bits,vb,Hq,Hkv,dtype,lens,recent,n_split", [
+    (576, 4, 4, 8, 1, torch.bfloat16, [300, 77, 1], None, None),
+    (576, 4, 2, 16, 1, torch.bfloat16, [300, 77], [0, 9], 3),          # 16 heads per KV head: two groups of 8; exact tail
+    (576, 4, 8, 8, 2, torch.bfloat16, [130, 513], None, 2),            # 8-bit values (a ring of two blocks)
+    (576, 4, 4, 8, 2, torch.float16, [300, 77], [5, 0], None),         # fp16 pages: zero points on the fp16 MFMA
+    (576, 3, 4, 11, 1, torch.bfloat16, [700, 33], None, 4),            # 11 heads: groups of 6 and 5; 3-bit keys
+    (512, 3, 4, 8, 2, torch.bfloat16, [300, 77], None, None),          # a multiple of 128: lane-major key words
+    (512, 4, 2, 4, 4, torch.bfloat16, [64, 1000], None, 5),
+    (320, 3, 2, 5, 1, torch.bfloat16, [257, 31], None, 2),             # five wavefronts, two and a half chunks
+    (704, 3, 2, 8, 1, torch.bfloat16, [300, 77], None, None),          # the widest head the kernel takes
+    (640, 2, 4, 3, 1, torch.bfloat16, [2100, 500], None, 2)])          # 2-bit keys; table registers move on (more than 64 pages)
+def test_decode_wide_heads_on_the_matrix_cores(gpu, d, key_bits, vb, Hq, Hkv, dtype, lens, recent, n_split):
+    """Head sizes above 256 (512 / 576: the latent sizes the reference's layer set-up meets, integration/vllm.py:376-381)
+    run the matrix-core kernel that works on a block of 32 tokens per workgroup: against the oracle on the same
+    store (ragged lengths, splits without tokens, an exact tail), and against the general kernel, which the
+    option "wide_heads" = 0 selects."""
+    pool, _ = _make_pool(gpu, d, key_bits, vb, Hkv, 4, dtype)
+    assert pool.page_kernel() == 2, "the shape has no wide-head kernel"
+    outs = {}
+    try:
+        for mode in (1, 0):
+            _set_option("wide_heads", mode)
+            _progress(f"decode d={d} kb={key_bits} vb={vb} Hq={Hq} Hkv={Hkv} {dtype} n_split={n_split} wide_heads={mode}")
+            outs[mode] = _decode_case(gpu, d, key_bits, vb, len(lens), Hq, Hkv, lens, recent, seed=700 + d + vb,
+                                      n_split=n_split, dtype=dtype, return_out=True)
+    finally:
+        _set_option("wide_heads", 1)
+    c = cosine(outs[1], outs[0])
+    _progress(f"   wide-head kernel against the general kernel: cosine {c:.7f}")
+    assert c >= COS_GATE
+
+
 # ------------------------------------------------------------------ block tables are bounded on the device
 @pytest.mark.parametrize("d,key_bits,vb,dtype,T", [(128, 3, 4, torch.bfloat16, 70), (256, 3, 2, torch.bfloat16, 5000),
                                                      (64, 2, 2, torch.float16, 70), (128, 3, 2, torch.float32, 40),

@@ -70,6 +70,7 @@ _SIGNATURES = {
     "tq_append_kv_from_blocks": (C.c_int, [_vp, _vp, _i, _i, _i, _i, _i64, _i64, _i64, _vp, _i, _vp, _vp, _vp, _i,
                                            C.POINTER(TqLayer), C.POINTER(TqPageLayout), _vp, _i64, _vp]),
     "tq_pool_export": (C.c_int, [_vp, _i64, _i, _vp, _i, C.POINTER(TqPageLayout), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "tq_decode_page_kernel": (C.c_int, [C.POINTER(TqLayer), C.POINTER(TqPageLayout)]),
     "tq_decode_workspace_bytes": (C.c_size_t, [_i, _i, _i, _i]),
     "tq_decode_attn_paged": (C.c_int, [_vp, _i, _i, _i, _i, _vp, _i64, _vp, _i, _vp, _f, C.POINTER(TqLayer),
                                        C.POINTER(TqPageLayout), _vp, _vp, _i, _i64, _i64, _i64, _vp, _vp, _vp, _i, _vp]),

@@ -15,7 +15,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libtq_hip.so")
 # (the matrix-core page kernel is instantiated by one file per head size, so that they compile side by side)
 SOURCES = ["tq_decode_mfma_d128.hip", "tq_decode_mfma_d128_f16.hip", "tq_decode_mfma_d64.hip", "tq_decode_mfma_d64_f16.hip",
-           "tq_decode_mfma_d256.hip", "tq_quantize_mfma.hip",
+           "tq_decode_mfma_d256.hip", "tq_quantize_mfma.hip", "tq_decode_wide.hip",
            "tq_quantize.hip", "tq_score.hip", "tq_decode.hip", "tq_decode_mfma.hip", "tq_probe.hip"]
 
 # packed-fp32 instructions stay off: some of their forms have produced wrong

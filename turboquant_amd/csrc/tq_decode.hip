@@ -964,6 +964,7 @@ std::atomic<int> opt_prep_mfma{1};
 std::atomic<int> opt_sequence_walkers{-1};
 std::atomic<int> opt_prep_words{-1};
 std::atomic<int> opt_append_small{-1};
+std::atomic<int> opt_wide_heads{1};
 }  // namespace tq
 
 extern "C" int tq_set_option(const char* name, int64_t value) {
@@ -986,6 +987,7 @@ extern "C" int tq_set_option(const char* name, int64_t value) {
   }
   if (!std::strcmp(name, "tail_chunks")) { opt_tail_chunks.store(value != 0); return TQ_OK; }
   if (!std::strcmp(name, "merge_row_groups")) { opt_merge_row_groups.store(value != 0); return TQ_OK; }
+  if (!std::strcmp(name, "wide_heads")) { opt_wide_heads.store(value != 0); return TQ_OK; }
   if (!std::strcmp(name, "append_small")) {
     if (value < -1 || value > (1 << 24)) return TQ_EINVAL;
     opt_append_small.store((int)value);
@@ -1011,6 +1013,12 @@ extern "C" int tq_set_option(const char* name, int64_t value) {
     return TQ_OK;
   }
   return TQ_EINVAL;
+}
+
+extern "C" int tq_decode_page_kernel(const tq_layer* layer, const tq_page_layout* layout) {
+  if (!layer || !layout) return TQ_ENULL;
+  if (layer->Pi_colsum && layer->S_colsum && decode_mfma_has_kernel(*layer, *layout)) return 1;
+  return decode_wide_has_kernel(*layer, *layout) ? 2 : 0;
 }
 
 extern "C" size_t tq_decode_workspace_bytes(int B, int Hq, int d, int n_split) {
@@ -1272,6 +1280,12 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
                     : TQ_EUNSUPPORTED;
   if (mf > 0) return mf;
   if (mf == TQ_OK && fm.out != nullptr) return TQ_OK;         // merged in the launch
+  // head sizes above 256: the matrix-core kernel that works on a block per workgroup
+  if ((stages & 2) && mf == TQ_EUNSUPPORTED) {
+    mf = launch_decode_wide(q_rot, q_sk, B, Hq, Hkv, pool, block_table, bt_stride, seq_lens, sm_scale, *layer, *layout,
+                            parts, n_parts, n_split, len_sub, max_pages, pool_pages, st);
+    if (mf > 0) return mf;
+  }
   if ((stages & 2) && mf == TQ_EUNSUPPORTED) {      // no matrix-core kernel for this shape: general kernel
     if (dtype < TQ_F32 || dtype > TQ_BF16) return TQ_EINVAL;
     const int gp4 = (G + 3) / 4, gp = 4 * gp4;      // query heads rounded up to a multiple of 4

@@ -114,6 +114,15 @@ int launch_decode_mfma(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv,
                        int max_pages, int num_pages, const FusedMerge& fm, bool wide_wg,
                        hipStream_t st);
 
+// The matrix-core kernel for head sizes above 256 (tq_decode_wide.hip; a workgroup per block of 32 tokens): reads the
+// fp32 rotated / sketched queries the general kernel reads and writes the same partials.  TQ_EUNSUPPORTED when the
+// shape has no such kernel (nothing was launched).
+bool decode_wide_has_kernel(const tq_layer& ly, const tq_page_layout& L);
+int launch_decode_wide(const float* q_rot, const float* q_sk, int B, int Hq, int Hkv, const uint8_t* pool,
+                       const int32_t* block_table, int bt_stride, const int32_t* seq_lens, float sm_scale,
+                       const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts, int n_split, int len_sub,
+                       int max_pages, int num_pages, hipStream_t st);
+
 // Whether a step of this shape runs workgroups of eight wavefronts: the caller then passes HALF its split count
 // (and wide_wg = true) to launch_decode_mfma and uses that count for everything that follows.
 bool decode_mfma_wide_workgroups(int d, int G, int n_split, int max_pages);

@@ -1,0 +1,745 @@
+// Page kernel on the matrix cores for wide heads: head_dim a multiple of 64 above 256, up to 704 (512 and 576 are the
+// latent sizes of multi-head latent attention; the reference ships a codebook for 576, codebooks/codebook_d576_b3.json,
+// and sizes its layers from impl.head_size / impl.kv_lora_rank, integration/vllm.py:376-381).  Same semantics as the
+// other page kernels (score.py:114-173 over compressed pages): partials (m, l, acc[d]) per context split.
+//
+// A wide head does not fit the per-wavefront design of the head_dim 64 / 128 / 256 kernel (its query operands and
+// accumulators would need several hundred registers), so here a whole workgroup works on one block of 32 tokens
+// (two pages) at a time:
+//   * one wavefront per 64 channels plus a helper wavefront (d + 64 threads), one workgroup per compute unit;
+//   * the pages travel HBM -> LDS as they lie in memory (LDS-direct loads, a kilobyte per instruction), the key
+//     part of a page (bit planes, norms) and its value part (codes, scales, zero points) into rings of their
+//     own, two or three blocks deep, so that the next block(s) arrive while the current ones are worked on;
+//   * the fp6 query operands of v_mfma_scale_f32_16x16x128_f8f6f4 (four terms per value, as the preparation
+//     kernel of the other sizes packs them) are built by the workgroup itself from the fp32 rotated / sketched
+//     queries and stay in LDS;
+//   * scores: the (page, 128-coordinate chunk) pairs of a block are dealt to the wavefronts, the stored bit
+//     planes are the fp4 operand, partial sums meet in LDS;
+//   * softmax: the helper wavefront, online, log2 domain, against a reference that moves lazily;
+//   * values: every wavefront takes the two groups of 32 channels it owns: codes masked in place are bf16
+//     denormals (B operand), softmax weight x group scale is the A operand (rows 0..7 the heads with the even
+//     group's scales, rows 8..15 with the odd group's), zero points through one more MFMA.
+// The stages are pipelined over the blocks: while the wavefronts accumulate the values of block j they score
+// block j + 1; its softmax follows.  Two workgroup barriers per block.  The step's other launches (rotation,
+// exact tail, merge) are those of the general kernel.
+
+#include "tq_decode_mfma_impl.h"
+
+namespace tq {
+
+constexpr int WD_BLK = 32;                 // tokens per iteration (two pages)
+constexpr int WD_QA_OP = 64 * 6;           // dwords of one packed operand: [64 lanes][4] then [64 lanes][2]
+constexpr int WD_MAX_WAVES = 12;           // head_dim 768
+constexpr int WD_MAX_CHUNKS = 6;           // 128-coordinate chunks of head_dim 768
+constexpr int WD_SMALL_FLOATS = 256 + 256 + 8 + 8 + 32 + 16 + 16 + WD_MAX_WAVES * 32;     // s_p, s_pv, s_alpha, s_flag, s_stat, s_mult, s_coef, s_z
+constexpr int WD_LDS_BYTES = 160 * 1024;
+
+// -DWD_PROF (a profiling build, never the shipped one): every wavefront of workgroup (0, 0, 0) sums the time it
+// spends in each part of an iteration (100 MHz counter); tq_debug_wide_prof copies the sums out.
+#ifdef WD_PROF
+__device__ unsigned long long wd_prof[WD_MAX_WAVES * 8];
+#define WD_T(k) do { const unsigned long long t_ = wall_clock64(); wd_t[k] += t_ - wd_last; wd_last = t_; } while (0)
+#else
+#define WD_T(k)
+#endif
+
+__device__ __forceinline__ void wd_wait_vm(int n) {
+  switch (n) {
+    case 0: stage_wait<0>(); break;
+    case 1: stage_wait<1>(); break;
+    case 2: stage_wait<2>(); break;
+    case 3: stage_wait<3>(); break;
+    case 4: stage_wait<4>(); break;
+    case 5: stage_wait<5>(); break;
+    case 6: stage_wait<6>(); break;
+    case 7: stage_wait<7>(); break;
+    case 8: stage_wait<8>(); break;
+    case 9: stage_wait<9>(); break;
+    case 10: stage_wait<10>(); break;
+    case 11: stage_wait<11>(); break;
+    case 12: stage_wait<12>(); break;
+    case 13: stage_wait<13>(); break;
+    case 14: stage_wait<14>(); break;
+    case 15: stage_wait<15>(); break;
+    case 16: stage_wait<16>(); break;
+    default: stage_wait<0>(); break;       // (stricter than asked: always safe)
+  }
+}
+
+// MB stored index planes; the codebooks the quantiser makes have NX = 0, 0, 1, 4 multi-bit Walsh terms for
+// MB = 1..4, so MB + NX + 1 term planes go through the score MFMAs.
+template <int VB, int MB>
+__global__ void __launch_bounds__(768)
+decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_sk, int Hq, int Hkv, int kv_div,
+                   const uint8_t* __restrict__ pool, const int32_t* __restrict__ block_table, int bt_stride,
+                   const int32_t* __restrict__ seq_lens, float sm_scale, tq_layer ly, tq_page_layout L,
+                   float* __restrict__ parts, int n_parts, int n_split, int len_sub, int max_pages, int num_pages,
+                   int nring, int kslot, int vslot) {
+  constexpr int NX = MB == 3 ? 1 : (MB == 4 ? 4 : 0), NTP = MB + NX + 1;
+  const bool f16p = L.dtype == TQ_F16;
+  const int d = ly.d, W = d >> 5, WPLT = (d + 127) >> 7;
+  const int tid = threadIdx.x, lane = tid & 63;
+  // NW wavefronts own 64 channels each; one more (the helper, wavefront NW) owns none: it runs the softmax and takes
+  // score units like the others (head_dim 576: ten units for ten wavefronts)
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), NW = ((int)blockDim.x >> 6) - 1, NWS = NW + 1;
+  const bool helper = wave == NW;
+  const int n = lane & 15, kb = lane >> 4;
+  const int split = blockIdx.x, b = blockIdx.z;
+  // the query heads of a KV head form kv_div groups of at most 8 (consecutive groups read the same pages)
+  const int g_tot = Hq / Hkv, kvh = (int)blockIdx.y / kv_div, grp = (int)blockIdx.y - kvh * kv_div;
+  const int g_max = (g_tot + kv_div - 1) / kv_div;
+  const int qbase = kvh * g_tot + grp * g_max;
+  const int G = min(g_max, g_tot - grp * g_max);
+  if (G <= 0) return;
+
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  uint32_t* qa_lds = (uint32_t*)smem_raw;                         // [NTP][WPLT][2 row sets][WD_QA_OP]
+  float* s_part = (float*)(qa_lds + NTP * WPLT * 2 * WD_QA_OP);   // [2 WPLT units][64 lanes][4]
+  float* s_p = s_part + 2 * WPLT * 256;                           // [8 heads][32 tokens] softmax weights
+  float* s_pv = s_p + 256;                                        // the same weights times 2^(80 - bit position of the token's code)
+  float* s_alpha = s_pv + 256;                                    // [8]
+  int* s_flag = (int*)(s_alpha + 8);                              // [0]: the block's softmax moved a reference
+  float* s_stat = s_alpha + 16;                                   // [8][4]: E_index, E_sign, constant parts of the score
+  float* s_mult = s_stat + 32;                                    // [8][2]: multipliers of q_rot / q_sk
+  float* s_coef = s_mult + 16;                                    // [16] coefficient of each term plane
+  float* s_z = s_coef + 16;                                       // [waves][16 rows][2 groups] zero-point sums
+  unsigned char* kring = (unsigned char*)(s_z + WD_MAX_WAVES * 32);   // [nring][2 pages][kslot]: bytes [0, off_vdata) of a page
+  unsigned char* vring = kring + nring * 2 * kslot;                   // [nring][2 pages][vslot]: bytes [off_vdata, page_bytes)
+
+  // ---------------------------------------------------------------- work range
+  const int seq_len = max(min(seq_lens[b], max_pages * TQ_PAGE_TOKENS) - len_sub, 0);
+  const int n_pages = (seq_len + TQ_PAGE_TOKENS - 1) / TQ_PAGE_TOKENS;
+  const int n_blocks = (seq_len + WD_BLK - 1) / WD_BLK;
+  const int per_split = (n_blocks + n_split - 1) / n_split;
+  const int blk_begin = split * per_split, blk_end = min(blk_begin + per_split, n_blocks);
+  if (blk_begin >= blk_end) {                                     // nothing to read: an empty partial
+    for (int o = tid; o < G * (d + 2); o += blockDim.x) {
+      const int g = o / (d + 2), e = o - g * (d + 2);
+      parts[(((int64_t)b * Hq + qbase + g) * n_parts + split) * (d + 2) + e] = e == 0 ? MF_NEG * 0.6931471805599453f : 0.0f;
+    }
+    return;
+  }
+  const int32_t* bt = block_table + (int64_t)b * bt_stride;
+  const uint8_t* pool_h = pool + (int64_t)kvh * L.page_bytes;
+  const uint32_t page_stride32 = (uint32_t)((int64_t)Hkv * L.page_bytes);
+  // Page numbers: lane l of tbl_a holds the table entry of page pbase + l, tbl_b that of page pbase + 64 + l (entries
+  // past the end of the sequence repeat the last one, whose tokens are masked by position; an entry outside the
+  // pool becomes page 0 with the top bit set: its tokens get no weight).  Looked up with a lane read; the pair
+  // moves on 64 pages at a time, long before the entries are needed.
+  int pbase = 2 * blk_begin;
+  auto load_tbl = [&](int first) -> int {
+    const int raw = bt[min(first + lane, n_pages - 1)];
+    return (unsigned)raw < (unsigned)num_pages ? raw : (int)0x80000000;
+  };
+  int tbl_a = load_tbl(pbase), tbl_b = load_tbl(pbase + 64);
+  // (used here, so that the compiler waits for the loads here and knows of no pending load inside the loop: a wait of
+  // its own there would be for everything outstanding, the page requests included)
+  asm volatile("" : "+v"(tbl_a), "+v"(tbl_b));
+  auto page_entry = [&](int page) -> int {
+    const int rel = __builtin_amdgcn_readfirstlane(min(page, n_pages - 1) - pbase);
+    return rel < 64 ? __builtin_amdgcn_readlane(tbl_a, rel) : __builtin_amdgcn_readlane(tbl_b, rel - 64);
+  };
+  // Requests for the key part / value part of the next block of each kind into its ring slot: a kilobyte per
+  // instruction, dealt to the wavefronts; every wavefront issues the same number per block (the waits below count
+  // them), surplus ones repeat the last piece; the last piece of a part re-reads its final 16 bytes into the slot's
+  // padding.  Blocks are requested in order, so the block and its slot are running counters; behind the last block
+  // of the range the requests repeat it (into the slot it already has).  What does not depend on the block - which
+  // page of the pair, the offset inside the page, the offset inside the slot - is worked out once.
+  const int kbytes = L.off_vdata, vbytes = L.page_bytes - L.off_vdata;
+  const int PK = kslot >> 10, PV = vslot >> 10;
+  const int OPS_K = (2 * PK + NWS - 1) / NWS, OPS_V = (2 * PV + NWS - 1) / NWS, OPS = OPS_K + OPS_V;
+  constexpr int WD_MAX_OPS = 4;                 // per kind (the plan on the host keeps to it)
+  struct Req { int blk, slot; uint32_t src_off[WD_MAX_OPS]; int lds_off[WD_MAX_OPS]; int pg[WD_MAX_OPS]; };
+  auto req_init = [&](Req& r, int pieces, int slot_bytes, int part_off, int part_bytes) {
+    r.blk = blk_begin;
+    r.slot = 0;
+#pragma unroll
+    for (int k = 0; k < WD_MAX_OPS; ++k) {
+      const int piece = min(wave + k * NWS, 2 * pieces - 1);
+      const int pg = piece >= pieces ? 1 : 0, pc = piece - pg * pieces;
+      r.pg[k] = pg;
+      r.src_off[k] = (uint32_t)(part_off + min(pc * 1024 + lane * 16, part_bytes - 16));
+      r.lds_off[k] = pg * slot_bytes + pc * 1024;
+    }
+  };
+  Req rq_k, rq_v;
+  req_init(rq_k, PK, kslot, 0, kbytes);
+  req_init(rq_v, PV, vslot, kbytes, vbytes);
+  const uint32_t kring_lds = (uint32_t)(uintptr_t)kring, vring_lds = (uint32_t)(uintptr_t)vring;
+  auto issue = [&](Req& r, uint32_t ring_lds, int slot_bytes, int ops) __attribute__((always_inline)) {
+    const uint32_t pid0 = (uint32_t)page_entry(2 * r.blk) & 0x7fffffffu, pid1 = (uint32_t)page_entry(2 * r.blk + 1) & 0x7fffffffu;
+    const uint8_t* base0 = pool_h + (uint64_t)pid0 * page_stride32;
+    const uint8_t* base1 = pool_h + (uint64_t)pid1 * page_stride32;
+    const uint32_t slot_lds = ring_lds + (uint32_t)(r.slot * 2 * slot_bytes);
+#pragma unroll
+    for (int k = 0; k < WD_MAX_OPS; ++k)
+      if (k < ops)
+        dma16<0>((r.pg[k] ? base1 : base0) + r.src_off[k], (uint32_t)__builtin_amdgcn_readfirstlane((int)(slot_lds + (uint32_t)r.lds_off[k])));
+    if (r.blk < blk_end - 1) {
+      ++r.blk;
+      r.slot = r.slot + 1 == nring ? 0 : r.slot + 1;
+    }
+  };
+  auto issue_keys = [&]() __attribute__((always_inline)) { issue(rq_k, kring_lds, kslot, OPS_K); };
+  auto issue_vals = [&]() __attribute__((always_inline)) { issue(rq_v, vring_lds, vslot, OPS_V); };
+  // the first blocks are on their way while the operands are prepared: the keys of the first block, then groups of
+  // (keys of block i + 1, values of block i)
+  issue_keys();
+  for (int i = 0; i < nring - 1; ++i) {
+    issue_keys();
+    issue_vals();
+  }
+
+  // ---------------------------------------------------------------- query operands (as the preparation kernel packs them)
+  float cmax = 0.0f;
+  for (int t = 0; t < ly.n_terms; ++t) cmax = fmaxf(cmax, fabsf(ly.term_coef[t]));
+  int xpl = 0;                                  // four bits per multi-bit term: the stored planes it XORs
+  {
+    int seen = 0;
+    for (int t = 0; t < ly.n_terms; ++t) {
+      if (__builtin_popcount(ly.term_mask[t]) > 1 && seen < NX) {
+        int pl = 0;
+        for (int k2 = 0; k2 < MB; ++k2)
+          if (ly.term_mask[t] & (1 << k2)) pl |= 1 << (MB - 1 - k2);
+        xpl |= pl << (4 * seen++);
+      }
+    }
+    xpl = __builtin_amdgcn_readfirstlane(xpl);
+  }
+  if (tid < 16) {
+    float coef = 1.0f;                          // the sign plane
+    if (tid < MB) {
+      coef = 0.0f;
+      for (int t = 0; t < ly.n_terms; ++t)
+        if (ly.term_mask[t] == (1 << (MB - 1 - tid))) coef = ly.term_coef[t];
+    } else if (tid < MB + NX) {
+      coef = 0.0f;
+      int seen = 0;
+      for (int t = 0; t < ly.n_terms; ++t) {
+        if (__builtin_popcount(ly.term_mask[t]) > 1) {
+          if (seen == tid - MB) coef = ly.term_coef[t];
+          ++seen;
+        }
+      }
+    }
+    s_coef[tid] = coef;
+  }
+  // row statistics, a wavefront per head: the largest |q_rot_j| / |q_sk_j| bound the operands (a power of two
+  // 2^E above the bound goes into the MFMA's block scale), the sums give the constant parts of the score
+  for (int r = wave; r < 8; r += NWS) {
+    float mr = 0.0f, ms = 0.0f, s1 = 0.0f, s2 = 0.0f;
+    if (r < G) {
+      const float* xr = q_rot + ((int64_t)b * Hq + qbase + r) * d;
+      const float* xs = q_sk + ((int64_t)b * Hq + qbase + r) * d;
+      float x[WD_MAX_WAVES], y[WD_MAX_WAVES];   // (all loads first: one memory latency)
+#pragma unroll
+      for (int k = 0; k < WD_MAX_WAVES; ++k) {
+        const int c = min(lane + 64 * k, d - 1);
+        x[k] = xr[c];
+        y[k] = xs[c];
+      }
+#pragma unroll
+      for (int k = 0; k < WD_MAX_WAVES; ++k) {
+        const bool in = lane + 64 * k < d;
+        mr = fmaxf(mr, in ? fabsf(x[k]) : 0.0f);
+        ms = fmaxf(ms, in ? fabsf(y[k]) : 0.0f);
+        s1 += in ? x[k] : 0.0f;
+        s2 += in ? y[k] : 0.0f;
+      }
+    }
+    mr = wave_max_fast(mr); ms = wave_max_fast(ms);
+    s1 = wave_sum_fast(s1); s2 = wave_sum_fast(s2);
+    if (lane == 0) {
+      const float k = sm_scale * 1.4426950408889634f;
+      // bound < 2^e: e = exponent field - 126, kept within +-100
+      const int e1 = min(max((int)((__float_as_uint(fabsf(k) * mr * cmax) >> 23) & 255u) - 126, -100), 100);
+      const int e2 = min(max((int)((__float_as_uint(2.0f * fabsf(k * ly.qjl_scale) * ms) >> 23) & 255u) - 126, -100), 100);
+      const bool live = r < G;
+      s_stat[r * 4 + 0] = live ? (float)e1 : 0.0f;
+      s_stat[r * 4 + 1] = live ? (float)e2 : 0.0f;
+      s_stat[r * 4 + 2] = live ? k * ly.term_const * s1 : 0.0f;
+      s_stat[r * 4 + 3] = live ? -k * ly.qjl_scale * s2 : 0.0f;
+      s_mult[r * 2 + 0] = live ? k * __uint_as_float((uint32_t)(127 - e1) << 23) : 0.0f;
+      s_mult[r * 2 + 1] = live ? 2.0f * k * ly.qjl_scale * __uint_as_float((uint32_t)(127 - e2) << 23) : 0.0f;
+    }
+  }
+  __syncthreads();
+  // one lane per (term plane, head, plane word): the word's 32 values as four fp6 terms (the packing conversion
+  // of gfx950 and its inverse for the residual), written where lane (row 2 head + term % 2, quarter word % 4) of
+  // operand (plane, chunk word / 4, row set term / 2) reads them.  Rows of absent heads and the words past the
+  // head's last one (a head that is not a multiple of 128 wide) are zero.
+  {
+    typedef float f32x16_t __attribute__((ext_vector_type(16)));
+    typedef float f32x32_t __attribute__((ext_vector_type(32)));
+    typedef uint32_t u32x6_t __attribute__((ext_vector_type(6)));
+    const int n_items = NTP * 8 * 4 * WPLT;
+    for (int item = tid; item < n_items; item += blockDim.x) {
+      const int g = item & 7, j = (item >> 3) % (4 * WPLT), tp = (item >> 3) / (4 * WPLT);
+      const bool is_sign = tp == NTP - 1, live = g < G && j < W;
+      uint32_t* op0 = qa_lds + ((tp * WPLT + (j >> 2)) * 2) * WD_QA_OP;
+      const int slot0 = 2 * g + 16 * (j & 3);
+      if (!live) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          uint32_t* op = op0 + (t >> 1) * WD_QA_OP;
+          *(u32x4*)(op + (slot0 + (t & 1)) * 4) = u32x4{0, 0, 0, 0};
+          *(uint2*)(op + 64 * 4 + (slot0 + (t & 1)) * 2) = make_uint2(0u, 0u);
+        }
+        continue;
+      }
+      const float base = 4.0f * (is_sign ? s_mult[2 * g + 1] : s_coef[tp] * s_mult[2 * g]);
+      // (the rows start on 8-byte boundaries of the workspace, not always on 16-byte ones)
+      const float2* src = (const float2*)((is_sign ? q_sk : q_rot) + ((int64_t)b * Hq + qbase + g) * d + 32 * j);
+      float x[32];
+#pragma unroll
+      for (int k = 0; k < 16; ++k) {
+        const float2 v2 = src[k];
+        x[2 * k] = v2.x; x[2 * k + 1] = v2.y;
+      }
+      f32x16_t va, vb;                      // contraction indices 0, 2, 4, ... and 1, 3, 5, ...
+#pragma unroll
+      for (int kloc = 0; kloc < 32; ++kloc) {
+        const int c = 4 * (kloc & 7) + (kloc >> 3), t4 = kloc >> 3;      // coordinate within the word
+        // (the page kernel takes three of a nibble's four bits in place, as the fp4 numbers 0.5, 1, 2)
+        const float v = x[c] * (base * (t4 == 1 ? 0.5f : (t4 == 2 ? 0.25f : 1.0f)));
+        if (kloc & 1) vb[kloc >> 1] = v;
+        else va[kloc >> 1] = v;
+      }
+      const float one = 1.0f;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        u32x6_t code;
+        asm volatile("v_cvt_scalef32_2xpk16_fp6_f32 %0, %1, %2, %3" : "=&v"(code) : "v"(va), "v"(vb), "v"(one));
+        uint32_t* op = op0 + (t >> 1) * WD_QA_OP;
+        *(u32x4*)(op + (slot0 + (t & 1)) * 4) = u32x4{code[0], code[1], code[2], code[3]};
+        *(uint2*)(op + 64 * 4 + (slot0 + (t & 1)) * 2) = make_uint2(code[4], code[5]);
+        if (t < 3) {
+          f32x32_t r;
+          asm volatile("v_cvt_scalef32_pk32_f32_fp6 %0, %1, %2" : "=&v"(r) : "v"(code), "v"(one));
+#pragma unroll
+          for (int k = 0; k < 16; ++k) {
+            va[k] = (va[k] - r[2 * k]) * 32.0f;
+            vb[k] = (vb[k] - r[2 * k + 1]) * 32.0f;
+          }
+        }
+      }
+    }
+  }
+  __syncthreads();
+  // E8M0 block-scale codes of this lane's operand row (head n / 2; row 2g + t holds term t of row set 0 and term
+  // t + 2 of row set 1): index planes row set 0, 1, sign plane row set 0, 1.  4 v / 2^E is stored, so term t
+  // carries 2^(E - 2 - 5t); the fp4 bit value 0.5 carries 2^1.
+  int sa;
+  {
+    const int e1 = 127 + (int)s_stat[(n >> 1) * 4 + 0], e2 = 127 + (int)s_stat[(n >> 1) * 4 + 1];
+    const int t01 = (n & 1) ? 7 : 2, t23 = t01 + 10;
+    sa = (e1 - t01) | ((e1 - t23) << 8) | ((e2 - t01) << 16) | ((e2 - t23) << 24);
+  }
+  const int sb = 127 + 1;
+  // constant parts of the scores of the heads the helper wavefront sees in the softmax (heads 2 kb, 2 kb + 1)
+  const float c_idx0 = s_stat[(2 * kb) * 4 + 2], c_idx1 = s_stat[(2 * kb + 1) * 4 + 2];
+  const float c_sgn0 = s_stat[(2 * kb) * 4 + 3], c_sgn1 = s_stat[(2 * kb + 1) * 4 + 3];
+
+  // ---------------------------------------------------------------- state
+  f32x4 acc[4];                                 // channel tiles 4 wave .. 4 wave + 3
+#pragma unroll
+  for (int c = 0; c < 4; ++c) acc[c] = f32x4{0, 0, 0, 0};
+  f32x4 zacc = {0, 0, 0, 0};
+  float m_run[2] = {MF_NEG, MF_NEG}, l_run[2] = {0.0f, 0.0f};     // helper wavefront: heads 2 kb, 2 kb + 1
+  const uint32_t m0 = VB == 2 ? 0x00030003u : (VB == 4 ? 0x000F000Fu : 0x00FF00FFu);
+  const uint32_t m1 = VB == 2 ? 0x000C000Cu : 0x00F000F0u, m2 = 0x00300030u, m3 = 0x00C000C0u;
+  // existing tokens of page pg of block blk: a prefix (none on a page outside the pool)
+  auto tokens_of = [&](int blk, int pg) -> int {
+    return page_entry(2 * blk + pg) < 0 ? 0 : min(max(seq_len - blk * WD_BLK - 16 * pg, 0), 16);
+  };
+
+  // ---- scores of block blk: unit u = (page u % 2, chunk u / 2), dealt from the helper wavefront down
+  auto score_units = [&](int ring_slot) __attribute__((always_inline)) {
+    const unsigned char* kslot0 = kring + (ring_slot * 2) * kslot;
+    for (int u = NW - wave; u < 2 * WPLT; u += NWS) {
+      const int pg = u & 1, i = u >> 1;
+      const unsigned char* kp = kslot0 + pg * kslot;
+      const int j = 4 * i + kb;
+      const bool jl = j < W;
+      const int jc = jl ? j : W - 1;
+      // the key words, then the planes in groups of at most five: every LDS read of a group (its operands of both row
+      // sets) before the group's first MFMA
+      uint32_t kw[MB + 1];
+#pragma unroll
+      for (int p = 0; p <= MB; ++p) {
+        const uint32_t w = *(const uint32_t*)(kp + key_word_off(L, p, jc, n));
+        kw[p] = jl ? w : 0u;
+      }
+      f32x4 dm0 = {0, 0, 0, 0}, dm1 = {0, 0, 0, 0}, dq0 = {0, 0, 0, 0}, dq1 = {0, 0, 0, 0};
+      constexpr int TPG = NTP > 5 ? 5 : NTP;
+#pragma unroll
+      for (int t0 = 0; t0 < NTP; t0 += TPG) {
+        i32x8 a[TPG][2];
+#pragma unroll
+        for (int q = 0; q < TPG; ++q)
+#pragma unroll
+          for (int rs = 0; rs < 2; ++rs) {
+            const int tp = t0 + q < NTP ? t0 + q : NTP - 1;
+            const uint32_t* op = qa_lds + ((tp * WPLT + i) * 2 + rs) * WD_QA_OP;
+            const u32x4 lo = *(const u32x4*)(op + lane * 4);
+            const uint2 hi = *(const uint2*)(op + 64 * 4 + lane * 2);
+            a[q][rs] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi.x, (int)hi.y, 0, 0};
+          }
+#pragma unroll
+        for (int q = 0; q < TPG; ++q) {
+          const int tp = t0 + q;
+          if (tp < NTP) {
+            uint32_t x;
+            if (tp == NTP - 1) x = kw[MB];
+            else if (tp < MB) x = kw[tp < MB ? tp : 0];
+            else {
+              const int pl = (xpl >> (4 * (tp - MB))) & 15;
+              x = 0;
+#pragma unroll
+              for (int p = 0; p < MB; ++p) x ^= ((pl >> p) & 1) ? kw[p] : 0u;
+            }
+            const uint32_t b0 = x & 0x11111111u, b1 = x & 0x22222222u, b2 = x & 0x44444444u, b3 = (x >> 3) & 0x11111111u;
+            if (tp == NTP - 1) {
+              dq0 = mfma_f8f4<2>(a[q][0], b0, b1, b2, b3, dq0, sa, sb);
+              dq1 = mfma_f8f4<3>(a[q][1], b0, b1, b2, b3, dq1, sa, sb);
+            } else {
+              dm0 = mfma_f8f4<0>(a[q][0], b0, b1, b2, b3, dm0, sa, sb);
+              dm1 = mfma_f8f4<1>(a[q][1], b0, b1, b2, b3, dm1, sa, sb);
+            }
+          }
+        }
+        if (NTP > TPG) __builtin_amdgcn_sched_barrier(0);       // (the next group's operands after this group's MFMAs)
+      }
+      // lane (token n, rows 4 kb .. 4 kb + 3 = terms of heads 2 kb, 2 kb + 1)
+      *(f32x4*)(s_part + (u * 64 + lane) * 4) = f32x4{(dm0[0] + dm0[1]) + (dm1[0] + dm1[1]), (dm0[2] + dm0[3]) + (dm1[2] + dm1[3]),
+                                                      (dq0[0] + dq0[1]) + (dq1[0] + dq1[1]), (dq0[2] + dq0[3]) + (dq1[2] + dq1[3])};
+    }
+  };
+
+  // ---- softmax of block blk (log2 domain, running reference), the helper wavefront: lane (token n of either page, heads
+  // 2 kb, 2 kb + 1)
+  auto softmax = [&](int blk, int ring_slot) __attribute__((always_inline)) {
+    const unsigned char* kslot0 = kring + (ring_slot * 2) * kslot;
+    float s[2][2];
+    bool valid[2];
+    f32x4 t[2][WD_MAX_CHUNKS];
+    f32x2 meta[2];
+#pragma unroll
+    for (int pg = 0; pg < 2; ++pg) {
+      meta[pg] = *(const f32x2*)(kslot0 + pg * kslot + L.off_meta + n * 8);
+#pragma unroll
+      for (int i = 0; i < WD_MAX_CHUNKS; ++i) t[pg][i] = *(const f32x4*)(s_part + ((2 * min(i, WPLT - 1) + pg) * 64 + lane) * 4);
+    }
+#pragma unroll
+    for (int pg = 0; pg < 2; ++pg) {
+      f32x4 sum = t[pg][0];
+#pragma unroll
+      for (int i = 1; i < WD_MAX_CHUNKS; ++i) {
+        const f32x4 v = t[pg][i];
+        sum += i < WPLT ? v : f32x4{0, 0, 0, 0};
+      }
+      valid[pg] = n < tokens_of(blk, pg);
+      const float v0 = fmaf(meta[pg][0], sum[0] + c_idx0, meta[pg][1] * (sum[2] + c_sgn0));
+      const float v1 = fmaf(meta[pg][0], sum[1] + c_idx1, meta[pg][1] * (sum[3] + c_sgn1));
+      s[0][pg] = valid[pg] ? v0 : MF_NEG;
+      s[1][pg] = valid[pg] ? v1 : MF_NEG;
+    }
+    // The reference of a head (weights are exp2(score - reference)) only moves when a score exceeds it by more than
+    // a small slack, so the usual block rescales nothing; weights are at most 2^REF_SLACK.
+    constexpr float REF_SLACK = 4.0f;
+    // 2^(80 - s), s the bit position the code of token n has in its 16-bit half of a value operand register
+    const float kpow = VB == 2 ? ((n & 3) == 0 ? 0x1p80f : ((n & 3) == 1 ? 0x1p78f : ((n & 3) == 2 ? 0x1p76f : 0x1p74f)))
+                               : (VB == 4 ? ((n & 1) ? 0x1p76f : 0x1p80f) : 0x1p80f);
+    bool moved = false;
+#pragma unroll
+    for (int jj = 0; jj < 2; ++jj) {
+      const int g = 2 * kb + jj;
+      const float mx = row_max16(fmaxf(s[jj][0], s[jj][1]));
+      const bool move = mx > m_run[jj] + REF_SLACK;
+      const float m_new = move ? mx : m_run[jj];
+      const float alpha = move ? __builtin_amdgcn_exp2f(m_run[jj] - m_new) : 1.0f;
+      moved |= move;
+      m_run[jj] = m_new;
+      const float p0 = valid[0] ? __builtin_amdgcn_exp2f(s[jj][0] - m_new) : 0.0f;
+      const float p1 = valid[1] ? __builtin_amdgcn_exp2f(s[jj][1] - m_new) : 0.0f;
+      l_run[jj] = fmaf(l_run[jj], alpha, p0 + p1);
+      s_p[g * 32 + n] = p0;
+      s_p[g * 32 + 16 + n] = p1;
+      s_pv[g * 32 + n] = p0 * kpow;
+      s_pv[g * 32 + 16 + n] = p1 * kpow;
+      if (n == 0) s_alpha[g] = alpha;
+    }
+    const bool any_moved = __builtin_amdgcn_ballot_w64(moved) != 0;
+    if (lane == 0) s_flag[0] = any_moved ? 1 : 0;
+  };
+
+  // ---- values of block blk: lane = (row n: head n % 8 with the scales of group 2 wave + n / 8; tokens
+  // 8 (kb % 2) .. of page kb / 2)
+  auto values = [&](int blk, int ring_slot) __attribute__((always_inline)) {
+    const int hd = n & 7, gpar = n >> 3, pg = kb >> 1, u = kb & 1;
+    // this lane's page in the value ring; offsets are those of the page record minus the key part
+    const unsigned char* vp = vring + (ring_slot * 2 + pg) * vslot - L.off_vdata;
+    const float* prow = s_p + hd * 32 + pg * 16;
+    const float* pvrow = s_pv + hd * 32 + pg * 16;
+    const bool rescale = __builtin_amdgcn_readfirstlane(s_flag[0]) != 0;
+    // some tokens of the block do not exist (the ragged end of the sequence, a page outside the pool)
+    const bool partial = tokens_of(blk, 0) < 16 || tokens_of(blk, 1) < 16;
+    // weights in natural token order 8u .. 8u + 7 (the zero points' operand)
+    float pn[8];
+    {
+      const f32x4 t0 = *(const f32x4*)(prow + 8 * u), t1 = *(const f32x4*)(prow + 8 * u + 4);
+      pn[0] = t0[0]; pn[1] = t0[1]; pn[2] = t0[2]; pn[3] = t0[3];
+      pn[4] = t1[0]; pn[5] = t1[1]; pn[6] = t1[2]; pn[7] = t1[3];
+    }
+    // weights (with the code position folded in) and scales of the tokens whose codes this lane's operand registers
+    // hold: register r carries token tk(r, 0) in its low half and tk(r, 1) in its high half
+    float pw[4][2], sc[4][2];
+    const unsigned char* srow = vp + L.off_vscale + ((2 * wave + gpar) * 16) * 2;
+    auto widen = [&](uint32_t w, float& lo, float& hi) {
+      lo = f16p ? f16_lo(w) : __uint_as_float(w << 16);
+      hi = f16p ? f16_hi(w) : __uint_as_float(w & 0xffff0000u);
+    };
+    if (VB == 2) {
+      // tk(r, h) = 4u + r + 8h
+      const f32x4 t0 = *(const f32x4*)(pvrow + 4 * u), t1 = *(const f32x4*)(pvrow + 4 * u + 8);
+      const uint2 s0 = *(const uint2*)(srow + (4 * u) * 2), s1 = *(const uint2*)(srow + (4 * u + 8) * 2);
+      float f0[4], f1[4];
+      widen(s0.x, f0[0], f0[1]); widen(s0.y, f0[2], f0[3]);
+      widen(s1.x, f1[0], f1[1]); widen(s1.y, f1[2], f1[3]);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) { pw[r][0] = t0[r]; pw[r][1] = t1[r]; sc[r][0] = f0[r]; sc[r][1] = f1[r]; }
+    } else {
+      const f32x4 t0 = *(const f32x4*)(pvrow + 8 * u), t1 = *(const f32x4*)(pvrow + 8 * u + 4);
+      const float pv[8] = {t0[0], t0[1], t0[2], t0[3], t1[0], t1[1], t1[2], t1[3]};
+      const u32x4 sv = *(const u32x4*)(srow + (8 * u) * 2);
+      float f[8];
+      widen(sv[0], f[0], f[1]); widen(sv[1], f[2], f[3]); widen(sv[2], f[4], f[5]); widen(sv[3], f[6], f[7]);
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const int k = VB == 4 ? r + 4 * h : 4 * (r >> 1) + (r & 1) + 2 * h;     // token - 8u
+          pw[r][h] = pv[k];
+          sc[r][h] = f[k];
+        }
+    }
+    u32x4 bz = *(const u32x4*)(vp + L.off_vzero + ((2 * wave + (n & 1)) * 16 + 8 * u) * 2);
+    uint32_t fw[4][VB == 8 ? 2 : 1];
+#pragma unroll
+    for (int cc = 0; cc < 4; ++cc) {
+      const uint32_t* field = (const uint32_t*)(vp + L.off_vdata + (n * (d >> 4) + 4 * wave + cc) * (VB * 2));
+      if (VB == 2) fw[cc][0] = field[0] >> (8 * u);
+      else if (VB == 4) fw[cc][0] = field[u];
+      else { fw[cc][0] = field[2 * u]; fw[cc][VB == 8 ? 1 : 0] = field[2 * u + 1]; }
+    }
+    if (rescale) {
+      const f32x4 a4 = *(const f32x4*)(s_alpha + 4 * (kb & 1));   // accumulator rows 4 kb .. 4 kb + 3 = heads 4 (kb % 2) ..
+#pragma unroll
+      for (int c = 0; c < 4; ++c) acc[c] *= a4;
+      zacc *= a4;
+    }
+    // a code masked in place at bit s of its 16-bit half is the bf16 number code x 2^(s - 133); the weight carries 2^(80 - s)
+    u32x4 aw;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float w0 = pw[r][0] * sc[r][0], w1 = pw[r][1] * sc[r][1];
+      if (partial) {      // (a slot past the end of the sequence may hold any scale: its weight is an exact zero)
+        w0 = pw[r][0] != 0.0f ? w0 : 0.0f;
+        w1 = pw[r][1] != 0.0f ? w1 : 0.0f;
+      }
+      aw[r] = pack_bf16(w0, w1);
+    }
+    // zero points of this wavefront's two groups (columns n % 2; the other columns repeat them)
+    {
+      u32x4 ap;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) ap[r] = f16p ? pack_f16(pn[2 * r], pn[2 * r + 1]) : pack_bf16(pn[2 * r], pn[2 * r + 1]);
+      if (partial) {
+        const int left = tokens_of(blk, pg) - 8 * u;            // existing tokens among this lane's eight
+#pragma unroll
+        for (int r = 0; r < 4; ++r) bz[r] &= (2 * r < left ? 0x0000ffffu : 0u) | (2 * r + 1 < left ? 0xffff0000u : 0u);
+      }
+      zacc = f16p ? mfma_f16(ap, bz, zacc) : mfma(ap, bz, zacc);
+    }
+#pragma unroll
+    for (int cc = 0; cc < 4; ++cc) {
+      u32x4 bc;
+      if (VB == 2) {
+        const uint32_t x = fw[cc][0];
+        bc = u32x4{x & m0, x & m1, x & m2, x & m3};
+      } else if (VB == 4) {
+        const uint32_t x = fw[cc][0], x8 = x >> 8;
+        bc = u32x4{x & m0, x & m1, x8 & m0, x8 & m1};
+      } else {
+        const uint32_t x = fw[cc][0], y = fw[cc][VB == 8 ? 1 : 0];
+        bc = u32x4{x & m0, (x >> 8) & m0, y & m0, (y >> 8) & m0};
+      }
+      acc[cc] = mfma(aw, bc, acc[cc]);
+    }
+  };
+
+  // ---------------------------------------------------------------- the blocks
+  // Iteration j: the values of block j beside the scores of block j + 1, then the softmax of block j + 1; the first
+  // iteration (j = first block - 1) only scores.  Requests outstanding at the top of iteration j, oldest first:
+  // (keys j + 1, values j), ..., (keys j + nring - 1, values j + nring - 2); the first group has to have landed.
+#ifdef WD_PROF
+  unsigned long long wd_t[8] = {0, 0, 0, 0, 0, 0, 0, 0}, wd_last = wall_clock64();
+#endif
+  int ks = 0, vs = 0;                           // ring slots of the keys of block j + 1 and the values of block j
+  for (int j = blk_begin - 1; j < blk_end; ++j) {
+    WD_T(7);
+    wd_wait_vm(OPS * (j < blk_begin ? nring - 1 : nring - 2));
+    WD_T(0);
+    __syncthreads();      // every wavefront's requests have landed; everyone is done with the slots refilled next, and sees the softmax of block j
+    WD_T(1);
+    if (2 * j >= pbase + 64) {                  // (uniform) the table registers move on
+      pbase += 64;
+      tbl_a = tbl_b;
+      tbl_b = load_tbl(pbase + 64);
+      asm volatile("" : "+v"(tbl_b));           // (the wait for this load: here, once in 32 blocks)
+    }
+    if (j >= blk_begin) {
+      issue_keys();
+      issue_vals();
+      WD_T(2);
+      if (!helper) values(j, vs);
+      vs = vs + 1 == nring ? 0 : vs + 1;
+      WD_T(3);
+    }
+    if (j + 1 < blk_end) score_units(ks);
+    WD_T(4);
+    __syncthreads();
+    WD_T(5);
+    if (helper && j + 1 < blk_end) softmax(j + 1, ks);
+    ks = ks + 1 == nring ? 0 : ks + 1;
+    WD_T(6);
+  }
+#ifdef WD_PROF
+  if (blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && lane == 0)
+    for (int k = 0; k < 8; ++k) wd_prof[wave * 8 + k] = wd_t[k];
+#endif
+
+  // ---------------------------------------------------------------- the partial (m, l, acc[d]) of every head
+  stage_wait<0>();                              // the surplus requests of the last trips have landed
+  __syncthreads();
+  if (n < 2 && !helper) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) s_z[(wave * 16 + 4 * kb + i) * 2 + n] = zacc[i];
+  }
+  if (helper) {
+#pragma unroll
+    for (int jj = 0; jj < 2; ++jj) {
+      const float lsum = row_sum16(l_run[jj]);
+      const int g = 2 * kb + jj;
+      if (n == 0 && g < G) {
+        float* r = parts + (((int64_t)b * Hq + qbase + g) * n_parts + split) * (d + 2);
+        r[0] = m_run[jj] * 0.6931471805599453f;     // natural-log domain
+        r[1] = lsum;
+      }
+    }
+  }
+  __syncthreads();
+  // accumulator rows 0..7 hold the heads for the tiles of the even group (tiles 0, 1), rows 8..15 for the odd
+  // group (tiles 2, 3); the zero-point sums have the same rows in both halves
+  if (!helper) {
+    const int par = kb >> 1;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int g = 4 * (kb & 1) + i;
+      if (g < G) {
+        const float z = s_z[(wave * 16 + 4 * kb + i) * 2 + par];
+        float* row = parts + (((int64_t)b * Hq + qbase + g) * n_parts + split) * (d + 2) + 2 + 64 * wave + 32 * par + n;
+        row[0] = fmaf(par ? acc[2][i] : acc[0][i], 0x1p53f, z);
+        row[16] = fmaf(par ? acc[3][i] : acc[1][i], 0x1p53f, z);
+      }
+    }
+  }
+}
+
+// LDS plan of the kernel for a layer: ring depth, slot sizes, bytes; false when it does not fit
+static bool wide_plan(const tq_layer& ly, const tq_page_layout& L, int& nring, int& kslot, int& vslot, size_t& smem) {
+  const int d = ly.d, wplt = (d + 127) / 128, mb = ly.mse_bits;
+  int nx = 0;
+  for (int t = 0; t < ly.n_terms; ++t)
+    if (__builtin_popcount(ly.term_mask[t]) > 1) ++nx;
+  if (mb < 1 || mb > 4 || nx != (mb == 3 ? 1 : (mb == 4 ? 4 : 0))) return false;
+  const int ntp = mb + nx + 1;
+  kslot = ((L.off_vdata + 1023) / 1024) * 1024;
+  vslot = ((L.page_bytes - L.off_vdata + 1023) / 1024) * 1024;
+  const size_t fixed = (size_t)ntp * wplt * 2 * WD_QA_OP * 4 + (size_t)2 * wplt * 1024 + (size_t)WD_SMALL_FLOATS * 4;
+  const size_t block = (size_t)2 * (kslot + vslot);
+  if (fixed + 2 * block > (size_t)WD_LDS_BYTES) return false;
+  nring = fixed + 3 * block <= (size_t)WD_LDS_BYTES ? 3 : 2;
+  // (the waits count the requests of the blocks behind the current one: an immediate operand, sixteen at most)
+  const int nw = d / 64 + 1, ops = (2 * (kslot / 1024) + nw - 1) / nw + (2 * (vslot / 1024) + nw - 1) / nw;
+  if ((2 * (kslot / 1024) + nw - 1) / nw > 4 || (2 * (vslot / 1024) + nw - 1) / nw > 4) return false;
+  if (ops * (nring - 1) > 16) nring = 2;
+  if (ops * (nring - 1) > 16) return false;
+  smem = fixed + (size_t)nring * block;
+  return true;
+}
+
+bool decode_wide_has_kernel(const tq_layer& ly, const tq_page_layout& L) {
+  const int d = ly.d;
+  if (opt_wide_heads.load(std::memory_order_relaxed) == 0) return false;
+  // (d + 64 threads: at most twelve wavefronts, three per SIMD, with the helper)
+  if (d <= 256 || d > 704 || (d & 63) || L.d != d || L.mse_bits != ly.mse_bits) return false;
+  if ((L.dtype != TQ_BF16 && L.dtype != TQ_F16) || L.group_size != 32) return false;
+  if (L.value_bits != 2 && L.value_bits != 4 && L.value_bits != 8) return false;
+  if (ly.n_terms <= 0) return false;
+  int nring, kslot, vslot;
+  size_t smem;
+  return wide_plan(ly, L, nring, kslot, vslot, smem);
+}
+
+// Returns TQ_EUNSUPPORTED when the shape has no wide-head kernel (nothing was launched).
+int launch_decode_wide(const float* q_rot, const float* q_sk, int B, int Hq, int Hkv, const uint8_t* pool,
+                       const int32_t* block_table, int bt_stride, const int32_t* seq_lens, float sm_scale,
+                       const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts, int n_split, int len_sub,
+                       int max_pages, int num_pages, hipStream_t st) {
+  if (!decode_wide_has_kernel(ly, L)) return TQ_EUNSUPPORTED;
+  const int g_tot = Hq / Hkv, kv_div = (g_tot + 7) / 8;
+  if (g_tot < 1 || g_tot > 16 || (int64_t)Hkv * kv_div > 65535) return TQ_EUNSUPPORTED;
+  int nring, kslot, vslot;
+  size_t smem;
+  wide_plan(ly, L, nring, kslot, vslot, smem);
+  const dim3 grid(n_split, Hkv * kv_div, B), block(ly.d + 64);      // (one wavefront more than channels / 64: the helper)
+  hipEvent_t t_start = nullptr, t_stop = nullptr;
+  const bool timed = take_time_hook(0, t_start, t_stop);
+#define TQ_LAUNCH_WIDE(VB, MB)                                                                                        \
+  {                                                                                                                   \
+    auto kern = decode_wide_kernel<VB, MB>;                                                                           \
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);     \
+    if (e != hipSuccess) return (int)e;                                                                               \
+    if (timed)                                                                                                        \
+      hipExtLaunchKernelGGL(kern, grid, block, smem, st, t_start, t_stop, 0, q_rot, q_sk, Hq, Hkv, kv_div, pool,      \
+                            block_table, bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts, n_split, len_sub,      \
+                            max_pages, num_pages, nring, kslot, vslot);                                               \
+    else                                                                                                              \
+      kern<<<grid, block, smem, st>>>(q_rot, q_sk, Hq, Hkv, kv_div, pool, block_table, bt_stride, seq_lens, sm_scale, \
+                                      ly, L, parts, n_parts, n_split, len_sub, max_pages, num_pages, nring, kslot,    \
+                                      vslot);                                                                         \
+  }
+#define TQ_LAUNCH_WIDE_MB(VB)                        \
+  {                                                  \
+    if (ly.mse_bits == 1) TQ_LAUNCH_WIDE(VB, 1)      \
+    else if (ly.mse_bits == 2) TQ_LAUNCH_WIDE(VB, 2) \
+    else if (ly.mse_bits == 3) TQ_LAUNCH_WIDE(VB, 3) \
+    else TQ_LAUNCH_WIDE(VB, 4)                       \
+  }
+  if (L.value_bits == 2) TQ_LAUNCH_WIDE_MB(2)
+  else if (L.value_bits == 4) TQ_LAUNCH_WIDE_MB(4)
+  else TQ_LAUNCH_WIDE_MB(8)
+#undef TQ_LAUNCH_WIDE_MB
+#undef TQ_LAUNCH_WIDE
+  TQ_CHECK_LAUNCH();
+  return TQ_OK;
+}
+
+}  // namespace tq
+
+#ifdef WD_PROF
+extern "C" int tq_debug_wide_prof(unsigned long long* host, int n) {
+  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(tq::wd_prof), (size_t)n * 8);
+}
+#endif

@@ -167,6 +167,16 @@ class PagedKVPool:
                 v_zeros.data_ptr(), _ffi.stream_ptr(dev)), "tq_pool_export")
         return idx, signs, norms, rnorms, v_data, v_scales, v_zeros
 
+    def page_kernel(self) -> int:
+        """Which page kernel the library runs for this pool's layer (tq_decode_page_kernel): 0 the general
+        vector-ALU kernel, 1 the matrix-core kernel of head_dim 64 / 128 / 256, 2 the matrix-core kernel of the
+        head sizes above 256."""
+        ly = self.quantizer._layer()
+        rc = _ffi.lib().tq_decode_page_kernel(C.byref(ly), C.byref(self.layout))
+        if rc < 0:
+            _ffi.check(rc, "tq_decode_page_kernel")
+        return int(rc)
+
     def _matrix_core_shape(self, Hq: Optional[int]) -> bool:
         """Whether decode runs on the matrix-core page kernel (head_dim 64 / 128 / 256, 16-bit pools, up to 4-bit
         keys - 5-bit at head_dim 128 -, at most 16 query heads per KV head); only the split heuristic depends on it."""
@@ -189,6 +199,13 @@ class PagedKVPool:
         General kernel: it hides its memory latency by occupancy, so about eight workgroups per CU, each
         with at least one 256-token chunk."""
         pairs = max(1, B * self.num_kv_heads)
+        if self.head_dim > 256 and self.page_kernel() == 2:
+            # head sizes above 256: one workgroup per compute unit, a block of 32 tokens at a time; each workgroup
+            # first packs its query operands, so it should have at least 16 blocks
+            if Hq is not None:
+                pairs *= (Hq // self.num_kv_heads + 7) // 8
+            blocks = max(1, (max_len + 31) // 32)
+            return int(max(1, min(max(1, 256 // pairs), max(1, blocks // 16), 512)))
         if not self._matrix_core_shape(Hq):
             chunks = max(1, (max_len + 255) // 256)
             return int(max(1, min(2048 // pairs, chunks, 512)))
