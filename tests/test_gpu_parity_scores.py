@@ -235,7 +235,9 @@ def test_decode_wide_heads_on_the_matrix_cores(gpu, d, key_bits, vb, Hq, Hkv, dt
     assert pool.page_kernel() == 2, "the shape has no wide-head kernel"
     outs = {}
     try:
-        for mode in (1, 0):
+        # 1: as shipped (head_dim 512 / 576: the instantiations with constant page geometry), 2: the instantiation
+        # that takes the geometry at run time (what the other head sizes run), 0: the general kernel
+        for mode in (1, 2, 0) if d in (512, 576) else (1, 0):
             _set_option("wide_heads", mode)
             _progress(f"decode d={d} kb={key_bits} vb={vb} Hq={Hq} Hkv={Hkv} {dtype} n_split={n_split} wide_heads={mode}")
             outs[mode] = _decode_case(gpu, d, key_bits, vb, len(lens), Hq, Hkv, lens, recent, seed=700 + d + vb,
@@ -245,6 +247,8 @@ def test_decode_wide_heads_on_the_matrix_cores(gpu, d, key_bits, vb, Hq, Hkv, dt
     c = cosine(outs[1], outs[0])
     _progress(f"   wide-head kernel against the general kernel: cosine {c:.7f}")
     assert c >= COS_GATE
+    if 2 in outs:
+        assert torch.equal(outs[1], outs[2]), "constant and run-time geometry disagree"
 
 
 # ------------------------------------------------------------------ block tables are bounded on the device
@@ -300,7 +304,8 @@ def test_append_never_writes_through_a_bad_table_entry(gpu, d, key_bits, vb, dty
 
 
 @pytest.mark.parametrize("d,key_bits,vb,Hq,Hkv,dtype", [(128, 3, 4, 8, 2, torch.bfloat16), (256, 3, 2, 16, 2, torch.bfloat16),
-                                                         (64, 3, 2, 4, 1, torch.bfloat16), (128, 3, 2, 4, 2, torch.float32)])
+                                                         (64, 3, 2, 4, 1, torch.bfloat16), (128, 3, 2, 4, 2, torch.float32),
+                                                         (576, 4, 4, 8, 1, torch.bfloat16), (512, 3, 2, 4, 2, torch.float16)])
 def test_decode_gives_no_weight_to_pages_outside_the_pool(gpu, d, key_bits, vb, Hq, Hkv, dtype):
     """Decode with table entries outside [0, num_pages): those pages' tokens get no weight, so the result is
     the attention over the remaining tokens - checked against the oracle on exactly those tokens

@@ -987,7 +987,11 @@ extern "C" int tq_set_option(const char* name, int64_t value) {
   }
   if (!std::strcmp(name, "tail_chunks")) { opt_tail_chunks.store(value != 0); return TQ_OK; }
   if (!std::strcmp(name, "merge_row_groups")) { opt_merge_row_groups.store(value != 0); return TQ_OK; }
-  if (!std::strcmp(name, "wide_heads")) { opt_wide_heads.store(value != 0); return TQ_OK; }
+  if (!std::strcmp(name, "wide_heads")) {
+    if (value < 0 || value > 2) return TQ_EINVAL;
+    opt_wide_heads.store((int)value);
+    return TQ_OK;
+  }
   if (!std::strcmp(name, "append_small")) {
     if (value < -1 || value > (1 << 24)) return TQ_EINVAL;
     opt_append_small.store((int)value);

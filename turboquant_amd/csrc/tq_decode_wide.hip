@@ -31,7 +31,7 @@ constexpr int WD_BLK = 32;                 // tokens per iteration (two pages)
 constexpr int WD_QA_OP = 64 * 6;           // dwords of one packed operand: [64 lanes][4] then [64 lanes][2]
 constexpr int WD_MAX_WAVES = 12;           // head_dim 768
 constexpr int WD_MAX_CHUNKS = 6;           // 128-coordinate chunks of head_dim 768
-constexpr int WD_SMALL_FLOATS = 256 + 256 + 8 + 8 + 32 + 16 + 16 + WD_MAX_WAVES * 32;     // s_p, s_pv, s_alpha, s_flag, s_stat, s_mult, s_coef, s_z
+constexpr int WD_SMALL_FLOATS = 2 * (256 + 256 + 8 + 8 + 64) + 32 + 16 + 16 + WD_MAX_WAVES * 32;   // two of (s_p, s_pv, s_alpha, s_flag, s_meta), s_stat, s_mult, s_coef, s_z
 constexpr int WD_LDS_BYTES = 160 * 1024;
 
 // -DWD_PROF (a profiling build, never the shipped one): every wavefront of workgroup (0, 0, 0) sums the time it
@@ -66,22 +66,66 @@ __device__ __forceinline__ void wd_wait_vm(int n) {
   }
 }
 
+// The page geometry tq_page_layout_init gives 16-bit pages with groups of 32, and the kernel's LDS plan, as functions
+// the compiler can evaluate: the instantiations for the head sizes 512 and 576 have every offset, slot size and trip
+// count as a constant (a wavefront's scalar registers hold a fraction of what the run-time version keeps in them).
+struct WideGeom { int off_meta, off_vdata, off_vscale, off_vzero, page_bytes, key_lane_major; };
+__host__ __device__ constexpr WideGeom wide_geom(int d, int mb, int vb) {
+  WideGeom g{};
+  int off = (mb + 1) * (d / 8) * TQ_PAGE_TOKENS;
+  g.off_meta = off;   off += 8 * TQ_PAGE_TOKENS;
+  g.off_vdata = off;  off += d * vb * 2;
+  g.off_vscale = off; off += (d / 32) * TQ_PAGE_TOKENS * 2;
+  g.off_vzero = off;  off += (d / 32) * TQ_PAGE_TOKENS * 2;
+  g.page_bytes = (off + 127) & ~127;
+  g.key_lane_major = (d % 128 == 0 || d == 64) ? 1 : 0;
+  return g;
+}
+struct WidePlan { int nring, kslot, vslot, smem; bool ok; };
+__host__ __device__ constexpr WidePlan wide_plan_of(int d, int mb, int off_vdata, int page_bytes) {
+  WidePlan p{};
+  const int wplt = (d + 127) / 128, ntp = mb + (mb == 3 ? 1 : (mb == 4 ? 4 : 0)) + 1;
+  p.kslot = off_vdata;                          // (multiples of 16; a slot is as long as its part of the page)
+  p.vslot = page_bytes - off_vdata;
+  const int qa_stride = wplt * WD_QA_OP - (d % 128 ? WD_QA_OP / 2 : 0);
+  const int fixed = ntp * 2 * qa_stride * 4 + 2 * 2 * wplt * 1024 + WD_SMALL_FLOATS * 4;
+  const int block = 2 * (p.kslot + p.vslot);
+  p.nring = fixed + 3 * block <= WD_LDS_BYTES ? 3 : 2;
+  // (the waits count the requests of the iteration behind the current one: an immediate operand, sixteen at most;
+  // a wavefront keeps the constants of at most four requests of a kind)
+  const int nw = d / 64 + 1, ops_k = (2 * ((p.kslot + 1023) / 1024) + nw - 1) / nw, ops_v = (2 * ((p.vslot + 1023) / 1024) + nw - 1) / nw;
+  p.ok = p.kslot >= 1024 && p.vslot >= 1024 && fixed + 2 * block <= WD_LDS_BYTES && ops_k <= 4 && ops_v <= 4 && ops_k + ops_v <= 16;
+  p.smem = fixed + p.nring * block;
+  return p;
+}
+
 // MB stored index planes; the codebooks the quantiser makes have NX = 0, 0, 1, 4 multi-bit Walsh terms for
 // MB = 1..4, so MB + NX + 1 term planes go through the score MFMAs.
-template <int VB, int MB>
+// D: the head size as a constant (512, 576), or 0: taken from the layer at run time.  F16P: fp16 pages.
+template <int D, int VB, int MB, bool F16P>
 __global__ void __launch_bounds__(768)
 decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_sk, int Hq, int Hkv, int kv_div,
                    const uint8_t* __restrict__ pool, const int32_t* __restrict__ block_table, int bt_stride,
-                   const int32_t* __restrict__ seq_lens, float sm_scale, tq_layer ly, tq_page_layout L,
+                   const int32_t* __restrict__ seq_lens, float sm_scale, tq_layer ly, tq_page_layout L_rt,
                    float* __restrict__ parts, int n_parts, int n_split, int len_sub, int max_pages, int num_pages,
-                   int nring, int kslot, int vslot) {
+                   int nring_rt, int kslot_rt, int vslot_rt) {
   constexpr int NX = MB == 3 ? 1 : (MB == 4 ? 4 : 0), NTP = MB + NX + 1;
-  const bool f16p = L.dtype == TQ_F16;
-  const int d = ly.d, W = d >> 5, WPLT = (d + 127) >> 7;
+  constexpr bool f16p = F16P;                   // fp16 pages: scales and zero points are fp16 numbers
+  const int d = D ? D : ly.d, W = d >> 5, WPLT = (d + 127) >> 7;
+  // the page geometry and the LDS plan: constants when the head size is one
+  constexpr WideGeom GC = wide_geom(D ? D : 512, MB, VB);
+  constexpr WidePlan PC = wide_plan_of(D ? D : 512, MB, GC.off_vdata, GC.page_bytes);
+  tq_page_layout L = L_rt;
+  if (D) {
+    L.d = D; L.mse_bits = MB; L.value_bits = VB; L.group_size = 32; L.key_lane_major = GC.key_lane_major; L.off_keys = 0;
+    L.off_meta = GC.off_meta; L.off_vdata = GC.off_vdata; L.off_vscale = GC.off_vscale; L.off_vzero = GC.off_vzero;
+    L.page_bytes = GC.page_bytes;
+  }
+  const int nring = D ? PC.nring : nring_rt, kslot = D ? PC.kslot : kslot_rt, vslot = D ? PC.vslot : vslot_rt;
   const int tid = threadIdx.x, lane = tid & 63;
   // NW wavefronts own 64 channels each; one more (the helper, wavefront NW) owns none: it runs the softmax and takes
   // score units like the others (head_dim 576: ten units for ten wavefronts)
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), NW = ((int)blockDim.x >> 6) - 1, NWS = NW + 1;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), NW = D ? D / 64 : ((int)blockDim.x >> 6) - 1, NWS = NW + 1;
   const bool helper = wave == NW;
   const int n = lane & 15, kb = lane >> 4;
   const int split = blockIdx.x, b = blockIdx.z;
@@ -93,13 +137,19 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
   if (G <= 0) return;
 
   extern __shared__ __align__(16) unsigned char smem_raw[];
-  uint32_t* qa_lds = (uint32_t*)smem_raw;                         // [NTP][WPLT][2 row sets][WD_QA_OP]
-  float* s_part = (float*)(qa_lds + NTP * WPLT * 2 * WD_QA_OP);   // [2 WPLT units][64 lanes][4]
-  float* s_p = s_part + 2 * WPLT * 256;                           // [8 heads][32 tokens] softmax weights
-  float* s_pv = s_p + 256;                                        // the same weights times 2^(80 - bit position of the token's code)
-  float* s_alpha = s_pv + 256;                                    // [8]
-  int* s_flag = (int*)(s_alpha + 8);                              // [0]: the block's softmax moved a reference
-  float* s_stat = s_alpha + 16;                                   // [8][4]: E_index, E_sign, constant parts of the score
+  // Query operands: per (term plane, row set) the chunks one after another; a last chunk of 64 coordinates (head_dim
+  // not a multiple of 128) takes half an operand - the slots of the lanes of its upper two coordinate quarters do not
+  // exist: those lanes read what follows (always finite as fp6) against key words that are zero.
+  const bool half_chunk = (d & 127) != 0;
+  const int QA_STRIDE = WPLT * WD_QA_OP - (half_chunk ? WD_QA_OP / 2 : 0);    // dwords per (term plane, row set)
+  uint32_t* qa_lds = (uint32_t*)smem_raw;                         // [NTP][2 row sets][QA_STRIDE]
+  float* s_part = (float*)(qa_lds + NTP * 2 * QA_STRIDE);         // [2][2 WPLT units][64 lanes][4]
+  float* s_p = s_part + 2 * 2 * WPLT * 256;                       // [2][8 heads][32 tokens] softmax weights
+  float* s_pv = s_p + 2 * 256;                                    // [2]... the same weights times 2^(80 - bit position of the token's code)
+  float* s_alpha = s_pv + 2 * 256;                                // [2][8]
+  int* s_flag = (int*)(s_alpha + 2 * 8);                          // [2][8], [0] used: the block's softmax moved a reference
+  float* s_meta = s_alpha + 4 * 8;                                // [2][2 pages][16 tokens][norm, residual norm]
+  float* s_stat = s_meta + 2 * 64;                                // [8][4]: E_index, E_sign, constant parts of the score
   float* s_mult = s_stat + 32;                                    // [8][2]: multipliers of q_rot / q_sk
   float* s_coef = s_mult + 16;                                    // [16] coefficient of each term plane
   float* s_z = s_coef + 16;                                       // [waves][16 rows][2 groups] zero-point sums
@@ -131,13 +181,23 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
     const int raw = bt[min(first + lane, n_pages - 1)];
     return (unsigned)raw < (unsigned)num_pages ? raw : (int)0x80000000;
   };
+  // Block tables are device data nobody has checked: every wavefront looks once at the entries of the workgroup's
+  // range, a lane per entry; only a workgroup that finds one outside the pool looks at the entries again, block by block.
+  bool has_bad;
+  {
+    bool bad = false;
+    const int e1 = min(2 * blk_end, n_pages);
+    for (int e = 2 * blk_begin + lane; e < e1; e += 64) bad |= (unsigned)bt[e] >= (unsigned)num_pages;
+    has_bad = __builtin_amdgcn_ballot_w64(bad) != 0;
+  }
   int tbl_a = load_tbl(pbase), tbl_b = load_tbl(pbase + 64);
   // (used here, so that the compiler waits for the loads here and knows of no pending load inside the loop: a wait of
   // its own there would be for everything outstanding, the page requests included)
   asm volatile("" : "+v"(tbl_a), "+v"(tbl_b));
   auto page_entry = [&](int page) -> int {
     const int rel = __builtin_amdgcn_readfirstlane(min(page, n_pages - 1) - pbase);
-    return rel < 64 ? __builtin_amdgcn_readlane(tbl_a, rel) : __builtin_amdgcn_readlane(tbl_b, rel - 64);
+    const int ea = __builtin_amdgcn_readlane(tbl_a, rel & 63), eb = __builtin_amdgcn_readlane(tbl_b, rel & 63);
+    return rel < 64 ? ea : eb;
   };
   // Requests for the key part / value part of the next block of each kind into its ring slot: a kilobyte per
   // instruction, dealt to the wavefronts; every wavefront issues the same number per block (the waits below count
@@ -146,7 +206,7 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
   // of the range the requests repeat it (into the slot it already has).  What does not depend on the block - which
   // page of the pair, the offset inside the page, the offset inside the slot - is worked out once.
   const int kbytes = L.off_vdata, vbytes = L.page_bytes - L.off_vdata;
-  const int PK = kslot >> 10, PV = vslot >> 10;
+  const int PK = (kbytes + 1023) >> 10, PV = (vbytes + 1023) >> 10;
   const int OPS_K = (2 * PK + NWS - 1) / NWS, OPS_V = (2 * PV + NWS - 1) / NWS, OPS = OPS_K + OPS_V;
   constexpr int WD_MAX_OPS = 4;                 // per kind (the plan on the host keeps to it)
   struct Req { int blk, slot; uint32_t src_off[WD_MAX_OPS]; int lds_off[WD_MAX_OPS]; int pg[WD_MAX_OPS]; };
@@ -158,8 +218,9 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
       const int piece = min(wave + k * NWS, 2 * pieces - 1);
       const int pg = piece >= pieces ? 1 : 0, pc = piece - pg * pieces;
       r.pg[k] = pg;
-      r.src_off[k] = (uint32_t)(part_off + min(pc * 1024 + lane * 16, part_bytes - 16));
-      r.lds_off[k] = pg * slot_bytes + pc * 1024;
+      const int at = min(pc * 1024, part_bytes - 1024);     // (the last piece overlaps the one before it: a slot is as long as its part)
+      r.src_off[k] = (uint32_t)(part_off + at + lane * 16);
+      r.lds_off[k] = pg * slot_bytes + at;
     }
   };
   Req rq_k, rq_v;
@@ -182,13 +243,8 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
   };
   auto issue_keys = [&]() __attribute__((always_inline)) { issue(rq_k, kring_lds, kslot, OPS_K); };
   auto issue_vals = [&]() __attribute__((always_inline)) { issue(rq_v, vring_lds, vslot, OPS_V); };
-  // the first blocks are on their way while the operands are prepared: the keys of the first block, then groups of
-  // (keys of block i + 1, values of block i)
-  issue_keys();
-  for (int i = 0; i < nring - 1; ++i) {
-    issue_keys();
-    issue_vals();
-  }
+  // the keys of the first blocks are on their way while the operands are prepared
+  for (int i = 0; i < nring - 1; ++i) issue_keys();
 
   // ---------------------------------------------------------------- query operands (as the preparation kernel packs them)
   float cmax = 0.0f;
@@ -276,14 +332,16 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
     for (int item = tid; item < n_items; item += blockDim.x) {
       const int g = item & 7, j = (item >> 3) % (4 * WPLT), tp = (item >> 3) / (4 * WPLT);
       const bool is_sign = tp == NTP - 1, live = g < G && j < W;
-      uint32_t* op0 = qa_lds + ((tp * WPLT + (j >> 2)) * 2) * WD_QA_OP;
+      if (j >= W) continue;                 // (no slot: see half_chunk)
+      uint32_t* op0 = qa_lds + (tp * 2) * QA_STRIDE + (j >> 2) * WD_QA_OP;
       const int slot0 = 2 * g + 16 * (j & 3);
+      const int hi_at = half_chunk && (j >> 2) == WPLT - 1 ? 32 * 4 : 64 * 4;      // the operand's [lanes][2] part
       if (!live) {
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-          uint32_t* op = op0 + (t >> 1) * WD_QA_OP;
+          uint32_t* op = op0 + (t >> 1) * QA_STRIDE;
           *(u32x4*)(op + (slot0 + (t & 1)) * 4) = u32x4{0, 0, 0, 0};
-          *(uint2*)(op + 64 * 4 + (slot0 + (t & 1)) * 2) = make_uint2(0u, 0u);
+          *(uint2*)(op + hi_at + (slot0 + (t & 1)) * 2) = make_uint2(0u, 0u);
         }
         continue;
       }
@@ -310,9 +368,9 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
       for (int t = 0; t < 4; ++t) {
         u32x6_t code;
         asm volatile("v_cvt_scalef32_2xpk16_fp6_f32 %0, %1, %2, %3" : "=&v"(code) : "v"(va), "v"(vb), "v"(one));
-        uint32_t* op = op0 + (t >> 1) * WD_QA_OP;
+        uint32_t* op = op0 + (t >> 1) * QA_STRIDE;
         *(u32x4*)(op + (slot0 + (t & 1)) * 4) = u32x4{code[0], code[1], code[2], code[3]};
-        *(uint2*)(op + 64 * 4 + (slot0 + (t & 1)) * 2) = make_uint2(code[4], code[5]);
+        *(uint2*)(op + hi_at + (slot0 + (t & 1)) * 2) = make_uint2(code[4], code[5]);
         if (t < 3) {
           f32x32_t r;
           asm volatile("v_cvt_scalef32_pk32_f32_fp6 %0, %1, %2" : "=&v"(r) : "v"(code), "v"(one));
@@ -350,16 +408,21 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
   const uint32_t m1 = VB == 2 ? 0x000C000Cu : 0x00F000F0u, m2 = 0x00300030u, m3 = 0x00C000C0u;
   // existing tokens of page pg of block blk: a prefix (none on a page outside the pool)
   auto tokens_of = [&](int blk, int pg) -> int {
-    return page_entry(2 * blk + pg) < 0 ? 0 : min(max(seq_len - blk * WD_BLK - 16 * pg, 0), 16);
+    if (has_bad && page_entry(2 * blk + pg) < 0) return 0;
+    return min(max(seq_len - blk * WD_BLK - 16 * pg, 0), 16);
   };
 
   // ---- scores of block blk: unit u = (page u % 2, chunk u / 2), dealt from the helper wavefront down
-  auto score_units = [&](int ring_slot) __attribute__((always_inline)) {
+  auto score_units = [&](int ring_slot, int pb) __attribute__((always_inline)) {
     const unsigned char* kslot0 = kring + (ring_slot * 2) * kslot;
+    float* part = s_part + pb * (2 * WPLT * 256);
     for (int u = NW - wave; u < 2 * WPLT; u += NWS) {
       const int pg = u & 1, i = u >> 1;
       const unsigned char* kp = kslot0 + pg * kslot;
       const int j = 4 * i + kb;
+      const int hi_at = half_chunk && i == WPLT - 1 ? 32 * 4 : 64 * 4;
+      // (the unit of a page's first chunk hands the page's norms to the softmax, which runs an iteration later)
+      if (i == 0 && kb == 0) *(f32x2*)(s_meta + pb * 64 + pg * 32 + n * 2) = *(const f32x2*)(kp + L.off_meta + n * 8);
       const bool jl = j < W;
       const int jc = jl ? j : W - 1;
       // the key words, then the planes in groups of at most five: every LDS read of a group (its operands of both row
@@ -380,9 +443,9 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
 #pragma unroll
           for (int rs = 0; rs < 2; ++rs) {
             const int tp = t0 + q < NTP ? t0 + q : NTP - 1;
-            const uint32_t* op = qa_lds + ((tp * WPLT + i) * 2 + rs) * WD_QA_OP;
+            const uint32_t* op = qa_lds + (tp * 2 + rs) * QA_STRIDE + i * WD_QA_OP;
             const u32x4 lo = *(const u32x4*)(op + lane * 4);
-            const uint2 hi = *(const uint2*)(op + 64 * 4 + lane * 2);
+            const uint2 hi = *(const uint2*)(op + hi_at + lane * 2);
             a[q][rs] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi.x, (int)hi.y, 0, 0};
           }
 #pragma unroll
@@ -411,24 +474,26 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
         if (NTP > TPG) __builtin_amdgcn_sched_barrier(0);       // (the next group's operands after this group's MFMAs)
       }
       // lane (token n, rows 4 kb .. 4 kb + 3 = terms of heads 2 kb, 2 kb + 1)
-      *(f32x4*)(s_part + (u * 64 + lane) * 4) = f32x4{(dm0[0] + dm0[1]) + (dm1[0] + dm1[1]), (dm0[2] + dm0[3]) + (dm1[2] + dm1[3]),
+      *(f32x4*)(part + (u * 64 + lane) * 4) = f32x4{(dm0[0] + dm0[1]) + (dm1[0] + dm1[1]), (dm0[2] + dm0[3]) + (dm1[2] + dm1[3]),
                                                       (dq0[0] + dq0[1]) + (dq1[0] + dq1[1]), (dq0[2] + dq0[3]) + (dq1[2] + dq1[3])};
     }
   };
 
   // ---- softmax of block blk (log2 domain, running reference), the helper wavefront: lane (token n of either page, heads
   // 2 kb, 2 kb + 1)
-  auto softmax = [&](int blk, int ring_slot) __attribute__((always_inline)) {
-    const unsigned char* kslot0 = kring + (ring_slot * 2) * kslot;
+  auto softmax = [&](int blk, int pb) __attribute__((always_inline)) {
+    const float* part = s_part + pb * (2 * WPLT * 256);
+    float* sp = s_p + pb * 256;
+    float* spv = s_pv + pb * 256;
     float s[2][2];
     bool valid[2];
     f32x4 t[2][WD_MAX_CHUNKS];
     f32x2 meta[2];
 #pragma unroll
     for (int pg = 0; pg < 2; ++pg) {
-      meta[pg] = *(const f32x2*)(kslot0 + pg * kslot + L.off_meta + n * 8);
+      meta[pg] = *(const f32x2*)(s_meta + pb * 64 + pg * 32 + n * 2);
 #pragma unroll
-      for (int i = 0; i < WD_MAX_CHUNKS; ++i) t[pg][i] = *(const f32x4*)(s_part + ((2 * min(i, WPLT - 1) + pg) * 64 + lane) * 4);
+      for (int i = 0; i < WD_MAX_CHUNKS; ++i) t[pg][i] = *(const f32x4*)(part + ((2 * min(i, WPLT - 1) + pg) * 64 + lane) * 4);
     }
 #pragma unroll
     for (int pg = 0; pg < 2; ++pg) {
@@ -463,25 +528,25 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
       const float p0 = valid[0] ? __builtin_amdgcn_exp2f(s[jj][0] - m_new) : 0.0f;
       const float p1 = valid[1] ? __builtin_amdgcn_exp2f(s[jj][1] - m_new) : 0.0f;
       l_run[jj] = fmaf(l_run[jj], alpha, p0 + p1);
-      s_p[g * 32 + n] = p0;
-      s_p[g * 32 + 16 + n] = p1;
-      s_pv[g * 32 + n] = p0 * kpow;
-      s_pv[g * 32 + 16 + n] = p1 * kpow;
-      if (n == 0) s_alpha[g] = alpha;
+      sp[g * 32 + n] = p0;
+      sp[g * 32 + 16 + n] = p1;
+      spv[g * 32 + n] = p0 * kpow;
+      spv[g * 32 + 16 + n] = p1 * kpow;
+      if (n == 0) s_alpha[pb * 8 + g] = alpha;
     }
     const bool any_moved = __builtin_amdgcn_ballot_w64(moved) != 0;
-    if (lane == 0) s_flag[0] = any_moved ? 1 : 0;
+    if (lane == 0) s_flag[pb * 8] = any_moved ? 1 : 0;
   };
 
   // ---- values of block blk: lane = (row n: head n % 8 with the scales of group 2 wave + n / 8; tokens
   // 8 (kb % 2) .. of page kb / 2)
-  auto values = [&](int blk, int ring_slot) __attribute__((always_inline)) {
+  auto values = [&](int blk, int ring_slot, int pb) __attribute__((always_inline)) {
     const int hd = n & 7, gpar = n >> 3, pg = kb >> 1, u = kb & 1;
     // this lane's page in the value ring; offsets are those of the page record minus the key part
     const unsigned char* vp = vring + (ring_slot * 2 + pg) * vslot - L.off_vdata;
-    const float* prow = s_p + hd * 32 + pg * 16;
-    const float* pvrow = s_pv + hd * 32 + pg * 16;
-    const bool rescale = __builtin_amdgcn_readfirstlane(s_flag[0]) != 0;
+    const float* prow = s_p + pb * 256 + hd * 32 + pg * 16;
+    const float* pvrow = s_pv + pb * 256 + hd * 32 + pg * 16;
+    const bool rescale = __builtin_amdgcn_readfirstlane(s_flag[pb * 8]) != 0;
     // some tokens of the block do not exist (the ragged end of the sequence, a page outside the pool)
     const bool partial = tokens_of(blk, 0) < 16 || tokens_of(blk, 1) < 16;
     // weights in natural token order 8u .. 8u + 7 (the zero points' operand)
@@ -533,7 +598,7 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
       else { fw[cc][0] = field[2 * u]; fw[cc][VB == 8 ? 1 : 0] = field[2 * u + 1]; }
     }
     if (rescale) {
-      const f32x4 a4 = *(const f32x4*)(s_alpha + 4 * (kb & 1));   // accumulator rows 4 kb .. 4 kb + 3 = heads 4 (kb % 2) ..
+      const f32x4 a4 = *(const f32x4*)(s_alpha + pb * 8 + 4 * (kb & 1));   // accumulator rows 4 kb .. 4 kb + 3 = heads 4 (kb % 2) ..
 #pragma unroll
       for (int c = 0; c < 4; ++c) acc[c] *= a4;
       zacc *= a4;
@@ -579,40 +644,41 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
   };
 
   // ---------------------------------------------------------------- the blocks
-  // Iteration j: the values of block j beside the scores of block j + 1, then the softmax of block j + 1; the first
-  // iteration (j = first block - 1) only scores.  Requests outstanding at the top of iteration j, oldest first:
-  // (keys j + 1, values j), ..., (keys j + nring - 1, values j + nring - 2); the first group has to have landed.
+  // Three stages, a block apart, between two barriers: iteration t accumulates the values of block t, runs the
+  // softmax of block t + 1 (the helper) and scores block t + 2; the score sums, the norms and the softmax weights are
+  // double-buffered (block % 2).  Iteration t requests the keys of block t + nring + 1 and the values of block
+  // t + nring - 1 into the slots the blocks t + 1 and t - 1 had, so at its top the requests of iteration t - nring + 1
+  // (keys t + 2, values t) have to have landed and those of the nring - 2 iterations after it may be outstanding.
+  int ks = 0, vs = 0;                           // ring slots of the keys of block t + 2 and the values of block t
 #ifdef WD_PROF
   unsigned long long wd_t[8] = {0, 0, 0, 0, 0, 0, 0, 0}, wd_last = wall_clock64();
 #endif
-  int ks = 0, vs = 0;                           // ring slots of the keys of block j + 1 and the values of block j
-  for (int j = blk_begin - 1; j < blk_end; ++j) {
+  for (int t = blk_begin - 2; t < blk_end; ++t) {
     WD_T(7);
-    wd_wait_vm(OPS * (j < blk_begin ? nring - 1 : nring - 2));
+    // (the iterations before block 0's values are requested issue keys only)
+    wd_wait_vm(nring == 2 ? 0 : OPS_K + (t - 1 >= blk_begin - nring + 1 ? OPS_V : 0));
     WD_T(0);
-    __syncthreads();      // every wavefront's requests have landed; everyone is done with the slots refilled next, and sees the softmax of block j
+    __syncthreads();
     WD_T(1);
-    if (2 * j >= pbase + 64) {                  // (uniform) the table registers move on
+    if (t >= blk_begin && 2 * t >= pbase + 64) {                  // (uniform) the table registers move on
       pbase += 64;
       tbl_a = tbl_b;
       tbl_b = load_tbl(pbase + 64);
       asm volatile("" : "+v"(tbl_b));           // (the wait for this load: here, once in 32 blocks)
     }
-    if (j >= blk_begin) {
-      issue_keys();
-      issue_vals();
-      WD_T(2);
-      if (!helper) values(j, vs);
+    issue_keys();
+    if (t >= blk_begin - nring + 1) issue_vals();
+    WD_T(2);
+    if (t >= blk_begin) {
+      if (!helper) values(t, vs, t & 1);
       vs = vs + 1 == nring ? 0 : vs + 1;
-      WD_T(3);
     }
-    if (j + 1 < blk_end) score_units(ks);
-    WD_T(4);
-    __syncthreads();
-    WD_T(5);
-    if (helper && j + 1 < blk_end) softmax(j + 1, ks);
+    WD_T(3);
+    if (t + 2 < blk_end) score_units(ks, t & 1);
     ks = ks + 1 == nring ? 0 : ks + 1;
-    WD_T(6);
+    WD_T(4);
+    if (helper && t + 1 >= blk_begin && t + 1 < blk_end) softmax(t + 1, (t + 1) & 1);
+    WD_T(5);
   }
 #ifdef WD_PROF
   if (blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && lane == 0)
@@ -658,25 +724,21 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
 
 // LDS plan of the kernel for a layer: ring depth, slot sizes, bytes; false when it does not fit
 static bool wide_plan(const tq_layer& ly, const tq_page_layout& L, int& nring, int& kslot, int& vslot, size_t& smem) {
-  const int d = ly.d, wplt = (d + 127) / 128, mb = ly.mse_bits;
+  const int mb = ly.mse_bits;
   int nx = 0;
   for (int t = 0; t < ly.n_terms; ++t)
     if (__builtin_popcount(ly.term_mask[t]) > 1) ++nx;
   if (mb < 1 || mb > 4 || nx != (mb == 3 ? 1 : (mb == 4 ? 4 : 0))) return false;
-  const int ntp = mb + nx + 1;
-  kslot = ((L.off_vdata + 1023) / 1024) * 1024;
-  vslot = ((L.page_bytes - L.off_vdata + 1023) / 1024) * 1024;
-  const size_t fixed = (size_t)ntp * wplt * 2 * WD_QA_OP * 4 + (size_t)2 * wplt * 1024 + (size_t)WD_SMALL_FLOATS * 4;
-  const size_t block = (size_t)2 * (kslot + vslot);
-  if (fixed + 2 * block > (size_t)WD_LDS_BYTES) return false;
-  nring = fixed + 3 * block <= (size_t)WD_LDS_BYTES ? 3 : 2;
-  // (the waits count the requests of the blocks behind the current one: an immediate operand, sixteen at most)
-  const int nw = d / 64 + 1, ops = (2 * (kslot / 1024) + nw - 1) / nw + (2 * (vslot / 1024) + nw - 1) / nw;
-  if ((2 * (kslot / 1024) + nw - 1) / nw > 4 || (2 * (vslot / 1024) + nw - 1) / nw > 4) return false;
-  if (ops * (nring - 1) > 16) nring = 2;
-  if (ops * (nring - 1) > 16) return false;
-  smem = fixed + (size_t)nring * block;
-  return true;
+  const WidePlan p = wide_plan_of(ly.d, mb, L.off_vdata, L.page_bytes);
+  nring = p.nring; kslot = p.kslot; vslot = p.vslot; smem = (size_t)p.smem;
+  return p.ok;
+}
+
+// whether the page layout is the one the constant-geometry instantiations assume
+static bool wide_geom_matches(const tq_page_layout& L) {
+  const WideGeom g = wide_geom(L.d, L.mse_bits, L.value_bits);
+  return L.off_keys == 0 && L.off_meta == g.off_meta && L.off_vdata == g.off_vdata && L.off_vscale == g.off_vscale &&
+         L.off_vzero == g.off_vzero && L.page_bytes == g.page_bytes && L.key_lane_major == g.key_lane_major && L.group_size == 32;
 }
 
 bool decode_wide_has_kernel(const tq_layer& ly, const tq_page_layout& L) {
@@ -706,9 +768,9 @@ int launch_decode_wide(const float* q_rot, const float* q_sk, int B, int Hq, int
   const dim3 grid(n_split, Hkv * kv_div, B), block(ly.d + 64);      // (one wavefront more than channels / 64: the helper)
   hipEvent_t t_start = nullptr, t_stop = nullptr;
   const bool timed = take_time_hook(0, t_start, t_stop);
-#define TQ_LAUNCH_WIDE(VB, MB)                                                                                        \
+#define TQ_LAUNCH_WIDE(D, VB, MB)                                                                                     \
   {                                                                                                                   \
-    auto kern = decode_wide_kernel<VB, MB>;                                                                           \
+    auto kern = L.dtype == TQ_F16 ? decode_wide_kernel<D, VB, MB, true> : decode_wide_kernel<D, VB, MB, false>;                                                                        \
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);     \
     if (e != hipSuccess) return (int)e;                                                                               \
     if (timed)                                                                                                        \
@@ -720,16 +782,25 @@ int launch_decode_wide(const float* q_rot, const float* q_sk, int B, int Hq, int
                                       ly, L, parts, n_parts, n_split, len_sub, max_pages, num_pages, nring, kslot,    \
                                       vslot);                                                                         \
   }
-#define TQ_LAUNCH_WIDE_MB(VB)                        \
-  {                                                  \
-    if (ly.mse_bits == 1) TQ_LAUNCH_WIDE(VB, 1)      \
-    else if (ly.mse_bits == 2) TQ_LAUNCH_WIDE(VB, 2) \
-    else if (ly.mse_bits == 3) TQ_LAUNCH_WIDE(VB, 3) \
-    else TQ_LAUNCH_WIDE(VB, 4)                       \
+#define TQ_LAUNCH_WIDE_MB(D, VB)                        \
+  {                                                     \
+    if (ly.mse_bits == 1) TQ_LAUNCH_WIDE(D, VB, 1)      \
+    else if (ly.mse_bits == 2) TQ_LAUNCH_WIDE(D, VB, 2) \
+    else if (ly.mse_bits == 3) TQ_LAUNCH_WIDE(D, VB, 3) \
+    else TQ_LAUNCH_WIDE(D, VB, 4)                       \
   }
-  if (L.value_bits == 2) TQ_LAUNCH_WIDE_MB(2)
-  else if (L.value_bits == 4) TQ_LAUNCH_WIDE_MB(4)
-  else TQ_LAUNCH_WIDE_MB(8)
+#define TQ_LAUNCH_WIDE_VB(D)                            \
+  {                                                     \
+    if (L.value_bits == 2) TQ_LAUNCH_WIDE_MB(D, 2)      \
+    else if (L.value_bits == 4) TQ_LAUNCH_WIDE_MB(D, 4) \
+    else TQ_LAUNCH_WIDE_MB(D, 8)                        \
+  }
+  // the head sizes of latent attention have instantiations with constant geometry (for the layout the library makes)
+  const bool fixed_geom = wide_geom_matches(L) && opt_wide_heads.load(std::memory_order_relaxed) != 2;
+  if (fixed_geom && ly.d == 576) TQ_LAUNCH_WIDE_VB(576)
+  else if (fixed_geom && ly.d == 512) TQ_LAUNCH_WIDE_VB(512)
+  else TQ_LAUNCH_WIDE_VB(0)
+#undef TQ_LAUNCH_WIDE_VB
 #undef TQ_LAUNCH_WIDE_MB
 #undef TQ_LAUNCH_WIDE
   TQ_CHECK_LAUNCH();

@@ -16,6 +16,10 @@ namespace tq {
 // slices meet in LDS.
 constexpr int ROT_COLS = 32, ROT_SLICES = 8;
 
+// BATCH: matrix rows of both matrices requested before the first is used (8, 16 or 24, a divisor of the d / 8 rows a
+// thread contracts): the kernel is a chain of memory latencies, one per batch (head_dim 576: 9 -> 3; the sums add in
+// the same order whatever the batch).
+template <int BATCH>
 __global__ void __launch_bounds__(ROT_COLS * ROT_SLICES)
 rotate_query_kernel(const void* __restrict__ q, int dtype, int64_t rows, int R, tq_layer ly, float* __restrict__ q_rot,
                     float* __restrict__ q_sk) {
@@ -33,11 +37,11 @@ rotate_query_kernel(const void* __restrict__ q, int dtype, int64_t rows, int R, 
   float a[ROT_MAX_ROWS], b[ROT_MAX_ROWS];
 #pragma unroll
   for (int r = 0; r < ROT_MAX_ROWS; ++r) a[r] = b[r] = 0.0f;
-  // eight matrix rows at a time: all sixteen loads are in flight before the first use
-  for (int ib = i0; ib < i0 + per; ib += 8) {
-    float mp[8], ms[8];
+  // BATCH matrix rows at a time: all their loads are in flight before the first use
+  for (int ib = i0; ib < i0 + per; ib += BATCH) {
+    float mp[BATCH], ms[BATCH];
 #pragma unroll
-    for (int k = 0; k < 8; ++k) {
+    for (int k = 0; k < BATCH; ++k) {
       mp[k] = ly.PiT[(int64_t)(ib + k) * d + j];
       ms[k] = ly.ST[(int64_t)(ib + k) * d + j];
     }
@@ -45,7 +49,7 @@ rotate_query_kernel(const void* __restrict__ q, int dtype, int64_t rows, int R, 
     for (int r = 0; r < ROT_MAX_ROWS; ++r) {
       if (r < R) {
 #pragma unroll
-        for (int k = 0; k < 8; ++k) {
+        for (int k = 0; k < BATCH; ++k) {
           const float x = sq[r * d + ib + k];
           a[r] = fmaf(x, mp[k], a[r]);
           b[r] = fmaf(x, ms[k], b[r]);
@@ -479,8 +483,11 @@ int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* 
   const int R = (int)(rows < ROT_MAX_ROWS ? rows : ROT_MAX_ROWS);      // rows per workgroup
   if (R < 1 || d % ROT_COLS || d % (8 * ROT_SLICES)) return TQ_EUNSUPPORTED;
   size_t smem = (size_t)(R * d + 2 * ROT_SLICES * R * ROT_COLS) * sizeof(float);
-  rotate_query_kernel<<<dim3((unsigned)((rows + R - 1) / R), d / ROT_COLS), dim3(ROT_COLS * ROT_SLICES), smem, st>>>(
-      q, dtype, rows, R, *layer, q_rot, q_sk);
+  const dim3 rgrid((unsigned)((rows + R - 1) / R), d / ROT_COLS), rblock(ROT_COLS * ROT_SLICES);
+  const int per = d / ROT_SLICES;
+  if (per % 24 == 0) rotate_query_kernel<24><<<rgrid, rblock, smem, st>>>(q, dtype, rows, R, *layer, q_rot, q_sk);
+  else if (per % 16 == 0) rotate_query_kernel<16><<<rgrid, rblock, smem, st>>>(q, dtype, rows, R, *layer, q_rot, q_sk);
+  else rotate_query_kernel<8><<<rgrid, rblock, smem, st>>>(q, dtype, rows, R, *layer, q_rot, q_sk);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return (int)e;
   return TQ_OK;
