@@ -19,14 +19,18 @@ constexpr int ROT_COLS = 32, ROT_SLICES = 8;
 // BATCH: matrix rows of both matrices requested before the first is used (8, 16 or 24, a divisor of the d / 8 rows a
 // thread contracts): the kernel is a chain of memory latencies, one per batch (head_dim 576: 9 -> 3; the sums add in
 // the same order whatever the batch).
-template <int BATCH>
-__global__ void __launch_bounds__(ROT_COLS * ROT_SLICES)
+// HALVES (1 or 2): a workgroup of HALVES x 256 threads takes HALVES x 8 rows; the halves run the same loads a
+// moment apart, so the second finds the matrix lines in the compute unit's cache: with many rows half the traffic
+// from L2 for the same work per thread (128 rows at head_dim 576: 42 -> 21 MB).
+template <int BATCH, int HALVES>
+__global__ void __launch_bounds__(ROT_COLS * ROT_SLICES * HALVES)
 rotate_query_kernel(const void* __restrict__ q, int dtype, int64_t rows, int R, tq_layer ly, float* __restrict__ q_rot,
                     float* __restrict__ q_sk) {
-  extern __shared__ float sm[];
-  const int d = ly.d, tid = threadIdx.x, jl = tid % ROT_COLS, sl = tid / ROT_COLS;
+  extern __shared__ __align__(16) float sm[];
+  constexpr int T1 = ROT_COLS * ROT_SLICES;
+  const int d = ly.d, tid = threadIdx.x, half = tid / T1, t1 = tid - half * T1, jl = t1 % ROT_COLS, sl = t1 / ROT_COLS;
   const int j = blockIdx.y * ROT_COLS + jl;
-  float* sq = sm;                                  // [R][d] inputs
+  float* sq = sm;                                  // [R][d] inputs (R rows per workgroup: up to 8 per half)
   float* pa = sq + R * d;                          // [ROT_SLICES][R][ROT_COLS] partial sums
   float* pb = pa + ROT_SLICES * R * ROT_COLS;
   const int64_t row0 = (int64_t)blockIdx.x * R;
@@ -34,6 +38,7 @@ rotate_query_kernel(const void* __restrict__ q, int dtype, int64_t rows, int R, 
   for (int o = tid; o < R * d; o += blockDim.x) sq[o] = o < nr * d ? load_as_f32(q, row0 * d + o, dtype) : 0.0f;
   __syncthreads();
   const int per = d / ROT_SLICES, i0 = sl * per;
+  const int r0 = half * ROT_MAX_ROWS, RH = min(R - r0, ROT_MAX_ROWS);      // this half's rows: r0 .. r0 + RH - 1
   float a[ROT_MAX_ROWS], b[ROT_MAX_ROWS];
 #pragma unroll
   for (int r = 0; r < ROT_MAX_ROWS; ++r) a[r] = b[r] = 0.0f;
@@ -47,21 +52,25 @@ rotate_query_kernel(const void* __restrict__ q, int dtype, int64_t rows, int R, 
     }
 #pragma unroll
     for (int r = 0; r < ROT_MAX_ROWS; ++r) {
-      if (r < R) {
+      if (r < RH) {
 #pragma unroll
-        for (int k = 0; k < BATCH; ++k) {
-          const float x = sq[r * d + ib + k];
-          a[r] = fmaf(x, mp[k], a[r]);
-          b[r] = fmaf(x, ms[k], b[r]);
+        for (int k4 = 0; k4 < BATCH / 4; ++k4) {
+          const float4 x4 = *(const float4*)(sq + (r0 + r) * d + ib + 4 * k4);      // (ib and d are multiples of 8)
+          const float xs[4] = {x4.x, x4.y, x4.z, x4.w};
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            a[r] = fmaf(xs[k], mp[4 * k4 + k], a[r]);
+            b[r] = fmaf(xs[k], ms[4 * k4 + k], b[r]);
+          }
         }
       }
     }
   }
 #pragma unroll
   for (int r = 0; r < ROT_MAX_ROWS; ++r) {
-    if (r < R) {
-      pa[(sl * R + r) * ROT_COLS + jl] = a[r];
-      pb[(sl * R + r) * ROT_COLS + jl] = b[r];
+    if (r < RH) {
+      pa[(sl * R + r0 + r) * ROT_COLS + jl] = a[r];
+      pb[(sl * R + r0 + r) * ROT_COLS + jl] = b[r];
     }
   }
   __syncthreads();
@@ -480,14 +489,33 @@ int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* 
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? TQ_OK : (int)e;
   }
-  const int R = (int)(rows < ROT_MAX_ROWS ? rows : ROT_MAX_ROWS);      // rows per workgroup
+  // rows per workgroup: 8, or 16 (two halves of 256 threads) when that still leaves a workgroup for half the compute units
+  const bool wide_rows = rows >= 32 && ((rows + 15) / 16) * (d / ROT_COLS) >= device_compute_units() / 2;
+  const int max_r = wide_rows ? 16 : ROT_MAX_ROWS;
+  const int R = (int)(rows < max_r ? rows : max_r);
   if (R < 1 || d % ROT_COLS || d % (8 * ROT_SLICES)) return TQ_EUNSUPPORTED;
   size_t smem = (size_t)(R * d + 2 * ROT_SLICES * R * ROT_COLS) * sizeof(float);
-  const dim3 rgrid((unsigned)((rows + R - 1) / R), d / ROT_COLS), rblock(ROT_COLS * ROT_SLICES);
+  const dim3 rgrid((unsigned)((rows + R - 1) / R), d / ROT_COLS), rblock(ROT_COLS * ROT_SLICES * (wide_rows ? 2 : 1));
   const int per = d / ROT_SLICES;
-  if (per % 24 == 0) rotate_query_kernel<24><<<rgrid, rblock, smem, st>>>(q, dtype, rows, R, *layer, q_rot, q_sk);
-  else if (per % 16 == 0) rotate_query_kernel<16><<<rgrid, rblock, smem, st>>>(q, dtype, rows, R, *layer, q_rot, q_sk);
-  else rotate_query_kernel<8><<<rgrid, rblock, smem, st>>>(q, dtype, rows, R, *layer, q_rot, q_sk);
+#define TQ_ROTATE(BATCH, MAXR)                                                                                         \
+  {                                                                                                                    \
+    auto kern = rotate_query_kernel<BATCH, MAXR>;                                                                      \
+    if (smem > 48 * 1024) {                                                                                            \
+      hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);    \
+      if (e != hipSuccess) return (int)e;                                                                              \
+    }                                                                                                                  \
+    kern<<<rgrid, rblock, smem, st>>>(q, dtype, rows, R, *layer, q_rot, q_sk);                                         \
+  }
+#define TQ_ROTATE_R(BATCH)                 \
+  {                                        \
+    if (wide_rows) TQ_ROTATE(BATCH, 2)     \
+    else TQ_ROTATE(BATCH, 1)               \
+  }
+  if (per % 24 == 0) TQ_ROTATE_R(24)
+  else if (per % 16 == 0) TQ_ROTATE_R(16)
+  else TQ_ROTATE_R(8)
+#undef TQ_ROTATE_R
+#undef TQ_ROTATE
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return (int)e;
   return TQ_OK;
