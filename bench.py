@@ -481,8 +481,8 @@ def cpu_quantize_baseline(k, v, tq, sample_tokens=32768):
 
 # (sequences, context, query heads, KV heads, head_dim, key bits, value bits): every family of decode kernels -
 # head_dim 64 / 128 / 256 on the matrix cores with 2- / 3- / 4-bit keys and 2- / 4- / 8-bit values, 1 to 16 query
-# heads per KV head (11 as 6 + 5), 5-bit keys at head_dim 128, short and long contexts - and the general kernel's shape
-# (head_dim 576)
+# heads per KV head (11 as 6 + 5), 5-bit keys at head_dim 128, short and long contexts - and the head sizes of latent
+# attention (512, 576) on the kernel that works on a block per workgroup
 SHAPE_TABLE = [
     (4, 131072, 16, 2, 256, 3, 2), (4, 131072, 16, 2, 256, 2, 2), (4, 131072, 16, 2, 256, 4, 2),
     (4, 131072, 16, 2, 256, 3, 4), (4, 131072, 8, 2, 256, 3, 2), (4, 131072, 2, 2, 256, 3, 2),
@@ -493,7 +493,8 @@ SHAPE_TABLE = [
     (1, 131072, 32, 8, 128, 3, 4),
     (16, 8192, 32, 8, 64, 3, 4), (16, 8192, 32, 8, 64, 2, 2), (16, 8192, 32, 8, 64, 4, 4), (16, 8192, 64, 8, 64, 3, 4),
     (32, 32768, 32, 8, 64, 3, 4),
-    (16, 8192, 8, 1, 576, 4, 4), (16, 8192, 32, 8, 128, 5, 4), (16, 8192, 64, 8, 128, 5, 4), (16, 8192, 32, 8, 128, 3, 8),
+    (16, 8192, 8, 1, 576, 4, 4), (32, 8192, 8, 1, 576, 4, 4), (4, 32768, 16, 1, 576, 4, 4), (16, 8192, 8, 1, 512, 3, 4),
+    (16, 8192, 32, 8, 128, 5, 4), (16, 8192, 64, 8, 128, 5, 4), (16, 8192, 32, 8, 128, 3, 8),
     (16, 8192, 88, 8, 128, 3, 4),
 ]
 
@@ -511,6 +512,8 @@ def shape_table(device, steps, warmup):
         hyb = hybrid_step_bench(w, steps, warmup)
         rows.append({"sequences": B, "context": N, "q_heads": Hq, "kv_heads": Hkv, "head_dim": d, "key_bits": kb,
                      "value_bits": vb, "n_split": w.n_split, "bytes_per_step": w.bytes,
+                     "page_kernel": ("general (vector ALU)", "matrix cores, a block per wavefront",
+                                     "matrix cores, a block per workgroup")[w.pools[0].page_kernel()],
                      "step_us": round(ms * 1e3, 2), "step_pct_hbm_peak": round(100.0 * w.bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 1),
                      "page_kernel_us": round(kern * 1e3, 2),
                      "page_kernel_pct_hbm_peak": round(100.0 * w.bytes / (kern * 1e-3) / 1e9 / HBM_PEAK_GBS, 1),
