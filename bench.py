@@ -499,12 +499,12 @@ SHAPE_TABLE = [
 ]
 
 
-def shape_table(device, steps, warmup):
+def shape_table(device, steps, warmup, table=None):
     """Whole-step and page-kernel times of SHAPE_TABLE's decode shapes (timing only; N(0,1) data from the card's
     generator), compressed-only and with the newest 128 tokens exact."""
     import torch
     rows = []
-    for (B, N, Hq, Hkv, d, kb, vb) in SHAPE_TABLE:
+    for (B, N, Hq, Hkv, d, kb, vb) in (table or SHAPE_TABLE):
         w = DecodeWorkload("shape", B, N, Hq, Hkv, d, kb, vb, n_pools=2 if B * N * Hkv >= 1 << 22 else 4, seed=5,
                            dist="normal", device=device, device_data=True)
         ms, _ = time_steps(w.step, steps, warmup)
@@ -572,6 +572,42 @@ def phase_stamps(device, reps=40):
     return out
 
 
+def wide_phases(device, reps=20):
+    """Time the wavefronts of one workgroup of the wide-head page kernel (head_dim 576) spend in each part of its loop,
+    summed over the workgroup's blocks.  Needs a library built with -DWD_PROF (every wavefront of workgroup (0, 0, 0)
+    then sums the 100 MHz real-time counter between the parts)."""
+    import ctypes
+    import numpy as np
+    import torch
+    from turboquant_amd import _ffi
+    lib = _ffi.lib()
+    if not hasattr(lib, "tq_debug_wide_prof"):
+        raise SystemExit("this libtq_hip.so has no phase sums: build it with TQ_EXTRA_HIPCC_FLAGS=-DWD_PROF")
+    fn = lib.tq_debug_wide_prof
+    fn.argtypes = [ctypes.c_void_p, ctypes.c_int]
+    B, N, Hq, Hkv, d, kb, vb = 16, 8192, 8, 1, 576, 4, 4
+    w = DecodeWorkload("wide head", B, N, Hq, Hkv, d, kb, vb, n_pools=2, seed=5, dist="normal", device=device, device_data=True)
+    for i in range(300):
+        w.step(i)
+    torch.cuda.synchronize()
+    kern = time_kernel_stage(w, 100, 20)
+    acc = []
+    for r in range(reps):
+        w.step(r)
+        torch.cuda.synchronize()
+        buf = (ctypes.c_ulonglong * 96)()
+        if fn(buf, 96) != 0:
+            raise SystemExit("reading the phase sums failed")
+        acc.append(np.frombuffer(buf, dtype=np.uint64).reshape(12, 8).astype(np.float64))
+    a = np.mean(acc, axis=0) / 100.0                      # microseconds
+    names = {0: "wait for page data", 1: "barrier", 2: "page requests", 3: "values", 4: "scores", 5: "softmax", 7: "loop overhead"}
+    n_waves = d // 64 + 1
+    return {"workload": f"{B} x {N}, {Hq} q / {Hkv} KV heads, head_dim {d}, keys {kb}b, values {vb}b", "n_split": w.n_split,
+            "blocks_per_workgroup": (N // 32) // w.n_split, "kernel_us_with_the_counters_in": round(kern * 1e3, 2),
+            "sums_over_the_loop_us": [{"wavefront": wv, **{names[k]: round(float(a[wv, k]), 2) for k in names},
+                                       "total": round(float(a[wv].sum()), 2)} for wv in range(n_waves)]}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -593,6 +629,10 @@ def main():
                     help="per-phase times inside the page kernel of the long-context and the 16 x 8192 workloads, from "
                          "the real-time counter stamps of a library built with TQ_EXTRA_HIPCC_FLAGS=-DTQ_STAMPS "
                          "(a profiling build; the shipped one has no stamps and this mode then exits)")
+    ap.add_argument("--shape", action="append", default=[], metavar="B,N,Hq,Hkv,d,key_bits,value_bits",
+                    help="with --shapes semantics, time this decode shape instead of the table (repeatable)")
+    ap.add_argument("--wide-phases", action="store_true",
+                    help="per-part time sums of the wide-head page kernel's loop (needs a library built with -DWD_PROF)")
     ap.add_argument("--quantize-only", action="store_true",
                     help="run the prefill-quantize leg alone and print its object (for profiles of its kernels)")
     args = ap.parse_args()
@@ -610,9 +650,16 @@ def main():
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
 
-    if args.shapes:
+    if args.shapes or args.shape:
+        table = [tuple(int(x) for x in sh.split(",")) for sh in args.shape] or SHAPE_TABLE
+        if any(len(sh) != 7 for sh in table):
+            raise SystemExit("--shape takes seven comma-separated integers: B,N,Hq,Hkv,d,key_bits,value_bits")
         print(json.dumps({"metric": "decode step over a table of shapes, 1 GPU", "steps": args.steps, "warmup": args.warmup,
-                          "shapes": shape_table(device, args.steps, args.warmup)}))
+                          "shapes": shape_table(device, args.steps, args.warmup, table)}))
+        return
+
+    if args.wide_phases:
+        print(json.dumps({"metric": "wide-head page kernel, time per part of the loop, 1 GPU", "phases": wide_phases(device)}))
         return
 
     if args.phase_stamps:

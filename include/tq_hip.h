@@ -362,6 +362,10 @@ void tq_time_next_key_kernel(void *start_event, void *stop_event);
  *   "wide_workgroups"  1 (default): at head_dim 64 / 128, with an even split count and at most 16 blocks of 64 tokens
  *                      per wavefront (judged by the width of the block table), a step runs workgroups of 8
  *                      wavefronts on half the split count it was given; 0: always 4 wavefronts per workgroup.
+ *   "wide_heads"       1 (default): head sizes 320 .. 704 (16-bit pages, value groups of 32) run the matrix-core page kernel
+ *                      that works on a block of 32 tokens per workgroup, 512 and 576 in instantiations with constant page
+ *                      geometry; 2: every such head size on the instantiation that takes the geometry at run time (same
+ *                      result bit for bit); 0: the general vector-ALU kernel (results agree to rounding).
  *   "append_small"     -1 (default), 0, or a tile count: an append to pages of at most this many 16-vector tiles (-1: two
  *                      per compute unit) gives every tile a workgroup that computes that tile only - the page write of
  *                      a decode step, a token per sequence; 0: always workgroups over groups of tiles.  Same bytes.

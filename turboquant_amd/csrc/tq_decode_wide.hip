@@ -200,19 +200,18 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
     return rel < 64 ? ea : eb;
   };
   // Requests for the key part / value part of the next block of each kind into its ring slot: a kilobyte per
-  // instruction, dealt to the wavefronts; every wavefront issues the same number per block (the waits below count
-  // them), surplus ones repeat the last piece; the last piece of a part re-reads its final 16 bytes into the slot's
-  // padding.  Blocks are requested in order, so the block and its slot are running counters; behind the last block
-  // of the range the requests repeat it (into the slot it already has).  What does not depend on the block - which
-  // page of the pair, the offset inside the page, the offset inside the slot - is worked out once.
+  // instruction, the pieces dealt to the wavefronts (a wavefront counts its own requests in the waits below, so the
+  // numbers need not be equal).  Blocks are requested in order, so the block and its slot are running counters;
+  // behind the last block of the range the requests repeat it (into the slot it already has).  What does not depend
+  // on the block - which page of the pair, the offset inside the page, the offset inside the slot - is worked out once.
   const int kbytes = L.off_vdata, vbytes = L.page_bytes - L.off_vdata;
   const int PK = (kbytes + 1023) >> 10, PV = (vbytes + 1023) >> 10;
-  const int OPS_K = (2 * PK + NWS - 1) / NWS, OPS_V = (2 * PV + NWS - 1) / NWS, OPS = OPS_K + OPS_V;
   constexpr int WD_MAX_OPS = 4;                 // per kind (the plan on the host keeps to it)
-  struct Req { int blk, slot; uint32_t src_off[WD_MAX_OPS]; int lds_off[WD_MAX_OPS]; int pg[WD_MAX_OPS]; };
+  struct Req { int blk, slot, n; uint32_t src_off[WD_MAX_OPS]; int lds_off[WD_MAX_OPS]; int pg[WD_MAX_OPS]; };
   auto req_init = [&](Req& r, int pieces, int slot_bytes, int part_off, int part_bytes) {
     r.blk = blk_begin;
     r.slot = 0;
+    r.n = wave < 2 * pieces ? (2 * pieces - wave + NWS - 1) / NWS : 0;      // pieces wave, wave + NWS, ...
 #pragma unroll
     for (int k = 0; k < WD_MAX_OPS; ++k) {
       const int piece = min(wave + k * NWS, 2 * pieces - 1);
@@ -227,22 +226,23 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
   req_init(rq_k, PK, kslot, 0, kbytes);
   req_init(rq_v, PV, vslot, kbytes, vbytes);
   const uint32_t kring_lds = (uint32_t)(uintptr_t)kring, vring_lds = (uint32_t)(uintptr_t)vring;
-  auto issue = [&](Req& r, uint32_t ring_lds, int slot_bytes, int ops) __attribute__((always_inline)) {
+  auto issue = [&](Req& r, uint32_t ring_lds, int slot_bytes) __attribute__((always_inline)) {
     const uint32_t pid0 = (uint32_t)page_entry(2 * r.blk) & 0x7fffffffu, pid1 = (uint32_t)page_entry(2 * r.blk + 1) & 0x7fffffffu;
     const uint8_t* base0 = pool_h + (uint64_t)pid0 * page_stride32;
     const uint8_t* base1 = pool_h + (uint64_t)pid1 * page_stride32;
     const uint32_t slot_lds = ring_lds + (uint32_t)(r.slot * 2 * slot_bytes);
 #pragma unroll
     for (int k = 0; k < WD_MAX_OPS; ++k)
-      if (k < ops)
+      if (k < r.n)
         dma16<0>((r.pg[k] ? base1 : base0) + r.src_off[k], (uint32_t)__builtin_amdgcn_readfirstlane((int)(slot_lds + (uint32_t)r.lds_off[k])));
     if (r.blk < blk_end - 1) {
       ++r.blk;
       r.slot = r.slot + 1 == nring ? 0 : r.slot + 1;
     }
   };
-  auto issue_keys = [&]() __attribute__((always_inline)) { issue(rq_k, kring_lds, kslot, OPS_K); };
-  auto issue_vals = [&]() __attribute__((always_inline)) { issue(rq_v, vring_lds, vslot, OPS_V); };
+  auto issue_keys = [&]() __attribute__((always_inline)) { issue(rq_k, kring_lds, kslot); };
+  auto issue_vals = [&]() __attribute__((always_inline)) { issue(rq_v, vring_lds, vslot); };
+  const int OPS_K = rq_k.n, OPS_V = rq_v.n;     // this wavefront's requests per block
   // the keys of the first blocks are on their way while the operands are prepared
   for (int i = 0; i < nring - 1; ++i) issue_keys();
 
@@ -650,6 +650,7 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
   // t + nring - 1 into the slots the blocks t + 1 and t - 1 had, so at its top the requests of iteration t - nring + 1
   // (keys t + 2, values t) have to have landed and those of the nring - 2 iterations after it may be outstanding.
   int ks = 0, vs = 0;                           // ring slots of the keys of block t + 2 and the values of block t
+  const int issue_at = helper ? 2 : wave % 3;
 #ifdef WD_PROF
   unsigned long long wd_t[8] = {0, 0, 0, 0, 0, 0, 0, 0}, wd_last = wall_clock64();
 #endif
@@ -666,17 +667,24 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
       tbl_b = load_tbl(pbase + 64);
       asm volatile("" : "+v"(tbl_b));           // (the wait for this load: here, once in 32 blocks)
     }
-    issue_keys();
-    if (t >= blk_begin - nring + 1) issue_vals();
+    // (the requests of a compute unit's wavefronts all pass through its one address unit: a third of the wavefronts
+    // issue theirs here, a third between the stages, a third behind them)
+    auto requests = [&]() __attribute__((always_inline)) {
+      issue_keys();
+      if (t >= blk_begin - nring + 1) issue_vals();
+    };
+    if (issue_at == 0) requests();
     WD_T(2);
     if (t >= blk_begin) {
       if (!helper) values(t, vs, t & 1);
       vs = vs + 1 == nring ? 0 : vs + 1;
     }
     WD_T(3);
+    if (issue_at == 1) requests();
     if (t + 2 < blk_end) score_units(ks, t & 1);
     ks = ks + 1 == nring ? 0 : ks + 1;
     WD_T(4);
+    if (issue_at == 2) requests();
     if (helper && t + 1 >= blk_begin && t + 1 < blk_end) softmax(t + 1, (t + 1) & 1);
     WD_T(5);
   }
