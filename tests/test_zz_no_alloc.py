@@ -43,7 +43,7 @@ def _both(gpu, pool, tq, q, table, seq, n_split, rk=None, rv=None, rl=None):
 # (8-bit values and 5-bit keys at head_dim 128 run the matrix-core kernel too; the last case, 5-bit keys at head_dim 64,
 # has no matrix-core kernel: the general page kernel runs on the static area)
 @pytest.mark.parametrize("d,key_bits,vb,Hq,Hkv", [(128, 3, 4, 8, 2), (256, 3, 2, 16, 2), (64, 3, 2, 4, 1), (128, 3, 8, 8, 2),
-                                                   (128, 5, 4, 8, 2), (64, 5, 2, 10, 2)])
+                                                   (128, 5, 4, 8, 2), (64, 5, 2, 10, 2), (576, 4, 4, 8, 1)])
 def test_static_scratch_decode_equals_the_workspace_form_on_consecutive_calls(gpu, d, key_bits, vb, Hq, Hkv):
     g = torch.Generator().manual_seed(d + Hq)
     B, N = 3, 900

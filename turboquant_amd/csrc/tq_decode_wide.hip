@@ -38,9 +38,12 @@ constexpr int WD_LDS_BYTES = 160 * 1024;
 // spends in each part of an iteration (100 MHz counter); tq_debug_wide_prof copies the sums out.
 #ifdef WD_PROF
 __device__ unsigned long long wd_prof[WD_MAX_WAVES * 8];
+__device__ unsigned long long wd_prof2[WD_MAX_WAVES * 8];   // prologue / epilogue stamps (absolute)
+#define WD_P(k) do { wd_p[k] = wall_clock64(); } while (0)
 #define WD_T(k) do { const unsigned long long t_ = wall_clock64(); wd_t[k] += t_ - wd_last; wd_last = t_; } while (0)
 #else
 #define WD_T(k)
+#define WD_P(k)
 #endif
 
 __device__ __forceinline__ void wd_wait_vm(int n) {
@@ -93,7 +96,7 @@ __host__ __device__ constexpr WidePlan wide_plan_of(int d, int mb, int off_vdata
   p.nring = fixed + 3 * block <= WD_LDS_BYTES ? 3 : 2;
   // (the waits count the requests of the iteration behind the current one: an immediate operand, sixteen at most;
   // a wavefront keeps the constants of at most four requests of a kind)
-  const int nw = d / 64 + 1, ops_k = (2 * ((p.kslot + 1023) / 1024) + nw - 1) / nw, ops_v = (2 * ((p.vslot + 1023) / 1024) + nw - 1) / nw;
+  const int nw = d / 64, ops_k = (2 * ((p.kslot + 1023) / 1024) + nw - 1) / nw, ops_v = (2 * ((p.vslot + 1023) / 1024) + nw - 1) / nw;
   p.ok = p.kslot >= 1024 && p.vslot >= 1024 && fixed + 2 * block <= WD_LDS_BYTES && ops_k <= 4 && ops_v <= 4 && ops_k + ops_v <= 16;
   p.smem = fixed + p.nring * block;
   return p;
@@ -136,6 +139,10 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
   const int G = min(g_max, g_tot - grp * g_max);
   if (G <= 0) return;
 
+#ifdef WD_PROF
+  unsigned long long wd_p[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#endif
+  WD_P(0);
   extern __shared__ __align__(16) unsigned char smem_raw[];
   // Query operands: per (term plane, row set) the chunks one after another; a last chunk of 64 coordinates (head_dim
   // not a multiple of 128) takes half an operand - the slots of the lanes of its upper two coordinate quarters do not
@@ -211,10 +218,12 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
   auto req_init = [&](Req& r, int pieces, int slot_bytes, int part_off, int part_bytes) {
     r.blk = blk_begin;
     r.slot = 0;
-    r.n = wave < 2 * pieces ? (2 * pieces - wave + NWS - 1) / NWS : 0;      // pieces wave, wave + NWS, ...
+    // pieces wave, wave + NW, ... for the channel wavefronts; none for the helper, whose chain (score unit, softmax) is
+    // the longest of an iteration
+    r.n = wave < NW && wave < 2 * pieces ? (2 * pieces - wave + NW - 1) / NW : 0;
 #pragma unroll
     for (int k = 0; k < WD_MAX_OPS; ++k) {
-      const int piece = min(wave + k * NWS, 2 * pieces - 1);
+      const int piece = min(wave + k * NW, 2 * pieces - 1);
       const int pg = piece >= pieces ? 1 : 0, pc = piece - pg * pieces;
       r.pg[k] = pg;
       const int at = min(pc * 1024, part_bytes - 1024);     // (the last piece overlaps the one before it: a slot is as long as its part)
@@ -244,7 +253,9 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
   auto issue_vals = [&]() __attribute__((always_inline)) { issue(rq_v, vring_lds, vslot); };
   const int OPS_K = rq_k.n, OPS_V = rq_v.n;     // this wavefront's requests per block
   // the keys of the first blocks are on their way while the operands are prepared
+  WD_P(1);
   for (int i = 0; i < nring - 1; ++i) issue_keys();
+  WD_P(2);
 
   // ---------------------------------------------------------------- query operands (as the preparation kernel packs them)
   float cmax = 0.0f;
@@ -320,6 +331,7 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
     }
   }
   __syncthreads();
+  WD_P(3);
   // one lane per (term plane, head, plane word): the word's 32 values as four fp6 terms (the packing conversion
   // of gfx950 and its inverse for the residual), written where lane (row 2 head + term % 2, quarter word % 4) of
   // operand (plane, chunk word / 4, row set term / 2) reads them.  Rows of absent heads and the words past the
@@ -384,6 +396,7 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
     }
   }
   __syncthreads();
+  WD_P(4);
   // E8M0 block-scale codes of this lane's operand row (head n / 2; row 2g + t holds term t of row set 0 and term
   // t + 2 of row set 1): index planes row set 0, 1, sign plane row set 0, 1.  4 v / 2^E is stored, so term t
   // carries 2^(E - 2 - 5t); the fp4 bit value 0.5 carries 2^1.
@@ -688,6 +701,7 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
     if (helper && t + 1 >= blk_begin && t + 1 < blk_end) softmax(t + 1, (t + 1) & 1);
     WD_T(5);
   }
+  WD_P(5);
 #ifdef WD_PROF
   if (blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && lane == 0)
     for (int k = 0; k < 8; ++k) wd_prof[wave * 8 + k] = wd_t[k];
@@ -728,6 +742,11 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
       }
     }
   }
+  WD_P(6);
+#ifdef WD_PROF
+  if (blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && lane == 0)
+    for (int k = 0; k < 8; ++k) wd_prof2[wave * 8 + k] = wd_p[k];
+#endif
 }
 
 // LDS plan of the kernel for a layer: ring depth, slot sizes, bytes; false when it does not fit
@@ -820,5 +839,8 @@ int launch_decode_wide(const float* q_rot, const float* q_sk, int B, int Hq, int
 #ifdef WD_PROF
 extern "C" int tq_debug_wide_prof(unsigned long long* host, int n) {
   return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(tq::wd_prof), (size_t)n * 8);
+}
+extern "C" int tq_debug_wide_prof2(unsigned long long* host, int n) {
+  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(tq::wd_prof2), (size_t)n * 8);
 }
 #endif
