@@ -6,7 +6,7 @@
 // A wide head does not fit the per-wavefront design of the head_dim 64 / 128 / 256 kernel (its query operands and
 // accumulators would need several hundred registers), so here a whole workgroup works on one block of 32 tokens
 // (two pages) at a time:
-//   * one wavefront per 64 channels plus a helper wavefront (d + 64 threads), one workgroup per compute unit;
+//   * one wavefront per 64 channels plus one or two helper wavefronts, one workgroup per compute unit;
 //   * the pages travel HBM -> LDS as they lie in memory (LDS-direct loads, a kilobyte per instruction), the key
 //     part of a page (bit planes, norms) and its value part (codes, scales, zero points) into rings of their
 //     own, two or three blocks deep, so that the next block(s) arrive while the current ones are worked on;
@@ -126,9 +126,11 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
   }
   const int nring = D ? PC.nring : nring_rt, kslot = D ? PC.kslot : kslot_rt, vslot = D ? PC.vslot : vslot_rt;
   const int tid = threadIdx.x, lane = tid & 63;
-  // NW wavefronts own 64 channels each; one more (the helper, wavefront NW) owns none: it runs the softmax and takes
-  // score units like the others (head_dim 576: ten units for ten wavefronts)
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), NW = D ? D / 64 : ((int)blockDim.x >> 6) - 1, NWS = NW + 1;
+  // NW wavefronts own 64 channels each and take a score unit each.  Wavefront NW owns no channels: it runs the softmax
+  // (and the score units the others leave over, when it is the only helper).  A second helper, wavefront NW + 1, is
+  // launched when the block has more units than channel wavefronts and the workgroup has room (head_dim 576: nine
+  // channel wavefronts, ten units): it takes the units left over, so that no wavefront's chain is two stages long.
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), NWS = (int)blockDim.x >> 6, NW = D ? D / 64 : ly.d >> 6;
   const bool helper = wave == NW;
   const int n = lane & 15, kb = lane >> 4;
   const int split = blockIdx.x, b = blockIdx.z;
@@ -425,11 +427,14 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
     return min(max(seq_len - blk * WD_BLK - 16 * pg, 0), 16);
   };
 
-  // ---- scores of block blk: unit u = (page u % 2, chunk u / 2), dealt from the helper wavefront down
+  // ---- scores of block blk: unit u = (page u % 2, chunk u / 2)
   auto score_units = [&](int ring_slot, int pb) __attribute__((always_inline)) {
     const unsigned char* kslot0 = kring + (ring_slot * 2) * kslot;
     float* part = s_part + pb * (2 * WPLT * 256);
-    for (int u = NW - wave; u < 2 * WPLT; u += NWS) {
+    // unit `wave` for a channel wavefront; the units from NW on for the last wavefront of the workgroup (the second
+    // helper, or the only one)
+    const bool leftovers = wave == NWS - 1;
+    for (int u = wave < NW ? wave : (leftovers ? NW : 2 * WPLT); u < 2 * WPLT; u += leftovers ? 1 : 2 * WPLT) {
       const int pg = u & 1, i = u >> 1;
       const unsigned char* kp = kslot0 + pg * kslot;
       const int j = 4 * i + kb;
@@ -663,7 +668,7 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
   // t + nring - 1 into the slots the blocks t + 1 and t - 1 had, so at its top the requests of iteration t - nring + 1
   // (keys t + 2, values t) have to have landed and those of the nring - 2 iterations after it may be outstanding.
   int ks = 0, vs = 0;                           // ring slots of the keys of block t + 2 and the values of block t
-  const int issue_at = helper ? 2 : wave % 3;
+  const int issue_at = wave >= NW ? 2 : wave % 3;
 #ifdef WD_PROF
   unsigned long long wd_t[8] = {0, 0, 0, 0, 0, 0, 0, 0}, wd_last = wall_clock64();
 #endif
@@ -689,7 +694,7 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
     if (issue_at == 0) requests();
     WD_T(2);
     if (t >= blk_begin) {
-      if (!helper) values(t, vs, t & 1);
+      if (wave < NW) values(t, vs, t & 1);
       vs = vs + 1 == nring ? 0 : vs + 1;
     }
     WD_T(3);
@@ -710,7 +715,7 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
   // ---------------------------------------------------------------- the partial (m, l, acc[d]) of every head
   stage_wait<0>();                              // the surplus requests of the last trips have landed
   __syncthreads();
-  if (n < 2 && !helper) {
+  if (n < 2 && wave < NW) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) s_z[(wave * 16 + 4 * kb + i) * 2 + n] = zacc[i];
   }
@@ -729,7 +734,7 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
   __syncthreads();
   // accumulator rows 0..7 hold the heads for the tiles of the even group (tiles 0, 1), rows 8..15 for the odd
   // group (tiles 2, 3); the zero-point sums have the same rows in both halves
-  if (!helper) {
+  if (wave < NW) {
     const int par = kb >> 1;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -792,7 +797,11 @@ int launch_decode_wide(const float* q_rot, const float* q_sk, int B, int Hq, int
   int nring, kslot, vslot;
   size_t smem;
   wide_plan(ly, L, nring, kslot, vslot, smem);
-  const dim3 grid(n_split, Hkv * kv_div, B), block(ly.d + 64);      // (one wavefront more than channels / 64: the helper)
+  // one wavefront more than channels / 64 (the helper), two when the block's units outnumber the channel wavefronts
+  // and twelve wavefronts are not exceeded
+  const int nw = ly.d / 64, units = 2 * ((ly.d + 127) / 128);
+  const int helpers = units > nw && nw + 2 <= WD_MAX_WAVES ? 2 : 1;
+  const dim3 grid(n_split, Hkv * kv_div, B), block((nw + helpers) * 64);
   hipEvent_t t_start = nullptr, t_stop = nullptr;
   const bool timed = take_time_hook(0, t_start, t_stop);
 #define TQ_LAUNCH_WIDE(D, VB, MB)                                                                                     \
