@@ -601,8 +601,8 @@ def wide_phases(device, reps=20):
         acc.append(np.frombuffer(buf, dtype=np.uint64).reshape(12, 8).astype(np.float64))
     a = np.mean(acc, axis=0) / 100.0                      # microseconds
     names = {0: "wait for page data", 1: "barrier", 2: "page requests", 3: "values", 4: "scores", 5: "softmax", 7: "loop overhead"}
-    units, nw = 2 * ((d + 127) // 128), d // 64
-    n_waves = nw + (2 if units > nw and nw + 2 <= 12 else 1)      # channel wavefronts + helpers
+    nw = d // 64
+    n_waves = nw + (2 if nw + 2 <= 12 else 1)      # channel wavefronts + helpers
     return {"workload": f"{B} x {N}, {Hq} q / {Hkv} KV heads, head_dim {d}, keys {kb}b, values {vb}b", "n_split": w.n_split,
             "blocks_per_workgroup": (N // 32) // w.n_split, "kernel_us_with_the_counters_in": round(kern * 1e3, 2),
             "sums_over_the_loop_us": [{"wavefront": wv, **{names[k]: round(float(a[wv, k]), 2) for k in names},

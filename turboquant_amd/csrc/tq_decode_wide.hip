@@ -47,26 +47,15 @@ __device__ unsigned long long wd_prof2[WD_MAX_WAVES * 8];   // prologue / epilog
 #endif
 
 __device__ __forceinline__ void wd_wait_vm(int n) {
+#define WD_W(k) case k: stage_wait<k>(); break;
   switch (n) {
-    case 0: stage_wait<0>(); break;
-    case 1: stage_wait<1>(); break;
-    case 2: stage_wait<2>(); break;
-    case 3: stage_wait<3>(); break;
-    case 4: stage_wait<4>(); break;
-    case 5: stage_wait<5>(); break;
-    case 6: stage_wait<6>(); break;
-    case 7: stage_wait<7>(); break;
-    case 8: stage_wait<8>(); break;
-    case 9: stage_wait<9>(); break;
-    case 10: stage_wait<10>(); break;
-    case 11: stage_wait<11>(); break;
-    case 12: stage_wait<12>(); break;
-    case 13: stage_wait<13>(); break;
-    case 14: stage_wait<14>(); break;
-    case 15: stage_wait<15>(); break;
-    case 16: stage_wait<16>(); break;
+    WD_W(0) WD_W(1) WD_W(2) WD_W(3) WD_W(4) WD_W(5) WD_W(6) WD_W(7) WD_W(8) WD_W(9) WD_W(10) WD_W(11) WD_W(12) WD_W(13) WD_W(14) WD_W(15)
+    WD_W(16) WD_W(17) WD_W(18) WD_W(19) WD_W(20) WD_W(21) WD_W(22) WD_W(23) WD_W(24) WD_W(25) WD_W(26) WD_W(27) WD_W(28) WD_W(29) WD_W(30)
+    WD_W(31) WD_W(32) WD_W(33) WD_W(34) WD_W(35) WD_W(36) WD_W(37) WD_W(38) WD_W(39) WD_W(40) WD_W(41) WD_W(42) WD_W(43) WD_W(44) WD_W(45)
+    WD_W(46) WD_W(47) WD_W(48)
     default: stage_wait<0>(); break;       // (stricter than asked: always safe)
   }
+#undef WD_W
 }
 
 // The page geometry tq_page_layout_init gives 16-bit pages with groups of 32, and the kernel's LDS plan, as functions
@@ -97,7 +86,8 @@ __host__ __device__ constexpr WidePlan wide_plan_of(int d, int mb, int off_vdata
   // (the waits count the requests of the iteration behind the current one: an immediate operand, sixteen at most;
   // a wavefront keeps the constants of at most four requests of a kind)
   const int nw = d / 64, ops_k = (2 * ((p.kslot + 1023) / 1024) + nw - 1) / nw, ops_v = (2 * ((p.vslot + 1023) / 1024) + nw - 1) / nw;
-  p.ok = p.kslot >= 1024 && p.vslot >= 1024 && fixed + 2 * block <= WD_LDS_BYTES && ops_k <= 4 && ops_v <= 4 && ops_k + ops_v <= 16;
+  p.ok = p.kslot >= 1024 && p.vslot >= 1024 && fixed + 2 * block <= WD_LDS_BYTES && (p.nring == 2 || 2 * ((p.kslot + 1023) / 1024 + (p.vslot + 1023) / 1024) <= 48);
+  (void)ops_k; (void)ops_v;
   p.smem = fixed + p.nring * block;
   return p;
 }
@@ -126,10 +116,10 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
   }
   const int nring = D ? PC.nring : nring_rt, kslot = D ? PC.kslot : kslot_rt, vslot = D ? PC.vslot : vslot_rt;
   const int tid = threadIdx.x, lane = tid & 63;
-  // NW wavefronts own 64 channels each and take a score unit each.  Wavefront NW owns no channels: it runs the softmax
-  // (and the score units the others leave over, when it is the only helper).  A second helper, wavefront NW + 1, is
-  // launched when the block has more units than channel wavefronts and the workgroup has room (head_dim 576: nine
-  // channel wavefronts, ten units): it takes the units left over, so that no wavefront's chain is two stages long.
+  // NW wavefronts own 64 channels each and take a score unit each.  Wavefront NW owns no channels: it runs the softmax.
+  // The last wavefront of the workgroup - a second helper, or the same one when the workgroup has no room for two -
+  // issues the page requests and takes the score units the channel wavefronts leave over (head_dim 576: nine
+  // channel wavefronts, ten units), so that no wavefront's chain in an iteration is much longer than values + one unit.
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), NWS = (int)blockDim.x >> 6, NW = D ? D / 64 : ly.d >> 6;
   const bool helper = wave == NW;
   const int n = lane & 15, kb = lane >> 4;
@@ -215,45 +205,32 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
   // on the block - which page of the pair, the offset inside the page, the offset inside the slot - is worked out once.
   const int kbytes = L.off_vdata, vbytes = L.page_bytes - L.off_vdata;
   const int PK = (kbytes + 1023) >> 10, PV = (vbytes + 1023) >> 10;
-  constexpr int WD_MAX_OPS = 4;                 // per kind (the plan on the host keeps to it)
-  struct Req { int blk, slot, n; uint32_t src_off[WD_MAX_OPS]; int lds_off[WD_MAX_OPS]; int pg[WD_MAX_OPS]; };
-  auto req_init = [&](Req& r, int pieces, int slot_bytes, int part_off, int part_bytes) {
-    r.blk = blk_begin;
-    r.slot = 0;
-    // pieces wave, wave + NW, ... for the channel wavefronts; none for the helper, whose chain (score unit, softmax) is
-    // the longest of an iteration
-    r.n = wave < NW && wave < 2 * pieces ? (2 * pieces - wave + NW - 1) / NW : 0;
-#pragma unroll
-    for (int k = 0; k < WD_MAX_OPS; ++k) {
-      const int piece = min(wave + k * NW, 2 * pieces - 1);
-      const int pg = piece >= pieces ? 1 : 0, pc = piece - pg * pieces;
-      r.pg[k] = pg;
-      const int at = min(pc * 1024, part_bytes - 1024);     // (the last piece overlaps the one before it: a slot is as long as its part)
-      r.src_off[k] = (uint32_t)(part_off + at + lane * 16);
-      r.lds_off[k] = pg * slot_bytes + at;
-    }
-  };
-  Req rq_k, rq_v;
-  req_init(rq_k, PK, kslot, 0, kbytes);
-  req_init(rq_v, PV, vslot, kbytes, vbytes);
+  // One wavefront - the last of the workgroup, a helper - issues every request (the channel wavefronts' chains are the
+  // longest of an iteration; a request costs a wavefront a third of a microsecond of its time whoever issues it).
+  const bool requester = wave == NWS - 1;
+  struct Req { int blk, slot; };
+  Req rq_k{blk_begin, 0}, rq_v{blk_begin, 0};
   const uint32_t kring_lds = (uint32_t)(uintptr_t)kring, vring_lds = (uint32_t)(uintptr_t)vring;
-  auto issue = [&](Req& r, uint32_t ring_lds, int slot_bytes) __attribute__((always_inline)) {
-    const uint32_t pid0 = (uint32_t)page_entry(2 * r.blk) & 0x7fffffffu, pid1 = (uint32_t)page_entry(2 * r.blk + 1) & 0x7fffffffu;
-    const uint8_t* base0 = pool_h + (uint64_t)pid0 * page_stride32;
-    const uint8_t* base1 = pool_h + (uint64_t)pid1 * page_stride32;
-    const uint32_t slot_lds = ring_lds + (uint32_t)(r.slot * 2 * slot_bytes);
-#pragma unroll
-    for (int k = 0; k < WD_MAX_OPS; ++k)
-      if (k < r.n)
-        dma16<0>((r.pg[k] ? base1 : base0) + r.src_off[k], (uint32_t)__builtin_amdgcn_readfirstlane((int)(slot_lds + (uint32_t)r.lds_off[k])));
+  auto issue = [&](Req& r, uint32_t ring_lds, int slot_bytes, int pieces, int part_off, int part_bytes) __attribute__((always_inline)) {
+    if (requester) {
+      const uint32_t slot_lds = ring_lds + (uint32_t)(r.slot * 2 * slot_bytes);
+      for (int pg = 0; pg < 2; ++pg) {
+        const uint32_t pid = (uint32_t)page_entry(2 * r.blk + pg) & 0x7fffffffu;
+        const uint8_t* base = pool_h + (uint64_t)pid * page_stride32 + part_off + lane * 16;
+        for (int pc = 0; pc < pieces; ++pc) {
+          const int at = min(pc * 1024, part_bytes - 1024);     // (the last piece overlaps the one before it: a slot is as long as its part)
+          dma16<0>(base + at, (uint32_t)__builtin_amdgcn_readfirstlane((int)(slot_lds + (uint32_t)(pg * slot_bytes + at))));
+        }
+      }
+    }
     if (r.blk < blk_end - 1) {
       ++r.blk;
       r.slot = r.slot + 1 == nring ? 0 : r.slot + 1;
     }
   };
-  auto issue_keys = [&]() __attribute__((always_inline)) { issue(rq_k, kring_lds, kslot); };
-  auto issue_vals = [&]() __attribute__((always_inline)) { issue(rq_v, vring_lds, vslot); };
-  const int OPS_K = rq_k.n, OPS_V = rq_v.n;     // this wavefront's requests per block
+  auto issue_keys = [&]() __attribute__((always_inline)) { issue(rq_k, kring_lds, kslot, PK, 0, kbytes); };
+  auto issue_vals = [&]() __attribute__((always_inline)) { issue(rq_v, vring_lds, vslot, PV, kbytes, vbytes); };
+  const int OPS_K = requester ? 2 * PK : 0, OPS_V = requester ? 2 * PV : 0;     // this wavefront's requests per block
   // the keys of the first blocks are on their way while the operands are prepared
   WD_P(1);
   for (int i = 0; i < nring - 1; ++i) issue_keys();
@@ -668,7 +645,7 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
   // t + nring - 1 into the slots the blocks t + 1 and t - 1 had, so at its top the requests of iteration t - nring + 1
   // (keys t + 2, values t) have to have landed and those of the nring - 2 iterations after it may be outstanding.
   int ks = 0, vs = 0;                           // ring slots of the keys of block t + 2 and the values of block t
-  const int issue_at = wave >= NW ? 2 : wave % 3;
+  const int issue_at = 0;
 #ifdef WD_PROF
   unsigned long long wd_t[8] = {0, 0, 0, 0, 0, 0, 0, 0}, wd_last = wall_clock64();
 #endif
@@ -797,10 +774,11 @@ int launch_decode_wide(const float* q_rot, const float* q_sk, int B, int Hq, int
   int nring, kslot, vslot;
   size_t smem;
   wide_plan(ly, L, nring, kslot, vslot, smem);
-  // one wavefront more than channels / 64 (the helper), two when the block's units outnumber the channel wavefronts
-  // and twelve wavefronts are not exceeded
+  // helpers beside the d / 64 channel wavefronts: one for the softmax, one for the page requests and the score units the
+  // channel wavefronts leave over (one for both when that would be more than twelve wavefronts)
   const int nw = ly.d / 64, units = 2 * ((ly.d + 127) / 128);
-  const int helpers = units > nw && nw + 2 <= WD_MAX_WAVES ? 2 : 1;
+  const int helpers = nw + 2 <= WD_MAX_WAVES ? 2 : 1;
+  (void)units;
   const dim3 grid(n_split, Hkv * kv_div, B), block((nw + helpers) * 64);
   hipEvent_t t_start = nullptr, t_stop = nullptr;
   const bool timed = take_time_hook(0, t_start, t_stop);
