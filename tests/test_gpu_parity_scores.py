@@ -251,6 +251,15 @@ def test_decode_wide_heads_on_the_matrix_cores(gpu, d, key_bits, vb, Hq, Hkv, dt
         assert torch.equal(outs[1], outs[2]), "constant and run-time geometry disagree"
 
 
+def test_decode_head_dim_576_at_the_bench_shape_against_the_oracle(gpu):
+    """Two sequences of the 16 x 8192 step bench.py times at head_dim 576 (8 query heads on one KV head, 4-bit keys,
+    4-bit values; 16 splits of 16 blocks, the table registers of a workgroup move on): every sequence against the
+    oracle on the same store."""
+    _progress("decode d=576 at 2 x 8192")
+    worst = _decode_case(gpu, 576, 4, 4, 2, 8, 1, [8192, 8000], None, seed=576, n_split=16)
+    _progress(f"   worst cosine {worst:.7f}")
+
+
 # ------------------------------------------------------------------ block tables are bounded on the device
 @pytest.mark.parametrize("d,key_bits,vb,dtype,T", [(128, 3, 4, torch.bfloat16, 70), (256, 3, 2, torch.bfloat16, 5000),
                                                      (64, 2, 2, torch.float16, 70), (128, 3, 2, torch.float32, 40),

@@ -6,22 +6,24 @@
 // A wide head does not fit the per-wavefront design of the head_dim 64 / 128 / 256 kernel (its query operands and
 // accumulators would need several hundred registers), so here a whole workgroup works on one block of 32 tokens
 // (two pages) at a time:
-//   * one wavefront per 64 channels plus one or two helper wavefronts, one workgroup per compute unit;
-//   * the pages travel HBM -> LDS as they lie in memory (LDS-direct loads, a kilobyte per instruction), the key
-//     part of a page (bit planes, norms) and its value part (codes, scales, zero points) into rings of their
-//     own, two or three blocks deep, so that the next block(s) arrive while the current ones are worked on;
+//   * one wavefront per 64 channels plus two helper wavefronts (one, when twelve wavefronts do not hold two), one
+//     workgroup per compute unit;
+//   * the pages travel HBM -> LDS as they lie in memory (LDS-direct loads, a kilobyte per instruction, all issued by a
+//     helper wavefront): the key part of a page (bit planes, norms) and its value part (codes, scales, zero points)
+//     into rings of their own, two or three blocks deep, so that the next block(s) arrive while the current ones
+//     are worked on;
 //   * the fp6 query operands of v_mfma_scale_f32_16x16x128_f8f6f4 (four terms per value, as the preparation
 //     kernel of the other sizes packs them) are built by the workgroup itself from the fp32 rotated / sketched
 //     queries and stay in LDS;
 //   * scores: the (page, 128-coordinate chunk) pairs of a block are dealt to the wavefronts, the stored bit
 //     planes are the fp4 operand, partial sums meet in LDS;
-//   * softmax: the helper wavefront, online, log2 domain, against a reference that moves lazily;
-//   * values: every wavefront takes the two groups of 32 channels it owns: codes masked in place are bf16
+//   * softmax: a helper wavefront, online, log2 domain, against a reference that moves lazily;
+//   * values: every channel wavefront takes the two groups of 32 channels it owns: codes masked in place are bf16
 //     denormals (B operand), softmax weight x group scale is the A operand (rows 0..7 the heads with the even
 //     group's scales, rows 8..15 with the odd group's), zero points through one more MFMA.
-// The stages are pipelined over the blocks: while the wavefronts accumulate the values of block j they score
-// block j + 1; its softmax follows.  Two workgroup barriers per block.  The step's other launches (rotation,
-// exact tail, merge) are those of the general kernel.
+// The stages are pipelined over the blocks, three a block apart between two barriers: the values of block t, the
+// softmax of block t + 1, the scores of block t + 2.  The step's other launches (rotation, exact tail, merge) are
+// those of the general kernel.
 
 #include "tq_decode_mfma_impl.h"
 
@@ -198,11 +200,9 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
     const int ea = __builtin_amdgcn_readlane(tbl_a, rel & 63), eb = __builtin_amdgcn_readlane(tbl_b, rel & 63);
     return rel < 64 ? ea : eb;
   };
-  // Requests for the key part / value part of the next block of each kind into its ring slot: a kilobyte per
-  // instruction, the pieces dealt to the wavefronts (a wavefront counts its own requests in the waits below, so the
-  // numbers need not be equal).  Blocks are requested in order, so the block and its slot are running counters;
-  // behind the last block of the range the requests repeat it (into the slot it already has).  What does not depend
-  // on the block - which page of the pair, the offset inside the page, the offset inside the slot - is worked out once.
+  // Requests for the key part / value part of the next block of each kind into its ring slot, a kilobyte per
+  // instruction.  Blocks are requested in order, so the block and its slot are running counters (every wavefront keeps
+  // them); behind the last block of the range the requests repeat it (into the slot it already has).
   const int kbytes = L.off_vdata, vbytes = L.page_bytes - L.off_vdata;
   const int PK = (kbytes + 1023) >> 10, PV = (vbytes + 1023) >> 10;
   // One wavefront - the last of the workgroup, a helper - issues every request (the channel wavefronts' chains are the
@@ -645,7 +645,6 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
   // t + nring - 1 into the slots the blocks t + 1 and t - 1 had, so at its top the requests of iteration t - nring + 1
   // (keys t + 2, values t) have to have landed and those of the nring - 2 iterations after it may be outstanding.
   int ks = 0, vs = 0;                           // ring slots of the keys of block t + 2 and the values of block t
-  const int issue_at = 0;
 #ifdef WD_PROF
   unsigned long long wd_t[8] = {0, 0, 0, 0, 0, 0, 0, 0}, wd_last = wall_clock64();
 #endif
@@ -662,24 +661,17 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
       tbl_b = load_tbl(pbase + 64);
       asm volatile("" : "+v"(tbl_b));           // (the wait for this load: here, once in 32 blocks)
     }
-    // (the requests of a compute unit's wavefronts all pass through its one address unit: a third of the wavefronts
-    // issue theirs here, a third between the stages, a third behind them)
-    auto requests = [&]() __attribute__((always_inline)) {
-      issue_keys();
-      if (t >= blk_begin - nring + 1) issue_vals();
-    };
-    if (issue_at == 0) requests();
+    issue_keys();
+    if (t >= blk_begin - nring + 1) issue_vals();
     WD_T(2);
     if (t >= blk_begin) {
       if (wave < NW) values(t, vs, t & 1);
       vs = vs + 1 == nring ? 0 : vs + 1;
     }
     WD_T(3);
-    if (issue_at == 1) requests();
     if (t + 2 < blk_end) score_units(ks, t & 1);
     ks = ks + 1 == nring ? 0 : ks + 1;
     WD_T(4);
-    if (issue_at == 2) requests();
     if (helper && t + 1 >= blk_begin && t + 1 < blk_end) softmax(t + 1, (t + 1) & 1);
     WD_T(5);
   }
