@@ -234,21 +234,29 @@ def test_decode_wide_heads_on_the_matrix_cores(gpu, d, key_bits, vb, Hq, Hkv, dt
     pool, _ = _make_pool(gpu, d, key_bits, vb, Hkv, 4, dtype)
     assert pool.page_kernel() == 2, "the shape has no wide-head kernel"
     outs = {}
+    # as shipped (operands packed by the rotation launch; head_dim 512 / 576: the instantiations with constant page
+    # geometry); operands packed by every page-kernel workgroup; the instantiation that takes the geometry at run time
+    # (what the other head sizes run); the general kernel
+    variants = [("shipped", 1, 1), ("packed in the page kernel", 1, 0)]
+    if d in (512, 576):
+        variants.append(("geometry at run time", 2, 1))
+    variants.append(("general kernel", 0, 1))
     try:
-        # 1: as shipped (head_dim 512 / 576: the instantiations with constant page geometry), 2: the instantiation
-        # that takes the geometry at run time (what the other head sizes run), 0: the general kernel
-        for mode in (1, 2, 0) if d in (512, 576) else (1, 0):
-            _set_option("wide_heads", mode)
-            _progress(f"decode d={d} kb={key_bits} vb={vb} Hq={Hq} Hkv={Hkv} {dtype} n_split={n_split} wide_heads={mode}")
-            outs[mode] = _decode_case(gpu, d, key_bits, vb, len(lens), Hq, Hkv, lens, recent, seed=700 + d + vb,
+        for name, wide, pre in variants:
+            _set_option("wide_heads", wide)
+            _set_option("wide_prepack", pre)
+            _progress(f"decode d={d} kb={key_bits} vb={vb} Hq={Hq} Hkv={Hkv} {dtype} n_split={n_split}: {name}")
+            outs[name] = _decode_case(gpu, d, key_bits, vb, len(lens), Hq, Hkv, lens, recent, seed=700 + d + vb,
                                       n_split=n_split, dtype=dtype, return_out=True)
     finally:
         _set_option("wide_heads", 1)
-    c = cosine(outs[1], outs[0])
-    _progress(f"   wide-head kernel against the general kernel: cosine {c:.7f}")
-    assert c >= COS_GATE
-    if 2 in outs:
-        assert torch.equal(outs[1], outs[2]), "constant and run-time geometry disagree"
+        _set_option("wide_prepack", 1)
+    for name in ("packed in the page kernel", "general kernel"):
+        c = cosine(outs["shipped"], outs[name])
+        _progress(f"   shipped against {name}: cosine {c:.7f}")
+        assert c >= COS_GATE
+    if "geometry at run time" in outs:
+        assert torch.equal(outs["shipped"], outs["geometry at run time"]), "constant and run-time geometry disagree"
 
 
 def test_decode_head_dim_576_at_the_bench_shape_against_the_oracle(gpu):

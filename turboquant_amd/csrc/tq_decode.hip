@@ -940,7 +940,7 @@ using namespace tq;
 namespace tq {
 int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* layer, float* q_rot, float* q_sk,
                         float* q_stat, uint32_t* qa_pack, int G, float sm_scale, hipStream_t st, bool q_rot_unused,
-                        unsigned long long* arrivals, const PagePrefetch* prefetch, int g_tot);
+                        unsigned long long* arrivals, const PagePrefetch* prefetch, int g_tot, const WidePack* wide);
 bool prep_on_matrix_cores(const void* q, int dtype, int64_t rows, const tq_layer* layer, int G, int g_tot);
 }  // namespace tq
 
@@ -965,6 +965,7 @@ std::atomic<int> opt_sequence_walkers{-1};
 std::atomic<int> opt_prep_words{-1};
 std::atomic<int> opt_append_small{-1};
 std::atomic<int> opt_wide_heads{1};
+std::atomic<int> opt_wide_prepack{1};
 }  // namespace tq
 
 extern "C" int tq_set_option(const char* name, int64_t value) {
@@ -987,6 +988,7 @@ extern "C" int tq_set_option(const char* name, int64_t value) {
   }
   if (!std::strcmp(name, "tail_chunks")) { opt_tail_chunks.store(value != 0); return TQ_OK; }
   if (!std::strcmp(name, "merge_row_groups")) { opt_merge_row_groups.store(value != 0); return TQ_OK; }
+  if (!std::strcmp(name, "wide_prepack")) { opt_wide_prepack.store(value != 0); return TQ_OK; }
   if (!std::strcmp(name, "wide_heads")) {
     if (value < 0 || value > 2) return TQ_EINVAL;
     opt_wide_heads.store((int)value);
@@ -1121,6 +1123,18 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   float* q_stat = q_sk + (size_t)B * Hq * d;
   unsigned long long* arrivals = (unsigned long long*)(q_stat + (size_t)4 * B * Hq);    // 8-byte aligned: every term above is even
   uint32_t* qa_pack = (uint32_t*)(arrivals + counter_words(B, Hq));
+  // Head sizes of the wide-head page kernel: the rotation launch also packs the kernel's query operands (one copy per
+  // group of heads, instead of one per page-kernel workgroup) and writes the row statistics.  All stages of a step
+  // decide alike, from the layer, the layout and the options.
+  WidePack wide_pre;
+  if (!mfma_shape && kv_div && decode_wide_has_kernel(*layer, *layout) && layer->Pi_colsum && layer->S_colsum &&
+      opt_wide_prepack.load(std::memory_order_relaxed) != 0 && decode_wide_term_planes(*layer) > 0 &&
+      (size_t)B * Hkv * kv_div * decode_wide_term_planes(*layer) * 2 * wide_qa_stride(d) + 4 <= decode_mfma_pack_words(B, Hq, d)) {
+    wide_pre.qa = (uint32_t*)(((uintptr_t)qa_pack + 15) & ~(uintptr_t)15);      // (16-byte pieces are fetched and stored)
+    wide_pre.q_stat = q_stat;
+    wide_pre.Hq = Hq; wide_pre.Hkv = Hkv; wide_pre.kv_div = kv_div; wide_pre.ntp = decode_wide_term_planes(*layer);
+    wide_pre.sm_scale = sm_scale;
+  }
 
   if (tail && ts.paged && !words) return TQ_EUNSUPPORTED;       // a paged exact cache has to be word-aligned
   TailArgs ta;
@@ -1229,7 +1243,7 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
     } else {
       int rc = launch_rotate_query(q, dtype, (int64_t)B * Hq, layer, q_rot, q_sk, q_stat,
                                    mfma_shape ? qa_pack : nullptr, mfma_shape ? Gq : G, sm_scale, st, mfma_shape,
-                                   fm.counters, &pf, mfma_shape ? g_tot : 0);
+                                   fm.counters, &pf, mfma_shape ? g_tot : 0, wide_pre.qa ? &wide_pre : nullptr);
       if (rc) return rc;
     }
   }
@@ -1287,7 +1301,7 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   // head sizes above 256: the matrix-core kernel that works on a block per workgroup
   if ((stages & 2) && mf == TQ_EUNSUPPORTED) {
     mf = launch_decode_wide(q_rot, q_sk, B, Hq, Hkv, pool, block_table, bt_stride, seq_lens, sm_scale, *layer, *layout,
-                            parts, n_parts, n_split, len_sub, max_pages, pool_pages, st);
+                            parts, n_parts, n_split, len_sub, max_pages, pool_pages, wide_pre, st);
     if (mf > 0) return mf;
   }
   if ((stages & 2) && mf == TQ_EUNSUPPORTED) {      // no matrix-core kernel for this shape: general kernel
@@ -1417,6 +1431,8 @@ size_t decode_scratch_need(int B, int Hq, int Hkv, int n_split, const tq_layer& 
     for (int t = 0; t < ly.n_terms; ++t)
       if (__builtin_popcount(ly.term_mask[t]) > 1) ++planes;
     words = (size_t)B * Hkv * kv_div * planes * (d >= 128 ? d / 128 : 1) * 2 * 64 * 8;
+  } else if (kv_div && d > 256 && decode_wide_term_planes(ly) > 0) {
+    words = (size_t)B * Hkv * kv_div * decode_wide_term_planes(ly) * 2 * wide_qa_stride(d) + 4;
   }
   return (floats + words) * 4;
 }

@@ -114,6 +114,20 @@ int launch_decode_mfma(uint32_t* qa_pack, float* q_stat, int B, int Hq, int Hkv,
                        int max_pages, int num_pages, const FusedMerge& fm, bool wide_wg,
                        hipStream_t st);
 
+// Packed query operands of the wide-head kernel (head sizes 320 .. 704), written by the rotation launch of the step
+// and read by every page-kernel workgroup of the group: per group of at most 8 query heads of a KV head
+// [term plane][row set][chunk] operands of WD_QA_OP dwords ([64 lanes][4] then [64 lanes][2]); a last chunk of 64
+// coordinates takes half an operand ([32][4] then [32][2]).  q_stat per query row: {E_index, E_sign, constant part of the
+// index score, of the sign score}.
+constexpr int WD_QA_OP = 64 * 6;
+__host__ __device__ constexpr int wide_qa_stride(int d) { return ((d + 127) / 128) * WD_QA_OP - (d % 128 ? WD_QA_OP / 2 : 0); }   // dwords per (plane, row set)
+struct WidePack {
+  uint32_t* qa = nullptr;            // nullptr: the page kernel packs its operands itself
+  float* q_stat = nullptr;
+  int Hq = 0, Hkv = 0, kv_div = 1, ntp = 0;
+  float sm_scale = 0.0f;
+};
+
 // The matrix-core kernel for head sizes above 256 (tq_decode_wide.hip; a workgroup per block of 32 tokens): reads the
 // fp32 rotated / sketched queries the general kernel reads and writes the same partials.  TQ_EUNSUPPORTED when the
 // shape has no such kernel (nothing was launched).
@@ -121,7 +135,9 @@ bool decode_wide_has_kernel(const tq_layer& ly, const tq_page_layout& L);
 int launch_decode_wide(const float* q_rot, const float* q_sk, int B, int Hq, int Hkv, const uint8_t* pool,
                        const int32_t* block_table, int bt_stride, const int32_t* seq_lens, float sm_scale,
                        const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts, int n_split, int len_sub,
-                       int max_pages, int num_pages, hipStream_t st);
+                       int max_pages, int num_pages, const WidePack& pre, hipStream_t st);
+// term planes of a layer on that kernel (0: its codebook has other Walsh terms than the kernel takes)
+int decode_wide_term_planes(const tq_layer& ly);
 
 // Whether a step of this shape runs workgroups of eight wavefronts: the caller then passes HALF its split count
 // (and wide_wg = true) to launch_decode_mfma and uses that count for everything that follows.

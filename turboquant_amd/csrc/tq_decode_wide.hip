@@ -30,7 +30,6 @@
 namespace tq {
 
 constexpr int WD_BLK = 32;                 // tokens per iteration (two pages)
-constexpr int WD_QA_OP = 64 * 6;           // dwords of one packed operand: [64 lanes][4] then [64 lanes][2]
 constexpr int WD_MAX_WAVES = 12;           // head_dim 768
 constexpr int WD_MAX_CHUNKS = 6;           // 128-coordinate chunks of head_dim 768
 constexpr int WD_SMALL_FLOATS = 2 * (256 + 256 + 8 + 8 + 64) + 32 + 16 + 16 + WD_MAX_WAVES * 32;   // two of (s_p, s_pv, s_alpha, s_flag, s_meta), s_stat, s_mult, s_coef, s_z
@@ -103,7 +102,8 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
                    const uint8_t* __restrict__ pool, const int32_t* __restrict__ block_table, int bt_stride,
                    const int32_t* __restrict__ seq_lens, float sm_scale, tq_layer ly, tq_page_layout L_rt,
                    float* __restrict__ parts, int n_parts, int n_split, int len_sub, int max_pages, int num_pages,
-                   int nring_rt, int kslot_rt, int vslot_rt) {
+                   int nring_rt, int kslot_rt, int vslot_rt, const uint32_t* __restrict__ qa_pre,
+                   const float* __restrict__ q_stat_pre) {
   constexpr int NX = MB == 3 ? 1 : (MB == 4 ? 4 : 0), NTP = MB + NX + 1;
   constexpr bool f16p = F16P;                   // fp16 pages: scales and zero points are fp16 numbers
   const int d = D ? D : ly.d, W = d >> 5, WPLT = (d + 127) >> 7;
@@ -236,9 +236,7 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
   for (int i = 0; i < nring - 1; ++i) issue_keys();
   WD_P(2);
 
-  // ---------------------------------------------------------------- query operands (as the preparation kernel packs them)
-  float cmax = 0.0f;
-  for (int t = 0; t < ly.n_terms; ++t) cmax = fmaxf(cmax, fabsf(ly.term_coef[t]));
+  // ---------------------------------------------------------------- query operands
   int xpl = 0;                                  // four bits per multi-bit term: the stored planes it XORs
   {
     int seen = 0;
@@ -252,6 +250,39 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
     }
     xpl = __builtin_amdgcn_readfirstlane(xpl);
   }
+  if (qa_pre != nullptr) {
+    // Packed by the step's rotation launch, one copy per group of heads: fetched as they lie in memory, a kilobyte per
+    // instruction, every wavefront its share; the statistics of the group's rows with them.
+    const int total = NTP * 2 * QA_STRIDE * 4;  // bytes
+    const uint8_t* src = (const uint8_t*)(qa_pre + ((int64_t)b * gridDim.y + blockIdx.y) * (NTP * 2 * QA_STRIDE));
+    const uint32_t qa_at = (uint32_t)(uintptr_t)qa_lds;
+    for (int pc = wave; pc < (total + 1023) >> 10; pc += NWS) {
+      const int at = min(pc * 1024, total - 1024);
+      dma16<0>(src + at + lane * 16, (uint32_t)__builtin_amdgcn_readfirstlane((int)(qa_at + (uint32_t)at)));
+    }
+    if (tid < 32) s_stat[tid] = (tid >> 2) < G ? q_stat_pre[((int64_t)b * Hq + qbase + (tid >> 2)) * 4 + (tid & 3)] : 0.0f;
+    stage_wait<0>();
+    __syncthreads();
+    WD_P(3);
+    // rows of the heads the group does not have: zero (nobody wrote them)
+    for (int item = tid; item < NTP * (8 - G) * W; item += blockDim.x) {
+      const int g = G + item % (8 - G), rest = item / (8 - G), j = rest % W, tp = rest / W;
+      uint32_t* op0 = qa_lds + (tp * 2) * QA_STRIDE + (j >> 2) * WD_QA_OP;
+      const int slot0 = 2 * g + 16 * (j & 3);
+      const int hi_at = half_chunk && (j >> 2) == WPLT - 1 ? 32 * 4 : 64 * 4;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        uint32_t* op = op0 + (t >> 1) * QA_STRIDE;
+        *(u32x4*)(op + (slot0 + (t & 1)) * 4) = u32x4{0, 0, 0, 0};
+        *(uint2*)(op + hi_at + (slot0 + (t & 1)) * 2) = make_uint2(0u, 0u);
+      }
+    }
+    __syncthreads();
+    WD_P(4);
+  } else {
+  // packed here, as the preparation kernel of the other head sizes packs them
+  float cmax = 0.0f;
+  for (int t = 0; t < ly.n_terms; ++t) cmax = fmaxf(cmax, fabsf(ly.term_coef[t]));
   if (tid < 16) {
     float coef = 1.0f;                          // the sign plane
     if (tid < MB) {
@@ -376,6 +407,7 @@ decode_wide_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_
   }
   __syncthreads();
   WD_P(4);
+  }
   // E8M0 block-scale codes of this lane's operand row (head n / 2; row 2g + t holds term t of row set 0 and term
   // t + 2 of row set 1): index planes row set 0, 1, sign plane row set 0, 1.  4 v / 2^E is stored, so term t
   // carries 2^(E - 2 - 5t); the fp4 bit value 0.5 carries 2^1.
@@ -755,11 +787,20 @@ bool decode_wide_has_kernel(const tq_layer& ly, const tq_page_layout& L) {
   return wide_plan(ly, L, nring, kslot, vslot, smem);
 }
 
+int decode_wide_term_planes(const tq_layer& ly) {
+  const int mb = ly.mse_bits;
+  int nx = 0;
+  for (int t = 0; t < ly.n_terms; ++t)
+    if (__builtin_popcount(ly.term_mask[t]) > 1) ++nx;
+  if (mb < 1 || mb > 4 || ly.n_terms <= 0 || nx != (mb == 3 ? 1 : (mb == 4 ? 4 : 0))) return 0;
+  return mb + nx + 1;
+}
+
 // Returns TQ_EUNSUPPORTED when the shape has no wide-head kernel (nothing was launched).
 int launch_decode_wide(const float* q_rot, const float* q_sk, int B, int Hq, int Hkv, const uint8_t* pool,
                        const int32_t* block_table, int bt_stride, const int32_t* seq_lens, float sm_scale,
                        const tq_layer& ly, const tq_page_layout& L, float* parts, int n_parts, int n_split, int len_sub,
-                       int max_pages, int num_pages, hipStream_t st) {
+                       int max_pages, int num_pages, const WidePack& pre, hipStream_t st) {
   if (!decode_wide_has_kernel(ly, L)) return TQ_EUNSUPPORTED;
   const int g_tot = Hq / Hkv, kv_div = (g_tot + 7) / 8;
   if (g_tot < 1 || g_tot > 16 || (int64_t)Hkv * kv_div > 65535) return TQ_EUNSUPPORTED;
@@ -782,11 +823,11 @@ int launch_decode_wide(const float* q_rot, const float* q_sk, int B, int Hq, int
     if (timed)                                                                                                        \
       hipExtLaunchKernelGGL(kern, grid, block, smem, st, t_start, t_stop, 0, q_rot, q_sk, Hq, Hkv, kv_div, pool,      \
                             block_table, bt_stride, seq_lens, sm_scale, ly, L, parts, n_parts, n_split, len_sub,      \
-                            max_pages, num_pages, nring, kslot, vslot);                                               \
+                            max_pages, num_pages, nring, kslot, vslot, pre.qa, pre.q_stat);                           \
     else                                                                                                              \
       kern<<<grid, block, smem, st>>>(q_rot, q_sk, Hq, Hkv, kv_div, pool, block_table, bt_stride, seq_lens, sm_scale, \
                                       ly, L, parts, n_parts, n_split, len_sub, max_pages, num_pages, nring, kslot,    \
-                                      vslot);                                                                         \
+                                      vslot, pre.qa, pre.q_stat);                                                     \
   }
 #define TQ_LAUNCH_WIDE_MB(D, VB)                        \
   {                                                     \

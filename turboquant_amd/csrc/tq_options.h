@@ -17,6 +17,7 @@ extern std::atomic<int> opt_prep_mfma;           // decode: bf16 queries at head
 extern std::atomic<int> opt_sequence_walkers;     // decode, one split, head_dim 64 / 128: wavefronts that walk a (sequence, head group): 4, 2, 1, or -1 = as many of those as keep the whole launch resident
 extern std::atomic<int> opt_prep_words;           // decode, matrix-core preparation: a workgroup per tile of query rows, a plane word per wavefront (1), a workgroup per (tile, word) (0), -1: the first when the second would not be resident at once
 extern std::atomic<int> opt_append_small;         // key quantiser into pages: up to this many 16-vector tiles get a workgroup each that computes one tile (0: never, -1: two per compute unit)
+extern std::atomic<int> opt_wide_prepack;          // decode, wide-head kernel: the rotation launch packs the query operands (0: every page-kernel workgroup its own)
 extern std::atomic<int> opt_wide_heads;             // decode: head sizes above 256 run the workgroup-per-block matrix-core kernel (0: the general kernel)
 extern std::atomic<int> opt_merge_in_kernel;    // decode: few context splits are merged by the last workgroup of the page kernel
 }  // namespace tq

@@ -22,10 +22,16 @@ constexpr int ROT_COLS = 32, ROT_SLICES = 8;
 // HALVES (1 or 2): a workgroup of HALVES x 256 threads takes HALVES x 8 rows; the halves run the same loads a
 // moment apart, so the second finds the matrix lines in the compute unit's cache: with many rows half the traffic
 // from L2 for the same work per thread (128 rows at head_dim 576: 42 -> 21 MB).
-template <int BATCH, int HALVES>
+// PACK (a decode step at a head size of the wide-head page kernel): the workgroup also turns its 32 columns - one
+// plane word - of every row into the kernel's fp6 query operands (four terms per value, as prep_query_body packs them
+// for the other head sizes) and writes them where the page-kernel workgroups of the row's head group fetch them,
+// and the workgroups of the first word write the rows' statistics.  The operands are normalised by bounds every
+// workgroup can compute from the raw query: |q_rot_j| <= ||q|| (Pi is orthogonal) and |q_sk_j| <= ||q|| max_j ||S_j||;
+// the sums over all coordinates the scores need are q . colsum(Pi), q . colsum(S).
+template <int BATCH, int HALVES, bool PACK>
 __global__ void __launch_bounds__(ROT_COLS * ROT_SLICES * HALVES)
 rotate_query_kernel(const void* __restrict__ q, int dtype, int64_t rows, int R, tq_layer ly, float* __restrict__ q_rot,
-                    float* __restrict__ q_sk) {
+                    float* __restrict__ q_sk, WidePack wp) {
   extern __shared__ __align__(16) float sm[];
   constexpr int T1 = ROT_COLS * ROT_SLICES;
   const int d = ly.d, tid = threadIdx.x, half = tid / T1, t1 = tid - half * T1, jl = t1 % ROT_COLS, sl = t1 / ROT_COLS;
@@ -37,6 +43,68 @@ rotate_query_kernel(const void* __restrict__ q, int dtype, int64_t rows, int R, 
   const int nr = (int)((rows - row0) < R ? (rows - row0) : R);
   for (int o = tid; o < R * d; o += blockDim.x) sq[o] = o < nr * d ? load_as_f32(q, row0 * d + o, dtype) : 0.0f;
   __syncthreads();
+  float* s_rot = pb + ROT_SLICES * R * ROT_COLS;   // PACK: [R][ROT_COLS] this word's rotated values, then the sketched ones
+  float* s_sk = s_rot + R * ROT_COLS;
+  float* s_rs = s_sk + R * ROT_COLS;               // PACK: [R][2] multipliers of q_rot / q_sk
+  float* s_cf = s_rs + 2 * R;                      // PACK: [16] coefficient of each term plane
+  if constexpr (PACK) {
+    // row statistics, a wavefront per row (every workgroup of the rows computes the same ones)
+    const int lane = tid & 63, wv = tid >> 6, n_wv = (int)blockDim.x >> 6;
+    float cmax = 0.0f;
+    for (int t = 0; t < ly.n_terms; ++t) cmax = fmaxf(cmax, fabsf(ly.term_coef[t]));
+    // (this lane's column sums: requested once, for all rows)
+    constexpr int CS = 12;                         // d <= 768
+    float cs1[CS], cs2[CS];
+#pragma unroll
+    for (int k = 0; k < CS; ++k) {
+      const int c = min(lane + 64 * k, d - 1);
+      cs1[k] = ly.Pi_colsum[c];
+      cs2[k] = ly.S_colsum[c];
+    }
+    for (int r = wv; r < nr; r += n_wv) {
+      float ss = 0.0f, s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+      for (int k = 0; k < CS; ++k) {
+        const int c = lane + 64 * k;
+        const float x = c < d ? sq[r * d + c] : 0.0f;
+        ss = fmaf(x, x, ss);
+        s1 = fmaf(x, cs1[k], s1);
+        s2 = fmaf(x, cs2[k], s2);
+      }
+      ss = wave_sum_fast(ss); s1 = wave_sum_fast(s1); s2 = wave_sum_fast(s2);
+      if (lane == 0) {
+        const float nq = sqrtf(ss), k = wp.sm_scale * 1.4426950408889634f;
+        // bound < 2^e: e = exponent field - 126, kept within +-100
+        const int e1 = min(max((int)((__float_as_uint(fabsf(k) * nq * cmax) >> 23) & 255u) - 126, -100), 100);
+        const int e2 = min(max((int)((__float_as_uint(2.0f * fabsf(k * ly.qjl_scale) * nq * ly.S_rownorm_max) >> 23) & 255u) - 126, -100), 100);
+        s_rs[2 * r] = k * __uint_as_float((uint32_t)(127 - e1) << 23);
+        s_rs[2 * r + 1] = 2.0f * k * ly.qjl_scale * __uint_as_float((uint32_t)(127 - e2) << 23);
+        if (blockIdx.y == 0) {
+          float* st = wp.q_stat + (row0 + r) * 4;
+          st[0] = (float)e1; st[1] = (float)e2; st[2] = k * ly.term_const * s1; st[3] = -k * ly.qjl_scale * s2;
+        }
+      }
+    }
+    if (tid < 16) {                                // coefficient of term plane tid (as the page kernel orders them)
+      const int mb = ly.mse_bits;
+      float coef = 1.0f;                           // the sign plane
+      if (tid < mb) {
+        coef = 0.0f;
+        for (int t = 0; t < ly.n_terms; ++t)
+          if (ly.term_mask[t] == (1 << (mb - 1 - tid))) coef = ly.term_coef[t];
+      } else if (tid < wp.ntp - 1) {
+        coef = 0.0f;
+        int seen = 0;
+        for (int t = 0; t < ly.n_terms; ++t) {
+          if (__builtin_popcount(ly.term_mask[t]) > 1) {
+            if (seen == tid - mb) coef = ly.term_coef[t];
+            ++seen;
+          }
+        }
+      }
+      s_cf[tid] = coef;
+    }
+  }
   const int per = d / ROT_SLICES, i0 = sl * per;
   const int r0 = half * ROT_MAX_ROWS, RH = min(R - r0, ROT_MAX_ROWS);      // this half's rows: r0 .. r0 + RH - 1
   float a[ROT_MAX_ROWS], b[ROT_MAX_ROWS];
@@ -80,6 +148,71 @@ rotate_query_kernel(const void* __restrict__ q, int dtype, int64_t rows, int R, 
     for (int k = 0; k < ROT_SLICES; ++k) { ra += pa[(k * R + r) * ROT_COLS + c]; rb += pb[(k * R + r) * ROT_COLS + c]; }
     q_rot[(row0 + r) * d + blockIdx.y * ROT_COLS + c] = ra;
     q_sk[(row0 + r) * d + blockIdx.y * ROT_COLS + c] = rb;
+    if constexpr (PACK) {
+      s_rot[o] = ra;
+      s_sk[o] = rb;
+    }
+  }
+  if constexpr (PACK) {
+    __syncthreads();
+    // one lane per (term plane, row): the word's 32 values as four fp6 terms (the packing conversion of gfx950 and its
+    // inverse for the residual), written where lane (row 2 g + term % 2, quarter word % 4) of operand (plane, row set
+    // term / 2, chunk word / 4) of the row's head group reads them
+    typedef float f32x16_t __attribute__((ext_vector_type(16)));
+    typedef float f32x32_t __attribute__((ext_vector_type(32)));
+    typedef uint32_t u32x6_t __attribute__((ext_vector_type(6)));
+    const int ntp = wp.ntp, j = blockIdx.y, W = d >> 5;
+    const int qa_stride = wide_qa_stride(d);
+    const bool half_op = (d & 127) != 0 && (j >> 2) == ((d + 127) >> 7) - 1;
+    const int hi_at = half_op ? 32 * 4 : 64 * 4;
+    (void)W;
+    for (int it = tid; it < ntp * nr; it += blockDim.x) {
+      const int tp = it / nr, r = it - tp * nr;
+      const bool is_sign = tp == ntp - 1;
+      // the row's place: sequence, head, group of at most 8 heads of its KV head, slot in the group
+      const int row = (int)row0 + r;                   // (32-bit arithmetic: the launcher checks the row count)
+      const int bq = row / wp.Hq, head = row - bq * wp.Hq;
+      const int g_tot = wp.Hq / wp.Hkv, kvh = head / g_tot, hh = head - kvh * g_tot;
+      const int g_max = (g_tot + wp.kv_div - 1) / wp.kv_div, grp = hh / g_max, g = hh - grp * g_max;
+      const int64_t group = ((int64_t)bq * wp.Hkv + kvh) * wp.kv_div + grp;
+      const float base = 4.0f * (is_sign ? s_rs[2 * r + 1] : s_cf[tp] * s_rs[2 * r]);
+      const float4* src = (const float4*)((is_sign ? s_sk : s_rot) + r * ROT_COLS);
+      float x[32];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const float4 v4 = src[k];
+        x[4 * k] = v4.x; x[4 * k + 1] = v4.y; x[4 * k + 2] = v4.z; x[4 * k + 3] = v4.w;
+      }
+      f32x16_t va, vb;                      // contraction indices 0, 2, 4, ... and 1, 3, 5, ...
+#pragma unroll
+      for (int kloc = 0; kloc < 32; ++kloc) {
+        const int c = 4 * (kloc & 7) + (kloc >> 3), t4 = kloc >> 3;      // coordinate within the word
+        // (the page kernel takes three of a nibble's four bits in place, as the fp4 numbers 0.5, 1, 2)
+        const float v = x[c] * (base * (t4 == 1 ? 0.5f : (t4 == 2 ? 0.25f : 1.0f)));
+        if (kloc & 1) vb[kloc >> 1] = v;
+        else va[kloc >> 1] = v;
+      }
+      uint32_t* op0 = wp.qa + group * (int64_t)(ntp * 2 * qa_stride) + (tp * 2) * qa_stride + (j >> 2) * WD_QA_OP;
+      const int slot0 = 2 * g + 16 * (j & 3);
+      const float one = 1.0f;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        u32x6_t code;
+        asm volatile("v_cvt_scalef32_2xpk16_fp6_f32 %0, %1, %2, %3" : "=&v"(code) : "v"(va), "v"(vb), "v"(one));
+        uint32_t* op = op0 + (t >> 1) * qa_stride;
+        *(uint4*)(op + (slot0 + (t & 1)) * 4) = make_uint4(code[0], code[1], code[2], code[3]);
+        *(uint2*)(op + hi_at + (slot0 + (t & 1)) * 2) = make_uint2(code[4], code[5]);
+        if (t < 3) {
+          f32x32_t rr;
+          asm volatile("v_cvt_scalef32_pk32_f32_fp6 %0, %1, %2" : "=&v"(rr) : "v"(code), "v"(one));
+#pragma unroll
+          for (int k = 0; k < 16; ++k) {
+            va[k] = (va[k] - rr[2 * k]) * 32.0f;
+            vb[k] = (vb[k] - rr[2 * k + 1]) * 32.0f;
+          }
+        }
+      }
+    }
   }
 }
 
@@ -410,7 +543,7 @@ bool prep_on_matrix_cores(const void* q, int dtype, int64_t rows, const tq_layer
 // cores), not the fp32 rotated / sketched queries
 int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* layer, float* q_rot, float* q_sk,
                         float* q_stat, uint32_t* qa_pack, int G, float sm_scale, hipStream_t st, bool q_rot_unused,
-                        unsigned long long* arrivals, const PagePrefetch* prefetch, int g_tot) {
+                        unsigned long long* arrivals, const PagePrefetch* prefetch, int g_tot, const WidePack* wide) {
   const int d = layer->d;
   if (qa_pack) {       // operands of the matrix-core decode kernel wanted
     // g_tot: query heads per KV head when its groups of G are unequal (0: the rows are whole groups of G)
@@ -494,17 +627,20 @@ int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* 
   const int max_r = wide_rows ? 16 : ROT_MAX_ROWS;
   const int R = (int)(rows < max_r ? rows : max_r);
   if (R < 1 || d % ROT_COLS || d % (8 * ROT_SLICES)) return TQ_EUNSUPPORTED;
-  size_t smem = (size_t)(R * d + 2 * ROT_SLICES * R * ROT_COLS) * sizeof(float);
+  const bool pack = wide != nullptr && wide->qa != nullptr && wide->q_stat != nullptr && layer->Pi_colsum && layer->S_colsum &&
+                    wide->ntp >= 2 && wide->ntp <= 9 && rows % wide->Hq == 0 && rows < (1 << 30) && d <= 768;
+  size_t smem = (size_t)(R * d + 2 * ROT_SLICES * R * ROT_COLS + (pack ? 2 * R * ROT_COLS + 2 * R + 16 : 0)) * sizeof(float);
+  const WidePack wp = pack ? *wide : WidePack{};
   const dim3 rgrid((unsigned)((rows + R - 1) / R), d / ROT_COLS), rblock(ROT_COLS * ROT_SLICES * (wide_rows ? 2 : 1));
   const int per = d / ROT_SLICES;
 #define TQ_ROTATE(BATCH, MAXR)                                                                                         \
   {                                                                                                                    \
-    auto kern = rotate_query_kernel<BATCH, MAXR>;                                                                      \
+    auto kern = pack ? rotate_query_kernel<BATCH, MAXR, true> : rotate_query_kernel<BATCH, MAXR, false>;             \
     if (smem > 48 * 1024) {                                                                                            \
       hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);    \
       if (e != hipSuccess) return (int)e;                                                                              \
     }                                                                                                                  \
-    kern<<<rgrid, rblock, smem, st>>>(q, dtype, rows, R, *layer, q_rot, q_sk);                                         \
+    kern<<<rgrid, rblock, smem, st>>>(q, dtype, rows, R, *layer, q_rot, q_sk, wp);                                     \
   }
 #define TQ_ROTATE_R(BATCH)                 \
   {                                        \
@@ -529,7 +665,7 @@ extern "C" int tq_rotate_query(const void* q, int dtype, int64_t rows, const tq_
   if (!q || !q_rot || !q_sk) return TQ_ENULL;
   if (rows < 0 || dtype < TQ_F32 || dtype > TQ_BF16) return TQ_EINVAL;
   if (rows == 0) return TQ_OK;
-  return launch_rotate_query(q, dtype, rows, layer, q_rot, q_sk, nullptr, nullptr, 1, 0.0f, (hipStream_t)stream, false, nullptr, nullptr, 0);
+  return launch_rotate_query(q, dtype, rows, layer, q_rot, q_sk, nullptr, nullptr, 1, 0.0f, (hipStream_t)stream, false, nullptr, nullptr, 0, nullptr);
 }
 
 extern "C" int tq_score(const void* q, int dtype, int64_t batch, int64_t n_q, const uint8_t* idx, const uint8_t* signs,
