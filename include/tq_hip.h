@@ -366,6 +366,9 @@ void tq_time_next_key_kernel(void *start_event, void *stop_event);
  *                      that works on a block of 32 tokens per workgroup, 512 and 576 in instantiations with constant page
  *                      geometry; 2: every such head size on the instantiation that takes the geometry at run time (same
  *                      result bit for bit); 0: the general vector-ALU kernel (results agree to rounding).
+ *   "wide_prepack"     1 (default): at the head sizes of that kernel the rotation launch of a decode step packs the kernel's
+ *                      query operands once per group of heads; 0: every page-kernel workgroup packs its own (results agree to
+ *                      rounding: the operands are normalised by other bounds).
  *   "append_small"     -1 (default), 0, or a tile count: an append to pages of at most this many 16-vector tiles (-1: two
  *                      per compute unit) gives every tile a workgroup that computes that tile only - the page write of
  *                      a decode step, a token per sequence; 0: always workgroups over groups of tiles.  Same bytes.
