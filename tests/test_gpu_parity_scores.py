@@ -237,24 +237,34 @@ def test_decode_wide_heads_on_the_matrix_cores(gpu, d, key_bits, vb, Hq, Hkv, dt
     # as shipped (operands packed by the rotation launch; head_dim 512 / 576: the instantiations with constant page
     # geometry); operands packed by every page-kernel workgroup; the instantiation that takes the geometry at run time
     # (what the other head sizes run); the general kernel
-    variants = [("shipped", 1, 1), ("packed in the page kernel", 1, 0)]
+    # (bf16 queries are rotated and packed on the matrix cores; "prep_mfma" = 0 leaves that to the vector ALU)
+    variants = [("shipped", 1, 1, 1), ("packed in the page kernel", 1, 0, 1)]
+    if dtype == torch.bfloat16:
+        variants.append(("rotated on the vector ALU", 1, 1, 0))
     if d in (512, 576):
-        variants.append(("geometry at run time", 2, 1))
-    variants.append(("general kernel", 0, 1))
+        variants.append(("geometry at run time", 2, 1, 1))
+    variants.append(("general kernel", 0, 1, 1))
     try:
-        for name, wide, pre in variants:
+        for name, wide, pre, rot in variants:
             _set_option("wide_heads", wide)
             _set_option("wide_prepack", pre)
+            _set_option("prep_mfma", rot)
             _progress(f"decode d={d} kb={key_bits} vb={vb} Hq={Hq} Hkv={Hkv} {dtype} n_split={n_split}: {name}")
             outs[name] = _decode_case(gpu, d, key_bits, vb, len(lens), Hq, Hkv, lens, recent, seed=700 + d + vb,
                                       n_split=n_split, dtype=dtype, return_out=True)
     finally:
         _set_option("wide_heads", 1)
         _set_option("wide_prepack", 1)
-    for name in ("packed in the page kernel", "general kernel"):
+        _set_option("prep_mfma", 1)
+    for name in ("packed in the page kernel", "rotated on the vector ALU", "general kernel"):
+        if name not in outs:
+            continue
         c = cosine(outs["shipped"], outs[name])
         _progress(f"   shipped against {name}: cosine {c:.7f}")
         assert c >= COS_GATE
+    if "rotated on the vector ALU" in outs:      # the same operands to rounding: outputs within a rounding step of the output type
+        a, b = outs["shipped"].float(), outs["rotated on the vector ALU"].float()
+        assert float((a - b).abs().max()) <= 2.0 ** -7 * float(a.abs().max())
     if "geometry at run time" in outs:
         assert torch.equal(outs["shipped"], outs["geometry at run time"]), "constant and run-time geometry disagree"
 

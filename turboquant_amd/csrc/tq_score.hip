@@ -16,6 +16,123 @@ namespace tq {
 // slices meet in LDS.
 constexpr int ROT_COLS = 32, ROT_SLICES = 8;
 
+// coefficient of term plane tp as the wide-head page kernel orders them: the index planes from the highest bit down,
+// the multi-bit Walsh terms, the sign plane
+__device__ __forceinline__ float wide_term_plane_coef(const tq_layer& ly, int ntp, int tp) {
+  const int mb = ly.mse_bits;
+  float coef = 1.0f;                               // the sign plane
+  if (tp < mb) {
+    coef = 0.0f;
+    for (int t = 0; t < ly.n_terms; ++t)
+      if (ly.term_mask[t] == (1 << (mb - 1 - tp))) coef = ly.term_coef[t];
+  } else if (tp < ntp - 1) {
+    coef = 0.0f;
+    int seen = 0;
+    for (int t = 0; t < ly.n_terms; ++t) {
+      if (__builtin_popcount(ly.term_mask[t]) > 1) {
+        if (seen == tp - mb) coef = ly.term_coef[t];
+        ++seen;
+      }
+    }
+  }
+  return coef;
+}
+
+// PACK epilogue of the rotation kernels: plane word j (32 coordinates) of nr query rows from row0 on, as the wide-head
+// page kernel's fp6 operands.  s_rot / s_sk: [row][32] rotated / sketched values of the word; s_rs: [row][2] the
+// rows' multipliers; s_cf: coefficient of each term plane.
+__device__ __forceinline__ void wide_pack_word(const WidePack& wp, int d, int nr, int row0, int j, const float* s_rot,
+                                               const float* s_sk, const float* s_rs, const float* s_cf, int tid,
+                                               int n_threads) {
+  // one lane per (term plane, row): the word's 32 values as four fp6 terms (the packing conversion of gfx950 and its
+  // inverse for the residual), written where lane (row 2 g + term % 2, quarter word % 4) of operand (plane, row set
+  // term / 2, chunk word / 4) of the row's head group reads them
+  typedef float f32x16_t __attribute__((ext_vector_type(16)));
+  typedef float f32x32_t __attribute__((ext_vector_type(32)));
+  typedef uint32_t u32x6_t __attribute__((ext_vector_type(6)));
+  const int ntp = wp.ntp;
+  const int qa_stride = wide_qa_stride(d);
+  const bool half_op = (d & 127) != 0 && (j >> 2) == ((d + 127) >> 7) - 1;
+  const int hi_at = half_op ? 32 * 4 : 64 * 4;
+  for (int it = tid; it < ntp * nr; it += n_threads) {
+    const int tp = it / nr, r = it - tp * nr;
+    const bool is_sign = tp == ntp - 1;
+    // the row's place: sequence, head, group of at most 8 heads of its KV head, slot in the group
+    const int row = row0 + r;                        // (32-bit arithmetic: the launcher checks the row count)
+    const int bq = row / wp.Hq, head = row - bq * wp.Hq;
+    const int g_tot = wp.Hq / wp.Hkv, kvh = head / g_tot, hh = head - kvh * g_tot;
+    const int g_max = (g_tot + wp.kv_div - 1) / wp.kv_div, grp = hh / g_max, g = hh - grp * g_max;
+    const int64_t group = ((int64_t)bq * wp.Hkv + kvh) * wp.kv_div + grp;
+    const float base = 4.0f * (is_sign ? s_rs[2 * r + 1] : s_cf[tp] * s_rs[2 * r]);
+    const float4* src = (const float4*)((is_sign ? s_sk : s_rot) + r * ROT_COLS);
+    float x[32];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const float4 v4 = src[k];
+      x[4 * k] = v4.x; x[4 * k + 1] = v4.y; x[4 * k + 2] = v4.z; x[4 * k + 3] = v4.w;
+    }
+    f32x16_t va, vb;                      // contraction indices 0, 2, 4, ... and 1, 3, 5, ...
+#pragma unroll
+    for (int kloc = 0; kloc < 32; ++kloc) {
+      const int c = 4 * (kloc & 7) + (kloc >> 3), t4 = kloc >> 3;      // coordinate within the word
+      // (the page kernel takes three of a nibble's four bits in place, as the fp4 numbers 0.5, 1, 2)
+      const float v = x[c] * (base * (t4 == 1 ? 0.5f : (t4 == 2 ? 0.25f : 1.0f)));
+      if (kloc & 1) vb[kloc >> 1] = v;
+      else va[kloc >> 1] = v;
+    }
+    uint32_t* op0 = wp.qa + group * (int64_t)(ntp * 2 * qa_stride) + (tp * 2) * qa_stride + (j >> 2) * WD_QA_OP;
+    const int slot0 = 2 * g + 16 * (j & 3);
+    const float one = 1.0f;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      u32x6_t code;
+      asm volatile("v_cvt_scalef32_2xpk16_fp6_f32 %0, %1, %2, %3" : "=&v"(code) : "v"(va), "v"(vb), "v"(one));
+      uint32_t* op = op0 + (t >> 1) * qa_stride;
+      *(uint4*)(op + (slot0 + (t & 1)) * 4) = make_uint4(code[0], code[1], code[2], code[3]);
+      *(uint2*)(op + hi_at + (slot0 + (t & 1)) * 2) = make_uint2(code[4], code[5]);
+      if (t < 3) {
+        f32x32_t rr;
+        asm volatile("v_cvt_scalef32_pk32_f32_fp6 %0, %1, %2" : "=&v"(rr) : "v"(code), "v"(one));
+#pragma unroll
+        for (int k = 0; k < 16; ++k) {
+          va[k] = (va[k] - rr[2 * k]) * 32.0f;
+          vb[k] = (vb[k] - rr[2 * k + 1]) * 32.0f;
+        }
+      }
+    }
+  }
+}
+
+// sq[0 .. tot) = elements off .. off + have of q as fp32, zeros behind them (off, have and tot multiples of 8):
+// 16-byte loads, all of a thread's in flight together, when q allows them
+__device__ __forceinline__ void rows_to_lds(const void* __restrict__ q, int dtype, int64_t off, int have, int tot,
+                                            float* __restrict__ sq, int tid, int n_threads) {
+  if ((((uintptr_t)q) & 15) == 0 && dtype != TQ_F32) {
+    const uint4* src = (const uint4*)((const uint16_t*)q + off);
+    const bool bf = dtype == TQ_BF16;
+#pragma unroll 4
+    for (int c = tid; c < tot / 8; c += n_threads) {
+      const uint4 w = 8 * c < have ? src[c] : make_uint4(0u, 0u, 0u, 0u);
+      const uint32_t ws[4] = {w.x, w.y, w.z, w.w};
+      float v[8];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        v[2 * k] = bf ? __uint_as_float(ws[k] << 16) : f16_bits_to_f32((uint16_t)(ws[k] & 0xffffu));
+        v[2 * k + 1] = bf ? __uint_as_float(ws[k] & 0xffff0000u) : f16_bits_to_f32((uint16_t)(ws[k] >> 16));
+      }
+      *(float4*)(sq + 8 * c) = make_float4(v[0], v[1], v[2], v[3]);
+      *(float4*)(sq + 8 * c + 4) = make_float4(v[4], v[5], v[6], v[7]);
+    }
+  } else if ((((uintptr_t)q) & 15) == 0) {
+    const float4* src = (const float4*)((const float*)q + off);
+#pragma unroll 4
+    for (int c = tid; c < tot / 4; c += n_threads)
+      *(float4*)(sq + 4 * c) = 4 * c < have ? src[c] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+  } else {
+    for (int o = tid; o < tot; o += n_threads) sq[o] = o < have ? load_as_f32(q, off + o, dtype) : 0.0f;
+  }
+}
+
 // BATCH: matrix rows of both matrices requested before the first is used (8, 16 or 24, a divisor of the d / 8 rows a
 // thread contracts): the kernel is a chain of memory latencies, one per batch (head_dim 576: 9 -> 3; the sums add in
 // the same order whatever the batch).
@@ -41,7 +158,25 @@ rotate_query_kernel(const void* __restrict__ q, int dtype, int64_t rows, int R, 
   float* pb = pa + ROT_SLICES * R * ROT_COLS;
   const int64_t row0 = (int64_t)blockIdx.x * R;
   const int nr = (int)((rows - row0) < R ? (rows - row0) : R);
-  for (int o = tid; o < R * d; o += blockDim.x) sq[o] = o < nr * d ? load_as_f32(q, row0 * d + o, dtype) : 0.0f;
+  // the first batch of matrix rows (and, below, the column sums) is requested before the queries: neither depends on them
+  const int per = d / ROT_SLICES, i0 = sl * per;
+  float mp[BATCH], ms[BATCH];
+#pragma unroll
+  for (int k = 0; k < BATCH; ++k) {
+    mp[k] = ly.PiT[(int64_t)(i0 + k) * d + j];
+    ms[k] = ly.ST[(int64_t)(i0 + k) * d + j];
+  }
+  constexpr int CS = PACK ? 12 : 1;                // column sums of a lane (PACK; d <= 768)
+  float cs1[CS], cs2[CS];
+  if constexpr (PACK) {
+#pragma unroll
+    for (int k = 0; k < CS; ++k) {
+      const int c = min((tid & 63) + 64 * k, d - 1);
+      cs1[k] = ly.Pi_colsum[c];
+      cs2[k] = ly.S_colsum[c];
+    }
+  }
+  rows_to_lds(q, dtype, row0 * d, nr * d, R * d, sq, tid, (int)blockDim.x);
   __syncthreads();
   float* s_rot = pb + ROT_SLICES * R * ROT_COLS;   // PACK: [R][ROT_COLS] this word's rotated values, then the sketched ones
   float* s_sk = s_rot + R * ROT_COLS;
@@ -52,15 +187,6 @@ rotate_query_kernel(const void* __restrict__ q, int dtype, int64_t rows, int R, 
     const int lane = tid & 63, wv = tid >> 6, n_wv = (int)blockDim.x >> 6;
     float cmax = 0.0f;
     for (int t = 0; t < ly.n_terms; ++t) cmax = fmaxf(cmax, fabsf(ly.term_coef[t]));
-    // (this lane's column sums: requested once, for all rows)
-    constexpr int CS = 12;                         // d <= 768
-    float cs1[CS], cs2[CS];
-#pragma unroll
-    for (int k = 0; k < CS; ++k) {
-      const int c = min(lane + 64 * k, d - 1);
-      cs1[k] = ly.Pi_colsum[c];
-      cs2[k] = ly.S_colsum[c];
-    }
     for (int r = wv; r < nr; r += n_wv) {
       float ss = 0.0f, s1 = 0.0f, s2 = 0.0f;
 #pragma unroll
@@ -85,38 +211,20 @@ rotate_query_kernel(const void* __restrict__ q, int dtype, int64_t rows, int R, 
         }
       }
     }
-    if (tid < 16) {                                // coefficient of term plane tid (as the page kernel orders them)
-      const int mb = ly.mse_bits;
-      float coef = 1.0f;                           // the sign plane
-      if (tid < mb) {
-        coef = 0.0f;
-        for (int t = 0; t < ly.n_terms; ++t)
-          if (ly.term_mask[t] == (1 << (mb - 1 - tid))) coef = ly.term_coef[t];
-      } else if (tid < wp.ntp - 1) {
-        coef = 0.0f;
-        int seen = 0;
-        for (int t = 0; t < ly.n_terms; ++t) {
-          if (__builtin_popcount(ly.term_mask[t]) > 1) {
-            if (seen == tid - mb) coef = ly.term_coef[t];
-            ++seen;
-          }
-        }
-      }
-      s_cf[tid] = coef;
-    }
+    if (tid < 16) s_cf[tid] = wide_term_plane_coef(ly, wp.ntp, tid);
   }
-  const int per = d / ROT_SLICES, i0 = sl * per;
   const int r0 = half * ROT_MAX_ROWS, RH = min(R - r0, ROT_MAX_ROWS);      // this half's rows: r0 .. r0 + RH - 1
   float a[ROT_MAX_ROWS], b[ROT_MAX_ROWS];
 #pragma unroll
   for (int r = 0; r < ROT_MAX_ROWS; ++r) a[r] = b[r] = 0.0f;
   // BATCH matrix rows at a time: all their loads are in flight before the first use
   for (int ib = i0; ib < i0 + per; ib += BATCH) {
-    float mp[BATCH], ms[BATCH];
+    if (ib > i0) {                                         // (the same for every thread)
 #pragma unroll
-    for (int k = 0; k < BATCH; ++k) {
-      mp[k] = ly.PiT[(int64_t)(ib + k) * d + j];
-      ms[k] = ly.ST[(int64_t)(ib + k) * d + j];
+      for (int k = 0; k < BATCH; ++k) {
+        mp[k] = ly.PiT[(int64_t)(ib + k) * d + j];
+        ms[k] = ly.ST[(int64_t)(ib + k) * d + j];
+      }
     }
 #pragma unroll
     for (int r = 0; r < ROT_MAX_ROWS; ++r) {
@@ -155,65 +263,141 @@ rotate_query_kernel(const void* __restrict__ q, int dtype, int64_t rows, int R, 
   }
   if constexpr (PACK) {
     __syncthreads();
-    // one lane per (term plane, row): the word's 32 values as four fp6 terms (the packing conversion of gfx950 and its
-    // inverse for the residual), written where lane (row 2 g + term % 2, quarter word % 4) of operand (plane, row set
-    // term / 2, chunk word / 4) of the row's head group reads them
-    typedef float f32x16_t __attribute__((ext_vector_type(16)));
-    typedef float f32x32_t __attribute__((ext_vector_type(32)));
-    typedef uint32_t u32x6_t __attribute__((ext_vector_type(6)));
-    const int ntp = wp.ntp, j = blockIdx.y, W = d >> 5;
-    const int qa_stride = wide_qa_stride(d);
-    const bool half_op = (d & 127) != 0 && (j >> 2) == ((d + 127) >> 7) - 1;
-    const int hi_at = half_op ? 32 * 4 : 64 * 4;
-    (void)W;
-    for (int it = tid; it < ntp * nr; it += blockDim.x) {
-      const int tp = it / nr, r = it - tp * nr;
-      const bool is_sign = tp == ntp - 1;
-      // the row's place: sequence, head, group of at most 8 heads of its KV head, slot in the group
-      const int row = (int)row0 + r;                   // (32-bit arithmetic: the launcher checks the row count)
-      const int bq = row / wp.Hq, head = row - bq * wp.Hq;
-      const int g_tot = wp.Hq / wp.Hkv, kvh = head / g_tot, hh = head - kvh * g_tot;
-      const int g_max = (g_tot + wp.kv_div - 1) / wp.kv_div, grp = hh / g_max, g = hh - grp * g_max;
-      const int64_t group = ((int64_t)bq * wp.Hkv + kvh) * wp.kv_div + grp;
-      const float base = 4.0f * (is_sign ? s_rs[2 * r + 1] : s_cf[tp] * s_rs[2 * r]);
-      const float4* src = (const float4*)((is_sign ? s_sk : s_rot) + r * ROT_COLS);
-      float x[32];
+    wide_pack_word(wp, d, nr, (int)row0, (int)blockIdx.y, s_rot, s_sk, s_rs, s_cf, tid, (int)blockDim.x);
+  }
+}
+
+// The rotation with the PACK epilogue on the matrix cores, for bf16 queries and the split matrices of the layer
+// (tq_layer::Pi_split / S_split: three bf16 terms in MFMA operand order; a bf16 query is an exact single term, so
+// v_mfma_f32_16x16x32_bf16 gives fp32-accurate products).  A workgroup of eight wavefronts owns sixteen consecutive
+// query rows and one plane word (32 coordinates); wavefront (half word jt, product m, contraction half kh) runs
+// KPW = d / 64 contraction steps x 3 terms with the matrix as the row operand and the queries as the column operand.
+// Everything a wavefront needs is requested up front - its queries, a share of the column sums for the row statistics,
+// then the matrix terms - so the statistics are summed while the terms are on their way: one memory latency in all.
+// The halves meet in LDS; the rest is the vector-ALU kernel's epilogue.
+constexpr int ROTM_THREADS = 512, ROTM_LD = 36;
+__host__ __device__ inline int rotate_mfma_smem_floats() {
+  return 4 * 16 * ROTM_LD + 8 * 16 * 4 + 2 * 16 * ROT_COLS + 2 * 16 + 16;
+}
+
+template <int KPW>
+__global__ void __launch_bounds__(ROTM_THREADS)
+rotate_mfma_kernel(const uint16_t* __restrict__ q, int64_t rows, tq_layer ly, float* __restrict__ q_rot,
+                   float* __restrict__ q_sk, WidePack wp) {
+  extern __shared__ __align__(16) float sm[];
+  constexpr int KS = 2 * KPW, D = 32 * KS;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 15, kb = lane >> 4;
+  const int jt = wave & 1, m = (wave >> 1) & 1, kh = wave >> 2, share = wave & 3;
+  const int word = blockIdx.y;
+  const int64_t row0 = (int64_t)blockIdx.x * 16;
+  const int nr = (int)(rows - row0 < 16 ? rows - row0 : 16);
+  float* part = sm;                                  // [kh][m][16 rows][ROTM_LD]
+  float* s_st = part + 4 * 16 * ROTM_LD;             // [8 wavefronts][16 rows][4] partial statistics
+  float* s_rot = s_st + 8 * 16 * 4;                  // [16][32] the word's rotated values, then the sketched ones
+  float* s_sk = s_rot + 16 * ROT_COLS;
+  float* s_rs = s_sk + 16 * ROT_COLS;                // [16][2] multipliers of q_rot / q_sk
+  float* s_cf = s_rs + 2 * 16;                       // [16] coefficient of each term plane
+  // column operands: lane (row n, block kb) holds q[n][32 ks + 8 kb .. + 7]; rows beyond the last are zero
+  const uint16_t* qrow = q + (row0 + (n < nr ? n : nr - 1)) * D + kb * 8;
+  prep_u32x4 qb[KPW];
 #pragma unroll
-      for (int k = 0; k < 8; ++k) {
-        const float4 v4 = src[k];
-        x[4 * k] = v4.x; x[4 * k + 1] = v4.y; x[4 * k + 2] = v4.z; x[4 * k + 3] = v4.w;
-      }
-      f32x16_t va, vb;                      // contraction indices 0, 2, 4, ... and 1, 3, 5, ...
+  for (int k = 0; k < KPW; ++k) qb[k] = *(const prep_u32x4*)(qrow + (kh * KPW + k) * 32);
+  // this wavefront's share of the statistics: steps share, share + 4, ... of its contraction half
+  constexpr int NS = (KPW + 3) / 4;
+  prep_u32x4 xq[NS];
+  prep_f32x4 c1[NS][2], c2[NS][2];
 #pragma unroll
-      for (int kloc = 0; kloc < 32; ++kloc) {
-        const int c = 4 * (kloc & 7) + (kloc >> 3), t4 = kloc >> 3;      // coordinate within the word
-        // (the page kernel takes three of a nibble's four bits in place, as the fp4 numbers 0.5, 1, 2)
-        const float v = x[c] * (base * (t4 == 1 ? 0.5f : (t4 == 2 ? 0.25f : 1.0f)));
-        if (kloc & 1) vb[kloc >> 1] = v;
-        else va[kloc >> 1] = v;
-      }
-      uint32_t* op0 = wp.qa + group * (int64_t)(ntp * 2 * qa_stride) + (tp * 2) * qa_stride + (j >> 2) * WD_QA_OP;
-      const int slot0 = 2 * g + 16 * (j & 3);
-      const float one = 1.0f;
+  for (int i = 0; i < NS; ++i) {
+    const int kl = share + 4 * i < KPW ? share + 4 * i : 0;            // (a step that does not exist counts for nothing)
+    const int ks = kh * KPW + kl;
+    xq[i] = *(const prep_u32x4*)(qrow + ks * 32);
+    c1[i][0] = *(const prep_f32x4*)(ly.Pi_colsum + ks * 32 + kb * 8);
+    c1[i][1] = *(const prep_f32x4*)(ly.Pi_colsum + ks * 32 + kb * 8 + 4);
+    c2[i][0] = *(const prep_f32x4*)(ly.S_colsum + ks * 32 + kb * 8);
+    c2[i][1] = *(const prep_f32x4*)(ly.S_colsum + ks * 32 + kb * 8 + 4);
+  }
+  // row operands: the three bf16 terms of 16 matrix rows
+  prep_u32x4 ma[3][KPW];
+  {
+    const uint16_t* mat = m ? ly.S_split : ly.Pi_split;
 #pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        u32x6_t code;
-        asm volatile("v_cvt_scalef32_2xpk16_fp6_f32 %0, %1, %2, %3" : "=&v"(code) : "v"(va), "v"(vb), "v"(one));
-        uint32_t* op = op0 + (t >> 1) * qa_stride;
-        *(uint4*)(op + (slot0 + (t & 1)) * 4) = make_uint4(code[0], code[1], code[2], code[3]);
-        *(uint2*)(op + hi_at + (slot0 + (t & 1)) * 2) = make_uint2(code[4], code[5]);
-        if (t < 3) {
-          f32x32_t rr;
-          asm volatile("v_cvt_scalef32_pk32_f32_fp6 %0, %1, %2" : "=&v"(rr) : "v"(code), "v"(one));
+    for (int t = 0; t < 3; ++t) {
+      const uint16_t* base = mat + (((int64_t)(t * (D / 16) + word * 2 + jt) * KS + kh * KPW) * 64 + lane) * 8;
 #pragma unroll
-          for (int k = 0; k < 16; ++k) {
-            va[k] = (va[k] - rr[2 * k]) * 32.0f;
-            vb[k] = (vb[k] - rr[2 * k + 1]) * 32.0f;
-          }
-        }
-      }
+      for (int k = 0; k < KPW; ++k) ma[t][k] = *(const prep_u32x4*)(base + k * (64 * 8));
     }
   }
+  {
+    float ss = 0.0f, s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NS; ++i) {
+      const bool real = share + 4 * i < KPW && n < nr;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float xl = real ? __uint_as_float(xq[i][e] << 16) : 0.0f;
+        const float xh = real ? __uint_as_float(xq[i][e] & 0xffff0000u) : 0.0f;
+        const float cl1 = c1[i][e >> 1][2 * (e & 1)], ch1 = c1[i][e >> 1][2 * (e & 1) + 1];
+        const float cl2 = c2[i][e >> 1][2 * (e & 1)], ch2 = c2[i][e >> 1][2 * (e & 1) + 1];
+        ss = fmaf(xl, xl, fmaf(xh, xh, ss));
+        s1 = fmaf(xl, cl1, fmaf(xh, ch1, s1));
+        s2 = fmaf(xl, cl2, fmaf(xh, ch2, s2));
+      }
+    }
+    ss += __shfl_xor(ss, 16, 64); s1 += __shfl_xor(s1, 16, 64); s2 += __shfl_xor(s2, 16, 64);
+    ss += __shfl_xor(ss, 32, 64); s1 += __shfl_xor(s1, 32, 64); s2 += __shfl_xor(s2, 32, 64);
+    if (kb == 0) *(float4*)(s_st + (wave * 16 + n) * 4) = make_float4(ss, s1, s2, 0.0f);
+  }
+  if (n >= nr) {
+#pragma unroll
+    for (int k = 0; k < KPW; ++k) qb[k] = prep_u32x4{0u, 0u, 0u, 0u};
+  }
+  prep_f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+  for (int t = 2; t >= 0; --t)                                         // the small terms first
+#pragma unroll
+    for (int k = 0; k < KPW; ++k)
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(prep_bf16x8, ma[t][k]),
+                                                    __builtin_bit_cast(prep_bf16x8, qb[k]), acc, 0, 0, 0);
+  // result register i of lane (row n, quarter kb) is coordinate 16 jt + 4 kb + i of query row n
+  *(prep_f32x4*)(part + ((kh * 2 + m) * 16 + n) * ROTM_LD + jt * 16 + 4 * kb) = acc;
+  __syncthreads();
+  {
+    const int r = tid >> 5, c = tid & 31;                              // 512 threads: a (row, coordinate) each
+    const float ra = part[(0 * 16 + r) * ROTM_LD + c] + part[(2 * 16 + r) * ROTM_LD + c];
+    const float rb = part[(1 * 16 + r) * ROTM_LD + c] + part[(3 * 16 + r) * ROTM_LD + c];
+    s_rot[tid] = ra;
+    s_sk[tid] = rb;
+    if (r < nr) {
+      q_rot[(row0 + r) * D + word * ROT_COLS + c] = ra;
+      q_sk[(row0 + r) * D + word * ROT_COLS + c] = rb;
+    }
+  }
+  if (tid < 16) {                                                      // the statistics of row tid
+    const int r = tid;
+    float ss = 0.0f, s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+    for (int w = 0; w < 8; ++w) {
+      const float4 p = *(const float4*)(s_st + (w * 16 + r) * 4);
+      ss += p.x; s1 += p.y; s2 += p.z;
+    }
+    float cmax = 0.0f;
+    for (int t = 0; t < ly.n_terms; ++t) cmax = fmaxf(cmax, fabsf(ly.term_coef[t]));
+    const float nq = sqrtf(ss), k = wp.sm_scale * 1.4426950408889634f;
+    // bound < 2^e: e = exponent field - 126, kept within +-100
+    const int e1 = min(max((int)((__float_as_uint(fabsf(k) * nq * cmax) >> 23) & 255u) - 126, -100), 100);
+    const int e2 = min(max((int)((__float_as_uint(2.0f * fabsf(k * ly.qjl_scale) * nq * ly.S_rownorm_max) >> 23) & 255u) - 126, -100), 100);
+    s_rs[2 * r] = k * __uint_as_float((uint32_t)(127 - e1) << 23);
+    s_rs[2 * r + 1] = 2.0f * k * ly.qjl_scale * __uint_as_float((uint32_t)(127 - e2) << 23);
+    if (word == 0 && r < nr) {
+      float* st = wp.q_stat + (row0 + r) * 4;
+      st[0] = (float)e1; st[1] = (float)e2; st[2] = k * ly.term_const * s1; st[3] = -k * ly.qjl_scale * s2;
+    }
+  } else if (tid >= 64 && tid < 80) {
+    s_cf[tid - 64] = wide_term_plane_coef(ly, wp.ntp, tid - 64);
+  }
+  __syncthreads();
+  wide_pack_word(wp, D, nr, (int)row0, word, s_rot, s_sk, s_rs, s_cf, tid, ROTM_THREADS);
 }
 
 template <int PER, int DT, bool PACKED>
@@ -629,8 +813,22 @@ int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* 
   if (R < 1 || d % ROT_COLS || d % (8 * ROT_SLICES)) return TQ_EUNSUPPORTED;
   const bool pack = wide != nullptr && wide->qa != nullptr && wide->q_stat != nullptr && layer->Pi_colsum && layer->S_colsum &&
                     wide->ntp >= 2 && wide->ntp <= 9 && rows % wide->Hq == 0 && rows < (1 << 30) && d <= 768;
-  size_t smem = (size_t)(R * d + 2 * ROT_SLICES * R * ROT_COLS + (pack ? 2 * R * ROT_COLS + 2 * R + 16 : 0)) * sizeof(float);
   const WidePack wp = pack ? *wide : WidePack{};
+  // bf16 queries with the layer's split matrices: rotation and packing on the matrix cores
+  if (pack && dtype == TQ_BF16 && layer->Pi_split && layer->S_split && (((uintptr_t)q) & 15) == 0 && d % 64 == 0 &&
+      d >= 320 && d <= 704 && opt_prep_mfma.load(std::memory_order_relaxed) != 0) {
+    const dim3 mgrid((unsigned)((rows + 15) / 16), d / ROT_COLS), mblock(ROTM_THREADS);
+    const size_t msm = (size_t)rotate_mfma_smem_floats() * sizeof(float);
+#define TQ_ROTM(KPW) \
+  case KPW: rotate_mfma_kernel<KPW><<<mgrid, mblock, msm, st>>>((const uint16_t*)q, rows, *layer, q_rot, q_sk, wp); break;
+    switch (d / 64) {
+      TQ_ROTM(5) TQ_ROTM(6) TQ_ROTM(7) TQ_ROTM(8) TQ_ROTM(9) TQ_ROTM(10) TQ_ROTM(11)
+    }
+#undef TQ_ROTM
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? TQ_OK : (int)e;
+  }
+  size_t smem = (size_t)(R * d + 2 * ROT_SLICES * R * ROT_COLS + (pack ? 2 * R * ROT_COLS + 2 * R + 16 : 0)) * sizeof(float);
   const dim3 rgrid((unsigned)((rows + R - 1) / R), d / ROT_COLS), rblock(ROT_COLS * ROT_SLICES * (wide_rows ? 2 : 1));
   const int per = d / ROT_SLICES;
 #define TQ_ROTATE(BATCH, MAXR)                                                                                         \

@@ -131,12 +131,15 @@ class TurboQuantMSE(torch.nn.Module):
         key = (self.Pi.data_ptr(), self.Pi._version, None if S is None else (S.data_ptr(), S._version))
         if self._splits is None or self._splits[0] != key:
             self._PiT = self.Pi.T.contiguous()
-            # only head_dim 128 / 256 have a matrix-core kernel; other sizes pass no split operands
-            mk = _ffi.split_bf16x3 if self.dim in (128, 256) else (lambda m: None)
+            # head_dim 128 / 256 have matrix-core quantise / de-quantise kernels; the head sizes of the wide-head decode
+            # kernel (320 ... 704 in steps of 64) rotate their queries on the matrix cores, which takes Pi and S only
+            wide = self.dim % 64 == 0 and 320 <= self.dim <= 704
+            mk = _ffi.split_bf16x3 if (self.dim in (128, 256) or wide) else (lambda m: None)
+            mkt = (lambda m: None) if wide else mk
             # head_dim 128: Pi^T also as fp6 terms, for the centroid contraction on the block-scaled MFMA
             fp6 = _ffi.split_fp6x5(self._PiT) if (self.dim == 128 and S is not None) else None
-            self._splits = (key, (mk(self.Pi), mk(self._PiT), None if S is None else mk(S),
-                                  None if ST is None else mk(ST), fp6))
+            self._splits = (key, (mk(self.Pi), mkt(self._PiT), None if S is None else mk(S),
+                                  None if ST is None else mkt(ST), fp6))
         qc = None
         if S is not None:
             if getattr(self, "_query_consts", None) is None or self._query_consts[0] != key:
