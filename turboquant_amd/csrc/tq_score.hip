@@ -43,7 +43,7 @@ __device__ __forceinline__ float wide_term_plane_coef(const tq_layer& ly, int nt
 // rows' multipliers; s_cf: coefficient of each term plane.
 __device__ __forceinline__ void wide_pack_word(const WidePack& wp, int d, int nr, int row0, int j, const float* s_rot,
                                                const float* s_sk, const float* s_rs, const float* s_cf, int tid,
-                                               int n_threads) {
+                                               int n_threads, int tp_begin, int tp_end) {
   // one lane per (term plane, row): the word's 32 values as four fp6 terms (the packing conversion of gfx950 and its
   // inverse for the residual), written where lane (row 2 g + term % 2, quarter word % 4) of operand (plane, row set
   // term / 2, chunk word / 4) of the row's head group reads them
@@ -54,7 +54,7 @@ __device__ __forceinline__ void wide_pack_word(const WidePack& wp, int d, int nr
   const int qa_stride = wide_qa_stride(d);
   const bool half_op = (d & 127) != 0 && (j >> 2) == ((d + 127) >> 7) - 1;
   const int hi_at = half_op ? 32 * 4 : 64 * 4;
-  for (int it = tid; it < ntp * nr; it += n_threads) {
+  for (int it = tp_begin * nr + tid; it < tp_end * nr; it += n_threads) {      // (term planes tp_begin .. tp_end - 1)
     const int tp = it / nr, r = it - tp * nr;
     const bool is_sign = tp == ntp - 1;
     // the row's place: sequence, head, group of at most 8 heads of its KV head, slot in the group
@@ -263,59 +263,64 @@ rotate_query_kernel(const void* __restrict__ q, int dtype, int64_t rows, int R, 
   }
   if constexpr (PACK) {
     __syncthreads();
-    wide_pack_word(wp, d, nr, (int)row0, (int)blockIdx.y, s_rot, s_sk, s_rs, s_cf, tid, (int)blockDim.x);
+    wide_pack_word(wp, d, nr, (int)row0, (int)blockIdx.y, s_rot, s_sk, s_rs, s_cf, tid, (int)blockDim.x, 0, wp.ntp);
   }
 }
 
 // The rotation with the PACK epilogue on the matrix cores, for bf16 queries and the split matrices of the layer
 // (tq_layer::Pi_split / S_split: three bf16 terms in MFMA operand order; a bf16 query is an exact single term, so
-// v_mfma_f32_16x16x32_bf16 gives fp32-accurate products).  A workgroup of eight wavefronts owns sixteen consecutive
-// query rows and one plane word (32 coordinates); wavefront (half word jt, product m, contraction half kh) runs
-// KPW = d / 64 contraction steps x 3 terms with the matrix as the row operand and the queries as the column operand.
-// Everything a wavefront needs is requested up front - its queries, a share of the column sums for the row statistics,
-// then the matrix terms - so the statistics are summed while the terms are on their way: one memory latency in all.
-// The halves meet in LDS; the rest is the vector-ALU kernel's epilogue.
-constexpr int ROTM_THREADS = 512, ROTM_LD = 36;
+// v_mfma_f32_16x16x32_bf16 gives fp32-accurate products).  A workgroup of four wavefronts owns sixteen consecutive
+// query rows, one plane word (32 coordinates) and one of the two products (0: q Pi^T, whose values fill the
+// index and term planes of the operands; 1: q S^T, the sign plane) - a compute unit moves 64 bytes per cycle, and the
+// matrix terms of both products in one workgroup made the second half of its wavefronts wait 2 us for the first.
+// Wavefront (half word jt, contraction half kh) runs KPW = d / 64 contraction steps x 3 terms with the matrix as the
+// row operand and the queries as the column operand.  Everything a wavefront needs is requested up front - its
+// queries, a share of the column sums for the row statistics, then the matrix terms - so the statistics are summed
+// while the terms are on their way: one memory latency in all.  The halves meet in LDS, then the packing.
+constexpr int ROTM_THREADS = 256, ROTM_LD = 36;
 __host__ __device__ inline int rotate_mfma_smem_floats() {
-  return 4 * 16 * ROTM_LD + 8 * 16 * 4 + 2 * 16 * ROT_COLS + 2 * 16 + 16;
+  return 2 * 16 * ROTM_LD + 4 * 16 * 2 + 16 * ROT_COLS + 2 * 16 + 16;
 }
 
 template <int KPW>
 __global__ void __launch_bounds__(ROTM_THREADS)
-rotate_mfma_kernel(const uint16_t* __restrict__ q, int64_t rows, tq_layer ly, float* __restrict__ q_rot,
+rotate_mfma_kernel(const uint16_t* __restrict__ q, int64_t rows, int n_tiles, tq_layer ly, float* __restrict__ q_rot,
                    float* __restrict__ q_sk, WidePack wp) {
   extern __shared__ __align__(16) float sm[];
   constexpr int KS = 2 * KPW, D = 32 * KS;
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = lane & 15, kb = lane >> 4;
-  const int jt = wave & 1, m = (wave >> 1) & 1, kh = wave >> 2, share = wave & 3;
-  const int word = blockIdx.y;
-  const int64_t row0 = (int64_t)blockIdx.x * 16;
+  const int jt = wave & 1, kh = wave >> 1;
+  // Workgroup -> (plane word, product, row tile): workgroups go to the card's eight dies in turn, each die with an L2
+  // of its own, so the (word, product) pairs are dealt to the dies - pair p to die p % 8 - and all row tiles of a
+  // pair run on its die: the matrix terms are fetched into one L2, not into all eight.
+  const int id = blockIdx.x, pair = (id & 7) + 8 * ((id >> 3) / n_tiles);
+  if (pair >= 2 * KS) return;                        // (the pairs do not divide among eight dies)
+  const int word = pair >> 1, m = pair & 1;
+  const int64_t row0 = (int64_t)((id >> 3) % n_tiles) * 16;
   const int nr = (int)(rows - row0 < 16 ? rows - row0 : 16);
-  float* part = sm;                                  // [kh][m][16 rows][ROTM_LD]
-  float* s_st = part + 4 * 16 * ROTM_LD;             // [8 wavefronts][16 rows][4] partial statistics
-  float* s_rot = s_st + 8 * 16 * 4;                  // [16][32] the word's rotated values, then the sketched ones
-  float* s_sk = s_rot + 16 * ROT_COLS;
-  float* s_rs = s_sk + 16 * ROT_COLS;                // [16][2] multipliers of q_rot / q_sk
+  float* part = sm;                                  // [kh][16 rows][ROTM_LD]
+  float* s_st = part + 2 * 16 * ROTM_LD;             // [4 wavefronts][16 rows][2] partial statistics
+  float* s_val = s_st + 4 * 16 * 2;                  // [16][32] the word's rotated (sketched) values
+  float* s_rs = s_val + 16 * ROT_COLS;               // [16][2] multipliers of q_rot / q_sk (this product's is set)
   float* s_cf = s_rs + 2 * 16;                       // [16] coefficient of each term plane
   // column operands: lane (row n, block kb) holds q[n][32 ks + 8 kb .. + 7]; rows beyond the last are zero
   const uint16_t* qrow = q + (row0 + (n < nr ? n : nr - 1)) * D + kb * 8;
   prep_u32x4 qb[KPW];
 #pragma unroll
   for (int k = 0; k < KPW; ++k) qb[k] = *(const prep_u32x4*)(qrow + (kh * KPW + k) * 32);
-  // this wavefront's share of the statistics: steps share, share + 4, ... of its contraction half
-  constexpr int NS = (KPW + 3) / 4;
+  // this wavefront's share of the statistics: steps jt, jt + 2, ... of its contraction half
+  constexpr int NS = (KPW + 1) / 2;
+  const float* colsum = m ? ly.S_colsum : ly.Pi_colsum;
   prep_u32x4 xq[NS];
-  prep_f32x4 c1[NS][2], c2[NS][2];
+  prep_f32x4 cs[NS][2];
 #pragma unroll
   for (int i = 0; i < NS; ++i) {
-    const int kl = share + 4 * i < KPW ? share + 4 * i : 0;            // (a step that does not exist counts for nothing)
+    const int kl = jt + 2 * i < KPW ? jt + 2 * i : 0;                  // (a step that does not exist counts for nothing)
     const int ks = kh * KPW + kl;
     xq[i] = *(const prep_u32x4*)(qrow + ks * 32);
-    c1[i][0] = *(const prep_f32x4*)(ly.Pi_colsum + ks * 32 + kb * 8);
-    c1[i][1] = *(const prep_f32x4*)(ly.Pi_colsum + ks * 32 + kb * 8 + 4);
-    c2[i][0] = *(const prep_f32x4*)(ly.S_colsum + ks * 32 + kb * 8);
-    c2[i][1] = *(const prep_f32x4*)(ly.S_colsum + ks * 32 + kb * 8 + 4);
+    cs[i][0] = *(const prep_f32x4*)(colsum + ks * 32 + kb * 8);
+    cs[i][1] = *(const prep_f32x4*)(colsum + ks * 32 + kb * 8 + 4);
   }
   // row operands: the three bf16 terms of 16 matrix rows
   prep_u32x4 ma[3][KPW];
@@ -329,24 +334,21 @@ rotate_mfma_kernel(const uint16_t* __restrict__ q, int64_t rows, tq_layer ly, fl
     }
   }
   {
-    float ss = 0.0f, s1 = 0.0f, s2 = 0.0f;
+    float ss = 0.0f, s1 = 0.0f;
 #pragma unroll
     for (int i = 0; i < NS; ++i) {
-      const bool real = share + 4 * i < KPW && n < nr;
+      const bool real = jt + 2 * i < KPW && n < nr;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const float xl = real ? __uint_as_float(xq[i][e] << 16) : 0.0f;
         const float xh = real ? __uint_as_float(xq[i][e] & 0xffff0000u) : 0.0f;
-        const float cl1 = c1[i][e >> 1][2 * (e & 1)], ch1 = c1[i][e >> 1][2 * (e & 1) + 1];
-        const float cl2 = c2[i][e >> 1][2 * (e & 1)], ch2 = c2[i][e >> 1][2 * (e & 1) + 1];
         ss = fmaf(xl, xl, fmaf(xh, xh, ss));
-        s1 = fmaf(xl, cl1, fmaf(xh, ch1, s1));
-        s2 = fmaf(xl, cl2, fmaf(xh, ch2, s2));
+        s1 = fmaf(xl, cs[i][e >> 1][2 * (e & 1)], fmaf(xh, cs[i][e >> 1][2 * (e & 1) + 1], s1));
       }
     }
-    ss += __shfl_xor(ss, 16, 64); s1 += __shfl_xor(s1, 16, 64); s2 += __shfl_xor(s2, 16, 64);
-    ss += __shfl_xor(ss, 32, 64); s1 += __shfl_xor(s1, 32, 64); s2 += __shfl_xor(s2, 32, 64);
-    if (kb == 0) *(float4*)(s_st + (wave * 16 + n) * 4) = make_float4(ss, s1, s2, 0.0f);
+    ss += __shfl_xor(ss, 16, 64); s1 += __shfl_xor(s1, 16, 64);
+    ss += __shfl_xor(ss, 32, 64); s1 += __shfl_xor(s1, 32, 64);
+    if (kb == 0) *(float2*)(s_st + (wave * 16 + n) * 2) = make_float2(ss, s1);
   }
   if (n >= nr) {
 #pragma unroll
@@ -360,44 +362,45 @@ rotate_mfma_kernel(const uint16_t* __restrict__ q, int64_t rows, tq_layer ly, fl
       acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(prep_bf16x8, ma[t][k]),
                                                     __builtin_bit_cast(prep_bf16x8, qb[k]), acc, 0, 0, 0);
   // result register i of lane (row n, quarter kb) is coordinate 16 jt + 4 kb + i of query row n
-  *(prep_f32x4*)(part + ((kh * 2 + m) * 16 + n) * ROTM_LD + jt * 16 + 4 * kb) = acc;
+  *(prep_f32x4*)(part + (kh * 16 + n) * ROTM_LD + jt * 16 + 4 * kb) = acc;
   __syncthreads();
-  {
-    const int r = tid >> 5, c = tid & 31;                              // 512 threads: a (row, coordinate) each
-    const float ra = part[(0 * 16 + r) * ROTM_LD + c] + part[(2 * 16 + r) * ROTM_LD + c];
-    const float rb = part[(1 * 16 + r) * ROTM_LD + c] + part[(3 * 16 + r) * ROTM_LD + c];
-    s_rot[tid] = ra;
-    s_sk[tid] = rb;
-    if (r < nr) {
-      q_rot[(row0 + r) * D + word * ROT_COLS + c] = ra;
-      q_sk[(row0 + r) * D + word * ROT_COLS + c] = rb;
-    }
+  float* dst = m ? q_sk : q_rot;
+#pragma unroll
+  for (int o = tid; o < 16 * ROT_COLS; o += ROTM_THREADS) {            // a (row, coordinate) of the word
+    const int r = o >> 5, c = o & 31;
+    const float v = part[r * ROTM_LD + c] + part[(16 + r) * ROTM_LD + c];
+    s_val[o] = v;
+    if (r < nr) dst[(row0 + r) * D + word * ROT_COLS + c] = v;
   }
   if (tid < 16) {                                                      // the statistics of row tid
     const int r = tid;
-    float ss = 0.0f, s1 = 0.0f, s2 = 0.0f;
+    float ss = 0.0f, s1 = 0.0f;
 #pragma unroll
-    for (int w = 0; w < 8; ++w) {
-      const float4 p = *(const float4*)(s_st + (w * 16 + r) * 4);
-      ss += p.x; s1 += p.y; s2 += p.z;
+    for (int w = 0; w < 4; ++w) {
+      const float2 p = *(const float2*)(s_st + (w * 16 + r) * 2);
+      ss += p.x; s1 += p.y;
     }
-    float cmax = 0.0f;
-    for (int t = 0; t < ly.n_terms; ++t) cmax = fmaxf(cmax, fabsf(ly.term_coef[t]));
     const float nq = sqrtf(ss), k = wp.sm_scale * 1.4426950408889634f;
+    float* st = wp.q_stat + (row0 + r) * 4;
     // bound < 2^e: e = exponent field - 126, kept within +-100
-    const int e1 = min(max((int)((__float_as_uint(fabsf(k) * nq * cmax) >> 23) & 255u) - 126, -100), 100);
-    const int e2 = min(max((int)((__float_as_uint(2.0f * fabsf(k * ly.qjl_scale) * nq * ly.S_rownorm_max) >> 23) & 255u) - 126, -100), 100);
-    s_rs[2 * r] = k * __uint_as_float((uint32_t)(127 - e1) << 23);
-    s_rs[2 * r + 1] = 2.0f * k * ly.qjl_scale * __uint_as_float((uint32_t)(127 - e2) << 23);
-    if (word == 0 && r < nr) {
-      float* st = wp.q_stat + (row0 + r) * 4;
-      st[0] = (float)e1; st[1] = (float)e2; st[2] = k * ly.term_const * s1; st[3] = -k * ly.qjl_scale * s2;
+    if (m == 0) {
+      float cmax = 0.0f;
+      for (int t = 0; t < ly.n_terms; ++t) cmax = fmaxf(cmax, fabsf(ly.term_coef[t]));
+      const int e1 = min(max((int)((__float_as_uint(fabsf(k) * nq * cmax) >> 23) & 255u) - 126, -100), 100);
+      s_rs[2 * r] = k * __uint_as_float((uint32_t)(127 - e1) << 23);
+      if (word == 0 && r < nr) { st[0] = (float)e1; st[2] = k * ly.term_const * s1; }
+    } else {
+      const int e2 = min(max((int)((__float_as_uint(2.0f * fabsf(k * ly.qjl_scale) * nq * ly.S_rownorm_max) >> 23) & 255u) - 126, -100), 100);
+      s_rs[2 * r + 1] = 2.0f * k * ly.qjl_scale * __uint_as_float((uint32_t)(127 - e2) << 23);
+      if (word == 0 && r < nr) { st[1] = (float)e2; st[3] = -k * ly.qjl_scale * s1; }
     }
   } else if (tid >= 64 && tid < 80) {
     s_cf[tid - 64] = wide_term_plane_coef(ly, wp.ntp, tid - 64);
   }
   __syncthreads();
-  wide_pack_word(wp, D, nr, (int)row0, word, s_rot, s_sk, s_rs, s_cf, tid, ROTM_THREADS);
+  // the index and term planes from the rotated values, the sign plane from the sketched ones
+  wide_pack_word(wp, D, nr, (int)row0, word, s_val, s_val, s_rs, s_cf, tid, ROTM_THREADS, m ? wp.ntp - 1 : 0,
+                 m ? wp.ntp : wp.ntp - 1);
 }
 
 template <int PER, int DT, bool PACKED>
@@ -817,10 +820,11 @@ int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* 
   // bf16 queries with the layer's split matrices: rotation and packing on the matrix cores
   if (pack && dtype == TQ_BF16 && layer->Pi_split && layer->S_split && (((uintptr_t)q) & 15) == 0 && d % 64 == 0 &&
       d >= 320 && d <= 704 && opt_prep_mfma.load(std::memory_order_relaxed) != 0) {
-    const dim3 mgrid((unsigned)((rows + 15) / 16), d / ROT_COLS), mblock(ROTM_THREADS);
+    const int n_tiles = (int)((rows + 15) / 16), pair_rounds = (2 * (d / ROT_COLS) + 7) / 8;
+    const dim3 mgrid((unsigned)(8 * pair_rounds * n_tiles)), mblock(ROTM_THREADS);
     const size_t msm = (size_t)rotate_mfma_smem_floats() * sizeof(float);
 #define TQ_ROTM(KPW) \
-  case KPW: rotate_mfma_kernel<KPW><<<mgrid, mblock, msm, st>>>((const uint16_t*)q, rows, *layer, q_rot, q_sk, wp); break;
+  case KPW: rotate_mfma_kernel<KPW><<<mgrid, mblock, msm, st>>>((const uint16_t*)q, rows, n_tiles, *layer, q_rot, q_sk, wp); break;
     switch (d / 64) {
       TQ_ROTM(5) TQ_ROTM(6) TQ_ROTM(7) TQ_ROTM(8) TQ_ROTM(9) TQ_ROTM(10) TQ_ROTM(11)
     }
