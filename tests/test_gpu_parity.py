@@ -1083,7 +1083,9 @@ def test_stream_read_probe_runs_and_rejects_bad_arguments(gpu):
 @pytest.mark.parametrize("d,dtype,Hq,Hkv,ring,n_split", [(128, torch.bfloat16, 16, 4, 128, None), (256, torch.bfloat16, 16, 2, 128, None),
                                                            (64, torch.float16, 8, 2, 200, None), (128, torch.float32, 4, 2, 48, None),
                                                            (256, torch.bfloat16, 16, 2, 128, 12),       # many splits: the exact tokens
-                                                           (128, torch.float16, 4, 1, 100, 9)])         # are shared by 2 / 4 workgroups
+                                                           (128, torch.float16, 4, 1, 100, 9),          # are shared by 2 / 4 workgroups
+                                                           (576, torch.bfloat16, 8, 1, 128, None),      # wide heads: the exact tail in the
+                                                           (512, torch.bfloat16, 16, 2, 100, 5)])       # launch of the matrix-core rotation
 def test_ring_entry_reads_the_exact_cache_in_place(gpu, d, dtype, Hq, Hkv, ring, n_split):
     """tq_decode_attn_paged_ring takes the exact recent tokens (score.py:99-111) straight from a paged exact
     cache through the block table; it must equal, bit for bit, gathering those rows with torch indexing and

@@ -269,6 +269,43 @@ def test_decode_wide_heads_on_the_matrix_cores(gpu, d, key_bits, vb, Hq, Hkv, dt
         assert torch.equal(outs["shipped"], outs["geometry at run time"]), "constant and run-time geometry disagree"
 
 
+@pytest.mark.parametrize("d,key_bits,vb,Hq,Hkv,lens,recent", [(576, 4, 4, 8, 1, [300, 77, 40], [128, 9, 0]),
+                                                              (512, 3, 2, 16, 2, [130, 513], [100, 100])])
+def test_hybrid_step_of_wide_heads_with_the_exact_tail_in_the_rotation_launch(gpu, d, key_bits, vb, Hq, Hkv, lens, recent):
+    """A whole hybrid step (score.py:99-111 + 138-173) with bf16 queries at head_dim 512 / 576 runs the exact-tail
+    workgroups in the launch of the matrix-core rotation.  The stages called apart (rotation, then tail + page
+    kernel + merge as launches of their own) do the same arithmetic: same output, bit for bit."""
+    g = torch.Generator().manual_seed(31 * d + vb)
+    B, max_len = len(lens), max(lens)
+    pages_per_seq = (max_len + 15) // 16
+    pool, _ = _make_pool(gpu, d, key_bits, vb, Hkv, B * pages_per_seq + 2, torch.bfloat16)
+    assert pool.page_kernel() == 2
+    table = torch.randperm(B * pages_per_seq + 2, generator=g)[: B * pages_per_seq].to(torch.int32).reshape(B, pages_per_seq).to(gpu)
+    k = torch.randn(B, max_len, Hkv, d, generator=g).bfloat16().to(gpu)
+    v = torch.randn(B, max_len, Hkv, d, generator=g).bfloat16().to(gpu)
+    pool.append(k, v, table)
+    q = torch.randn(B, Hq, d, generator=g).bfloat16().to(gpu)
+    rk = torch.randn(B, max(recent), Hkv, d, generator=g).bfloat16().to(gpu)
+    rv = torch.randn(B, max(recent), Hkv, d, generator=g).bfloat16().to(gpu)
+    seq = torch.tensor(lens, dtype=torch.int32, device=gpu)
+    rl = torch.tensor(recent, dtype=torch.int32, device=gpu)
+    n_split = 3
+    _progress(f"hybrid step d={d} lens={lens} recent={recent}: one call, then staged")
+    whole = pool.decode_attention(q, table, seq, recent_k=rk, recent_v=rv, recent_len=rl, n_split=n_split, max_len=max_len).clone()
+    ws = pool.workspace(B, Hq, n_split)
+    staged = torch.empty_like(q)
+    for stages in (1, 6):
+        pool.decode_attention(q, table, seq, recent_k=rk, recent_v=rv, recent_len=rl, n_split=n_split, max_len=max_len,
+                              workspace=ws, out=staged, stages=stages)
+    torch.cuda.synchronize()
+    assert torch.equal(whole, staged)
+    # against the oracle on the first sequence (history and exact tokens)
+    kc, vc = _store_from_oracle_view(pool, table[0], lens[0])
+    ref = O.hybrid_attention(q[0:1].cpu(), kc, vc, max(lens[0], O.MIN_HISTORY), params_of(pool.quantizer), Hkv,
+                             rk[0, :recent[0]].cpu(), rv[0, :recent[0]].cpu())
+    assert cosine(whole[0:1].cpu(), ref) >= COS_GATE
+
+
 def test_decode_head_dim_576_at_the_bench_shape_against_the_oracle(gpu):
     """Two sequences of the 16 x 8192 step bench.py times at head_dim 576 (8 query heads on one KV head, 4-bit keys,
     4-bit values; 16 splits of 16 blocks, the table registers of a workgroup move on): every sequence against the

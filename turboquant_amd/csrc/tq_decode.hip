@@ -832,6 +832,22 @@ prep_tail_kernel(TailArgs A, int n_tail, int B, int Gq, tq_layer ly, float* __re
   }
 }
 
+// The same for the head sizes of the wide-head page kernel with bf16 queries: the exact-tail workgroups and the rotation /
+// operand packing on the matrix cores (rotate_mfma_body: the first 256 threads of its workgroups) in one launch.
+template <int KPW, bool PAGED>
+__global__ void __launch_bounds__(TAIL_THREADS)
+rotate_tail_kernel(TailArgs A, int n_tail, int B, int n_tiles, tq_layer ly, float* __restrict__ q_rot,
+                   float* __restrict__ q_sk, WidePack wp) {
+  extern __shared__ __align__(16) float sm[];
+  const int id = blockIdx.x;
+  if (id < n_tail) {
+    const int per_z = A.Hkv * B;
+    exact_tail_words_body<TQ_BF16, 1, PAGED, true>(A, id % A.Hkv, (id / A.Hkv) % B, id / per_z, sm);
+  } else if (threadIdx.x < ROTM_THREADS) {
+    rotate_mfma_body<KPW>((const uint16_t*)A.q, (int64_t)B * A.Hq, n_tiles, ly, q_rot, q_sk, wp, id - n_tail, sm);
+  }
+}
+
 // n_parts partials are merged per row; consecutive rows are part_stride partials apart.
 // gridDim.y workgroups per row, each with an equal share of the row's channels (all of them repeat the
 // small weight computation).  A thread owns a pair of channels and every S-th part (S = 256 / pairs
@@ -942,6 +958,7 @@ int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* 
                         float* q_stat, uint32_t* qa_pack, int G, float sm_scale, hipStream_t st, bool q_rot_unused,
                         unsigned long long* arrivals, const PagePrefetch* prefetch, int g_tot, const WidePack* wide);
 bool prep_on_matrix_cores(const void* q, int dtype, int64_t rows, const tq_layer* layer, int G, int g_tot);
+bool rotate_on_matrix_cores(const void* q, int dtype, int64_t rows, const tq_layer* layer, const WidePack* wide);
 }  // namespace tq
 
 static size_t parts_floats(int B, int Hq, int d, int n_parts) { return (size_t)B * Hq * n_parts * (d + 2); }
@@ -1238,6 +1255,33 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
       }
 #undef TQ_LAUNCH_PT_DT
 #undef TQ_LAUNCH_PT
+      TQ_CHECK_LAUNCH();
+      tail_done = true;
+    } else if (tail && ta.wide && stages == 7 && (d == 512 || d == 576) && static_cast<int64_t>(n_tail) <= 4 * device_compute_units() &&
+               rotate_on_matrix_cores(q, dtype, (int64_t)B * Hq, layer, wide_pre.qa ? &wide_pre : nullptr)) {
+      // Hybrid step at the head sizes of latent attention: the exact tail shares the launch of the rotation
+      // (16 x 8192 at head_dim 576: one launch of 13 us instead of 10 + 13)
+      const int n_tiles = (B * Hq + 15) / 16, pair_rounds = (2 * (d / ROT_COLS) + 7) / 8;
+      size_t fsm = tail_words_smem(d, recent_rows, ta.tile_words);
+      if ((size_t)rotate_mfma_smem_floats() * sizeof(float) > fsm) fsm = (size_t)rotate_mfma_smem_floats() * sizeof(float);
+#define TQ_LAUNCH_RT(KPW, PAGED)                                                                                     \
+  {                                                                                                                  \
+    auto kern = rotate_tail_kernel<KPW, PAGED>;                                                                      \
+    if (fsm > 48 * 1024) {                                                                                           \
+      hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)fsm);   \
+      if (e != hipSuccess) return (int)e;                                                                            \
+    }                                                                                                                \
+    kern<<<dim3((unsigned)(n_tail + 8 * pair_rounds * n_tiles)), dim3(TAIL_THREADS), fsm, st>>>(                     \
+        ta, n_tail, B, n_tiles, *layer, q_rot, q_sk, wide_pre);                                                      \
+  }
+      if (d == 576) {
+        if (ts.paged) TQ_LAUNCH_RT(9, true)
+        else TQ_LAUNCH_RT(9, false)
+      } else {
+        if (ts.paged) TQ_LAUNCH_RT(8, true)
+        else TQ_LAUNCH_RT(8, false)
+      }
+#undef TQ_LAUNCH_RT
       TQ_CHECK_LAUNCH();
       tail_done = true;
     } else {

@@ -14,94 +14,7 @@ namespace tq {
 // ROT_COLS x ROT_SLICES threads: thread (j, s) sums slice s of the contraction for
 // its column of every row, so each matrix element is read once per workgroup; the
 // slices meet in LDS.
-constexpr int ROT_COLS = 32, ROT_SLICES = 8;
-
-// coefficient of term plane tp as the wide-head page kernel orders them: the index planes from the highest bit down,
-// the multi-bit Walsh terms, the sign plane
-__device__ __forceinline__ float wide_term_plane_coef(const tq_layer& ly, int ntp, int tp) {
-  const int mb = ly.mse_bits;
-  float coef = 1.0f;                               // the sign plane
-  if (tp < mb) {
-    coef = 0.0f;
-    for (int t = 0; t < ly.n_terms; ++t)
-      if (ly.term_mask[t] == (1 << (mb - 1 - tp))) coef = ly.term_coef[t];
-  } else if (tp < ntp - 1) {
-    coef = 0.0f;
-    int seen = 0;
-    for (int t = 0; t < ly.n_terms; ++t) {
-      if (__builtin_popcount(ly.term_mask[t]) > 1) {
-        if (seen == tp - mb) coef = ly.term_coef[t];
-        ++seen;
-      }
-    }
-  }
-  return coef;
-}
-
-// PACK epilogue of the rotation kernels: plane word j (32 coordinates) of nr query rows from row0 on, as the wide-head
-// page kernel's fp6 operands.  s_rot / s_sk: [row][32] rotated / sketched values of the word; s_rs: [row][2] the
-// rows' multipliers; s_cf: coefficient of each term plane.
-__device__ __forceinline__ void wide_pack_word(const WidePack& wp, int d, int nr, int row0, int j, const float* s_rot,
-                                               const float* s_sk, const float* s_rs, const float* s_cf, int tid,
-                                               int n_threads, int tp_begin, int tp_end) {
-  // one lane per (term plane, row): the word's 32 values as four fp6 terms (the packing conversion of gfx950 and its
-  // inverse for the residual), written where lane (row 2 g + term % 2, quarter word % 4) of operand (plane, row set
-  // term / 2, chunk word / 4) of the row's head group reads them
-  typedef float f32x16_t __attribute__((ext_vector_type(16)));
-  typedef float f32x32_t __attribute__((ext_vector_type(32)));
-  typedef uint32_t u32x6_t __attribute__((ext_vector_type(6)));
-  const int ntp = wp.ntp;
-  const int qa_stride = wide_qa_stride(d);
-  const bool half_op = (d & 127) != 0 && (j >> 2) == ((d + 127) >> 7) - 1;
-  const int hi_at = half_op ? 32 * 4 : 64 * 4;
-  for (int it = tp_begin * nr + tid; it < tp_end * nr; it += n_threads) {      // (term planes tp_begin .. tp_end - 1)
-    const int tp = it / nr, r = it - tp * nr;
-    const bool is_sign = tp == ntp - 1;
-    // the row's place: sequence, head, group of at most 8 heads of its KV head, slot in the group
-    const int row = row0 + r;                        // (32-bit arithmetic: the launcher checks the row count)
-    const int bq = row / wp.Hq, head = row - bq * wp.Hq;
-    const int g_tot = wp.Hq / wp.Hkv, kvh = head / g_tot, hh = head - kvh * g_tot;
-    const int g_max = (g_tot + wp.kv_div - 1) / wp.kv_div, grp = hh / g_max, g = hh - grp * g_max;
-    const int64_t group = ((int64_t)bq * wp.Hkv + kvh) * wp.kv_div + grp;
-    const float base = 4.0f * (is_sign ? s_rs[2 * r + 1] : s_cf[tp] * s_rs[2 * r]);
-    const float4* src = (const float4*)((is_sign ? s_sk : s_rot) + r * ROT_COLS);
-    float x[32];
-#pragma unroll
-    for (int k = 0; k < 8; ++k) {
-      const float4 v4 = src[k];
-      x[4 * k] = v4.x; x[4 * k + 1] = v4.y; x[4 * k + 2] = v4.z; x[4 * k + 3] = v4.w;
-    }
-    f32x16_t va, vb;                      // contraction indices 0, 2, 4, ... and 1, 3, 5, ...
-#pragma unroll
-    for (int kloc = 0; kloc < 32; ++kloc) {
-      const int c = 4 * (kloc & 7) + (kloc >> 3), t4 = kloc >> 3;      // coordinate within the word
-      // (the page kernel takes three of a nibble's four bits in place, as the fp4 numbers 0.5, 1, 2)
-      const float v = x[c] * (base * (t4 == 1 ? 0.5f : (t4 == 2 ? 0.25f : 1.0f)));
-      if (kloc & 1) vb[kloc >> 1] = v;
-      else va[kloc >> 1] = v;
-    }
-    uint32_t* op0 = wp.qa + group * (int64_t)(ntp * 2 * qa_stride) + (tp * 2) * qa_stride + (j >> 2) * WD_QA_OP;
-    const int slot0 = 2 * g + 16 * (j & 3);
-    const float one = 1.0f;
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      u32x6_t code;
-      asm volatile("v_cvt_scalef32_2xpk16_fp6_f32 %0, %1, %2, %3" : "=&v"(code) : "v"(va), "v"(vb), "v"(one));
-      uint32_t* op = op0 + (t >> 1) * qa_stride;
-      *(uint4*)(op + (slot0 + (t & 1)) * 4) = make_uint4(code[0], code[1], code[2], code[3]);
-      *(uint2*)(op + hi_at + (slot0 + (t & 1)) * 2) = make_uint2(code[4], code[5]);
-      if (t < 3) {
-        f32x32_t rr;
-        asm volatile("v_cvt_scalef32_pk32_f32_fp6 %0, %1, %2" : "=&v"(rr) : "v"(code), "v"(one));
-#pragma unroll
-        for (int k = 0; k < 16; ++k) {
-          va[k] = (va[k] - rr[2 * k]) * 32.0f;
-          vb[k] = (vb[k] - rr[2 * k + 1]) * 32.0f;
-        }
-      }
-    }
-  }
-}
+constexpr int ROT_SLICES = 8;      // (ROT_COLS = 32 output columns per workgroup: tq_prep.h)
 
 // sq[0 .. tot) = elements off .. off + have of q as fp32, zeros behind them (off, have and tot multiples of 8):
 // 16-byte loads, all of a thread's in flight together, when q allows them
@@ -267,140 +180,13 @@ rotate_query_kernel(const void* __restrict__ q, int dtype, int64_t rows, int R, 
   }
 }
 
-// The rotation with the PACK epilogue on the matrix cores, for bf16 queries and the split matrices of the layer
-// (tq_layer::Pi_split / S_split: three bf16 terms in MFMA operand order; a bf16 query is an exact single term, so
-// v_mfma_f32_16x16x32_bf16 gives fp32-accurate products).  A workgroup of four wavefronts owns sixteen consecutive
-// query rows, one plane word (32 coordinates) and one of the two products (0: q Pi^T, whose values fill the
-// index and term planes of the operands; 1: q S^T, the sign plane) - a compute unit moves 64 bytes per cycle, and the
-// matrix terms of both products in one workgroup made the second half of its wavefronts wait 2 us for the first.
-// Wavefront (half word jt, contraction half kh) runs KPW = d / 64 contraction steps x 3 terms with the matrix as the
-// row operand and the queries as the column operand.  Everything a wavefront needs is requested up front - its
-// queries, a share of the column sums for the row statistics, then the matrix terms - so the statistics are summed
-// while the terms are on their way: one memory latency in all.  The halves meet in LDS, then the packing.
-constexpr int ROTM_THREADS = 256, ROTM_LD = 36;
-__host__ __device__ inline int rotate_mfma_smem_floats() {
-  return 2 * 16 * ROTM_LD + 4 * 16 * 2 + 16 * ROT_COLS + 2 * 16 + 16;
-}
-
+// the rotation on the matrix cores (rotate_mfma_body, tq_prep.h) as a launch of its own
 template <int KPW>
 __global__ void __launch_bounds__(ROTM_THREADS)
 rotate_mfma_kernel(const uint16_t* __restrict__ q, int64_t rows, int n_tiles, tq_layer ly, float* __restrict__ q_rot,
                    float* __restrict__ q_sk, WidePack wp) {
   extern __shared__ __align__(16) float sm[];
-  constexpr int KS = 2 * KPW, D = 32 * KS;
-  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int n = lane & 15, kb = lane >> 4;
-  const int jt = wave & 1, kh = wave >> 1;
-  // Workgroup -> (plane word, product, row tile): workgroups go to the card's eight dies in turn, each die with an L2
-  // of its own, so the (word, product) pairs are dealt to the dies - pair p to die p % 8 - and all row tiles of a
-  // pair run on its die: the matrix terms are fetched into one L2, not into all eight.
-  const int id = blockIdx.x, pair = (id & 7) + 8 * ((id >> 3) / n_tiles);
-  if (pair >= 2 * KS) return;                        // (the pairs do not divide among eight dies)
-  const int word = pair >> 1, m = pair & 1;
-  const int64_t row0 = (int64_t)((id >> 3) % n_tiles) * 16;
-  const int nr = (int)(rows - row0 < 16 ? rows - row0 : 16);
-  float* part = sm;                                  // [kh][16 rows][ROTM_LD]
-  float* s_st = part + 2 * 16 * ROTM_LD;             // [4 wavefronts][16 rows][2] partial statistics
-  float* s_val = s_st + 4 * 16 * 2;                  // [16][32] the word's rotated (sketched) values
-  float* s_rs = s_val + 16 * ROT_COLS;               // [16][2] multipliers of q_rot / q_sk (this product's is set)
-  float* s_cf = s_rs + 2 * 16;                       // [16] coefficient of each term plane
-  // column operands: lane (row n, block kb) holds q[n][32 ks + 8 kb .. + 7]; rows beyond the last are zero
-  const uint16_t* qrow = q + (row0 + (n < nr ? n : nr - 1)) * D + kb * 8;
-  prep_u32x4 qb[KPW];
-#pragma unroll
-  for (int k = 0; k < KPW; ++k) qb[k] = *(const prep_u32x4*)(qrow + (kh * KPW + k) * 32);
-  // this wavefront's share of the statistics: steps jt, jt + 2, ... of its contraction half
-  constexpr int NS = (KPW + 1) / 2;
-  const float* colsum = m ? ly.S_colsum : ly.Pi_colsum;
-  prep_u32x4 xq[NS];
-  prep_f32x4 cs[NS][2];
-#pragma unroll
-  for (int i = 0; i < NS; ++i) {
-    const int kl = jt + 2 * i < KPW ? jt + 2 * i : 0;                  // (a step that does not exist counts for nothing)
-    const int ks = kh * KPW + kl;
-    xq[i] = *(const prep_u32x4*)(qrow + ks * 32);
-    cs[i][0] = *(const prep_f32x4*)(colsum + ks * 32 + kb * 8);
-    cs[i][1] = *(const prep_f32x4*)(colsum + ks * 32 + kb * 8 + 4);
-  }
-  // row operands: the three bf16 terms of 16 matrix rows
-  prep_u32x4 ma[3][KPW];
-  {
-    const uint16_t* mat = m ? ly.S_split : ly.Pi_split;
-#pragma unroll
-    for (int t = 0; t < 3; ++t) {
-      const uint16_t* base = mat + (((int64_t)(t * (D / 16) + word * 2 + jt) * KS + kh * KPW) * 64 + lane) * 8;
-#pragma unroll
-      for (int k = 0; k < KPW; ++k) ma[t][k] = *(const prep_u32x4*)(base + k * (64 * 8));
-    }
-  }
-  {
-    float ss = 0.0f, s1 = 0.0f;
-#pragma unroll
-    for (int i = 0; i < NS; ++i) {
-      const bool real = jt + 2 * i < KPW && n < nr;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const float xl = real ? __uint_as_float(xq[i][e] << 16) : 0.0f;
-        const float xh = real ? __uint_as_float(xq[i][e] & 0xffff0000u) : 0.0f;
-        ss = fmaf(xl, xl, fmaf(xh, xh, ss));
-        s1 = fmaf(xl, cs[i][e >> 1][2 * (e & 1)], fmaf(xh, cs[i][e >> 1][2 * (e & 1) + 1], s1));
-      }
-    }
-    ss += __shfl_xor(ss, 16, 64); s1 += __shfl_xor(s1, 16, 64);
-    ss += __shfl_xor(ss, 32, 64); s1 += __shfl_xor(s1, 32, 64);
-    if (kb == 0) *(float2*)(s_st + (wave * 16 + n) * 2) = make_float2(ss, s1);
-  }
-  if (n >= nr) {
-#pragma unroll
-    for (int k = 0; k < KPW; ++k) qb[k] = prep_u32x4{0u, 0u, 0u, 0u};
-  }
-  prep_f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-  for (int t = 2; t >= 0; --t)                                         // the small terms first
-#pragma unroll
-    for (int k = 0; k < KPW; ++k)
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(prep_bf16x8, ma[t][k]),
-                                                    __builtin_bit_cast(prep_bf16x8, qb[k]), acc, 0, 0, 0);
-  // result register i of lane (row n, quarter kb) is coordinate 16 jt + 4 kb + i of query row n
-  *(prep_f32x4*)(part + (kh * 16 + n) * ROTM_LD + jt * 16 + 4 * kb) = acc;
-  __syncthreads();
-  float* dst = m ? q_sk : q_rot;
-#pragma unroll
-  for (int o = tid; o < 16 * ROT_COLS; o += ROTM_THREADS) {            // a (row, coordinate) of the word
-    const int r = o >> 5, c = o & 31;
-    const float v = part[r * ROTM_LD + c] + part[(16 + r) * ROTM_LD + c];
-    s_val[o] = v;
-    if (r < nr) dst[(row0 + r) * D + word * ROT_COLS + c] = v;
-  }
-  if (tid < 16) {                                                      // the statistics of row tid
-    const int r = tid;
-    float ss = 0.0f, s1 = 0.0f;
-#pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      const float2 p = *(const float2*)(s_st + (w * 16 + r) * 2);
-      ss += p.x; s1 += p.y;
-    }
-    const float nq = sqrtf(ss), k = wp.sm_scale * 1.4426950408889634f;
-    float* st = wp.q_stat + (row0 + r) * 4;
-    // bound < 2^e: e = exponent field - 126, kept within +-100
-    if (m == 0) {
-      float cmax = 0.0f;
-      for (int t = 0; t < ly.n_terms; ++t) cmax = fmaxf(cmax, fabsf(ly.term_coef[t]));
-      const int e1 = min(max((int)((__float_as_uint(fabsf(k) * nq * cmax) >> 23) & 255u) - 126, -100), 100);
-      s_rs[2 * r] = k * __uint_as_float((uint32_t)(127 - e1) << 23);
-      if (word == 0 && r < nr) { st[0] = (float)e1; st[2] = k * ly.term_const * s1; }
-    } else {
-      const int e2 = min(max((int)((__float_as_uint(2.0f * fabsf(k * ly.qjl_scale) * nq * ly.S_rownorm_max) >> 23) & 255u) - 126, -100), 100);
-      s_rs[2 * r + 1] = 2.0f * k * ly.qjl_scale * __uint_as_float((uint32_t)(127 - e2) << 23);
-      if (word == 0 && r < nr) { st[1] = (float)e2; st[3] = -k * ly.qjl_scale * s1; }
-    }
-  } else if (tid >= 64 && tid < 80) {
-    s_cf[tid - 64] = wide_term_plane_coef(ly, wp.ntp, tid - 64);
-  }
-  __syncthreads();
-  // the index and term planes from the rotated values, the sign plane from the sketched ones
-  wide_pack_word(wp, D, nr, (int)row0, word, s_val, s_val, s_rs, s_cf, tid, ROTM_THREADS, m ? wp.ntp - 1 : 0,
-                 m ? wp.ntp : wp.ntp - 1);
+  rotate_mfma_body<KPW>(q, rows, n_tiles, ly, q_rot, q_sk, wp, (int)blockIdx.x, sm);
 }
 
 template <int PER, int DT, bool PACKED>
@@ -726,6 +512,19 @@ bool prep_on_matrix_cores(const void* q, int dtype, int64_t rows, const tq_layer
          mfma_opt != 0 && (d == 128 || n_mprep >= 64 || mfma_opt > 1);
 }
 
+// Whether the rotation launch of a decode step also packs the wide-head page kernel's query operands ...
+static bool rotate_packs(int64_t rows, const tq_layer* layer, const WidePack* wide) {
+  return wide != nullptr && wide->qa != nullptr && wide->q_stat != nullptr && layer->Pi_colsum && layer->S_colsum &&
+         wide->ntp >= 2 && wide->ntp <= 9 && rows % wide->Hq == 0 && rows < (1 << 30) && layer->d <= 768;
+}
+// ... and whether it does so on the matrix cores (bf16 queries with the layer's split matrices)
+bool rotate_on_matrix_cores(const void* q, int dtype, int64_t rows, const tq_layer* layer, const WidePack* wide) {
+  const int d = layer->d;
+  return rotate_packs(rows, layer, wide) && dtype == TQ_BF16 && layer->Pi_split && layer->S_split &&
+         (((uintptr_t)q) & 15) == 0 && d % 64 == 0 && d >= 320 && d <= 704 &&
+         opt_prep_mfma.load(std::memory_order_relaxed) != 0;
+}
+
 // q_rot_unused: the caller only needs the packed operands and statistics (the page kernel on the matrix
 // cores), not the fp32 rotated / sketched queries
 int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* layer, float* q_rot, float* q_sk,
@@ -814,12 +613,10 @@ int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* 
   const int max_r = wide_rows ? 16 : ROT_MAX_ROWS;
   const int R = (int)(rows < max_r ? rows : max_r);
   if (R < 1 || d % ROT_COLS || d % (8 * ROT_SLICES)) return TQ_EUNSUPPORTED;
-  const bool pack = wide != nullptr && wide->qa != nullptr && wide->q_stat != nullptr && layer->Pi_colsum && layer->S_colsum &&
-                    wide->ntp >= 2 && wide->ntp <= 9 && rows % wide->Hq == 0 && rows < (1 << 30) && d <= 768;
+  const bool pack = rotate_packs(rows, layer, wide);
   const WidePack wp = pack ? *wide : WidePack{};
   // bf16 queries with the layer's split matrices: rotation and packing on the matrix cores
-  if (pack && dtype == TQ_BF16 && layer->Pi_split && layer->S_split && (((uintptr_t)q) & 15) == 0 && d % 64 == 0 &&
-      d >= 320 && d <= 704 && opt_prep_mfma.load(std::memory_order_relaxed) != 0) {
+  if (rotate_on_matrix_cores(q, dtype, rows, layer, wide)) {
     const int n_tiles = (int)((rows + 15) / 16), pair_rounds = (2 * (d / ROT_COLS) + 7) / 8;
     const dim3 mgrid((unsigned)(8 * pair_rounds * n_tiles)), mblock(ROTM_THREADS);
     const size_t msm = (size_t)rotate_mfma_smem_floats() * sizeof(float);
