@@ -16,6 +16,7 @@
 
 #include <chrono>
 #include <cstring>
+#include <type_traits>
 
 #include <hip/hip_ext.h>
 
@@ -676,23 +677,30 @@ __device__ __forceinline__ void exact_tail_words_body(const TailArgs& A, int h, 
       }
       __syncthreads();
     }
-    // (a thread takes two tokens per trip, 64 apart, against one read of the query values)
+    // (a thread takes two tokens per trip, 64 apart, against one read of the query values; one when the chunk
+    // has no second token for anybody: the share of a workgroup that splits the exact tokens with others)
     const int seg = tid & 7;
     constexpr int TPT = TAIL_THREADS / 8;
-    for (int t0 = 0; t0 < n; t0 += 2 * TPT) {                        // uniform trip count: the lane exchanges need every lane
-      const int t[2] = {t0 + (tid >> 3), t0 + (tid >> 3) + TPT};
-      const uint32_t* row0 = ktile + (t[0] < n ? t[0] : 0) * ldw;
-      const uint32_t* row1 = ktile + (t[1] < n ? t[1] : 0) * ldw;
-      float a[2][4] = {{0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}};
+    auto score_trip = [&](int t0, auto nt_tag) __attribute__((always_inline)) {
+      constexpr int NT = decltype(nt_tag)::value;
+      int t[NT];
+      const uint32_t* row[NT];
+      float a[NT][4];
+#pragma unroll
+      for (int u = 0; u < NT; ++u) {
+        t[u] = t0 + (tid >> 3) + u * TPT;
+        row[u] = ktile + (t[u] < n ? t[u] : 0) * ldw;
+        a[u][0] = a[u][1] = a[u][2] = a[u][3] = 0.0f;
+      }
       for (int cw = seg; cw < W; cw += 8) {
-        float x[2][2];
-        TailWord<DT>::unpack(row0[cw], x[0]);
-        TailWord<DT>::unpack(row1[cw], x[1]);
+        float x[NT][2];
+#pragma unroll
+        for (int u = 0; u < NT; ++u) TailWord<DT>::unpack(row[u][cw], x[u]);
 #pragma unroll
         for (int e = 0; e < EPW; ++e) {
           const float4 q4 = *reinterpret_cast<const float4*>(sq + (cw * EPW + e) * GC);
 #pragma unroll
-          for (int u = 0; u < 2; ++u) {
+          for (int u = 0; u < NT; ++u) {
             a[u][0] = fmaf(x[u][e], q4.x, a[u][0]);
             a[u][1] = fmaf(x[u][e], q4.y, a[u][1]);
             a[u][2] = fmaf(x[u][e], q4.z, a[u][2]);
@@ -701,13 +709,17 @@ __device__ __forceinline__ void exact_tail_words_body(const TailArgs& A, int h, 
         }
       }
 #pragma unroll
-      for (int u = 0; u < 2; ++u) {
+      for (int u = 0; u < NT; ++u) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) a[u][g] = lanes_sum_dpp<8>(a[u][g]);
         if (seg == 0 && t[u] < n)
           *reinterpret_cast<float4*>(ss + (c0 + t[u]) * GC) =
               make_float4(a[u][0] * sm_scale, a[u][1] * sm_scale, a[u][2] * sm_scale, a[u][3] * sm_scale);
       }
+    };
+    for (int t0 = 0; t0 < n; t0 += 2 * TPT) {                        // uniform trip count: the lane exchanges need every lane
+      if (t0 + TPT < n) score_trip(t0, std::integral_constant<int, 2>{});
+      else score_trip(t0, std::integral_constant<int, 1>{});
     }
   }
   __syncthreads();
