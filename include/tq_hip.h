@@ -252,7 +252,9 @@ size_t tq_decode_workspace_bytes(int B, int Hq, int d, int n_split);
  * exact tail (compute_hybrid_attention, score.py:29-173; kernel semantics of
  * triton_kernels.py:209-356 with GQA sharing, paging and split-K added).
  * q (B, Hq, d) `dtype` contiguous (it need not be the pages' dtype); query head h
- * reads KV head h / (Hq/Hkv).
+ * reads KV head h / (Hq/Hkv); Hq / Hkv is any whole number up to 128 (the reference's
+ * _matmul_attend, score.py:138-173, takes any ratio): the page kernels serve a KV head's
+ * heads in groups of at most 8 (matrix cores) or 16 (general kernel).
  * seq_lens[b] compressed tokens of sequence b sit in block_table[b*bt_stride + i]:
  * bt_stride > 0 is a row of that many entries per sequence; bt_stride < 0 one row of -bt_stride entries
  * shared by all sequences; 0 one shared row of unchecked length.  A length beyond the row is cut to

@@ -306,6 +306,25 @@ def test_hybrid_step_of_wide_heads_with_the_exact_tail_in_the_rotation_launch(gp
     assert cosine(whole[0:1].cpu(), ref) >= COS_GATE
 
 
+@pytest.mark.parametrize("d,key_bits,vb,Hq,Hkv,dtype,lens,recent,n_split", [
+    (576, 4, 4, 128, 1, torch.bfloat16, [300, 77], None, 2),           # multi-head latent attention: 128 heads on one latent
+    (512, 3, 2, 40, 2, torch.bfloat16, [130, 513], [7, 0], None),      # 20 heads per KV head: groups of 7, 7, 6; exact tail
+    (128, 3, 4, 71, 1, torch.bfloat16, [200, 37, 512], None, 2),       # multi-query attention with an odd head count
+    (128, 4, 2, 64, 2, torch.float16, [300, 77], [9, 0], None),        # 32 heads per KV head, fp16, exact tail
+    (256, 3, 2, 48, 2, torch.bfloat16, [700, 33], None, 4),            # 24 heads per KV head: three groups of 8
+    (64, 3, 4, 20, 1, torch.bfloat16, [257, 31], None, None),          # head_dim 64: groups of 7, 7, 6
+    (128, 3, 2, 40, 2, torch.float32, [200, 37], [5, 0], None),        # fp32 pages: the general kernel, groups of 10
+    (192, 3, 4, 33, 1, torch.bfloat16, [300, 77], None, 3)])           # a head size of the general kernel: groups of 11
+def test_decode_more_than_sixteen_query_heads_per_kv_head(gpu, d, key_bits, vb, Hq, Hkv, dtype, lens, recent, n_split):
+    """_matmul_attend (score.py:138-173) takes any ratio of query heads to KV heads (multi-query and multi-head latent
+    attention put 32 - 128 heads on one KV head): the matrix-core page kernels serve a KV head's heads in groups of at
+    most 8, whatever their number up to 128, and the general kernel in groups of at most 16.  Every sequence against
+    the oracle on the same store."""
+    _progress(f"decode d={d} kb={key_bits} vb={vb} Hq={Hq} Hkv={Hkv} {dtype}")
+    worst = _decode_case(gpu, d, key_bits, vb, len(lens), Hq, Hkv, lens, recent, seed=1300 + Hq, n_split=n_split, dtype=dtype)
+    _progress(f"   worst cosine {worst:.7f}")
+
+
 def test_decode_head_dim_576_at_the_bench_shape_against_the_oracle(gpu):
     """Two sequences of the 16 x 8192 step bench.py times at head_dim 576 (8 query heads on one KV head, 4-bit keys,
     4-bit values; 16 splits of 16 blocks, the table registers of a workgroup move on): every sequence against the

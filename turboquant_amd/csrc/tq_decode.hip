@@ -33,7 +33,8 @@ static __device__ __align__(256) unsigned char scratch[TQ_NOALLOC_SCRATCH_BYTES]
 
 namespace tq {
 
-constexpr int G_MAX = 16;      // query heads per KV head handled by one workgroup
+constexpr int G_MAX = 16;      // query heads per KV head handled by one workgroup of the general page kernel
+constexpr int G_LIMIT = 128;   // ... and per KV head in all: the matrix-core kernels serve them in groups of at most 8
 constexpr float NEG_BIG = -1.0e30f;
 
 // General page kernel (vector ALU) for the shapes without a matrix-core kernel: any head_dim that is a
@@ -71,10 +72,14 @@ __global__ void __launch_bounds__(GEN_THREADS)
 decode_pages_kernel(const float* __restrict__ q_rot, const float* __restrict__ q_sk, int Hq, int Hkv,
                     const uint8_t* __restrict__ pool, const int32_t* __restrict__ block_table, int bt_stride,
                     const int32_t* __restrict__ seq_lens, float sm_scale, tq_layer ly, tq_page_layout L,
-                    float* __restrict__ parts, int n_parts, int n_split, int len_sub, int max_pages, int num_pages) {
+                    float* __restrict__ parts, int n_parts, int n_split, int len_sub, int max_pages, int num_pages,
+                    int head_groups) {
   constexpr int GP = 4 * GP4;
-  const int d = ly.d, mb = ly.mse_bits, G = Hq / Hkv, words = d >> 5;
-  const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int d = ly.d, mb = ly.mse_bits, words = d >> 5;
+  // the query heads of a KV head in head_groups groups of at most G_MAX (workgroups blockIdx.y = KV head x groups + group)
+  const int g_all = Hq / Hkv, g_per = (g_all + head_groups - 1) / head_groups;
+  const int split = blockIdx.x, h = (int)blockIdx.y / head_groups, b = blockIdx.z;
+  const int g0 = ((int)blockIdx.y - h * head_groups) * g_per, G = min(g_per, g_all - g0);
   const int tid = threadIdx.x;
 
   extern __shared__ __align__(16) float smem[];
@@ -88,7 +93,7 @@ decode_pages_kernel(const float* __restrict__ q_rot, const float* __restrict__ q
 
   for (int o = tid; o < d * GP; o += GEN_THREADS) {
     const int c = o / GP, g = o - c * GP;
-    const int64_t row = (int64_t)b * Hq + h * G + (g < G ? g : 0);
+    const int64_t row = (int64_t)b * Hq + h * g_all + g0 + (g < G ? g : 0);
     s_rot[o] = g < G ? q_rot[row * d + c] : 0.0f;
     s_sk[o] = g < G ? q_sk[row * d + c] : 0.0f;
   }
@@ -277,7 +282,7 @@ decode_pages_kernel(const float* __restrict__ q_rot, const float* __restrict__ q
       aa += s_red[(t * GP + g) * d + ch];
       ll += s_ml[t * GP + g];
     }
-    float* out = parts + (((int64_t)b * Hq + h * G + g) * n_parts + split) * (d + 2);
+    float* out = parts + (((int64_t)b * Hq + h * g_all + g0 + g) * n_parts + split) * (d + 2);
     if (ch == 0) { out[0] = s_ml[4 * GP + g]; out[1] = ll; }
     out[2 + ch] = aa;
   }
@@ -1111,7 +1116,7 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   const int pool_pages = (int)(num_pages < 0x7fffffff ? num_pages : 0x7fffffff);
   const int d = layer->d, G = Hq / Hkv;
   if (d != layout->d || layer->mse_bits != layout->mse_bits) return TQ_EINVAL;
-  if (d < 64 || d > 768 || (d & 63) || G > G_MAX) return TQ_EUNSUPPORTED;
+  if (d < 64 || d > 768 || (d & 63) || G > G_LIMIT) return TQ_EUNSUPPORTED;
   if (layout->value_bits != 2 && layout->value_bits != 4 && layout->value_bits != 8) return TQ_EUNSUPPORTED;
   const bool tail = recent_k != nullptr && recent_rows > 0;
   if (tail && !recent_v) return TQ_ENULL;
@@ -1362,11 +1367,14 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   }
   if ((stages & 2) && mf == TQ_EUNSUPPORTED) {      // no matrix-core kernel for this shape: general kernel
     if (dtype < TQ_F32 || dtype > TQ_BF16) return TQ_EINVAL;
-    const int gp4 = (G + 3) / 4, gp = 4 * gp4;      // query heads rounded up to a multiple of 4
+    // (more than G_MAX query heads per KV head: groups of equal size, a workgroup each)
+    const int head_groups = (G + G_MAX - 1) / G_MAX, g_per = (G + head_groups - 1) / head_groups;
+    if ((int64_t)Hkv * head_groups > 65535) return TQ_EUNSUPPORTED;
+    const int gp4 = (g_per + 3) / 4, gp = 4 * gp4;      // query heads rounded up to a multiple of 4
     const int tg = d < GEN_THREADS ? GEN_THREADS / d : 1;
     const size_t work = (size_t)gp * (GEN_CHUNK > tg * d ? GEN_CHUNK : tg * d);    // weights, then slice partials
     const size_t smem = ((size_t)2 * d * gp + 32 + work) * sizeof(float);
-    dim3 grid(n_split, Hkv, B), block(GEN_THREADS);
+    dim3 grid(n_split, Hkv * head_groups, B), block(GEN_THREADS);
     // an armed pair of timing events goes to this kernel's dispatch as it would to the matrix-core kernel's
     hipEvent_t t_start = nullptr, t_stop = nullptr;
     const bool timed = take_time_hook(0, t_start, t_stop);
@@ -1380,10 +1388,10 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
     if (timed)                                                                                            \
       hipExtLaunchKernelGGL(kern, grid, block, smem, st, t_start, t_stop, 0, q_rot, q_sk, Hq, Hkv, pool, block_table,  \
                             bt_stride, seq_lens, sm_scale, *layer, *layout, parts, n_parts, n_split, len_sub,          \
-                            max_pages, pool_pages);                                                                      \
+                            max_pages, pool_pages, head_groups);                                                         \
     else                                                                                                  \
       kern<<<grid, block, smem, st>>>(q_rot, q_sk, Hq, Hkv, pool, block_table, bt_stride, seq_lens, sm_scale, *layer,  \
-                                      *layout, parts, n_parts, n_split, len_sub, max_pages, pool_pages);   \
+                                      *layout, parts, n_parts, n_split, len_sub, max_pages, pool_pages, head_groups); \
   }
 #define TQ_LAUNCH_DEC_G(VB)                                                      \
   {                                                                              \

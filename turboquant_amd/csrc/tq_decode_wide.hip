@@ -803,7 +803,7 @@ int launch_decode_wide(const float* q_rot, const float* q_sk, int B, int Hq, int
                        int max_pages, int num_pages, const WidePack& pre, hipStream_t st) {
   if (!decode_wide_has_kernel(ly, L)) return TQ_EUNSUPPORTED;
   const int g_tot = Hq / Hkv, kv_div = (g_tot + 7) / 8;
-  if (g_tot < 1 || g_tot > 16 || (int64_t)Hkv * kv_div > 65535) return TQ_EUNSUPPORTED;
+  if (g_tot < 1 || g_tot > 128 || (int64_t)Hkv * kv_div > 65535) return TQ_EUNSUPPORTED;
   int nring, kslot, vslot;
   size_t smem;
   wide_plan(ly, L, nring, kslot, vslot, smem);

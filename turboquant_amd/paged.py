@@ -179,7 +179,7 @@ class PagedKVPool:
 
     def _matrix_core_shape(self, Hq: Optional[int]) -> bool:
         """Whether decode runs on the matrix-core page kernel (head_dim 64 / 128 / 256, 16-bit pools, up to 4-bit
-        keys - 5-bit at head_dim 128 -, at most 16 query heads per KV head); only the split heuristic depends on it."""
+        keys - 5-bit at head_dim 128 -, at most 128 query heads per KV head); only the split heuristic depends on it."""
         if self.head_dim not in (64, 128, 256) or self.dtype not in (torch.bfloat16, torch.float16):
             return False
         if self.quantizer.bits - 1 > 4 or self.value_bits not in (2, 4, 8) or self.value_group_size not in (32, 64):
@@ -190,7 +190,7 @@ class PagedKVPool:
             return False                                     # 5-bit keys: head_dim 128 only
         if Hq is None:
             return True
-        return max(1, Hq // self.num_kv_heads) <= 16        # (more than 8 heads per KV head: groups of at most 8)
+        return max(1, Hq // self.num_kv_heads) <= 128       # (more than 8 heads per KV head: groups of at most 8)
 
     def default_splits(self, B: int, max_len: int, Hq: Optional[int] = None) -> int:
         """Split count of the page-streaming kernel.  Matrix-core kernel: its workgroups (4 wavefronts,
