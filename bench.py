@@ -496,6 +496,7 @@ SHAPE_TABLE = [
     (16, 8192, 8, 1, 576, 4, 4), (32, 8192, 8, 1, 576, 4, 4), (4, 32768, 16, 1, 576, 4, 4), (16, 8192, 8, 1, 512, 3, 4),
     (16, 8192, 32, 8, 128, 5, 4), (16, 8192, 64, 8, 128, 5, 4), (16, 8192, 32, 8, 128, 3, 8),
     (16, 8192, 88, 8, 128, 3, 4),
+    (16, 8192, 128, 1, 576, 4, 4), (16, 8192, 64, 1, 128, 3, 4),      # 128 heads on one latent; multi-query attention
 ]
 
 

@@ -308,6 +308,8 @@ def test_hybrid_step_of_wide_heads_with_the_exact_tail_in_the_rotation_launch(gp
 
 @pytest.mark.parametrize("d,key_bits,vb,Hq,Hkv,dtype,lens,recent,n_split", [
     (576, 4, 4, 128, 1, torch.bfloat16, [300, 77], None, 2),           # multi-head latent attention: 128 heads on one latent
+    (576, 4, 2, 120, 1, torch.bfloat16, [40, 17, 33, 16, 5, 64, 48, 31, 20], None, 1),     # 1080 query rows: the rotation takes
+                                                                       # six row tiles per workgroup, the last tile half full
     (512, 3, 2, 40, 2, torch.bfloat16, [130, 513], [7, 0], None),      # 20 heads per KV head: groups of 7, 7, 6; exact tail
     (128, 3, 4, 71, 1, torch.bfloat16, [200, 37, 512], None, 2),       # multi-query attention with an odd head count
     (128, 4, 2, 64, 2, torch.float16, [300, 77], [9, 0], None),        # 32 heads per KV head, fp16, exact tail

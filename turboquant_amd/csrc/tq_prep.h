@@ -628,6 +628,145 @@ __device__ __forceinline__ void rotate_mfma_body(const uint16_t* __restrict__ q,
                  m ? wp.ntp : wp.ntp - 1);
 }
 
+// The same rotation for thousands of rows (more workgroups than the card holds at once): a workgroup takes `tpw`
+// consecutive row tiles of its (plane word, product) pair against ONE fetch of the matrix terms and column sums
+// (2048 rows at head_dim 576 as a workgroup per tile pulled 560 MB of terms through the L2s).  First every tile's
+// products, sums and statistics - the matrix terms stay in registers, the halves meet in LDS buffers that alternate
+// by tile, the results wait in LDS -, then the packing of all tiles, which needs the registers the terms held.
+constexpr int ROTM_MAX_TPW = 8;
+__host__ __device__ inline int rotate_mfma_tiles_smem_floats(int tpw) {
+  return 2 * (2 * 16 * ROTM_LD + 4 * 16 * 2) + tpw * (16 * ROT_COLS + 2 * 16) + 16;
+}
+
+template <int KPW>
+__device__ __forceinline__ void rotate_mfma_tiles_body(const uint16_t* __restrict__ q, int64_t rows, int n_tiles, int tpw,
+                                                       const tq_layer& ly, float* __restrict__ q_rot,
+                                                       float* __restrict__ q_sk, const WidePack& wp, int id, float* sm) {
+  constexpr int KS = 2 * KPW, D = 32 * KS;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 15, kb = lane >> 4;
+  const int jt = wave & 1, kh = wave >> 1;
+  const int n_tg = (n_tiles + tpw - 1) / tpw;
+  const int pair = (id & 7) + 8 * ((id >> 3) / n_tg);              // (pair p on die p % 8, as in rotate_mfma_body)
+  if (pair >= 2 * KS) return;
+  const int word = pair >> 1, m = pair & 1;
+  const int tile0 = ((id >> 3) % n_tg) * tpw, tile1 = min(tile0 + tpw, n_tiles);
+  float* part = sm;                                  // [2 buffers][kh][16 rows][ROTM_LD]
+  float* s_st = part + 2 * 2 * 16 * ROTM_LD;         // [2 buffers][4 wavefronts][16 rows][2]
+  float* s_val = s_st + 2 * 4 * 16 * 2;              // [tpw][16][32]
+  float* s_rs = s_val + tpw * 16 * ROT_COLS;         // [tpw][16][2]
+  float* s_cf = s_rs + tpw * 2 * 16;                 // [16]
+  constexpr int NS = (KPW + 1) / 2;
+  const float* colsum = m ? ly.S_colsum : ly.Pi_colsum;
+  prep_f32x4 cs[NS][2];
+#pragma unroll
+  for (int i = 0; i < NS; ++i) {
+    const int kl = jt + 2 * i < KPW ? jt + 2 * i : 0;
+    const int ks = kh * KPW + kl;
+    cs[i][0] = *(const prep_f32x4*)(colsum + ks * 32 + kb * 8);
+    cs[i][1] = *(const prep_f32x4*)(colsum + ks * 32 + kb * 8 + 4);
+  }
+  prep_u32x4 ma[3][KPW];
+  {
+    const uint16_t* mat = m ? ly.S_split : ly.Pi_split;
+#pragma unroll
+    for (int t = 0; t < 3; ++t) {
+      const uint16_t* base = mat + (((int64_t)(t * (D / 16) + word * 2 + jt) * KS + kh * KPW) * 64 + lane) * 8;
+#pragma unroll
+      for (int k = 0; k < KPW; ++k) ma[t][k] = *(const prep_u32x4*)(base + k * (64 * 8));
+    }
+  }
+  if (tid >= 64 && tid < 80) s_cf[tid - 64] = wide_term_plane_coef(ly, wp.ntp, tid - 64);
+  float cmax = 0.0f;
+  for (int t = 0; t < ly.n_terms; ++t) cmax = fmaxf(cmax, fabsf(ly.term_coef[t]));
+  float* dst = m ? q_sk : q_rot;
+#pragma unroll 1
+  for (int tile = tile0; tile < tile1; ++tile) {
+    const int buf = (tile - tile0) & 1, ti = tile - tile0;
+    const int64_t row0 = (int64_t)tile * 16;
+    const int nr = (int)(rows - row0 < 16 ? rows - row0 : 16);
+    const uint16_t* qrow = q + (row0 + (n < nr ? n : nr - 1)) * D + kb * 8;
+    prep_u32x4 qb[KPW];
+#pragma unroll
+    for (int k = 0; k < KPW; ++k) qb[k] = *(const prep_u32x4*)(qrow + (kh * KPW + k) * 32);
+    if (n >= nr) {
+#pragma unroll
+      for (int k = 0; k < KPW; ++k) qb[k] = prep_u32x4{0u, 0u, 0u, 0u};
+    }
+    {  // this wavefront's share of the statistics: steps jt, jt + 2, ... of its contraction half
+      float ss = 0.0f, s1 = 0.0f;
+#pragma unroll
+      for (int i = 0; i < NS; ++i) {
+        const bool real = jt + 2 * i < KPW;
+        // (step 2 i + jt of the operand registers, picked with masks: an index that depends on the wavefront would
+        // move the registers to scratch memory)
+        const uint32_t odd = jt ? 0xffffffffu : 0u;
+        const int KO = 2 * i + 1 < KPW ? 2 * i + 1 : 2 * i;      // (a constant once the loop is unrolled)
+        prep_u32x4 x4;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) x4[e] = (qb[KO][e] & odd) | (qb[2 * i][e] & ~odd);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float xl = real ? __uint_as_float(x4[e] << 16) : 0.0f;
+          const float xh = real ? __uint_as_float(x4[e] & 0xffff0000u) : 0.0f;
+          ss = fmaf(xl, xl, fmaf(xh, xh, ss));
+          s1 = fmaf(xl, cs[i][e >> 1][2 * (e & 1)], fmaf(xh, cs[i][e >> 1][2 * (e & 1) + 1], s1));
+        }
+      }
+      ss += __shfl_xor(ss, 16, 64); s1 += __shfl_xor(s1, 16, 64);
+      ss += __shfl_xor(ss, 32, 64); s1 += __shfl_xor(s1, 32, 64);
+      if (kb == 0) *(float2*)(s_st + ((buf * 4 + wave) * 16 + n) * 2) = make_float2(ss, s1);
+    }
+    prep_f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int t = 2; t >= 0; --t)
+#pragma unroll
+      for (int k = 0; k < KPW; ++k)
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(prep_bf16x8, ma[t][k]),
+                                                      __builtin_bit_cast(prep_bf16x8, qb[k]), acc, 0, 0, 0);
+    *(prep_f32x4*)(part + ((buf * 2 + kh) * 16 + n) * ROTM_LD + jt * 16 + 4 * kb) = acc;
+    // (one barrier per tile: the buffers alternate, and a thread two tiles ahead has passed the barrier of the tile
+    // between, which every reader of this buffer reaches only after its reads)
+    __syncthreads();
+#pragma unroll
+    for (int o = tid; o < 16 * ROT_COLS; o += ROTM_THREADS) {
+      const int r = o >> 5, c = o & 31;
+      const float v = part[((buf * 2) * 16 + r) * ROTM_LD + c] + part[((buf * 2 + 1) * 16 + r) * ROTM_LD + c];
+      s_val[ti * 16 * ROT_COLS + o] = v;
+      if (r < nr) dst[(row0 + r) * D + word * ROT_COLS + c] = v;
+    }
+    if (tid < 16) {
+      const int r = tid;
+      float ss = 0.0f, s1 = 0.0f;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const float2 p = *(const float2*)(s_st + ((buf * 4 + w) * 16 + r) * 2);
+        ss += p.x; s1 += p.y;
+      }
+      const float nq = sqrtf(ss), k = wp.sm_scale * 1.4426950408889634f;
+      float* st = wp.q_stat + (row0 + r) * 4;
+      if (m == 0) {
+        const int e1 = min(max((int)((__float_as_uint(fabsf(k) * nq * cmax) >> 23) & 255u) - 126, -100), 100);
+        s_rs[ti * 32 + 2 * r] = k * __uint_as_float((uint32_t)(127 - e1) << 23);
+        if (word == 0 && r < nr) { st[0] = (float)e1; st[2] = k * ly.term_const * s1; }
+      } else {
+        const int e2 = min(max((int)((__float_as_uint(2.0f * fabsf(k * ly.qjl_scale) * nq * ly.S_rownorm_max) >> 23) & 255u) - 126, -100), 100);
+        s_rs[ti * 32 + 2 * r + 1] = 2.0f * k * ly.qjl_scale * __uint_as_float((uint32_t)(127 - e2) << 23);
+        if (word == 0 && r < nr) { st[1] = (float)e2; st[3] = -k * ly.qjl_scale * s1; }
+      }
+    }
+  }
+  __syncthreads();
+#pragma unroll 1
+  for (int tile = tile0; tile < tile1; ++tile) {
+    const int ti = tile - tile0;
+    const int64_t row0 = (int64_t)tile * 16;
+    const int nr = (int)(rows - row0 < 16 ? rows - row0 : 16);
+    wide_pack_word(wp, D, nr, (int)row0, word, s_val + ti * 16 * ROT_COLS, s_val + ti * 16 * ROT_COLS, s_rs + ti * 32, s_cf, tid,
+                   ROTM_THREADS, m ? wp.ntp - 1 : 0, m ? wp.ntp : wp.ntp - 1);
+  }
+}
+
 __host__ __device__ inline int prep_mfma_smem_floats() { return 2 * 16 * PREP_MFMA_LD + 32; }
 
 template <int D, bool WW>

@@ -189,6 +189,14 @@ rotate_mfma_kernel(const uint16_t* __restrict__ q, int64_t rows, int n_tiles, tq
   rotate_mfma_body<KPW>(q, rows, n_tiles, ly, q_rot, q_sk, wp, (int)blockIdx.x, sm);
 }
 
+template <int KPW>
+__global__ void __launch_bounds__(ROTM_THREADS)
+rotate_mfma_tiles_kernel(const uint16_t* __restrict__ q, int64_t rows, int n_tiles, int tpw, tq_layer ly,
+                         float* __restrict__ q_rot, float* __restrict__ q_sk, WidePack wp) {
+  extern __shared__ __align__(16) float sm[];
+  rotate_mfma_tiles_body<KPW>(q, rows, n_tiles, tpw, ly, q_rot, q_sk, wp, (int)blockIdx.x, sm);
+}
+
 template <int PER, int DT, bool PACKED>
 __global__ void __launch_bounds__(PREP_COLS * PREP_SLICES)
 prep_query_kernel(const void* __restrict__ q, int G, int gpw, int64_t n_rows, int g_tot, tq_layer ly, float sm_scale,
@@ -618,6 +626,23 @@ int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* 
   // bf16 queries with the layer's split matrices: rotation and packing on the matrix cores
   if (rotate_on_matrix_cores(q, dtype, rows, layer, wide)) {
     const int n_tiles = (int)((rows + 15) / 16), pair_rounds = (2 * (d / ROT_COLS) + 7) / 8;
+    // more workgroups than the card holds at once (two per compute unit of the kernel below): several row tiles per workgroup
+    const int64_t slots = 2 * (int64_t)device_compute_units();
+    int tpw = (int)((8 * (int64_t)pair_rounds * n_tiles + slots - 1) / slots);
+    tpw = tpw > ROTM_MAX_TPW ? ROTM_MAX_TPW : tpw;
+    if (tpw > 1) {
+      const int n_tg = (n_tiles + tpw - 1) / tpw;
+      const dim3 tgrid((unsigned)(8 * pair_rounds * n_tg));
+      const size_t tsm = (size_t)rotate_mfma_tiles_smem_floats(tpw) * sizeof(float);
+#define TQ_ROTT(KPW) \
+  case KPW: rotate_mfma_tiles_kernel<KPW><<<tgrid, dim3(ROTM_THREADS), tsm, st>>>((const uint16_t*)q, rows, n_tiles, tpw, *layer, q_rot, q_sk, wp); break;
+      switch (d / 64) {
+        TQ_ROTT(5) TQ_ROTT(6) TQ_ROTT(7) TQ_ROTT(8) TQ_ROTT(9) TQ_ROTT(10) TQ_ROTT(11)
+      }
+#undef TQ_ROTT
+      hipError_t e = hipGetLastError();
+      return e == hipSuccess ? TQ_OK : (int)e;
+    }
     const dim3 mgrid((unsigned)(8 * pair_rounds * n_tiles)), mblock(ROTM_THREADS);
     const size_t msm = (size_t)rotate_mfma_smem_floats() * sizeof(float);
 #define TQ_ROTM(KPW) \
