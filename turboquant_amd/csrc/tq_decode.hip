@@ -1127,6 +1127,7 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
   // groups of Gq = ceil(G / kv_div) heads, the last one of fewer when G does not divide (11 heads: 6 + 5)
   const int kv_div = (G + 7) / 8;
   const int Gq = (G + kv_div - 1) / kv_div;
+  if ((int64_t)Hkv * kv_div > 65535) return TQ_EUNSUPPORTED;      // (head groups are a grid dimension)
   // (the same table the launchers dispatch over: a shape without an instantiation keeps its split count and takes
   // the general kernel's preparation, which writes the fp32 rotated / sketched queries that kernel reads)
   const bool mfma_shape = kv_div && layer->Pi_colsum && layer->S_colsum && decode_mfma_has_kernel(*layer, *layout);
