@@ -96,50 +96,65 @@ key_tile_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
     su[t * d + j] = E::round(sx[t * d + j] / den);
   }
   __syncthreads();
-  // (4) y = u Pi^T (fp32), bucketise
-  float acc[TILE];
+  // The three contractions: a thread owns two columns (c0, c0 + d / 2) of eight tokens - the lower half of the
+  // workgroup the tile's first eight tokens, the upper half the others - so an LDS read of four vector elements feeds
+  // eight multiply-adds (with one column of sixteen tokens per thread the loop waited for LDS: nine wavefronts reading
+  // the same sixteen rows).  Every (token, column) sum still runs over the contraction in ascending order.
+  constexpr int TH = TILE / 2;
+  const int hd = d >> 1, upper = j >= hd ? 1 : 0, c0 = j - upper * hd, t_lo = upper * TH;
+  float acc[TH][2];
+  auto contract = [&](const float* __restrict__ M) __attribute__((always_inline)) {
 #pragma unroll
-  for (int t = 0; t < TILE; ++t) acc[t] = 0.0f;
-  for (int i = 0; i < d; i += 4) {
-    float m0 = ly.PiT[(int64_t)(i + 0) * d + j], m1 = ly.PiT[(int64_t)(i + 1) * d + j];
-    float m2 = ly.PiT[(int64_t)(i + 2) * d + j], m3 = ly.PiT[(int64_t)(i + 3) * d + j];
+    for (int t = 0; t < TH; ++t) acc[t][0] = acc[t][1] = 0.0f;
+    for (int i = 0; i < d; i += 4) {
+      float m[4][2];
 #pragma unroll
-    for (int t = 0; t < TILE; ++t) {
-      float4 u = *(const float4*)(su + t * d + i);
-      acc[t] = fmaf(u.x, m0, acc[t]); acc[t] = fmaf(u.y, m1, acc[t]);
-      acc[t] = fmaf(u.z, m2, acc[t]); acc[t] = fmaf(u.w, m3, acc[t]);
+      for (int k = 0; k < 4; ++k) {
+        m[k][0] = M[(int64_t)(i + k) * d + c0];
+        m[k][1] = M[(int64_t)(i + k) * d + c0 + hd];
+      }
+#pragma unroll
+      for (int t = 0; t < TH; ++t) {
+        const float4 u = *(const float4*)(su + (t_lo + t) * d + i);
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+          acc[t][c] = fmaf(u.x, m[0][c], acc[t][c]); acc[t][c] = fmaf(u.y, m[1][c], acc[t][c]);
+          acc[t][c] = fmaf(u.z, m[2][c], acc[t][c]); acc[t][c] = fmaf(u.w, m[3][c], acc[t][c]);
+        }
+      }
     }
-  }
+  };
+  // (4) y = u Pi^T (fp32), bucketise
+  contract(ly.PiT);
   __syncthreads();   // everyone is done reading su
 #pragma unroll
-  for (int t = 0; t < TILE; ++t) {
-    float yv = acc[t];
-    unsigned idx = 0;
-    for (int k = 0; k < n_thr; ++k) idx += !(yv <= ly.thresholds[k]);
-    sidx[t * d + j] = (uint8_t)idx;
-    su[t * d + j] = scent[idx];
-    if constexpr (std::is_same<Sink, KeyFlatSink>::value) {
-      if (sink.y_dbg && svalid[t]) sink.y_dbg[((int64_t)tile * TILE + t) * d + j] = yv;
+  for (int t = 0; t < TH; ++t) {
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      const int tt = t_lo + t, jc = c0 + c * hd;
+      float yv = acc[t][c];
+      unsigned idx = 0;
+      for (int k = 0; k < n_thr; ++k) idx += !(yv <= ly.thresholds[k]);
+      sidx[tt * d + jc] = (uint8_t)idx;
+      su[tt * d + jc] = scent[idx];
+      if constexpr (std::is_same<Sink, KeyFlatSink>::value) {
+        if (sink.y_dbg && svalid[tt]) sink.y_dbg[((int64_t)tile * TILE + tt) * d + jc] = yv;
+      }
     }
   }
   __syncthreads();
   if (!mse_only) {
     // (5) x_hat = (c Pi) * norm ; r = x - x_hat ; rho = ||r|| (quantizer.py:241-245)
-#pragma unroll
-    for (int t = 0; t < TILE; ++t) acc[t] = 0.0f;
-    for (int i = 0; i < d; i += 4) {
-      float m0 = ly.Pi[(int64_t)(i + 0) * d + j], m1 = ly.Pi[(int64_t)(i + 1) * d + j];
-      float m2 = ly.Pi[(int64_t)(i + 2) * d + j], m3 = ly.Pi[(int64_t)(i + 3) * d + j];
-#pragma unroll
-      for (int t = 0; t < TILE; ++t) {
-        float4 u = *(const float4*)(su + t * d + i);
-        acc[t] = fmaf(u.x, m0, acc[t]); acc[t] = fmaf(u.y, m1, acc[t]);
-        acc[t] = fmaf(u.z, m2, acc[t]); acc[t] = fmaf(u.w, m3, acc[t]);
-      }
-    }
+    contract(ly.Pi);
     __syncthreads();
 #pragma unroll
-    for (int t = 0; t < TILE; ++t) su[t * d + j] = sx[t * d + j] - acc[t] * snorm[t];
+    for (int t = 0; t < TH; ++t) {
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+        const int tt = t_lo + t, jc = c0 + c * hd;
+        su[tt * d + jc] = sx[tt * d + jc] - acc[t][c] * snorm[tt];
+      }
+    }
     __syncthreads();
     for (int t = wave; t < TILE; t += n_wave) {
       float ss = 0.0f;
@@ -148,23 +163,16 @@ key_tile_kernel(const void* __restrict__ x, Source src, tq_layer ly, Sink sink, 
       if (lane == 0) srn[t] = sqrtf(ss);
     }
     // (6) p = r S^T ; sign bits (quantizer.py:248-249)
+    contract(ly.ST);
 #pragma unroll
-    for (int t = 0; t < TILE; ++t) acc[t] = 0.0f;
-    for (int i = 0; i < d; i += 4) {
-      float m0 = ly.ST[(int64_t)(i + 0) * d + j], m1 = ly.ST[(int64_t)(i + 1) * d + j];
-      float m2 = ly.ST[(int64_t)(i + 2) * d + j], m3 = ly.ST[(int64_t)(i + 3) * d + j];
+    for (int t = 0; t < TH; ++t) {
 #pragma unroll
-      for (int t = 0; t < TILE; ++t) {
-        float4 u = *(const float4*)(su + t * d + i);
-        acc[t] = fmaf(u.x, m0, acc[t]); acc[t] = fmaf(u.y, m1, acc[t]);
-        acc[t] = fmaf(u.z, m2, acc[t]); acc[t] = fmaf(u.w, m3, acc[t]);
-      }
-    }
-#pragma unroll
-    for (int t = 0; t < TILE; ++t) {
-      ssgn[t * d + j] = acc[t] > 0.0f;
-      if constexpr (std::is_same<Sink, KeyFlatSink>::value) {
-        if (sink.p_dbg && svalid[t]) sink.p_dbg[((int64_t)tile * TILE + t) * d + j] = acc[t];
+      for (int c = 0; c < 2; ++c) {
+        const int tt = t_lo + t, jc = c0 + c * hd;
+        ssgn[tt * d + jc] = acc[t][c] > 0.0f;
+        if constexpr (std::is_same<Sink, KeyFlatSink>::value) {
+          if (sink.p_dbg && svalid[tt]) sink.p_dbg[((int64_t)tile * TILE + tt) * d + jc] = acc[t][c];
+        }
       }
     }
   }
