@@ -72,7 +72,7 @@ typedef struct tq_layer {
    *   ((((t*(d/16) + row/16)*(d/32) + col/32)*4 + (col%32)/8)*16 + row%16)*8 + col%8.
    * ST_split (the transpose of S) serves the de-quantiser.  NULL selects the vector-ALU
    * kernels.  At the head sizes of the wide-head decode kernel (320 ... 704 in steps of 64)
-   * Pi_split and S_split alone serve the decode step's query rotation (bf16 queries); the
+   * Pi_split and S_split alone serve the decode step's query rotation (bf16 / fp16 queries); the
    * transposes may stay NULL there.                                                    */
   const uint16_t *Pi_split, *PiT_split, *S_split, *ST_split;
   /* Optional constants of the fused query-preparation kernel of the decode path:
@@ -355,8 +355,8 @@ void tq_time_next_key_kernel(void *start_event, void *stop_event);
  *                      workgroups on, are rotated, sketched and packed on the matrix cores (three-term bf16 products
  *                      with Pi_split / S_split: fp32-accurate, summed in another order than the vector-ALU kernel,
  *                      so outputs agree to rounding, not bit for bit); 2: wherever the kernel applies; 0: never.
- *                      At the head sizes of the wide-head kernel, 1 or 2: bf16 queries are rotated and packed on the
- *                      matrix cores when the layer has Pi_split and S_split.
+ *                      At the head sizes of the wide-head kernel, 1 or 2: bf16 and fp16 queries are rotated and packed
+ *                      on the matrix cores when the layer has Pi_split and S_split.
  *   "merge_in_kernel"  1 (default): a compressed-only decode step on the matrix-core kernel with at most 8 context
  *                      splits has its splits merged by the last workgroup of the page kernel (two launches per
  *                      step); 0: always the separate merge kernel.

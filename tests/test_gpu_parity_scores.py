@@ -237,10 +237,8 @@ def test_decode_wide_heads_on_the_matrix_cores(gpu, d, key_bits, vb, Hq, Hkv, dt
     # as shipped (operands packed by the rotation launch; head_dim 512 / 576: the instantiations with constant page
     # geometry); operands packed by every page-kernel workgroup; the instantiation that takes the geometry at run time
     # (what the other head sizes run); the general kernel
-    # (bf16 queries are rotated and packed on the matrix cores; "prep_mfma" = 0 leaves that to the vector ALU)
-    variants = [("shipped", 1, 1, 1), ("packed in the page kernel", 1, 0, 1)]
-    if dtype == torch.bfloat16:
-        variants.append(("rotated on the vector ALU", 1, 1, 0))
+    # (bf16 and fp16 queries are rotated and packed on the matrix cores; "prep_mfma" = 0 leaves that to the vector ALU)
+    variants = [("shipped", 1, 1, 1), ("packed in the page kernel", 1, 0, 1), ("rotated on the vector ALU", 1, 1, 0)]
     if d in (512, 576):
         variants.append(("geometry at run time", 2, 1, 1))
     variants.append(("general kernel", 0, 1, 1))

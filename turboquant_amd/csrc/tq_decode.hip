@@ -1275,7 +1275,7 @@ static int decode_stages(const void* q, int dtype, int B, int Hq, int Hkv, const
 #undef TQ_LAUNCH_PT
       TQ_CHECK_LAUNCH();
       tail_done = true;
-    } else if (tail && ta.wide && stages == 7 && (d == 512 || d == 576) && static_cast<int64_t>(n_tail) <= 4 * device_compute_units() &&
+    } else if (tail && ta.wide && stages == 7 && dtype == TQ_BF16 && (d == 512 || d == 576) && static_cast<int64_t>(n_tail) <= 4 * device_compute_units() &&
                rotate_on_matrix_cores(q, dtype, (int64_t)B * Hq, layer, wide_pre.qa ? &wide_pre : nullptr)) {
       // Hybrid step at the head sizes of latent attention: the exact tail shares the launch of the rotation
       // (16 x 8192 at head_dim 576: one launch of 13 us instead of 10 + 13)

@@ -508,7 +508,9 @@ __host__ __device__ inline int rotate_mfma_smem_floats() {
 }
 
 // (id: the workgroup's place among the launch's rotation workgroups; the first ROTM_THREADS threads of a workgroup)
-template <int KPW>
+// F16Q: fp16 queries - a value of 11 significant bits is the exact sum of two bf16 terms (the rounded value and the
+// remainder), so every matrix term meets two query operands instead of one.
+template <int KPW, bool F16Q = false>
 __device__ __forceinline__ void rotate_mfma_body(const uint16_t* __restrict__ q, int64_t rows, int n_tiles, const tq_layer& ly,
                                                  float* __restrict__ q_rot, float* __restrict__ q_sk, const WidePack& wp,
                                                  int id, float* sm) {
@@ -565,8 +567,8 @@ __device__ __forceinline__ void rotate_mfma_body(const uint16_t* __restrict__ q,
       const bool real = jt + 2 * i < KPW && n < nr;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const float xl = real ? __uint_as_float(xq[i][e] << 16) : 0.0f;
-        const float xh = real ? __uint_as_float(xq[i][e] & 0xffff0000u) : 0.0f;
+        const float xl = real ? (F16Q ? f16_bits_to_f32((uint16_t)(xq[i][e] & 0xffffu)) : __uint_as_float(xq[i][e] << 16)) : 0.0f;
+        const float xh = real ? (F16Q ? f16_bits_to_f32((uint16_t)(xq[i][e] >> 16)) : __uint_as_float(xq[i][e] & 0xffff0000u)) : 0.0f;
         ss = fmaf(xl, xl, fmaf(xh, xh, ss));
         s1 = fmaf(xl, cs[i][e >> 1][2 * (e & 1)], fmaf(xh, cs[i][e >> 1][2 * (e & 1) + 1], s1));
       }
@@ -579,13 +581,37 @@ __device__ __forceinline__ void rotate_mfma_body(const uint16_t* __restrict__ q,
 #pragma unroll
     for (int k = 0; k < KPW; ++k) qb[k] = prep_u32x4{0u, 0u, 0u, 0u};
   }
+  prep_u32x4 ql[F16Q ? KPW : 1];                                       // fp16 queries: qb becomes the rounded values, ql the remainders
+  if constexpr (F16Q) {
+#pragma unroll
+    for (int k = 0; k < KPW; ++k) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        // (the packed conversion rounds to nearest even; the remainders have at most four significant bits: exact)
+        typedef float rot_f32x2 __attribute__((ext_vector_type(2)));
+        typedef __bf16 rot_bf16x2 __attribute__((ext_vector_type(2)));
+        const rot_f32x2 x = {f16_bits_to_f32((uint16_t)(qb[k][e] & 0xffffu)), f16_bits_to_f32((uint16_t)(qb[k][e] >> 16))};
+        const uint32_t hi = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, rot_bf16x2));
+        const rot_f32x2 rem = {x[0] - __uint_as_float(hi << 16), x[1] - __uint_as_float(hi & 0xffff0000u)};
+        qb[k][e] = hi;
+        ql[k][e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(rem, rot_bf16x2));
+      }
+    }
+  }
   prep_f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-  for (int t = 2; t >= 0; --t)                                         // the small terms first
+  for (int t = 2; t >= 0; --t) {                                       // the small terms first
+    if constexpr (F16Q) {
+#pragma unroll
+      for (int k = 0; k < KPW; ++k)
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(prep_bf16x8, ma[t][k]),
+                                                      __builtin_bit_cast(prep_bf16x8, ql[k]), acc, 0, 0, 0);
+    }
 #pragma unroll
     for (int k = 0; k < KPW; ++k)
       acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(prep_bf16x8, ma[t][k]),
                                                     __builtin_bit_cast(prep_bf16x8, qb[k]), acc, 0, 0, 0);
+  }
   // result register i of lane (row n, quarter kb) is coordinate 16 jt + 4 kb + i of query row n
   *(prep_f32x4*)(part + (kh * 16 + n) * ROTM_LD + jt * 16 + 4 * kb) = acc;
   __syncthreads();

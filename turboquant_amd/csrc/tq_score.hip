@@ -181,12 +181,12 @@ rotate_query_kernel(const void* __restrict__ q, int dtype, int64_t rows, int R, 
 }
 
 // the rotation on the matrix cores (rotate_mfma_body, tq_prep.h) as a launch of its own
-template <int KPW>
+template <int KPW, bool F16Q>
 __global__ void __launch_bounds__(ROTM_THREADS)
 rotate_mfma_kernel(const uint16_t* __restrict__ q, int64_t rows, int n_tiles, tq_layer ly, float* __restrict__ q_rot,
                    float* __restrict__ q_sk, WidePack wp) {
   extern __shared__ __align__(16) float sm[];
-  rotate_mfma_body<KPW>(q, rows, n_tiles, ly, q_rot, q_sk, wp, (int)blockIdx.x, sm);
+  rotate_mfma_body<KPW, F16Q>(q, rows, n_tiles, ly, q_rot, q_sk, wp, (int)blockIdx.x, sm);
 }
 
 template <int KPW>
@@ -526,10 +526,20 @@ static bool rotate_packs(int64_t rows, const tq_layer* layer, const WidePack* wi
          wide->ntp >= 2 && wide->ntp <= 9 && rows % wide->Hq == 0 && rows < (1 << 30) && layer->d <= 768;
 }
 // ... and whether it does so on the matrix cores (bf16 queries with the layer's split matrices)
+// row tiles a rotation workgroup takes: one while the card holds all workgroups at once (two per compute unit of the
+// kernel that takes several)
+static int rotate_tiles_per_workgroup(int64_t rows, int d) {
+  const int64_t n_tiles = (rows + 15) / 16, pair_rounds = (2 * (d / ROT_COLS) + 7) / 8;
+  const int64_t slots = 2 * (int64_t)device_compute_units();
+  const int64_t tpw = (8 * pair_rounds * n_tiles + slots - 1) / slots;
+  return (int)(tpw > ROTM_MAX_TPW ? ROTM_MAX_TPW : (tpw < 1 ? 1 : tpw));
+}
+// (bf16 queries; fp16 queries as two bf16 terms while a workgroup takes one row tile)
 bool rotate_on_matrix_cores(const void* q, int dtype, int64_t rows, const tq_layer* layer, const WidePack* wide) {
   const int d = layer->d;
-  return rotate_packs(rows, layer, wide) && dtype == TQ_BF16 && layer->Pi_split && layer->S_split &&
+  return rotate_packs(rows, layer, wide) && layer->Pi_split && layer->S_split &&
          (((uintptr_t)q) & 15) == 0 && d % 64 == 0 && d >= 320 && d <= 704 &&
+         (dtype == TQ_BF16 || (dtype == TQ_F16 && rotate_tiles_per_workgroup(rows, d) == 1)) &&
          opt_prep_mfma.load(std::memory_order_relaxed) != 0;
 }
 
@@ -627,9 +637,7 @@ int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* 
   if (rotate_on_matrix_cores(q, dtype, rows, layer, wide)) {
     const int n_tiles = (int)((rows + 15) / 16), pair_rounds = (2 * (d / ROT_COLS) + 7) / 8;
     // more workgroups than the card holds at once (two per compute unit of the kernel below): several row tiles per workgroup
-    const int64_t slots = 2 * (int64_t)device_compute_units();
-    int tpw = (int)((8 * (int64_t)pair_rounds * n_tiles + slots - 1) / slots);
-    tpw = tpw > ROTM_MAX_TPW ? ROTM_MAX_TPW : tpw;
+    const int tpw = rotate_tiles_per_workgroup(rows, d);
     if (tpw > 1) {
       const int n_tg = (n_tiles + tpw - 1) / tpw;
       const dim3 tgrid((unsigned)(8 * pair_rounds * n_tg));
@@ -646,7 +654,10 @@ int launch_rotate_query(const void* q, int dtype, int64_t rows, const tq_layer* 
     const dim3 mgrid((unsigned)(8 * pair_rounds * n_tiles)), mblock(ROTM_THREADS);
     const size_t msm = (size_t)rotate_mfma_smem_floats() * sizeof(float);
 #define TQ_ROTM(KPW) \
-  case KPW: rotate_mfma_kernel<KPW><<<mgrid, mblock, msm, st>>>((const uint16_t*)q, rows, n_tiles, *layer, q_rot, q_sk, wp); break;
+  case KPW:                                                                                                            \
+    if (dtype == TQ_F16) rotate_mfma_kernel<KPW, true><<<mgrid, mblock, msm, st>>>((const uint16_t*)q, rows, n_tiles, *layer, q_rot, q_sk, wp); \
+    else rotate_mfma_kernel<KPW, false><<<mgrid, mblock, msm, st>>>((const uint16_t*)q, rows, n_tiles, *layer, q_rot, q_sk, wp);               \
+    break;
     switch (d / 64) {
       TQ_ROTM(5) TQ_ROTM(6) TQ_ROTM(7) TQ_ROTM(8) TQ_ROTM(9) TQ_ROTM(10) TQ_ROTM(11)
     }
