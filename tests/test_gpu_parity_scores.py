@@ -267,6 +267,37 @@ def test_decode_wide_heads_on_the_matrix_cores(gpu, d, key_bits, vb, Hq, Hkv, dt
         assert torch.equal(outs["shipped"], outs["geometry at run time"]), "constant and run-time geometry disagree"
 
 
+@pytest.mark.parametrize("d,rows", [(128, 20), (576, 20), (576, 7), (256, 33)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_rotate_query_entry_point_on_every_input_dtype_and_alignment(gpu, d, rows, dtype):
+    """tq_rotate_query: q_rot = q Pi^T, q_sk = q S^T (triton_kernels.py:527-528) in fp32, for queries of every input
+    dtype.  Queries that start on a 16-byte boundary are staged with 16-byte loads, others element by element: the same
+    bits either way, and within fp32 rounding of a float64 product."""
+    import ctypes as C
+    from turboquant_amd import _ffi
+    from turboquant_amd.quantizer import TurboQuantProd
+    tq = TurboQuantProd(d, bits=3, device=gpu, seed=5)
+    ly = tq._layer()
+    g = torch.Generator().manual_seed(17 * d + rows)
+    q = torch.randn(rows, d, generator=g).to(dtype)
+    buf = torch.zeros(rows * d + 8, dtype=dtype, device=gpu)
+    outs = []
+    for shift in (0, 1):                               # element offset of the queries inside a 16-byte aligned buffer
+        buf[shift:shift + rows * d] = q.to(gpu).reshape(-1)
+        q_rot = torch.empty(rows, d, dtype=torch.float32, device=gpu)
+        q_sk = torch.empty(rows, d, dtype=torch.float32, device=gpu)
+        with _ffi.on_device(gpu):
+            _ffi.check(_ffi.lib().tq_rotate_query(buf.data_ptr() + shift * buf.element_size(), _ffi.dtype_tag(dtype), rows, C.byref(ly),
+                                                  q_rot.data_ptr(), q_sk.data_ptr(), _ffi.stream_ptr(gpu)), "tq_rotate_query")
+        torch.cuda.synchronize()
+        outs.append((q_rot.cpu(), q_sk.cpu()))
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+    q64 = q.double()
+    for got, M in ((outs[0][0], tq.mse_quantizer.Pi), (outs[0][1], tq.S)):
+        want = q64 @ M.detach().cpu().double().T
+        assert float((got.double() - want).abs().max()) <= 1e-5 * float(want.abs().max())
+
+
 @pytest.mark.parametrize("d,key_bits,vb,Hq,Hkv,lens,recent", [(576, 4, 4, 8, 1, [300, 77, 40], [128, 9, 0]),
                                                               (512, 3, 2, 16, 2, [130, 513], [100, 100])])
 def test_hybrid_step_of_wide_heads_with_the_exact_tail_in_the_rotation_launch(gpu, d, key_bits, vb, Hq, Hkv, lens, recent):
