@@ -531,7 +531,10 @@ static bool rotate_packs(int64_t rows, const tq_layer* layer, const WidePack* wi
 static int rotate_tiles_per_workgroup(int64_t rows, int d) {
   const int64_t n_tiles = (rows + 15) / 16, pair_rounds = (2 * (d / ROT_COLS) + 7) / 8;
   const int64_t slots = 2 * (int64_t)device_compute_units();
-  const int64_t tpw = (8 * pair_rounds * n_tiles + slots - 1) / slots;
+  // (workgroups of a (word, product) pair the card has room for: the tiles are shared out among that many, so that
+  // the launch is one round of workgroups and not one and a bit)
+  const int64_t per_pair = slots / (8 * pair_rounds) > 0 ? slots / (8 * pair_rounds) : 1;
+  const int64_t tpw = (n_tiles + per_pair - 1) / per_pair;
   return (int)(tpw > ROTM_MAX_TPW ? ROTM_MAX_TPW : (tpw < 1 ? 1 : tpw));
 }
 // (bf16 queries; fp16 queries as two bf16 terms while a workgroup takes one row tile)
